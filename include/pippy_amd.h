@@ -1,0 +1,223 @@
+/*
+ * pippy_amd.h -- C ABI of the MI355X (gfx950) kernels behind the PiPPy-compatible
+ * pipeline-stage hot path.
+ *
+ * The reference (pytorch/PiPPy 0.2.0) is pure Python and reaches all arithmetic through
+ * torch calls; it has no FFI of its own.  Each entry point below names the reference call
+ * site (file:line under the reference tree) whose torch call it replaces.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless a comment says "host";
+ *   - `stream` is a hipStream_t passed as void*; every launch is asynchronous on it;
+ *   - functions return PP_OK (0) or a PP_ERR_* code and never throw; pp_last_error() returns
+ *     a thread-local, human-readable description of the last failure;
+ *   - no entry point allocates or frees device memory: outputs and workspaces are
+ *     caller-provided;
+ *   - bf16 values are raw uint16 bit patterns (upper half of an IEEE fp32).
+ */
+#ifndef PIPPY_AMD_H
+#define PIPPY_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PP_OK 0
+#define PP_ERR_INVALID 1     /* bad argument (null pointer, negative size, misalignment) */
+#define PP_ERR_UNSUPPORTED 2 /* shape / layout / dtype combination not implemented */
+#define PP_ERR_LAUNCH 3      /* HIP reported an error at launch */
+
+typedef void* pp_stream;
+
+int pp_abi_version(void);
+const char* pp_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Microbatch split / merge.
+ *   split: pippy/microbatch.py:139-141  torch.tensor_split(v, n, dim)   (made contiguous)
+ *   merge: pippy/microbatch.py:415      torch.cat(values, dim)
+ * Both are row copies: a tensor of shape [outer, dim, inner] is `outer` rows per chunk, each a
+ * contiguous run of dim_chunk*inner elements.  Bit-exact for any element type (bytes move).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct pp_copy_seg {
+    const void* src;
+    void* dst;
+    int64_t n_rows;     /* rows to copy */
+    int64_t row_bytes;  /* contiguous bytes per row */
+    int64_t src_stride; /* bytes between consecutive source rows */
+    int64_t dst_stride; /* bytes between consecutive destination rows */
+} pp_copy_seg;
+
+#define PP_COPY_MAX_SEGS 64
+
+/* Copies up to PP_COPY_MAX_SEGS independent row segments in one launch.  `segs` is a HOST array. */
+int pp_copy_rows(const pp_copy_seg* segs, int n_segs, pp_stream stream);
+
+/* src: contiguous [outer, dim, inner_bytes]; dsts[i] (host array of device pointers): contiguous
+ * [outer, dim_i, inner_bytes] with dim_i from the tensor_split rule (the first dim % n_chunks
+ * chunks get ceil(dim / n_chunks), the rest floor).  Requires 1 <= n_chunks <= PP_COPY_MAX_SEGS. */
+int pp_split_copy(const void* src, void* const* dsts, int n_chunks, int64_t outer, int64_t dim,
+                  int64_t inner_bytes, pp_stream stream);
+
+/* srcs[i] (host array): contiguous [outer, chunk_dims[i], inner_bytes]; dst: contiguous
+ * [outer, sum(chunk_dims), inner_bytes]. */
+int pp_merge_copy(void* dst, const void* const* srcs, const int64_t* chunk_dims, int n_chunks,
+                  int64_t outer, int64_t inner_bytes, pp_stream stream);
+
+/* Generic strided gather of an N-d view (ndim <= 8) into a contiguous destination; one element
+ * (elem_bytes in {1,2,4,8,16}) per lane.  Used for inputs that are not contiguous to begin with.
+ * `sizes` / `src_strides` (in elements) are HOST arrays. */
+int pp_strided_copy_nd(void* dst, const void* src, int ndim, const int64_t* sizes,
+                       const int64_t* src_strides, int elem_bytes, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Gradient accumulation across microbatches.
+ *   pippy/_backward.py:67-69 (autograd AccumulateGrad reached from torch.autograd.backward)
+ *   acc[i] = (init ? 0 : acc[i]) + (float)g[i], one IEEE fp32 add per element, so the result is
+ *   bit-identical to torch `acc.add_(g.float())` applied in the same microbatch order.
+ * ---------------------------------------------------------------------------------------- */
+int pp_grad_accum_f32_bf16(float* acc, const uint16_t* g, int64_t n, int init, pp_stream stream);
+int pp_grad_accum_f32_f32(float* acc, const float* g, int64_t n, int init, pp_stream stream);
+/* fills n bytes with a byte value (used instead of hipMemsetAsync so that callers may capture) */
+int pp_fill_bytes(void* dst, int value, int64_t n_bytes, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * bf16 GEMM on MFMA with fp32 accumulation and fused epilogues.
+ *   forward  F.linear inside the stage module      pippy/_PipelineStage.py:420-428
+ *   backward dI / dW of the same linear            pippy/_backward.py:67-69
+ *   C[M,N] = epilogue( sum_k A(m,k) * B(n,k) )
+ * ---------------------------------------------------------------------------------------- */
+enum pp_gemm_epilogue {
+    PP_EPI_NONE = 0,          /* C = acc                                                    */
+    PP_EPI_BIAS = 1,          /* C = acc + bias[n]                                          */
+    PP_EPI_BIAS_GELU_ERF = 2, /* aux_out = acc + bias[n] (if non-null); C = gelu_erf(that)  */
+    PP_EPI_BIAS_GELU_TANH = 3,/* same with the tanh approximation                           */
+    PP_EPI_BIAS_RESIDUAL = 4, /* C = acc + bias[n] + aux_in[m,n]   (bias may be null)       */
+    PP_EPI_DGELU_ERF = 5,     /* C = acc * gelu_erf'(aux_in[m,n])                           */
+    PP_EPI_DGELU_TANH = 6,    /* C = acc * gelu_tanh'(aux_in[m,n])                          */
+    PP_EPI_ACCUM_F32 = 7,     /* C(fp32) = (beta ? C : 0) + acc     (fused grad accumulate) */
+    PP_EPI_BIAS_RELU = 8,     /* C = max(acc + bias[n], 0)                                  */
+    PP_EPI_DRELU = 9          /* C = aux_in[m,n] > 0 ? acc : 0                              */
+};
+
+enum pp_dtype { PP_BF16 = 0, PP_F32 = 1 };
+
+typedef struct pp_gemm_desc {
+    const void* A;  /* a_trans == 0: [M, K] row-major, lda >= K;  a_trans == 1: [K, M], lda >= M */
+    const void* B;  /* b_trans == 0: [N, K] row-major, ldb >= K;  b_trans == 1: [K, N], ldb >= N */
+    void* C;        /* [M, N] row-major, ldc >= N; bf16 unless c_dtype == PP_F32 */
+    int64_t M, N, K;
+    int64_t lda, ldb, ldc; /* in elements */
+    int32_t a_trans, b_trans;
+    int32_t epilogue;      /* enum pp_gemm_epilogue */
+    int32_t c_dtype;       /* enum pp_dtype */
+    const void* bias;      /* bf16 [N] or null */
+    const void* aux_in;    /* bf16 [M, N] with ld_aux (residual / saved pre-activation) */
+    void* aux_out;         /* bf16 [M, N] with ld_aux (pre-activation to save) or null */
+    int64_t ld_aux;
+    int32_t beta;          /* PP_EPI_ACCUM_F32: 0 overwrite, 1 accumulate */
+    int32_t reserved;
+} pp_gemm_desc;
+
+/* Requirements: A, B 16-byte aligned; K % 8 == 0; lda, ldb % 8 == 0; a transposed operand needs
+ * its contiguous extent (M resp. N) % 8 == 0; ldc, ld_aux % 4 == 0 (bf16) . */
+int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
+
+/* fp32 GEMM with the same descriptor (A, B, C, bias, aux fp32; config 1 of the baseline, the
+ * README MLP).  Only a_trans / b_trans, NONE, BIAS, BIAS_RELU, DRELU and ACCUM_F32 epilogues. */
+int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
+
+/* db[n] = sum_m dY[m, n]  (bias gradient of a linear; part of the dW pass).
+ * out is bf16 [N] (out_dtype PP_BF16) or fp32 [N]; workspace: fp32 [ws_rows = ceil(M/128), N]. */
+int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, int out_dtype,
+                   float* workspace, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * LayerNorm (F.layer_norm inside the stage module; backward via pippy/_backward.py:67-69).
+ * x, y, dy, dx: bf16 [rows, C]; gamma, beta: bf16 [C]; mean, rstd: fp32 [rows].
+ * ---------------------------------------------------------------------------------------- */
+int pp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                     float* rstd, int64_t rows, int64_t C, float eps, pp_stream stream);
+/* dx = LN'(dy) (+ dres if non-null): the input-gradient pass */
+int pp_layernorm_bwd_input(const void* dy, const void* x, const void* gamma, const float* mean,
+                           const float* rstd, const void* dres, void* dx, int64_t rows, int64_t C,
+                           pp_stream stream);
+/* dgamma, dbeta (bf16 [C] or fp32 by out_dtype): the weight-gradient pass.
+ * workspace: fp32 [2, ceil(rows/128), C]. */
+int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean, const float* rstd,
+                            void* dgamma, void* dbeta, int out_dtype, float* workspace,
+                            int64_t rows, int64_t C, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Multi-head attention, flash style (F.scaled_dot_product_attention inside the stage module).
+ * q, k, v: bf16, element (b, s, h, d) at base + b*stride_b + s*stride_s + h*head_dim + d, so the
+ * three can alias one fused [B, S, 3*H*D] projection output.  o: bf16 [B, S, H*D] contiguous.
+ * lse: fp32 [B, H, S] (log-sum-exp of the scaled scores; saved for backward).
+ * head_dim in {64, 128}; S % 64 == 0.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct pp_attn_desc {
+    const void* q; const void* k; const void* v;
+    void* o; float* lse;
+    const void* d_o;       /* backward only: bf16 [B, S, H*D] */
+    void* dq; void* dk; void* dv; /* backward only: same addressing as q, k, v */
+    float* delta;          /* backward workspace: fp32 [B, H, S] */
+    int64_t B, S, H, D;
+    int64_t stride_b, stride_s; /* of q/k/v (and dq/dk/dv), in elements */
+    float scale;           /* usually 1/sqrt(D) */
+    int32_t causal;
+} pp_attn_desc;
+int pp_attn_fwd(const pp_attn_desc* desc, pp_stream stream);
+int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Token + position embedding (F.embedding inside the first stage).
+ * y[t, :] = wte[ids[t], :] + (wpe ? wpe[t % seq, :] : 0);  ids int64 [n_tok]; bf16 tables.
+ * ---------------------------------------------------------------------------------------- */
+int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, void* y, int64_t n_tok,
+                 int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
+/* d_wte (fp32 [vocab, C]) += scatter(dy) with atomics; d_wpe (fp32 [seq, C]) += sum over batch */
+int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe, int64_t n_tok,
+                 int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Cross-entropy loss of one microbatch (loss_fn at pippy/PipelineSchedule.py:154-155 when it is
+ * torch cross_entropy with mean reduction) fused with its gradient.
+ * logits bf16 [rows, ld] (first V columns valid); target int64 [rows] (ignore_index skipped);
+ * loss: fp32 [1]; dlogits bf16 [rows, ld] (columns >= V written as 0) or null (loss only);
+ * workspace: fp32 [rows + 2].
+ * ---------------------------------------------------------------------------------------- */
+int pp_ce_loss(const void* logits, const int64_t* target, float* loss, void* dlogits,
+               float* workspace, int64_t rows, int64_t V, int64_t ld, int64_t ignore_index,
+               int logits_dtype, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Launch list: a host array of tagged descriptors executed in order on one stream.  One call
+ * replays a whole stage forward / input-gradient / weight-gradient pass for one microbatch
+ * (pippy/_PipelineStage.py:452-550) without returning to Python between kernels.
+ * ---------------------------------------------------------------------------------------- */
+enum pp_op_kind {
+    PP_OP_GEMM_BF16 = 1, PP_OP_GEMM_F32 = 2, PP_OP_COLSUM = 3, PP_OP_LN_FWD = 4,
+    PP_OP_LN_BWD_INPUT = 5, PP_OP_LN_BWD_WEIGHT = 6, PP_OP_ATTN_FWD = 7, PP_OP_ATTN_BWD = 8,
+    PP_OP_EMBED_FWD = 9, PP_OP_EMBED_BWD = 10, PP_OP_CE_LOSS = 11, PP_OP_ACCUM_BF16 = 12,
+    PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15
+};
+
+typedef struct pp_op {
+    int32_t kind;   /* enum pp_op_kind */
+    int32_t flags;
+    void* p[10];
+    int64_t i[12];
+    float f[2];
+    int32_t j[6];
+} pp_op;
+
+/* Runs ops[0..n) in order; stops at the first failure and returns its code (the index of the
+ * failing op is in pp_last_error()). */
+int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIPPY_AMD_H */

@@ -1,0 +1,74 @@
+"""fp32 CPU statements of the arithmetic a stage module performs.
+
+The reference runs the user's ``nn.Module.forward`` (pippy/_PipelineStage.py:420-428) and one
+``torch.autograd.backward`` (pippy/_backward.py:67-69); these are the torch calls the transformer
+and MLP stage modules of the baseline configurations reduce to.  All functions take and return
+fp32 CPU tensors; gradients come from autograd on these functions.
+
+Pinning: every function here is a direct torch library routine or a closed form checked against
+one in tests/test_oracle.py (gelu closed forms vs F.gelu, attention vs
+F.scaled_dot_product_attention, layer norm vs F.layer_norm, cross entropy vs F.cross_entropy).
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def linear(x, w, b=None):
+    return F.linear(x, w, b)
+
+
+def gelu_erf(x):
+    return 0.5 * x * (1.0 + torch.erf(x / math.sqrt(2.0)))
+
+
+def gelu_tanh(x):
+    return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
+
+
+def layer_norm(x, gamma, beta, eps):
+    mean = x.mean(-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(-1, keepdim=True)
+    y = (x - mean) / torch.sqrt(var + eps) * gamma
+    return y + beta if beta is not None else y
+
+
+def attention(q, k, v, causal, scale=None):
+    """q, k, v: [B, H, S, D] -> [B, H, S, D] (softmax(q k^T * scale + mask) v)."""
+    D = q.shape[-1]
+    scale = D ** -0.5 if scale is None else scale
+    s = torch.matmul(q, k.transpose(-1, -2)) * scale
+    if causal:
+        S = q.shape[-2]
+        mask = torch.ones(S, S, dtype=torch.bool).tril()
+        s = s.masked_fill(~mask, float("-inf"))
+    return torch.matmul(torch.softmax(s, dim=-1), v)
+
+
+def attention_fused_qkv(qkv, H, causal):
+    """qkv: [B, S, 3*H*D] (q | k | v on the last dim) -> [B, S, H*D]."""
+    B, S, three = qkv.shape
+    HD = three // 3
+    D = HD // H
+    q, k, v = (t.reshape(B, S, H, D).transpose(1, 2) for t in qkv.split(HD, dim=-1))
+    o = attention(q, k, v, causal)
+    return o.transpose(1, 2).reshape(B, S, HD)
+
+
+def cross_entropy_mean(logits, target, ignore_index=-100):
+    """Mean negative log-likelihood over rows whose target is not ignore_index."""
+    lse = torch.logsumexp(logits, dim=-1)
+    valid = target != ignore_index
+    safe = torch.where(valid, target, torch.zeros_like(target))
+    picked = logits.gather(-1, safe.unsqueeze(-1)).squeeze(-1)
+    per_row = torch.where(valid, lse - picked, torch.zeros_like(lse))
+    return per_row.sum() / valid.sum().clamp(min=1)
+
+
+def embedding(ids, wte, wpe=None):
+    y = wte[ids]
+    if wpe is not None:
+        S = ids.shape[-1]
+        y = y + wpe[:S]
+    return y

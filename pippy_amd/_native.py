@@ -1,0 +1,374 @@
+"""ctypes binding of ``libpippy_amd.so`` (the C ABI declared in ``include/pippy_amd.h``).
+
+There is no CPU fallback: if the library is missing, every kernel call raises.  Tensors are passed
+as raw device pointers and launches go to torch's current HIP stream, so they order with torch
+work on that stream.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from ._build import LIB_PATH
+
+PP_OK = 0
+PP_BF16, PP_F32 = 0, 1
+
+# enum pp_gemm_epilogue
+EPI_NONE, EPI_BIAS, EPI_BIAS_GELU_ERF, EPI_BIAS_GELU_TANH, EPI_BIAS_RESIDUAL = 0, 1, 2, 3, 4
+EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7, 8, 9
+
+# enum pp_op_kind
+(OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
+ OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
+ OP_FILL) = range(1, 16)
+
+PP_COPY_MAX_SEGS = 64
+
+# every symbol include/pippy_amd.h declares
+EXPORTED_SYMBOLS = (
+    "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
+    "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
+    "pp_gemm_bf16", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
+    "pp_ce_loss", "pp_run_ops",
+)
+
+
+class CopySeg(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("n_rows", C.c_int64),
+                ("row_bytes", C.c_int64), ("src_stride", C.c_int64), ("dst_stride", C.c_int64)]
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p),
+                ("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64),
+                ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
+                ("a_trans", C.c_int32), ("b_trans", C.c_int32),
+                ("epilogue", C.c_int32), ("c_dtype", C.c_int32),
+                ("bias", C.c_void_p), ("aux_in", C.c_void_p), ("aux_out", C.c_void_p),
+                ("ld_aux", C.c_int64), ("beta", C.c_int32), ("reserved", C.c_int32)]
+
+
+class AttnDesc(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+                ("o", C.c_void_p), ("lse", C.c_void_p), ("d_o", C.c_void_p),
+                ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+                ("delta", C.c_void_p),
+                ("B", C.c_int64), ("S", C.c_int64), ("H", C.c_int64), ("D", C.c_int64),
+                ("stride_b", C.c_int64), ("stride_s", C.c_int64),
+                ("scale", C.c_float), ("causal", C.c_int32)]
+
+
+class Op(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("flags", C.c_int32), ("p", C.c_void_p * 10),
+                ("i", C.c_int64 * 12), ("f", C.c_float * 2), ("j", C.c_int32 * 6)]
+
+
+_lib: Optional[C.CDLL] = None
+
+
+class NativeLibraryError(RuntimeError):
+    pass
+
+
+def lib() -> C.CDLL:
+    """Loads the kernel library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise NativeLibraryError(
+            f"{LIB_PATH} is missing: build it with `python -m pippy_amd._build` "
+            "(there is no CPU fallback for the pipeline-stage kernels)")
+    L = C.CDLL(str(LIB_PATH))
+    L.pp_last_error.restype = C.c_char_p
+    L.pp_abi_version.restype = C.c_int
+    vp, i64, i32, f32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
+    sigs = {
+        "pp_copy_rows": [C.POINTER(CopySeg), i32, vp],
+        "pp_split_copy": [vp, C.POINTER(vp), i32, i64, i64, i64, vp],
+        "pp_merge_copy": [vp, C.POINTER(vp), C.POINTER(i64), i32, i64, i64, vp],
+        "pp_strided_copy_nd": [vp, vp, i32, C.POINTER(i64), C.POINTER(i64), i32, vp],
+        "pp_grad_accum_f32_bf16": [vp, vp, i64, i32, vp],
+        "pp_grad_accum_f32_f32": [vp, vp, i64, i32, vp],
+        "pp_fill_bytes": [vp, i32, i64, vp],
+        "pp_gemm_bf16": [C.POINTER(GemmDesc), vp],
+        "pp_gemm_f32": [C.POINTER(GemmDesc), vp],
+        "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
+        "pp_layernorm_fwd": [vp, vp, vp, vp, vp, vp, i64, i64, f32, vp],
+        "pp_layernorm_bwd_input": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp],
+        "pp_layernorm_bwd_weight": [vp, vp, vp, vp, vp, vp, i32, vp, i64, i64, vp],
+        "pp_attn_fwd": [C.POINTER(AttnDesc), vp],
+        "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
+        "pp_embed_fwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
+        "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
+        "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
+        "pp_run_ops": [C.POINTER(Op), i32, vp],
+    }
+    for name, argtypes in sigs.items():
+        fn = getattr(L, name)
+        fn.argtypes = argtypes
+        fn.restype = C.c_int
+    _lib = L
+    return L
+
+
+def check(rc: int, what: str) -> None:
+    if rc != PP_OK:
+        msg = lib().pp_last_error()
+        raise RuntimeError(f"{what} failed with code {rc}: {msg.decode() if msg else ''}")
+
+
+def current_stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def require_cuda(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "pippy_amd kernels take device tensors; got a tensor on "
+                f"{t.device} (there is no CPU path)")
+
+
+# ---- microbatch copies ----------------------------------------------------------------------
+def copy_rows(segs: Sequence[tuple]) -> None:
+    """segs: (src_ptr, dst_ptr, n_rows, row_bytes, src_stride, dst_stride) tuples."""
+    if not segs:
+        return
+    arr = (CopySeg * len(segs))()
+    for a, s in zip(arr, segs):
+        a.src, a.dst, a.n_rows, a.row_bytes, a.src_stride, a.dst_stride = s
+    for i0 in range(0, len(segs), PP_COPY_MAX_SEGS):
+        n = min(PP_COPY_MAX_SEGS, len(segs) - i0)
+        sub = C.cast(C.byref(arr, i0 * C.sizeof(CopySeg)), C.POINTER(CopySeg))
+        check(lib().pp_copy_rows(sub, n, current_stream()), "pp_copy_rows")
+
+
+def split_copy(src: torch.Tensor, dsts: Sequence[torch.Tensor], dim: int) -> None:
+    require_cuda(src, *dsts)
+    assert src.is_contiguous() and all(d.is_contiguous() for d in dsts)
+    outer = 1
+    for s in src.shape[:dim]:
+        outer *= s
+    inner = src.element_size()
+    for s in src.shape[dim + 1:]:
+        inner *= s
+    arr = (C.c_void_p * len(dsts))(*[d.data_ptr() for d in dsts])
+    check(lib().pp_split_copy(src.data_ptr(), arr, len(dsts), outer, src.shape[dim], inner,
+                              current_stream()), "pp_split_copy")
+
+
+def merge_copy(dst: torch.Tensor, srcs: Sequence[torch.Tensor], dim: int) -> None:
+    require_cuda(dst, *srcs)
+    assert dst.is_contiguous() and all(s.is_contiguous() for s in srcs)
+    outer = 1
+    for s in dst.shape[:dim]:
+        outer *= s
+    inner = dst.element_size()
+    for s in dst.shape[dim + 1:]:
+        inner *= s
+    n = len(srcs)
+    ptrs = (C.c_void_p * n)(*[s.data_ptr() for s in srcs])
+    dims = (C.c_int64 * n)(*[s.shape[dim] for s in srcs])
+    check(lib().pp_merge_copy(dst.data_ptr(), ptrs, dims, n, outer, inner, current_stream()),
+          "pp_merge_copy")
+
+
+def strided_copy_nd(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """dst (contiguous) <- src (any strides), same shape and dtype."""
+    require_cuda(dst, src)
+    assert dst.is_contiguous() and dst.shape == src.shape and dst.dtype == src.dtype
+    nd = src.dim()
+    sizes = (C.c_int64 * max(nd, 1))(*src.shape)
+    strides = (C.c_int64 * max(nd, 1))(*src.stride())
+    check(lib().pp_strided_copy_nd(dst.data_ptr(), src.data_ptr(), nd, sizes, strides,
+                                   src.element_size(), current_stream()), "pp_strided_copy_nd")
+
+
+# ---- gradient accumulation ------------------------------------------------------------------
+def grad_accum(acc: torch.Tensor, g: torch.Tensor, init: bool = False) -> None:
+    require_cuda(acc, g)
+    assert acc.dtype == torch.float32 and acc.is_contiguous() and g.is_contiguous()
+    assert acc.numel() == g.numel()
+    if g.dtype == torch.bfloat16:
+        check(lib().pp_grad_accum_f32_bf16(acc.data_ptr(), g.data_ptr(), acc.numel(), int(init),
+                                           current_stream()), "pp_grad_accum_f32_bf16")
+    elif g.dtype == torch.float32:
+        check(lib().pp_grad_accum_f32_f32(acc.data_ptr(), g.data_ptr(), acc.numel(), int(init),
+                                          current_stream()), "pp_grad_accum_f32_f32")
+    else:
+        raise TypeError(f"grad_accum: unsupported gradient dtype {g.dtype}")
+
+
+def fill_bytes(t: torch.Tensor, value: int = 0) -> None:
+    require_cuda(t)
+    assert t.is_contiguous()
+    check(lib().pp_fill_bytes(t.data_ptr(), value, t.numel() * t.element_size(),
+                              current_stream()), "pp_fill_bytes")
+
+
+# ---- GEMM -------------------------------------------------------------------------------------
+def gemm_desc(A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, *, a_trans: bool = False,
+              b_trans: bool = False, epilogue: int = EPI_NONE, bias: Optional[torch.Tensor] = None,
+              aux_in: Optional[torch.Tensor] = None, aux_out: Optional[torch.Tensor] = None,
+              beta: int = 0) -> GemmDesc:
+    """A: [M,K] (or [K,M] if a_trans); B: [N,K] (or [K,N] if b_trans); Cm: [M,N].
+    Row-major 2-d tensors whose last stride is 1 (a row stride larger than the row is fine)."""
+    require_cuda(A, B, Cm, bias, aux_in, aux_out)
+    for t in (A, B, Cm, aux_in, aux_out):
+        if t is not None:
+            assert t.dim() == 2 and t.stride(1) == 1, "GEMM operands are row-major 2-d"
+    M, N = Cm.shape
+    K = A.shape[0] if a_trans else A.shape[1]
+    assert (A.shape[1] if a_trans else A.shape[0]) == M, "A does not match C"
+    assert (B.shape[1] if b_trans else B.shape[0]) == N, "B does not match C"
+    assert (B.shape[0] if b_trans else B.shape[1]) == K, "A and B disagree on K"
+    d = GemmDesc()
+    d.A, d.B, d.C = A.data_ptr(), B.data_ptr(), Cm.data_ptr()
+    d.M, d.N, d.K = M, N, K
+    d.lda, d.ldb, d.ldc = A.stride(0), B.stride(0), Cm.stride(0)
+    d.a_trans, d.b_trans = int(a_trans), int(b_trans)
+    d.epilogue = epilogue
+    d.c_dtype = PP_F32 if Cm.dtype == torch.float32 else PP_BF16
+    d.bias = ptr(bias)
+    d.aux_in = ptr(aux_in)
+    d.aux_out = ptr(aux_out)
+    ld_aux = 0
+    for t in (aux_in, aux_out):
+        if t is not None:
+            assert t.shape == Cm.shape
+            assert ld_aux in (0, t.stride(0)), "aux_in and aux_out share one leading dimension"
+            ld_aux = t.stride(0)
+    d.ld_aux = ld_aux
+    d.beta = beta
+    return d
+
+
+def gemm_bf16(A, B, Cm, **kw) -> None:
+    assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16
+    d = gemm_desc(A, B, Cm, **kw)
+    check(lib().pp_gemm_bf16(C.byref(d), current_stream()), "pp_gemm_bf16")
+
+
+def gemm_f32(A, B, Cm, **kw) -> None:
+    assert A.dtype == torch.float32 and B.dtype == torch.float32 and Cm.dtype == torch.float32
+    d = gemm_desc(A, B, Cm, **kw)
+    check(lib().pp_gemm_f32(C.byref(d), current_stream()), "pp_gemm_f32")
+
+
+def colsum(dY: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor) -> None:
+    require_cuda(dY, out, workspace)
+    M, N = dY.shape
+    assert dY.stride(1) == 1 and out.numel() == N and workspace.dtype == torch.float32
+    assert workspace.numel() >= ((M + 127) // 128) * N
+    check(lib().pp_colsum_bf16(dY.data_ptr(), M, N, dY.stride(0), out.data_ptr(),
+                               PP_F32 if out.dtype == torch.float32 else PP_BF16,
+                               workspace.data_ptr(), current_stream()), "pp_colsum_bf16")
+
+
+# ---- LayerNorm --------------------------------------------------------------------------------
+def layernorm_fwd(x, gamma, beta, y, mean, rstd, eps: float) -> None:
+    require_cuda(x, gamma, beta, y, mean, rstd)
+    rows, Cc = x.shape
+    check(lib().pp_layernorm_fwd(x.data_ptr(), gamma.data_ptr(), ptr(beta), y.data_ptr(),
+                                 mean.data_ptr(), rstd.data_ptr(), rows, Cc, eps,
+                                 current_stream()), "pp_layernorm_fwd")
+
+
+def layernorm_bwd_input(dy, x, gamma, mean, rstd, dres, dx) -> None:
+    require_cuda(dy, x, gamma, mean, rstd, dres, dx)
+    rows, Cc = x.shape
+    check(lib().pp_layernorm_bwd_input(dy.data_ptr(), x.data_ptr(), gamma.data_ptr(),
+                                       mean.data_ptr(), rstd.data_ptr(), ptr(dres), dx.data_ptr(),
+                                       rows, Cc, current_stream()), "pp_layernorm_bwd_input")
+
+
+def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:
+    require_cuda(dy, x, mean, rstd, dgamma, dbeta, workspace)
+    rows, Cc = x.shape
+    assert workspace.numel() >= 2 * ((rows + 127) // 128) * Cc
+    check(lib().pp_layernorm_bwd_weight(dy.data_ptr(), x.data_ptr(), mean.data_ptr(),
+                                        rstd.data_ptr(), dgamma.data_ptr(), ptr(dbeta),
+                                        PP_F32 if dgamma.dtype == torch.float32 else PP_BF16,
+                                        workspace.data_ptr(), rows, Cc, current_stream()),
+          "pp_layernorm_bwd_weight")
+
+
+# ---- attention --------------------------------------------------------------------------------
+def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, causal: bool,
+              scale: Optional[float] = None, d_o: Optional[torch.Tensor] = None,
+              dqkv: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None) -> AttnDesc:
+    """qkv: [B, S, 3*H*D] fused projection output (q | k | v along the last dim)."""
+    require_cuda(qkv, o, lse, d_o, dqkv, delta)
+    B, S, three_hd = qkv.shape
+    HD = three_hd // 3
+    D = HD // H
+    assert qkv.stride(2) == 1 and o.is_contiguous() and o.shape == (B, S, HD)
+    es = qkv.element_size()
+    d = AttnDesc()
+    base = qkv.data_ptr()
+    d.q, d.k, d.v = base, base + HD * es, base + 2 * HD * es
+    d.o, d.lse = o.data_ptr(), lse.data_ptr()
+    d.B, d.S, d.H, d.D = B, S, H, D
+    d.stride_b, d.stride_s = qkv.stride(0), qkv.stride(1)
+    d.scale = scale if scale is not None else D ** -0.5
+    d.causal = int(causal)
+    if d_o is not None:
+        assert dqkv is not None and delta is not None
+        assert dqkv.shape == qkv.shape and dqkv.stride() == qkv.stride() and d_o.is_contiguous()
+        gb = dqkv.data_ptr()
+        d.d_o = d_o.data_ptr()
+        d.dq, d.dk, d.dv = gb, gb + HD * es, gb + 2 * HD * es
+        d.delta = delta.data_ptr()
+    return d
+
+
+def attn_fwd(qkv, o, lse, H, causal, scale=None) -> None:
+    d = attn_desc(qkv, o, lse, H, causal, scale)
+    check(lib().pp_attn_fwd(C.byref(d), current_stream()), "pp_attn_fwd")
+
+
+def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None) -> None:
+    d = attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta)
+    check(lib().pp_attn_bwd(C.byref(d), current_stream()), "pp_attn_bwd")
+
+
+# ---- embedding / loss -------------------------------------------------------------------------
+def embed_fwd(ids, wte, wpe, y, seq: int) -> None:
+    require_cuda(ids, wte, wpe, y)
+    assert ids.dtype == torch.int64 and ids.is_contiguous() and y.is_contiguous()
+    vocab, Cc = wte.shape
+    check(lib().pp_embed_fwd(ids.data_ptr(), wte.data_ptr(), ptr(wpe), y.data_ptr(), ids.numel(),
+                             seq, Cc, vocab, current_stream()), "pp_embed_fwd")
+
+
+def embed_bwd(ids, dy, d_wte, d_wpe, seq: int) -> None:
+    require_cuda(ids, dy, d_wte, d_wpe)
+    vocab, Cc = d_wte.shape
+    check(lib().pp_embed_bwd(ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), ptr(d_wpe),
+                             ids.numel(), seq, Cc, vocab, current_stream()), "pp_embed_bwd")
+
+
+def ce_loss(logits, target, loss, dlogits, workspace, V: int, ignore_index: int = -100) -> None:
+    """logits: [rows, ld] with the first V columns valid (ld = logits.stride(0))."""
+    require_cuda(logits, target, loss, dlogits, workspace)
+    rows = logits.shape[0]
+    assert logits.stride(1) == 1 and target.numel() == rows and workspace.numel() >= rows + 2
+    if dlogits is not None:
+        assert dlogits.stride() == logits.stride()
+    check(lib().pp_ce_loss(logits.data_ptr(), target.data_ptr(), loss.data_ptr(), ptr(dlogits),
+                           workspace.data_ptr(), rows, V, logits.stride(0), ignore_index,
+                           PP_F32 if logits.dtype == torch.float32 else PP_BF16,
+                           current_stream()), "pp_ce_loss")
+
+
+def run_ops(ops, n: int) -> None:
+    check(lib().pp_run_ops(ops, n, current_stream()), "pp_run_ops")

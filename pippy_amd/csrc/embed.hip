@@ -1,0 +1,106 @@
+// Token + position embedding lookup and its gradient (HBM-bound gathers / scatters).
+#include "common.h"
+
+namespace pp {
+
+// One wave per token; each lane moves 16-byte chunks of the row.
+__global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restrict__ ids,
+                                                        const uint16_t* __restrict__ wte,
+                                                        const uint16_t* __restrict__ wpe,
+                                                        uint16_t* __restrict__ y, int64_t n_tok,
+                                                        int64_t seq, int C, int64_t vocab) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tok) return;
+    int64_t id = ids[t];
+    // out-of-range ids read row 0 rather than faulting; callers validate ids on the host side
+    if (id < 0 || id >= vocab) id = 0;
+    const uint4* src = reinterpret_cast<const uint4*>(wte + id * C);
+    const uint4* pos = wpe ? reinterpret_cast<const uint4*>(wpe + (t % seq) * C) : nullptr;
+    uint4* dst = reinterpret_cast<uint4*>(y + t * C);
+    for (int c = lane; c < (C >> 3); c += 64) {
+        uint4 a = src[c];
+        if (pos) {
+            const uint4 b = pos[c];
+            a.x = pack_bf16(bf16lo(a.x) + bf16lo(b.x), bf16hi(a.x) + bf16hi(b.x));
+            a.y = pack_bf16(bf16lo(a.y) + bf16lo(b.y), bf16hi(a.y) + bf16hi(b.y));
+            a.z = pack_bf16(bf16lo(a.z) + bf16lo(b.z), bf16hi(a.z) + bf16hi(b.z));
+            a.w = pack_bf16(bf16lo(a.w) + bf16lo(b.w), bf16hi(a.w) + bf16hi(b.w));
+        }
+        dst[c] = a;
+    }
+}
+
+// d_wte[ids[t], :] += dy[t, :] with fp32 atomics (rows repeat when a token id repeats).
+__global__ __launch_bounds__(256) void embed_bwd_wte_kernel(const int64_t* __restrict__ ids,
+                                                            const uint16_t* __restrict__ dy,
+                                                            float* __restrict__ d_wte, int64_t n_tok,
+                                                            int C, int64_t vocab) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tok) return;
+    const int64_t id = ids[t];
+    if (id < 0 || id >= vocab) return;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(dy + t * C);
+    float* dst = d_wte + id * C;
+    for (int c = lane; c < (C >> 1); c += 64) {
+        const uint32_t w = src[c];
+        unsafeAtomicAdd(dst + 2 * c, bf16lo(w));
+        unsafeAtomicAdd(dst + 2 * c + 1, bf16hi(w));
+    }
+}
+
+// d_wpe[p, :] += sum_b dy[b*seq + p, :]; each (p, column) has one owner, summed in batch order.
+__global__ __launch_bounds__(256) void embed_bwd_wpe_kernel(const uint16_t* __restrict__ dy,
+                                                            float* __restrict__ d_wpe, int64_t n_tok,
+                                                            int64_t seq, int C) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over seq * C/2
+    const int half_c = C >> 1;
+    if (idx >= seq * half_c) return;
+    const int64_t p = idx / half_c;
+    const int c = (int)(idx - p * half_c);
+    float s0 = 0.f, s1 = 0.f;
+    for (int64_t t = p; t < n_tok; t += seq) {
+        const uint32_t w = reinterpret_cast<const uint32_t*>(dy + t * C)[c];
+        s0 += bf16lo(w);
+        s1 += bf16hi(w);
+    }
+    float* dst = d_wpe + p * C + 2 * c;
+    dst[0] += s0;
+    dst[1] += s1;
+}
+
+}  // namespace pp
+
+using namespace pp;
+
+extern "C" int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, void* y,
+                            int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream) {
+    if (n_tok < 0 || seq <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_fwd: bad shape");
+    if (C % 8) return fail(PP_ERR_UNSUPPORTED, "pp_embed_fwd: C %% 8 != 0");
+    if (n_tok == 0) return PP_OK;
+    if (!ids || !wte || !y) return fail(PP_ERR_INVALID, "pp_embed_fwd: null pointer");
+    if (!aligned(wte, 16) || !aligned(wpe, 16) || !aligned(y, 16))
+        return fail(PP_ERR_INVALID, "pp_embed_fwd: pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(embed_fwd_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), ids, (const uint16_t*)wte, (const uint16_t*)wpe,
+                       (uint16_t*)y, n_tok, seq, (int)C, vocab);
+    return check_launch("embed_fwd_kernel");
+}
+
+extern "C" int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe,
+                            int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream) {
+    if (n_tok < 0 || seq <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_bwd: bad shape");
+    if (C % 2) return fail(PP_ERR_UNSUPPORTED, "pp_embed_bwd: C %% 2 != 0");
+    if (n_tok == 0) return PP_OK;
+    if (!ids || !dy || !d_wte) return fail(PP_ERR_INVALID, "pp_embed_bwd: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(embed_bwd_wte_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0, st, ids,
+                       (const uint16_t*)dy, d_wte, n_tok, (int)C, vocab);
+    if (d_wpe) {
+        const int64_t work = seq * (C / 2);
+        hipLaunchKernelGGL(embed_bwd_wpe_kernel, dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st,
+                           (const uint16_t*)dy, d_wpe, n_tok, seq, (int)C);
+    }
+    return check_launch("embed_bwd");
+}

@@ -1,0 +1,328 @@
+// bf16 GEMM for gfx950 on v_mfma_f32_32x32x16_bf16 with LDS-staged tiles and fused epilogues.
+//
+//   C[M,N] = epilogue( sum_k A(m,k) * B(n,k) ),  fp32 accumulation.
+//
+// Tiling: a work-group of 256 lanes (4 waves, 2x2) owns a BM x BN output tile and walks K in steps
+// of 64.  Operand tiles live in LDS as [row][64 k] bf16 (128 B per row) with the 16-byte chunk
+// index XOR-swizzled by the row so that both the staging writes and the ds_read_b128 fragment
+// reads spread over all banks.  An operand whose memory layout is [K][rows] (the weight in the
+// input-gradient GEMM, both operands in the weight-gradient GEMM) is transposed on the way in:
+// each lane loads 4 k-rows x 8 rows and writes 8 x 8-byte k-runs.  Global loads for tile t+1 are
+// issued before the MFMAs of tile t (register double buffering, two LDS buffers, one barrier per
+// K step).
+//
+// The MFMA is issued with the B fragment as its first operand, so a lane ends up holding, for one
+// output row m, groups of 4 consecutive columns n: stores and epilogue reads are 8-byte vectors.
+#include "tile.h"
+#include <math.h>
+
+namespace pp {
+
+struct GemmArgs {
+    const uint16_t* A;
+    const uint16_t* B;
+    void* C;
+    int64_t M, N, K, lda, ldb, ldc;
+    const uint16_t* bias;
+    const uint16_t* aux_in;
+    uint16_t* aux_out;
+    int64_t ld_aux;
+    int beta;
+    uint32_t tiles_m, tiles_n, n_blocks;
+};
+
+// ---- epilogue math --------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_erf(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(u));
+}
+__device__ __forceinline__ float dgelu_erf(float x) {
+    const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
+    const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
+    return cdf + x * pdf;
+}
+__device__ __forceinline__ float dgelu_tanh(float x) {
+    const float k = 0.79788456080286535588f, c = 0.044715f;
+    const float u = k * (x + c * x * x * x);
+    const float t = tanhf(u);
+    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * k * (1.0f + 3.0f * c * x * x);
+}
+
+// Applies the epilogue to 4 consecutive columns n0..n0+3 of row m and stores them.
+template <int EPI, bool CF32>
+__device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t n0, float v0, float v1,
+                                          float v2, float v3, bool vec_ok) {
+    if (m >= g.M || n0 >= g.N) return;
+    float v[4] = {v0, v1, v2, v3};
+    const int nv = (g.N - n0 >= 4) ? 4 : (int)(g.N - n0);
+    const bool full = vec_ok && nv == 4;
+
+    if (EPI == PP_EPI_BIAS || EPI == PP_EPI_BIAS_GELU_ERF || EPI == PP_EPI_BIAS_GELU_TANH ||
+        EPI == PP_EPI_BIAS_RESIDUAL || EPI == PP_EPI_BIAS_RELU) {
+        if (g.bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nv) v[e] += bf16_to_f32(g.bias[n0 + e]);
+        }
+    }
+    if (EPI == PP_EPI_BIAS_RESIDUAL || EPI == PP_EPI_DGELU_ERF || EPI == PP_EPI_DGELU_TANH ||
+        EPI == PP_EPI_DRELU) {
+        float a[4] = {0.f, 0.f, 0.f, 0.f};
+        const uint16_t* ap = g.aux_in + m * g.ld_aux + n0;
+        if (full) {
+            const uint2 w = *reinterpret_cast<const uint2*>(ap);
+            a[0] = bf16lo(w.x); a[1] = bf16hi(w.x); a[2] = bf16lo(w.y); a[3] = bf16hi(w.y);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nv) a[e] = bf16_to_f32(ap[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (EPI == PP_EPI_BIAS_RESIDUAL) v[e] += a[e];
+            if (EPI == PP_EPI_DGELU_ERF) v[e] *= dgelu_erf(a[e]);
+            if (EPI == PP_EPI_DGELU_TANH) v[e] *= dgelu_tanh(a[e]);
+            if (EPI == PP_EPI_DRELU) v[e] = a[e] > 0.f ? v[e] : 0.f;
+        }
+    }
+    if (EPI == PP_EPI_BIAS_GELU_ERF || EPI == PP_EPI_BIAS_GELU_TANH) {
+        if (g.aux_out) {
+            uint16_t* op = g.aux_out + m * g.ld_aux + n0;
+            if (full) {
+                *reinterpret_cast<uint2*>(op) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nv) op[e] = f32_to_bf16(v[e]);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            v[e] = (EPI == PP_EPI_BIAS_GELU_ERF) ? gelu_erf(v[e]) : gelu_tanh(v[e]);
+    }
+    if (EPI == PP_EPI_BIAS_RELU) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+    }
+
+    if (CF32) {
+        float* cp = static_cast<float*>(g.C) + m * g.ldc + n0;
+        if (EPI == PP_EPI_ACCUM_F32 && g.beta) {
+            if (full) {
+                const float4 old = *reinterpret_cast<const float4*>(cp);
+                *reinterpret_cast<float4*>(cp) =
+                    make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nv) cp[e] += v[e];
+            }
+        } else {
+            if (full) {
+                *reinterpret_cast<float4*>(cp) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nv) cp[e] = v[e];
+            }
+        }
+    } else {
+        uint16_t* cp = static_cast<uint16_t*>(g.C) + m * g.ldc + n0;
+        if (full) {
+            *reinterpret_cast<uint2*>(cp) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nv) cp[e] = f32_to_bf16(v[e]);
+        }
+    }
+}
+
+// ---- the kernel -----------------------------------------------------------------------------
+template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs g) {
+    constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    constexpr int kStageElems = (BM + BN) * BK;  // one LDS buffer: A tile then B tile
+
+    // XCD-aware remap: consecutive hardware block ids round-robin over the 8 XCDs; give each XCD
+    // a contiguous range of tiles so that its private L2 sees a compact set of A/B panels.
+    uint32_t bid = blockIdx.x;
+    {
+        const uint32_t per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
+        bid = (bid & 7) * per_xcd + (bid >> 3);
+    }
+    if (bid >= g.n_blocks) return;
+    const uint32_t tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+    Stage<BM, AT> sa;
+    Stage<BN, BT> sb;
+    const int64_t nk = (g.K + BK - 1) / BK;
+
+    sa.load(g.A, g.lda, m0, g.M, 0, g.K, tid);
+    sb.load(g.B, g.ldb, n0, g.N, 0, g.K, tid);
+    sa.store(smem, tid);
+    sb.store(smem + BM * BK, tid);
+    __syncthreads();
+
+    for (int64_t kt = 0; kt < nk; ++kt) {
+        const int cur = (int)(kt & 1);
+        if (kt + 1 < nk) {
+            sa.load(g.A, g.lda, m0, g.M, (kt + 1) * BK, g.K, tid);
+            sb.load(g.B, g.ldb, n0, g.N, (kt + 1) * BK, g.K, tid);
+        }
+        const uint16_t* a_s = smem + cur * kStageElems;
+        const uint16_t* b_s = a_s + BM * BK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8_t af[TM], bf[TN];
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const int row = wm0 + t * 32 + l32;
+                af[t] = *reinterpret_cast<const bf16x8_t*>(a_s + row * BK + (((2 * ks + lh) ^ swz(row)) << 3));
+            }
+#pragma unroll
+            for (int t = 0; t < TN; ++t) {
+                const int row = wn0 + t * 32 + l32;
+                bf[t] = *reinterpret_cast<const bf16x8_t*>(b_s + row * BK + (((2 * ks + lh) ^ swz(row)) << 3));
+            }
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[a], af[b], acc[a][b], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            sa.store(smem + (cur ^ 1) * kStageElems, tid);
+            sb.store(smem + (cur ^ 1) * kStageElems + BM * BK, tid);
+        }
+        __syncthreads();
+    }
+
+    // D[i][j]: i = n within the 32x32 tile = 8*(v/4) + 4*lh + v%4, j = m within the tile = l32.
+    const bool vec_ok = CF32 ? ((g.ldc & 3) == 0 && aligned(g.C, 16))
+                             : ((g.ldc & 3) == 0 && aligned(g.C, 8) && (g.ld_aux & 3) == 0 &&
+                                aligned(g.aux_in, 8) && aligned(g.aux_out, 8));
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b) {
+            const int64_t m = m0 + wm0 + b * 32 + l32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t n = n0 + wn0 + a * 32 + 8 * q + 4 * lh;
+                epilogue4<EPI, CF32>(g, m, n, acc[a][b][4 * q + 0], acc[a][b][4 * q + 1],
+                                     acc[a][b][4 * q + 2], acc[a][b][4 * q + 3], vec_ok);
+            }
+        }
+}
+
+template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
+static int launch_gemm(const GemmArgs& g0, hipStream_t st) {
+    GemmArgs g = g0;
+    g.tiles_m = (uint32_t)((g.M + BM - 1) / BM);
+    g.tiles_n = (uint32_t)((g.N + BN - 1) / BN);
+    const uint64_t nb = (uint64_t)g.tiles_m * g.tiles_n;
+    if (nb > 0x7fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: too many tiles");
+    g.n_blocks = (uint32_t)nb;
+    const uint32_t grid = (uint32_t)((nb + 7) / 8 * 8);
+    const size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
+    static const hipError_t attr_rc = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr_rc != hipSuccess)
+        return fail(PP_ERR_LAUNCH, "pp_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds,
+                    hipGetErrorString(attr_rc));
+    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+                       lds, st, g);
+    return check_launch("gemm_bf16_kernel");
+}
+
+template <int EPI, bool CF32>
+static int dispatch_layout(const GemmArgs& g, int at, int bt, hipStream_t st) {
+    if (!at && !bt) return launch_gemm<128, 128, false, false, EPI, CF32>(g, st);
+    if (!at && bt) return launch_gemm<128, 128, false, true, EPI, CF32>(g, st);
+    if (at && !bt) return launch_gemm<128, 128, true, false, EPI, CF32>(g, st);
+    return launch_gemm<128, 128, true, true, EPI, CF32>(g, st);
+}
+
+}  // namespace pp
+
+using namespace pp;
+
+extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
+    if (!d) return fail(PP_ERR_INVALID, "pp_gemm_bf16: null descriptor");
+    if (d->M < 0 || d->N < 0 || d->K < 0) return fail(PP_ERR_INVALID, "pp_gemm_bf16: negative size");
+    if (d->M == 0 || d->N == 0) return PP_OK;
+    if (!d->A || !d->B || !d->C) return fail(PP_ERR_INVALID, "pp_gemm_bf16: null operand");
+    if (!aligned(d->A, 16) || !aligned(d->B, 16))
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: A and B must be 16-byte aligned");
+    if ((d->K & 7) || (d->lda & 7) || (d->ldb & 7))
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: K, lda, ldb must be multiples of 8 (K=%lld lda=%lld ldb=%lld)",
+                    (long long)d->K, (long long)d->lda, (long long)d->ldb);
+    if (d->a_trans && (d->M & 7)) return fail(PP_ERR_INVALID, "pp_gemm_bf16: transposed A needs M %% 8 == 0");
+    if (d->b_trans && (d->N & 7)) return fail(PP_ERR_INVALID, "pp_gemm_bf16: transposed B needs N %% 8 == 0");
+    if (d->lda < (d->a_trans ? d->M : d->K) || d->ldb < (d->b_trans ? d->N : d->K) || d->ldc < d->N)
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: leading dimension too small");
+    const int epi = d->epilogue;
+    const bool needs_aux = epi == PP_EPI_BIAS_RESIDUAL || epi == PP_EPI_DGELU_ERF ||
+                           epi == PP_EPI_DGELU_TANH || epi == PP_EPI_DRELU;
+    if (needs_aux && (!d->aux_in || d->ld_aux < d->N))
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: epilogue %d needs aux_in with ld_aux >= N", epi);
+    if (d->aux_out && d->ld_aux < d->N) return fail(PP_ERR_INVALID, "pp_gemm_bf16: ld_aux < N");
+    const bool cf32 = d->c_dtype == PP_F32;
+    if (epi == PP_EPI_ACCUM_F32 && !cf32)
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: PP_EPI_ACCUM_F32 needs an fp32 C");
+
+    GemmArgs g;
+    g.A = static_cast<const uint16_t*>(d->A);
+    g.B = static_cast<const uint16_t*>(d->B);
+    g.C = d->C;
+    g.M = d->M; g.N = d->N; g.K = d->K;
+    g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc;
+    g.bias = static_cast<const uint16_t*>(d->bias);
+    g.aux_in = static_cast<const uint16_t*>(d->aux_in);
+    g.aux_out = static_cast<uint16_t*>(d->aux_out);
+    g.ld_aux = d->ld_aux;
+    g.beta = d->beta;
+    g.tiles_m = g.tiles_n = g.n_blocks = 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int at = d->a_trans ? 1 : 0, bt = d->b_trans ? 1 : 0;
+
+    if (cf32) {
+        switch (epi) {
+            case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, true>(g, at, bt, st);
+            case PP_EPI_ACCUM_F32: return dispatch_layout<PP_EPI_ACCUM_F32, true>(g, at, bt, st);
+            default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d with fp32 C", epi);
+        }
+    }
+    switch (epi) {
+        case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, false>(g, at, bt, st);
+        case PP_EPI_BIAS: return dispatch_layout<PP_EPI_BIAS, false>(g, at, bt, st);
+        case PP_EPI_BIAS_GELU_ERF: return dispatch_layout<PP_EPI_BIAS_GELU_ERF, false>(g, at, bt, st);
+        case PP_EPI_BIAS_GELU_TANH: return dispatch_layout<PP_EPI_BIAS_GELU_TANH, false>(g, at, bt, st);
+        case PP_EPI_BIAS_RESIDUAL: return dispatch_layout<PP_EPI_BIAS_RESIDUAL, false>(g, at, bt, st);
+        case PP_EPI_DGELU_ERF: return dispatch_layout<PP_EPI_DGELU_ERF, false>(g, at, bt, st);
+        case PP_EPI_DGELU_TANH: return dispatch_layout<PP_EPI_DGELU_TANH, false>(g, at, bt, st);
+        case PP_EPI_BIAS_RELU: return dispatch_layout<PP_EPI_BIAS_RELU, false>(g, at, bt, st);
+        case PP_EPI_DRELU: return dispatch_layout<PP_EPI_DRELU, false>(g, at, bt, st);
+        default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d", epi);
+    }
+}

@@ -1,0 +1,197 @@
+// Cross-entropy (mean over non-ignored rows) fused with its gradient w.r.t. the logits.
+// HBM-bound: each logits row is read from memory once and kept in registers across the max,
+// sum-of-exponentials and gradient passes; the gradient row is written once.
+#include "common.h"
+#include <math.h>
+
+namespace pp {
+
+// ws[rows] = number of valid targets, ws[rows + 1] = 1 / max(count, 1)
+__global__ __launch_bounds__(256) void ce_count_kernel(const int64_t* __restrict__ target, int64_t rows,
+                                                       int64_t V, int64_t ignore_index,
+                                                       float* __restrict__ ws) {
+    __shared__ int part[4];
+    int c = 0;
+    for (int64_t r = threadIdx.x; r < rows; r += 256) {
+        const int64_t t = target[r];
+        c += (t != ignore_index && t >= 0 && t < V) ? 1 : 0;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int n = part[0] + part[1] + part[2] + part[3];
+        ws[rows] = (float)n;
+        ws[rows + 1] = 1.0f / (float)(n > 0 ? n : 1);
+    }
+}
+
+constexpr int kCeThreads = 1024;
+
+__device__ __forceinline__ float block_reduce_max(float v, float* sh) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = sh[0];
+#pragma unroll
+    for (int i = 1; i < kCeThreads / 64; ++i) r = fmaxf(r, sh[i]);
+    return r;
+}
+__device__ __forceinline__ float block_reduce_sum(float v, float* sh) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < kCeThreads / 64; ++i) r += sh[i];
+    return r;
+}
+
+// bf16 logits, one work-group per row, NC 16-byte chunks per lane held in registers.
+template <int NC>
+__global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
+    const uint16_t* __restrict__ logits, const int64_t* __restrict__ target, uint16_t* __restrict__ dlogits,
+    float* __restrict__ ws, int64_t rows, int V, int64_t ld, int64_t ignore_index) {
+    __shared__ float sh[kCeThreads / 64];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const uint16_t* xr = logits + row * ld;
+    const int nchunk_v = (V + 7) >> 3;          // chunks holding at least one valid column
+    const int nchunk_ld = (int)(ld >> 3);       // chunks to write (padding gets zeros)
+    uint4 w[NC];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+        const int c = tid + kCeThreads * i;
+        if (c < nchunk_v) {
+            w[i] = *reinterpret_cast<const uint4*>(xr + (int64_t)c * 8);
+            const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
+                                bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (c * 8 + e < V) mx = fmaxf(mx, f[e]);
+        }
+    }
+    mx = block_reduce_max(mx, sh);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+        const int c = tid + kCeThreads * i;
+        if (c < nchunk_v) {
+            const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
+                                bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (c * 8 + e < V) s += expf(f[e] - mx);
+        }
+    }
+    s = block_reduce_sum(s, sh);
+    const float lse = mx + logf(s);
+    const int64_t t = target[row];
+    const bool valid = (t != ignore_index && t >= 0 && t < V);
+    if (tid == 0) ws[row] = valid ? (lse - bf16_to_f32(xr[valid ? t : 0])) : 0.f;
+    if (!dlogits) return;
+    const float scale = valid ? ws[rows + 1] : 0.f;
+    uint16_t* dr = dlogits + row * ld;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+        const int c = tid + kCeThreads * i;
+        if (c < nchunk_ld) {
+            float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (c < nchunk_v) {
+                const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
+                                    bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int col = c * 8 + e;
+                    if (col < V) o[e] = (expf(f[e] - lse) - (col == t ? 1.0f : 0.0f)) * scale;
+                }
+            }
+            *reinterpret_cast<uint4*>(dr + (int64_t)c * 8) =
+                make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
+                           pack_bf16(o[6], o[7]));
+        }
+    }
+}
+
+// fp32 logits (small class counts): one wave per row, three passes over the row.
+__global__ __launch_bounds__(256) void ce_row_f32_kernel(const float* __restrict__ logits,
+                                                         const int64_t* __restrict__ target,
+                                                         float* __restrict__ dlogits, float* __restrict__ ws,
+                                                         int64_t rows, int V, int64_t ld,
+                                                         int64_t ignore_index) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = logits + row * ld;
+    float mx = -INFINITY;
+    for (int c = lane; c < V; c += 64) mx = fmaxf(mx, xr[c]);
+    mx = wave_max(mx);
+    float s = 0.f;
+    for (int c = lane; c < V; c += 64) s += expf(xr[c] - mx);
+    s = wave_sum(s);
+    const float lse = mx + logf(s);
+    const int64_t t = target[row];
+    const bool valid = (t != ignore_index && t >= 0 && t < V);
+    if (lane == 0) ws[row] = valid ? (lse - xr[valid ? t : 0]) : 0.f;
+    if (!dlogits) return;
+    const float scale = valid ? ws[rows + 1] : 0.f;
+    float* dr = dlogits + row * ld;
+    for (int c = lane; c < ld; c += 64)
+        dr[c] = (c < V) ? (expf(xr[c] - lse) - (c == t ? 1.0f : 0.0f)) * scale : 0.f;
+}
+
+// loss = (sum_r ws[r]) / count, summed in a fixed order
+__global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restrict__ ws, int64_t rows,
+                                                          float* __restrict__ loss) {
+    __shared__ float part[256];
+    float s = 0.f;
+    for (int64_t r = threadIdx.x; r < rows; r += 256) s += ws[r];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) loss[0] = part[0] * ws[rows + 1];
+}
+
+}  // namespace pp
+
+using namespace pp;
+
+extern "C" int pp_ce_loss(const void* logits, const int64_t* target, float* loss, void* dlogits,
+                          float* workspace, int64_t rows, int64_t V, int64_t ld, int64_t ignore_index,
+                          int logits_dtype, pp_stream stream) {
+    if (rows < 0 || V <= 0 || ld < V) return fail(PP_ERR_INVALID, "pp_ce_loss: bad shape");
+    if (!logits || !target || !loss || !workspace) return fail(PP_ERR_INVALID, "pp_ce_loss: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(256), 0, st, target, rows, V, ignore_index, workspace);
+    if (rows > 0) {
+        if (logits_dtype == PP_F32) {
+            hipLaunchKernelGGL(ce_row_f32_kernel, dim3((uint32_t)((rows + 3) / 4)), dim3(256), 0, st,
+                               (const float*)logits, target, (float*)dlogits, workspace, rows, (int)V, ld,
+                               ignore_index);
+        } else {
+            if ((ld % 8) || !aligned(logits, 16) || !aligned(dlogits, 16))
+                return fail(PP_ERR_INVALID, "pp_ce_loss: bf16 logits need ld %% 8 == 0 and 16-byte alignment");
+            const int64_t chunks = ld / 8;
+            const int nc = (int)((chunks + kCeThreads - 1) / kCeThreads);
+            const dim3 grid((uint32_t)rows), block(kCeThreads);
+#define PP_CE_LAUNCH(NC)                                                                              \
+    hipLaunchKernelGGL(ce_row_bf16_kernel<NC>, grid, block, 0, st, (const uint16_t*)logits, target,   \
+                       (uint16_t*)dlogits, workspace, rows, (int)V, ld, ignore_index)
+            if (nc <= 1) PP_CE_LAUNCH(1);
+            else if (nc <= 2) PP_CE_LAUNCH(2);
+            else if (nc <= 4) PP_CE_LAUNCH(4);
+            else if (nc <= 8) PP_CE_LAUNCH(8);
+            else return fail(PP_ERR_UNSUPPORTED, "pp_ce_loss: more than 65536 classes");
+#undef PP_CE_LAUNCH
+        }
+    }
+    hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(256), 0, st, workspace, rows, loss);
+    return check_launch("ce_loss");
+}

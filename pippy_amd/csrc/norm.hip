@@ -1,0 +1,313 @@
+// LayerNorm forward / input-gradient / weight-gradient and the bias-gradient column sum.
+// All HBM-bound: one wave owns one row and keeps it in registers (a single read of x per pass);
+// column reductions are two-stage (per-128-row partials, then an ordered final sum), so results
+// do not depend on scheduling.
+#include "common.h"
+
+namespace pp {
+
+constexpr int kRowsPerBlock = 4;  // one wave per row
+
+// ---- forward ----------------------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(256) void layernorm_fwd_kernel(const uint16_t* __restrict__ x,
+                                                            const uint16_t* __restrict__ gamma,
+                                                            const uint16_t* __restrict__ beta,
+                                                            uint16_t* __restrict__ y,
+                                                            float* __restrict__ mean_out,
+                                                            float* __restrict__ rstd_out, int64_t rows,
+                                                            int C, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nchunk = C >> 3;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * C);
+    float v[NV][8];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunk) {
+            const uint4 w = xr[c];
+            v[i][0] = bf16lo(w.x); v[i][1] = bf16hi(w.x); v[i][2] = bf16lo(w.y); v[i][3] = bf16hi(w.y);
+            v[i][4] = bf16lo(w.z); v[i][5] = bf16hi(w.z); v[i][6] = bf16lo(w.w); v[i][7] = bf16hi(w.w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += v[i][e];
+        }
+    }
+    const float mean = wave_sum(s) / (float)C;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunk) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float d = v[i][e] - mean;
+                q += d * d;
+            }
+        }
+    }
+    const float var = wave_sum(q) / (float)C;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    if (lane == 0) {
+        mean_out[row] = mean;
+        rstd_out[row] = rstd;
+    }
+    uint4* yr = reinterpret_cast<uint4*>(y + row * C);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunk) {
+            const uint4 gw = reinterpret_cast<const uint4*>(gamma)[c];
+            const float gf[8] = {bf16lo(gw.x), bf16hi(gw.x), bf16lo(gw.y), bf16hi(gw.y),
+                                 bf16lo(gw.z), bf16hi(gw.z), bf16lo(gw.w), bf16hi(gw.w)};
+            float bfv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (beta) {
+                const uint4 bw = reinterpret_cast<const uint4*>(beta)[c];
+                bfv[0] = bf16lo(bw.x); bfv[1] = bf16hi(bw.x); bfv[2] = bf16lo(bw.y); bfv[3] = bf16hi(bw.y);
+                bfv[4] = bf16lo(bw.z); bfv[5] = bf16hi(bw.z); bfv[6] = bf16lo(bw.w); bfv[7] = bf16hi(bw.w);
+            }
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (v[i][e] - mean) * rstd * gf[e] + bfv[e];
+            yr[c] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
+                               pack_bf16(o[6], o[7]));
+        }
+    }
+}
+
+// ---- input gradient ---------------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(256) void layernorm_bwd_input_kernel(
+    const uint16_t* __restrict__ dy, const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+    const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+    const uint16_t* __restrict__ dres, uint16_t* __restrict__ dx, int64_t rows, int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nchunk = C >> 3;
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * C);
+    const uint4* gr = reinterpret_cast<const uint4*>(dy + row * C);
+    float xh[NV][8], wd[NV][8];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunk) {
+            const uint4 xw = xr[c], dw = gr[c], gw = reinterpret_cast<const uint4*>(gamma)[c];
+            const float xf[8] = {bf16lo(xw.x), bf16hi(xw.x), bf16lo(xw.y), bf16hi(xw.y),
+                                 bf16lo(xw.z), bf16hi(xw.z), bf16lo(xw.w), bf16hi(xw.w)};
+            const float df[8] = {bf16lo(dw.x), bf16hi(dw.x), bf16lo(dw.y), bf16hi(dw.y),
+                                 bf16lo(dw.z), bf16hi(dw.z), bf16lo(dw.w), bf16hi(dw.w)};
+            const float gf[8] = {bf16lo(gw.x), bf16hi(gw.x), bf16lo(gw.y), bf16hi(gw.y),
+                                 bf16lo(gw.z), bf16hi(gw.z), bf16lo(gw.w), bf16hi(gw.w)};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                xh[i][e] = (xf[e] - mean) * rstd;
+                wd[i][e] = df[e] * gf[e];
+                s1 += wd[i][e] * xh[i][e];
+                s2 += wd[i][e];
+            }
+        }
+    }
+    const float c1 = wave_sum(s1) / (float)C;
+    const float c2 = wave_sum(s2) / (float)C;
+    uint4* outr = reinterpret_cast<uint4*>(dx + row * C);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        if (c < nchunk) {
+            float o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (wd[i][e] - c1 * xh[i][e] - c2) * rstd;
+            if (dres) {
+                const uint4 rw = reinterpret_cast<const uint4*>(dres + row * C)[c];
+                o[0] += bf16lo(rw.x); o[1] += bf16hi(rw.x); o[2] += bf16lo(rw.y); o[3] += bf16hi(rw.y);
+                o[4] += bf16lo(rw.z); o[5] += bf16hi(rw.z); o[6] += bf16lo(rw.w); o[7] += bf16hi(rw.w);
+            }
+            outr[c] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
+                                 pack_bf16(o[6], o[7]));
+        }
+    }
+}
+
+// ---- column reductions (dgamma / dbeta / bias gradient) ---------------------------------------
+// Stage 1: block (rb, cb) reduces rows [128*rb, 128*rb+128) of columns [256*cb, 256*cb+256).
+// Lane layout: 32 column chunks (8 columns each) x 8 row phases.
+template <bool WITH_X>
+__global__ __launch_bounds__(256) void colreduce_partial_kernel(
+    const uint16_t* __restrict__ dy, int64_t ld_dy, const uint16_t* __restrict__ x,
+    const float* __restrict__ mean_in, const float* __restrict__ rstd_in, float* __restrict__ part_g,
+    float* __restrict__ part_b, int64_t rows, int64_t C) {
+    __shared__ float red[8][32][8 + 1];
+    const int cc = threadIdx.x & 31, rp = threadIdx.x >> 5;
+    const int64_t col0 = (int64_t)blockIdx.y * 256 + cc * 8;
+    const int64_t row_begin = (int64_t)blockIdx.x * 128;
+    float sg[8] = {0, 0, 0, 0, 0, 0, 0, 0}, sb[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (col0 < C) {
+        for (int it = 0; it < 16; ++it) {
+            const int64_t r = row_begin + it * 8 + rp;
+            if (r < rows) {
+                const uint4 dw = *reinterpret_cast<const uint4*>(dy + r * ld_dy + col0);
+                const float df[8] = {bf16lo(dw.x), bf16hi(dw.x), bf16lo(dw.y), bf16hi(dw.y),
+                                     bf16lo(dw.z), bf16hi(dw.z), bf16lo(dw.w), bf16hi(dw.w)};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sb[e] += df[e];
+                if (WITH_X) {
+                    const float mean = mean_in[r], rstd = rstd_in[r];
+                    const uint4 xw = *reinterpret_cast<const uint4*>(x + r * C + col0);
+                    const float xf[8] = {bf16lo(xw.x), bf16hi(xw.x), bf16lo(xw.y), bf16hi(xw.y),
+                                         bf16lo(xw.z), bf16hi(xw.z), bf16lo(xw.w), bf16hi(xw.w)};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sg[e] += df[e] * ((xf[e] - mean) * rstd);
+                }
+            }
+        }
+    }
+    // reduce the 8 row phases in a fixed order
+#pragma unroll
+    for (int pass = 0; pass < (WITH_X ? 2 : 1); ++pass) {
+        float* s = pass == 0 ? sb : sg;
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[rp][cc][e] = s[e];
+        __syncthreads();
+        if (rp == 0 && col0 < C) {
+            float* out = (pass == 0 ? part_b : part_g) + (int64_t)blockIdx.x * C + col0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = 0.f;
+#pragma unroll
+                for (int p = 0; p < 8; ++p) t += red[p][cc][e];
+                out[e] = t;
+            }
+        }
+    }
+}
+
+// Stage 2: ordered sum of the per-row-block partials, one lane per column.
+__global__ __launch_bounds__(256) void colreduce_final_kernel(const float* __restrict__ part,
+                                                              int64_t n_part, int64_t C, void* out,
+                                                              int out_f32) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float t = 0.f;
+    for (int64_t p = 0; p < n_part; ++p) t += part[p * C + c];
+    if (out_f32) static_cast<float*>(out)[c] = t;
+    else static_cast<uint16_t*>(out)[c] = f32_to_bf16(t);
+}
+
+template <int NV>
+static void launch_ln_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                          float* rstd, int64_t rows, int C, float eps, hipStream_t st) {
+    const uint32_t nb = (uint32_t)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+    hipLaunchKernelGGL(layernorm_fwd_kernel<NV>, dim3(nb), dim3(256), 0, st, (const uint16_t*)x,
+                       (const uint16_t*)gamma, (const uint16_t*)beta, (uint16_t*)y, mean, rstd, rows, C, eps);
+}
+template <int NV>
+static void launch_ln_bwd_in(const void* dy, const void* x, const void* gamma, const float* mean,
+                             const float* rstd, const void* dres, void* dx, int64_t rows, int C,
+                             hipStream_t st) {
+    const uint32_t nb = (uint32_t)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+    hipLaunchKernelGGL(layernorm_bwd_input_kernel<NV>, dim3(nb), dim3(256), 0, st, (const uint16_t*)dy,
+                       (const uint16_t*)x, (const uint16_t*)gamma, mean, rstd, (const uint16_t*)dres,
+                       (uint16_t*)dx, rows, C);
+}
+
+static int ln_check(const char* who, int64_t rows, int64_t C) {
+    if (rows < 0 || C <= 0) return fail(PP_ERR_INVALID, "%s: bad shape", who);
+    if (C % 8) return fail(PP_ERR_UNSUPPORTED, "%s: C %% 8 != 0 (C=%lld)", who, (long long)C);
+    if (C > 64 * 8 * 16) return fail(PP_ERR_UNSUPPORTED, "%s: C > 8192", who);
+    return PP_OK;
+}
+
+}  // namespace pp
+
+using namespace pp;
+
+extern "C" int pp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y,
+                                float* mean, float* rstd, int64_t rows, int64_t C, float eps,
+                                pp_stream stream) {
+    int rc = ln_check("pp_layernorm_fwd", rows, C);
+    if (rc) return rc;
+    if (rows == 0) return PP_OK;
+    if (!x || !gamma || !y || !mean || !rstd) return fail(PP_ERR_INVALID, "pp_layernorm_fwd: null pointer");
+    if (!aligned(x, 16) || !aligned(y, 16) || !aligned(gamma, 16) || !aligned(beta, 16))
+        return fail(PP_ERR_INVALID, "pp_layernorm_fwd: pointers must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int nv = (int)((C / 8 + 63) / 64);
+    if (nv <= 1) launch_ln_fwd<1>(x, gamma, beta, y, mean, rstd, rows, (int)C, eps, st);
+    else if (nv <= 2) launch_ln_fwd<2>(x, gamma, beta, y, mean, rstd, rows, (int)C, eps, st);
+    else if (nv <= 4) launch_ln_fwd<4>(x, gamma, beta, y, mean, rstd, rows, (int)C, eps, st);
+    else if (nv <= 8) launch_ln_fwd<8>(x, gamma, beta, y, mean, rstd, rows, (int)C, eps, st);
+    else launch_ln_fwd<16>(x, gamma, beta, y, mean, rstd, rows, (int)C, eps, st);
+    return check_launch("layernorm_fwd_kernel");
+}
+
+extern "C" int pp_layernorm_bwd_input(const void* dy, const void* x, const void* gamma,
+                                      const float* mean, const float* rstd, const void* dres,
+                                      void* dx, int64_t rows, int64_t C, pp_stream stream) {
+    int rc = ln_check("pp_layernorm_bwd_input", rows, C);
+    if (rc) return rc;
+    if (rows == 0) return PP_OK;
+    if (!dy || !x || !gamma || !mean || !rstd || !dx)
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input: null pointer");
+    if (!aligned(x, 16) || !aligned(dy, 16) || !aligned(gamma, 16) || !aligned(dres, 16) || !aligned(dx, 16))
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input: pointers must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int nv = (int)((C / 8 + 63) / 64);
+    if (nv <= 1) launch_ln_bwd_in<1>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
+    else if (nv <= 2) launch_ln_bwd_in<2>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
+    else if (nv <= 4) launch_ln_bwd_in<4>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
+    else if (nv <= 8) launch_ln_bwd_in<8>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
+    else launch_ln_bwd_in<16>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
+    return check_launch("layernorm_bwd_input_kernel");
+}
+
+extern "C" int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean,
+                                       const float* rstd, void* dgamma, void* dbeta, int out_dtype,
+                                       float* workspace, int64_t rows, int64_t C, pp_stream stream) {
+    if (rows < 0 || C <= 0) return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: bad shape");
+    if (C % 8) return fail(PP_ERR_UNSUPPORTED, "pp_layernorm_bwd_weight: C %% 8 != 0");
+    if (!dy || !x || !mean || !rstd || !dgamma || !workspace)
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: null pointer");
+    if (!aligned(x, 16) || !aligned(dy, 16))
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: pointers must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t n_part = (rows + 127) / 128;
+    float* part_b = workspace;
+    float* part_g = workspace + n_part * C;
+    if (n_part > 0) {
+        dim3 grid((uint32_t)n_part, (uint32_t)((C + 255) / 256));
+        hipLaunchKernelGGL(colreduce_partial_kernel<true>, grid, dim3(256), 0, st, (const uint16_t*)dy, C,
+                           (const uint16_t*)x, mean, rstd, part_g, part_b, rows, C);
+    }
+    const uint32_t nb = (uint32_t)((C + 255) / 256);
+    hipLaunchKernelGGL(colreduce_final_kernel, dim3(nb), dim3(256), 0, st, part_g, n_part, C, dgamma,
+                       out_dtype == PP_F32);
+    if (dbeta)
+        hipLaunchKernelGGL(colreduce_final_kernel, dim3(nb), dim3(256), 0, st, part_b, n_part, C, dbeta,
+                           out_dtype == PP_F32);
+    return check_launch("layernorm_bwd_weight");
+}
+
+extern "C" int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out,
+                              int out_dtype, float* workspace, pp_stream stream) {
+    if (M < 0 || N <= 0 || ld < N) return fail(PP_ERR_INVALID, "pp_colsum_bf16: bad shape");
+    if ((N % 8) || (ld % 8)) return fail(PP_ERR_UNSUPPORTED, "pp_colsum_bf16: N and ld must be multiples of 8");
+    if (!dY || !out || !workspace) return fail(PP_ERR_INVALID, "pp_colsum_bf16: null pointer");
+    if (!aligned(dY, 16)) return fail(PP_ERR_INVALID, "pp_colsum_bf16: dY must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t n_part = (M + 127) / 128;
+    if (n_part > 0) {
+        dim3 grid((uint32_t)n_part, (uint32_t)((N + 255) / 256));
+        hipLaunchKernelGGL(colreduce_partial_kernel<false>, grid, dim3(256), 0, st, (const uint16_t*)dY, ld,
+                           (const uint16_t*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                           (float*)nullptr, workspace, M, N);
+    }
+    hipLaunchKernelGGL(colreduce_final_kernel, dim3((uint32_t)((N + 255) / 256)), dim3(256), 0, st,
+                       workspace, n_part, N, out, out_dtype == PP_F32);
+    return check_launch("colsum");
+}

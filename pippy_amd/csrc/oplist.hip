@@ -1,0 +1,86 @@
+// Launch list: replays a host array of tagged descriptors on one stream.  A pipeline stage
+// compiles its forward / input-gradient / weight-gradient pass for one microbatch into such a
+// list once, so that a pass costs one call from the host language instead of one per kernel.
+#include "common.h"
+
+using namespace pp;
+
+static int run_one(const pp_op& op, pp_stream st) {
+    switch (op.kind) {
+        case PP_OP_GEMM_BF16:
+        case PP_OP_GEMM_F32: {
+            pp_gemm_desc d;
+            d.A = op.p[0]; d.B = op.p[1]; d.C = op.p[2];
+            d.bias = op.p[3]; d.aux_in = op.p[4]; d.aux_out = op.p[5];
+            d.M = op.i[0]; d.N = op.i[1]; d.K = op.i[2];
+            d.lda = op.i[3]; d.ldb = op.i[4]; d.ldc = op.i[5]; d.ld_aux = op.i[6];
+            d.a_trans = op.j[0]; d.b_trans = op.j[1]; d.epilogue = op.j[2]; d.c_dtype = op.j[3];
+            d.beta = op.j[4]; d.reserved = 0;
+            return op.kind == PP_OP_GEMM_BF16 ? pp_gemm_bf16(&d, st) : pp_gemm_f32(&d, st);
+        }
+        case PP_OP_COLSUM:
+            return pp_colsum_bf16(op.p[0], op.i[0], op.i[1], op.i[2], op.p[1], op.j[0],
+                                  static_cast<float*>(op.p[2]), st);
+        case PP_OP_LN_FWD:
+            return pp_layernorm_fwd(op.p[0], op.p[1], op.p[2], op.p[3], static_cast<float*>(op.p[4]),
+                                    static_cast<float*>(op.p[5]), op.i[0], op.i[1], op.f[0], st);
+        case PP_OP_LN_BWD_INPUT:
+            return pp_layernorm_bwd_input(op.p[0], op.p[1], op.p[2], static_cast<const float*>(op.p[3]),
+                                          static_cast<const float*>(op.p[4]), op.p[5], op.p[6], op.i[0],
+                                          op.i[1], st);
+        case PP_OP_LN_BWD_WEIGHT:
+            return pp_layernorm_bwd_weight(op.p[0], op.p[1], static_cast<const float*>(op.p[2]),
+                                           static_cast<const float*>(op.p[3]), op.p[4], op.p[5], op.j[0],
+                                           static_cast<float*>(op.p[6]), op.i[0], op.i[1], st);
+        case PP_OP_ATTN_FWD:
+        case PP_OP_ATTN_BWD: {
+            pp_attn_desc d;
+            d.q = op.p[0]; d.k = op.p[1]; d.v = op.p[2]; d.o = op.p[3];
+            d.lse = static_cast<float*>(op.p[4]); d.d_o = op.p[5];
+            d.dq = op.p[6]; d.dk = op.p[7]; d.dv = op.p[8]; d.delta = static_cast<float*>(op.p[9]);
+            d.B = op.i[0]; d.S = op.i[1]; d.H = op.i[2]; d.D = op.i[3];
+            d.stride_b = op.i[4]; d.stride_s = op.i[5];
+            d.scale = op.f[0]; d.causal = op.j[0];
+            return op.kind == PP_OP_ATTN_FWD ? pp_attn_fwd(&d, st) : pp_attn_bwd(&d, st);
+        }
+        case PP_OP_EMBED_FWD:
+            return pp_embed_fwd(static_cast<const int64_t*>(op.p[0]), op.p[1], op.p[2], op.p[3], op.i[0],
+                                op.i[1], op.i[2], op.i[3], st);
+        case PP_OP_EMBED_BWD:
+            return pp_embed_bwd(static_cast<const int64_t*>(op.p[0]), op.p[1], static_cast<float*>(op.p[2]),
+                                static_cast<float*>(op.p[3]), op.i[0], op.i[1], op.i[2], op.i[3], st);
+        case PP_OP_CE_LOSS:
+            return pp_ce_loss(op.p[0], static_cast<const int64_t*>(op.p[1]), static_cast<float*>(op.p[2]),
+                              op.p[3], static_cast<float*>(op.p[4]), op.i[0], op.i[1], op.i[2], op.i[3],
+                              op.j[0], st);
+        case PP_OP_ACCUM_BF16:
+            return pp_grad_accum_f32_bf16(static_cast<float*>(op.p[0]), static_cast<const uint16_t*>(op.p[1]),
+                                          op.i[0], op.j[0], st);
+        case PP_OP_ACCUM_F32:
+            return pp_grad_accum_f32_f32(static_cast<float*>(op.p[0]), static_cast<const float*>(op.p[1]),
+                                         op.i[0], op.j[0], st);
+        case PP_OP_COPY_ROWS: {
+            pp_copy_seg s;
+            s.src = op.p[0]; s.dst = op.p[1];
+            s.n_rows = op.i[0]; s.row_bytes = op.i[1]; s.src_stride = op.i[2]; s.dst_stride = op.i[3];
+            return pp_copy_rows(&s, 1, st);
+        }
+        case PP_OP_FILL:
+            return pp_fill_bytes(op.p[0], op.j[0], op.i[0], st);
+        default:
+            return fail(PP_ERR_INVALID, "unknown op kind %d", op.kind);
+    }
+}
+
+extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
+    if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PP_ERR_INVALID, "pp_run_ops: bad list");
+    for (int i = 0; i < n_ops; ++i) {
+        const int rc = run_one(ops[i], stream);
+        if (rc != PP_OK) {
+            char msg[400];
+            snprintf(msg, sizeof msg, "%s", pp_last_error());
+            return fail(rc, "pp_run_ops: op %d (kind %d): %s", i, ops[i].kind, msg);
+        }
+    }
+    return PP_OK;
+}

@@ -1,0 +1,433 @@
+"""Parity of each HIP kernel, called through the C ABI, against the CPU oracle.
+
+Byte-moving and accumulate kernels must be bit-exact; bf16 arithmetic kernels must stay within
+2e-2 max relative error per tensor of the fp32 oracle; fp32 kernels within 1e-5.
+"""
+import math
+
+import pytest
+import torch
+
+from _util import BF16_TOL, F32_TOL, assert_close_rel
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def native():
+    from pippy_amd import _native
+    _native.lib()
+    return _native
+
+
+def note(msg):
+    print(msg, flush=True)
+
+
+# ---- split / merge -------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.int64])
+@pytest.mark.parametrize("shape,dim,n", [
+    ((256, 512), 0, 4), ((7, 33, 5), 1, 4), ((3, 10, 17), 2, 3), ((64, 512), 0, 8),
+    ((5, 9), 1, 9), ((2, 1024, 50), 1, 8), ((129,), 0, 4),
+])
+def test_split_merge_bit_exact(dtype, shape, dim, n):
+    N = native()
+    torch.manual_seed(0)
+    if dtype.is_floating_point:
+        x = torch.randn(shape, device=DEV).to(dtype)
+    else:
+        x = torch.randint(0, 127, shape, device=DEV).to(dtype)
+    ref = [c.contiguous() for c in torch.tensor_split(x, n, dim)]
+    outs = [torch.empty_like(c) for c in ref]
+    N.split_copy(x, outs, dim)
+    for i, (a, b) in enumerate(zip(outs, ref)):
+        assert torch.equal(a, b), f"split chunk {i}"
+    merged = torch.empty_like(x)
+    N.merge_copy(merged, outs, dim)
+    assert torch.equal(merged, x)
+    assert torch.equal(merged, torch.cat(ref, dim))
+
+
+def test_merge_uneven_and_strided_rows():
+    N = native()
+    torch.manual_seed(1)
+    # concatenation of chunks with arbitrary sizes along dim 1
+    chunks = [torch.randn(4, d, 6, device=DEV, dtype=torch.bfloat16) for d in (1, 5, 2, 9)]
+    ref = torch.cat(chunks, 1)
+    out = torch.empty_like(ref)
+    N.merge_copy(out, chunks, 1)
+    assert torch.equal(out, ref)
+    # rows with a padded source stride and an odd row length (vocabulary-like)
+    V, ld, rows = 1001, 1008, 37
+    src = torch.randn(rows, ld, device=DEV).to(torch.bfloat16)
+    dst = torch.empty(rows, V, device=DEV, dtype=torch.bfloat16)
+    N.copy_rows([(src.data_ptr(), dst.data_ptr(), rows, V * 2, ld * 2, V * 2)])
+    assert torch.equal(dst, src[:, :V])
+
+
+def test_strided_copy_nd():
+    N = native()
+    x = torch.arange(2 * 3 * 4 * 5, device=DEV, dtype=torch.float32).reshape(2, 3, 4, 5)
+    v = x.permute(2, 0, 3, 1)[1:, :, ::2]
+    out = torch.empty(v.shape, device=DEV, dtype=v.dtype)
+    N.strided_copy_nd(out, v)
+    assert torch.equal(out, v.contiguous())
+
+
+def test_merge_large_logits_shape():
+    """Full-size merge of config 3's logits is checked by a round trip (split then merge)."""
+    N = native()
+    x = torch.randn(8, 1024, 50257, device=DEV, dtype=torch.bfloat16)  # 0.82 GB
+    outs = [torch.empty(2, 1024, 50257, device=DEV, dtype=torch.bfloat16) for _ in range(4)]
+    N.split_copy(x, outs, 0)
+    back = torch.empty_like(x)
+    N.merge_copy(back, outs, 0)
+    assert torch.equal(back, x)
+    assert torch.equal(outs[3], x[6:8])
+
+
+# ---- gradient accumulation -------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 7, 8, 4096 + 3, 768 * 3072, 21_300_000 + 5])
+@pytest.mark.parametrize("gdtype", [torch.bfloat16, torch.float32])
+def test_grad_accum_bit_exact(n, gdtype):
+    N = native()
+    torch.manual_seed(n % 97)
+    M = 4
+    gs = [(torch.randn(n, device=DEV) * (10.0 ** (m - 2))).to(gdtype) for m in range(M)]
+    acc = torch.full((n,), float("nan"), device=DEV, dtype=torch.float32)
+    for m, g in enumerate(gs):
+        N.grad_accum(acc, g, init=(m == 0))
+    ref = gs[0].float().clone()
+    for g in gs[1:]:
+        ref.add_(g.float())
+    assert torch.equal(acc, ref)
+    # the same on the CPU: the oracle's sequential fp32 adds
+    ref_cpu = gs[0].float().cpu().clone()
+    for g in gs[1:]:
+        ref_cpu.add_(g.float().cpu())
+    assert torch.equal(acc.cpu(), ref_cpu)
+
+
+def test_grad_accum_init_keeps_negative_zero():
+    N = native()
+    g = torch.tensor([-0.0, 0.0, 1.5, -2.0] * 4, device=DEV, dtype=torch.bfloat16)
+    acc = torch.empty(16, device=DEV, dtype=torch.float32)
+    N.grad_accum(acc, g, init=True)
+    assert torch.equal(acc.view(torch.int32), g.float().view(torch.int32))
+
+
+def test_fill_bytes():
+    N = native()
+    t = torch.full((1000003,), 7, device=DEV, dtype=torch.uint8)
+    N.fill_bytes(t[3:], 0)
+    assert int(t[:3].sum()) == 21 and int(t[3:].sum()) == 0
+
+
+# ---- GEMM ----------------------------------------------------------------------------------------
+def _gemm_ref(A, B, a_trans, b_trans):
+    a = A.float().cpu()
+    b = B.float().cpu()
+    a = a.t() if a_trans else a
+    b = b.t() if b_trans else b
+    return a @ b.t()
+
+
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 768), (200, 136, 72), (4096, 768, 768),
+                                   (1000, 1001, 264), (64, 8, 8)])
+def test_gemm_bf16_layouts(a_trans, b_trans, M, N, K):
+    Nn = native()
+    if a_trans and M % 8:
+        pytest.skip("transposed A needs M % 8 == 0")
+    if b_trans and N % 8:
+        pytest.skip("transposed B needs N % 8 == 0")
+    torch.manual_seed(M + N + K)
+    A = torch.randn((K, M) if a_trans else (M, K), device=DEV).to(torch.bfloat16)
+    B = torch.randn((K, N) if b_trans else (N, K), device=DEV).to(torch.bfloat16)
+    ldc = (N + 3) // 4 * 4
+    Cbuf = torch.full((M, ldc), float("nan"), device=DEV, dtype=torch.bfloat16)
+    C = Cbuf[:, :N]
+    note(f"gemm {M}x{N}x{K} at={a_trans} bt={b_trans}")
+    Nn.gemm_bf16(A, B, C, a_trans=a_trans, b_trans=b_trans)
+    torch.cuda.synchronize()
+    ref = _gemm_ref(A, B, a_trans, b_trans)
+    assert_close_rel(C, ref, BF16_TOL, "gemm")
+    # fp32 output is exact up to summation order: much tighter than bf16 rounding
+    C32 = torch.empty(M, ldc, device=DEV, dtype=torch.float32)[:, :N]
+    Nn.gemm_bf16(A, B, C32, a_trans=a_trans, b_trans=b_trans)
+    assert_close_rel(C32, ref, 1e-5, "gemm fp32 out")
+
+
+def test_gemm_bf16_epilogues():
+    Nn = native()
+    torch.manual_seed(5)
+    M, N, K = 384, 264, 136
+    A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    W = (torch.randn(N, K, device=DEV) * 0.1).to(torch.bfloat16)
+    bias = torch.randn(N, device=DEV).to(torch.bfloat16)
+    R = torch.randn(M, N, device=DEV).to(torch.bfloat16)
+    a, w, b, r = A.float().cpu(), W.float().cpu(), bias.float().cpu(), R.float().cpu()
+    lin = a @ w.t()
+
+    C = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    Nn.gemm_bf16(A, W, C, epilogue=Nn.EPI_BIAS, bias=bias)
+    assert_close_rel(C, lin + b, BF16_TOL, "bias")
+
+    for epi, fn in ((Nn.EPI_BIAS_GELU_ERF, O.gelu_erf), (Nn.EPI_BIAS_GELU_TANH, O.gelu_tanh)):
+        pre = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+        Nn.gemm_bf16(A, W, C, epilogue=epi, bias=bias, aux_out=pre)
+        assert_close_rel(pre, lin + b, BF16_TOL, "pre-activation")
+        assert_close_rel(C, fn(lin + b), BF16_TOL, "gelu")
+        # without saving the pre-activation
+        C2 = torch.empty_like(C)
+        Nn.gemm_bf16(A, W, C2, epilogue=epi, bias=bias)
+        assert torch.equal(C, C2)
+
+    Nn.gemm_bf16(A, W, C, epilogue=Nn.EPI_BIAS_RESIDUAL, bias=bias, aux_in=R)
+    assert_close_rel(C, lin + b + r, BF16_TOL, "bias+residual")
+    Nn.gemm_bf16(A, W, C, epilogue=Nn.EPI_BIAS_RESIDUAL, aux_in=R)
+    assert_close_rel(C, lin + r, BF16_TOL, "residual")
+
+    Nn.gemm_bf16(A, W, C, epilogue=Nn.EPI_BIAS_RELU, bias=bias)
+    assert_close_rel(C, torch.relu(lin + b), BF16_TOL, "relu")
+    Nn.gemm_bf16(A, W, C, epilogue=Nn.EPI_DRELU, aux_in=R)
+    assert_close_rel(C, lin * (r > 0), BF16_TOL, "drelu")
+
+    for epi, fn in ((Nn.EPI_DGELU_ERF, O.gelu_erf), (Nn.EPI_DGELU_TANH, O.gelu_tanh)):
+        h = r.clone().requires_grad_(True)
+        fn(h).backward(lin)
+        Nn.gemm_bf16(A, W, C, epilogue=epi, aux_in=R)
+        assert_close_rel(C, h.grad, BF16_TOL, "dgelu")
+
+    acc = torch.randn(M, N, device=DEV, dtype=torch.float32)
+    acc0 = acc.cpu().clone()
+    Nn.gemm_bf16(A, W, acc, epilogue=Nn.EPI_ACCUM_F32, beta=1)
+    assert_close_rel(acc, acc0 + lin, 1e-5, "accumulate")
+    Nn.gemm_bf16(A, W, acc, epilogue=Nn.EPI_ACCUM_F32, beta=0)
+    assert_close_rel(acc, lin, 1e-5, "accumulate init")
+
+
+def test_gemm_bf16_rejects_bad_arguments():
+    Nn = native()
+    A = torch.zeros(16, 12, device=DEV, dtype=torch.bfloat16)
+    B = torch.zeros(16, 12, device=DEV, dtype=torch.bfloat16)
+    C = torch.zeros(16, 16, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        Nn.gemm_bf16(A, B, C)
+
+
+def test_gemm_f32():
+    Nn = native()
+    torch.manual_seed(6)
+    for (M, N, K, at, bt) in [(64, 512, 512, False, False), (64, 10, 256, False, False),
+                              (70, 33, 19, False, True), (512, 1024, 64, True, True),
+                              (64, 512, 1024, False, True)]:
+        A = torch.randn((K, M) if at else (M, K), device=DEV)
+        B = torch.randn((K, N) if bt else (N, K), device=DEV)
+        bias = torch.randn(N, device=DEV)
+        C = torch.empty(M, N, device=DEV)
+        ref = _gemm_ref(A, B, at, bt)
+        Nn.gemm_f32(A, B, C, a_trans=at, b_trans=bt)
+        assert_close_rel(C, ref, F32_TOL, "gemm_f32")
+        Nn.gemm_f32(A, B, C, a_trans=at, b_trans=bt, epilogue=Nn.EPI_BIAS_RELU, bias=bias)
+        assert_close_rel(C, torch.relu(ref + bias.cpu()), F32_TOL, "gemm_f32 relu")
+        R = torch.randn(M, N, device=DEV)
+        Nn.gemm_f32(A, B, C, a_trans=at, b_trans=bt, epilogue=Nn.EPI_DRELU, aux_in=R)
+        assert_close_rel(C, ref * (R.cpu() > 0), F32_TOL, "gemm_f32 drelu")
+        acc = torch.randn(M, N, device=DEV)
+        acc0 = acc.cpu().clone()
+        Nn.gemm_f32(A, B, acc, a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_F32, beta=1)
+        assert_close_rel(acc, acc0 + ref, F32_TOL, "gemm_f32 accumulate")
+
+
+# ---- column sums / LayerNorm ------------------------------------------------------------------
+@pytest.mark.parametrize("M,N", [(4096, 768), (100, 264), (1, 8)])
+def test_colsum(M, N):
+    Nn = native()
+    torch.manual_seed(7)
+    dY = torch.randn(M, N, device=DEV).to(torch.bfloat16)
+    ws = torch.empty(((M + 127) // 128) * N, device=DEV)
+    out32 = torch.empty(N, device=DEV)
+    Nn.colsum(dY, out32, ws)
+    assert_close_rel(out32, dY.float().cpu().sum(0), 1e-5, "colsum fp32")
+    out16 = torch.empty(N, device=DEV, dtype=torch.bfloat16)
+    Nn.colsum(dY, out16, ws)
+    assert_close_rel(out16, dY.float().cpu().sum(0), BF16_TOL, "colsum bf16")
+
+
+@pytest.mark.parametrize("rows,C", [(4096, 768), (37, 1024), (5, 8), (130, 4096)])
+def test_layernorm(rows, C):
+    Nn = native()
+    torch.manual_seed(8)
+    x = (torch.randn(rows, C, device=DEV) * 2 + 0.5).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(C, device=DEV)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(C, device=DEV)).to(torch.bfloat16)
+    dy = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+    dres = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+    y = torch.empty_like(x)
+    mean = torch.empty(rows, device=DEV)
+    rstd = torch.empty(rows, device=DEV)
+    eps = 1e-5
+    Nn.layernorm_fwd(x, gamma, beta, y, mean, rstd, eps)
+
+    xr = x.float().cpu().requires_grad_(True)
+    gr = gamma.float().cpu().requires_grad_(True)
+    br = beta.float().cpu().requires_grad_(True)
+    yr = O.layer_norm(xr, gr, br, eps)
+    assert_close_rel(y, yr, BF16_TOL, "ln fwd")
+    assert_close_rel(mean, xr.detach().mean(-1), 1e-4, "ln mean")
+    yr.backward(dy.float().cpu())
+
+    dx = torch.empty_like(x)
+    Nn.layernorm_bwd_input(dy, x, gamma, mean, rstd, None, dx)
+    assert_close_rel(dx, xr.grad, BF16_TOL, "ln dx")
+    Nn.layernorm_bwd_input(dy, x, gamma, mean, rstd, dres, dx)
+    assert_close_rel(dx, xr.grad + dres.float().cpu(), BF16_TOL, "ln dx + residual")
+
+    ws = torch.empty(2 * ((rows + 127) // 128) * C, device=DEV)
+    dg = torch.empty(C, device=DEV)
+    db = torch.empty(C, device=DEV)
+    Nn.layernorm_bwd_weight(dy, x, mean, rstd, dg, db, ws)
+    assert_close_rel(dg, gr.grad, 1e-3, "ln dgamma")
+    assert_close_rel(db, br.grad, 1e-4, "ln dbeta")
+    dg16 = torch.empty(C, device=DEV, dtype=torch.bfloat16)
+    db16 = torch.empty(C, device=DEV, dtype=torch.bfloat16)
+    Nn.layernorm_bwd_weight(dy, x, mean, rstd, dg16, db16, ws)
+    assert_close_rel(dg16, gr.grad, BF16_TOL, "ln dgamma bf16")
+    assert_close_rel(db16, br.grad, BF16_TOL, "ln dbeta bf16")
+
+
+# ---- embedding / loss ----------------------------------------------------------------------------
+def test_embedding():
+    Nn = native()
+    torch.manual_seed(9)
+    vocab, seq, C, B = 1000, 128, 768, 3
+    wte = torch.randn(vocab, C, device=DEV).to(torch.bfloat16)
+    wpe = torch.randn(seq, C, device=DEV).to(torch.bfloat16)
+    ids = torch.randint(0, vocab, (B, seq), device=DEV)
+    ids[0, :5] = 7  # repeated ids exercise the atomic scatter
+    y = torch.empty(B * seq, C, device=DEV, dtype=torch.bfloat16)
+    Nn.embed_fwd(ids, wte, wpe, y, seq)
+    ref = O.embedding(ids.cpu(), wte.float().cpu(), wpe.float().cpu()).reshape(B * seq, C)
+    # a single bf16 rounding of an fp32 sum: identical to torch's bf16 add
+    assert torch.equal(y.cpu(), (wte[ids.reshape(-1)] + wpe.repeat(B, 1)).cpu())
+    assert_close_rel(y, ref, BF16_TOL, "embed fwd")
+    y2 = torch.empty_like(y)
+    Nn.embed_fwd(ids, wte, None, y2, seq)
+    assert torch.equal(y2, wte[ids.reshape(-1)])
+
+    dy = torch.randn(B * seq, C, device=DEV).to(torch.bfloat16)
+    d_wte = torch.zeros(vocab, C, device=DEV)
+    d_wpe = torch.zeros(seq, C, device=DEV)
+    Nn.embed_bwd(ids, dy, d_wte, d_wpe, seq)
+    wr = wte.float().cpu().requires_grad_(True)
+    pr = wpe.float().cpu().requires_grad_(True)
+    O.embedding(ids.cpu(), wr, pr).reshape(B * seq, C).backward(dy.float().cpu())
+    assert_close_rel(d_wte, wr.grad, 1e-5, "d_wte")
+    assert_close_rel(d_wpe, pr.grad, 1e-5, "d_wpe")
+
+
+@pytest.mark.parametrize("rows,V,ld", [(64, 1000, 1000), (33, 1001, 1008), (128, 50257, 50304), (16, 8, 8)])
+def test_ce_loss_bf16(rows, V, ld):
+    Nn = native()
+    torch.manual_seed(10)
+    buf = (torch.randn(rows, ld, device=DEV) * 3).to(torch.bfloat16)
+    logits = buf[:, :V] if ld != V else buf
+    target = torch.randint(0, V, (rows,), device=DEV)
+    target[::7] = -100
+    loss = torch.empty(1, device=DEV)
+    dbuf = torch.full((rows, ld), float("nan"), device=DEV, dtype=torch.bfloat16)
+    ws = torch.empty(rows + 2, device=DEV)
+    Nn.ce_loss(buf, target, loss, dbuf, ws, V)
+    lr = logits.float().cpu().requires_grad_(True)
+    ref = O.cross_entropy_mean(lr, target.cpu())
+    ref.backward()
+    assert_close_rel(loss, ref.detach().reshape(1), 1e-5, "ce loss")
+    assert_close_rel(dbuf[:, :V], lr.grad, BF16_TOL, "ce dlogits")
+    if ld != V:
+        assert float(dbuf[:, V:].float().abs().max()) == 0.0
+    # loss only
+    loss2 = torch.empty(1, device=DEV)
+    Nn.ce_loss(buf, target, loss2, None, ws, V)
+    assert torch.equal(loss, loss2)
+
+
+def test_ce_loss_f32():
+    Nn = native()
+    torch.manual_seed(11)
+    rows, V = 64, 10
+    logits = torch.randn(rows, V, device=DEV) * 2
+    target = torch.randint(0, V, (rows,), device=DEV)
+    loss = torch.empty(1, device=DEV)
+    dl = torch.empty_like(logits)
+    ws = torch.empty(rows + 2, device=DEV)
+    Nn.ce_loss(logits, target, loss, dl, ws, V)
+    lr = logits.cpu().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(lr, target.cpu())
+    ref.backward()
+    assert_close_rel(loss, ref.detach().reshape(1), F32_TOL, "ce f32 loss")
+    assert_close_rel(dl, lr.grad, F32_TOL, "ce f32 grad")
+
+
+# ---- attention -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,S,H", [(1, 128, 1), (2, 256, 3), (1, 1024, 2)])
+def test_attention(causal, B, S, H):
+    Nn = native()
+    torch.manual_seed(12 + S)
+    D = 64
+    qkv = torch.randn(B, S, 3 * H * D, device=DEV).to(torch.bfloat16)
+    o = torch.full((B, S, H * D), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    note(f"attention fwd B={B} S={S} H={H} causal={causal}")
+    Nn.attn_fwd(qkv, o, lse, H, causal)
+    torch.cuda.synchronize()
+    qr = qkv.float().cpu().requires_grad_(True)
+    ref = O.attention_fused_qkv(qr, H, causal)
+    assert_close_rel(o, ref, BF16_TOL, "attention fwd")
+
+    d_o = torch.randn(B, S, H * D, device=DEV).to(torch.bfloat16)
+    dqkv = torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    note(f"attention bwd B={B} S={S} H={H} causal={causal}")
+    Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal)
+    torch.cuda.synchronize()
+    ref.backward(d_o.float().cpu())
+    HD = H * D
+    for name, sl in (("dq", slice(0, HD)), ("dk", slice(HD, 2 * HD)), ("dv", slice(2 * HD, 3 * HD))):
+        assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"attention {name}")
+
+
+# ---- launch list ---------------------------------------------------------------------------------
+def test_run_ops_matches_direct_calls():
+    import ctypes as C
+    Nn = native()
+    torch.manual_seed(13)
+    M, N, K = 256, 128, 64
+    A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    W = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    bias = torch.randn(N, device=DEV).to(torch.bfloat16)
+    C1 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    C2 = torch.empty_like(C1)
+    acc1 = torch.zeros(M * N, device=DEV)
+    acc2 = torch.zeros(M * N, device=DEV)
+    Nn.gemm_bf16(A, W, C1, epilogue=Nn.EPI_BIAS, bias=bias)
+    Nn.grad_accum(acc1, C1.reshape(-1), init=True)
+    ops = (Nn.Op * 2)()
+    g = ops[0]
+    g.kind = Nn.OP_GEMM_BF16
+    g.p[0], g.p[1], g.p[2], g.p[3] = A.data_ptr(), W.data_ptr(), C2.data_ptr(), bias.data_ptr()
+    g.i[0], g.i[1], g.i[2], g.i[3], g.i[4], g.i[5] = M, N, K, K, K, N
+    g.j[2], g.j[3] = Nn.EPI_BIAS, Nn.PP_BF16
+    a = ops[1]
+    a.kind = Nn.OP_ACCUM_BF16
+    a.p[0], a.p[1] = acc2.data_ptr(), C2.data_ptr()
+    a.i[0] = M * N
+    a.j[0] = 1
+    Nn.run_ops(ops, 2)
+    assert torch.equal(C1, C2) and torch.equal(acc1, acc2)
+    ops[1].kind = 999
+    with pytest.raises(RuntimeError, match="op 1"):
+        Nn.run_ops(ops, 2)
