@@ -134,6 +134,13 @@ int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
 int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, int out_dtype,
                    float* workspace, pp_stream stream);
 
+/* dz[i] = dy[i] * act'(aux[i]) for act 0 = relu (aux: the activation's output or input),
+ * 1 = gelu (erf form, aux: pre-activation), 2 = gelu (tanh form); dtype PP_BF16 or PP_F32.
+ * Backward of an activation that stands between two separately lowered linears
+ * (torch.relu in examples/basic/example_train.py:19-22, differentiated by pippy/_backward.py:67-69). */
+int pp_activation_bwd(const void* dy, const void* aux, void* dz, int64_t n, int act, int dtype,
+                      pp_stream stream);
+
 /* ------------------------------------------------------------------------------------------
  * LayerNorm (F.layer_norm inside the stage module; backward via pippy/_backward.py:67-69).
  * x, y, dy, dx: bf16 [rows, C]; gamma, beta: bf16 [C]; mean, rstd: fp32 [rows].
@@ -201,8 +208,27 @@ enum pp_op_kind {
     PP_OP_GEMM_BF16 = 1, PP_OP_GEMM_F32 = 2, PP_OP_COLSUM = 3, PP_OP_LN_FWD = 4,
     PP_OP_LN_BWD_INPUT = 5, PP_OP_LN_BWD_WEIGHT = 6, PP_OP_ATTN_FWD = 7, PP_OP_ATTN_BWD = 8,
     PP_OP_EMBED_FWD = 9, PP_OP_EMBED_BWD = 10, PP_OP_CE_LOSS = 11, PP_OP_ACCUM_BF16 = 12,
-    PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15
+    PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16
 };
+
+/* Field use per kind (unused fields are ignored):
+ *   GEMM_*        p: A B C bias aux_in aux_out | i: M N K lda ldb ldc ld_aux | j: a_trans b_trans
+ *                 epilogue c_dtype beta
+ *   COLSUM        p: dY out workspace | i: M N ld | j: out_dtype
+ *   LN_FWD        p: x gamma beta y mean rstd | i: rows C | f: eps
+ *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C
+ *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
+ *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
+ *                 | j: causal
+ *   EMBED_FWD     p: ids wte wpe y | i: n_tok seq C vocab
+ *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab
+ *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype
+ *   ACCUM_*       p: acc g | i: n | j: init
+ *   COPY_ROWS     p: src dst | i: n_rows row_bytes src_stride dst_stride
+ *   FILL          p: dst | i: n_bytes | j: value
+ *   ACT_BWD       p: dy aux dz | i: n | j: act dtype
+ * flags bit 0 (PP_OP_SKIP): the op is stepped over. */
+#define PP_OP_SKIP 1
 
 typedef struct pp_op {
     int32_t kind;   /* enum pp_op_kind */

@@ -1,0 +1,268 @@
+"""Pipeline front end: split a model into stage modules (mirrors the public part of
+``pippy/_IR.py``: ``pipeline``, ``Pipe``, ``SplitPoint``, ``pipe_split``,
+``annotate_split_points``, ``ArgsChunkSpec``, ``KwargsChunkSpec``).
+
+The reference exports the model with ``torch.export`` and cuts the ATen graph at ``pipe_split``
+markers (``_IR.py:679-1125``).  This front end runs once at set-up and does no device work, so it
+is kept small: the model is traced with ``torch.fx`` at module granularity (a module that does not
+contain a split point stays one node, so stage modules keep whole layers that the stage runtime
+can lower to kernels), markers are placed from ``split_spec`` or from ``pipe_split()`` calls in the
+model's ``forward``, and ``torch.fx.passes.split_module`` cuts the graph.  As in the reference,
+stage ``i`` is ``pipe.split_gm.submod_i`` and its parameters keep their original qualified names.
+"""
+from __future__ import annotations
+
+import logging
+from dataclasses import dataclass
+from enum import Enum
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+import torch.fx as fx
+import torch.nn as nn
+from torch.fx.passes.split_module import split_module
+
+from .microbatch import TensorChunkSpec, split_args_kwargs_into_chunks
+from .stage_modules import NativeBlock
+
+logger = logging.getLogger(__name__)
+
+
+def pipe_split():
+    """Marks a stage boundary when called inside a model's ``forward``
+    (reference ``_IR.py:319-342``).  A no-op outside of ``pipeline()``."""
+    return None
+
+
+class SplitPoint(Enum):
+    BEGINNING = 1
+    END = 2
+
+
+class PipeSplitWrapper:
+    """Kept for source compatibility: ``PipeSplitWrapper.SplitPoint`` (reference ``_IR.py:1299-1303``)."""
+    SplitPoint = SplitPoint
+
+
+class _ModuleGranularityTracer(fx.Tracer):
+    def __init__(self, split_names: Optional[List[str]]):
+        super().__init__(autowrap_functions=(pipe_split,))
+        self._split_names = split_names
+
+    def is_leaf_module(self, m: nn.Module, qualname: str) -> bool:
+        if isinstance(m, NativeBlock):
+            return True
+        if self._split_names is None:
+            return super().is_leaf_module(m, qualname)
+        # descend only into modules that contain a split point
+        is_ancestor = any(s.startswith(qualname + ".") for s in self._split_names)
+        if is_ancestor:
+            return False
+        if qualname in self._split_names:
+            return True
+        return super().is_leaf_module(m, qualname)
+
+
+def _insert_markers(gm_graph: fx.Graph, split_spec: Dict[str, SplitPoint]):
+    for name, point in split_spec.items():
+        hits = [n for n in gm_graph.nodes if n.op == "call_module" and n.target == name]
+        if not hits:
+            raise ValueError(f"Specified split point {name!r} is not a module called by the model")
+        node = hits[0] if point == SplitPoint.BEGINNING else hits[-1]
+        if point == SplitPoint.BEGINNING:
+            with gm_graph.inserting_before(node):
+                gm_graph.call_function(pipe_split, (), {})
+        elif point == SplitPoint.END:
+            with gm_graph.inserting_after(node):
+                gm_graph.call_function(pipe_split, (), {})
+        else:
+            raise ValueError(f"Unknown split point type {point}")
+
+
+@dataclass
+class PipeInfo:
+    """What the stage runtime needs from the front end (reference ``_IR.py:509-516``)."""
+    graph: fx.Graph
+    num_stages: int
+    num_chunks: int
+    has_loss_and_backward: bool
+    args_chunk_spec: Optional[Tuple[Any, ...]] = None
+    kwargs_chunk_spec: Optional[Dict[str, Any]] = None
+
+
+class Pipe(nn.Module):
+    """A model cut into stage modules ``split_gm.submod_0 .. submod_{n-1}``
+    (reference ``_IR.py:494-1291``).  Calling a ``Pipe`` runs the stages one after another in this
+    process, without microbatching (reference ``Pipe.forward``, ``_IR.py:620-651``)."""
+
+    # set by the ArgsChunkSpec / KwargsChunkSpec context managers
+    args_chunk_spec: Optional[Tuple[Any, ...]] = None
+    kwargs_chunk_spec: Optional[Dict[str, Any]] = None
+
+    PipeInfo = PipeInfo
+
+    def __init__(self, split_gm: fx.GraphModule, num_stages: int, has_loss_and_backward: bool = False,
+                 loss_spec=None):
+        super().__init__()
+        self.split_gm = split_gm
+        self.num_stages = num_stages
+        self.has_loss_and_backward = has_loss_and_backward
+        self.loss_spec = loss_spec
+        self.pipe_info: Optional[PipeInfo] = None
+
+    def forward(self, *args, **kwargs):
+        return self.split_gm(*args, **kwargs)
+
+    def get_stage_module(self, stage_idx: int) -> nn.Module:
+        if stage_idx < 0 or stage_idx >= self.num_stages:
+            raise ValueError(f"Invalid stage index {stage_idx}!")
+        return getattr(self.split_gm, f"submod_{stage_idx}")
+
+    def info(self) -> PipeInfo:
+        if self.pipe_info is None:
+            raise RuntimeError("Pipe info is not available. Please use the `pipeline` method to create the `Pipe` object.")
+        return self.pipe_info
+
+    def __str__(self):
+        return self.split_gm.__str__()
+
+    def __repr__(self):
+        return self.split_gm.__repr__()
+
+    @staticmethod
+    def _from_traced(mod: nn.Module, graph: fx.Graph) -> "Pipe":
+        # number the partitions by the markers and drop the markers
+        part = 0
+        part_of: Dict[fx.Node, int] = {}
+        markers = []
+        for n in graph.nodes:
+            if n.op == "call_function" and n.target is pipe_split:
+                part += 1
+                markers.append(n)
+                continue
+            part_of[n] = part
+        for m in markers:
+            graph.erase_node(m)
+        gm = fx.GraphModule(mod, graph)
+        orig_target = {n.name: n.target for n in graph.nodes if n.op in ("call_module", "get_attr")}
+        split = split_module(gm, mod, lambda n: part_of[n], keep_original_order=True)
+        num_stages = part + 1
+        # split_module flattens qualified names ("h.0" -> "h_0"); rebuild every stage module from the
+        # original model with the original targets so that parameter names are unchanged
+        # (the reference re-outlines for the same reason, ``_IR.py:765-769``)
+        for name, sub in list(split.named_children()):
+            if not name.startswith("submod_"):
+                continue
+            for n in sub.graph.nodes:
+                if n.op in ("call_module", "get_attr") and n.name in orig_target:
+                    n.target = orig_target[n.name]
+            setattr(split, name, fx.GraphModule(mod, sub.graph, class_name=name))
+        found = [n for n, _ in split.named_children() if n.startswith("submod_")]
+        if len(found) != num_stages:
+            raise RuntimeError(f"expected {num_stages} stage modules after splitting, found {found} "
+                               "(an empty stage: two split points with nothing between them)")
+        # a parameter may live in one stage only (reference ``_IR.py:871-879``)
+        owner: Dict[int, str] = {}
+        for name, sub in split.named_children():
+            for pn, p in sub.named_parameters():
+                if id(p) in owner and owner[id(p)] != name:
+                    raise NotImplementedError(
+                        f"Parameter {pn} is used in stages {owner[id(p)]} and {name}; parameters shared "
+                        "between stages (e.g. tied embeddings) are not supported")
+                owner[id(p)] = name
+        return Pipe(split, num_stages)
+
+    @staticmethod
+    def from_tracing(mod: nn.Module, num_chunks: int, example_args: Tuple[Any, ...],
+                     example_kwargs: Optional[Dict[str, Any]] = None,
+                     split_policy: Optional[Callable[[fx.GraphModule], fx.GraphModule]] = None,
+                     split_spec: Optional[Dict[str, SplitPoint]] = None) -> "Pipe":
+        args_chunk_spec = Pipe.args_chunk_spec
+        kwargs_chunk_spec = Pipe.kwargs_chunk_spec
+        # validates the chunk specs against the example inputs (reference ``_IR.py:1172-1178``)
+        split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks, args_chunk_spec,
+                                      kwargs_chunk_spec)
+        names = list(split_spec.keys()) if split_spec else None
+        graph = _ModuleGranularityTracer(names).trace(mod)
+        if split_spec:
+            _insert_markers(graph, split_spec)
+        if split_policy is not None:
+            gm = split_policy(fx.GraphModule(mod, graph))
+            graph = gm.graph
+        pipe = Pipe._from_traced(mod, graph)
+        pipe.pipe_info = PipeInfo(graph=pipe.split_gm.graph, num_stages=pipe.num_stages,
+                                  num_chunks=num_chunks, has_loss_and_backward=False,
+                                  args_chunk_spec=args_chunk_spec, kwargs_chunk_spec=kwargs_chunk_spec)
+        return pipe
+
+
+def annotate_split_points(mod: nn.Module, spec: Dict[str, SplitPoint]):
+    """Wraps the named submodules so that their ``forward`` calls ``pipe_split()`` before
+    (BEGINNING) or after (END) itself (reference ``_IR.py:1306-1338``)."""
+    for qualname, split_type in spec.items():
+        try:
+            target = mod.get_submodule(qualname)
+        except AttributeError as e:
+            raise AttributeError(f"Specified target {qualname} referenced nonexistent module") from e
+        orig_forward = target.forward
+
+        def make(orig_forward=orig_forward, split_type=split_type):
+            def forward(*args, **kwargs):
+                if split_type == SplitPoint.BEGINNING:
+                    pipe_split()
+                out = orig_forward(*args, **kwargs)
+                if split_type == SplitPoint.END:
+                    pipe_split()
+                return out
+            return forward
+
+        target.forward = make()
+
+
+def pipeline(module: nn.Module, num_chunks: int, example_args: Tuple[Any, ...],
+             example_kwargs: Optional[Dict[str, Any]] = None,
+             split_spec: Optional[Dict[str, SplitPoint]] = None,
+             split_policy: Optional[Callable[[fx.GraphModule], fx.GraphModule]] = None) -> Pipe:
+    """Splits ``module`` into pipeline stages (reference ``_IR.py:1341-1395``).
+
+    ``split_spec`` maps submodule names to ``SplitPoint.BEGINNING`` / ``END``; alternatively the
+    model's ``forward`` may call ``pipe_split()``, or ``split_policy`` may place the markers on the
+    traced graph.  ``num_chunks`` and the example inputs describe one full batch; the chunk specs
+    in force (``ArgsChunkSpec`` / ``KwargsChunkSpec``) are recorded for the schedules."""
+    if split_spec is not None and split_policy is not None:
+        raise ValueError("Cannot specify both `split_spec` and `split_policy`. Please use only one of them.")
+    return Pipe.from_tracing(mod=module, num_chunks=num_chunks, example_args=example_args,
+                             example_kwargs=example_kwargs, split_policy=split_policy,
+                             split_spec=split_spec)
+
+
+class ArgsChunkSpec:
+    """Context manager that sets the chunk spec of positional args for ``pipeline()``
+    (reference ``_IR.py:1399-1424``)."""
+
+    def __init__(self, chunk_dims: Tuple[int, ...]):
+        self.args_chunk_spec = tuple(TensorChunkSpec(d) for d in chunk_dims)
+
+    def __enter__(self):
+        self._saved = Pipe.args_chunk_spec
+        Pipe.args_chunk_spec = self.args_chunk_spec
+        return self.args_chunk_spec
+
+    def __exit__(self, exc_type, exc_val, traceback):
+        Pipe.args_chunk_spec = self._saved
+
+
+class KwargsChunkSpec:
+    """Context manager that sets the chunk spec of keyword args for ``pipeline()``
+    (reference ``_IR.py:1427-1451``)."""
+
+    def __init__(self, chunk_dims: Dict[str, int]):
+        self.kwargs_chunk_spec = {k: TensorChunkSpec(d) for k, d in chunk_dims.items()}
+
+    def __enter__(self):
+        self._saved = Pipe.kwargs_chunk_spec
+        Pipe.kwargs_chunk_spec = self.kwargs_chunk_spec
+        return self.kwargs_chunk_spec
+
+    def __exit__(self, exc_type, exc_val, traceback):
+        Pipe.kwargs_chunk_spec = self._saved

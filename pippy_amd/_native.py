@@ -23,7 +23,9 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7
 # enum pp_op_kind
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
- OP_FILL) = range(1, 16)
+ OP_FILL, OP_ACT_BWD) = range(1, 17)
+OP_SKIP = 1
+ACT_RELU, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
 
 PP_COPY_MAX_SEGS = 64
 
@@ -33,7 +35,7 @@ EXPORTED_SYMBOLS = (
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
     "pp_gemm_bf16", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
-    "pp_ce_loss", "pp_run_ops",
+    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd",
 )
 
 
@@ -107,6 +109,7 @@ def lib() -> C.CDLL:
         "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
+        "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -368,6 +371,15 @@ def ce_loss(logits, target, loss, dlogits, workspace, V: int, ignore_index: int 
                            workspace.data_ptr(), rows, V, logits.stride(0), ignore_index,
                            PP_F32 if logits.dtype == torch.float32 else PP_BF16,
                            current_stream()), "pp_ce_loss")
+
+
+def activation_bwd(dy, aux, dz, act: int) -> None:
+    require_cuda(dy, aux, dz)
+    assert dy.is_contiguous() and aux.is_contiguous() and dz.is_contiguous()
+    assert dy.numel() == aux.numel() == dz.numel() and dy.dtype == aux.dtype == dz.dtype
+    check(lib().pp_activation_bwd(dy.data_ptr(), aux.data_ptr(), dz.data_ptr(), dy.numel(), act,
+                                  PP_F32 if dy.dtype == torch.float32 else PP_BF16,
+                                  current_stream()), "pp_activation_bwd")
 
 
 def run_ops(ops, n: int) -> None:

@@ -1,0 +1,502 @@
+"""Stage programs: a stage module lowered to launch lists of HIP kernels.
+
+The reference executes a stage by calling the user's ``nn.Module`` (``_PipelineStage.py:420-428``)
+and one fused ``torch.autograd.backward`` (``_backward.py:67-69``).  Here a stage whose module is
+built from the blocks in ``stage_modules.py`` is *lowered* once per microbatch slot into three
+launch lists over pre-allocated device buffers:
+
+* ``F``  forward;
+* ``I``  input-gradient pass (dI): gradients w.r.t. the stage input;
+* ``W``  weight-gradient pass (dW): parameter gradients, then their fp32 accumulation.
+
+A fused backward is ``I`` followed by ``W``; a zero-bubble schedule runs them apart.  Lists are
+replayed with one ``pp_run_ops`` call each, so the host language is left once per pass.
+
+HBM layout per stage: one flat parameter arena (module parameters are views into it, names
+unchanged), one flat staging arena for the per-microbatch parameter gradients in the parameter
+dtype, and one flat fp32 accumulator arena; per microbatch slot, the activations saved for
+backward and the stage output plus the gradient buffer of that output (the next stage writes its
+input gradient straight into it: the hand-off is a pointer, not a copy).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import _native as N
+
+_ALIGN_ELEMS = 128  # every arena entry starts on a 256-byte boundary
+
+
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
+class ParamArena:
+    """Flat storage of one stage's parameters, gradient staging and fp32 accumulators."""
+
+    def __init__(self, module: nn.Module, device: torch.device):
+        params = [(n, p) for n, p in module.named_parameters()]
+        if not params:
+            self.dtype = torch.bfloat16
+        else:
+            dts = {p.dtype for _, p in params}
+            if len(dts) != 1:
+                raise RuntimeError(f"a native stage needs one parameter dtype, found {dts}")
+            self.dtype = dts.pop()
+        if self.dtype not in (torch.bfloat16, torch.float32):
+            raise RuntimeError(f"native stages support bf16 or fp32 parameters, not {self.dtype}")
+        pad_rows: Dict[int, int] = {}
+        direct = set()
+        for mod in module.modules():
+            for p, rows in getattr(mod, "_pp_padded_rows", lambda: [])():
+                pad_rows[id(p)] = rows
+            for p in getattr(mod, "_pp_direct_acc_params", lambda: [])():
+                direct.add(id(p))
+        # parameters whose gradient goes through the staging arena come first; the single
+        # accumulate op of a W pass covers [0, staged_total)
+        params = [q for q in params if id(q[1]) not in direct] + [q for q in params if id(q[1]) in direct]
+        self.entries: Dict[int, Tuple[int, int, Tuple[int, ...]]] = {}  # id(p) -> (off, numel, padded shape)
+        off = 0
+        self.staged_total = 0
+        for _, p in params:
+            if id(p) in direct and self.staged_total == 0:
+                self.staged_total = off
+            shape = tuple(p.shape)
+            if id(p) in pad_rows:
+                shape = (pad_rows[id(p)],) + shape[1:]
+            numel = 1
+            for s in shape:
+                numel *= s
+            self.entries[id(p)] = (off, numel, shape)
+            off = _round_up(off + numel, _ALIGN_ELEMS)
+        self.total = off
+        if not direct:
+            self.staged_total = off
+        elif all(id(p) in direct for _, p in params):
+            self.staged_total = 0
+        self.device = device
+        self.params = torch.zeros(max(off, 1), dtype=self.dtype, device=device)
+        self.staging = torch.zeros(max(off, 1), dtype=self.dtype, device=device)
+        self.acc = torch.zeros(max(off, 1), dtype=torch.float32, device=device)
+        for _, p in params:
+            o, _n, _shape = self.entries[id(p)]
+            view = self.params[o:o + p.numel()].view(p.shape)
+            view.copy_(p.detach().to(device))
+            p.data = view
+        self.named = params
+
+    def _slice(self, flat: torch.Tensor, p: nn.Parameter, padded: bool) -> torch.Tensor:
+        o, numel, shape = self.entries[id(p)]
+        if padded:
+            return flat[o:o + numel].view(shape)
+        return flat[o:o + p.numel()].view(p.shape)
+
+    def weight(self, p, padded=True):
+        return self._slice(self.params, p, padded)
+
+    def grad_staging(self, p, padded=True):
+        return self._slice(self.staging, p, padded)
+
+    def grad_acc(self, p, padded=True):
+        return self._slice(self.acc, p, padded)
+
+
+# ---- op constructors (host-side shape checks happen here, before anything is launched) ----------
+def _p(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def op_gemm(A, B, Cm, *, a_trans=False, b_trans=False, epilogue=N.EPI_NONE, bias=None, aux_in=None,
+            aux_out=None, beta=0) -> N.Op:
+    f32 = A.dtype == torch.float32
+    d = N.gemm_desc(A, B, Cm, a_trans=a_trans, b_trans=b_trans, epilogue=epilogue, bias=bias,
+                    aux_in=aux_in, aux_out=aux_out, beta=beta)
+    if bias is not None:
+        assert bias.numel() == Cm.shape[1] and bias.dtype == A.dtype
+    op = N.Op()
+    op.kind = N.OP_GEMM_F32 if f32 else N.OP_GEMM_BF16
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = d.A, d.B, d.C, d.bias, d.aux_in, d.aux_out
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5], op.i[6] = d.M, d.N, d.K, d.lda, d.ldb, d.ldc, d.ld_aux
+    op.j[0], op.j[1], op.j[2], op.j[3], op.j[4] = d.a_trans, d.b_trans, d.epilogue, d.c_dtype, d.beta
+    return op
+
+
+def op_colsum(dY, out, ws) -> N.Op:
+    M, Nn = dY.shape
+    assert dY.stride(1) == 1 and out.numel() == Nn and ws.numel() >= ((M + 127) // 128) * Nn
+    op = N.Op()
+    op.kind = N.OP_COLSUM
+    op.p[0], op.p[1], op.p[2] = dY.data_ptr(), out.data_ptr(), ws.data_ptr()
+    op.i[0], op.i[1], op.i[2] = M, Nn, dY.stride(0)
+    op.j[0] = N.PP_F32 if out.dtype == torch.float32 else N.PP_BF16
+    return op
+
+
+def op_act_bwd(dy, aux, dz, act) -> N.Op:
+    assert dy.is_contiguous() and aux.is_contiguous() and dz.is_contiguous()
+    assert dy.numel() == aux.numel() == dz.numel() and dy.dtype == aux.dtype == dz.dtype
+    op = N.Op()
+    op.kind = N.OP_ACT_BWD
+    op.p[0], op.p[1], op.p[2] = dy.data_ptr(), aux.data_ptr(), dz.data_ptr()
+    op.i[0] = dy.numel()
+    op.j[0] = act
+    op.j[1] = N.PP_F32 if dy.dtype == torch.float32 else N.PP_BF16
+    return op
+
+
+def op_ln_fwd(x, gamma, beta, y, mean, rstd, eps) -> N.Op:
+    rows, Cc = x.shape
+    assert x.is_contiguous() and y.is_contiguous() and y.shape == x.shape
+    assert gamma.numel() == Cc and mean.numel() == rows and rstd.numel() == rows
+    op = N.Op()
+    op.kind = N.OP_LN_FWD
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = (x.data_ptr(), gamma.data_ptr(), _p(beta),
+                                                            y.data_ptr(), mean.data_ptr(), rstd.data_ptr())
+    op.i[0], op.i[1] = rows, Cc
+    op.f[0] = eps
+    return op
+
+
+def op_ln_bwd_input(dy, x, gamma, mean, rstd, dres, dx) -> N.Op:
+    rows, Cc = x.shape
+    for t in (dy, x, dx) + ((dres,) if dres is not None else ()):
+        assert t.is_contiguous() and t.shape == x.shape
+    op = N.Op()
+    op.kind = N.OP_LN_BWD_INPUT
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5], op.p[6] = (
+        dy.data_ptr(), x.data_ptr(), gamma.data_ptr(), mean.data_ptr(), rstd.data_ptr(), _p(dres),
+        dx.data_ptr())
+    op.i[0], op.i[1] = rows, Cc
+    return op
+
+
+def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
+    rows, Cc = x.shape
+    assert dy.is_contiguous() and x.is_contiguous() and dy.shape == x.shape
+    assert dgamma.numel() == Cc and ws.numel() >= 2 * ((rows + 127) // 128) * Cc
+    op = N.Op()
+    op.kind = N.OP_LN_BWD_WEIGHT
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5], op.p[6] = (
+        dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dgamma.data_ptr(), _p(dbeta),
+        ws.data_ptr())
+    op.i[0], op.i[1] = rows, Cc
+    op.j[0] = N.PP_F32 if dgamma.dtype == torch.float32 else N.PP_BF16
+    return op
+
+
+def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None) -> N.Op:
+    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta)
+    op = N.Op()
+    op.kind = kind
+    for k, v in enumerate((d.q, d.k, d.v, d.o, d.lse, d.d_o, d.dq, d.dk, d.dv, d.delta)):
+        op.p[k] = v
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5] = d.B, d.S, d.H, d.D, d.stride_b, d.stride_s
+    op.f[0] = d.scale
+    op.j[0] = d.causal
+    return op
+
+
+def op_embed_fwd(ids, wte, wpe, y, seq) -> N.Op:
+    vocab, Cc = wte.shape
+    assert ids.dtype == torch.int64 and y.shape == (ids.numel(), Cc) and y.is_contiguous()
+    op = N.Op()
+    op.kind = N.OP_EMBED_FWD
+    op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), wte.data_ptr(), _p(wpe), y.data_ptr()
+    op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
+    return op
+
+
+def op_embed_bwd(ids, dy, d_wte, d_wpe, seq) -> N.Op:
+    vocab, Cc = d_wte.shape
+    assert d_wte.dtype == torch.float32 and dy.shape == (ids.numel(), Cc) and dy.is_contiguous()
+    op = N.Op()
+    op.kind = N.OP_EMBED_BWD
+    op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), _p(d_wpe)
+    op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
+    return op
+
+
+def op_ce_loss(logits, target, loss, dlogits, ws, V, ignore_index) -> N.Op:
+    rows = logits.shape[0]
+    assert logits.stride(1) == 1 and ws.numel() >= rows + 2 and target.numel() == rows
+    if dlogits is not None:
+        assert dlogits.stride() == logits.stride() and dlogits.shape[0] == rows
+    op = N.Op()
+    op.kind = N.OP_CE_LOSS
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = (logits.data_ptr(), target.data_ptr(),
+                                                   loss.data_ptr(), _p(dlogits), ws.data_ptr())
+    op.i[0], op.i[1], op.i[2], op.i[3] = rows, V, logits.stride(0), ignore_index
+    op.j[0] = N.PP_F32 if logits.dtype == torch.float32 else N.PP_BF16
+    return op
+
+
+def op_accum(acc, g, init=False) -> N.Op:
+    assert acc.dtype == torch.float32 and acc.numel() == g.numel()
+    op = N.Op()
+    op.kind = N.OP_ACCUM_F32 if g.dtype == torch.float32 else N.OP_ACCUM_BF16
+    op.p[0], op.p[1] = acc.data_ptr(), g.data_ptr()
+    op.i[0] = acc.numel()
+    op.j[0] = int(init)
+    return op
+
+
+def op_fill(t, value=0) -> N.Op:
+    assert t.is_contiguous()
+    op = N.Op()
+    op.kind = N.OP_FILL
+    op.p[0] = t.data_ptr()
+    op.i[0] = t.numel() * t.element_size()
+    op.j[0] = value
+    return op
+
+
+OP_SKIP = N.OP_SKIP  # pp_op.flags bit: the runner steps over the op
+
+
+class OpList:
+    """A growable list of descriptors, frozen into one ctypes array before its first replay."""
+
+    def __init__(self):
+        self.ops: List[N.Op] = []
+        self._arr = None
+
+    def append(self, op: N.Op) -> int:
+        assert self._arr is None, "list is frozen"
+        self.ops.append(op)
+        return len(self.ops) - 1
+
+    def freeze(self):
+        n = len(self.ops)
+        arr = (N.Op * max(n, 1))()
+        for k, op in enumerate(self.ops):
+            C.memmove(C.byref(arr, k * C.sizeof(N.Op)), C.byref(op), C.sizeof(N.Op))
+        self._arr = arr
+        self.n = n
+
+    def run(self):
+        if self._arr is None:
+            self.freeze()
+        if self.n:
+            N.run_ops(self._arr, self.n)
+
+    def __getitem__(self, k) -> N.Op:
+        if self._arr is None:
+            self.freeze()
+        return self._arr[k]
+
+    def find_pointer(self, ptr: int) -> List[Tuple[int, int]]:
+        if self._arr is None:
+            self.freeze()
+        hits = []
+        for k in range(self.n):
+            for q in range(10):
+                if self._arr[k].p[q] == ptr:
+                    hits.append((k, q))
+        return hits
+
+
+class MicrobatchProgram:
+    """Launch lists and buffers of one (stage, microbatch slot)."""
+
+    def __init__(self):
+        self.F = OpList()
+        self.I = OpList()
+        self.W = OpList()
+        self.acts: Dict[str, torch.Tensor] = {}
+        self.input_slot: Optional[torch.Tensor] = None
+        self.output: Optional[torch.Tensor] = None       # what the next stage (or the user) sees
+        self.output_grad: Optional[torch.Tensor] = None  # gradient of `output`, same layout
+        self.input_grad: Optional[torch.Tensor] = None
+        self.in_key = None
+        self.input_patches: List[Tuple[OpList, int, int]] = []
+        self.init_toggle_fill: List[int] = []   # W ops that run only on the first accumulation
+        self.init_toggle_accum: List[int] = []  # W ops whose init flag follows the stage state
+        self.init_toggle_beta: List[int] = []   # W GEMMs that accumulate in their epilogue
+        self.loss_ops: Dict[int, Tuple[OpList, torch.Tensor, torch.Tensor]] = {}
+
+
+class Builder:
+    """Handed to ``block.lower``: allocates buffers and records ops for one microbatch slot."""
+
+    def __init__(self, stage_prog: "StageProgram", mb: int, prog: MicrobatchProgram):
+        self.sp = stage_prog
+        self.mb = mb
+        self.prog = prog
+        self.training = stage_prog.training
+        self.fused_accumulate = stage_prog.fused_accumulate
+        self._scope: List[str] = []
+        self._backward: List[Callable] = []
+        self.device = stage_prog.device
+
+    # -- naming
+    def scope(self, name: str):
+        b = self
+
+        class _S:
+            def __enter__(self_inner):
+                b._scope.append(name)
+
+            def __exit__(self_inner, *exc):
+                b._scope.pop()
+        return _S()
+
+    def _key(self, name: str) -> str:
+        return ".".join(self._scope + [name])
+
+    # -- buffers
+    def act(self, name, shape, dtype=None) -> torch.Tensor:
+        """Per-microbatch buffer that lives from forward until the matching backward."""
+        t = torch.empty(tuple(shape), dtype=dtype or self.sp.act_dtype, device=self.device)
+        self.prog.acts[self._key(name)] = t
+        return t
+
+    def grad(self, name, shape, dtype=None) -> torch.Tensor:
+        """Gradient buffer written in the I pass and read in the W pass.  Shared by all
+        microbatches of the stage when I and W run back to back; per microbatch when the schedule
+        may defer W (zero-bubble)."""
+        if self.sp.split_backward:
+            return self.act("grad:" + name, shape, dtype)
+        return self.sp.shared(self._key("grad:" + name), shape, dtype or self.sp.act_dtype)
+
+    def scratch(self, name, shape, dtype) -> torch.Tensor:
+        """Workspace valid inside one kernel sequence (never carried across passes)."""
+        return self.sp.shared("scratch:" + name, shape, dtype, exact=False)
+
+    # -- parameters
+    def weight(self, p, padded=True):
+        return self.sp.arena.weight(p, padded)
+
+    def grad_target(self, p, padded=True):
+        """Where the W pass writes this parameter's microbatch gradient: the staging arena (then one
+        accumulate op folds the arena into fp32), or the fp32 accumulator when the GEMM epilogue
+        accumulates itself."""
+        return self.sp.arena.grad_staging(p, padded)
+
+    def grad_acc(self, p, padded=True):
+        return self.sp.arena.grad_acc(p, padded)
+
+    # -- ops
+    def f(self, op):
+        return self.prog.F.append(op)
+
+    def i(self, op):
+        return self.prog.I.append(op)
+
+    def w(self, op):
+        return self.prog.W.append(op)
+
+    def w_weight_gemm(self, dY2d, X2d, p, padded=True):
+        """dW[out, in] = dY^T X for a linear weight ``p``: bf16/fp32 into staging, or fused fp32
+        accumulation."""
+        if self.fused_accumulate:
+            k = self.w(op_gemm(dY2d, X2d, self.grad_acc(p, padded), a_trans=True, b_trans=True,
+                               epilogue=N.EPI_ACCUM_F32, beta=1))
+            self.prog.init_toggle_beta.append(k)
+        else:
+            self.w(op_gemm(dY2d, X2d, self.grad_target(p, padded), a_trans=True, b_trans=True))
+
+    def on_backward(self, fn: Callable):
+        self._backward.append(fn)
+
+
+class StageProgram:
+    """All microbatch programs of one stage plus its arenas and shared buffers."""
+
+    def __init__(self, blocks: Sequence[nn.Module], module: nn.Module, device, training: bool,
+                 split_backward: bool, fused_accumulate: bool, is_first: bool, is_last: bool):
+        self.blocks = list(blocks)
+        self.device = device
+        self.training = training
+        self.split_backward = split_backward
+        self.fused_accumulate = fused_accumulate
+        self.is_first = is_first
+        self.is_last = is_last
+        self.arena = ParamArena(module, device)
+        self.act_dtype = self.arena.dtype
+        self._shared: Dict[str, torch.Tensor] = {}
+        self.mbs: Dict[int, MicrobatchProgram] = {}
+        self.acc_initialized = False  # False: the next W pass overwrites the accumulators
+
+    def shared(self, key, shape, dtype, exact=True) -> torch.Tensor:
+        shape = tuple(shape)
+        numel = 1
+        for s in shape:
+            numel *= s
+        t = self._shared.get(key)
+        if t is None or t.dtype != dtype or t.numel() < numel or (exact and t.numel() != numel):
+            t = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
+            self._shared[key] = t
+        return t[:numel].view(shape)
+
+    def ones_f32(self, n: int) -> torch.Tensor:
+        """A [1, n] row of ones (the left operand that turns an fp32 GEMM into a column sum)."""
+        t = self._shared.get("ones_f32")
+        if t is None or t.numel() < n:
+            t = torch.ones(max(n, 1), dtype=torch.float32, device=self.device)
+            self._shared["ones_f32"] = t
+        return t[:n].view(1, n)
+
+    def build(self, mb: int, x: torch.Tensor, dx_target: Optional[torch.Tensor]) -> MicrobatchProgram:
+        """Lowers every block for microbatch slot ``mb`` with input ``x`` (a real buffer: the
+        previous stage's output slot, or this stage's own input slot on the first stage).
+        ``dx_target`` is the buffer the gradient w.r.t. ``x`` must be written to (the previous
+        stage's output-gradient slot) or None when nobody consumes it."""
+        prog = MicrobatchProgram()
+        b = Builder(self, mb, prog)
+        prog.in_key = (tuple(x.shape), x.dtype, x.data_ptr(), _p(dx_target))
+        prog.input_slot = x
+        h = x
+        for k, blk in enumerate(self.blocks):
+            with b.scope(f"{k}"):
+                h = blk.lower(b, h)
+        prog.output = h
+        if self.training:
+            # gradient of the output, in the (possibly padded) layout of the buffer behind it;
+            # zero-filled once so that padding columns stay zero for every later use
+            out_buf = getattr(h, "_pp_padded", None)
+            if out_buf is None:
+                gbuf = torch.zeros(h.shape, dtype=h.dtype, device=self.device)
+                prog.output_grad = gbuf
+            else:
+                gbuf = torch.zeros(out_buf.shape, dtype=out_buf.dtype, device=self.device)
+                prog.output_grad = _like_view(gbuf, h, out_buf)
+            prog.output_grad_buf = gbuf
+            dy = gbuf
+            fns = b._backward
+            assert len(fns) == len(self.blocks), "every block registers exactly one backward emitter"
+            for idx in reversed(range(len(fns))):
+                first = idx == 0
+                need_dx = (not first) or (dx_target is not None)
+                dy = fns[idx](dy, need_dx, dx_target if first else None)
+            if dx_target is not None:
+                assert dy is not None and dy.data_ptr() == dx_target.data_ptr()
+            prog.input_grad = dy
+            # fold this microbatch's staged parameter gradients into the fp32 accumulators
+            if not self.fused_accumulate and self.arena.staged_total:
+                n = self.arena.staged_total
+                k = prog.W.append(op_accum(self.arena.acc[:n], self.arena.staging[:n], init=False))
+                prog.init_toggle_accum.append(k)
+        prog.F.freeze()
+        prog.I.freeze()
+        prog.W.freeze()
+        self.mbs[mb] = prog
+        return prog
+
+    def set_accumulate_mode(self, prog: MicrobatchProgram, init: bool) -> None:
+        """Patches the W list for the first (init) or a later microbatch of an accumulation."""
+        for k in prog.init_toggle_accum:
+            prog.W[k].j[0] = int(init)
+        for k in prog.init_toggle_beta:
+            prog.W[k].j[4] = 0 if init else 1
+        for k in prog.init_toggle_fill:
+            prog.W[k].flags = 0 if init else OP_SKIP
+
+
+def _like_view(padded_grad: torch.Tensor, out_view: torch.Tensor, padded_out: torch.Tensor) -> torch.Tensor:
+    """The view of ``padded_grad`` that corresponds to ``out_view`` inside ``padded_out``."""
+    off = (out_view.data_ptr() - padded_out.data_ptr()) // out_view.element_size()
+    return torch.as_strided(padded_grad, out_view.shape, out_view.stride(), off)

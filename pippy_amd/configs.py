@@ -1,0 +1,45 @@
+"""Model definitions of the baseline configurations, built from lowerable stage blocks.
+
+These are the shapes the throughput metric is quoted on: random-initialised (std 0.02), no
+checkpoint needed.  Each model is a plain ``nn.Module`` whose ``forward`` applies its children
+in order, so ``pipeline(model, ..., split_spec={"h.3": SplitPoint.BEGINNING, ...})`` cuts it into
+stages that lower to HIP launch lists.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .stage_modules import LMHead, TokenEmbedding, TransformerLayer
+
+
+class DecoderLM(nn.Module):
+    """GPT-2-shaped decoder: token + position embedding, pre-LayerNorm causal transformer layers
+    with tanh-GELU, final LayerNorm and an untied vocabulary projection."""
+
+    def __init__(self, vocab=50257, max_seq=1024, dim=768, n_layers=12, n_heads=12, ffn=3072,
+                 dtype=torch.bfloat16, causal=True, pre_ln=True, activation="gelu_tanh", eps=1e-5):
+        super().__init__()
+        self.embed = TokenEmbedding(vocab, max_seq, dim, dtype=dtype)
+        self.h = nn.ModuleList([
+            TransformerLayer(dim, n_heads, ffn, causal=causal, pre_ln=pre_ln, activation=activation,
+                             eps=eps, dtype=dtype) for _ in range(n_layers)])
+        self.head = LMHead(dim, vocab, final_ln=pre_ln, eps=eps, dtype=dtype)
+
+    def forward(self, ids):
+        x = self.embed(ids)
+        for layer in self.h:
+            x = layer(x)
+        return self.head(x)
+
+
+def gpt2_small(dtype=torch.bfloat16) -> DecoderLM:
+    """12 layers, width 768, 12 heads, FFN 3072, vocabulary 50257, sequence 1024."""
+    return DecoderLM(dtype=dtype)
+
+
+def equal_split_spec(n_layers: int, n_stages: int, prefix: str = "h"):
+    """Split points that give every stage ``n_layers / n_stages`` consecutive layers."""
+    from ._IR import SplitPoint
+    per = n_layers // n_stages
+    return {f"{prefix}.{per * s}": SplitPoint.BEGINNING for s in range(1, n_stages)}

@@ -14,7 +14,7 @@
 // The MFMA is issued with the B fragment as its first operand, so a lane ends up holding, for one
 // output row m, groups of 4 consecutive columns n: stores and epilogue reads are 8-byte vectors.
 #include "tile.h"
-#include <math.h>
+#include "act_math.h"
 
 namespace pp {
 
@@ -30,26 +30,6 @@ struct GemmArgs {
     int beta;
     uint32_t tiles_m, tiles_n, n_blocks;
 };
-
-// ---- epilogue math --------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_erf(float x) {
-    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
-}
-__device__ __forceinline__ float gelu_tanh(float x) {
-    const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(u));
-}
-__device__ __forceinline__ float dgelu_erf(float x) {
-    const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
-    const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
-    return cdf + x * pdf;
-}
-__device__ __forceinline__ float dgelu_tanh(float x) {
-    const float k = 0.79788456080286535588f, c = 0.044715f;
-    const float u = k * (x + c * x * x * x);
-    const float t = tanhf(u);
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * k * (1.0f + 3.0f * c * x * x);
-}
 
 // Applies the epilogue to 4 consecutive columns n0..n0+3 of row m and stores them.
 template <int EPI, bool CF32>

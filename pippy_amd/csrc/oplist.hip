@@ -67,6 +67,8 @@ static int run_one(const pp_op& op, pp_stream st) {
         }
         case PP_OP_FILL:
             return pp_fill_bytes(op.p[0], op.j[0], op.i[0], st);
+        case PP_OP_ACT_BWD:
+            return pp_activation_bwd(op.p[0], op.p[1], op.p[2], op.i[0], op.j[0], op.j[1], st);
         default:
             return fail(PP_ERR_INVALID, "unknown op kind %d", op.kind);
     }
@@ -75,6 +77,7 @@ static int run_one(const pp_op& op, pp_stream st) {
 extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PP_ERR_INVALID, "pp_run_ops: bad list");
     for (int i = 0; i < n_ops; ++i) {
+        if (ops[i].flags & PP_OP_SKIP) continue;
         const int rc = run_one(ops[i], stream);
         if (rc != PP_OK) {
             char msg[400];

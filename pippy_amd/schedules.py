@@ -1,0 +1,281 @@
+"""Pipeline schedules (mirrors ``pippy/PipelineSchedule.py`` of the reference).
+
+Same classes, constructor arguments, ``step`` / ``_step_microbatches`` contract and error types.
+The difference is where stages live: the reference runs one process per pipeline rank and each
+process executes the loop of its own rank; here all stages are virtual stages of one GPU, so a
+schedule builds the per-rank programs from the reference's index formulas
+(``_schedule_order.py``), merges them into one dependency-respecting order and executes that.
+Per-stage forward order and backward order are unchanged (microbatches ascending), hence so are
+all results, including the fp32 gradient accumulation order.
+
+Single-stage schedule classes (``ScheduleGPipe``, ``Schedule1F1B``) accept, besides one stage as
+in the reference, the list of all stages of the pipeline: that is how a multi-stage pipeline is
+run on one device.
+"""
+from __future__ import annotations
+
+import logging
+from abc import ABC, abstractmethod
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+from torch.profiler import record_function
+
+from . import _schedule_order as order
+from .microbatch import merge_chunks, split_args_kwargs_into_chunks
+from .stage import PipelineStageBase, link_stages
+
+logger = logging.getLogger(__name__)
+
+
+class PipelineSchedule(ABC):
+    def __init__(self, n_microbatches: int, loss_fn: Optional[Callable[..., torch.Tensor]] = None,
+                 output_merge_spec: Optional[Union[Dict[str, Any], Tuple[Any]]] = None):
+        self._n_microbatches = n_microbatches
+        self._loss_fn = loss_fn
+        self._output_merge_spec = output_merge_spec
+        self._has_backward = self._loss_fn is not None
+        self._pipe_info = None
+        self._internal_losses: List[torch.Tensor] = []
+        self._stages: List[PipelineStageBase] = []
+        logger.info(f"Using {self.__class__.__name__}")
+
+    # -- losses (reference ``PipelineSchedule.py:39-80``) -------------------------------------------
+    def _maybe_compute_loss(self, stage, output, target_mbs, mb_index):
+        if stage.is_last and self._has_backward:
+            if target_mbs is None:
+                raise RuntimeError("a loss function was given but no target")
+            loss = self._compute_loss(stage, output, target_mbs[mb_index], mb_index)
+            self._internal_losses.append(loss)
+
+    def _maybe_get_loss(self, stage, mb_index):
+        valid_index = 0 <= mb_index < len(self._internal_losses)
+        if stage.is_last and self._has_backward and valid_index:
+            return self._internal_losses[mb_index]
+        elif len(self._internal_losses) != 0 and not valid_index:
+            raise RuntimeError(
+                f"Loss for microbatch {mb_index} is not available. "
+                f"Available losses for microbatches: {self._internal_losses}")
+        else:
+            return None
+
+    def _update_losses(self, stages, losses):
+        if not isinstance(stages, list):
+            stages = [stages]
+        contains_last_stage = any(stage.is_last for stage in stages)
+        if contains_last_stage and losses is not None:
+            if len(self._internal_losses) != self._n_microbatches:
+                raise RuntimeError(
+                    f"Expecting {self._n_microbatches} losses but got {len(self._internal_losses)}")
+            losses.clear()
+            losses.extend(self._internal_losses)
+        self._internal_losses.clear()
+
+    def _compute_loss(self, stage, output, target, mb_index):
+        return stage.compute_loss(self._loss_fn, output, target, mb_index)
+
+    # -- input checks (reference ``PipelineSchedule.py:114-152``) -----------------------------------
+    def _check_inputs(self, arg_mbs=None, kwarg_mbs=None, target_mbs=None, losses=None):
+        def check_type_and_len(mbs, name: str):
+            if not isinstance(mbs, list):
+                raise TypeError(f"{name} must be a list but got a {type(mbs)}")
+            if len(mbs) != self._n_microbatches:
+                raise ValueError(f"Expecting {self._n_microbatches} {name} but got {len(mbs)}")
+
+        if arg_mbs is not None:
+            check_type_and_len(arg_mbs, "arg_mbs")
+        else:
+            arg_mbs = [()] * self._n_microbatches
+        if kwarg_mbs is not None:
+            check_type_and_len(kwarg_mbs, "kwarg_mbs")
+        else:
+            kwarg_mbs = [{}] * self._n_microbatches
+        if target_mbs is not None:
+            check_type_and_len(target_mbs, "target_mbs")
+        if losses is not None and not isinstance(losses, list):
+            raise TypeError(f"losses must be a list but got a {type(losses)}")
+        return arg_mbs, kwarg_mbs
+
+    def _split_inputs(self, args: Tuple[Any, ...], kwargs: Optional[Dict[str, Any]] = None):
+        """Full batch -> microbatches (reference ``PipelineSchedule.py:157-187``)."""
+        if self._pipe_info is not None:
+            args_chunk_spec = self._pipe_info.args_chunk_spec
+            kwargs_chunk_spec = self._pipe_info.kwargs_chunk_spec
+        else:
+            args_chunk_spec = None
+            kwargs_chunk_spec = None
+        if args or kwargs:
+            return split_args_kwargs_into_chunks(args, kwargs, self._n_microbatches, args_chunk_spec,
+                                                 kwargs_chunk_spec)
+        return [()] * self._n_microbatches, [{}] * self._n_microbatches
+
+    def _merge_outputs(self, output_chunks: List[Any]) -> Any:
+        """Microbatch outputs -> full batch (reference ``PipelineSchedule.py:189-197``)."""
+        return merge_chunks(output_chunks, self._output_merge_spec)
+
+    # -- execution of a merged action order on the device -------------------------------------------
+    def _execute(self, actions: Sequence[order.Action], arg_mbs, kwarg_mbs, target_mbs):
+        by_index = {s.stage_index: s for s in self._stages}
+        for kind, s, m in actions:
+            stage = by_index[s]
+            if kind == "F":
+                with record_function(f"Stage {s} Forward {m}"):
+                    if stage.fwd_chunk_id != m:
+                        raise RuntimeError(f"stage {s}: forward order broken ({stage.fwd_chunk_id} != {m})")
+                    a = arg_mbs[m] if stage.is_first else ()
+                    k = kwarg_mbs[m] if stage.is_first else {}
+                    output = stage.forward_one_chunk(a, k)
+                    self._maybe_compute_loss(stage, output, target_mbs, m)
+            elif kind == "B":
+                with record_function(f"Stage {s} Backward {m}"):
+                    if stage.bwd_chunk_id != m:
+                        raise RuntimeError(f"stage {s}: backward order broken ({stage.bwd_chunk_id} != {m})")
+                    stage.backward_one_chunk(loss=self._maybe_get_loss(stage, m))
+            elif kind == "I":
+                with record_function(f"Stage {s} BackwardInput {m}"):
+                    stage.backward_input_one_chunk(loss=self._maybe_get_loss(stage, m))
+            elif kind == "W":
+                with record_function(f"Stage {s} BackwardWeight {m}"):
+                    stage.backward_weight_one_chunk()
+            else:
+                raise ValueError(f"unknown action {kind}")
+
+    @abstractmethod
+    def _rank_programs(self) -> List[List[order.Action]]:
+        """One action program per virtual pipeline rank."""
+
+    def _step_microbatches(self, arg_mbs: Optional[List] = None, kwarg_mbs: Optional[List] = None,
+                           target_mbs: Optional[List] = None, losses: Optional[List] = None):
+        """Runs one iteration over lists of microbatches (reference ``PipelineSchedule.py:83-98``)."""
+        arg_mbs, kwarg_mbs = self._check_inputs(arg_mbs, kwarg_mbs, target_mbs, losses)
+        num_stages = self._stages[0].num_stages
+        present = sorted(s.stage_index for s in self._stages)
+        if present != list(range(num_stages)):
+            raise RuntimeError(
+                f"this schedule holds stages {present} of a {num_stages}-stage pipeline; all stages "
+                "run as virtual stages on one device, so every stage must be given to the schedule "
+                "(there is no inter-process transport)")
+        actions = order.merge_rank_programs(self._rank_programs(), num_stages)
+        self._execute(actions, arg_mbs, kwarg_mbs, target_mbs)
+        self._update_losses(self._stages, losses)
+
+    def step(self, *args, target=None, losses: Optional[List] = None, **kwargs):
+        """Runs one iteration on a whole batch: split, run the microbatches, merge
+        (reference ``PipelineSchedule.py:254-276,490-514``)."""
+        for stage in self._stages:
+            stage.clear_runtime_states()
+        args_split, kwargs_split = self._split_inputs(args, kwargs)
+        if target is not None:
+            targets_split = list(torch.tensor_split(target, self._n_microbatches))
+        else:
+            targets_split = None
+        self._step_microbatches(args_split, kwargs_split, targets_split, losses)
+        for stage in self._stages:
+            if stage.is_last:
+                return self._merge_outputs(stage.output_chunks)
+        return None
+
+    def zero_grad(self):
+        for stage in self._stages:
+            stage.zero_grad()
+
+    def _adopt_stages(self, stages: List[PipelineStageBase]):
+        self._stages = link_stages(stages)
+        self._num_stages = self._stages[0].num_stages
+        self._pipe_info = getattr(self._stages[0], "pipe_info", None)
+        for stage in self._stages:
+            stage.has_backward = self._has_backward
+
+
+class PipelineScheduleSingle(PipelineSchedule):
+    """Schedules whose ranks own one stage each (reference ``PipelineSchedule.py:225-276``)."""
+
+    def __init__(self, stage: Union[PipelineStageBase, List[PipelineStageBase]], n_microbatches: int,
+                 loss_fn: Optional[Callable] = None,
+                 output_merge_spec: Optional[Union[Dict[str, Any], Tuple[Any]]] = None):
+        super().__init__(n_microbatches=n_microbatches, loss_fn=loss_fn, output_merge_spec=output_merge_spec)
+        stages = list(stage) if isinstance(stage, (list, tuple)) else [stage]
+        self._adopt_stages(stages)
+        self._stage = self._stages[0]
+
+
+class ScheduleGPipe(PipelineScheduleSingle):
+    """All forwards, then all backwards (reference ``PipelineSchedule.py:279-355``)."""
+
+    def _rank_programs(self):
+        return [order.gpipe_rank_program(s.stage_index, self._n_microbatches, self._has_backward)
+                for s in self._stages]
+
+
+class Schedule1F1B(PipelineScheduleSingle):
+    """One-forward-one-backward (reference ``PipelineSchedule.py:358-449``)."""
+
+    def _rank_programs(self):
+        return [order.one_f_one_b_rank_program(s.stage_index, self._num_stages, self._n_microbatches,
+                                               self._has_backward) for s in self._stages]
+
+
+class ScheduleZeroBubble(PipelineScheduleSingle):
+    """1F1B with the backward split into an input-gradient and a deferred weight-gradient pass.
+    Not part of the reference (its backward is one fused autograd call); needs native stages."""
+
+    def __init__(self, stage, n_microbatches, loss_fn=None, output_merge_spec=None):
+        super().__init__(stage, n_microbatches, loss_fn, output_merge_spec)
+        if not self._has_backward:
+            raise ValueError("a zero-bubble schedule needs a loss function")
+        for s in self._stages:
+            if not s.is_native:
+                raise RuntimeError("zero-bubble needs stages that lower to native input/weight passes")
+            s.split_backward = True
+
+    def _rank_programs(self):
+        return [order.zero_bubble_rank_program(s.stage_index, self._num_stages, self._n_microbatches)
+                for s in self._stages]
+
+
+class PipelineScheduleMulti(PipelineSchedule):
+    """Schedules whose ranks own several stages (reference ``PipelineSchedule.py:452-514``)."""
+
+    def __init__(self, stages: List[PipelineStageBase], n_microbatches: int,
+                 loss_fn: Optional[Callable] = None,
+                 output_merge_spec: Optional[Union[Dict[str, Any], Tuple[Any]]] = None):
+        if len(stages) <= 1:
+            raise ValueError(f"Multi-stage schedule expects at least two stages but got {len(stages)}")
+        super().__init__(n_microbatches=n_microbatches, loss_fn=loss_fn, output_merge_spec=output_merge_spec)
+        self._adopt_stages(list(stages))
+        self.pp_group_size = self._stages[0].group_size
+
+    def _local_stages(self, rank: int) -> List[int]:
+        return [s.stage_index for s in self._stages if s.group_rank == rank]
+
+
+class ScheduleLoopedBFS(PipelineScheduleMulti):
+    """Breadth-first over the local stages (reference ``PipelineSchedule.py:517-569``)."""
+
+    def _rank_programs(self):
+        return [order.looped_bfs_rank_program(self._local_stages(r), self._n_microbatches, self._has_backward)
+                for r in range(self.pp_group_size)]
+
+
+class ScheduleInterleaved1F1B(PipelineScheduleMulti):
+    """Interleaved 1F1B (reference ``PipelineSchedule.py:572-778``)."""
+
+    def __init__(self, stages: List[PipelineStageBase], n_microbatches: int,
+                 loss_fn: Optional[Callable] = None,
+                 output_merge_spec: Optional[Union[Dict[str, Any], Tuple[Any]]] = None):
+        if len(stages) > 0:
+            group_size = stages[0].group_size
+            if n_microbatches % group_size != 0:
+                raise ValueError(
+                    "Interleaved 1F1B requires the number of microbatches to be a "
+                    f"multiple of the number of pipeline ranks ({group_size}), "
+                    f"but got {n_microbatches}.")
+        super().__init__(stages=stages, n_microbatches=n_microbatches, loss_fn=loss_fn,
+                         output_merge_spec=output_merge_spec)
+        self.n_local_stages = len(self._local_stages(0))
+        self.rank = 0
+
+    def _rank_programs(self):
+        return [order.interleaved_rank_program(r, self.pp_group_size, self._local_stages(r),
+                                               self._n_microbatches, self._has_backward)
+                for r in range(self.pp_group_size)]

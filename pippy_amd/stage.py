@@ -1,0 +1,480 @@
+"""Pipeline stage runtime (mirrors ``pippy/_PipelineStage.py`` and ``pippy/ManualPipelineStage.py``).
+
+Every stage of the pipeline is a *virtual* stage on one GPU.  The reference moves a microbatch's
+activation from stage s to stage s+1 (and its gradient back) with ``dist.P2POp`` send/recv pairs
+into per-microbatch receive buffers (``_PipelineStage.py:210-341``); here the producer's output
+slot *is* the consumer's input, and the consumer's input-gradient pass writes straight into the
+producer's output-gradient slot: the hand-off is a pointer, no bytes move.
+
+Two execution modes per stage:
+
+* native: the stage module lowers to HIP launch lists (``_program.py``); forward, input-gradient
+  and weight-gradient passes are separate entry points and parameter gradients are accumulated in
+  fp32 by the accumulate kernel (or by the dW GEMM epilogue when ``fused_accumulate`` is set);
+* eager: any other ``nn.Module`` runs through torch autograd on the GPU exactly as the reference
+  does (``forward_one_chunk`` / ``stage_backward``), with the same caching rules.
+"""
+from __future__ import annotations
+
+import logging
+from typing import Any, Dict, List, Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+
+from . import _native as N
+from . import _program as P
+from ._backward import stage_backward
+from ._lowering import lower_stage_module
+from ._utils import flatten_args
+from .losses import as_native_loss
+
+logger = logging.getLogger(__name__)
+
+
+class VirtualGroup:
+    """Stands in for the reference's process group: ``size`` virtual pipeline ranks that all live
+    in this process.  ``stage_index % size`` is a stage's rank (wrap-around placement,
+    ``_PipelineStage.py:129-136``)."""
+
+    def __init__(self, size: int):
+        if size < 1:
+            raise ValueError("a virtual group needs at least one rank")
+        self._size = size
+
+    def size(self) -> int:
+        return self._size
+
+
+def _group_size(group) -> int:
+    if group is None:
+        return 1
+    if isinstance(group, int):
+        return group
+    if isinstance(group, VirtualGroup):
+        return group.size()
+    try:  # a real torch.distributed group of this (single) process
+        import torch.distributed as dist
+        return dist.get_world_size(group)
+    except Exception as e:  # pragma: no cover
+        raise TypeError(f"unsupported group object {group!r}") from e
+
+
+class PipelineStageBase:
+    """State and per-microbatch entry points shared by ``PipelineStage`` and
+    ``ManualPipelineStage`` (reference ``_PipelineStage.py:72-551``)."""
+
+    def __init__(self, submodule: nn.Module, stage_index: int, num_stages: int,
+                 device: Union[torch.device, str], num_microbatches: int, group=None, *,
+                 fused_accumulate: bool = False, force_eager: bool = False):
+        if stage_index >= num_stages:
+            raise ValueError(f"Stage index {stage_index} is out of range of {num_stages}")
+        self.submod = submodule
+        self.stage_index = stage_index
+        self.num_stages = num_stages
+        self.device = torch.device(device)
+        self.chunks = num_microbatches
+        self.group = group
+        self.group_size = _group_size(group)
+        self.group_rank = stage_index % self.group_size
+        if self.group_size > self.num_stages:
+            raise RuntimeError(
+                f"Pipeline group size {self.group_size} cannot be larger than number of stages {self.num_stages}")
+        self.stage_index_to_group_rank = {i: i % self.group_size for i in range(num_stages)}
+
+        # run-time state (reference names)
+        self.fwd_cache: Dict[int, Tuple[Any, List[torch.Tensor]]] = {}
+        self.fwd_chunk_id = 0
+        self.bwd_chunk_id = 0
+        self.bwd_weight_chunk_id = 0
+        self.output_chunks: List[Any] = []
+        self.grads_input: List[Optional[torch.Tensor]] = []
+        self._has_backward = False
+        self.log_prefix = f"[Stage {self.stage_index}]"
+
+        # neighbours on the device; set by the schedule
+        self._prev: Optional["PipelineStageBase"] = None
+        self._next: Optional["PipelineStageBase"] = None
+        self._fwd_done: Dict[int, bool] = {}
+        self._bwd_done: Dict[int, bool] = {}
+        self._input_grads: Dict[int, List[Optional[torch.Tensor]]] = {}  # eager hand-off
+        self._bridge: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}  # generic loss on a native stage
+
+        self.fused_accumulate = fused_accumulate
+        self.split_backward = False
+        self._blocks = None if force_eager else lower_stage_module(submodule)
+        self._program: Optional[P.StageProgram] = None
+        if self._blocks is None:
+            self.submod.to(self.device)
+
+    # -- reference properties -----------------------------------------------------------------
+    @property
+    def has_backward(self) -> bool:
+        return self._has_backward
+
+    @has_backward.setter
+    def has_backward(self, has_backward: bool):
+        self._has_backward = has_backward
+
+    @property
+    def is_first(self):
+        return self.stage_index == 0
+
+    @property
+    def is_last(self):
+        return self.stage_index == self.num_stages - 1
+
+    @property
+    def is_native(self) -> bool:
+        return self._blocks is not None
+
+    # The reference's schedules ask a stage for P2P op lists around every forward / backward.
+    # With device-local hand-off there is nothing to post; the methods remain for API parity.
+    def get_fwd_recv_ops(self):
+        return []
+
+    def get_bwd_recv_ops(self):
+        return []
+
+    def get_fwd_send_ops(self):
+        return []
+
+    def get_bwd_send_ops(self):
+        return []
+
+    def _configure_data_parallel_mode(self, last_backward: bool):
+        """No data-parallel wrapper exists on one GPU (reference ``_PipelineStage.py:409-418``)."""
+
+    def clear_runtime_states(self) -> None:
+        """Resets per-step state (reference ``_PipelineStage.py:343-366``)."""
+        self.fwd_chunk_id = 0
+        self.bwd_chunk_id = 0
+        self.bwd_weight_chunk_id = 0
+        self.fwd_cache.clear()
+        self.output_chunks.clear()
+        self._fwd_done.clear()
+        self._bwd_done.clear()
+        self._input_grads.clear()
+        self._bridge.clear()
+
+    # -- program management ---------------------------------------------------------------------
+    def _stage_program(self) -> P.StageProgram:
+        if self._program is None:
+            self._program = P.StageProgram(self._blocks, self.submod, self.device,
+                                           training=self.has_backward,
+                                           split_backward=self.split_backward,
+                                           fused_accumulate=self.fused_accumulate,
+                                           is_first=self.is_first, is_last=self.is_last)
+            self._publish_grad_views()
+        elif self._program.training != self.has_backward or \
+                self._program.split_backward != self.split_backward:
+            # the schedule changed between steps (e.g. inference after training): re-lower
+            self._program.training = self.has_backward
+            self._program.split_backward = self.split_backward
+            self._program.mbs.clear()
+        return self._program
+
+    def _publish_grad_views(self):
+        """fp32 parameters get their accumulator as ``.grad``; bf16 parameters expose it as
+        ``.main_grad`` (torch does not allow an fp32 ``.grad`` on a bf16 parameter)."""
+        arena = self._program.arena
+        for _, p in arena.named:
+            view = arena.grad_acc(p, padded=False)
+            p.main_grad = view
+
+    def zero_grad(self):
+        """Forget accumulated parameter gradients: the next weight-gradient pass overwrites the
+        fp32 accumulators instead of adding to them."""
+        if self._program is not None:
+            self._program.acc_initialized = False
+        for p in self.submod.parameters():
+            p.grad = None
+
+    def materialize_grads(self):
+        """Sets ``param.grad`` from the fp32 accumulators (cast to the parameter dtype) so that a
+        stock torch optimizer can step; fp32 parameters share memory with the accumulator."""
+        if self._program is None:
+            return
+        for _, p in self._program.arena.named:
+            p.grad = p.main_grad if p.dtype == torch.float32 else p.main_grad.to(p.dtype)
+
+    def _input_for(self, mb: int, args, kwargs):
+        """(x, dx_target, patch_input) of microbatch ``mb`` for a native stage."""
+        if self.is_first:
+            if kwargs:
+                raise RuntimeError(f"{self.log_prefix} native stages take positional tensor inputs only")
+            tensors = [a for a in args if isinstance(a, torch.Tensor)]
+            if len(tensors) != 1 or len(args) != 1:
+                raise RuntimeError(
+                    f"{self.log_prefix} a native stage takes exactly one tensor input, got {len(args)} args")
+            x = tensors[0]
+            if not x.is_cuda:
+                raise RuntimeError(f"{self.log_prefix} input is on {x.device}; move it to {self.device}")
+            return x, None, True
+        prev = self._prev
+        if prev is None:
+            raise RuntimeError(
+                f"{self.log_prefix} is not linked to stage {self.stage_index - 1}: pass every stage of "
+                "the pipeline to the schedule (all stages are virtual stages of this process)")
+        if not prev._fwd_done.get(mb):
+            raise RuntimeError(f"{self.log_prefix} activation of microbatch {mb} has not been produced")
+        if prev.is_native:
+            pprog = prev._program.mbs[mb]
+            x = pprog.output
+            dx = getattr(pprog, "output_grad_buf", None) if self.has_backward else None
+            if x.dim() and not x.is_contiguous():
+                raise RuntimeError(f"{self.log_prefix} received a non-contiguous activation")
+            return x, dx, False
+        out = prev.output_chunks[mb]
+        if not isinstance(out, torch.Tensor):
+            raise RuntimeError(f"{self.log_prefix} native stages take a single tensor from the previous stage")
+        x = out.detach().contiguous()
+        dx = torch.zeros_like(x) if self.has_backward else None
+        self._input_grads[mb] = [dx]
+        return x, dx, False
+
+    # -- forward ----------------------------------------------------------------------------------
+    def forward_one_chunk(self, args: Tuple[Any, ...] = (), kwargs: Optional[Dict[str, Any]] = None):
+        """Forward of the next microbatch (reference ``_PipelineStage.py:452-510``)."""
+        mb = self.fwd_chunk_id
+        try:
+            if self.is_native:
+                output, flat_inputs = self._forward_native(mb, args, kwargs or {})
+            else:
+                output, flat_inputs = self._forward_eager(mb, args, kwargs or {})
+        except Exception as e:
+            raise RuntimeError(f"{self.log_prefix} failed to run forward of microbatch {mb}: {e}") from e
+        if type(output) is list:
+            output = tuple(output)
+        output_tuple = output if type(output) is tuple else (output,)
+        self.output_chunks.append(output)
+        self.fwd_cache[mb] = (output_tuple, flat_inputs)
+        self._fwd_done[mb] = True
+        self.fwd_chunk_id += 1
+        return output
+
+    def _forward_native(self, mb, args, kwargs):
+        sp = self._stage_program()
+        x, dx_target, patch = self._input_for(mb, args, kwargs)
+        prog = sp.mbs.get(mb)
+        if patch:
+            if not x.is_contiguous() or (x.data_ptr() % 16):
+                xc = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+                N.strided_copy_nd(xc, x)
+                x = xc
+            key = (tuple(x.shape), x.dtype)
+            if prog is None or prog.in_key[:2] != key:
+                slot = torch.empty(x.shape, dtype=x.dtype, device=self.device)
+                prog = sp.build(mb, slot, None)
+                prog.input_patches = [(lst, k, q) for lst in (prog.F, prog.I, prog.W)
+                                      for (k, q) in lst.find_pointer(slot.data_ptr())]
+            for lst, k, q in prog.input_patches:
+                lst[k].p[q] = x.data_ptr()
+        else:
+            key = (tuple(x.shape), x.dtype, x.data_ptr(), P._p(dx_target))
+            if prog is None or prog.in_key != key:
+                prog = sp.build(mb, x, dx_target)
+        prog.F.run()
+        return prog.output, [x]
+
+    def _forward_eager(self, mb, args, kwargs):
+        if self.is_first:
+            composite_args, composite_kwargs = args, kwargs
+        else:
+            prev = self._prev
+            if prev is None:
+                raise RuntimeError(
+                    f"{self.log_prefix} is not linked to stage {self.stage_index - 1}: pass every stage "
+                    "of the pipeline to the schedule")
+            if not prev._fwd_done.get(mb):
+                raise RuntimeError(f"{self.log_prefix} activation of microbatch {mb} has not been produced")
+            out = prev.output_chunks[mb]
+            outs = out if isinstance(out, tuple) else (out,)
+            recv = []
+            for o in outs:
+                if isinstance(o, torch.Tensor):
+                    o = o.detach()
+                    if self.has_backward and o.is_floating_point():
+                        o = o.requires_grad_(True)
+                recv.append(o)
+            composite_args, composite_kwargs = tuple(recv), {}
+        output = self.submod(*composite_args, **composite_kwargs)
+        flat_inputs = flatten_args(composite_args) + flatten_args(composite_kwargs)
+        return output, flat_inputs
+
+    # -- loss ---------------------------------------------------------------------------------------
+    def compute_loss(self, loss_fn, output, target, mb: int) -> torch.Tensor:
+        """Runs ``loss_fn`` for microbatch ``mb`` of the last stage
+        (reference ``PipelineSchedule.py:39-45``)."""
+        if not self.is_native:
+            return loss_fn(output, target)
+        prog = self._program.mbs[mb]
+        native = as_native_loss(loss_fn)
+        logits = getattr(prog.output, "_pp_padded", None)
+        if native is not None and (not getattr(native, "_requires_2d", False) or output.dim() == 2):
+            V = output.shape[-1]
+            if logits is None:
+                logits = prog.output.reshape(-1, V)
+            rows = logits.shape[0]
+            if target.numel() != rows or target.dtype != torch.int64:
+                raise RuntimeError(
+                    f"cross entropy expects {rows} int64 targets, got {target.numel()} of {target.dtype}")
+            if not target.is_contiguous():
+                tc = torch.empty(target.shape, dtype=target.dtype, device=target.device)
+                N.strided_copy_nd(tc, target)
+                target = tc
+            entry = prog.loss_ops.get(id(loss_fn))
+            if entry is None:
+                loss = torch.empty(1, dtype=torch.float32, device=self.device)
+                ws = torch.empty(rows + 2, dtype=torch.float32, device=self.device)
+                dl = prog.output_grad_buf.view(logits.shape) if self.has_backward else None
+                lst = P.OpList()
+                lst.append(P.op_ce_loss(logits, target, loss, dl, ws, V, native.ignore_index))
+                lst.freeze()
+                entry = (lst, loss, ws)
+                prog.loss_ops[id(loss_fn)] = entry
+            lst, loss, _ = entry
+            lst[0].p[1] = target.data_ptr()
+            lst.run()
+            self._loss_targets = getattr(self, "_loss_targets", {})
+            self._loss_targets[mb] = target  # keep alive until the kernel has run
+            return loss.view(())
+        # any other callable: autograd on a detached copy of the output
+        leaf = output.detach().requires_grad_(self.has_backward)
+        loss = loss_fn(leaf, target)
+        self._bridge[mb] = (leaf, loss)
+        return loss
+
+    # -- backward -----------------------------------------------------------------------------------
+    def backward_one_chunk(self, loss=None):
+        """Full backward of the next microbatch (reference ``_PipelineStage.py:512-550``):
+        input-gradient pass followed by the weight-gradient pass."""
+        mb = self.bwd_chunk_id
+        if self.is_native:
+            self._backward_input_native(mb, loss)
+            self.bwd_chunk_id += 1
+            self._backward_weight_native(mb)
+            self.bwd_weight_chunk_id += 1
+        else:
+            self._backward_eager(mb, loss)
+            self.bwd_chunk_id += 1
+            self.bwd_weight_chunk_id += 1
+
+    def backward_input_one_chunk(self, loss=None):
+        """Input-gradient pass only (dI): produces the gradient the previous stage waits for and
+        keeps what the weight-gradient pass needs."""
+        if not self.is_native:
+            raise RuntimeError("split backward needs a native stage")
+        if not self.split_backward:
+            raise RuntimeError("enable split_backward (zero-bubble schedules do) before the first forward")
+        mb = self.bwd_chunk_id
+        self._backward_input_native(mb, loss)
+        self.bwd_chunk_id += 1
+
+    def backward_weight_one_chunk(self):
+        """Weight-gradient pass (dW) of the oldest microbatch whose input-gradient pass has run."""
+        if not self.is_native:
+            raise RuntimeError("split backward needs a native stage")
+        mb = self.bwd_weight_chunk_id
+        if mb >= self.bwd_chunk_id:
+            raise RuntimeError(f"{self.log_prefix} weight-gradient pass of microbatch {mb} before its input-gradient pass")
+        self._backward_weight_native(mb)
+        self.bwd_weight_chunk_id += 1
+
+    def _backward_input_native(self, mb, loss):
+        if mb not in self.fwd_cache:
+            raise RuntimeError(f"{self.log_prefix} backward of microbatch {mb} before its forward")
+        self.fwd_cache.pop(mb)
+        prog = self._program.mbs[mb]
+        if self.is_last:
+            if mb in self._bridge:
+                leaf, lss = self._bridge.pop(mb)
+                lss.backward()
+                prog.output_grad.copy_(leaf.grad)
+            elif loss is None:
+                raise RuntimeError(f"{self.log_prefix} last stage needs the loss of microbatch {mb}")
+        else:
+            nxt = self._next
+            if nxt is None or not nxt._bwd_done.get(mb):
+                raise RuntimeError(f"{self.log_prefix} gradient of microbatch {mb} has not been produced")
+            if not nxt.is_native:
+                g = nxt._input_grads[mb][0]
+                prog.output_grad.copy_(g)
+        prog.I.run()
+        self._bwd_done[mb] = True
+        self.grads_input = [prog.input_grad]
+
+    def _backward_weight_native(self, mb):
+        sp = self._program
+        prog = sp.mbs[mb]
+        fp32_params = sp.arena.dtype == torch.float32
+        if fp32_params and sp.acc_initialized and any(p.grad is None for _, p in sp.arena.named):
+            # the user cleared the gradients (optimizer.zero_grad()): start a new accumulation
+            sp.acc_initialized = False
+        sp.set_accumulate_mode(prog, init=not sp.acc_initialized)
+        prog.W.run()
+        sp.acc_initialized = True
+        if fp32_params:
+            for _, p in sp.arena.named:
+                if p.grad is None:
+                    p.grad = p.main_grad
+
+    def _backward_eager(self, mb, loss):
+        stage_output, input_values = self.fwd_cache.pop(mb)
+        if self.is_last:
+            bwd_kwargs = {"stage_output": loss, "output_grads": None, "input_values": input_values}
+        else:
+            nxt = self._next
+            if nxt is None or not nxt._bwd_done.get(mb):
+                raise RuntimeError(f"{self.log_prefix} gradient of microbatch {mb} has not been produced")
+            if nxt.is_native:
+                grads = (nxt._program.mbs[mb].input_grad,)
+            else:
+                grads = tuple(nxt._input_grads[mb])
+            bwd_kwargs = {"stage_output": stage_output, "output_grads": grads, "input_values": input_values}
+        self.grads_input = stage_backward(**bwd_kwargs)
+        self._input_grads[mb] = list(self.grads_input)
+        self._bwd_done[mb] = True
+
+
+class PipelineStage(PipelineStageBase):
+    """A stage built from a ``Pipe`` (reference ``_PipelineStage.py:818-833``)."""
+
+    def __init__(self, pipe, stage_index: int, device, group=None, **kw):
+        self.pipe = pipe
+        self.pipe_info = pipe.info()
+        submod = pipe.get_stage_module(stage_index)
+        super().__init__(submod, stage_index, pipe.num_stages, device, self.pipe_info.num_chunks,
+                         group, **kw)
+
+
+class ManualPipelineStage(PipelineStageBase):
+    """A stage built from a hand-written module (reference ``ManualPipelineStage.py:178-307``).
+    ``input_args`` / ``output_args`` are example microbatch values; the reference uses them to size
+    its receive buffers and to exchange shapes between ranks.  Here shapes are taken from the live
+    tensors, so the examples are only checked for consistency."""
+
+    def __init__(self, submodule: nn.Module, stage_index: int, num_stages: int, device,
+                 num_microbatches: int, input_args=None, output_args=None, group=None, **kw):
+        super().__init__(submodule, stage_index, num_stages, device, num_microbatches, group, **kw)
+        self.inputs = _to_tuple(input_args)
+        self.outputs = _to_tuple(output_args)
+
+
+def _to_tuple(v):
+    if v is None:
+        return ()
+    return tuple(v) if isinstance(v, (tuple, list)) else (v,)
+
+
+def link_stages(stages: List[PipelineStageBase]) -> List[PipelineStageBase]:
+    """Wires the device-local hand-off between consecutive stages and returns them sorted."""
+    ordered = sorted(stages, key=lambda s: s.stage_index)
+    idx = [s.stage_index for s in ordered]
+    if len(set(idx)) != len(idx):
+        raise ValueError(f"duplicate stage indices {idx}")
+    by_index = {s.stage_index: s for s in ordered}
+    for s in ordered:
+        s._prev = by_index.get(s.stage_index - 1)
+        s._next = by_index.get(s.stage_index + 1)
+    return ordered

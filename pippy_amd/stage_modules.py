@@ -1,0 +1,425 @@
+"""Stage building blocks that lower to HIP launch lists.
+
+Each block is an ordinary ``nn.Module``: its ``forward`` is the torch statement of what it
+computes (used for tracing, for un-pipelined comparison runs and by the CPU oracle), and its
+``lower`` emits the kernels that compute the same thing on the GPU for one microbatch slot,
+registering one backward emitter that produces the input-gradient (I) and weight-gradient (W)
+ops.  These are the modules the reference would run through ``submod(*args)``
+(``pippy/_PipelineStage.py:420-428``) and differentiate with ``torch.autograd.backward``
+(``pippy/_backward.py:67-69``).
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _native as N
+from . import _program as P
+
+
+class NativeBlock(nn.Module):
+    """Base class of lowerable blocks."""
+
+    def lower(self, b: "P.Builder", x: torch.Tensor) -> torch.Tensor:  # pragma: no cover
+        raise NotImplementedError
+
+    def _pp_padded_rows(self) -> List[Tuple[nn.Parameter, int]]:
+        """(parameter, padded leading size) pairs for parameters stored with padding."""
+        return []
+
+    def _pp_direct_acc_params(self) -> List[nn.Parameter]:
+        """Parameters whose gradient is added straight into the fp32 accumulator."""
+        return []
+
+
+def _as2d(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape(-1, t.shape[-1])
+
+
+# ---- lowering helpers for standard layers ------------------------------------------------------
+def lower_linear(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, *, epilogue=N.EPI_BIAS,
+                 aux_in=None, save_pre=False, out: Optional[torch.Tensor] = None):
+    """y = epilogue(x W^T + bias).  Returns (y, pre_activation or None)."""
+    W = b.weight(lin.weight)
+    bias = b.weight(lin.bias) if lin.bias is not None else None
+    T = x2d.shape[0]
+    y = out if out is not None else b.act(name, (T, W.shape[0]))
+    pre = b.act(name + ".pre", (T, W.shape[0])) if save_pre else None
+    if bias is None and epilogue == N.EPI_BIAS:
+        epilogue = N.EPI_NONE
+    b.f(P.op_gemm(x2d, W, y, epilogue=epilogue, bias=bias, aux_in=aux_in, aux_out=pre))
+    return y, pre
+
+
+def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
+    """db = column sum of dY (W pass)."""
+    if lin.bias is None:
+        return
+    if dY2d.dtype == torch.float32:
+        # fp32 stages are small: ones[1, T] @ dY through the fp32 GEMM is an ordered column sum
+        ones = b.sp.ones_f32(dY2d.shape[0])
+        if b.fused_accumulate:
+            k = b.w(P.op_gemm(ones, dY2d, b.grad_acc(lin.bias).view(1, -1), b_trans=True,
+                              epilogue=N.EPI_ACCUM_F32, beta=1))
+            b.prog.init_toggle_beta.append(k)
+        else:
+            b.w(P.op_gemm(ones, dY2d, b.grad_target(lin.bias).view(1, -1), b_trans=True))
+        return
+    M, Nn = dY2d.shape
+    ws = b.scratch("colsum", (((M + 127) // 128) * Nn,), torch.float32)
+    if b.fused_accumulate:
+        tmp = b.scratch("colsum_out", (Nn,), torch.float32)
+        b.w(P.op_colsum(dY2d, tmp, ws))
+        b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(lin.bias), tmp)))
+    else:
+        b.w(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
+
+
+def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, dY2d: torch.Tensor, *,
+                    need_dx=True, dx_out=None, dx_epilogue=N.EPI_NONE, dx_aux=None, padded=True):
+    """I: dX = epilogue(dY W); W: dW = dY^T X, db = colsum(dY)."""
+    W = b.weight(lin.weight, padded)
+    dx = None
+    if need_dx:
+        dx = dx_out if dx_out is not None else b.grad(name + ".dx", (dY2d.shape[0], W.shape[1]))
+        b.i(P.op_gemm(dY2d, W, dx, b_trans=True, epilogue=dx_epilogue, aux_in=dx_aux))
+    b.w_weight_gemm(dY2d, x2d, lin.weight, padded)
+    bias_grad(b, lin, dY2d)
+    return dx
+
+
+def lower_layernorm(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d: torch.Tensor):
+    T, Cc = x2d.shape
+    y = b.act(name, (T, Cc))
+    mean = b.act(name + ".mean", (T,), torch.float32)
+    rstd = b.act(name + ".rstd", (T,), torch.float32)
+    b.f(P.op_ln_fwd(x2d, b.weight(ln.weight), b.weight(ln.bias) if ln.bias is not None else None, y,
+                    mean, rstd, ln.eps))
+    return y, mean, rstd
+
+
+def layernorm_backward(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d, mean, rstd, dy2d, dres=None,
+                       dx_out=None):
+    """I: dx = LN'(dy) + dres; W: dgamma, dbeta."""
+    T, Cc = x2d.shape
+    dx = dx_out if dx_out is not None else b.grad(name + ".dx", (T, Cc))
+    b.i(P.op_ln_bwd_input(dy2d, x2d, b.weight(ln.weight), mean, rstd, dres, dx))
+    ws = b.scratch("ln_bwd", (2 * ((T + 127) // 128) * Cc,), torch.float32)
+    has_bias = ln.bias is not None
+    if b.fused_accumulate:
+        dg = b.scratch("ln_dg", (Cc,), torch.float32)
+        db = b.scratch("ln_db", (Cc,), torch.float32)
+        b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, dg, db if has_bias else None, ws))
+        b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(ln.weight), dg)))
+        if has_bias:
+            b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(ln.bias), db)))
+    else:
+        b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
+                               b.grad_target(ln.bias) if has_bias else None, ws))
+    return dx
+
+
+_ACT_EPI = {None: N.EPI_BIAS, "relu": N.EPI_BIAS_RELU, "gelu_erf": N.EPI_BIAS_GELU_ERF,
+            "gelu_tanh": N.EPI_BIAS_GELU_TANH}
+_ACT_DEPI = {"gelu_erf": N.EPI_DGELU_ERF, "gelu_tanh": N.EPI_DGELU_TANH}
+_ACT_KIND = {"relu": N.ACT_RELU, "gelu_erf": N.ACT_GELU_ERF, "gelu_tanh": N.ACT_GELU_TANH}
+
+
+def _torch_act(y, activation):
+    if activation == "relu":
+        return torch.relu(y)
+    if activation == "gelu_erf":
+        return F.gelu(y)
+    if activation == "gelu_tanh":
+        return F.gelu(y, approximate="tanh")
+    return y
+
+
+# ---- blocks ---------------------------------------------------------------------------------------
+class LinearAct(NativeBlock):
+    """``activation(linear(x))`` around a standard ``nn.Linear`` (activation: None, "relu",
+    "gelu_erf", "gelu_tanh").  The stage lowering builds it from an ``nn.Linear`` followed by an
+    activation; it wraps the original module, so parameter names stay those of the user's model."""
+
+    def __init__(self, lin: nn.Linear, activation: Optional[str] = None):
+        super().__init__()
+        assert activation in _ACT_EPI
+        self.lin = lin
+        self.activation = activation
+
+    def forward(self, x):
+        return _torch_act(self.lin(x), self.activation)
+
+    def lower(self, b, x):
+        x2d = _as2d(x)
+        act = self.activation
+        save_pre = b.training and act in ("gelu_erf", "gelu_tanh")
+        y, pre = lower_linear(b, "y", self.lin, x2d, epilogue=_ACT_EPI[act], save_pre=save_pre)
+        out = y.view(x.shape[:-1] + (y.shape[-1],))
+
+        def bwd(dy, need_dx, dx_out):
+            dy2d = _as2d(dy)
+            if act is not None:
+                dz = b.grad("dz", dy2d.shape, dy2d.dtype)
+                # relu' can be read off the output; gelu' needs the pre-activation
+                b.i(P.op_act_bwd(dy2d, y if act == "relu" else pre, dz, _ACT_KIND[act]))
+                dy2d = dz
+            dx = linear_backward(b, "lin", self.lin, x2d, dy2d, need_dx=need_dx,
+                                 dx_out=_as2d(dx_out) if dx_out is not None else None)
+            return None if dx is None else dx.view(x.shape)
+
+        b.on_backward(bwd)
+        return out
+
+
+class LayerNormBlock(NativeBlock):
+    """A stand-alone ``nn.LayerNorm`` over the last dimension."""
+
+    def __init__(self, ln: nn.LayerNorm):
+        super().__init__()
+        self.ln = ln
+
+    def forward(self, x):
+        return self.ln(x)
+
+    def lower(self, b, x):
+        x2d = _as2d(x)
+        y, mean, rstd = lower_layernorm(b, "y", self.ln, x2d)
+
+        def bwd(dy, need_dx, dx_out):
+            dx = layernorm_backward(b, "ln", self.ln, x2d, mean, rstd, _as2d(dy),
+                                    dx_out=_as2d(dx_out) if dx_out is not None else None)
+            return dx.view(x.shape)
+
+        b.on_backward(bwd)
+        return y.view(x.shape)
+
+
+class TokenEmbedding(NativeBlock):
+    """Token + learned position embedding: ``wte[ids] + wpe[:S]`` (GPT-2 style)."""
+
+    def __init__(self, vocab: int, max_seq: int, dim: int, dtype=torch.bfloat16, init_std=0.02):
+        super().__init__()
+        self.wte = nn.Embedding(vocab, dim, dtype=dtype)
+        self.wpe = nn.Embedding(max_seq, dim, dtype=dtype)
+        nn.init.normal_(self.wte.weight, std=init_std)
+        nn.init.normal_(self.wpe.weight, std=init_std)
+
+    def forward(self, ids):
+        S = ids.shape[-1]
+        pos = torch.arange(S, device=ids.device)
+        return self.wte(ids) + self.wpe(pos)
+
+    def _pp_direct_acc_params(self):
+        return [self.wte.weight, self.wpe.weight]
+
+    def lower(self, b, ids):
+        if ids.dtype != torch.int64 or ids.dim() != 2:
+            raise RuntimeError(f"TokenEmbedding expects int64 ids of shape [batch, seq], got "
+                               f"{ids.dtype} {tuple(ids.shape)}")
+        Bn, S = ids.shape
+        wte, wpe = b.weight(self.wte.weight), b.weight(self.wpe.weight)
+        if S > wpe.shape[0]:
+            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
+        Cc = wte.shape[1]
+        y = b.act("y", (Bn, S, Cc))
+        b.f(P.op_embed_fwd(ids, wte, wpe, y.view(Bn * S, Cc), S))
+
+        def bwd(dy, need_dx, dx_out):
+            # scatter-add straight into the fp32 accumulators (zeroed on the first accumulation)
+            acc_wte, acc_wpe = b.grad_acc(self.wte.weight), b.grad_acc(self.wpe.weight)
+            b.prog.init_toggle_fill.append(b.w(P.op_fill(acc_wte)))
+            b.prog.init_toggle_fill.append(b.w(P.op_fill(acc_wpe)))
+            b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S))
+            return None
+
+        b.on_backward(bwd)
+        return y
+
+
+class TransformerLayer(NativeBlock):
+    """One transformer layer: multi-head self-attention and a GELU feed-forward, pre-LayerNorm
+    (GPT-2) or post-LayerNorm (BERT).  Parameter names follow GPT-2 (``ln_1``, ``attn.c_attn``,
+    ``attn.c_proj``, ``ln_2``, ``mlp.c_fc``, ``mlp.c_proj``) with ``nn.Linear`` weights [out, in]."""
+
+    def __init__(self, dim: int, n_heads: int, ffn: int, *, causal: bool = True, pre_ln: bool = True,
+                 activation: str = "gelu_tanh", eps: float = 1e-5, dtype=torch.bfloat16, init_std=0.02):
+        super().__init__()
+        assert dim % n_heads == 0 and activation in ("gelu_tanh", "gelu_erf")
+        self.dim, self.n_heads, self.ffn = dim, n_heads, ffn
+        self.causal, self.pre_ln, self.activation = causal, pre_ln, activation
+        self.ln_1 = nn.LayerNorm(dim, eps=eps, dtype=dtype)
+        self.attn = nn.Module()
+        self.attn.c_attn = nn.Linear(dim, 3 * dim, dtype=dtype)
+        self.attn.c_proj = nn.Linear(dim, dim, dtype=dtype)
+        self.ln_2 = nn.LayerNorm(dim, eps=eps, dtype=dtype)
+        self.mlp = nn.Module()
+        self.mlp.c_fc = nn.Linear(dim, ffn, dtype=dtype)
+        self.mlp.c_proj = nn.Linear(ffn, dim, dtype=dtype)
+        for lin in (self.attn.c_attn, self.attn.c_proj, self.mlp.c_fc, self.mlp.c_proj):
+            nn.init.normal_(lin.weight, std=init_std)
+            nn.init.zeros_(lin.bias)
+
+    # torch statement of the layer
+    def _attention(self, h):
+        Bn, S, Cc = h.shape
+        H, D = self.n_heads, Cc // self.n_heads
+        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self.attn.c_attn(h).split(Cc, dim=-1))
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal)
+        return self.attn.c_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
+
+    def forward(self, x):
+        if self.pre_ln:
+            x = x + self._attention(self.ln_1(x))
+            return x + self.mlp.c_proj(_torch_act(self.mlp.c_fc(self.ln_2(x)), self.activation))
+        x = self.ln_1(x + self._attention(x))
+        return self.ln_2(x + self.mlp.c_proj(_torch_act(self.mlp.c_fc(x), self.activation)))
+
+    def lower(self, b, x):
+        if x.dim() != 3:
+            raise RuntimeError(f"TransformerLayer expects [batch, seq, dim], got {tuple(x.shape)}")
+        Bn, S, Cc = x.shape
+        if Cc != self.dim:
+            raise RuntimeError(f"TransformerLayer of width {self.dim} got width {Cc}")
+        return self._lower_pre_ln(b, x) if self.pre_ln else self._lower_post_ln(b, x)
+
+    def _lower_pre_ln(self, b, x):
+        Bn, S, Cc = x.shape
+        T, H = Bn * S, self.n_heads
+        x2d = x.view(T, Cc)
+        act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
+        ln1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, x2d)
+        qkv, _ = lower_linear(b, "qkv", self.attn.c_attn, ln1)
+        att = b.act("att", (T, Cc))
+        lse = b.act("lse", (Bn, H, S), torch.float32)
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
+        x2, _ = lower_linear(b, "x2", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
+        ln2, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, x2)
+        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, ln2, epilogue=act, save_pre=b.training)
+        y, _ = lower_linear(b, "y", self.mlp.c_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+
+        def bwd(dy, need_dx, dx_out):
+            dy2d = dy.view(T, Cc)
+            # feed-forward: dI through c_proj carries gelu'(h_pre) in its epilogue
+            d_hpre = linear_backward(b, "c_proj", self.mlp.c_proj, h, dy2d, dx_epilogue=dact, dx_aux=h_pre)
+            d_ln2 = linear_backward(b, "c_fc", self.mlp.c_fc, ln2, d_hpre)
+            d_x2 = layernorm_backward(b, "ln2", self.ln_2, x2, mean2, rstd2, d_ln2, dres=dy2d)
+            # attention
+            d_att = linear_backward(b, "attn_proj", self.attn.c_proj, att, d_x2)
+            dqkv = b.grad("dqkv", (T, 3 * Cc))
+            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
+            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            d_ln1 = linear_backward(b, "c_attn", self.attn.c_attn, ln1, dqkv)
+            dx = layernorm_backward(b, "ln1", self.ln_1, x2d, mean1, rstd1, d_ln1, dres=d_x2,
+                                    dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            return dx.view(Bn, S, Cc)
+
+        b.on_backward(bwd)
+        return y.view(Bn, S, Cc)
+
+    def _lower_post_ln(self, b, x):
+        if b.training:
+            raise NotImplementedError("post-LayerNorm transformer layers are lowered for inference only")
+        Bn, S, Cc = x.shape
+        T, H = Bn * S, self.n_heads
+        x2d = x.view(T, Cc)
+        qkv, _ = lower_linear(b, "qkv", self.attn.c_attn, x2d)
+        att = b.act("att", (T, Cc))
+        lse = b.act("lse", (Bn, H, S), torch.float32)
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
+        a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
+        x1, _, _ = lower_layernorm(b, "ln1", self.ln_1, a)
+        h, _ = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=_ACT_EPI[self.activation])
+        f, _ = lower_linear(b, "f", self.mlp.c_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x1)
+        y, _, _ = lower_layernorm(b, "ln2", self.ln_2, f)
+        b.on_backward(lambda dy, need_dx, dx_out: None)
+        return y.view(Bn, S, Cc)
+
+
+class LMHead(NativeBlock):
+    """Final LayerNorm and the (untied) vocabulary projection.  The weight is stored with its
+    vocabulary dimension padded to a multiple of 128 (zero rows) so that logits rows are 256-byte
+    aligned; the block's output is the [.., vocab] view of the padded logits buffer."""
+
+    VOCAB_ALIGN = 128
+
+    def __init__(self, dim: int, vocab: int, *, final_ln: bool = True, eps: float = 1e-5,
+                 dtype=torch.bfloat16, init_std=0.02):
+        super().__init__()
+        self.dim, self.vocab = dim, vocab
+        self.ln_f = nn.LayerNorm(dim, eps=eps, dtype=dtype) if final_ln else None
+        self.lm_head = nn.Linear(dim, vocab, bias=False, dtype=dtype)
+        nn.init.normal_(self.lm_head.weight, std=init_std)
+
+    @property
+    def padded_vocab(self):
+        return (self.vocab + self.VOCAB_ALIGN - 1) // self.VOCAB_ALIGN * self.VOCAB_ALIGN
+
+    def _pp_padded_rows(self):
+        return [(self.lm_head.weight, self.padded_vocab)]
+
+    def forward(self, x):
+        if self.ln_f is not None:
+            x = self.ln_f(x)
+        return self.lm_head(x)
+
+    def lower(self, b, x):
+        Bn, S, Cc = x.shape
+        T, V, Vp = Bn * S, self.vocab, self.padded_vocab
+        x2d = x.view(T, Cc)
+        if self.ln_f is not None:
+            h, mean, rstd = lower_layernorm(b, "ln_f", self.ln_f, x2d)
+        else:
+            h = x2d
+        logits = b.act("logits", (T, Vp))
+        lower_linear(b, "logits", self.lm_head, h, out=logits)
+        out = logits.view(Bn, S, Vp)[..., :V]
+        out._pp_padded = logits
+
+        def bwd(dy, need_dx, dx_out):
+            # dy is the padded [T, Vp] gradient buffer of the logits
+            d_h = linear_backward(b, "lm_head", self.lm_head, h, dy.view(T, Vp), need_dx=need_dx,
+                                  dx_out=(dx_out.view(T, Cc) if (dx_out is not None and self.ln_f is None)
+                                          else None))
+            if not need_dx:
+                return None
+            if self.ln_f is None:
+                return d_h.view(Bn, S, Cc)
+            dx = layernorm_backward(b, "ln_f", self.ln_f, x2d, mean, rstd, d_h,
+                                    dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            return dx.view(Bn, S, Cc)
+
+        b.on_backward(bwd)
+        return out
+
+
+class StageSequence(nn.Module):
+    """A stage module that applies its children in order.  Children keep the names they had in the
+    un-split model (``add_block("transformer.h.3", layer)`` registers nested containers), so a
+    stage's ``state_dict`` keys are a subset of the original model's."""
+
+    def __init__(self):
+        super().__init__()
+        self._order: List[str] = []
+
+    def add_block(self, fqn: str, module: nn.Module):
+        parts = fqn.split(".")
+        parent = self
+        for p in parts[:-1]:
+            if not hasattr(parent, p):
+                parent.add_module(p, nn.Module())
+            parent = getattr(parent, p)
+        parent.add_module(parts[-1], module)
+        self._order.append(fqn)
+
+    def blocks(self) -> List[nn.Module]:
+        return [self.get_submodule(f) for f in self._order]
+
+    def forward(self, x):
+        for blk in self.blocks():
+            x = blk(x)
+        return x

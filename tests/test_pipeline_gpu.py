@@ -1,0 +1,219 @@
+"""End-to-end parity of the pipeline (split -> staged forward/backward -> accumulate -> merge) on
+the GPU against the fp32 CPU oracle, through the reference's own API surface."""
+import copy
+
+import pytest
+import torch
+
+from _util import BF16_TOL, F32_TOL, assert_close_rel, max_rel
+from oracle import pipeline as OP
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def note(msg):
+    print(msg, flush=True)
+
+
+def _fp32_cpu_copy(model):
+    ref = copy.deepcopy(model).float().cpu()
+    return ref
+
+
+def _build_decoder(n_stages, n_layers=4, M=4, vocab=1000, seq=128, dim=128, heads=2, ffn=512, seed=0,
+                   fused=False, group=None):
+    import pippy_amd as pp
+    from pippy_amd.configs import DecoderLM, equal_split_spec
+    torch.manual_seed(seed)
+    model = DecoderLM(vocab=vocab, max_seq=seq, dim=dim, n_layers=n_layers, n_heads=heads, ffn=ffn)
+    ref = _fp32_cpu_copy(model)
+    ids = torch.randint(0, vocab, (2 * M, seq))
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(n_layers, n_stages))
+    assert pipe.num_stages == n_stages
+    stages = [pp.PipelineStage(pipe, i, DEV, group=group, fused_accumulate=fused) for i in range(n_stages)]
+    ref_stages = []
+    keys = list(ref.state_dict().keys())
+    # stage s of the oracle = the same children of the fp32 copy
+    import torch.nn as nn
+    per = n_layers // n_stages
+    for s in range(n_stages):
+        mods = []
+        if s == 0:
+            mods.append(ref.embed)
+        mods += [ref.h[i] for i in range(per * s, per * (s + 1))]
+        if s == n_stages - 1:
+            mods.append(ref.head)
+        ref_stages.append(nn.Sequential(*mods))
+    return model, ref, stages, ref_stages, ids
+
+
+def _ce(out, tgt):
+    return torch.nn.functional.cross_entropy(out.reshape(-1, out.shape[-1]), tgt.reshape(-1))
+
+
+def _check_against_oracle(model, ref, stages, ref_stages, ids, schedule_cls, M, steps=1):
+    import pippy_amd as pp
+    vocab = model.head.vocab
+    torch.manual_seed(123)
+    target = torch.randint(0, vocab, ids.shape)
+    sched = schedule_cls(stages, M, loss_fn=pp.CrossEntropyLoss())
+    for step in range(steps):
+        losses = []
+        out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+        torch.cuda.synchronize()
+    for p in ref.parameters():
+        p.grad = None
+    ref_out, ref_losses = None, None
+    for step in range(steps):
+        ref_out, ref_losses = OP.step(ref_stages, ids, target, M, _ce)
+    assert out.shape == ref_out.shape and out.is_contiguous()
+    assert_close_rel(out, ref_out, BF16_TOL, "merged logits")
+    assert len(losses) == M
+    for m in range(M):
+        assert_close_rel(losses[m].reshape(1), ref_losses[m].reshape(1), BF16_TOL, f"loss {m}")
+    named = dict(model.named_parameters())
+    worst = 0.0
+    for name, rp in ref.named_parameters():
+        g = named[name].main_grad
+        err = max_rel(g, rp.grad)
+        worst = max(worst, err)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+    note(f"{schedule_cls.__name__}: worst grad error {worst:.3e}")
+    return out, losses, {n: named[n].main_grad.clone() for n in named}
+
+
+@pytest.mark.parametrize("n_stages", [1, 2, 4])
+def test_decoder_gpipe_matches_oracle(n_stages):
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(n_stages, M=M)
+    _check_against_oracle(model, ref, stages, ref_stages, ids, pp.ScheduleGPipe, M)
+
+
+def test_schedules_agree_bitwise_and_match_oracle():
+    """Per stage, forward and backward run in ascending microbatch order in every schedule, so
+    all results are identical across schedules (embedding gradients use fp32 atomics whose order
+    inside one microbatch is not fixed, so they get a 1e-6 relative allowance)."""
+    import pippy_amd as pp
+    M = 4
+    results = {}
+    for name, cls, group in (("gpipe", pp.ScheduleGPipe, None), ("1f1b", pp.Schedule1F1B, None),
+                             ("bfs", pp.ScheduleLoopedBFS, 2), ("interleaved", pp.ScheduleInterleaved1F1B, 2),
+                             ("interleaved_g1", pp.ScheduleInterleaved1F1B, 1),
+                             ("zero_bubble", pp.ScheduleZeroBubble, None)):
+        model, ref, stages, ref_stages, ids = _build_decoder(4, M=M, group=group)
+        note(f"schedule {name}")
+        results[name] = _check_against_oracle(model, ref, stages, ref_stages, ids, cls, M)
+    base_out, base_losses, base_grads = results["gpipe"]
+    for name, (out, losses, grads) in results.items():
+        assert torch.equal(out, base_out), f"{name}: merged output differs from GPipe"
+        for a, b in zip(losses, base_losses):
+            assert torch.equal(a, b), f"{name}: loss differs from GPipe"
+        for k in grads:
+            if k.startswith("embed."):
+                assert max_rel(grads[k], base_grads[k]) <= 1e-6, f"{name}: {k}"
+            else:
+                assert torch.equal(grads[k], base_grads[k]), f"{name}: grad of {k} differs from GPipe"
+
+
+def test_two_steps_accumulate_then_zero_grad():
+    """Gradients keep accumulating across steps until zero_grad, as with autograd's .grad
+    (reference test_grad.py:78-82 runs two steps with zero_grad in between)."""
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M, steps=2)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    sched.zero_grad()
+    _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M, steps=1)
+
+
+def test_fused_accumulate_matches_oracle():
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M, fused=True)
+    _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M)
+
+
+def test_inference_gpipe_forward_only():
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    sched = pp.ScheduleGPipe(stages, M)
+    out = sched.step(ids.to(DEV))
+    ref_out, _ = OP.step(ref_stages, ids, None, M, None)
+    assert_close_rel(out, ref_out, BF16_TOL, "inference logits")
+
+
+def test_generic_loss_fn_bridge():
+    """Any callable works as loss_fn: it runs under autograd on the last stage's output."""
+    import pippy_amd as pp
+    M = 2
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    target = torch.randint(0, 1000, ids.shape)
+    sched = pp.ScheduleGPipe(stages, M, loss_fn=lambda o, t: _ce(o.float(), t))
+    losses = []
+    sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    for p in ref.parameters():
+        p.grad = None
+    _, ref_losses = OP.step(ref_stages, ids, target, M, _ce)
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        assert_close_rel(named[name].main_grad, rp.grad, BF16_TOL, name)
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.reshape(1), b.reshape(1), BF16_TOL, "loss")
+
+
+def test_readme_mlp_fp32_matches_oracle():
+    """Configuration 1: the README MLP (examples/basic/example_train.py:9-45 of the reference),
+    fp32, 2 stages split at layer1, GPipe over 4 microbatches of 64, cross entropy."""
+    import torch.nn as nn
+    import pippy_amd as pp
+
+    class MyNetworkBlock(nn.Module):
+        def __init__(self, i, o):
+            super().__init__()
+            self.lin = nn.Linear(i, o)
+
+        def forward(self, x):
+            return torch.relu(self.lin(x))
+
+    class MyNetwork(nn.Module):
+        def __init__(self):
+            super().__init__()
+            dims = [512, 1024, 256]
+            prev = 512
+            self.num_layers = len(dims)
+            for i, d in enumerate(dims):
+                self.add_module(f"layer{i}", MyNetworkBlock(prev, d))
+                prev = d
+            self.output_proj = nn.Linear(prev, 10)
+
+        def forward(self, x):
+            for i in range(self.num_layers):
+                x = getattr(self, f"layer{i}")(x)
+            return self.output_proj(x)
+
+    torch.manual_seed(0)
+    model = MyNetwork()
+    ref = copy.deepcopy(model)
+    x = torch.randn(256, 512)
+    y = torch.randint(0, 10, (256,))
+    M = 4
+    pipe = pp.pipeline(model, M, (x,), split_spec={"layer1": pp.SplitPoint.BEGINNING})
+    assert pipe.num_stages == 2
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert all(s.is_native for s in stages)
+    sched = pp.ScheduleGPipe(stages, M, loss_fn=nn.CrossEntropyLoss())
+    losses = []
+    out = sched.step(x.to(DEV), target=y.to(DEV), losses=losses)
+    ref_stages = [nn.Sequential(ref.layer0), nn.Sequential(ref.layer1, ref.layer2, ref.output_proj)]
+    ref_out, ref_losses = OP.step(ref_stages, x, y, M, nn.functional.cross_entropy)
+    assert_close_rel(out, ref_out, F32_TOL, "mlp output")
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.reshape(1), b.reshape(1), F32_TOL, "mlp loss")
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        assert_close_rel(named[name].grad, rp.grad, F32_TOL, f"mlp grad {name}")
+        assert named[name].grad.data_ptr() == named[name].main_grad.data_ptr()
