@@ -104,7 +104,12 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
                 return None
             blocks.append(LayerNormBlock(m))
         else:
-            return None
+            # a user container (e.g. a block that wraps a linear and an activation): lower it as
+            # a chain of its own and splice the result in
+            sub = lower_stage_module(m)
+            if sub is None:
+                return None
+            blocks.extend(sub)
         i += 1
     return blocks or None
 

@@ -400,7 +400,18 @@ class Builder:
             self.w(op_gemm(dY2d, X2d, self.grad_target(p, padded), a_trans=True, b_trans=True))
 
     def on_backward(self, fn: Callable):
-        self._backward.append(fn)
+        """Registers the block's backward emitter ``fn(dy, need_dx, dx_out) -> dx``; it runs later,
+        in reverse block order, under the naming scope that is current now."""
+        scope = list(self._scope)
+
+        def scoped(dy, need_dx, dx_out):
+            saved, self._scope = self._scope, list(scope)
+            try:
+                return fn(dy, need_dx, dx_out)
+            finally:
+                self._scope = saved
+
+        self._backward.append(scoped)
 
 
 class StageProgram:
@@ -422,23 +433,26 @@ class StageProgram:
         self.acc_initialized = False  # False: the next W pass overwrites the accumulators
 
     def shared(self, key, shape, dtype, exact=True) -> torch.Tensor:
+        # Launch lists hold raw pointers into these buffers, so a buffer is never replaced or
+        # freed once handed out: the size is part of the key.
         shape = tuple(shape)
         numel = 1
         for s in shape:
             numel *= s
-        t = self._shared.get(key)
-        if t is None or t.dtype != dtype or t.numel() < numel or (exact and t.numel() != numel):
+        full_key = (key, numel, dtype)
+        t = self._shared.get(full_key)
+        if t is None:
             t = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
-            self._shared[key] = t
+            self._shared[full_key] = t
         return t[:numel].view(shape)
 
     def ones_f32(self, n: int) -> torch.Tensor:
         """A [1, n] row of ones (the left operand that turns an fp32 GEMM into a column sum)."""
-        t = self._shared.get("ones_f32")
-        if t is None or t.numel() < n:
+        t = self._shared.get(("ones_f32", n))
+        if t is None:
             t = torch.ones(max(n, 1), dtype=torch.float32, device=self.device)
-            self._shared["ones_f32"] = t
-        return t[:n].view(1, n)
+            self._shared[("ones_f32", n)] = t
+        return t.view(1, n)
 
     def build(self, mb: int, x: torch.Tensor, dx_target: Optional[torch.Tensor]) -> MicrobatchProgram:
         """Lowers every block for microbatch slot ``mb`` with input ``x`` (a real buffer: the

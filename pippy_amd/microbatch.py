@@ -233,39 +233,66 @@ def split_args_kwargs_into_chunks(
 
 
 # ---- merge -------------------------------------------------------------------------------------
-def _row_view(t: torch.Tensor, dim: int):
-    """Describes ``t`` as rows for a concatenation along ``dim``: returns (n_rows, row_bytes,
-    row_stride_bytes) if every row [outer index] is one contiguous run, else None."""
-    es = t.element_size()
-    nd = t.dim()
-    # dims dim..nd-1 must be densely packed
-    expect = 1
-    for d in range(nd - 1, dim - 1, -1):
-        if t.size(d) != 1 and t.stride(d) != expect:
-            return None
-        expect *= t.size(d)
-    row_elems = expect
-    # dims 0..dim-1 must collapse to a single stride
-    outer = 1
-    for s in t.shape[:dim]:
-        outer *= s
-    if outer <= 1:
-        return (outer, row_elems * es, row_elems * es)
+def _collapse(t: torch.Tensor, dims: Sequence[int]):
+    """(count, stride) if the listed dims of ``t`` walk memory with one uniform stride, else None
+    (size-1 dims are ignored; an empty walk is (1, 0))."""
     stride = None
-    mult = 1
-    for d in range(dim - 1, -1, -1):
+    count = 1
+    for d in reversed(list(dims)):
         if t.size(d) == 1:
             continue
         if stride is None:
             stride = t.stride(d)
-            mult = t.size(d)
-        else:
-            if t.stride(d) != stride * mult:
-                return None
-            mult *= t.size(d)
-    if stride is None or stride < row_elems:
+        elif t.stride(d) != stride * count:
+            return None
+        count *= t.size(d)
+    return (count, stride if stride is not None else 0)
+
+
+def _row_view(t: torch.Tensor, dim: int):
+    """Describes ``t`` as uniformly strided rows for a concatenation along ``dim``.  Returns
+    (n_rows, row_bytes, row_stride_bytes, rows_per_outer) or None.  ``rows_per_outer`` is how many
+    consecutive rows belong to one index of the dims before ``dim`` (the destination jumps after
+    that many rows unless there is a single outer index)."""
+    es = t.element_size()
+    nd = t.dim()
+    # k = first dim of the densely packed trailing block
+    expect = 1
+    k = nd
+    for d in range(nd - 1, -1, -1):
+        if t.size(d) != 1 and t.stride(d) != expect:
+            break
+        expect *= t.size(d)
+        k = d
+    outer = 1
+    for s_ in t.shape[:dim]:
+        outer *= s_
+    if k <= dim:
+        # whole [dim..] slabs are contiguous: one row per outer index
+        row_elems = 1
+        for s_ in t.shape[dim:]:
+            row_elems *= s_
+        col = _collapse(t, range(0, dim))
+        if col is None:
+            return None
+        count, stride = col
+        if count > 1 and stride < row_elems:
+            return None
+        return (outer, row_elems * es, (stride if count > 1 else row_elems) * es, 1)
+    # the dense block is smaller than a slab: rows are the dense blocks; the destination is only
+    # uniformly strided when a single outer index exists
+    if outer != 1:
         return None
-    return (outer, row_elems * es, stride * es)
+    row_elems = 1
+    for s_ in t.shape[k:]:
+        row_elems *= s_
+    col = _collapse(t, range(0, k))
+    if col is None:
+        return None
+    count, stride = col
+    if count > 1 and stride < row_elems:
+        return None
+    return (count, row_elems * es, (stride if count > 1 else row_elems) * es, count)
 
 
 def cat_chunks(values: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
@@ -300,6 +327,7 @@ def cat_chunks(values: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
         return out
     outer, inner = _rows(shape, dim, first.element_size())
     segs = []
+    keep_alive = []  # staging tensors must outlive the enqueue of the copy that reads them
     lo = 0
     for v in values:
         d = v.size(dim)
@@ -308,14 +336,21 @@ def cat_chunks(values: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
             if rv is None:  # arbitrary strides: gather into a contiguous staging tensor first
                 tmp = torch.empty(v.shape, dtype=v.dtype, device=v.device)
                 _native.strided_copy_nd(tmp, v)
+                keep_alive.append(tmp)
                 v = tmp
-                rv = (outer, d * inner, d * inner)
-            n_rows, row_bytes, src_stride = rv
-            assert row_bytes == d * inner
-            segs.append((v.data_ptr(), out.data_ptr() + lo * inner, outer, row_bytes, src_stride,
-                         total * inner))
+                rv = (outer, d * inner, d * inner, 1)
+            n_rows, row_bytes, src_stride, rows_per_outer = rv
+            if rows_per_outer == 1:
+                assert row_bytes == d * inner and n_rows == outer
+                dst_stride = total * inner
+            else:
+                assert outer == 1 and n_rows * row_bytes == d * inner
+                dst_stride = row_bytes
+            segs.append((v.data_ptr(), out.data_ptr() + lo * inner, n_rows, row_bytes, src_stride,
+                         dst_stride))
         lo += d
     _native.copy_rows(segs)
+    del keep_alive
     return out
 
 

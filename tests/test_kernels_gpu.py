@@ -431,3 +431,20 @@ def test_run_ops_matches_direct_calls():
     ops[1].kind = 999
     with pytest.raises(RuntimeError, match="op 1"):
         Nn.run_ops(ops, 2)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32_TOL), (torch.bfloat16, BF16_TOL)])
+@pytest.mark.parametrize("act", ["relu", "gelu_erf", "gelu_tanh"])
+def test_activation_bwd(dtype, tol, act):
+    Nn = native()
+    torch.manual_seed(14)
+    n = 64 * 512 + 5
+    aux = torch.randn(n, device=DEV).to(dtype)
+    dy = torch.randn(n, device=DEV).to(dtype)
+    dz = torch.empty_like(dy)
+    kind = {"relu": Nn.ACT_RELU, "gelu_erf": Nn.ACT_GELU_ERF, "gelu_tanh": Nn.ACT_GELU_TANH}[act]
+    Nn.activation_bwd(dy, aux, dz, kind)
+    a = aux.float().cpu().requires_grad_(True)
+    fn = {"relu": torch.relu, "gelu_erf": O.gelu_erf, "gelu_tanh": O.gelu_tanh}[act]
+    fn(a).backward(dy.float().cpu())
+    assert_close_rel(dz, a.grad, tol, f"activation bwd {act}")
