@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Throughput of the pipeline-stage hot path on one MI355X.
+
+Workload (configs[2] of BASELINE.json, the one the metric's target is quoted on): a
+GPT-2-small-shaped decoder (12 layers, d_model 768, 12 heads, FFN 3072, tanh-GELU, pre-LayerNorm,
+causal attention, vocabulary 50257, sequence 1024) cut into 4 virtual stages of 3 layers on one
+GPU, trained with Schedule1F1B over a batch of 32 split into 8 microbatches of 4; bf16 weights and
+activations, fp32 gradient accumulation; synthetic tokens, random-initialised weights.
+
+One "step" is one ``schedule.step()``: microbatch split, 32 stage forwards, 8 cross-entropy
+losses, 32 stage backwards (input- and weight-gradient passes), fp32 gradient accumulation and
+the merge of the 8 logits chunks.  Inputs are resident in HBM before the timed region.
+
+Prints one JSON line: tokens/s, the MFMA roofline of the dominant kernel (the bf16 GEMM, timed
+per launch with HIP events on its own stream in a second, instrumented pass over the same steps)
+and the CPU baseline (the oracle's fp32 restatement of the reference step on this box's cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+
+
+def build(args):
+    import pippy_amd as pp
+    from pippy_amd.configs import DecoderLM, equal_split_spec
+    torch.manual_seed(0)
+    model = DecoderLM(vocab=args.vocab, max_seq=args.seq, dim=args.dim, n_layers=args.layers,
+                      n_heads=args.heads, ffn=args.ffn)
+    ids = torch.randint(0, args.vocab, (args.batch, args.seq))
+    target = torch.randint(0, args.vocab, (args.batch, args.seq))
+    pipe = pp.pipeline(model, args.microbatches, (ids,),
+                       split_spec=equal_split_spec(args.layers, args.stages))
+    stages = [pp.PipelineStage(pipe, i, "cuda", fused_accumulate=args.fused_accumulate)
+              for i in range(args.stages)]
+    sched_cls = {"1f1b": pp.Schedule1F1B, "gpipe": pp.ScheduleGPipe,
+                 "zero_bubble": pp.ScheduleZeroBubble}[args.schedule]
+    sched = sched_cls(stages, args.microbatches, loss_fn=pp.CrossEntropyLoss())
+    return model, sched, stages, ids.cuda(), target.cuda()
+
+
+def flops_per_step(args):
+    """Algorithmic FLOPs of one training step: matmul 2mnk, attention dense, backward 2x forward."""
+    T = args.batch * args.seq
+    d, f, V, L, S = args.dim, args.ffn, args.vocab, args.layers, args.seq
+    per_token_fwd = L * (2 * d * 3 * d + 2 * d * d + 2 * 2 * d * f + 4 * S * d) + 2 * d * V
+    return 3.0 * per_token_fwd * T
+
+
+def cpu_baseline(args, sample_microbatches=2):
+    """The oracle's statement of the reference step (fp32, torch CPU kernels, this box's cores) on a
+    bounded sample of the same workload: the first microbatches of one step through all stages,
+    forward, loss and backward in the reference's order."""
+    from oracle import pipeline as OP
+    from pippy_amd.configs import DecoderLM
+    import torch.nn as nn
+    torch.manual_seed(0)
+    model = DecoderLM(vocab=args.vocab, max_seq=args.seq, dim=args.dim, n_layers=args.layers,
+                      n_heads=args.heads, ffn=args.ffn, dtype=torch.float32)
+    per = args.layers // args.stages
+    stages = []
+    for s in range(args.stages):
+        mods = ([model.embed] if s == 0 else []) + [model.h[i] for i in range(per * s, per * (s + 1))]
+        if s == args.stages - 1:
+            mods.append(model.head)
+        stages.append(nn.Sequential(*mods))
+    mb = args.batch // args.microbatches
+    n = sample_microbatches
+    ids = torch.randint(0, args.vocab, (mb * n, args.seq))
+    target = torch.randint(0, args.vocab, (mb * n, args.seq))
+
+    def ce(o, t):
+        return torch.nn.functional.cross_entropy(o.reshape(-1, o.shape[-1]), t.reshape(-1))
+
+    t0 = time.perf_counter()
+    OP.step(stages, ids, target, n, ce)
+    dt = time.perf_counter() - t0
+    return {"value": round(ids.numel() / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{n} of {args.microbatches} microbatches ({ids.numel()} tokens) of one step: "
+                      f"fp32 forward+loss+backward through all {args.stages} stages in the reference's "
+                      f"order, one process, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--schedule", default="1f1b", choices=["1f1b", "gpipe", "zero_bubble"])
+    ap.add_argument("--fused-accumulate", action="store_true",
+                    help="accumulate fp32 gradients in the dW GEMM epilogue instead of the accumulate kernel")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    # workload shape (defaults: GPT-2 small, configs[2])
+    ap.add_argument("--vocab", type=int, default=50257)
+    ap.add_argument("--seq", type=int, default=1024)
+    ap.add_argument("--dim", type=int, default=768)
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--heads", type=int, default=12)
+    ap.add_argument("--ffn", type=int, default=3072)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--microbatches", type=int, default=8)
+    ap.add_argument("--stages", type=int, default=4)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs every pipeline stage as a virtual stage on ONE GPU; "
+              "there is no multi-GPU path to measure (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    from pippy_amd import _native as N
+    N.lib()  # fail loudly if the kernel library is missing
+    model, sched, stages, ids, target = build(args)
+    tokens = ids.numel()
+
+    def step():
+        sched.zero_grad()
+        losses = []
+        out = sched.step(ids, target=target, losses=losses)
+        return out, losses
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out, losses = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = tokens * args.steps / dt
+    loss0 = float(losses[0])
+
+    result = {
+        "metric": "tokens/sec per schedule step on 1 MI355X + stage GEMM MFMA util %",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"GPT-2-small-shaped decoder ({args.layers} layers, d_model {args.dim}, "
+                               f"{args.heads} heads, FFN {args.ffn}, vocab {args.vocab}, seq {args.seq}), "
+                               f"{args.stages} virtual stages on one GPU, schedule {args.schedule}, "
+                               f"batch {args.batch} in {args.microbatches} microbatches, bf16 with fp32 "
+                               f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})",
+                   "global_batch": args.batch, "seq_len": args.seq},
+        "step_tflops": round(flops_per_step(args) / (ms_per_step * 1e-3) / 1e12, 1),
+        "loss_microbatch0": round(loss0, 4),
+    }
+
+    if not args.no_roofline:
+        # Instrumented pass: the same steps with every launch-list op bracketed by HIP events on
+        # its stream.  Kept apart from the timed region above so that event records do not perturb
+        # `value`; the kernels, shapes and order are identical.
+        n_prof = max(1, min(args.steps, 3))
+        N.profile_start(1 << 17)
+        for _ in range(n_prof):
+            step()
+        torch.cuda.synchronize()
+        N.profile_stop()
+        ms, work, cnt = N.profile_read(N.OP_GEMM_BF16)
+        achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+        result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
+                              "traffic": None, "kernel": "gemm_bf16_kernel",
+                              "launches_per_step": cnt // n_prof,
+                              "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
+                              "gemm_ms_per_step": round(ms / n_prof, 3)}
+        hbm = {}
+        for name, kind in (("grad_accumulate", N.OP_ACCUM_BF16), ("cross_entropy", N.OP_CE_LOSS),
+                           ("layernorm_fwd", N.OP_LN_FWD), ("layernorm_bwd_input", N.OP_LN_BWD_INPUT)):
+            kms, kwork, kcnt = N.profile_read(kind)
+            if kcnt:
+                gbs = kwork / (kms * 1e-3) / 1e9
+                hbm[name] = {"achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(gbs / HBM_PEAK_GBS, 4), "ms_per_step": round(kms / n_prof, 3)}
+        for name, kind in (("attention_fwd", N.OP_ATTN_FWD), ("attention_bwd", N.OP_ATTN_BWD)):
+            kms, kwork, kcnt = N.profile_read(kind)
+            if kcnt:
+                tf = kwork / (kms * 1e-3) / 1e12
+                hbm[name] = {"achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s (dense count)",
+                             "frac": round(tf / MFMA_PEAK_TFLOPS, 4), "ms_per_step": round(kms / n_prof, 3)}
+        # the merge of the logits chunks runs outside the launch lists: time it alone
+        from pippy_amd.microbatch import merge_chunks
+        chunks = stages[-1].output_chunks
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        merge_chunks(chunks, None)
+        ev0.record()
+        for _ in range(5):
+            merged = merge_chunks(chunks, None)
+        ev1.record()
+        torch.cuda.synchronize()
+        mms = ev0.elapsed_time(ev1) / 5
+        mbytes = 2.0 * merged.numel() * merged.element_size()
+        hbm["merge"] = {"achieved": round(mbytes / (mms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(mbytes / (mms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(mms, 3)}
+        result["other_kernels"] = hbm
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -243,6 +243,18 @@ typedef struct pp_op {
  * failing op is in pp_last_error()). */
 int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Per-launch timing of launch-list ops (measurement aid; no reference counterpart).  Between
+ * pp_profile_start and pp_profile_stop every op run by pp_run_ops is bracketed by two HIP events on
+ * its stream (host-side event objects only; no device memory).  pp_profile_read waits for the
+ * recorded events and returns, for one op kind, the summed elapsed milliseconds, the summed
+ * algorithmic work (FLOPs for GEMM and attention kinds, bytes for the HBM-bound kinds) and the
+ * number of launches.  Not thread-safe.
+ * ---------------------------------------------------------------------------------------- */
+int pp_profile_start(int max_records);
+int pp_profile_stop(void);
+int pp_profile_read(int kind, double* total_ms, double* total_work, int64_t* count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,9 +28,15 @@ from .stage_modules import NativeBlock
 logger = logging.getLogger(__name__)
 
 
+_active_tracer: Optional["fx.Tracer"] = None
+
+
 def pipe_split():
     """Marks a stage boundary when called inside a model's ``forward``
-    (reference ``_IR.py:319-342``).  A no-op outside of ``pipeline()``."""
+    (reference ``_IR.py:319-342``).  A no-op outside of ``pipeline()``; while ``pipeline()`` traces
+    the model it records a marker node at the current position of the graph."""
+    if _active_tracer is not None:
+        _active_tracer.create_proxy("call_function", pipe_split, (), {})
     return None
 
 
@@ -46,8 +52,16 @@ class PipeSplitWrapper:
 
 class _ModuleGranularityTracer(fx.Tracer):
     def __init__(self, split_names: Optional[List[str]]):
-        super().__init__(autowrap_functions=(pipe_split,))
+        super().__init__()
         self._split_names = split_names
+
+    def trace(self, root, concrete_args=None):
+        global _active_tracer
+        saved, _active_tracer = _active_tracer, self
+        try:
+            return super().trace(root, concrete_args)
+        finally:
+            _active_tracer = saved
 
     def is_leaf_module(self, m: nn.Module, qualname: str) -> bool:
         if isinstance(m, NativeBlock):

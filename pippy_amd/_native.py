@@ -35,7 +35,8 @@ EXPORTED_SYMBOLS = (
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
     "pp_gemm_bf16", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
-    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd",
+    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_profile_start", "pp_profile_stop",
+    "pp_profile_read",
 )
 
 
@@ -110,6 +111,9 @@ def lib() -> C.CDLL:
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
         "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
+        "pp_profile_start": [i32],
+        "pp_profile_stop": [],
+        "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -384,3 +388,19 @@ def activation_bwd(dy, aux, dz, act: int) -> None:
 
 def run_ops(ops, n: int) -> None:
     check(lib().pp_run_ops(ops, n, current_stream()), "pp_run_ops")
+
+
+# ---- per-launch timing ---------------------------------------------------------------------------
+def profile_start(max_records: int = 1 << 16) -> None:
+    check(lib().pp_profile_start(max_records), "pp_profile_start")
+
+
+def profile_stop() -> None:
+    check(lib().pp_profile_stop(), "pp_profile_stop")
+
+
+def profile_read(kind: int):
+    """(total_ms, total_work, count) of the ops of one kind recorded since profile_start."""
+    ms, work, cnt = C.c_double(), C.c_double(), C.c_int64()
+    check(lib().pp_profile_read(kind, C.byref(ms), C.byref(work), C.byref(cnt)), "pp_profile_read")
+    return ms.value, work.value, cnt.value

@@ -2,6 +2,7 @@
 // compiles its forward / input-gradient / weight-gradient pass for one microbatch into such a
 // list once, so that a pass costs one call from the host language instead of one per kernel.
 #include "common.h"
+#include <vector>
 
 using namespace pp;
 
@@ -74,11 +75,119 @@ static int run_one(const pp_op& op, pp_stream st) {
     }
 }
 
+// ---- per-launch timing with HIP events ---------------------------------------------------------
+// When a profile is active every executed op is bracketed by two events recorded on the op's own
+// stream; pp_profile_read synchronises and sums elapsed time and algorithmic work per op kind.
+namespace {
+struct ProfRecord {
+    hipEvent_t a, b;
+    int kind;
+    double work;
+};
+std::vector<ProfRecord> g_prof;
+size_t g_prof_used = 0;
+bool g_prof_on = false;
+long long g_prof_dropped = 0;
+
+// Algorithmic work of one op: FLOPs for MFMA-bound kinds, bytes for HBM-bound kinds.
+double op_work(const pp_op& op) {
+    switch (op.kind) {
+        case PP_OP_GEMM_BF16:
+        case PP_OP_GEMM_F32:
+            return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
+        case PP_OP_ATTN_FWD:  // dense count: QK^T and PV
+            return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[1] * (double)op.i[1] * (double)op.i[3];
+        case PP_OP_ATTN_BWD:  // dQ, dK, dV, dP and the recomputed scores
+            return 10.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[1] * (double)op.i[1] * (double)op.i[3];
+        case PP_OP_ACCUM_BF16:
+            return (double)op.i[0] * (op.j[0] ? 6.0 : 10.0);
+        case PP_OP_ACCUM_F32:
+            return (double)op.i[0] * (op.j[0] ? 8.0 : 12.0);
+        case PP_OP_COPY_ROWS:
+            return 2.0 * (double)op.i[0] * (double)op.i[1];
+        case PP_OP_LN_FWD:
+            return 4.0 * (double)op.i[0] * (double)op.i[1];  // read x, write y (bf16)
+        case PP_OP_LN_BWD_INPUT:
+            return (op.p[5] ? 8.0 : 6.0) * (double)op.i[0] * (double)op.i[1];
+        case PP_OP_LN_BWD_WEIGHT:
+            return 4.0 * (double)op.i[0] * (double)op.i[1];
+        case PP_OP_COLSUM:
+            return 2.0 * (double)op.i[0] * (double)op.i[1];
+        case PP_OP_CE_LOSS:  // read logits, write their gradient
+            return (op.p[3] ? 2.0 : 1.0) * (double)op.i[0] * (double)op.i[2] * (op.j[0] == PP_F32 ? 4.0 : 2.0);
+        case PP_OP_EMBED_FWD:
+            return 6.0 * (double)op.i[0] * (double)op.i[2];
+        case PP_OP_EMBED_BWD:
+            return 10.0 * (double)op.i[0] * (double)op.i[2];
+        case PP_OP_FILL:
+            return (double)op.i[0];
+        case PP_OP_ACT_BWD:
+            return 3.0 * (double)op.i[0] * (op.j[1] == PP_F32 ? 4.0 : 2.0);
+        default:
+            return 0.0;
+    }
+}
+}  // namespace
+
+extern "C" int pp_profile_start(int max_records) {
+    if (max_records <= 0) return fail(PP_ERR_INVALID, "pp_profile_start: max_records <= 0");
+    if (g_prof.size() < (size_t)max_records) {
+        const size_t old = g_prof.size();
+        g_prof.resize((size_t)max_records);
+        for (size_t i = old; i < g_prof.size(); ++i) {
+            if (hipEventCreate(&g_prof[i].a) != hipSuccess || hipEventCreate(&g_prof[i].b) != hipSuccess) {
+                g_prof.resize(i);
+                return fail(PP_ERR_LAUNCH, "pp_profile_start: cannot create events");
+            }
+        }
+    }
+    g_prof_used = 0;
+    g_prof_dropped = 0;
+    g_prof_on = true;
+    return PP_OK;
+}
+
+extern "C" int pp_profile_stop(void) {
+    g_prof_on = false;
+    return PP_OK;
+}
+
+extern "C" int pp_profile_read(int kind, double* total_ms, double* total_work, int64_t* count) {
+    if (!total_ms || !total_work || !count) return fail(PP_ERR_INVALID, "pp_profile_read: null pointer");
+    *total_ms = 0.0;
+    *total_work = 0.0;
+    *count = 0;
+    for (size_t i = 0; i < g_prof_used; ++i) {
+        const ProfRecord& r = g_prof[i];
+        if (r.kind != kind) continue;
+        if (hipEventSynchronize(r.b) != hipSuccess) return fail(PP_ERR_LAUNCH, "pp_profile_read: event sync failed");
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, r.a, r.b) != hipSuccess) return fail(PP_ERR_LAUNCH, "pp_profile_read: elapsed failed");
+        *total_ms += ms;
+        *total_work += r.work;
+        *count += 1;
+    }
+    if (g_prof_dropped) return fail(PP_ERR_UNSUPPORTED, "pp_profile_read: %lld ops were not recorded (pool too small)", g_prof_dropped);
+    return PP_OK;
+}
+
 extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PP_ERR_INVALID, "pp_run_ops: bad list");
     for (int i = 0; i < n_ops; ++i) {
         if (ops[i].flags & PP_OP_SKIP) continue;
+        ProfRecord* rec = nullptr;
+        if (g_prof_on) {
+            if (g_prof_used < g_prof.size()) {
+                rec = &g_prof[g_prof_used++];
+                rec->kind = ops[i].kind;
+                rec->work = op_work(ops[i]);
+                (void)hipEventRecord(rec->a, static_cast<hipStream_t>(stream));
+            } else {
+                ++g_prof_dropped;
+            }
+        }
         const int rc = run_one(ops[i], stream);
+        if (rec) (void)hipEventRecord(rec->b, static_cast<hipStream_t>(stream));
         if (rc != PP_OK) {
             char msg[400];
             snprintf(msg, sizeof msg, "%s", pp_last_error());

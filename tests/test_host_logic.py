@@ -1,0 +1,369 @@
+"""Host-side logic that needs no GPU: microbatch bookkeeping, schedule orders, the splitting
+front end, error behaviour, and the C ABI surface of the built library."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+from collections import namedtuple
+
+import pytest
+import torch
+import torch.nn as nn
+
+import pippy_amd as pp
+from oracle import schedules as OS
+from pippy_amd import _native, _schedule_order as order
+from pippy_amd import microbatch as MB
+from pippy_amd._lowering import lower_stage_module
+from pippy_amd.microbatch import (TensorChunkSpec, _Replicate, chunk_sizes, merge_chunks,
+                                  split_args_kwargs_into_chunks, sum_reducer)
+from pippy_amd.stage import ManualPipelineStage
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- microbatch split (views of host tensors; no data movement) -----------------------------------
+def test_split_shapes_of_the_reference_test():
+    """test/test_microbatch.py:17-34 of the reference."""
+    d = 512
+    x0, x1, x2 = torch.randn(128, d), torch.randn(256, d), torch.randn(512, d)
+    args, kwargs = (x0, x1, x2), {"x0": x0, "x1": x1, "x2": x2}
+    a, k = split_args_kwargs_into_chunks(args, kwargs, 2)
+    assert len(a) == 2 and len(k) == 2
+    assert a[0][0].shape == (64, d) and a[1][0].shape == (64, d)
+    assert a[0][1].shape == (128, d) and a[0][2].shape == (256, d)
+    assert k[0]["x0"].shape == (64, d) and k[0]["x1"].shape == (128, d) and k[1]["x2"].shape == (256, d)
+    # chunks are views of the caller's tensors, as in the reference (no bytes move)
+    assert a[1][0].data_ptr() == x0[64:].data_ptr()
+    for i, x in enumerate(args):
+        assert torch.equal(torch.cat([c[i] for c in a]), x)
+
+
+@pytest.mark.parametrize("size,n", [(10, 4), (3, 3), (8, 8), (1, 1), (50257, 8), (0, 3)])
+def test_chunk_sizes_match_tensor_split(size, n):
+    ref = [t.shape[0] for t in torch.tensor_split(torch.empty(size, device="meta"), n)]
+    assert chunk_sizes(size, n) == ref
+
+
+def test_replicate_and_namedtuple_chunking():
+    """test/test_ir.py:598-680 of the reference (the split part)."""
+    NT = namedtuple("NT", ["my_tensor", "my_integer"])
+    x, nt = torch.randn(5, 3), NT(torch.randn(5, 3), 42)
+    a, k = split_args_kwargs_into_chunks((x,), {"input_nt": nt}, chunks=5, args_chunk_spec=(_Replicate,),
+                                         kwargs_chunk_spec={"input_nt": NT(TensorChunkSpec(0), _Replicate)})
+    assert len(a) == 5 and len(k) == 5
+    for i in range(5):
+        assert a[i][0] is x
+        assert isinstance(k[i]["input_nt"], NT) and k[i]["input_nt"].my_integer == 42
+        assert torch.equal(k[i]["input_nt"].my_tensor, nt.my_tensor[i:i + 1])
+
+
+def test_fewer_rows_than_chunks_shrinks_or_raises():
+    a, k = split_args_kwargs_into_chunks((torch.randn(3, 2),), None, 8)
+    assert len(a) == 3  # first tensor decides (reference microbatch.py:120-129)
+    with pytest.raises(RuntimeError, match="smaller than the number of chunks"):
+        split_args_kwargs_into_chunks((torch.randn(8, 2), torch.randn(3, 2)), None, 8)
+
+
+def test_split_error_types():
+    with pytest.raises(ValueError):
+        split_args_kwargs_into_chunks(((torch.randn(4, 2), torch.randn(4, 2)),), None, 2,
+                                      args_chunk_spec=(TensorChunkSpec(0),))
+    with pytest.raises(TypeError, match="Unrecognized chunk spec"):
+        split_args_kwargs_into_chunks((torch.randn(4, 2),), None, 2, args_chunk_spec=(object(),))
+
+
+def test_debug_mask_layout_on_host():
+    """test/test_ir.py:696-709 of the reference: full-size chunks, zero outside the own slice."""
+    x = torch.randn(5, 3)
+    MB._debug_mask_minibatches = True
+    try:
+        a, _ = split_args_kwargs_into_chunks((x,), None, 5)
+    finally:
+        MB._debug_mask_minibatches = False
+    for i, (c,) in enumerate(a):
+        assert c.shape == x.shape
+        assert torch.equal(c[i:i + 1], x[i:i + 1])
+        assert float(c[:i].abs().sum()) == 0 and float(c[i + 1:].abs().sum()) == 0
+
+
+def test_merge_reducer_and_replicated_leaves_on_host():
+    chunks = [{"loss": torch.tensor(float(i)), "tag": "same"} for i in range(4)]
+    out = merge_chunks(chunks, {"loss": sum_reducer, "tag": None})
+    assert out["tag"] == "same" and float(out["loss"]) == 6.0
+    with pytest.raises(ValueError, match="did not match chunk spec"):
+        merge_chunks([(torch.zeros(1), torch.zeros(1))], (TensorChunkSpec(0),))
+    with pytest.raises(RuntimeError, match="no CPU data path"):
+        merge_chunks([torch.zeros(2, 2), torch.zeros(2, 2)], None)
+
+
+def test_row_view_descriptions():
+    buf = torch.empty(256, 1024, dtype=torch.bfloat16)
+    v = buf.view(2, 128, 1024)[..., :1000]          # padded logits rows
+    assert MB._row_view(v, 0) == (256, 2000, 2048, 256)
+    c = torch.empty(4, 5, 6)
+    assert MB._row_view(c, 0) == (1, 480, 480, 1)
+    assert MB._row_view(c, 1) == (4, 120, 120, 1)
+    assert MB._row_view(torch.empty(4, 6, 5).transpose(1, 2), 0) is None
+
+
+# ---- schedule orders ----------------------------------------------------------------------------------
+def test_1f1b_phases_known_answer():
+    assert [order.one_f_one_b_phases(s, 4, 8) for s in range(4)] == [(6, 2, 6), (4, 4, 4), (2, 6, 2), (0, 8, 0)]
+
+
+@pytest.mark.parametrize("S,M", [(1, 1), (2, 4), (4, 8), (4, 2), (3, 7)])
+def test_rank_programs_equal_the_simulated_reference(S, M):
+    for s in range(S):
+        assert order.gpipe_rank_program(s, M, True) == list(OS.gpipe_rank(s, M))
+        assert order.one_f_one_b_rank_program(s, S, M, True) == list(OS.one_f_one_b_rank(s, S, M))
+        assert order.one_f_one_b_rank_program(s, S, M, False) == list(OS.one_f_one_b_rank(s, S, M, False))
+
+
+@pytest.mark.parametrize("G,n_local,M", [(1, 2, 8), (2, 2, 4), (2, 2, 8), (4, 2, 8), (2, 3, 4)])
+def test_multi_stage_rank_programs_equal_the_simulated_reference(G, n_local, M):
+    S = G * n_local
+    for r in range(G):
+        local = [s for s in range(S) if s % G == r]
+        assert order.interleaved_rank_program(r, G, local, M) == list(OS.interleaved_rank(r, G, local, M))
+        assert order.looped_bfs_rank_program(local, M, True) == list(OS.looped_bfs_rank(local, M))
+
+
+def _invariants(actions, S, M, split=False):
+    pos = {a: i for i, a in enumerate(actions)}
+    assert len(pos) == len(actions)
+    bk = "I" if split else "B"
+    for s in range(S):
+        for m in range(M):
+            if s > 0:
+                assert pos[("F", s - 1, m)] < pos[("F", s, m)]
+            if s < S - 1:
+                assert pos[(bk, s + 1, m)] < pos[(bk, s, m)]
+            assert pos[("F", s, m)] < pos[(bk, s, m)]
+            if split:
+                assert pos[("I", s, m)] < pos[("W", s, m)]
+            if m > 0:
+                assert pos[("F", s, m - 1)] < pos[("F", s, m)]
+                assert pos[(bk, s, m - 1)] < pos[(bk, s, m)]
+                if split:
+                    assert pos[("W", s, m - 1)] < pos[("W", s, m)]
+
+
+@pytest.mark.parametrize("S,M", [(1, 3), (2, 4), (4, 8), (4, 16), (3, 2)])
+def test_merged_orders_respect_dependencies(S, M):
+    progs = [order.one_f_one_b_rank_program(s, S, M, True) for s in range(S)]
+    merged = order.merge_rank_programs(progs, S)
+    assert len(merged) == 2 * S * M
+    _invariants(merged, S, M)
+    zb = order.merge_rank_programs([order.zero_bubble_rank_program(s, S, M) for s in range(S)], S)
+    assert len(zb) == 3 * S * M
+    _invariants(zb, S, M, split=True)
+
+
+def test_merge_detects_deadlock():
+    with pytest.raises(RuntimeError, match="dead-lock"):
+        order.merge_rank_programs([[("B", 0, 0), ("F", 0, 0)]], 1)
+
+
+# ---- front end ------------------------------------------------------------------------------------------
+class _Block(nn.Module):
+    def __init__(self, i, o):
+        super().__init__()
+        self.lin = nn.Linear(i, o)
+
+    def forward(self, x):
+        return torch.relu(self.lin(x))
+
+
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.num_layers = 3
+        prev = 16
+        for i, d in enumerate([16, 32, 8]):
+            self.add_module(f"layer{i}", _Block(prev, d))
+            prev = d
+        self.output_proj = nn.Linear(prev, 4)
+
+    def forward(self, x):
+        for i in range(self.num_layers):
+            x = getattr(self, f"layer{i}")(x)
+        return self.output_proj(x)
+
+
+def test_pipeline_splits_and_keeps_parameter_names():
+    """test/test_pipe.py:78-110 of the reference: stage count, output equality, stage state_dict
+    keys are a partition of the original keys."""
+    torch.manual_seed(0)
+    mod = _Net()
+    x = torch.randn(8, 16)
+    pipe = pp.pipeline(mod, 4, (x,), split_spec={"layer1": pp.SplitPoint.BEGINNING,
+                                                 "layer2": pp.SplitPoint.END})
+    assert pipe.num_stages == 3
+    assert torch.equal(pipe(x), mod(x))
+    old = set(mod.state_dict().keys())
+    seen = set()
+    for i in range(pipe.num_stages):
+        keys = set(pipe.get_stage_module(i).state_dict().keys())
+        assert keys <= old and not (keys & seen)
+        seen |= keys
+    assert seen == old
+    info = pipe.info()
+    assert info.num_stages == 3 and info.num_chunks == 4
+    assert all(lower_stage_module(pipe.get_stage_module(i)) is not None for i in range(3))
+
+
+def test_pipe_split_calls_in_forward():
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = nn.Linear(4, 4), nn.Linear(4, 4)
+
+        def forward(self, x):
+            x = self.a(x)
+            pp.pipe_split()
+            return self.b(x)
+
+    m = M()
+    x = torch.randn(2, 4)
+    pipe = pp.pipeline(m, 2, (x,))
+    assert pipe.num_stages == 2 and torch.equal(pipe(x), m(x))
+
+
+def test_annotate_split_points_and_errors():
+    m = _Net()
+    pp.annotate_split_points(m, {"layer2": pp.SplitPoint.BEGINNING})
+    x = torch.randn(4, 16)
+    ref = m(x)
+    pipe = pp.pipeline(m, 2, (x,))
+    assert pipe.num_stages == 2 and torch.equal(pipe(x), ref)
+    with pytest.raises(ValueError, match="Cannot specify both"):
+        pp.pipeline(_Net(), 2, (x,), split_spec={"layer1": pp.SplitPoint.END}, split_policy=lambda g: g)
+    with pytest.raises(ValueError, match="not a module called"):
+        pp.pipeline(_Net(), 2, (x,), split_spec={"nope": pp.SplitPoint.END})
+    with pytest.raises(ValueError, match="Invalid stage index"):
+        pipe.get_stage_module(5)
+
+
+def test_shared_parameters_are_rejected():
+    class Tied(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = nn.Linear(4, 4, bias=False)
+            self.mid = nn.Linear(4, 4)
+
+        def forward(self, x):
+            x = self.emb(x)
+            pp.pipe_split()
+            return self.emb(self.mid(x))
+
+    with pytest.raises(NotImplementedError, match="shared"):
+        pp.pipeline(Tied(), 2, (torch.randn(2, 4),))
+
+
+def test_chunk_spec_context_managers():
+    """test/test_chunkspec.py:42-62 of the reference."""
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(4, 4)
+
+        def forward(self, x, y, z=None):
+            return self.lin(x) + y + z
+
+    x, y, z = torch.randn(6, 4), torch.randn(6, 4), torch.randn(6, 4)
+    with pp.ArgsChunkSpec((0, 0)), pp.KwargsChunkSpec({"z": 0}):
+        pipe = pp.pipeline(M(), 3, (x, y), {"z": z})
+    info = pipe.info()
+    assert [s.split_dim for s in info.args_chunk_spec] == [0, 0]
+    assert info.kwargs_chunk_spec["z"].split_dim == 0
+    assert pp.Pipe.args_chunk_spec is None and pp.Pipe.kwargs_chunk_spec is None
+
+
+def test_lowering_decisions():
+    from pippy_amd.configs import DecoderLM
+    m = DecoderLM(vocab=64, max_seq=16, dim=64, n_layers=2, n_heads=1, ffn=128)
+    names = [type(b).__name__ for b in lower_stage_module(m)]
+    assert names == ["TokenEmbedding", "TransformerLayer", "TransformerLayer", "LMHead"]
+    assert [type(b).__name__ for b in lower_stage_module(_Net())] == ["LinearAct"] * 4
+
+    class Skip(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = nn.Linear(4, 4)
+
+        def forward(self, x):
+            return x + self.a(x)
+
+    assert lower_stage_module(Skip()) is None  # not a chain: runs through autograd instead
+
+
+# ---- stage / schedule argument checking (reference test_pipeline_schedule.py:477-521) ----------------
+def _host_stages(n):
+    mods = [nn.Linear(4, 4) for _ in range(n)]
+    return [ManualPipelineStage(mods[i], i, n, "cpu", 8, input_args=torch.zeros(1, 4)) for i in range(n)]
+
+
+def test_stage_constructor_errors():
+    with pytest.raises(ValueError, match="out of range"):
+        ManualPipelineStage(nn.Linear(2, 2), 3, 2, "cpu", 4)
+    with pytest.raises(RuntimeError, match="cannot be larger than number of stages"):
+        ManualPipelineStage(nn.Linear(2, 2), 0, 2, "cpu", 4, group=4)
+
+
+def test_schedule_input_checks():
+    sched = pp.Schedule1F1B(_host_stages(1), 8)
+    with pytest.raises(ValueError):
+        sched._step_microbatches([(i,) for i in range(7)])
+    with pytest.raises(TypeError):
+        sched._step_microbatches(torch.ones(8, 4, 8))
+    with pytest.raises(TypeError):
+        sched._step_microbatches([(torch.zeros(1, 4),)] * 8, losses=1)
+    with pytest.raises(ValueError, match="at least two stages"):
+        pp.ScheduleInterleaved1F1B(_host_stages(1), 8)
+    stages = [ManualPipelineStage(nn.Linear(4, 4), i, 4, "cpu", 8, group=2) for i in range(4)]
+    with pytest.raises(ValueError, match="multiple of the number of pipeline ranks"):
+        pp.ScheduleInterleaved1F1B(stages, 7)
+    partial = [ManualPipelineStage(nn.Linear(4, 4), 1, 3, "cpu", 8)]
+    with pytest.raises(RuntimeError, match="every stage must be given"):
+        pp.ScheduleGPipe(partial, 8)._step_microbatches([()] * 8)
+
+
+def test_product_code_never_imports_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "pippy_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), f
+
+
+# ---- C ABI --------------------------------------------------------------------------------------------
+def _header_functions():
+    text = open(os.path.join(ROOT, "include", "pippy_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _header_functions()
+    assert names and set(names) == set(_native.EXPORTED_SYMBOLS)
+    lib = ctypes.CDLL(str(_native.LIB_PATH))
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert _native.lib().pp_abi_version() == 1
+
+
+def test_ctypes_structs_match_the_header(tmp_path):
+    src = tmp_path / "sizes.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "pippy_amd.h"\n'
+                   'int main(void){printf("%zu %zu %zu %zu %zu %zu %zu\\n", sizeof(pp_copy_seg), '
+                   'sizeof(pp_gemm_desc), sizeof(pp_attn_desc), sizeof(pp_op), offsetof(pp_op, i), '
+                   'offsetof(pp_op, j), offsetof(pp_gemm_desc, bias));return 0;}\n')
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
+    N = _native
+    want = [ctypes.sizeof(N.CopySeg), ctypes.sizeof(N.GemmDesc), ctypes.sizeof(N.AttnDesc), ctypes.sizeof(N.Op),
+            N.Op.i.offset, N.Op.j.offset, N.GemmDesc.bias.offset]
+    assert got == want

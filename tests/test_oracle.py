@@ -1,0 +1,206 @@
+"""Pins the CPU oracle: every oracle function is checked against something it did not come from
+(a torch library routine, a closed form, a known-answer vector held by the reference, or an
+invariant), chosen so that a dropped term, a wrong sign or a wrong index fails."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from oracle import microbatch as OM
+from oracle import ops as O
+from oracle import pipeline as OP
+from oracle import schedules as OS
+
+
+# ---- arithmetic statements -------------------------------------------------------------------------
+def test_gelu_forms_match_torch():
+    x = torch.linspace(-6, 6, 2001, dtype=torch.float64)
+    assert torch.allclose(O.gelu_erf(x), F.gelu(x), atol=1e-12)
+    assert torch.allclose(O.gelu_tanh(x), F.gelu(x, approximate="tanh"), atol=1e-12)
+    # special values: gelu(0) = 0, gelu(x) -> x for large x, -> 0 for very negative x
+    assert O.gelu_erf(torch.tensor(0.0)) == 0 and O.gelu_tanh(torch.tensor(0.0)) == 0
+    assert abs(O.gelu_erf(torch.tensor(10.0, dtype=torch.float64)).item() - 10.0) < 1e-12
+
+
+def test_layer_norm_matches_torch_and_is_normalised():
+    torch.manual_seed(0)
+    x = torch.randn(7, 48, dtype=torch.float64) * 3 + 1
+    g, b = torch.randn(48, dtype=torch.float64), torch.randn(48, dtype=torch.float64)
+    assert torch.allclose(O.layer_norm(x, g, b, 1e-5), F.layer_norm(x, (48,), g, b, 1e-5), atol=1e-12)
+    y = O.layer_norm(x, torch.ones(48, dtype=torch.float64), None, 0.0)
+    assert torch.allclose(y.mean(-1), torch.zeros(7, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose((y * y).mean(-1), torch.ones(7, dtype=torch.float64), atol=1e-12)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_matches_sdpa_and_brute_force(causal):
+    torch.manual_seed(1)
+    q, k, v = (torch.randn(2, 3, 9, 4, dtype=torch.float64) for _ in range(3))
+    ref = F.scaled_dot_product_attention(q, k, v, is_causal=causal)
+    assert torch.allclose(O.attention(q, k, v, causal), ref, atol=1e-12)
+    # brute force, one query at a time
+    out = torch.zeros_like(q)
+    for b in range(2):
+        for h in range(3):
+            for i in range(9):
+                n = i + 1 if causal else 9
+                w = torch.tensor([math.exp(float(q[b, h, i] @ k[b, h, j]) / 2.0) for j in range(n)],
+                                 dtype=torch.float64)
+                out[b, h, i] = (w[:, None] * v[b, h, :n]).sum(0) / w.sum()
+    assert torch.allclose(O.attention(q, k, v, causal), out, atol=1e-10)
+    # fused-qkv layout is the same function
+    qkv = torch.cat([t.transpose(1, 2).reshape(2, 9, 12) for t in (q, k, v)], dim=-1)
+    assert torch.allclose(O.attention_fused_qkv(qkv, 3, causal), ref.transpose(1, 2).reshape(2, 9, 12), atol=1e-12)
+
+
+def test_cross_entropy_matches_torch_with_ignore_index():
+    torch.manual_seed(2)
+    logits = torch.randn(11, 17, dtype=torch.float64)
+    target = torch.randint(0, 17, (11,))
+    target[[2, 7]] = -100
+    assert torch.allclose(O.cross_entropy_mean(logits, target), F.cross_entropy(logits, target), atol=1e-12)
+    # uniform logits: loss = log(V)
+    assert abs(O.cross_entropy_mean(torch.zeros(4, 17, dtype=torch.float64), torch.arange(4)).item()
+               - math.log(17)) < 1e-12
+
+
+def test_embedding_matches_torch():
+    torch.manual_seed(3)
+    wte, wpe = torch.randn(20, 6), torch.randn(8, 6)
+    ids = torch.randint(0, 20, (3, 5))
+    ref = F.embedding(ids, wte) + F.embedding(torch.arange(5), wpe)
+    assert torch.equal(O.embedding(ids, wte, wpe), ref)
+
+
+# ---- split / merge / accumulate --------------------------------------------------------------------
+@pytest.mark.parametrize("shape,dim,n", [((128, 512), 0, 2), ((256, 512), 0, 2), ((512, 512), 0, 2),
+                                         ((7, 33, 5), 1, 4), ((3, 10, 17), 2, 3), ((5, 9), 1, 9)])
+def test_numpy_split_merge_match_torch(shape, dim, n):
+    rng = np.random.default_rng(0)
+    x = rng.integers(0, 2 ** 16, size=shape, dtype=np.uint16)
+    chunks = OM.split(x, n, dim)
+    ref = torch.tensor_split(torch.from_numpy(x.astype(np.int32)), n, dim)
+    assert len(chunks) == len(ref)
+    for c, r in zip(chunks, ref):
+        assert c.shape == tuple(r.shape) and np.array_equal(c.astype(np.int32), r.numpy())
+    assert np.array_equal(OM.merge(chunks, dim), x)
+    assert np.array_equal(OM.merge(chunks, dim).astype(np.int32),
+                          torch.cat(list(ref), dim).numpy())
+
+
+def test_split_shapes_held_by_the_reference_test():
+    """test/test_microbatch.py:17-34 of the reference: 128/256/512 rows of 512 in two chunks."""
+    for rows, expect in ((128, 64), (256, 128), (512, 256)):
+        chunks = OM.split(np.zeros((rows, 512), np.float32), 2, 0)
+        assert [c.shape for c in chunks] == [(expect, 512)] * 2
+
+
+def test_chunk_bounds_rule():
+    # first size % n chunks get one more (torch.tensor_split's documented rule)
+    assert [len(r) for r in OM.chunk_bounds(10, 4)] == [3, 3, 2, 2]
+    assert [len(r) for r in OM.chunk_bounds(3, 5)] == [1, 1, 1, 0, 0]
+    assert [len(r) for r in OM.chunk_bounds(8, 8)] == [1] * 8
+
+
+def test_accumulate_fp32_matches_torch_sequence():
+    torch.manual_seed(4)
+    gs = [(torch.randn(1000) * 10.0 ** (m - 2)).to(torch.bfloat16) for m in range(5)]
+    bits = [g.view(torch.int16).numpy().view(np.uint16) for g in gs]
+    acc = OM.accumulate_fp32(bits)
+    ref = gs[0].float().clone()
+    for g in gs[1:]:
+        ref.add_(g.float())
+    assert np.array_equal(acc.view(np.uint32), ref.numpy().view(np.uint32))
+    # order matters in floating point: the reversed order differs somewhere
+    rev = OM.accumulate_fp32(bits[::-1])
+    assert not np.array_equal(rev.view(np.uint32), acc.view(np.uint32))
+
+
+# ---- one pipelined step ----------------------------------------------------------------------------
+class _MLP(nn.Module):
+    def __init__(self, d):
+        super().__init__()
+        self.a, self.b, self.c = nn.Linear(d, d), nn.Linear(d, d), nn.Linear(d, d)
+
+    def forward(self, x):
+        return self.c(torch.relu(self.b(torch.relu(self.a(x)))))
+
+
+def test_pipeline_step_matches_unpipelined_run():
+    """The reference's own relative checks (test_fwd.py:80-84, test_grad.py:103-136): the merged
+    output equals the un-pipelined output, the summed microbatch losses equal the full-batch loss
+    of a sum-reduction loss, and gradients equal the un-pipelined gradients."""
+    import copy
+    torch.manual_seed(5)
+    model = _MLP(16).double()
+    ref = copy.deepcopy(model)
+    x, t = torch.randn(12, 16, dtype=torch.float64), torch.randn(12, 16, dtype=torch.float64)
+    loss_fn = nn.MSELoss(reduction="sum")
+    stages = [nn.Sequential(model.a, nn.ReLU()), nn.Sequential(model.b, nn.ReLU()), nn.Sequential(model.c)]
+    out, losses = OP.step(stages, x, t, 4, loss_fn)
+    ref_out = ref(x)
+    ref_loss = loss_fn(ref_out, t)
+    ref_loss.backward()
+    assert torch.allclose(out, ref_out.detach(), atol=1e-12)
+    assert torch.allclose(sum(losses), ref_loss.detach(), atol=1e-10)
+    for (n, p), (_, rp) in zip(model.named_parameters(), ref.named_parameters()):
+        assert torch.allclose(p.grad, rp.grad, atol=1e-10), n
+    # no 1/M scaling: a mean-reduction loss gives M times the full-batch gradient scale difference
+    assert len(losses) == 4
+
+
+def test_pipeline_step_ragged_batch():
+    torch.manual_seed(6)
+    model = _MLP(8)
+    x = torch.randn(10, 8)
+    out, _ = OP.step([model], x, None, 4, None)
+    assert out.shape == (10, 8) and torch.allclose(out, model(x))
+
+
+# ---- schedule orders --------------------------------------------------------------------------------
+def test_1f1b_phase_table_quoted_by_the_reference():
+    """pippy/PipelineSchedule.py:373-377: 4 stages, 8 microbatches."""
+    table = [OS.one_f_one_b_counts(s, 4, 8) for s in range(4)]
+    assert table == [(6, 2, 6), (4, 4, 4), (2, 6, 2), (0, 8, 0)]
+
+
+def _check_order_invariants(order, S, M):
+    pos = {a: i for i, a in enumerate(order)}
+    assert len(pos) == len(order) == 2 * S * M
+    for s in range(S):
+        for m in range(M):
+            assert ("F", s, m) in pos and ("B", s, m) in pos
+            if s > 0:
+                assert pos[("F", s - 1, m)] < pos[("F", s, m)]
+            if s < S - 1:
+                assert pos[("B", s + 1, m)] < pos[("B", s, m)]
+            assert pos[("F", s, m)] < pos[("B", s, m)]
+            if m > 0:
+                assert pos[("F", s, m - 1)] < pos[("F", s, m)]
+                assert pos[("B", s, m - 1)] < pos[("B", s, m)]
+
+
+@pytest.mark.parametrize("S,M", [(1, 1), (2, 4), (4, 8), (4, 2), (3, 7)])
+def test_simulated_orders_satisfy_pipeline_invariants(S, M):
+    _check_order_invariants(OS.simulate([OS.gpipe_rank(s, M) for s in range(S)], S), S, M)
+    _check_order_invariants(OS.simulate([OS.one_f_one_b_rank(s, S, M) for s in range(S)], S), S, M)
+
+
+@pytest.mark.parametrize("G,n_local,M", [(1, 2, 8), (2, 2, 4), (2, 2, 8), (4, 2, 8), (2, 3, 4)])
+def test_interleaved_and_bfs_orders(G, n_local, M):
+    S = G * n_local
+    local = [[s for s in range(S) if s % G == r] for r in range(G)]
+    _check_order_invariants(OS.simulate([OS.interleaved_rank(r, G, local[r], M) for r in range(G)], S), S, M)
+    _check_order_invariants(OS.simulate([OS.looped_bfs_rank(local[r], M) for r in range(G)], S), S, M)
+
+
+def test_single_rank_interleaved_order():
+    """One rank, two local stages, M = 8: warm-up 1, 15 forward/backward pairs, cool-down 1."""
+    prog = list(OS.interleaved_rank(0, 1, [0, 1], 8))
+    assert prog[:5] == [("F", 0, 0), ("F", 1, 0), ("B", 1, 0), ("F", 0, 1), ("B", 0, 0)]
+    assert prog[-1] == ("B", 0, 7) and len(prog) == 32
+    kinds = "".join(k for k, _, _ in prog)
+    assert kinds == "F" + "FB" * 15 + "B"
