@@ -152,21 +152,23 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs 
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    Stage<BM, AT> sa;
-    Stage<BN, BT> sb;
-    const int64_t nk = (g.K + BK - 1) / BK;
+    BufStage<BM, AT> sa;
+    BufStage<BN, BT> sb;
+    sa.init(g.A, g.lda, m0, g.M, g.K, tid);
+    sb.init(g.B, g.ldb, n0, g.N, g.K, tid);
+    const int nk = (int)((g.K + BK - 1) / BK);
 
-    sa.load(g.A, g.lda, m0, g.M, 0, g.K, tid);
-    sb.load(g.B, g.ldb, n0, g.N, 0, g.K, tid);
-    sa.store(smem, tid);
-    sb.store(smem + BM * BK, tid);
+    sa.load(0);
+    sb.load(0);
+    sa.store(smem);
+    sb.store(smem + BM * BK);
     __syncthreads();
 
-    for (int64_t kt = 0; kt < nk; ++kt) {
-        const int cur = (int)(kt & 1);
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
         if (kt + 1 < nk) {
-            sa.load(g.A, g.lda, m0, g.M, (kt + 1) * BK, g.K, tid);
-            sb.load(g.B, g.ldb, n0, g.N, (kt + 1) * BK, g.K, tid);
+            sa.load((kt + 1) * BK);
+            sb.load((kt + 1) * BK);
         }
         const uint16_t* a_s = smem + cur * kStageElems;
         const uint16_t* b_s = a_s + BM * BK;
@@ -190,8 +192,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs 
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[a], af[b], acc[a][b], 0, 0, 0);
         }
         if (kt + 1 < nk) {
-            sa.store(smem + (cur ^ 1) * kStageElems, tid);
-            sb.store(smem + (cur ^ 1) * kStageElems + BM * BK, tid);
+            sa.store(smem + (cur ^ 1) * kStageElems);
+            sb.store(smem + (cur ^ 1) * kStageElems + BM * BK);
         }
         __syncthreads();
     }
@@ -261,6 +263,13 @@ extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
     if (d->b_trans && (d->N & 7)) return fail(PP_ERR_INVALID, "pp_gemm_bf16: transposed B needs N %% 8 == 0");
     if (d->lda < (d->a_trans ? d->M : d->K) || d->ldb < (d->b_trans ? d->N : d->K) || d->ldc < d->N)
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: leading dimension too small");
+    {
+        // staging uses 32-bit byte offsets from the tile origin
+        const uint64_t a_bytes = (uint64_t)(d->a_trans ? d->K : d->M) * (uint64_t)d->lda * 2;
+        const uint64_t b_bytes = (uint64_t)(d->b_trans ? d->K : d->N) * (uint64_t)d->ldb * 2;
+        if (a_bytes >= 0x7ffffff0ull || b_bytes >= 0x7ffffff0ull)
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: an operand spans 2 GiB or more");
+    }
     const int epi = d->epilogue;
     const bool needs_aux = epi == PP_EPI_BIAS_RESIDUAL || epi == PP_EPI_DGELU_ERF ||
                            epi == PP_EPI_DGELU_TANH || epi == PP_EPI_DRELU;

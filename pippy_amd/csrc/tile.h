@@ -124,4 +124,123 @@ struct Stage<ROWS, true> {
     __device__ __forceinline__ void store(uint16_t* lds, int tid) { sstore_tr<ROWS>(r, lds, tid); }
 };
 
+
+// ---- buffer-resource staging (branch-free global loads) ---------------------------------------
+// Same tiles as above, loaded with raw buffer loads: the hardware range check returns zero for
+// addresses past the end of the operand, so rows (k-contiguous operands) and k indices (transposed
+// operands) beyond the matrix need no branches; 32-bit offsets replace 64-bit address arithmetic.
+// The remaining edge (k tail of a k-contiguous operand, row tail of a transposed one) is masked
+// with selects, and only in tiles that touch it.  Operands must span less than 4 GiB from the tile
+// origin.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint64_t bytes) {
+    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+
+template <int ROWS, bool TR, int NTHREADS = kGemmThreads>
+struct BufStage;
+
+template <int ROWS, int NTHREADS>
+struct BufStage<ROWS, false, NTHREADS> {
+    static constexpr int kChunks = ROWS * 8 / NTHREADS;
+    static_assert(ROWS * 8 % NTHREADS == 0, "tile rows must divide evenly over the lanes");
+    u32x4_t r[kChunks];
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voff[kChunks];
+    int soff[kChunks];
+    int kcol;  // first k of this lane's chunk within a tile
+    int K;
+    __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
+                                         int64_t rows_total, int64_t K_, int tid) {
+        rsrc = make_rsrc(base + row0 * ld, (uint64_t)(rows_total - row0) * (uint64_t)ld * 2);
+        K = (int)K_;
+        kcol = (tid & 7) * 8;
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) {
+            const int id = tid + NTHREADS * i;
+            const int row = id >> 3, ch = id & 7;
+            voff[i] = (int)((row * ld + ch * 8) * 2);
+            soff[i] = row * BK + ((ch ^ swz(row)) << 3);
+        }
+    }
+    __device__ __forceinline__ void load(int k0) {
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i)
+            r[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[i] + k0 * 2, 0, 0);
+        if (k0 + BK > K) {  // k tail: this lane's chunk may lie past K
+            if (k0 + kcol >= K) {
+#pragma unroll
+                for (int i = 0; i < kChunks; ++i) r[i] = u32x4_t{0, 0, 0, 0};
+            }
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t* lds) const {
+#pragma unroll
+        for (int i = 0; i < kChunks; ++i) *reinterpret_cast<u32x4_t*>(lds + soff[i]) = r[i];
+    }
+};
+
+template <int ROWS, int NTHREADS>
+struct BufStage<ROWS, true, NTHREADS> {
+    static constexpr int kHalfBlocks = (BK / 4) * (ROWS / 8);
+    static constexpr int kPer = (kHalfBlocks + NTHREADS - 1) / NTHREADS;
+    u32x4_t r[kPer * 4];
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voff[kPer];
+    int ld2;          // bytes per k row
+    __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
+                                         int64_t rows_total, int64_t K_, int tid) {
+        const uint64_t bytes = ((uint64_t)K_ * (uint64_t)ld - (uint64_t)row0) * 2;
+        // keep the "nothing to load" offset out of range: cap the resource below it
+        rsrc = make_rsrc(base + row0, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
+        ld2 = (int)(ld * 2);
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int id = tid + NTHREADS * i;
+            const int mc = id % (ROWS / 8), kq = id / (ROWS / 8);
+            const bool valid = id < kHalfBlocks && (row0 + mc * 8 < rows_total);
+            // lanes with nothing to load aim past the end of the buffer: the range check returns 0
+            voff[i] = valid ? (int)((kq * 4 * ld + mc * 8) * 2) : (int)0x7ffffff0;
+        }
+    }
+    __device__ __forceinline__ void load(int k0) {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                r[i * 4 + kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[i] + (k0 + kk) * ld2, 0, 0);
+            }
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int id = tid + NTHREADS * i;
+            if (id < kHalfBlocks) {
+                const int mc = id % (ROWS / 8), kq = id / (ROWS / 8);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int w = j >> 1;
+                    const uint32_t x0 = r[i * 4 + 0][w], x1 = r[i * 4 + 1][w];
+                    const uint32_t x2 = r[i * 4 + 2][w], x3 = r[i * 4 + 3][w];
+                    uint2 o;
+                    if (j & 1) {
+                        o.x = (x0 >> 16) | (x1 & 0xffff0000u);
+                        o.y = (x2 >> 16) | (x3 & 0xffff0000u);
+                    } else {
+                        o.x = (x0 & 0xffffu) | (x1 << 16);
+                        o.y = (x2 & 0xffffu) | (x3 << 16);
+                    }
+                    const int row = mc * 8 + j;
+                    *reinterpret_cast<uint2*>(lds + row * BK + (((kq >> 1) ^ swz(row)) << 3) +
+                                              ((kq & 1) << 2)) = o;
+                }
+            }
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t* lds) const { store(lds, threadIdx.x); }
+};
+
 }  // namespace pp
