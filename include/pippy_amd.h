@@ -125,6 +125,13 @@ typedef struct pp_gemm_desc {
  * its contiguous extent (M resp. N) % 8 == 0; ldc, ld_aux % 4 == 0 (bf16) . */
 int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
 
+/* Several independent GEMMs in one launch (up to PP_GEMM_MAX_GROUP; longer lists are split).  All
+ * descriptors must agree in a_trans, b_trans, epilogue and c_dtype.  The weight-gradient GEMMs of
+ * one stage and microbatch (pippy/_backward.py:67-69 reaches them through autograd one by one) are
+ * small but independent of each other: grouped, their tiles fill the GPU together. */
+#define PP_GEMM_MAX_GROUP 16
+int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream);
+
 /* fp32 GEMM with the same descriptor (A, B, C, bias, aux fp32; config 1 of the baseline, the
  * README MLP).  Only a_trans / b_trans, NONE, BIAS, BIAS_RELU, DRELU and ACCUM_F32 epilogues. */
 int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
@@ -227,8 +234,11 @@ enum pp_op_kind {
  *   COPY_ROWS     p: src dst | i: n_rows row_bytes src_stride dst_stride
  *   FILL          p: dst | i: n_bytes | j: value
  *   ACT_BWD       p: dy aux dz | i: n | j: act dtype
- * flags bit 0 (PP_OP_SKIP): the op is stepped over. */
+ * flags bit 0 (PP_OP_SKIP): the op is stepped over.
+ * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
+ * GEMM_BF16 ops next to it (they must not depend on each other). */
 #define PP_OP_SKIP 1
+#define PP_OP_GROUPED 2
 
 typedef struct pp_op {
     int32_t kind;   /* enum pp_op_kind */

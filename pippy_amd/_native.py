@@ -25,6 +25,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD) = range(1, 17)
 OP_SKIP = 1
+OP_GROUPED = 2
 ACT_RELU, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
 
 PP_COPY_MAX_SEGS = 64
@@ -33,7 +34,7 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read",
@@ -100,6 +101,7 @@ def lib() -> C.CDLL:
         "pp_fill_bytes": [vp, i32, i64, vp],
         "pp_gemm_bf16": [C.POINTER(GemmDesc), vp],
         "pp_gemm_f32": [C.POINTER(GemmDesc), vp],
+        "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
         "pp_layernorm_fwd": [vp, vp, vp, vp, vp, vp, i64, i64, f32, vp],
         "pp_layernorm_bwd_input": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp],
@@ -263,6 +265,15 @@ def gemm_bf16(A, B, Cm, **kw) -> None:
     assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16
     d = gemm_desc(A, B, Cm, **kw)
     check(lib().pp_gemm_bf16(C.byref(d), current_stream()), "pp_gemm_bf16")
+
+
+def gemm_bf16_grouped(problems) -> None:
+    """problems: list of (A, B, C, kwargs) sharing layout flags, epilogue and output dtype."""
+    arr = (GemmDesc * len(problems))()
+    for k, (A, B, Cm, kw) in enumerate(problems):
+        d = gemm_desc(A, B, Cm, **kw)
+        C.memmove(C.byref(arr, k * C.sizeof(GemmDesc)), C.byref(d), C.sizeof(GemmDesc))
+    check(lib().pp_gemm_bf16_grouped(arr, len(problems), current_stream()), "pp_gemm_bf16_grouped")
 
 
 def gemm_f32(A, B, Cm, **kw) -> None:

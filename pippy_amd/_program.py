@@ -330,6 +330,8 @@ class Builder:
         self.fused_accumulate = stage_prog.fused_accumulate
         self._scope: List[str] = []
         self._backward: List[Callable] = []
+        self._w_gemm: List[Tuple[N.Op, Optional[str]]] = []
+        self._w_other: List[Tuple[N.Op, Optional[str]]] = []
         self.device = stage_prog.device
 
     # -- naming
@@ -386,18 +388,26 @@ class Builder:
     def i(self, op):
         return self.prog.I.append(op)
 
-    def w(self, op):
-        return self.prog.W.append(op)
+    def w(self, op, tag: Optional[str] = None):
+        """Queues an op of the weight-gradient pass.  ``tag`` names how the op follows the
+        accumulation state: "accum" (its init flag), "beta" (GEMM epilogue accumulate), "fill"
+        (runs only when an accumulation starts)."""
+        self._w_other.append((op, tag))
 
     def w_weight_gemm(self, dY2d, X2d, p, padded=True):
         """dW[out, in] = dY^T X for a linear weight ``p``: bf16/fp32 into staging, or fused fp32
         accumulation."""
+        # all dW GEMMs of a pass only read buffers that the input-gradient pass has finished, so
+        # they are independent of each other: they go first and are marked for grouped launch
         if self.fused_accumulate:
-            k = self.w(op_gemm(dY2d, X2d, self.grad_acc(p, padded), a_trans=True, b_trans=True,
-                               epilogue=N.EPI_ACCUM_F32, beta=1))
-            self.prog.init_toggle_beta.append(k)
+            op = op_gemm(dY2d, X2d, self.grad_acc(p, padded), a_trans=True, b_trans=True,
+                         epilogue=N.EPI_ACCUM_F32, beta=1)
+            op.flags |= N.OP_GROUPED
+            self._w_gemm.append((op, "beta"))
         else:
-            self.w(op_gemm(dY2d, X2d, self.grad_target(p, padded), a_trans=True, b_trans=True))
+            op = op_gemm(dY2d, X2d, self.grad_target(p, padded), a_trans=True, b_trans=True)
+            op.flags |= N.OP_GROUPED
+            self._w_gemm.append((op, None))
 
     def on_backward(self, fn: Callable):
         """Registers the block's backward emitter ``fn(dy, need_dx, dx_out) -> dx``; it runs later,
@@ -489,6 +499,12 @@ class StageProgram:
             if dx_target is not None:
                 assert dy is not None and dy.data_ptr() == dx_target.data_ptr()
             prog.input_grad = dy
+            toggles = {"accum": prog.init_toggle_accum, "beta": prog.init_toggle_beta,
+                       "fill": prog.init_toggle_fill}
+            for op, tag in b._w_gemm + b._w_other:
+                k = prog.W.append(op)
+                if tag is not None:
+                    toggles[tag].append(k)
             # fold this microbatch's staged parameter gradients into the fp32 accumulators
             if not self.fused_accumulate and self.arena.staged_total:
                 n = self.arena.staged_total
@@ -507,7 +523,10 @@ class StageProgram:
         for k in prog.init_toggle_beta:
             prog.W[k].j[4] = 0 if init else 1
         for k in prog.init_toggle_fill:
-            prog.W[k].flags = 0 if init else OP_SKIP
+            if init:
+                prog.W[k].flags &= ~OP_SKIP
+            else:
+                prog.W[k].flags |= OP_SKIP
 
 
 def _like_view(padded_grad: torch.Tensor, out_view: torch.Tensor, padded_out: torch.Tensor) -> torch.Tensor:

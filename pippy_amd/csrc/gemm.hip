@@ -15,6 +15,7 @@
 // output row m, groups of 4 consecutive columns n: stores and epilogue reads are 8-byte vectors.
 #include "tile.h"
 #include "act_math.h"
+#include <vector>
 
 namespace pp {
 
@@ -122,22 +123,21 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t 
 }
 
 // ---- the kernel -----------------------------------------------------------------------------
+extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+
+// XCD-aware remap: consecutive hardware block ids round-robin over the 8 XCDs; give each XCD a
+// contiguous range of tiles so that its private L2 sees a compact set of A/B panels.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t bid, uint32_t grid) {
+    const uint32_t per_xcd = grid >> 3;  // the grid is a multiple of 8
+    return (bid & 7) * per_xcd + (bid >> 3);
+}
+
+// One BM x BN output tile of one problem.
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
-__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs g) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
     constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     constexpr int kStageElems = (BM + BN) * BK;  // one LDS buffer: A tile then B tile
-
-    // XCD-aware remap: consecutive hardware block ids round-robin over the 8 XCDs; give each XCD
-    // a contiguous range of tiles so that its private L2 sees a compact set of A/B panels.
-    uint32_t bid = blockIdx.x;
-    {
-        const uint32_t per_xcd = gridDim.x >> 3;  // gridDim.x is a multiple of 8
-        bid = (bid & 7) * per_xcd + (bid >> 3);
-    }
-    if (bid >= g.n_blocks) return;
-    const uint32_t tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -217,42 +217,138 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs 
 }
 
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
-static int launch_gemm(const GemmArgs& g0, hipStream_t st) {
-    GemmArgs g = g0;
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs g) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks) return;
+    gemm_tile<BM, BN, AT, BT, EPI, CF32>(g, bid % g.tiles_m, bid / g.tiles_m);
+}
+
+// Several independent problems in one grid: the tiles of problem i are the block ids
+// [tile_start[i], tile_start[i + 1]).
+struct GemmGroupArgs {
+    GemmArgs p[PP_GEMM_MAX_GROUP];
+    uint32_t tile_start[PP_GEMM_MAX_GROUP + 1];
+    int n;
+};
+
+template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const GemmGroupArgs ga) {
+    uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= ga.tile_start[ga.n]) return;
+    int i = 0;
+    while (i + 1 < ga.n && bid >= ga.tile_start[i + 1]) ++i;
+    bid -= ga.tile_start[i];
+    const GemmArgs& g = ga.p[i];
+    gemm_tile<BM, BN, AT, BT, EPI, CF32>(g, bid % g.tiles_m, bid / g.tiles_m);
+}
+
+template <typename Kernel>
+static int reserve_lds(Kernel kernel, size_t lds) {
+    const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (rc != hipSuccess)
+        return fail(PP_ERR_LAUNCH, "pp_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(rc));
+    return PP_OK;
+}
+
+template <int BM, int BN>
+static int count_tiles(GemmArgs& g) {
     g.tiles_m = (uint32_t)((g.M + BM - 1) / BM);
     g.tiles_n = (uint32_t)((g.N + BN - 1) / BN);
     const uint64_t nb = (uint64_t)g.tiles_m * g.tiles_n;
-    if (nb > 0x7fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: too many tiles");
+    if (nb > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: too many tiles");
     g.n_blocks = (uint32_t)nb;
-    const uint32_t grid = (uint32_t)((nb + 7) / 8 * 8);
-    const size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
-    static const hipError_t attr_rc = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (attr_rc != hipSuccess)
-        return fail(PP_ERR_LAUNCH, "pp_gemm_bf16: cannot reserve %zu bytes of LDS: %s", lds,
-                    hipGetErrorString(attr_rc));
-    hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
-                       lds, st, g);
-    return check_launch("gemm_bf16_kernel");
+    return PP_OK;
+}
+
+template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
+static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
+    constexpr size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
+    if (n == 1) {
+        GemmArgs g = probs[0];
+        int rc = count_tiles<BM, BN>(g);
+        if (rc) return rc;
+        static const int attr_rc = reserve_lds(&gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>, lds);
+        if (attr_rc) return attr_rc;
+        const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
+        hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+                           lds, st, g);
+        return check_launch("gemm_bf16_kernel");
+    }
+    if constexpr (EPI == PP_EPI_NONE || EPI == PP_EPI_ACCUM_F32) {
+        static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, EPI, CF32>, lds);
+        if (attr_rc) return attr_rc;
+        for (int i0 = 0; i0 < n; i0 += PP_GEMM_MAX_GROUP) {
+            GemmGroupArgs ga;
+            ga.n = (n - i0 < PP_GEMM_MAX_GROUP) ? n - i0 : PP_GEMM_MAX_GROUP;
+            uint64_t total = 0;
+            for (int i = 0; i < ga.n; ++i) {
+                ga.p[i] = probs[i0 + i];
+                int rc = count_tiles<BM, BN>(ga.p[i]);
+                if (rc) return rc;
+                ga.tile_start[i] = (uint32_t)total;
+                total += ga.p[i].n_blocks;
+            }
+            if (total > 0x7fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_grouped: too many tiles");
+            ga.tile_start[ga.n] = (uint32_t)total;
+            if (total == 0) continue;
+            const uint32_t grid = (uint32_t)((total + 7) / 8 * 8);
+            hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid),
+                               dim3(kGemmThreads), lds, st, ga);
+            int rc = check_launch("gemm_bf16_group_kernel");
+            if (rc) return rc;
+        }
+        return PP_OK;
+    } else {
+        // epilogues that chain kernels are launched one by one
+        for (int i = 0; i < n; ++i) {
+            int rc = launch_gemm<BM, BN, AT, BT, EPI, CF32>(probs + i, 1, st);
+            if (rc) return rc;
+        }
+        return PP_OK;
+    }
 }
 
 template <int EPI, bool CF32>
-static int dispatch_layout(const GemmArgs& g, int at, int bt, hipStream_t st) {
-    if (!at && !bt) return launch_gemm<128, 128, false, false, EPI, CF32>(g, st);
-    if (!at && bt) return launch_gemm<128, 128, false, true, EPI, CF32>(g, st);
-    if (at && !bt) return launch_gemm<128, 128, true, false, EPI, CF32>(g, st);
-    return launch_gemm<128, 128, true, true, EPI, CF32>(g, st);
+static int dispatch_layout(const GemmArgs* g, int n, int at, int bt, hipStream_t st) {
+    if (!at && !bt) return launch_gemm<128, 128, false, false, EPI, CF32>(g, n, st);
+    if (!at && bt) return launch_gemm<128, 128, false, true, EPI, CF32>(g, n, st);
+    if (at && !bt) return launch_gemm<128, 128, true, false, EPI, CF32>(g, n, st);
+    return launch_gemm<128, 128, true, true, EPI, CF32>(g, n, st);
 }
 
-}  // namespace pp
+static int dispatch(const GemmArgs* g, int n, int at, int bt, int epi, bool cf32, hipStream_t st) {
+    if (cf32) {
+        switch (epi) {
+            case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, true>(g, n, at, bt, st);
+            case PP_EPI_ACCUM_F32: return dispatch_layout<PP_EPI_ACCUM_F32, true>(g, n, at, bt, st);
+            default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d with fp32 C", epi);
+        }
+    }
+    switch (epi) {
+        case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, false>(g, n, at, bt, st);
+        case PP_EPI_BIAS: return dispatch_layout<PP_EPI_BIAS, false>(g, n, at, bt, st);
+        case PP_EPI_BIAS_GELU_ERF: return dispatch_layout<PP_EPI_BIAS_GELU_ERF, false>(g, n, at, bt, st);
+        case PP_EPI_BIAS_GELU_TANH: return dispatch_layout<PP_EPI_BIAS_GELU_TANH, false>(g, n, at, bt, st);
+        case PP_EPI_BIAS_RESIDUAL: return dispatch_layout<PP_EPI_BIAS_RESIDUAL, false>(g, n, at, bt, st);
+        case PP_EPI_DGELU_ERF: return dispatch_layout<PP_EPI_DGELU_ERF, false>(g, n, at, bt, st);
+        case PP_EPI_DGELU_TANH: return dispatch_layout<PP_EPI_DGELU_TANH, false>(g, n, at, bt, st);
+        case PP_EPI_BIAS_RELU: return dispatch_layout<PP_EPI_BIAS_RELU, false>(g, n, at, bt, st);
+        case PP_EPI_DRELU: return dispatch_layout<PP_EPI_DRELU, false>(g, n, at, bt, st);
+        default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d", epi);
+    }
+}
 
-using namespace pp;
-
-extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
+// Validates one descriptor and converts it to kernel arguments.  Returns PP_OK with *empty set
+// when the problem has no output (M or N zero).
+static int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
+    *empty = false;
     if (!d) return fail(PP_ERR_INVALID, "pp_gemm_bf16: null descriptor");
     if (d->M < 0 || d->N < 0 || d->K < 0) return fail(PP_ERR_INVALID, "pp_gemm_bf16: negative size");
-    if (d->M == 0 || d->N == 0) return PP_OK;
+    if (d->M == 0 || d->N == 0) {
+        *empty = true;
+        return PP_OK;
+    }
     if (!d->A || !d->B || !d->C) return fail(PP_ERR_INVALID, "pp_gemm_bf16: null operand");
     if (!aligned(d->A, 16) || !aligned(d->B, 16))
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: A and B must be 16-byte aligned");
@@ -276,42 +372,53 @@ extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
     if (needs_aux && (!d->aux_in || d->ld_aux < d->N))
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: epilogue %d needs aux_in with ld_aux >= N", epi);
     if (d->aux_out && d->ld_aux < d->N) return fail(PP_ERR_INVALID, "pp_gemm_bf16: ld_aux < N");
-    const bool cf32 = d->c_dtype == PP_F32;
-    if (epi == PP_EPI_ACCUM_F32 && !cf32)
+    if (epi == PP_EPI_ACCUM_F32 && d->c_dtype != PP_F32)
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: PP_EPI_ACCUM_F32 needs an fp32 C");
+    g->A = static_cast<const uint16_t*>(d->A);
+    g->B = static_cast<const uint16_t*>(d->B);
+    g->C = d->C;
+    g->M = d->M; g->N = d->N; g->K = d->K;
+    g->lda = d->lda; g->ldb = d->ldb; g->ldc = d->ldc;
+    g->bias = static_cast<const uint16_t*>(d->bias);
+    g->aux_in = static_cast<const uint16_t*>(d->aux_in);
+    g->aux_out = static_cast<uint16_t*>(d->aux_out);
+    g->ld_aux = d->ld_aux;
+    g->beta = d->beta;
+    g->tiles_m = g->tiles_n = g->n_blocks = 0;
+    return PP_OK;
+}
 
+}  // namespace pp
+
+using namespace pp;
+
+extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
     GemmArgs g;
-    g.A = static_cast<const uint16_t*>(d->A);
-    g.B = static_cast<const uint16_t*>(d->B);
-    g.C = d->C;
-    g.M = d->M; g.N = d->N; g.K = d->K;
-    g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc;
-    g.bias = static_cast<const uint16_t*>(d->bias);
-    g.aux_in = static_cast<const uint16_t*>(d->aux_in);
-    g.aux_out = static_cast<uint16_t*>(d->aux_out);
-    g.ld_aux = d->ld_aux;
-    g.beta = d->beta;
-    g.tiles_m = g.tiles_n = g.n_blocks = 0;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const int at = d->a_trans ? 1 : 0, bt = d->b_trans ? 1 : 0;
+    bool empty;
+    int rc = convert(d, &g, &empty);
+    if (rc || empty) return rc;
+    return dispatch(&g, 1, d->a_trans ? 1 : 0, d->b_trans ? 1 : 0, d->epilogue, d->c_dtype == PP_F32,
+                    static_cast<hipStream_t>(stream));
+}
 
-    if (cf32) {
-        switch (epi) {
-            case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, true>(g, at, bt, st);
-            case PP_EPI_ACCUM_F32: return dispatch_layout<PP_EPI_ACCUM_F32, true>(g, at, bt, st);
-            default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d with fp32 C", epi);
-        }
+extern "C" int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream) {
+    if (n < 0 || (n > 0 && !descs)) return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped: bad list");
+    if (n == 0) return PP_OK;
+    std::vector<GemmArgs> probs;
+    probs.reserve(n);
+    const pp_gemm_desc& f = descs[0];
+    for (int i = 0; i < n; ++i) {
+        const pp_gemm_desc& d = descs[i];
+        if ((d.a_trans != 0) != (f.a_trans != 0) || (d.b_trans != 0) != (f.b_trans != 0) ||
+            d.epilogue != f.epilogue || d.c_dtype != f.c_dtype)
+            return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped: problem %d differs in layout, epilogue or dtype", i);
+        GemmArgs g;
+        bool empty;
+        int rc = convert(&d, &g, &empty);
+        if (rc) return rc;
+        if (!empty) probs.push_back(g);
     }
-    switch (epi) {
-        case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, false>(g, at, bt, st);
-        case PP_EPI_BIAS: return dispatch_layout<PP_EPI_BIAS, false>(g, at, bt, st);
-        case PP_EPI_BIAS_GELU_ERF: return dispatch_layout<PP_EPI_BIAS_GELU_ERF, false>(g, at, bt, st);
-        case PP_EPI_BIAS_GELU_TANH: return dispatch_layout<PP_EPI_BIAS_GELU_TANH, false>(g, at, bt, st);
-        case PP_EPI_BIAS_RESIDUAL: return dispatch_layout<PP_EPI_BIAS_RESIDUAL, false>(g, at, bt, st);
-        case PP_EPI_DGELU_ERF: return dispatch_layout<PP_EPI_DGELU_ERF, false>(g, at, bt, st);
-        case PP_EPI_DGELU_TANH: return dispatch_layout<PP_EPI_DGELU_TANH, false>(g, at, bt, st);
-        case PP_EPI_BIAS_RELU: return dispatch_layout<PP_EPI_BIAS_RELU, false>(g, at, bt, st);
-        case PP_EPI_DRELU: return dispatch_layout<PP_EPI_DRELU, false>(g, at, bt, st);
-        default: return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: epilogue %d", epi);
-    }
+    if (probs.empty()) return PP_OK;
+    return dispatch(probs.data(), (int)probs.size(), f.a_trans ? 1 : 0, f.b_trans ? 1 : 0, f.epilogue,
+                    f.c_dtype == PP_F32, static_cast<hipStream_t>(stream));
 }

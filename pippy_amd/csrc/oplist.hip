@@ -6,17 +6,36 @@
 
 using namespace pp;
 
+static pp_gemm_desc gemm_desc_of(const pp_op& op) {
+    pp_gemm_desc d;
+    d.A = op.p[0]; d.B = op.p[1]; d.C = op.p[2];
+    d.bias = op.p[3]; d.aux_in = op.p[4]; d.aux_out = op.p[5];
+    d.M = op.i[0]; d.N = op.i[1]; d.K = op.i[2];
+    d.lda = op.i[3]; d.ldb = op.i[4]; d.ldc = op.i[5]; d.ld_aux = op.i[6];
+    d.a_trans = op.j[0]; d.b_trans = op.j[1]; d.epilogue = op.j[2]; d.c_dtype = op.j[3];
+    d.beta = op.j[4]; d.reserved = 0;
+    return d;
+}
+
+// Number of ops starting at ops[i] that can go into one grouped GEMM launch (0: not groupable).
+static int group_length(const pp_op* ops, int i, int n_ops) {
+    const pp_op& f = ops[i];
+    if (f.kind != PP_OP_GEMM_BF16 || !(f.flags & PP_OP_GROUPED) || (f.flags & PP_OP_SKIP)) return 0;
+    int len = 1;
+    while (i + len < n_ops) {
+        const pp_op& o = ops[i + len];
+        if (o.kind != PP_OP_GEMM_BF16 || !(o.flags & PP_OP_GROUPED) || (o.flags & PP_OP_SKIP)) break;
+        if (o.j[0] != f.j[0] || o.j[1] != f.j[1] || o.j[2] != f.j[2] || o.j[3] != f.j[3]) break;
+        ++len;
+    }
+    return len;
+}
+
 static int run_one(const pp_op& op, pp_stream st) {
     switch (op.kind) {
         case PP_OP_GEMM_BF16:
         case PP_OP_GEMM_F32: {
-            pp_gemm_desc d;
-            d.A = op.p[0]; d.B = op.p[1]; d.C = op.p[2];
-            d.bias = op.p[3]; d.aux_in = op.p[4]; d.aux_out = op.p[5];
-            d.M = op.i[0]; d.N = op.i[1]; d.K = op.i[2];
-            d.lda = op.i[3]; d.ldb = op.i[4]; d.ldc = op.i[5]; d.ld_aux = op.i[6];
-            d.a_trans = op.j[0]; d.b_trans = op.j[1]; d.epilogue = op.j[2]; d.c_dtype = op.j[3];
-            d.beta = op.j[4]; d.reserved = 0;
+            const pp_gemm_desc d = gemm_desc_of(op);
             return op.kind == PP_OP_GEMM_BF16 ? pp_gemm_bf16(&d, st) : pp_gemm_f32(&d, st);
         }
         case PP_OP_COLSUM:
@@ -175,24 +194,35 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PP_ERR_INVALID, "pp_run_ops: bad list");
     for (int i = 0; i < n_ops; ++i) {
         if (ops[i].flags & PP_OP_SKIP) continue;
+        const int glen = group_length(ops, i, n_ops);
         ProfRecord* rec = nullptr;
         if (g_prof_on) {
             if (g_prof_used < g_prof.size()) {
                 rec = &g_prof[g_prof_used++];
                 rec->kind = ops[i].kind;
                 rec->work = op_work(ops[i]);
+                for (int q = 1; q < glen; ++q) rec->work += op_work(ops[i + q]);
                 (void)hipEventRecord(rec->a, static_cast<hipStream_t>(stream));
             } else {
                 ++g_prof_dropped;
             }
         }
-        const int rc = run_one(ops[i], stream);
+        int rc;
+        if (glen > 1) {
+            std::vector<pp_gemm_desc> descs;
+            descs.reserve(glen);
+            for (int q = 0; q < glen; ++q) descs.push_back(gemm_desc_of(ops[i + q]));
+            rc = pp_gemm_bf16_grouped(descs.data(), glen, stream);
+        } else {
+            rc = run_one(ops[i], stream);
+        }
         if (rec) (void)hipEventRecord(rec->b, static_cast<hipStream_t>(stream));
         if (rc != PP_OK) {
             char msg[400];
             snprintf(msg, sizeof msg, "%s", pp_last_error());
             return fail(rc, "pp_run_ops: op %d (kind %d): %s", i, ops[i].kind, msg);
         }
+        if (glen > 1) i += glen - 1;
     }
     return PP_OK;
 }

@@ -62,9 +62,8 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
         # fp32 stages are small: ones[1, T] @ dY through the fp32 GEMM is an ordered column sum
         ones = b.sp.ones_f32(dY2d.shape[0])
         if b.fused_accumulate:
-            k = b.w(P.op_gemm(ones, dY2d, b.grad_acc(lin.bias).view(1, -1), b_trans=True,
-                              epilogue=N.EPI_ACCUM_F32, beta=1))
-            b.prog.init_toggle_beta.append(k)
+            b.w(P.op_gemm(ones, dY2d, b.grad_acc(lin.bias).view(1, -1), b_trans=True,
+                          epilogue=N.EPI_ACCUM_F32, beta=1), tag="beta")
         else:
             b.w(P.op_gemm(ones, dY2d, b.grad_target(lin.bias).view(1, -1), b_trans=True))
         return
@@ -73,7 +72,7 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
     if b.fused_accumulate:
         tmp = b.scratch("colsum_out", (Nn,), torch.float32)
         b.w(P.op_colsum(dY2d, tmp, ws))
-        b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(lin.bias), tmp)))
+        b.w(P.op_accum(b.grad_acc(lin.bias), tmp), tag="accum")
     else:
         b.w(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
 
@@ -113,9 +112,9 @@ def layernorm_backward(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d, mean, r
         dg = b.scratch("ln_dg", (Cc,), torch.float32)
         db = b.scratch("ln_db", (Cc,), torch.float32)
         b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, dg, db if has_bias else None, ws))
-        b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(ln.weight), dg)))
+        b.w(P.op_accum(b.grad_acc(ln.weight), dg), tag="accum")
         if has_bias:
-            b.prog.init_toggle_accum.append(b.w(P.op_accum(b.grad_acc(ln.bias), db)))
+            b.w(P.op_accum(b.grad_acc(ln.bias), db), tag="accum")
     else:
         b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
                                b.grad_target(ln.bias) if has_bias else None, ws))
@@ -231,8 +230,8 @@ class TokenEmbedding(NativeBlock):
         def bwd(dy, need_dx, dx_out):
             # scatter-add straight into the fp32 accumulators (zeroed on the first accumulation)
             acc_wte, acc_wpe = b.grad_acc(self.wte.weight), b.grad_acc(self.wpe.weight)
-            b.prog.init_toggle_fill.append(b.w(P.op_fill(acc_wte)))
-            b.prog.init_toggle_fill.append(b.w(P.op_fill(acc_wpe)))
+            b.w(P.op_fill(acc_wte), tag="fill")
+            b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S))
             return None
 
