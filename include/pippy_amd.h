@@ -148,6 +148,26 @@ int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, 
 int pp_activation_bwd(const void* dy, const void* aux, void* dz, int64_t n, int act, int dtype,
                       pp_stream stream);
 
+/* Column reductions of one weight-gradient pass in two launches.  Per descriptor:
+ *   out_sum[c] = sum_r dy[r, c]                                   (bias gradient / dbeta), and, if
+ *   out_dot is non-null, out_dot[c] = sum_r dy[r, c] * (x[r, c] - mean[r]) * rstd[r]   (dgamma).
+ * workspace: fp32 [2, ceil(rows / 128), C] per descriptor, distinct between descriptors.  Sums are
+ * formed in a fixed order, so results do not depend on scheduling. */
+typedef struct pp_colreduce_desc {
+    const void* dy;      /* bf16 [rows, C] with row stride ld_dy */
+    const void* x;       /* bf16 [rows, C] contiguous, or null */
+    const float* mean;   /* fp32 [rows] (with x) */
+    const float* rstd;   /* fp32 [rows] (with x) */
+    void* out_sum;       /* [C] or null */
+    void* out_dot;       /* [C] or null */
+    float* workspace;
+    int64_t ld_dy, rows, C;
+    int32_t out_dtype;   /* PP_BF16 or PP_F32 */
+    int32_t reserved;
+} pp_colreduce_desc;
+#define PP_COLREDUCE_MAX_GROUP 24
+int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_stream stream);
+
 /* ------------------------------------------------------------------------------------------
  * LayerNorm (F.layer_norm inside the stage module; backward via pippy/_backward.py:67-69).
  * x, y, dy, dx: bf16 [rows, C]; gamma, beta: bf16 [C]; mean, rstd: fp32 [rows].
@@ -236,7 +256,8 @@ enum pp_op_kind {
  *   ACT_BWD       p: dy aux dz | i: n | j: act dtype
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
- * GEMM_BF16 ops next to it (they must not depend on each other). */
+ * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped
+ * COLSUM / LN_BWD_WEIGHT ops run as one pp_colreduce_grouped call (distinct workspaces needed). */
 #define PP_OP_SKIP 1
 #define PP_OP_GROUPED 2
 

@@ -34,7 +34,7 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read",
@@ -54,6 +54,13 @@ class GemmDesc(C.Structure):
                 ("epilogue", C.c_int32), ("c_dtype", C.c_int32),
                 ("bias", C.c_void_p), ("aux_in", C.c_void_p), ("aux_out", C.c_void_p),
                 ("ld_aux", C.c_int64), ("beta", C.c_int32), ("reserved", C.c_int32)]
+
+
+class ColReduceDesc(C.Structure):
+    _fields_ = [("dy", C.c_void_p), ("x", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p),
+                ("out_sum", C.c_void_p), ("out_dot", C.c_void_p), ("workspace", C.c_void_p),
+                ("ld_dy", C.c_int64), ("rows", C.c_int64), ("C", C.c_int64),
+                ("out_dtype", C.c_int32), ("reserved", C.c_int32)]
 
 
 class AttnDesc(C.Structure):
@@ -103,6 +110,7 @@ def lib() -> C.CDLL:
         "pp_gemm_f32": [C.POINTER(GemmDesc), vp],
         "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
+        "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],
         "pp_layernorm_fwd": [vp, vp, vp, vp, vp, vp, i64, i64, f32, vp],
         "pp_layernorm_bwd_input": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp],
         "pp_layernorm_bwd_weight": [vp, vp, vp, vp, vp, vp, i32, vp, i64, i64, vp],
@@ -290,6 +298,22 @@ def colsum(dY: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor) -> None
     check(lib().pp_colsum_bf16(dY.data_ptr(), M, N, dY.stride(0), out.data_ptr(),
                                PP_F32 if out.dtype == torch.float32 else PP_BF16,
                                workspace.data_ptr(), current_stream()), "pp_colsum_bf16")
+
+
+def colreduce_grouped(items) -> None:
+    """items: dicts with dy, out_sum and/or out_dot, workspace and, for out_dot, x, mean, rstd."""
+    arr = (ColReduceDesc * len(items))()
+    for d, it in zip(arr, items):
+        dy = it["dy"]
+        require_cuda(dy, it.get("x"), it.get("out_sum"), it.get("out_dot"), it["workspace"])
+        d.dy, d.ld_dy, d.rows, d.C = dy.data_ptr(), dy.stride(0), dy.shape[0], dy.shape[1]
+        d.x, d.mean, d.rstd = ptr(it.get("x")), ptr(it.get("mean")), ptr(it.get("rstd"))
+        d.out_sum, d.out_dot = ptr(it.get("out_sum")), ptr(it.get("out_dot"))
+        d.workspace = it["workspace"].data_ptr()
+        assert it["workspace"].numel() >= 2 * ((dy.shape[0] + 127) // 128) * dy.shape[1]
+        out = it.get("out_sum") if it.get("out_sum") is not None else it.get("out_dot")
+        d.out_dtype = PP_F32 if out.dtype == torch.float32 else PP_BF16
+    check(lib().pp_colreduce_grouped(arr, len(items), current_stream()), "pp_colreduce_grouped")
 
 
 # ---- LayerNorm --------------------------------------------------------------------------------

@@ -127,7 +127,7 @@ def op_gemm(A, B, Cm, *, a_trans=False, b_trans=False, epilogue=N.EPI_NONE, bias
 
 def op_colsum(dY, out, ws) -> N.Op:
     M, Nn = dY.shape
-    assert dY.stride(1) == 1 and out.numel() == Nn and ws.numel() >= ((M + 127) // 128) * Nn
+    assert dY.stride(1) == 1 and out.numel() == Nn and ws.numel() >= 2 * ((M + 127) // 128) * Nn
     op = N.Op()
     op.kind = N.OP_COLSUM
     op.p[0], op.p[1], op.p[2] = dY.data_ptr(), out.data_ptr(), ws.data_ptr()
@@ -331,6 +331,7 @@ class Builder:
         self._scope: List[str] = []
         self._backward: List[Callable] = []
         self._w_gemm: List[Tuple[N.Op, Optional[str]]] = []
+        self._w_reduce: List[Tuple[N.Op, Optional[str]]] = []
         self._w_other: List[Tuple[N.Op, Optional[str]]] = []
         self.device = stage_prog.device
 
@@ -363,6 +364,17 @@ class Builder:
         if self.sp.split_backward:
             return self.act("grad:" + name, shape, dtype)
         return self.sp.shared(self._key("grad:" + name), shape, dtype or self.sp.act_dtype)
+
+    def workspace(self, name, shape, dtype) -> torch.Tensor:
+        """Stage-shared workspace with a name of its own (for ops that run concurrently with
+        others in a grouped launch and therefore cannot share scratch)."""
+        return self.sp.shared("ws:" + name, shape, dtype)
+
+    def w_reduce(self, op):
+        """Queues a column reduction of the weight-gradient pass; all of them run grouped, after
+        the grouped dW GEMMs."""
+        op.flags |= N.OP_GROUPED
+        self._w_reduce.append((op, None))
 
     def scratch(self, name, shape, dtype) -> torch.Tensor:
         """Workspace valid inside one kernel sequence (never carried across passes)."""
@@ -501,7 +513,7 @@ class StageProgram:
             prog.input_grad = dy
             toggles = {"accum": prog.init_toggle_accum, "beta": prog.init_toggle_beta,
                        "fill": prog.init_toggle_fill}
-            for op, tag in b._w_gemm + b._w_other:
+            for op, tag in b._w_gemm + b._w_reduce + b._w_other:
                 k = prog.W.append(op)
                 if tag is not None:
                     toggles[tag].append(k)

@@ -199,6 +199,101 @@ __global__ __launch_bounds__(256) void colreduce_final_kernel(const float* __res
     else static_cast<uint16_t*>(out)[c] = f32_to_bf16(t);
 }
 
+// ---- grouped column reductions -------------------------------------------------------------------
+// All bias-gradient and LayerNorm weight-gradient reductions of one weight-gradient pass in two
+// launches (partials, then ordered final sums) instead of two or three tiny launches each.
+constexpr int kMaxColGroup = PP_COLREDUCE_MAX_GROUP;
+
+struct ColDesc {
+    const uint16_t* dy;
+    const uint16_t* x;
+    const float* mean;
+    const float* rstd;
+    void* out_sum;
+    void* out_dot;
+    float* ws;       // [2][n_part][C]: sums, then dots
+    int64_t ld_dy;
+    int rows, C, n_part, n_cb, out_f32;
+};
+
+struct ColGroupArgs {
+    ColDesc d[kMaxColGroup];
+    uint32_t part_start[kMaxColGroup + 1];   // block ranges of the partial kernel
+    uint32_t final_start[kMaxColGroup + 1];  // block ranges of the final kernel
+    int n;
+};
+
+__global__ __launch_bounds__(256) void colgroup_partial_kernel(const ColGroupArgs ga) {
+    __shared__ float red[8][32][8 + 1];
+    uint32_t b = blockIdx.x;
+    int i = 0;
+    while (i + 1 < ga.n && b >= ga.part_start[i + 1]) ++i;
+    b -= ga.part_start[i];
+    const ColDesc& d = ga.d[i];
+    const int rb = b / d.n_cb, cb = b % d.n_cb;
+    const int cc = threadIdx.x & 31, rp = threadIdx.x >> 5;
+    const int col0 = cb * 256 + cc * 8;
+    const int row_begin = rb * 128;
+    const bool with_x = d.x != nullptr;
+    float sg[8] = {0, 0, 0, 0, 0, 0, 0, 0}, sb[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (col0 < d.C) {
+        for (int it = 0; it < 16; ++it) {
+            const int r = row_begin + it * 8 + rp;
+            if (r < d.rows) {
+                const uint4 dw = *reinterpret_cast<const uint4*>(d.dy + (int64_t)r * d.ld_dy + col0);
+                const float df[8] = {bf16lo(dw.x), bf16hi(dw.x), bf16lo(dw.y), bf16hi(dw.y),
+                                     bf16lo(dw.z), bf16hi(dw.z), bf16lo(dw.w), bf16hi(dw.w)};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sb[e] += df[e];
+                if (with_x) {
+                    const float mean = d.mean[r], rstd = d.rstd[r];
+                    const uint4 xw = *reinterpret_cast<const uint4*>(d.x + (int64_t)r * d.C + col0);
+                    const float xf[8] = {bf16lo(xw.x), bf16hi(xw.x), bf16lo(xw.y), bf16hi(xw.y),
+                                         bf16lo(xw.z), bf16hi(xw.z), bf16lo(xw.w), bf16hi(xw.w)};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sg[e] += df[e] * ((xf[e] - mean) * rstd);
+                }
+            }
+        }
+    }
+    for (int pass = 0; pass < (with_x ? 2 : 1); ++pass) {
+        const float* s = pass == 0 ? sb : sg;
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[rp][cc][e] = s[e];
+        __syncthreads();
+        if (rp == 0 && col0 < d.C) {
+            float* out = d.ws + ((int64_t)pass * d.n_part + rb) * d.C + col0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = 0.f;
+#pragma unroll
+                for (int p = 0; p < 8; ++p) t += red[p][cc][e];
+                out[e] = t;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void colgroup_final_kernel(const ColGroupArgs ga) {
+    uint32_t b = blockIdx.x;
+    int i = 0;
+    while (i + 1 < ga.n && b >= ga.final_start[i + 1]) ++i;
+    b -= ga.final_start[i];
+    const ColDesc& d = ga.d[i];
+    const int c = b * 256 + threadIdx.x;
+    if (c >= d.C) return;
+    for (int pass = 0; pass < 2; ++pass) {
+        void* out = pass == 0 ? d.out_sum : d.out_dot;
+        if (!out || (pass == 1 && !d.x)) continue;
+        const float* part = d.ws + (int64_t)pass * d.n_part * d.C;
+        float t = 0.f;
+        for (int p = 0; p < d.n_part; ++p) t += part[(int64_t)p * d.C + c];
+        if (d.out_f32) static_cast<float*>(out)[c] = t;
+        else static_cast<uint16_t*>(out)[c] = f32_to_bf16(t);
+    }
+}
+
 template <int NV>
 static void launch_ln_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
                           float* rstd, int64_t rows, int C, float eps, hipStream_t st) {
@@ -310,4 +405,46 @@ extern "C" int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, 
     hipLaunchKernelGGL(colreduce_final_kernel, dim3((uint32_t)((N + 255) / 256)), dim3(256), 0, st,
                        workspace, n_part, N, out, out_dtype == PP_F32);
     return check_launch("colsum");
+}
+
+extern "C" int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_stream stream) {
+    if (n < 0 || (n > 0 && !descs)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: bad list");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (int i0 = 0; i0 < n; i0 += kMaxColGroup) {
+        ColGroupArgs ga;
+        ga.n = 0;
+        uint64_t pb = 0, fb = 0;
+        const int cnt = (n - i0 < kMaxColGroup) ? n - i0 : kMaxColGroup;
+        for (int i = 0; i < cnt; ++i) {
+            const pp_colreduce_desc& s = descs[i0 + i];
+            if (s.rows < 0 || s.C <= 0 || s.ld_dy < s.C) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: bad shape in %d", i0 + i);
+            if ((s.C % 8) || (s.ld_dy % 8)) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: C and ld must be multiples of 8");
+            if (!s.dy || !s.workspace || (!s.out_sum && !s.out_dot)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: null pointer in %d", i0 + i);
+            if (s.out_dot && (!s.x || !s.mean || !s.rstd)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: out_dot needs x, mean, rstd");
+            if (!aligned(s.dy, 16) || !aligned(s.x, 16)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: dy and x must be 16-byte aligned");
+            if (s.rows > 0x7fffffff || s.C > 0x7fffffff) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: shape too large");
+            ColDesc& d = ga.d[ga.n];
+            d.dy = static_cast<const uint16_t*>(s.dy);
+            d.x = s.out_dot ? static_cast<const uint16_t*>(s.x) : nullptr;
+            d.mean = s.mean; d.rstd = s.rstd;
+            d.out_sum = s.out_sum; d.out_dot = s.out_dot;
+            d.ws = s.workspace;
+            d.ld_dy = s.ld_dy;
+            d.rows = (int)s.rows; d.C = (int)s.C;
+            d.n_part = (int)((s.rows + 127) / 128);
+            d.n_cb = (int)((s.C + 255) / 256);
+            d.out_f32 = s.out_dtype == PP_F32;
+            ga.part_start[ga.n] = (uint32_t)pb;
+            ga.final_start[ga.n] = (uint32_t)fb;
+            pb += (uint64_t)d.n_part * d.n_cb;
+            fb += (uint64_t)d.n_cb;
+            ++ga.n;
+        }
+        if (pb > 0x7fffffffull) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: too many blocks");
+        ga.part_start[ga.n] = (uint32_t)pb;
+        ga.final_start[ga.n] = (uint32_t)fb;
+        if (pb) hipLaunchKernelGGL(colgroup_partial_kernel, dim3((uint32_t)pb), dim3(256), 0, st, ga);
+        if (fb) hipLaunchKernelGGL(colgroup_final_kernel, dim3((uint32_t)fb), dim3(256), 0, st, ga);
+    }
+    return check_launch("colreduce_grouped");
 }

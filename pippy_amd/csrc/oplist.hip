@@ -31,6 +31,37 @@ static int group_length(const pp_op* ops, int i, int n_ops) {
     return len;
 }
 
+static bool is_colreduce(const pp_op& o) {
+    return (o.kind == PP_OP_COLSUM || o.kind == PP_OP_LN_BWD_WEIGHT) && (o.flags & PP_OP_GROUPED) &&
+           !(o.flags & PP_OP_SKIP);
+}
+
+static int colreduce_group_length(const pp_op* ops, int i, int n_ops) {
+    if (!is_colreduce(ops[i])) return 0;
+    int len = 1;
+    while (i + len < n_ops && is_colreduce(ops[i + len])) ++len;
+    return len;
+}
+
+static pp_colreduce_desc colreduce_desc_of(const pp_op& op) {
+    pp_colreduce_desc d;
+    if (op.kind == PP_OP_COLSUM) {
+        d.dy = op.p[0]; d.x = nullptr; d.mean = nullptr; d.rstd = nullptr;
+        d.out_sum = op.p[1]; d.out_dot = nullptr;
+        d.workspace = static_cast<float*>(op.p[2]);
+        d.rows = op.i[0]; d.C = op.i[1]; d.ld_dy = op.i[2];
+    } else {
+        d.dy = op.p[0]; d.x = op.p[1];
+        d.mean = static_cast<const float*>(op.p[2]); d.rstd = static_cast<const float*>(op.p[3]);
+        d.out_dot = op.p[4]; d.out_sum = op.p[5];
+        d.workspace = static_cast<float*>(op.p[6]);
+        d.rows = op.i[0]; d.C = op.i[1]; d.ld_dy = op.i[1];
+    }
+    d.out_dtype = op.j[0];
+    d.reserved = 0;
+    return d;
+}
+
 static int run_one(const pp_op& op, pp_stream st) {
     switch (op.kind) {
         case PP_OP_GEMM_BF16:
@@ -194,7 +225,9 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     if (n_ops < 0 || (n_ops > 0 && !ops)) return fail(PP_ERR_INVALID, "pp_run_ops: bad list");
     for (int i = 0; i < n_ops; ++i) {
         if (ops[i].flags & PP_OP_SKIP) continue;
-        const int glen = group_length(ops, i, n_ops);
+        int glen = group_length(ops, i, n_ops);
+        const int clen = glen ? 0 : colreduce_group_length(ops, i, n_ops);
+        if (clen > 1) glen = clen;
         ProfRecord* rec = nullptr;
         if (g_prof_on) {
             if (g_prof_used < g_prof.size()) {
@@ -208,7 +241,12 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
             }
         }
         int rc;
-        if (glen > 1) {
+        if (clen > 1) {
+            std::vector<pp_colreduce_desc> descs;
+            descs.reserve(clen);
+            for (int q = 0; q < clen; ++q) descs.push_back(colreduce_desc_of(ops[i + q]));
+            rc = pp_colreduce_grouped(descs.data(), clen, stream);
+        } else if (glen > 1) {
             std::vector<pp_gemm_desc> descs;
             descs.reserve(glen);
             for (int q = 0; q < glen; ++q) descs.push_back(gemm_desc_of(ops[i + q]));

@@ -68,13 +68,14 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
             b.w(P.op_gemm(ones, dY2d, b.grad_target(lin.bias).view(1, -1), b_trans=True))
         return
     M, Nn = dY2d.shape
-    ws = b.scratch("colsum", (((M + 127) // 128) * Nn,), torch.float32)
+    # reductions of one pass run as one grouped launch: every op needs a workspace of its own
+    ws = b.workspace("colsum:" + str(id(lin)), (2 * ((M + 127) // 128) * Nn,), torch.float32)
     if b.fused_accumulate:
-        tmp = b.scratch("colsum_out", (Nn,), torch.float32)
-        b.w(P.op_colsum(dY2d, tmp, ws))
+        tmp = b.workspace("colsum_out:" + str(id(lin)), (Nn,), torch.float32)
+        b.w_reduce(P.op_colsum(dY2d, tmp, ws))
         b.w(P.op_accum(b.grad_acc(lin.bias), tmp), tag="accum")
     else:
-        b.w(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
+        b.w_reduce(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
 
 
 def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, dY2d: torch.Tensor, *,
@@ -106,18 +107,18 @@ def layernorm_backward(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d, mean, r
     T, Cc = x2d.shape
     dx = dx_out if dx_out is not None else b.grad(name + ".dx", (T, Cc))
     b.i(P.op_ln_bwd_input(dy2d, x2d, b.weight(ln.weight), mean, rstd, dres, dx))
-    ws = b.scratch("ln_bwd", (2 * ((T + 127) // 128) * Cc,), torch.float32)
+    ws = b.workspace("ln_bwd:" + str(id(ln)), (2 * ((T + 127) // 128) * Cc,), torch.float32)
     has_bias = ln.bias is not None
     if b.fused_accumulate:
-        dg = b.scratch("ln_dg", (Cc,), torch.float32)
-        db = b.scratch("ln_db", (Cc,), torch.float32)
-        b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, dg, db if has_bias else None, ws))
+        dg = b.workspace("ln_dg:" + str(id(ln)), (Cc,), torch.float32)
+        db = b.workspace("ln_db:" + str(id(ln)), (Cc,), torch.float32)
+        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, dg, db if has_bias else None, ws))
         b.w(P.op_accum(b.grad_acc(ln.weight), dg), tag="accum")
         if has_bias:
             b.w(P.op_accum(b.grad_acc(ln.bias), db), tag="accum")
     else:
-        b.w(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
-                               b.grad_target(ln.bias) if has_bias else None, ws))
+        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
+                                      b.grad_target(ln.bias) if has_bias else None, ws))
     return dx
 
 

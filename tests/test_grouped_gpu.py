@@ -41,3 +41,36 @@ def test_grouped_rejects_mixed_configurations():
     C = torch.zeros(16, 16, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="differs"):
         N.gemm_bf16_grouped([(A, A, C, {}), (A, A, C, dict(epilogue=N.EPI_BIAS_RELU))])
+
+
+def test_grouped_column_reductions_equal_single_calls():
+    from pippy_amd import _native as N
+    torch.manual_seed(1)
+    items, refs = [], []
+    for k, (rows, C, with_x, f32) in enumerate([(4096, 768, True, False), (4096, 2304, False, False),
+                                                 (300, 264, True, True), (1, 8, False, True)] * 8):
+        dy = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+        odt = torch.float32 if f32 else torch.bfloat16
+        n_part = (rows + 127) // 128
+        it = {"dy": dy, "out_sum": torch.empty(C, device=DEV, dtype=odt),
+              "workspace": torch.empty(2 * n_part * C, device=DEV)}
+        ref_sum = torch.empty(C, device=DEV, dtype=odt)
+        ref_dot = None
+        ws = torch.empty(2 * n_part * C, device=DEV)
+        if with_x:
+            x = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+            mean = x.float().mean(-1)
+            rstd = 1.0 / torch.sqrt(x.float().var(-1, unbiased=False) + 1e-5)
+            it.update(x=x, mean=mean, rstd=rstd, out_dot=torch.empty(C, device=DEV, dtype=odt))
+            ref_dot = torch.empty(C, device=DEV, dtype=odt)
+            N.layernorm_bwd_weight(dy, x, mean, rstd, ref_dot, ref_sum, ws)
+        else:
+            N.colsum(dy, ref_sum, ws)
+        items.append(it)
+        refs.append((ref_sum, ref_dot))
+    N.colreduce_grouped(items)
+    torch.cuda.synchronize()
+    for it, (ref_sum, ref_dot) in zip(items, refs):
+        assert torch.equal(it["out_sum"], ref_sum)
+        if ref_dot is not None:
+            assert torch.equal(it["out_dot"], ref_dot)
