@@ -141,6 +141,12 @@ int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
 int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, int out_dtype,
                    float* workspace, pp_stream stream);
 
+/* dst[c, r] = src[r, c] for bf16 (any 2-byte type).  Used once per optimizer step to keep a
+ * transposed copy of every linear weight, so that the input-gradient GEMM dX = dY W
+ * (pippy/_backward.py:67-69) reads both operands k-contiguously. */
+int pp_transpose_bf16(const void* src, int64_t rows, int64_t cols, int64_t ld_src, void* dst,
+                      int64_t ld_dst, pp_stream stream);
+
 /* dz[i] = dy[i] * act'(aux[i]) for act 0 = relu (aux: the activation's output or input),
  * 1 = gelu (erf form, aux: pre-activation), 2 = gelu (tanh form); dtype PP_BF16 or PP_F32.
  * Backward of an activation that stands between two separately lowered linears

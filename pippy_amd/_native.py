@@ -36,7 +36,7 @@ EXPORTED_SYMBOLS = (
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
     "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
-    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_profile_start", "pp_profile_stop",
+    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read",
 )
 
@@ -121,6 +121,7 @@ def lib() -> C.CDLL:
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
         "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
+        "pp_transpose_bf16": [vp, i64, i64, i64, vp, i64, vp],
         "pp_profile_start": [i32],
         "pp_profile_stop": [],
         "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
@@ -419,6 +420,15 @@ def activation_bwd(dy, aux, dz, act: int) -> None:
     check(lib().pp_activation_bwd(dy.data_ptr(), aux.data_ptr(), dz.data_ptr(), dy.numel(), act,
                                   PP_F32 if dy.dtype == torch.float32 else PP_BF16,
                                   current_stream()), "pp_activation_bwd")
+
+
+def transpose_bf16(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst[c, r] = src[r, c]; 2-d, 2-byte elements, unit inner strides."""
+    require_cuda(src, dst)
+    assert src.dim() == 2 and dst.dim() == 2 and src.stride(1) == 1 and dst.stride(1) == 1
+    assert dst.shape == (src.shape[1], src.shape[0]) and src.element_size() == 2 == dst.element_size()
+    check(lib().pp_transpose_bf16(src.data_ptr(), src.shape[0], src.shape[1], src.stride(0),
+                                  dst.data_ptr(), dst.stride(0), current_stream()), "pp_transpose_bf16")
 
 
 def run_ops(ops, n: int) -> None:

@@ -88,6 +88,33 @@ class ParamArena:
             view.copy_(p.detach().to(device))
             p.data = view
         self.named = params
+        # transposed copies of linear weights ([in, out]) for the input-gradient GEMMs
+        self._transposed: Dict[int, Tuple[nn.Parameter, torch.Tensor]] = {}
+        self._versions = None
+
+    def weight_t(self, p: nn.Parameter) -> torch.Tensor:
+        """[in, out_padded] copy of a 2-d weight, kept in step with the parameter by
+        ``refresh_transposed``."""
+        ent = self._transposed.get(id(p))
+        if ent is None:
+            w = self.weight(p, padded=True)
+            t = torch.empty((w.shape[1], w.shape[0]), dtype=w.dtype, device=self.device)
+            N.transpose_bf16(w, t)
+            ent = (p, t)
+            self._transposed[id(p)] = ent
+        return ent[1]
+
+    def refresh_transposed(self) -> None:
+        """Re-transposes the weights whose parameter changed since the last call (an optimizer
+        step bumps the parameter's version counter)."""
+        if not self._transposed:
+            return
+        versions = tuple(p._version for p, _ in self._transposed.values())
+        if versions == self._versions:
+            return
+        self._versions = versions
+        for p, t in self._transposed.values():
+            N.transpose_bf16(self.weight(p, padded=True), t)
 
     def _slice(self, flat: torch.Tensor, p: nn.Parameter, padded: bool) -> torch.Tensor:
         o, numel, shape = self.entries[id(p)]
@@ -383,6 +410,9 @@ class Builder:
     # -- parameters
     def weight(self, p, padded=True):
         return self.sp.arena.weight(p, padded)
+
+    def weight_t(self, p):
+        return self.sp.arena.weight_t(p)
 
     def grad_target(self, p, padded=True):
         """Where the W pass writes this parameter's microbatch gradient: the staging arena (then one

@@ -147,6 +147,8 @@ class PipelineStageBase:
 
     def clear_runtime_states(self) -> None:
         """Resets per-step state (reference ``_PipelineStage.py:343-366``)."""
+        if self._program is not None:
+            self._program.arena.refresh_transposed()
         self.fwd_chunk_id = 0
         self.bwd_chunk_id = 0
         self.bwd_weight_chunk_id = 0

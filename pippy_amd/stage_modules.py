@@ -85,7 +85,11 @@ def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor
     dx = None
     if need_dx:
         dx = dx_out if dx_out is not None else b.grad(name + ".dx", (dY2d.shape[0], W.shape[1]))
-        b.i(P.op_gemm(dY2d, W, dx, b_trans=True, epilogue=dx_epilogue, aux_in=dx_aux))
+        if W.dtype == torch.bfloat16:
+            # dX = dY W with the transposed weight copy: both operands k-contiguous
+            b.i(P.op_gemm(dY2d, b.weight_t(lin.weight), dx, epilogue=dx_epilogue, aux_in=dx_aux))
+        else:
+            b.i(P.op_gemm(dY2d, W, dx, b_trans=True, epilogue=dx_epilogue, aux_in=dx_aux))
     b.w_weight_gemm(dY2d, x2d, lin.weight, padded)
     bias_grad(b, lin, dY2d)
     return dx

@@ -74,3 +74,40 @@ def test_grouped_column_reductions_equal_single_calls():
         assert torch.equal(it["out_sum"], ref_sum)
         if ref_dot is not None:
             assert torch.equal(it["out_dot"], ref_dot)
+
+
+def test_transpose_and_weight_refresh_after_optimizer_step():
+    """The transposed weight copies used by the input-gradient GEMMs follow parameter updates."""
+    import copy
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from pippy_amd import _native as N
+    x = torch.randn(130, 77, device=DEV).to(torch.bfloat16)
+    t = torch.empty(77, 130, device=DEV, dtype=torch.bfloat16)
+    N.transpose_bf16(x, t)
+    assert torch.equal(t, x.t())
+
+    import pippy_amd as pp
+    from oracle import pipeline as OP
+    from test_pipeline_gpu import _build_decoder, _ce
+    from _util import BF16_TOL, max_rel
+    M = 2
+    model, ref, stages, ref_stages, ids = _build_decoder(2, n_layers=2, M=M)
+    target = torch.randint(0, 1000, ids.shape)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    sched.step(ids.to(DEV), target=target.to(DEV))
+    # "optimizer step": perturb every parameter in place on both sides, then compare a fresh step
+    torch.manual_seed(7)
+    with torch.no_grad():
+        for (n, p), (_, rp) in zip(model.named_parameters(), ref.named_parameters()):
+            d = (torch.randn(rp.shape) * 0.02).to(torch.bfloat16)
+            p.add_(d.to(DEV))
+            rp.copy_(p.detach().float().cpu())
+    sched.zero_grad()
+    sched.step(ids.to(DEV), target=target.to(DEV))
+    for p in ref.parameters():
+        p.grad = None
+    OP.step(ref_stages, ids, target, M, _ce)
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        assert max_rel(named[name].main_grad, rp.grad) <= BF16_TOL, name
