@@ -95,6 +95,88 @@ __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) 
     }
 }
 
+// Rows whose start is not 16-byte aligned (e.g. a row length of 50257 bf16 elements): the
+// destination is aligned per row by a short scalar head, the body moves as aligned 16-byte stores
+// fed by unaligned 16-byte loads, and a scalar tail finishes the row.  A = common alignment (bytes)
+// of all pointers, strides and row lengths.
+template <int A>
+struct __attribute__((packed, aligned(A))) Unaligned16 {
+    uint32_t w[4];
+};
+
+template <int A>
+__global__ __launch_bounds__(kThreads) void copy_rows_unaligned_kernel(const CopyTable t) {
+    typedef typename VecT<A>::type elem;
+    uint32_t b = blockIdx.x;
+    int s = 0;
+    while (s + 1 < t.n && b >= t.block_start[s + 1]) ++s;
+    b -= t.block_start[s];
+    const DevSeg& g = t.seg[s];
+    const int tid = threadIdx.x;
+    const int64_t row = b / g.col_blocks;
+    const uint32_t cblk = b % g.col_blocks;
+    const char* sp = g.src + row * g.src_stride;
+    char* dp = g.dst + row * g.dst_stride;
+    int64_t head = (16 - (reinterpret_cast<uintptr_t>(dp) & 15)) & 15;
+    if (head > g.row_bytes) head = g.row_bytes;
+    const int64_t nv = (g.row_bytes - head) >> 4;
+    const int64_t v0 = (int64_t)cblk * (kThreads * kUnroll);
+    uint4 r[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t vi = v0 + u * kThreads + tid;
+        if (vi < nv) {
+            const Unaligned16<A> v = *reinterpret_cast<const Unaligned16<A>*>(sp + head + vi * 16);
+            r[u] = make_uint4(v.w[0], v.w[1], v.w[2], v.w[3]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t vi = v0 + u * kThreads + tid;
+        if (vi < nv) *reinterpret_cast<uint4*>(dp + head + vi * 16) = r[u];
+    }
+    if (cblk == 0) {
+        for (int64_t i = (int64_t)tid * A; i < head; i += kThreads * A)
+            *reinterpret_cast<elem*>(dp + i) = *reinterpret_cast<const elem*>(sp + i);
+    }
+    if (cblk == g.col_blocks - 1) {
+        for (int64_t i = head + nv * 16 + (int64_t)tid * A; i < g.row_bytes; i += kThreads * A)
+            *reinterpret_cast<elem*>(dp + i) = *reinterpret_cast<const elem*>(sp + i);
+    }
+}
+
+template <int A>
+static int launch_unaligned(const pp_copy_seg* segs, int n, hipStream_t stream) {
+    CopyTable t;
+    uint64_t blocks = 0;
+    int m = 0;
+    for (int i = 0; i < n; ++i) {
+        const pp_copy_seg& s = segs[i];
+        if (s.n_rows == 0 || s.row_bytes == 0) continue;
+        DevSeg& d = t.seg[m];
+        d.src = static_cast<const char*>(s.src);
+        d.dst = static_cast<char*>(s.dst);
+        d.n_rows = s.n_rows;
+        d.row_bytes = s.row_bytes;
+        d.src_stride = s.src_stride;
+        d.dst_stride = s.dst_stride;
+        d.rows_per_block = 1;
+        const int64_t vecs = s.row_bytes / 16;
+        const int64_t per = (int64_t)kThreads * kUnroll;
+        d.col_blocks = (uint32_t)((vecs + per - 1) / per);
+        if (d.col_blocks == 0) d.col_blocks = 1;
+        t.block_start[m] = (uint32_t)blocks;
+        blocks += (uint64_t)s.n_rows * d.col_blocks;
+        if (blocks > 0x7fffffffull) return fail(PP_ERR_UNSUPPORTED, "pp_copy_rows: too many blocks");
+        ++m;
+    }
+    if (m == 0) return PP_OK;
+    t.block_start[m] = (uint32_t)blocks;
+    t.n = m;
+    hipLaunchKernelGGL(copy_rows_unaligned_kernel<A>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, t);
+    return check_launch("copy_rows_unaligned_kernel");
+}
+
 static int pick_vec(const pp_copy_seg* segs, int n) {
     uint64_t bits = 0;
     for (int i = 0; i < n; ++i) {
@@ -164,7 +246,21 @@ static int copy_rows_impl(const pp_copy_seg* segs, int n_segs, hipStream_t strea
     for (int i0 = 0; i0 < n_segs; i0 += kMaxSegs) {
         const int n = (n_segs - i0 < kMaxSegs) ? n_segs - i0 : kMaxSegs;
         int rc;
-        switch (pick_vec(segs + i0, n)) {
+        const int vec = pick_vec(segs + i0, n);
+        bool long_rows = true;
+        for (int i = 0; i < n; ++i)
+            if (segs[i0 + i].n_rows > 0 && segs[i0 + i].row_bytes < 2048) long_rows = false;
+        if (vec < 16 && long_rows) {
+            switch (vec) {
+                case 8: rc = launch_unaligned<8>(segs + i0, n, stream); break;
+                case 4: rc = launch_unaligned<4>(segs + i0, n, stream); break;
+                case 2: rc = launch_unaligned<2>(segs + i0, n, stream); break;
+                default: rc = launch_unaligned<1>(segs + i0, n, stream); break;
+            }
+            if (rc != PP_OK) return rc;
+            continue;
+        }
+        switch (vec) {
             case 16: rc = launch_table<16>(segs + i0, n, stream); break;
             case 8: rc = launch_table<8>(segs + i0, n, stream); break;
             case 4: rc = launch_table<4>(segs + i0, n, stream); break;

@@ -111,3 +111,20 @@ def test_transpose_and_weight_refresh_after_optimizer_step():
     named = dict(model.named_parameters())
     for name, rp in ref.named_parameters():
         assert max_rel(named[name].main_grad, rp.grad) <= BF16_TOL, name
+
+
+@pytest.mark.parametrize("dtype,V,ld,rows", [(torch.bfloat16, 50257, 50304, 64), (torch.uint8, 4099, 4112, 33),
+                                              (torch.float32, 1027, 1030, 17), (torch.bfloat16, 1025, 1025, 9)])
+def test_copy_rows_with_unaligned_rows_is_bit_exact(dtype, V, ld, rows):
+    """Rows that do not start on 16-byte boundaries take the head / aligned body / tail path."""
+    from pippy_amd import _native as N
+    torch.manual_seed(2)
+    es = torch.empty(0, dtype=dtype).element_size()
+    src = (torch.randn(rows, ld, device=DEV) * 100).to(dtype)
+    dst = torch.zeros(rows * V + 16, device=DEV, dtype=dtype)
+    for shift in (0, 1, 3):   # destination start misaligned by `shift` elements
+        dst.zero_()
+        N.copy_rows([(src.data_ptr(), dst.data_ptr() + shift * es, rows, V * es, ld * es, V * es)])
+        got = dst[shift:shift + rows * V].view(rows, V)
+        assert torch.equal(got, src[:, :V])
+        assert float(dst[:shift].float().abs().sum()) == 0 and float(dst[shift + rows * V:].float().abs().sum()) == 0
