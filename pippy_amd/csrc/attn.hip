@@ -63,7 +63,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t q0 = (int64_t)blockIdx.x * 128;
+    // causal: late query blocks have the most key blocks; launch them first
+    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 128;
     const int64_t qw0 = q0 + 32 * wave;
     const int64_t qi = qw0 + l32;  // this lane's query row
 
@@ -119,28 +120,28 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
             }
             // sacc[t][v]: kv = kv0 + 32 t + 8 (v/4) + 4 lh + v%4, q = qi
             const bool diag = CAUSAL && (kv0 + 63 > qw0);
+            // m_run tracks the maximum of the raw scores; c > 0, so scaling commutes with max
             float mloc = -INFINITY;
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    float s = sacc[t][v] * c;
                     if (diag) {
                         const int64_t kv = kv0 + 32 * t + 8 * (v >> 2) + 4 * lh + (v & 3);
-                        if (kv > qi) s = -INFINITY;
+                        if (kv > qi) sacc[t][v] = -INFINITY;
                     }
-                    sacc[t][v] = s;
-                    mloc = fmaxf(mloc, s);
+                    mloc = fmaxf(mloc, sacc[t][v]);
                 }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             const float m_new = fmaxf(m_run, mloc);
-            const float alpha = exp2f(m_run - m_new);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+            const float mc = m_new * c;
             float psum = 0.f;
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const float p = exp2f(sacc[t][v] - m_new);
+                    const float p = __builtin_amdgcn_exp2f(fmaf(sacc[t][v], c, -mc));
                     sacc[t][v] = p;
                     psum += p;
                 }
@@ -180,7 +181,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
                 make_uint2(pack_bf16(oacc[dt][4 * g + 0] * inv_l, oacc[dt][4 * g + 1] * inv_l),
                            pack_bf16(oacc[dt][4 * g + 2] * inv_l, oacc[dt][4 * g + 3] * inv_l));
         }
-    if (lh == 0) a.lse[(b * a.H + h) * a.S + qi] = m_run * kLn2 + logf(l_run);
+    if (lh == 0) a.lse[(b * a.H + h) * a.S + qi] = m_run * a.scale + logf(l_run);
 }
 
 // ---- backward: delta[b, h, q] = sum_d dO * O ---------------------------------------------------
@@ -329,7 +330,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int v = 4 * g + e;
-                    float p = exp2f(sacc[v] * c - lq[e]);
+                    float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lq[e]));
                     if (diag) {
                         const int64_t qrow = qt0 + 8 * g + 4 * lh + e;
                         if (kvi > qrow) p = 0.f;
@@ -381,7 +382,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t q0 = (int64_t)blockIdx.x * 128;
+    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 128;
     const int64_t qw0 = q0 + 32 * wave;
     const int64_t qi = qw0 + l32;
 
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
             float dsv[16];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float p = exp2f(sacc[v] * c - lse_q);
+                float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lse_q));
                 if (diag) {
                     const int64_t kv = kt0 + 8 * (v >> 2) + 4 * lh + (v & 3);
                     if (kv > qi) p = 0.f;

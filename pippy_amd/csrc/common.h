@@ -34,17 +34,18 @@ __host__ __device__ inline bool aligned(const void* p, size_t a) {
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
+typedef __bf16 pp_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float pp_f32x2_t __attribute__((ext_vector_type(2)));
+// fp32 -> bf16, round-to-nearest-even, through the hardware conversion (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const pp_f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pp_bf16x2_t));
+}
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-    uint32_t bias = 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>((u + bias) >> 16);
+    return static_cast<uint16_t>(pack_bf16(f, 0.f) & 0xffffu);
 }
 __device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
-}
 
 // Sum / max over the 64 lanes of a wave (every lane gets the result).
 __device__ __forceinline__ float wave_sum(float v) {
