@@ -13,6 +13,14 @@
 //
 // The MFMA is issued with the B fragment as its first operand, so a lane ends up holding, for one
 // output row m, groups of 4 consecutive columns n: stores and epilogue reads are 8-byte vectors.
+//
+// When both operands are k-contiguous (forward GEMMs, input-gradient GEMMs against a transposed
+// weight copy) the tiles are staged with direct-to-LDS buffer loads instead: no staging registers,
+// no ds_write, a pipeline of 2 or 3 LDS stages with the barrier placed in the middle of the last
+// k16 step of a tile, LDS fragment reads interleaved one-to-one with the MFMAs of the previous
+// step, tiles visited in an order that keeps an XCD on a compact patch of C, and an epilogue that
+// passes the fp32 accumulators through LDS so that every global access of the epilogue (C, bias,
+// auxiliary tensors) is a full line.
 #include "tile.h"
 #include "act_math.h"
 #include <vector>
@@ -216,6 +224,159 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint32_t tile_m, ui
         }
 }
 
+// Tile order of the direct-to-LDS kernels: bands of kGroupM tile rows, walked m-fastest, so that
+// the tiles resident on an XCD at one time share few A and B panels.
+constexpr uint32_t kGroupM = 8;
+__device__ __forceinline__ void grouped_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n,
+                                             uint32_t* tile_m, uint32_t* tile_n) {
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t grp = bid / per_group, rem = bid % per_group;
+    const uint32_t rows = min(kGroupM, tiles_m - grp * kGroupM);
+    *tile_m = grp * kGroupM + rem % rows;
+    *tile_n = rem / rows;
+}
+
+// One BM x BN output tile, both operands k-contiguous, NS LDS stages filled by direct-to-LDS loads.
+template <int BM, int BN, int NS, int EPI, bool CF32>
+__device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
+    constexpr int WTM = BM / 2, WTN = BN / 2;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int kStageElems = (BM + BN) * BK;
+    constexpr int LPT = DmaStage<BM>::kLoads + DmaStage<BN>::kLoads;  // loads per tile per wave
+    static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int a = 0; a < TN; ++a)
+#pragma unroll
+        for (int b = 0; b < TM; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+    DmaStage<BM> sa;
+    DmaStage<BN> sb;
+    sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
+    sb.init(g.B, g.ldb, n0, g.N, g.K, wave, lane);
+    const int nk = (int)((g.K + BK - 1) / BK);
+    auto issue = [&](int stage, int kt) {
+        sa.load(smem + stage * kStageElems, kt * BK, wave);
+        sb.load(smem + stage * kStageElems + BM * BK, kt * BK, wave);
+    };
+
+    // fragment addresses within a stage: row base and the row's swizzle
+    int fa_off[TM], fb_off[TN], fa_sw[TM], fb_sw[TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t) {
+        const int r = wm0 + t * 32 + l32;
+        fa_off[t] = r * BK;
+        fa_sw[t] = swz(r);
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const int r = wn0 + t * 32 + l32;
+        fb_off[t] = BM * BK + r * BK;
+        fb_sw[t] = swz(r);
+    }
+    bf16x8_t fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int sel, const uint16_t* st, int ks) {
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+            fa[sel][t] = *reinterpret_cast<const bf16x8_t*>(st + fa_off[t] + (((2 * ks + lh) ^ fa_sw[t]) << 3));
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+            fb[sel][t] = *reinterpret_cast<const bf16x8_t*>(st + fb_off[t] + (((2 * ks + lh) ^ fb_sw[t]) << 3));
+    };
+    auto mma = [&](int sel, int a_lo, int a_hi) {
+#pragma unroll
+        for (int a = a_lo; a < a_hi; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[sel][a], fa[sel][b], acc[a][b], 0, 0, 0);
+    };
+    // one MFMA, one LDS read, ... then the remaining MFMAs of the step
+    auto interleave = [&]() {
+#pragma unroll
+        for (int i = 0; i < TM + TN; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+    };
+
+    // prologue: tiles 0 .. NS-1 in flight, tile 0 awaited
+#pragma unroll
+    for (int t = 0; t < NS; ++t)
+        if (t < nk) issue(t, t);
+    if (nk >= NS) wait_vmcnt<(NS - 1) * LPT>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, smem, 0);
+
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        const uint16_t* st = smem + stage * kStageElems;
+        read_frags(1, st, 1); mma(0, 0, TN); interleave();
+        read_frags(0, st, 2); mma(1, 0, TN); interleave();
+        read_frags(1, st, 3); mma(0, 0, TN); interleave();
+        mma(1, 0, TN / 2);
+        // tile kt+1 must have landed; tiles kt+2 .. kt+NS-1 may stay in flight
+        const int ahead = nk - 2 - kt;
+        if (NS >= 4 && ahead >= 2) wait_vmcnt<(NS >= 4 ? 2 : 0) * LPT>();
+        else if (NS >= 3 && ahead >= 1) wait_vmcnt<(NS >= 3 ? 1 : 0) * LPT>();
+        else wait_vmcnt<0>();
+        wait_lds();  // this wave's reads of the current stage are done: the stage may be refilled
+        __builtin_amdgcn_s_barrier();
+        if (kt + NS < nk) issue(stage, kt + NS);
+        stage = stage + 1 == NS ? 0 : stage + 1;
+        if (kt + 1 < nk) read_frags(0, smem + stage * kStageElems, 0);
+        mma(1, TN / 2, TN);
+    }
+
+    // Epilogue: one band of 32 rows at a time goes through a wave-private LDS region as fp32,
+    // [32][WTN] with the 16-byte unit index XORed by the row, and comes back with lanes running
+    // along n, so that epilogue4 reads and writes whole lines.
+    wait_lds();
+    __builtin_amdgcn_s_barrier();  // every wave is done with the stages
+    float* cw = reinterpret_cast<float*>(smem) + wave * (32 * WTN);
+    constexpr int UPR = WTN / 4;   // 16-byte units per row
+    constexpr int RPP = 64 / UPR;  // rows per pass of the wave
+    const int ru = lane % UPR, rr = lane / UPR;
+    const bool vec_ok = CF32 ? ((g.ldc & 3) == 0 && aligned(g.C, 16))
+                             : ((g.ldc & 3) == 0 && aligned(g.C, 8) && (g.ld_aux & 3) == 0 &&
+                                aligned(g.aux_in, 8) && aligned(g.aux_out, 8));
+#pragma unroll
+    for (int b = 0; b < TM; ++b) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int u = a * 8 + 2 * q + lh;
+                *reinterpret_cast<float4*>(cw + l32 * WTN + ((u ^ (l32 & (UPR - 1))) << 2)) =
+                    make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
+            }
+#pragma unroll
+        for (int i = 0; i < 32 / RPP; ++i) {
+            const int m = i * RPP + rr;
+            const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
+            epilogue4<EPI, CF32>(g, m0 + wm0 + b * 32 + m, n0 + wn0 + ru * 4, v.x, v.y, v.z, v.w, vec_ok);
+        }
+    }
+}
+
+template <int BM, int BN, int NS, int EPI, bool CF32>
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_dma_kernel(const GemmArgs g) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks) return;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    gemm_tile_dma<BM, BN, NS, EPI, CF32>(g, tile_m, tile_n);
+}
+
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs g) {
     const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
@@ -268,6 +429,23 @@ static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
         GemmArgs g = probs[0];
         int rc = count_tiles<BM, BN>(g);
         if (rc) return rc;
+        if constexpr (!AT && !BT) {
+            // up to one tile per CU: a deeper pipeline in one resident block; more: two blocks per CU
+            const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
+            if (g.n_blocks <= 256) {
+                constexpr size_t lds3 = (size_t)3 * (BM + BN) * BK * sizeof(uint16_t);
+                static const int attr3 = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, 3, EPI, CF32>, lds3);
+                if (attr3) return attr3;
+                hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, 3, EPI, CF32>), dim3(grid),
+                                   dim3(kGemmThreads), lds3, st, g);
+            } else {
+                static const int attr2 = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, 2, EPI, CF32>, lds);
+                if (attr2) return attr2;
+                hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, 2, EPI, CF32>), dim3(grid),
+                                   dim3(kGemmThreads), lds, st, g);
+            }
+            return check_launch("gemm_bf16_dma_kernel");
+        }
         static const int attr_rc = reserve_lds(&gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>, lds);
         if (attr_rc) return attr_rc;
         const uint32_t grid = (g.n_blocks + 7) / 8 * 8;

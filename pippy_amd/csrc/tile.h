@@ -243,4 +243,65 @@ struct BufStage<ROWS, true, NTHREADS> {
     __device__ __forceinline__ void store(uint16_t* lds) const { store(lds, threadIdx.x); }
 };
 
+// ---- direct-to-LDS staging -------------------------------------------------------------------
+// A buffer load with the lds modifier writes each lane's 16 bytes to LDS at (wave-uniform base +
+// 16 * lane) without passing through registers, so one wave instruction fills 1 KiB = 8 tile rows.
+// The XOR swizzle is applied on the global side: lane l of a row fetches chunk (l & 7) ^ swz(row).
+// Loads complete in order, so "tile t has landed" is a vmcnt wait that leaves the younger tiles in
+// flight.  Only k-contiguous operands can be staged this way.
+typedef __attribute__((address_space(3))) void* lds_void_ptr_t;
+
+__device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint16_t* lds_wave_base,
+                                                 int voffset, int soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr_t)lds_wave_base, 16, voffset, soffset, 0, 0);
+#endif
+}
+
+// s_waitcnt with only the vector-memory counter constrained (N outstanding loads allowed).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+// s_waitcnt lgkmcnt(0): every LDS access of this wave has completed.
+__device__ __forceinline__ void wait_lds() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
+template <int ROWS>
+struct DmaStage {
+    static constexpr int kLoads = ROWS / 8 / 4;  // 1 KiB pieces per wave, 4 waves
+    static_assert(ROWS % 32 == 0, "tile rows must divide over 4 waves x 8 rows");
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voff[kLoads];
+    int kcol[kLoads];  // first k of this lane's chunk within a tile
+    int K;
+    __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
+                                         int64_t rows_total, int64_t K_, int wave, int lane) {
+        const uint64_t bytes = (uint64_t)(rows_total - row0) * (uint64_t)ld * 2;
+        rsrc = make_rsrc(base + row0 * ld, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
+        K = (int)K_;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            const int row = (i * 4 + wave) * 8 + (lane >> 3);
+            const int ch = (lane & 7) ^ swz(row);
+            voff[i] = (int)((row * ld + ch * 8) * 2);
+            kcol[i] = ch * 8;
+        }
+    }
+    // Issues the loads of the k-tile starting at k0 into the LDS tile at `lds` ([ROWS][64] bf16).
+    __device__ __forceinline__ void load(uint16_t* lds, int k0, int wave) const {
+        if (k0 + BK <= K) {
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i)
+                load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i], k0 * 2);
+        } else {
+            // k tail: chunks past K aim beyond the end of the buffer, which the range check zero-fills
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i)
+                load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512,
+                                 k0 + kcol[i] < K ? voff[i] + k0 * 2 : (int)0x7ffffff0, 0);
+        }
+    }
+};
+
 }  // namespace pp
