@@ -3,24 +3,21 @@
 //   C[M,N] = epilogue( sum_k A(m,k) * B(n,k) ),  fp32 accumulation.
 //
 // Tiling: a work-group of 256 lanes (4 waves, 2x2) owns a BM x BN output tile and walks K in steps
-// of 64.  Operand tiles live in LDS as [row][64 k] bf16 (128 B per row) with the 16-byte chunk
-// index XOR-swizzled by the row so that both the staging writes and the ds_read_b128 fragment
-// reads spread over all banks.  An operand whose memory layout is [K][rows] (the weight in the
-// input-gradient GEMM, both operands in the weight-gradient GEMM) is transposed on the way in:
-// each lane loads 4 k-rows x 8 rows and writes 8 x 8-byte k-runs.  Global loads for tile t+1 are
-// issued before the MFMAs of tile t (register double buffering, two LDS buffers, one barrier per
-// K step).
+// of 64.  Tiles are staged with direct-to-LDS buffer loads (no staging registers, no ds_write):
+//   * a k-contiguous operand (memory [rows][ld]) lives in LDS as [row][64 k] with the 16-byte chunk
+//     index XOR-swizzled by the row, and fragments are plain ds_read_b128;
+//   * a transposed operand (memory [K][ld]: the weight of an input-gradient GEMM, both operands of a
+//     weight-gradient GEMM) lives in LDS as it does in memory, [64 k][rows], and fragments come out
+//     through ds_read_b64_tr_b16, which transposes 4 k x 16 rows across each 16 lanes.
+// The loads of up to 3 tiles are in flight (vmcnt waits leave the younger ones outstanding); the
+// single barrier of a tile sits in the middle of its last k16 step, after which the stage it just
+// finished is refilled; the LDS reads of a k16 step are interleaved with the MFMAs of the step
+// before.  Tiles are visited in bands of 8 tile rows so that an XCD stays on a compact patch of C.
 //
 // The MFMA is issued with the B fragment as its first operand, so a lane ends up holding, for one
-// output row m, groups of 4 consecutive columns n: stores and epilogue reads are 8-byte vectors.
-//
-// When both operands are k-contiguous (forward GEMMs, input-gradient GEMMs against a transposed
-// weight copy) the tiles are staged with direct-to-LDS buffer loads instead: no staging registers,
-// no ds_write, a pipeline of 2 or 3 LDS stages with the barrier placed in the middle of the last
-// k16 step of a tile, LDS fragment reads interleaved one-to-one with the MFMAs of the previous
-// step, tiles visited in an order that keeps an XCD on a compact patch of C, and an epilogue that
-// passes the fp32 accumulators through LDS so that every global access of the epilogue (C, bias,
-// auxiliary tensors) is a full line.
+// output row m, groups of 4 consecutive columns n.  The epilogue passes the fp32 accumulators
+// through LDS, 32 rows at a time, and comes back with lanes running along n, so that every global
+// access of the epilogue (C, bias, auxiliary tensors) covers whole lines.
 #include "tile.h"
 #include "act_math.h"
 #include <vector>
@@ -140,90 +137,6 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t bid, uint32_t grid) {
     return (bid & 7) * per_xcd + (bid >> 3);
 }
 
-// One BM x BN output tile of one problem.
-template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
-    constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
-    constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int kStageElems = (BM + BN) * BK;  // one LDS buffer: A tile then B tile
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
-    const int l32 = lane & 31, lh = lane >> 5;
-
-    f32x16_t acc[TN][TM];
-#pragma unroll
-    for (int a = 0; a < TN; ++a)
-#pragma unroll
-        for (int b = 0; b < TM; ++b)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
-
-    BufStage<BM, AT> sa;
-    BufStage<BN, BT> sb;
-    sa.init(g.A, g.lda, m0, g.M, g.K, tid);
-    sb.init(g.B, g.ldb, n0, g.N, g.K, tid);
-    const int nk = (int)((g.K + BK - 1) / BK);
-
-    sa.load(0);
-    sb.load(0);
-    sa.store(smem);
-    sb.store(smem + BM * BK);
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
-            sa.load((kt + 1) * BK);
-            sb.load((kt + 1) * BK);
-        }
-        const uint16_t* a_s = smem + cur * kStageElems;
-        const uint16_t* b_s = a_s + BM * BK;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8_t af[TM], bf[TN];
-#pragma unroll
-            for (int t = 0; t < TM; ++t) {
-                const int row = wm0 + t * 32 + l32;
-                af[t] = *reinterpret_cast<const bf16x8_t*>(a_s + row * BK + (((2 * ks + lh) ^ swz(row)) << 3));
-            }
-#pragma unroll
-            for (int t = 0; t < TN; ++t) {
-                const int row = wn0 + t * 32 + l32;
-                bf[t] = *reinterpret_cast<const bf16x8_t*>(b_s + row * BK + (((2 * ks + lh) ^ swz(row)) << 3));
-            }
-#pragma unroll
-            for (int a = 0; a < TN; ++a)
-#pragma unroll
-                for (int b = 0; b < TM; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf[a], af[b], acc[a][b], 0, 0, 0);
-        }
-        if (kt + 1 < nk) {
-            sa.store(smem + (cur ^ 1) * kStageElems);
-            sb.store(smem + (cur ^ 1) * kStageElems + BM * BK);
-        }
-        __syncthreads();
-    }
-
-    // D[i][j]: i = n within the 32x32 tile = 8*(v/4) + 4*lh + v%4, j = m within the tile = l32.
-    const bool vec_ok = CF32 ? ((g.ldc & 3) == 0 && aligned(g.C, 16))
-                             : ((g.ldc & 3) == 0 && aligned(g.C, 8) && (g.ld_aux & 3) == 0 &&
-                                aligned(g.aux_in, 8) && aligned(g.aux_out, 8));
-#pragma unroll
-    for (int a = 0; a < TN; ++a)
-#pragma unroll
-        for (int b = 0; b < TM; ++b) {
-            const int64_t m = m0 + wm0 + b * 32 + l32;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int64_t n = n0 + wn0 + a * 32 + 8 * q + 4 * lh;
-                epilogue4<EPI, CF32>(g, m, n, acc[a][b][4 * q + 0], acc[a][b][4 * q + 1],
-                                     acc[a][b][4 * q + 2], acc[a][b][4 * q + 3], vec_ok);
-            }
-        }
-}
-
 // Tile order of the direct-to-LDS kernels: bands of kGroupM tile rows, walked m-fastest, so that
 // the tiles resident on an XCD at one time share few A and B panels.
 constexpr uint32_t kGroupM = 8;
@@ -236,20 +149,29 @@ __device__ __forceinline__ void grouped_tile(uint32_t bid, uint32_t tiles_m, uin
     *tile_n = rem / rows;
 }
 
-// One BM x BN output tile, both operands k-contiguous, NS LDS stages filled by direct-to-LDS loads.
-template <int BM, int BN, int NS, int EPI, bool CF32>
+// Scheduling hint for one k16 step: R LDS reads (the fragments of the next step) spread evenly
+// between M MFMAs.
+template <int R, int M, int I>
+__device__ __forceinline__ void interleave_reads() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, R * (I + 1) / M - R * I / M, 0);
+    if constexpr (I + 1 < M) interleave_reads<R, M, I + 1>();
+}
+
+// One BM x BN output tile with NS LDS stages filled by direct-to-LDS loads.
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
 __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int kStageElems = (BM + BN) * BK;
-    constexpr int LPT = DmaStage<BM>::kLoads + DmaStage<BN>::kLoads;  // loads per tile per wave
+    constexpr int LPT = DmaStage<BM, AT>::kLoads + DmaStage<BN, BT>::kLoads;  // loads per tile per wave
+    constexpr int kReadsPerStep = TM * FragReader<BM, AT>::kReads + TN * FragReader<BN, BT>::kReads;
     static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
-    const int l32 = lane & 31, lh = lane >> 5;
 
     f32x16_t acc[TN][TM];
 #pragma unroll
@@ -259,8 +181,8 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    DmaStage<BM> sa;
-    DmaStage<BN> sb;
+    DmaStage<BM, AT> sa;
+    DmaStage<BN, BT> sb;
     sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
     sb.init(g.B, g.ldb, n0, g.N, g.K, wave, lane);
     const int nk = (int)((g.K + BK - 1) / BK);
@@ -269,28 +191,18 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
         sb.load(smem + stage * kStageElems + BM * BK, kt * BK, wave);
     };
 
-    // fragment addresses within a stage: row base and the row's swizzle
-    int fa_off[TM], fb_off[TN], fa_sw[TM], fb_sw[TN];
+    FragReader<BM, AT> ra[TM];
+    FragReader<BN, BT> rb[TN];
 #pragma unroll
-    for (int t = 0; t < TM; ++t) {
-        const int r = wm0 + t * 32 + l32;
-        fa_off[t] = r * BK;
-        fa_sw[t] = swz(r);
-    }
+    for (int t = 0; t < TM; ++t) ra[t].init(wm0 + t * 32, lane);
 #pragma unroll
-    for (int t = 0; t < TN; ++t) {
-        const int r = wn0 + t * 32 + l32;
-        fb_off[t] = BM * BK + r * BK;
-        fb_sw[t] = swz(r);
-    }
+    for (int t = 0; t < TN; ++t) rb[t].init(wn0 + t * 32, lane);
     bf16x8_t fa[2][TM], fb[2][TN];
     auto read_frags = [&](int sel, const uint16_t* st, int ks) {
 #pragma unroll
-        for (int t = 0; t < TM; ++t)
-            fa[sel][t] = *reinterpret_cast<const bf16x8_t*>(st + fa_off[t] + (((2 * ks + lh) ^ fa_sw[t]) << 3));
+        for (int t = 0; t < TM; ++t) fa[sel][t] = ra[t].read(st, ks);
 #pragma unroll
-        for (int t = 0; t < TN; ++t)
-            fb[sel][t] = *reinterpret_cast<const bf16x8_t*>(st + fb_off[t] + (((2 * ks + lh) ^ fb_sw[t]) << 3));
+        for (int t = 0; t < TN; ++t) fb[sel][t] = rb[t].read(st + BM * BK, ks);
     };
     auto mma = [&](int sel, int a_lo, int a_hi) {
 #pragma unroll
@@ -299,15 +211,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
             for (int b = 0; b < TM; ++b)
                 acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[sel][a], fa[sel][b], acc[a][b], 0, 0, 0);
     };
-    // one MFMA, one LDS read, ... then the remaining MFMAs of the step
-    auto interleave = [&]() {
-#pragma unroll
-        for (int i = 0; i < TM + TN; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
-    };
+    auto interleave = [&]() { interleave_reads<kReadsPerStep, TM * TN, 0>(); };
 
     // prologue: tiles 0 .. NS-1 in flight, tile 0 awaited
 #pragma unroll
@@ -342,6 +246,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     // along n, so that epilogue4 reads and writes whole lines.
     wait_lds();
     __builtin_amdgcn_s_barrier();  // every wave is done with the stages
+    const int l32 = lane & 31, lh = lane >> 5;
     float* cw = reinterpret_cast<float*>(smem) + wave * (32 * WTN);
     constexpr int UPR = WTN / 4;   // 16-byte units per row
     constexpr int RPP = 64 / UPR;  // rows per pass of the wave
@@ -368,20 +273,13 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     }
 }
 
-template <int BM, int BN, int NS, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_dma_kernel(const GemmArgs g) {
     const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= g.n_blocks) return;
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, NS, EPI, CF32>(g, tile_m, tile_n);
-}
-
-template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
-__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_kernel(const GemmArgs g) {
-    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
-    if (bid >= g.n_blocks) return;
-    gemm_tile<BM, BN, AT, BT, EPI, CF32>(g, bid % g.tiles_m, bid / g.tiles_m);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32>(g, tile_m, tile_n);
 }
 
 // Several independent problems in one grid: the tiles of problem i are the block ids
@@ -392,7 +290,7 @@ struct GemmGroupArgs {
     int n;
 };
 
-template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const GemmGroupArgs ga) {
     uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= ga.tile_start[ga.n]) return;
@@ -400,7 +298,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const Gem
     while (i + 1 < ga.n && bid >= ga.tile_start[i + 1]) ++i;
     bid -= ga.tile_start[i];
     const GemmArgs& g = ga.p[i];
-    gemm_tile<BM, BN, AT, BT, EPI, CF32>(g, bid % g.tiles_m, bid / g.tiles_m);
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32>(g, tile_m, tile_n);
 }
 
 template <typename Kernel>
@@ -422,40 +322,43 @@ static int count_tiles(GemmArgs& g) {
     return PP_OK;
 }
 
+// Pipeline depth: with at most one tile per CU a block has the CU to itself and takes 3 stages;
+// with more tiles 2 stages leave room for two resident blocks, whose prologues and epilogues overlap
+// each other's main loops.
+constexpr uint32_t kComputeUnits = 256;
+
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+static int launch_single(const GemmArgs& g, hipStream_t st) {
+    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32>, lds);
+    if (attr_rc) return attr_rc;
+    const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+                       lds, st, g);
+    return check_launch("gemm_bf16_dma_kernel");
+}
+
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+static int launch_group(const GemmGroupArgs& ga, hipStream_t st) {
+    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32>, lds);
+    if (attr_rc) return attr_rc;
+    const uint32_t grid = (ga.tile_start[ga.n] + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+                       lds, st, ga);
+    return check_launch("gemm_bf16_group_kernel");
+}
+
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
 static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
-    constexpr size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
     if (n == 1) {
         GemmArgs g = probs[0];
         int rc = count_tiles<BM, BN>(g);
         if (rc) return rc;
-        if constexpr (!AT && !BT) {
-            // up to one tile per CU: a deeper pipeline in one resident block; more: two blocks per CU
-            const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
-            if (g.n_blocks <= 256) {
-                constexpr size_t lds3 = (size_t)3 * (BM + BN) * BK * sizeof(uint16_t);
-                static const int attr3 = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, 3, EPI, CF32>, lds3);
-                if (attr3) return attr3;
-                hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, 3, EPI, CF32>), dim3(grid),
-                                   dim3(kGemmThreads), lds3, st, g);
-            } else {
-                static const int attr2 = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, 2, EPI, CF32>, lds);
-                if (attr2) return attr2;
-                hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, 2, EPI, CF32>), dim3(grid),
-                                   dim3(kGemmThreads), lds, st, g);
-            }
-            return check_launch("gemm_bf16_dma_kernel");
-        }
-        static const int attr_rc = reserve_lds(&gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>, lds);
-        if (attr_rc) return attr_rc;
-        const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
-        hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
-                           lds, st, g);
-        return check_launch("gemm_bf16_kernel");
+        return g.n_blocks <= kComputeUnits ? launch_single<BM, BN, AT, BT, 3, EPI, CF32>(g, st)
+                                           : launch_single<BM, BN, AT, BT, 2, EPI, CF32>(g, st);
     }
     if constexpr (EPI == PP_EPI_NONE || EPI == PP_EPI_ACCUM_F32) {
-        static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, EPI, CF32>, lds);
-        if (attr_rc) return attr_rc;
         for (int i0 = 0; i0 < n; i0 += PP_GEMM_MAX_GROUP) {
             GemmGroupArgs ga;
             ga.n = (n - i0 < PP_GEMM_MAX_GROUP) ? n - i0 : PP_GEMM_MAX_GROUP;
@@ -470,10 +373,8 @@ static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
             if (total > 0x7fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_grouped: too many tiles");
             ga.tile_start[ga.n] = (uint32_t)total;
             if (total == 0) continue;
-            const uint32_t grid = (uint32_t)((total + 7) / 8 * 8);
-            hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, EPI, CF32>), dim3(grid),
-                               dim3(kGemmThreads), lds, st, ga);
-            int rc = check_launch("gemm_bf16_group_kernel");
+            int rc = total <= kComputeUnits ? launch_group<BM, BN, AT, BT, 3, EPI, CF32>(ga, st)
+                                            : launch_group<BM, BN, AT, BT, 2, EPI, CF32>(ga, st);
             if (rc) return rc;
         }
         return PP_OK;

@@ -267,8 +267,12 @@ __device__ __forceinline__ void wait_vmcnt() {
 // s_waitcnt lgkmcnt(0): every LDS access of this wave has completed.
 __device__ __forceinline__ void wait_lds() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 
+template <int ROWS, bool TR>
+struct DmaStage;
+
+// K-contiguous operand: memory [rows][ld]; LDS tile [ROWS][64 k], chunk index XORed with swz(row).
 template <int ROWS>
-struct DmaStage {
+struct DmaStage<ROWS, false> {
     static constexpr int kLoads = ROWS / 8 / 4;  // 1 KiB pieces per wave, 4 waves
     static_assert(ROWS % 32 == 0, "tile rows must divide over 4 waves x 8 rows");
     __amdgpu_buffer_rsrc_t rsrc;
@@ -288,7 +292,7 @@ struct DmaStage {
             kcol[i] = ch * 8;
         }
     }
-    // Issues the loads of the k-tile starting at k0 into the LDS tile at `lds` ([ROWS][64] bf16).
+    // Issues the loads of the k-tile starting at k0 into the LDS tile at `lds`.
     __device__ __forceinline__ void load(uint16_t* lds, int k0, int wave) const {
         if (k0 + BK <= K) {
 #pragma unroll
@@ -301,6 +305,89 @@ struct DmaStage {
                 load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512,
                                  k0 + kcol[i] < K ? voff[i] + k0 * 2 : (int)0x7ffffff0, 0);
         }
+    }
+};
+
+// Transposed operand: memory [K][ld] with the tile's rows contiguous; LDS tile [64 k][ROWS] as in
+// memory, the 16-byte chunk index of k-row k XORed with (k & 3) << 2 so that the four k-rows a
+// transposing read touches at once fall into different banks.
+template <int ROWS>
+struct DmaStage<ROWS, true> {
+    static constexpr int kChunksPerRow = ROWS / 8;
+    static constexpr int kRowsPerLoad = 64 / kChunksPerRow;
+    static constexpr int kLoads = BK / kRowsPerLoad / 4;
+    static_assert(ROWS % 128 == 0 && ROWS <= 512, "transposed tiles are staged 128 rows at a time");
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voff[kLoads];
+    int ld2;  // bytes per k-row of the operand
+    __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
+                                         int64_t rows_total, int64_t K_, int wave, int lane) {
+        const uint64_t bytes = ((uint64_t)K_ * (uint64_t)ld - (uint64_t)row0) * 2;
+        rsrc = make_rsrc(base + row0, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
+        ld2 = (int)(ld * 2);
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            const int krow = (i * 4 + wave) * kRowsPerLoad + lane / kChunksPerRow;
+            const int ch = (lane % kChunksPerRow) ^ ((krow & 3) << 2);
+            const bool valid = row0 + ch * 8 < rows_total;
+            // k is part of the lane offset so that k-rows past K fail the range check and read as 0
+            voff[i] = valid ? (int)((krow * ld + ch * 8) * 2) : (int)0x7ffffff0;
+        }
+    }
+    __device__ __forceinline__ void load(uint16_t* lds, int k0, int wave) const {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i)
+            load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i] + k0 * ld2, 0);
+    }
+};
+
+// ---- MFMA operand fragments out of a staged tile ------------------------------------------------
+// Fragment of v_mfma_f32_32x32x16_bf16 for 32 tile rows starting at r0: lane l holds, for row
+// r0 + l % 32, the 8 consecutive k values 16 * ks + 8 * (l / 32) ...
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr_t;
+
+template <int ROWS, bool TR>
+struct FragReader;
+
+template <int ROWS>
+struct FragReader<ROWS, false> {
+    static constexpr int kReads = 1;  // LDS instructions per fragment
+    int off, sw, lh;
+    __device__ __forceinline__ void init(int r0, int lane) {
+        const int r = r0 + (lane & 31);
+        off = r * BK;
+        sw = swz(r);
+        lh = lane >> 5;
+    }
+    __device__ __forceinline__ bf16x8_t read(const uint16_t* tile, int ks) const {
+        return *reinterpret_cast<const bf16x8_t*>(tile + off + (((2 * ks + lh) ^ sw) << 3));
+    }
+};
+
+// Transposing read: in each block of 16 lanes, lane 4 j + i fetches 4 consecutive rows
+// (8 bytes) of k-row j, and ds_read_b64_tr_b16 hands lane m of the block the 4 k values of row m.
+template <int ROWS>
+struct FragReader<ROWS, true> {
+    static constexpr int kReads = 2;
+    int off;
+    __device__ __forceinline__ void init(int r0, int lane) {
+        const int blk = lane >> 4, g = blk >> 1, mb = blk & 1;
+        const int j = (lane & 15) >> 2, i = lane & 3;
+        const int m = r0 + 16 * mb + 4 * i;
+        off = (8 * g + j) * ROWS + (((m >> 3) ^ (j << 2)) << 3) + (m & 7);
+    }
+    __device__ __forceinline__ bf16x8_t read(const uint16_t* tile, int ks) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        const uint16_t* p = tile + off + ks * 16 * ROWS;
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_t)p);
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_t)(p + 4 * ROWS));
+        const s16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8_t, v);
+#else
+        return bf16x8_t{};
+#endif
     }
 };
 
