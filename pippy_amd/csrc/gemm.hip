@@ -37,26 +37,63 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n, n_blocks;
 };
 
-// Applies the epilogue to 4 consecutive columns n0..n0+3 of row m and stores them.
+constexpr bool epi_has_bias(int epi) {
+    return epi == PP_EPI_BIAS || epi == PP_EPI_BIAS_GELU_ERF || epi == PP_EPI_BIAS_GELU_TANH ||
+           epi == PP_EPI_BIAS_RESIDUAL || epi == PP_EPI_BIAS_RELU;
+}
+constexpr bool epi_reads_aux(int epi) {
+    return epi == PP_EPI_BIAS_RESIDUAL || epi == PP_EPI_DGELU_ERF || epi == PP_EPI_DGELU_TANH ||
+           epi == PP_EPI_DRELU;
+}
+constexpr bool epi_is_gelu(int epi) { return epi == PP_EPI_BIAS_GELU_ERF || epi == PP_EPI_BIAS_GELU_TANH; }
+
+// The bias of 4 consecutive columns starting at n0 (zero past N or without a bias).
+template <int EPI>
+__device__ __forceinline__ void load_bias4(const GemmArgs& g, int64_t n0, float (&bias)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bias[e] = 0.f;
+    if (!epi_has_bias(EPI) || !g.bias || n0 >= g.N) return;
+    if (n0 + 3 < g.N && aligned(g.bias + n0, 8)) {
+        const uint2 w = *reinterpret_cast<const uint2*>(g.bias + n0);
+        bias[0] = bf16lo(w.x); bias[1] = bf16hi(w.x); bias[2] = bf16lo(w.y); bias[3] = bf16hi(w.y);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (n0 + e < g.N) bias[e] = bf16_to_f32(g.bias[n0 + e]);
+    }
+}
+
+// The arithmetic of the epilogue on 4 values: v becomes the output, pre the value before the
+// activation (what a GELU epilogue saves for the backward pass).
+template <int EPI>
+__device__ __forceinline__ void epilogue_math4(float (&v)[4], float (&pre)[4], const float (&bias)[4],
+                                               const float (&a)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (epi_has_bias(EPI)) v[e] += bias[e];
+        if (EPI == PP_EPI_BIAS_RESIDUAL) v[e] += a[e];
+        if (EPI == PP_EPI_DGELU_ERF) v[e] *= dgelu_erf(a[e]);
+        if (EPI == PP_EPI_DGELU_TANH) v[e] *= dgelu_tanh(a[e]);
+        if (EPI == PP_EPI_DRELU) v[e] = a[e] > 0.f ? v[e] : 0.f;
+        pre[e] = v[e];
+        if (EPI == PP_EPI_BIAS_GELU_ERF) v[e] = gelu_erf(v[e]);
+        if (EPI == PP_EPI_BIAS_GELU_TANH) v[e] = gelu_tanh(v[e]);
+        if (EPI == PP_EPI_BIAS_RELU) v[e] = fmaxf(v[e], 0.f);
+    }
+}
+
+// Applies the epilogue to 4 consecutive columns n0..n0+3 of row m and stores them; handles rows
+// and columns past the edge of C and unaligned operands.
 template <int EPI, bool CF32>
 __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t n0, float v0, float v1,
-                                          float v2, float v3, bool vec_ok) {
+                                          float v2, float v3, const float (&bias)[4], bool vec_ok) {
     if (m >= g.M || n0 >= g.N) return;
-    float v[4] = {v0, v1, v2, v3};
+    float v[4] = {v0, v1, v2, v3}, pre[4];
     const int nv = (g.N - n0 >= 4) ? 4 : (int)(g.N - n0);
     const bool full = vec_ok && nv == 4;
 
-    if (EPI == PP_EPI_BIAS || EPI == PP_EPI_BIAS_GELU_ERF || EPI == PP_EPI_BIAS_GELU_TANH ||
-        EPI == PP_EPI_BIAS_RESIDUAL || EPI == PP_EPI_BIAS_RELU) {
-        if (g.bias) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (e < nv) v[e] += bf16_to_f32(g.bias[n0 + e]);
-        }
-    }
-    if (EPI == PP_EPI_BIAS_RESIDUAL || EPI == PP_EPI_DGELU_ERF || EPI == PP_EPI_DGELU_TANH ||
-        EPI == PP_EPI_DRELU) {
-        float a[4] = {0.f, 0.f, 0.f, 0.f};
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    if (epi_reads_aux(EPI)) {
         const uint16_t* ap = g.aux_in + m * g.ld_aux + n0;
         if (full) {
             const uint2 w = *reinterpret_cast<const uint2*>(ap);
@@ -66,32 +103,17 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t 
             for (int e = 0; e < 4; ++e)
                 if (e < nv) a[e] = bf16_to_f32(ap[e]);
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (EPI == PP_EPI_BIAS_RESIDUAL) v[e] += a[e];
-            if (EPI == PP_EPI_DGELU_ERF) v[e] *= dgelu_erf(a[e]);
-            if (EPI == PP_EPI_DGELU_TANH) v[e] *= dgelu_tanh(a[e]);
-            if (EPI == PP_EPI_DRELU) v[e] = a[e] > 0.f ? v[e] : 0.f;
-        }
     }
-    if (EPI == PP_EPI_BIAS_GELU_ERF || EPI == PP_EPI_BIAS_GELU_TANH) {
-        if (g.aux_out) {
-            uint16_t* op = g.aux_out + m * g.ld_aux + n0;
-            if (full) {
-                *reinterpret_cast<uint2*>(op) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-            } else {
+    epilogue_math4<EPI>(v, pre, bias, a);
+    if (epi_is_gelu(EPI) && g.aux_out) {
+        uint16_t* op = g.aux_out + m * g.ld_aux + n0;
+        if (full) {
+            *reinterpret_cast<uint2*>(op) = make_uint2(pack_bf16(pre[0], pre[1]), pack_bf16(pre[2], pre[3]));
+        } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (e < nv) op[e] = f32_to_bf16(v[e]);
-            }
+            for (int e = 0; e < 4; ++e)
+                if (e < nv) op[e] = f32_to_bf16(pre[e]);
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            v[e] = (EPI == PP_EPI_BIAS_GELU_ERF) ? gelu_erf(v[e]) : gelu_tanh(v[e]);
-    }
-    if (EPI == PP_EPI_BIAS_RELU) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
     }
 
     if (CF32) {
@@ -254,6 +276,13 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     const bool vec_ok = CF32 ? ((g.ldc & 3) == 0 && aligned(g.C, 16))
                              : ((g.ldc & 3) == 0 && aligned(g.C, 8) && (g.ld_aux & 3) == 0 &&
                                 aligned(g.aux_in, 8) && aligned(g.aux_out, 8));
+    const int64_t gn = n0 + wn0 + ru * 4;  // this lane's 4 columns, the same in every pass
+    float bias[4];
+    load_bias4<EPI>(g, gn, bias);
+    // a tile in the interior of C with aligned operands takes the path without bounds checks, in
+    // which the loads of a band (LDS, auxiliary tensor, old C) are issued before any arithmetic
+    const bool interior = vec_ok && m0 + BM <= g.M && n0 + BN <= g.N;
+    constexpr int kPasses = 32 / RPP;
 #pragma unroll
     for (int b = 0; b < TM; ++b) {
 #pragma unroll
@@ -264,11 +293,56 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
                 *reinterpret_cast<float4*>(cw + l32 * WTN + ((u ^ (l32 & (UPR - 1))) << 2)) =
                     make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
             }
+        const int64_t gm = m0 + wm0 + b * 32 + rr;  // row of pass 0; pass i adds i * RPP
+        if (interior) {
+            float4 v4[kPasses];
+            uint2 aw[kPasses];
+            float4 old[kPasses];
 #pragma unroll
-        for (int i = 0; i < 32 / RPP; ++i) {
-            const int m = i * RPP + rr;
-            const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
-            epilogue4<EPI, CF32>(g, m0 + wm0 + b * 32 + m, n0 + wn0 + ru * 4, v.x, v.y, v.z, v.w, vec_ok);
+            for (int i = 0; i < kPasses; ++i) {
+                const int m = i * RPP + rr;
+                v4[i] = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
+            }
+            if (epi_reads_aux(EPI)) {
+#pragma unroll
+                for (int i = 0; i < kPasses; ++i)
+                    aw[i] = *reinterpret_cast<const uint2*>(g.aux_in + (gm + i * RPP) * g.ld_aux + gn);
+            }
+            if (CF32 && EPI == PP_EPI_ACCUM_F32 && g.beta) {
+#pragma unroll
+                for (int i = 0; i < kPasses; ++i)
+                    old[i] = *reinterpret_cast<const float4*>(static_cast<const float*>(g.C) + (gm + i * RPP) * g.ldc + gn);
+            }
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                float v[4] = {v4[i].x, v4[i].y, v4[i].z, v4[i].w}, pre[4];
+                float av[4] = {0.f, 0.f, 0.f, 0.f};
+                if (epi_reads_aux(EPI)) {
+                    av[0] = bf16lo(aw[i].x); av[1] = bf16hi(aw[i].x); av[2] = bf16lo(aw[i].y); av[3] = bf16hi(aw[i].y);
+                }
+                epilogue_math4<EPI>(v, pre, bias, av);
+                const int64_t row = gm + i * RPP;
+                if (epi_is_gelu(EPI) && g.aux_out)
+                    *reinterpret_cast<uint2*>(g.aux_out + row * g.ld_aux + gn) =
+                        make_uint2(pack_bf16(pre[0], pre[1]), pack_bf16(pre[2], pre[3]));
+                if (CF32) {
+                    float* cp = static_cast<float*>(g.C) + row * g.ldc + gn;
+                    if (EPI == PP_EPI_ACCUM_F32 && g.beta)
+                        *reinterpret_cast<float4*>(cp) = make_float4(old[i].x + v[0], old[i].y + v[1], old[i].z + v[2], old[i].w + v[3]);
+                    else
+                        *reinterpret_cast<float4*>(cp) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(g.C) + row * g.ldc + gn) =
+                        make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                const int m = i * RPP + rr;
+                const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
+                epilogue4<EPI, CF32>(g, gm + i * RPP, gn, v.x, v.y, v.z, v.w, bias, vec_ok);
+            }
         }
     }
 }
