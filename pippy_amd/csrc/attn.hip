@@ -1,15 +1,22 @@
 // Flash-style multi-head attention for gfx950 (forward, and a two-kernel deterministic backward)
-// on v_mfma_f32_32x32x16_bf16.
+// on v_mfma_f32_32x32x16_bf16, head dimension 64.
 //
 // Forward: a work-group owns 128 query rows of one (batch, head); each of its 4 waves owns 32 rows.
-// Keys/values stream through LDS in blocks of 64.  Scores are produced transposed,
+// Keys/values stream through LDS in blocks of 64 rows.  Scores are produced transposed,
 // S^T[kv][q] = K Q^T, so that a lane holds one query column: the online-softmax statistics are
 // per-lane scalars (one cross-lane exchange with lane^32 per reduction) and the probabilities sit
 // in registers in exactly the form the second MFMA wants as its B operand for
-// O^T[d][q] += V^T[d][kv] P^T[kv][q].  V is transposed on its way into LDS.
+// O^T[d][q] += V^T[d][kv] P^T[kv][q].
 //
 // Backward: delta = rowsum(dO * O); one kernel parallel over key blocks produces dK and dV, one
 // kernel parallel over query blocks produces dQ.  No atomics: results are run-to-run identical.
+//
+// Staging: every streamed operand is a 64 x 64 bf16 tile kept in LDS exactly as it lies in memory
+// ([row][d], 128 B per row, 16-byte chunks XOR-swizzled by the row), filled by direct-to-LDS buffer
+// loads, three stages deep with one barrier per block of 64 rows.  A fragment whose MFMA k index
+// runs along d is a ds_read_b128 of one row; a fragment whose k index runs along the tile's rows
+// (V^T in the forward pass, K^T, Q^T and dO^T in the backward pass) comes out of the same tile
+// through ds_read_b64_tr_b16, so no transposed copy is ever made.
 #include "tile.h"
 #include <math.h>
 
@@ -29,18 +36,6 @@ union Frag {
     uint4 u;
     bf16x8_t v;
 };
-
-// Two 8-byte k-runs (chunks chunk0 and chunk0 + 1, offset 4*lh) of one row of a swizzled tile.
-__device__ __forceinline__ bf16x8_t read_runs(const uint16_t* tile, int row, int chunk0, int lh) {
-    const uint2 a = *reinterpret_cast<const uint2*>(tile + row * BK + (((chunk0) ^ swz(row)) << 3) + 4 * lh);
-    const uint2 b = *reinterpret_cast<const uint2*>(tile + row * BK + (((chunk0 + 1) ^ swz(row)) << 3) + 4 * lh);
-    Frag f;
-    f.u = make_uint4(a.x, a.y, b.x, b.y);
-    return f.v;
-}
-__device__ __forceinline__ bf16x8_t read_chunk(const uint16_t* tile, int row, int chunk) {
-    return *reinterpret_cast<const bf16x8_t*>(tile + row * BK + ((chunk ^ swz(row)) << 3));
-}
 __device__ __forceinline__ bf16x8_t pack8(const float* p) {
     Frag f;
     f.u = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
@@ -49,18 +44,87 @@ __device__ __forceinline__ bf16x8_t pack8(const float* p) {
 }
 
 constexpr float kLog2e = 1.44269504088896340736f;
-constexpr float kLn2 = 0.69314718055994530942f;
+constexpr int kTile = 64 * 64;  // elements of one staged tile
+constexpr int kAttnStages = 3;
+
+// Chunk swizzle of a staged tile.  Rows r and r+1 start 32 banks apart; the first term spreads 16
+// consecutive rows read at one chunk index (ds_read_b128 fragments), the second separates rows r
+// and r+2, which a transposing read touches together.
+__device__ __forceinline__ int swz_attn(int r) { return ((r ^ (r >> 3)) & 7) ^ ((r & 2) << 1); }
+
+// Direct-to-LDS loader of 64-row tiles out of a [rows][stride] operand (64 d = 128 B per row).
+struct AttnTileLoader {
+    __amdgpu_buffer_rsrc_t rsrc;
+    int voff[2];
+    int row_bytes;
+    __device__ __forceinline__ void init(const uint16_t* base, int64_t stride, int64_t rows, int wave, int lane) {
+        rsrc = make_rsrc(base, (uint64_t)rows * (uint64_t)stride * 2);
+        row_bytes = (int)(stride * 2);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int row = (i * 4 + wave) * 8 + (lane >> 3);
+            voff[i] = row * row_bytes + (((lane & 7) ^ swz_attn(row)) << 4);
+        }
+    }
+    __device__ __forceinline__ void load(uint16_t* lds, int64_t row0, int wave) const {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i], (int)row0 * row_bytes);
+    }
+};
+
+// 64 consecutive floats into LDS with one wave instruction.
+__device__ __forceinline__ void load_floats_to_lds(__amdgpu_buffer_rsrc_t rsrc, float* lds, int64_t first, int lane) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr_t)lds, 4, lane * 4, (int)first * 4, 0, 0);
+#endif
+}
+
+// Fragment with k along d: row `row` of the tile, 16-byte chunk `chunk`.
+__device__ __forceinline__ bf16x8_t read_row_frag(const uint16_t* tile, int row, int chunk) {
+    return *reinterpret_cast<const bf16x8_t*>(tile + row * 64 + ((chunk ^ swz_attn(row)) << 3));
+}
+
+// Fragment with k along the tile's rows, for 32 columns d0 .. d0+31 and the 16 rows r0 .. r0+15.
+// The k slots of lane group g = lane / 32 are rows r0 + 4g .. + 3 and r0 + 8 + 4g .. + 3: the order
+// in which a lane of a 32x32 MFMA result holds 8 of its 16 values, so that probabilities computed
+// in registers can be the other operand without a shuffle.  Inside each block of 16 lanes, lane
+// 4j + i fetches columns 4i .. 4i+3 of row j, and the hardware hands lane m the 4 rows of column m.
+__device__ __forceinline__ bf16x8_t read_col_frag(const uint16_t* tile, int r0, int d0, int lane) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int g = lane >> 5, mb = (lane >> 4) & 1, j = (lane & 15) >> 2, i = lane & 3;
+    const int d = d0 + 16 * mb + 4 * i;
+    const int r_lo = r0 + 4 * g + j, r_hi = r_lo + 8;
+    const uint16_t* p_lo = tile + r_lo * 64 + (((d >> 3) ^ swz_attn(r_lo)) << 3) + (d & 7);
+    const uint16_t* p_hi = tile + r_hi * 64 + (((d >> 3) ^ swz_attn(r_hi)) << 3) + (d & 7);
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_t)p_lo);
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr_t)p_hi);
+    const s16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, v);
+#else
+    return bf16x8_t{};
+#endif
+}
+
+// Pipeline step shared by the three kernels: block j of `nb` has landed for every wave, and the
+// stage that block j-1 occupied is free.  `lpt` loads per block per wave.
+template <int LPT>
+__device__ __forceinline__ void await_block(int64_t j, int64_t nb) {
+    if (j + 1 < nb) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+}
 
 // ---- forward ----------------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
-    constexpr int DS = D / 64;   // 64-wide sub-tiles along d
-    constexpr int KS = D / 16;   // MFMA k steps along d
-    constexpr int DT = D / 32;   // 32-row tiles of O^T
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[DS][64 * BK];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * BK];
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+    static_assert(D == 64, "head dimension 64");
+    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
+    constexpr int kStage = 2 * kTile;  // K tile, V tile
+    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
     // causal: late query blocks have the most key blocks; launch them first
@@ -69,13 +133,22 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     const int64_t qi = qw0 + l32;  // this lane's query row
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
-    const uint16_t* kp = a.k + b * a.stride_b + h * D;
-    const uint16_t* vp = a.v + b * a.stride_b + h * D;
+    AttnTileLoader lk, lv;
+    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
+    auto issue = [&](int stage, int64_t j) {
+        lk.load(lds + stage * kStage, j * 64, wave);
+        lv.load(lds + stage * kStage + kTile, j * 64, wave);
+    };
 
     bf16x8_t qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
         qf[ks] = *reinterpret_cast<const bf16x8_t*>(qp + qi * a.stride_s + 16 * ks + 8 * lh);
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+        if (t < n_blocks) issue(t, t);
 
     f32x16_t oacc[DT];
 #pragma unroll
@@ -85,24 +158,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     float m_run = -INFINITY, l_run = 0.f;
     const float c = a.scale * kLog2e;
 
-    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
-    Stage<64, false> sk[DS];
-    Stage<D, true> sv;
-#pragma unroll
-    for (int s = 0; s < DS; ++s) sk[s].load(kp, a.stride_s, 0, a.S, 64 * s, D, tid);
-    sv.load(vp, a.stride_s, 0, D, 0, a.S, tid);
-
+    int stage = 0;
     for (int64_t j = 0; j < n_blocks; ++j) {
         const int64_t kv0 = j * 64;
-#pragma unroll
-        for (int s = 0; s < DS; ++s) sk[s].store(Ks[s], tid);
-        sv.store(Vt, tid);
-        __syncthreads();
-        if (j + 1 < n_blocks) {
-#pragma unroll
-            for (int s = 0; s < DS; ++s) sk[s].load(kp, a.stride_s, kv0 + 64, a.S, 64 * s, D, tid);
-            sv.load(vp, a.stride_s, 0, D, kv0 + 64, a.S, tid);
-        }
+        await_block<4>(j, n_blocks);
+        if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
+        const uint16_t* Ks = lds + stage * kStage;
+        const uint16_t* Vs = Ks + kTile;
+        stage = stage + 1 == NS ? 0 : stage + 1;
         const bool active = !CAUSAL || (kv0 <= qw0 + 31);
         if (active) {
             f32x16_t sacc[2];
@@ -114,7 +177,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
             for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t kf = read_chunk(Ks[ks / 4], 32 * t + l32, 2 * (ks % 4) + lh);
+                    const bf16x8_t kf = read_row_frag(Ks, 32 * t + l32, 2 * ks + lh);
                     sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[t], 0, 0, 0);
                 }
             }
@@ -162,12 +225,11 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
                     const bf16x8_t pb = pack8(pv);
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
-                        const bf16x8_t vf = read_runs(Vt, 32 * dt + l32, 4 * t + 2 * gp, lh);
+                        const bf16x8_t vf = read_col_frag(Vs, 32 * t + 16 * gp, 32 * dt, lane);
                         oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, oacc[dt], 0, 0, 0);
                     }
                 }
         }
-        __syncthreads();
     }
 
     const float inv_l = 1.0f / l_run;
@@ -215,29 +277,40 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
 
 // ---- backward: dK, dV (parallel over key blocks) ------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
-    constexpr int DS = D / 64, KS = D / 16, DT = D / 32;
-    __shared__ __attribute__((aligned(16))) uint16_t Qs[DS][64 * BK];   // [q][d]
-    __shared__ __attribute__((aligned(16))) uint16_t Os[DS][64 * BK];   // dO [q][d]
-    __shared__ __attribute__((aligned(16))) uint16_t Qt[D * BK];        // [d][q]
-    __shared__ __attribute__((aligned(16))) uint16_t Ot[D * BK];        // dO [d][q]
-    __shared__ __attribute__((aligned(16))) float lse_s[64];
-    __shared__ __attribute__((aligned(16))) float delta_s[64];
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
+    static_assert(D == 64, "head dimension 64");
+    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
+    constexpr int kStage = 2 * kTile + 256;  // Q tile, dO tile, 64 lse, 64 delta
+    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
     const int64_t kv0 = (int64_t)blockIdx.x * 128;
     const int64_t kvw0 = kv0 + 32 * wave;
     const int64_t kvi = kvw0 + l32;  // this lane's key row
 
-    const uint16_t* qp = a.q + b * a.stride_b + h * D;
     const uint16_t* kp = a.k + b * a.stride_b + h * D;
     const uint16_t* vp = a.v + b * a.stride_b + h * D;
     const int64_t ldo = a.H * D;
-    const uint16_t* dop = a.d_o + b * a.S * ldo + h * D;
-    const float* lsep = a.lse + (b * a.H + h) * a.S;
-    const float* deltap = a.delta + (b * a.H + h) * a.S;
+    AttnTileLoader lq, ldo_;
+    lq.init(a.q + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    ldo_.init(a.d_o + b * a.S * ldo + h * D, ldo, a.S, wave, lane);
+    // waves 0 and 2 fetch lse, waves 1 and 3 delta (the same values twice: every wave issues the
+    // same number of loads, which keeps the vmcnt arithmetic uniform)
+    const float* stat = ((wave & 1) ? a.delta : a.lse) + (b * a.H + h) * a.S;
+    const __amdgpu_buffer_rsrc_t rstat = make_rsrc(stat, (uint64_t)a.S * 4);
+    const int stat_off = 2 * kTile + ((wave & 1) ? 128 : 0);
+
+    const int64_t jq_begin = CAUSAL ? kv0 / 64 : 0;
+    const int64_t nb = a.S / 64 - jq_begin;
+    auto issue = [&](int stage, int64_t j) {
+        uint16_t* st = lds + stage * kStage;
+        lq.load(st, (jq_begin + j) * 64, wave);
+        ldo_.load(st + kTile, (jq_begin + j) * 64, wave);
+        load_floats_to_lds(rstat, reinterpret_cast<float*>(st + stat_off), (jq_begin + j) * 64, lane);
+    };
 
     bf16x8_t kf[KS], vf[KS];
 #pragma unroll
@@ -245,6 +318,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
         kf[ks] = *reinterpret_cast<const bf16x8_t*>(kp + kvi * a.stride_s + 16 * ks + 8 * lh);
         vf[ks] = *reinterpret_cast<const bf16x8_t*>(vp + kvi * a.stride_s + 16 * ks + 8 * lh);
     }
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+        if (t < nb) issue(t, t);
+
     f32x16_t dvacc[DT], dkacc[DT];
 #pragma unroll
     for (int t = 0; t < DT; ++t)
@@ -255,52 +332,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
         }
     const float c = a.scale * kLog2e;
 
-    const int64_t jq_begin = CAUSAL ? kv0 / 64 : 0;
-    const int64_t jq_end = a.S / 64;
-    Stage<64, false> sq[DS], so[DS];
-    Stage<D, true> sqt, sot;
-    float lse_r = 0.f, delta_r = 0.f;
-    {
-        const int64_t qc0 = jq_begin * 64;
-#pragma unroll
-        for (int s = 0; s < DS; ++s) {
-            sq[s].load(qp, a.stride_s, qc0, a.S, 64 * s, D, tid);
-            so[s].load(dop, ldo, qc0, a.S, 64 * s, D, tid);
-        }
-        sqt.load(qp, a.stride_s, 0, D, qc0, a.S, tid);
-        sot.load(dop, ldo, 0, D, qc0, a.S, tid);
-        if (tid < 64) {
-            lse_r = lsep[qc0 + tid] * kLog2e;
-            delta_r = deltap[qc0 + tid];
-        }
-    }
-    for (int64_t jq = jq_begin; jq < jq_end; ++jq) {
-        const int64_t qc0 = jq * 64;
-#pragma unroll
-        for (int s = 0; s < DS; ++s) {
-            sq[s].store(Qs[s], tid);
-            so[s].store(Os[s], tid);
-        }
-        sqt.store(Qt, tid);
-        sot.store(Ot, tid);
-        if (tid < 64) {
-            lse_s[tid] = lse_r;
-            delta_s[tid] = delta_r;
-        }
-        __syncthreads();
-        if (jq + 1 < jq_end) {
-#pragma unroll
-            for (int s = 0; s < DS; ++s) {
-                sq[s].load(qp, a.stride_s, qc0 + 64, a.S, 64 * s, D, tid);
-                so[s].load(dop, ldo, qc0 + 64, a.S, 64 * s, D, tid);
-            }
-            sqt.load(qp, a.stride_s, 0, D, qc0 + 64, a.S, tid);
-            sot.load(dop, ldo, 0, D, qc0 + 64, a.S, tid);
-            if (tid < 64) {
-                lse_r = lsep[qc0 + 64 + tid] * kLog2e;
-                delta_r = deltap[qc0 + 64 + tid];
-            }
-        }
+    int stage = 0;
+    for (int64_t j = 0; j < nb; ++j) {
+        const int64_t qc0 = (jq_begin + j) * 64;
+        await_block<5>(j, nb);
+        if (j + NS - 1 < nb) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
+        const uint16_t* Qs = lds + stage * kStage;
+        const uint16_t* Os = Qs + kTile;
+        const float* lse_s = reinterpret_cast<const float*>(Qs + 2 * kTile);
+        const float* delta_s = lse_s + 64;
+        stage = stage + 1 == NS ? 0 : stage + 1;
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const int64_t qt0 = qc0 + 32 * qt;
@@ -313,8 +354,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t qfr = read_chunk(Qs[ks / 4], 32 * qt + l32, 2 * (ks % 4) + lh);
-                const bf16x8_t ofr = read_chunk(Os[ks / 4], 32 * qt + l32, 2 * (ks % 4) + lh);
+                const bf16x8_t qfr = read_row_frag(Qs, 32 * qt + l32, 2 * ks + lh);
+                const bf16x8_t ofr = read_row_frag(Os, 32 * qt + l32, 2 * ks + lh);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr, kf[ks], sacc, 0, 0, 0);
                 dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ofr, vf[ks], dpacc, 0, 0, 0);
             }
@@ -325,18 +366,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
             for (int g = 0; g < 4; ++g) {
                 const float4 l4 = *reinterpret_cast<const float4*>(lse_s + 32 * qt + 8 * g + 4 * lh);
                 const float4 d4 = *reinterpret_cast<const float4*>(delta_s + 32 * qt + 8 * g + 4 * lh);
-                const float lq[4] = {l4.x, l4.y, l4.z, l4.w};
-                const float dq_[4] = {d4.x, d4.y, d4.z, d4.w};
+                const float lq4[4] = {l4.x * kLog2e, l4.y * kLog2e, l4.z * kLog2e, l4.w * kLog2e};
+                const float dq4[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int v = 4 * g + e;
-                    float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lq[e]));
+                    float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lq4[e]));
                     if (diag) {
                         const int64_t qrow = qt0 + 8 * g + 4 * lh + e;
                         if (kvi > qrow) p = 0.f;
                     }
                     pv[v] = p;
-                    dsv[v] = p * (dpacc[v] - dq_[e]);
+                    dsv[v] = p * (dpacc[v] - dq4[e]);
                 }
             }
 #pragma unroll
@@ -345,14 +386,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
                 const bf16x8_t dsb = pack8(dsv + 8 * gp);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t otf = read_runs(Ot, 32 * dt + l32, 4 * qt + 2 * gp, lh);
-                    const bf16x8_t qtf = read_runs(Qt, 32 * dt + l32, 4 * qt + 2 * gp, lh);
+                    const bf16x8_t otf = read_col_frag(Os, 32 * qt + 16 * gp, 32 * dt, lane);
+                    const bf16x8_t qtf = read_col_frag(Qs, 32 * qt + 16 * gp, 32 * dt, lane);
                     dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(otf, pb, dvacc[dt], 0, 0, 0);
                     dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtf, dsb, dkacc[dt], 0, 0, 0);
                 }
             }
         }
-        __syncthreads();
     }
     // dvacc[dt][v]: d = 32 dt + 8 (v/4) + 4 lh + v%4, kv = kvi
     uint16_t* dkp = a.dk + b * a.stride_b + h * D + kvi * a.stride_s;
@@ -373,13 +413,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
 
 // ---- backward: dQ (parallel over query blocks) ---------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
-    constexpr int DS = D / 64, KS = D / 16, DT = D / 32;
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[DS][64 * BK];  // [kv][d]
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[DS][64 * BK];  // [kv][d]
-    __shared__ __attribute__((aligned(16))) uint16_t Kt[D * BK];       // [d][kv]
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+    static_assert(D == 64, "head dimension 64");
+    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
+    constexpr int kStage = 2 * kTile;  // K tile, V tile
+    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
     const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 128;
@@ -387,10 +428,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
     const int64_t qi = qw0 + l32;
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
-    const uint16_t* kp = a.k + b * a.stride_b + h * D;
-    const uint16_t* vp = a.v + b * a.stride_b + h * D;
     const int64_t ldo = a.H * D;
     const uint16_t* dop = a.d_o + b * a.S * ldo + h * D;
+    AttnTileLoader lk, lv;
+    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
+    auto issue = [&](int stage, int64_t j) {
+        lk.load(lds + stage * kStage, j * 64, wave);
+        lv.load(lds + stage * kStage + kTile, j * 64, wave);
+    };
 
     bf16x8_t qf[KS], dof[KS];
 #pragma unroll
@@ -400,6 +447,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
     }
     const float lse_q = a.lse[(b * a.H + h) * a.S + qi] * kLog2e;
     const float delta_q = a.delta[(b * a.H + h) * a.S + qi];
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+        if (t < n_blocks) issue(t, t);
     const float c = a.scale * kLog2e;
 
     f32x16_t dqacc[DT];
@@ -408,33 +458,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) dqacc[t][e] = 0.f;
 
-    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
-    Stage<64, false> sk[DS], sv[DS];
-    Stage<D, true> skt;
-#pragma unroll
-    for (int s = 0; s < DS; ++s) {
-        sk[s].load(kp, a.stride_s, 0, a.S, 64 * s, D, tid);
-        sv[s].load(vp, a.stride_s, 0, a.S, 64 * s, D, tid);
-    }
-    skt.load(kp, a.stride_s, 0, D, 0, a.S, tid);
-
+    int stage = 0;
     for (int64_t j = 0; j < n_blocks; ++j) {
         const int64_t kv0 = j * 64;
-#pragma unroll
-        for (int s = 0; s < DS; ++s) {
-            sk[s].store(Ks[s], tid);
-            sv[s].store(Vs[s], tid);
-        }
-        skt.store(Kt, tid);
-        __syncthreads();
-        if (j + 1 < n_blocks) {
-#pragma unroll
-            for (int s = 0; s < DS; ++s) {
-                sk[s].load(kp, a.stride_s, kv0 + 64, a.S, 64 * s, D, tid);
-                sv[s].load(vp, a.stride_s, kv0 + 64, a.S, 64 * s, D, tid);
-            }
-            skt.load(kp, a.stride_s, 0, D, kv0 + 64, a.S, tid);
-        }
+        await_block<4>(j, n_blocks);
+        if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
+        const uint16_t* Ks = lds + stage * kStage;
+        const uint16_t* Vs = Ks + kTile;
+        stage = stage + 1 == NS ? 0 : stage + 1;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int64_t kt0 = kv0 + 32 * t;
@@ -447,8 +478,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t kfr = read_chunk(Ks[ks / 4], 32 * t + l32, 2 * (ks % 4) + lh);
-                const bf16x8_t vfr = read_chunk(Vs[ks / 4], 32 * t + l32, 2 * (ks % 4) + lh);
+                const bf16x8_t kfr = read_row_frag(Ks, 32 * t + l32, 2 * ks + lh);
+                const bf16x8_t vfr = read_row_frag(Vs, 32 * t + l32, 2 * ks + lh);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[ks], sacc, 0, 0, 0);
                 dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[ks], dpacc, 0, 0, 0);
             }
@@ -469,12 +500,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
                 const bf16x8_t dsb = pack8(dsv + 8 * gp);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t ktf = read_runs(Kt, 32 * dt + l32, 4 * t + 2 * gp, lh);
+                    const bf16x8_t ktf = read_col_frag(Ks, 32 * t + 16 * gp, 32 * dt, lane);
                     dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf, dsb, dqacc[dt], 0, 0, 0);
                 }
             }
         }
-        __syncthreads();
     }
     uint16_t* dqp = a.dq + b * a.stride_b + h * D + qi * a.stride_s;
 #pragma unroll
