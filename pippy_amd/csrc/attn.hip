@@ -1,15 +1,21 @@
 // Flash-style multi-head attention for gfx950 (forward, and a two-kernel deterministic backward)
 // on v_mfma_f32_32x32x16_bf16, head dimension 64.
 //
-// Forward: a work-group owns 128 query rows of one (batch, head); each of its 4 waves owns 32 rows.
-// Keys/values stream through LDS in blocks of 64 rows.  Scores are produced transposed,
+// Forward: a work-group owns 64 query rows of one (batch, head) and streams keys/values through LDS
+// in blocks of 64 rows.  Its 4 waves are 2 groups of 32 query rows x 2 halves of every key block:
+// the two waves of a row group keep separate softmax statistics and output accumulators over their
+// 32 of every 64 keys and merge them once, through LDS, after the last block.  That halves the
+// length of the dependent chain MFMA -> softmax -> MFMA per key block, which is what bounds a causal
+// launch (its longest work-group, not its total work).  Scores are produced transposed,
 // S^T[kv][q] = K Q^T, so that a lane holds one query column: the online-softmax statistics are
 // per-lane scalars (one cross-lane exchange with lane^32 per reduction) and the probabilities sit
 // in registers in exactly the form the second MFMA wants as its B operand for
 // O^T[d][q] += V^T[d][kv] P^T[kv][q].
 //
-// Backward: delta = rowsum(dO * O); one kernel parallel over key blocks produces dK and dV, one
-// kernel parallel over query blocks produces dQ.  No atomics: results are run-to-run identical.
+// Backward: delta = rowsum(dO * O); one kernel parallel over key blocks (64 keys) produces dK and
+// dV, one kernel parallel over query blocks (64 queries) produces dQ, with the same 2 x 2 split of
+// the waves: partial sums of the two halves are added in a fixed order through LDS.  No atomics:
+// results are run-to-run identical.
 //
 // Staging: every streamed operand is a 64 x 64 bf16 tile kept in LDS exactly as it lies in memory
 // ([row][d], 128 B per row, 16-byte chunks XOR-swizzled by the row), filled by direct-to-LDS buffer
@@ -117,7 +123,7 @@ __device__ __forceinline__ void await_block(int64_t j, int64_t nb) {
 
 // ---- forward ----------------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
     static_assert(D == 64, "head dimension 64");
     constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
     constexpr int kStage = 2 * kTile;  // K tile, V tile
@@ -125,18 +131,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave & 1, half = wave >> 1;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
     // causal: late query blocks have the most key blocks; launch them first
-    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 128;
-    const int64_t qw0 = q0 + 32 * wave;
+    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 64;
+    const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;  // this lane's query row
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
     AttnTileLoader lk, lv;
     lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
-    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
+    const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
     auto issue = [&](int stage, int64_t j) {
         lk.load(lds + stage * kStage, j * 64, wave);
         lv.load(lds + stage * kStage + kTile, j * 64, wave);
@@ -160,54 +167,47 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
     int stage = 0;
     for (int64_t j = 0; j < n_blocks; ++j) {
-        const int64_t kv0 = j * 64;
+        const int64_t kt0 = j * 64 + 32 * half;  // first key of this wave's half block
         await_block<4>(j, n_blocks);
         if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Ks = lds + stage * kStage;
         const uint16_t* Vs = Ks + kTile;
         stage = stage + 1 == NS ? 0 : stage + 1;
-        const bool active = !CAUSAL || (kv0 <= qw0 + 31);
+        const bool active = !CAUSAL || (kt0 <= qw0 + 31);
         if (active) {
-            f32x16_t sacc[2];
+            f32x16_t sacc;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
+            for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t kf = read_row_frag(Ks, 32 * t + l32, 2 * ks + lh);
-                    sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[t], 0, 0, 0);
-                }
+                const bf16x8_t kf = read_row_frag(Ks, 32 * half + l32, 2 * ks + lh);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
             }
-            // sacc[t][v]: kv = kv0 + 32 t + 8 (v/4) + 4 lh + v%4, q = qi
-            const bool diag = CAUSAL && (kv0 + 63 > qw0);
+            // sacc[v]: kv = kt0 + 8 (v/4) + 4 lh + v%4, q = qi
+            const bool diag = CAUSAL && (kt0 + 31 > qw0);
             // m_run tracks the maximum of the raw scores; c > 0, so scaling commutes with max
             float mloc = -INFINITY;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    if (diag) {
-                        const int64_t kv = kv0 + 32 * t + 8 * (v >> 2) + 4 * lh + (v & 3);
-                        if (kv > qi) sacc[t][v] = -INFINITY;
-                    }
-                    mloc = fmaxf(mloc, sacc[t][v]);
+            for (int v = 0; v < 16; ++v) {
+                if (diag) {
+                    const int64_t kv = kt0 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                    if (kv > qi) sacc[v] = -INFINITY;
                 }
+                mloc = fmaxf(mloc, sacc[v]);
+            }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            // a row whose keys of this half block are all masked keeps its statistics
             const float m_new = fmaxf(m_run, mloc);
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-            const float mc = m_new * c;
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+            const float mc = m_use * c;
             float psum = 0.f;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float p = __builtin_amdgcn_exp2f(fmaf(sacc[t][v], c, -mc));
-                    sacc[t][v] = p;
-                    psum += p;
-                }
+            for (int v = 0; v < 16; ++v) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -mc));
+                sacc[v] = p;
+                psum += p;
+            }
             psum += __shfl_xor(psum, 32, 64);
             l_run = l_run * alpha + psum;
             m_run = m_new;
@@ -216,34 +216,55 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int gp = 0; gp < 2; ++gp) {
+                float pv[8];
 #pragma unroll
-                for (int gp = 0; gp < 2; ++gp) {
-                    float pv[8];
+                for (int e = 0; e < 8; ++e) pv[e] = sacc[8 * gp + e];
+                const bf16x8_t pb = pack8(pv);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) pv[e] = sacc[t][8 * gp + e];
-                    const bf16x8_t pb = pack8(pv);
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        const bf16x8_t vf = read_col_frag(Vs, 32 * t + 16 * gp, 32 * dt, lane);
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, oacc[dt], 0, 0, 0);
-                    }
+                for (int dt = 0; dt < DT; ++dt) {
+                    const bf16x8_t vf = read_col_frag(Vs, 32 * half + 16 * gp, 32 * dt, lane);
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, oacc[dt], 0, 0, 0);
                 }
+            }
         }
     }
 
-    const float inv_l = 1.0f / l_run;
-    uint16_t* op = a.o + (b * a.S + qi) * (a.H * D) + h * D;
+    // merge the two halves of every key block: [grp][34 values][64 lanes] floats
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+    float* xs = reinterpret_cast<float*>(lds) + grp * (34 * 64) + lane;
+    if (half == 1) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int d = 32 * dt + 8 * g + 4 * lh;
-            *reinterpret_cast<uint2*>(op + d) =
-                make_uint2(pack_bf16(oacc[dt][4 * g + 0] * inv_l, oacc[dt][4 * g + 1] * inv_l),
-                           pack_bf16(oacc[dt][4 * g + 2] * inv_l, oacc[dt][4 * g + 3] * inv_l));
-        }
-    if (lh == 0) a.lse[(b * a.H + h) * a.S + qi] = m_run * a.scale + logf(l_run);
+            for (int e = 0; e < 16; ++e) xs[(16 * dt + e) * 64] = oacc[dt][e];
+        xs[32 * 64] = m_run;
+        xs[33 * 64] = l_run;
+    }
+    __syncthreads();
+    if (half == 0) {
+        const float m1 = xs[32 * 64], l1 = xs[33 * 64];
+        const float m = fmaxf(m_run, m1);  // finite: key 0 is visible to every query
+        const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c);
+        const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * c);
+        const float l = l_run * a0 + l1 * a1;
+        const float inv_l = 1.0f / l;
+        const float w0 = a0 * inv_l, w1 = a1 * inv_l;
+        uint16_t* op = a.o + (b * a.S + qi) * (a.H * D) + h * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    o[e] = oacc[dt][4 * g + e] * w0 + xs[(16 * dt + 4 * g + e) * 64] * w1;
+                const int d = 32 * dt + 8 * g + 4 * lh;
+                *reinterpret_cast<uint2*>(op + d) = make_uint2(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]));
+            }
+        if (lh == 0) a.lse[(b * a.H + h) * a.S + qi] = m * a.scale + logf(l);
+    }
 }
 
 // ---- backward: delta[b, h, q] = sum_d dO * O ---------------------------------------------------
@@ -277,7 +298,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
 
 // ---- backward: dK, dV (parallel over key blocks) ------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) {
     static_assert(D == 64, "head dimension 64");
     constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
     constexpr int kStage = 2 * kTile + 256;  // Q tile, dO tile, 64 lse, 64 delta
@@ -285,10 +306,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave & 1, half = wave >> 1;  // 32 keys of the block x 32 of every 64 queries
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t kv0 = (int64_t)blockIdx.x * 128;
-    const int64_t kvw0 = kv0 + 32 * wave;
+    const int64_t kv0 = (int64_t)blockIdx.x * 64;
+    const int64_t kvw0 = kv0 + 32 * grp;
     const int64_t kvi = kvw0 + l32;  // this lane's key row
 
     const uint16_t* kp = a.k + b * a.stride_b + h * D;
@@ -342,10 +364,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
         const float* lse_s = reinterpret_cast<const float*>(Qs + 2 * kTile);
         const float* delta_s = lse_s + 64;
         stage = stage + 1 == NS ? 0 : stage + 1;
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-            const int64_t qt0 = qc0 + 32 * qt;
-            if (CAUSAL && (qt0 + 31 < kvw0)) continue;  // every query precedes every key: masked
+        const int qt = half;
+        const int64_t qt0 = qc0 + 32 * qt;
+        if (!CAUSAL || (qt0 + 31 >= kvw0)) {  // else every query precedes every key: masked
             f32x16_t sacc, dpacc;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
@@ -394,6 +415,29 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             }
         }
     }
+    // add the partial sums of the two query halves: [grp][32 values][64 lanes] floats, dV then dK
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+    float* xs = reinterpret_cast<float*>(lds) + grp * (32 * 64) + lane;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        f32x16_t(&acc)[DT] = pass == 0 ? dvacc : dkacc;
+        if (half == 1) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) xs[(16 * dt + e) * 64] = acc[dt][e];
+        }
+        __syncthreads();
+        if (half == 0) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[dt][e] += xs[(16 * dt + e) * 64];
+        }
+        __syncthreads();
+    }
+    if (half != 0) return;
     // dvacc[dt][v]: d = 32 dt + 8 (v/4) + 4 lh + v%4, kv = kvi
     uint16_t* dkp = a.dk + b * a.stride_b + h * D + kvi * a.stride_s;
     uint16_t* dvp = a.dv + b * a.stride_b + h * D + kvi * a.stride_s;
@@ -413,7 +457,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 
 // ---- backward: dQ (parallel over query blocks) ---------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
     static_assert(D == 64, "head dimension 64");
     constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
     constexpr int kStage = 2 * kTile;  // K tile, V tile
@@ -421,10 +465,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave & 1, half = wave >> 1;  // 32 queries of the block x 32 of every 64 keys
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 128;
-    const int64_t qw0 = q0 + 32 * wave;
+    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 64;
+    const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
@@ -433,7 +478,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     AttnTileLoader lk, lv;
     lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
-    const int64_t n_blocks = CAUSAL ? (q0 + 128 + 63) / 64 : a.S / 64;
+    const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
     auto issue = [&](int stage, int64_t j) {
         lk.load(lds + stage * kStage, j * 64, wave);
         lv.load(lds + stage * kStage + kTile, j * 64, wave);
@@ -466,10 +511,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
         const uint16_t* Ks = lds + stage * kStage;
         const uint16_t* Vs = Ks + kTile;
         stage = stage + 1 == NS ? 0 : stage + 1;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int64_t kt0 = kv0 + 32 * t;
-            if (CAUSAL && (kt0 > qw0 + 31)) continue;
+        const int t = half;
+        const int64_t kt0 = kv0 + 32 * t;
+        if (!CAUSAL || (kt0 <= qw0 + 31)) {
             f32x16_t sacc, dpacc;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
@@ -506,6 +550,22 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
             }
         }
     }
+    // add the partial sums of the two key halves: [grp][32 values][64 lanes] floats
+    wait_lds();
+    __builtin_amdgcn_s_barrier();
+    float* xs = reinterpret_cast<float*>(lds) + grp * (32 * 64) + lane;
+    if (half == 1) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) xs[(16 * dt + e) * 64] = dqacc[dt][e];
+    }
+    __syncthreads();
+    if (half != 0) return;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dqacc[dt][e] += xs[(16 * dt + e) * 64];
     uint16_t* dqp = a.dq + b * a.stride_b + h * D + qi * a.stride_s;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -533,7 +593,7 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
         if (!aligned(d->d_o, 16) || !aligned(d->dq, 16) || !aligned(d->dk, 16) || !aligned(d->dv, 16))
             return fail(PP_ERR_INVALID, "%s: gradients must be 16-byte aligned", who);
     }
-    if (d->S / 128 > 65535 || d->H > 65535 || d->B > 65535) return fail(PP_ERR_UNSUPPORTED, "%s: grid too large", who);
+    if (d->S / 64 > 65535 || d->H > 65535 || d->B > 65535) return fail(PP_ERR_UNSUPPORTED, "%s: grid too large", who);
     return PP_OK;
 }
 
@@ -560,7 +620,7 @@ extern "C" int pp_attn_fwd(const pp_attn_desc* d, pp_stream stream) {
     if (d->B == 0 || d->S == 0) return PP_OK;
     const AttnArgs a = to_args(d);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    dim3 grid((uint32_t)(d->S / 128), (uint32_t)d->H, (uint32_t)d->B);
+    dim3 grid((uint32_t)(d->S / 64), (uint32_t)d->H, (uint32_t)d->B);
     if (d->causal) hipLaunchKernelGGL((attn_fwd_kernel<64, true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((attn_fwd_kernel<64, false>), grid, dim3(256), 0, st, a);
     return check_launch("attn_fwd_kernel");
@@ -573,7 +633,7 @@ extern "C" int pp_attn_bwd(const pp_attn_desc* d, pp_stream stream) {
     const AttnArgs a = to_args(d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((uint32_t)((d->B * d->S + 3) / 4)), dim3(256), 0, st, a);
-    dim3 grid((uint32_t)(d->S / 128), (uint32_t)d->H, (uint32_t)d->B);
+    dim3 grid((uint32_t)(d->S / 64), (uint32_t)d->H, (uint32_t)d->B);
     if (d->causal) {
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<64, true>), grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL((attn_bwd_dq_kernel<64, true>), grid, dim3(256), 0, st, a);
