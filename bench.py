@@ -173,7 +173,7 @@ def main():
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
-                              "traffic": None, "kernel": "gemm_bf16_kernel",
+                              "traffic": None, "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel",
                               "launches_per_step": cnt // n_prof,
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
                               "gemm_ms_per_step": round(ms / n_prof, 3)}

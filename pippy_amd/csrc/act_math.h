@@ -9,27 +9,30 @@ namespace pp {
 __device__ __forceinline__ float gelu_erf(float x) {
     return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
-// tanh through the hardware exp2 and reciprocal: 1 - 2 / (e^(2u) + 1).  The absolute error is a few
-// 1e-7 everywhere (e^(2u) = inf gives exactly 1, e^(2u) = 0 exactly -1), which is what the GELU
-// forms below need: they multiply tanh by values of order one.
-__device__ __forceinline__ float fast_tanh(float u) {
-    const float e = __builtin_amdgcn_exp2f(u * 2.88539008177792681472f);
-    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-}
+// The tanh form of GELU written through the logistic function: with u = k (x + c x^3),
+//   0.5 x (1 + tanh(u)) = x * s,   s = 1 / (1 + e^(-2u)),
+// so one hardware exp2 and one reciprocal do the transcendental work.  e^(-2u) = inf gives s = 0
+// and e^(-2u) = 0 gives s = 1 exactly; the absolute error of s is a few 1e-8.
+constexpr float kGeluK = 0.79788456080286535588f, kGeluC = 0.044715f;
+constexpr float kGeluA = -2.0f * 1.44269504088896340736f * kGeluK;  // exponent of 2 per unit of x
+constexpr float kGeluB = kGeluA * kGeluC;                          // ... per unit of x^3
 __device__ __forceinline__ float gelu_tanh(float x) {
-    const float u = 0.79788456080286535588f * (x + 0.044715f * x * x * x);
-    return 0.5f * x * (1.0f + fast_tanh(u));
+    const float x2 = x * x;
+    const float e = __builtin_amdgcn_exp2f(x * fmaf(x2, kGeluB, kGeluA));
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 __device__ __forceinline__ float dgelu_erf(float x) {
     const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
     const float pdf = 0.39894228040143267794f * __expf(-0.5f * x * x);
     return cdf + x * pdf;
 }
+// d/dx [x s] = s + x s (1 - s) 2 u',  u' = k (1 + 3 c x^2).
 __device__ __forceinline__ float dgelu_tanh(float x) {
-    const float k = 0.79788456080286535588f, c = 0.044715f;
-    const float u = k * (x + c * x * x * x);
-    const float t = fast_tanh(u);
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * k * (1.0f + 3.0f * c * x * x);
+    const float x2 = x * x;
+    const float e = __builtin_amdgcn_exp2f(x * fmaf(x2, kGeluB, kGeluA));
+    const float s = __builtin_amdgcn_rcpf(1.0f + e);
+    const float du2 = fmaf(x2, 6.0f * kGeluK * kGeluC, 2.0f * kGeluK);
+    return s * fmaf(x * du2, 1.0f - s, 1.0f);
 }
 
 }  // namespace pp

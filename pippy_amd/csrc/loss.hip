@@ -28,6 +28,7 @@ __global__ __launch_bounds__(256) void ce_count_kernel(const int64_t* __restrict
 }
 
 constexpr int kCeThreads = 1024;
+constexpr float kLog2e = 1.44269504088896340736f;
 
 __device__ __forceinline__ float block_reduce_max(float v, float* sh) {
     v = wave_max(v);
@@ -51,6 +52,11 @@ __device__ __forceinline__ float block_reduce_sum(float v, float* sh) {
 }
 
 // bf16 logits, one work-group per row, NC 16-byte chunks per lane held in registers.
+// The kernel is bound by VALU issue as much as by HBM, so the per-element work is kept minimal:
+// columns past V are turned into -inf when the row is loaded (no bounds checks afterwards), the
+// exponentials exp(x - max) of the sum pass replace the logits in the registers (as bf16) and the
+// gradient pass only scales them, and the "- 1" of the target column is a single scalar store by
+// the lane that owns it.
 template <int NC>
 __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
     const uint16_t* __restrict__ logits, const int64_t* __restrict__ target, uint16_t* __restrict__ dlogits,
@@ -61,58 +67,69 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
     const uint16_t* xr = logits + row * ld;
     const int nchunk_v = (V + 7) >> 3;          // chunks holding at least one valid column
     const int nchunk_ld = (int)(ld >> 3);       // chunks to write (padding gets zeros)
+    constexpr uint32_t kNegInf2 = 0xff80ff80u;  // two bf16 -inf
     uint4 w[NC];
-    float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
         const int c = tid + kCeThreads * i;
+        w[i] = make_uint4(kNegInf2, kNegInf2, kNegInf2, kNegInf2);
         if (c < nchunk_v) {
             w[i] = *reinterpret_cast<const uint4*>(xr + (int64_t)c * 8);
-            const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
-                                bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+            if (c * 8 + 8 > V) {  // the one chunk that straddles V
+                uint32_t u[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (c * 8 + e < V) mx = fmaxf(mx, f[e]);
+                for (int e = 0; e < 8; ++e)
+                    if (c * 8 + e >= V)
+                        u[e >> 1] = (e & 1) ? ((u[e >> 1] & 0x0000ffffu) | 0xff800000u)
+                                            : ((u[e >> 1] & 0xffff0000u) | 0x0000ff80u);
+                w[i] = make_uint4(u[0], u[1], u[2], u[3]);
+            }
         }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+        mx = fmaxf(mx, fmaxf(fmaxf(bf16lo(w[i].x), bf16hi(w[i].x)), fmaxf(bf16lo(w[i].y), bf16hi(w[i].y))));
+        mx = fmaxf(mx, fmaxf(fmaxf(bf16lo(w[i].z), bf16hi(w[i].z)), fmaxf(bf16lo(w[i].w), bf16hi(w[i].w))));
     }
     mx = block_reduce_max(mx, sh);
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-        const int c = tid + kCeThreads * i;
-        if (c < nchunk_v) {
-            const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
-                                bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+        const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
+                            bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
+        float ex[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (c * 8 + e < V) s += expf(f[e] - mx);
+        for (int e = 0; e < 8; ++e) {
+            ex[e] = __builtin_amdgcn_exp2f((f[e] - mx) * kLog2e);
+            s += ex[e];
         }
+        w[i] = make_uint4(pack_bf16(ex[0], ex[1]), pack_bf16(ex[2], ex[3]), pack_bf16(ex[4], ex[5]),
+                          pack_bf16(ex[6], ex[7]));
     }
     s = block_reduce_sum(s, sh);
     const float lse = mx + logf(s);
     const int64_t t = target[row];
     const bool valid = (t != ignore_index && t >= 0 && t < V);
-    if (tid == 0) ws[row] = valid ? (lse - bf16_to_f32(xr[valid ? t : 0])) : 0.f;
+    const float xt = valid ? bf16_to_f32(xr[t]) : 0.f;
+    if (tid == 0) ws[row] = valid ? (lse - xt) : 0.f;
     if (!dlogits) return;
     const float scale = valid ? ws[rows + 1] : 0.f;
+    const float ps = scale / s;  // exp(x - max) * ps = softmax * scale
     uint16_t* dr = dlogits + row * ld;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
         const int c = tid + kCeThreads * i;
         if (c < nchunk_ld) {
-            float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (c < nchunk_v) {
-                const float f[8] = {bf16lo(w[i].x), bf16hi(w[i].x), bf16lo(w[i].y), bf16hi(w[i].y),
-                                    bf16lo(w[i].z), bf16hi(w[i].z), bf16lo(w[i].w), bf16hi(w[i].w)};
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int col = c * 8 + e;
-                    if (col < V) o[e] = (expf(f[e] - lse) - (col == t ? 1.0f : 0.0f)) * scale;
-                }
-            }
             *reinterpret_cast<uint4*>(dr + (int64_t)c * 8) =
-                make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
-                           pack_bf16(o[6], o[7]));
+                make_uint4(pack_bf16(bf16lo(w[i].x) * ps, bf16hi(w[i].x) * ps),
+                           pack_bf16(bf16lo(w[i].y) * ps, bf16hi(w[i].y) * ps),
+                           pack_bf16(bf16lo(w[i].z) * ps, bf16hi(w[i].z) * ps),
+                           pack_bf16(bf16lo(w[i].w) * ps, bf16hi(w[i].w) * ps));
+            // the target column, by the lane that has just written its chunk (same-address stores
+            // of one lane stay in order)
+            if (valid && c == (int)(t >> 3))
+                dr[t] = f32_to_bf16((__builtin_amdgcn_exp2f((xt - mx) * kLog2e) / s - 1.0f) * scale);
         }
     }
 }
