@@ -133,9 +133,13 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave & 1, half = wave >> 1;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int64_t b = blockIdx.z, h = blockIdx.y;
-    // causal: late query blocks have the most key blocks; launch them first
-    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 64;
+    // all blocks of a (batch, head) on one XCD; causal: late query blocks have the most key blocks
+    // and go first
+    const uint32_t nx = (uint32_t)(a.S / 64);
+    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
+    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
+    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - vid % nx : vid % nx) * 64;
     const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;  // this lane's query row
 
@@ -308,8 +312,11 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave & 1, half = wave >> 1;  // 32 keys of the block x 32 of every 64 queries
     const int l32 = lane & 31, lh = lane >> 5;
-    const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t kv0 = (int64_t)blockIdx.x * 64;
+    const uint32_t nx = (uint32_t)(a.S / 64);
+    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
+    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
+    const int64_t kv0 = (int64_t)(vid % nx) * 64;  // early key blocks see the most queries and go first
     const int64_t kvw0 = kv0 + 32 * grp;
     const int64_t kvi = kvw0 + l32;  // this lane's key row
 
@@ -467,8 +474,11 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave & 1, half = wave >> 1;  // 32 queries of the block x 32 of every 64 keys
     const int l32 = lane & 31, lh = lane >> 5;
-    const int64_t b = blockIdx.z, h = blockIdx.y;
-    const int64_t q0 = (int64_t)(CAUSAL ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * 64;
+    const uint32_t nx = (uint32_t)(a.S / 64);
+    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
+    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
+    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - vid % nx : vid % nx) * 64;
     const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;
 
@@ -593,7 +603,7 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
         if (!aligned(d->d_o, 16) || !aligned(d->dq, 16) || !aligned(d->dk, 16) || !aligned(d->dv, 16))
             return fail(PP_ERR_INVALID, "%s: gradients must be 16-byte aligned", who);
     }
-    if (d->S / 64 > 65535 || d->H > 65535 || d->B > 65535) return fail(PP_ERR_UNSUPPORTED, "%s: grid too large", who);
+    if ((d->S / 64) * d->H * d->B > 0x7fffff00ll) return fail(PP_ERR_UNSUPPORTED, "%s: grid too large", who);
     return PP_OK;
 }
 
@@ -620,7 +630,7 @@ extern "C" int pp_attn_fwd(const pp_attn_desc* d, pp_stream stream) {
     if (d->B == 0 || d->S == 0) return PP_OK;
     const AttnArgs a = to_args(d);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    dim3 grid((uint32_t)(d->S / 64), (uint32_t)d->H, (uint32_t)d->B);
+    const dim3 grid((uint32_t)(((d->S / 64) * d->H * d->B + 7) / 8 * 8));
     if (d->causal) hipLaunchKernelGGL((attn_fwd_kernel<64, true>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((attn_fwd_kernel<64, false>), grid, dim3(256), 0, st, a);
     return check_launch("attn_fwd_kernel");
@@ -633,7 +643,7 @@ extern "C" int pp_attn_bwd(const pp_attn_desc* d, pp_stream stream) {
     const AttnArgs a = to_args(d);
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((uint32_t)((d->B * d->S + 3) / 4)), dim3(256), 0, st, a);
-    dim3 grid((uint32_t)(d->S / 64), (uint32_t)d->H, (uint32_t)d->B);
+    const dim3 grid((uint32_t)(((d->S / 64) * d->H * d->B + 7) / 8 * 8));
     if (d->causal) {
         hipLaunchKernelGGL((attn_bwd_dkv_kernel<64, true>), grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL((attn_bwd_dq_kernel<64, true>), grid, dim3(256), 0, st, a);

@@ -152,13 +152,6 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t 
 // ---- the kernel -----------------------------------------------------------------------------
 extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
-// XCD-aware remap: consecutive hardware block ids round-robin over the 8 XCDs; give each XCD a
-// contiguous range of tiles so that its private L2 sees a compact set of A/B panels.
-__device__ __forceinline__ uint32_t xcd_remap(uint32_t bid, uint32_t grid) {
-    const uint32_t per_xcd = grid >> 3;  // the grid is a multiple of 8
-    return (bid & 7) * per_xcd + (bid >> 3);
-}
-
 // Tile order of the direct-to-LDS kernels: bands of kGroupM tile rows, walked m-fastest, so that
 // the tiles resident on an XCD at one time share few A and B panels.
 constexpr uint32_t kGroupM = 8;

@@ -18,6 +18,16 @@ constexpr int kGemmThreads = 256;
 
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
+// Consecutive hardware work-group ids go round-robin over the 8 XCDs, each with a private L2.  This
+// remap gives every XCD a contiguous range of logical ids (the grid must be a multiple of 8 and
+// logical ids past the real count are skipped by the caller), so that work-groups sharing operands
+// share an L2.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t bid, uint32_t grid) {
+    const uint32_t per_xcd = grid >> 3;
+    return (bid & 7) * per_xcd + (bid >> 3);
+}
+
+
 // ---- global -> register staging -----------------------------------------------------------
 // K-contiguous operand: memory [rows_total][ld], tile = ROWS x 64.
 template <int ROWS>
