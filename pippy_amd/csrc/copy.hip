@@ -30,12 +30,17 @@ struct CopyTable {
 };
 
 template <int V> struct VecT;
-template <> struct VecT<16> { typedef uint4 type; };
-template <> struct VecT<8> { typedef uint2 type; };
+// native vector types: arrays of them stay in registers
+typedef unsigned int copy_u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int copy_u32x2_t __attribute__((ext_vector_type(2)));
+template <> struct VecT<16> { typedef copy_u32x4_t type; };
+template <> struct VecT<8> { typedef copy_u32x2_t type; };
 template <> struct VecT<4> { typedef uint32_t type; };
 template <> struct VecT<2> { typedef uint16_t type; };
 template <> struct VecT<1> { typedef uint8_t type; };
 
+// Loads are unconditional (an index past the end is clamped to the last vector, whose value is then
+// not stored): a load under a branch would keep the staging values out of registers.
 template <int V>
 __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) {
     typedef typename VecT<V>::type vec;
@@ -48,17 +53,18 @@ __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) 
 
     if (g.rows_per_block == 1) {
         // long rows: this block owns one tile of one row
-        const int64_t row = b / g.col_blocks;
-        const int64_t cblk = b % g.col_blocks;
-        const int64_t base = cblk * (int64_t)(kThreads * kUnroll * V);
+        const uint32_t row = b / g.col_blocks;
+        const uint32_t cblk = b - row * g.col_blocks;
+        const int64_t base = (int64_t)cblk * (kThreads * kUnroll * V);
         const char* sp = g.src + row * g.src_stride + base;
         char* dp = g.dst + row * g.dst_stride + base;
-        const int64_t left = g.row_bytes - base;
+        const int64_t left = g.row_bytes - base;  // > 0, a multiple of V
+        const int64_t last = left - V;
         vec r[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int64_t off = (int64_t)(u * kThreads + tid) * V;
-            if (off < left) r[u] = *reinterpret_cast<const vec*>(sp + off);
+            r[u] = *reinterpret_cast<const vec*>(sp + (off < left ? off : last));
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -71,25 +77,22 @@ __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) 
         int64_t nr = g.n_rows - row0;
         if (nr > g.rows_per_block) nr = g.rows_per_block;
         const uint32_t vpr = (uint32_t)(g.row_bytes / V);
-        const uint32_t total = (uint32_t)nr * vpr;
+        const uint32_t total = (uint32_t)nr * vpr;  // > 0
         for (uint32_t idx0 = 0; idx0 < total; idx0 += kThreads * kUnroll) {
             vec r[kUnroll];
-            uint32_t rr[kUnroll], cc[kUnroll];
+            int64_t doff[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 const uint32_t idx = idx0 + u * kThreads + tid;
-                rr[u] = idx / vpr;
-                cc[u] = idx - rr[u] * vpr;
-                if (idx < total)
-                    r[u] = *reinterpret_cast<const vec*>(g.src + (row0 + rr[u]) * g.src_stride +
-                                                         (int64_t)cc[u] * V);
+                const uint32_t cl = idx < total ? idx : total - 1;
+                const uint32_t rr = cl / vpr, cc = cl - rr * vpr;
+                r[u] = *reinterpret_cast<const vec*>(g.src + (row0 + rr) * g.src_stride + (int64_t)cc * V);
+                doff[u] = (row0 + rr) * g.dst_stride + (int64_t)cc * V;
             }
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) {
                 const uint32_t idx = idx0 + u * kThreads + tid;
-                if (idx < total)
-                    *reinterpret_cast<vec*>(g.dst + (row0 + rr[u]) * g.dst_stride +
-                                            (int64_t)cc[u] * V) = r[u];
+                if (idx < total) *reinterpret_cast<vec*>(g.dst + doff[u]) = r[u];
             }
         }
     }
