@@ -106,6 +106,8 @@ def main():
     ap.add_argument("--fused-accumulate", action="store_true",
                     help="accumulate fp32 gradients in the dW GEMM epilogue instead of the accumulate kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--serial-stages", action="store_true",
+                    help="run all virtual stages on one stream instead of one stream per stage")
     ap.add_argument("--no-roofline", action="store_true")
     # workload shape (defaults: GPT-2 small, configs[2])
     ap.add_argument("--vocab", type=int, default=50257)
@@ -131,6 +133,7 @@ def main():
     N.lib()  # fail loudly if the kernel library is missing
     model, sched, stages, ids, target = build(args)
     tokens = ids.numel()
+    sched.concurrent_stages = not args.serial_stages
 
     def step():
         sched.zero_grad()
@@ -169,12 +172,16 @@ def main():
         # Instrumented pass: the same steps with every launch-list op bracketed by HIP events on
         # its stream.  Kept apart from the timed region above so that event records do not perturb
         # `value`; the kernels, shapes and order are identical.
+        # The stages run one after the other here (one stream), so that a launch's duration is its
+        # own and not that of kernels of other stages sharing the device with it.
         n_prof = max(1, min(args.steps, 3))
+        sched.concurrent_stages = False
         N.profile_start(1 << 17)
         for _ in range(n_prof):
             step()
         torch.cuda.synchronize()
         N.profile_stop()
+        sched.concurrent_stages = not args.serial_stages
         ms, work, cnt = N.profile_read(N.OP_GEMM_BF16)
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,

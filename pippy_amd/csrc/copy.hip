@@ -10,7 +10,7 @@ namespace pp {
 
 constexpr int kMaxSegs = 32;  // per launch; pp_copy_rows loops for longer tables
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+constexpr int kUnroll = 2;  // 8 KiB per work-group measured best for the logits merge
 
 struct DevSeg {
     const char* src;

@@ -15,6 +15,7 @@ run on one device.
 from __future__ import annotations
 
 import logging
+import os
 from abc import ABC, abstractmethod
 from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple, Union
 
@@ -38,6 +39,11 @@ class PipelineSchedule(ABC):
         self._pipe_info = None
         self._internal_losses: List[torch.Tensor] = []
         self._stages: List[PipelineStageBase] = []
+        self._by_index: Dict[int, PipelineStageBase] = {}
+        #: run every virtual stage on a HIP stream of its own (natively lowered stages only)
+        self.concurrent_stages = True
+        self._streams = None
+        self._events: Dict[Any, Any] = {}
         logger.info(f"Using {self.__class__.__name__}")
 
     # -- losses (reference ``PipelineSchedule.py:39-80``) -------------------------------------------
@@ -114,31 +120,88 @@ class PipelineSchedule(ABC):
         return merge_chunks(output_chunks, self._output_merge_spec)
 
     # -- execution of a merged action order on the device -------------------------------------------
+    def _stage_streams(self):
+        """One HIP stream per virtual stage, or None when the actions run on the caller's stream.
+
+        Stages are independent between hand-offs, exactly like ranks of a real pipeline, so their
+        launch lists may overlap on the device: a kernel that leaves CUs idle (a GEMM with fewer
+        tiles than CUs, the tail of any grid, the dependent chain of a causal attention block)
+        shares the machine with a kernel of another stage.  Only natively lowered stages qualify:
+        their buffers are allocated once, so no allocator block changes hands between streams."""
+        if not self.concurrent_stages or os.environ.get("PIPPY_AMD_SERIAL_STAGES") == "1":
+            return None
+        if len(self._stages) < 2 or not all(getattr(st, "is_native", False) for st in self._stages):
+            return None
+        dev = self._stages[0].device
+        if torch.device(dev).type != "cuda":
+            return None
+        if self._streams is None or len(self._streams) != len(self._stages):
+            self._streams = {st.stage_index: torch.cuda.Stream(device=dev) for st in self._stages}
+            self._events = {}
+        return self._streams
+
+    def _event(self, key):
+        ev = self._events.get(key)
+        if ev is None:
+            ev = self._events[key] = torch.cuda.Event()
+        return ev
+
     def _execute(self, actions: Sequence[order.Action], arg_mbs, kwarg_mbs, target_mbs):
-        by_index = {s.stage_index: s for s in self._stages}
+        streams = self._stage_streams()
+        if streams is None:
+            for kind, s, m in actions:
+                self._run_action(kind, s, m, arg_mbs, kwarg_mbs, target_mbs)
+            return
+        # hand-offs become events: forward (s, m) waits for forward (s-1, m), backward (s, m) for
+        # backward (s+1, m); everything of one stage stays in order on that stage's stream
+        main = torch.cuda.current_stream()
+        start = self._event("start")
+        start.record(main)
+        for st in streams.values():
+            st.wait_event(start)
+        last = max(streams)
         for kind, s, m in actions:
-            stage = by_index[s]
-            if kind == "F":
-                with record_function(f"Stage {s} Forward {m}"):
-                    if stage.fwd_chunk_id != m:
-                        raise RuntimeError(f"stage {s}: forward order broken ({stage.fwd_chunk_id} != {m})")
-                    a = arg_mbs[m] if stage.is_first else ()
-                    k = kwarg_mbs[m] if stage.is_first else {}
-                    output = stage.forward_one_chunk(a, k)
-                    self._maybe_compute_loss(stage, output, target_mbs, m)
-            elif kind == "B":
-                with record_function(f"Stage {s} Backward {m}"):
-                    if stage.bwd_chunk_id != m:
-                        raise RuntimeError(f"stage {s}: backward order broken ({stage.bwd_chunk_id} != {m})")
-                    stage.backward_one_chunk(loss=self._maybe_get_loss(stage, m))
-            elif kind == "I":
-                with record_function(f"Stage {s} BackwardInput {m}"):
-                    stage.backward_input_one_chunk(loss=self._maybe_get_loss(stage, m))
-            elif kind == "W":
-                with record_function(f"Stage {s} BackwardWeight {m}"):
-                    stage.backward_weight_one_chunk()
-            else:
-                raise ValueError(f"unknown action {kind}")
+            st = streams[s]
+            with torch.cuda.stream(st):
+                if kind == "F":
+                    if s > 0:
+                        st.wait_event(self._event(("F", s - 1, m)))
+                elif kind in ("B", "I"):
+                    if s < last:
+                        st.wait_event(self._event(("B", s + 1, m)))
+                self._run_action(kind, s, m, arg_mbs, kwarg_mbs, target_mbs)
+                if kind == "F":
+                    self._event(("F", s, m)).record(st)
+                elif kind in ("B", "I"):
+                    self._event(("B", s, m)).record(st)
+        for s, st in streams.items():
+            done = self._event(("done", s))
+            done.record(st)
+            main.wait_event(done)
+
+    def _run_action(self, kind, s, m, arg_mbs, kwarg_mbs, target_mbs):
+        stage = self._by_index[s]
+        if kind == "F":
+            with record_function(f"Stage {s} Forward {m}"):
+                if stage.fwd_chunk_id != m:
+                    raise RuntimeError(f"stage {s}: forward order broken ({stage.fwd_chunk_id} != {m})")
+                a = arg_mbs[m] if stage.is_first else ()
+                k = kwarg_mbs[m] if stage.is_first else {}
+                output = stage.forward_one_chunk(a, k)
+                self._maybe_compute_loss(stage, output, target_mbs, m)
+        elif kind == "B":
+            with record_function(f"Stage {s} Backward {m}"):
+                if stage.bwd_chunk_id != m:
+                    raise RuntimeError(f"stage {s}: backward order broken ({stage.bwd_chunk_id} != {m})")
+                stage.backward_one_chunk(loss=self._maybe_get_loss(stage, m))
+        elif kind == "I":
+            with record_function(f"Stage {s} BackwardInput {m}"):
+                stage.backward_input_one_chunk(loss=self._maybe_get_loss(stage, m))
+        elif kind == "W":
+            with record_function(f"Stage {s} BackwardWeight {m}"):
+                stage.backward_weight_one_chunk()
+        else:
+            raise ValueError(f"unknown action {kind}")
 
     @abstractmethod
     def _rank_programs(self) -> List[List[order.Action]]:
@@ -181,6 +244,8 @@ class PipelineSchedule(ABC):
 
     def _adopt_stages(self, stages: List[PipelineStageBase]):
         self._stages = link_stages(stages)
+        self._by_index = {st.stage_index: st for st in self._stages}
+        self._streams = None
         self._num_stages = self._stages[0].num_stages
         self._pipe_info = getattr(self._stages[0], "pipe_info", None)
         for stage in self._stages:
