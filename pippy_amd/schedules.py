@@ -43,6 +43,7 @@ class PipelineSchedule(ABC):
         #: run every virtual stage on a HIP stream of its own (natively lowered stages only)
         self.concurrent_stages = True
         self._streams = None
+        self._w_streams = None
         self._events: Dict[Any, Any] = {}
         logger.info(f"Using {self.__class__.__name__}")
 
@@ -137,6 +138,9 @@ class PipelineSchedule(ABC):
             return None
         if self._streams is None or len(self._streams) != len(self._stages):
             self._streams = {st.stage_index: torch.cuda.Stream(device=dev) for st in self._stages}
+            # deferred weight-gradient passes ("W" actions) read per-microbatch buffers only, so they
+            # get a stream of their own next to the stage's forward / input-gradient stream
+            self._w_streams = {st.stage_index: torch.cuda.Stream(device=dev) for st in self._stages}
             self._events = {}
         return self._streams
 
@@ -157,10 +161,22 @@ class PipelineSchedule(ABC):
         main = torch.cuda.current_stream()
         start = self._event("start")
         start.record(main)
-        for st in streams.values():
+        w_streams = self._w_streams
+        for st in list(streams.values()) + list(w_streams.values()):
             st.wait_event(start)
         last = max(streams)
+        used_w = set()
         for kind, s, m in actions:
+            if kind == "W":
+                # after the input-gradient pass of the same microbatch; W passes of a stage stay in
+                # microbatch order among themselves, which keeps the accumulation order
+                wm = self._by_index[s].bwd_weight_chunk_id
+                st = w_streams[s]
+                used_w.add(s)
+                with torch.cuda.stream(st):
+                    st.wait_event(self._event(("B", s, wm)))
+                    self._run_action(kind, s, m, arg_mbs, kwarg_mbs, target_mbs)
+                continue
             st = streams[s]
             with torch.cuda.stream(st):
                 if kind == "F":
@@ -177,6 +193,10 @@ class PipelineSchedule(ABC):
         for s, st in streams.items():
             done = self._event(("done", s))
             done.record(st)
+            main.wait_event(done)
+        for s in used_w:
+            done = self._event(("done_w", s))
+            done.record(w_streams[s])
             main.wait_event(done)
 
     def _run_action(self, kind, s, m, arg_mbs, kwarg_mbs, target_mbs):
