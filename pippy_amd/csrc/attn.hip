@@ -190,21 +190,31 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
             // sacc[v]: kv = kt0 + 8 (v/4) + 4 lh + v%4, q = qi
             const bool diag = CAUSAL && (kt0 + 31 > qw0);
             // m_run tracks the maximum of the raw scores; c > 0, so scaling commutes with max
+            if (diag) {  // wave-uniform: only blocks on the diagonal pay for the mask
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (kt0 + 8 * (v >> 2) + 4 * lh + (v & 3) > qi) sacc[v] = -INFINITY;
+            }
             float mloc = -INFINITY;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                if (diag) {
-                    const int64_t kv = kt0 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                    if (kv > qi) sacc[v] = -INFINITY;
-                }
-                mloc = fmaxf(mloc, sacc[v]);
-            }
+            for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, sacc[v]);
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-            // a row whose keys of this half block are all masked keeps its statistics
-            const float m_new = fmaxf(m_run, mloc);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-            const float mc = m_use * c;
+            // The reference maximum of a row only has to keep the exponentials in range, so it is
+            // moved (and the accumulators rescaled) only when some row of the wave exceeds it by
+            // more than 2^8 after scaling; that happens in the first block of a row and almost
+            // never again.  Any reference gives the same softmax after the final division.
+            if (__ballot(mloc * c > m_run * c + 8.0f)) {
+                const float m_new = fmaxf(m_run, mloc);
+                const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
+                l_run *= alpha;
+                m_run = m_new;
+#pragma unroll
+                for (int t = 0; t < DT; ++t)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+            }
+            // a row whose keys have all been masked so far has no reference yet: its scores are -inf
+            const float mc = (m_run == -INFINITY ? 0.f : m_run) * c;
             float psum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -213,12 +223,7 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
                 psum += p;
             }
             psum += __shfl_xor(psum, 32, 64);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
-#pragma unroll
-            for (int t = 0; t < DT; ++t)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) oacc[t][e] *= alpha;
+            l_run += psum;
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
                 float pv[8];
@@ -393,20 +398,22 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const float4 l4 = *reinterpret_cast<const float4*>(lse_s + 32 * qt + 8 * g + 4 * lh);
-                const float4 d4 = *reinterpret_cast<const float4*>(delta_s + 32 * qt + 8 * g + 4 * lh);
                 const float lq4[4] = {l4.x * kLog2e, l4.y * kLog2e, l4.z * kLog2e, l4.w * kLog2e};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    pv[4 * g + e] = __builtin_amdgcn_exp2f(fmaf(sacc[4 * g + e], c, -lq4[e]));
+            }
+            if (diag) {  // wave-uniform: only blocks on the diagonal pay for the mask
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (kvi > qt0 + 8 * (v >> 2) + 4 * lh + (v & 3)) pv[v] = 0.f;
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 d4 = *reinterpret_cast<const float4*>(delta_s + 32 * qt + 8 * g + 4 * lh);
                 const float dq4[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = 4 * g + e;
-                    float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lq4[e]));
-                    if (diag) {
-                        const int64_t qrow = qt0 + 8 * g + 4 * lh + e;
-                        if (kvi > qrow) p = 0.f;
-                    }
-                    pv[v] = p;
-                    dsv[v] = p * (dpacc[v] - dq4[e]);
-                }
+                for (int e = 0; e < 4; ++e) dsv[4 * g + e] = pv[4 * g + e] * (dpacc[4 * g + e] - dq4[e]);
             }
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
@@ -541,14 +548,14 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
             const bool diag = CAUSAL && (kt0 + 31 > qw0);
             float dsv[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float p = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lse_q));
-                if (diag) {
-                    const int64_t kv = kt0 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                    if (kv > qi) p = 0.f;
-                }
-                dsv[v] = p * (dpacc[v] - delta_q);
+            for (int v = 0; v < 16; ++v) dsv[v] = __builtin_amdgcn_exp2f(fmaf(sacc[v], c, -lse_q));
+            if (diag) {  // wave-uniform: only blocks on the diagonal pay for the mask
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (kt0 + 8 * (v >> 2) + 4 * lh + (v & 3) > qi) dsv[v] = 0.f;
             }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dsv[v] *= dpacc[v] - delta_q;
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
                 const bf16x8_t dsb = pack8(dsv + 8 * gp);
