@@ -219,6 +219,19 @@ def main():
         mbytes = 2.0 * merged.numel() * merged.element_size()
         hbm["merge"] = {"achieved": round(mbytes / (mms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(mbytes / (mms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(mms, 3)}
+        # the optimizer step that follows schedule.step() in training: timed alone, outside `value`
+        import pippy_amd as pp
+        opt = pp.FusedAdamW(stages, lr=1e-4, weight_decay=0.1)
+        opt.step()
+        ev0.record()
+        for _ in range(5):
+            opt.step()
+        ev1.record()
+        torch.cuda.synchronize()
+        oms = ev0.elapsed_time(ev1) / 5
+        obytes = sum(a.total for a in (st.param_arena() for st in stages)) * 24.0  # g 4, m 8, v 8, bf16 p 4
+        hbm["adamw_step"] = {"achieved": round(obytes / (oms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(obytes / (oms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(oms, 3)}
         result["other_kernels"] = hbm
 
     if not args.no_cpu_baseline:

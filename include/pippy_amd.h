@@ -84,6 +84,26 @@ int pp_grad_accum_f32_f32(float* acc, const float* g, int64_t n, int init, pp_st
 int pp_fill_bytes(void* dst, int value, int64_t n_bytes, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Optimizer step on the fp32 accumulators: what the reference's users run right after
+ * schedule.step() (test/test_optim.py:83-99, `optim.SGD(stage.submod.parameters(), ...)`), here as
+ * one launch over a stage's flat parameter range.  `param` is bf16 or fp32 (enum pp_dtype), `grad`
+ * the fp32 accumulator, state buffers fp32, `master` an optional fp32 copy of bf16 parameters that
+ * takes the update (param becomes its rounding) or null.  n % 4 == 0; pointers aligned to 4
+ * elements.  Arithmetic follows torch.optim's single-tensor SGD / AdamW operation by operation.
+ *   SGD:   d = g + wd p;  buf = first_step ? d : momentum buf + (1 - dampening) d;
+ *          d = nesterov ? d + momentum buf : buf  (momentum != 0);  p -= lr d
+ *   AdamW: p *= 1 - lr wd;  m += (1 - beta1)(g - m);  v = beta2 v + (1 - beta2) g g;
+ *          p -= lr / bias_correction1 * m / (sqrt(v) / bias_correction2_sqrt + eps)
+ * ---------------------------------------------------------------------------------------- */
+int pp_sgd_step(void* param, int param_dtype, float* master, const float* grad, float* momentum_buf,
+                int64_t n, float lr, float momentum, float dampening, float weight_decay, int nesterov,
+                int first_step, int maximize, pp_stream stream);
+int pp_adamw_step(void* param, int param_dtype, float* master, const float* grad, float* exp_avg,
+                  float* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps,
+                  float weight_decay, float bias_correction1, float bias_correction2_sqrt, int maximize,
+                  pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
  * bf16 GEMM on MFMA with fp32 accumulation and fused epilogues.
  *   forward  F.linear inside the stage module      pippy/_PipelineStage.py:420-428
  *   backward dI / dW of the same linear            pippy/_backward.py:67-69

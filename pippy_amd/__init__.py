@@ -7,6 +7,7 @@ virtual stages on one GPU; see ``schedules.py``.
 from ._IR import (ArgsChunkSpec, KwargsChunkSpec, Pipe, PipeSplitWrapper, SplitPoint,
                   annotate_split_points, pipe_split, pipeline)
 from .losses import CrossEntropyLoss
+from .optim import FusedAdamW, FusedSGD
 from .microbatch import TensorChunkSpec, merge_chunks, split_args_kwargs_into_chunks, sum_reducer
 from .schedules import (Schedule1F1B, ScheduleGPipe, ScheduleInterleaved1F1B, ScheduleLoopedBFS,
                         ScheduleZeroBubble)
@@ -19,5 +20,5 @@ __all__ = [
     "KwargsChunkSpec", "TensorChunkSpec", "PipelineStage", "ManualPipelineStage", "Schedule1F1B",
     "ScheduleGPipe", "ScheduleInterleaved1F1B", "ScheduleLoopedBFS", "ScheduleZeroBubble",
     "split_args_kwargs_into_chunks", "merge_chunks", "sum_reducer", "CrossEntropyLoss",
-    "VirtualGroup", "PipeSplitWrapper",
+    "VirtualGroup", "PipeSplitWrapper", "FusedSGD", "FusedAdamW",
 ]

@@ -37,7 +37,7 @@ EXPORTED_SYMBOLS = (
     "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
-    "pp_profile_read",
+    "pp_profile_read", "pp_sgd_step", "pp_adamw_step",
 )
 
 
@@ -125,6 +125,8 @@ def lib() -> C.CDLL:
         "pp_profile_start": [i32],
         "pp_profile_stop": [],
         "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
+        "pp_sgd_step": [vp, i32, vp, vp, vp, i64, f32, f32, f32, f32, i32, i32, i32, vp],
+        "pp_adamw_step": [vp, i32, vp, vp, vp, vp, i64, f32, f32, f32, f32, f32, f32, f32, i32, vp],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -224,6 +226,44 @@ def grad_accum(acc: torch.Tensor, g: torch.Tensor, init: bool = False) -> None:
                                           current_stream()), "pp_grad_accum_f32_f32")
     else:
         raise TypeError(f"grad_accum: unsupported gradient dtype {g.dtype}")
+
+
+# ---- optimizer step ---------------------------------------------------------------------------
+def _pp_dtype(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return 0
+    if t.dtype == torch.float32:
+        return 1
+    raise TypeError(f"unsupported parameter dtype {t.dtype}")
+
+
+def sgd_step(param, grad, buf, *, master=None, lr, momentum=0.0, dampening=0.0, weight_decay=0.0,
+             nesterov=False, first_step=False, maximize=False) -> None:
+    """Flat tensors: ``param`` bf16/fp32, ``grad`` / ``buf`` / ``master`` fp32 of the same length."""
+    require_cuda(param, grad)
+    assert grad.dtype == torch.float32 and param.is_contiguous() and grad.is_contiguous()
+    assert grad.numel() == param.numel()
+    for t in (buf, master):
+        assert t is None or (t.dtype == torch.float32 and t.numel() == param.numel() and t.is_contiguous())
+    check(lib().pp_sgd_step(param.data_ptr(), _pp_dtype(param), _p_or_none(master), grad.data_ptr(),
+                            _p_or_none(buf), param.numel(), lr, momentum, dampening, weight_decay,
+                            int(nesterov), int(first_step), int(maximize), current_stream()), "pp_sgd_step")
+
+
+def adamw_step(param, grad, exp_avg, exp_avg_sq, *, master=None, lr, beta1, beta2, eps, weight_decay,
+               bias_correction1, bias_correction2_sqrt, maximize=False) -> None:
+    require_cuda(param, grad, exp_avg, exp_avg_sq)
+    assert grad.dtype == torch.float32 and param.is_contiguous() and grad.is_contiguous()
+    for t in (grad, exp_avg, exp_avg_sq, master):
+        assert t is None or (t.dtype == torch.float32 and t.numel() == param.numel() and t.is_contiguous())
+    check(lib().pp_adamw_step(param.data_ptr(), _pp_dtype(param), _p_or_none(master), grad.data_ptr(),
+                              exp_avg.data_ptr(), exp_avg_sq.data_ptr(), param.numel(), lr, beta1, beta2, eps,
+                              weight_decay, bias_correction1, bias_correction2_sqrt, int(maximize),
+                              current_stream()), "pp_adamw_step")
+
+
+def _p_or_none(t):
+    return None if t is None else t.data_ptr()
 
 
 def fill_bytes(t: torch.Tensor, value: int = 0) -> None:

@@ -91,6 +91,7 @@ class ParamArena:
         # transposed copies of linear weights ([in, out]) for the input-gradient GEMMs
         self._transposed: Dict[int, Tuple[nn.Parameter, torch.Tensor]] = {}
         self._versions = None
+        self._epoch = 0  # bumped by updates that write the arena directly (fused optimizers)
 
     def weight_t(self, p: nn.Parameter) -> torch.Tensor:
         """[in, out_padded] copy of a 2-d weight, kept in step with the parameter by
@@ -109,12 +110,16 @@ class ParamArena:
         step bumps the parameter's version counter)."""
         if not self._transposed:
             return
-        versions = tuple(p._version for p, _ in self._transposed.values())
+        versions = (self._epoch,) + tuple(p._version for p, _ in self._transposed.values())
         if versions == self._versions:
             return
         self._versions = versions
         for p, t in self._transposed.values():
             N.transpose_bf16(self.weight(p, padded=True), t)
+
+    def mark_updated(self) -> None:
+        """The parameter arena was written behind the parameters' version counters."""
+        self._epoch += 1
 
     def _slice(self, flat: torch.Tensor, p: nn.Parameter, padded: bool) -> torch.Tensor:
         o, numel, shape = self.entries[id(p)]

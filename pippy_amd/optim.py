@@ -1,0 +1,120 @@
+"""Optimizer step on the fp32 gradient accumulators of natively lowered stages.
+
+The reference's users build a ``torch.optim`` optimizer over ``stage.submod.parameters()`` and call
+``optimizer.step()`` after ``schedule.step()`` (reference ``test/test_optim.py:83-99``).  A lowered
+stage keeps its parameters, and the fp32 sums of their microbatch gradients, in flat arenas, so the
+same update is one HIP launch per stage: ``FusedSGD`` and ``FusedAdamW`` follow ``torch.optim.SGD``
+and ``torch.optim.AdamW`` (same hyper-parameters, same arithmetic operation by operation), read the
+fp32 accumulators instead of ``param.grad`` and keep their state in fp32.
+
+    opt = FusedAdamW(stages, lr=3e-4, weight_decay=0.1)
+    for batch, target in data:
+        opt.zero_grad()
+        schedule.step(batch, target=target, losses=losses)
+        opt.step()
+"""
+from __future__ import annotations
+
+import math
+from typing import Iterable, List, Optional
+
+import torch
+
+from . import _native as N
+
+
+class _FusedOptimizer:
+    def __init__(self, stages, master_weights: bool):
+        stages = list(stages) if isinstance(stages, (list, tuple)) else [stages]
+        if not stages:
+            raise ValueError("optimizer got no stages")
+        self._stages = stages
+        self._arenas = []
+        for st in stages:
+            if not getattr(st, "is_native", False):
+                raise RuntimeError(
+                    f"stage {getattr(st, 'stage_index', '?')} is not lowered to HIP launch lists; use a "
+                    "torch.optim optimizer on stage.submod.parameters() after stage.materialize_grads()")
+            self._arenas.append(st.param_arena())
+        self._master: List[Optional[torch.Tensor]] = []
+        for a in self._arenas:
+            if master_weights and a.dtype == torch.bfloat16:
+                self._master.append(a.params.to(torch.float32))
+            else:
+                self._master.append(None)
+        self._steps = 0
+
+    def zero_grad(self, set_to_none: bool = True):
+        """Clears the accumulated gradients of every stage (the next weight-gradient pass starts
+        the sums afresh)."""
+        for st in self._stages:
+            st.zero_grad()
+
+    def _after_update(self):
+        for a in self._arenas:
+            a.mark_updated()
+
+    @property
+    def master_weights(self) -> List[Optional[torch.Tensor]]:
+        return self._master
+
+
+class FusedSGD(_FusedOptimizer):
+    """``torch.optim.SGD`` over the arenas of lowered stages."""
+
+    def __init__(self, stages, lr: float, momentum: float = 0.0, dampening: float = 0.0,
+                 weight_decay: float = 0.0, nesterov: bool = False, *, maximize: bool = False,
+                 master_weights: bool = False):
+        if lr < 0.0:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if momentum < 0.0:
+            raise ValueError(f"Invalid momentum value: {momentum}")
+        if weight_decay < 0.0:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        if nesterov and (momentum <= 0 or dampening != 0):
+            raise ValueError("Nesterov momentum requires a momentum and zero dampening")
+        super().__init__(stages, master_weights)
+        self.lr, self.momentum, self.dampening = lr, momentum, dampening
+        self.weight_decay, self.nesterov, self.maximize = weight_decay, nesterov, maximize
+        self._buf = [torch.zeros_like(a.acc) if momentum != 0 else None for a in self._arenas]
+
+    @torch.no_grad()
+    def step(self):
+        for a, buf, master in zip(self._arenas, self._buf, self._master):
+            N.sgd_step(a.params, a.acc, buf, master=master, lr=self.lr, momentum=self.momentum,
+                       dampening=self.dampening, weight_decay=self.weight_decay, nesterov=self.nesterov,
+                       first_step=self._steps == 0, maximize=self.maximize)
+        self._steps += 1
+        self._after_update()
+
+
+class FusedAdamW(_FusedOptimizer):
+    """``torch.optim.AdamW`` (no amsgrad) over the arenas of lowered stages."""
+
+    def __init__(self, stages, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
+                 weight_decay: float = 1e-2, *, maximize: bool = False, master_weights: bool = False):
+        if lr < 0.0:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if eps < 0.0:
+            raise ValueError(f"Invalid epsilon value: {eps}")
+        if not 0.0 <= betas[0] < 1.0 or not 0.0 <= betas[1] < 1.0:
+            raise ValueError(f"Invalid betas: {betas}")
+        if weight_decay < 0.0:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        super().__init__(stages, master_weights)
+        self.lr, self.betas, self.eps = lr, tuple(betas), eps
+        self.weight_decay, self.maximize = weight_decay, maximize
+        self._m = [torch.zeros_like(a.acc) for a in self._arenas]
+        self._v = [torch.zeros_like(a.acc) for a in self._arenas]
+
+    @torch.no_grad()
+    def step(self):
+        self._steps += 1
+        b1, b2 = self.betas
+        bc1 = 1.0 - b1 ** self._steps
+        bc2_sqrt = math.sqrt(1.0 - b2 ** self._steps)
+        for a, m, v, master in zip(self._arenas, self._m, self._v, self._master):
+            N.adamw_step(a.params, a.acc, m, v, master=master, lr=self.lr, beta1=b1, beta2=b2, eps=self.eps,
+                         weight_decay=self.weight_decay, bias_correction1=bc1, bias_correction2_sqrt=bc2_sqrt,
+                         maximize=self.maximize)
+        self._after_update()

@@ -176,6 +176,13 @@ class PipelineStageBase:
             self._program.mbs.clear()
         return self._program
 
+    def param_arena(self) -> "P.ParamArena":
+        """The flat parameter / fp32-accumulator storage of a natively lowered stage (what the fused
+        optimizers step on)."""
+        if not self.is_native:
+            raise RuntimeError(f"{self.log_prefix} is not lowered to launch lists and has no arena")
+        return self._stage_program().arena
+
     def _publish_grad_views(self):
         """fp32 parameters get their accumulator as ``.grad``; bf16 parameters expose it as
         ``.main_grad`` (torch does not allow an fp32 ``.grad`` on a bf16 parameter)."""

@@ -448,3 +448,100 @@ def test_activation_bwd(dtype, tol, act):
     fn = {"relu": torch.relu, "gelu_erf": O.gelu_erf, "gelu_tanh": O.gelu_tanh}[act]
     fn(a).backward(dy.float().cpu())
     assert_close_rel(dz, a.grad, tol, f"activation bwd {act}")
+
+
+# ---- optimizer step on the fp32 accumulators -----------------------------------------------------
+from oracle import optim as OO
+import numpy as np
+
+
+def _bf16_ulp_diff(a: torch.Tensor, b: torch.Tensor) -> int:
+    ia = a.view(torch.int16).to(torch.int32)
+    ib = b.view(torch.int16).to(torch.int32)
+    return int((ia - ib).abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("momentum,dampening,wd,nesterov", [(0.0, 0.0, 0.0, False), (0.9, 0.0, 0.01, False),
+                                                            (0.9, 0.0, 0.0, True), (0.8, 0.2, 0.1, False)])
+@pytest.mark.parametrize("master", [False, True])
+def test_sgd_step_matches_oracle(dtype, momentum, dampening, wd, nesterov, master):
+    if master and dtype != torch.bfloat16:
+        pytest.skip("a master copy goes with bf16 parameters")
+    N = native()
+    n = 4 * 1000 + 4
+    g0 = torch.Generator().manual_seed(11)
+    p_host = torch.randn(n, generator=g0).to(dtype)
+    p = p_host.cuda()
+    mst = p.float() if master else None
+    buf = torch.zeros(n, device="cuda") if momentum else None
+    p_o = p_host.float().numpy().copy()
+    buf_o = None
+    for step in range(3):
+        grad = torch.randn(n, generator=g0)
+        N.sgd_step(p, grad.cuda(), buf, master=mst, lr=0.05, momentum=momentum, dampening=dampening,
+                   weight_decay=wd, nesterov=nesterov, first_step=step == 0)
+        p_o, buf_o = OO.sgd_step(p_o, grad.numpy(), buf_o, lr=0.05, momentum=momentum, dampening=dampening,
+                                 weight_decay=wd, nesterov=nesterov, first_step=step == 0)
+        if dtype == torch.float32:
+            assert_close_rel(p.cpu(), torch.from_numpy(p_o), 2e-6, "sgd fp32 parameters")
+        elif master:
+            assert_close_rel(mst.cpu(), torch.from_numpy(p_o), 2e-6, "sgd master copy")
+            assert _bf16_ulp_diff(p.cpu(), torch.from_numpy(OO.round_bf16(p_o)).to(torch.bfloat16)) <= 1
+        else:
+            # the parameter is re-rounded to bf16 every step; the oracle does the same
+            p_o = OO.round_bf16(p_o)
+            assert _bf16_ulp_diff(p.cpu(), torch.from_numpy(p_o).to(torch.bfloat16)) <= 1
+            p_o = p.cpu().float().numpy().copy()  # continue from the device value so 1-ulp ties do not compound
+        if momentum:
+            assert_close_rel(buf.cpu(), torch.from_numpy(buf_o), 2e-6, "sgd momentum buffer")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,master", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("wd", [0.0, 0.1])
+def test_adamw_step_matches_oracle(dtype, master, wd):
+    N = native()
+    n = 4 * 777
+    g0 = torch.Generator().manual_seed(13)
+    p_host = torch.randn(n, generator=g0).to(dtype)
+    p = p_host.cuda()
+    mst = p.float() if master else None
+    m = torch.zeros(n, device="cuda")
+    v = torch.zeros(n, device="cuda")
+    p_o = p_host.float().numpy().copy()
+    m_o = np.zeros(n, np.float32)
+    v_o = np.zeros(n, np.float32)
+    lr, b1, b2, eps = 1e-2, 0.9, 0.95, 1e-8
+    for step in range(1, 4):
+        grad = torch.randn(n, generator=g0)
+        N.adamw_step(p, grad.cuda(), m, v, master=mst, lr=lr, beta1=b1, beta2=b2, eps=eps, weight_decay=wd,
+                     bias_correction1=1 - b1 ** step, bias_correction2_sqrt=math.sqrt(1 - b2 ** step))
+        p_o, m_o, v_o = OO.adamw_step(p_o, grad.numpy(), m_o, v_o, lr=lr, beta1=b1, beta2=b2, eps=eps,
+                                      weight_decay=wd, step=step)
+        assert_close_rel(m.cpu(), torch.from_numpy(m_o), 2e-6, "adamw exp_avg")
+        assert_close_rel(v.cpu(), torch.from_numpy(v_o), 2e-6, "adamw exp_avg_sq")
+        if dtype == torch.float32:
+            assert_close_rel(p.cpu(), torch.from_numpy(p_o), 3e-6, "adamw fp32 parameters")
+        elif master:
+            assert_close_rel(mst.cpu(), torch.from_numpy(p_o), 3e-6, "adamw master copy")
+            assert _bf16_ulp_diff(p.cpu(), torch.from_numpy(OO.round_bf16(p_o)).to(torch.bfloat16)) <= 1
+        else:
+            assert _bf16_ulp_diff(p.cpu(), torch.from_numpy(OO.round_bf16(p_o)).to(torch.bfloat16)) <= 1
+            p_o = p.cpu().float().numpy().copy()
+
+
+@pytest.mark.gpu
+def test_optimizer_steps_reject_bad_arguments():
+    N = native()
+    p = torch.zeros(6, device="cuda")
+    g = torch.zeros(6, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        N.sgd_step(p, g, None, lr=0.1)
+    p = torch.zeros(8, device="cuda")
+    g = torch.zeros(8, device="cuda")
+    with pytest.raises(RuntimeError, match="momentum needs"):
+        N.sgd_step(p, g, None, lr=0.1, momentum=0.9)
+    with pytest.raises(RuntimeError, match="master copy goes with bf16"):
+        N.sgd_step(p, g, None, master=torch.zeros(8, device="cuda"), lr=0.1)

@@ -204,3 +204,53 @@ def test_single_rank_interleaved_order():
     assert prog[-1] == ("B", 0, 7) and len(prog) == 32
     kinds = "".join(k for k, _, _ in prog)
     assert kinds == "F" + "FB" * 15 + "B"
+
+
+# ---- optimizer updates: pinned against torch.optim itself (CPU fp32) ----------------------------
+from oracle import optim as OO
+
+
+@pytest.mark.parametrize("momentum,dampening,wd,nesterov,maximize", [
+    (0.0, 0.0, 0.0, False, False), (0.9, 0.0, 0.0, False, False), (0.9, 0.1, 0.01, False, False),
+    (0.9, 0.0, 0.05, True, False), (0.5, 0.0, 0.0, False, True)])
+def test_sgd_oracle_matches_torch_optim(momentum, dampening, wd, nesterov, maximize):
+    g = torch.Generator().manual_seed(3)
+    p = nn.Parameter(torch.randn(257, generator=g))
+    opt = torch.optim.SGD([p], lr=0.05, momentum=momentum, dampening=dampening, weight_decay=wd,
+                          nesterov=nesterov, maximize=maximize)
+    p_o, buf = p.detach().numpy().copy(), None
+    for step in range(3):
+        grad = torch.randn(257, generator=g)
+        p.grad = grad.clone()
+        opt.step()
+        p_o, buf = OO.sgd_step(p_o, grad.numpy(), buf, lr=0.05, momentum=momentum, dampening=dampening,
+                               weight_decay=wd, nesterov=nesterov, first_step=step == 0, maximize=maximize)
+        np.testing.assert_allclose(p_o, p.detach().numpy(), rtol=2e-6, atol=1e-7)
+    # closed form without momentum: p_T = p_0 - lr * sum(g)
+    assert OO.sgd_step(np.ones(4, np.float32), np.full(4, 2.0, np.float32), None, lr=0.25)[0].tolist() == [0.5] * 4
+
+
+@pytest.mark.parametrize("wd,maximize", [(0.0, False), (0.1, False), (0.01, True)])
+def test_adamw_oracle_matches_torch_optim(wd, maximize):
+    g = torch.Generator().manual_seed(5)
+    p = nn.Parameter(torch.randn(300, generator=g))
+    opt = torch.optim.AdamW([p], lr=1e-2, betas=(0.9, 0.95), eps=1e-8, weight_decay=wd, maximize=maximize)
+    p_o = p.detach().numpy().copy()
+    m = np.zeros(300, np.float32)
+    v = np.zeros(300, np.float32)
+    for step in range(1, 5):
+        grad = torch.randn(300, generator=g)
+        p.grad = grad.clone()
+        opt.step()
+        p_o, m, v = OO.adamw_step(p_o, grad.numpy(), m, v, lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8,
+                                  weight_decay=wd, step=step, maximize=maximize)
+        np.testing.assert_allclose(p_o, p.detach().numpy(), rtol=3e-6, atol=1e-7)
+    # first step of Adam moves every coordinate by lr * sign(g) (up to eps), whatever |g| is
+    q, _, _ = OO.adamw_step(np.zeros(3, np.float32), np.array([1e-3, -5.0, 40.0], np.float32), np.zeros(3, np.float32),
+                            np.zeros(3, np.float32), lr=0.1, beta1=0.9, beta2=0.999, eps=1e-12, weight_decay=0.0, step=1)
+    np.testing.assert_allclose(q, [-0.1, 0.1, -0.1], rtol=1e-5)
+
+
+def test_round_bf16_matches_torch():
+    x = torch.randn(1000, generator=torch.Generator().manual_seed(0)) * 7
+    np.testing.assert_array_equal(OO.round_bf16(x.numpy()), x.to(torch.bfloat16).float().numpy())

@@ -234,3 +234,56 @@ def test_readme_mlp_fp32_matches_oracle():
     for name, rp in ref.named_parameters():
         assert_close_rel(named[name].grad, rp.grad, F32_TOL, f"mlp grad {name}")
         assert named[name].grad.data_ptr() == named[name].main_grad.data_ptr()
+
+
+def test_fused_optimizer_trains_like_the_oracle():
+    """schedule.step() + optimizer.step() twice (reference test_optim.py:83-99): parameter updates,
+    the momentum-carrying second update and the losses of the second step (which run on the updated
+    weights and their refreshed transposed copies) against the oracle pipeline stepped with the
+    oracle's SGD."""
+    import pippy_amd as pp
+    from oracle import optim as OO
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    torch.manual_seed(7)
+    target = torch.randint(0, model.head.vocab, ids.shape)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    lr, mom = 1.0, 0.9
+    opt = pp.FusedSGD(stages, lr=lr, momentum=mom, master_weights=True)
+    named = dict(model.named_parameters())
+    ref_named = dict(ref.named_parameters())
+    arenas = [st.param_arena() for st in stages]
+
+    def master_of(name):
+        """fp32 master copy of one parameter (a slice of its stage's flat master array)."""
+        k = next(i for i, a in enumerate(arenas) if id(named[name]) in a.entries)
+        return arenas[k]._slice(opt.master_weights[k], named[name], padded=False).detach().cpu().clone()
+
+    bufs = {}
+    prev = {n: master_of(n) for n in named}
+    for step in range(2):
+        opt.zero_grad()
+        losses = []
+        sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+        opt.step()
+        torch.cuda.synchronize()
+        for p in ref.parameters():
+            p.grad = None
+        _, ref_losses = OP.step(ref_stages, ids, target, M, _ce)
+        for m in range(M):
+            assert_close_rel(losses[m].reshape(1), ref_losses[m].reshape(1), BF16_TOL, f"step {step} loss {m}")
+        worst = 0.0
+        for name, rp in ref_named.items():
+            new, bufs[name] = OO.sgd_step(rp.detach().numpy(), rp.grad.numpy(), bufs.get(name), lr=lr,
+                                          momentum=mom, first_step=step == 0)
+            ref_update = torch.from_numpy(new) - rp.detach()
+            with torch.no_grad():
+                rp.copy_(torch.from_numpy(new))
+            cur = master_of(name)
+            err = max_rel(cur - prev[name], ref_update)
+            worst = max(worst, err)
+            assert err <= BF16_TOL, f"step {step} update of {name}: max relative error {err:.3e}"
+            # the bf16 parameter is the rounding of its master copy
+            assert torch.equal(named[name].detach().cpu(), cur.to(torch.bfloat16))
+            prev[name] = cur
+        note(f"optimizer step {step}: worst update error {worst:.3e}")
