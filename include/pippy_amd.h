@@ -233,10 +233,12 @@ int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
  * Token + position embedding (F.embedding inside the first stage).
- * y[t, :] = wte[ids[t], :] + (wpe ? wpe[t % seq, :] : 0);  ids int64 [n_tok]; bf16 tables.
+ * y[t, :] = wte[ids[t], :] + (wpe ? wpe[t % seq, :] : 0) + (extra_row ? extra_row[:] : 0), summed in
+ * fp32 and rounded once;  ids int64 [n_tok]; bf16 tables; extra_row is one bf16 row [C] added to
+ * every token (the token-type-0 row of a BERT embedding) or null.
  * ---------------------------------------------------------------------------------------- */
-int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, void* y, int64_t n_tok,
-                 int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
+int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, const void* extra_row, void* y,
+                 int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
 /* d_wte (fp32 [vocab, C]) += scatter(dy) with atomics; d_wpe (fp32 [seq, C]) += sum over batch */
 int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe, int64_t n_tok,
                  int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
@@ -273,7 +275,7 @@ enum pp_op_kind {
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
  *                 | j: causal
- *   EMBED_FWD     p: ids wte wpe y | i: n_tok seq C vocab
+ *   EMBED_FWD     p: ids wte wpe y extra_row | i: n_tok seq C vocab
  *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype
  *   ACCUM_*       p: acc g | i: n | j: init

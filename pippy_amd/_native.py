@@ -116,7 +116,7 @@ def lib() -> C.CDLL:
         "pp_layernorm_bwd_weight": [vp, vp, vp, vp, vp, vp, i32, vp, i64, i64, vp],
         "pp_attn_fwd": [C.POINTER(AttnDesc), vp],
         "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
-        "pp_embed_fwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
+        "pp_embed_fwd": [vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
@@ -425,12 +425,13 @@ def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None) -> None:
 
 
 # ---- embedding / loss -------------------------------------------------------------------------
-def embed_fwd(ids, wte, wpe, y, seq: int) -> None:
+def embed_fwd(ids, wte, wpe, y, seq: int, extra_row=None) -> None:
     require_cuda(ids, wte, wpe, y)
     assert ids.dtype == torch.int64 and ids.is_contiguous() and y.is_contiguous()
     vocab, Cc = wte.shape
-    check(lib().pp_embed_fwd(ids.data_ptr(), wte.data_ptr(), ptr(wpe), y.data_ptr(), ids.numel(),
-                             seq, Cc, vocab, current_stream()), "pp_embed_fwd")
+    assert extra_row is None or (extra_row.numel() == Cc and extra_row.is_contiguous())
+    check(lib().pp_embed_fwd(ids.data_ptr(), wte.data_ptr(), ptr(wpe), ptr(extra_row), y.data_ptr(),
+                             ids.numel(), seq, Cc, vocab, current_stream()), "pp_embed_fwd")
 
 
 def embed_bwd(ids, dy, d_wte, d_wpe, seq: int) -> None:

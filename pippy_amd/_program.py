@@ -232,12 +232,14 @@ def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None) -> N.
     return op
 
 
-def op_embed_fwd(ids, wte, wpe, y, seq) -> N.Op:
+def op_embed_fwd(ids, wte, wpe, y, seq, extra_row=None) -> N.Op:
     vocab, Cc = wte.shape
     assert ids.dtype == torch.int64 and y.shape == (ids.numel(), Cc) and y.is_contiguous()
+    assert extra_row is None or (extra_row.numel() == Cc and extra_row.is_contiguous())
     op = N.Op()
     op.kind = N.OP_EMBED_FWD
     op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), wte.data_ptr(), _p(wpe), y.data_ptr()
+    op.p[4] = _p(extra_row)
     op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
     return op
 

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .stage_modules import LMHead, TokenEmbedding, TransformerLayer
+from .stage_modules import EncoderEmbedding, LMHead, TokenEmbedding, TransformerLayer
 
 
 class DecoderLM(nn.Module):
@@ -36,6 +36,30 @@ class DecoderLM(nn.Module):
 def gpt2_small(dtype=torch.bfloat16) -> DecoderLM:
     """12 layers, width 768, 12 heads, FFN 3072, vocabulary 50257, sequence 1024."""
     return DecoderLM(dtype=dtype)
+
+
+class EncoderModel(nn.Module):
+    """BERT-shaped encoder: word + position + token-type embedding with LayerNorm, post-LayerNorm
+    bidirectional transformer layers with erf-GELU; returns the last hidden state."""
+
+    def __init__(self, vocab=30522, max_seq=512, dim=768, n_layers=12, n_heads=12, ffn=3072,
+                 dtype=torch.bfloat16, eps=1e-12):
+        super().__init__()
+        self.embed = EncoderEmbedding(vocab, max_seq, dim, eps=eps, dtype=dtype)
+        self.h = nn.ModuleList([
+            TransformerLayer(dim, n_heads, ffn, causal=False, pre_ln=False, activation="gelu_erf",
+                             eps=eps, dtype=dtype) for _ in range(n_layers)])
+
+    def forward(self, ids):
+        x = self.embed(ids)
+        for layer in self.h:
+            x = layer(x)
+        return x
+
+
+def bert_base(dtype=torch.bfloat16) -> EncoderModel:
+    """12 layers, hidden 768, 12 heads, FFN 3072, vocabulary 30522, sequence 512."""
+    return EncoderModel(dtype=dtype)
 
 
 def equal_split_spec(n_layers: int, n_stages: int, prefix: str = "h"):

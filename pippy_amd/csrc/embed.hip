@@ -7,6 +7,7 @@ namespace pp {
 __global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restrict__ ids,
                                                         const uint16_t* __restrict__ wte,
                                                         const uint16_t* __restrict__ wpe,
+                                                        const uint16_t* __restrict__ extra_row,
                                                         uint16_t* __restrict__ y, int64_t n_tok,
                                                         int64_t seq, int C, int64_t vocab) {
     const int lane = threadIdx.x & 63;
@@ -17,15 +18,25 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restric
     if (id < 0 || id >= vocab) id = 0;
     const uint4* src = reinterpret_cast<const uint4*>(wte + id * C);
     const uint4* pos = wpe ? reinterpret_cast<const uint4*>(wpe + (t % seq) * C) : nullptr;
+    const uint4* ext = reinterpret_cast<const uint4*>(extra_row);
     uint4* dst = reinterpret_cast<uint4*>(y + t * C);
     for (int c = lane; c < (C >> 3); c += 64) {
         uint4 a = src[c];
-        if (pos) {
-            const uint4 b = pos[c];
-            a.x = pack_bf16(bf16lo(a.x) + bf16lo(b.x), bf16hi(a.x) + bf16hi(b.x));
-            a.y = pack_bf16(bf16lo(a.y) + bf16lo(b.y), bf16hi(a.y) + bf16hi(b.y));
-            a.z = pack_bf16(bf16lo(a.z) + bf16lo(b.z), bf16hi(a.z) + bf16hi(b.z));
-            a.w = pack_bf16(bf16lo(a.w) + bf16lo(b.w), bf16hi(a.w) + bf16hi(b.w));
+        if (pos || ext) {
+            // the sum is formed in fp32 and rounded once
+            float f[8] = {bf16lo(a.x), bf16hi(a.x), bf16lo(a.y), bf16hi(a.y),
+                          bf16lo(a.z), bf16hi(a.z), bf16lo(a.w), bf16hi(a.w)};
+            if (pos) {
+                const uint4 b = pos[c];
+                f[0] += bf16lo(b.x); f[1] += bf16hi(b.x); f[2] += bf16lo(b.y); f[3] += bf16hi(b.y);
+                f[4] += bf16lo(b.z); f[5] += bf16hi(b.z); f[6] += bf16lo(b.w); f[7] += bf16hi(b.w);
+            }
+            if (ext) {
+                const uint4 b = ext[c];
+                f[0] += bf16lo(b.x); f[1] += bf16hi(b.x); f[2] += bf16lo(b.y); f[3] += bf16hi(b.y);
+                f[4] += bf16lo(b.z); f[5] += bf16hi(b.z); f[6] += bf16lo(b.w); f[7] += bf16hi(b.w);
+            }
+            a = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
         }
         dst[c] = a;
     }
@@ -74,17 +85,17 @@ __global__ __launch_bounds__(256) void embed_bwd_wpe_kernel(const uint16_t* __re
 
 using namespace pp;
 
-extern "C" int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, void* y,
-                            int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream) {
+extern "C" int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, const void* extra_row,
+                            void* y, int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream) {
     if (n_tok < 0 || seq <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_fwd: bad shape");
     if (C % 8) return fail(PP_ERR_UNSUPPORTED, "pp_embed_fwd: C %% 8 != 0");
     if (n_tok == 0) return PP_OK;
     if (!ids || !wte || !y) return fail(PP_ERR_INVALID, "pp_embed_fwd: null pointer");
-    if (!aligned(wte, 16) || !aligned(wpe, 16) || !aligned(y, 16))
+    if (!aligned(wte, 16) || !aligned(wpe, 16) || !aligned(extra_row, 16) || !aligned(y, 16))
         return fail(PP_ERR_INVALID, "pp_embed_fwd: pointers must be 16-byte aligned");
     hipLaunchKernelGGL(embed_fwd_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), ids, (const uint16_t*)wte, (const uint16_t*)wpe,
-                       (uint16_t*)y, n_tok, seq, (int)C, vocab);
+                       (const uint16_t*)extra_row, (uint16_t*)y, n_tok, seq, (int)C, vocab);
     return check_launch("embed_fwd_kernel");
 }
 

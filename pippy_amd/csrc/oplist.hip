@@ -95,7 +95,7 @@ static int run_one(const pp_op& op, pp_stream st) {
             return op.kind == PP_OP_ATTN_FWD ? pp_attn_fwd(&d, st) : pp_attn_bwd(&d, st);
         }
         case PP_OP_EMBED_FWD:
-            return pp_embed_fwd(static_cast<const int64_t*>(op.p[0]), op.p[1], op.p[2], op.p[3], op.i[0],
+            return pp_embed_fwd(static_cast<const int64_t*>(op.p[0]), op.p[1], op.p[2], op.p[4], op.p[3], op.i[0],
                                 op.i[1], op.i[2], op.i[3], st);
         case PP_OP_EMBED_BWD:
             return pp_embed_bwd(static_cast<const int64_t*>(op.p[0]), op.p[1], static_cast<float*>(op.p[2]),

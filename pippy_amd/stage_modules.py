@@ -244,6 +244,68 @@ class TokenEmbedding(NativeBlock):
         return y
 
 
+class EncoderEmbedding(NativeBlock):
+    """BERT-style embedding: ``LayerNorm(word[ids] + position[:S] + token_type[0])``.  All tokens
+    are of type 0, which is what the encoder computes when no ``token_type_ids`` are passed."""
+
+    def __init__(self, vocab: int, max_seq: int, dim: int, n_types: int = 2, eps: float = 1e-12,
+                 dtype=torch.bfloat16, init_std=0.02):
+        super().__init__()
+        self.word_embeddings = nn.Embedding(vocab, dim, dtype=dtype)
+        self.position_embeddings = nn.Embedding(max_seq, dim, dtype=dtype)
+        self.token_type_embeddings = nn.Embedding(n_types, dim, dtype=dtype)
+        self.LayerNorm = nn.LayerNorm(dim, eps=eps, dtype=dtype)
+        for emb in (self.word_embeddings, self.position_embeddings, self.token_type_embeddings):
+            nn.init.normal_(emb.weight, std=init_std)
+
+    def forward(self, ids):
+        S = ids.shape[-1]
+        pos = torch.arange(S, device=ids.device)
+        # one rounding of the three-term sum, as the lowered kernel does
+        e = (self.word_embeddings(ids).float() + self.position_embeddings(pos).float()
+             + self.token_type_embeddings.weight[0].float()).to(self.word_embeddings.weight.dtype)
+        return self.LayerNorm(e)
+
+    def _pp_direct_acc_params(self):
+        return [self.word_embeddings.weight, self.position_embeddings.weight]
+
+    def lower(self, b, ids):
+        if ids.dtype != torch.int64 or ids.dim() != 2:
+            raise RuntimeError(f"EncoderEmbedding expects int64 ids of shape [batch, seq], got "
+                               f"{ids.dtype} {tuple(ids.shape)}")
+        Bn, S = ids.shape
+        wte, wpe = b.weight(self.word_embeddings.weight), b.weight(self.position_embeddings.weight)
+        wtt = b.weight(self.token_type_embeddings.weight)
+        if S > wpe.shape[0]:
+            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
+        Cc = wte.shape[1]
+        T = Bn * S
+        e = b.act("e", (T, Cc))
+        b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0]))
+        y, mean, rstd = lower_layernorm(b, "ln", self.LayerNorm, e)
+
+        def bwd(dy, need_dx, dx_out):
+            de = layernorm_backward(b, "ln", self.LayerNorm, e, mean, rstd, dy.view(T, Cc))
+            acc_wte = b.grad_acc(self.word_embeddings.weight)
+            acc_wpe = b.grad_acc(self.position_embeddings.weight)
+            b.w(P.op_fill(acc_wte), tag="fill")
+            b.w(P.op_fill(acc_wpe), tag="fill")
+            b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S))
+            # the type-0 row receives the gradient of every token; the other rows none
+            g_tt = b.grad_target(self.token_type_embeddings.weight)
+            ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)
+            if b.fused_accumulate:
+                tmp = b.workspace("colsum_out:tt", (Cc,), torch.float32)
+                b.w_reduce(P.op_colsum(de, tmp, ws))
+                b.w(P.op_accum(b.grad_acc(self.token_type_embeddings.weight)[0], tmp), tag="accum")
+            else:
+                b.w_reduce(P.op_colsum(de, g_tt[0], ws))
+            return None
+
+        b.on_backward(bwd)
+        return y.view(Bn, S, Cc)
+
+
 class TransformerLayer(NativeBlock):
     """One transformer layer: multi-head self-attention and a GELU feed-forward, pre-LayerNorm
     (GPT-2) or post-LayerNorm (BERT).  Parameter names follow GPT-2 (``ln_1``, ``attn.c_attn``,
@@ -326,21 +388,38 @@ class TransformerLayer(NativeBlock):
         return y.view(Bn, S, Cc)
 
     def _lower_post_ln(self, b, x):
-        if b.training:
-            raise NotImplementedError("post-LayerNorm transformer layers are lowered for inference only")
         Bn, S, Cc = x.shape
         T, H = Bn * S, self.n_heads
         x2d = x.view(T, Cc)
+        act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         qkv, _ = lower_linear(b, "qkv", self.attn.c_attn, x2d)
         att = b.act("att", (T, Cc))
         lse = b.act("lse", (Bn, H, S), torch.float32)
         b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
         a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
-        x1, _, _ = lower_layernorm(b, "ln1", self.ln_1, a)
-        h, _ = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=_ACT_EPI[self.activation])
+        x1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, a)
+        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act, save_pre=b.training)
         f, _ = lower_linear(b, "f", self.mlp.c_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x1)
-        y, _, _ = lower_layernorm(b, "ln2", self.ln_2, f)
-        b.on_backward(lambda dy, need_dx, dx_out: None)
+        y, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, f)
+
+        def bwd(dy, need_dx, dx_out):
+            # a sum of two gradients in front of a LayerNorm is formed by the residual epilogue
+            # (without a bias) of the input-gradient GEMM that produces one of them
+            d_f = layernorm_backward(b, "ln2", self.ln_2, f, mean2, rstd2, dy.view(T, Cc))
+            d_hpre = linear_backward(b, "c_proj", self.mlp.c_proj, h, d_f, dx_epilogue=dact, dx_aux=h_pre)
+            d_x1 = linear_backward(b, "c_fc", self.mlp.c_fc, x1, d_hpre, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+                                   dx_aux=d_f)
+            d_a = layernorm_backward(b, "ln1", self.ln_1, a, mean1, rstd1, d_x1)
+            d_att = linear_backward(b, "attn_proj", self.attn.c_proj, att, d_a)
+            dqkv = b.grad("dqkv", (T, 3 * Cc))
+            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
+            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            dx = linear_backward(b, "c_attn", self.attn.c_attn, x2d, dqkv, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+                                 dx_aux=d_a, dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            return dx.view(Bn, S, Cc)
+
+        b.on_backward(bwd)
         return y.view(Bn, S, Cc)
 
 

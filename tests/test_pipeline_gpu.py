@@ -287,3 +287,89 @@ def test_fused_optimizer_trains_like_the_oracle():
             assert torch.equal(named[name].detach().cpu(), cur.to(torch.bfloat16))
             prev[name] = cur
         note(f"optimizer step {step}: worst update error {worst:.3e}")
+
+
+# ---- BERT-shaped encoder (post-LayerNorm, bidirectional attention, erf-GELU) ----------------------
+def _build_encoder(n_stages, n_layers=4, M=4, vocab=1000, seq=128, dim=128, heads=2, ffn=512, seed=0):
+    import pippy_amd as pp
+    import torch.nn as nn
+    from pippy_amd.configs import EncoderModel, equal_split_spec
+    torch.manual_seed(seed)
+    model = EncoderModel(vocab=vocab, max_seq=seq, dim=dim, n_layers=n_layers, n_heads=heads, ffn=ffn)
+    # LayerNorm weights away from their (1, 0) initial values, so that their gradients are exercised
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, nn.LayerNorm):
+                m.weight.add_(0.1 * torch.randn_like(m.weight))
+                m.bias.add_(0.1 * torch.randn_like(m.bias))
+    ref = _fp32_cpu_copy(model)
+    ids = torch.randint(0, vocab, (2 * M, seq))
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(n_layers, n_stages))
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(n_stages)]
+    per = n_layers // n_stages
+    ref_stages = []
+    for s in range(n_stages):
+        mods = [ref.embed] if s == 0 else []
+        mods += [ref.h[i] for i in range(per * s, per * (s + 1))]
+        ref_stages.append(nn.Sequential(*mods))
+    return model, ref, stages, ref_stages, ids
+
+
+def test_encoder_inference_gpipe_matches_oracle():
+    """Config 2 at a reduced size: GPipe fill-drain forward of a post-LayerNorm encoder in 4 stages."""
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_encoder(4, M=M)
+    assert all(st.is_native for st in stages)
+    out = pp.ScheduleGPipe(stages, M).step(ids.to(DEV))
+    ref_out, _ = OP.step(ref_stages, ids, None, M, None)
+    assert out.shape == ref_out.shape == (2 * M, 128, 128)
+    assert_close_rel(out, ref_out, BF16_TOL, "encoder hidden states")
+
+
+def test_encoder_training_post_layernorm_matches_oracle():
+    """Post-LayerNorm layers and the three-table embedding through forward, dI and dW passes."""
+    import pippy_amd as pp
+    M = 2
+    model, ref, stages, ref_stages, ids = _build_encoder(2, n_layers=2, M=M)
+    torch.manual_seed(5)
+    target = torch.randn(2 * M, 128, 128)
+
+    def loss_fn(o, t):
+        return ((o.float() - t) ** 2).sum() * 1e-2
+
+    sched = pp.Schedule1F1B(stages, M, loss_fn=loss_fn)
+    losses = []
+    sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    for p in ref.parameters():
+        p.grad = None
+    _, ref_losses = OP.step(ref_stages, ids, target, M, loss_fn)
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.reshape(1), b.reshape(1), BF16_TOL, "loss")
+    named = dict(model.named_parameters())
+    worst = 0.0
+    for name, rp in ref.named_parameters():
+        err = max_rel(named[name].main_grad, rp.grad)
+        worst = max(worst, err)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+    note(f"post-LN encoder: worst grad error {worst:.3e}")
+
+
+def test_encoder_bert_base_full_size_layernorm_invariant():
+    """Config 2 at full size (12 layers, hidden 768, seq 512, batch 64 in 8 microbatches, 4 stages):
+    the last op of a post-LayerNorm encoder is a LayerNorm with weight 1 and bias 0 at
+    initialisation, so every output row has mean 0 and variance 1 whatever came before."""
+    import pippy_amd as pp
+    from pippy_amd.configs import bert_base, equal_split_spec
+    torch.manual_seed(0)
+    model = bert_base()
+    M = 8
+    ids = torch.randint(0, 30522, (64, 512))
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(12, 4))
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(4)]
+    out = pp.ScheduleGPipe(stages, M).step(ids.to(DEV))
+    assert out.shape == (64, 512, 768) and out.is_contiguous()
+    o = out.float()
+    assert torch.isfinite(o).all()
+    assert o.mean(-1).abs().max() < 2e-2
+    assert (o.var(-1, unbiased=False) - 1).abs().max() < 3e-2
