@@ -174,6 +174,22 @@ int pp_transpose_bf16(const void* src, int64_t rows, int64_t cols, int64_t ld_sr
 int pp_activation_bwd(const void* dy, const void* aux, void* dz, int64_t n, int act, int dtype,
                       pp_stream stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Element-wise pieces of a Llama-style layer (inside the stage module in the reference; backward
+ * through pippy/_backward.py:67-69).  bf16, n % 8 == 0, 16-byte aligned pointers.
+ *   SwiGLU:  h = silu(g) * u;   dg = dh * u * silu'(g),  du = dh * silu(g)
+ *   RoPE (rotate-half form, in place): for the first n_heads heads of width D of every row of
+ *   x [n_tok, ld]:  (x[i], x[i + D/2]) -> (x[i] c - x[i + D/2] s,  x[i + D/2] c + x[i] s)  with
+ *   c, s = cos_table / sin_table [seq, D/2] (fp32) at position t % seq;  inverse != 0 applies the
+ *   transposed rotation (the backward pass).  A fused [q | k | v] projection is rotated with
+ *   n_heads = q heads + k heads.
+ * ---------------------------------------------------------------------------------------- */
+int pp_swiglu_fwd(const void* g, const void* u, void* h, int64_t n, pp_stream stream);
+int pp_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int64_t n,
+                  pp_stream stream);
+int pp_rope(void* x, const float* cos_table, const float* sin_table, int64_t n_tok, int64_t seq,
+            int64_t n_heads, int64_t D, int64_t ld, int inverse, pp_stream stream);
+
 /* Column reductions of one weight-gradient pass in two launches.  Per descriptor:
  *   out_sum[c] = sum_r dy[r, c]                                   (bias gradient / dbeta), and, if
  *   out_dot is non-null, out_dot[c] = sum_r dy[r, c] * (x[r, c] - mean[r]) * rstd[r]   (dgamma).
@@ -197,6 +213,8 @@ int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_stream stream
 /* ------------------------------------------------------------------------------------------
  * LayerNorm (F.layer_norm inside the stage module; backward via pippy/_backward.py:67-69).
  * x, y, dy, dx: bf16 [rows, C]; gamma, beta: bf16 [C]; mean, rstd: fp32 [rows].
+ * A null `mean` selects RMSNorm in all three calls: nothing is subtracted, rstd = 1 / sqrt(mean(x^2)
+ * + eps), there is no beta and no dbeta.
  * ---------------------------------------------------------------------------------------- */
 int pp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
                      float* rstd, int64_t rows, int64_t C, float eps, pp_stream stream);
@@ -263,7 +281,8 @@ enum pp_op_kind {
     PP_OP_GEMM_BF16 = 1, PP_OP_GEMM_F32 = 2, PP_OP_COLSUM = 3, PP_OP_LN_FWD = 4,
     PP_OP_LN_BWD_INPUT = 5, PP_OP_LN_BWD_WEIGHT = 6, PP_OP_ATTN_FWD = 7, PP_OP_ATTN_BWD = 8,
     PP_OP_EMBED_FWD = 9, PP_OP_EMBED_BWD = 10, PP_OP_CE_LOSS = 11, PP_OP_ACCUM_BF16 = 12,
-    PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16
+    PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16,
+    PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -282,6 +301,9 @@ enum pp_op_kind {
  *   COPY_ROWS     p: src dst | i: n_rows row_bytes src_stride dst_stride
  *   FILL          p: dst | i: n_bytes | j: value
  *   ACT_BWD       p: dy aux dz | i: n | j: act dtype
+ *   SWIGLU_FWD    p: g u h | i: n
+ *   SWIGLU_BWD    p: g u dh dg du | i: n
+ *   ROPE          p: x cos sin | i: n_tok seq n_heads D ld | j: inverse
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped

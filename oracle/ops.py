@@ -7,7 +7,9 @@ fp32 CPU tensors; gradients come from autograd on these functions.
 
 Pinning: every function here is a direct torch library routine or a closed form checked against
 one in tests/test_oracle.py (gelu closed forms vs F.gelu, attention vs
-F.scaled_dot_product_attention, layer norm vs F.layer_norm, cross entropy vs F.cross_entropy).
+F.scaled_dot_product_attention, layer norm vs F.layer_norm, cross entropy vs F.cross_entropy,
+rms norm vs F.rms_norm, silu vs F.silu, the rotary embedding vs a complex-number rotation and its
+norm / relative-position invariants).
 """
 import math
 
@@ -32,6 +34,28 @@ def layer_norm(x, gamma, beta, eps):
     var = ((x - mean) ** 2).mean(-1, keepdim=True)
     y = (x - mean) / torch.sqrt(var + eps) * gamma
     return y + beta if beta is not None else y
+
+
+def rms_norm(x, gamma, eps):
+    return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gamma
+
+
+def swiglu(g, u):
+    return g * torch.sigmoid(g) * u
+
+
+def rope_tables(seq, D, theta=10000.0):
+    """cos, sin [seq, D/2] (fp32): angle of position p and frequency index i is p * theta^(-2i/D)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.arange(seq, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return torch.cos(ang), torch.sin(ang)
+
+
+def rope(x, cos, sin):
+    """Rotate-half rotary embedding.  x: [..., S, D]; cos, sin: [S, D/2]."""
+    half = x.shape[-1] // 2
+    a, b = x[..., :half], x[..., half:]
+    return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
 
 
 def attention(q, k, v, causal, scale=None):

@@ -23,7 +23,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7
 # enum pp_op_kind
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
- OP_FILL, OP_ACT_BWD) = range(1, 17)
+ OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE) = range(1, 20)
 OP_SKIP = 1
 OP_GROUPED = 2
 ACT_RELU, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
@@ -37,7 +37,7 @@ EXPORTED_SYMBOLS = (
     "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
-    "pp_profile_read", "pp_sgd_step", "pp_adamw_step",
+    "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
 )
 
 
@@ -125,6 +125,9 @@ def lib() -> C.CDLL:
         "pp_profile_start": [i32],
         "pp_profile_stop": [],
         "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
+        "pp_swiglu_fwd": [vp, vp, vp, i64, vp],
+        "pp_swiglu_bwd": [vp, vp, vp, vp, vp, i64, vp],
+        "pp_rope": [vp, vp, vp, i64, i64, i64, i64, i64, i32, vp],
         "pp_sgd_step": [vp, i32, vp, vp, vp, i64, f32, f32, f32, f32, i32, i32, i32, vp],
         "pp_adamw_step": [vp, i32, vp, vp, vp, vp, i64, f32, f32, f32, f32, f32, f32, f32, i32, vp],
     }
@@ -266,6 +269,30 @@ def _p_or_none(t):
     return None if t is None else t.data_ptr()
 
 
+# ---- Llama-style element-wise pieces ----------------------------------------------------------
+def swiglu_fwd(g, u, h) -> None:
+    require_cuda(g, u, h)
+    assert g.is_contiguous() and u.is_contiguous() and h.is_contiguous() and g.numel() == u.numel() == h.numel()
+    check(lib().pp_swiglu_fwd(g.data_ptr(), u.data_ptr(), h.data_ptr(), g.numel(), current_stream()), "pp_swiglu_fwd")
+
+
+def swiglu_bwd(g, u, dh, dg, du) -> None:
+    require_cuda(g, u, dh, dg, du)
+    for t in (g, u, dh, dg, du):
+        assert t.is_contiguous() and t.numel() == g.numel()
+    check(lib().pp_swiglu_bwd(g.data_ptr(), u.data_ptr(), dh.data_ptr(), dg.data_ptr(), du.data_ptr(), g.numel(),
+                              current_stream()), "pp_swiglu_bwd")
+
+
+def rope(x2d, cos, sin, seq: int, n_heads: int, D: int, inverse: bool = False) -> None:
+    """In-place rotation of the first ``n_heads`` heads of every row of ``x2d`` [tokens, ld]."""
+    require_cuda(x2d, cos, sin)
+    assert x2d.dim() == 2 and x2d.stride(1) == 1 and cos.dtype == torch.float32 and sin.dtype == torch.float32
+    assert cos.shape == sin.shape == (seq, D // 2) and cos.is_contiguous() and sin.is_contiguous()
+    check(lib().pp_rope(x2d.data_ptr(), cos.data_ptr(), sin.data_ptr(), x2d.shape[0], seq, n_heads, D,
+                        x2d.stride(0), int(inverse), current_stream()), "pp_rope")
+
+
 def fill_bytes(t: torch.Tensor, value: int = 0) -> None:
     require_cuda(t)
     assert t.is_contiguous()
@@ -362,7 +389,7 @@ def layernorm_fwd(x, gamma, beta, y, mean, rstd, eps: float) -> None:
     require_cuda(x, gamma, beta, y, mean, rstd)
     rows, Cc = x.shape
     check(lib().pp_layernorm_fwd(x.data_ptr(), gamma.data_ptr(), ptr(beta), y.data_ptr(),
-                                 mean.data_ptr(), rstd.data_ptr(), rows, Cc, eps,
+                                 ptr(mean), rstd.data_ptr(), rows, Cc, eps,
                                  current_stream()), "pp_layernorm_fwd")
 
 
@@ -370,7 +397,7 @@ def layernorm_bwd_input(dy, x, gamma, mean, rstd, dres, dx) -> None:
     require_cuda(dy, x, gamma, mean, rstd, dres, dx)
     rows, Cc = x.shape
     check(lib().pp_layernorm_bwd_input(dy.data_ptr(), x.data_ptr(), gamma.data_ptr(),
-                                       mean.data_ptr(), rstd.data_ptr(), ptr(dres), dx.data_ptr(),
+                                       ptr(mean), rstd.data_ptr(), ptr(dres), dx.data_ptr(),
                                        rows, Cc, current_stream()), "pp_layernorm_bwd_input")
 
 
@@ -378,7 +405,7 @@ def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:
     require_cuda(dy, x, mean, rstd, dgamma, dbeta, workspace)
     rows, Cc = x.shape
     assert workspace.numel() >= 2 * ((rows + 127) // 128) * Cc
-    check(lib().pp_layernorm_bwd_weight(dy.data_ptr(), x.data_ptr(), mean.data_ptr(),
+    check(lib().pp_layernorm_bwd_weight(dy.data_ptr(), x.data_ptr(), ptr(mean),
                                         rstd.data_ptr(), dgamma.data_ptr(), ptr(dbeta),
                                         PP_F32 if dgamma.dtype == torch.float32 else PP_BF16,
                                         workspace.data_ptr(), rows, Cc, current_stream()),

@@ -180,14 +180,48 @@ def op_act_bwd(dy, aux, dz, act) -> N.Op:
     return op
 
 
+def op_swiglu_fwd(g, u, h) -> N.Op:
+    assert g.is_contiguous() and u.is_contiguous() and h.is_contiguous()
+    assert g.numel() == u.numel() == h.numel() and g.numel() % 8 == 0 and g.dtype == torch.bfloat16
+    op = N.Op()
+    op.kind = N.OP_SWIGLU_FWD
+    op.p[0], op.p[1], op.p[2] = g.data_ptr(), u.data_ptr(), h.data_ptr()
+    op.i[0] = g.numel()
+    return op
+
+
+def op_swiglu_bwd(g, u, dh, dg, du) -> N.Op:
+    for t in (g, u, dh, dg, du):
+        assert t.is_contiguous() and t.numel() == g.numel() and t.dtype == torch.bfloat16
+    op = N.Op()
+    op.kind = N.OP_SWIGLU_BWD
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = (g.data_ptr(), u.data_ptr(), dh.data_ptr(), dg.data_ptr(),
+                                                   du.data_ptr())
+    op.i[0] = g.numel()
+    return op
+
+
+def op_rope(x2d, cos, sin, seq, n_heads, D, inverse=False) -> N.Op:
+    assert x2d.dim() == 2 and x2d.stride(1) == 1 and x2d.dtype == torch.bfloat16
+    assert cos.shape == sin.shape == (seq, D // 2) and cos.dtype == sin.dtype == torch.float32
+    assert n_heads * D <= x2d.stride(0) and x2d.shape[0] % seq == 0
+    op = N.Op()
+    op.kind = N.OP_ROPE
+    op.p[0], op.p[1], op.p[2] = x2d.data_ptr(), cos.data_ptr(), sin.data_ptr()
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4] = x2d.shape[0], seq, n_heads, D, x2d.stride(0)
+    op.j[0] = int(inverse)
+    return op
+
+
 def op_ln_fwd(x, gamma, beta, y, mean, rstd, eps) -> N.Op:
     rows, Cc = x.shape
     assert x.is_contiguous() and y.is_contiguous() and y.shape == x.shape
-    assert gamma.numel() == Cc and mean.numel() == rows and rstd.numel() == rows
+    assert gamma.numel() == Cc and rstd.numel() == rows and (mean is None or mean.numel() == rows)
+    assert mean is not None or beta is None, "RMSNorm (mean=None) has no beta"
     op = N.Op()
     op.kind = N.OP_LN_FWD
     op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = (x.data_ptr(), gamma.data_ptr(), _p(beta),
-                                                            y.data_ptr(), mean.data_ptr(), rstd.data_ptr())
+                                                            y.data_ptr(), _p(mean), rstd.data_ptr())
     op.i[0], op.i[1] = rows, Cc
     op.f[0] = eps
     return op
@@ -200,7 +234,7 @@ def op_ln_bwd_input(dy, x, gamma, mean, rstd, dres, dx) -> N.Op:
     op = N.Op()
     op.kind = N.OP_LN_BWD_INPUT
     op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5], op.p[6] = (
-        dy.data_ptr(), x.data_ptr(), gamma.data_ptr(), mean.data_ptr(), rstd.data_ptr(), _p(dres),
+        dy.data_ptr(), x.data_ptr(), gamma.data_ptr(), _p(mean), rstd.data_ptr(), _p(dres),
         dx.data_ptr())
     op.i[0], op.i[1] = rows, Cc
     return op
@@ -213,7 +247,7 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
     op = N.Op()
     op.kind = N.OP_LN_BWD_WEIGHT
     op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5], op.p[6] = (
-        dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dgamma.data_ptr(), _p(dbeta),
+        dy.data_ptr(), x.data_ptr(), _p(mean), rstd.data_ptr(), dgamma.data_ptr(), _p(dbeta),
         ws.data_ptr())
     op.i[0], op.i[1] = rows, Cc
     op.j[0] = N.PP_F32 if dgamma.dtype == torch.float32 else N.PP_BF16

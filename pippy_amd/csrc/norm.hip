@@ -35,7 +35,8 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const uint16_t* __re
             for (int e = 0; e < 8; ++e) s += v[i][e];
         }
     }
-    const float mean = wave_sum(s) / (float)C;
+    // a null mean_out selects RMSNorm: nothing is subtracted and rstd = 1 / sqrt(mean(x^2) + eps)
+    const float mean = mean_out ? wave_sum(s) / (float)C : 0.f;
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -51,7 +52,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const uint16_t* __re
     const float var = wave_sum(q) / (float)C;
     const float rstd = 1.0f / sqrtf(var + eps);
     if (lane == 0) {
-        mean_out[row] = mean;
+        if (mean_out) mean_out[row] = mean;
         rstd_out[row] = rstd;
     }
     uint4* yr = reinterpret_cast<uint4*>(y + row * C);
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_input_kernel(
     const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int nchunk = C >> 3;
-    const float mean = mean_in[row], rstd = rstd_in[row];
+    const float mean = mean_in ? mean_in[row] : 0.f, rstd = rstd_in[row];  // null mean: RMSNorm
     const uint4* xr = reinterpret_cast<const uint4*>(x + row * C);
     const uint4* gr = reinterpret_cast<const uint4*>(dy + row * C);
     float xh[NV][8], wd[NV][8];
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_input_kernel(
         }
     }
     const float c1 = wave_sum(s1) / (float)C;
-    const float c2 = wave_sum(s2) / (float)C;
+    const float c2 = mean_in ? wave_sum(s2) / (float)C : 0.f;
     uint4* outr = reinterpret_cast<uint4*>(dx + row * C);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(256) void colreduce_partial_kernel(
 #pragma unroll
                 for (int e = 0; e < 8; ++e) sb[e] += df[e];
                 if (WITH_X) {
-                    const float mean = mean_in[r], rstd = rstd_in[r];
+                    const float mean = mean_in ? mean_in[r] : 0.f, rstd = rstd_in[r];
                     const uint4 xw = *reinterpret_cast<const uint4*>(x + r * C + col0);
                     const float xf[8] = {bf16lo(xw.x), bf16hi(xw.x), bf16lo(xw.y), bf16hi(xw.y),
                                          bf16lo(xw.z), bf16hi(xw.z), bf16lo(xw.w), bf16hi(xw.w)};
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(256) void colgroup_partial_kernel(const ColGroupArg
 #pragma unroll
                 for (int e = 0; e < 8; ++e) sb[e] += df[e];
                 if (with_x) {
-                    const float mean = d.mean[r], rstd = d.rstd[r];
+                    const float mean = d.mean ? d.mean[r] : 0.f, rstd = d.rstd[r];
                     const uint4 xw = *reinterpret_cast<const uint4*>(d.x + (int64_t)r * d.C + col0);
                     const float xf[8] = {bf16lo(xw.x), bf16hi(xw.x), bf16lo(xw.y), bf16hi(xw.y),
                                          bf16lo(xw.z), bf16hi(xw.z), bf16lo(xw.w), bf16hi(xw.w)};
@@ -328,7 +329,8 @@ extern "C" int pp_layernorm_fwd(const void* x, const void* gamma, const void* be
     int rc = ln_check("pp_layernorm_fwd", rows, C);
     if (rc) return rc;
     if (rows == 0) return PP_OK;
-    if (!x || !gamma || !y || !mean || !rstd) return fail(PP_ERR_INVALID, "pp_layernorm_fwd: null pointer");
+    if (!x || !gamma || !y || !rstd) return fail(PP_ERR_INVALID, "pp_layernorm_fwd: null pointer");
+    if (!mean && beta) return fail(PP_ERR_INVALID, "pp_layernorm_fwd: RMSNorm (null mean) has no beta");
     if (!aligned(x, 16) || !aligned(y, 16) || !aligned(gamma, 16) || !aligned(beta, 16))
         return fail(PP_ERR_INVALID, "pp_layernorm_fwd: pointers must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -347,7 +349,7 @@ extern "C" int pp_layernorm_bwd_input(const void* dy, const void* x, const void*
     int rc = ln_check("pp_layernorm_bwd_input", rows, C);
     if (rc) return rc;
     if (rows == 0) return PP_OK;
-    if (!dy || !x || !gamma || !mean || !rstd || !dx)
+    if (!dy || !x || !gamma || !rstd || !dx)
         return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input: null pointer");
     if (!aligned(x, 16) || !aligned(dy, 16) || !aligned(gamma, 16) || !aligned(dres, 16) || !aligned(dx, 16))
         return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input: pointers must be 16-byte aligned");
@@ -366,7 +368,7 @@ extern "C" int pp_layernorm_bwd_weight(const void* dy, const void* x, const floa
                                        float* workspace, int64_t rows, int64_t C, pp_stream stream) {
     if (rows < 0 || C <= 0) return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: bad shape");
     if (C % 8) return fail(PP_ERR_UNSUPPORTED, "pp_layernorm_bwd_weight: C %% 8 != 0");
-    if (!dy || !x || !mean || !rstd || !dgamma || !workspace)
+    if (!dy || !x || !rstd || !dgamma || !workspace)
         return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: null pointer");
     if (!aligned(x, 16) || !aligned(dy, 16))
         return fail(PP_ERR_INVALID, "pp_layernorm_bwd_weight: pointers must be 16-byte aligned");
@@ -420,7 +422,7 @@ extern "C" int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_st
             if (s.rows < 0 || s.C <= 0 || s.ld_dy < s.C) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: bad shape in %d", i0 + i);
             if ((s.C % 8) || (s.ld_dy % 8)) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: C and ld must be multiples of 8");
             if (!s.dy || !s.workspace || (!s.out_sum && !s.out_dot)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: null pointer in %d", i0 + i);
-            if (s.out_dot && (!s.x || !s.mean || !s.rstd)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: out_dot needs x, mean, rstd");
+            if (s.out_dot && (!s.x || !s.rstd)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: out_dot needs x and rstd");
             if (!aligned(s.dy, 16) || !aligned(s.x, 16)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: dy and x must be 16-byte aligned");
             if (s.rows > 0x7fffffff || s.C > 0x7fffffff) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: shape too large");
             ColDesc& d = ga.d[ga.n];

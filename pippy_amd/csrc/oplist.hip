@@ -120,6 +120,13 @@ static int run_one(const pp_op& op, pp_stream st) {
             return pp_fill_bytes(op.p[0], op.j[0], op.i[0], st);
         case PP_OP_ACT_BWD:
             return pp_activation_bwd(op.p[0], op.p[1], op.p[2], op.i[0], op.j[0], op.j[1], st);
+        case PP_OP_SWIGLU_FWD:
+            return pp_swiglu_fwd(op.p[0], op.p[1], op.p[2], op.i[0], st);
+        case PP_OP_SWIGLU_BWD:
+            return pp_swiglu_bwd(op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.i[0], st);
+        case PP_OP_ROPE:
+            return pp_rope(op.p[0], static_cast<const float*>(op.p[1]), static_cast<const float*>(op.p[2]),
+                           op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.j[0], st);
         default:
             return fail(PP_ERR_INVALID, "unknown op kind %d", op.kind);
     }
@@ -173,6 +180,12 @@ double op_work(const pp_op& op) {
             return (double)op.i[0];
         case PP_OP_ACT_BWD:
             return 3.0 * (double)op.i[0] * (op.j[1] == PP_F32 ? 4.0 : 2.0);
+        case PP_OP_SWIGLU_FWD:
+            return 6.0 * (double)op.i[0];
+        case PP_OP_SWIGLU_BWD:
+            return 10.0 * (double)op.i[0];
+        case PP_OP_ROPE:
+            return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[3];
         default:
             return 0.0;
     }

@@ -545,3 +545,72 @@ def test_optimizer_steps_reject_bad_arguments():
         N.sgd_step(p, g, None, lr=0.1, momentum=0.9)
     with pytest.raises(RuntimeError, match="master copy goes with bf16"):
         N.sgd_step(p, g, None, master=torch.zeros(8, device="cuda"), lr=0.1)
+
+
+# ---- RMSNorm, SwiGLU, RoPE ----------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,C", [(64, 4096), (37, 1024), (5, 128)])
+def test_rmsnorm_matches_oracle(rows, C):
+    N = native()
+    g0 = torch.Generator().manual_seed(rows)
+    x = (torch.randn(rows, C, generator=g0) * 2).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(C, generator=g0)).to(torch.bfloat16)
+    dy = torch.randn(rows, C, generator=g0).to(torch.bfloat16)
+    dres = torch.randn(rows, C, generator=g0).to(torch.bfloat16)
+    xd, wd, dyd, dresd = x.cuda(), w.cuda(), dy.cuda(), dres.cuda()
+    y = torch.empty_like(xd)
+    rstd = torch.empty(rows, device="cuda")
+    N.layernorm_fwd(xd, wd, None, y, None, rstd, 1e-5)
+    xr = x.float().requires_grad_(True)
+    wr = w.float().requires_grad_(True)
+    yr = O.rms_norm(xr, wr, 1e-5)
+    assert_close_rel(y, yr.detach(), BF16_TOL, "rmsnorm forward")
+    yr.backward(dy.float())
+    dx = torch.empty_like(xd)
+    N.layernorm_bwd_input(dyd, xd, wd, None, rstd, dresd, dx)
+    assert_close_rel(dx, xr.grad + dres.float(), BF16_TOL, "rmsnorm input gradient (+ residual)")
+    dgamma = torch.empty(C, device="cuda")
+    ws = torch.empty(2 * ((rows + 127) // 128) * C, device="cuda")
+    N.layernorm_bwd_weight(dyd, xd, None, rstd, dgamma, None, ws)
+    assert_close_rel(dgamma, wr.grad, 1e-3, "rmsnorm weight gradient")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [8, 2048 * 11008, 1000 * 8])
+def test_swiglu_matches_oracle(n):
+    N = native()
+    g0 = torch.Generator().manual_seed(n % 97)
+    g = (torch.randn(n, generator=g0) * 2).to(torch.bfloat16)
+    u = torch.randn(n, generator=g0).to(torch.bfloat16)
+    dh = torch.randn(n, generator=g0).to(torch.bfloat16)
+    gd, ud, dhd = g.cuda(), u.cuda(), dh.cuda()
+    h = torch.empty_like(gd)
+    N.swiglu_fwd(gd, ud, h)
+    gr, ur = g.float().requires_grad_(True), u.float().requires_grad_(True)
+    hr = O.swiglu(gr, ur)
+    assert_close_rel(h, hr.detach(), BF16_TOL, "swiglu forward")
+    hr.backward(dh.float())
+    dg, du = torch.empty_like(gd), torch.empty_like(gd)
+    N.swiglu_bwd(gd, ud, dhd, dg, du)
+    assert_close_rel(dg, gr.grad, BF16_TOL, "swiglu gate gradient")
+    assert_close_rel(du, ur.grad, BF16_TOL, "swiglu up gradient")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,S,H,D", [(2, 64, 3, 64), (1, 2048, 4, 128), (3, 16, 2, 32)])
+def test_rope_matches_oracle_and_inverts(B, S, H, D):
+    N = native()
+    g0 = torch.Generator().manual_seed(S + D)
+    qkv = torch.randn(B * S, 3 * H * D, generator=g0).to(torch.bfloat16)
+    cos, sin = O.rope_tables(S, D)
+    x = qkv.cuda()
+    N.rope(x, cos.cuda(), sin.cuda(), S, 2 * H, D)
+    ref = qkv.float().view(B, S, 3, H, D).clone()
+    ref[:, :, 0] = O.rope(ref[:, :, 0].transpose(1, 2), cos, sin).transpose(1, 2)
+    ref[:, :, 1] = O.rope(ref[:, :, 1].transpose(1, 2), cos, sin).transpose(1, 2)
+    assert_close_rel(x, ref.view(B * S, 3 * H * D), BF16_TOL, "rope on the q and k heads")
+    # the v third of every row is untouched, bit for bit
+    assert torch.equal(x.view(B * S, 3, H * D)[:, 2].cpu(), qkv.view(B * S, 3, H * D)[:, 2])
+    # the inverse rotation brings q and k back (two bf16 roundings away)
+    N.rope(x, cos.cuda(), sin.cuda(), S, 2 * H, D, inverse=True)
+    assert_close_rel(x, qkv.float(), BF16_TOL, "rope followed by its transpose")

@@ -254,3 +254,34 @@ def test_adamw_oracle_matches_torch_optim(wd, maximize):
 def test_round_bf16_matches_torch():
     x = torch.randn(1000, generator=torch.Generator().manual_seed(0)) * 7
     np.testing.assert_array_equal(OO.round_bf16(x.numpy()), x.to(torch.bfloat16).float().numpy())
+
+
+# ---- Llama-style pieces ------------------------------------------------------------------------
+def test_rms_norm_and_swiglu_match_torch():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(5, 48, generator=g) * 3
+    w = torch.randn(48, generator=g)
+    torch.testing.assert_close(O.rms_norm(x, w, 1e-5), F.rms_norm(x, (48,), w, 1e-5))
+    a, b = torch.randn(7, 16, generator=g), torch.randn(7, 16, generator=g)
+    torch.testing.assert_close(O.swiglu(a, b), F.silu(a) * b)
+
+
+def test_rope_is_a_complex_rotation_with_relative_position_property():
+    g = torch.Generator().manual_seed(4)
+    S, D = 12, 8
+    cos, sin = O.rope_tables(S, D, theta=100.0)
+    x = torch.randn(2, 3, S, D, generator=g)
+    y = O.rope(x, cos, sin)
+    # pairs (x[i], x[i + D/2]) rotate as complex numbers by angle p * theta^(-2i/D)
+    z = torch.complex(x[..., :D // 2], x[..., D // 2:])
+    inv_freq = 100.0 ** (-torch.arange(0, D, 2, dtype=torch.float32) / D)
+    rot = torch.polar(torch.ones(S, D // 2), torch.arange(S, dtype=torch.float32)[:, None] * inv_freq)
+    zr = z * rot
+    torch.testing.assert_close(y, torch.cat([zr.real, zr.imag], dim=-1))
+    # rotations preserve norms, position 0 is the identity, and q.k depends on the distance only
+    torch.testing.assert_close(y.norm(dim=-1), x.norm(dim=-1))
+    torch.testing.assert_close(y[..., 0, :], x[..., 0, :])
+    q = torch.randn(D, generator=g).expand(S, D)
+    k = torch.randn(D, generator=g).expand(S, D)
+    qr, kr = O.rope(q, cos, sin), O.rope(k, cos, sin)
+    torch.testing.assert_close((qr[5] * kr[2]).sum(), (qr[9] * kr[6]).sum(), rtol=1e-4, atol=1e-5)
