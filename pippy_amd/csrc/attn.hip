@@ -1,5 +1,5 @@
 // Flash-style multi-head attention for gfx950 (forward, and a two-kernel deterministic backward)
-// on v_mfma_f32_32x32x16_bf16, head dimension 64.
+// on v_mfma_f32_32x32x16_bf16, head dimension 64 or 128.
 //
 // Forward: a work-group owns 64 query rows of one (batch, head) and streams keys/values through LDS
 // in blocks of 64 rows.  Its 4 waves are 2 groups of 32 query rows x 2 halves of every key block:
@@ -17,9 +17,10 @@
 // the waves: partial sums of the two halves are added in a fixed order through LDS.  No atomics:
 // results are run-to-run identical.
 //
-// Staging: every streamed operand is a 64 x 64 bf16 tile kept in LDS exactly as it lies in memory
-// ([row][d], 128 B per row, 16-byte chunks XOR-swizzled by the row), filled by direct-to-LDS buffer
-// loads, three stages deep with one barrier per block of 64 rows.  A fragment whose MFMA k index
+// Staging: every streamed operand is a block of 64 rows kept in LDS exactly as it lies in memory,
+// as one 64 x 64 bf16 tile per 64 columns of the head ([row][d], 128 B per row, 16-byte chunks
+// XOR-swizzled by the row), filled by direct-to-LDS buffer loads, three stages deep (two for head
+// dimension 128) with one barrier per block of 64 rows.  A fragment whose MFMA k index
 // runs along d is a ds_read_b128 of one row; a fragment whose k index runs along the tile's rows
 // (V^T in the forward pass, K^T, Q^T and dO^T in the backward pass) comes out of the same tile
 // through ds_read_b64_tr_b16, so no transposed copy is ever made.
@@ -51,14 +52,17 @@ __device__ __forceinline__ bf16x8_t pack8(const float* p) {
 
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kTile = 64 * 64;  // elements of one staged tile
-constexpr int kAttnStages = 3;
+// LDS stages: 3 x 16 KiB for head dimension 64 (three work-groups per CU), 2 x 32 KiB for 128
+constexpr int attn_stages(int D) { return D == 64 ? 3 : 2; }
 
 // Chunk swizzle of a staged tile.  Rows r and r+1 start 32 banks apart; the first term spreads 16
 // consecutive rows read at one chunk index (ds_read_b128 fragments), the second separates rows r
 // and r+2, which a transposing read touches together.
 __device__ __forceinline__ int swz_attn(int r) { return ((r ^ (r >> 3)) & 7) ^ ((r & 2) << 1); }
 
-// Direct-to-LDS loader of 64-row tiles out of a [rows][stride] operand (64 d = 128 B per row).
+// Direct-to-LDS loader of 64-row blocks out of a [rows][stride] operand: DS tiles of 64 columns
+// (128 B per row and tile), tile s at lds + s * kTile.
+template <int DS>
 struct AttnTileLoader {
     __amdgpu_buffer_rsrc_t rsrc;
     int voff[2];
@@ -74,8 +78,11 @@ struct AttnTileLoader {
     }
     __device__ __forceinline__ void load(uint16_t* lds, int64_t row0, int wave) const {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i], (int)row0 * row_bytes);
+        for (int s = 0; s < DS; ++s)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                load_to_lds_b128(rsrc, lds + s * kTile + (i * 4 + wave) * 512, voff[i] + s * 128,
+                                 (int)row0 * row_bytes);
     }
 };
 
@@ -113,21 +120,26 @@ __device__ __forceinline__ bf16x8_t read_col_frag(const uint16_t* tile, int r0, 
 }
 
 // Pipeline step shared by the three kernels: block j of `nb` has landed for every wave, and the
-// stage that block j-1 occupied is free.  `lpt` loads per block per wave.
-template <int LPT>
+// stage that block j-1 occupied is free.  LPT loads per block per wave; with NS stages, NS - 2
+// younger blocks may stay in flight.
+template <int LPT, int NS>
 __device__ __forceinline__ void await_block(int64_t j, int64_t nb) {
-    if (j + 1 < nb) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
+    static_assert(NS == 2 || NS == 3, "two or three stages");
+    if (NS == 3 && j + 1 < nb) wait_vmcnt<(NS == 3 ? LPT : 0)>(); else wait_vmcnt<0>();
     wait_lds();
     __builtin_amdgcn_s_barrier();
 }
 
+extern __shared__ __attribute__((aligned(16))) uint16_t attn_lds[];
+
 // ---- forward ----------------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
-    static_assert(D == 64, "head dimension 64");
-    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
-    constexpr int kStage = 2 * kTile;  // K tile, V tile
-    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
+__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const AttnArgs a) {
+    static_assert(D == 64 || D == 128, "head dimension 64 or 128");
+    constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = attn_stages(D);
+    constexpr int kOperand = DS * kTile;   // one staged 64-row block of K or V
+    constexpr int kStage = 2 * kOperand;
+    uint16_t* const lds = attn_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -144,13 +156,13 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
     const int64_t qi = qw0 + l32;  // this lane's query row
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
-    AttnTileLoader lk, lv;
+    AttnTileLoader<DS> lk, lv;
     lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
     auto issue = [&](int stage, int64_t j) {
         lk.load(lds + stage * kStage, j * 64, wave);
-        lv.load(lds + stage * kStage + kTile, j * 64, wave);
+        lv.load(lds + stage * kStage + kOperand, j * 64, wave);
     };
 
     bf16x8_t qf[KS];
@@ -172,10 +184,10 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
     int stage = 0;
     for (int64_t j = 0; j < n_blocks; ++j) {
         const int64_t kt0 = j * 64 + 32 * half;  // first key of this wave's half block
-        await_block<4>(j, n_blocks);
+        await_block<4 * DS, NS>(j, n_blocks);
         if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Ks = lds + stage * kStage;
-        const uint16_t* Vs = Ks + kTile;
+        const uint16_t* Vs = Ks + kOperand;
         stage = stage + 1 == NS ? 0 : stage + 1;
         const bool active = !CAUSAL || (kt0 <= qw0 + 31);
         if (active) {
@@ -184,7 +196,7 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
             for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t kf = read_row_frag(Ks, 32 * half + l32, 2 * ks + lh);
+                const bf16x8_t kf = read_row_frag(Ks + (ks / 4) * kTile, 32 * half + l32, 2 * (ks % 4) + lh);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
             }
             // sacc[v]: kv = kt0 + 8 (v/4) + 4 lh + v%4, q = qi
@@ -232,28 +244,29 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const AttnArgs a) {
                 const bf16x8_t pb = pack8(pv);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t vf = read_col_frag(Vs, 32 * half + 16 * gp, 32 * dt, lane);
+                    const bf16x8_t vf = read_col_frag(Vs + (dt / 2) * kTile, 32 * half + 16 * gp, 32 * (dt % 2), lane);
                     oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, oacc[dt], 0, 0, 0);
                 }
             }
         }
     }
 
-    // merge the two halves of every key block: [grp][34 values][64 lanes] floats
+    // merge the two halves of every key block: [grp][16 DT + 2 values][64 lanes] floats
     wait_lds();
     __builtin_amdgcn_s_barrier();
-    float* xs = reinterpret_cast<float*>(lds) + grp * (34 * 64) + lane;
+    constexpr int kVals = 16 * DT + 2;
+    float* xs = reinterpret_cast<float*>(lds) + grp * (kVals * 64) + lane;
     if (half == 1) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) xs[(16 * dt + e) * 64] = oacc[dt][e];
-        xs[32 * 64] = m_run;
-        xs[33 * 64] = l_run;
+        xs[16 * DT * 64] = m_run;
+        xs[(16 * DT + 1) * 64] = l_run;
     }
     __syncthreads();
     if (half == 0) {
-        const float m1 = xs[32 * 64], l1 = xs[33 * 64];
+        const float m1 = xs[16 * DT * 64], l1 = xs[(16 * DT + 1) * 64];
         const float m = fmaxf(m_run, m1);  // finite: key 0 is visible to every query
         const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c);
         const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * c);
@@ -307,11 +320,12 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
 
 // ---- backward: dK, dV (parallel over key blocks) ------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) {
-    static_assert(D == 64, "head dimension 64");
-    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
-    constexpr int kStage = 2 * kTile + 256;  // Q tile, dO tile, 64 lse, 64 delta
-    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
+__global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(const AttnArgs a) {
+    static_assert(D == 64 || D == 128, "head dimension 64 or 128");
+    constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = attn_stages(D);
+    constexpr int kOperand = DS * kTile;     // one staged 64-row block of Q or dO
+    constexpr int kStage = 2 * kOperand + 256;  // Q, dO, 64 lse, 64 delta
+    uint16_t* const lds = attn_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -328,21 +342,21 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
     const uint16_t* kp = a.k + b * a.stride_b + h * D;
     const uint16_t* vp = a.v + b * a.stride_b + h * D;
     const int64_t ldo = a.H * D;
-    AttnTileLoader lq, ldo_;
+    AttnTileLoader<DS> lq, ldo_;
     lq.init(a.q + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     ldo_.init(a.d_o + b * a.S * ldo + h * D, ldo, a.S, wave, lane);
     // waves 0 and 2 fetch lse, waves 1 and 3 delta (the same values twice: every wave issues the
     // same number of loads, which keeps the vmcnt arithmetic uniform)
     const float* stat = ((wave & 1) ? a.delta : a.lse) + (b * a.H + h) * a.S;
     const __amdgpu_buffer_rsrc_t rstat = make_rsrc(stat, (uint64_t)a.S * 4);
-    const int stat_off = 2 * kTile + ((wave & 1) ? 128 : 0);
+    const int stat_off = 2 * kOperand + ((wave & 1) ? 128 : 0);
 
     const int64_t jq_begin = CAUSAL ? kv0 / 64 : 0;
     const int64_t nb = a.S / 64 - jq_begin;
     auto issue = [&](int stage, int64_t j) {
         uint16_t* st = lds + stage * kStage;
         lq.load(st, (jq_begin + j) * 64, wave);
-        ldo_.load(st + kTile, (jq_begin + j) * 64, wave);
+        ldo_.load(st + kOperand, (jq_begin + j) * 64, wave);
         load_floats_to_lds(rstat, reinterpret_cast<float*>(st + stat_off), (jq_begin + j) * 64, lane);
     };
 
@@ -369,11 +383,11 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
     int stage = 0;
     for (int64_t j = 0; j < nb; ++j) {
         const int64_t qc0 = (jq_begin + j) * 64;
-        await_block<5>(j, nb);
+        await_block<4 * DS + 1, NS>(j, nb);
         if (j + NS - 1 < nb) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Qs = lds + stage * kStage;
-        const uint16_t* Os = Qs + kTile;
-        const float* lse_s = reinterpret_cast<const float*>(Qs + 2 * kTile);
+        const uint16_t* Os = Qs + kOperand;
+        const float* lse_s = reinterpret_cast<const float*>(Qs + 2 * kOperand);
         const float* delta_s = lse_s + 64;
         stage = stage + 1 == NS ? 0 : stage + 1;
         const int qt = half;
@@ -387,8 +401,8 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t qfr = read_row_frag(Qs, 32 * qt + l32, 2 * ks + lh);
-                const bf16x8_t ofr = read_row_frag(Os, 32 * qt + l32, 2 * ks + lh);
+                const bf16x8_t qfr = read_row_frag(Qs + (ks / 4) * kTile, 32 * qt + l32, 2 * (ks % 4) + lh);
+                const bf16x8_t ofr = read_row_frag(Os + (ks / 4) * kTile, 32 * qt + l32, 2 * (ks % 4) + lh);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr, kf[ks], sacc, 0, 0, 0);
                 dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ofr, vf[ks], dpacc, 0, 0, 0);
             }
@@ -421,18 +435,18 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
                 const bf16x8_t dsb = pack8(dsv + 8 * gp);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t otf = read_col_frag(Os, 32 * qt + 16 * gp, 32 * dt, lane);
-                    const bf16x8_t qtf = read_col_frag(Qs, 32 * qt + 16 * gp, 32 * dt, lane);
+                    const bf16x8_t otf = read_col_frag(Os + (dt / 2) * kTile, 32 * qt + 16 * gp, 32 * (dt % 2), lane);
+                    const bf16x8_t qtf = read_col_frag(Qs + (dt / 2) * kTile, 32 * qt + 16 * gp, 32 * (dt % 2), lane);
                     dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(otf, pb, dvacc[dt], 0, 0, 0);
                     dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtf, dsb, dkacc[dt], 0, 0, 0);
                 }
             }
         }
     }
-    // add the partial sums of the two query halves: [grp][32 values][64 lanes] floats, dV then dK
+    // add the partial sums of the two query halves: [grp][16 DT values][64 lanes] floats, dV then dK
     wait_lds();
     __builtin_amdgcn_s_barrier();
-    float* xs = reinterpret_cast<float*>(lds) + grp * (32 * 64) + lane;
+    float* xs = reinterpret_cast<float*>(lds) + grp * (16 * DT * 64) + lane;
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
         f32x16_t(&acc)[DT] = pass == 0 ? dvacc : dkacc;
@@ -471,11 +485,12 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dkv_kernel(const AttnArgs a) 
 
 // ---- backward: dQ (parallel over query blocks) ---------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
-    static_assert(D == 64, "head dimension 64");
-    constexpr int KS = D / 16, DT = D / 32, NS = kAttnStages;
-    constexpr int kStage = 2 * kTile;  // K tile, V tile
-    __shared__ __attribute__((aligned(16))) uint16_t lds[NS * kStage];
+__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+    static_assert(D == 64 || D == 128, "head dimension 64 or 128");
+    constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = attn_stages(D);
+    constexpr int kOperand = DS * kTile;   // one staged 64-row block of K or V
+    constexpr int kStage = 2 * kOperand;
+    uint16_t* const lds = attn_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -492,13 +507,13 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
     const int64_t ldo = a.H * D;
     const uint16_t* dop = a.d_o + b * a.S * ldo + h * D;
-    AttnTileLoader lk, lv;
+    AttnTileLoader<DS> lk, lv;
     lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
     auto issue = [&](int stage, int64_t j) {
         lk.load(lds + stage * kStage, j * 64, wave);
-        lv.load(lds + stage * kStage + kTile, j * 64, wave);
+        lv.load(lds + stage * kStage + kOperand, j * 64, wave);
     };
 
     bf16x8_t qf[KS], dof[KS];
@@ -523,10 +538,10 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
     int stage = 0;
     for (int64_t j = 0; j < n_blocks; ++j) {
         const int64_t kv0 = j * 64;
-        await_block<4>(j, n_blocks);
+        await_block<4 * DS, NS>(j, n_blocks);
         if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Ks = lds + stage * kStage;
-        const uint16_t* Vs = Ks + kTile;
+        const uint16_t* Vs = Ks + kOperand;
         stage = stage + 1 == NS ? 0 : stage + 1;
         const int t = half;
         const int64_t kt0 = kv0 + 32 * t;
@@ -539,8 +554,8 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
             }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t kfr = read_row_frag(Ks, 32 * t + l32, 2 * ks + lh);
-                const bf16x8_t vfr = read_row_frag(Vs, 32 * t + l32, 2 * ks + lh);
+                const bf16x8_t kfr = read_row_frag(Ks + (ks / 4) * kTile, 32 * t + l32, 2 * (ks % 4) + lh);
+                const bf16x8_t vfr = read_row_frag(Vs + (ks / 4) * kTile, 32 * t + l32, 2 * (ks % 4) + lh);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[ks], sacc, 0, 0, 0);
                 dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[ks], dpacc, 0, 0, 0);
             }
@@ -561,16 +576,16 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
                 const bf16x8_t dsb = pack8(dsv + 8 * gp);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t ktf = read_col_frag(Ks, 32 * t + 16 * gp, 32 * dt, lane);
+                    const bf16x8_t ktf = read_col_frag(Ks + (dt / 2) * kTile, 32 * t + 16 * gp, 32 * (dt % 2), lane);
                     dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf, dsb, dqacc[dt], 0, 0, 0);
                 }
             }
         }
     }
-    // add the partial sums of the two key halves: [grp][32 values][64 lanes] floats
+    // add the partial sums of the two key halves: [grp][16 DT values][64 lanes] floats
     wait_lds();
     __builtin_amdgcn_s_barrier();
-    float* xs = reinterpret_cast<float*>(lds) + grp * (32 * 64) + lane;
+    float* xs = reinterpret_cast<float*>(lds) + grp * (16 * DT * 64) + lane;
     if (half == 1) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -598,7 +613,8 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(const AttnArgs a) {
 static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
     if (!d) return fail(PP_ERR_INVALID, "%s: null descriptor", who);
     if (d->B < 0 || d->S < 0 || d->H <= 0) return fail(PP_ERR_INVALID, "%s: bad shape", who);
-    if (d->D != 64) return fail(PP_ERR_UNSUPPORTED, "%s: head_dim %lld (only 64 is built)", who, (long long)d->D);
+    if (d->D != 64 && d->D != 128)
+        return fail(PP_ERR_UNSUPPORTED, "%s: head_dim %lld (64 and 128 are built)", who, (long long)d->D);
     if (d->S % 128) return fail(PP_ERR_UNSUPPORTED, "%s: S %% 128 != 0 (S=%lld)", who, (long long)d->S);
     if ((d->stride_s % 8) || (d->stride_b % 8)) return fail(PP_ERR_INVALID, "%s: strides must be multiples of 8", who);
     if (d->stride_s < d->H * d->D) return fail(PP_ERR_INVALID, "%s: stride_s < H*D", who);
@@ -627,6 +643,48 @@ static AttnArgs to_args(const pp_attn_desc* d) {
     return a;
 }
 
+// Dynamic LDS of the three kernels: stages, or the merge buffers of the epilogue if those are larger.
+static size_t attn_lds_bytes(int D, bool dkv) {
+    const size_t stage = (size_t)2 * (D / 64) * kTile * 2 + (dkv ? 512 : 0);
+    const size_t merge = (size_t)2 * (16 * (D / 32) + 2) * 64 * 4;
+    const size_t stages = (size_t)attn_stages(D) * stage;
+    return stages > merge ? stages : merge;
+}
+
+template <auto kernel>
+static int attn_launch(const char* name, dim3 grid, size_t lds, hipStream_t st, const AttnArgs& a) {
+    // one attribute call per kernel (the kernel is a template argument, so is the static) and process
+    static const hipError_t attr_rc =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr_rc != hipSuccess)
+        return fail(PP_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS: %s", name, lds, hipGetErrorString(attr_rc));
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, a);
+    return check_launch(name);
+}
+
+template <int D>
+static int attn_fwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
+    const size_t lds = attn_lds_bytes(D, false);
+    return d->causal ? attn_launch<attn_fwd_kernel<D, true>>("attn_fwd_kernel", grid, lds, st, a)
+                     : attn_launch<attn_fwd_kernel<D, false>>("attn_fwd_kernel", grid, lds, st, a);
+}
+
+template <int D>
+static int attn_bwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
+    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((uint32_t)((d->B * d->S + 3) / 4)), dim3(256), 0, st, a);
+    int rc = check_launch("attn_delta_kernel");
+    if (rc) return rc;
+    const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false);
+    if (d->causal) {
+        rc = attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+        if (rc) return rc;
+        return attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+    }
+    rc = attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+    if (rc) return rc;
+    return attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+}
+
 }  // namespace pp
 
 using namespace pp;
@@ -636,11 +694,9 @@ extern "C" int pp_attn_fwd(const pp_attn_desc* d, pp_stream stream) {
     if (rc) return rc;
     if (d->B == 0 || d->S == 0) return PP_OK;
     const AttnArgs a = to_args(d);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((uint32_t)(((d->S / 64) * d->H * d->B + 7) / 8 * 8));
-    if (d->causal) hipLaunchKernelGGL((attn_fwd_kernel<64, true>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<64, false>), grid, dim3(256), 0, st, a);
-    return check_launch("attn_fwd_kernel");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return d->D == 64 ? attn_fwd_d<64>(d, a, grid, st) : attn_fwd_d<128>(d, a, grid, st);
 }
 
 extern "C" int pp_attn_bwd(const pp_attn_desc* d, pp_stream stream) {
@@ -648,15 +704,7 @@ extern "C" int pp_attn_bwd(const pp_attn_desc* d, pp_stream stream) {
     if (rc) return rc;
     if (d->B == 0 || d->S == 0) return PP_OK;
     const AttnArgs a = to_args(d);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((uint32_t)((d->B * d->S + 3) / 4)), dim3(256), 0, st, a);
     const dim3 grid((uint32_t)(((d->S / 64) * d->H * d->B + 7) / 8 * 8));
-    if (d->causal) {
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<64, true>), grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<64, true>), grid, dim3(256), 0, st, a);
-    } else {
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<64, false>), grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<64, false>), grid, dim3(256), 0, st, a);
-    }
-    return check_launch("attn_bwd");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return d->D == 64 ? attn_bwd_d<64>(d, a, grid, st) : attn_bwd_d<128>(d, a, grid, st);
 }

@@ -373,15 +373,15 @@ def test_ce_loss_f32():
 
 # ---- attention -----------------------------------------------------------------------------------
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("B,S,H", [(1, 128, 1), (2, 256, 3), (1, 1024, 2)])
-def test_attention(causal, B, S, H):
+@pytest.mark.parametrize("B,S,H,D", [(1, 128, 1, 64), (2, 256, 3, 64), (1, 1024, 2, 64),
+                                     (1, 128, 1, 128), (2, 256, 3, 128), (1, 2048, 2, 128)])
+def test_attention(causal, B, S, H, D):
     Nn = native()
     torch.manual_seed(12 + S)
-    D = 64
     qkv = torch.randn(B, S, 3 * H * D, device=DEV).to(torch.bfloat16)
     o = torch.full((B, S, H * D), float("nan"), device=DEV, dtype=torch.bfloat16)
     lse = torch.empty(B, H, S, device=DEV)
-    note(f"attention fwd B={B} S={S} H={H} causal={causal}")
+    note(f"attention fwd B={B} S={S} H={H} D={D} causal={causal}")
     Nn.attn_fwd(qkv, o, lse, H, causal)
     torch.cuda.synchronize()
     qr = qkv.float().cpu().requires_grad_(True)
@@ -391,7 +391,7 @@ def test_attention(causal, B, S, H):
     d_o = torch.randn(B, S, H * D, device=DEV).to(torch.bfloat16)
     dqkv = torch.full_like(qkv, float("nan"))
     delta = torch.empty(B, H, S, device=DEV)
-    note(f"attention bwd B={B} S={S} H={H} causal={causal}")
+    note(f"attention bwd B={B} S={S} H={H} D={D} causal={causal}")
     Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal)
     torch.cuda.synchronize()
     ref.backward(d_o.float().cpu())
