@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .stage_modules import EncoderEmbedding, LMHead, TokenEmbedding, TransformerLayer
+from .stage_modules import EncoderEmbedding, LlamaLayer, LMHead, TokenEmbedding, TransformerLayer
 
 
 class DecoderLM(nn.Module):
@@ -60,6 +60,27 @@ class EncoderModel(nn.Module):
 def bert_base(dtype=torch.bfloat16) -> EncoderModel:
     """12 layers, hidden 768, 12 heads, FFN 3072, vocabulary 30522, sequence 512."""
     return EncoderModel(dtype=dtype)
+
+
+class LlamaStage(nn.Module):
+    """One pipeline stage's share of a Llama-style decoder: ``n_layers`` decoder layers applied to
+    incoming activations ``[batch, seq, dim]`` (no embedding, no head)."""
+
+    def __init__(self, n_layers=8, dim=4096, n_heads=32, ffn=11008, eps=1e-5, rope_theta=1e4,
+                 dtype=torch.bfloat16):
+        super().__init__()
+        self.layers = nn.ModuleList([
+            LlamaLayer(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype) for _ in range(n_layers)])
+
+    def forward(self, x):
+        for layer in self.layers:
+            x = layer(x)
+        return x
+
+
+def llama2_7b_stage(dtype=torch.bfloat16) -> LlamaStage:
+    """8 of the 32 layers of a Llama-2-7B-shaped model: width 4096, 32 heads of 128, SwiGLU 11008."""
+    return LlamaStage(dtype=dtype)
 
 
 def equal_split_spec(n_layers: int, n_stages: int, prefix: str = "h"):

@@ -423,6 +423,135 @@ class TransformerLayer(NativeBlock):
         return y.view(Bn, S, Cc)
 
 
+def rope_tables(seq: int, head_dim: int, theta: float, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos, sin [seq, head_dim / 2] in fp32: the angle of position p and frequency index i is
+    p * theta^(-2 i / head_dim)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+    ang = torch.arange(seq, dtype=torch.float32, device=device)[:, None] * inv_freq[None, :]
+    return torch.cos(ang).contiguous(), torch.sin(ang).contiguous()
+
+
+def _apply_rope(x, cos, sin):
+    """Rotate-half rotary embedding on [batch, heads, seq, head_dim] (torch statement of the block)."""
+    half = x.shape[-1] // 2
+    a, b = x[..., :half].float(), x[..., half:].float()
+    return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(x.dtype)
+
+
+def lower_rmsnorm(b: "P.Builder", name: str, norm: nn.Module, x2d: torch.Tensor):
+    T, Cc = x2d.shape
+    y = b.act(name, (T, Cc))
+    rstd = b.act(name + ".rstd", (T,), torch.float32)
+    b.f(P.op_ln_fwd(x2d, b.weight(norm.weight), None, y, None, rstd, norm.eps))
+    return y, rstd
+
+
+def rmsnorm_backward(b: "P.Builder", name: str, norm: nn.Module, x2d, rstd, dy2d, dres=None, dx_out=None):
+    """I: dx = RMSNorm'(dy) + dres; W: dgamma."""
+    T, Cc = x2d.shape
+    dx = dx_out if dx_out is not None else b.grad(name + ".dx", (T, Cc))
+    b.i(P.op_ln_bwd_input(dy2d, x2d, b.weight(norm.weight), None, rstd, dres, dx))
+    ws = b.workspace("rms_bwd:" + str(id(norm)), (2 * ((T + 127) // 128) * Cc,), torch.float32)
+    if b.fused_accumulate:
+        dg = b.workspace("rms_dg:" + str(id(norm)), (Cc,), torch.float32)
+        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, None, rstd, dg, None, ws))
+        b.w(P.op_accum(b.grad_acc(norm.weight), dg), tag="accum")
+    else:
+        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, None, rstd, b.grad_target(norm.weight), None, ws))
+    return dx
+
+
+class LlamaLayer(NativeBlock):
+    """One Llama-style decoder layer: RMSNorm, causal self-attention with rotary position embedding
+    on a fused q|k|v projection, RMSNorm, SwiGLU feed-forward; no biases.  Parameter names follow the
+    Hugging Face layer (``input_layernorm``, ``self_attn.o_proj``, ``post_attention_layernorm``,
+    ``mlp.gate_proj / up_proj / down_proj``) except for the fused ``self_attn.qkv_proj``."""
+
+    def __init__(self, dim: int, n_heads: int, ffn: int, *, eps: float = 1e-5, rope_theta: float = 1e4,
+                 dtype=torch.bfloat16, init_std=0.02):
+        super().__init__()
+        assert dim % n_heads == 0 and (dim // n_heads) in (64, 128), "head dimension 64 or 128"
+        self.dim, self.n_heads, self.ffn = dim, n_heads, ffn
+        self.eps, self.rope_theta = eps, rope_theta
+        self.input_layernorm = nn.RMSNorm(dim, eps=eps, dtype=dtype)
+        self.self_attn = nn.Module()
+        self.self_attn.qkv_proj = nn.Linear(dim, 3 * dim, bias=False, dtype=dtype)
+        self.self_attn.o_proj = nn.Linear(dim, dim, bias=False, dtype=dtype)
+        self.post_attention_layernorm = nn.RMSNorm(dim, eps=eps, dtype=dtype)
+        self.mlp = nn.Module()
+        self.mlp.gate_proj = nn.Linear(dim, ffn, bias=False, dtype=dtype)
+        self.mlp.up_proj = nn.Linear(dim, ffn, bias=False, dtype=dtype)
+        self.mlp.down_proj = nn.Linear(ffn, dim, bias=False, dtype=dtype)
+        for lin in (self.self_attn.qkv_proj, self.self_attn.o_proj, self.mlp.gate_proj, self.mlp.up_proj,
+                    self.mlp.down_proj):
+            nn.init.normal_(lin.weight, std=init_std)
+
+    # torch statement of the layer
+    def forward(self, x):
+        Bn, S, Cc = x.shape
+        H, D = self.n_heads, Cc // self.n_heads
+        cos, sin = rope_tables(S, D, self.rope_theta, x.device)
+        h = self.input_layernorm(x)
+        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self.self_attn.qkv_proj(h).split(Cc, dim=-1))
+        q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + self.self_attn.o_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
+        h = self.post_attention_layernorm(x)
+        return x + self.mlp.down_proj(F.silu(self.mlp.gate_proj(h)) * self.mlp.up_proj(h))
+
+    def lower(self, b, x):
+        if x.dim() != 3 or x.shape[-1] != self.dim:
+            raise RuntimeError(f"LlamaLayer of width {self.dim} expects [batch, seq, dim], got {tuple(x.shape)}")
+        Bn, S, Cc = x.shape
+        T, H = Bn * S, self.n_heads
+        D = Cc // H
+        x2d = x.view(T, Cc)
+        cos = b.sp.shared(f"rope_cos:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
+        sin = b.sp.shared(f"rope_sin:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
+        c, s_ = rope_tables(S, D, self.rope_theta, x.device)
+        cos.copy_(c)
+        sin.copy_(s_)
+        n1, rstd1 = lower_rmsnorm(b, "n1", self.input_layernorm, x2d)
+        qkv, _ = lower_linear(b, "qkv", self.self_attn.qkv_proj, n1)
+        b.f(P.op_rope(qkv, cos, sin, S, 2 * H, D))
+        att = b.act("att", (T, Cc))
+        lse = b.act("lse", (Bn, H, S), torch.float32)
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, True))
+        x2, _ = lower_linear(b, "x2", self.self_attn.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
+        n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
+        g, _ = lower_linear(b, "g", self.mlp.gate_proj, n2)
+        u, _ = lower_linear(b, "u", self.mlp.up_proj, n2)
+        h = b.act("h", (T, self.ffn))
+        b.f(P.op_swiglu_fwd(g, u, h))
+        y, _ = lower_linear(b, "y", self.mlp.down_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+
+        def bwd(dy, need_dx, dx_out):
+            dy2d = dy.view(T, Cc)
+            d_h = linear_backward(b, "down", self.mlp.down_proj, h, dy2d)
+            dg = b.grad("dg", (T, self.ffn))
+            du = b.grad("du", (T, self.ffn))
+            b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
+            # the two branches that read n2 add up in the residual epilogue of the second GEMM
+            d_n2a = linear_backward(b, "gate", self.mlp.gate_proj, n2, dg)
+            d_n2 = linear_backward(b, "up", self.mlp.up_proj, n2, du, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+                                   dx_aux=d_n2a)
+            d_x2 = rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+            d_att = linear_backward(b, "o", self.self_attn.o_proj, att, d_x2)
+            dqkv = b.grad("dqkv", (T, 3 * Cc))
+            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
+            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, True,
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            # gradients w.r.t. the rotated q and k go back through the transposed rotation
+            b.i(P.op_rope(dqkv, cos, sin, S, 2 * H, D, inverse=True))
+            d_n1 = linear_backward(b, "qkv", self.self_attn.qkv_proj, n1, dqkv)
+            dx = rmsnorm_backward(b, "n1", self.input_layernorm, x2d, rstd1, d_n1, dres=d_x2,
+                                  dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            return dx.view(Bn, S, Cc)
+
+        b.on_backward(bwd)
+        return y.view(Bn, S, Cc)
+
+
 class LMHead(NativeBlock):
     """Final LayerNorm and the (untied) vocabulary projection.  The weight is stored with its
     vocabulary dimension padded to a multiple of 128 (zero rows) so that logits rows are 256-byte
