@@ -450,3 +450,41 @@ def test_llama_two_stages_1f1b_hand_off_matches_oracle():
     assert_close_rel(out, ref_out, BF16_TOL, "stage output")
     worst = _llama_grads_match(model, ref, losses, ref_losses, ref_out, upstream)
     note(f"Llama layers, two stages: worst grad error {worst:.3e}")
+
+
+def test_llama2_7b_stage_full_size_schedule_and_scaling_invariants():
+    """Config 4 at full size (8 layers, width 4096, 32 heads of 128, SwiGLU 11008, sequence 2048,
+    16 microbatches of one sequence).  Two properties that hold at any size: the zero-bubble schedule
+    (dI and dW as separate passes) accumulates bit-identical gradients to 1F1B, because each
+    parameter receives its microbatch contributions in the same order; and the backward pass is
+    linear in the upstream gradient, so doubling it (exact in binary floating point) doubles every
+    accumulated gradient bit for bit."""
+    import pippy_amd as pp
+    from pippy_amd.configs import llama2_7b_stage
+    torch.manual_seed(0)
+    M = 16
+    with torch.device(DEV):
+        model = llama2_7b_stage()
+        x = torch.randn(M, 2048, 4096).to(torch.bfloat16)
+        upstream = torch.randn(M, 2048, 4096) * 1e-2
+    stage = pp.ManualPipelineStage(model, 0, 1, DEV, M, input_args=(x[:1],))
+    assert stage.is_native
+
+    def grads_after(schedule_cls, up):
+        sched = schedule_cls([stage], M, loss_fn=_upstream_loss)
+        sched.zero_grad()
+        out = sched.step(x, target=up)
+        return out, [p.main_grad.clone() for p in model.layers[0].parameters()] + \
+                    [p.main_grad.clone() for p in model.layers[7].parameters()]
+
+    out_zb, g_zb = grads_after(pp.ScheduleZeroBubble, upstream)
+    assert out_zb.shape == x.shape and torch.isfinite(out_zb.float()).all()
+    assert all(torch.isfinite(g).all() and g.abs().max() > 0 for g in g_zb)
+    out_1f1b, g_1f1b = grads_after(pp.Schedule1F1B, upstream)
+    assert torch.equal(out_zb, out_1f1b)
+    for a, b in zip(g_zb, g_1f1b):
+        assert torch.equal(a, b)
+    del g_1f1b
+    _, g_2x = grads_after(pp.ScheduleZeroBubble, upstream * 2)
+    for a, b in zip(g_zb, g_2x):
+        assert torch.equal(a * 2, b)
