@@ -2,7 +2,7 @@
 
 A stage lowers when it is a chain: its forward applies one lowerable piece after another to a
 single tensor.  Lowerable pieces are the blocks of ``stage_modules`` and the standard torch layers
-``nn.Linear`` (optionally followed by ReLU / GELU) and ``nn.LayerNorm``.  Anything else returns
+``nn.Linear`` (optionally followed by ReLU / GELU), ``nn.LayerNorm`` and ``nn.RMSNorm``.  Anything else returns
 None and the stage runs through torch autograd like the reference does.
 """
 from __future__ import annotations
@@ -15,9 +15,9 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .stage_modules import LayerNormBlock, LinearAct, NativeBlock, StageSequence
+from .stage_modules import LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence
 
-_LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout)
+_LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout)
 
 
 class _ChainTracer(fx.Tracer):
@@ -103,6 +103,10 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
             if len(m.normalized_shape) != 1 or not m.elementwise_affine:
                 return None
             blocks.append(LayerNormBlock(m))
+        elif isinstance(m, nn.RMSNorm):
+            if len(m.normalized_shape) != 1 or m.weight is None or m.eps is None:
+                return None
+            blocks.append(RMSNormBlock(m))
         else:
             # a user container (e.g. a block that wraps a linear and an activation): lower it as
             # a chain of its own and splice the result in

@@ -461,6 +461,29 @@ def rmsnorm_backward(b: "P.Builder", name: str, norm: nn.Module, x2d, rstd, dy2d
     return dx
 
 
+class RMSNormBlock(NativeBlock):
+    """A stand-alone ``nn.RMSNorm`` over the last dimension (the final norm of a Llama-style model)."""
+
+    def __init__(self, norm: nn.Module):
+        super().__init__()
+        self.norm = norm
+
+    def forward(self, x):
+        return self.norm(x)
+
+    def lower(self, b, x):
+        x2d = _as2d(x)
+        y, rstd = lower_rmsnorm(b, "y", self.norm, x2d)
+
+        def bwd(dy, need_dx, dx_out):
+            dx = rmsnorm_backward(b, "rms", self.norm, x2d, rstd, _as2d(dy),
+                                  dx_out=_as2d(dx_out) if dx_out is not None else None)
+            return dx.view(x.shape)
+
+        b.on_backward(bwd)
+        return y.view(x.shape)
+
+
 class LlamaLayer(NativeBlock):
     """One Llama-style decoder layer: RMSNorm, causal self-attention with rotary position embedding
     on a fused q|k|v projection, RMSNorm, SwiGLU feed-forward; no biases.  Parameter names follow the

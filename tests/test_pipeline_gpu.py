@@ -488,3 +488,33 @@ def test_llama2_7b_stage_full_size_schedule_and_scaling_invariants():
     _, g_2x = grads_after(pp.ScheduleZeroBubble, upstream * 2)
     for a, b in zip(g_zb, g_2x):
         assert torch.equal(a * 2, b)
+
+
+def test_llama_last_stage_with_final_rmsnorm_and_head_matches_oracle():
+    """The last stage of a Llama-style pipeline as a user would write it: decoder layers, the final
+    ``nn.RMSNorm`` and a bias-free ``nn.Linear`` head as plain torch layers, cross-entropy loss."""
+    import pippy_amd as pp
+    import torch.nn as nn
+    from pippy_amd.stage_modules import LlamaLayer
+    torch.manual_seed(2)
+    M, S, dim, vocab = 2, 128, 128, 384
+    model = nn.Sequential(LlamaLayer(dim, 2, 256), nn.RMSNorm(dim, eps=1e-5, dtype=torch.bfloat16),
+                          nn.Linear(dim, vocab, bias=False, dtype=torch.bfloat16))
+    with torch.no_grad():
+        model[1].weight.add_(0.1 * torch.randn_like(model[1].weight))
+    ref = _fp32_cpu_copy(model)
+    x = torch.randn(2 * M, S, dim).to(torch.bfloat16)
+    target = torch.randint(0, vocab, (2 * M, S))
+    stage = pp.ManualPipelineStage(model, 0, 1, DEV, M, input_args=(x[:2].to(DEV),))
+    assert stage.is_native
+    sched = pp.Schedule1F1B([stage], M, loss_fn=_ce)
+    losses = []
+    out = sched.step(x.to(DEV), target=target.to(DEV), losses=losses)
+    ref_out, ref_losses = OP.step([ref], x.float(), target, M, _ce)
+    assert_close_rel(out, ref_out, BF16_TOL, "logits")
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.detach().reshape(1), b.detach().reshape(1), BF16_TOL, "loss")
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        err = max_rel(named[name].main_grad, rp.grad)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
