@@ -152,6 +152,24 @@ int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
 #define PP_GEMM_MAX_GROUP 16
 int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream);
 
+/* One GEMM per segment of a row-partitioned operand, with the segment bounds in DEVICE memory:
+ * seg_start[0 .. n_seg] ascending row indices (int32), read by the kernel, so that sizes produced on
+ * the device (the token counts of the experts of a mixture-of-experts layer, which the reference
+ * would reach as one F.linear per expert inside the stage module, pippy/_PipelineStage.py:420-428)
+ * never travel to the host.  seg_ptr[0 .. n_seg) is a device array of device pointers.
+ *   PP_SEG_ROWS: for every segment e,  C[r0:r1, :] = epilogue(A[r0:r1, :] * B_e^T)  with
+ *     B_e = seg_ptr[e] ([N, K], ldb), r0 = seg_start[e], r1 = seg_start[e + 1]; desc->M is the total
+ *     row count (an upper bound for the grid), desc->B is ignored; a_trans = b_trans = 0, bf16 C,
+ *     epilogue NONE or BIAS_RESIDUAL with a null bias (C = A B^T + aux_in, rows as in C).
+ *   PP_SEG_K: for every segment e,  C_e = A[r0:r1, :]^T * B[r0:r1, :]  with C_e = seg_ptr[e]
+ *     ([M, N], ldc): the weight gradient of expert e; desc->K is the total row count, desc->C is
+ *     ignored; a_trans = b_trans = 1; bf16 C with NONE (an empty segment writes zeros) or fp32 C
+ *     with ACCUM_F32 / beta. */
+enum pp_gemm_seg_mode { PP_SEG_ROWS = 0, PP_SEG_K = 1 };
+#define PP_GEMM_MAX_SEGMENTS 1024
+int pp_gemm_bf16_segmented(const pp_gemm_desc* desc, const int32_t* seg_start, const void* const* seg_ptr,
+                           int n_seg, int mode, pp_stream stream);
+
 /* fp32 GEMM with the same descriptor (A, B, C, bias, aux fp32; config 1 of the baseline, the
  * README MLP).  Only a_trans / b_trans, NONE, BIAS, BIAS_RELU, DRELU and ACCUM_F32 epilogues. */
 int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
@@ -189,6 +207,42 @@ int pp_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* 
                   pp_stream stream);
 int pp_rope(void* x, const float* cos_table, const float* sin_table, int64_t n_tok, int64_t seq,
             int64_t n_heads, int64_t D, int64_t ld, int inverse, pp_stream stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Routing of a top-2 mixture-of-experts layer (a Mixtral-style block inside the stage module;
+ * forward through pippy/_PipelineStage.py:420-428, backward through pippy/_backward.py:67-69).
+ * T tokens, E experts, topk slots per token; flat slot f = t * topk + k; permuted rows are grouped
+ * by expert and ordered by ascending f inside an expert.  All index arrays are int32 in device
+ * memory; nothing is read back by the host.
+ *   pp_moe_router_top2: logits bf16 [T, ld] -> topk_idx [T, 2] (the two largest logits, the lower
+ *     expert index winning a tie) and gate fp32 [T, 2] = softmax over all experts renormalised
+ *     over the selected pair.
+ *   pp_moe_permute: expert_of_slot [n_slots] -> seg_start [E + 1] (first row of every expert;
+ *     seg_start[E] = rows placed), row_src [n_slots] (flat slot of every row), pos [n_slots] (row
+ *     of every flat slot; -1 and dropped for an expert id outside [0, E)).  E <= 64.
+ *   pp_moe_gather: dst[r, :] = scale[f] * src[f / topk, :] with f = row_src[r] for r < *n_rows_dev
+ *     (null: r < R); scale null = plain gather.  Tokens -> expert rows, and the weighted
+ *     scatter of the output gradient in the backward pass.
+ *   pp_moe_combine: out[t, :] = resid[t, :] + sum_k gate[f] * y[pos[f], :] (resid, gate optional),
+ *     fp32 sum with one rounding.  Expert rows -> tokens, and the sum of the expert input
+ *     gradients in the backward pass.
+ *   pp_moe_gate_bwd: dlogits bf16 [T, ld_dl]: gradient of the loss w.r.t. the router logits given
+ *     dout [T, C] and the expert outputs y [rows, C]; zero for experts that were not selected.
+ * bf16 rows: 16-byte aligned, leading dimensions and C multiples of 8.
+ * ---------------------------------------------------------------------------------------- */
+int pp_moe_router_top2(const void* logits, int64_t ld, int64_t T, int E, int32_t* topk_idx, float* gate,
+                       pp_stream stream);
+int pp_moe_permute(const int32_t* expert_of_slot, int64_t n_slots, int E, int32_t* seg_start,
+                   int32_t* row_src, int32_t* pos, pp_stream stream);
+int pp_moe_gather(const void* src, int64_t ld_src, const int32_t* row_src, const int32_t* n_rows_dev,
+                  int topk, const float* scale, void* dst, int64_t ld_dst, int64_t R, int64_t C,
+                  pp_stream stream);
+int pp_moe_combine(const void* y, int64_t ld_y, const int32_t* pos, const float* gate, int topk,
+                   const void* resid, int64_t ld_resid, void* out, int64_t ld_out, int64_t T, int64_t C,
+                   pp_stream stream);
+int pp_moe_gate_bwd(const void* dout, int64_t ld_dout, const void* y, int64_t ld_y, const int32_t* pos,
+                    const int32_t* topk_idx, const float* gate, int topk, int E, void* dlogits,
+                    int64_t ld_dl, int64_t T, int64_t C, pp_stream stream);
 
 /* Column reductions of one weight-gradient pass in two launches.  Per descriptor:
  *   out_sum[c] = sum_r dy[r, c]                                   (bias gradient / dbeta), and, if
@@ -282,7 +336,9 @@ enum pp_op_kind {
     PP_OP_LN_BWD_INPUT = 5, PP_OP_LN_BWD_WEIGHT = 6, PP_OP_ATTN_FWD = 7, PP_OP_ATTN_BWD = 8,
     PP_OP_EMBED_FWD = 9, PP_OP_EMBED_BWD = 10, PP_OP_CE_LOSS = 11, PP_OP_ACCUM_BF16 = 12,
     PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16,
-    PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19
+    PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
+    PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
+    PP_OP_MOE_GATE_BWD = 25
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -304,6 +360,12 @@ enum pp_op_kind {
  *   SWIGLU_FWD    p: g u h | i: n
  *   SWIGLU_BWD    p: g u dh dg du | i: n
  *   ROPE          p: x cos sin | i: n_tok seq n_heads D ld | j: inverse
+ *   GEMM_SEG      as GEMM_BF16, and p[6]: seg_start p[7]: seg_ptr | i[7]: n_seg | j[5]: mode
+ *   MOE_ROUTER    p: logits topk_idx gate | i: ld T E
+ *   MOE_PERMUTE   p: expert_of_slot seg_start row_src pos | i: n_slots E
+ *   MOE_GATHER    p: src row_src n_rows_dev scale dst | i: ld_src topk ld_dst R C
+ *   MOE_COMBINE   p: y pos gate resid out | i: ld_y topk ld_resid ld_out T C
+ *   MOE_GATE_BWD  p: dout y pos topk_idx gate dlogits | i: ld_dout ld_y topk E ld_dl T C
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped

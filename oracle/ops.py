@@ -9,7 +9,9 @@ Pinning: every function here is a direct torch library routine or a closed form 
 one in tests/test_oracle.py (gelu closed forms vs F.gelu, attention vs
 F.scaled_dot_product_attention, layer norm vs F.layer_norm, cross entropy vs F.cross_entropy,
 rms norm vs F.rms_norm, silu vs F.silu, the rotary embedding vs a complex-number rotation and its
-norm / relative-position invariants).
+norm / relative-position invariants; top-2 routing vs torch.topk on tie-free logits, the expert
+permutation vs a stable argsort, the sparse mixture-of-experts layer vs the dense sum over all
+experts with zero weight for the experts not selected).
 """
 import math
 
@@ -95,4 +97,49 @@ def embedding(ids, wte, wpe=None):
     if wpe is not None:
         S = ids.shape[-1]
         y = y + wpe[:S]
+    return y
+
+
+# ---- top-2 mixture of experts (Mixtral-style block) -------------------------------------------
+def moe_route_top2(logits):
+    """Softmax over all experts, the two largest probabilities (the lower expert index wins a tie),
+    renormalised to sum to one.  Returns (idx int64 [T, 2], gate fp32 [T, 2], first slot = largest)."""
+    probs = torch.softmax(logits.float(), dim=-1)
+    # a stable descending sort keeps the lower index first among equal values
+    order = torch.sort(probs, dim=-1, descending=True, stable=True).indices
+    idx = order[:, :2]
+    top = probs.gather(-1, idx)
+    return idx, top / top.sum(-1, keepdim=True)
+
+
+def moe_permutation(expert_of_slot, E):
+    """Rows grouped by expert, ascending flat slot inside an expert.  Returns (seg_start [E + 1],
+    row_src [n], pos [n]) as int64 tensors."""
+    flat = expert_of_slot.reshape(-1).long()
+    row_src = torch.sort(flat, stable=True).indices
+    pos = torch.empty_like(row_src)
+    pos[row_src] = torch.arange(flat.numel())
+    counts = torch.bincount(flat, minlength=E)
+    seg_start = torch.cat([torch.zeros(1, dtype=torch.long), counts.cumsum(0)])
+    return seg_start, row_src, pos
+
+
+def moe_top2(x, w_router, w1, w2, w3, idx=None):
+    """y[t] = sum over the two selected experts e of gate[t, e] * w2_e (silu(w1_e x[t]) * (w3_e x[t])).
+    ``w1, w3`` [E, ffn, d], ``w2`` [E, d, ffn], ``w_router`` [E, d].  ``idx`` ([T, 2]) forces the
+    selection (the weights are then the renormalised probabilities of the forced pair)."""
+    logits = F.linear(x, w_router)
+    if idx is None:
+        idx, gate = moe_route_top2(logits)
+    else:
+        top = torch.softmax(logits.float(), dim=-1).gather(-1, idx)
+        gate = top / top.sum(-1, keepdim=True)
+    y = torch.zeros_like(x)
+    for e in range(w1.shape[0]):
+        tok, slot = torch.where(idx == e)
+        if tok.numel() == 0:
+            continue
+        xe = x[tok]
+        ye = F.linear(swiglu(F.linear(xe, w1[e]), F.linear(xe, w3[e])), w2[e])
+        y = y.index_add(0, tok, gate[tok, slot, None] * ye)
     return y

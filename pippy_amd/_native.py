@@ -23,7 +23,9 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7
 # enum pp_op_kind
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
- OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE) = range(1, 20)
+ OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
+ OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD) = range(1, 26)
+SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
 ACT_RELU, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
@@ -38,6 +40,8 @@ EXPORTED_SYMBOLS = (
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
+    "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
+    "pp_moe_gate_bwd",
 )
 
 
@@ -128,6 +132,12 @@ def lib() -> C.CDLL:
         "pp_swiglu_fwd": [vp, vp, vp, i64, vp],
         "pp_swiglu_bwd": [vp, vp, vp, vp, vp, i64, vp],
         "pp_rope": [vp, vp, vp, i64, i64, i64, i64, i64, i32, vp],
+        "pp_gemm_bf16_segmented": [C.POINTER(GemmDesc), vp, vp, i32, i32, vp],
+        "pp_moe_router_top2": [vp, i64, i64, i32, vp, vp, vp],
+        "pp_moe_permute": [vp, i64, i32, vp, vp, vp, vp],
+        "pp_moe_gather": [vp, i64, vp, vp, i32, vp, vp, i64, i64, i64, vp],
+        "pp_moe_combine": [vp, i64, vp, vp, i32, vp, i64, vp, i64, i64, i64, vp],
+        "pp_moe_gate_bwd": [vp, i64, vp, i64, vp, vp, vp, i32, i32, vp, i64, i64, i64, vp],
         "pp_sgd_step": [vp, i32, vp, vp, vp, i64, f32, f32, f32, f32, i32, i32, i32, vp],
         "pp_adamw_step": [vp, i32, vp, vp, vp, vp, i64, f32, f32, f32, f32, f32, f32, f32, i32, vp],
     }
@@ -291,6 +301,95 @@ def rope(x2d, cos, sin, seq: int, n_heads: int, D: int, inverse: bool = False) -
     assert cos.shape == sin.shape == (seq, D // 2) and cos.is_contiguous() and sin.is_contiguous()
     check(lib().pp_rope(x2d.data_ptr(), cos.data_ptr(), sin.data_ptr(), x2d.shape[0], seq, n_heads, D,
                         x2d.stride(0), int(inverse), current_stream()), "pp_rope")
+
+
+# ---- mixture-of-experts routing and segmented GEMMs ---------------------------------------------
+def gemm_bf16_segmented(A, B_or_C_list: torch.Tensor, Cm, seg_start: torch.Tensor, mode: int, *, other=None,
+                        N: Optional[int] = None, ld: Optional[int] = None, epilogue: int = EPI_NONE,
+                        aux_in=None, beta: int = 0, c_dtype=None) -> None:
+    """Segmented GEMM (see ``pp_gemm_bf16_segmented``).
+
+    rows mode: ``A`` [R, K], ``Cm`` [R, N]; ``B_or_C_list`` is an int64 device tensor of per-segment B
+    pointers ([N, K] each, leading dimension ``ld``).
+    k mode: ``A`` [R, M] and ``other`` [R, N] are the transposed operands; ``B_or_C_list`` holds the
+    per-segment C pointers ([M, N], leading dimension ``ld``, dtype ``c_dtype``); ``Cm`` is None."""
+    require_cuda(A, B_or_C_list, seg_start, Cm, other, aux_in)
+    assert seg_start.dtype == torch.int32 and B_or_C_list.dtype == torch.int64
+    n_seg = seg_start.numel() - 1
+    assert B_or_C_list.numel() == n_seg
+    d = GemmDesc()
+    if mode == SEG_ROWS:
+        assert A.stride(1) == 1 and Cm.stride(1) == 1 and A.shape[0] == Cm.shape[0]
+        d.A, d.B, d.C = A.data_ptr(), None, Cm.data_ptr()
+        d.M, d.N, d.K = A.shape[0], Cm.shape[1], A.shape[1]
+        d.lda, d.ldb, d.ldc = A.stride(0), ld if ld is not None else A.shape[1], Cm.stride(0)
+        d.a_trans = d.b_trans = 0
+        d.c_dtype = PP_BF16
+        if aux_in is not None:
+            assert aux_in.shape == Cm.shape and aux_in.stride(1) == 1
+            d.aux_in, d.ld_aux = aux_in.data_ptr(), aux_in.stride(0)
+    else:
+        assert other is not None and A.shape[0] == other.shape[0] and A.stride(1) == 1 and other.stride(1) == 1
+        d.A, d.B, d.C = A.data_ptr(), other.data_ptr(), None
+        d.M, d.N, d.K = A.shape[1], other.shape[1], A.shape[0]
+        d.lda, d.ldb, d.ldc = A.stride(0), other.stride(0), ld if ld is not None else other.shape[1]
+        d.a_trans = d.b_trans = 1
+        d.c_dtype = PP_F32 if c_dtype == torch.float32 else PP_BF16
+    d.epilogue, d.beta = epilogue, beta
+    check(lib().pp_gemm_bf16_segmented(C.byref(d), seg_start.data_ptr(), B_or_C_list.data_ptr(), n_seg, mode,
+                                       current_stream()), "pp_gemm_bf16_segmented")
+
+
+def moe_router_top2(logits, topk_idx, gate) -> None:
+    require_cuda(logits, topk_idx, gate)
+    T, E = logits.shape
+    assert logits.dtype == torch.bfloat16 and logits.stride(1) == 1
+    assert topk_idx.dtype == torch.int32 and topk_idx.is_contiguous() and topk_idx.numel() == 2 * T
+    assert gate.dtype == torch.float32 and gate.is_contiguous() and gate.numel() == 2 * T
+    check(lib().pp_moe_router_top2(logits.data_ptr(), logits.stride(0), T, E, topk_idx.data_ptr(), gate.data_ptr(),
+                                   current_stream()), "pp_moe_router_top2")
+
+
+def moe_permute(expert_of_slot, E: int, seg_start, row_src, pos) -> None:
+    require_cuda(expert_of_slot, seg_start, row_src, pos)
+    n = expert_of_slot.numel()
+    for t in (expert_of_slot, seg_start, row_src, pos):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert seg_start.numel() == E + 1 and row_src.numel() == n and pos.numel() == n
+    check(lib().pp_moe_permute(expert_of_slot.data_ptr(), n, E, seg_start.data_ptr(), row_src.data_ptr(),
+                               pos.data_ptr(), current_stream()), "pp_moe_permute")
+
+
+def moe_gather(src, row_src, topk: int, dst, *, scale=None, n_rows=None) -> None:
+    require_cuda(src, row_src, dst, scale, n_rows)
+    assert src.stride(1) == 1 and dst.stride(1) == 1 and src.shape[1] == dst.shape[1]
+    assert row_src.dtype == torch.int32 and row_src.numel() == dst.shape[0]
+    assert scale is None or (scale.dtype == torch.float32 and scale.is_contiguous())
+    check(lib().pp_moe_gather(src.data_ptr(), src.stride(0), row_src.data_ptr(), _p_or_none(n_rows), topk,
+                              _p_or_none(scale), dst.data_ptr(), dst.stride(0), dst.shape[0], dst.shape[1],
+                              current_stream()), "pp_moe_gather")
+
+
+def moe_combine(y, pos, topk: int, out, *, gate=None, resid=None) -> None:
+    require_cuda(y, pos, out, gate, resid)
+    T, Cc = out.shape
+    assert y.stride(1) == 1 and out.stride(1) == 1 and y.shape[1] == Cc
+    assert pos.dtype == torch.int32 and pos.numel() == T * topk
+    assert gate is None or (gate.dtype == torch.float32 and gate.is_contiguous() and gate.numel() == T * topk)
+    assert resid is None or (resid.shape == out.shape and resid.stride(1) == 1)
+    check(lib().pp_moe_combine(y.data_ptr(), y.stride(0), pos.data_ptr(), _p_or_none(gate), topk,
+                               _p_or_none(resid), resid.stride(0) if resid is not None else 0, out.data_ptr(),
+                               out.stride(0), T, Cc, current_stream()), "pp_moe_combine")
+
+
+def moe_gate_bwd(dout, y, pos, topk_idx, gate, E: int, dlogits) -> None:
+    require_cuda(dout, y, pos, topk_idx, gate, dlogits)
+    T, Cc = dout.shape
+    topk = pos.numel() // T
+    assert dlogits.shape == (T, E) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
+    check(lib().pp_moe_gate_bwd(dout.data_ptr(), dout.stride(0), y.data_ptr(), y.stride(0), pos.data_ptr(),
+                                topk_idx.data_ptr(), gate.data_ptr(), topk, E, dlogits.data_ptr(),
+                                dlogits.stride(0), T, Cc, current_stream()), "pp_moe_gate_bwd")
 
 
 def fill_bytes(t: torch.Tensor, value: int = 0) -> None:

@@ -213,6 +213,102 @@ def op_rope(x2d, cos, sin, seq, n_heads, D, inverse=False) -> N.Op:
     return op
 
 
+def op_gemm_seg(mode, A, ptr_list, seg_start, *, Cm=None, other=None, n_cols=None, ld=None,
+                epilogue=N.EPI_NONE, aux_in=None, beta=0, c_f32=False) -> N.Op:
+    """Segmented GEMM over the expert segments of permuted rows (sizes read on the device).
+    rows mode: Cm[r0:r1] = A[r0:r1] B_e^T (+ aux_in), B_e [n_cols = Cm.shape[1], K] with leading
+    dimension ``ld`` from ``ptr_list``.  k mode: C_e = A[r0:r1]^T other[r0:r1], C_e [A.shape[1],
+    other.shape[1]] with leading dimension ``ld`` from ``ptr_list``."""
+    assert seg_start.dtype == torch.int32 and ptr_list.dtype == torch.int64
+    assert ptr_list.numel() == seg_start.numel() - 1
+    op = N.Op()
+    op.kind = N.OP_GEMM_SEG
+    if mode == N.SEG_ROWS:
+        assert A.stride(1) == 1 and Cm.stride(1) == 1 and A.shape[0] == Cm.shape[0]
+        assert A.dtype == torch.bfloat16 and Cm.dtype == torch.bfloat16
+        op.p[0], op.p[1], op.p[2] = A.data_ptr(), None, Cm.data_ptr()
+        op.i[0], op.i[1], op.i[2] = A.shape[0], Cm.shape[1], A.shape[1]
+        op.i[3], op.i[4], op.i[5] = A.stride(0), ld if ld is not None else A.shape[1], Cm.stride(0)
+        if aux_in is not None:
+            assert aux_in.shape == Cm.shape and aux_in.stride(1) == 1
+            op.p[4], op.i[6] = aux_in.data_ptr(), aux_in.stride(0)
+        op.j[0], op.j[1], op.j[3] = 0, 0, N.PP_BF16
+    else:
+        assert A.stride(1) == 1 and other.stride(1) == 1 and A.shape[0] == other.shape[0]
+        op.p[0], op.p[1], op.p[2] = A.data_ptr(), other.data_ptr(), None
+        op.i[0], op.i[1], op.i[2] = A.shape[1], other.shape[1], A.shape[0]
+        op.i[3], op.i[4], op.i[5] = A.stride(0), other.stride(0), ld if ld is not None else other.shape[1]
+        op.j[0], op.j[1], op.j[3] = 1, 1, N.PP_F32 if c_f32 else N.PP_BF16
+    op.j[2], op.j[4], op.j[5] = epilogue, beta, mode
+    op.p[6], op.p[7] = seg_start.data_ptr(), ptr_list.data_ptr()
+    op.i[7] = ptr_list.numel()
+    return op
+
+
+def op_moe_router(logits, topk_idx, gate) -> N.Op:
+    T, E = logits.shape
+    assert logits.dtype == torch.bfloat16 and logits.stride(1) == 1
+    assert topk_idx.dtype == torch.int32 and topk_idx.numel() == 2 * T and topk_idx.is_contiguous()
+    assert gate.dtype == torch.float32 and gate.numel() == 2 * T and gate.is_contiguous()
+    op = N.Op()
+    op.kind = N.OP_MOE_ROUTER
+    op.p[0], op.p[1], op.p[2] = logits.data_ptr(), topk_idx.data_ptr(), gate.data_ptr()
+    op.i[0], op.i[1], op.i[2] = logits.stride(0), T, E
+    return op
+
+
+def op_moe_permute(expert_of_slot, E, seg_start, row_src, pos) -> N.Op:
+    n = expert_of_slot.numel()
+    for t in (expert_of_slot, seg_start, row_src, pos):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert seg_start.numel() == E + 1 and row_src.numel() == n and pos.numel() == n
+    op = N.Op()
+    op.kind = N.OP_MOE_PERMUTE
+    op.p[0], op.p[1], op.p[2], op.p[3] = (expert_of_slot.data_ptr(), seg_start.data_ptr(), row_src.data_ptr(),
+                                          pos.data_ptr())
+    op.i[0], op.i[1] = n, E
+    return op
+
+
+def op_moe_gather(src, row_src, topk, dst, scale=None, n_rows=None) -> N.Op:
+    assert src.stride(1) == 1 and dst.stride(1) == 1 and src.shape[1] == dst.shape[1]
+    assert row_src.dtype == torch.int32 and row_src.numel() == dst.shape[0]
+    assert scale is None or (scale.dtype == torch.float32 and scale.is_contiguous())
+    op = N.Op()
+    op.kind = N.OP_MOE_GATHER
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = src.data_ptr(), row_src.data_ptr(), _p(n_rows), _p(scale), dst.data_ptr()
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4] = src.stride(0), topk, dst.stride(0), dst.shape[0], dst.shape[1]
+    return op
+
+
+def op_moe_combine(y, pos, topk, out, gate=None, resid=None) -> N.Op:
+    T, Cc = out.shape
+    assert y.stride(1) == 1 and out.stride(1) == 1 and y.shape[1] == Cc
+    assert pos.dtype == torch.int32 and pos.numel() == T * topk
+    assert gate is None or (gate.dtype == torch.float32 and gate.numel() == T * topk and gate.is_contiguous())
+    assert resid is None or (resid.shape == out.shape and resid.stride(1) == 1)
+    op = N.Op()
+    op.kind = N.OP_MOE_COMBINE
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = y.data_ptr(), pos.data_ptr(), _p(gate), _p(resid), out.data_ptr()
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5] = (y.stride(0), topk, resid.stride(0) if resid is not None else 0,
+                                                          out.stride(0), T, Cc)
+    return op
+
+
+def op_moe_gate_bwd(dout, y, pos, topk_idx, gate, E, dlogits) -> N.Op:
+    T, Cc = dout.shape
+    topk = pos.numel() // T
+    assert dlogits.shape == (T, E) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
+    assert dout.stride(1) == 1 and y.stride(1) == 1 and y.shape[1] == Cc
+    op = N.Op()
+    op.kind = N.OP_MOE_GATE_BWD
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = (dout.data_ptr(), y.data_ptr(), pos.data_ptr(),
+                                                          topk_idx.data_ptr(), gate.data_ptr(), dlogits.data_ptr())
+    op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5], op.i[6] = (dout.stride(0), y.stride(0), topk, E,
+                                                                     dlogits.stride(0), T, Cc)
+    return op
+
+
 def op_ln_fwd(x, gamma, beta, y, mean, rstd, eps) -> N.Op:
     rows, Cc = x.shape
     assert x.is_contiguous() and y.is_contiguous() and y.shape == x.shape

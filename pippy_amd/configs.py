@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .stage_modules import EncoderEmbedding, LlamaLayer, LMHead, TokenEmbedding, TransformerLayer
+from .stage_modules import EncoderEmbedding, LlamaLayer, LMHead, MoELayer, TokenEmbedding, TransformerLayer
 
 
 class DecoderLM(nn.Module):
@@ -81,6 +81,33 @@ class LlamaStage(nn.Module):
 def llama2_7b_stage(dtype=torch.bfloat16) -> LlamaStage:
     """8 of the 32 layers of a Llama-2-7B-shaped model: width 4096, 32 heads of 128, SwiGLU 11008."""
     return LlamaStage(dtype=dtype)
+
+
+class MoEDecoderLM(nn.Module):
+    """Mixtral-shaped decoder: token embedding (positions enter through the rotary embedding),
+    decoder layers whose feed-forward is a top-2 mixture of SwiGLU experts, final RMSNorm and an
+    untied vocabulary projection."""
+
+    def __init__(self, vocab=32000, dim=1024, n_layers=8, n_heads=16, ffn=4096, n_experts=8,
+                 dtype=torch.bfloat16, eps=1e-5, rope_theta=1e6):
+        super().__init__()
+        self.embed = TokenEmbedding(vocab, 0, dim, dtype=dtype, positions=False)
+        self.h = nn.ModuleList([
+            MoELayer(dim, n_heads, ffn, n_experts, eps=eps, rope_theta=rope_theta, dtype=dtype)
+            for _ in range(n_layers)])
+        self.head = LMHead(dim, vocab, final_ln="rms", eps=eps, dtype=dtype)
+
+    def forward(self, ids):
+        x = self.embed(ids)
+        for layer in self.h:
+            x = layer(x)
+        return self.head(x)
+
+
+def mixtral_style(dtype=torch.bfloat16) -> MoEDecoderLM:
+    """8 layers (2 stages of 4), width 1024, 16 heads of 64, 8 experts with SwiGLU 4096, top-2 router,
+    vocabulary 32000."""
+    return MoEDecoderLM(dtype=dtype)
 
 
 def equal_split_spec(n_layers: int, n_stages: int, prefix: str = "h"):

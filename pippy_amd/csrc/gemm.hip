@@ -370,6 +370,72 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const Gem
     gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32>(g, tile_m, tile_n);
 }
 
+// Segmented problems: the rows of one operand are partitioned into consecutive segments whose
+// bounds seg_start[0 .. n_seg] live in device memory (the token counts of the experts of a
+// mixture-of-experts layer), so the sizes are only known on the device and the grid is an upper
+// bound.
+//   rows mode: segment e is the GEMM of rows [seg_start[e], seg_start[e+1]) of A (and of C and the
+//              auxiliary tensors) with its own B = seg_ptr[e];
+//   k mode:    segment e reduces over k-rows [seg_start[e], seg_start[e+1]) of transposed A and B
+//              into its own C = seg_ptr[e] (an empty segment writes zeros / adds nothing).
+struct GemmSegArgs {
+    GemmArgs g;  // rows mode: M = total rows, B unused;  k mode: K = total rows, C unused
+    const int32_t* seg_start;
+    const void* const* seg_ptr;
+    int n_seg;
+};
+
+template <int BM, int BN, int NS, int EPI>
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_rows_kernel(const GemmSegArgs sa) {
+    // tiles of every segment, then an XCD-contiguous numbering of exactly that many ids
+    uint32_t total = 0;
+    for (int e = 0; e < sa.n_seg; ++e)
+        total += (uint32_t)((sa.seg_start[e + 1] - sa.seg_start[e] + BM - 1) / BM) * sa.g.tiles_n;
+    const uint32_t total8 = (total + 7) & ~7u;
+    if (blockIdx.x >= total8) return;
+    uint32_t bid = xcd_remap(blockIdx.x, total8);
+    if (bid >= total) return;
+    int e = 0;
+    int32_t r0 = sa.seg_start[0], r1 = r0;
+    uint32_t tiles_m = 0;
+    for (; e < sa.n_seg; ++e) {
+        r1 = sa.seg_start[e + 1];
+        tiles_m = (uint32_t)((r1 - r0 + BM - 1) / BM);
+        const uint32_t nt = tiles_m * sa.g.tiles_n;
+        if (bid < nt) break;
+        bid -= nt;
+        r0 = r1;
+    }
+    GemmArgs g = sa.g;
+    g.M = r1 - r0;
+    g.A += (int64_t)r0 * g.lda;
+    g.B = static_cast<const uint16_t*>(sa.seg_ptr[e]);
+    g.C = static_cast<uint16_t*>(g.C) + (int64_t)r0 * g.ldc;
+    if (g.aux_in) g.aux_in += (int64_t)r0 * g.ld_aux;
+    if (g.aux_out) g.aux_out += (int64_t)r0 * g.ld_aux;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, tiles_m, g.tiles_n, &tile_m, &tile_n);
+    gemm_tile_dma<BM, BN, false, false, NS, EPI, false>(g, tile_m, tile_n);
+}
+
+template <int BM, int BN, int NS, int EPI, bool CF32>
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_k_kernel(const GemmSegArgs sa) {
+    uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    const uint32_t per_seg = sa.g.tiles_m * sa.g.tiles_n;
+    if (bid >= per_seg * (uint32_t)sa.n_seg) return;
+    const int e = (int)(bid / per_seg);
+    bid -= (uint32_t)e * per_seg;
+    const int32_t r0 = sa.seg_start[e], r1 = sa.seg_start[e + 1];
+    GemmArgs g = sa.g;
+    g.K = r1 - r0;
+    g.A += (int64_t)r0 * g.lda;
+    g.B += (int64_t)r0 * g.ldb;
+    g.C = const_cast<void*>(sa.seg_ptr[e]);
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    gemm_tile_dma<BM, BN, true, true, NS, EPI, CF32>(g, tile_m, tile_n);
+}
+
 template <typename Kernel>
 static int reserve_lds(Kernel kernel, size_t lds) {
     const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -534,9 +600,84 @@ static int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
     return PP_OK;
 }
 
+template <int EPI>
+static int launch_seg_rows(GemmSegArgs& sa, hipStream_t st) {
+    constexpr int BM = 128, BN = 128, NS = 2;
+    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_seg_rows_kernel<BM, BN, NS, EPI>, lds);
+    if (attr_rc) return attr_rc;
+    sa.g.tiles_n = (uint32_t)((sa.g.N + BN - 1) / BN);
+    // every segment may end in a partly filled tile row
+    const uint64_t bound = ((uint64_t)(sa.g.M + BM - 1) / BM + (uint64_t)sa.n_seg) * sa.g.tiles_n;
+    if (bound > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: too many tiles");
+    const uint32_t grid = ((uint32_t)bound + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_seg_rows_kernel<BM, BN, NS, EPI>), dim3(grid), dim3(kGemmThreads), lds, st, sa);
+    return check_launch("gemm_bf16_seg_rows_kernel");
+}
+
+template <int EPI, bool CF32>
+static int launch_seg_k(GemmSegArgs& sa, hipStream_t st) {
+    constexpr int BM = 128, BN = 128, NS = 2;
+    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_seg_k_kernel<BM, BN, NS, EPI, CF32>, lds);
+    if (attr_rc) return attr_rc;
+    int rc = count_tiles<BM, BN>(sa.g);
+    if (rc) return rc;
+    const uint64_t total = (uint64_t)sa.g.n_blocks * (uint64_t)sa.n_seg;
+    if (total > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: too many tiles");
+    const uint32_t grid = ((uint32_t)total + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_seg_k_kernel<BM, BN, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads), lds, st, sa);
+    return check_launch("gemm_bf16_seg_k_kernel");
+}
+
 }  // namespace pp
 
 using namespace pp;
+
+extern "C" int pp_gemm_bf16_segmented(const pp_gemm_desc* d, const int32_t* seg_start,
+                                      const void* const* seg_ptr, int n_seg, int mode, pp_stream stream) {
+    if (!d || !seg_start || !seg_ptr || n_seg < 1 || n_seg > PP_GEMM_MAX_SEGMENTS)
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16_segmented: bad segment list (n_seg=%d)", n_seg);
+    if (mode != PP_SEG_ROWS && mode != PP_SEG_K)
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16_segmented: unknown mode %d", mode);
+    // the operand that every segment brings itself is checked on its first use only for null here:
+    // its pointers live in device memory
+    pp_gemm_desc dd = *d;
+    if (mode == PP_SEG_ROWS) {
+        if (dd.a_trans || dd.b_trans)
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: rows mode takes k-contiguous A and B");
+        if (dd.epilogue != PP_EPI_NONE && dd.epilogue != PP_EPI_BIAS_RESIDUAL)
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: rows mode epilogue %d", dd.epilogue);
+        if (dd.c_dtype != PP_BF16) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: rows mode writes bf16");
+        if (dd.bias) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: no bias");
+        dd.B = dd.A;  // placeholder that passes the checks; the kernel takes B from seg_ptr
+    } else {
+        if (!dd.a_trans || !dd.b_trans)
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: k mode takes transposed A and B");
+        if (!((dd.epilogue == PP_EPI_NONE && dd.c_dtype == PP_BF16) ||
+              (dd.epilogue == PP_EPI_ACCUM_F32 && dd.c_dtype == PP_F32)))
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: k mode writes bf16 or accumulates into fp32");
+        dd.C = const_cast<void*>(dd.A);
+        dd.K = (dd.K + 7) & ~(int64_t)7;  // the reduction length of a segment need not be a multiple of 8
+    }
+    GemmSegArgs sa;
+    bool empty;
+    int rc = convert(&dd, &sa.g, &empty);
+    if (rc || empty) return rc;
+    sa.g.K = (mode == PP_SEG_K) ? d->K : sa.g.K;
+    sa.seg_start = seg_start;
+    sa.seg_ptr = seg_ptr;
+    sa.n_seg = n_seg;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mode == PP_SEG_ROWS) {
+        sa.g.B = nullptr;
+        return dd.epilogue == PP_EPI_NONE ? launch_seg_rows<PP_EPI_NONE>(sa, st)
+                                          : launch_seg_rows<PP_EPI_BIAS_RESIDUAL>(sa, st);
+    }
+    sa.g.C = nullptr;
+    return dd.c_dtype == PP_F32 ? launch_seg_k<PP_EPI_ACCUM_F32, true>(sa, st)
+                                : launch_seg_k<PP_EPI_NONE, false>(sa, st);
+}
 
 extern "C" int pp_gemm_bf16(const pp_gemm_desc* d, pp_stream stream) {
     GemmArgs g;

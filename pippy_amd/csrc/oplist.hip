@@ -127,6 +127,30 @@ static int run_one(const pp_op& op, pp_stream st) {
         case PP_OP_ROPE:
             return pp_rope(op.p[0], static_cast<const float*>(op.p[1]), static_cast<const float*>(op.p[2]),
                            op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.j[0], st);
+        case PP_OP_GEMM_SEG: {
+            const pp_gemm_desc d = gemm_desc_of(op);
+            return pp_gemm_bf16_segmented(&d, static_cast<const int32_t*>(op.p[6]),
+                                          static_cast<const void* const*>(op.p[7]), (int)op.i[7], op.j[5], st);
+        }
+        case PP_OP_MOE_ROUTER:
+            return pp_moe_router_top2(op.p[0], op.i[0], op.i[1], (int)op.i[2], static_cast<int32_t*>(op.p[1]),
+                                      static_cast<float*>(op.p[2]), st);
+        case PP_OP_MOE_PERMUTE:
+            return pp_moe_permute(static_cast<const int32_t*>(op.p[0]), op.i[0], (int)op.i[1],
+                                  static_cast<int32_t*>(op.p[1]), static_cast<int32_t*>(op.p[2]),
+                                  static_cast<int32_t*>(op.p[3]), st);
+        case PP_OP_MOE_GATHER:
+            return pp_moe_gather(op.p[0], op.i[0], static_cast<const int32_t*>(op.p[1]),
+                                 static_cast<const int32_t*>(op.p[2]), (int)op.i[1],
+                                 static_cast<const float*>(op.p[3]), op.p[4], op.i[2], op.i[3], op.i[4], st);
+        case PP_OP_MOE_COMBINE:
+            return pp_moe_combine(op.p[0], op.i[0], static_cast<const int32_t*>(op.p[1]),
+                                  static_cast<const float*>(op.p[2]), (int)op.i[1], op.p[3], op.i[2], op.p[4],
+                                  op.i[3], op.i[4], op.i[5], st);
+        case PP_OP_MOE_GATE_BWD:
+            return pp_moe_gate_bwd(op.p[0], op.i[0], op.p[1], op.i[1], static_cast<const int32_t*>(op.p[2]),
+                                   static_cast<const int32_t*>(op.p[3]), static_cast<const float*>(op.p[4]),
+                                   (int)op.i[2], (int)op.i[3], op.p[5], op.i[4], op.i[5], op.i[6], st);
         default:
             return fail(PP_ERR_INVALID, "unknown op kind %d", op.kind);
     }

@@ -183,6 +183,14 @@ class PipelineStageBase:
             raise RuntimeError(f"{self.log_prefix} is not lowered to launch lists and has no arena")
         return self._stage_program().arena
 
+    def saved_activations(self, mb: int) -> Dict[str, torch.Tensor]:
+        """The buffers a natively lowered stage keeps for microbatch ``mb`` between its forward and
+        backward pass, by scoped name (for inspection, e.g. the expert selection of a
+        mixture-of-experts layer: keys ending in ``topk_idx``)."""
+        if not self.is_native:
+            raise RuntimeError(f"{self.log_prefix} is not lowered to launch lists")
+        return dict(self._stage_program().mbs[mb].acts)
+
     def _publish_grad_views(self):
         """fp32 parameters get their accumulator as ``.grad``; bf16 parameters expose it as
         ``.main_grad`` (torch does not allow an fp32 ``.grad`` on a bf16 parameter)."""

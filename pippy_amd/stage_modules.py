@@ -203,30 +203,37 @@ class LayerNormBlock(NativeBlock):
 
 
 class TokenEmbedding(NativeBlock):
-    """Token + learned position embedding: ``wte[ids] + wpe[:S]`` (GPT-2 style)."""
+    """Token + learned position embedding: ``wte[ids] + wpe[:S]`` (GPT-2 style);
+    ``positions=False`` leaves the position table out (models with rotary embeddings)."""
 
-    def __init__(self, vocab: int, max_seq: int, dim: int, dtype=torch.bfloat16, init_std=0.02):
+    def __init__(self, vocab: int, max_seq: int, dim: int, dtype=torch.bfloat16, init_std=0.02,
+                 positions: bool = True):
         super().__init__()
         self.wte = nn.Embedding(vocab, dim, dtype=dtype)
-        self.wpe = nn.Embedding(max_seq, dim, dtype=dtype)
         nn.init.normal_(self.wte.weight, std=init_std)
-        nn.init.normal_(self.wpe.weight, std=init_std)
+        self.wpe = None
+        if positions:
+            self.wpe = nn.Embedding(max_seq, dim, dtype=dtype)
+            nn.init.normal_(self.wpe.weight, std=init_std)
 
     def forward(self, ids):
+        if self.wpe is None:
+            return self.wte(ids)
         S = ids.shape[-1]
         pos = torch.arange(S, device=ids.device)
         return self.wte(ids) + self.wpe(pos)
 
     def _pp_direct_acc_params(self):
-        return [self.wte.weight, self.wpe.weight]
+        return [self.wte.weight] + ([self.wpe.weight] if self.wpe is not None else [])
 
     def lower(self, b, ids):
         if ids.dtype != torch.int64 or ids.dim() != 2:
             raise RuntimeError(f"TokenEmbedding expects int64 ids of shape [batch, seq], got "
                                f"{ids.dtype} {tuple(ids.shape)}")
         Bn, S = ids.shape
-        wte, wpe = b.weight(self.wte.weight), b.weight(self.wpe.weight)
-        if S > wpe.shape[0]:
+        wte = b.weight(self.wte.weight)
+        wpe = b.weight(self.wpe.weight) if self.wpe is not None else None
+        if wpe is not None and S > wpe.shape[0]:
             raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
         Cc = wte.shape[1]
         y = b.act("y", (Bn, S, Cc))
@@ -234,9 +241,11 @@ class TokenEmbedding(NativeBlock):
 
         def bwd(dy, need_dx, dx_out):
             # scatter-add straight into the fp32 accumulators (zeroed on the first accumulation)
-            acc_wte, acc_wpe = b.grad_acc(self.wte.weight), b.grad_acc(self.wpe.weight)
+            acc_wte = b.grad_acc(self.wte.weight)
+            acc_wpe = b.grad_acc(self.wpe.weight) if self.wpe is not None else None
             b.w(P.op_fill(acc_wte), tag="fill")
-            b.w(P.op_fill(acc_wpe), tag="fill")
+            if acc_wpe is not None:
+                b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S))
             return None
 
@@ -519,12 +528,15 @@ class LlamaLayer(NativeBlock):
         q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
         o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         x = x + self.self_attn.o_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
-        h = self.post_attention_layernorm(x)
-        return x + self.mlp.down_proj(F.silu(self.mlp.gate_proj(h)) * self.mlp.up_proj(h))
+        return x + self._feed_forward(self.post_attention_layernorm(x))
+
+    def _feed_forward(self, h):
+        return self.mlp.down_proj(F.silu(self.mlp.gate_proj(h)) * self.mlp.up_proj(h))
 
     def lower(self, b, x):
         if x.dim() != 3 or x.shape[-1] != self.dim:
-            raise RuntimeError(f"LlamaLayer of width {self.dim} expects [batch, seq, dim], got {tuple(x.shape)}")
+            raise RuntimeError(f"{type(self).__name__} of width {self.dim} expects [batch, seq, dim], got "
+                               f"{tuple(x.shape)}")
         Bn, S, Cc = x.shape
         T, H = Bn * S, self.n_heads
         D = Cc // H
@@ -541,24 +553,10 @@ class LlamaLayer(NativeBlock):
         lse = b.act("lse", (Bn, H, S), torch.float32)
         b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, True))
         x2, _ = lower_linear(b, "x2", self.self_attn.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
-        n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
-        g, _ = lower_linear(b, "g", self.mlp.gate_proj, n2)
-        u, _ = lower_linear(b, "u", self.mlp.up_proj, n2)
-        h = b.act("h", (T, self.ffn))
-        b.f(P.op_swiglu_fwd(g, u, h))
-        y, _ = lower_linear(b, "y", self.mlp.down_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+        y, ffn_backward = self._lower_feed_forward(b, x2)
 
         def bwd(dy, need_dx, dx_out):
-            dy2d = dy.view(T, Cc)
-            d_h = linear_backward(b, "down", self.mlp.down_proj, h, dy2d)
-            dg = b.grad("dg", (T, self.ffn))
-            du = b.grad("du", (T, self.ffn))
-            b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
-            # the two branches that read n2 add up in the residual epilogue of the second GEMM
-            d_n2a = linear_backward(b, "gate", self.mlp.gate_proj, n2, dg)
-            d_n2 = linear_backward(b, "up", self.mlp.up_proj, n2, du, dx_epilogue=N.EPI_BIAS_RESIDUAL,
-                                   dx_aux=d_n2a)
-            d_x2 = rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+            d_x2 = ffn_backward(dy.view(T, Cc))
             d_att = linear_backward(b, "o", self.self_attn.o_proj, att, d_x2)
             dqkv = b.grad("dqkv", (T, 3 * Cc))
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
@@ -574,6 +572,164 @@ class LlamaLayer(NativeBlock):
         b.on_backward(bwd)
         return y.view(Bn, S, Cc)
 
+    def _lower_feed_forward(self, b, x2):
+        """Emits y = x2 + FFN(RMSNorm(x2)); returns (y, emitter of the backward: dy -> d_x2)."""
+        T = x2.shape[0]
+        n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
+        g, _ = lower_linear(b, "g", self.mlp.gate_proj, n2)
+        u, _ = lower_linear(b, "u", self.mlp.up_proj, n2)
+        h = b.act("h", (T, self.ffn))
+        b.f(P.op_swiglu_fwd(g, u, h))
+        y, _ = lower_linear(b, "y", self.mlp.down_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+
+        def backward(dy2d):
+            d_h = linear_backward(b, "down", self.mlp.down_proj, h, dy2d)
+            dg = b.grad("dg", (T, self.ffn))
+            du = b.grad("du", (T, self.ffn))
+            b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
+            # the two branches that read n2 add up in the residual epilogue of the second GEMM
+            d_n2a = linear_backward(b, "gate", self.mlp.gate_proj, n2, dg)
+            d_n2 = linear_backward(b, "up", self.mlp.up_proj, n2, du, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+                                   dx_aux=d_n2a)
+            return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+
+        return y, backward
+
+
+class _Expert(nn.Module):
+    """SwiGLU expert with Mixtral's parameter names: w2(silu(w1 x) * w3 x)."""
+
+    def __init__(self, dim, ffn, dtype, init_std):
+        super().__init__()
+        self.w1 = nn.Linear(dim, ffn, bias=False, dtype=dtype)
+        self.w2 = nn.Linear(ffn, dim, bias=False, dtype=dtype)
+        self.w3 = nn.Linear(dim, ffn, bias=False, dtype=dtype)
+        for lin in (self.w1, self.w2, self.w3):
+            nn.init.normal_(lin.weight, std=init_std)
+
+    def forward(self, x):
+        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+
+class MoELayer(LlamaLayer):
+    """A Mixtral-style decoder layer: the attention half of ``LlamaLayer`` and, in place of the dense
+    feed-forward, a sparse mixture of ``n_experts`` SwiGLU experts of which a softmax router picks
+    two per token (weights renormalised over the pair).  Parameters: ``block_sparse_moe.gate`` and
+    ``block_sparse_moe.experts.<e>.w1 / w2 / w3``.  The launch-list form takes 8, 16, .. 64 experts.
+
+    ``forced_routing`` (a list of int64 [tokens, 2] tensors, one per forward call, consumed in
+    order) overrides the expert selection of the torch statement; a comparison against a lower
+    precision run uses it so that tokens whose second and third logits nearly tie do not count as
+    errors of the arithmetic."""
+
+    TOPK = 2
+
+    def __init__(self, dim: int, n_heads: int, ffn: int, n_experts: int = 8, *, eps: float = 1e-5,
+                 rope_theta: float = 1e6, dtype=torch.bfloat16, init_std=0.02):
+        super().__init__(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype, init_std=init_std)
+        del self.mlp
+        assert 2 <= n_experts <= 64
+        self.n_experts = n_experts
+        self.block_sparse_moe = nn.Module()
+        self.block_sparse_moe.gate = nn.Linear(dim, n_experts, bias=False, dtype=dtype)
+        nn.init.normal_(self.block_sparse_moe.gate.weight, std=init_std)
+        self.block_sparse_moe.experts = nn.ModuleList([_Expert(dim, ffn, dtype, init_std) for _ in range(n_experts)])
+        self.forced_routing = None
+
+    def _feed_forward(self, h):
+        shape = h.shape
+        h = h.reshape(-1, shape[-1])
+        moe = self.block_sparse_moe
+        probs = torch.softmax(moe.gate(h).float(), dim=-1)
+        if self.forced_routing:
+            idx = self.forced_routing.pop(0).to(h.device)
+        else:
+            idx = torch.sort(probs, dim=-1, descending=True, stable=True).indices[:, :2]
+        top = probs.gather(-1, idx)
+        gate = top / top.sum(-1, keepdim=True)
+        y = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
+        for e, expert in enumerate(moe.experts):
+            tok, slot = torch.where(idx == e)
+            if tok.numel():
+                y = y.index_add(0, tok, gate[tok, slot, None] * expert(h[tok]).float())
+        return y.to(h.dtype).reshape(shape)
+
+    def _pointer_list(self, b, name, tensors):
+        t = b.sp.shared(f"moe_ptrs:{id(self)}:{name}", (len(tensors),), torch.int64)
+        t.copy_(torch.tensor([x.data_ptr() for x in tensors], dtype=torch.int64))
+        return t
+
+    def _lower_feed_forward(self, b, x2):
+        T, Cc = x2.shape
+        E, K, ffn = self.n_experts, self.TOPK, self.ffn
+        if E % 8:
+            # the router GEMMs run with the expert count as a leading dimension and as a reduction length
+            raise RuntimeError(f"MoELayer lowers with a multiple of 8 experts, got {E}")
+        R = T * K
+        moe = self.block_sparse_moe
+        experts = list(moe.experts)
+        n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
+        logits = b.act("router_logits", (T, E))
+        lower_linear(b, "router", moe.gate, n2, out=logits)
+        idx = b.act("topk_idx", (T, K), torch.int32)
+        gate = b.act("gate", (T, K), torch.float32)
+        b.f(P.op_moe_router(logits, idx, gate))
+        seg = b.act("seg_start", (E + 1,), torch.int32)
+        row_src = b.act("row_src", (R,), torch.int32)
+        pos = b.act("pos", (R,), torch.int32)
+        b.f(P.op_moe_permute(idx.view(-1), E, seg, row_src, pos))
+        xp = b.act("xp", (R, Cc))
+        b.f(P.op_moe_gather(n2, row_src, K, xp))
+        w1 = self._pointer_list(b, "w1", [b.weight(ex.w1.weight) for ex in experts])
+        w2 = self._pointer_list(b, "w2", [b.weight(ex.w2.weight) for ex in experts])
+        w3 = self._pointer_list(b, "w3", [b.weight(ex.w3.weight) for ex in experts])
+        g = b.act("g", (R, ffn))
+        u = b.act("u", (R, ffn))
+        h = b.act("h", (R, ffn))
+        yp = b.act("yp", (R, Cc))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w1, seg, Cm=g))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w3, seg, Cm=u))
+        b.f(P.op_swiglu_fwd(g, u, h))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, h, w2, seg, Cm=yp))
+        y = b.act("y", (T, Cc))
+        b.f(P.op_moe_combine(yp, pos, K, y, gate=gate.view(-1), resid=x2))
+
+        def backward(dy2d):
+            # expert rows receive the output gradient of their token times the routing weight
+            d_yp = b.grad("d_yp", (R, Cc))
+            b.i(P.op_moe_gather(dy2d, row_src, K, d_yp, scale=gate.view(-1)))
+            dlogits = b.grad("dlogits", (T, E))
+            b.i(P.op_moe_gate_bwd(dy2d, yp, pos, idx, gate, E, dlogits))
+            w2t = self._pointer_list(b, "w2t", [b.weight_t(ex.w2.weight) for ex in experts])
+            w1t = self._pointer_list(b, "w1t", [b.weight_t(ex.w1.weight) for ex in experts])
+            w3t = self._pointer_list(b, "w3t", [b.weight_t(ex.w3.weight) for ex in experts])
+            d_h = b.grad("d_h", (R, ffn))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, d_yp, w2t, seg, Cm=d_h))
+            dg = b.grad("dg", (R, ffn))
+            du = b.grad("du", (R, ffn))
+            b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
+            d_xp = b.grad("d_xp", (R, Cc))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=d_xp))
+            # token gradient: its two expert rows, plus the router branch in the GEMM epilogue
+            d_n2a = b.grad("d_n2a", (T, Cc))
+            b.i(P.op_moe_combine(d_xp, pos, K, d_n2a))
+            d_n2 = linear_backward(b, "router", moe.gate, n2, dlogits, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+                                   dx_aux=d_n2a)
+            # expert weight gradients: one segmented GEMM per projection, reduced over each expert's rows
+            for name, dy_rows, x_rows in (("w1", dg, xp), ("w3", du, xp), ("w2", d_yp, h)):
+                params = [getattr(ex, name).weight for ex in experts]
+                if b.fused_accumulate:
+                    ptrs = self._pointer_list(b, "acc_" + name, [b.grad_acc(p) for p in params])
+                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, epilogue=N.EPI_ACCUM_F32,
+                                      beta=1, c_f32=True), tag="beta")
+                else:
+                    ptrs = self._pointer_list(b, "stage_" + name, [b.grad_target(p) for p in params])
+                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows))
+            return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+
+        return y, backward
+
 
 class LMHead(NativeBlock):
     """Final LayerNorm and the (untied) vocabulary projection.  The weight is stored with its
@@ -582,11 +738,15 @@ class LMHead(NativeBlock):
 
     VOCAB_ALIGN = 128
 
-    def __init__(self, dim: int, vocab: int, *, final_ln: bool = True, eps: float = 1e-5,
+    def __init__(self, dim: int, vocab: int, *, final_ln=True, eps: float = 1e-5,
                  dtype=torch.bfloat16, init_std=0.02):
+        """``final_ln``: True (LayerNorm), "rms" (RMSNorm) or False (no final normalisation)."""
         super().__init__()
         self.dim, self.vocab = dim, vocab
-        self.ln_f = nn.LayerNorm(dim, eps=eps, dtype=dtype) if final_ln else None
+        if final_ln == "rms":
+            self.ln_f = nn.RMSNorm(dim, eps=eps, dtype=dtype)
+        else:
+            self.ln_f = nn.LayerNorm(dim, eps=eps, dtype=dtype) if final_ln else None
         self.lm_head = nn.Linear(dim, vocab, bias=False, dtype=dtype)
         nn.init.normal_(self.lm_head.weight, std=init_std)
 
@@ -606,7 +766,10 @@ class LMHead(NativeBlock):
         Bn, S, Cc = x.shape
         T, V, Vp = Bn * S, self.vocab, self.padded_vocab
         x2d = x.view(T, Cc)
-        if self.ln_f is not None:
+        rms = isinstance(self.ln_f, nn.RMSNorm)
+        if rms:
+            h, rstd = lower_rmsnorm(b, "ln_f", self.ln_f, x2d)
+        elif self.ln_f is not None:
             h, mean, rstd = lower_layernorm(b, "ln_f", self.ln_f, x2d)
         else:
             h = x2d
@@ -624,8 +787,11 @@ class LMHead(NativeBlock):
                 return None
             if self.ln_f is None:
                 return d_h.view(Bn, S, Cc)
-            dx = layernorm_backward(b, "ln_f", self.ln_f, x2d, mean, rstd, d_h,
-                                    dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            dx_view = dx_out.view(T, Cc) if dx_out is not None else None
+            if rms:
+                dx = rmsnorm_backward(b, "ln_f", self.ln_f, x2d, rstd, d_h, dx_out=dx_view)
+            else:
+                dx = layernorm_backward(b, "ln_f", self.ln_f, x2d, mean, rstd, d_h, dx_out=dx_view)
             return dx.view(Bn, S, Cc)
 
         b.on_backward(bwd)

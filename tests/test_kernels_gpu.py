@@ -614,3 +614,165 @@ def test_rope_matches_oracle_and_inverts(B, S, H, D):
     # the inverse rotation brings q and k back (two bf16 roundings away)
     N.rope(x, cos.cuda(), sin.cuda(), S, 2 * H, D, inverse=True)
     assert_close_rel(x, qkv.float(), BF16_TOL, "rope followed by its transpose")
+
+
+# ---- mixture-of-experts routing and segmented GEMMs ---------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,E", [(2048, 8), (77, 3), (1000, 64)])
+def test_moe_router_top2_matches_oracle(T, E):
+    N = native()
+    torch.manual_seed(0)
+    logits = (torch.randn(T, E) * 0.6).to(torch.bfloat16)     # bf16 values: ties do occur
+    logits[0] = 1.0                                            # a row of equal logits
+    idx = torch.empty(T, 2, dtype=torch.int32, device=DEV)
+    gate = torch.empty(T, 2, dtype=torch.float32, device=DEV)
+    N.moe_router_top2(logits.to(DEV), idx, gate)
+    ref_idx, ref_gate = O.moe_route_top2(logits.float())
+    assert torch.equal(idx.cpu().long(), ref_idx)
+    assert (gate.cpu() - ref_gate).abs().max() <= 1e-6
+    # where the three largest values are distinct the selection is torch.topk's
+    top3 = torch.topk(logits.float(), min(3, E), -1).values
+    clean = (top3[:, 0] != top3[:, 1]) & ((top3[:, 1] != top3[:, 2]) if E > 2 else True)
+    assert clean.sum() > T // 2
+    assert torch.equal(idx.cpu().long()[clean], torch.topk(logits.float(), 2, -1).indices[clean])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,E", [(4096, 8), (5001, 3), (10, 64), (0, 4)])
+def test_moe_permute_bit_exact(n, E):
+    N = native()
+    torch.manual_seed(1)
+    slots = torch.randint(0, E, (n,), dtype=torch.int32)
+    if n > 100:
+        slots[slots == 1] = 0                                  # an expert without tokens
+    seg = torch.full((E + 1,), -7, dtype=torch.int32, device=DEV)
+    row_src = torch.full((n,), -7, dtype=torch.int32, device=DEV)
+    pos = torch.full((n,), -7, dtype=torch.int32, device=DEV)
+    N.moe_permute(slots.to(DEV), E, seg, row_src, pos)
+    ref_seg, ref_rows, ref_pos = O.moe_permutation(slots, E)
+    assert torch.equal(seg.cpu().long(), ref_seg)
+    assert torch.equal(row_src.cpu().long(), ref_rows)
+    assert torch.equal(pos.cpu().long(), ref_pos)
+
+
+@pytest.mark.gpu
+def test_moe_permute_drops_slots_with_an_invalid_expert():
+    N = native()
+    slots = torch.tensor([2, 9, 0, -1, 2, 1], dtype=torch.int32)
+    seg = torch.empty(4, dtype=torch.int32, device=DEV)
+    row_src = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+    pos = torch.empty(6, dtype=torch.int32, device=DEV)
+    N.moe_permute(slots.to(DEV), 3, seg, row_src, pos)
+    assert seg.tolist() == [0, 1, 2, 4]
+    assert row_src.tolist()[:4] == [2, 5, 0, 4]
+    assert pos.tolist() == [2, -1, 0, -1, 3, 1]
+
+
+@pytest.mark.gpu
+def test_moe_gather_and_combine():
+    N = native()
+    torch.manual_seed(2)
+    T, Cc, K, E = 300, 256, 2, 8
+    x = torch.randn(T, Cc).to(torch.bfloat16)
+    slots = torch.randint(0, E, (T * K,), dtype=torch.int32)
+    _, row_src, pos = O.moe_permutation(slots, E)
+    gate = torch.rand(T * K)
+    xd, rows_d, pos_d, gate_d = x.to(DEV), row_src.int().to(DEV), pos.int().to(DEV), gate.to(DEV)
+    out = torch.empty(T * K, Cc, dtype=torch.bfloat16, device=DEV)
+    N.moe_gather(xd, rows_d, K, out)
+    assert torch.equal(out.cpu(), x[row_src // K])               # a plain gather moves bytes
+    N.moe_gather(xd, rows_d, K, out, scale=gate_d)
+    ref = (gate[row_src, None] * x[row_src // K].float())
+    assert torch.equal(out.cpu(), ref.to(torch.bfloat16))        # one product, one rounding
+    # only the first *n_rows rows are written
+    out.fill_(7)
+    n_rows = torch.tensor([10], dtype=torch.int32, device=DEV)
+    N.moe_gather(xd, rows_d, K, out, n_rows=n_rows)
+    assert torch.equal(out[:10].cpu(), x[row_src[:10] // K]) and bool((out[10:] == 7).all())
+    # combine: resid + sum_k gate * y[pos]
+    y = torch.randn(T * K, Cc).to(torch.bfloat16)
+    resid = torch.randn(T, Cc).to(torch.bfloat16)
+    res = torch.empty(T, Cc, dtype=torch.bfloat16, device=DEV)
+    N.moe_combine(y.to(DEV), pos_d, K, res, gate=gate_d, resid=resid.to(DEV))
+    ref = resid.float() + (gate.view(T, K, 1) * y.float()[pos].view(T, K, Cc)).sum(1)
+    assert_close_rel(res, ref, 4e-3, "combine")                  # one bf16 rounding of an fp32 sum
+    N.moe_combine(y.to(DEV), pos_d, K, res)
+    assert_close_rel(res, y.float()[pos].view(T, K, Cc).sum(1), 4e-3, "unweighted combine")
+
+
+@pytest.mark.gpu
+def test_moe_gate_bwd_matches_autograd():
+    N = native()
+    torch.manual_seed(3)
+    T, Cc, E, K = 200, 128, 8, 2
+    logits = (torch.randn(T, E) * 0.6).to(torch.bfloat16)
+    idx, gate = O.moe_route_top2(logits.float())
+    _, row_src, pos = O.moe_permutation(idx, E)
+    y = torch.randn(T * K, Cc).to(torch.bfloat16)
+    dout = (torch.randn(T, Cc) * 0.1).to(torch.bfloat16)
+    # autograd through softmax -> gather -> renormalise -> weighted sum of the expert rows
+    lg = logits.float().requires_grad_()
+    top = torch.softmax(lg, -1).gather(-1, idx)
+    g = top / top.sum(-1, keepdim=True)
+    out = (g.unsqueeze(-1) * y.float()[pos].view(T, K, Cc)).sum(1)
+    out.backward(dout.float())
+    dl = torch.empty(T, E, dtype=torch.bfloat16, device=DEV)
+    N.moe_gate_bwd(dout.to(DEV), y.to(DEV), pos.int().to(DEV), idx.int().to(DEV), gate.to(DEV), E, dl)
+    assert_close_rel(dl, lg.grad, BF16_TOL, "router logit gradient")
+    unselected = torch.ones(T, E, dtype=torch.bool).scatter(1, idx, False)
+    assert bool((dl.cpu()[unselected] == 0).all())
+
+
+def _segments(R, E, seed):
+    g = torch.Generator().manual_seed(seed)
+    cuts = torch.sort(torch.randint(0, R + 1, (E - 1,), generator=g)).values
+    seg = torch.cat([torch.zeros(1, dtype=torch.long), cuts, torch.tensor([R])])
+    return seg
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,K,Nn,E", [(4096, 1024, 512, 8), (1000, 256, 384, 5), (130, 64, 128, 3)])
+def test_segmented_gemm_rows_mode(R, K, Nn, E):
+    N = native()
+    torch.manual_seed(4)
+    seg = _segments(R, E, R)
+    seg[2] = seg[1]                                              # an empty segment
+    A = (torch.randn(R, K) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(E, Nn, K) * 0.05).to(torch.bfloat16)
+    aux = torch.randn(R, Nn).to(torch.bfloat16)
+    Ad, Wd, auxd = A.to(DEV), W.to(DEV), aux.to(DEV)
+    ptrs = torch.tensor([Wd[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    segd = seg.int().to(DEV)
+    ref = torch.empty(R, Nn)
+    for e in range(E):
+        r0, r1 = int(seg[e]), int(seg[e + 1])
+        ref[r0:r1] = A[r0:r1].float() @ W[e].float().T
+    Cm = torch.full((R, Nn), 3.0, dtype=torch.bfloat16, device=DEV)
+    N.gemm_bf16_segmented(Ad, ptrs, Cm, segd, N.SEG_ROWS)
+    assert_close_rel(Cm, ref, BF16_TOL, "segmented rows")
+    N.gemm_bf16_segmented(Ad, ptrs, Cm, segd, N.SEG_ROWS, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=auxd)
+    assert_close_rel(Cm, ref + aux.float(), BF16_TOL, "segmented rows + residual")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,M,Nn,E", [(4096, 512, 1024, 8), (1000, 128, 136, 4), (50, 8, 64, 3)])
+def test_segmented_gemm_k_mode(R, M, Nn, E):
+    N = native()
+    torch.manual_seed(5)
+    seg = _segments(R, E, R + 1)
+    seg[2] = seg[1]
+    dY = (torch.randn(R, M) * 0.5).to(torch.bfloat16)
+    X = (torch.randn(R, Nn) * 0.5).to(torch.bfloat16)
+    ref = torch.stack([dY[int(seg[e]):int(seg[e + 1])].float().T @ X[int(seg[e]):int(seg[e + 1])].float()
+                       for e in range(E)])
+    segd = seg.int().to(DEV)
+    out = torch.full((E, M, Nn), 3.0, dtype=torch.bfloat16, device=DEV)
+    ptrs = torch.tensor([out[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    N.gemm_bf16_segmented(dY.to(DEV), ptrs, None, segd, N.SEG_K, other=X.to(DEV))
+    assert_close_rel(out, ref, BF16_TOL, "segmented k")
+    assert bool((out[1] == 0).all())                             # the empty segment writes zeros
+    acc = torch.ones(E, M, Nn, dtype=torch.float32, device=DEV)
+    ptrs = torch.tensor([acc[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    N.gemm_bf16_segmented(dY.to(DEV), ptrs, None, segd, N.SEG_K, other=X.to(DEV), epilogue=N.EPI_ACCUM_F32,
+                          beta=1, c_dtype=torch.float32)
+    assert_close_rel(acc, ref + 1.0, 1e-3, "segmented k, fp32 accumulate")

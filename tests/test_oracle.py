@@ -285,3 +285,67 @@ def test_rope_is_a_complex_rotation_with_relative_position_property():
     k = torch.randn(D, generator=g).expand(S, D)
     qr, kr = O.rope(q, cos, sin), O.rope(k, cos, sin)
     torch.testing.assert_close((qr[5] * kr[2]).sum(), (qr[9] * kr[6]).sum(), rtol=1e-4, atol=1e-5)
+
+
+# ---- top-2 mixture of experts ------------------------------------------------------------------
+def test_moe_routing_matches_topk_and_breaks_ties_towards_the_lower_index():
+    from oracle import ops as O
+    torch.manual_seed(0)
+    logits = torch.randn(500, 8)
+    idx, gate = O.moe_route_top2(logits)
+    probs = torch.softmax(logits, -1)
+    top_v, top_i = torch.topk(probs, 2, dim=-1)     # fp32 normal draws: no ties
+    assert torch.equal(idx, top_i)
+    assert torch.allclose(gate, top_v / top_v.sum(-1, keepdim=True), atol=1e-7)
+    assert torch.allclose(gate.sum(-1), torch.ones(500), atol=1e-6)
+    # renormalising over the pair is the softmax of the two logits alone
+    two = torch.softmax(logits.gather(-1, idx), -1)
+    assert torch.allclose(gate, two, atol=1e-6)
+    tied = torch.tensor([[1.0, 3.0, 3.0, 3.0], [2.0, 2.0, 2.0, 2.0], [0.0, 1.0, 5.0, 1.0]])
+    idx, gate = O.moe_route_top2(tied)
+    assert idx.tolist() == [[1, 2], [0, 1], [2, 1]]
+    assert torch.allclose(gate[:2], torch.full((2, 2), 0.5))
+
+
+def test_moe_permutation_matches_brute_force():
+    from oracle import ops as O
+    torch.manual_seed(1)
+    E = 5
+    slots = torch.randint(0, E, (37, 2))
+    seg, row_src, pos = O.moe_permutation(slots, E)
+    flat = slots.reshape(-1).tolist()
+    rows = [f for e in range(E) for f in range(len(flat)) if flat[f] == e]
+    assert row_src.tolist() == rows
+    assert [rows.index(f) for f in range(len(flat))] == pos.tolist()
+    assert seg.tolist() == [sum(1 for v in flat if v < e) for e in range(E + 1)]
+
+
+def test_moe_layer_equals_dense_sum_with_zero_weights_and_module_statement():
+    from oracle import ops as O
+    from pippy_amd.stage_modules import MoELayer
+    torch.manual_seed(2)
+    T, d, ffn, E = 40, 32, 48, 6
+    layer = MoELayer(64, 1, ffn, E, dtype=torch.float32)     # only its feed-forward half is used
+    x = torch.randn(T, 64)
+    moe = layer.block_sparse_moe
+    w1 = torch.stack([e.w1.weight for e in moe.experts])
+    w2 = torch.stack([e.w2.weight for e in moe.experts])
+    w3 = torch.stack([e.w3.weight for e in moe.experts])
+    with torch.no_grad():
+        moe.gate.weight.mul_(20)     # spread the routing probabilities
+        y = O.moe_top2(x, moe.gate.weight, w1, w2, w3)
+        # dense statement: every expert on every token, weight zero unless selected
+        probs = torch.softmax(x @ moe.gate.weight.T, -1)
+        top_v, top_i = torch.topk(probs, 2, -1)
+        dense_gate = torch.zeros(T, E).scatter(1, top_i, top_v / top_v.sum(-1, keepdim=True))
+        dense = sum(dense_gate[:, e, None] * (torch.nn.functional.silu(x @ w1[e].T) * (x @ w3[e].T)) @ w2[e].T
+                    for e in range(E))
+        assert torch.allclose(y, dense, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(layer._feed_forward(x), y, rtol=1e-5, atol=1e-6)
+        # a forced selection is honoured by both statements
+        forced = torch.stack([torch.arange(T) % E, (torch.arange(T) + 1) % E], 1)
+        layer.forced_routing = [forced]
+        y_forced = layer._feed_forward(x)
+        assert layer.forced_routing == []
+        assert torch.allclose(y_forced, O.moe_top2(x, moe.gate.weight, w1, w2, w3, idx=forced), rtol=1e-5, atol=1e-6)
+        assert not torch.allclose(y_forced, y, atol=1e-3)

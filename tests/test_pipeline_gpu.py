@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from _util import BF16_TOL, F32_TOL, assert_close_rel, max_rel
+from oracle import ops as OO
 from oracle import pipeline as OP
 
 pytestmark = pytest.mark.gpu
@@ -518,3 +519,69 @@ def test_llama_last_stage_with_final_rmsnorm_and_head_matches_oracle():
     for name, rp in ref.named_parameters():
         err = max_rel(named[name].main_grad, rp.grad)
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+
+
+# ---- Mixtral-style mixture of experts under interleaved 1F1B (config 5) ---------------------------
+def _moe_reference_stages(ref, n_stages, per):
+    import torch.nn as nn
+    out = []
+    for s in range(n_stages):
+        mods = [ref.embed] if s == 0 else []
+        mods += [ref.h[i] for i in range(per * s, per * (s + 1))]
+        if s == n_stages - 1:
+            mods.append(ref.head)
+        out.append(nn.Sequential(*mods))
+    return out
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_moe_interleaved_1f1b_matches_oracle(fused):
+    """Config 5 at a reduced size: two virtual stages of MoE layers on one rank under interleaved
+    1F1B.  The fp32 oracle is given the expert selection of the bf16 run (a token whose second and
+    third router logits nearly tie may legitimately flip under rounding); that the selection itself
+    is the top-2 of the run's own logits is checked separately."""
+    import pippy_amd as pp
+    from pippy_amd.configs import MoEDecoderLM, equal_split_spec
+    torch.manual_seed(0)
+    M, S, vocab, L, E = 4, 128, 512, 4, 8
+    model = MoEDecoderLM(vocab=vocab, dim=128, n_layers=L, n_heads=2, ffn=256, n_experts=E)
+    with torch.no_grad():
+        for layer in model.h:
+            layer.block_sparse_moe.gate.weight.mul_(10)     # decisive routing: few near-ties
+    ref = _fp32_cpu_copy(model)
+    ids = torch.randint(0, vocab, (2 * M, S))
+    target = torch.randint(0, vocab, (2 * M, S))
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(L, 2))
+    stages = [pp.PipelineStage(pipe, i, DEV, group=1, fused_accumulate=fused) for i in range(2)]
+    assert all(st.is_native for st in stages)
+    sched = pp.ScheduleInterleaved1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    losses = []
+    out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    torch.cuda.synchronize()
+    # the run's own routing: top-2 of its router logits, every token placed once per slot
+    routing = [[] for _ in range(L)]
+    for s, st in enumerate(stages):
+        for m in range(M):
+            acts = st.saved_activations(m)
+            idx = [v for k, v in acts.items() if k.endswith("topk_idx")]
+            logits = [v for k, v in acts.items() if k.endswith("router_logits")]
+            seg = [v for k, v in acts.items() if k.endswith("seg_start")]
+            assert len(idx) == L // 2
+            for j in range(L // 2):
+                want, _ = OO.moe_route_top2(logits[j].float().cpu())
+                assert torch.equal(idx[j].cpu().long(), want)
+                assert int(seg[j][-1]) == 2 * 2 * S and int(seg[j][0]) == 0
+                routing[s * (L // 2) + j].append(idx[j].cpu().long())
+    for l in range(L):
+        ref.h[l].forced_routing = list(routing[l])
+    ref_out, ref_losses = OP.step(_moe_reference_stages(ref, 2, L // 2), ids, target, M, _ce)
+    assert_close_rel(out, ref_out, BF16_TOL, "merged logits")
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.reshape(1), b.reshape(1), BF16_TOL, "loss")
+    named = dict(model.named_parameters())
+    worst = 0.0
+    for name, rp in ref.named_parameters():
+        err = max_rel(named[name].main_grad, rp.grad)
+        worst = max(worst, err)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+    note(f"MoE interleaved 1F1B (fused accumulate {fused}): worst grad error {worst:.3e}")
