@@ -585,3 +585,58 @@ def test_moe_interleaved_1f1b_matches_oracle(fused):
         worst = max(worst, err)
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
     note(f"MoE interleaved 1F1B (fused accumulate {fused}): worst grad error {worst:.3e}")
+
+
+def test_moe_mixtral_style_full_size_routing_and_schedule_invariants():
+    """Config 5 at full size (2 virtual stages of 4 layers, width 1024, 16 heads, 8 experts with
+    SwiGLU 4096, top-2, sequence 1024, batch 16 in 8 microbatches, vocabulary 32000).  Properties
+    that hold at any size: every (token, slot) pair lands in exactly one expert row, the two experts
+    of a token differ, the routing weights of a token sum to one, the expert row ranges tile
+    [0, 2 * tokens); and interleaved 1F1B gives bit-identical losses and gradients to GPipe."""
+    import pippy_amd as pp
+    from pippy_amd.configs import mixtral_style, equal_split_spec
+    torch.manual_seed(0)
+    M = 8
+    with torch.device(DEV):
+        model = mixtral_style()
+    ids = torch.randint(0, 32000, (16, 1024), device=DEV)
+    target = torch.randint(0, 32000, (16, 1024), device=DEV)
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(8, 2))
+    stages = [pp.PipelineStage(pipe, i, DEV, group=1) for i in range(2)]
+    assert all(st.is_native for st in stages)
+    probe = [model.h[0].block_sparse_moe.experts[3].w1.weight, model.h[7].block_sparse_moe.experts[0].w2.weight,
+             model.h[4].block_sparse_moe.gate.weight, model.h[2].self_attn.qkv_proj.weight,
+             model.h[5].post_attention_layernorm.weight]
+    results = []
+    for cls in (pp.ScheduleInterleaved1F1B, pp.ScheduleGPipe):
+        sched = cls(stages, M, loss_fn=pp.CrossEntropyLoss())
+        sched.zero_grad()
+        losses = []
+        out = sched.step(ids, target=target, losses=losses)
+        results.append((out, [l.clone() for l in losses], [p.main_grad.clone() for p in probe]))
+        if cls is pp.ScheduleInterleaved1F1B:
+            T = 2 * 1024
+            for st in stages:
+                for m in (0, M - 1):
+                    acts = st.saved_activations(m)
+                    for key in [k for k in acts if k.endswith("topk_idx")]:
+                        pre = key[:-len("topk_idx")]
+                        idx, gate = acts[key], acts[pre + "gate"]
+                        seg, row_src, pos = acts[pre + "seg_start"], acts[pre + "row_src"], acts[pre + "pos"]
+                        assert bool((idx[:, 0] != idx[:, 1]).all()) and int(idx.min()) >= 0 and int(idx.max()) < 8
+                        assert float((gate.sum(-1) - 1).abs().max()) <= 1e-6
+                        assert int(seg[0]) == 0 and int(seg[-1]) == 2 * T and bool((seg[1:] >= seg[:-1]).all())
+                        assert torch.equal(torch.sort(pos).values.long(), torch.arange(2 * T, device=DEV))
+                        assert torch.equal(row_src.long()[pos.long()], torch.arange(2 * T, device=DEV))
+                        # rows of expert e hold slots routed to e
+                        expert_of_row = idx.reshape(-1).long()[row_src.long()]
+                        bounds = torch.bucketize(torch.arange(2 * T, device=DEV), seg[1:].long(), right=True)
+                        assert torch.equal(expert_of_row, bounds)
+    (out_a, loss_a, g_a), (out_b, loss_b, g_b) = results
+    assert torch.isfinite(out_a.float()).all() and torch.equal(out_a, out_b)
+    for a, b in zip(loss_a, loss_b):
+        assert torch.equal(a, b)
+    # at initialisation the loss of a uniform guess over 32000 classes
+    assert abs(float(loss_a[0]) - 10.37) < 0.5
+    for a, b in zip(g_a, g_b):
+        assert torch.isfinite(a).all() and float(a.abs().max()) > 0 and torch.equal(a, b)
