@@ -164,13 +164,38 @@ class Pipe(nn.Module):
         # split_module flattens qualified names ("h.0" -> "h_0"); rebuild every stage module from the
         # original model with the original targets so that parameter names are unchanged
         # (the reference re-outlines for the same reason, ``_IR.py:765-769``)
+        # parameters and buffers that the model's own forward reads (``self.scale``) stay behind in
+        # the root as get_attr nodes feeding the stage call; they belong to the stage that uses them,
+        # under their original name (the reference sinks them the same way, ``_IR.py:785-895``)
+        sunk: Dict[str, Dict[int, str]] = {}
+        for call in split.graph.nodes:
+            if call.op != "call_module" or not str(call.target).startswith("submod_"):
+                continue
+            keep = []
+            for i, a in enumerate(call.args):
+                if isinstance(a, fx.Node) and a.op == "get_attr":
+                    sunk.setdefault(call.target, {})[i] = orig_target.get(a.name, a.target)
+                else:
+                    keep.append(a)
+            call.args = tuple(keep)
+        for n in list(split.graph.nodes):
+            if n.op == "get_attr" and not n.users:
+                split.graph.erase_node(n)
         for name, sub in list(split.named_children()):
             if not name.startswith("submod_"):
                 continue
             for n in sub.graph.nodes:
                 if n.op in ("call_module", "get_attr") and n.name in orig_target:
                     n.target = orig_target[n.name]
+            placeholders = [n for n in sub.graph.nodes if n.op == "placeholder"]
+            for i, target in sunk.get(name, {}).items():
+                ph = placeholders[i]
+                with sub.graph.inserting_after(ph):
+                    attr = sub.graph.create_node("get_attr", target)
+                ph.replace_all_uses_with(attr)
+                sub.graph.erase_node(ph)
             setattr(split, name, fx.GraphModule(mod, sub.graph, class_name=name))
+        split.recompile()
         found = [n for n, _ in split.named_children() if n.startswith("submod_")]
         if len(found) != num_stages:
             raise RuntimeError(f"expected {num_stages} stage modules after splitting, found {found} "

@@ -58,6 +58,35 @@ class _FusedOptimizer:
     def master_weights(self) -> List[Optional[torch.Tensor]]:
         return self._master
 
+    # -- checkpointing: state per parameter, keyed by the name it has in its stage module (which is
+    # the name in the un-split model), so that a state dict survives a different split
+    def _flat_state(self) -> dict:
+        """name -> list of flat fp32 state tensors, one per stage arena (None where unused)."""
+        return {"master": self._master}
+
+    def state_dict(self) -> dict:
+        state = {}
+        flats = self._flat_state()
+        for st, arena, k in zip(self._stages, self._arenas, range(len(self._arenas))):
+            for name, p in st.submod.named_parameters():
+                entry = {}
+                for key, per_stage in flats.items():
+                    if per_stage[k] is not None:
+                        entry[key] = arena._slice(per_stage[k], p, False).detach().cpu().clone()
+                state[name] = entry
+        return {"step": self._steps, "state": state}
+
+    def load_state_dict(self, sd: dict) -> None:
+        flats = self._flat_state()
+        for st, arena, k in zip(self._stages, self._arenas, range(len(self._arenas))):
+            for name, p in st.submod.named_parameters():
+                if name not in sd["state"]:
+                    raise KeyError(f"optimizer state of {name} is missing")
+                for key, per_stage in flats.items():
+                    if per_stage[k] is not None:
+                        arena._slice(per_stage[k], p, False).copy_(sd["state"][name][key])
+        self._steps = int(sd["step"])
+
 
 class FusedSGD(_FusedOptimizer):
     """``torch.optim.SGD`` over the arenas of lowered stages."""
@@ -77,6 +106,9 @@ class FusedSGD(_FusedOptimizer):
         self.lr, self.momentum, self.dampening = lr, momentum, dampening
         self.weight_decay, self.nesterov, self.maximize = weight_decay, nesterov, maximize
         self._buf = [torch.zeros_like(a.acc) if momentum != 0 else None for a in self._arenas]
+
+    def _flat_state(self):
+        return {"momentum_buffer": self._buf, "master": self._master}
 
     @torch.no_grad()
     def step(self):
@@ -106,6 +138,9 @@ class FusedAdamW(_FusedOptimizer):
         self.weight_decay, self.maximize = weight_decay, maximize
         self._m = [torch.zeros_like(a.acc) for a in self._arenas]
         self._v = [torch.zeros_like(a.acc) for a in self._arenas]
+
+    def _flat_state(self):
+        return {"exp_avg": self._m, "exp_avg_sq": self._v, "master": self._master}
 
     @torch.no_grad()
     def step(self):

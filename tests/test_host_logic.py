@@ -246,6 +246,36 @@ def test_annotate_split_points_and_errors():
         pipe.get_stage_module(5)
 
 
+def test_root_level_parameters_and_buffers_move_into_the_stage_that_reads_them():
+    """A tensor that the model's forward reads itself (not through a child module) belongs to the
+    stage that uses it, under its original name (reference ``_IR.py:785-895`` sinks them)."""
+    import pippy_amd as pp
+
+    class Scaled(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = nn.Linear(4, 4)
+            self.b = nn.Linear(4, 4)
+            self.gain = nn.Parameter(torch.full((4,), 2.0))
+            self.register_buffer("shift", torch.arange(4.0))
+
+        def forward(self, x):
+            x = self.a(x) + self.shift
+            pp.pipe_split()
+            return self.b(x) * self.gain
+
+    torch.manual_seed(0)
+    model = Scaled()
+    x = torch.randn(6, 4)
+    pipe = pp.pipeline(model, 2, (x,))
+    s0, s1 = pipe.get_stage_module(0), pipe.get_stage_module(1)
+    assert set(s0.state_dict()) == {"a.weight", "a.bias", "shift"}
+    assert set(s1.state_dict()) == {"b.weight", "b.bias", "gain"}
+    assert dict(s1.named_parameters())["gain"] is model.gain
+    assert len([n for n in s1.graph.nodes if n.op == "placeholder"]) == 1
+    assert torch.equal(pipe(x), model(x))
+
+
 def test_shared_parameters_are_rejected():
     class Tied(nn.Module):
         def __init__(self):
