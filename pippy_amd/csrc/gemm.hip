@@ -165,7 +165,9 @@ __device__ __forceinline__ void grouped_tile(uint32_t bid, uint32_t tiles_m, uin
 }
 
 // Scheduling hint for one k16 step: R LDS reads (the fragments of the next step) spread evenly
-// between M MFMAs.
+// between M MFMAs.  (Issuing all reads right after the first MFMA, with the tile's barrier at the
+// start of its last step, measured slower on the transformer shapes: 41.0 against 38.6 ms of GEMM
+// time per GPT-2-small step.)
 template <int R, int M, int I>
 __device__ __forceinline__ void interleave_reads() {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -173,15 +175,18 @@ __device__ __forceinline__ void interleave_reads() {
     if constexpr (I + 1 < M) interleave_reads<R, M, I + 1>();
 }
 
-// One BM x BN output tile with NS LDS stages filled by direct-to-LDS loads.
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+// One BM x BN output tile with NS LDS stages of KT values of k, filled by direct-to-LDS loads.
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int kStageElems = (BM + BN) * BK;
-    constexpr int LPT = DmaStage<BM, AT>::kLoads + DmaStage<BN, BT>::kLoads;  // loads per tile per wave
-    constexpr int kReadsPerStep = TM * FragReader<BM, AT>::kReads + TN * FragReader<BN, BT>::kReads;
+    constexpr int KS = KT / 16;  // MFMA k-steps per tile
+    constexpr int kStageElems = (BM + BN) * KT;
+    constexpr int LPT = DmaStage<BM, AT, KT>::kLoads + DmaStage<BN, BT, KT>::kLoads;  // loads per tile per wave
+    constexpr int kReadsPerStep = TM * FragReader<BM, AT, KT>::kReads + TN * FragReader<BN, BT, KT>::kReads;
     static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
+    static_assert(KS >= 2 && TN % 2 == 0, "the last k-step is split in two halves around the barrier");
+    static_assert(NS * kStageElems * 2 >= 4 * 32 * WTN * 4, "the epilogue stages fp32 bands in the tile memory");
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -196,18 +201,18 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    DmaStage<BM, AT> sa;
-    DmaStage<BN, BT> sb;
+    DmaStage<BM, AT, KT> sa;
+    DmaStage<BN, BT, KT> sb;
     sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
     sb.init(g.B, g.ldb, n0, g.N, g.K, wave, lane);
-    const int nk = (int)((g.K + BK - 1) / BK);
+    const int nk = (int)((g.K + KT - 1) / KT);
     auto issue = [&](int stage, int kt) {
-        sa.load(smem + stage * kStageElems, kt * BK, wave);
-        sb.load(smem + stage * kStageElems + BM * BK, kt * BK, wave);
+        sa.load(smem + stage * kStageElems, kt * KT, wave);
+        sb.load(smem + stage * kStageElems + BM * KT, kt * KT, wave);
     };
 
-    FragReader<BM, AT> ra[TM];
-    FragReader<BN, BT> rb[TN];
+    FragReader<BM, AT, KT> ra[TM];
+    FragReader<BN, BT, KT> rb[TN];
 #pragma unroll
     for (int t = 0; t < TM; ++t) ra[t].init(wm0 + t * 32, lane);
 #pragma unroll
@@ -217,7 +222,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
         for (int t = 0; t < TM; ++t) fa[sel][t] = ra[t].read(st, ks);
 #pragma unroll
-        for (int t = 0; t < TN; ++t) fb[sel][t] = rb[t].read(st + BM * BK, ks);
+        for (int t = 0; t < TN; ++t) fb[sel][t] = rb[t].read(st + BM * KT, ks);
     };
     auto mma = [&](int sel, int a_lo, int a_hi) {
 #pragma unroll
@@ -237,12 +242,16 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     read_frags(0, smem, 0);
 
     int stage = 0;
+    constexpr int kLast = (KS - 1) & 1;  // fragment set of a tile's last k-step
     for (int kt = 0; kt < nk; ++kt) {
         const uint16_t* st = smem + stage * kStageElems;
-        read_frags(1, st, 1); mma(0, 0, TN); interleave();
-        read_frags(0, st, 2); mma(1, 0, TN); interleave();
-        read_frags(1, st, 3); mma(0, 0, TN); interleave();
-        mma(1, 0, TN / 2);
+#pragma unroll
+        for (int ks = 1; ks < KS; ++ks) {
+            read_frags(ks & 1, st, ks);
+            mma((ks - 1) & 1, 0, TN);
+            interleave();
+        }
+        mma(kLast, 0, TN / 2);
         // tile kt+1 must have landed; tiles kt+2 .. kt+NS-1 may stay in flight
         const int ahead = nk - 2 - kt;
         if (NS >= 4 && ahead >= 2) wait_vmcnt<(NS >= 4 ? 2 : 0) * LPT>();
@@ -253,7 +262,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
         if (kt + NS < nk) issue(stage, kt + NS);
         stage = stage + 1 == NS ? 0 : stage + 1;
         if (kt + 1 < nk) read_frags(0, smem + stage * kStageElems, 0);
-        mma(1, TN / 2, TN);
+        mma(kLast, TN / 2, TN);
     }
 
     // Epilogue: one band of 32 rows at a time goes through a wave-private LDS region as fp32,
@@ -340,13 +349,13 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     }
 }
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_dma_kernel(const GemmArgs g) {
     const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= g.n_blocks) return;
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32>(g, tile_m, tile_n);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT>(g, tile_m, tile_n);
 }
 
 // Several independent problems in one grid: the tiles of problem i are the block ids
@@ -459,14 +468,15 @@ static int count_tiles(GemmArgs& g) {
 // with more tiles 2 stages leave room for two resident blocks, whose prologues and epilogues overlap
 // each other's main loops.
 constexpr uint32_t kComputeUnits = 256;
+constexpr int64_t kBigTileMinTiles = 1024;  // 256 x 256 tiles are used from this many of them
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 static int launch_single(const GemmArgs& g, hipStream_t st) {
-    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
-    static const int attr_rc = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32>, lds);
+    constexpr size_t lds = (size_t)NS * (BM + BN) * KT * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
     if (attr_rc) return attr_rc;
     const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+    hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid), dim3(kGemmThreads),
                        lds, st, g);
     return check_launch("gemm_bf16_dma_kernel");
 }
@@ -485,6 +495,16 @@ static int launch_group(const GemmGroupArgs& ga, hipStream_t st) {
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
 static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
     if (n == 1) {
+        if constexpr (EPI == PP_EPI_NONE && !CF32 && BM == 128 && !AT && !BT) {
+            // a large output with both operands k-contiguous: 256 x 256 tiles halve the LDS and L2
+            // traffic per MFMA (vocabulary projection 4096 x 50304 x 768: 776 against 707 TFLOP/s)
+            GemmArgs big = probs[0];
+            if (((big.M + 255) / 256) * ((big.N + 255) / 256) >= kBigTileMinTiles) {
+                int rc = count_tiles<256, 256>(big);
+                if (rc) return rc;
+                return launch_single<256, 256, AT, BT, 2, EPI, CF32>(big, st);
+            }
+        }
         GemmArgs g = probs[0];
         int rc = count_tiles<BM, BN>(g);
         if (rc) return rc;

@@ -160,6 +160,22 @@ def test_gemm_bf16_layouts(a_trans, b_trans, M, N, K):
     assert_close_rel(C32, ref, 1e-5, "gemm fp32 out")
 
 
+def test_gemm_bf16_large_output_takes_256_wide_tiles():
+    """Outputs of at least 1024 tiles of 256 x 256 (both operands k-contiguous, no epilogue) run on
+    the 256-wide tile variant: edges in M and N, a k tail, and a ragged leading dimension."""
+    Nn = native()
+    torch.manual_seed(11)
+    M, N, K = 8192 - 40, 8192 + 264, 136
+    A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    B = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    Cbuf = torch.full((M, N + 4), float("nan"), device=DEV, dtype=torch.bfloat16)
+    C = Cbuf[:, :N]
+    Nn.gemm_bf16(A, B, C)
+    ref = A.float() @ B.float().t()          # on the GPU in fp32: the CPU would take a minute
+    assert_close_rel(C, ref.cpu(), BF16_TOL, "gemm, 256-wide tiles")
+    assert bool(torch.isnan(Cbuf[:, N:]).all())
+
+
 def test_gemm_bf16_epilogues():
     Nn = native()
     torch.manual_seed(5)
