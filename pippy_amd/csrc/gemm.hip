@@ -366,7 +366,7 @@ struct GemmGroupArgs {
     int n;
 };
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const GemmGroupArgs ga) {
     uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= ga.tile_start[ga.n]) return;
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const Gem
     const GemmArgs& g = ga.p[i];
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32>(g, tile_m, tile_n);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT>(g, tile_m, tile_n);
 }
 
 // Segmented problems: the rows of one operand are partitioned into consecutive segments whose
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_k_kernel(const Gem
     g.C = const_cast<void*>(sa.seg_ptr[e]);
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, true, true, NS, EPI, CF32>(g, tile_m, tile_n);
+    gemm_tile_dma<BM, BN, true, true, NS, EPI, CF32, 32>(g, tile_m, tile_n);
 }
 
 template <typename Kernel>
@@ -481,13 +481,13 @@ static int launch_single(const GemmArgs& g, hipStream_t st) {
     return check_launch("gemm_bf16_dma_kernel");
 }
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 static int launch_group(const GemmGroupArgs& ga, hipStream_t st) {
-    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
-    static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32>, lds);
+    constexpr size_t lds = (size_t)NS * (BM + BN) * KT * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
     if (attr_rc) return attr_rc;
     const uint32_t grid = (ga.tile_start[ga.n] + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads),
+    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid), dim3(kGemmThreads),
                        lds, st, ga);
     return check_launch("gemm_bf16_group_kernel");
 }
@@ -638,7 +638,7 @@ static int launch_seg_rows(GemmSegArgs& sa, hipStream_t st) {
 template <int EPI, bool CF32>
 static int launch_seg_k(GemmSegArgs& sa, hipStream_t st) {
     constexpr int BM = 128, BN = 128, NS = 2;
-    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    constexpr size_t lds = (size_t)NS * (BM + BN) * 32 * sizeof(uint16_t);  // tiles of 32 k: with about 8 k-tiles per expert, four work-groups per CU cover each other's prologues
     static const int attr_rc = reserve_lds(&gemm_bf16_seg_k_kernel<BM, BN, NS, EPI, CF32>, lds);
     if (attr_rc) return attr_rc;
     int rc = count_tiles<BM, BN>(sa.g);
