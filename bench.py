@@ -62,7 +62,7 @@ def flops_per_step(args):
     return 3.0 * per_token_fwd * T
 
 
-def cpu_baseline(args, sample_microbatches=2):
+def cpu_baseline(args, sample_microbatches=4):
     """The oracle's statement of the reference step (fp32, torch CPU kernels, this box's cores) on a
     bounded sample of the same workload: the first microbatches of one step through all stages,
     forward, loss and backward in the reference's order."""
