@@ -294,9 +294,32 @@ class PipelineStageBase:
         prog.F.run()
         return prog.output, [x]
 
+    def _received(self, value):
+        if isinstance(value, torch.Tensor):
+            value = value.detach()
+            if self.has_backward and value.is_floating_point():
+                value = value.requires_grad_(True)
+        return value
+
     def _forward_eager(self, mb, args, kwargs):
+        routes = getattr(self, "_arg_routes", None)
         if self.is_first:
             composite_args, composite_kwargs = args, kwargs
+        elif routes is not None:
+            # inputs as the pipe's graph wires them: any earlier stage, any of its outputs
+            recv = []
+            for src, out_idx in routes:
+                producer = self._stages.get(src)
+                if producer is None:
+                    raise RuntimeError(
+                        f"{self.log_prefix} takes an input from stage {src}: pass every stage of the "
+                        "pipeline to the schedule")
+                if not producer._fwd_done.get(mb):
+                    raise RuntimeError(
+                        f"{self.log_prefix} activation of microbatch {mb} from stage {src} has not been produced")
+                out = producer.output_chunks[mb]
+                recv.append(self._received(out[out_idx] if out_idx is not None else out))
+            composite_args, composite_kwargs = tuple(recv), {}
         else:
             prev = self._prev
             if prev is None:
@@ -307,14 +330,7 @@ class PipelineStageBase:
                 raise RuntimeError(f"{self.log_prefix} activation of microbatch {mb} has not been produced")
             out = prev.output_chunks[mb]
             outs = out if isinstance(out, tuple) else (out,)
-            recv = []
-            for o in outs:
-                if isinstance(o, torch.Tensor):
-                    o = o.detach()
-                    if self.has_backward and o.is_floating_point():
-                        o = o.requires_grad_(True)
-                recv.append(o)
-            composite_args, composite_kwargs = tuple(recv), {}
+            composite_args, composite_kwargs = tuple(self._received(o) for o in outs), {}
         output = self.submod(*composite_args, **composite_kwargs)
         flat_inputs = flatten_args(composite_args) + flatten_args(composite_kwargs)
         return output, flat_inputs
@@ -436,17 +452,46 @@ class PipelineStageBase:
                 if p.grad is None:
                     p.grad = p.main_grad
 
+    def _grad_from(self, consumer: "PipelineStageBase", pos: int, mb: int):
+        if not consumer._bwd_done.get(mb):
+            raise RuntimeError(
+                f"{self.log_prefix} gradient of microbatch {mb} from stage {consumer.stage_index} has not been produced")
+        if consumer.is_native:
+            return consumer._program.mbs[mb].input_grad
+        return consumer._input_grads[mb][pos]
+
     def _backward_eager(self, mb, loss):
         stage_output, input_values = self.fwd_cache.pop(mb)
+        consumers = getattr(self, "_out_consumers", None)
         if self.is_last:
             bwd_kwargs = {"stage_output": loss, "output_grads": None, "input_values": input_values}
+        elif consumers is not None:
+            # every output with its gradient: the sum over the stages that consumed it (the reference
+            # stops at one consumer per output, ``_PipelineStage.py:790-793``)
+            outs, grads = [], []
+            for out_idx, users in consumers.items():
+                total = None
+                for dst, pos in users:
+                    g = self._grad_from(self._stages[dst], pos, mb)
+                    if g is not None:
+                        total = g if total is None else total + g
+                if total is not None:
+                    if out_idx is not None:
+                        outs.append(stage_output[out_idx])
+                    elif isinstance(stage_output, (tuple, list)) and len(stage_output) == 1:
+                        outs.append(stage_output[0])  # the cache holds a single output as a 1-tuple
+                    else:
+                        outs.append(stage_output)
+                    grads.append(total)
+            bwd_kwargs = {"stage_output": tuple(outs), "output_grads": tuple(grads), "input_values": input_values}
         else:
             nxt = self._next
-            if nxt is None or not nxt._bwd_done.get(mb):
-                raise RuntimeError(f"{self.log_prefix} gradient of microbatch {mb} has not been produced")
-            if nxt.is_native:
-                grads = (nxt._program.mbs[mb].input_grad,)
-            else:
+            if nxt is None:
+                raise RuntimeError(f"{self.log_prefix} is not linked to stage {self.stage_index + 1}")
+            grads = (self._grad_from(nxt, 0, mb),) if nxt.is_native else None
+            if grads is None:
+                if not nxt._bwd_done.get(mb):
+                    raise RuntimeError(f"{self.log_prefix} gradient of microbatch {mb} has not been produced")
                 grads = tuple(nxt._input_grads[mb])
             bwd_kwargs = {"stage_output": stage_output, "output_grads": grads, "input_values": input_values}
         self.grads_input = stage_backward(**bwd_kwargs)
@@ -454,15 +499,73 @@ class PipelineStageBase:
         self._bwd_done[mb] = True
 
 
+def _stage_wiring(pipe, stage_index: int):
+    """How the pipe's graph feeds stage ``stage_index`` and who consumes its outputs
+    (reference ``_PipelineStage.py:649-768``).  Returns (routes, consumers, is_chain):
+    routes: per positional input (source stage, output index or None), None for the first stage whose
+    inputs are the user's; consumers: output index (None: the single output) -> [(stage, input
+    position)]; is_chain: the only input is the whole output of the previous stage and the only
+    consumer of the output is the next stage."""
+    import operator
+    nodes = [n for n in pipe.split_gm.graph.nodes if n.op == "call_module" and str(n.target).startswith("submod_")]
+    index_of = {n: i for i, n in enumerate(nodes)}
+    node = nodes[stage_index]
+
+    def source(arg):
+        out_idx = None
+        while arg.op == "call_function" and arg.target is operator.getitem:
+            out_idx = arg.args[1] if out_idx is None else out_idx
+            arg = arg.args[0]
+        return arg, out_idx
+
+    routes = []
+    for arg in node.args:
+        src, out_idx = source(arg)
+        if src.op == "placeholder":
+            if stage_index != 0:
+                raise NotImplementedError(
+                    f"stage {stage_index} reads the model input '{src.name}': only the first stage may "
+                    "(reference _PipelineStage.py:462-470)")
+            routes = None
+            break
+        if src not in index_of:
+            raise RuntimeError(f"stage {stage_index}: unsupported input node {src.format_node()}")
+        routes.append((index_of[src], out_idx))
+    consumers = {}
+    for user in node.users:
+        if user.op == "call_function" and user.target is operator.getitem:
+            dsts = consumers.setdefault(user.args[1], [])
+            for gu in user.users:
+                if gu in index_of:
+                    dsts += [(index_of[gu], pos) for pos, a in enumerate(gu.args) if a is user]
+        elif user in index_of:
+            consumers.setdefault(None, [])
+            consumers[None] += [(index_of[user], pos) for pos, a in enumerate(user.args) if a is node]
+    chain_in = stage_index == 0 or routes == [(stage_index - 1, None)]
+    chain_out = stage_index == len(nodes) - 1 or consumers == {None: [(stage_index + 1, 0)]}
+    if stage_index == 0 and len(node.args) != 1:
+        chain_in = True  # the lowering itself checks that a native first stage takes one tensor
+    return routes, consumers, chain_in and chain_out
+
+
 class PipelineStage(PipelineStageBase):
-    """A stage built from a ``Pipe`` (reference ``_PipelineStage.py:818-833``)."""
+    """A stage built from a ``Pipe`` (reference ``_PipelineStage.py:818-833``).  Inputs follow the
+    pipe's graph: a stage may take several values, from any earlier stage (skip connections,
+    reference ``test/test_skip_conn.py:20-45``); such a stage runs through autograd, and so does one
+    whose output feeds more than the next stage."""
 
     def __init__(self, pipe, stage_index: int, device, group=None, **kw):
         self.pipe = pipe
         self.pipe_info = pipe.info()
         submod = pipe.get_stage_module(stage_index)
+        routes, consumers, is_chain = _stage_wiring(pipe, stage_index)
+        if not is_chain:
+            kw["force_eager"] = True
         super().__init__(submod, stage_index, pipe.num_stages, device, self.pipe_info.num_chunks,
                          group, **kw)
+        if not is_chain or not self.is_native:
+            self._arg_routes = routes
+            self._out_consumers = consumers if stage_index != pipe.num_stages - 1 else None
 
 
 class ManualPipelineStage(PipelineStageBase):
@@ -494,4 +597,5 @@ def link_stages(stages: List[PipelineStageBase]) -> List[PipelineStageBase]:
     for s in ordered:
         s._prev = by_index.get(s.stage_index - 1)
         s._next = by_index.get(s.stage_index + 1)
+        s._stages = by_index
     return ordered

@@ -682,3 +682,57 @@ def test_checkpoint_round_trip_resumes_training_bit_for_bit(tmp_path):
     sd_a, sd_b = model_a.state_dict(), model_b.state_dict()
     for k in sd_a:
         assert torch.equal(sd_a[k], sd_b[k]), k
+
+
+# ---- skip connections: a stage fed by several earlier stages --------------------------------------
+class _SkipNet(torch.nn.Module):
+    """The model of the reference's skip-connection test (``test/test_skip_conn.py:20-45``)."""
+
+    def __init__(self, d=16):
+        super().__init__()
+        self.mm_param0 = torch.nn.Parameter(torch.randn(d, d) * 0.3)
+        self.mm_param1 = torch.nn.Parameter(torch.randn(d, d) * 0.3)
+        self.mm_param2 = torch.nn.Parameter(torch.randn(d, d) * 0.3)
+        self.lin1 = torch.nn.Linear(d, d)
+        self.lin2 = torch.nn.Linear(d, d)
+
+    def forward(self, x, y):
+        import pippy_amd as pp
+        x = torch.mm(x, self.mm_param0)
+        x = torch.relu(x + y)
+        skip_conn = x
+        pp.pipe_split()
+        x = self.lin1(torch.mm(x, self.mm_param1))
+        pp.pipe_split()
+        x = torch.mm(torch.relu(x), self.mm_param2)
+        pp.pipe_split()
+        return torch.relu(self.lin2(x + skip_conn))
+
+
+@pytest.mark.parametrize("schedule", ["ScheduleGPipe", "Schedule1F1B"])
+def test_skip_connection_forward_and_backward_match_the_unsplit_model(schedule):
+    import pippy_amd as pp
+    torch.manual_seed(0)
+    model = _SkipNet()
+    x, y, target = (torch.randn(8, 16, device=DEV) for _ in range(3))
+    pipe = pp.pipeline(model, 4, (x.cpu(),), {"y": y.cpu()})
+    assert pipe.num_stages == 4
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(4)]
+    assert not any(st.is_native for st in stages)
+    loss_fn = torch.nn.MSELoss(reduction="sum")
+    sched = getattr(pp, schedule)(stages, 4, loss_fn=loss_fn)
+    losses = []
+    out = sched.step(x, y=y, target=target, losses=losses)
+    ref = copy.deepcopy(model)   # the stages moved the parameters to the GPU
+    for p in ref.parameters():
+        p.grad = None
+    ref_out = ref(x, y)
+    loss_fn(ref_out, target).backward()
+    torch.testing.assert_close(out, ref_out)
+    torch.testing.assert_close(sum(losses), loss_fn(ref_out, target))
+    # stage 0's output has two consumers (stages 1 and 3): its gradient is their sum
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        g = named[name].grad
+        assert g is not None, name
+        torch.testing.assert_close(g, rp.grad, rtol=1e-4, atol=1e-5)
