@@ -4,6 +4,7 @@ Public names mirror ``pippy/__init__.py:2-43`` of the reference so that a script
 ``pippy`` runs against this package by changing the import.  All stages of a pipeline run as
 virtual stages on one GPU; see ``schedules.py``.
 """
+from . import _debug  # noqa: F401  (sets the logging level from PIPPY_VERBOSITY)
 from ._IR import (ArgsChunkSpec, KwargsChunkSpec, Pipe, PipeSplitWrapper, SplitPoint,
                   annotate_split_points, pipe_split, pipeline)
 from .losses import CrossEntropyLoss

@@ -397,3 +397,19 @@ def test_ctypes_structs_match_the_header(tmp_path):
     want = [ctypes.sizeof(N.CopySeg), ctypes.sizeof(N.GemmDesc), ctypes.sizeof(N.AttnDesc), ctypes.sizeof(N.Op),
             N.Op.i.offset, N.Op.j.offset, N.GemmDesc.bias.offset]
     assert got == want
+
+
+def test_verbosity_from_the_environment():
+    """PIPPY_VERBOSITY sets the package logger's level; an unknown value falls back to WARNING
+    (reference ``pippy/_debug.py:13-18``)."""
+    import logging
+    from pippy_amd import _debug
+    try:
+        assert _debug.configure("DEBUG") == "DEBUG"
+        assert logging.getLogger("pippy_amd").level == logging.DEBUG
+        assert logging.getLogger("pippy_amd.schedules").getEffectiveLevel() == logging.DEBUG
+        assert _debug.configure("LOUD") == "WARNING"
+        assert logging.getLogger("pippy_amd").level == logging.WARNING
+    finally:
+        _debug.configure()
+    assert _debug.map_debug_info([torch.zeros(2, 3), 5]) == ["Tensor((2, 3), grad=False)", "5"]
