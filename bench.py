@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Throughput of the pipeline-stage hot path on one MI355X.
 
-Workload (configs[2] of BASELINE.json, the one the metric's target is quoted on): a
+Workload (the training configuration the headline metric is quoted on): a
 GPT-2-small-shaped decoder (12 layers, d_model 768, 12 heads, FFN 3072, tanh-GELU, pre-LayerNorm,
 causal attention, vocabulary 50257, sequence 1024) cut into 4 virtual stages of 3 layers on one
 GPU, trained with Schedule1F1B over a batch of 32 split into 8 microbatches of 4; bf16 weights and
