@@ -175,9 +175,12 @@ __device__ __forceinline__ void interleave_reads() {
     if constexpr (I + 1 < M) interleave_reads<R, M, I + 1>();
 }
 
-// One BM x BN output tile with NS LDS stages of KT values of k, filled by direct-to-LDS loads.
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
-__device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
+// Main loop of one BM x BN output tile over the k-tiles [kt_begin, kt_end) of KT values each, through
+// NS LDS stages filled by direct-to-LDS loads; the products are added to acc.  Starts with a barrier,
+// so that it may follow an epilogue (or another main loop) that used the same LDS.
+template <int BM, int BN, bool AT, bool BT, int NS, int KT>
+__device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n, int kt_begin,
+                                              int kt_end, f32x16_t (&acc)[BN / 64][BM / 64]) {
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int KS = KT / 16;  // MFMA k-steps per tile
@@ -193,22 +196,14 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
 
-    f32x16_t acc[TN][TM];
-#pragma unroll
-    for (int a = 0; a < TN; ++a)
-#pragma unroll
-        for (int b = 0; b < TM; ++b)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
-
     DmaStage<BM, AT, KT> sa;
     DmaStage<BN, BT, KT> sb;
     sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
     sb.init(g.B, g.ldb, n0, g.N, g.K, wave, lane);
-    const int nk = (int)((g.K + KT - 1) / KT);
+    const int nk = kt_end - kt_begin;
     auto issue = [&](int stage, int kt) {
-        sa.load(smem + stage * kStageElems, kt * KT, wave);
-        sb.load(smem + stage * kStageElems + BM * KT, kt * KT, wave);
+        sa.load(smem + stage * kStageElems, (kt_begin + kt) * KT, wave);
+        sb.load(smem + stage * kStageElems + BM * KT, (kt_begin + kt) * KT, wave);
     };
 
     FragReader<BM, AT, KT> ra[TM];
@@ -234,6 +229,8 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
     auto interleave = [&]() { interleave_reads<kReadsPerStep, TM * TN, 0>(); };
 
     // prologue: tiles 0 .. NS-1 in flight, tile 0 awaited
+    wait_lds();
+    __builtin_amdgcn_s_barrier();  // whatever used the stages before is done with them
 #pragma unroll
     for (int t = 0; t < NS; ++t)
         if (t < nk) issue(t, t);
@@ -264,10 +261,20 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
         if (kt + 1 < nk) read_frags(0, smem + stage * kStageElems, 0);
         mma(kLast, TN / 2, TN);
     }
+}
 
-    // Epilogue: one band of 32 rows at a time goes through a wave-private LDS region as fp32,
-    // [32][WTN] with the 16-byte unit index XORed by the row, and comes back with lanes running
-    // along n, so that epilogue4 reads and writes whole lines.
+// Epilogue of one BM x BN tile: one band of 32 rows at a time goes through a wave-private LDS region
+// as fp32, [32][WTN] with the 16-byte unit index XORed by the row, and comes back with lanes running
+// along n, so that epilogue4 reads and writes whole lines.
+template <int BM, int BN, int EPI, bool CF32>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
+                                              f32x16_t (&acc)[BN / 64][BM / 64]) {
+    constexpr int WTM = BM / 2, WTN = BN / 2;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
     wait_lds();
     __builtin_amdgcn_s_barrier();  // every wave is done with the stages
     const int l32 = lane & 31, lh = lane >> 5;
@@ -347,6 +354,20 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
             }
         }
     }
+}
+
+// One whole output tile: main loop over all of K, then the epilogue.
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
+__device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
+    f32x16_t acc[BN / 64][BM / 64];
+#pragma unroll
+    for (int a = 0; a < BN / 64; ++a)
+#pragma unroll
+        for (int b = 0; b < BM / 64; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+    gemm_mainloop<BM, BN, AT, BT, NS, KT>(g, tile_m, tile_n, 0, (int)((g.K + KT - 1) / KT), acc);
+    gemm_epilogue<BM, BN, EPI, CF32>(g, tile_m, tile_n, acc);
 }
 
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
