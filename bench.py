@@ -219,6 +219,24 @@ def main():
         mbytes = 2.0 * merged.numel() * merged.element_size()
         hbm["merge"] = {"achieved": round(mbytes / (mms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(mbytes / (mms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(mms, 3)}
+        # the split kernel at a size that shows its bandwidth: the step's own split moves 0.5 MB of
+        # token ids (and a split along dim 0 of a contiguous tensor is a set of views), so the merged
+        # logits are split along the sequence dimension, which copies every chunk
+        from pippy_amd.microbatch import TensorChunkSpec, split_args_kwargs_into_chunks
+        spec = (TensorChunkSpec(1),)
+        split_args_kwargs_into_chunks((merged,), None, args.microbatches, spec)
+        ev0.record()
+        for _ in range(5):
+            split_args_kwargs_into_chunks((merged,), None, args.microbatches, spec)
+        ev1.record()
+        torch.cuda.synchronize()
+        sms = ev0.elapsed_time(ev1) / 5
+        hbm["split_logits_sized"] = {"achieved": round(mbytes / (sms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                                     "unit": "GB/s", "frac": round(mbytes / (sms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                     "ms": round(sms, 3),
+                                     "note": "8-way split of the merged logits along dim 1; not part of the "
+                                             "step, whose own split is 0.5 MB of token ids"}
+        del merged
         # the optimizer step that follows schedule.step() in training: timed alone, outside `value`
         import pippy_amd as pp
         opt = pp.FusedAdamW(stages, lr=1e-4, weight_decay=0.1)

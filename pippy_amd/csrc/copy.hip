@@ -64,12 +64,12 @@ __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int64_t off = (int64_t)(u * kThreads + tid) * V;
-            r[u] = *reinterpret_cast<const vec*>(sp + (off < left ? off : last));
+            r[u] = __builtin_nontemporal_load(reinterpret_cast<const vec*>(sp + (off < left ? off : last)));
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int64_t off = (int64_t)(u * kThreads + tid) * V;
-            if (off < left) *reinterpret_cast<vec*>(dp + off) = r[u];
+            if (off < left) __builtin_nontemporal_store(r[u], reinterpret_cast<vec*>(dp + off));
         }
     } else {
         // short rows: several whole rows per block
@@ -102,10 +102,13 @@ __global__ __launch_bounds__(kThreads) void copy_rows_kernel(const CopyTable t) 
 // destination is aligned per row by a short scalar head, the body moves as aligned 16-byte stores
 // fed by unaligned 16-byte loads, and a scalar tail finishes the row.  A = common alignment (bytes)
 // of all pointers, strides and row lengths.
-template <int A>
-struct __attribute__((packed, aligned(A))) Unaligned16 {
-    uint32_t w[4];
-};
+template <int A> struct Unaligned16;
+#define PP_UNALIGNED16(A)                                                                    \
+    template <> struct Unaligned16<A> {                                                      \
+        typedef unsigned int type __attribute__((ext_vector_type(4), aligned(A)));          \
+    };
+PP_UNALIGNED16(1) PP_UNALIGNED16(2) PP_UNALIGNED16(4) PP_UNALIGNED16(8)
+#undef PP_UNALIGNED16
 
 template <int A>
 __global__ __launch_bounds__(kThreads) void copy_rows_unaligned_kernel(const CopyTable t) {
@@ -129,14 +132,18 @@ __global__ __launch_bounds__(kThreads) void copy_rows_unaligned_kernel(const Cop
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t vi = v0 + u * kThreads + tid;
         if (vi < nv) {
-            const Unaligned16<A> v = *reinterpret_cast<const Unaligned16<A>*>(sp + head + vi * 16);
-            r[u] = make_uint4(v.w[0], v.w[1], v.w[2], v.w[3]);
+            typedef typename Unaligned16<A>::type src_vec;
+            const copy_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const src_vec*>(sp + head + vi * 16));
+            r[u] = make_uint4(v.x, v.y, v.z, v.w);
         }
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t vi = v0 + u * kThreads + tid;
-        if (vi < nv) *reinterpret_cast<uint4*>(dp + head + vi * 16) = r[u];
+        if (vi < nv) {
+            const copy_u32x4_t w = {r[u].x, r[u].y, r[u].z, r[u].w};
+            __builtin_nontemporal_store(w, reinterpret_cast<copy_u32x4_t*>(dp + head + vi * 16));
+        }
     }
     if (cblk == 0) {
         for (int64_t i = (int64_t)tid * A; i < head; i += kThreads * A)
