@@ -37,9 +37,12 @@ GEMM_TRAFFIC_BYTES_PER_LAUNCH = 114.8e6
 
 
 def build(args):
+    """Model, schedule, stages and the step's inputs for the chosen workload."""
     import pippy_amd as pp
     from pippy_amd.configs import DecoderLM, equal_split_spec
     torch.manual_seed(0)
+    if args.workload != "gpt2":
+        return build_other(args)
     model = DecoderLM(vocab=args.vocab, max_seq=args.seq, dim=args.dim, n_layers=args.layers,
                       n_heads=args.heads, ffn=args.ffn)
     ids = torch.randint(0, args.vocab, (args.batch, args.seq))
@@ -52,6 +55,74 @@ def build(args):
                  "zero_bubble": pp.ScheduleZeroBubble}[args.schedule]
     sched = sched_cls(stages, args.microbatches, loss_fn=pp.CrossEntropyLoss())
     return model, sched, stages, ids.cuda(), target.cuda()
+
+
+def _upstream_loss(out, upstream):
+    """A loss whose gradient w.r.t. the stage output is `upstream` (what a middle stage receives)."""
+    return (out.float() * upstream).sum()
+
+
+def build_other(args):
+    """The other baseline configurations at full size (each sets its own shape; the --vocab ... --stages
+    options only shape the default workload).  Sets args.describe / args.tokens / args.flops."""
+    import pippy_amd as pp
+    from pippy_amd.configs import bert_base, equal_split_spec, llama2_7b_stage, mixtral_style
+    if args.workload == "bert":
+        # BERT-base-shaped encoder, inference, GPipe: batch 64 x 512 in 8 microbatches, 4 stages
+        model = bert_base()
+        ids = torch.randint(0, 30522, (64, 512))
+        pipe = pp.pipeline(model, 8, (ids,), split_spec=equal_split_spec(12, 4))
+        stages = [pp.PipelineStage(pipe, i, "cuda") for i in range(4)]
+        sched = pp.ScheduleGPipe(stages, 8)
+        args.tokens, args.training = ids.numel(), False
+        per_token = 12 * (2 * 768 * 3 * 768 + 2 * 768 * 768 + 4 * 768 * 3072 + 4 * 512 * 768)
+        args.flops = float(per_token) * ids.numel()
+        args.describe = ("BERT-base-shaped encoder (12 post-LayerNorm layers, hidden 768, 12 heads, FFN 3072, "
+                         "vocab 30522, seq 512), inference, 4 virtual stages on one GPU, schedule gpipe, "
+                         "batch 64 in 8 microbatches, bf16")
+        args.batch, args.seq = 64, 512
+        return model, sched, stages, ids.cuda(), None
+    if args.workload == "llama":
+        # one stage of a Llama-2-7B-shaped PP=4 pipeline, zero-bubble: 16 microbatches of one sequence
+        M = 16
+        with torch.device("cuda"):
+            model = llama2_7b_stage()
+            x = torch.randn(M, 2048, 4096).to(torch.bfloat16)
+            upstream = torch.randn(M, 2048, 4096) * 1e-2
+        stage = pp.ManualPipelineStage(model, 0, 1, "cuda", M, input_args=(x[:1],),
+                                       fused_accumulate=args.fused_accumulate)
+        sched = pp.ScheduleZeroBubble([stage], M, loss_fn=_upstream_loss)
+        T = M * 2048
+        per_layer = 4 * 4096 ** 2 + 3 * 4096 * 11008
+        args.tokens, args.training = T, True
+        args.flops = 3.0 * (2.0 * T * per_layer * 8 + 8 * 4.0 * T * 2048 * 4096)
+        args.describe = ("one stage (8 layers) of a Llama-2-7B-shaped pipeline (d_model 4096, 32 heads of 128, "
+                         "SwiGLU 11008, RMSNorm, RoPE, seq 2048), zero-bubble schedule with separate dI and dW "
+                         "passes, 16 microbatches of one sequence, upstream gradients N(0, 1e-2), bf16 with fp32 "
+                         f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+        args.batch, args.seq = M, 2048
+        return model, sched, [stage], x, upstream
+    if args.workload == "moe":
+        # Mixtral-style MoE, interleaved 1F1B: 2 virtual stages of 4 layers on one rank
+        with torch.device("cuda"):
+            model = mixtral_style()
+        ids = torch.randint(0, 32000, (16, 1024))
+        target = torch.randint(0, 32000, (16, 1024))
+        pipe = pp.pipeline(model, 8, (ids,), split_spec=equal_split_spec(8, 2))
+        stages = [pp.PipelineStage(pipe, i, "cuda", group=1, fused_accumulate=args.fused_accumulate)
+                  for i in range(2)]
+        sched = pp.ScheduleInterleaved1F1B(stages, 8, loss_fn=pp.CrossEntropyLoss())
+        T = ids.numel()
+        active = 4 * 1024 ** 2 + 2 * 3 * 1024 * 4096 + 8 * 1024   # attention, two experts, router
+        args.tokens, args.training = T, True
+        args.flops = 3.0 * (2.0 * T * (active * 8 + 1024 * 32000) + 8 * 4.0 * T * 1024 * 1024)
+        args.describe = ("Mixtral-style decoder (8 layers in 2 virtual stages, d_model 1024, 16 heads, 8 experts "
+                         "with SwiGLU 4096, top-2 router, vocab 32000, seq 1024), schedule interleaved 1f1b on one "
+                         "rank, batch 16 in 8 microbatches, bf16 with fp32 gradient accumulation "
+                         f"({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+        args.batch, args.seq = 16, 1024
+        return model, sched, stages, ids.cuda(), target.cuda()
+    raise ValueError(args.workload)
 
 
 def flops_per_step(args):
@@ -109,6 +180,10 @@ def main():
     ap.add_argument("--serial-stages", action="store_true",
                     help="run all virtual stages on one stream instead of one stream per stage")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe"],
+                    help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
+                         "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
+                         "configurations at full size")
     # workload shape (defaults: GPT-2 small, configs[2])
     ap.add_argument("--vocab", type=int, default=50257)
     ap.add_argument("--seq", type=int, default=1024)
@@ -132,12 +207,16 @@ def main():
     from pippy_amd import _native as N
     N.lib()  # fail loudly if the kernel library is missing
     model, sched, stages, ids, target = build(args)
-    tokens = ids.numel()
+    default_workload = args.workload == "gpt2"
+    tokens = ids.numel() if default_workload else args.tokens
+    training = True if default_workload else args.training
     sched.concurrent_stages = not args.serial_stages
 
     def step():
-        sched.zero_grad()
         losses = []
+        if not training:
+            return sched.step(ids), losses
+        sched.zero_grad()
         out = sched.step(ids, target=target, losses=losses)
         return out, losses
 
@@ -151,21 +230,23 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     value = tokens * args.steps / dt
-    loss0 = float(losses[0])
+    loss0 = float(losses[0]) if losses else None
 
     result = {
         "metric": "tokens/sec per schedule step on 1 MI355X + stage GEMM MFMA util %",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"GPT-2-small-shaped decoder ({args.layers} layers, d_model {args.dim}, "
-                               f"{args.heads} heads, FFN {args.ffn}, vocab {args.vocab}, seq {args.seq}), "
-                               f"{args.stages} virtual stages on one GPU, schedule {args.schedule}, "
-                               f"batch {args.batch} in {args.microbatches} microbatches, bf16 with fp32 "
-                               f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})",
+        "config": {"workload": (f"GPT-2-small-shaped decoder ({args.layers} layers, d_model {args.dim}, "
+                                f"{args.heads} heads, FFN {args.ffn}, vocab {args.vocab}, seq {args.seq}), "
+                                f"{args.stages} virtual stages on one GPU, schedule {args.schedule}, "
+                                f"batch {args.batch} in {args.microbatches} microbatches, bf16 with fp32 "
+                                f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+                               if default_workload else args.describe,
                    "global_batch": args.batch, "seq_len": args.seq},
-        "step_tflops": round(flops_per_step(args) / (ms_per_step * 1e-3) / 1e12, 1),
-        "loss_microbatch0": round(loss0, 4),
+        "step_tflops": round((flops_per_step(args) if default_workload else args.flops)
+                             / (ms_per_step * 1e-3) / 1e12, 1),
+        "loss_microbatch0": round(loss0, 4) if loss0 is not None else None,
     }
 
     if not args.no_roofline:
@@ -183,11 +264,14 @@ def main():
         N.profile_stop()
         sched.concurrent_stages = not args.serial_stages
         ms, work, cnt = N.profile_read(N.OP_GEMM_BF16)
+        sms_, swork, scnt = N.profile_read(N.OP_GEMM_SEG)   # expert GEMMs of a mixture-of-experts layer
+        ms, work, cnt = ms + sms_, work + swork, cnt + scnt
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
-                              "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
-                              "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel",
+                              "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
+                              "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel"
+                                        + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else ""),
                               "launches_per_step": cnt // n_prof,
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
                               "gemm_ms_per_step": round(ms / n_prof, 3)}
@@ -205,6 +289,10 @@ def main():
                 tf = kwork / (kms * 1e-3) / 1e12
                 hbm[name] = {"achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s (dense count)",
                              "frac": round(tf / MFMA_PEAK_TFLOPS, 4), "ms_per_step": round(kms / n_prof, 3)}
+        if not default_workload:
+            result["other_kernels"] = hbm
+            print(json.dumps(result))
+            return
         # the merge of the logits chunks runs outside the launch lists: time it alone
         from pippy_amd.microbatch import merge_chunks
         chunks = stages[-1].output_chunks
@@ -252,7 +340,7 @@ def main():
                              "frac": round(obytes / (oms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(oms, 3)}
         result["other_kernels"] = hbm
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and default_workload:
         result["cpu_baseline"] = cpu_baseline(args)
 
     print(json.dumps(result))

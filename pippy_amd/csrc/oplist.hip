@@ -175,6 +175,7 @@ double op_work(const pp_op& op) {
     switch (op.kind) {
         case PP_OP_GEMM_BF16:
         case PP_OP_GEMM_F32:
+        case PP_OP_GEMM_SEG:  // the segments partition the rows (rows mode: M, k mode: K)
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_ATTN_FWD:  // dense count: QK^T and PV
             return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[1] * (double)op.i[1] * (double)op.i[3];
@@ -210,6 +211,10 @@ double op_work(const pp_op& op) {
             return 10.0 * (double)op.i[0];
         case PP_OP_ROPE:
             return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[3];
+        case PP_OP_MOE_GATHER:  // read and write R rows of C bf16
+            return 4.0 * (double)op.i[3] * (double)op.i[4];
+        case PP_OP_MOE_COMBINE:  // read topk rows (+ the residual), write one, per token
+            return 2.0 * ((double)op.i[1] + (op.p[3] ? 2.0 : 1.0)) * (double)op.i[4] * (double)op.i[5];
         default:
             return 0.0;
     }
