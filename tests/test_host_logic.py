@@ -24,18 +24,25 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 # ---- microbatch split (views of host tensors; no data movement) -----------------------------------
+def _golden(name):
+    import json
+    with open(os.path.join(ROOT, "tests", "golden", name)) as f:
+        return json.load(f)
+
+
 def test_split_shapes_of_the_reference_test():
-    """test/test_microbatch.py:17-34 of the reference."""
-    d = 512
-    x0, x1, x2 = torch.randn(128, d), torch.randn(256, d), torch.randn(512, d)
-    args, kwargs = (x0, x1, x2), {"x0": x0, "x1": x1, "x2": x2}
-    a, k = split_args_kwargs_into_chunks(args, kwargs, 2)
-    assert len(a) == 2 and len(k) == 2
-    assert a[0][0].shape == (64, d) and a[1][0].shape == (64, d)
-    assert a[0][1].shape == (128, d) and a[0][2].shape == (256, d)
-    assert k[0]["x0"].shape == (64, d) and k[0]["x1"].shape == (128, d) and k[1]["x2"].shape == (256, d)
+    """The chunk shapes that test/test_microbatch.py:17-34 of the reference asserts."""
+    gold = _golden("microbatch_split_shapes.json")
+    d, n = gold["width"], gold["chunks"]
+    xs = [torch.randn(r, d) for r in gold["rows"]]
+    args, kwargs = tuple(xs), {f"x{i}": x for i, x in enumerate(xs)}
+    a, k = split_args_kwargs_into_chunks(args, kwargs, n)
+    assert len(a) == n and len(k) == n
+    for c in range(n):
+        assert [tuple(t.shape) for t in a[c]] == [(r, d) for r in gold["chunk_rows"][c]]
+        assert [tuple(k[c][f"x{i}"].shape) for i in range(len(xs))] == [(r, d) for r in gold["chunk_rows"][c]]
     # chunks are views of the caller's tensors, as in the reference (no bytes move)
-    assert a[1][0].data_ptr() == x0[64:].data_ptr()
+    assert a[1][0].data_ptr() == xs[0][64:].data_ptr()
     for i, x in enumerate(args):
         assert torch.equal(torch.cat([c[i] for c in a]), x)
 
@@ -110,7 +117,10 @@ def test_row_view_descriptions():
 
 # ---- schedule orders ----------------------------------------------------------------------------------
 def test_1f1b_phases_known_answer():
-    assert [order.one_f_one_b_phases(s, 4, 8) for s in range(4)] == [(6, 2, 6), (4, 4, 4), (2, 6, 2), (0, 8, 0)]
+    """The worked example in the reference's comment at PipelineSchedule.py:373-377."""
+    gold = _golden("schedule_1f1b_phases.json")
+    S, M = gold["num_stages"], gold["num_microbatches"]
+    assert [list(order.one_f_one_b_phases(s, S, M)) for s in range(S)] == gold["phases_per_stage"]
 
 
 @pytest.mark.parametrize("S,M", [(1, 1), (2, 4), (4, 8), (4, 2), (3, 7)])
