@@ -156,7 +156,9 @@ def check(rc: int, what: str) -> None:
 
 
 def current_stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current HIP stream (what ``torch.cuda.current_stream().cuda_stream``
+    returns, without building the Python wrapper objects: this is called once per launch list)."""
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:

@@ -21,6 +21,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 from torch.profiler import record_function
+from contextlib import nullcontext
 
 from . import _schedule_order as order
 from .microbatch import merge_chunks, split_args_kwargs_into_chunks
@@ -199,10 +200,16 @@ class PipelineSchedule(ABC):
             done.record(w_streams[s])
             main.wait_event(done)
 
+    @staticmethod
+    def _range(name: str):
+        """A profiler range with the reference's names (``PipelineSchedule.py:540,557``); entering one
+        costs tens of microseconds, so it is only opened while a torch profiler is recording."""
+        return record_function(name) if torch.autograd.profiler._is_profiler_enabled else nullcontext()
+
     def _run_action(self, kind, s, m, arg_mbs, kwarg_mbs, target_mbs):
         stage = self._by_index[s]
         if kind == "F":
-            with record_function(f"Stage {s} Forward {m}"):
+            with self._range(f"Stage {s} Forward {m}"):
                 if stage.fwd_chunk_id != m:
                     raise RuntimeError(f"stage {s}: forward order broken ({stage.fwd_chunk_id} != {m})")
                 a = arg_mbs[m] if stage.is_first else ()
@@ -210,15 +217,15 @@ class PipelineSchedule(ABC):
                 output = stage.forward_one_chunk(a, k)
                 self._maybe_compute_loss(stage, output, target_mbs, m)
         elif kind == "B":
-            with record_function(f"Stage {s} Backward {m}"):
+            with self._range(f"Stage {s} Backward {m}"):
                 if stage.bwd_chunk_id != m:
                     raise RuntimeError(f"stage {s}: backward order broken ({stage.bwd_chunk_id} != {m})")
                 stage.backward_one_chunk(loss=self._maybe_get_loss(stage, m))
         elif kind == "I":
-            with record_function(f"Stage {s} BackwardInput {m}"):
+            with self._range(f"Stage {s} BackwardInput {m}"):
                 stage.backward_input_one_chunk(loss=self._maybe_get_loss(stage, m))
         elif kind == "W":
-            with record_function(f"Stage {s} BackwardWeight {m}"):
+            with self._range(f"Stage {s} BackwardWeight {m}"):
                 stage.backward_weight_one_chunk()
         else:
             raise ValueError(f"unknown action {kind}")
