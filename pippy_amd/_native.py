@@ -319,6 +319,8 @@ def gemm_bf16_segmented(A, B_or_C_list: torch.Tensor, Cm, seg_start: torch.Tenso
     assert seg_start.dtype == torch.int32 and B_or_C_list.dtype == torch.int64
     n_seg = seg_start.numel() - 1
     assert B_or_C_list.numel() == n_seg
+    if mode not in (SEG_ROWS, SEG_K):
+        raise ValueError(f"unknown mode {mode}: SEG_ROWS or SEG_K")
     d = GemmDesc()
     if mode == SEG_ROWS:
         assert A.stride(1) == 1 and Cm.stride(1) == 1 and A.shape[0] == Cm.shape[0]

@@ -792,3 +792,41 @@ def test_segmented_gemm_k_mode(R, M, Nn, E):
     N.gemm_bf16_segmented(dY.to(DEV), ptrs, None, segd, N.SEG_K, other=X.to(DEV), epilogue=N.EPI_ACCUM_F32,
                           beta=1, c_dtype=torch.float32)
     assert_close_rel(acc, ref + 1.0, 1e-3, "segmented k, fp32 accumulate")
+
+
+@pytest.mark.gpu
+def test_moe_and_segmented_entry_points_reject_bad_arguments():
+    Nn = native()
+    seg = torch.tensor([0, 4, 8], dtype=torch.int32, device=DEV)
+    A = torch.zeros(8, 64, device=DEV, dtype=torch.bfloat16)
+    W = torch.zeros(2, 16, 64, device=DEV, dtype=torch.bfloat16)
+    ptrs = torch.tensor([W[0].data_ptr(), W[1].data_ptr()], dtype=torch.int64, device=DEV)
+    Cm = torch.zeros(8, 16, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="rows mode epilogue"):
+        Nn.gemm_bf16_segmented(A, ptrs, Cm, seg, Nn.SEG_ROWS, epilogue=Nn.EPI_BIAS_RELU)
+    with pytest.raises(ValueError, match="unknown mode"):
+        Nn.gemm_bf16_segmented(A, ptrs, Cm, seg, 7)
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        Nn.gemm_bf16_segmented(A[:, :60], ptrs, Cm, seg, Nn.SEG_ROWS)
+    logits = torch.zeros(4, 1, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="pp_moe_router_top2"):
+        Nn.moe_router_top2(logits, torch.zeros(4, 2, dtype=torch.int32, device=DEV),
+                           torch.zeros(4, 2, device=DEV))
+    slots = torch.zeros(4, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="at most 64 experts"):
+        Nn.moe_permute(slots, 65, torch.zeros(66, dtype=torch.int32, device=DEV), slots.clone(), slots.clone())
+    x = torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16)       # width not a multiple of 8
+    with pytest.raises(RuntimeError, match="pp_moe_gather"):
+        Nn.moe_gather(x, slots, 1, torch.zeros(4, 12, device=DEV, dtype=torch.bfloat16))
+
+
+@pytest.mark.gpu
+def test_moe_layer_with_an_expert_count_that_is_not_a_multiple_of_8_raises_on_lowering():
+    import pippy_amd as pp
+    from pippy_amd.stage_modules import MoELayer
+    layer = MoELayer(128, 2, 256, n_experts=4)
+    x = torch.randn(2, 128, 128, device=DEV).to(torch.bfloat16)
+    stage = pp.ManualPipelineStage(layer, 0, 1, DEV, 1, input_args=(x,))
+    assert stage.is_native
+    with pytest.raises(RuntimeError, match="multiple of 8 experts"):
+        pp.ScheduleGPipe([stage], 1).step(x)
