@@ -137,6 +137,12 @@ class Pipe(nn.Module):
             raise RuntimeError("Pipe info is not available. Please use the `pipeline` method to create the `Pipe` object.")
         return self.pipe_info
 
+    def build_stage(self, stage_index: int, device, group=None, **kw):
+        """The runtime stage for ``stage_index`` (the spelling of the reference's examples,
+        ``examples/llama/pippy_llama.py:36-39``); same as ``PipelineStage(pipe, stage_index, device, group)``."""
+        from .stage import PipelineStage
+        return PipelineStage(self, stage_index, device, group, **kw)
+
     def __str__(self):
         return self.split_gm.__str__()
 
@@ -258,18 +264,30 @@ def annotate_split_points(mod: nn.Module, spec: Dict[str, SplitPoint]):
         target.forward = make()
 
 
-def pipeline(module: nn.Module, num_chunks: int, example_args: Tuple[Any, ...],
+def pipeline(module: nn.Module, num_chunks: Optional[int] = None, example_args: Optional[Tuple[Any, ...]] = None,
              example_kwargs: Optional[Dict[str, Any]] = None,
              split_spec: Optional[Dict[str, SplitPoint]] = None,
-             split_policy: Optional[Callable[[fx.GraphModule], fx.GraphModule]] = None) -> Pipe:
+             split_policy: Optional[Callable[[fx.GraphModule], fx.GraphModule]] = None, *,
+             mb_args: Optional[Tuple[Any, ...]] = None, mb_kwargs: Optional[Dict[str, Any]] = None) -> Pipe:
     """Splits ``module`` into pipeline stages (reference ``_IR.py:1341-1395``).
 
     ``split_spec`` maps submodule names to ``SplitPoint.BEGINNING`` / ``END``; alternatively the
     model's ``forward`` may call ``pipe_split()``, or ``split_policy`` may place the markers on the
     traced graph.  ``num_chunks`` and the example inputs describe one full batch; the chunk specs
-    in force (``ArgsChunkSpec`` / ``KwargsChunkSpec``) are recorded for the schedules."""
+    in force (``ArgsChunkSpec`` / ``KwargsChunkSpec``) are recorded for the schedules.
+
+    The reference's examples are written against the later spelling of this call,
+    ``pipeline(module, mb_args=..., mb_kwargs=...)`` with the inputs of ONE microbatch
+    (``examples/huggingface/pippy_gpt2.py:50-65``); it is accepted too: the number of microbatches
+    is then the schedule's ``n_microbatches``."""
     if split_spec is not None and split_policy is not None:
         raise ValueError("Cannot specify both `split_spec` and `split_policy`. Please use only one of them.")
+    if mb_args is not None or mb_kwargs is not None:
+        if num_chunks is not None or example_args is not None or example_kwargs is not None:
+            raise ValueError("pass either (num_chunks, example_args, example_kwargs) or (mb_args, mb_kwargs)")
+        num_chunks, example_args, example_kwargs = 1, tuple(mb_args or ()), mb_kwargs
+    if num_chunks is None or example_args is None:
+        raise TypeError("pipeline() needs num_chunks and example_args (or mb_args)")
     return Pipe.from_tracing(mod=module, num_chunks=num_chunks, example_args=example_args,
                              example_kwargs=example_kwargs, split_policy=split_policy,
                              split_spec=split_spec)

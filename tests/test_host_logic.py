@@ -423,3 +423,23 @@ def test_verbosity_from_the_environment():
     finally:
         _debug.configure()
     assert _debug.map_debug_info([torch.zeros(2, 3), 5]) == ["Tensor((2, 3), grad=False)", "5"]
+
+
+def test_pipeline_accepts_the_microbatch_spelling_and_build_stage():
+    """``pipeline(module, mb_args=...)`` and ``pipe.build_stage(i, device)``, as the reference's examples
+    call them (examples/huggingface/pippy_gpt2.py:50-65, examples/llama/pippy_llama.py:36-39)."""
+    torch.manual_seed(0)
+    model = _Net()
+    x = torch.randn(8, 16)
+    a = pp.pipeline(model, 4, (x,), split_spec={"layer1": pp.SplitPoint.BEGINNING})
+    b = pp.pipeline(model, mb_args=(x[:2],), split_spec={"layer1": pp.SplitPoint.BEGINNING})
+    assert a.num_stages == b.num_stages == 2
+    for i in range(2):
+        assert list(a.get_stage_module(i).state_dict()) == list(b.get_stage_module(i).state_dict())
+    assert torch.equal(b(x), model(x))
+    stage = b.build_stage(1, "cpu")
+    assert isinstance(stage, pp.PipelineStage) and stage.stage_index == 1 and stage.num_stages == 2
+    with pytest.raises(ValueError, match="either"):
+        pp.pipeline(model, 4, (x,), mb_args=(x,))
+    with pytest.raises(TypeError, match="num_chunks"):
+        pp.pipeline(model)
