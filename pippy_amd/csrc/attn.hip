@@ -615,7 +615,7 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
     if (d->B < 0 || d->S < 0 || d->H <= 0) return fail(PP_ERR_INVALID, "%s: bad shape", who);
     if (d->D != 64 && d->D != 128)
         return fail(PP_ERR_UNSUPPORTED, "%s: head_dim %lld (64 and 128 are built)", who, (long long)d->D);
-    if (d->S % 128) return fail(PP_ERR_UNSUPPORTED, "%s: S %% 128 != 0 (S=%lld)", who, (long long)d->S);
+    if (d->S % 64) return fail(PP_ERR_UNSUPPORTED, "%s: S %% 64 != 0 (S=%lld)", who, (long long)d->S);
     if ((d->stride_s % 8) || (d->stride_b % 8)) return fail(PP_ERR_INVALID, "%s: strides must be multiples of 8", who);
     if (d->stride_s < d->H * d->D) return fail(PP_ERR_INVALID, "%s: stride_s < H*D", who);
     if (!d->q || !d->k || !d->v || !d->o || !d->lse) return fail(PP_ERR_INVALID, "%s: null pointer", who);
