@@ -175,26 +175,38 @@ __device__ __forceinline__ void interleave_reads() {
     if constexpr (I + 1 < M) interleave_reads<R, M, I + 1>();
 }
 
+// How the 4 waves of a work-group share a BM x BN tile: 2 x 2 when BN is a multiple of 64, else 4 x 1
+// (a 128 x 96 tile: each wave 32 rows by 96 columns).  A wave's part is TM x TN MFMA tiles of 32 x 32.
+template <int BM, int BN>
+struct WaveTile {
+    static constexpr int WGN = (BN % 64 == 0) ? 2 : 1;
+    static constexpr int WGM = 4 / WGN;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    static constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "a wave's part of the tile is made of 32 x 32 MFMA tiles");
+};
+
 // Main loop of one BM x BN output tile over the k-tiles [kt_begin, kt_end) of KT values each, through
 // NS LDS stages filled by direct-to-LDS loads; the products are added to acc.  Starts with a barrier,
 // so that it may follow an epilogue (or another main loop) that used the same LDS.
 template <int BM, int BN, bool AT, bool BT, int NS, int KT>
 __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n, int kt_begin,
-                                              int kt_end, f32x16_t (&acc)[BN / 64][BM / 64]) {
-    constexpr int WTM = BM / 2, WTN = BN / 2;
-    constexpr int TM = WTM / 32, TN = WTN / 32;
+                                              int kt_end,
+                                              f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
+    typedef WaveTile<BM, BN> WT;
+    constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     constexpr int KS = KT / 16;  // MFMA k-steps per tile
     constexpr int kStageElems = (BM + BN) * KT;
     constexpr int LPT = DmaStage<BM, AT, KT>::kLoads + DmaStage<BN, BT, KT>::kLoads;  // loads per tile per wave
     constexpr int kReadsPerStep = TM * FragReader<BM, AT, KT>::kReads + TN * FragReader<BN, BT, KT>::kReads;
     static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
-    static_assert(KS >= 2 && TN % 2 == 0, "the last k-step is split in two halves around the barrier");
+    static_assert(KS >= 2 && TN >= 2, "the last k-step is split in two parts around the barrier");
     static_assert(NS * kStageElems * 2 >= 4 * 32 * WTN * 4, "the epilogue stages fp32 bands in the tile memory");
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
+    const int wm0 = (wave % WT::WGM) * WTM, wn0 = (wave / WT::WGM) * WTN;
 
     DmaStage<BM, AT, KT> sa;
     DmaStage<BN, BT, KT> sb;
@@ -268,20 +280,27 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
 // along n, so that epilogue4 reads and writes whole lines.
 template <int BM, int BN, int EPI, bool CF32>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
-                                              f32x16_t (&acc)[BN / 64][BM / 64]) {
-    constexpr int WTM = BM / 2, WTN = BN / 2;
-    constexpr int TM = WTM / 32, TN = WTN / 32;
+                                              f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
+    typedef WaveTile<BM, BN> WT;
+    constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave & 1) * WTM, wn0 = (wave >> 1) * WTN;
+    const int wm0 = (wave % WT::WGM) * WTM, wn0 = (wave / WT::WGM) * WTN;
     wait_lds();
     __builtin_amdgcn_s_barrier();  // every wave is done with the stages
     const int l32 = lane & 31, lh = lane >> 5;
     float* cw = reinterpret_cast<float*>(smem) + wave * (32 * WTN);
     constexpr int UPR = WTN / 4;   // 16-byte units per row
     constexpr int RPP = 64 / UPR;  // rows per pass of the wave
+    static_assert(UPR % 8 == 0 && 32 % RPP == 0, "the unit swizzle works on groups of 8 units");
+    // With 24 units per row (96 columns) two rows fill 48 lanes of a pass and 16 lanes sit out.
+    const bool lane_on = lane < RPP * UPR;
     const int ru = lane % UPR, rr = lane / UPR;
+    // unit u of row r lives at unit (u with its low 3 bits XORed by r) when UPR is not a power of two
+    auto unit_at = [](int u, int r) {
+        return (UPR & (UPR - 1)) == 0 ? (u ^ (r & (UPR - 1))) : ((u & ~7) | ((u ^ r) & 7));
+    };
     const bool vec_ok = CF32 ? ((g.ldc & 3) == 0 && aligned(g.C, 16))
                              : ((g.ldc & 3) == 0 && aligned(g.C, 8) && (g.ld_aux & 3) == 0 &&
                                 aligned(g.aux_in, 8) && aligned(g.aux_out, 8));
@@ -299,18 +318,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int u = a * 8 + 2 * q + lh;
-                *reinterpret_cast<float4*>(cw + l32 * WTN + ((u ^ (l32 & (UPR - 1))) << 2)) =
+                *reinterpret_cast<float4*>(cw + l32 * WTN + (unit_at(u, l32) << 2)) =
                     make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
             }
         const int64_t gm = m0 + wm0 + b * 32 + rr;  // row of pass 0; pass i adds i * RPP
-        if (interior) {
+        if (interior && lane_on) {
             float4 v4[kPasses];
             uint2 aw[kPasses];
             float4 old[kPasses];
 #pragma unroll
             for (int i = 0; i < kPasses; ++i) {
                 const int m = i * RPP + rr;
-                v4[i] = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
+                v4[i] = *reinterpret_cast<const float4*>(cw + m * WTN + (unit_at(ru, m) << 2));
             }
             if (epi_reads_aux(EPI)) {
 #pragma unroll
@@ -345,11 +364,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
                         make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
                 }
             }
-        } else {
+        } else if (lane_on) {
 #pragma unroll
             for (int i = 0; i < kPasses; ++i) {
                 const int m = i * RPP + rr;
-                const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + ((ru ^ (m & (UPR - 1))) << 2));
+                const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + (unit_at(ru, m) << 2));
                 epilogue4<EPI, CF32>(g, gm + i * RPP, gn, v.x, v.y, v.z, v.w, bias, vec_ok);
             }
         }
@@ -359,11 +378,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
 // One whole output tile: main loop over all of K, then the epilogue.
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
-    f32x16_t acc[BN / 64][BM / 64];
+    f32x16_t acc[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM];
 #pragma unroll
-    for (int a = 0; a < BN / 64; ++a)
+    for (int a = 0; a < WaveTile<BM, BN>::TN; ++a)
 #pragma unroll
-        for (int b = 0; b < BM / 64; ++b)
+        for (int b = 0; b < WaveTile<BM, BN>::TM; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
     gemm_mainloop<BM, BN, AT, BT, NS, KT>(g, tile_m, tile_n, 0, (int)((g.K + KT - 1) / KT), acc);
@@ -524,6 +543,26 @@ static int launch_gemm(const GemmArgs* probs, int n, hipStream_t st) {
                 int rc = count_tiles<256, 256>(big);
                 if (rc) return rc;
                 return launch_single<256, 256, AT, BT, 2, EPI, CF32>(big, st);
+            }
+        }
+        if constexpr (BM == 128 && BN == 128 && !AT && !BT) {
+            // an output that leaves CUs idle on 128-wide tiles but fills them on 96-wide ones
+            // (4096 x 768: 192 tiles against 256)
+            GemmArgs narrow = probs[0];
+            const int64_t rows = (narrow.M + 127) / 128;
+            const int64_t t128 = rows * ((narrow.N + 127) / 128), t96 = rows * ((narrow.N + 95) / 96);
+            if (t128 < kComputeUnits && t96 > t128 && t96 <= kComputeUnits) {
+                int rc = count_tiles<128, 96>(narrow);
+                if (rc) return rc;
+                return launch_single<128, 96, AT, BT, 3, EPI, CF32>(narrow, st);
+            }
+            // an output that needs a second, mostly empty wave of 128-wide tiles (two work-groups per
+            // CU: 512 at once) but fits one wave of 192-wide ones (4096 x 3072: 768 tiles against 512)
+            const int64_t t192 = rows * ((narrow.N + 191) / 192);
+            if (t128 > 2 * kComputeUnits && t128 < 4 * kComputeUnits && t192 <= 2 * kComputeUnits) {
+                int rc = count_tiles<128, 192>(narrow);
+                if (rc) return rc;
+                return launch_single<128, 192, AT, BT, 2, EPI, CF32>(narrow, st);
             }
         }
         GemmArgs g = probs[0];

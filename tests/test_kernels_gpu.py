@@ -136,7 +136,7 @@ def _gemm_ref(A, B, a_trans, b_trans):
 
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 768), (200, 136, 72), (4096, 768, 768),
-                                   (1000, 1001, 264), (64, 8, 8)])
+                                   (1000, 1001, 264), (64, 8, 8), (4088, 2296, 72)])
 def test_gemm_bf16_layouts(a_trans, b_trans, M, N, K):
     Nn = native()
     if a_trans and M % 8:
@@ -176,10 +176,12 @@ def test_gemm_bf16_large_output_takes_256_wide_tiles():
     assert bool(torch.isnan(Cbuf[:, N:]).all())
 
 
-def test_gemm_bf16_epilogues():
+@pytest.mark.parametrize("M,N,K", [(384, 264, 136), (512, 380, 136), (4096, 768, 264), (4096, 2304, 136)])
+def test_gemm_bf16_epilogues(M, N, K):
+    """The second and third shapes run on 96-column tiles (they fill more CUs than 128-column ones),
+    the last on 192-column tiles (one wave of work-groups instead of one and a bit)."""
     Nn = native()
     torch.manual_seed(5)
-    M, N, K = 384, 264, 136
     A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     W = (torch.randn(N, K, device=DEV) * 0.1).to(torch.bfloat16)
     bias = torch.randn(N, device=DEV).to(torch.bfloat16)
