@@ -2,8 +2,12 @@
 //
 //   C[M,N] = epilogue( sum_k A(m,k) * B(n,k) ),  fp32 accumulation.
 //
-// Tiling: a work-group of 256 lanes (4 waves, 2x2) owns a BM x BN output tile and walks K in steps
-// of 64.  Tiles are staged with direct-to-LDS buffer loads (no staging registers, no ds_write):
+// Tiling: a work-group of 256 lanes (4 waves) owns a BM x BN output tile and walks K in steps of 64
+// (32 for the segmented weight gradients).  The tile shape is chosen per problem so that the grid
+// fits the 256 CUs: 128 x 128 by default (waves 2 x 2), 128 x 96 (waves 4 x 1) when that puts a tile
+// on more CUs, 128 x 192 when it replaces a full wave of work-groups plus a mostly empty one by a
+// single wave, 256 x 256 for very large outputs.  Tiles are staged with direct-to-LDS buffer loads
+// (no staging registers, no ds_write):
 //   * a k-contiguous operand (memory [rows][ld]) lives in LDS as [row][64 k] with the 16-byte chunk
 //     index XOR-swizzled by the row, and fragments are plain ds_read_b128;
 //   * a transposed operand (memory [K][ld]: the weight of an input-gradient GEMM, both operands of a
