@@ -1,4 +1,4 @@
-// fp32 GEMM (SIMT, LDS-tiled) for the small fp32 MLP configuration.  Same descriptor and operand
+// fp32 GEMM on the fp32 matrix cores for the small fp32 MLP configuration.  Same descriptor and operand
 // conventions as the bf16 MFMA GEMM: C[M,N] = epilogue( sum_k A(m,k) * B(n,k) ).
 #include "common.h"
 
@@ -16,77 +16,102 @@ struct GemmF32Args {
     int a_trans, b_trans;
 };
 
-constexpr int FT = 64;   // output tile edge
-constexpr int FK = 16;   // k step
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmF32Args g) {
-    __shared__ float As[FK][FT + 1];
-    __shared__ float Bs[FK][FT + 1];
-    const int tid = threadIdx.x;
-    const int tx = tid & 15, ty = tid >> 4;  // 16 x 16 lanes, 4 x 4 outputs each
-    const int64_t m0 = (int64_t)blockIdx.x * FT, n0 = (int64_t)blockIdx.y * FT;
-    float acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+constexpr int FT = 32;       // output tile edge: one 32 x 32 MFMA tile per work-group
+constexpr int FW = 8;        // waves per work-group; each takes every 8th k-chunk
+constexpr int FC = 8;        // k values per chunk (4 MFMA steps of k = 2)
+constexpr int FU = 8;        // chunks whose loads a wave has in flight at a time
 
-    for (int64_t k0 = 0; k0 < g.K; k0 += FK) {
-        // 64 x 16 elements per operand, 4 per lane
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int id = tid + 256 * i;
-            int r, k;
-            if (g.a_trans) { r = id & 63; k = id >> 6; } else { k = id & 15; r = id >> 4; }
-            const int64_t gm = m0 + r, gk = k0 + k;
-            float v = 0.f;
-            if (gm < g.M && gk < g.K) v = g.a_trans ? g.A[gk * g.lda + gm] : g.A[gm * g.lda + gk];
-            As[k][r] = v;
-            if (g.b_trans) { r = id & 63; k = id >> 6; } else { k = id & 15; r = id >> 4; }
-            const int64_t gn = n0 + r, gk2 = k0 + k;
-            v = 0.f;
-            if (gn < g.N && gk2 < g.K) v = g.b_trans ? g.B[gk2 * g.ldb + gn] : g.B[gn * g.ldb + gk2];
-            Bs[k][r] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < FK; ++k) {
-            float a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = Bs[k][tx * 4 + j];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
-        }
-        __syncthreads();
+// The four k values that lane (row, h) feeds to the 4 MFMA steps of a chunk starting at k0:
+// k0 + 4h + {0,1,2,3}.  A and B use the same assignment, so step e of a chunk multiplies
+// k = k0 + e (lanes 0-31) and k0 + 4 + e (lanes 32-63) on both sides.
+__device__ __forceinline__ float4 load_chunk(const float* X, int64_t ld, bool trans, int64_t row, bool row_ok,
+                                             int64_t k, int64_t K, bool vec_ok) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (!row_ok || k >= K) return v;
+    if (!trans) {
+        const float* p = X + row * ld + k;
+        if (vec_ok && k + 3 < K) return *reinterpret_cast<const float4*>(p);
+        v.x = p[0];
+        if (k + 1 < K) v.y = p[1];
+        if (k + 2 < K) v.z = p[2];
+        if (k + 3 < K) v.w = p[3];
+    } else {
+        const float* p = X + k * ld + row;
+        v.x = p[0];
+        if (k + 1 < K) v.y = p[ld];
+        if (k + 2 < K) v.z = p[2 * ld];
+        if (k + 3 < K) v.w = p[3 * ld];
     }
+    return v;
+}
+
+// One 32 x 32 tile of C per work-group.  The problems this kernel serves are small (a few tiles,
+// K up to a few thousand), so the time of a launch is the length of one work-group's dependent
+// chain: the 8 waves split K between them (chunk c goes to wave c mod 8), every wave reads its
+// operands straight from memory into the lanes of v_mfma_f32_32x32x2_f32 with 8 chunks of loads in
+// flight, and the 8 partial tiles are summed through LDS in wave order (so the result does not
+// depend on timing).
+template <int EPI>
+__global__ __launch_bounds__(FW * 64) void gemm_f32_kernel(const GemmF32Args g) {
+    __shared__ float part[FW][FT][FT];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t m0 = (int64_t)blockIdx.x * FT, n0 = (int64_t)blockIdx.y * FT;
+    const int64_t am = m0 + r, bn = n0 + r;
+    const bool a_ok = am < g.M, b_ok = bn < g.N;
+    const bool a_vec = !g.a_trans && (g.lda & 3) == 0 && aligned(g.A, 16);
+    const bool b_vec = !g.b_trans && (g.ldb & 3) == 0 && aligned(g.B, 16);
+
+    f32x16_t acc;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t m = m0 + ty * 4 + i;
-        if (m >= g.M) continue;
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    const int64_t n_chunks = (g.K + FC - 1) / FC;
+    for (int64_t c0 = wave; c0 < n_chunks; c0 += (int64_t)FW * FU) {
+        float4 a[FU], b[FU];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int64_t n = n0 + tx * 4 + j;
-            if (n >= g.N) continue;
-            float v = acc[i][j];
-            if ((EPI == PP_EPI_BIAS || EPI == PP_EPI_BIAS_RELU) && g.bias) v += g.bias[n];
-            if (EPI == PP_EPI_BIAS_RELU) v = fmaxf(v, 0.f);
-            if (EPI == PP_EPI_DRELU) v = g.aux_in[m * g.ld_aux + n] > 0.f ? v : 0.f;
-            float* cp = g.C + m * g.ldc + n;
-            if (EPI == PP_EPI_ACCUM_F32 && g.beta) v += *cp;
-            *cp = v;
+        for (int u = 0; u < FU; ++u) {
+            const int64_t k = (c0 + (int64_t)u * FW) * FC + 4 * h;  // past K for chunks beyond the last
+            a[u] = load_chunk(g.A, g.lda, g.a_trans, am, a_ok, k, g.K, a_vec);
+            b[u] = load_chunk(g.B, g.ldb, g.b_trans, bn, b_ok, k, g.K, b_vec);
         }
+#pragma unroll
+        for (int u = 0; u < FU; ++u) {
+            if (c0 + (int64_t)u * FW >= n_chunks) break;  // the same for every lane of the wave
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, b[u].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, b[u].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].z, b[u].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].w, b[u].w, acc, 0, 0, 0);
+        }
+    }
+    // accumulator element e of lane (r, h) is C(m = 8 (e / 4) + 4 h + e % 4, n = r)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) part[wave][8 * (e >> 2) + 4 * h + (e & 3)][r] = acc[e];
+    __syncthreads();
+    for (int o = tid; o < FT * FT; o += FW * 64) {
+        const int i = o >> 5, j = o & 31;
+        const int64_t m = m0 + i, n = n0 + j;
+        if (m >= g.M || n >= g.N) continue;
+        float v = part[0][i][j];
+#pragma unroll
+        for (int w = 1; w < FW; ++w) v += part[w][i][j];
+        if ((EPI == PP_EPI_BIAS || EPI == PP_EPI_BIAS_RELU) && g.bias) v += g.bias[n];
+        if (EPI == PP_EPI_BIAS_RELU) v = fmaxf(v, 0.f);
+        if (EPI == PP_EPI_DRELU) v = g.aux_in[m * g.ld_aux + n] > 0.f ? v : 0.f;
+        float* cp = g.C + m * g.ldc + n;
+        if (EPI == PP_EPI_ACCUM_F32 && g.beta) v += *cp;
+        *cp = v;
     }
 }
 
 template <int EPI>
 static int launch_f32(const GemmF32Args& g, hipStream_t st) {
-    dim3 grid((uint32_t)((g.M + FT - 1) / FT), (uint32_t)((g.N + FT - 1) / FT));
-    hipLaunchKernelGGL(gemm_f32_kernel<EPI>, grid, dim3(256), 0, st, g);
+    const int64_t tm = (g.M + FT - 1) / FT, tn = (g.N + FT - 1) / FT;
+    if (tm > 0x7fffffff || tn > 65535) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_f32: output too large");
+    dim3 grid((uint32_t)tm, (uint32_t)tn);
+    hipLaunchKernelGGL(gemm_f32_kernel<EPI>, grid, dim3(FW * 64), 0, st, g);
     return check_launch("gemm_f32_kernel");
 }
 

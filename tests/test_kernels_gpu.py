@@ -241,7 +241,8 @@ def test_gemm_f32():
     torch.manual_seed(6)
     for (M, N, K, at, bt) in [(64, 512, 512, False, False), (64, 10, 256, False, False),
                               (70, 33, 19, False, True), (512, 1024, 64, True, True),
-                              (64, 512, 1024, False, True)]:
+                              (64, 512, 1024, False, True), (1, 1, 1, False, False),
+                              (33, 65, 2051, True, False), (256, 10, 64, True, True)]:
         A = torch.randn((K, M) if at else (M, K), device=DEV)
         B = torch.randn((K, N) if bt else (N, K), device=DEV)
         bias = torch.randn(N, device=DEV)
