@@ -99,7 +99,7 @@ def build_other(args):
         args.describe = ("one stage (8 layers) of a Llama-2-7B-shaped pipeline (d_model 4096, 32 heads of 128, "
                          "SwiGLU 11008, RMSNorm, RoPE, seq 2048), zero-bubble schedule with separate dI and dW "
                          "passes, 16 microbatches of one sequence, upstream gradients N(0, 1e-2), bf16 with fp32 "
-                         f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+                         f"gradient accumulation ({args.accumulate_text})")
         args.batch, args.seq = M, 2048
         return model, sched, [stage], x, upstream
     if args.workload == "moe":
@@ -119,7 +119,7 @@ def build_other(args):
         args.describe = ("Mixtral-style decoder (8 layers in 2 virtual stages, d_model 1024, 16 heads, 8 experts "
                          "with SwiGLU 4096, top-2 router, vocab 32000, seq 1024), schedule interleaved 1f1b on one "
                          "rank, batch 16 in 8 microbatches, bf16 with fp32 gradient accumulation "
-                         f"({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+                         f"({args.accumulate_text})")
         args.batch, args.seq = 16, 1024
         return model, sched, stages, ids.cuda(), target.cuda()
     raise ValueError(args.workload)
@@ -175,7 +175,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--schedule", default="1f1b", choices=["1f1b", "gpipe", "zero_bubble"])
     ap.add_argument("--fused-accumulate", action="store_true",
-                    help="accumulate fp32 gradients in the dW GEMM epilogue instead of the accumulate kernel")
+                    help="add the unrounded fp32 sums of the dW GEMMs to the accumulators (default: rounded "
+                         "to bf16 first, the bits of a bf16 gradient folded in by the accumulate kernel)")
+    ap.add_argument("--staged-accumulate", action="store_true",
+                    help="write every gradient to the bf16 staging arena and fold it in with the accumulate "
+                         "kernel (the same bits as the default, one more pass over the parameters)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--serial-stages", action="store_true",
                     help="run all virtual stages on one stream instead of one stream per stage")
@@ -195,6 +199,11 @@ def main():
     ap.add_argument("--microbatches", type=int, default=8)
     ap.add_argument("--stages", type=int, default=4)
     args = ap.parse_args()
+    if args.staged_accumulate:
+        args.fused_accumulate = "staged"
+    args.accumulate_text = {False: "added in the dW GEMM epilogue, rounded to bf16 first",
+                            True: "unrounded sums added in the dW GEMM epilogue",
+                            "staged": "staging arena + accumulate kernel"}[args.fused_accumulate]
 
     if args.gpus != 1:
         print("bench.py: this build runs every pipeline stage as a virtual stage on ONE GPU; "
@@ -241,7 +250,7 @@ def main():
                                 f"{args.heads} heads, FFN {args.ffn}, vocab {args.vocab}, seq {args.seq}), "
                                 f"{args.stages} virtual stages on one GPU, schedule {args.schedule}, "
                                 f"batch {args.batch} in {args.microbatches} microbatches, bf16 with fp32 "
-                                f"gradient accumulation ({'GEMM epilogue' if args.fused_accumulate else 'accumulate kernel'})")
+                                f"gradient accumulation ({args.accumulate_text})")
                                if default_workload else args.describe,
                    "global_batch": args.batch, "seq_len": args.seq},
         "step_tflops": round((flops_per_step(args) if default_workload else args.flops)
@@ -276,7 +285,10 @@ def main():
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
                               "gemm_ms_per_step": round(ms / n_prof, 3)}
         hbm = {}
-        for name, kind in (("grad_accumulate", N.OP_ACCUM_BF16), ("cross_entropy", N.OP_CE_LOSS),
+        # with the default accumulation the in-step accumulate launches only cover the small
+        # tensors (biases, LayerNorm): the kernel's bandwidth is measured at arena size below
+        accum_rows = (("grad_accumulate", N.OP_ACCUM_BF16),) if args.fused_accumulate == "staged" else ()
+        for name, kind in accum_rows + (("cross_entropy", N.OP_CE_LOSS),
                            ("layernorm_fwd", N.OP_LN_FWD), ("layernorm_bwd_input", N.OP_LN_BWD_INPUT)):
             kms, kwork, kcnt = N.profile_read(kind)
             if kcnt:
@@ -325,6 +337,24 @@ def main():
                                      "note": "8-way split of the merged logits along dim 1; not part of the "
                                              "step, whose own split is 0.5 MB of token ids"}
         del merged
+        # the accumulate kernel over a whole stage arena (what a staged weight-gradient pass runs)
+        arena = max((st.param_arena() for st in stages), key=lambda a: a.total)
+        acc_t, g_t = torch.zeros_like(arena.acc), torch.zeros_like(arena.staging)
+        N.grad_accum(acc_t, g_t, init=False)
+        ev0.record()
+        for _ in range(5):
+            N.grad_accum(acc_t, g_t, init=False)
+        ev1.record()
+        torch.cuda.synchronize()
+        ams = ev0.elapsed_time(ev1) / 5
+        abytes = 10.0 * acc_t.numel()
+        hbm["grad_accumulate_arena_sized"] = {
+            "achieved": round(abytes / (ams * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(abytes / (ams * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms": round(ams, 3),
+            "note": f"pp_grad_accum_f32_bf16 over {acc_t.numel()} elements (the largest stage's arena), 10 B per "
+                    "element; in the step the weight gradients are accumulated by their GEMM's epilogue unless "
+                    "--staged-accumulate"}
+        del acc_t, g_t
         # the optimizer step that follows schedule.step() in training: timed alone, outside `value`
         import pippy_amd as pp
         opt = pp.FusedAdamW(stages, lr=1e-4, weight_decay=0.1)

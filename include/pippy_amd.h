@@ -119,7 +119,9 @@ enum pp_gemm_epilogue {
     PP_EPI_DGELU_TANH = 6,    /* C = acc * gelu_tanh'(aux_in[m,n])                          */
     PP_EPI_ACCUM_F32 = 7,     /* C(fp32) = (beta ? C : 0) + acc     (fused grad accumulate) */
     PP_EPI_BIAS_RELU = 8,     /* C = max(acc + bias[n], 0)                                  */
-    PP_EPI_DRELU = 9          /* C = aux_in[m,n] > 0 ? acc : 0                              */
+    PP_EPI_DRELU = 9,         /* C = aux_in[m,n] > 0 ? acc : 0                              */
+    PP_EPI_ACCUM_ROUNDED = 10 /* C(fp32) = (beta ? C : 0) + float(bf16(acc)): bit for bit what a
+                                 bf16 C followed by pp_grad_accum_f32_bf16 leaves in C           */
 };
 
 enum pp_dtype { PP_BF16 = 0, PP_F32 = 1 };
@@ -137,7 +139,7 @@ typedef struct pp_gemm_desc {
     const void* aux_in;    /* bf16 [M, N] with ld_aux (residual / saved pre-activation) */
     void* aux_out;         /* bf16 [M, N] with ld_aux (pre-activation to save) or null */
     int64_t ld_aux;
-    int32_t beta;          /* PP_EPI_ACCUM_F32: 0 overwrite, 1 accumulate */
+    int32_t beta;          /* PP_EPI_ACCUM_F32 / _ROUNDED: 0 overwrite, 1 accumulate */
     int32_t reserved;
 } pp_gemm_desc;
 
@@ -164,7 +166,7 @@ int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream);
  *   PP_SEG_K: for every segment e,  C_e = A[r0:r1, :]^T * B[r0:r1, :]  with C_e = seg_ptr[e]
  *     ([M, N], ldc): the weight gradient of expert e; desc->K is the total row count, desc->C is
  *     ignored; a_trans = b_trans = 1; bf16 C with NONE (an empty segment writes zeros) or fp32 C
- *     with ACCUM_F32 / beta. */
+ *     with ACCUM_F32 or ACCUM_ROUNDED / beta. */
 enum pp_gemm_seg_mode { PP_SEG_ROWS = 0, PP_SEG_K = 1 };
 #define PP_GEMM_MAX_SEGMENTS 1024
 int pp_gemm_bf16_segmented(const pp_gemm_desc* desc, const int32_t* seg_start, const void* const* seg_ptr,

@@ -18,7 +18,7 @@ PP_BF16, PP_F32 = 0, 1
 
 # enum pp_gemm_epilogue
 EPI_NONE, EPI_BIAS, EPI_BIAS_GELU_ERF, EPI_BIAS_GELU_TANH, EPI_BIAS_RESIDUAL = 0, 1, 2, 3, 4
-EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU = 5, 6, 7, 8, 9
+EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCUM_ROUNDED = 5, 6, 7, 8, 9, 10
 
 # enum pp_op_kind
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,

@@ -58,7 +58,11 @@ class ParamArena:
                 direct.add(id(p))
         # parameters whose gradient goes through the staging arena come first; the single
         # accumulate op of a W pass covers [0, staged_total)
-        params = [q for q in params if id(q[1]) not in direct] + [q for q in params if id(q[1]) in direct]
+        # and among them matrices before vectors: the weight-gradient GEMMs add into the accumulators
+        # themselves, so what is left for the accumulate op is (normally) one range of small tensors
+        params = [q for q in params if id(q[1]) not in direct and q[1].dim() >= 2] + \
+                 [q for q in params if id(q[1]) not in direct and q[1].dim() < 2] + \
+                 [q for q in params if id(q[1]) in direct]
         self.entries: Dict[int, Tuple[int, int, Tuple[int, ...]]] = {}  # id(p) -> (off, numel, padded shape)
         off = 0
         self.staged_total = 0
@@ -126,6 +130,21 @@ class ParamArena:
         if padded:
             return flat[o:o + numel].view(shape)
         return flat[o:o + p.numel()].view(p.shape)
+
+    def staged_ranges(self, skip_ids) -> List[Tuple[int, int]]:
+        """[begin, end) element ranges of the staging arena that hold gradients, leaving out the
+        parameters in ``skip_ids``; neighbours are merged (alignment gaps hold zeros)."""
+        ranges: List[Tuple[int, int]] = []
+        for _, p in self.named:
+            o, numel, _shape = self.entries[id(p)]
+            if o >= self.staged_total or id(p) in skip_ids:
+                continue
+            end = min(_round_up(o + numel, _ALIGN_ELEMS), self.staged_total)
+            if ranges and ranges[-1][1] == o:
+                ranges[-1] = (ranges[-1][0], end)
+            else:
+                ranges.append((o, end))
+        return ranges
 
     def weight(self, p, padded=True):
         return self._slice(self.params, p, padded)
@@ -552,9 +571,8 @@ class Builder:
         return self.sp.arena.weight_t(p)
 
     def grad_target(self, p, padded=True):
-        """Where the W pass writes this parameter's microbatch gradient: the staging arena (then one
-        accumulate op folds the arena into fp32), or the fp32 accumulator when the GEMM epilogue
-        accumulates itself."""
+        """Where the W pass writes a microbatch gradient that no GEMM epilogue accumulates: the
+        staging arena, which the accumulate ops at the end of the pass fold into fp32."""
         return self.sp.arena.grad_staging(p, padded)
 
     def grad_acc(self, p, padded=True):
@@ -578,15 +596,27 @@ class Builder:
         accumulation."""
         # all dW GEMMs of a pass only read buffers that the input-gradient pass has finished, so
         # they are independent of each other: they go first and are marked for grouped launch
-        if self.fused_accumulate:
-            op = op_gemm(dY2d, X2d, self.grad_acc(p, padded), a_trans=True, b_trans=True,
-                         epilogue=N.EPI_ACCUM_F32, beta=1)
+        epi = self.weight_grad_epilogue(p)
+        if epi is not None:
+            op = op_gemm(dY2d, X2d, self.grad_acc(p, padded), a_trans=True, b_trans=True, epilogue=epi, beta=1)
             op.flags |= N.OP_GROUPED
             self._w_gemm.append((op, "beta"))
         else:
             op = op_gemm(dY2d, X2d, self.grad_target(p, padded), a_trans=True, b_trans=True)
             op.flags |= N.OP_GROUPED
             self._w_gemm.append((op, None))
+
+    def weight_grad_epilogue(self, p) -> Optional[int]:
+        """The GEMM epilogue that adds the gradient of weight ``p`` to its fp32 accumulator, or None
+        when the gradient goes through the staging arena.  ``fused_accumulate`` adds the fp32 sums;
+        the default adds them rounded to the parameter dtype, which leaves bit for bit what a
+        gradient written in that dtype and folded in by the accumulate kernel would."""
+        if self.sp.staged_weight_grads:
+            return None
+        self.sp.epilogue_accumulated.add(id(p))
+        if self.fused_accumulate or p.dtype == torch.float32:
+            return N.EPI_ACCUM_F32
+        return N.EPI_ACCUM_ROUNDED
 
     def on_backward(self, fn: Callable):
         """Registers the block's backward emitter ``fn(dy, need_dx, dx_out) -> dx``; it runs later,
@@ -612,7 +642,15 @@ class StageProgram:
         self.device = device
         self.training = training
         self.split_backward = split_backward
-        self.fused_accumulate = fused_accumulate
+        # fused_accumulate: False - weight-gradient GEMMs add their sums, rounded to the parameter
+        # dtype, to the fp32 accumulators (the same bits as the staged form); True - they add the
+        # unrounded fp32 sums; "staged" - every gradient is written to the staging arena in the
+        # parameter dtype and folded in by the accumulate kernel (the literal form of the contract)
+        if fused_accumulate not in (False, True, "staged"):
+            raise ValueError(f"fused_accumulate must be False, True or 'staged', not {fused_accumulate!r}")
+        self.fused_accumulate = fused_accumulate is True
+        self.staged_weight_grads = fused_accumulate == "staged"
+        self.epilogue_accumulated = set()  # ids of the parameters whose GEMM epilogue accumulates
         self.is_first = is_first
         self.is_last = is_last
         self.arena = ParamArena(module, device)
@@ -685,10 +723,10 @@ class StageProgram:
                 if tag is not None:
                     toggles[tag].append(k)
             # fold this microbatch's staged parameter gradients into the fp32 accumulators
-            if not self.fused_accumulate and self.arena.staged_total:
-                n = self.arena.staged_total
-                k = prog.W.append(op_accum(self.arena.acc[:n], self.arena.staging[:n], init=False))
-                prog.init_toggle_accum.append(k)
+            if not self.fused_accumulate:
+                for lo, hi in self.arena.staged_ranges(self.epilogue_accumulated):
+                    k = prog.W.append(op_accum(self.arena.acc[lo:hi], self.arena.staging[lo:hi], init=False))
+                    prog.init_toggle_accum.append(k)
         prog.F.freeze()
         prog.I.freeze()
         prog.W.freeze()

@@ -38,6 +38,7 @@ struct GemmArgs {
     uint16_t* aux_out;
     int64_t ld_aux;
     int beta;
+    int round_bf16;  // fp32 C: round the sums to bf16 before they are stored or added
     uint32_t tiles_m, tiles_n, n_blocks;
 };
 
@@ -122,6 +123,10 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t 
 
     if (CF32) {
         float* cp = static_cast<float*>(g.C) + m * g.ldc + n0;
+        if (EPI == PP_EPI_ACCUM_F32 && g.round_bf16) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = bf16_to_f32(f32_to_bf16(v[e]));
+        }
         if (EPI == PP_EPI_ACCUM_F32 && g.beta) {
             if (full) {
                 const float4 old = *reinterpret_cast<const float4*>(cp);
@@ -359,6 +364,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
                         make_uint2(pack_bf16(pre[0], pre[1]), pack_bf16(pre[2], pre[3]));
                 if (CF32) {
                     float* cp = static_cast<float*>(g.C) + row * g.ldc + gn;
+                    if (EPI == PP_EPI_ACCUM_F32 && g.round_bf16) {
+                        const uint32_t w0 = pack_bf16(v[0], v[1]), w1 = pack_bf16(v[2], v[3]);
+                        v[0] = bf16lo(w0); v[1] = bf16hi(w0); v[2] = bf16lo(w1); v[3] = bf16hi(w1);
+                    }
                     if (EPI == PP_EPI_ACCUM_F32 && g.beta)
                         *reinterpret_cast<float4*>(cp) = make_float4(old[i].x + v[0], old[i].y + v[1], old[i].z + v[2], old[i].w + v[3]);
                     else
@@ -614,6 +623,7 @@ static int dispatch_layout(const GemmArgs* g, int n, int at, int bt, hipStream_t
 }
 
 static int dispatch(const GemmArgs* g, int n, int at, int bt, int epi, bool cf32, hipStream_t st) {
+    if (epi == PP_EPI_ACCUM_ROUNDED) epi = PP_EPI_ACCUM_F32;  // the same kernels; GemmArgs::round_bf16 is set
     if (cf32) {
         switch (epi) {
             case PP_EPI_NONE: return dispatch_layout<PP_EPI_NONE, true>(g, n, at, bt, st);
@@ -662,14 +672,14 @@ static int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
         if (a_bytes >= 0x7ffffff0ull || b_bytes >= 0x7ffffff0ull)
             return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16: an operand spans 2 GiB or more");
     }
-    const int epi = d->epilogue;
+    const int epi = d->epilogue == PP_EPI_ACCUM_ROUNDED ? PP_EPI_ACCUM_F32 : d->epilogue;
     const bool needs_aux = epi == PP_EPI_BIAS_RESIDUAL || epi == PP_EPI_DGELU_ERF ||
                            epi == PP_EPI_DGELU_TANH || epi == PP_EPI_DRELU;
     if (needs_aux && (!d->aux_in || d->ld_aux < d->N))
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: epilogue %d needs aux_in with ld_aux >= N", epi);
     if (d->aux_out && d->ld_aux < d->N) return fail(PP_ERR_INVALID, "pp_gemm_bf16: ld_aux < N");
     if (epi == PP_EPI_ACCUM_F32 && d->c_dtype != PP_F32)
-        return fail(PP_ERR_INVALID, "pp_gemm_bf16: PP_EPI_ACCUM_F32 needs an fp32 C");
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: PP_EPI_ACCUM_F32 / PP_EPI_ACCUM_ROUNDED need an fp32 C");
     g->A = static_cast<const uint16_t*>(d->A);
     g->B = static_cast<const uint16_t*>(d->B);
     g->C = d->C;
@@ -680,6 +690,7 @@ static int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
     g->aux_out = static_cast<uint16_t*>(d->aux_out);
     g->ld_aux = d->ld_aux;
     g->beta = d->beta;
+    g->round_bf16 = d->epilogue == PP_EPI_ACCUM_ROUNDED;
     g->tiles_m = g->tiles_n = g->n_blocks = 0;
     return PP_OK;
 }
@@ -739,7 +750,7 @@ extern "C" int pp_gemm_bf16_segmented(const pp_gemm_desc* d, const int32_t* seg_
         if (!dd.a_trans || !dd.b_trans)
             return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: k mode takes transposed A and B");
         if (!((dd.epilogue == PP_EPI_NONE && dd.c_dtype == PP_BF16) ||
-              (dd.epilogue == PP_EPI_ACCUM_F32 && dd.c_dtype == PP_F32)))
+              ((dd.epilogue == PP_EPI_ACCUM_F32 || dd.epilogue == PP_EPI_ACCUM_ROUNDED) && dd.c_dtype == PP_F32)))
             return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: k mode writes bf16 or accumulates into fp32");
         dd.C = const_cast<void*>(dd.A);
         dd.K = (dd.K + 7) & ~(int64_t)7;  // the reduction length of a segment need not be a multiple of 8

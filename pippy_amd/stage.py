@@ -10,7 +10,10 @@ Two execution modes per stage:
 
 * native: the stage module lowers to HIP launch lists (``_program.py``); forward, input-gradient
   and weight-gradient passes are separate entry points and parameter gradients are accumulated in
-  fp32 by the accumulate kernel (or by the dW GEMM epilogue when ``fused_accumulate`` is set);
+  fp32: ``acc += float(g)`` with ``g`` the microbatch gradient in the parameter dtype, microbatches
+  ascending (weight gradients by the epilogue of their GEMM, the small tensors by the accumulate
+  kernel; ``fused_accumulate=True`` adds the unrounded fp32 sums instead, ``"staged"`` sends every
+  gradient through the staging arena and the accumulate kernel, with the same bits as the default);
 * eager: any other ``nn.Module`` runs through torch autograd on the GPU exactly as the reference
   does (``forward_one_chunk`` / ``stage_backward``), with the same caching rules.
 """
@@ -66,7 +69,7 @@ class PipelineStageBase:
 
     def __init__(self, submodule: nn.Module, stage_index: int, num_stages: int,
                  device: Union[torch.device, str], num_microbatches: int, group=None, *,
-                 fused_accumulate: bool = False, force_eager: bool = False):
+                 fused_accumulate: Union[bool, str] = False, force_eager: bool = False):
         if stage_index >= num_stages:
             raise ValueError(f"Stage index {stage_index} is out of range of {num_stages}")
         self.submod = submodule

@@ -61,9 +61,10 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
     if dY2d.dtype == torch.float32:
         # fp32 stages are small: ones[1, T] @ dY through the fp32 GEMM is an ordered column sum
         ones = b.sp.ones_f32(dY2d.shape[0])
-        if b.fused_accumulate:
-            b.w(P.op_gemm(ones, dY2d, b.grad_acc(lin.bias).view(1, -1), b_trans=True,
-                          epilogue=N.EPI_ACCUM_F32, beta=1), tag="beta")
+        epi = b.weight_grad_epilogue(lin.bias)
+        if epi is not None:
+            b.w(P.op_gemm(ones, dY2d, b.grad_acc(lin.bias).view(1, -1), b_trans=True, epilogue=epi, beta=1),
+                tag="beta")
         else:
             b.w(P.op_gemm(ones, dY2d, b.grad_target(lin.bias).view(1, -1), b_trans=True))
         return
@@ -719,9 +720,12 @@ class MoELayer(LlamaLayer):
             # expert weight gradients: one segmented GEMM per projection, reduced over each expert's rows
             for name, dy_rows, x_rows in (("w1", dg, xp), ("w3", du, xp), ("w2", d_yp, h)):
                 params = [getattr(ex, name).weight for ex in experts]
-                if b.fused_accumulate:
+                epis = {b.weight_grad_epilogue(p) for p in params}
+                assert len(epis) == 1
+                epi = epis.pop()
+                if epi is not None:
                     ptrs = self._pointer_list(b, "acc_" + name, [b.grad_acc(p) for p in params])
-                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, epilogue=N.EPI_ACCUM_F32,
+                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, epilogue=epi,
                                       beta=1, c_f32=True), tag="beta")
                 else:
                     ptrs = self._pointer_list(b, "stage_" + name, [b.grad_target(p) for p in params])

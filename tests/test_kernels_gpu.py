@@ -227,6 +227,37 @@ def test_gemm_bf16_epilogues(M, N, K):
     assert_close_rel(acc, lin, 1e-5, "accumulate init")
 
 
+@pytest.mark.parametrize("M,N,K,at,bt", [(768, 2304, 4096, True, True), (200, 136, 264, True, True),
+                                          (256, 96, 512, False, False), (4096, 768, 64, False, True)])
+def test_gemm_bf16_rounded_accumulate_is_bit_exact(M, N, K, at, bt):
+    """PP_EPI_ACCUM_ROUNDED leaves in an fp32 C what a bf16 C followed by the accumulate kernel
+    leaves (``acc = float(g)`` when it starts an accumulation, ``acc += float(g)`` after)."""
+    Nn = native()
+    torch.manual_seed(21)
+    A = torch.randn((K, M) if at else (M, K), device=DEV).to(torch.bfloat16)
+    B = torch.randn((K, N) if bt else (N, K), device=DEV).to(torch.bfloat16)
+    g = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    Nn.gemm_bf16(A, B, g, a_trans=at, b_trans=bt)
+    start = torch.randn(M, N, device=DEV)
+    want = start.clone()
+    Nn.grad_accum(want.view(-1), g.view(-1), init=False)
+    got = start.clone()
+    Nn.gemm_bf16(A, B, got, a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_ROUNDED, beta=1)
+    assert torch.equal(got, want)
+    assert torch.equal(want, start + g.float())
+    Nn.gemm_bf16(A, B, got, a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_ROUNDED, beta=0)
+    assert torch.equal(got, g.float())
+    # the same through a grouped launch
+    got2 = start.clone()
+    other = torch.zeros(M, N, device=DEV)
+    kw = dict(a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_ROUNDED, beta=1)
+    Nn.gemm_bf16_grouped([(A, B, got2, kw), (A, B, other, kw)])
+    assert torch.equal(got2, want) and torch.equal(other, g.float())
+    bad = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="fp32 C"):
+        Nn.gemm_bf16(A, B, bad, a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_ROUNDED)
+
+
 def test_gemm_bf16_rejects_bad_arguments():
     Nn = native()
     A = torch.zeros(16, 12, device=DEV, dtype=torch.bfloat16)
@@ -796,6 +827,13 @@ def test_segmented_gemm_k_mode(R, M, Nn, E):
     N.gemm_bf16_segmented(dY.to(DEV), ptrs, None, segd, N.SEG_K, other=X.to(DEV), epilogue=N.EPI_ACCUM_F32,
                           beta=1, c_dtype=torch.float32)
     assert_close_rel(acc, ref + 1.0, 1e-3, "segmented k, fp32 accumulate")
+    # rounded accumulation: the bits of the bf16 result added by the accumulate kernel
+    start = torch.randn(E, M, Nn, device=DEV)
+    rounded = start.clone()
+    ptrs = torch.tensor([rounded[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    N.gemm_bf16_segmented(dY.to(DEV), ptrs, None, segd, N.SEG_K, other=X.to(DEV), epilogue=N.EPI_ACCUM_ROUNDED,
+                          beta=1, c_dtype=torch.float32)
+    assert torch.equal(rounded, start + out.float())
 
 
 @pytest.mark.gpu

@@ -137,6 +137,29 @@ def test_fused_accumulate_matches_oracle():
     _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M)
 
 
+def test_epilogue_accumulation_leaves_the_bits_of_the_staged_form():
+    """The default adds each weight gradient, rounded to bf16, to the fp32 accumulator in the
+    epilogue of its GEMM; ``fused_accumulate="staged"`` writes every gradient to the staging arena
+    in bf16 and folds the arena in with the accumulate kernel (``acc += float(g)``).  Both must
+    leave the same bits after two steps of four microbatches (embedding gradients use atomics)."""
+    import pippy_amd as pp
+    M = 4
+    grads = {}
+    for mode in (False, "staged"):
+        model, ref, stages, ref_stages, ids = _build_decoder(2, M=M, fused=mode)
+        _, _, grads[mode] = _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M, steps=2)
+        n_accum = [sum(1 for k in range(st._program.mbs[0].W.n)
+                       if st._program.mbs[0].W[k].kind in (pp._native.OP_ACCUM_BF16, pp._native.OP_ACCUM_F32))
+                   for st in stages]
+        note(f"fused_accumulate={mode!r}: accumulate launches per weight-gradient pass {n_accum}")
+        assert all(n == 1 for n in n_accum)
+    for k in grads[False]:
+        if k.startswith("embed."):
+            assert max_rel(grads[False][k], grads["staged"][k]) <= 1e-6, k
+        else:
+            assert torch.equal(grads[False][k], grads["staged"][k]), f"grad of {k}"
+
+
 def test_inference_gpipe_forward_only():
     import pippy_amd as pp
     M = 4
@@ -534,7 +557,7 @@ def _moe_reference_stages(ref, n_stages, per):
     return out
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fused", [False, True, "staged"])
 def test_moe_interleaved_1f1b_matches_oracle(fused):
     """Config 5 at a reduced size: two virtual stages of MoE layers on one rank under interleaved
     1F1B.  The fp32 oracle is given the expert selection of the bf16 run (a token whose second and
