@@ -646,10 +646,10 @@ class StageProgram:
         # dtype, to the fp32 accumulators (the same bits as the staged form); True - they add the
         # unrounded fp32 sums; "staged" - every gradient is written to the staging arena in the
         # parameter dtype and folded in by the accumulate kernel (the literal form of the contract)
-        if fused_accumulate not in (False, True, "staged"):
+        if isinstance(fused_accumulate, str) and fused_accumulate != "staged":
             raise ValueError(f"fused_accumulate must be False, True or 'staged', not {fused_accumulate!r}")
-        self.fused_accumulate = fused_accumulate is True
         self.staged_weight_grads = fused_accumulate == "staged"
+        self.fused_accumulate = bool(fused_accumulate) and not self.staged_weight_grads
         self.epilogue_accumulated = set()  # ids of the parameters whose GEMM epilogue accumulates
         self.is_first = is_first
         self.is_last = is_last
@@ -723,10 +723,10 @@ class StageProgram:
                 if tag is not None:
                     toggles[tag].append(k)
             # fold this microbatch's staged parameter gradients into the fp32 accumulators
-            if not self.fused_accumulate:
-                for lo, hi in self.arena.staged_ranges(self.epilogue_accumulated):
-                    k = prog.W.append(op_accum(self.arena.acc[lo:hi], self.arena.staging[lo:hi], init=False))
-                    prog.init_toggle_accum.append(k)
+            # (those that no GEMM epilogue has added already)
+            for lo, hi in self.arena.staged_ranges(self.epilogue_accumulated):
+                k = prog.W.append(op_accum(self.arena.acc[lo:hi], self.arena.staging[lo:hi], init=False))
+                prog.init_toggle_accum.append(k)
         prog.F.freeze()
         prog.I.freeze()
         prog.W.freeze()

@@ -71,12 +71,7 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
     M, Nn = dY2d.shape
     # reductions of one pass run as one grouped launch: every op needs a workspace of its own
     ws = b.workspace("colsum:" + str(id(lin)), (2 * ((M + 127) // 128) * Nn,), torch.float32)
-    if b.fused_accumulate:
-        tmp = b.workspace("colsum_out:" + str(id(lin)), (Nn,), torch.float32)
-        b.w_reduce(P.op_colsum(dY2d, tmp, ws))
-        b.w(P.op_accum(b.grad_acc(lin.bias), tmp), tag="accum")
-    else:
-        b.w_reduce(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
+    b.w_reduce(P.op_colsum(dY2d, b.grad_target(lin.bias), ws))
 
 
 def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, dY2d: torch.Tensor, *,
@@ -114,16 +109,8 @@ def layernorm_backward(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d, mean, r
     b.i(P.op_ln_bwd_input(dy2d, x2d, b.weight(ln.weight), mean, rstd, dres, dx))
     ws = b.workspace("ln_bwd:" + str(id(ln)), (2 * ((T + 127) // 128) * Cc,), torch.float32)
     has_bias = ln.bias is not None
-    if b.fused_accumulate:
-        dg = b.workspace("ln_dg:" + str(id(ln)), (Cc,), torch.float32)
-        db = b.workspace("ln_db:" + str(id(ln)), (Cc,), torch.float32)
-        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, dg, db if has_bias else None, ws))
-        b.w(P.op_accum(b.grad_acc(ln.weight), dg), tag="accum")
-        if has_bias:
-            b.w(P.op_accum(b.grad_acc(ln.bias), db), tag="accum")
-    else:
-        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
-                                      b.grad_target(ln.bias) if has_bias else None, ws))
+    b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, mean, rstd, b.grad_target(ln.weight),
+                                  b.grad_target(ln.bias) if has_bias else None, ws))
     return dx
 
 
@@ -304,12 +291,7 @@ class EncoderEmbedding(NativeBlock):
             # the type-0 row receives the gradient of every token; the other rows none
             g_tt = b.grad_target(self.token_type_embeddings.weight)
             ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)
-            if b.fused_accumulate:
-                tmp = b.workspace("colsum_out:tt", (Cc,), torch.float32)
-                b.w_reduce(P.op_colsum(de, tmp, ws))
-                b.w(P.op_accum(b.grad_acc(self.token_type_embeddings.weight)[0], tmp), tag="accum")
-            else:
-                b.w_reduce(P.op_colsum(de, g_tt[0], ws))
+            b.w_reduce(P.op_colsum(de, g_tt[0], ws))
             return None
 
         b.on_backward(bwd)
@@ -462,12 +444,7 @@ def rmsnorm_backward(b: "P.Builder", name: str, norm: nn.Module, x2d, rstd, dy2d
     dx = dx_out if dx_out is not None else b.grad(name + ".dx", (T, Cc))
     b.i(P.op_ln_bwd_input(dy2d, x2d, b.weight(norm.weight), None, rstd, dres, dx))
     ws = b.workspace("rms_bwd:" + str(id(norm)), (2 * ((T + 127) // 128) * Cc,), torch.float32)
-    if b.fused_accumulate:
-        dg = b.workspace("rms_dg:" + str(id(norm)), (Cc,), torch.float32)
-        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, None, rstd, dg, None, ws))
-        b.w(P.op_accum(b.grad_acc(norm.weight), dg), tag="accum")
-    else:
-        b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, None, rstd, b.grad_target(norm.weight), None, ws))
+    b.w_reduce(P.op_ln_bwd_weight(dy2d, x2d, None, rstd, b.grad_target(norm.weight), None, ws))
     return dx
 
 
