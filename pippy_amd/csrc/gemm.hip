@@ -287,7 +287,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
 // Epilogue of one BM x BN tile: one band of 32 rows at a time goes through a wave-private LDS region
 // as fp32, [32][WTN] with the 16-byte unit index XORed by the row, and comes back with lanes running
 // along n, so that epilogue4 reads and writes whole lines.
-template <int BM, int BN, int EPI, bool CF32>
+template <int BM, int BN, int EPI, bool CF32, int EB = 0>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
                                               f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
     typedef WaveTile<BM, BN> WT;
@@ -332,26 +332,32 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
             }
         const int64_t gm = m0 + wm0 + b * 32 + rr;  // row of pass 0; pass i adds i * RPP
         if (interior && lane_on) {
+          // EB passes at a time (all of them by default): fewer values in flight for a kernel that
+          // counts on many resident waves rather than on long runs of independent loads
+          constexpr int kBatch = EB > 0 && EB < kPasses ? EB : kPasses;
+          static_assert(kPasses % kBatch == 0, "the passes of a band split into whole batches");
+#pragma unroll
+          for (int i0 = 0; i0 < kPasses; i0 += kBatch) {
             float4 v4[kPasses];
             uint2 aw[kPasses];
             float4 old[kPasses];
 #pragma unroll
-            for (int i = 0; i < kPasses; ++i) {
+            for (int i = i0; i < i0 + kBatch; ++i) {
                 const int m = i * RPP + rr;
                 v4[i] = *reinterpret_cast<const float4*>(cw + m * WTN + (unit_at(ru, m) << 2));
             }
             if (epi_reads_aux(EPI)) {
 #pragma unroll
-                for (int i = 0; i < kPasses; ++i)
+                for (int i = i0; i < i0 + kBatch; ++i)
                     aw[i] = *reinterpret_cast<const uint2*>(g.aux_in + (gm + i * RPP) * g.ld_aux + gn);
             }
             if (CF32 && EPI == PP_EPI_ACCUM_F32 && g.beta) {
 #pragma unroll
-                for (int i = 0; i < kPasses; ++i)
+                for (int i = i0; i < i0 + kBatch; ++i)
                     old[i] = *reinterpret_cast<const float4*>(static_cast<const float*>(g.C) + (gm + i * RPP) * g.ldc + gn);
             }
 #pragma unroll
-            for (int i = 0; i < kPasses; ++i) {
+            for (int i = i0; i < i0 + kBatch; ++i) {
                 float v[4] = {v4[i].x, v4[i].y, v4[i].z, v4[i].w}, pre[4];
                 float av[4] = {0.f, 0.f, 0.f, 0.f};
                 if (epi_reads_aux(EPI)) {
@@ -377,6 +383,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
                         make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
                 }
             }
+          }
         } else if (lane_on) {
 #pragma unroll
             for (int i = 0; i < kPasses; ++i) {
@@ -389,7 +396,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
 }
 
 // One whole output tile: main loop over all of K, then the epilogue.
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK, int EB = 0>
 __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
     f32x16_t acc[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM];
 #pragma unroll
@@ -399,7 +406,7 @@ __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
     gemm_mainloop<BM, BN, AT, BT, NS, KT>(g, tile_m, tile_n, 0, (int)((g.K + KT - 1) / KT), acc);
-    gemm_epilogue<BM, BN, EPI, CF32>(g, tile_m, tile_n, acc);
+    gemm_epilogue<BM, BN, EPI, CF32, EB>(g, tile_m, tile_n, acc);
 }
 
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
@@ -523,7 +530,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_k_kernel(const Gem
     g.C = const_cast<void*>(sa.seg_ptr[e]);
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, true, true, NS, EPI, CF32, 32>(g, tile_m, tile_n);
+    gemm_tile_dma<BM, BN, true, true, NS, EPI, CF32, 32, 2>(g, tile_m, tile_n);
 }
 
 template <typename Kernel>
