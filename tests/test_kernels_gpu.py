@@ -782,7 +782,8 @@ def _segments(R, E, seed):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("R,K,Nn,E", [(4096, 1024, 512, 8), (1000, 256, 384, 5), (130, 64, 128, 3)])
+@pytest.mark.parametrize("R,K,Nn,E", [(4096, 1024, 512, 8), (1000, 256, 384, 5), (130, 64, 128, 3),
+                                      (3000, 64, 136, 63), (3000, 64, 136, 64), (2000, 64, 128, 130)])
 def test_segmented_gemm_rows_mode(R, K, Nn, E):
     N = native()
     torch.manual_seed(4)
