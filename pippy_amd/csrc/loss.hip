@@ -57,8 +57,14 @@ __device__ __forceinline__ float block_reduce_sum(float v, float* sh) {
 // exponentials exp(x - max) of the sum pass replace the logits in the registers (as bf16) and the
 // gradient pass only scales them, and the "- 1" of the target column is a single scalar store by
 // the lane that owns it.
+// Rows are read and written through buffer instructions: one VGPR byte offset per lane serves every
+// chunk (the chunk's 16 KiB stride is a scalar offset), which keeps the kernel within 64 VGPRs, so
+// that two work-groups of 16 waves share a CU and one row's store phase overlaps the other's load
+// phase; chunks past the row's end read as zero and are not written.
+typedef unsigned int ce_u32x4_t __attribute__((ext_vector_type(4)));
+
 template <int NC>
-__global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
+__global__ __launch_bounds__(kCeThreads, 8) void ce_row_bf16_kernel(
     const uint16_t* __restrict__ logits, const int64_t* __restrict__ target, uint16_t* __restrict__ dlogits,
     float* __restrict__ ws, int64_t rows, int V, int64_t ld, int64_t ignore_index) {
     __shared__ float sh[kCeThreads / 64];
@@ -66,24 +72,27 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
     const int tid = threadIdx.x;
     const uint16_t* xr = logits + row * ld;
     const int nchunk_v = (V + 7) >> 3;          // chunks holding at least one valid column
-    const int nchunk_ld = (int)(ld >> 3);       // chunks to write (padding gets zeros)
     constexpr uint32_t kNegInf2 = 0xff80ff80u;  // two bf16 -inf
+    const __amdgpu_buffer_rsrc_t src =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(xr), 0, nchunk_v * 16, 0x00020000);
+    const int voff = tid * 16;
     uint4 w[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-        const int c = tid + kCeThreads * i;
-        w[i] = make_uint4(kNegInf2, kNegInf2, kNegInf2, kNegInf2);
-        if (c < nchunk_v) {
-            w[i] = *reinterpret_cast<const uint4*>(xr + (int64_t)c * 8);
-            if (c * 8 + 8 > V) {  // the one chunk that straddles V
-                uint32_t u[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
+        const ce_u32x4_t r = __builtin_amdgcn_raw_buffer_load_b128(src, voff, i * kCeThreads * 16, 0);
+        w[i] = make_uint4(r.x, r.y, r.z, r.w);
+    }
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (c * 8 + e >= V)
-                        u[e >> 1] = (e & 1) ? ((u[e >> 1] & 0x0000ffffu) | 0xff800000u)
-                                            : ((u[e >> 1] & 0xffff0000u) | 0x0000ff80u);
-                w[i] = make_uint4(u[0], u[1], u[2], u[3]);
-            }
+    for (int i = 0; i < NC; ++i) {
+        const int c = tid + kCeThreads * i;
+        if (c * 8 + 8 > V) {  // the chunk that straddles V, and the chunks past it
+            uint32_t u[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (c * 8 + e >= V)
+                    u[e >> 1] = (e & 1) ? ((u[e >> 1] & 0x0000ffffu) | 0xff800000u)
+                                        : ((u[e >> 1] & 0xffff0000u) | 0x0000ff80u);
+            w[i] = make_uint4(u[0], u[1], u[2], u[3]);
         }
     }
     float mx = -INFINITY;
@@ -91,8 +100,13 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
     for (int i = 0; i < NC; ++i) {
         mx = fmaxf(mx, fmaxf(fmaxf(bf16lo(w[i].x), bf16hi(w[i].x)), fmaxf(bf16lo(w[i].y), bf16hi(w[i].y))));
         mx = fmaxf(mx, fmaxf(fmaxf(bf16lo(w[i].z), bf16hi(w[i].z)), fmaxf(bf16lo(w[i].w), bf16hi(w[i].w))));
+        __builtin_amdgcn_sched_barrier(0);  // one chunk's temporaries at a time
     }
     mx = block_reduce_max(mx, sh);
+    // The row stays packed across the reduction: without this the compiler keeps the 8 * NC unpacked
+    // values of the max pass alive for the sum pass, which doubles the kernel's registers.
+#pragma unroll
+    for (int i = 0; i < NC; ++i) asm volatile("" : "+v"(w[i].x), "+v"(w[i].y), "+v"(w[i].z), "+v"(w[i].w));
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
@@ -106,6 +120,9 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
         }
         w[i] = make_uint4(pack_bf16(ex[0], ex[1]), pack_bf16(ex[2], ex[3]), pack_bf16(ex[4], ex[5]),
                           pack_bf16(ex[6], ex[7]));
+        // pack here, not where the values are used: the fp32 exponentials must not stay alive
+        asm volatile("" : "+v"(w[i].x), "+v"(w[i].y), "+v"(w[i].z), "+v"(w[i].w));
+        __builtin_amdgcn_sched_barrier(0);
     }
     s = block_reduce_sum(s, sh);
     const float lse = mx + logf(s);
@@ -117,21 +134,20 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_bf16_kernel(
     const float scale = valid ? ws[rows + 1] : 0.f;
     const float ps = scale / s;  // exp(x - max) * ps = softmax * scale
     uint16_t* dr = dlogits + row * ld;
+    // ld / 8 chunks are written (padding columns get exp(-inf) * ps = 0); stores past them are dropped
+    const __amdgpu_buffer_rsrc_t dst = __builtin_amdgcn_make_buffer_rsrc(dr, 0, (int)(ld >> 3) * 16, 0x00020000);
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-        const int c = tid + kCeThreads * i;
-        if (c < nchunk_ld) {
-            *reinterpret_cast<uint4*>(dr + (int64_t)c * 8) =
-                make_uint4(pack_bf16(bf16lo(w[i].x) * ps, bf16hi(w[i].x) * ps),
-                           pack_bf16(bf16lo(w[i].y) * ps, bf16hi(w[i].y) * ps),
-                           pack_bf16(bf16lo(w[i].z) * ps, bf16hi(w[i].z) * ps),
-                           pack_bf16(bf16lo(w[i].w) * ps, bf16hi(w[i].w) * ps));
-            // the target column, by the lane that has just written its chunk (same-address stores
-            // of one lane stay in order)
-            if (valid && c == (int)(t >> 3))
-                dr[t] = f32_to_bf16((__builtin_amdgcn_exp2f((xt - mx) * kLog2e) / s - 1.0f) * scale);
-        }
+        const ce_u32x4_t o = {pack_bf16(bf16lo(w[i].x) * ps, bf16hi(w[i].x) * ps),
+                              pack_bf16(bf16lo(w[i].y) * ps, bf16hi(w[i].y) * ps),
+                              pack_bf16(bf16lo(w[i].z) * ps, bf16hi(w[i].z) * ps),
+                              pack_bf16(bf16lo(w[i].w) * ps, bf16hi(w[i].w) * ps)};
+        __builtin_amdgcn_raw_buffer_store_b128(o, dst, voff, i * kCeThreads * 16, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    // the target column, by the lane that wrote its chunk (same-address stores of one lane stay in order)
+    if (valid && (int)((t >> 3) & (kCeThreads - 1)) == tid)
+        dr[t] = f32_to_bf16((__builtin_amdgcn_exp2f((xt - mx) * kLog2e) / s - 1.0f) * scale);
 }
 
 // fp32 logits (small class counts): one wave per row, three passes over the row.
