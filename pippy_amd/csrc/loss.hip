@@ -55,8 +55,8 @@ __device__ __forceinline__ float block_reduce_sum(float v, float* sh) {
 // The kernel is bound by VALU issue as much as by HBM, so the per-element work is kept minimal:
 // columns past V are turned into -inf when the row is loaded (no bounds checks afterwards), the
 // exponentials exp(x - max) of the sum pass replace the logits in the registers (as bf16) and the
-// gradient pass only scales them, and the "- 1" of the target column is a single scalar store by
-// the lane that owns it.
+// gradient pass only scales them; the "- 1" of the target column is patched into the chunk that
+// holds it before that chunk is stored.
 // Rows are read and written through buffer instructions: one VGPR byte offset per lane serves every
 // chunk (the chunk's 16 KiB stride is a scalar offset), which keeps the kernel within 64 VGPRs, so
 // that two work-groups of 16 waves share a CU and one row's store phase overlaps the other's load
@@ -136,18 +136,30 @@ __global__ __launch_bounds__(kCeThreads, 8) void ce_row_bf16_kernel(
     uint16_t* dr = dlogits + row * ld;
     // ld / 8 chunks are written (padding columns get exp(-inf) * ps = 0); stores past them are dropped
     const __amdgpu_buffer_rsrc_t dst = __builtin_amdgcn_make_buffer_rsrc(dr, 0, (int)(ld >> 3) * 16, 0x00020000);
+    // the target column gets softmax - 1: patched into its chunk by the lane that stores it
+    const int tc = valid ? (int)(t >> 3) : -1;
+    const uint32_t corr = f32_to_bf16((__builtin_amdgcn_exp2f((xt - mx) * kLog2e) / s - 1.0f) * scale);
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-        const ce_u32x4_t o = {pack_bf16(bf16lo(w[i].x) * ps, bf16hi(w[i].x) * ps),
-                              pack_bf16(bf16lo(w[i].y) * ps, bf16hi(w[i].y) * ps),
-                              pack_bf16(bf16lo(w[i].z) * ps, bf16hi(w[i].z) * ps),
-                              pack_bf16(bf16lo(w[i].w) * ps, bf16hi(w[i].w) * ps)};
+        ce_u32x4_t o = {pack_bf16(bf16lo(w[i].x) * ps, bf16hi(w[i].x) * ps),
+                        pack_bf16(bf16lo(w[i].y) * ps, bf16hi(w[i].y) * ps),
+                        pack_bf16(bf16lo(w[i].z) * ps, bf16hi(w[i].z) * ps),
+                        pack_bf16(bf16lo(w[i].w) * ps, bf16hi(w[i].w) * ps)};
+        if (tid + kCeThreads * i == tc) {
+            const int e = (int)(t & 7);
+            const uint32_t keep = (e & 1) ? 0x0000ffffu : 0xffff0000u, put = (e & 1) ? (corr << 16) : corr;
+            if ((e >> 1) == 0) o.x = (o.x & keep) | put;
+            if ((e >> 1) == 1) o.y = (o.y & keep) | put;
+            if ((e >> 1) == 2) o.z = (o.z & keep) | put;
+            if ((e >> 1) == 3) o.w = (o.w & keep) | put;
+        }
         __builtin_amdgcn_raw_buffer_store_b128(o, dst, voff, i * kCeThreads * 16, 0);
+        // The next chunk's arithmetic reuses the registers this store reads.  The compiler pads a
+        // 128-bit buffer store with wait states only when its scalar offset is not a register; with
+        // the offset in an SGPR some lanes were seen to store the overwritten value, so pad by hand.
+        asm volatile("s_nop 3");
         __builtin_amdgcn_sched_barrier(0);
     }
-    // the target column, by the lane that wrote its chunk (same-address stores of one lane stay in order)
-    if (valid && (int)((t >> 3) & (kCeThreads - 1)) == tid)
-        dr[t] = f32_to_bf16((__builtin_amdgcn_exp2f((xt - mx) * kLog2e) / s - 1.0f) * scale);
 }
 
 // fp32 logits (small class counts): one wave per row, three passes over the row.

@@ -404,6 +404,37 @@ def test_ce_loss_bf16(rows, V, ld):
     assert torch.equal(loss, loss2)
 
 
+@pytest.mark.parametrize("rows,V", [(4096, 50257), (2048, 32000)])
+def test_ce_loss_bf16_full_size_is_exact_per_element_and_repeatable(rows, V):
+    """The logits of a whole microbatch (every CU holds two rows at a time): each gradient element
+    against softmax - onehot computed by torch on the GPU in fp32, not only the largest error of the
+    tensor, the same bits on every run, and the same bits when the gradient overwrites the logits."""
+    Nn = native()
+    torch.manual_seed(12)
+    ld = (V + 127) // 128 * 128
+    buf = torch.zeros(rows, ld, device=DEV, dtype=torch.bfloat16)
+    buf[:, :V] = torch.randn(rows, V, device=DEV).to(torch.bfloat16)
+    target = torch.randint(0, V, (rows,), device=DEV)
+    runs = []
+    for _ in range(3):
+        loss = torch.empty(1, device=DEV)
+        d = torch.full((rows, ld), float("nan"), device=DEV, dtype=torch.bfloat16)
+        Nn.ce_loss(buf, target, loss, d, torch.empty(rows + 2, device=DEV), V)
+        runs.append((loss, d))
+    ref = torch.softmax(buf[:, :V].float(), -1)
+    ref[torch.arange(rows, device=DEV), target] -= 1
+    ref /= rows
+    got = runs[0][1][:, :V].float()
+    # bf16 rounding of the result (2^-8 relative) plus that of the stored exponentials
+    assert bool(((got - ref).abs() <= 2.0 ** -6 * ref.abs() + 1e-9).all())
+    assert bool((runs[0][1][:, V:] == 0).all())
+    for loss, d in runs[1:]:
+        assert torch.equal(loss, runs[0][0]) and torch.equal(d, runs[0][1])
+    inplace = buf.clone()
+    Nn.ce_loss(inplace, target, torch.empty(1, device=DEV), inplace, torch.empty(rows + 2, device=DEV), V)
+    assert torch.equal(inplace, runs[0][1])
+
+
 def test_ce_loss_f32():
     Nn = native()
     torch.manual_seed(11)
