@@ -188,14 +188,29 @@ __global__ __launch_bounds__(256) void colreduce_partial_kernel(
     }
 }
 
+// part[0], part[stride], ... summed in that order; the loads of 8 terms are issued together, the
+// additions stay a chain (a loop of load-then-add pays one memory latency per term).
+__device__ __forceinline__ float ordered_column_sum(const float* __restrict__ part, int64_t n, int64_t stride) {
+    float t = 0.f;
+    int64_t p = 0;
+    for (; p + 8 <= n; p += 8) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = part[(p + k) * stride];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t += v[k];
+    }
+    for (; p < n; ++p) t += part[p * stride];
+    return t;
+}
+
 // Stage 2: ordered sum of the per-row-block partials, one lane per column.
 __global__ __launch_bounds__(256) void colreduce_final_kernel(const float* __restrict__ part,
                                                               int64_t n_part, int64_t C, void* out,
                                                               int out_f32) {
     const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    float t = 0.f;
-    for (int64_t p = 0; p < n_part; ++p) t += part[p * C + c];
+    const float t = ordered_column_sum(part + c, n_part, C);
     if (out_f32) static_cast<float*>(out)[c] = t;
     else static_cast<uint16_t*>(out)[c] = f32_to_bf16(t);
 }
@@ -288,8 +303,7 @@ __global__ __launch_bounds__(256) void colgroup_final_kernel(const ColGroupArgs 
         void* out = pass == 0 ? d.out_sum : d.out_dot;
         if (!out || (pass == 1 && !d.x)) continue;
         const float* part = d.ws + (int64_t)pass * d.n_part * d.C;
-        float t = 0.f;
-        for (int p = 0; p < d.n_part; ++p) t += part[(int64_t)p * d.C + c];
+        const float t = ordered_column_sum(part + c, d.n_part, d.C);
         if (d.out_f32) static_cast<float*>(out)[c] = t;
         else static_cast<uint16_t*>(out)[c] = f32_to_bf16(t);
     }
