@@ -388,21 +388,6 @@ typedef struct pp_op {
  * failing op is in pp_last_error()). */
 int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream);
 
-/* The same, replayed as a HIP graph once the list has settled (no reference counterpart: the
- * reference issues every kernel from Python).  The cache belongs to one list; it is keyed by a hash
- * of the descriptor bytes, so a list whose pointers or flags are patched between runs gets one graph
- * per variant (at most 6; the least recently used one is dropped).  A variant runs eagerly twice
- * before it is captured; on the default stream, while per-launch timing is on, or after a failed
- * capture the call is pp_run_ops.  Unless `always` is non-zero a variant is only captured when it is
- * bound by launching its kernels rather than by running them (at least 8 ops averaging under 8 us of
- * estimated work): lists of large kernels gain nothing from a graph.  Lists hold kernel launches
- * only (no memset or copy nodes).  Not thread-safe. */
-typedef void* pp_graph_cache;
-int pp_graph_cache_create(pp_graph_cache* out);
-int pp_graph_cache_destroy(pp_graph_cache cache);
-int pp_graph_cache_size(pp_graph_cache cache); /* graphs currently instantiated */
-int pp_run_ops_graphed(const pp_op* ops, int n_ops, pp_stream stream, pp_graph_cache cache, int always);
-
 /* ------------------------------------------------------------------------------------------
  * Per-launch timing of launch-list ops (measurement aid; no reference counterpart).  Between
  * pp_profile_start and pp_profile_stop every op run by pp_run_ops is bracketed by two HIP events on

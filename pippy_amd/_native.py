@@ -7,7 +7,6 @@ work on that stream.
 from __future__ import annotations
 
 import ctypes as C
-import os
 from typing import Optional, Sequence
 
 import torch
@@ -39,8 +38,7 @@ EXPORTED_SYMBOLS = (
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
     "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
-    "pp_ce_loss", "pp_run_ops", "pp_run_ops_graphed", "pp_graph_cache_create", "pp_graph_cache_destroy",
-    "pp_graph_cache_size", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
+    "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
     "pp_moe_gate_bwd",
@@ -126,10 +124,6 @@ def lib() -> C.CDLL:
         "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
-        "pp_run_ops_graphed": [C.POINTER(Op), i32, vp, vp, i32],
-        "pp_graph_cache_create": [C.POINTER(vp)],
-        "pp_graph_cache_destroy": [vp],
-        "pp_graph_cache_size": [vp],
         "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
         "pp_transpose_bf16": [vp, i64, i64, i64, vp, i64, vp],
         "pp_profile_start": [i32],
@@ -610,39 +604,6 @@ def transpose_bf16(src: torch.Tensor, dst: torch.Tensor) -> None:
 
 def run_ops(ops, n: int) -> None:
     check(lib().pp_run_ops(ops, n, current_stream()), "pp_run_ops")
-
-
-class GraphCache:
-    """The HIP graphs of one launch list (``pp_graph_cache``), freed with the object."""
-
-    def __init__(self):
-        self._h = C.c_void_p()
-        check(lib().pp_graph_cache_create(C.byref(self._h)), "pp_graph_cache_create")
-
-    def __len__(self) -> int:
-        return int(lib().pp_graph_cache_size(self._h))
-
-    def __del__(self):
-        h, self._h = getattr(self, "_h", None), None
-        if h:
-            try:
-                lib().pp_graph_cache_destroy(h)
-            except Exception:  # interpreter shutdown
-                pass
-
-
-GRAPH_MIN_OPS = 8  # shorter lists are never captured unless PIPPY_AMD_GRAPHS=2 (kMinOpsForGraph)
-
-
-def graph_mode() -> int:
-    """PIPPY_AMD_GRAPHS: 0 - launch lists always run kernel by kernel; 1 (default) - a list that is
-    bound by launching its kernels is replayed as a HIP graph; 2 - every list is."""
-    v = os.environ.get("PIPPY_AMD_GRAPHS", "1")
-    return int(v) if v in ("0", "1", "2") else 1
-
-
-def run_ops_graphed(ops, n: int, cache: GraphCache, always: bool = False) -> None:
-    check(lib().pp_run_ops_graphed(ops, n, current_stream(), cache._h, int(always)), "pp_run_ops_graphed")
 
 
 # ---- per-launch timing ---------------------------------------------------------------------------

@@ -446,7 +446,6 @@ class OpList:
     def __init__(self):
         self.ops: List[N.Op] = []
         self._arr = None
-        self._graphs = None  # N.GraphCache, created with the first graphed run
 
     def append(self, op: N.Op) -> int:
         assert self._arr is None, "list is frozen"
@@ -464,14 +463,7 @@ class OpList:
     def run(self):
         if self._arr is None:
             self.freeze()
-        if not self.n:
-            return
-        mode = N.graph_mode()
-        if mode:
-            if self._graphs is None:
-                self._graphs = N.GraphCache()
-            N.run_ops_graphed(self._arr, self.n, self._graphs, always=mode == 2)
-        else:
+        if self.n:
             N.run_ops(self._arr, self.n)
 
     def __getitem__(self, k) -> N.Op:

@@ -306,157 +306,3 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     }
     return PP_OK;
 }
-
-// ---- launch lists replayed as HIP graphs ------------------------------------------------------
-// A launch list is a fixed sequence of kernel launches (no allocation, no memset, no host
-// synchronisation), so once its descriptors stop changing it can be captured into a graph and
-// replayed with one call.  The cache is keyed by a hash of the descriptor bytes: patching a pointer
-// or a flag of the list simply selects (or creates) another graph.
-namespace pp {
-
-struct GraphEntry {
-    uint64_t hash = 0;
-    int n_ops = 0;
-    int seen = 0;          // eager runs of exactly this content
-    bool refused = false;  // capture failed once: stay eager
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
-    uint64_t last_use = 0;
-};
-
-struct GraphCache {
-    std::vector<GraphEntry> entries;
-    uint64_t clock = 0;
-};
-
-constexpr size_t kMaxGraphsPerList = 6;
-constexpr int kEagerRunsBeforeCapture = 2;
-
-// A graph pays when the list is bound by launching its kernels, not by running them: measured on
-// this part, a 2-stage decoder of width 128 steps 2.8 times faster with graphs (1.7 against 4.8 ms),
-// lists of two to four kernels run slower (one graph launch costs more than a few kernel launches)
-// and the GPT-2-small step, whose kernels average 40 us, loses 1 %.  The estimate below prices
-// MFMA-bound ops at 400 TFLOP/s and the others at 3 TB/s.
-constexpr int kMinOpsForGraph = 8;
-constexpr double kMaxAvgOpMicrosForGraph = 8.0;
-
-static bool launch_bound(const pp_op* ops, int n) {
-    int launches = 0;
-    double us = 0.0;
-    for (int i = 0; i < n; ++i) {
-        if (ops[i].flags & PP_OP_SKIP) continue;
-        ++launches;
-        const int k = ops[i].kind;
-        const bool mfma = k == PP_OP_GEMM_BF16 || k == PP_OP_GEMM_F32 || k == PP_OP_GEMM_SEG ||
-                          k == PP_OP_ATTN_FWD || k == PP_OP_ATTN_BWD;
-        us += op_work(ops[i]) / (mfma ? 400e6 : 3e6);
-    }
-    return launches >= kMinOpsForGraph && us <= kMaxAvgOpMicrosForGraph * launches;
-}
-
-static uint64_t hash_ops(const pp_op* ops, int n) {
-    // FNV-1a over 64-bit words (pp_op is a multiple of 8 bytes)
-    static_assert(sizeof(pp_op) % 8 == 0, "pp_op hashes as 64-bit words");
-    const uint64_t* w = reinterpret_cast<const uint64_t*>(ops);
-    const size_t nw = (size_t)n * sizeof(pp_op) / 8;
-    uint64_t h = 1469598103934665603ull ^ (uint64_t)n;
-    for (size_t i = 0; i < nw; ++i) {
-        h ^= w[i];
-        h *= 1099511628211ull;
-    }
-    return h;
-}
-
-static void release(GraphEntry& e) {
-    if (e.exec) (void)hipGraphExecDestroy(e.exec);
-    if (e.graph) (void)hipGraphDestroy(e.graph);
-    e.exec = nullptr;
-    e.graph = nullptr;
-}
-
-}  // namespace pp
-
-extern "C" int pp_graph_cache_create(pp_graph_cache* out) {
-    if (!out) return fail(PP_ERR_INVALID, "pp_graph_cache_create: null pointer");
-    *out = new GraphCache();
-    return PP_OK;
-}
-
-extern "C" int pp_graph_cache_destroy(pp_graph_cache cache) {
-    GraphCache* c = static_cast<GraphCache*>(cache);
-    if (!c) return PP_OK;
-    for (GraphEntry& e : c->entries) release(e);
-    delete c;
-    return PP_OK;
-}
-
-extern "C" int pp_graph_cache_size(pp_graph_cache cache) {
-    GraphCache* c = static_cast<GraphCache*>(cache);
-    int n = 0;
-    if (c)
-        for (const GraphEntry& e : c->entries) n += e.exec != nullptr;
-    return n;
-}
-
-extern "C" int pp_run_ops_graphed(const pp_op* ops, int n_ops, pp_stream stream, pp_graph_cache cache,
-                                  int always) {
-    GraphCache* c = static_cast<GraphCache*>(cache);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    // the default stream cannot be captured; per-op timing needs the ops as separate launches
-    if (!c || !st || g_prof_on || n_ops <= 0) return pp_run_ops(ops, n_ops, stream);
-    const uint64_t h = hash_ops(ops, n_ops);
-    GraphEntry* e = nullptr;
-    for (GraphEntry& x : c->entries)
-        if (x.hash == h && x.n_ops == n_ops) e = &x;
-    if (!e) {
-        if (c->entries.size() >= kMaxGraphsPerList) {
-            size_t victim = 0;
-            for (size_t i = 1; i < c->entries.size(); ++i)
-                if (c->entries[i].last_use < c->entries[victim].last_use) victim = i;
-            release(c->entries[victim]);
-            c->entries.erase(c->entries.begin() + victim);
-        }
-        c->entries.emplace_back();
-        e = &c->entries.back();
-        e->hash = h;
-        e->n_ops = n_ops;
-        e->refused = !always && !launch_bound(ops, n_ops);
-    }
-    e->last_use = ++c->clock;
-    if (e->exec) {
-        if (hipGraphLaunch(e->exec, st) != hipSuccess) return fail(PP_ERR_LAUNCH, "pp_run_ops_graphed: graph launch failed");
-        return PP_OK;
-    }
-    if (e->refused || e->seen < kEagerRunsBeforeCapture) {
-        ++e->seen;
-        return pp_run_ops(ops, n_ops, stream);
-    }
-    // Every kernel of this list has run eagerly before (one-time function attributes are set), so
-    // the capture records launches only; nothing executes until the graph is launched below.
-    if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess) {
-        (void)hipGetLastError();
-        e->refused = true;
-        return pp_run_ops(ops, n_ops, stream);
-    }
-    const int rc = pp_run_ops(ops, n_ops, stream);
-    hipGraph_t graph = nullptr;
-    const hipError_t end = hipStreamEndCapture(st, &graph);
-    if (rc != PP_OK || end != hipSuccess || !graph) {
-        (void)hipGetLastError();
-        if (graph) (void)hipGraphDestroy(graph);
-        e->refused = true;
-        if (rc != PP_OK) return rc;  // a bad descriptor: the message is already set
-        return pp_run_ops(ops, n_ops, stream);
-    }
-    hipGraphExec_t exec = nullptr;
-    if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess || !exec) {
-        (void)hipGetLastError();
-        (void)hipGraphDestroy(graph);
-        e->refused = true;
-        return pp_run_ops(ops, n_ops, stream);
-    }
-    e->graph = graph;
-    e->exec = exec;
-    if (hipGraphLaunch(exec, st) != hipSuccess) return fail(PP_ERR_LAUNCH, "pp_run_ops_graphed: graph launch failed");
-    return PP_OK;
-}

@@ -63,9 +63,6 @@ def _group_size(group) -> int:
         raise TypeError(f"unsupported group object {group!r}") from e
 
 
-_INPUT_COPY_BYTES = 1 << 20  # first-stage inputs up to this size are copied into a fixed slot
-
-
 class PipelineStageBase:
     """State and per-microbatch entry points shared by ``PipelineStage`` and
     ``ManualPipelineStage`` (reference ``_PipelineStage.py:72-551``)."""
@@ -281,27 +278,18 @@ class PipelineStageBase:
         x, dx_target, patch = self._input_for(mb, args, kwargs)
         prog = sp.mbs.get(mb)
         if patch:
+            if not x.is_contiguous() or (x.data_ptr() % 16):
+                xc = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+                N.strided_copy_nd(xc, x)
+                x = xc
             key = (tuple(x.shape), x.dtype)
             if prog is None or prog.in_key[:2] != key:
                 slot = torch.empty(x.shape, dtype=x.dtype, device=self.device)
                 prog = sp.build(mb, slot, None)
                 prog.input_patches = [(lst, k, q) for lst in (prog.F, prog.I, prog.W)
                                       for (k, q) in lst.find_pointer(slot.data_ptr())]
-            mode = N.graph_mode()
-            if x.numel() * x.element_size() <= _INPUT_COPY_BYTES and \
-                    (mode == 2 or (mode == 1 and prog.F.n >= N.GRAPH_MIN_OPS)):
-                # a small input (token ids) is copied into the slot the lists were built on: their
-                # descriptors then stay the same from step to step and the lists can run as graphs
-                N.strided_copy_nd(prog.input_slot, x)
-                src = prog.input_slot
-            else:
-                src = x
-                if not x.is_contiguous() or (x.data_ptr() % 16):
-                    src = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-                    N.strided_copy_nd(src, x)
             for lst, k, q in prog.input_patches:
-                lst[k].p[q] = src.data_ptr()
-            x = src
+                lst[k].p[q] = x.data_ptr()
         else:
             key = (tuple(x.shape), x.dtype, x.data_ptr(), P._p(dx_target))
             if prog is None or prog.in_key != key:
