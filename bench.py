@@ -182,7 +182,7 @@ def main():
                          "kernel (the same bits as the default, one more pass over the parameters)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--serial-stages", action="store_true",
-                    help="run all virtual stages on one stream instead of one stream per stage")
+                    help="run all virtual stages on one stream instead of two")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
