@@ -482,6 +482,55 @@ def test_attention(causal, B, S, H, D):
         assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"attention {name}")
 
 
+@pytest.mark.parametrize("B,S,H,D,causal", [(4, 1024, 12, 64, True), (8, 512, 12, 64, False),
+                                           (1, 2048, 32, 128, True)])
+def test_attention_full_size_with_equal_keys_is_a_running_mean(B, S, H, D, causal):
+    """The attention shapes of the full-size configurations.  When all keys of a head are the same
+    vector every allowed score is equal, so row i of the output is the mean of the values 0..i
+    (causal) or of all values, whatever the queries are, and the log-sum-exp is that score plus
+    log(count): closed forms computed with cumsum, no O(S^2) reference."""
+    Nn = native()
+    torch.manual_seed(S + D)
+    HD = H * D
+    qkv = torch.randn(B, S, 3 * HD, device=DEV).to(torch.bfloat16)
+    key = torch.randn(B, 1, HD, device=DEV).to(torch.bfloat16)
+    qkv[..., HD:2 * HD] = key                    # one key vector per (batch, head)
+    o = torch.full((B, S, HD), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    Nn.attn_fwd(qkv, o, lse, H, causal)
+    v = qkv[..., 2 * HD:].float()
+    count = torch.arange(1, S + 1, device=DEV, dtype=torch.float32) if causal else \
+        torch.full((S,), float(S), device=DEV)
+    want = v.cumsum(1) / count.view(1, S, 1) if causal else v.mean(1, keepdim=True).expand(B, S, HD)
+    # probabilities are rounded to bf16 before the second product: 2^-9 relative per term
+    assert float((o.float() - want).abs().max()) <= 2e-2 * float(want.abs().max())
+    q = qkv[..., :HD].float().view(B, S, H, D)
+    score = (q * key.float().view(B, 1, H, D)).sum(-1) / math.sqrt(D)          # [B, S, H]
+    want_lse = score.permute(0, 2, 1) + torch.log(count).view(1, 1, S)
+    assert float((lse - want_lse).abs().max()) <= 1e-2 * max(1.0, float(want_lse.abs().max()))
+
+
+@pytest.mark.parametrize("M,N,K,at,bt", [(4096, 768, 768, False, False), (4096, 2304, 768, False, False),
+                                         (4096, 50304, 768, False, False), (4096, 768, 50304, False, False),
+                                         (3072, 768, 4096, True, True), (2048, 11008, 4096, False, False)])
+def test_gemm_bf16_full_size_selects_rows_exactly(M, N, K, at, bt):
+    """GEMM shapes of the full-size configurations (every tile shape the dispatcher picks).  With
+    one-hot rows in A the product is a row selection of B: C[m, :] = B[:, k_m], which bf16
+    reproduces exactly, so every element of C checks the indexing of its tile bit for bit."""
+    Nn = native()
+    g = torch.Generator(device=DEV).manual_seed(M + N + K)
+    pick = torch.randint(0, K, (M,), device=DEV, generator=g)
+    A = torch.zeros(M, K, device=DEV, dtype=torch.bfloat16)
+    A[torch.arange(M, device=DEV), pick] = 1
+    Bm = torch.randn(N, K, device=DEV, generator=g).to(torch.bfloat16)
+    want = Bm[:, pick].t().contiguous()
+    Aop = A.t().contiguous() if at else A
+    Bop = Bm.t().contiguous() if bt else Bm
+    C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    Nn.gemm_bf16(Aop, Bop, C, a_trans=at, b_trans=bt)
+    assert torch.equal(C, want)
+
+
 # ---- launch list ---------------------------------------------------------------------------------
 def test_run_ops_matches_direct_calls():
     import ctypes as C
