@@ -379,6 +379,37 @@ def test_embedding():
     assert_close_rel(d_wpe, pr.grad, 1e-5, "d_wpe")
 
 
+def test_embedding_and_layernorm_full_size_closed_forms():
+    """The embedding and LayerNorm shapes of the GPT-2-small stage (4096 tokens, width 768, 50257
+    tokens in the table).  A zero position table makes the embedding an exact gather; rows of the
+    form s_r * (+1, -1, +1, ...) have mean 0 and variance s_r^2, so LayerNorm returns +-gamma + beta
+    for every row."""
+    Nn = native()
+    torch.manual_seed(31)
+    vocab, seq, C, B = 50257, 1024, 768, 4
+    wte = torch.randn(vocab, C, device=DEV).to(torch.bfloat16)
+    ids = torch.randint(0, vocab, (B, seq), device=DEV)
+    y = torch.full((B * seq, C), float("nan"), device=DEV, dtype=torch.bfloat16)
+    Nn.embed_fwd(ids, wte, torch.zeros(seq, C, device=DEV, dtype=torch.bfloat16), y, seq)
+    assert torch.equal(y, wte[ids.reshape(-1)])
+
+    rows = B * seq
+    sign = torch.ones(C, device=DEV)
+    sign[1::2] = -1
+    scale = torch.exp2(torch.randint(-6, 7, (rows, 1), device=DEV).float())   # exact in bf16
+    x = (scale * sign).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(C, device=DEV)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(C, device=DEV)).to(torch.bfloat16)
+    out = torch.empty_like(x)
+    mean = torch.empty(rows, device=DEV)
+    rstd = torch.empty(rows, device=DEV)
+    Nn.layernorm_fwd(x, gamma, beta, out, mean, rstd, 0.0)
+    want = (sign * gamma.float() + beta.float()).to(torch.bfloat16).expand(rows, C)
+    assert float(mean.abs().max()) == 0.0
+    assert float((rstd * scale.view(-1) - 1).abs().max()) <= 1e-6
+    assert torch.equal(out, want)
+
+
 @pytest.mark.parametrize("rows,V,ld", [(64, 1000, 1000), (33, 1001, 1008), (128, 50257, 50304), (16, 8, 8)])
 def test_ce_loss_bf16(rows, V, ld):
     Nn = native()
