@@ -918,6 +918,51 @@ def test_segmented_gemm_rows_mode(R, K, Nn, E):
 
 
 @pytest.mark.gpu
+def test_segmented_gemms_full_size_equal_one_dense_gemm_per_expert():
+    """The expert GEMMs of the Mixtral-style configuration (4096 permuted rows, 8 ragged segments,
+    1024 -> 4096): the segmented kernels run the dense kernel's tile code, so rows mode must give
+    the bits of one dense GEMM per expert, k mode those of one transposed dense GEMM per expert
+    (also through the rounded accumulation), and a second run the same bits again."""
+    N = native()
+    torch.manual_seed(41)
+    R, K, Nn, E = 4096, 1024, 4096, 8
+    bounds = [0, 450, 1010, 1500, 1500, 2560, 3100, 3620, 4096]     # one empty segment
+    seg = torch.tensor(bounds, dtype=torch.int32, device=DEV)
+    A = (torch.randn(R, K, device=DEV) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(E, Nn, K, device=DEV) * 0.05).to(torch.bfloat16)
+    ptrs = torch.tensor([W[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    want = torch.zeros(R, Nn, device=DEV, dtype=torch.bfloat16)
+    for e in range(E):
+        r0, r1 = bounds[e], bounds[e + 1]
+        if r1 > r0:
+            N.gemm_bf16(A[r0:r1], W[e], want[r0:r1])
+    for _ in range(2):
+        got = torch.full((R, Nn), float("nan"), device=DEV, dtype=torch.bfloat16)
+        N.gemm_bf16_segmented(A, ptrs, got, seg, N.SEG_ROWS)
+        assert torch.equal(got, want)
+    # k mode: dW_e = dY[r0:r1]^T X[r0:r1], accumulated on top of earlier sums
+    dY = (torch.randn(R, Nn, device=DEV) * 0.5).to(torch.bfloat16)
+    start = torch.randn(E, Nn, K, device=DEV)
+    want_acc = start.clone()
+    g = torch.empty(Nn, K, device=DEV, dtype=torch.bfloat16)
+    for e in range(E):
+        r0, r1 = bounds[e], bounds[e + 1]
+        if r1 > r0:
+            rows = (r1 - r0 + 7) // 8 * 8          # the dense entry point wants K in multiples of 8
+            dYp = torch.zeros(rows, Nn, device=DEV, dtype=torch.bfloat16)
+            Xp = torch.zeros(rows, K, device=DEV, dtype=torch.bfloat16)
+            dYp[:r1 - r0], Xp[:r1 - r0] = dY[r0:r1], A[r0:r1]
+            N.gemm_bf16(dYp, Xp, g, a_trans=True, b_trans=True)
+            want_acc[e] += g.float()
+    for _ in range(2):
+        acc = start.clone()
+        aptrs = torch.tensor([acc[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+        N.gemm_bf16_segmented(dY, aptrs, None, seg, N.SEG_K, other=A, epilogue=N.EPI_ACCUM_ROUNDED, beta=1,
+                              c_dtype=torch.float32)
+        assert torch.equal(acc, want_acc)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("R,M,Nn,E", [(4096, 512, 1024, 8), (1000, 128, 136, 4), (50, 8, 64, 3)])
 def test_segmented_gemm_k_mode(R, M, Nn, E):
     N = native()
