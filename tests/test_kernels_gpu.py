@@ -519,7 +519,8 @@ def test_attention_full_size_with_equal_keys_is_a_running_mean(B, S, H, D, causa
     """The attention shapes of the full-size configurations.  When all keys of a head are the same
     vector every allowed score is equal, so row i of the output is the mean of the values 0..i
     (causal) or of all values, whatever the queries are, and the log-sum-exp is that score plus
-    log(count): closed forms computed with cumsum, no O(S^2) reference."""
+    log(count): closed forms computed with cumsum, no O(S^2) reference.  Backward: dQ vanishes and
+    dV is a (reversed) cumulative sum of dO / count."""
     Nn = native()
     torch.manual_seed(S + D)
     HD = H * D
@@ -539,6 +540,20 @@ def test_attention_full_size_with_equal_keys_is_a_running_mean(B, S, H, D, causa
     score = (q * key.float().view(B, 1, H, D)).sum(-1) / math.sqrt(D)          # [B, S, H]
     want_lse = score.permute(0, 2, 1) + torch.log(count).view(1, 1, S)
     assert float((lse - want_lse).abs().max()) <= 1e-2 * max(1.0, float(want_lse.abs().max()))
+    # backward: uniform probabilities do not depend on the queries, so dQ = 0, and
+    # dV[j] = sum over the rows i that see key j of dO[i] / count[i] (a reversed cumsum when causal)
+    d_o = torch.randn(B, S, HD, device=DEV).to(torch.bfloat16)
+    dqkv = torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal)
+    w = d_o.float() / count.view(1, S, 1)
+    want_dv = w.flip(1).cumsum(1).flip(1) if causal else w.sum(1, keepdim=True).expand(B, S, HD)
+    got_dv = dqkv[..., 2 * HD:].float()
+    assert float((got_dv - want_dv).abs().max()) <= 2e-2 * float(want_dv.abs().max())
+    # dQ is a sum of terms that cancel: compare with the size of the terms, |dO| |V| |K| / sqrt(D)
+    term = float(d_o.float().abs().max() * v.abs().max() * key.float().abs().max()) / math.sqrt(D)
+    assert float(dqkv[..., :HD].float().abs().max()) <= 2e-2 * term
+    assert bool(torch.isfinite(dqkv.float()).all())
 
 
 @pytest.mark.parametrize("M,N,K,at,bt", [(4096, 768, 768, False, False), (4096, 2304, 768, False, False),
