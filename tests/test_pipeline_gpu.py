@@ -1,6 +1,7 @@
 """End-to-end parity of the pipeline (split -> staged forward/backward -> accumulate -> merge) on
 the GPU against the fp32 CPU oracle, through the reference's own API surface."""
 import copy
+import math
 
 import pytest
 import torch
@@ -116,6 +117,42 @@ def test_schedules_agree_bitwise_and_match_oracle():
                 assert max_rel(grads[k], base_grads[k]) <= 1e-6, f"{name}: {k}"
             else:
                 assert torch.equal(grads[k], base_grads[k]), f"{name}: grad of {k} differs from GPipe"
+
+
+def test_gpt2_small_full_size_schedules_and_repeats_agree_bit_for_bit():
+    """The headline configuration at full size (12 layers of width 768, vocabulary 50257, 32 x 1024
+    tokens in 8 microbatches, 4 virtual stages on two streams): 1F1B twice and GPipe once must give
+    the same logits, losses and (sampled) gradient accumulators bit for bit, and the loss of a
+    uniform guess at initialisation.  Races between the stage streams or schedule-dependent
+    accumulation order would show here."""
+    import pippy_amd as pp
+    from pippy_amd.configs import DecoderLM, equal_split_spec
+    torch.manual_seed(0)
+    M = 8
+    with torch.device(DEV):
+        model = DecoderLM(vocab=50257, max_seq=1024, dim=768, n_layers=12, n_heads=12, ffn=3072)
+    ids = torch.randint(0, 50257, (32, 1024), device=DEV)
+    target = torch.randint(0, 50257, (32, 1024), device=DEV)
+    pipe = pp.pipeline(model, M, (ids,), split_spec=equal_split_spec(12, 4))
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(4)]
+    assert all(st.is_native for st in stages)
+    named = dict(model.named_parameters())
+    probe = ["h.0.attn.c_attn.weight", "h.5.mlp.c_proj.weight", "h.11.ln_2.weight", "h.7.attn.c_proj.bias",
+             "h.3.mlp.c_fc.weight", "h.9.ln_1.bias"] + [n for n in named if n.startswith("head.")]
+    assert all(n in named for n in probe) and len(probe) >= 7
+    results = []
+    for cls in (pp.Schedule1F1B, pp.ScheduleGPipe, pp.Schedule1F1B):
+        sched = cls(stages, M, loss_fn=pp.CrossEntropyLoss())
+        sched.zero_grad()
+        losses = []
+        out = sched.step(ids, target=target, losses=losses)
+        results.append((out, torch.stack(losses).clone(), [named[n].main_grad.clone() for n in probe]))
+    base = results[0]
+    assert torch.isfinite(base[0].float()).all() and abs(float(base[1][0]) - math.log(50257)) < 0.3
+    for out, losses, grads in results[1:]:
+        assert torch.equal(out, base[0]) and torch.equal(losses, base[1])
+        for n, a, b in zip(probe, grads, base[2]):
+            assert float(a.abs().max()) > 0 and torch.equal(a, b), f"grad of {n}"
 
 
 def test_two_steps_accumulate_then_zero_grad():
