@@ -147,6 +147,15 @@ typedef struct pp_gemm_desc {
  * its contiguous extent (M resp. N) % 8 == 0; ldc, ld_aux % 4 == 0 (bf16) . */
 int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
 
+/* pp_gemm_bf16 with a workspace of `workspace_elems` floats (16-byte aligned) that lets the library
+ * split a long reduction: for k-contiguous A and B, a plain bf16 C (epilogue NONE, N and ldc
+ * multiples of 4) with at most 64 tiles of 256 x 256 it runs up to 8 splits of K, of at least 4096
+ * each, on 256 x 256 tiles (each into its own fp32 copy of C, splits * M * N floats) and adds the copies
+ * in split order; any other problem, or a workspace that is too small, runs as pp_gemm_bf16.  The
+ * input-gradient GEMM of a vocabulary projection (F.linear backward with K = vocabulary) is the case
+ * it is for.  The workspace must not be shared by launches that may overlap. */
+int pp_gemm_bf16_splitk(const pp_gemm_desc* desc, float* workspace, int64_t workspace_elems, pp_stream stream);
+
 /* Several independent GEMMs in one launch (up to PP_GEMM_MAX_GROUP; longer lists are split).  All
  * descriptors must agree in a_trans, b_trans, epilogue and c_dtype.  The weight-gradient GEMMs of
  * one stage and microbatch (pippy/_backward.py:67-69 reaches them through autograd one by one) are
@@ -345,7 +354,8 @@ enum pp_op_kind {
 
 /* Field use per kind (unused fields are ignored):
  *   GEMM_*        p: A B C bias aux_in aux_out | i: M N K lda ldb ldc ld_aux | j: a_trans b_trans
- *                 epilogue c_dtype beta
+ *                 epilogue c_dtype beta; GEMM_BF16 also p[8]: split-K workspace or null, i[10]: its
+ *                 size in floats (then the op is pp_gemm_bf16_splitk)
  *   COLSUM        p: dY out workspace | i: M N ld | j: out_dtype
  *   LN_FWD        p: x gamma beta y mean rstd | i: rows C | f: eps
  *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C

@@ -36,7 +36,7 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
@@ -112,6 +112,7 @@ def lib() -> C.CDLL:
         "pp_fill_bytes": [vp, i32, i64, vp],
         "pp_gemm_bf16": [C.POINTER(GemmDesc), vp],
         "pp_gemm_f32": [C.POINTER(GemmDesc), vp],
+        "pp_gemm_bf16_splitk": [C.POINTER(GemmDesc), vp, i64, vp],
         "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
         "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],
@@ -444,6 +445,16 @@ def gemm_bf16(A, B, Cm, **kw) -> None:
     assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16
     d = gemm_desc(A, B, Cm, **kw)
     check(lib().pp_gemm_bf16(C.byref(d), current_stream()), "pp_gemm_bf16")
+
+
+def gemm_bf16_splitk(A, B, Cm, workspace: torch.Tensor, **kw) -> None:
+    """``gemm_bf16`` that may split a long K over several work-groups per tile, through ``workspace``
+    (fp32, up to 8 copies of C)."""
+    require_cuda(workspace)
+    assert workspace.dtype == torch.float32 and workspace.is_contiguous()
+    d = gemm_desc(A, B, Cm, **kw)
+    check(lib().pp_gemm_bf16_splitk(C.byref(d), workspace.data_ptr(), workspace.numel(), current_stream()),
+          "pp_gemm_bf16_splitk")
 
 
 def gemm_bf16_grouped(problems) -> None:

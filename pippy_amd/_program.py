@@ -162,7 +162,8 @@ def _p(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def op_gemm(A, B, Cm, *, a_trans=False, b_trans=False, epilogue=N.EPI_NONE, bias=None, aux_in=None,
-            aux_out=None, beta=0) -> N.Op:
+            aux_out=None, beta=0, splitk_workspace=None) -> N.Op:
+    """``splitk_workspace`` (fp32) lets the library split a long reduction (``pp_gemm_bf16_splitk``)."""
     f32 = A.dtype == torch.float32
     d = N.gemm_desc(A, B, Cm, a_trans=a_trans, b_trans=b_trans, epilogue=epilogue, bias=bias,
                     aux_in=aux_in, aux_out=aux_out, beta=beta)
@@ -173,7 +174,20 @@ def op_gemm(A, B, Cm, *, a_trans=False, b_trans=False, epilogue=N.EPI_NONE, bias
     op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = d.A, d.B, d.C, d.bias, d.aux_in, d.aux_out
     op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5], op.i[6] = d.M, d.N, d.K, d.lda, d.ldb, d.ldc, d.ld_aux
     op.j[0], op.j[1], op.j[2], op.j[3], op.j[4] = d.a_trans, d.b_trans, d.epilogue, d.c_dtype, d.beta
+    if splitk_workspace is not None:
+        assert not f32 and splitk_workspace.dtype == torch.float32 and splitk_workspace.is_contiguous()
+        op.p[8], op.i[10] = splitk_workspace.data_ptr(), splitk_workspace.numel()
     return op
+
+
+def splitk_copies(M: int, Nn: int, K: int) -> int:
+    """How many fp32 copies of an [M, Nn] output a k-split of this problem can use (0: none): at most
+    64 tiles of 256 x 256, splits of at least 4096 along K, at most 8 (the library's own rule)."""
+    tiles = ((M + 255) // 256) * ((Nn + 255) // 256)
+    if tiles > 64:
+        return 0
+    splits = min(256 // tiles, ((K + 63) // 64) // 64, 8)
+    return splits if splits >= 2 else 0
 
 
 def op_colsum(dY, out, ws) -> N.Op:

@@ -418,6 +418,50 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_dma_kernel(const GemmA
     gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT>(g, tile_m, tile_n);
 }
 
+// Split along K on 256 x 256 tiles, for an output with few tiles and a long reduction (the input
+// gradient of a vocabulary projection: 4096 x 768 with K = 50304).  Large tiles load half as many
+// operand bytes per FLOP as 128-wide ones, and the split makes enough of them to fill the CUs.
+// Split s of a tile reduces k-tiles [s * kt_per_split, (s + 1) * kt_per_split) into its own fp32
+// copy of C in the workspace; splitk_reduce_kernel adds the copies in split order.
+__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_splitk_kernel(const GemmArgs g, float* ws, int splits,
+                                                                       int kt_per_split) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks * (uint32_t)splits) return;
+    const int split = (int)(bid / g.n_blocks);
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid % g.n_blocks, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    f32x16_t acc[WaveTile<256, 256>::TN][WaveTile<256, 256>::TM];
+#pragma unroll
+    for (int a = 0; a < WaveTile<256, 256>::TN; ++a)
+#pragma unroll
+        for (int b = 0; b < WaveTile<256, 256>::TM; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+    const int nk = (int)((g.K + BK - 1) / BK);
+    const int kb = min(nk, split * kt_per_split), ke = min(nk, kb + kt_per_split);
+    gemm_mainloop<256, 256, false, false, 2, BK>(g, tile_m, tile_n, kb, ke, acc);
+    GemmArgs part = g;
+    part.C = ws + (size_t)split * (size_t)g.M * (size_t)g.N;
+    part.ldc = g.N;
+    gemm_epilogue<256, 256, PP_EPI_NONE, true>(part, tile_m, tile_n, acc);
+}
+
+// C (bf16) = ws[0] + ws[1] + ... + ws[splits - 1], added in that order; N and ldc multiples of 4.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int64_t M,
+                                                            int64_t N, uint16_t* __restrict__ C, int64_t ldc) {
+    const int64_t n4 = N >> 2;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * n4) return;
+    const int64_t m = idx / n4, c = (idx - m * n4) << 2;
+    const int64_t plane = M * N;
+    float4 t = *reinterpret_cast<const float4*>(ws + m * N + c);
+    for (int s = 1; s < splits; ++s) {
+        const float4 v = *reinterpret_cast<const float4*>(ws + (int64_t)s * plane + m * N + c);
+        t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+    }
+    *reinterpret_cast<uint2*>(C + m * ldc + c) = make_uint2(pack_bf16(t.x, t.y), pack_bf16(t.z, t.w));
+}
+
 // Several independent problems in one grid: the tiles of problem i are the block ids
 // [tile_start[i], tile_start[i + 1]).
 struct GemmGroupArgs {
@@ -838,4 +882,47 @@ extern "C" int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream 
     if (probs.empty()) return PP_OK;
     return dispatch(probs.data(), (int)probs.size(), f.a_trans ? 1 : 0, f.b_trans ? 1 : 0, f.epilogue,
                     f.c_dtype == PP_F32, static_cast<hipStream_t>(stream));
+}
+
+// Number of k-splits on 256 x 256 tiles that pays for this problem, or 0: k-contiguous operands, a
+// plain bf16 C, at most a quarter of a wave of such tiles and at least 64 k-tiles left per split.
+static int splitk_plan(const pp_gemm_desc* d, int64_t workspace_elems, int* kt_per_split) {
+    if (d->a_trans || d->b_trans || d->epilogue != PP_EPI_NONE || d->c_dtype != PP_BF16) return 0;
+    if ((d->N & 3) || (d->ldc & 3) || !aligned(d->C, 8)) return 0;
+    const int64_t tiles = ((d->M + 255) / 256) * ((d->N + 255) / 256);
+    const int64_t nk = (d->K + BK - 1) / BK;
+    if (tiles <= 0 || tiles > kComputeUnits / 4) return 0;  // 2048 x 4096 x 11008 (128 tiles) is faster unsplit
+    int64_t splits = kComputeUnits / tiles;
+    if (splits > nk / 64) splits = nk / 64;
+    if (splits > 8) splits = 8;
+    if (splits > workspace_elems / (d->M * d->N)) splits = workspace_elems / (d->M * d->N);
+    if (splits < 2) return 0;
+    *kt_per_split = (int)((nk + splits - 1) / splits);
+    return (int)splits;
+}
+
+extern "C" int pp_gemm_bf16_splitk(const pp_gemm_desc* d, float* workspace, int64_t workspace_elems,
+                                   pp_stream stream) {
+    GemmArgs g;
+    bool empty;
+    int rc = convert(d, &g, &empty);
+    if (rc || empty) return rc;
+    int kt_per_split = 0;
+    const int splits = (workspace && aligned(workspace, 16)) ? splitk_plan(d, workspace_elems, &kt_per_split) : 0;
+    if (!splits) return pp_gemm_bf16(d, stream);
+    rc = count_tiles<256, 256>(g);
+    if (rc) return rc;
+    constexpr size_t lds = (size_t)2 * (256 + 256) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_splitk_kernel, lds);
+    if (attr_rc) return attr_rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t grid = (g.n_blocks * (uint32_t)splits + 7) / 8 * 8;
+    hipLaunchKernelGGL(gemm_bf16_splitk_kernel, dim3(grid), dim3(kGemmThreads), lds, st, g, workspace, splits,
+                       kt_per_split);
+    rc = check_launch("gemm_bf16_splitk_kernel");
+    if (rc) return rc;
+    const int64_t quads = g.M * (g.N >> 2);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((quads + 255) / 256)), dim3(256), 0, st, workspace,
+                       splits, g.M, g.N, static_cast<uint16_t*>(g.C), g.ldc);
+    return check_launch("splitk_reduce_kernel");
 }

@@ -67,6 +67,8 @@ static int run_one(const pp_op& op, pp_stream st) {
         case PP_OP_GEMM_BF16:
         case PP_OP_GEMM_F32: {
             const pp_gemm_desc d = gemm_desc_of(op);
+            if (op.kind == PP_OP_GEMM_BF16 && op.p[8])  // a workspace for a split along K
+                return pp_gemm_bf16_splitk(&d, static_cast<float*>(op.p[8]), op.i[10], st);
             return op.kind == PP_OP_GEMM_BF16 ? pp_gemm_bf16(&d, st) : pp_gemm_f32(&d, st);
         }
         case PP_OP_COLSUM:

@@ -82,8 +82,14 @@ def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor
     if need_dx:
         dx = dx_out if dx_out is not None else b.grad(name + ".dx", (dY2d.shape[0], W.shape[1]))
         if W.dtype == torch.bfloat16:
-            # dX = dY W with the transposed weight copy: both operands k-contiguous
-            b.i(P.op_gemm(dY2d, b.weight_t(lin.weight), dx, epilogue=dx_epilogue, aux_in=dx_aux))
+            # dX = dY W with the transposed weight copy: both operands k-contiguous; a long reduction
+            # into a small output (the vocabulary projection) is split along K through a workspace
+            ws = None
+            copies = P.splitk_copies(dY2d.shape[0], W.shape[1], dY2d.shape[1])
+            if copies and dx_epilogue == N.EPI_NONE:
+                ws = b.workspace("splitk", (copies * dY2d.shape[0] * W.shape[1],), torch.float32)
+            b.i(P.op_gemm(dY2d, b.weight_t(lin.weight), dx, epilogue=dx_epilogue, aux_in=dx_aux,
+                          splitk_workspace=ws))
         else:
             b.i(P.op_gemm(dY2d, W, dx, b_trans=True, epilogue=dx_epilogue, aux_in=dx_aux))
     b.w_weight_gemm(dY2d, x2d, lin.weight, padded)

@@ -577,6 +577,37 @@ def test_gemm_bf16_full_size_selects_rows_exactly(M, N, K, at, bt):
     assert torch.equal(C, want)
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 768, 50304), (512, 256, 16384), (300, 200, 9000), (4096, 768, 768)])
+def test_gemm_bf16_split_along_k(M, N, K):
+    """pp_gemm_bf16_splitk: a long reduction into a small output runs as several k-splits on
+    256 x 256 tiles whose fp32 partial results are added in split order; problems it is not meant
+    for (the last case) fall back to the ordinary kernel.  One-hot rows in A make the exact answer
+    a row selection of B; random operands are compared with the fp32 product, and two runs agree."""
+    Nn = native()
+    g = torch.Generator(device=DEV).manual_seed(M + K)
+    ws = torch.empty(8 * M * N, device=DEV, dtype=torch.float32)
+    pick = torch.randint(0, K, (M,), device=DEV, generator=g)
+    A = torch.zeros(M, K, device=DEV, dtype=torch.bfloat16)
+    A[torch.arange(M, device=DEV), pick] = 1
+    Bm = torch.randn(N, K, device=DEV, generator=g).to(torch.bfloat16)
+    C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    Nn.gemm_bf16_splitk(A, Bm, C, ws)
+    assert torch.equal(C, Bm[:, pick].t().contiguous())
+    A = (torch.randn(M, K, device=DEV, generator=g) * 0.5).to(torch.bfloat16)
+    runs = []
+    for _ in range(2):
+        C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+        ws.fill_(float("nan"))
+        Nn.gemm_bf16_splitk(A, Bm, C, ws)
+        runs.append(C)
+    assert torch.equal(runs[0], runs[1])
+    ref = A.float() @ Bm.float().t()
+    assert_close_rel(runs[0], ref.cpu(), BF16_TOL, "split-K GEMM")
+    small = torch.empty(M * N, device=DEV, dtype=torch.float32)     # room for one copy only: no split
+    Nn.gemm_bf16_splitk(A, Bm, C, small)
+    assert_close_rel(C, ref.cpu(), BF16_TOL, "split-K GEMM without room to split")
+
+
 # ---- launch list ---------------------------------------------------------------------------------
 def test_run_ops_matches_direct_calls():
     import ctypes as C
