@@ -228,6 +228,7 @@ def test_gemm_bf16_epilogues(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,at,bt", [(768, 2304, 4096, True, True), (200, 136, 264, True, True),
+                                          (50304, 768, 4096, True, True), (11008, 4096, 2048, True, True),
                                           (256, 96, 512, False, False), (4096, 768, 64, False, True)])
 def test_gemm_bf16_rounded_accumulate_is_bit_exact(M, N, K, at, bt):
     """PP_EPI_ACCUM_ROUNDED leaves in an fp32 C what a bf16 C followed by the accumulate kernel
