@@ -400,9 +400,8 @@ int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-launch timing of launch-list ops (measurement aid; no reference counterpart).  Between
- * pp_profile_start and pp_profile_stop every op run by pp_run_ops is timed with two HIP events
- * (host-side event objects only; no device memory): a GEMM op that is one kernel launch carries them
- * as the start and stop events of its dispatch, every other op is bracketed by them on its stream.  pp_profile_read waits for the
+ * pp_profile_start and pp_profile_stop every op run by pp_run_ops is bracketed by two HIP events on
+ * its stream (host-side event objects only; no device memory).  pp_profile_read waits for the
  * recorded events and returns, for one op kind, the summed elapsed milliseconds, the summed
  * algorithmic work (FLOPs for GEMM and attention kinds, bytes for the HBM-bound kinds) and the
  * number of launches.  Not thread-safe.

@@ -1,7 +1,6 @@
 // Shared helpers for the gfx950 kernels: status reporting, bf16 bit conversions, wave utilities.
 #pragma once
 #include <hip/hip_runtime.h>
-#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
@@ -18,25 +17,6 @@ inline int fail(int code, const char* fmt, ...) {
     vsnprintf(error_buffer(), 512, fmt, ap);
     va_end(ap);
     return code;
-}
-
-// Per-launch timing: while these are set, the next kernel started through launch_timed carries them as
-// its own start / stop events (the timestamps of the dispatch itself, without the gap before it).
-struct LaunchEvents {
-    hipEvent_t start = nullptr, stop = nullptr;
-    bool used = false;
-};
-LaunchEvents& launch_events();
-
-template <typename Kernel, typename... Args>
-inline void launch_timed(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t st, Args... args) {
-    LaunchEvents& ev = launch_events();
-    if (ev.start && !ev.used) {
-        ev.used = true;
-        hipExtLaunchKernelGGL(kernel, grid, block, lds, st, ev.start, ev.stop, 0, args...);
-    } else {
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, args...);
-    }
 }
 
 inline int check_launch(const char* what) {

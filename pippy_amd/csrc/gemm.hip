@@ -608,7 +608,8 @@ static int launch_single(const GemmArgs& g, hipStream_t st) {
     static const int attr_rc = reserve_lds(&gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
     if (attr_rc) return attr_rc;
     const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
-    launch_timed(&gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, dim3(grid), dim3(kGemmThreads), lds, st, g);
+    hipLaunchKernelGGL((gemm_bf16_dma_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid), dim3(kGemmThreads),
+                       lds, st, g);
     return check_launch("gemm_bf16_dma_kernel");
 }
 
@@ -618,8 +619,8 @@ static int launch_group(const GemmGroupArgs& ga, hipStream_t st) {
     static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
     if (attr_rc) return attr_rc;
     const uint32_t grid = (ga.tile_start[ga.n] + 7) / 8 * 8;
-    launch_timed(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, dim3(grid), dim3(kGemmThreads), lds, st,
-                 ga);
+    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid), dim3(kGemmThreads),
+                       lds, st, ga);
     return check_launch("gemm_bf16_group_kernel");
 }
 
@@ -784,7 +785,7 @@ static int launch_seg_rows(GemmSegArgs& sa, hipStream_t st) {
     const uint64_t bound = ((uint64_t)(sa.g.M + BM - 1) / BM + (uint64_t)sa.n_seg) * sa.g.tiles_n;
     if (bound > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: too many tiles");
     const uint32_t grid = ((uint32_t)bound + 7) / 8 * 8;
-    launch_timed(&gemm_bf16_seg_rows_kernel<BM, BN, NS, EPI>, dim3(grid), dim3(kGemmThreads), lds, st, sa);
+    hipLaunchKernelGGL((gemm_bf16_seg_rows_kernel<BM, BN, NS, EPI>), dim3(grid), dim3(kGemmThreads), lds, st, sa);
     return check_launch("gemm_bf16_seg_rows_kernel");
 }
 
@@ -799,7 +800,7 @@ static int launch_seg_k(GemmSegArgs& sa, hipStream_t st) {
     const uint64_t total = (uint64_t)sa.g.n_blocks * (uint64_t)sa.n_seg;
     if (total > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_segmented: too many tiles");
     const uint32_t grid = ((uint32_t)total + 7) / 8 * 8;
-    launch_timed(&gemm_bf16_seg_k_kernel<BM, BN, NS, EPI, CF32>, dim3(grid), dim3(kGemmThreads), lds, st, sa);
+    hipLaunchKernelGGL((gemm_bf16_seg_k_kernel<BM, BN, NS, EPI, CF32>), dim3(grid), dim3(kGemmThreads), lds, st, sa);
     return check_launch("gemm_bf16_seg_k_kernel");
 }
 

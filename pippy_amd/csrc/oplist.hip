@@ -270,28 +270,16 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
     for (int i = 0; i < n_ops; ++i) {
         if (ops[i].flags & PP_OP_SKIP) continue;
         int glen = group_length(ops, i, n_ops);
-        // while launches are timed a group is one kernel launch, so that a record is one dispatch
-        if (g_prof_on && glen > PP_GEMM_MAX_GROUP) glen = PP_GEMM_MAX_GROUP;
         const int clen = glen ? 0 : colreduce_group_length(ops, i, n_ops);
         if (clen > 1) glen = clen;
         ProfRecord* rec = nullptr;
-        // a GEMM that is a single kernel is timed by the dispatch's own start and stop events; ops
-        // of several kernels (column reductions, a GEMM split along K) by events on the stream
-        const int kind = ops[i].kind;
-        const bool one_kernel = (kind == PP_OP_GEMM_BF16 && !ops[i].p[8]) || kind == PP_OP_GEMM_SEG;
-        bool dispatch_timed = false;
         if (g_prof_on) {
             if (g_prof_used < g_prof.size()) {
                 rec = &g_prof[g_prof_used++];
                 rec->kind = ops[i].kind;
                 rec->work = op_work(ops[i]);
                 for (int q = 1; q < glen; ++q) rec->work += op_work(ops[i + q]);
-                if (one_kernel) {
-                    dispatch_timed = true;
-                    launch_events() = LaunchEvents{rec->a, rec->b, false};
-                } else {
-                    (void)hipEventRecord(rec->a, static_cast<hipStream_t>(stream));
-                }
+                (void)hipEventRecord(rec->a, static_cast<hipStream_t>(stream));
             } else {
                 ++g_prof_dropped;
             }
@@ -310,16 +298,7 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
         } else {
             rc = run_one(ops[i], stream);
         }
-        if (dispatch_timed) {
-            const bool used = launch_events().used;
-            launch_events() = LaunchEvents{};
-            if (!used) {  // nothing was launched (an empty problem): an empty interval on the stream
-                (void)hipEventRecord(rec->a, static_cast<hipStream_t>(stream));
-                (void)hipEventRecord(rec->b, static_cast<hipStream_t>(stream));
-            }
-        } else if (rec) {
-            (void)hipEventRecord(rec->b, static_cast<hipStream_t>(stream));
-        }
+        if (rec) (void)hipEventRecord(rec->b, static_cast<hipStream_t>(stream));
         if (rc != PP_OK) {
             char msg[400];
             snprintf(msg, sizeof msg, "%s", pp_last_error());

@@ -6,10 +6,6 @@ char* error_buffer() {
     static thread_local char buf[512] = {0};
     return buf;
 }
-LaunchEvents& launch_events() {
-    static thread_local LaunchEvents ev;
-    return ev;
-}
 }  // namespace pp
 
 extern "C" int pp_abi_version(void) { return 1; }
