@@ -12,8 +12,8 @@
 // in registers in exactly the form the second MFMA wants as its B operand for
 // O^T[d][q] += V^T[d][kv] P^T[kv][q].
 //
-// Backward: delta = rowsum(dO * O); one kernel parallel over key blocks (64 keys) produces dK and
-// dV, one kernel parallel over query blocks (64 queries) produces dQ, with the same 2 x 2 split of
+// Backward: one kernel parallel over query blocks (64 queries) produces dQ and delta = rowsum(dO * O),
+// one kernel parallel over key blocks (64 keys) then produces dK and dV, with the same 2 x 2 split of
 // the waves: partial sums of the two halves are added in a fixed order through LDS.  No atomics:
 // results are run-to-run identical.
 //
@@ -289,35 +289,6 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
     }
 }
 
-// ---- backward: delta[b, h, q] = sum_d dO * O ---------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
-    constexpr int LPH = D / 8;  // lanes per head
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // over B*S
-    if (row >= a.B * a.S) return;
-    const int64_t bidx = row / a.S, q = row - bidx * a.S;
-    const int64_t width = a.H * D;
-    const int nchunk = (int)(width >> 3);
-    for (int c0 = 0; c0 < nchunk; c0 += 64) {
-        const int cidx = c0 + lane;
-        float s = 0.f;
-        if (cidx < nchunk) {
-            const uint4 x = *reinterpret_cast<const uint4*>(a.d_o + row * width + (int64_t)cidx * 8);
-            const uint4 y = *reinterpret_cast<const uint4*>(a.o + row * width + (int64_t)cidx * 8);
-            s = bf16lo(x.x) * bf16lo(y.x) + bf16hi(x.x) * bf16hi(y.x) + bf16lo(x.y) * bf16lo(y.y) +
-                bf16hi(x.y) * bf16hi(y.y) + bf16lo(x.z) * bf16lo(y.z) + bf16hi(x.z) * bf16hi(y.z) +
-                bf16lo(x.w) * bf16lo(y.w) + bf16hi(x.w) * bf16hi(y.w);
-        }
-#pragma unroll
-        for (int o = LPH / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-        if (cidx < nchunk && (lane % LPH) == 0) {
-            const int64_t h = cidx / LPH;
-            a.delta[(bidx * a.H + h) * a.S + q] = s;
-        }
-    }
-}
-
 // ---- backward: dK, dV (parallel over key blocks) ------------------------------------------------
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(const AttnArgs a) {
@@ -523,7 +494,24 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
         dof[ks] = *reinterpret_cast<const bf16x8_t*>(dop + qi * ldo + 16 * ks + 8 * lh);
     }
     const float lse_q = a.lse[(b * a.H + h) * a.S + qi] * kLog2e;
-    const float delta_q = a.delta[(b * a.H + h) * a.S + qi];
+    // delta = rowsum(dO * O) of this lane's query row: the lane pair (lh = 0, 1) holds the row of dO, so
+    // the same pieces of O make the dot product; it is stored for the dK / dV kernel, which runs next
+    float delta_q = 0.f;
+    {
+        const uint16_t* op = a.o + b * a.S * ldo + h * D;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            Frag x, y;
+            x.v = dof[ks];
+            y.u = *reinterpret_cast<const uint4*>(op + qi * ldo + 16 * ks + 8 * lh);
+            delta_q += bf16lo(x.u.x) * bf16lo(y.u.x) + bf16hi(x.u.x) * bf16hi(y.u.x) +
+                       bf16lo(x.u.y) * bf16lo(y.u.y) + bf16hi(x.u.y) * bf16hi(y.u.y) +
+                       bf16lo(x.u.z) * bf16lo(y.u.z) + bf16hi(x.u.z) * bf16hi(y.u.z) +
+                       bf16lo(x.u.w) * bf16lo(y.u.w) + bf16hi(x.u.w) * bf16hi(y.u.w);
+        }
+        delta_q += __shfl_xor(delta_q, 32, 64);
+        if (half == 0 && lh == 0) a.delta[(b * a.H + h) * a.S + qi] = delta_q;
+    }
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t)
         if (t < n_blocks) issue(t, t);
@@ -671,18 +659,17 @@ static int attn_fwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipSt
 
 template <int D>
 static int attn_bwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
-    hipLaunchKernelGGL(attn_delta_kernel<D>, dim3((uint32_t)((d->B * d->S + 3) / 4)), dim3(256), 0, st, a);
-    int rc = check_launch("attn_delta_kernel");
-    if (rc) return rc;
+    // the dQ kernel goes first: it also computes delta = rowsum(dO * O), which the dK / dV kernel reads
     const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false);
+    int rc;
     if (d->causal) {
-        rc = attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+        rc = attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
         if (rc) return rc;
-        return attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+        return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
     }
-    rc = attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+    rc = attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
     if (rc) return rc;
-    return attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+    return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
 }
 
 }  // namespace pp
