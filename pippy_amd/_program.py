@@ -672,6 +672,9 @@ class StageProgram:
         self._shared: Dict[str, torch.Tensor] = {}
         self.mbs: Dict[int, MicrobatchProgram] = {}
         self.acc_initialized = False  # False: the next W pass overwrites the accumulators
+        # True once ``materialize_grads`` has set ``param.grad`` from the accumulators: a ``.grad`` that
+        # is None afterwards was cleared by the user's optimizer
+        self.grads_handed_over = False
 
     def shared(self, key, shape, dtype, exact=True) -> torch.Tensor:
         # Launch lists hold raw pointers into these buffers, so a buffer is never replaced or

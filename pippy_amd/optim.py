@@ -54,6 +54,12 @@ class _FusedOptimizer:
         for a in self._arenas:
             a.mark_updated()
 
+    def _has_grads(self, k: int) -> bool:
+        """False for a stage whose gradients were cleared and not produced again: its accumulators
+        hold the sums of an earlier step, and torch.optim skips parameters without a gradient."""
+        prog = self._stages[k]._program
+        return prog is not None and prog.acc_initialized
+
     @property
     def master_weights(self) -> List[Optional[torch.Tensor]]:
         return self._master
@@ -112,7 +118,9 @@ class FusedSGD(_FusedOptimizer):
 
     @torch.no_grad()
     def step(self):
-        for a, buf, master in zip(self._arenas, self._buf, self._master):
+        for k, (a, buf, master) in enumerate(zip(self._arenas, self._buf, self._master)):
+            if not self._has_grads(k):
+                continue
             N.sgd_step(a.params, a.acc, buf, master=master, lr=self.lr, momentum=self.momentum,
                        dampening=self.dampening, weight_decay=self.weight_decay, nesterov=self.nesterov,
                        first_step=self._steps == 0, maximize=self.maximize)
@@ -148,7 +156,9 @@ class FusedAdamW(_FusedOptimizer):
         b1, b2 = self.betas
         bc1 = 1.0 - b1 ** self._steps
         bc2_sqrt = math.sqrt(1.0 - b2 ** self._steps)
-        for a, m, v, master in zip(self._arenas, self._m, self._v, self._master):
+        for k, (a, m, v, master) in enumerate(zip(self._arenas, self._m, self._v, self._master)):
+            if not self._has_grads(k):
+                continue
             N.adamw_step(a.params, a.acc, m, v, master=master, lr=self.lr, beta1=b1, beta2=b2, eps=self.eps,
                          weight_decay=self.weight_decay, bias_correction1=bc1, bias_correction2_sqrt=bc2_sqrt,
                          maximize=self.maximize)

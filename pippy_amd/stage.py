@@ -20,6 +20,7 @@ Two execution modes per stage:
 from __future__ import annotations
 
 import logging
+import os
 from typing import Any, Dict, List, Optional, Tuple, Union
 
 import torch
@@ -33,6 +34,10 @@ from ._utils import flatten_args
 from .losses import as_native_loss
 
 logger = logging.getLogger(__name__)
+
+# PIPPY_AMD_CHECK_INPUTS=1: token ids and loss targets are range-checked on the host before the kernels
+# that index with them run (one device-to-host synchronisation per check; off by default)
+_CHECK_INPUTS = os.environ.get("PIPPY_AMD_CHECK_INPUTS") == "1"
 
 
 class VirtualGroup:
@@ -102,6 +107,7 @@ class PipelineStageBase:
         self._bwd_done: Dict[int, bool] = {}
         self._input_grads: Dict[int, List[Optional[torch.Tensor]]] = {}  # eager hand-off
         self._bridge: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}  # generic loss on a native stage
+        self._step_losses: Optional[torch.Tensor] = None
 
         self.fused_accumulate = fused_accumulate
         self.split_backward = False
@@ -161,6 +167,7 @@ class PipelineStageBase:
         self._bwd_done.clear()
         self._input_grads.clear()
         self._bridge.clear()
+        self._step_losses = None  # per-step buffer of the native losses, allocated by the first of them
 
     # -- program management ---------------------------------------------------------------------
     def _stage_program(self) -> P.StageProgram:
@@ -207,6 +214,7 @@ class PipelineStageBase:
         fp32 accumulators instead of adding to them."""
         if self._program is not None:
             self._program.acc_initialized = False
+            self._program.grads_handed_over = False
         for p in self.submod.parameters():
             p.grad = None
 
@@ -217,6 +225,9 @@ class PipelineStageBase:
             return
         for _, p in self._program.arena.named:
             p.grad = p.main_grad if p.dtype == torch.float32 else p.main_grad.to(p.dtype)
+        # from here on a cleared ``.grad`` (``optimizer.zero_grad()``) means "start a new accumulation",
+        # exactly as for fp32 parameters, whose ``.grad`` is the accumulator itself
+        self._program.grads_handed_over = True
 
     def _input_for(self, mb: int, args, kwargs):
         """(x, dx_target, patch_input) of microbatch ``mb`` for a native stage."""
@@ -278,6 +289,7 @@ class PipelineStageBase:
         x, dx_target, patch = self._input_for(mb, args, kwargs)
         prog = sp.mbs.get(mb)
         if patch:
+            xc = None
             if not x.is_contiguous() or (x.data_ptr() % 16):
                 xc = torch.empty(x.shape, dtype=x.dtype, device=x.device)
                 N.strided_copy_nd(xc, x)
@@ -290,12 +302,26 @@ class PipelineStageBase:
                                       for (k, q) in lst.find_pointer(slot.data_ptr())]
             for lst, k, q in prog.input_patches:
                 lst[k].p[q] = x.data_ptr()
+            # a deferred weight-gradient pass on another stream still reads the copy after the
+            # input-gradient pass has dropped the forward cache: the slot keeps it until its next forward
+            prog.input_copy = xc
+            if _CHECK_INPUTS and x.dtype == torch.int64:
+                self._check_ids(x)
         else:
             key = (tuple(x.shape), x.dtype, x.data_ptr(), P._p(dx_target))
             if prog is None or prog.in_key != key:
                 prog = sp.build(mb, x, dx_target)
         prog.F.run()
         return prog.output, [x]
+
+    def _check_ids(self, ids):
+        for blk in self._blocks:
+            table = getattr(blk, "wte", None) or getattr(blk, "word_embeddings", None)
+            if table is not None:
+                vocab = table.weight.shape[0]
+                if bool(((ids < 0) | (ids >= vocab)).any()):
+                    raise RuntimeError(f"{self.log_prefix} token id outside [0, {vocab})")
+                return
 
     def _received(self, value):
         if isinstance(value, torch.Tensor):
@@ -359,18 +385,29 @@ class PipelineStageBase:
                 tc = torch.empty(target.shape, dtype=target.dtype, device=target.device)
                 N.strided_copy_nd(tc, target)
                 target = tc
-            entry = prog.loss_ops.get(id(loss_fn))
+            # the launch list is cached per microbatch slot by what shapes it (never by the identity of
+            # the loss object, which a later object may reuse); the loss itself goes to a buffer that is
+            # allocated afresh every step, so the tensors a caller keeps are not overwritten by later steps
+            key = (native.ignore_index, V, self.has_backward)
+            entry = prog.loss_ops.get(key)
             if entry is None:
-                loss = torch.empty(1, dtype=torch.float32, device=self.device)
                 ws = torch.empty(rows + 2, dtype=torch.float32, device=self.device)
                 dl = prog.output_grad_buf.view(logits.shape) if self.has_backward else None
                 lst = P.OpList()
-                lst.append(P.op_ce_loss(logits, target, loss, dl, ws, V, native.ignore_index))
+                lst.append(P.op_ce_loss(logits, target, ws[:1], dl, ws, V, native.ignore_index))
                 lst.freeze()
-                entry = (lst, loss, ws)
-                prog.loss_ops[id(loss_fn)] = entry
-            lst, loss, _ = entry
+                entry = (lst, ws)
+                prog.loss_ops[key] = entry
+            lst, _ = entry
+            if self._step_losses is None:
+                self._step_losses = torch.empty(self.chunks, dtype=torch.float32, device=self.device)
+            if _CHECK_INPUTS:
+                bad = ((target < 0) | (target >= V)) & (target != native.ignore_index)
+                if bool(bad.any()):
+                    raise RuntimeError(f"cross entropy target outside [0, {V}) in microbatch {mb}")
+            loss = self._step_losses[mb:mb + 1]
             lst[0].p[1] = target.data_ptr()
+            lst[0].p[2] = loss.data_ptr()
             lst.run()
             self._loss_targets = getattr(self, "_loss_targets", {})
             self._loss_targets[mb] = target  # keep alive until the kernel has run
@@ -444,9 +481,11 @@ class PipelineStageBase:
         sp = self._program
         prog = sp.mbs[mb]
         fp32_params = sp.arena.dtype == torch.float32
-        if fp32_params and sp.acc_initialized and any(p.grad is None for _, p in sp.arena.named):
+        if (fp32_params or sp.grads_handed_over) and sp.acc_initialized and \
+                any(p.grad is None for _, p in sp.arena.named):
             # the user cleared the gradients (optimizer.zero_grad()): start a new accumulation
             sp.acc_initialized = False
+            sp.grads_handed_over = False
         sp.set_accumulate_mode(prog, init=not sp.acc_initialized)
         prog.W.run()
         sp.acc_initialized = True

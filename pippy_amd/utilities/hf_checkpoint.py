@@ -112,8 +112,9 @@ def load_checkpoint(model, index_filename: Union[str, os.PathLike], optim=None, 
                     checkpoint_prefix: Optional[str] = None):
     """Loads the tensors that ``model`` (a stage, a stage module or a whole model) owns from the
     checkpoint behind ``index_filename``; only the binaries that hold them are opened.  Values are
-    cast to the dtype of the tensor they replace (or ``dtype``) and copied in place.  Raises
-    ``RuntimeError`` when a tensor of ``model`` is not in the index."""
+    cast to the dtype of the tensor they replace and copied in place (stage tensors are views of the
+    stage's flat arenas and keep their dtype: a floating-point ``dtype`` that differs from it raises
+    ``RuntimeError``).  Also raises ``RuntimeError`` when a tensor of ``model`` is not in the index."""
     module = _module_of(model)
     folder = os.path.split(index_filename)[0]
     with open(index_filename, "r") as f:

@@ -350,6 +350,70 @@ def test_fused_optimizer_trains_like_the_oracle():
         note(f"optimizer step {step}: worst update error {worst:.3e}")
 
 
+def test_stock_optimizer_zero_grad_restarts_the_accumulation_on_bf16_stages():
+    """The loop of the reference's test_optim.py:85-99 with a torch optimizer on bf16 stages:
+    ``materialize_grads`` hands the fp32 sums over as ``param.grad``, ``optimizer.zero_grad()`` clears
+    them, and the next step must start a new accumulation.  With a zero learning rate both steps see
+    the same weights, so the sums after the second step equal those after the first bit for bit
+    (a stage that kept adding would hold twice the values)."""
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    torch.manual_seed(11)
+    target = torch.randint(0, model.head.vocab, ids.shape)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    params = [p for st in stages for p in st.submod.parameters()]
+    opt = torch.optim.SGD(params, lr=0.0)
+    named = dict(model.named_parameters())
+    embed = {n for n in named if "wte" in n or "wpe" in n}
+    first = None
+    for step in range(2):
+        sched.step(ids.to(DEV), target=target.to(DEV), losses=[])
+        for st in stages:
+            st.materialize_grads()
+        torch.cuda.synchronize()
+        for n, p in named.items():
+            assert p.grad is not None and p.grad.dtype == p.dtype
+            assert torch.equal(p.grad, p.main_grad.to(p.dtype)), n
+        sums = {n: p.main_grad.clone() for n, p in named.items()}
+        if first is None:
+            first = sums
+        opt.step()
+        opt.zero_grad()
+        assert all(p.grad is None for p in params)
+    for n in named:
+        assert torch.equal(sums[n], first[n]), f"{n}: the second step did not restart the accumulation"
+    # against the oracle: one step's gradients
+    for p in ref.parameters():
+        p.grad = None
+    OP.step(ref_stages, ids, target, M, _ce)
+    for n, rp in ref.named_parameters():
+        assert_close_rel(sums[n], rp.grad, BF16_TOL, f"grad of {n}")
+    del embed
+
+
+def test_fused_optimizer_skips_a_stage_whose_gradients_were_cleared():
+    """``zero_grad`` followed by ``step`` without a backward pass in between leaves the parameters
+    alone (torch.optim skips parameters without a gradient); the accumulators of the step before are
+    not applied a second time."""
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    torch.manual_seed(3)
+    target = torch.randint(0, model.head.vocab, ids.shape)
+    sched = pp.ScheduleGPipe(stages, M, loss_fn=pp.CrossEntropyLoss())
+    opt = pp.FusedSGD(stages, lr=0.5)
+    sched.step(ids.to(DEV), target=target.to(DEV), losses=[])
+    opt.step()
+    torch.cuda.synchronize()
+    after_one = {n: p.detach().clone() for n, p in model.named_parameters()}
+    opt.zero_grad()
+    opt.step()
+    torch.cuda.synchronize()
+    for n, p in model.named_parameters():
+        assert torch.equal(p.detach(), after_one[n]), n
+
+
 # ---- BERT-shaped encoder (post-LayerNorm, bidirectional attention, erf-GELU) ----------------------
 def _build_encoder(n_stages, n_layers=4, M=4, vocab=1000, seq=128, dim=128, heads=2, ffn=512, seed=0):
     import pippy_amd as pp
