@@ -99,65 +99,86 @@ def _split_tensor(v: torch.Tensor, n: int, dim: int) -> Sequence[torch.Tensor]:
     return tuple(outs)
 
 
-def _shard_dict_of_args(args_dict, args_chunk_spec, num_chunks):
-    """Flatten, split or replicate, regroup per chunk (``microbatch.py:66-194``)."""
-    args_sharded_replicated = {}
-    arg_specs = []
-    real_num_chunks = num_chunks
-    first_tensor = True
+class _Leaf:
+    """One flattened value of an argument and what the spec says to do with it: ``dim`` is the
+    dimension a tensor is cut along, or None for a value that every microbatch receives as it is."""
 
+    __slots__ = ("value", "dim")
+
+    def __init__(self, value, dim):
+        self.value = value
+        self.dim = dim
+
+
+def _plan_leaves(arg, chunk_spec) -> Tuple[List[_Leaf], Any]:
+    """Flattens one argument next to its spec (reference ``microbatch.py:97-113,169``)."""
+    values, tree = tree_flatten(arg)
+    rules, _ = tree_flatten(chunk_spec)
+    if len(values) != len(rules):
+        raise ValueError(
+            f"Argument value {arg} did not have the same number of "
+            f"values as as chunk spec {chunk_spec}")
+    leaves = []
+    for value, rule in zip(values, rules):
+        if rule is _Replicate or not isinstance(value, torch.Tensor):
+            leaves.append(_Leaf(value, None))
+        elif isinstance(rule, TensorChunkSpec):
+            leaves.append(_Leaf(value, rule.split_dim))
+        else:
+            raise TypeError(f"Unrecognized chunk spec: {rule}")
+    return leaves, tree
+
+
+def _settle_chunk_count(plans, num_chunks: int) -> int:
+    """How many chunks the arguments really give (reference ``microbatch.py:118-137``): the first
+    tensor that is cut may be shorter than ``num_chunks`` along its dimension, which lowers the count
+    with a warning; a later tensor that is shorter than the count is an error."""
+    count = num_chunks
+    seen_tensor = False
+    for key, leaves, _tree in plans:
+        for leaf in leaves:
+            if leaf.dim is None:
+                continue
+            extent = leaf.value.size(leaf.dim)
+            if extent < count:
+                if seen_tensor:
+                    raise RuntimeError(
+                        f"Arg {key} on chunking dimension has a size of {extent}, "
+                        f"smaller than the number of chunks {num_chunks}. "
+                        "PiPPy cannot reduce the number of chunks because "
+                        "other arguments have bigger chunk-dimension sizes. "
+                        "Please adjust your num_chunks setting.")
+                logger.warning(
+                    f"Tensor size on chunking dimension is {extent}, "
+                    f"downsizing the number of chunks from {num_chunks} to {extent}.")
+                count = extent
+            seen_tensor = True
+    return count
+
+
+def _shard_dict_of_args(args_dict, args_chunk_spec, num_chunks):
+    """Cuts a dict of arguments into a list of per-microbatch dicts (reference
+    ``microbatch.py:66-194``).  Three passes: pair every flattened value with its rule, settle the
+    chunk count, then cut each tensor once and deal the pieces out."""
     assert len(args_dict) == len(args_chunk_spec), (
         f"args_dict.keys() = {list(args_dict.keys())} "
         f"args_chunk_spec.keys() = {list(args_chunk_spec.keys())}")
+    plans = []
+    for key, arg in args_dict.items():
+        rule = args_chunk_spec[key]
+        assert rule is not None
+        leaves, tree = _plan_leaves(arg, rule)
+        plans.append((key, leaves, tree))
+    count = _settle_chunk_count(plans, num_chunks)
+    cut = _masked_chunks if _debug_mask_minibatches else _split_tensor
 
-    for arg_key, arg in args_dict.items():
-        flat, spec = tree_flatten(arg)
-        arg_specs.append(spec)
-        chunk_spec = args_chunk_spec[arg_key]
-        assert chunk_spec is not None
-        chunk_spec_flat, _ = tree_flatten(chunk_spec)
-        if len(flat) != len(chunk_spec_flat):
-            raise ValueError(
-                f"Argument value {arg} did not have the same number of "
-                f"values as as chunk spec {chunk_spec}")
-
-        sharded_arg_flat = []
-        for v, chunk_v in zip(flat, chunk_spec_flat):
-            if chunk_v is _Replicate or not isinstance(v, torch.Tensor):
-                sharded_arg_flat.append([v] * real_num_chunks)
-            elif isinstance(chunk_v, TensorChunkSpec):
-                v_split_dim_size = v.size(chunk_v.split_dim)
-                if v_split_dim_size < real_num_chunks:
-                    if first_tensor:
-                        logger.warning(
-                            f"Tensor size on chunking dimension is {v_split_dim_size}, "
-                            f"downsizing the number of chunks from {num_chunks} to {v_split_dim_size}.")
-                        real_num_chunks = v_split_dim_size
-                    else:
-                        raise RuntimeError(
-                            f"Arg {arg_key} on chunking dimension has a size of {v_split_dim_size}, "
-                            f"smaller than the number of chunks {num_chunks}. "
-                            "PiPPy cannot reduce the number of chunks because "
-                            "other arguments have bigger chunk-dimension sizes. "
-                            "Please adjust your num_chunks setting.")
-
-                if _debug_mask_minibatches:
-                    chunk_tensors = _masked_chunks(v, real_num_chunks, chunk_v.split_dim)
-                else:
-                    chunk_tensors = _split_tensor(v, real_num_chunks, chunk_v.split_dim)
-                sharded_arg_flat.append(chunk_tensors)
-                first_tensor = False
-            else:
-                raise TypeError(f"Unrecognized chunk spec: {chunk_v}")
-        args_sharded_replicated[arg_key] = sharded_arg_flat
-
-    args_split = []
-    for chunk_idx in range(real_num_chunks):
-        per_chunk_args = {}
-        for (key, arg), arg_spec in zip(args_sharded_replicated.items(), arg_specs):
-            per_chunk_args[key] = tree_unflatten([v_flat[chunk_idx] for v_flat in arg], arg_spec)
-        args_split.append(per_chunk_args)
-    return args_split
+    microbatches: List[Dict[Any, Any]] = [{} for _ in range(count)]
+    for key, leaves, tree in plans:
+        pieces = [cut(leaf.value, count, leaf.dim) if leaf.dim is not None else None for leaf in leaves]
+        for m, mb_args in enumerate(microbatches):
+            flat = [leaf.value if piece is None else piece[m] for leaf, piece in zip(leaves, pieces)]
+            mb_args[key] = tree_unflatten(flat, tree)
+    return microbatches
 
 
 def _masked_chunks(v: torch.Tensor, n: int, dim: int) -> List[torch.Tensor]:
@@ -205,31 +226,25 @@ def split_args_kwargs_into_chunks(
     args_chunk_spec: Optional[Tuple[TensorChunkSpec, ...]] = None,
     kwargs_chunk_spec: Optional[Dict[str, TensorChunkSpec]] = None,
 ) -> Tuple[List[Tuple], List[Dict]]:
-    """Split ``args`` / ``kwargs`` into ``chunks`` microbatches (``microbatch.py:197-300``)."""
-    if kwargs is None:
-        kwargs = {}
-    if args_chunk_spec is None:
-        args_chunk_spec = (TensorChunkSpec(DEFAULT_CHUNK_DIM),) * len(args)
-    if kwargs_chunk_spec is None:
-        kwargs_chunk_spec = dict.fromkeys(kwargs, TensorChunkSpec(DEFAULT_CHUNK_DIM))
+    """Split ``args`` / ``kwargs`` into ``chunks`` microbatches (reference ``microbatch.py:197-300``).
+    Without a spec every tensor is cut along dimension 0.  Positional and keyword arguments must end
+    up with the same number of chunks; when the keyword arguments settle on fewer, the positional
+    ones are cut again to that number."""
+    kwargs = {} if kwargs is None else kwargs
+    by_position = dict(enumerate(args))
+    default = TensorChunkSpec(DEFAULT_CHUNK_DIM)
+    position_rules = dict(enumerate(args_chunk_spec if args_chunk_spec is not None else (default,) * len(args)))
+    keyword_rules = kwargs_chunk_spec if kwargs_chunk_spec is not None else dict.fromkeys(kwargs, default)
 
-    args_split_dict = _shard_dict_of_args(dict(enumerate(args)), dict(enumerate(args_chunk_spec)), chunks)
-    real_num_chunks = len(args_split_dict)
-    kwargs_split = _shard_dict_of_args(kwargs, kwargs_chunk_spec, real_num_chunks)
-
-    if len(kwargs_split) < real_num_chunks:
-        # kwargs forced a smaller chunk count (e.g. args held no tensor): re-shard args to match
-        real_num_chunks = len(kwargs_split)
-        args_split_dict = _shard_dict_of_args(
-            dict(enumerate(args)), dict(enumerate(args_chunk_spec)), real_num_chunks)
-
-    if len(args_split_dict) != len(kwargs_split):
+    positional = _shard_dict_of_args(by_position, position_rules, chunks)
+    keyword = _shard_dict_of_args(kwargs, keyword_rules, len(positional))
+    if len(keyword) < len(positional):
+        positional = _shard_dict_of_args(by_position, position_rules, len(keyword))
+    if len(positional) != len(keyword):
         raise RuntimeError(
             "args and kwargs are split into different number of chunks: "
-            f"{len(args_split_dict)}, {len(kwargs_split)}")
-
-    args_split = [tuple(chunk_args[i] for i in range(len(chunk_args))) for chunk_args in args_split_dict]
-    return args_split, kwargs_split
+            f"{len(positional)}, {len(keyword)}")
+    return [tuple(mb[i] for i in range(len(args))) for mb in positional], keyword
 
 
 # ---- merge -------------------------------------------------------------------------------------
@@ -354,51 +369,49 @@ def cat_chunks(values: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
     return out
 
 
+def _own_slices(values: Sequence[torch.Tensor], dim: int) -> List[torch.Tensor]:
+    """Debug-mask mode: every microbatch value has the full batch shape and only the slice that the
+    split gave its microbatch is meaningful (reference ``microbatch.py:380-410``)."""
+    shape = values[0].shape
+    for v in values[1:]:
+        assert v.shape == shape
+    out, lo = [], 0
+    for v, size in zip(values, chunk_sizes(shape[dim], len(values))):
+        out.append(v.narrow(dim, lo, size))
+        lo += size
+    return out
+
+
+def _merge_leaf(rule, column: Sequence[Any]):
+    """One output leaf from its per-microbatch values (reference ``microbatch.py:374-429``)."""
+    if isinstance(rule, TensorChunkSpec):
+        values = _own_slices(column, rule.split_dim) if _debug_mask_minibatches else column
+        return cat_chunks(values, rule.split_dim)
+    if isinstance(rule, _CustomReducer):
+        total = rule.init_value
+        for value in column:
+            total = rule.reduce_fn(total, value)
+        return total
+    # anything else was replicated: every microbatch must hold the same value
+    for value in column[1:]:
+        assert value == column[0]
+    return column[0]
+
+
 def merge_chunks(chunks: List[Any], chunk_spec):
-    """Inverse of the split: merge per-microbatch values into one (``microbatch.py:303-432``)."""
-    if chunk_spec is not None:
-        spec_flattened, flatten_spec = tree_flatten(chunk_spec)
+    """Inverse of the split: per-microbatch values back into one (reference
+    ``microbatch.py:303-432``).  ``chunk_spec`` mirrors the structure of one chunk; None concatenates
+    every leaf along dimension 0."""
+    if chunk_spec is None:
+        leaves0, tree = tree_flatten(chunks[0])
+        rules = [TensorChunkSpec(DEFAULT_CHUNK_DIM)] * len(leaves0)
     else:
-        # default: every output leaf is concatenated along dim 0 (``microbatch.py:348-354``)
-        chunk0_flat, flatten_spec = tree_flatten(chunks[0])
-        spec_flattened = [TensorChunkSpec(DEFAULT_CHUNK_DIM)] * len(chunk0_flat)
-
-    chunks_flattened = []
+        rules, tree = tree_flatten(chunk_spec)
+    columns: List[List[Any]] = [[] for _ in rules]
     for chunk in chunks:
-        chunk_flattened, _ = tree_flatten(chunk)
-        if len(chunk_flattened) != len(spec_flattened):
+        leaves, _ = tree_flatten(chunk)
+        if len(leaves) != len(rules):
             raise ValueError(f"Chunk {chunk} did not match chunk spec {chunk_spec}")
-        chunks_flattened.append(chunk_flattened)
-
-    args_flattened = []
-    for arg_idx, arg in enumerate(spec_flattened):
-        if isinstance(arg, TensorChunkSpec):
-            partial_values = [c[arg_idx] for c in chunks_flattened]
-            if _debug_mask_minibatches:
-                # every chunk is full size; keep only its own slice (``microbatch.py:380-410``)
-                overall_shape = partial_values[0].shape
-                for val in partial_values[1:]:
-                    assert val.shape == overall_shape
-                sizes = chunk_sizes(overall_shape[arg.split_dim], len(partial_values))
-                values_to_cat = []
-                lo = 0
-                for val, size in zip(partial_values, sizes):
-                    idx = [slice(None)] * val.dim()
-                    idx[arg.split_dim] = slice(lo, lo + size)
-                    values_to_cat.append(val[tuple(idx)])
-                    lo += size
-            else:
-                values_to_cat = partial_values
-            args_flattened.append(cat_chunks(values_to_cat, arg.split_dim))
-        elif isinstance(arg, _CustomReducer):
-            reduced_val = arg.init_value
-            for chunk in chunks_flattened:
-                reduced_val = arg.reduce_fn(reduced_val, chunk[arg_idx])
-            args_flattened.append(reduced_val)
-        else:
-            value = chunks_flattened[0][arg_idx]
-            for chunk in chunks_flattened[1:]:
-                assert chunk[arg_idx] == value
-            args_flattened.append(value)
-
-    return tree_unflatten(args_flattened, flatten_spec)
+        for column, leaf in zip(columns, leaves):
+            column.append(leaf)
+    return tree_unflatten([_merge_leaf(rule, column) for rule, column in zip(rules, columns)], tree)
