@@ -50,72 +50,66 @@ class PipelineSchedule(ABC):
 
     # -- losses (reference ``PipelineSchedule.py:39-80``) -------------------------------------------
     def _maybe_compute_loss(self, stage, output, target_mbs, mb_index):
-        if stage.is_last and self._has_backward:
-            if target_mbs is None:
-                raise RuntimeError("a loss function was given but no target")
-            loss = self._compute_loss(stage, output, target_mbs[mb_index], mb_index)
-            self._internal_losses.append(loss)
+        if not (stage.is_last and self._has_backward):
+            return
+        if target_mbs is None:
+            raise RuntimeError("a loss function was given but no target")
+        self._internal_losses.append(self._compute_loss(stage, output, target_mbs[mb_index], mb_index))
 
     def _maybe_get_loss(self, stage, mb_index):
-        valid_index = 0 <= mb_index < len(self._internal_losses)
-        if stage.is_last and self._has_backward and valid_index:
-            return self._internal_losses[mb_index]
-        elif len(self._internal_losses) != 0 and not valid_index:
+        """The loss that the backward pass of microbatch ``mb_index`` starts from: only the last
+        stage of a training schedule has one."""
+        held = len(self._internal_losses)
+        if 0 <= mb_index < held:
+            return self._internal_losses[mb_index] if (stage.is_last and self._has_backward) else None
+        if held:
             raise RuntimeError(
                 f"Loss for microbatch {mb_index} is not available. "
                 f"Available losses for microbatches: {self._internal_losses}")
-        else:
-            return None
+        return None
 
     def _update_losses(self, stages, losses):
-        if not isinstance(stages, list):
-            stages = [stages]
-        contains_last_stage = any(stage.is_last for stage in stages)
-        if contains_last_stage and losses is not None:
+        """Hands the step's losses to the caller's list and forgets them."""
+        stages = stages if isinstance(stages, list) else [stages]
+        if losses is not None and any(st.is_last for st in stages):
             if len(self._internal_losses) != self._n_microbatches:
                 raise RuntimeError(
                     f"Expecting {self._n_microbatches} losses but got {len(self._internal_losses)}")
-            losses.clear()
-            losses.extend(self._internal_losses)
+            losses[:] = self._internal_losses
         self._internal_losses.clear()
 
     def _compute_loss(self, stage, output, target, mb_index):
         return stage.compute_loss(self._loss_fn, output, target, mb_index)
 
     # -- input checks (reference ``PipelineSchedule.py:114-152``) -----------------------------------
-    def _check_inputs(self, arg_mbs=None, kwarg_mbs=None, target_mbs=None, losses=None):
-        def check_type_and_len(mbs, name: str):
-            if not isinstance(mbs, list):
-                raise TypeError(f"{name} must be a list but got a {type(mbs)}")
-            if len(mbs) != self._n_microbatches:
-                raise ValueError(f"Expecting {self._n_microbatches} {name} but got {len(mbs)}")
+    def _require_microbatch_list(self, mbs, name: str):
+        if not isinstance(mbs, list):
+            raise TypeError(f"{name} must be a list but got a {type(mbs)}")
+        if len(mbs) != self._n_microbatches:
+            raise ValueError(f"Expecting {self._n_microbatches} {name} but got {len(mbs)}")
 
-        if arg_mbs is not None:
-            check_type_and_len(arg_mbs, "arg_mbs")
-        else:
-            arg_mbs = [()] * self._n_microbatches
-        if kwarg_mbs is not None:
-            check_type_and_len(kwarg_mbs, "kwarg_mbs")
-        else:
-            kwarg_mbs = [{}] * self._n_microbatches
-        if target_mbs is not None:
-            check_type_and_len(target_mbs, "target_mbs")
+    def _check_inputs(self, arg_mbs=None, kwarg_mbs=None, target_mbs=None, losses=None):
+        """Validates the per-microbatch lists; absent positional / keyword lists become empty ones."""
+        given = {"arg_mbs": arg_mbs, "kwarg_mbs": kwarg_mbs, "target_mbs": target_mbs}
+        for name, mbs in given.items():
+            if mbs is not None:
+                self._require_microbatch_list(mbs, name)
         if losses is not None and not isinstance(losses, list):
             raise TypeError(f"losses must be a list but got a {type(losses)}")
-        return arg_mbs, kwarg_mbs
+        n = self._n_microbatches
+        return (arg_mbs if arg_mbs is not None else [()] * n,
+                kwarg_mbs if kwarg_mbs is not None else [{}] * n)
 
     def _split_inputs(self, args: Tuple[Any, ...], kwargs: Optional[Dict[str, Any]] = None):
-        """Full batch -> microbatches (reference ``PipelineSchedule.py:157-187``)."""
-        if self._pipe_info is not None:
-            args_chunk_spec = self._pipe_info.args_chunk_spec
-            kwargs_chunk_spec = self._pipe_info.kwargs_chunk_spec
-        else:
-            args_chunk_spec = None
-            kwargs_chunk_spec = None
-        if args or kwargs:
-            return split_args_kwargs_into_chunks(args, kwargs, self._n_microbatches, args_chunk_spec,
-                                                 kwargs_chunk_spec)
-        return [()] * self._n_microbatches, [{}] * self._n_microbatches
+        """Full batch -> microbatches (reference ``PipelineSchedule.py:157-187``): the chunk specs are
+        those the pipe was traced with, dimension 0 everywhere without a pipe."""
+        n = self._n_microbatches
+        if not args and not kwargs:
+            return [()] * n, [{}] * n
+        info = self._pipe_info
+        return split_args_kwargs_into_chunks(args, kwargs, n,
+                                             info.args_chunk_spec if info is not None else None,
+                                             info.kwargs_chunk_spec if info is not None else None)
 
     def _merge_outputs(self, output_chunks: List[Any]) -> Any:
         """Microbatch outputs -> full batch (reference ``PipelineSchedule.py:189-197``)."""
