@@ -190,6 +190,18 @@ int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
 int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, int out_dtype,
                    float* workspace, pp_stream stream);
 
+/* pp_colsum_bf16 without a workspace argument.  No counterpart in the reference: it exists for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The partial sums go to an array that the library itself holds
+ * on every GPU it runs on (PP_COLSUM_NOALLOC_MAX_FLOATS floats = 4 MiB per GPU, held until the
+ * process ends); the call allocates and frees nothing.  Problems with ceil(M / 128) * N above that
+ * limit are rejected with PP_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls
+ * that may overlap on one GPU (different streams, different threads) race and must be serialised
+ * by the caller.  Results are bit-identical to pp_colsum_bf16. */
+#define PP_COLSUM_NOALLOC_MAX_FLOATS (1 << 20)
+int pp_colsum_bf16_noalloc(const void* dY, int64_t M, int64_t N, int64_t ld, void* out, int out_dtype,
+                           pp_stream stream);
+
 /* dst[c, r] = src[r, c] for bf16 (any 2-byte type).  Used once per optimizer step to keep a
  * transposed copy of every linear weight, so that the input-gradient GEMM dX = dY W
  * (pippy/_backward.py:67-69) reads both operands k-contiguously. */

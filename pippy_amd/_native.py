@@ -14,6 +14,8 @@ import torch
 from ._build import LIB_PATH
 
 PP_OK = 0
+PP_ERR_INVALID, PP_ERR_UNSUPPORTED, PP_ERR_LAUNCH = 1, 2, 3
+PP_COLSUM_NOALLOC_MAX_FLOATS = 1 << 20
 PP_BF16, PP_F32 = 0, 1
 
 # enum pp_gemm_epilogue
@@ -41,7 +43,7 @@ EXPORTED_SYMBOLS = (
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
-    "pp_moe_gate_bwd",
+    "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc",
 )
 
 
@@ -115,6 +117,7 @@ def lib() -> C.CDLL:
         "pp_gemm_bf16_splitk": [C.POINTER(GemmDesc), vp, i64, vp],
         "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
+        "pp_colsum_bf16_noalloc": [vp, i64, i64, i64, vp, i32, vp],
         "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],
         "pp_layernorm_fwd": [vp, vp, vp, vp, vp, vp, i64, i64, f32, vp],
         "pp_layernorm_bwd_input": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp],

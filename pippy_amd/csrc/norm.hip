@@ -423,6 +423,59 @@ extern "C" int pp_colsum_bf16(const void* dY, int64_t M, int64_t N, int64_t ld, 
     return check_launch("colsum");
 }
 
+// ---- column sum with the partial sums in a library-owned array -----------------------------------
+// For callers that cannot allocate (a loop under graph capture, a harness that forbids it): the
+// per-row-block partial sums of pp_colsum_bf16 live in a file-scope device array instead of a
+// caller-provided workspace.  Every GPU holds its own copy of the array at its own address, so the
+// address is looked up once per device, with that device current, and only that pointer is ever
+// handed to a kernel or a copy: the array's name is a host-side stand-in, not a device address.
+namespace pp {
+constexpr int64_t kColsumScratchFloats = PP_COLSUM_NOALLOC_MAX_FLOATS;
+static __device__ __align__(256) float g_colsum_scratch[kColsumScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static float* g_colsum_scratch_ptr[kMaxDevices];  // per device, null until looked up
+
+// The device address of the current device's copy of the array; null (and a message) on failure.
+static float* colsum_scratch_for_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        fail(PP_ERR_LAUNCH, "pp_colsum_bf16_noalloc: cannot identify the current device (%s)",
+             e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return nullptr;
+    }
+    float* p = __atomic_load_n(&g_colsum_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p) return p;
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_colsum_scratch));
+    if (e != hipSuccess || !sym) {
+        fail(PP_ERR_LAUNCH, "pp_colsum_bf16_noalloc: hipGetSymbolAddress failed on device %d: %s", dev,
+             hipGetErrorString(e));
+        return nullptr;
+    }
+    // two threads racing here look up the same address; the store is idempotent
+    __atomic_store_n(&g_colsum_scratch_ptr[dev], static_cast<float*>(sym), __ATOMIC_RELEASE);
+    return static_cast<float*>(sym);
+}
+}  // namespace pp
+
+extern "C" int pp_colsum_bf16_noalloc(const void* dY, int64_t M, int64_t N, int64_t ld, void* out,
+                                      int out_dtype, pp_stream stream) {
+    if (M < 0 || N <= 0 || ld < N) return fail(PP_ERR_INVALID, "pp_colsum_bf16_noalloc: bad shape");
+    const int64_t n_part = (M + 127) / 128;
+    if (n_part * N > kColsumScratchFloats)
+        return fail(PP_ERR_UNSUPPORTED,
+                    "pp_colsum_bf16_noalloc: ceil(M / 128) * N = %lld partial sums exceed the built-in "
+                    "array of %lld floats; use pp_colsum_bf16 with a workspace", (long long)(n_part * N),
+                    (long long)kColsumScratchFloats);
+    float* scratch = colsum_scratch_for_current_device();
+    if (!scratch) return PP_ERR_LAUNCH;
+    // every partial sum that the final kernel reads is written by the partial kernel of this call, so
+    // nothing left by an earlier call needs clearing
+    return pp_colsum_bf16(dY, M, N, ld, out, out_dtype, scratch, stream);
+}
+
 extern "C" int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_stream stream) {
     if (n < 0 || (n > 0 && !descs)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: bad list");
     hipStream_t st = static_cast<hipStream_t>(stream);
