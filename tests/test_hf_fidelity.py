@@ -1,0 +1,183 @@
+"""Pins the block definitions and the oracle's rotary embedding to an implementation outside this
+repository: Hugging Face ``transformers`` (importable in the build container; no download, random
+weights copied over).  What is pinned is configuration fidelity: layer order, ``gelu_new``, the
+q|k|v layout of the fused projection, rotate-half RoPE and its frequency table, the Mixtral routing
+(softmax over all experts, top-2, renormalised).  CPU only, fp32; never runs with ``-m gpu``.
+"""
+import pytest
+import torch
+
+transformers = pytest.importorskip("transformers")
+
+from oracle import ops as OO  # noqa: E402
+from pippy_amd import stage_modules as SM  # noqa: E402
+
+TOL = 2e-5
+
+
+def _close(a, b, what):
+    err = (a - b).abs().max().item() / max(b.abs().max().item(), 1e-30)
+    assert err <= TOL, f"{what}: max relative error {err:.3e}"
+
+
+@pytest.mark.parametrize("theta,D,seq", [(1e4, 128, 96), (1e6, 64, 40), (5e5, 32, 17)])
+def test_rope_tables_and_rotation_match_llama_rotary_embedding(theta, D, seq):
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding, apply_rotary_pos_emb
+    H = 2
+    cfg = LlamaConfig(hidden_size=H * D, num_attention_heads=H, num_key_value_heads=H, intermediate_size=64,
+                      num_hidden_layers=1, max_position_embeddings=4 * seq, rope_theta=theta, vocab_size=32)
+    if getattr(cfg, "rope_parameters", None) is not None:  # newer configs keep theta here
+        cfg.rope_parameters["rope_theta"] = theta
+    rot = LlamaRotaryEmbedding(cfg)
+    torch.manual_seed(0)
+    q, k = torch.randn(1, H, seq, D), torch.randn(1, H, seq, D)
+    pos = torch.arange(seq)[None]
+    cos_hf, sin_hf = rot(q, pos)                   # [1, seq, D]: the half table repeated twice
+    cos, sin = OO.rope_tables(seq, D, theta)       # [seq, D / 2]
+    _close(cos, cos_hf[0, :, :D // 2], "cos table")
+    _close(sin, sin_hf[0, :, :D // 2], "sin table")
+    assert torch.equal(cos_hf[0, :, :D // 2], cos_hf[0, :, D // 2:])
+    q_hf, k_hf = apply_rotary_pos_emb(q, k, cos_hf, sin_hf)
+    _close(OO.rope(q, cos, sin), q_hf, "rotated q")
+    _close(OO.rope(k, cos, sin), k_hf, "rotated k")
+    # the block's own table builder and torch statement agree with the oracle's
+    c2, s2 = SM.rope_tables(seq, D, theta, "cpu")
+    assert torch.equal(c2, cos) and torch.equal(s2, sin)
+    _close(SM._apply_rope(q, cos, sin), q_hf, "block rotation")
+
+
+def test_transformer_layer_is_a_gpt2_block():
+    """Pre-LayerNorm, causal, gelu_new; GPT-2 keeps its projections as Conv1D ([in, out] weights)."""
+    from transformers import GPT2Config
+    from transformers.models.gpt2.modeling_gpt2 import GPT2Block
+    dim, heads, ffn, S = 64, 4, 256, 24
+    cfg = GPT2Config(n_embd=dim, n_head=heads, n_layer=1, n_inner=ffn, n_positions=64, vocab_size=32,
+                     activation_function="gelu_new", resid_pdrop=0.0, attn_pdrop=0.0, embd_pdrop=0.0,
+                     layer_norm_epsilon=1e-5)
+    cfg._attn_implementation = "eager"
+    hf = GPT2Block(cfg, layer_idx=0).eval()
+    torch.manual_seed(1)
+    for p in hf.parameters():
+        torch.nn.init.normal_(p, std=0.2)
+    mine = SM.TransformerLayer(dim, heads, ffn, causal=True, pre_ln=True, activation="gelu_tanh", eps=1e-5,
+                               dtype=torch.float32)
+    sd = hf.state_dict()
+    with torch.no_grad():
+        for name, p in mine.named_parameters():
+            src = sd[name]
+            p.copy_(src.t() if (name.endswith("weight") and src.dim() == 2) else src)
+    x = torch.randn(2, S, dim)
+    # the causal mask is built by the enclosing model in this library version: hand it to the block
+    mask = torch.full((S, S), torch.finfo(torch.float32).min).triu(1)[None, None]
+    out_hf = hf(x, attention_mask=mask)
+    out_hf = out_hf[0] if isinstance(out_hf, tuple) else out_hf
+    _close(mine(x), out_hf, "GPT-2 block output")
+
+
+def test_transformer_layer_post_ln_is_a_bert_layer():
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertLayer
+    dim, heads, ffn, S = 64, 4, 256, 24
+    cfg = BertConfig(hidden_size=dim, num_attention_heads=heads, intermediate_size=ffn, num_hidden_layers=1,
+                     hidden_act="gelu", hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                     layer_norm_eps=1e-12, vocab_size=32)
+    cfg._attn_implementation = "eager"
+    hf = BertLayer(cfg).eval()
+    torch.manual_seed(2)
+    for p in hf.parameters():
+        torch.nn.init.normal_(p, std=0.2)
+    mine = SM.TransformerLayer(dim, heads, ffn, causal=False, pre_ln=False, activation="gelu_erf", eps=1e-12,
+                               dtype=torch.float32)
+    sd = hf.state_dict()
+    att = "attention.self."
+    with torch.no_grad():
+        mine.attn.c_attn.weight.copy_(torch.cat([sd[att + "query.weight"], sd[att + "key.weight"],
+                                                 sd[att + "value.weight"]], 0))
+        mine.attn.c_attn.bias.copy_(torch.cat([sd[att + "query.bias"], sd[att + "key.bias"], sd[att + "value.bias"]], 0))
+        mine.attn.c_proj.weight.copy_(sd["attention.output.dense.weight"])
+        mine.attn.c_proj.bias.copy_(sd["attention.output.dense.bias"])
+        mine.ln_1.weight.copy_(sd["attention.output.LayerNorm.weight"])
+        mine.ln_1.bias.copy_(sd["attention.output.LayerNorm.bias"])
+        mine.mlp.c_fc.weight.copy_(sd["intermediate.dense.weight"])
+        mine.mlp.c_fc.bias.copy_(sd["intermediate.dense.bias"])
+        mine.mlp.c_proj.weight.copy_(sd["output.dense.weight"])
+        mine.mlp.c_proj.bias.copy_(sd["output.dense.bias"])
+        mine.ln_2.weight.copy_(sd["output.LayerNorm.weight"])
+        mine.ln_2.bias.copy_(sd["output.LayerNorm.bias"])
+    x = torch.randn(2, S, dim)
+    out_hf = hf(x)
+    out_hf = out_hf[0] if isinstance(out_hf, tuple) else out_hf
+    _close(mine(x), out_hf, "BERT layer output")
+
+
+def _llama_position_embeddings(cfg, x, S):
+    from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+    return LlamaRotaryEmbedding(cfg)(x, torch.arange(S)[None])
+
+
+def test_llama_layer_is_a_llama_decoder_layer():
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaDecoderLayer
+    dim, heads, ffn, S, theta = 128, 2, 192, 24, 1e4
+    cfg = LlamaConfig(hidden_size=dim, num_attention_heads=heads, num_key_value_heads=heads,
+                      intermediate_size=ffn, num_hidden_layers=1, rms_norm_eps=1e-5, rope_theta=theta,
+                      max_position_embeddings=64, vocab_size=32, attention_dropout=0.0, hidden_act="silu")
+    if getattr(cfg, "rope_parameters", None) is not None:
+        cfg.rope_parameters["rope_theta"] = theta
+    cfg._attn_implementation = "eager"
+    hf = LlamaDecoderLayer(cfg, layer_idx=0).eval()
+    torch.manual_seed(3)
+    for p in hf.parameters():
+        torch.nn.init.normal_(p, std=0.1)
+    mine = SM.LlamaLayer(dim, heads, ffn, eps=1e-5, rope_theta=theta, dtype=torch.float32)
+    sd = hf.state_dict()
+    with torch.no_grad():
+        mine.self_attn.qkv_proj.weight.copy_(torch.cat([sd["self_attn.q_proj.weight"], sd["self_attn.k_proj.weight"],
+                                                        sd["self_attn.v_proj.weight"]], 0))
+        for name in ("self_attn.o_proj.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight",
+                     "input_layernorm.weight", "post_attention_layernorm.weight"):
+            mine.get_parameter(name).copy_(sd[name])
+    x = torch.randn(2, S, dim)
+    mask = torch.full((S, S), float("-inf")).triu(1)[None, None]
+    out_hf = hf(x, attention_mask=mask, position_ids=torch.arange(S)[None],
+                position_embeddings=_llama_position_embeddings(cfg, x, S))
+    out_hf = out_hf[0] if isinstance(out_hf, tuple) else out_hf
+    _close(mine(x), out_hf, "Llama decoder layer output")
+
+
+def test_moe_feed_forward_is_a_mixtral_sparse_moe_block():
+    from transformers import MixtralConfig
+    from transformers.models.mixtral.modeling_mixtral import MixtralSparseMoeBlock
+    dim, heads, ffn, E, T = 64, 1, 96, 8, 50
+    cfg = MixtralConfig(hidden_size=dim, intermediate_size=ffn, num_attention_heads=heads, num_key_value_heads=heads,
+                        num_local_experts=E, num_experts_per_tok=2, num_hidden_layers=1, vocab_size=32,
+                        router_jitter_noise=0.0, hidden_act="silu")
+    hf = MixtralSparseMoeBlock(cfg).eval()
+    torch.manual_seed(4)
+    for p in hf.parameters():
+        torch.nn.init.normal_(p, std=0.2)
+    mine = SM.MoELayer(dim, heads, ffn, E, dtype=torch.float32)
+    sd = hf.state_dict()
+    with torch.no_grad():
+        mine.block_sparse_moe.gate.weight.copy_(sd["gate.weight"])
+        if "experts.gate_up_proj" in sd:   # fused expert weights: [E, 2 ffn, dim] (gate rows, then up rows)
+            gu, dn = sd["experts.gate_up_proj"], sd["experts.down_proj"]
+            for e, ex in enumerate(mine.block_sparse_moe.experts):
+                ex.w1.weight.copy_(gu[e, :ffn])
+                ex.w3.weight.copy_(gu[e, ffn:])
+                ex.w2.weight.copy_(dn[e])
+        else:
+            for e, ex in enumerate(mine.block_sparse_moe.experts):
+                for w in ("w1", "w2", "w3"):
+                    getattr(ex, w).weight.copy_(sd[f"experts.{e}.{w}.weight"])
+    h = torch.randn(1, T, dim)
+    out_hf = hf(h)
+    out_hf = out_hf[0] if isinstance(out_hf, tuple) else out_hf
+    _close(mine._feed_forward(h), out_hf.reshape(1, T, dim), "Mixtral sparse MoE block output")
+    # and the oracle's own statement of the block
+    w1 = torch.stack([ex.w1.weight for ex in mine.block_sparse_moe.experts]).detach()
+    w2 = torch.stack([ex.w2.weight for ex in mine.block_sparse_moe.experts]).detach()
+    w3 = torch.stack([ex.w3.weight for ex in mine.block_sparse_moe.experts]).detach()
+    y = OO.moe_top2(h[0], sd["gate.weight"], w1, w2, w3)
+    _close(y, out_hf.reshape(T, dim), "oracle moe_top2")
