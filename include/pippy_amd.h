@@ -334,9 +334,14 @@ int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
  * ---------------------------------------------------------------------------------------- */
 int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, const void* extra_row, void* y,
                  int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
-/* d_wte (fp32 [vocab, C]) += scatter(dy) with atomics; d_wpe (fp32 [seq, C]) += sum over batch */
+/* Gradient of the lookup, added to fp32 accumulators (F.embedding's backward reached through
+ * pippy/_backward.py:67-69, followed by the accumulation into the parameter's gradient):
+ *   d_wte[v, :] += g[v, :],  g[v, :] = sum of dy[t, :] over the tokens t with ids[t] == v, formed in
+ *   fp32 in ascending t;  d_wpe[p, :] += sum over the batch of dy[b * seq + p, :] in ascending b.
+ * round_bf16 != 0 rounds g to bf16 before it is added: bit for bit what a bf16 gradient tensor folded
+ * in by pp_grad_accum_f32_bf16 leaves.  No atomics: results do not depend on scheduling.  C <= 8192. */
 int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe, int64_t n_tok,
-                 int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
+                 int64_t seq, int64_t C, int64_t vocab, int round_bf16, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
  * Cross-entropy loss of one microbatch (loss_fn at pippy/PipelineSchedule.py:154-155 when it is
@@ -375,7 +380,7 @@ enum pp_op_kind {
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
  *                 | j: causal
  *   EMBED_FWD     p: ids wte wpe y extra_row | i: n_tok seq C vocab
- *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab
+ *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab | j: round_bf16
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype
  *   ACCUM_*       p: acc g | i: n | j: init
  *   COPY_ROWS     p: src dst | i: n_rows row_bytes src_stride dst_stride

@@ -57,3 +57,22 @@ def accumulate_fp32(grads_bf16_bits: Sequence[np.ndarray]) -> np.ndarray:
     for g in grads_bf16_bits[1:]:
         acc = (acc + widen(g)).astype(np.float32)
     return acc
+
+
+def round_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns, round to nearest even (finite inputs)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def embedding_grad(ids: np.ndarray, dy_bf16_bits: np.ndarray, vocab: int, round_bf16: bool) -> np.ndarray:
+    """Gradient of ``F.embedding`` w.r.t. its table for one microbatch (reached from
+    pippy/_backward.py:67-69): row v is the sum of dy[t] over the tokens with ids[t] == v, formed in
+    fp32 in ascending t; ``round_bf16`` rounds it to bf16, the dtype of the table.  Returned as fp32.
+    ``np.add.at`` applies the additions one by one in index order."""
+    dy = (dy_bf16_bits.astype(np.uint32) << 16).view(np.float32)
+    g = np.zeros((vocab, dy.shape[1]), dtype=np.float32)
+    np.add.at(g, ids.reshape(-1), dy)
+    if round_bf16:
+        g = (round_to_bf16_bits(g).astype(np.uint32) << 16).view(np.float32)
+    return g

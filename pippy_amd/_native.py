@@ -125,7 +125,7 @@ def lib() -> C.CDLL:
         "pp_attn_fwd": [C.POINTER(AttnDesc), vp],
         "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
         "pp_embed_fwd": [vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
-        "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, vp],
+        "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
         "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
@@ -578,11 +578,11 @@ def embed_fwd(ids, wte, wpe, y, seq: int, extra_row=None) -> None:
                              ids.numel(), seq, Cc, vocab, current_stream()), "pp_embed_fwd")
 
 
-def embed_bwd(ids, dy, d_wte, d_wpe, seq: int) -> None:
+def embed_bwd(ids, dy, d_wte, d_wpe, seq: int, round_bf16: bool = False) -> None:
     require_cuda(ids, dy, d_wte, d_wpe)
     vocab, Cc = d_wte.shape
     check(lib().pp_embed_bwd(ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), ptr(d_wpe),
-                             ids.numel(), seq, Cc, vocab, current_stream()), "pp_embed_bwd")
+                             ids.numel(), seq, Cc, vocab, int(round_bf16), current_stream()), "pp_embed_bwd")
 
 
 def ce_loss(logits, target, loss, dlogits, workspace, V: int, ignore_index: int = -100) -> None:

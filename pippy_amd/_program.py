@@ -407,13 +407,16 @@ def op_embed_fwd(ids, wte, wpe, y, seq, extra_row=None) -> N.Op:
     return op
 
 
-def op_embed_bwd(ids, dy, d_wte, d_wpe, seq) -> N.Op:
+def op_embed_bwd(ids, dy, d_wte, d_wpe, seq, round_bf16=False) -> N.Op:
+    """``round_bf16``: the per-microbatch row sums are rounded to bf16 before they are added (the bits
+    of a bf16 gradient tensor folded into the fp32 accumulator)."""
     vocab, Cc = d_wte.shape
     assert d_wte.dtype == torch.float32 and dy.shape == (ids.numel(), Cc) and dy.is_contiguous()
     op = N.Op()
     op.kind = N.OP_EMBED_BWD
     op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), _p(d_wpe)
     op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
+    op.j[0] = int(round_bf16)
     return op
 
 

@@ -42,29 +42,71 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restric
     }
 }
 
-// d_wte[ids[t], :] += dy[t, :] with fp32 atomics (rows repeat when a token id repeats).
+// d_wte[id, :] += g[id, :] with g[id, :] the sum of dy[t, :] over the tokens t with ids[t] == id, added
+// in ascending t (fp32) and, with round_bf16, rounded to bf16 before it is added: the same bits as a
+// bf16 gradient tensor folded into the accumulator.  No atomics: one wave per token scans the ids; the
+// wave of the first occurrence of an id owns that row and sums all occurrences in order, every other
+// wave leaves at the first earlier occurrence it meets.  NW = 32-bit words (column pairs) per lane.
+template <int NW>
 __global__ __launch_bounds__(256) void embed_bwd_wte_kernel(const int64_t* __restrict__ ids,
                                                             const uint16_t* __restrict__ dy,
                                                             float* __restrict__ d_wte, int64_t n_tok,
-                                                            int C, int64_t vocab) {
+                                                            int C, int64_t vocab, int round_bf16) {
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tok) return;
     const int64_t id = ids[t];
     if (id < 0 || id >= vocab) return;
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(dy + t * C);
+    const int half_c = C >> 1;
+    float lo[NW], hi[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) lo[w] = hi[w] = 0.f;
+    for (int64_t base = 0; base < n_tok; base += 64) {
+        const int64_t idx = base + lane;
+        uint64_t mask = __ballot(idx < n_tok && ids[idx] == id);
+        if (base <= t) {
+            // occurrences before t: another wave owns the row
+            const uint64_t before = base + 64 <= t ? ~0ull : ((1ull << (t - base)) - 1ull);
+            if (mask & before) return;
+        }
+        while (mask) {
+            const int bit = __builtin_ctzll(mask);
+            mask &= mask - 1;
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(dy + (base + bit) * C);
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const int c = w * 64 + lane;
+                if (c < half_c) {
+                    const uint32_t v = src[c];
+                    lo[w] += bf16lo(v);
+                    hi[w] += bf16hi(v);
+                }
+            }
+        }
+    }
     float* dst = d_wte + id * C;
-    for (int c = lane; c < (C >> 1); c += 64) {
-        const uint32_t w = src[c];
-        unsafeAtomicAdd(dst + 2 * c, bf16lo(w));
-        unsafeAtomicAdd(dst + 2 * c + 1, bf16hi(w));
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const int c = w * 64 + lane;
+        if (c < half_c) {
+            float a = lo[w], b = hi[w];
+            if (round_bf16) {
+                const uint32_t r = pack_bf16(a, b);
+                a = bf16lo(r);
+                b = bf16hi(r);
+            }
+            float2* d2 = reinterpret_cast<float2*>(dst + 2 * c);
+            const float2 old = *d2;
+            *d2 = make_float2(old.x + a, old.y + b);
+        }
     }
 }
 
-// d_wpe[p, :] += sum_b dy[b*seq + p, :]; each (p, column) has one owner, summed in batch order.
+// d_wpe[p, :] += sum_b dy[b*seq + p, :]; each (p, column) has one owner, summed in batch order and,
+// with round_bf16, rounded to bf16 before it is added.
 __global__ __launch_bounds__(256) void embed_bwd_wpe_kernel(const uint16_t* __restrict__ dy,
                                                             float* __restrict__ d_wpe, int64_t n_tok,
-                                                            int64_t seq, int C) {
+                                                            int64_t seq, int C, int round_bf16) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over seq * C/2
     const int half_c = C >> 1;
     if (idx >= seq * half_c) return;
@@ -76,9 +118,21 @@ __global__ __launch_bounds__(256) void embed_bwd_wpe_kernel(const uint16_t* __re
         s0 += bf16lo(w);
         s1 += bf16hi(w);
     }
+    if (round_bf16) {
+        const uint32_t r = pack_bf16(s0, s1);
+        s0 = bf16lo(r);
+        s1 = bf16hi(r);
+    }
     float* dst = d_wpe + p * C + 2 * c;
     dst[0] += s0;
     dst[1] += s1;
+}
+
+template <int NW>
+static void launch_embed_bwd_wte(const int64_t* ids, const void* dy, float* d_wte, int64_t n_tok, int C,
+                                 int64_t vocab, int round_bf16, hipStream_t st) {
+    hipLaunchKernelGGL(embed_bwd_wte_kernel<NW>, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0, st, ids,
+                       (const uint16_t*)dy, d_wte, n_tok, C, vocab, round_bf16);
 }
 
 }  // namespace pp
@@ -100,18 +154,25 @@ extern "C" int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe
 }
 
 extern "C" int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe,
-                            int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream) {
+                            int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, int round_bf16,
+                            pp_stream stream) {
     if (n_tok < 0 || seq <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_bwd: bad shape");
     if (C % 2) return fail(PP_ERR_UNSUPPORTED, "pp_embed_bwd: C %% 2 != 0");
+    if (C > 8192) return fail(PP_ERR_UNSUPPORTED, "pp_embed_bwd: C > 8192");
     if (n_tok == 0) return PP_OK;
     if (!ids || !dy || !d_wte) return fail(PP_ERR_INVALID, "pp_embed_bwd: null pointer");
+    if (!aligned(dy, 4) || !aligned(d_wte, 8)) return fail(PP_ERR_INVALID, "pp_embed_bwd: misaligned pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(embed_bwd_wte_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0, st, ids,
-                       (const uint16_t*)dy, d_wte, n_tok, (int)C, vocab);
+    const int words = (int)((C / 2 + 63) / 64);
+    if (words <= 2) launch_embed_bwd_wte<2>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
+    else if (words <= 8) launch_embed_bwd_wte<8>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
+    else if (words <= 16) launch_embed_bwd_wte<16>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
+    else if (words <= 32) launch_embed_bwd_wte<32>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
+    else launch_embed_bwd_wte<64>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
     if (d_wpe) {
         const int64_t work = seq * (C / 2);
         hipLaunchKernelGGL(embed_bwd_wpe_kernel, dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st,
-                           (const uint16_t*)dy, d_wpe, n_tok, seq, (int)C);
+                           (const uint16_t*)dy, d_wpe, n_tok, seq, (int)C, round_bf16);
     }
     return check_launch("embed_bwd");
 }

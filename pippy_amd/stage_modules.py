@@ -234,13 +234,15 @@ class TokenEmbedding(NativeBlock):
         b.f(P.op_embed_fwd(ids, wte, wpe, y.view(Bn * S, Cc), S))
 
         def bwd(dy, need_dx, dx_out):
-            # scatter-add straight into the fp32 accumulators (zeroed on the first accumulation)
+            # added straight into the fp32 accumulators (zeroed on the first accumulation): per row the
+            # sum over its tokens in ascending order, rounded to bf16 first unless the stage adds
+            # unrounded sums (``fused_accumulate=True``)
             acc_wte = b.grad_acc(self.wte.weight)
             acc_wpe = b.grad_acc(self.wpe.weight) if self.wpe is not None else None
             b.w(P.op_fill(acc_wte), tag="fill")
             if acc_wpe is not None:
                 b.w(P.op_fill(acc_wpe), tag="fill")
-            b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S))
+            b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
             return None
 
         b.on_backward(bwd)
@@ -293,7 +295,7 @@ class EncoderEmbedding(NativeBlock):
             acc_wpe = b.grad_acc(self.position_embeddings.weight)
             b.w(P.op_fill(acc_wte), tag="fill")
             b.w(P.op_fill(acc_wpe), tag="fill")
-            b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S))
+            b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
             # the type-0 row receives the gradient of every token; the other rows none
             g_tt = b.grad_target(self.token_type_embeddings.weight)
             ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)

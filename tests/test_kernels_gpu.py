@@ -358,7 +358,7 @@ def test_embedding():
     wte = torch.randn(vocab, C, device=DEV).to(torch.bfloat16)
     wpe = torch.randn(seq, C, device=DEV).to(torch.bfloat16)
     ids = torch.randint(0, vocab, (B, seq), device=DEV)
-    ids[0, :5] = 7  # repeated ids exercise the atomic scatter
+    ids[0, :5] = 7  # repeated ids: one row receives several tokens
     y = torch.empty(B * seq, C, device=DEV, dtype=torch.bfloat16)
     Nn.embed_fwd(ids, wte, wpe, y, seq)
     ref = O.embedding(ids.cpu(), wte.float().cpu(), wpe.float().cpu()).reshape(B * seq, C)
@@ -378,6 +378,35 @@ def test_embedding():
     O.embedding(ids.cpu(), wr, pr).reshape(B * seq, C).backward(dy.float().cpu())
     assert_close_rel(d_wte, wr.grad, 1e-5, "d_wte")
     assert_close_rel(d_wpe, pr.grad, 1e-5, "d_wpe")
+
+
+@pytest.mark.parametrize("C,vocab,n_tok,seq", [(768, 50, 1024, 128), (64, 3, 333, 111), (4096, 17, 130, 65),
+                                               (1024, 32000, 2048, 1024)])
+@pytest.mark.parametrize("rounded", [False, True])
+def test_embedding_backward_is_ordered_and_bit_exact(C, vocab, n_tok, seq, rounded):
+    """Few distinct ids, so every row of the table receives many tokens: the row sums must equal the
+    oracle's one-by-one additions in ascending token order bit for bit, in both accumulation forms
+    (unrounded fp32 sums; sums rounded to bf16 first), on top of what the accumulator already holds,
+    and again on a second call."""
+    import numpy as np
+    from oracle import microbatch as OM
+    Nn = native()
+    g = torch.Generator().manual_seed(C + n_tok)
+    ids = torch.randint(0, vocab, (n_tok,), generator=g)
+    ids[-1] = ids[0]                      # the first and the last token share a row
+    dy = (torch.randn(n_tok, C, generator=g) * 3).to(torch.bfloat16)
+    start = torch.randn(vocab, C, generator=g)
+    start_p = torch.randn(seq, C, generator=g)
+    d_wte, d_wpe = start.to(DEV), start_p.to(DEV)
+    bits = dy.view(torch.int16).numpy().view(np.uint16)
+    gw = OM.embedding_grad(ids.numpy(), bits, vocab, rounded)
+    gp = OM.embedding_grad(np.arange(n_tok) % seq, bits, seq, rounded)
+    for call in range(2):
+        Nn.embed_bwd(ids.to(DEV), dy.to(DEV), d_wte, d_wpe, seq, round_bf16=rounded)
+        start = start + torch.from_numpy(gw)
+        start_p = start_p + torch.from_numpy(gp)
+        assert torch.equal(d_wte.cpu(), start), f"d_wte, call {call}"
+        assert torch.equal(d_wpe.cpu(), start_p), f"d_wpe, call {call}"
 
 
 def test_embedding_and_layernorm_full_size_closed_forms():

@@ -119,6 +119,30 @@ def test_accumulate_fp32_matches_torch_sequence():
     assert not np.array_equal(rev.view(np.uint32), acc.view(np.uint32))
 
 
+def test_embedding_grad_is_the_ordered_sum_and_matches_autograd():
+    torch.manual_seed(5)
+    vocab, n_tok, C = 7, 60, 16
+    ids = torch.randint(0, vocab, (n_tok,))
+    dy = torch.randn(n_tok, C).to(torch.bfloat16)
+    bits = dy.view(torch.int16).numpy().view(np.uint16)
+    g = OM.embedding_grad(ids.numpy(), bits, vocab, False)
+    # brute force: one fp32 addition per token, in order
+    ref = np.zeros((vocab, C), np.float32)
+    for t in range(n_tok):
+        ref[ids[t]] = ref[ids[t]] + dy[t].float().numpy()
+    assert np.array_equal(g.view(np.uint32), ref.view(np.uint32))
+    # autograd of F.embedding in fp64 agrees to rounding
+    w = torch.zeros(vocab, C, dtype=torch.float64, requires_grad=True)
+    torch.nn.functional.embedding(ids, w).backward(dy.double())
+    assert np.abs(g - w.grad.numpy()).max() <= 1e-5 * np.abs(w.grad.numpy()).max()
+    # the rounded form is torch's own bf16 rounding of those sums
+    gr = OM.embedding_grad(ids.numpy(), bits, vocab, True)
+    assert np.array_equal(gr, torch.from_numpy(g).to(torch.bfloat16).float().numpy())
+    x = torch.cat([torch.randn(4096) * 1e3, torch.tensor([0.0, -0.0, 1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8])])
+    assert np.array_equal(OM.round_to_bf16_bits(x.numpy()),
+                          x.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16))
+
+
 # ---- one pipelined step ----------------------------------------------------------------------------
 class _MLP(nn.Module):
     def __init__(self, d):
