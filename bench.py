@@ -13,7 +13,8 @@ the merge of the 8 logits chunks.  Inputs are resident in HBM before the timed r
 
 Prints one JSON line: tokens/s, the MFMA roofline of the dominant kernel (the bf16 GEMM, timed
 per launch with HIP events on its own stream in a second, instrumented pass over the same steps)
-and the CPU baseline (the oracle's fp32 restatement of the reference step on this box's cores).
+and the CPU baseline (the reference's own CPU path restated: one gloo process per stage, same schedule,
+on this box's cores, run before the GPU is touched).
 """
 import argparse
 import json
@@ -133,39 +134,53 @@ def flops_per_step(args):
     return 3.0 * per_token_fwd * T
 
 
-def cpu_baseline(args, sample_microbatches=4):
-    """The oracle's statement of the reference step (fp32, torch CPU kernels, this box's cores) on a
-    bounded sample of the same workload: the first microbatches of one step through all stages,
-    forward, loss and backward in the reference's order."""
-    from oracle import pipeline as OP
-    from pippy_amd.configs import DecoderLM
-    import torch.nn as nn
-    torch.manual_seed(0)
-    model = DecoderLM(vocab=args.vocab, max_seq=args.seq, dim=args.dim, n_layers=args.layers,
-                      n_heads=args.heads, ffn=args.ffn, dtype=torch.float32)
-    per = args.layers // args.stages
-    stages = []
-    for s in range(args.stages):
-        mods = ([model.embed] if s == 0 else []) + [model.h[i] for i in range(per * s, per * (s + 1))]
-        if s == args.stages - 1:
-            mods.append(model.head)
-        stages.append(nn.Sequential(*mods))
-    mb = args.batch // args.microbatches
-    n = sample_microbatches
-    ids = torch.randint(0, args.vocab, (mb * n, args.seq))
-    target = torch.randint(0, args.vocab, (mb * n, args.seq))
-
-    def ce(o, t):
-        return torch.nn.functional.cross_entropy(o.reshape(-1, o.shape[-1]), t.reshape(-1))
-
-    t0 = time.perf_counter()
-    OP.step(stages, ids, target, n, ce)
-    dt = time.perf_counter() - t0
-    return {"value": round(ids.numel() / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"{n} of {args.microbatches} microbatches ({ids.numel()} tokens) of one step: "
-                      f"fp32 forward+loss+backward through all {args.stages} stages in the reference's "
-                      f"order, one process, {dt:.1f} s"}
+def cpu_baseline(args, budget_seconds=45.0):
+    """The reference's own way of running this workload on host cores (its tests: backend gloo, one
+    process per stage, ``test/test_fwd.py:117-129``), restated in ``oracle/gloo_pipeline.py``: S fresh
+    CPU-only child processes over gloo on 127.0.0.1, each running its rank's program of the same 1F1B
+    schedule on its stage of the same model, ``cores // S`` threads each, in the arithmetic of the
+    configuration (bf16 parameters, activations and gradients).  One warm-up microbatch through the
+    whole pipeline, then one timed step; if the warm-up says a full step would overrun the budget the
+    first half (quarter ...) of the step's microbatches is timed instead, and ``sample`` says so.
+    Must be called before this process touches the GPU: the children are started from a parent that
+    holds no GPU state."""
+    import socket
+    import subprocess
+    cores = torch.get_num_threads()
+    S = args.stages
+    threads = max(1, cores // S)
+    with socket.socket() as sock:
+        sock.bind(("127.0.0.1", 0))
+        port = sock.getsockname()[1]
+    env = dict(os.environ, MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port), OMP_NUM_THREADS=str(threads),
+               HIP_VISIBLE_DEVICES="", CUDA_VISIBLE_DEVICES="")
+    common = ["--world", str(S), "--threads", str(threads), "--dtype", "bf16", "--vocab", str(args.vocab),
+              "--seq", str(args.seq), "--dim", str(args.dim), "--layers", str(args.layers), "--heads",
+              str(args.heads), "--ffn", str(args.ffn), "--batch", str(args.batch), "--microbatches",
+              str(args.microbatches), "--budget-seconds", str(budget_seconds)]
+    procs = [subprocess.Popen([sys.executable, "-m", "oracle.gloo_pipeline", "--rank", str(r)] + common, cwd=ROOT,
+                              env=env, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+             for r in range(S)]
+    try:
+        out0, _ = procs[0].communicate(timeout=420)
+        for p in procs[1:]:
+            p.wait(timeout=60)
+    except subprocess.TimeoutExpired:
+        for p in procs:
+            p.kill()
+        return {"value": None, "unit": "tokens/s", "cores": cores, "kind": "port",
+                "sample": "the CPU pipeline did not finish within 420 s and was stopped"}
+    if any(p.returncode for p in procs):
+        return {"value": None, "unit": "tokens/s", "cores": cores, "kind": "port",
+                "sample": f"a CPU pipeline process failed (exit codes {[p.returncode for p in procs]})"}
+    rep = json.loads([ln for ln in out0.splitlines() if ln.startswith("{")][-1])
+    n, M = rep["microbatches_timed"], rep["microbatches"]
+    what = "one full step" if n == M else f"the first {n} of {M} microbatches of one step"
+    return {"value": round(rep["tokens"] / rep["step_s"], 1), "unit": "tokens/s", "cores": S * threads,
+            "kind": "port", "dtype": "bf16", "processes": S, "threads_per_process": threads,
+            "sample": f"{what} ({rep['tokens']} tokens) of the same workload: {S} CPU processes over gloo, one "
+                      f"per stage, 1F1B, bf16, after a warm-up of {rep['warmup_microbatches']} microbatch "
+                      f"({rep['warmup_s']:.1f} s); timed {rep['step_s']:.1f} s"}
 
 
 def main():
@@ -209,9 +224,13 @@ def main():
         print("bench.py: this build runs every pipeline stage as a virtual stage on ONE GPU; "
               "there is no multi-GPU path to measure (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
-    if not torch.cuda.is_available():
+    if torch.cuda.device_count() < 1:   # counting devices does not initialise the GPU runtime
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
+    # the CPU baseline runs first, in child processes started while this process holds no GPU state
+    cpu_result = None
+    if not args.no_cpu_baseline and args.workload == "gpt2":
+        cpu_result = cpu_baseline(args)
 
     from pippy_amd import _native as N
     N.lib()  # fail loudly if the kernel library is missing
@@ -370,8 +389,8 @@ def main():
                              "frac": round(obytes / (oms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "ms_per_step": round(oms, 3)}
         result["other_kernels"] = hbm
 
-    if not args.no_cpu_baseline and default_workload:
-        result["cpu_baseline"] = cpu_baseline(args)
+    if cpu_result is not None:
+        result["cpu_baseline"] = cpu_result
 
     print(json.dumps(result))
 

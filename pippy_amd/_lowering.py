@@ -48,12 +48,16 @@ def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
     return None
 
 
+class NotLowerable(Exception):
+    """Why a stage module cannot run as launch lists (the message names the construct)."""
+
+
 def _chain_nodes(gm_graph: fx.Graph) -> Optional[List[fx.Node]]:
     """The compute nodes of a graph that is a pure chain (one placeholder, every node consuming
     exactly the previous node's value, the last one returned), else None."""
     placeholders = [n for n in gm_graph.nodes if n.op == "placeholder"]
     if len(placeholders) != 1:
-        return None
+        raise NotLowerable(f"the stage takes {len(placeholders)} inputs; a launch-list stage takes one tensor")
     prev = placeholders[0]
     chain = []
     for n in gm_graph.nodes:
@@ -69,7 +73,9 @@ def _chain_nodes(gm_graph: fx.Graph) -> Optional[List[fx.Node]]:
         tensor_args = [a for a in n.args if isinstance(a, fx.Node)]
         tensor_args += [a for a in n.kwargs.values() if isinstance(a, fx.Node)]
         if tensor_args != [prev] or len(prev.users) != 1:
-            return None
+            raise NotLowerable(f"node '{n.format_node()}' does not continue a chain of single-input layers "
+                               "(branches, residual adds and multi-input ops need one of the blocks of "
+                               "pippy_amd.stage_modules around them)")
         chain.append(n)
         prev = n
     return None
@@ -78,7 +84,7 @@ def _chain_nodes(gm_graph: fx.Graph) -> Optional[List[fx.Node]]:
 def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeBlock]]:
     nodes = _chain_nodes(graph)
     if nodes is None:
-        return None
+        raise NotLowerable("the stage does not return the value of its last layer")
     blocks: List[NativeBlock] = []
     i = 0
     while i < len(nodes):
@@ -88,7 +94,7 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
             i += 1
             continue
         if n.op != "call_module":
-            return None
+            raise NotLowerable(f"'{n.format_node()}' is not a module call or a supported activation")
         m = root.get_submodule(n.target)
         if isinstance(m, NativeBlock):
             blocks.append(m)
@@ -101,39 +107,55 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
                 blocks.append(LinearAct(m, None))
         elif isinstance(m, nn.LayerNorm):
             if len(m.normalized_shape) != 1 or not m.elementwise_affine:
-                return None
+                raise NotLowerable(f"LayerNorm '{n.target}' normalises over {len(m.normalized_shape)} dimensions "
+                                   "or has no affine parameters")
             blocks.append(LayerNormBlock(m))
         elif isinstance(m, nn.RMSNorm):
             if len(m.normalized_shape) != 1 or m.weight is None or m.eps is None:
-                return None
+                raise NotLowerable(f"RMSNorm '{n.target}' needs one normalised dimension, a weight and an eps")
             blocks.append(RMSNormBlock(m))
         else:
             # a user container (e.g. a block that wraps a linear and an activation): lower it as
             # a chain of its own and splice the result in
-            sub = lower_stage_module(m)
-            if sub is None:
-                return None
-            blocks.extend(sub)
+            blocks.extend(_lower(m))
         i += 1
-    return blocks or None
+    if not blocks:
+        raise NotLowerable("the stage holds no layer")
+    return blocks
 
 
-def lower_stage_module(submod: nn.Module) -> Optional[List[NativeBlock]]:
-    """Blocks of a lowerable stage module, or None when it has to run eagerly."""
+def _lower(submod: nn.Module) -> List[NativeBlock]:
     if isinstance(submod, NativeBlock):
         return [submod]
     if isinstance(submod, StageSequence):
         out: List[NativeBlock] = []
         for child in submod.blocks():
-            sub = lower_stage_module(child)
-            if sub is None:
-                return None
-            out.extend(sub)
-        return out or None
+            out.extend(_lower(child))
+        if not out:
+            raise NotLowerable("the stage holds no layer")
+        return out
     if isinstance(submod, fx.GraphModule):
         return blocks_from_graph(submod, submod.graph)
+    if isinstance(submod, (nn.Linear, nn.LayerNorm, nn.RMSNorm)):
+        # a stage that is one standard layer: the same rules as for that layer inside a chain
+        holder = nn.Module()
+        holder.layer = submod
+        g = fx.Graph()
+        g.output(g.call_module("layer", (g.placeholder("x"),)))
+        return blocks_from_graph(holder, g)
     try:
         graph = _ChainTracer().trace(submod)
-    except Exception:
-        return None
+    except Exception as e:
+        raise NotLowerable(f"torch.fx cannot trace {type(submod).__name__}: {type(e).__name__}: {e}") from e
     return blocks_from_graph(submod, graph)
+
+
+def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None) -> Optional[List[NativeBlock]]:
+    """Blocks of a lowerable stage module, or None when it has to run eagerly; the reason is then
+    appended to ``why``."""
+    try:
+        return _lower(submod)
+    except NotLowerable as e:
+        if why is not None:
+            why.append(str(e))
+        return None

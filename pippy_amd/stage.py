@@ -111,9 +111,20 @@ class PipelineStageBase:
 
         self.fused_accumulate = fused_accumulate
         self.split_backward = False
-        self._blocks = None if force_eager else lower_stage_module(submodule)
+        why: List[str] = []
+        if not force_eager and self.device.type != "cuda":
+            force_eager = True
+            why.append(f"its device is '{self.device}' and launch lists run on the GPU only")
+        self._blocks = None if force_eager else lower_stage_module(submodule, why)
         self._program: Optional[P.StageProgram] = None
+        #: why this stage runs through torch autograd instead of HIP launch lists (None: it is native)
+        self.eager_reason: Optional[str] = None
         if self._blocks is None:
+            self.eager_reason = why[0] if why else (
+                "its inputs or outputs are not a single tensor chain between consecutive stages"
+                if force_eager else "unknown")
+            logger.warning(f"{self.log_prefix} runs eagerly through torch autograd, not as HIP launch lists: "
+                           f"{self.eager_reason}")
             self.submod.to(self.device)
 
     # -- reference properties -----------------------------------------------------------------
@@ -278,11 +289,15 @@ class PipelineStageBase:
         if type(output) is list:
             output = tuple(output)
         output_tuple = output if type(output) is tuple else (output,)
+        self._check_live_shapes(flat_inputs, output_tuple)
         self.output_chunks.append(output)
         self.fwd_cache[mb] = (output_tuple, flat_inputs)
         self._fwd_done[mb] = True
         self.fwd_chunk_id += 1
         return output
+
+    def _check_live_shapes(self, flat_inputs, output_tuple) -> None:
+        """Hook for stages that were given example values (``ManualPipelineStage``)."""
 
     def _forward_native(self, mb, args, kwargs):
         sp = self._stage_program()
@@ -612,15 +627,58 @@ class PipelineStage(PipelineStageBase):
 
 class ManualPipelineStage(PipelineStageBase):
     """A stage built from a hand-written module (reference ``ManualPipelineStage.py:178-307``).
-    ``input_args`` / ``output_args`` are example microbatch values; the reference uses them to size
-    its receive buffers and to exchange shapes between ranks.  Here shapes are taken from the live
-    tensors, so the examples are only checked for consistency."""
+    ``input_args`` / ``output_args`` are example microbatch values; the reference sizes its receive
+    buffers from them and compares them between neighbouring ranks (``ManualPipelineStage.py:342-439``).
+    Here buffers take their shapes from the live tensors, and the examples are a contract that is
+    checked: every forward compares the shape and dtype of what the stage receives and produces with
+    the examples and raises ``ValueError`` on a mismatch; ``validate_stage_shapes`` compares the
+    examples of consecutive stages."""
 
     def __init__(self, submodule: nn.Module, stage_index: int, num_stages: int, device,
                  num_microbatches: int, input_args=None, output_args=None, group=None, **kw):
         super().__init__(submodule, stage_index, num_stages, device, num_microbatches, group, **kw)
         self.inputs = _to_tuple(input_args)
         self.outputs = _to_tuple(output_args)
+
+    @staticmethod
+    def _meta(values):
+        return [(tuple(v.shape), v.dtype) for v in values if isinstance(v, torch.Tensor)]
+
+    def _check_live_shapes(self, flat_inputs, output_tuple) -> None:
+        for what, examples, live in (("input", self.inputs, flat_inputs), ("output", self.outputs, output_tuple)):
+            want = self._meta(examples)
+            if not want:
+                continue
+            got = self._meta(live)
+            if got != want:
+                raise ValueError(
+                    f"{self.log_prefix} {what} of microbatch {self.fwd_chunk_id} has shape/dtype {got}, "
+                    f"but the stage was built with example {what}s {want}")
+
+
+def validate_stage_shapes(pipeline_stages: List["ManualPipelineStage"]) -> None:
+    """Checks that the example values the stages were built with fit together (reference
+    ``ManualPipelineStage.py:342-439``, without its all-gather: every stage lives in this process):
+    all stages agree on the number of stages, and the example output of stage i has the shapes of the
+    example input of stage i + 1 wherever both were given.  Raises ``ValueError``."""
+    if len(pipeline_stages) == 0:
+        raise ValueError("No pipeline stages provided.")
+    ordered = sorted(pipeline_stages, key=lambda st: st.stage_index)
+    num_stages = ordered[0].num_stages
+    for st in ordered:
+        if st.num_stages != num_stages:
+            raise ValueError(
+                f"Stage id {st.stage_index} has num stages ({st.num_stages}) which does not match num stages "
+                f"({num_stages}) of other stages.")
+    for a, b in zip(ordered, ordered[1:]):
+        if b.stage_index != a.stage_index + 1:
+            continue
+        out = [list(s) for s, _ in ManualPipelineStage._meta(a.outputs)]
+        inp = [list(s) for s, _ in ManualPipelineStage._meta(b.inputs)]
+        if out and inp and out != inp:
+            raise ValueError(
+                f"Stage_id {a.stage_index} output shape {out} at does not match stage_id {b.stage_index} "
+                f"input shape {inp}.")
 
 
 def _to_tuple(v):

@@ -443,3 +443,60 @@ def test_pipeline_accepts_the_microbatch_spelling_and_build_stage():
         pp.pipeline(model, 4, (x,), mb_args=(x,))
     with pytest.raises(TypeError, match="num_chunks"):
         pp.pipeline(model)
+
+
+# ---- example values of a hand-built stage are a checked contract (reference ManualPipelineStage.py:342-439)
+def test_manual_stage_checks_live_shapes_against_its_examples():
+    from pippy_amd.stage import validate_stage_shapes
+    lin = nn.Linear(4, 6)
+    kw = dict(force_eager=True)   # host tensors: the torch path (launch lists take device tensors)
+    stage = ManualPipelineStage(lin, 0, 1, "cpu", 2, input_args=torch.zeros(3, 4), output_args=torch.zeros(3, 6), **kw)
+    assert not stage.is_native and stage.eager_reason
+    sched = pp.ScheduleGPipe([stage], 2)
+    out = sched._step_microbatches([(torch.ones(3, 4),), (torch.ones(3, 4),)])
+    assert out is None and len(stage.output_chunks) == 2
+    stage.clear_runtime_states()
+    with pytest.raises(ValueError, match="example inputs"):
+        sched._step_microbatches([(torch.ones(2, 4),), (torch.ones(2, 4),)])
+    wrong_out = ManualPipelineStage(lin, 0, 1, "cpu", 1, input_args=torch.zeros(3, 4), output_args=torch.zeros(3, 5), **kw)
+    with pytest.raises(ValueError, match="example outputs"):
+        pp.ScheduleGPipe([wrong_out], 1)._step_microbatches([(torch.ones(3, 4),)])
+    wrong_dtype = ManualPipelineStage(lin, 0, 1, "cpu", 1, input_args=torch.zeros(3, 4, dtype=torch.float64), **kw)
+    with pytest.raises(ValueError, match="example inputs"):
+        pp.ScheduleGPipe([wrong_dtype], 1)._step_microbatches([(torch.ones(3, 4),)])
+
+    a = ManualPipelineStage(nn.Linear(4, 6), 0, 2, "cpu", 1, input_args=torch.zeros(3, 4), output_args=torch.zeros(3, 6))
+    b = ManualPipelineStage(nn.Linear(6, 2), 1, 2, "cpu", 1, input_args=torch.zeros(3, 6))
+    validate_stage_shapes([a, b])
+    c = ManualPipelineStage(nn.Linear(5, 2), 1, 2, "cpu", 1, input_args=torch.zeros(3, 5))
+    with pytest.raises(ValueError, match="does not match stage_id 1 input shape"):
+        validate_stage_shapes([a, c])
+    d = ManualPipelineStage(nn.Linear(6, 2), 1, 3, "cpu", 1, input_args=torch.zeros(3, 6))
+    with pytest.raises(ValueError, match="num stages"):
+        validate_stage_shapes([a, d])
+    with pytest.raises(ValueError, match="No pipeline stages"):
+        validate_stage_shapes([])
+
+
+def test_a_stage_that_cannot_be_lowered_says_why(caplog):
+    class Branchy(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = nn.Linear(4, 4)
+
+        def forward(self, x):
+            return x + self.a(x)
+
+    import logging
+    from pippy_amd._lowering import lower_stage_module
+    why = []
+    assert lower_stage_module(Branchy(), why) is None and "does not continue a chain" in why[0]
+    with caplog.at_level(logging.WARNING, logger="pippy_amd.stage"):
+        stage = ManualPipelineStage(Branchy(), 0, 1, "cpu", 1)
+    assert not stage.is_native and stage.eager_reason
+    assert any("runs eagerly" in r.getMessage() for r in caplog.records)
+    why = []
+    assert lower_stage_module(nn.Sequential(nn.Linear(4, 4), nn.ReLU(), nn.Linear(4, 2)), why) and not why
+    assert lower_stage_module(nn.Linear(4, 2), why) and not why
+    host = ManualPipelineStage(nn.Linear(4, 2), 0, 1, "cpu", 1)
+    assert not host.is_native and "GPU only" in host.eager_reason
