@@ -156,11 +156,16 @@ int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
  * it is for.  The workspace must not be shared by launches that may overlap. */
 int pp_gemm_bf16_splitk(const pp_gemm_desc* desc, float* workspace, int64_t workspace_elems, pp_stream stream);
 
-/* Several independent GEMMs in one launch (up to PP_GEMM_MAX_GROUP; longer lists are split).  All
- * descriptors must agree in a_trans, b_trans, epilogue and c_dtype.  The weight-gradient GEMMs of
- * one stage and microbatch (pippy/_backward.py:67-69 reaches them through autograd one by one) are
- * small but independent of each other: grouped, their tiles fill the GPU together. */
-#define PP_GEMM_MAX_GROUP 16
+/* Several independent GEMMs in one launch (longer lists go out as several launches of at most
+ * PP_GEMM_MAX_GROUP problems).  All descriptors must agree in a_trans, b_trans and c_dtype.  With a bf16
+ * C every problem may bring its own epilogue (any but the accumulating ones); with an fp32 C the
+ * problems are either all PP_EPI_NONE or all accumulating (PP_EPI_ACCUM_F32 / _ROUNDED and beta per
+ * problem).  The weight-gradient GEMMs of one stage and microbatch (pippy/_backward.py:67-69 reaches
+ * them through autograd one by one) are small but independent of each other, and so are the GEMMs that
+ * different pipeline stages reach at the same point of their passes (pippy/_PipelineStage.py:420-428 on
+ * different ranks): grouped, their tiles fill the GPU together.  A problem computes the same bits
+ * alone or in a group. */
+#define PP_GEMM_MAX_GROUP 28
 int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream);
 
 /* One GEMM per segment of a row-partitioned operand, with the segment bounds in DEVICE memory:

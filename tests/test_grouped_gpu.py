@@ -38,9 +38,60 @@ def test_grouped_weight_gradient_gemms_equal_single_launches(fused):
 def test_grouped_rejects_mixed_configurations():
     from pippy_amd import _native as N
     A = torch.zeros(16, 8, device=DEV, dtype=torch.bfloat16)
+    At = torch.zeros(8, 16, device=DEV, dtype=torch.bfloat16)
     C = torch.zeros(16, 16, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match="differs"):
-        N.gemm_bf16_grouped([(A, A, C, {}), (A, A, C, dict(epilogue=N.EPI_BIAS_RELU))])
+    Cf = torch.zeros(16, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="differs in layout"):
+        N.gemm_bf16_grouped([(A, A, C, {}), (At, A, C, dict(a_trans=True))])
+    with pytest.raises(RuntimeError, match="differs in layout or output dtype"):
+        N.gemm_bf16_grouped([(A, A, C, {}), (A, A, Cf, {})])
+    with pytest.raises(RuntimeError, match="mixes plain and accumulating"):
+        N.gemm_bf16_grouped([(A, A, Cf, {}), (A, A, Cf, dict(epilogue=N.EPI_ACCUM_F32, beta=1))])
+    with pytest.raises(RuntimeError, match="with bf16 C"):
+        N.gemm_bf16_grouped([(A, A, C, {}), (A, A, C, dict(epilogue=N.EPI_ACCUM_F32))])
+
+
+@pytest.mark.parametrize("M,K", [(4096, 768), (200, 136)])
+def test_grouped_problems_with_different_epilogues_equal_single_launches(M, K):
+    """The GEMMs that several stages reach at the same point of their passes go out as one launch in
+    which every problem brings its own epilogue; each must leave the bits of its own single launch
+    (the reduction order over k does not depend on the tile shape or on the neighbours in the grid)."""
+    from pippy_amd import _native as N
+    torch.manual_seed(3)
+
+    def problem(Nn, epi):
+        A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+        B = (torch.randn(Nn, K, device=DEV) * 0.05).to(torch.bfloat16)
+        kw = dict(epilogue=epi)
+        if epi in (N.EPI_BIAS, N.EPI_BIAS_GELU_TANH, N.EPI_BIAS_GELU_ERF, N.EPI_BIAS_RESIDUAL, N.EPI_BIAS_RELU):
+            kw["bias"] = torch.randn(Nn, device=DEV).to(torch.bfloat16)
+        if epi in (N.EPI_BIAS_RESIDUAL, N.EPI_DGELU_TANH, N.EPI_DGELU_ERF, N.EPI_DRELU):
+            kw["aux_in"] = torch.randn(M, Nn, device=DEV).to(torch.bfloat16)
+        return A, B, kw
+
+    specs = [(768, N.EPI_BIAS_RESIDUAL), (2304, N.EPI_BIAS), (3072, N.EPI_BIAS_GELU_TANH), (768, N.EPI_NONE),
+             (3072, N.EPI_DGELU_TANH), (264, N.EPI_BIAS_GELU_ERF), (136, N.EPI_DGELU_ERF), (520, N.EPI_BIAS_RELU),
+             (392, N.EPI_DRELU)]
+    group, singles = [], []
+    for Nn, epi in specs:
+        A, B, kw = problem(Nn, epi)
+        outs = []
+        for _ in range(2):
+            C = torch.full((M, Nn), 7.0, device=DEV, dtype=torch.bfloat16)
+            k2 = dict(kw)
+            if epi in (N.EPI_BIAS_GELU_TANH, N.EPI_BIAS_GELU_ERF):
+                k2["aux_out"] = torch.full((M, Nn), 7.0, device=DEV, dtype=torch.bfloat16)
+            outs.append((C, k2))
+        group.append((A, B, outs[0][0], outs[0][1]))
+        singles.append((A, B, outs[1][0], outs[1][1]))
+    N.gemm_bf16_grouped(group)
+    for A, B, C, kw in singles:
+        N.gemm_bf16(A, B, C, **kw)
+    torch.cuda.synchronize()
+    for (Nn, epi), g, s_ in zip(specs, group, singles):
+        assert torch.equal(g[2], s_[2]), f"C of N={Nn} epilogue {epi}"
+        if "aux_out" in g[3]:
+            assert torch.equal(g[3]["aux_out"], s_[3]["aux_out"]), f"saved pre-activation of N={Nn} epilogue {epi}"
 
 
 def test_grouped_column_reductions_equal_single_calls():
