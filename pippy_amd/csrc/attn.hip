@@ -132,6 +132,40 @@ __device__ __forceinline__ void await_block(int64_t j, int64_t nb) {
 
 extern __shared__ __attribute__((aligned(16))) uint16_t attn_lds[];
 
+// Which (batch, head) and which block a work-group takes.  All work-groups of a (batch, head) stay on
+// one XCD (their K and V share its L2).  `ord` counts a head's blocks from the longest: under a causal
+// mask block `ord` of the query-parallel kernels is query block nx - 1 - ord (it sees the most keys), of
+// the key-parallel kernel key block ord (it is seen by the most queries).
+//
+// A causal launch is bound by how the unequal blocks meet on a CU: with three resident work-groups
+// per CU and work-groups handed to the 32 CUs of an XCD in turn, CU c holds the work-groups c, c + 32
+// and c + 64 of its XCD; numbered head by head these are three blocks of the same length, so one CU
+// gets three longest blocks and another three shortest.  Here the blocks of an XCD are ranked by
+// length (all heads' longest first) and dealt out in rounds of 32 that alternate in direction, so
+// every CU's blocks add up to about the same length, and work-groups that start later (when more
+// exist than fit at once) are the short ones.  The assignment is a permutation of the same work, so
+// results do not depend on it.
+constexpr uint32_t kCusPerXcd = 32;
+__device__ __forceinline__ bool attn_block_of(uint32_t bid, uint32_t grid, uint32_t nx, uint32_t heads,
+                                              bool balance, uint32_t* bh, uint32_t* ord) {
+    if (balance && heads % 8 == 0) {
+        const uint32_t x = bid & 7, t = bid >> 3;      // XCD, arrival order inside it
+        const uint32_t g = heads / 8, per = nx * g;    // heads and work-groups per XCD
+        if (t >= per) return false;
+        const uint32_t r = t / kCusPerXcd, p = t % kCusPerXcd;
+        const bool whole_round = (r + 1) * kCusPerXcd <= per;
+        const uint32_t k = r * kCusPerXcd + (((r & 1) && whole_round) ? kCusPerXcd - 1 - p : p);
+        *bh = x * g + k % g;
+        *ord = k / g;
+        return true;
+    }
+    const uint32_t vid = xcd_remap(bid, grid);
+    if (vid >= nx * heads) return false;
+    *bh = vid / nx;
+    *ord = vid % nx;
+    return true;
+}
+
 // ---- forward ----------------------------------------------------------------------------------
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const AttnArgs a) {
@@ -145,13 +179,11 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave & 1, half = wave >> 1;
     const int l32 = lane & 31, lh = lane >> 5;
-    // all blocks of a (batch, head) on one XCD; causal: late query blocks have the most key blocks
-    // and go first
     const uint32_t nx = (uint32_t)(a.S / 64);
-    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
-    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
-    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
-    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - vid % nx : vid % nx) * 64;
+    uint32_t bh, ord;
+    if (!attn_block_of(blockIdx.x, gridDim.x, nx, (uint32_t)(a.H * a.B), CAUSAL, &bh, &ord)) return;
+    const int64_t b = bh / a.H, h = bh % a.H;
+    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - ord : ord) * 64;
     const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;  // this lane's query row
 
@@ -303,10 +335,10 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     const int grp = wave & 1, half = wave >> 1;  // 32 keys of the block x 32 of every 64 queries
     const int l32 = lane & 31, lh = lane >> 5;
     const uint32_t nx = (uint32_t)(a.S / 64);
-    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
-    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
-    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
-    const int64_t kv0 = (int64_t)(vid % nx) * 64;  // early key blocks see the most queries and go first
+    uint32_t bh, ord;
+    if (!attn_block_of(blockIdx.x, gridDim.x, nx, (uint32_t)(a.H * a.B), CAUSAL, &bh, &ord)) return;
+    const int64_t b = bh / a.H, h = bh % a.H;
+    const int64_t kv0 = (int64_t)ord * 64;  // early key blocks see the most queries
     const int64_t kvw0 = kv0 + 32 * grp;
     const int64_t kvi = kvw0 + l32;  // this lane's key row
 
@@ -468,10 +500,10 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
     const int grp = wave & 1, half = wave >> 1;  // 32 queries of the block x 32 of every 64 keys
     const int l32 = lane & 31, lh = lane >> 5;
     const uint32_t nx = (uint32_t)(a.S / 64);
-    const uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
-    if (vid >= nx * (uint32_t)(a.H * a.B)) return;
-    const int64_t b = vid / nx / a.H, h = vid / nx % a.H;
-    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - vid % nx : vid % nx) * 64;
+    uint32_t bh, ord;
+    if (!attn_block_of(blockIdx.x, gridDim.x, nx, (uint32_t)(a.H * a.B), CAUSAL, &bh, &ord)) return;
+    const int64_t b = bh / a.H, h = bh % a.H;
+    const int64_t q0 = (int64_t)(CAUSAL ? nx - 1 - ord : ord) * 64;
     const int64_t qw0 = q0 + 32 * grp;
     const int64_t qi = qw0 + l32;
 
