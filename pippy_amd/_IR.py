@@ -31,12 +31,30 @@ logger = logging.getLogger(__name__)
 _active_tracer: Optional["fx.Tracer"] = None
 
 
+# The marker as an operator, so that ``torch.export`` records it too (the reference registers
+# ``pippy::_pipe_split`` for the same purpose, ``_IR.py:319-329``): no inputs, no outputs, no effect.
+@torch.library.custom_op("pippy_amd::_pipe_split", mutates_args=())
+def _pipe_split_op() -> None:
+    return None
+
+
+@_pipe_split_op.register_fake
+def _pipe_split_fake() -> None:
+    return None
+
+
+fx.node._side_effectful_functions.add(torch.ops.pippy_amd._pipe_split.default)
+
+
 def pipe_split():
     """Marks a stage boundary when called inside a model's ``forward``
-    (reference ``_IR.py:319-342``).  A no-op outside of ``pipeline()``; while ``pipeline()`` traces
-    the model it records a marker node at the current position of the graph."""
+    (reference ``_IR.py:319-342``).  While ``pipeline()`` traces the model symbolically it records a
+    marker node at the current position of the graph; otherwise it calls the marker operator, which
+    does nothing when the model simply runs and which ``torch.export`` keeps in the exported graph."""
     if _active_tracer is not None:
         _active_tracer.create_proxy("call_function", pipe_split, (), {})
+        return None
+    torch.ops.pippy_amd._pipe_split()
     return None
 
 
@@ -91,6 +109,46 @@ def _insert_markers(gm_graph: fx.Graph, split_spec: Dict[str, SplitPoint]):
                 gm_graph.call_function(pipe_split, (), {})
         else:
             raise ValueError(f"Unknown split point type {point}")
+
+
+def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Optional[Dict[str, Any]],
+                     split_spec: Optional[Dict[str, SplitPoint]]) -> Tuple[fx.GraphModule, fx.Graph]:
+    """The route of the reference (``_IR.py:1141-1145``): ``torch.export`` on the inputs of one
+    microbatch, for models that symbolic tracing cannot follow (Python control flow on shapes, calls
+    torch.fx has no proxy for).  Returns the exported module, whose parameters and buffers keep their
+    qualified names, and its ATen-level graph with a ``pipe_split`` marker node at every stage
+    boundary: where the model called ``pipe_split()``, and where ``split_spec`` names a submodule (the
+    first / last node that the exporter recorded as coming from inside it)."""
+    ep = torch.export.export(mod, tuple(mb_args), dict(mb_kwargs or {}), strict=False)
+    gm = ep.module()
+    graph = gm.graph
+    for n in list(graph.nodes):
+        if n.op == "call_module" and str(n.target).startswith("_guards"):
+            graph.erase_node(n)   # shape guards of the example inputs: stages re-check nothing
+        elif n.op == "call_function" and n.target is torch.ops.pippy_amd._pipe_split.default:
+            n.target = pipe_split
+    compute = [n for n in graph.nodes if n.op in ("call_function", "call_method", "call_module")]
+    for name, point in (split_spec or {}).items():
+        inside = [n for n in compute
+                  if any(v[0] == name or v[0].startswith(name + ".")
+                         for v in (n.meta.get("nn_module_stack") or {}).values())]
+        if not inside:
+            raise ValueError(f"Specified split point {name!r} is not a module called by the model")
+        if point == SplitPoint.BEGINNING:
+            with graph.inserting_before(inside[0]):
+                graph.call_function(pipe_split, (), {})
+        elif point == SplitPoint.END:
+            with graph.inserting_after(inside[-1]):
+                graph.call_function(pipe_split, (), {})
+        else:
+            raise ValueError(f"Unknown split point type {point}")
+    # a model that returns one tensor exports as a one-element tuple plus an output spec: undo that
+    out = next(n for n in graph.nodes if n.op == "output")
+    spec = getattr(gm, "_out_spec", None)
+    if spec is not None and spec.num_leaves == 1 and spec.num_nodes == 1 and isinstance(out.args[0], (tuple, list)):
+        out.args = (out.args[0][0],)
+    graph.lint()
+    return gm, graph
 
 
 @dataclass
@@ -209,6 +267,8 @@ class Pipe(nn.Module):
         # a parameter may live in one stage only (reference ``_IR.py:871-879``)
         owner: Dict[int, str] = {}
         for name, sub in split.named_children():
+            if not name.startswith("submod_"):
+                continue
             for pn, p in sub.named_parameters():
                 if id(p) in owner and owner[id(p)] != name:
                     raise NotImplementedError(
@@ -228,13 +288,32 @@ class Pipe(nn.Module):
         split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks, args_chunk_spec,
                                       kwargs_chunk_spec)
         names = list(split_spec.keys()) if split_spec else None
-        graph = _ModuleGranularityTracer(names).trace(mod)
-        if split_spec:
-            _insert_markers(graph, split_spec)
+        root = mod
+        try:
+            graph = _ModuleGranularityTracer(names).trace(mod)
+            if split_spec:
+                _insert_markers(graph, split_spec)
+        except Exception as fx_error:
+            # symbolic tracing cannot follow this model: export it on the first microbatch's inputs, as
+            # the reference does (``_IR.py:1172-1185``); the stages are then ATen-level graphs
+            logger.warning(f"torch.fx symbolic tracing failed ({type(fx_error).__name__}: {fx_error}); "
+                           "falling back to torch.export: the stages are ATen-level graphs and run through "
+                           "torch autograd, not as HIP launch lists")
+            args_split, kwargs_split = split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks,
+                                                                     args_chunk_spec, kwargs_chunk_spec)
+            try:
+                root, graph = _export_and_mark(mod, args_split[0], kwargs_split[0], split_spec)
+            except ValueError:
+                raise
+            except Exception as export_error:
+                raise RuntimeError(
+                    f"pipeline(): neither torch.fx symbolic tracing ({type(fx_error).__name__}: {fx_error}) "
+                    f"nor torch.export ({type(export_error).__name__}: {export_error}) can trace this model"
+                ) from export_error
         if split_policy is not None:
-            gm = split_policy(fx.GraphModule(mod, graph))
+            gm = split_policy(fx.GraphModule(root, graph))
             graph = gm.graph
-        pipe = Pipe._from_traced(mod, graph)
+        pipe = Pipe._from_traced(root, graph)
         pipe.pipe_info = PipeInfo(graph=pipe.split_gm.graph, num_stages=pipe.num_stages,
                                   num_chunks=num_chunks, has_loss_and_backward=False,
                                   args_chunk_spec=args_chunk_spec, kwargs_chunk_spec=kwargs_chunk_spec)

@@ -1,0 +1,114 @@
+"""The ``torch.export`` route of the front end (reference ``pippy/_IR.py:1141-1145,679-1125``): a model
+that ``torch.fx`` symbolic tracing cannot follow is exported on the inputs of one microbatch and cut at
+the markers.  Checked with the invariants of the reference's ``test/test_pipe.py:78-110`` (stage count,
+``Pipe(x) == mod(x)``, the stages' state-dict keys partition the model's) and, end to end on the host,
+with those of ``test/test_fwd.py:80-84`` / ``test/test_grad.py:103-136`` (pipelined output and gradients
+equal the un-pipelined model's)."""
+import copy
+
+import pytest
+import torch
+import torch.fx as fx
+import torch.nn as nn
+
+import pippy_amd as pp
+
+
+class _Block(nn.Module):
+    def __init__(self, d):
+        super().__init__()
+        self.lin = nn.Linear(d, d)
+        self.ln = nn.LayerNorm(d)
+
+    def forward(self, x):
+        h = self.lin(x)
+        if h.shape[-1] > 4:      # Python control flow on a shape: symbolic tracing stops here
+            h = torch.relu(h)
+        return self.ln(h) + x
+
+
+class _Model(nn.Module):
+    def __init__(self, d=8, marker_at=None):
+        super().__init__()
+        self.scale = nn.Parameter(torch.rand(d) + 0.5)
+        self.marker_at = marker_at
+        self.layers = nn.ModuleList([_Block(d) for _ in range(4)])
+        self.head = nn.Linear(d, 3)
+
+    def forward(self, x):
+        x = x * self.scale
+        for i, layer in enumerate(self.layers):
+            if self.marker_at == i:
+                pp.pipe_split()
+            x = layer(x)
+        return self.head(x)
+
+
+def _check_partition(pipe, model):
+    keys = []
+    for i in range(pipe.num_stages):
+        stage_mod = pipe.get_stage_module(i)
+        keys += list(stage_mod.state_dict().keys())
+        for name, p in stage_mod.named_parameters():
+            assert p is model.get_parameter(name), f"{name} is not the model's own parameter"
+    assert sorted(keys) == sorted(model.state_dict().keys())
+
+
+def test_symbolic_tracing_really_fails_on_this_model():
+    with pytest.raises(Exception):
+        fx.symbolic_trace(_Model())
+
+
+@pytest.mark.parametrize("spec,marker_at,n_stages", [
+    ({"layers.1": pp.SplitPoint.BEGINNING, "layers.2": pp.SplitPoint.END}, None, 3),
+    (None, 2, 2),
+    ({"layers.3": pp.SplitPoint.BEGINNING}, 1, 3),
+])
+def test_export_fallback_keeps_names_and_results(spec, marker_at, n_stages):
+    torch.manual_seed(0)
+    model = _Model(marker_at=marker_at)
+    x = torch.randn(8, 8)
+    pipe = pp.pipeline(model, 4, (x,), split_spec=spec)
+    assert pipe.num_stages == n_stages
+    _check_partition(pipe, model)
+    assert torch.equal(pipe(x), model(x))
+    # the marker does nothing when the model simply runs
+    assert model(x).shape == (8, 3)
+
+
+def test_export_fallback_pipeline_trains_like_the_unsplit_model():
+    torch.manual_seed(1)
+    model = _Model()
+    ref = copy.deepcopy(model)
+    x, target = torch.randn(8, 8), torch.randn(8, 3)
+    pipe = pp.pipeline(model, 4, (x,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, "cpu") for i in range(pipe.num_stages)]
+    assert not any(st.is_native for st in stages)
+    loss_fn = nn.MSELoss(reduction="sum")
+    for cls in (pp.ScheduleGPipe, pp.Schedule1F1B):
+        for p in model.parameters():
+            p.grad = None
+        losses = []
+        # the microbatch lists are handed over directly: merging host tensors is not something this
+        # package does (its merge is a device kernel), so the chunks are compared after a torch.cat
+        for st in stages:
+            st.clear_runtime_states()
+        cls(stages, 4, loss_fn=loss_fn)._step_microbatches([(c,) for c in x.chunk(4)], None,
+                                                           list(target.chunk(4)), losses)
+        out = torch.cat(stages[-1].output_chunks)
+        for p in ref.parameters():
+            p.grad = None
+        ref_out = ref(x)
+        ref_loss = loss_fn(ref_out, target)
+        ref_loss.backward()
+        torch.testing.assert_close(out, ref_out)
+        torch.testing.assert_close(sum(losses), ref_loss)
+        for (n, p), (_, rp) in zip(model.named_parameters(), ref.named_parameters()):
+            # microbatch sums against one full-batch sum: fp32 rounding only (the reference's own
+            # backward test allows rtol 1e-2 / atol 5e-3, test/test_bwd.py:98)
+            torch.testing.assert_close(p.grad, rp.grad, rtol=1e-4, atol=1e-4, msg=lambda m, n=n: f"{n}: {m}")
+
+
+def test_split_point_that_is_not_in_the_model_raises_on_the_export_route_too():
+    with pytest.raises(ValueError, match="not a module called by the model"):
+        pp.pipeline(_Model(), 2, (torch.randn(4, 8),), split_spec={"nowhere": pp.SplitPoint.BEGINNING})
