@@ -137,26 +137,24 @@ extern __shared__ __attribute__((aligned(16))) uint16_t attn_lds[];
 // mask block `ord` of the query-parallel kernels is query block nx - 1 - ord (it sees the most keys), of
 // the key-parallel kernel key block ord (it is seen by the most queries).
 //
-// A causal launch is bound by how the unequal blocks meet on a CU: with three resident work-groups
-// per CU and work-groups handed to the 32 CUs of an XCD in turn, CU c holds the work-groups c, c + 32
-// and c + 64 of its XCD; numbered head by head these are three blocks of the same length, so one CU
-// gets three longest blocks and another three shortest.  Here the blocks of an XCD are ranked by
-// length (all heads' longest first) and dealt out in rounds of 32 that alternate in direction, so
-// every CU's blocks add up to about the same length, and work-groups that start later (when more
-// exist than fit at once) are the short ones.  The assignment is a permutation of the same work, so
-// results do not depend on it.
-constexpr uint32_t kCusPerXcd = 32;
+// A causal launch is bound by how its unequal blocks meet on the CUs.  Numbered head by head, the
+// work-groups that arrive on an XCD one after the other repeat the same ramp of lengths for every head,
+// and the CUs end up with very unequal sums (measured: as slow as the launch without a mask, which
+// does twice the work).  Here the blocks of an XCD are ranked by length across its heads, every head's
+// longest first, so that the work-groups which share a CU at any time are of about one length and the
+// late arrivals are the short ones: 24.7 -> 18.9 us forward and 62.8 -> 49.3 us backward at
+// [4, 12, 1024, 64].  (Dealing the ranked blocks to the CUs in rounds of alternating direction measured
+// the same for every round length from 8 to 96; fewer resident work-groups per CU, which lets the
+// dispatcher place the short blocks as slots free up, measured slower.)  The assignment is a
+// permutation of the same work, so results do not depend on it.
 __device__ __forceinline__ bool attn_block_of(uint32_t bid, uint32_t grid, uint32_t nx, uint32_t heads,
                                               bool balance, uint32_t* bh, uint32_t* ord) {
     if (balance && heads % 8 == 0) {
         const uint32_t x = bid & 7, t = bid >> 3;      // XCD, arrival order inside it
-        const uint32_t g = heads / 8, per = nx * g;    // heads and work-groups per XCD
-        if (t >= per) return false;
-        const uint32_t r = t / kCusPerXcd, p = t % kCusPerXcd;
-        const bool whole_round = (r + 1) * kCusPerXcd <= per;
-        const uint32_t k = r * kCusPerXcd + (((r & 1) && whole_round) ? kCusPerXcd - 1 - p : p);
-        *bh = x * g + k % g;
-        *ord = k / g;
+        const uint32_t g = heads / 8;                  // heads per XCD
+        if (t >= nx * g) return false;
+        *bh = x * g + t % g;
+        *ord = t / g;
         return true;
     }
     const uint32_t vid = xcd_remap(bid, grid);
