@@ -15,9 +15,11 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .stage_modules import LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence
+from .stage_modules import (LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence,
+                            WrappedLMHead, WrappedTokenEmbedding, WrappedTransformerLayer)
 
-_LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout)
+_LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout,
+               nn.Embedding)
 
 
 class _ChainTracer(fx.Tracer):
@@ -135,7 +137,13 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
             raise NotLowerable("the stage holds no layer")
         return out
     if isinstance(submod, fx.GraphModule):
-        return blocks_from_graph(submod, submod.graph)
+        try:
+            return blocks_from_graph(submod, submod.graph)
+        except NotLowerable as chain_reason:
+            try:
+                return blocks_from_residual_graph(submod)
+            except NotLowerable as residual_reason:
+                raise NotLowerable(f"{chain_reason}; as a residual transformer stack: {residual_reason}") from None
     if isinstance(submod, (nn.Linear, nn.LayerNorm, nn.RMSNorm)):
         # a stage that is one standard layer: the same rules as for that layer inside a chain
         holder = nn.Module()
@@ -147,7 +155,232 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
         graph = _ChainTracer().trace(submod)
     except Exception as e:
         raise NotLowerable(f"torch.fx cannot trace {type(submod).__name__}: {type(e).__name__}: {e}") from e
-    return blocks_from_graph(submod, graph)
+    try:
+        return blocks_from_graph(submod, graph)
+    except NotLowerable as chain_reason:
+        # not a chain of layers: maybe a transformer written with plain torch layers
+        try:
+            return blocks_from_residual_graph(submod)
+        except NotLowerable as residual_reason:
+            raise NotLowerable(f"{chain_reason}; as a residual transformer stack: {residual_reason}") from None
+
+
+# ---- transformers written with plain torch layers ---------------------------------------------------
+# Recognised, in this order along the stage: an optional embedding front (token table, optionally plus
+# a position table indexed by arange), any number of pre-LayerNorm residual pairs
+#     x = x + proj(scaled_dot_product_attention(split(qkv(ln(x)))))      x = x + fc2(gelu(fc1(ln(x))))
+# and an optional tail of a final LayerNorm and a bias-free vocabulary projection.  The walk only looks
+# at which layers feed which residual add; how the model reshapes between them is not parsed but
+# checked: the torch statement of the recognised blocks must reproduce the stage's own forward on a
+# random input (fp32, on the host), otherwise the stage stays with torch autograd.
+_SDPA = F.scaled_dot_product_attention
+_ADD_FNS = (operator.add, operator.iadd, torch.add)
+
+
+def _is_add(n: fx.Node) -> bool:
+    return (n.op == "call_function" and n.target in _ADD_FNS) or (n.op == "call_method" and n.target in ("add", "add_"))
+
+
+def _branch_layers(y: fx.Node, stream: fx.Node, order: dict) -> List[fx.Node]:
+    """The layer and function nodes that ``y`` is computed from, back to ``stream`` (in graph order)."""
+    seen, stack, found = set(), [y], []
+    while stack:
+        n = stack.pop()
+        if n in seen or n is stream:
+            continue
+        seen.add(n)
+        if n.op == "placeholder":
+            continue
+        if n.op == "call_module" or (n.op == "call_function" and n.target in (_SDPA, F.gelu, F.relu, torch.relu)) \
+                or _is_add(n):
+            found.append(n)
+        stack.extend(a for a in n.all_input_nodes)
+    return sorted(found, key=order.get)
+
+
+def _classify_branch(root: nn.Module, layers: List[fx.Node]):
+    """("attn", ln, qkv, proj, causal) or ("mlp", ln, fc1, fc2, activation) for a residual branch."""
+    mods = []
+    for n in layers:
+        if n.op == "call_module":
+            m = root.get_submodule(n.target)
+            if _activation_of(n, root) == "identity":
+                continue
+            mods.append((n, m))
+        elif _is_add(n):
+            raise NotLowerable(f"an addition inside a residual branch ('{n.format_node()}')")
+        else:
+            mods.append((n, None))
+    kinds = [type(m).__name__ if m is not None else ("sdpa" if n.target is _SDPA else "act") for n, m in mods]
+    if kinds == ["LayerNorm", "Linear", "sdpa", "Linear"]:
+        (_, ln), (_, qkv), (sd, _), (_, proj) = mods
+        if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
+            raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection of width 3 d")
+        kw = dict(sd.kwargs)
+        extra = sd.args[3:]
+        if kw.get("attn_mask") is not None or kw.get("dropout_p", 0.0) not in (0, 0.0) or kw.get("scale") is not None \
+                or kw.get("enable_gqa") or any(a is not None and a != 0.0 and a is not False for a in extra[:2]):
+            raise NotLowerable("scaled_dot_product_attention with a mask tensor, dropout, a custom scale or grouped "
+                               "queries")
+        causal = bool(kw.get("is_causal", extra[2] if len(extra) > 2 else False))
+        return ("attn", ln, qkv, proj, causal)
+    if len(kinds) == 4 and kinds[0] == "LayerNorm" and kinds[1] == "Linear" and kinds[3] == "Linear":
+        (_, ln), (_, fc1), (an, am), (_, fc2) = mods
+        act = _activation_of(an, root)
+        if act not in ("gelu_tanh", "gelu_erf"):
+            raise NotLowerable(f"feed-forward activation '{an.format_node()}' (tanh- and erf-GELU are built)")
+        if fc2.in_features != fc1.out_features or fc2.out_features != fc1.in_features:
+            raise NotLowerable("feed-forward projections do not map d -> f -> d")
+        return ("mlp", ln, fc1, fc2, act)
+    raise NotLowerable(f"a residual branch made of {kinds}")
+
+
+def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[NativeBlock]:
+    nodes = list(graph.nodes)
+    order = {n: i for i, n in enumerate(nodes)}
+    placeholders = [n for n in nodes if n.op == "placeholder"]
+    if len(placeholders) != 1:
+        raise NotLowerable(f"the stage takes {len(placeholders)} inputs; a launch-list stage takes one tensor")
+    out_node = next(n for n in nodes if n.op == "output")
+    result = out_node.args[0]
+    if isinstance(result, (tuple, list)):
+        if len(result) != 1:
+            raise NotLowerable("the stage returns several values")
+        result = result[0]
+    stream = placeholders[0]
+    blocks: List[NativeBlock] = []
+    # embedding front: the first addition of two embedding look-ups, or a lone token table
+    emb = [n for n in nodes if n.op == "call_module" and isinstance(root.get_submodule(n.target), nn.Embedding)]
+    if emb:
+        if len(emb) > 2 or emb[0].all_input_nodes != [stream]:
+            raise NotLowerable("embedding tables other than one token table (and one position table)")
+        wte = root.get_submodule(emb[0].target)
+        if len(emb) == 2:
+            joins = [n for n in nodes if _is_add(n) and set(_branch_layers(n, stream, order)) == {emb[0], emb[1], n}]
+            if not joins:
+                raise NotLowerable("token and position embeddings are not simply added")
+            stream = joins[0]
+            blocks.append(WrappedTokenEmbedding(wte, root.get_submodule(emb[1].target)))
+        else:
+            stream = emb[0]
+            blocks.append(WrappedTokenEmbedding(wte, None))
+        while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
+            stream = next(iter(stream.users))   # dropout that does nothing
+    # residual pairs
+    pending = None
+    while True:
+        adds = [u for u in stream.users if _is_add(u)]
+        if len(adds) != 1:
+            break
+        add = adds[0]
+        other = [a for a in add.all_input_nodes if a is not stream]
+        if len(other) != 1:
+            break
+        kind = _classify_branch(root, [n for n in _branch_layers(other[0], stream, order)])
+        if kind[0] == "attn":
+            if pending is not None:
+                raise NotLowerable("two attention branches in a row")
+            pending = kind
+        else:
+            if pending is None:
+                raise NotLowerable("a feed-forward branch without an attention branch before it")
+            _, ln1, qkv, proj, causal = pending
+            _, ln2, fc1, fc2, act = kind
+            d = qkv.in_features
+            if d % n_heads or d // n_heads not in (64, 128):
+                raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
+            blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
+            pending = None
+        stream = add
+        while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
+            stream = next(iter(stream.users))
+    if pending is not None:
+        raise NotLowerable("an attention branch without its feed-forward branch in the same stage")
+    # tail: what is left must be a chain of layers
+    tail = []
+    cur = stream
+    while cur is not result:
+        users = [u for u in cur.users]
+        if len(users) != 1:
+            raise NotLowerable(f"'{cur.format_node()}' feeds {len(users)} nodes after the last residual addition")
+        cur = users[0]
+        if cur.op == "output":
+            break
+        tail.append(cur)
+    tail_mods = []
+    for n in tail:
+        if _activation_of(n, root) == "identity":
+            continue
+        if n.op != "call_module":
+            raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
+        tail_mods.append(root.get_submodule(n.target))
+    kinds = [type(m).__name__ for m in tail_mods]
+    if kinds == ["LayerNorm", "Linear"] and tail_mods[1].bias is None:
+        blocks.append(WrappedLMHead(tail_mods[0], tail_mods[1]))
+    elif kinds == ["Linear"] and tail_mods[0].bias is None and blocks:
+        blocks.append(WrappedLMHead(None, tail_mods[0]))
+    else:
+        for m in tail_mods:
+            if isinstance(m, nn.LayerNorm):
+                blocks.append(LayerNormBlock(m))
+            elif isinstance(m, nn.Linear):
+                blocks.append(LinearAct(m, None))
+            else:
+                raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
+    if not any(isinstance(b, WrappedTransformerLayer) for b in blocks):
+        raise NotLowerable("no attention / feed-forward residual pair found")
+    return blocks
+
+
+def _example_input(blocks: List[NativeBlock]) -> torch.Tensor:
+    g = torch.Generator().manual_seed(0)
+    first = blocks[0]
+    if isinstance(first, WrappedTokenEmbedding):
+        seq = 16 if first.wpe is None else min(16, first.wpe.num_embeddings)
+        return torch.randint(0, first.wte.num_embeddings, (2, seq), generator=g)
+    d = next(b for b in blocks if isinstance(b, WrappedTransformerLayer)).dim
+    return torch.randn(2, 16, d, generator=g)
+
+
+def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
+    """Blocks of a stage that is a stack of plain-torch transformer layers, verified numerically."""
+    import copy
+    try:
+        graph = _ChainTracer().trace(submod)
+    except Exception as e:
+        raise NotLowerable(f"torch.fx cannot trace {type(submod).__name__}: {type(e).__name__}: {e}") from e
+    widths = {m.normalized_shape[0] for m in submod.modules()
+              if isinstance(m, nn.LayerNorm) and len(m.normalized_shape) == 1}
+    if len(widths) != 1:
+        raise NotLowerable("no single model width (the LayerNorms of the stage disagree)")
+    d = widths.pop()
+    candidates = [h for h in (d // 64, d // 128) if h >= 1 and d % h == 0]
+    if not candidates:
+        raise NotLowerable(f"model width {d} allows no head dimension of 64 or 128")
+    _residual_blocks(submod, graph, candidates[0])   # raises unless the structure is recognised
+    # the structure fits; which head count (if any) reproduces the stage is decided on an fp32 copy
+    try:
+        probe = copy.deepcopy(submod).float().cpu().eval()
+    except Exception as e:
+        raise NotLowerable(f"the stage module cannot be copied for verification: {e}") from e
+    probe_graph = _ChainTracer().trace(probe)
+    reasons = []
+    for n_heads in candidates:
+        trial = _residual_blocks(probe, probe_graph, n_heads)
+        x = _example_input(trial)
+        with torch.no_grad():
+            want = probe(x)
+            got = x
+            for blk in trial:
+                got = blk(got)
+        if isinstance(want, (tuple, list)):
+            want = want[0]
+        err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30) if got.shape == want.shape else 1.0
+        if err <= 1e-4:
+            return _residual_blocks(submod, graph, n_heads)
+        reasons.append(f"with {n_heads} heads the recognised blocks differ from the stage's own forward "
+                       f"(relative error {err:.2e})")
+    raise NotLowerable("; ".join(reasons))
 
 
 def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None) -> Optional[List[NativeBlock]]:

@@ -38,7 +38,7 @@ def _round_up(x: int, m: int) -> int:
 class ParamArena:
     """Flat storage of one stage's parameters, gradient staging and fp32 accumulators."""
 
-    def __init__(self, module: nn.Module, device: torch.device):
+    def __init__(self, module: nn.Module, device: torch.device, blocks: Sequence[nn.Module] = ()):
         params = [(n, p) for n, p in module.named_parameters()]
         if not params:
             self.dtype = torch.bfloat16
@@ -51,7 +51,11 @@ class ParamArena:
             raise RuntimeError(f"native stages support bf16 or fp32 parameters, not {self.dtype}")
         pad_rows: Dict[int, int] = {}
         direct = set()
-        for mod in module.modules():
+        # the blocks may be wrappers around the module's layers that are not part of the module itself
+        holders = {id(m): m for m in module.modules()}
+        for blk in blocks:
+            holders.update({id(m): m for m in blk.modules()})
+        for mod in holders.values():
             for p, rows in getattr(mod, "_pp_padded_rows", lambda: [])():
                 pad_rows[id(p)] = rows
             for p in getattr(mod, "_pp_direct_acc_params", lambda: [])():
@@ -670,7 +674,7 @@ class StageProgram:
         self.epilogue_accumulated = set()  # ids of the parameters whose GEMM epilogue accumulates
         self.is_first = is_first
         self.is_last = is_last
-        self.arena = ParamArena(module, device)
+        self.arena = ParamArena(module, device, self.blocks)
         self.act_dtype = self.arena.dtype
         self._shared: Dict[str, torch.Tensor] = {}
         self.mbs: Dict[int, MicrobatchProgram] = {}

@@ -787,6 +787,38 @@ class LMHead(NativeBlock):
         return out
 
 
+# ---- the same blocks around layers that a user's model already owns ---------------------------------
+# A model written with plain torch layers (``nn.Embedding``, ``nn.LayerNorm``, ``nn.Linear``,
+# ``F.scaled_dot_product_attention``, residual adds) is lowered by recognising these groupings in its
+# graph and wrapping the user's own layer objects: no parameter is copied or renamed.
+class WrappedTokenEmbedding(TokenEmbedding):
+    def __init__(self, wte: nn.Embedding, wpe: Optional[nn.Embedding]):
+        NativeBlock.__init__(self)
+        self.wte = wte
+        self.wpe = wpe
+
+
+class WrappedTransformerLayer(TransformerLayer):
+    def __init__(self, ln_1: nn.LayerNorm, c_attn: nn.Linear, c_proj: nn.Linear, ln_2: nn.LayerNorm,
+                 c_fc: nn.Linear, mlp_proj: nn.Linear, n_heads: int, causal: bool, activation: str):
+        NativeBlock.__init__(self)
+        self.dim, self.n_heads, self.ffn = c_proj.out_features, n_heads, c_fc.out_features
+        self.causal, self.pre_ln, self.activation = causal, True, activation
+        self.ln_1, self.ln_2 = ln_1, ln_2
+        self.attn = nn.Module()
+        self.attn.c_attn, self.attn.c_proj = c_attn, c_proj
+        self.mlp = nn.Module()
+        self.mlp.c_fc, self.mlp.c_proj = c_fc, mlp_proj
+
+
+class WrappedLMHead(LMHead):
+    def __init__(self, ln_f: Optional[nn.Module], lm_head: nn.Linear):
+        NativeBlock.__init__(self)
+        self.dim, self.vocab = lm_head.in_features, lm_head.out_features
+        self.ln_f = ln_f
+        self.lm_head = lm_head
+
+
 class StageSequence(nn.Module):
     """A stage module that applies its children in order.  Children keep the names they had in the
     un-split model (``add_block("transformer.h.3", layer)`` registers nested containers), so a

@@ -500,3 +500,41 @@ def test_a_stage_that_cannot_be_lowered_says_why(caplog):
     assert lower_stage_module(nn.Linear(4, 2), why) and not why
     host = ManualPipelineStage(nn.Linear(4, 2), 0, 1, "cpu", 1)
     assert not host.is_native and "GPU only" in host.eager_reason
+
+
+# ---- a transformer written with plain torch layers lowers to the same blocks --------------------------
+def test_plain_torch_transformer_is_recognised_and_verified():
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import GPT, Block
+    from pippy_amd._lowering import lower_stage_module
+    torch.manual_seed(0)
+    model = GPT(vocab=500, seq=64, d=128, h=2, L=4)
+    why = []
+    blocks = lower_stage_module(model, why)
+    assert [type(b).__name__ for b in blocks] == ["WrappedTokenEmbedding"] + ["WrappedTransformerLayer"] * 4 + ["WrappedLMHead"]
+    # the wrappers hold the model's own layers: nothing is copied or renamed
+    assert blocks[1].attn.c_attn is model.h[0].c_attn and blocks[-1].lm_head is model.lm_head
+    assert blocks[1].n_heads == 2 and blocks[1].causal and blocks[1].activation == "gelu_tanh"
+    # stages cut by the front end lower too, with the model's parameter names
+    ids = torch.randint(0, 500, (4, 64))
+    pipe = pp.pipeline(model, 2, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    kinds = [[type(b).__name__ for b in lower_stage_module(pipe.get_stage_module(i))] for i in range(2)]
+    assert kinds == [["WrappedTokenEmbedding"] + ["WrappedTransformerLayer"] * 2,
+                     ["WrappedTransformerLayer"] * 2 + ["WrappedLMHead"]]
+    assert "h.2.c_attn.weight" in pipe.get_stage_module(1).state_dict()
+
+    # a model whose heads are not what the kernels are built for stays with torch, and says why
+    why = []
+    assert lower_stage_module(GPT(d=96, h=3), why) is None and "head dimension" in why[0]
+
+    # a block that computes something else between the same layers fails the numerical check
+    class Scaled(Block):
+        def forward(self, x):
+            return super().forward(x) * 1.5
+
+    odd = GPT(vocab=500, seq=64, d=128, h=2, L=1)
+    odd.h[0] = Scaled(128, 2)
+    why = []
+    assert lower_stage_module(odd, why) is None
+    assert "residual" in why[0]

@@ -855,3 +855,58 @@ def test_skip_connection_forward_and_backward_match_the_unsplit_model(schedule):
         g = named[name].grad
         assert g is not None, name
         torch.testing.assert_close(g, rp.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_plain_torch_gpt_runs_natively_and_matches_the_oracle():
+    """A GPT-2-shaped model written without any block of this package (nn.Embedding, nn.LayerNorm,
+    nn.Linear, F.scaled_dot_product_attention, residual adds; the kind of model the reference is handed,
+    examples/huggingface/pippy_gpt2.py:50-65): both stages must run as launch lists, and logits, losses and
+    every parameter gradient must match the fp32 oracle run of the same model."""
+    import sys, os
+    import torch.nn as nn
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import GPT
+    import pippy_amd as pp
+    torch.manual_seed(0)
+    M, vocab, seq = 4, 1000, 128
+    model = GPT(vocab=vocab, seq=seq, d=128, h=2, L=4).to(torch.bfloat16)
+    ref = copy.deepcopy(model).float()
+    ids = torch.randint(0, vocab, (2 * M, seq))
+    target = torch.randint(0, vocab, (2 * M, seq))
+    pipe = pp.pipeline(model, M, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert all(st.is_native for st in stages), [st.eager_reason for st in stages]
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    losses = []
+    out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    torch.cuda.synchronize()
+
+    class Front(nn.Module):
+        def __init__(self, g):
+            super().__init__()
+            self.g = g
+
+        def forward(self, idx):
+            x = self.g.wte(idx) + self.g.wpe(torch.arange(idx.shape[1]))
+            for blk in self.g.h[:2]:
+                x = blk(x)
+            return x
+
+    class Back(nn.Module):
+        def __init__(self, g):
+            super().__init__()
+            self.g = g
+
+        def forward(self, x):
+            for blk in self.g.h[2:]:
+                x = blk(x)
+            return self.g.lm_head(self.g.ln_f(x))
+
+    ref_out, ref_losses = OP.step([Front(ref), Back(ref)], ids, target, M, _ce)
+    assert_close_rel(out, ref_out, BF16_TOL, "merged logits")
+    for m in range(M):
+        assert_close_rel(losses[m].reshape(1), ref_losses[m].reshape(1), BF16_TOL, f"loss {m}")
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        err = max_rel(named[name].main_grad, rp.grad)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
