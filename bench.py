@@ -294,12 +294,17 @@ def main():
         ms, work, cnt = N.profile_read(N.OP_GEMM_BF16)
         sms_, swork, scnt = N.profile_read(N.OP_GEMM_SEG)   # expert GEMMs of a mixture-of-experts layer
         ms, work, cnt = ms + sms_, work + swork, cnt + scnt
+        gcnt = 0
+        for kind in (N.OP_GEMM_SWIGLU, N.OP_GEMM_DSWIGLU):   # feed-forward GEMMs with SwiGLU in the epilogue
+            kms, kwork, kcnt = N.profile_read(kind)
+            ms, work, cnt, gcnt = ms + kms, work + kwork, cnt + kcnt, gcnt + kcnt
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
                               "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
                               "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
-                                        + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else ""),
+                                        + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else "")
+                                        + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else ""),
                               "launches_per_step": cnt // n_prof,
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
                               "gemm_ms_per_step": round(ms / n_prof, 3)}

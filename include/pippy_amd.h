@@ -236,6 +236,26 @@ int pp_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* 
 int pp_rope(void* x, const float* cos_table, const float* sin_table, int64_t n_tok, int64_t seq,
             int64_t n_heads, int64_t D, int64_t ld, int inverse, pp_stream stream);
 
+/* SwiGLU fused into the GEMMs on either side of it (the feed-forward of a Llama-style layer inside
+ * the stage module: forward through pippy/_PipelineStage.py:420-428, backward through
+ * pippy/_backward.py:67-69).  All operands bf16, k-contiguous; x, the weights 16-byte aligned with
+ * K, ldx, ldw multiples of 8; N a multiple of 8; gu, h, dgu 8-byte aligned with leading dimensions
+ * that are multiples of 4.
+ *   pp_gemm_bf16_swiglu:  g = x w_gate^T, u = x w_up^T (x [M, K], w_gate and w_up [N, K] with the same
+ *     ldw), both rounded to bf16 and stored side by side in gu [M, 2 N] (g in columns [0, N), u in
+ *     [N, 2 N)), and h [M, N] = silu(g) * u from the rounded values: the bits of two pp_gemm_bf16 calls
+ *     followed by pp_swiglu_fwd.
+ *   pp_gemm_bf16_dswiglu: dh = dy w_down_t^T (dy [M, K], w_down_t [N, K] the transposed down
+ *     projection) is rounded to bf16 and never stored; dgu [M, 2 N] receives dg = dh u silu'(g) in
+ *     columns [0, N) and du = dh silu(g) in [N, 2 N), g and u read from gu: the bits of pp_gemm_bf16
+ *     followed by pp_swiglu_bwd. */
+int pp_gemm_bf16_swiglu(const void* x, const void* w_gate, const void* w_up, void* gu, void* h, int64_t M,
+                        int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ld_gu, int64_t ldh,
+                        pp_stream stream);
+int pp_gemm_bf16_dswiglu(const void* dy, const void* w_down_t, const void* gu, void* dgu, int64_t M,
+                         int64_t N, int64_t K, int64_t ldy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu,
+                         pp_stream stream);
+
 /* ------------------------------------------------------------------------------------------
  * Routing of a top-2 mixture-of-experts layer (a Mixtral-style block inside the stage module;
  * forward through pippy/_PipelineStage.py:420-428, backward through pippy/_backward.py:67-69).
@@ -371,7 +391,7 @@ enum pp_op_kind {
     PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16,
     PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
     PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
-    PP_OP_MOE_GATE_BWD = 25
+    PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -400,6 +420,8 @@ enum pp_op_kind {
  *   MOE_GATHER    p: src row_src n_rows_dev scale dst | i: ld_src topk ld_dst R C
  *   MOE_COMBINE   p: y pos gate resid out | i: ld_y topk ld_resid ld_out T C
  *   MOE_GATE_BWD  p: dout y pos topk_idx gate dlogits | i: ld_dout ld_y topk E ld_dl T C
+ *   GEMM_SWIGLU   p: x w_gate w_up gu h | i: M N K ldx ldw ld_gu ldh
+ *   GEMM_DSWIGLU  p: dy w_down_t gu dgu | i: M N K ldy ldw ld_gu ld_dgu
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped

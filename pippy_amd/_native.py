@@ -26,7 +26,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
- OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD) = range(1, 26)
+ OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU) = range(1, 28)
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
@@ -43,7 +43,7 @@ EXPORTED_SYMBOLS = (
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
-    "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc",
+    "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc", "pp_gemm_bf16_swiglu", "pp_gemm_bf16_dswiglu",
 )
 
 
@@ -136,6 +136,8 @@ def lib() -> C.CDLL:
         "pp_swiglu_fwd": [vp, vp, vp, i64, vp],
         "pp_swiglu_bwd": [vp, vp, vp, vp, vp, i64, vp],
         "pp_rope": [vp, vp, vp, i64, i64, i64, i64, i64, i32, vp],
+        "pp_gemm_bf16_swiglu": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
+        "pp_gemm_bf16_dswiglu": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
         "pp_gemm_bf16_segmented": [C.POINTER(GemmDesc), vp, vp, i32, i32, vp],
         "pp_moe_router_top2": [vp, i64, i64, i32, vp, vp, vp],
         "pp_moe_permute": [vp, i64, i32, vp, vp, vp, vp],
@@ -298,6 +300,31 @@ def swiglu_bwd(g, u, dh, dg, du) -> None:
         assert t.is_contiguous() and t.numel() == g.numel()
     check(lib().pp_swiglu_bwd(g.data_ptr(), u.data_ptr(), dh.data_ptr(), dg.data_ptr(), du.data_ptr(), g.numel(),
                               current_stream()), "pp_swiglu_bwd")
+
+
+def gemm_swiglu(x, w_gate, w_up, gu, h) -> None:
+    """gu [M, 2 N] = [x w_gate^T | x w_up^T] (bf16) and h [M, N] = silu(gate) * up, in one kernel."""
+    require_cuda(x, w_gate, w_up, gu, h)
+    M, K = x.shape
+    Nn = w_gate.shape[0]
+    assert w_gate.shape == w_up.shape == (Nn, K) and gu.shape == (M, 2 * Nn) and h.shape == (M, Nn)
+    assert x.stride(1) == w_gate.stride(1) == w_up.stride(1) == gu.stride(1) == h.stride(1) == 1
+    assert w_gate.stride(0) == w_up.stride(0)
+    check(lib().pp_gemm_bf16_swiglu(x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), gu.data_ptr(), h.data_ptr(),
+                                    M, Nn, K, x.stride(0), w_gate.stride(0), gu.stride(0), h.stride(0),
+                                    current_stream()), "pp_gemm_bf16_swiglu")
+
+
+def gemm_dswiglu(dy, w_down_t, gu, dgu) -> None:
+    """dgu [M, 2 N] = [dg | du] from dh = dy w_down_t^T (never stored) and the saved gu = [g | u]."""
+    require_cuda(dy, w_down_t, gu, dgu)
+    M, K = dy.shape
+    Nn = w_down_t.shape[0]
+    assert w_down_t.shape == (Nn, K) and gu.shape == dgu.shape == (M, 2 * Nn)
+    assert dy.stride(1) == w_down_t.stride(1) == gu.stride(1) == dgu.stride(1) == 1
+    check(lib().pp_gemm_bf16_dswiglu(dy.data_ptr(), w_down_t.data_ptr(), gu.data_ptr(), dgu.data_ptr(), M, Nn, K,
+                                     dy.stride(0), w_down_t.stride(0), gu.stride(0), dgu.stride(0),
+                                     current_stream()), "pp_gemm_bf16_dswiglu")
 
 
 def rope(x2d, cos, sin, seq: int, n_heads: int, D: int, inverse: bool = False) -> None:

@@ -113,16 +113,35 @@ class ParamArena:
             self._transposed[id(p)] = ent
         return ent[1]
 
+    def weight_t_cat(self, p1: nn.Parameter, p2: nn.Parameter) -> torch.Tensor:
+        """[in, out1 + out2]: the transposed copies of two weights with the same input width side by
+        side, so that dY1 W1 + dY2 W2 is ONE product of [dY1 | dY2] with this matrix.  Kept in step
+        with both parameters by ``refresh_transposed``."""
+        key = ("cat", id(p1), id(p2))
+        ent = self._transposed.get(key)
+        if ent is None:
+            w1, w2 = self.weight(p1, padded=True), self.weight(p2, padded=True)
+            assert w1.shape[1] == w2.shape[1]
+            t = torch.empty((w1.shape[1], w1.shape[0] + w2.shape[0]), dtype=w1.dtype, device=self.device)
+            for k, (p, lo, hi) in enumerate(((p1, 0, w1.shape[0]), (p2, w1.shape[0], t.shape[1]))):
+                view = t[:, lo:hi]
+                N.transpose_bf16(self.weight(p, padded=True), view)
+                self._transposed[key + (k,)] = (p, view)
+            ent = (None, t)
+            self._transposed[key] = ent
+        return ent[1]
+
     def refresh_transposed(self) -> None:
         """Re-transposes the weights whose parameter changed since the last call (an optimizer
         step bumps the parameter's version counter)."""
         if not self._transposed:
             return
-        versions = (self._epoch,) + tuple(p._version for p, _ in self._transposed.values())
+        live = [(p, t) for p, t in self._transposed.values() if p is not None]
+        versions = (self._epoch,) + tuple(p._version for p, _ in live)
         if versions == self._versions:
             return
         self._versions = versions
-        for p, t in self._transposed.values():
+        for p, t in live:
             N.transpose_bf16(self.weight(p, padded=True), t)
 
     def mark_updated(self) -> None:
@@ -235,6 +254,39 @@ def op_swiglu_bwd(g, u, dh, dg, du) -> N.Op:
     op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = (g.data_ptr(), u.data_ptr(), dh.data_ptr(), dg.data_ptr(),
                                                    du.data_ptr())
     op.i[0] = g.numel()
+    return op
+
+
+def op_gemm_swiglu(x, w_gate, w_up, gu, h) -> N.Op:
+    """gu [T, 2 F] = [x w_gate^T | x w_up^T] and h [T, F] = silu(gate) * up in one GEMM kernel."""
+    T, K = x.shape
+    Fn = w_gate.shape[0]
+    assert w_gate.shape == w_up.shape == (Fn, K) and gu.shape == (T, 2 * Fn) and h.shape == (T, Fn)
+    for t in (x, w_gate, w_up, gu, h):
+        assert t.dtype == torch.bfloat16 and t.stride(1) == 1
+    assert w_gate.stride(0) == w_up.stride(0) and Fn % 8 == 0 and K % 8 == 0
+    op = N.Op()
+    op.kind = N.OP_GEMM_SWIGLU
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = (x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), gu.data_ptr(),
+                                                   h.data_ptr())
+    op.i[0], op.i[1], op.i[2] = T, Fn, K
+    op.i[3], op.i[4], op.i[5], op.i[6] = x.stride(0), w_gate.stride(0), gu.stride(0), h.stride(0)
+    return op
+
+
+def op_gemm_dswiglu(dy, w_down_t, gu, dgu) -> N.Op:
+    """dgu [T, 2 F] = [dg | du] from dh = dy w_down_t^T (not stored) and the saved gu = [g | u]."""
+    T, K = dy.shape
+    Fn = w_down_t.shape[0]
+    assert w_down_t.shape == (Fn, K) and gu.shape == dgu.shape == (T, 2 * Fn)
+    for t in (dy, w_down_t, gu, dgu):
+        assert t.dtype == torch.bfloat16 and t.stride(1) == 1
+    assert Fn % 8 == 0 and K % 8 == 0
+    op = N.Op()
+    op.kind = N.OP_GEMM_DSWIGLU
+    op.p[0], op.p[1], op.p[2], op.p[3] = dy.data_ptr(), w_down_t.data_ptr(), gu.data_ptr(), dgu.data_ptr()
+    op.i[0], op.i[1], op.i[2] = T, Fn, K
+    op.i[3], op.i[4], op.i[5], op.i[6] = dy.stride(0), w_down_t.stride(0), gu.stride(0), dgu.stride(0)
     return op
 
 
@@ -590,6 +642,9 @@ class Builder:
 
     def weight_t(self, p):
         return self.sp.arena.weight_t(p)
+
+    def weight_t_cat(self, p1, p2):
+        return self.sp.arena.weight_t_cat(p1, p2)
 
     def grad_target(self, p, padded=True):
         """Where the W pass writes a microbatch gradient that no GEMM epilogue accumulates: the

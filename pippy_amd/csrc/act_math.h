@@ -35,4 +35,18 @@ __device__ __forceinline__ float dgelu_tanh(float x) {
     return s * fmaf(x * du2, 1.0f - s, 1.0f);
 }
 
+// logistic function through the hardware exp2 and reciprocal
+__device__ __forceinline__ float sigmoid_fast(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * x));
+}
+// SwiGLU on values already rounded to the storage type: h = silu(g) u, and its two gradients
+// dg = dh u silu'(g), du = dh silu(g) with silu'(g) = s (1 + g (1 - s)), s = sigmoid(g).  The stand-alone
+// kernels and the GEMM epilogues share these, so that both leave the same bits.
+__device__ __forceinline__ float swiglu_value(float g, float u) { return g * sigmoid_fast(g) * u; }
+__device__ __forceinline__ void swiglu_grads(float g, float u, float dh, float* dg, float* du) {
+    const float s = sigmoid_fast(g);
+    *dg = dh * u * (s * fmaf(g, 1.0f - s, 1.0f));
+    *du = dh * (g * s);
+}
+
 }  // namespace pp

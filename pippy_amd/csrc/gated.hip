@@ -1,6 +1,7 @@
 // SwiGLU gate and rotary position embedding: the element-wise pieces of a Llama-style layer
 // (HBM-bound; 8 bf16 elements = 16 bytes per lane and access).
 #include "common.h"
+#include "act_math.h"
 
 namespace pp {
 
@@ -11,10 +12,6 @@ __device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
 __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
     return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
 }
-// logistic function through the hardware exp2 and reciprocal
-__device__ __forceinline__ float sigmoid_fast(float x) {
-    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * x));
-}
 
 // h = silu(g) * u
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint4* __restrict__ g, const uint4* __restrict__ u,
@@ -24,7 +21,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint4* __restrict
         unpack8(g[i], gf);
         unpack8(u[i], uf);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = gf[e] * sigmoid_fast(gf[e]) * uf[e];
+        for (int e = 0; e < 8; ++e) o[e] = swiglu_value(gf[e], uf[e]);
         h[i] = pack8(o);
     }
 }
@@ -39,11 +36,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* __restrict
         unpack8(u[i], uf);
         unpack8(dh[i], df);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float s = sigmoid_fast(gf[e]);
-            og[e] = df[e] * uf[e] * (s * fmaf(gf[e], 1.0f - s, 1.0f));
-            ou[e] = df[e] * (gf[e] * s);
-        }
+        for (int e = 0; e < 8; ++e) swiglu_grads(gf[e], uf[e], df[e], &og[e], &ou[e]);
         dg[i] = pack8(og);
         du[i] = pack8(ou);
     }

@@ -21,6 +21,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 struct GemmArgs {
     const uint16_t* A;
     const uint16_t* B;
+    const uint16_t* B2;  // second k-contiguous operand of a kernel that computes two products per tile
     void* C;
     int64_t M, N, K, lda, ldb, ldc;
     const uint16_t* bias;
@@ -224,7 +225,9 @@ struct WaveTile {
 // Main loop of one BM x BN output tile over the k-tiles [kt_begin, kt_end) of KT values each, through
 // NS LDS stages filled by direct-to-LDS loads; the products are added to acc.  Starts with a barrier,
 // so that it may follow an epilogue (or another main loop) that used the same LDS.
-template <int BM, int BN, bool AT, bool BT, int NS, int KT>
+// DUAL: the BN rows of the B tile are BN / 2 rows of g.B followed by the same BN / 2 rows of g.B2, so
+// that one tile holds two products of the same A rows (tile_n then counts blocks of BN / 2 rows).
+template <int BM, int BN, bool AT, bool BT, int NS, int KT, bool DUAL = false>
 __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n, int kt_begin,
                                               int kt_end,
                                               f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
@@ -232,7 +235,8 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
     constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     constexpr int KS = KT / 16;  // MFMA k-steps per tile
     constexpr int kStageElems = (BM + BN) * KT;
-    constexpr int LPT = DmaStage<BM, AT, KT>::kLoads + DmaStage<BN, BT, KT>::kLoads;  // loads per tile per wave
+    // loads per tile per wave (the two half loaders of a DUAL tile issue as many as one whole loader)
+    constexpr int LPT = DmaStage<BM, AT, KT>::kLoads + DmaStage<BN, BT, KT>::kLoads;
     constexpr int kReadsPerStep = TM * FragReader<BM, AT, KT>::kReads + TN * FragReader<BN, BT, KT>::kReads;
     static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
     static_assert(KS >= 2 && TN >= 2, "the last k-step is split in two parts around the barrier");
@@ -243,14 +247,18 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave % WT::WGM) * WTM, wn0 = (wave / WT::WGM) * WTN;
 
+    constexpr int BNL = DUAL ? BN / 2 : BN;  // rows that one loader of B brings
+    static_assert(!DUAL || (!AT && !BT), "two products per tile: k-contiguous operands");
     DmaStage<BM, AT, KT> sa;
-    DmaStage<BN, BT, KT> sb;
+    DmaStage<BNL, BT, KT> sb, sb2;
     sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
-    sb.init(g.B, g.ldb, n0, g.N, g.K, wave, lane);
+    sb.init(g.B, g.ldb, DUAL ? n0 / 2 : n0, g.N, g.K, wave, lane);
+    if (DUAL) sb2.init(g.B2, g.ldb, n0 / 2, g.N, g.K, wave, lane);
     const int nk = kt_end - kt_begin;
     auto issue = [&](int stage, int kt) {
         sa.load(smem + stage * kStageElems, (kt_begin + kt) * KT, wave);
         sb.load(smem + stage * kStageElems + BM * KT, (kt_begin + kt) * KT, wave);
+        if (DUAL) sb2.load(smem + stage * kStageElems + (BM + BNL) * KT, (kt_begin + kt) * KT, wave);
     };
 
     FragReader<BM, AT, KT> ra[TM];
@@ -530,6 +538,7 @@ static inline int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
     g->aux_out = static_cast<uint16_t*>(d->aux_out);
     g->ld_aux = d->ld_aux;
     g->beta = d->beta;
+    g->B2 = nullptr;
     g->round_bf16 = d->epilogue == PP_EPI_ACCUM_ROUNDED;
     g->epi = epi;
     g->tiles_m = g->tiles_n = g->n_blocks = 0;

@@ -562,6 +562,10 @@ class LlamaLayer(NativeBlock):
         """Emits y = x2 + FFN(RMSNorm(x2)); returns (y, emitter of the backward: dy -> d_x2)."""
         T = x2.shape[0]
         n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
+        mlp = self.mlp
+        if (x2.dtype == torch.bfloat16 and self.ffn % 8 == 0 and
+                all(lin.bias is None for lin in (mlp.gate_proj, mlp.up_proj, mlp.down_proj))):
+            return self._lower_feed_forward_fused(b, x2, n2, rstd2)
         g, _ = lower_linear(b, "g", self.mlp.gate_proj, n2)
         u, _ = lower_linear(b, "u", self.mlp.up_proj, n2)
         h = b.act("h", (T, self.ffn))
@@ -577,6 +581,32 @@ class LlamaLayer(NativeBlock):
             d_n2a = linear_backward(b, "gate", self.mlp.gate_proj, n2, dg)
             d_n2 = linear_backward(b, "up", self.mlp.up_proj, n2, du, dx_epilogue=N.EPI_BIAS_RESIDUAL,
                                    dx_aux=d_n2a)
+            return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+
+        return y, backward
+
+
+    def _lower_feed_forward_fused(self, b, x2, n2, rstd2):
+        """The bf16 feed-forward with SwiGLU inside the GEMMs around it: the gate and up products come
+        out of one kernel together with h = silu(g) * u; the input-gradient GEMM of the down projection
+        writes dg and du instead of dh; and the two input-gradient GEMMs of gate and up are one
+        product of [dg | du] with the two transposed weights side by side.  g, u, h, dg, du carry the
+        bits of the separate kernels; the gradient of the normalised input is one fp32 sum over both
+        branches (rounded once) instead of a rounded branch added in the epilogue of the other."""
+        T, ffn, mlp = x2.shape[0], self.ffn, self.mlp
+        gu = b.act("gu", (T, 2 * ffn))
+        h = b.act("h", (T, ffn))
+        b.f(P.op_gemm_swiglu(n2, b.weight(mlp.gate_proj.weight), b.weight(mlp.up_proj.weight), gu, h))
+        y, _ = lower_linear(b, "y", mlp.down_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+
+        def backward(dy2d):
+            dgu = b.grad("dgu", (T, 2 * ffn))
+            b.i(P.op_gemm_dswiglu(dy2d, b.weight_t(mlp.down_proj.weight), gu, dgu))
+            d_n2 = b.grad("gate_up.dx", (T, x2.shape[1]))
+            b.i(P.op_gemm(dgu, b.weight_t_cat(mlp.gate_proj.weight, mlp.up_proj.weight), d_n2))
+            linear_backward(b, "down", mlp.down_proj, h, dy2d, need_dx=False)
+            linear_backward(b, "gate", mlp.gate_proj, n2, dgu[:, :ffn], need_dx=False)
+            linear_backward(b, "up", mlp.up_proj, n2, dgu[:, ffn:], need_dx=False)
             return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
 
         return y, backward

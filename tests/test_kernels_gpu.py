@@ -835,6 +835,62 @@ def test_swiglu_matches_oracle(n):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,K,F", [(4096, 1024, 2816), (130, 72, 200), (1, 8, 8), (257, 4096, 344)])
+def test_gemm_fused_swiglu_equals_the_separate_kernels_and_the_oracle(M, K, F):
+    """The gate / up GEMM that applies SwiGLU in its epilogue, and the down projection's input-gradient
+    GEMM that applies its derivative, leave the bits of the GEMMs followed by the element-wise kernels
+    (values are rounded to bf16 at the same points); the oracle's fp32 feed-forward pins both."""
+    N = native()
+    g0 = torch.Generator().manual_seed(M + F)
+    x = torch.randn(M, K, generator=g0).to(torch.bfloat16)
+    wg = (torch.randn(F, K, generator=g0) / K ** 0.5 * 2).to(torch.bfloat16)
+    wu = (torch.randn(F, K, generator=g0) / K ** 0.5).to(torch.bfloat16)
+    wd = (torch.randn(K, F, generator=g0) / F ** 0.5).to(torch.bfloat16)   # down projection [out=K, in=F]
+    dy = torch.randn(M, K, generator=g0).to(torch.bfloat16)
+    xd, wgd, wud, dyd = x.cuda(), wg.cuda(), wu.cuda(), dy.cuda()
+    wdt = wd.t().contiguous().cuda()                                       # [F, K]
+    # separate kernels
+    g = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+    u, h, dh, dg, du = (torch.empty_like(g) for _ in range(5))
+    N.gemm_bf16(xd, wgd, g)
+    N.gemm_bf16(xd, wud, u)
+    N.swiglu_fwd(g, u, h)
+    N.gemm_bf16(dyd, wdt, dh)
+    N.swiglu_bwd(g, u, dh, dg, du)
+    # fused, into buffers with a recognisable fill so that stray writes show
+    gu = torch.full((M, 2 * F), 7.0, device="cuda", dtype=torch.bfloat16)
+    hf = torch.full((M, F), 7.0, device="cuda", dtype=torch.bfloat16)
+    dgu = torch.full((M, 2 * F), 7.0, device="cuda", dtype=torch.bfloat16)
+    N.gemm_swiglu(xd, wgd, wud, gu, hf)
+    N.gemm_dswiglu(dyd, wdt, gu, dgu)
+    torch.cuda.synchronize()
+    assert torch.equal(gu[:, :F], g) and torch.equal(gu[:, F:], u), "gate / up products"
+    assert torch.equal(hf, h), "activation"
+    assert torch.equal(dgu[:, :F], dg) and torch.equal(dgu[:, F:], du), "gate / up gradients"
+    # oracle: fp32 feed-forward and its autograd gradients
+    gr = (x.float() @ wg.float().t()).requires_grad_(True)
+    ur = (x.float() @ wu.float().t()).requires_grad_(True)
+    hr = O.swiglu(gr, ur)
+    assert_close_rel(hf, hr.detach(), BF16_TOL, "fused swiglu forward")
+    hr.backward(dy.float() @ wd.float())
+    assert_close_rel(dgu[:, :F], gr.grad, 2 * BF16_TOL, "fused gate gradient")
+    assert_close_rel(dgu[:, F:], ur.grad, 2 * BF16_TOL, "fused up gradient")
+
+
+@pytest.mark.gpu
+def test_gemm_fused_swiglu_rejects_bad_arguments():
+    N = native()
+    x = torch.zeros(16, 8, device="cuda", dtype=torch.bfloat16)
+    w = torch.zeros(12, 8, device="cuda", dtype=torch.bfloat16)   # N = 12 is not a multiple of 8
+    gu = torch.zeros(16, 24, device="cuda", dtype=torch.bfloat16)
+    h = torch.zeros(16, 12, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        N.gemm_swiglu(x, w, w, gu, h)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        N.gemm_dswiglu(x, w, gu, gu.clone())
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("B,S,H,D", [(2, 64, 3, 64), (1, 2048, 4, 128), (3, 16, 2, 32)])
 def test_rope_matches_oracle_and_inverts(B, S, H, D):
     N = native()

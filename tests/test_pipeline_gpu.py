@@ -544,6 +544,40 @@ def test_llama_stage_zero_bubble_matches_oracle():
     note(f"Llama stage, zero-bubble: worst grad error {worst:.3e}")
 
 
+def test_llama_fused_feed_forward_follows_parameter_updates_and_launches_fused_kernels():
+    """The feed-forward of a bf16 Llama layer runs as GEMMs with SwiGLU in their epilogues (no separate
+    element-wise launch), and the side-by-side transposed gate / up weights that its input-gradient GEMM
+    reads are refreshed after the parameters change."""
+    import pippy_amd as pp
+    from pippy_amd import _native as N
+    from pippy_amd.configs import LlamaStage
+    torch.manual_seed(5)
+    M, S, dim = 2, 128, 128
+    model = LlamaStage(n_layers=1, dim=dim, n_heads=2, ffn=328)   # 328: tiles with a ragged last column block
+    ref = _fp32_cpu_copy(model)
+    x = torch.randn(M, S, dim).to(torch.bfloat16)
+    upstream = torch.randn(M, S, dim) * 1e-2
+    stage = pp.ManualPipelineStage(model, 0, 1, DEV, M, input_args=(x[:1].to(DEV),))
+    sched = pp.ScheduleZeroBubble([stage], M, loss_fn=_upstream_loss)
+    sched.step(x.to(DEV), target=upstream.to(DEV))
+    prog = stage._program.mbs[0]
+    kinds_f = [op.kind for op in prog.F.ops]
+    kinds_i = [op.kind for op in prog.I.ops]
+    assert N.OP_GEMM_SWIGLU in kinds_f and N.OP_SWIGLU_FWD not in kinds_f
+    assert N.OP_GEMM_DSWIGLU in kinds_i and N.OP_SWIGLU_BWD not in kinds_i
+    torch.manual_seed(6)
+    with torch.no_grad():
+        for (n, p), (_, rp) in zip(model.named_parameters(), ref.named_parameters()):
+            p.add_((torch.randn(rp.shape) * 0.02).to(torch.bfloat16).to(DEV))
+            rp.copy_(p.detach().float().cpu())
+    sched.zero_grad()
+    losses = []
+    out = sched.step(x.to(DEV), target=upstream.to(DEV), losses=losses)
+    ref_out, ref_losses = OP.step([ref], x.float(), upstream, M, _upstream_loss)
+    assert_close_rel(out, ref_out, BF16_TOL, "stage output after the update")
+    _llama_grads_match(model, ref, losses, ref_losses, ref_out, upstream)
+
+
 def test_llama_two_stages_1f1b_hand_off_matches_oracle():
     """The same layers split into two traced stages: the input gradient of the second stage (through
     RMSNorm, rotary embedding and attention backward) feeds the first."""
