@@ -183,11 +183,11 @@ double op_work(const pp_op& op) {
     switch (op.kind) {
         case PP_OP_GEMM_BF16:
         case PP_OP_GEMM_F32:
-        case PP_OP_GEMM_SWIGLU:  // two products of N columns each
-            return 4.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_GEMM_DSWIGLU:
         case PP_OP_GEMM_SEG:  // the segments partition the rows (rows mode: M, k mode: K)
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
+        case PP_OP_GEMM_SWIGLU:  // two products of N columns each
+            return 4.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_ATTN_FWD:  // dense count: QK^T and PV
             return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[1] * (double)op.i[1] * (double)op.i[3];
         case PP_OP_ATTN_BWD:  // dQ, dK, dV, dP and the recomputed scores

@@ -1161,3 +1161,32 @@ def test_moe_layer_with_an_expert_count_that_is_not_a_multiple_of_8_raises_on_lo
     assert stage.is_native
     with pytest.raises(RuntimeError, match="multiple of 8 experts"):
         pp.ScheduleGPipe([stage], 1).step(x)
+
+
+@pytest.mark.gpu
+def test_launch_timer_counts_the_algorithmic_work_of_each_gemm_kind():
+    """The per-launch timer behind the bench's roofline figures must attribute 2 M N K flops to a GEMM
+    (4 M N K to the kernel that forms the gate and up products together): a slip here would scale every
+    reported MFMA fraction."""
+    from pippy_amd import _program as P
+    N = native()
+    M, K, F = 256, 128, 192
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w = torch.randn(F, K, device="cuda").to(torch.bfloat16)
+    wt = torch.randn(F, K, device="cuda").to(torch.bfloat16)
+    y = torch.empty(M, F, device="cuda", dtype=torch.bfloat16)
+    gu = torch.empty(M, 2 * F, device="cuda", dtype=torch.bfloat16)
+    dgu = torch.empty_like(gu)
+    ops = P.OpList()
+    ops.append(P.op_gemm(x, w, y))
+    ops.append(P.op_gemm(x, w, y))
+    ops.append(P.op_gemm_swiglu(x, w, w, gu, y))
+    ops.append(P.op_gemm_dswiglu(x, wt, gu, dgu))
+    N.profile_start(64)
+    ops.run()
+    torch.cuda.synchronize()
+    N.profile_stop()
+    for kind, want_work, want_count in ((N.OP_GEMM_BF16, 2 * 2.0 * M * F * K, 2), (N.OP_GEMM_SWIGLU, 4.0 * M * F * K, 1),
+                                        (N.OP_GEMM_DSWIGLU, 2.0 * M * F * K, 1)):
+        ms, work, cnt = N.profile_read(kind)
+        assert cnt == want_count and work == want_work and ms > 0, (kind, ms, work, cnt)
