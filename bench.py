@@ -31,10 +31,19 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # Bytes between the L2 caches and the fabric per GEMM launch, averaged over the GEMM launches of one
 # step of the default workload: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
-# counter reads for the logits merge, a copy of known size (summary under profiles/).  A counter run
-# cannot be made from inside this script, so the figure is carried here and only reported for the
-# default workload.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 113.1e6
+# counter reads for the logits merge, a copy of known size.  A counter run cannot be made from inside
+# this script: the figure is read from the tracked summary of the last such run and reported, with the
+# file it came from, for the default workload only.
+GEMM_TRAFFIC_FILE = os.path.join("profiles", "gemm_gpt2small_1f1b_hbm_traffic.json")
+
+
+def gemm_traffic():
+    """(bytes per launch or None, where the figure comes from)."""
+    try:
+        with open(os.path.join(ROOT, GEMM_TRAFFIC_FILE)) as f:
+            return float(json.load(f)["gemm_traffic_bytes_per_launch"]), GEMM_TRAFFIC_FILE
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def build(args):
@@ -183,6 +192,71 @@ def cpu_baseline(args, budget_seconds=45.0):
                       f"({rep['warmup_s']:.1f} s); timed {rep['step_s']:.1f} s"}
 
 
+GEMM_SHAPES = (
+    # (M, N, K, a_trans, b_trans, what)
+    (4096, 768, 768, 0, 0, "gpt2 attention projection"), (4096, 2304, 768, 0, 0, "gpt2 qkv"),
+    (4096, 3072, 768, 0, 0, "gpt2 feed-forward up"), (4096, 768, 3072, 0, 0, "gpt2 feed-forward down"),
+    (4096, 50304, 768, 0, 0, "gpt2 vocabulary projection"), (4096, 768, 50304, 0, 0, "its input gradient"),
+    (3072, 768, 4096, 1, 1, "gpt2 weight gradient (dY^T X over 4096 tokens)"),
+    (4096, 4096, 1024, 0, 0, "mid-sized"), (2048, 4096, 4096, 0, 0, "llama attention projection"),
+    (2048, 12288, 4096, 0, 0, "llama qkv"), (2048, 11008, 4096, 0, 0, "llama gate / up"),
+    (2048, 4096, 11008, 0, 0, "llama down"), (11008, 4096, 2048, 1, 1, "llama weight gradient"),
+    (8192, 8192, 8192, 0, 0, "large square"),
+)
+
+
+def gemm_shapes():
+    """One JSON line per shape: the library's GEMM and torch.matmul on the same operands, each timed over
+    rotating operand sets (so that operands are not L2-resident from the previous launch) with the shader
+    clock sampled by a one-wave probe on a second stream while the launches run."""
+    from pippy_amd import _native as N
+    N.lib()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    side = torch.cuda.Stream()
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
+
+    def timed(fns, flops):
+        for f in fns:
+            f()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = max(2, min(200, int(2e12 / flops)))   # a few milliseconds of work
+        ev0.record()
+        for _ in range(reps):
+            for f in fns:
+                f()
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1e3 / (reps * len(fns))
+        # the same launches again, enough of them to outlast the 2 ms probe
+        for _ in range(max(reps, int(4e3 / (us * len(fns))) + 1)):
+            for f in fns:
+                f()
+        N.clock_probe(clk, 2e-3, side.cuda_stream)
+        torch.cuda.synchronize()
+        c, w = clk.tolist()
+        return us, c / max(w, 1) * 100.0   # MHz
+
+    for (M, Nn, K, at, bt, what) in GEMM_SHAPES:
+        sets = []
+        for _ in range(3):
+            A = torch.randn((K, M) if at else (M, K), device=dev).to(torch.bfloat16)
+            B = (torch.randn((K, Nn) if bt else (Nn, K), device=dev) * 0.05).to(torch.bfloat16)
+            sets.append((A, B, torch.empty(M, Nn, device=dev, dtype=torch.bfloat16)))
+        flops = 2.0 * M * Nn * K
+        ours_us, ours_mhz = timed([(lambda s=s: N.gemm_bf16(s[0], s[1], s[2], a_trans=bool(at), b_trans=bool(bt)))
+                                   for s in sets], flops)
+        lib_us, lib_mhz = timed([(lambda s=s: torch.matmul(s[0].t() if at else s[0], s[1] if bt else s[1].t(),
+                                                           out=s[2])) for s in sets], flops)
+        print(json.dumps({"shape": [M, Nn, K], "a_trans": at, "b_trans": bt, "what": what,
+                          "us": round(ours_us, 1), "tflops": round(flops / ours_us / 1e6, 1),
+                          "shader_mhz": round(ours_mhz), "vendor_us": round(lib_us, 1),
+                          "vendor_tflops": round(flops / lib_us / 1e6, 1), "vendor_shader_mhz": round(lib_mhz)}),
+              flush=True)
+        del sets
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -199,6 +273,10 @@ def main():
     ap.add_argument("--serial-stages", action="store_true",
                     help="run all virtual stages on one stream instead of two")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--gemm-shapes", action="store_true",
+                    help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
+                         "events, cold operands), torch.matmul (the vendor library) on the same operands beside "
+                         "it, and sample the shader clock during each; one JSON line per shape")
     ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
                          "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
@@ -231,6 +309,10 @@ def main():
     cpu_result = None
     if not args.no_cpu_baseline and args.workload == "gpt2":
         cpu_result = cpu_baseline(args)
+
+    if args.gemm_shapes:
+        gemm_shapes()
+        return
 
     from pippy_amd import _native as N
     N.lib()  # fail loudly if the kernel library is missing
@@ -301,7 +383,8 @@ def main():
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
-                              "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
+                              "traffic": gemm_traffic()[0] if default_workload else None,
+                              "traffic_source": gemm_traffic()[1] if default_workload else None,
                               "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
                                         + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else "")
                                         + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else ""),

@@ -454,6 +454,12 @@ int pp_profile_start(int max_records);
 int pp_profile_stop(void);
 int pp_profile_read(int kind, double* total_ms, double* total_work, int64_t* count);
 
+/* Samples the shader clock (measurement aid; no reference counterpart): one wave idles for
+ * `wall_ticks` ticks of the constant 100 MHz counter (at most 1e8 = one second) and writes
+ * out[0] = shader clocks elapsed, out[1] = ticks elapsed (device memory, two int64).  Launched on a
+ * stream of its own beside other work, out[0] / out[1] * 100 MHz is the clock that work runs at. */
+int pp_clock_probe(int64_t* out, int64_t wall_ticks, pp_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

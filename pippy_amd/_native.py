@@ -44,6 +44,7 @@ EXPORTED_SYMBOLS = (
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
     "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc", "pp_gemm_bf16_swiglu", "pp_gemm_bf16_dswiglu",
+    "pp_clock_probe",
 )
 
 
@@ -132,6 +133,7 @@ def lib() -> C.CDLL:
         "pp_transpose_bf16": [vp, i64, i64, i64, vp, i64, vp],
         "pp_profile_start": [i32],
         "pp_profile_stop": [],
+        "pp_clock_probe": [vp, i64, vp],
         "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
         "pp_swiglu_fwd": [vp, vp, vp, i64, vp],
         "pp_swiglu_bwd": [vp, vp, vp, vp, vp, i64, vp],
@@ -654,6 +656,14 @@ def profile_start(max_records: int = 1 << 16) -> None:
 
 def profile_stop() -> None:
     check(lib().pp_profile_stop(), "pp_profile_stop")
+
+
+def clock_probe(out: torch.Tensor, seconds: float, stream: int) -> None:
+    """Launches the clock sampler on ``stream`` for ``seconds``; afterwards out[0] / out[1] * 1e8 is the
+    shader clock in Hz (``out``: two int64 on the device)."""
+    require_cuda(out)
+    assert out.dtype == torch.int64 and out.numel() >= 2 and out.is_contiguous()
+    check(lib().pp_clock_probe(out.data_ptr(), int(seconds * 1e8), stream), "pp_clock_probe")
 
 
 def profile_read(kind: int):

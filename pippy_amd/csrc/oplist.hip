@@ -232,6 +232,31 @@ double op_work(const pp_op& op) {
 }
 }  // namespace
 
+// One wave that idles for `wall_ticks` ticks of the constant 100 MHz counter and reports how many
+// shader clocks passed meanwhile: launched on a stream of its own beside other work, it samples the
+// clock that the work runs at.
+__global__ void clock_probe_kernel(long long* out, long long wall_ticks) {
+    const long long c0 = clock64(), w0 = wall_clock64();
+    long long w1 = w0;
+    while (w1 - w0 < wall_ticks) {
+        __builtin_amdgcn_s_sleep(8);
+        w1 = wall_clock64();
+    }
+    const long long c1 = clock64();
+    if (threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = w1 - w0;
+    }
+}
+
+extern "C" int pp_clock_probe(int64_t* out, int64_t wall_ticks, pp_stream stream) {
+    if (!out) return fail(PP_ERR_INVALID, "pp_clock_probe: null pointer");
+    if (wall_ticks < 0 || wall_ticks > 100000000) return fail(PP_ERR_INVALID, "pp_clock_probe: 0 <= wall_ticks <= 1e8 (one second)");
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<long long*>(out), (long long)wall_ticks);
+    return check_launch("clock_probe_kernel");
+}
+
 extern "C" int pp_profile_start(int max_records) {
     if (max_records <= 0) return fail(PP_ERR_INVALID, "pp_profile_start: max_records <= 0");
     if (g_prof.size() < (size_t)max_records) {
