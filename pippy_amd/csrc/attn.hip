@@ -165,17 +165,35 @@ __device__ __forceinline__ bool attn_block_of(uint32_t bid, uint32_t grid, uint3
 }
 
 // ---- forward ----------------------------------------------------------------------------------
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const AttnArgs a) {
+// WAVES = 4: key blocks of 64, each row group's two waves take 32 keys of every block.  WAVES = 8: key
+// blocks of 128 and four waves per row group.  A launch of few, short heads is bound by the chain of
+// dependent block steps of its longest work-group (load -> K Q^T -> softmax -> P V, about 0.6 us per
+// step whatever shares the CU), not by arithmetic: eight waves walk that chain in half the steps.
+template <int D, int WAVES>
+struct AttnFwdCfg {
+    static constexpr int kParts = WAVES / 2;             // waves per row group = parts of a key block
+    static constexpr int kBlockKeys = 32 * kParts;       // keys per block
+    static constexpr int kTilesPerOperand = (D / 64) * (kBlockKeys / 64);
+    static constexpr int kOperand = kTilesPerOperand * kTile;
+    static constexpr int kStage = 2 * kOperand;
+    static constexpr int kStages = (D == 64 && WAVES == 4) ? 3 : 2;
+    static constexpr size_t kMerge = (size_t)2 * (kParts - 1) * (16 * (D / 32) + 2) * 64 * 4;
+    static constexpr size_t kLds = (size_t)kStages * kStage * 2 > kMerge ? (size_t)kStages * kStage * 2 : kMerge;
+};
+
+template <int D, bool CAUSAL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) void attn_fwd_kernel(const AttnArgs a) {
     static_assert(D == 64 || D == 128, "head dimension 64 or 128");
-    constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = attn_stages(D);
-    constexpr int kOperand = DS * kTile;   // one staged 64-row block of K or V
-    constexpr int kStage = 2 * kOperand;
+    static_assert(WAVES == 4 || WAVES == 8, "two or four waves per row group");
+    typedef AttnFwdCfg<D, WAVES> Cfg;
+    constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = Cfg::kStages;
+    constexpr int P = Cfg::kParts, KB = Cfg::kBlockKeys, KT = KB / 64;  // KT: 64-row tiles per block and operand column
+    constexpr int kOperand = Cfg::kOperand, kStage = Cfg::kStage;
     uint16_t* const lds = attn_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = wave & 1, half = wave >> 1;
+    const int grp = wave & 1, part = wave >> 1;
     const int l32 = lane & 31, lh = lane >> 5;
     const uint32_t nx = (uint32_t)(a.S / 64);
     uint32_t bh, ord;
@@ -186,13 +204,17 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
     const int64_t qi = qw0 + l32;  // this lane's query row
 
     const uint16_t* qp = a.q + b * a.stride_b + h * D;
+    // the 64-row tiles of a block are loaded by sets of four waves: waves 4 .. 7 take the second 64 keys
+    const int lset = wave >> 2, lwave = wave & 3;
     AttnTileLoader<DS> lk, lv;
-    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
-    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
-    const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
+    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, lwave, lane);
+    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, lwave, lane);
+    const int64_t n_keys = CAUSAL ? q0 + 64 : a.S;
+    const int64_t n_blocks = (n_keys + KB - 1) / KB;
+    // LDS layout of an operand: [64-key tile of the block][64 columns of d] tiles of 64 x 64
     auto issue = [&](int stage, int64_t j) {
-        lk.load(lds + stage * kStage, j * 64, wave);
-        lv.load(lds + stage * kStage + kOperand, j * 64, wave);
+        lk.load(lds + stage * kStage + lset * DS * kTile, j * KB + 64 * lset, lwave);
+        lv.load(lds + stage * kStage + kOperand + lset * DS * kTile, j * KB + 64 * lset, lwave);
     };
 
     bf16x8_t qf[KS];
@@ -208,44 +230,55 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
     for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[t][e] = 0.f;
+    // l_run is this lane's share of the row sum (the other 16 of the wave's 32 keys are the partner
+    // lane's, lane ^ 32): the shares meet once, after the last block
     float m_run = -INFINITY, l_run = 0.f;
     const float c = a.scale * kLog2e;
+    const int partner = (lane ^ 32) << 2;  // byte index of the lane that holds the same query column
+    const int ktile = (32 * part) / 64, krow = (32 * part) % 64;  // this wave's keys inside the block
 
-    int stage = 0;
-    for (int64_t j = 0; j < n_blocks; ++j) {
-        const int64_t kt0 = j * 64 + 32 * half;  // first key of this wave's half block
+    // The loop over blocks is unrolled by the number of stages: the stage of a block is then a constant of
+    // its copy of the loop body, and the LDS addresses of the fragment reads are per-lane offsets computed
+    // once plus immediate offsets, instead of vector additions in every step.
+    for (int64_t j0 = 0; j0 < n_blocks; j0 += NS)
+      static_for<NS>([&](auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
+        const int64_t j = j0 + stage;
+        if (j >= n_blocks) return;
+        const int64_t kt0 = j * KB + 32 * part;  // first key of this wave's part of the block
         await_block<4 * DS, NS>(j, n_blocks);
         if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
-        const uint16_t* Ks = lds + stage * kStage;
+        const uint16_t* Ks = lds + stage * kStage + ktile * DS * kTile;
         const uint16_t* Vs = Ks + kOperand;
-        stage = stage + 1 == NS ? 0 : stage + 1;
-        const bool active = !CAUSAL || (kt0 <= qw0 + 31);
+        // keys past the sequence (a last block of 128 that is half full) or past every query of the wave
+        const bool active = kt0 < a.S && (!CAUSAL || (kt0 <= qw0 + 31));
         if (active) {
+            bf16x8_t kf[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf[ks] = read_row_frag(Ks + (ks / 4) * kTile, krow + l32, 2 * (ks % 4) + lh);
             f32x16_t sacc;
 #pragma unroll
             for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t kf = read_row_frag(Ks + (ks / 4) * kTile, 32 * half + l32, 2 * (ks % 4) + lh);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc, 0, 0, 0);
-            }
+            for (int ks = 0; ks < KS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], sacc, 0, 0, 0);
             // sacc[v]: kv = kt0 + 8 (v/4) + 4 lh + v%4, q = qi
-            const bool diag = CAUSAL && (kt0 + 31 > qw0);
-            // m_run tracks the maximum of the raw scores; c > 0, so scaling commutes with max
-            if (diag) {  // wave-uniform: only blocks on the diagonal pay for the mask
+            if (CAUSAL && (kt0 + 31 > qw0)) {  // wave-uniform: only blocks on the diagonal pay for the mask
+                const int lim = (int)(qi - kt0) - 4 * lh;  // keys 8 (v/4) + v%4 up to lim are visible
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    if (kt0 + 8 * (v >> 2) + 4 * lh + (v & 3) > qi) sacc[v] = -INFINITY;
+                    if (8 * (v >> 2) + (v & 3) > lim) sacc[v] = -INFINITY;
             }
             float mloc = -INFINITY;
 #pragma unroll
             for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, sacc[v]);
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             // The reference maximum of a row only has to keep the exponentials in range, so it is
             // moved (and the accumulators rescaled) only when some row of the wave exceeds it by
             // more than 2^8 after scaling; that happens in the first block of a row and almost
-            // never again.  Any reference gives the same softmax after the final division.
+            // never again.  Any reference gives the same softmax after the final division.  m_run
+            // tracks the maximum of the raw scores (c > 0, so scaling commutes with max) and is the
+            // same in both lanes of a query column.
             if (__ballot(mloc * c > m_run * c + 8.0f)) {
+                mloc = fmaxf(mloc, __int_as_float(__builtin_amdgcn_ds_bpermute(partner, __float_as_int(mloc))));
                 const float m_new = fmaxf(m_run, mloc);
                 const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
                 l_run *= alpha;
@@ -264,7 +297,6 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
                 sacc[v] = p;
                 psum += p;
             }
-            psum += __shfl_xor(psum, 32, 64);
             l_run += psum;
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
@@ -274,19 +306,21 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
                 const bf16x8_t pb = pack8(pv);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t vf = read_col_frag(Vs + (dt / 2) * kTile, 32 * half + 16 * gp, 32 * (dt % 2), lane);
+                    const bf16x8_t vf = read_col_frag(Vs + (dt / 2) * kTile, krow + 16 * gp, 32 * (dt % 2), lane);
                     oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, oacc[dt], 0, 0, 0);
                 }
             }
         }
-    }
+      });
+    l_run += __int_as_float(__builtin_amdgcn_ds_bpermute(partner, __float_as_int(l_run)));
 
-    // merge the two halves of every key block: [grp][16 DT + 2 values][64 lanes] floats
+    // merge the parts of every key block in a fixed order: [grp][part - 1][16 DT + 2 values][64 lanes] floats
     wait_lds();
-    __builtin_amdgcn_s_barrier();
+    __syncthreads();
     constexpr int kVals = 16 * DT + 2;
-    float* xs = reinterpret_cast<float*>(lds) + grp * (kVals * 64) + lane;
-    if (half == 1) {
+    float* const xs0 = reinterpret_cast<float*>(lds) + grp * ((P - 1) * kVals * 64) + lane;
+    if (part != 0) {
+        float* xs = xs0 + (part - 1) * (kVals * 64);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -295,14 +329,28 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
         xs[(16 * DT + 1) * 64] = l_run;
     }
     __syncthreads();
-    if (half == 0) {
-        const float m1 = xs[16 * DT * 64], l1 = xs[(16 * DT + 1) * 64];
-        const float m = fmaxf(m_run, m1);  // finite: key 0 is visible to every query
-        const float a0 = __builtin_amdgcn_exp2f((m_run - m) * c);
-        const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m1 - m) * c);
-        const float l = l_run * a0 + l1 * a1;
+    if (part == 0) {
+        float m = m_run;  // finite after the merge: key 0 is visible to every query
+#pragma unroll
+        for (int p = 1; p < P; ++p) m = fmaxf(m, xs0[(p - 1) * (kVals * 64) + 16 * DT * 64]);
+        const float a0 = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((m_run - m) * c);
+        float l = l_run * a0;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[dt][e] *= a0;
+#pragma unroll
+        for (int p = 1; p < P; ++p) {
+            const float* xs = xs0 + (p - 1) * (kVals * 64);
+            const float mp = xs[16 * DT * 64], lp = xs[(16 * DT + 1) * 64];
+            const float ap = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mp - m) * c);
+            l += lp * ap;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) oacc[dt][e] += xs[(16 * dt + e) * 64] * ap;
+        }
         const float inv_l = 1.0f / l;
-        const float w0 = a0 * inv_l, w1 = a1 * inv_l;
         uint16_t* op = a.o + (b * a.S + qi) * (a.H * D) + h * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -310,8 +358,7 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_fwd_kernel(const At
             for (int g = 0; g < 4; ++g) {
                 float o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    o[e] = oacc[dt][4 * g + e] * w0 + xs[(16 * dt + 4 * g + e) * 64] * w1;
+                for (int e = 0; e < 4; ++e) o[e] = oacc[dt][4 * g + e] * inv_l;
                 const int d = 32 * dt + 8 * g + 4 * lh;
                 *reinterpret_cast<uint2*>(op + d) = make_uint2(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]));
             }
@@ -381,6 +428,8 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
         }
     const float c = a.scale * kLog2e;
 
+    // (not unrolled by the number of stages as the other two kernels are: the per-lane offsets of its 24
+    // fragment reads per block would not fit the register budget of three work-groups per CU)
     int stage = 0;
     for (int64_t j = 0; j < nb; ++j) {
         const int64_t qc0 = (jq_begin + j) * 64;
@@ -553,14 +602,17 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
 #pragma unroll
         for (int e = 0; e < 16; ++e) dqacc[t][e] = 0.f;
 
-    int stage = 0;
-    for (int64_t j = 0; j < n_blocks; ++j) {
+    // unrolled by the number of stages (see the forward kernel)
+    for (int64_t j0 = 0; j0 < n_blocks; j0 += NS)
+      static_for<NS>([&](auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
+        const int64_t j = j0 + stage;
+        if (j >= n_blocks) return;
         const int64_t kv0 = j * 64;
         await_block<4 * DS, NS>(j, n_blocks);
         if (j + NS - 1 < n_blocks) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Ks = lds + stage * kStage;
         const uint16_t* Vs = Ks + kOperand;
-        stage = stage + 1 == NS ? 0 : stage + 1;
         const int t = half;
         const int64_t kt0 = kv0 + 32 * t;
         if (!CAUSAL || (kt0 <= qw0 + 31)) {
@@ -599,7 +651,7 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
                 }
             }
         }
-    }
+      });
     // add the partial sums of the two key halves: [grp][16 DT values][64 lanes] floats
     wait_lds();
     __builtin_amdgcn_s_barrier();
@@ -670,21 +722,36 @@ static size_t attn_lds_bytes(int D, bool dkv) {
 }
 
 template <auto kernel>
-static int attn_launch(const char* name, dim3 grid, size_t lds, hipStream_t st, const AttnArgs& a) {
+static int attn_launch(const char* name, dim3 grid, int threads, size_t lds, hipStream_t st, const AttnArgs& a) {
     // one attribute call per kernel (the kernel is a template argument, so is the static) and process
     static const hipError_t attr_rc =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr_rc != hipSuccess)
         return fail(PP_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS: %s", name, lds, hipGetErrorString(attr_rc));
-    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, a);
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, st, a);
     return check_launch(name);
+}
+
+// Eight waves per work-group when the launch has fewer than two work-groups per CU: its duration is
+// then the chain of its longest work-group (15.9 -> 10.9 us at [1, 12, 1024, 64] causal).  With more,
+// the four-wave form's three work-groups per CU keep the CUs busy and its smaller key blocks waste less
+// on the diagonal (18.6 against 20.6 us at [4, 12, 1024, 64] causal).
+static bool attn_fwd_wide(const pp_attn_desc* d) {
+    return d->D == 64 && (d->S / 64) * d->H * d->B < 2 * 256 && d->S >= 256;
 }
 
 template <int D>
 static int attn_fwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
-    const size_t lds = attn_lds_bytes(D, false);
-    return d->causal ? attn_launch<attn_fwd_kernel<D, true>>("attn_fwd_kernel", grid, lds, st, a)
-                     : attn_launch<attn_fwd_kernel<D, false>>("attn_fwd_kernel", grid, lds, st, a);
+    if constexpr (D == 64) {
+        if (attn_fwd_wide(d)) {
+            const size_t lds = AttnFwdCfg<D, 8>::kLds;
+            return d->causal ? attn_launch<attn_fwd_kernel<D, true, 8>>("attn_fwd_kernel", grid, 512, lds, st, a)
+                             : attn_launch<attn_fwd_kernel<D, false, 8>>("attn_fwd_kernel", grid, 512, lds, st, a);
+        }
+    }
+    const size_t lds = AttnFwdCfg<D, 4>::kLds;
+    return d->causal ? attn_launch<attn_fwd_kernel<D, true, 4>>("attn_fwd_kernel", grid, 256, lds, st, a)
+                     : attn_launch<attn_fwd_kernel<D, false, 4>>("attn_fwd_kernel", grid, 256, lds, st, a);
 }
 
 template <int D>
@@ -693,13 +760,13 @@ static int attn_bwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipSt
     const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false);
     int rc;
     if (d->causal) {
-        rc = attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+        rc = attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
         if (rc) return rc;
-        return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+        return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, 256, lds_kv, st, a);
     }
-    rc = attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, lds_q, st, a);
+    rc = attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
     if (rc) return rc;
-    return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, lds_kv, st, a);
+    return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, 256, lds_kv, st, a);
 }
 
 }  // namespace pp

@@ -8,16 +8,6 @@
 
 namespace pp {
 
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop that is unrolled by
-// construction, for bodies that index register arrays with the loop variable.
-template <int N, int I = 0, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<N, I + 1>(f);
-    }
-}
-
 struct GemmArgs {
     const uint16_t* A;
     const uint16_t* B;

@@ -10,11 +10,22 @@
 // 256 lanes (4 waves) cooperate.
 #pragma once
 #include "common.h"
+#include <type_traits>
 
 namespace pp {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop that is unrolled by
+// construction, for bodies that index register arrays with the loop variable.
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 constexpr int BK = 64;
 constexpr int kGemmThreads = 256;
