@@ -605,6 +605,55 @@ def test_llama_two_stages_1f1b_hand_off_matches_oracle():
     note(f"Llama layers, two stages: worst grad error {worst:.3e}")
 
 
+def test_split_backward_matches_the_library_split_of_autograd():
+    """The separate input-gradient and weight-gradient passes against the library routines that split
+    autograd the same way (torch.distributed.pipelining._backward.stage_backward_input /
+    stage_backward_weight, run on an fp32 CPU copy of the same two stages): the gradient that stage 1
+    hands to stage 0 for every microbatch, and the parameter gradients once the deferred weight
+    passes have run."""
+    import pippy_amd as pp
+    import torch.nn as nn
+    from torch.distributed.pipelining._backward import stage_backward_input, stage_backward_weight
+    from pippy_amd.configs import LlamaStage
+    torch.manual_seed(11)
+    M, S, dim = 2, 128, 128
+    model = LlamaStage(n_layers=2, dim=dim, n_heads=2, ffn=256)
+    ref = _fp32_cpu_copy(model)
+    x = torch.randn(2 * M, S, dim).to(torch.bfloat16)
+    upstream = torch.randn(2 * M, S, dim) * 1e-2
+    pipe = pp.pipeline(model, M, (x,), split_spec={"layers.1": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    sched = pp.ScheduleZeroBubble(stages, M, loss_fn=_upstream_loss)
+    sched.step(x.to(DEV), target=upstream.to(DEV))
+    torch.cuda.synchronize()
+
+    ref_stages = [nn.Sequential(ref.layers[0]), nn.Sequential(ref.layers[1])]
+    for p in ref.parameters():
+        p.grad = None
+    handed_over, deferred = [], []
+    for xm, um in zip(x.float().chunk(M), upstream.chunk(M)):
+        xm = xm.clone().requires_grad_(True)
+        h0 = ref_stages[0](xm)
+        h1_in = h0.detach().requires_grad_(True)
+        out = ref_stages[1](h1_in)
+        loss = _upstream_loss(out, um)
+        (d_h1,), groups1 = stage_backward_input([loss], None, [h1_in], ref_stages[1].parameters())
+        assert all(p.grad is None for p in ref_stages[1].parameters()), "the input pass leaves the weights alone"
+        _, groups0 = stage_backward_input([h0], [d_h1], [xm], ref_stages[0].parameters())
+        handed_over.append(d_h1)
+        deferred.append((groups0, groups1))
+    for groups0, groups1 in deferred:   # the weight passes run later, in microbatch order
+        stage_backward_weight(ref_stages[1].parameters(), groups1)
+        stage_backward_weight(ref_stages[0].parameters(), groups0)
+
+    for m in range(M):
+        got = stages[1]._program.mbs[m].input_grad
+        assert_close_rel(got.view(handed_over[m].shape), handed_over[m], BF16_TOL, f"input gradient of microbatch {m}")
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        assert max_rel(named[name].main_grad, rp.grad) <= BF16_TOL, f"grad of {name}"
+
+
 def test_llama2_7b_stage_full_size_schedule_and_scaling_invariants():
     """Config 4 at full size (8 layers, width 4096, 32 heads of 128, SwiGLU 11008, sequence 2048,
     16 microbatches of one sequence).  Two properties that hold at any size: the zero-bubble schedule
