@@ -210,6 +210,7 @@ def gemm_shapes():
     rotating operand sets (so that operands are not L2-resident from the previous launch) with the shader
     clock sampled by a one-wave probe on a second stream while the launches run."""
     from pippy_amd import _native as N
+    from pippy_amd._program import splitk_copies
     N.lib()
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
@@ -245,11 +246,17 @@ def gemm_shapes():
             B = (torch.randn((K, Nn) if bt else (Nn, K), device=dev) * 0.05).to(torch.bfloat16)
             sets.append((A, B, torch.empty(M, Nn, device=dev, dtype=torch.bfloat16)))
         flops = 2.0 * M * Nn * K
-        ours_us, ours_mhz = timed([(lambda s=s: N.gemm_bf16(s[0], s[1], s[2], a_trans=bool(at), b_trans=bool(bt)))
-                                   for s in sets], flops)
+        # as the stage lowers it: a long reduction into a small output goes through the k-split entry point
+        copies = 0 if (at or bt) else splitk_copies(M, Nn, K)
+        if copies:
+            ws = torch.empty(copies * M * Nn, device=dev)
+            ours = [(lambda s=s: N.gemm_bf16_splitk(s[0], s[1], s[2], ws)) for s in sets]
+        else:
+            ours = [(lambda s=s: N.gemm_bf16(s[0], s[1], s[2], a_trans=bool(at), b_trans=bool(bt))) for s in sets]
+        ours_us, ours_mhz = timed(ours, flops)
         lib_us, lib_mhz = timed([(lambda s=s: torch.matmul(s[0].t() if at else s[0], s[1] if bt else s[1].t(),
                                                            out=s[2])) for s in sets], flops)
-        print(json.dumps({"shape": [M, Nn, K], "a_trans": at, "b_trans": bt, "what": what,
+        print(json.dumps({"shape": [M, Nn, K], "a_trans": at, "b_trans": bt, "what": what, "k_splits": copies,
                           "us": round(ours_us, 1), "tflops": round(flops / ours_us / 1e6, 1),
                           "shader_mhz": round(ours_mhz), "vendor_us": round(lib_us, 1),
                           "vendor_tflops": round(flops / lib_us / 1e6, 1), "vendor_shader_mhz": round(lib_mhz)}),
@@ -385,7 +392,7 @@ def main():
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
                               "traffic": gemm_traffic()[0] if default_workload else None,
                               "traffic_source": gemm_traffic()[1] if default_workload else None,
-                              "kernel": "gemm_bf16_dma_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
+                              "kernel": "gemm_bf16_dma_kernel + gemm_bf16_dma8_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
                                         + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else "")
                                         + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else ""),
                               "launches_per_step": cnt // n_prof,

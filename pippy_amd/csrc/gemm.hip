@@ -39,32 +39,44 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_dma_kernel(const GemmA
     gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT>(g, tile_m, tile_n);
 }
 
+// The same tile on 8 waves (two per SIMD): each wave's part of the tile is half as large, and while one
+// wave of a SIMD waits for its fragments or at the barrier the other one's MFMAs run.
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
+__global__ __launch_bounds__(2 * kGemmThreads) void gemm_bf16_dma8_kernel(const GemmArgs g) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks) return;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT, 0, 8>(g, tile_m, tile_n);
+}
+
 // Split along K on 256 x 256 tiles, for an output with few tiles and a long reduction (the input
 // gradient of a vocabulary projection: 4096 x 768 with K = 50304).  Large tiles load half as many
 // operand bytes per FLOP as 128-wide ones, and the split makes enough of them to fill the CUs.
 // Split s of a tile reduces k-tiles [s * kt_per_split, (s + 1) * kt_per_split) into its own fp32
 // copy of C in the workspace; splitk_reduce_kernel adds the copies in split order.
-__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_splitk_kernel(const GemmArgs g, float* ws, int splits,
-                                                                       int kt_per_split) {
+__global__ __launch_bounds__(2 * kGemmThreads) void gemm_bf16_splitk_kernel(const GemmArgs g, float* ws, int splits,
+                                                                           int kt_per_split) {
     const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= g.n_blocks * (uint32_t)splits) return;
     const int split = (int)(bid / g.n_blocks);
     uint32_t tile_m, tile_n;
     grouped_tile(bid % g.n_blocks, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    f32x16_t acc[WaveTile<256, 256>::TN][WaveTile<256, 256>::TM];
+    typedef WaveTile<256, 256, 8> WT;  // 8 waves, as the 256 x 256 tiles of the single-problem kernel
+    f32x16_t acc[WT::TN][WT::TM];
 #pragma unroll
-    for (int a = 0; a < WaveTile<256, 256>::TN; ++a)
+    for (int a = 0; a < WT::TN; ++a)
 #pragma unroll
-        for (int b = 0; b < WaveTile<256, 256>::TM; ++b)
+        for (int b = 0; b < WT::TM; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
     const int nk = (int)((g.K + BK - 1) / BK);
     const int kb = min(nk, split * kt_per_split), ke = min(nk, kb + kt_per_split);
-    gemm_mainloop<256, 256, false, false, 2, BK>(g, tile_m, tile_n, kb, ke, acc);
+    gemm_mainloop<256, 256, false, false, 2, BK, false, 8>(g, tile_m, tile_n, kb, ke, acc);
     GemmArgs part = g;
     part.C = ws + (size_t)split * (size_t)g.M * (size_t)g.N;
     part.ldc = g.N;
-    gemm_epilogue<256, 256, PP_EPI_NONE, true>(part, tile_m, tile_n, acc);
+    gemm_epilogue<256, 256, PP_EPI_NONE, true, 0, 8>(part, tile_m, tile_n, acc);
 }
 
 // C (bf16) = ws[0] + ws[1] + ... + ws[splits - 1], added in that order; N and ldc multiples of 4.
@@ -180,7 +192,6 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_k_kernel(const Gem
 // Pipeline depth: with at most one tile per CU a block has the CU to itself and takes 3 stages;
 // with more tiles 2 stages leave room for two resident blocks, whose prologues and epilogues overlap
 // each other's main loops.
-constexpr int64_t kBigTileMinTiles = 1024;  // 256 x 256 tiles are used from this many of them
 
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
 static int launch_single(const GemmArgs& g, hipStream_t st) {
@@ -193,17 +204,33 @@ static int launch_single(const GemmArgs& g, hipStream_t st) {
     return check_launch("gemm_bf16_dma_kernel");
 }
 
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
+static int launch_single8(const GemmArgs& g, hipStream_t st) {
+    constexpr size_t lds = (size_t)NS * (BM + BN) * KT * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_dma8_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
+    if (attr_rc) return attr_rc;
+    const uint32_t grid = (g.n_blocks + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_dma8_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid),
+                       dim3(2 * kGemmThreads), lds, st, g);
+    return check_launch("gemm_bf16_dma8_kernel");
+}
+
 template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
 static int launch_gemm(const GemmArgs* probs, hipStream_t st) {
     {
         if constexpr (EPI == PP_EPI_NONE && !CF32 && BM == 128 && !AT && !BT) {
             // a large output with both operands k-contiguous: 256 x 256 tiles halve the LDS and L2
-            // traffic per MFMA (vocabulary projection 4096 x 50304 x 768: 776 against 707 TFLOP/s)
+            // traffic per MFMA; on 8 waves, so that every SIMD has a second wave to run while the first
+            // waits (vocabulary projection 4096 x 50304 x 768: 880 against 840 TFLOP/s on 4 waves and
+            // 710 on 128 x 128 tiles; 4096 x 4096 x 1024: 970 against 860).  Taken when the tiles fill at
+            // least four fifths of the rounds of 256 work-groups they need.
             GemmArgs big = probs[0];
-            if (((big.M + 255) / 256) * ((big.N + 255) / 256) >= kBigTileMinTiles) {
+            const int64_t t256 = ((big.M + 255) / 256) * ((big.N + 255) / 256);
+            const int64_t rounds = (t256 + kComputeUnits - 1) / kComputeUnits;
+            if (t256 >= kComputeUnits && 5 * t256 >= 4 * rounds * kComputeUnits) {
                 int rc = count_tiles<256, 256>(big);
                 if (rc) return rc;
-                return launch_single<256, 256, AT, BT, 2, EPI, CF32>(big, st);
+                return launch_single8<256, 256, AT, BT, 2, EPI, CF32>(big, st);
             }
         }
         if constexpr (BM == 128 && BN == 128 && !AT && !BT) {
@@ -387,7 +414,7 @@ extern "C" int pp_gemm_bf16_splitk(const pp_gemm_desc* d, float* workspace, int6
     if (attr_rc) return attr_rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t grid = (g.n_blocks * (uint32_t)splits + 7) / 8 * 8;
-    hipLaunchKernelGGL(gemm_bf16_splitk_kernel, dim3(grid), dim3(kGemmThreads), lds, st, g, workspace, splits,
+    hipLaunchKernelGGL(gemm_bf16_splitk_kernel, dim3(grid), dim3(2 * kGemmThreads), lds, st, g, workspace, splits,
                        kt_per_split);
     rc = check_launch("gemm_bf16_splitk_kernel");
     if (rc) return rc;

@@ -201,12 +201,13 @@ __device__ __forceinline__ void interleave_reads() {
     if constexpr (I + 1 < M) interleave_reads<R, M, I + 1>();
 }
 
-// How the 4 waves of a work-group share a BM x BN tile: 2 x 2 when BN is a multiple of 64, else 4 x 1
-// (a 128 x 96 tile: each wave 32 rows by 96 columns).  A wave's part is TM x TN MFMA tiles of 32 x 32.
-template <int BM, int BN>
+// How the W waves of a work-group share a BM x BN tile: two columns of waves when BN is a multiple of
+// 64 (4 waves: 2 x 2, 8 waves: 4 x 2), else one (a 128 x 96 tile: each of 4 waves 32 rows by 96
+// columns).  A wave's part is TM x TN MFMA tiles of 32 x 32.
+template <int BM, int BN, int W = 4>
 struct WaveTile {
     static constexpr int WGN = (BN % 64 == 0) ? 2 : 1;
-    static constexpr int WGM = 4 / WGN;
+    static constexpr int WGM = W / WGN;
     static constexpr int WTM = BM / WGM, WTN = BN / WGN;
     static constexpr int TM = WTM / 32, TN = WTN / 32;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "a wave's part of the tile is made of 32 x 32 MFMA tiles");
@@ -225,20 +226,20 @@ struct WaveTile {
 // so that it may follow an epilogue (or another main loop) that used the same LDS.
 // DUAL: the BN rows of the B tile are BN / 2 rows of g.B followed by the same BN / 2 rows of g.B2, so
 // that one tile holds two products of the same A rows (tile_n then counts blocks of BN / 2 rows).
-template <int BM, int BN, bool AT, bool BT, int NS, int KT, bool DUAL = false>
+template <int BM, int BN, bool AT, bool BT, int NS, int KT, bool DUAL = false, int W = 4>
 __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n, int kt_begin,
                                               int kt_end,
-                                              f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
-    typedef WaveTile<BM, BN> WT;
+                                              f32x16_t (&acc)[WaveTile<BM, BN, W>::TN][WaveTile<BM, BN, W>::TM]) {
+    typedef WaveTile<BM, BN, W> WT;
     constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     constexpr int KS = KT / 16;  // MFMA k-steps per tile
     constexpr int kStageElems = (BM + BN) * KT;
     // loads per tile per wave (the two half loaders of a DUAL tile issue as many as one whole loader)
-    constexpr int LPT = DmaStage<BM, AT, KT>::kLoads + DmaStage<BN, BT, KT>::kLoads;
+    constexpr int LPT = DmaStage<BM, AT, KT, W>::kLoads + DmaStage<BN, BT, KT, W>::kLoads;
     constexpr int kReadsPerStep = TM * FragReader<BM, AT, KT>::kReads + TN * FragReader<BN, BT, KT>::kReads;
     static_assert(NS >= 2 && NS <= 4 && (NS - 1) * LPT < 64, "pipeline depth exceeds vmcnt");
     static_assert(KS >= 2 && TN >= 2, "the last k-step is split in two parts around the barrier");
-    static_assert(NS * kStageElems * 2 >= 4 * 32 * WTN * 4, "the epilogue stages fp32 bands in the tile memory");
+    static_assert(NS * kStageElems * 2 >= W * 32 * WTN * 4, "the epilogue stages fp32 bands in the tile memory");
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -247,8 +248,8 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
 
     constexpr int BNL = DUAL ? BN / 2 : BN;  // rows that one loader of B brings
     static_assert(!DUAL || (!AT && !BT), "two products per tile: k-contiguous operands");
-    DmaStage<BM, AT, KT> sa;
-    DmaStage<BNL, BT, KT> sb, sb2;
+    DmaStage<BM, AT, KT, W> sa;
+    DmaStage<BNL, BT, KT, W> sb, sb2;
     sa.init(g.A, g.lda, m0, g.M, g.K, wave, lane);
     sb.init(g.B, g.ldb, DUAL ? n0 / 2 : n0, g.N, g.K, wave, lane);
     if (DUAL) sb2.init(g.B2, g.ldb, n0 / 2, g.N, g.K, wave, lane);
@@ -333,10 +334,10 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
 // Epilogue of one BM x BN tile: one band of 32 rows at a time goes through a wave-private LDS region
 // as fp32, [32][WTN] with the 16-byte unit index XORed by the row, and comes back with lanes running
 // along n, so that epilogue4 reads and writes whole lines.
-template <int BM, int BN, int EPI, bool CF32, int EB = 0>
+template <int BM, int BN, int EPI, bool CF32, int EB = 0, int W = 4>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
-                                              f32x16_t (&acc)[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM]) {
-    typedef WaveTile<BM, BN> WT;
+                                              f32x16_t (&acc)[WaveTile<BM, BN, W>::TN][WaveTile<BM, BN, W>::TM]) {
+    typedef WaveTile<BM, BN, W> WT;
     constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -447,17 +448,17 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
 }
 
 // One whole output tile: main loop over all of K, then the epilogue.
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK, int EB = 0>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK, int EB = 0, int W = 4>
 __device__ __forceinline__ void gemm_tile_dma(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n) {
-    f32x16_t acc[WaveTile<BM, BN>::TN][WaveTile<BM, BN>::TM];
+    f32x16_t acc[WaveTile<BM, BN, W>::TN][WaveTile<BM, BN, W>::TM];
 #pragma unroll
-    for (int a = 0; a < WaveTile<BM, BN>::TN; ++a)
+    for (int a = 0; a < WaveTile<BM, BN, W>::TN; ++a)
 #pragma unroll
-        for (int b = 0; b < WaveTile<BM, BN>::TM; ++b)
+        for (int b = 0; b < WaveTile<BM, BN, W>::TM; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
-    gemm_mainloop<BM, BN, AT, BT, NS, KT>(g, tile_m, tile_n, 0, (int)((g.K + KT - 1) / KT), acc);
-    gemm_epilogue<BM, BN, EPI, CF32, EB>(g, tile_m, tile_n, acc);
+    gemm_mainloop<BM, BN, AT, BT, NS, KT, false, W>(g, tile_m, tile_n, 0, (int)((g.K + KT - 1) / KT), acc);
+    gemm_epilogue<BM, BN, EPI, CF32, EB, W>(g, tile_m, tile_n, acc);
 }
 
 

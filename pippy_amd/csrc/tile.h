@@ -84,17 +84,18 @@ __device__ __forceinline__ void wait_vmcnt() {
 // s_waitcnt lgkmcnt(0): every LDS access of this wave has completed.
 __device__ __forceinline__ void wait_lds() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 
-template <int ROWS, bool TR, int KT = BK>
+// W waves (4 or 8) cooperate on a tile.
+template <int ROWS, bool TR, int KT = BK, int W = 4>
 struct DmaStage;
 
 // K-contiguous operand: memory [rows][ld]; LDS tile [ROWS][KT], chunk index XORed with swz_kt(row).
 // One wave load fills 1 KiB: 8 rows of 64 k or 16 rows of 32 k.
-template <int ROWS, int KT>
-struct DmaStage<ROWS, false, KT> {
+template <int ROWS, int KT, int W>
+struct DmaStage<ROWS, false, KT, W> {
     static constexpr int kChunks = KT / 8;              // 16-byte chunks per row
     static constexpr int kRowsPerLoad = 64 / kChunks;   // rows covered by one wave load
-    static constexpr int kLoads = ROWS / kRowsPerLoad / 4;
-    static_assert(ROWS % (kRowsPerLoad * 4) == 0, "tile rows must divide over the 4 waves' loads");
+    static constexpr int kLoads = ROWS / kRowsPerLoad / W;
+    static_assert(ROWS % (kRowsPerLoad * W) == 0, "tile rows must divide over the waves' loads");
     __amdgpu_buffer_rsrc_t rsrc;
     int voff[kLoads];
     int kcol[kLoads];  // first k of this lane's chunk within a tile
@@ -106,7 +107,7 @@ struct DmaStage<ROWS, false, KT> {
         K = (int)K_;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            const int row = (i * 4 + wave) * kRowsPerLoad + lane / kChunks;
+            const int row = (i * W + wave) * kRowsPerLoad + lane / kChunks;
             const int ch = (lane % kChunks) ^ swz_kt<KT>(row);
             voff[i] = (int)((row * ld + ch * 8) * 2);
             kcol[i] = ch * 8;
@@ -117,12 +118,12 @@ struct DmaStage<ROWS, false, KT> {
         if (k0 + KT <= K) {
 #pragma unroll
             for (int i = 0; i < kLoads; ++i)
-                load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i], k0 * 2);
+                load_to_lds_b128(rsrc, lds + (i * W + wave) * 512, voff[i], k0 * 2);
         } else {
             // k tail: chunks past K aim beyond the end of the buffer, which the range check zero-fills
 #pragma unroll
             for (int i = 0; i < kLoads; ++i)
-                load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512,
+                load_to_lds_b128(rsrc, lds + (i * W + wave) * 512,
                                  k0 + kcol[i] < K ? voff[i] + k0 * 2 : (int)0x7ffffff0, 0);
         }
     }
@@ -131,11 +132,11 @@ struct DmaStage<ROWS, false, KT> {
 // Transposed operand: memory [K][ld] with the tile's rows contiguous; LDS tile [KT][ROWS] as in
 // memory, the 16-byte chunk index of k-row k XORed with (k & 3) << 2 so that the four k-rows a
 // transposing read touches at once fall into different banks.
-template <int ROWS, int KT>
-struct DmaStage<ROWS, true, KT> {
+template <int ROWS, int KT, int W>
+struct DmaStage<ROWS, true, KT, W> {
     static constexpr int kChunksPerRow = ROWS / 8;
     static constexpr int kRowsPerLoad = 64 / kChunksPerRow;
-    static constexpr int kLoads = KT / kRowsPerLoad / 4;
+    static constexpr int kLoads = KT / kRowsPerLoad / W;
     static_assert(ROWS % 128 == 0 && ROWS <= 512, "transposed tiles are staged 128 rows at a time");
     static_assert(kLoads >= 1, "a wave load must not span more k-rows than a quarter of the tile");
     __amdgpu_buffer_rsrc_t rsrc;
@@ -148,7 +149,7 @@ struct DmaStage<ROWS, true, KT> {
         ld2 = (int)(ld * 2);
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            const int krow = (i * 4 + wave) * kRowsPerLoad + lane / kChunksPerRow;
+            const int krow = (i * W + wave) * kRowsPerLoad + lane / kChunksPerRow;
             const int ch = (lane % kChunksPerRow) ^ ((krow & 3) << 2);
             const bool valid = row0 + ch * 8 < rows_total;
             // k is part of the lane offset so that k-rows past K fail the range check and read as 0
@@ -158,7 +159,7 @@ struct DmaStage<ROWS, true, KT> {
     __device__ __forceinline__ void load(uint16_t* lds, int k0, int wave) const {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i)
-            load_to_lds_b128(rsrc, lds + (i * 4 + wave) * 512, voff[i] + k0 * ld2, 0);
+            load_to_lds_b128(rsrc, lds + (i * W + wave) * 512, voff[i] + k0 * ld2, 0);
     }
 };
 
