@@ -371,8 +371,10 @@ int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe,
 /* ------------------------------------------------------------------------------------------
  * Cross-entropy loss of one microbatch (loss_fn at pippy/PipelineSchedule.py:154-155 when it is
  * torch cross_entropy with mean reduction) fused with its gradient.
- * logits bf16 [rows, ld] (first V columns valid); target int64 [rows] (ignore_index skipped);
- * loss: fp32 [1]; dlogits bf16 [rows, ld] (columns >= V written as 0) or null (loss only);
+ * logits bf16 [rows, ld] (first V columns valid); target int64 [rows] (ignore_index skipped; so is a
+ * target outside [0, V), which torch rejects: callers that cannot trust their targets check them on the
+ * host); loss: fp32 [1], NaN when every row is skipped (the mean over no rows, as torch returns it; the
+ * gradient is zero then); dlogits bf16 [rows, ld] (columns >= V written as 0) or null (loss only);
  * workspace: fp32 [rows + 2].
  * ---------------------------------------------------------------------------------------- */
 int pp_ce_loss(const void* logits, const int64_t* target, float* loss, void* dlogits,

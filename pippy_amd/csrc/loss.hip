@@ -189,7 +189,8 @@ __global__ __launch_bounds__(256) void ce_row_f32_kernel(const float* __restrict
         dr[c] = (c < V) ? (expf(xr[c] - lse) - (c == t ? 1.0f : 0.0f)) * scale : 0.f;
 }
 
-// loss = (sum_r ws[r]) / count, summed in a fixed order
+// loss = (sum_r ws[r]) / count, summed in a fixed order; NaN when every row is ignored (the mean over no
+// rows, as torch.nn.functional.cross_entropy returns it; the gradient is zero then)
 __global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restrict__ ws, int64_t rows,
                                                           float* __restrict__ loss) {
     __shared__ float part[256];
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(256) void ce_finalize_kernel(const float* __restric
         if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
         __syncthreads();
     }
-    if (threadIdx.x == 0) loss[0] = part[0] * ws[rows + 1];
+    if (threadIdx.x == 0) loss[0] = ws[rows] > 0.f ? part[0] * ws[rows + 1] : __builtin_nanf("");
 }
 
 }  // namespace pp

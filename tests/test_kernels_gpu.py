@@ -496,6 +496,23 @@ def test_ce_loss_bf16_full_size_is_exact_per_element_and_repeatable(rows, V):
     assert torch.equal(inplace, runs[0][1])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_ce_loss_with_every_row_ignored_is_nan_with_zero_gradient(dtype):
+    """The mean over no rows: torch.nn.functional.cross_entropy returns NaN and a zero gradient."""
+    Nn = native()
+    rows, V = 24, 16
+    logits = torch.randn(rows, V, device=DEV).to(dtype)
+    target = torch.full((rows,), -100, device=DEV)
+    loss = torch.zeros(1, device=DEV)
+    dl = torch.full_like(logits, 7.0)
+    Nn.ce_loss(logits, target, loss, dl, torch.empty(rows + 2, device=DEV), V)
+    lr = logits.float().cpu().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(lr, target.cpu())
+    ref.backward()
+    assert torch.isnan(ref) and torch.isnan(loss).all()
+    assert float(lr.grad.abs().max()) == 0.0 and float(dl.float().abs().max()) == 0.0
+
+
 def test_ce_loss_f32():
     Nn = native()
     torch.manual_seed(11)
