@@ -256,10 +256,21 @@ def gemm_shapes():
         ours_us, ours_mhz = timed(ours, flops)
         lib_us, lib_mhz = timed([(lambda s=s: torch.matmul(s[0].t() if at else s[0], s[1] if bt else s[1].t(),
                                                            out=s[2])) for s in sets], flops)
+        # the per-layer shapes once more as 2 and 4 independent problems in one grouped launch: what the
+        # same-shaped GEMMs of several pipeline stages would cost each if the stages ran in lock step
+        grouped = {}
+        if flops < 3e10 and not copies:
+            for k in (2, 4):
+                more = [[(torch.randn_like(s[0]), torch.randn_like(s[1]) * 0.05, torch.empty_like(s[2]),
+                          dict(a_trans=bool(at), b_trans=bool(bt))) for _ in range(k)] for s in sets]
+                us_k, _ = timed([(lambda ps=ps: N.gemm_bf16_grouped(ps)) for ps in more], k * flops)
+                grouped[f"grouped{k}_us_each"] = round(us_k / k, 1)
+                del more
         print(json.dumps({"shape": [M, Nn, K], "a_trans": at, "b_trans": bt, "what": what, "k_splits": copies,
                           "us": round(ours_us, 1), "tflops": round(flops / ours_us / 1e6, 1),
                           "shader_mhz": round(ours_mhz), "vendor_us": round(lib_us, 1),
-                          "vendor_tflops": round(flops / lib_us / 1e6, 1), "vendor_shader_mhz": round(lib_mhz)}),
+                          "vendor_tflops": round(flops / lib_us / 1e6, 1), "vendor_shader_mhz": round(lib_mhz),
+                          **grouped}),
               flush=True)
         del sets
 
