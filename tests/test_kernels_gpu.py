@@ -534,7 +534,10 @@ def test_ce_loss_f32():
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,S,H,D", [(1, 128, 1, 64), (2, 256, 3, 64), (1, 1024, 2, 64),
                                      (1, 128, 1, 128), (2, 256, 3, 128), (1, 2048, 2, 128),
-                                     (1, 64, 2, 64), (2, 192, 1, 64), (1, 320, 2, 128), (3, 64, 1, 128)])
+                                     (1, 64, 2, 64), (2, 192, 1, 64), (1, 320, 2, 128), (3, 64, 1, 128),
+                                     # few work-groups, head dimension 64: key blocks of 128 on 8 waves, the last
+                                     # block half full when S is an odd multiple of 64
+                                     (2, 320, 2, 64), (1, 448, 3, 64)])
 def test_attention(causal, B, S, H, D):
     Nn = native()
     torch.manual_seed(12 + S)
