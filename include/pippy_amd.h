@@ -336,6 +336,9 @@ int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean, co
  * three can alias one fused [B, S, 3*H*D] projection output.  o: bf16 [B, S, H*D] contiguous.
  * lse: fp32 [B, H, S] (log-sum-exp of the scaled scores; saved for backward).
  * head_dim in {64, 128}; S % 64 == 0.
+ * Grouped-query attention: kv_group = G > 1 query heads share one key / value head, k and v (and dk,
+ * dv) then hold H / G heads, query head h reads key / value head h / G, and dk, dv are sums over the
+ * group (formed inside one work-group, in ascending query-head order); 0 or 1: one per query head.
  * ---------------------------------------------------------------------------------------- */
 typedef struct pp_attn_desc {
     const void* q; const void* k; const void* v;
@@ -347,6 +350,8 @@ typedef struct pp_attn_desc {
     int64_t stride_b, stride_s; /* of q/k/v (and dq/dk/dv), in elements */
     float scale;           /* usually 1/sqrt(D) */
     int32_t causal;
+    int32_t kv_group;      /* query heads per key / value head; 0 or 1: multi-head attention */
+    int32_t reserved;
 } pp_attn_desc;
 int pp_attn_fwd(const pp_attn_desc* desc, pp_stream stream);
 int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
@@ -405,7 +410,7 @@ enum pp_op_kind {
  *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
- *                 | j: causal
+ *                 | j: causal kv_group
  *   EMBED_FWD     p: ids wte wpe y extra_row | i: n_tok seq C vocab
  *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab | j: round_bf16
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype

@@ -72,14 +72,18 @@ def attention(q, k, v, causal, scale=None):
     return torch.matmul(torch.softmax(s, dim=-1), v)
 
 
-def attention_fused_qkv(qkv, H, causal):
-    """qkv: [B, S, 3*H*D] (q | k | v on the last dim) -> [B, S, H*D]."""
-    B, S, three = qkv.shape
-    HD = three // 3
-    D = HD // H
-    q, k, v = (t.reshape(B, S, H, D).transpose(1, 2) for t in qkv.split(HD, dim=-1))
+def attention_fused_qkv(qkv, H, causal, n_kv_heads=None):
+    """qkv: [B, S, (H + 2 H_kv) * D] (q | k | v on the last dim) -> [B, S, H*D].  With
+    ``n_kv_heads`` = H_kv < H (grouped-query attention) query heads g * H / H_kv .. (g + 1) * H / H_kv - 1
+    attend to key / value head g."""
+    B, S, width = qkv.shape
+    Hkv = H if n_kv_heads is None else n_kv_heads
+    D = width // (H + 2 * Hkv)
+    q, k, v = qkv.split([H * D, Hkv * D, Hkv * D], dim=-1)
+    q = q.reshape(B, S, H, D).transpose(1, 2)
+    k, v = (t.reshape(B, S, Hkv, D).transpose(1, 2).repeat_interleave(H // Hkv, dim=1) for t in (k, v))
     o = attention(q, k, v, causal)
-    return o.transpose(1, 2).reshape(B, S, HD)
+    return o.transpose(1, 2).reshape(B, S, H * D)
 
 
 def cross_entropy_mean(logits, target, ignore_index=-100):

@@ -77,7 +77,7 @@ class AttnDesc(C.Structure):
                 ("delta", C.c_void_p),
                 ("B", C.c_int64), ("S", C.c_int64), ("H", C.c_int64), ("D", C.c_int64),
                 ("stride_b", C.c_int64), ("stride_s", C.c_int64),
-                ("scale", C.c_float), ("causal", C.c_int32)]
+                ("scale", C.c_float), ("causal", C.c_int32), ("kv_group", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Op(C.Structure):
@@ -561,17 +561,22 @@ def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:
 # ---- attention --------------------------------------------------------------------------------
 def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, causal: bool,
               scale: Optional[float] = None, d_o: Optional[torch.Tensor] = None,
-              dqkv: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None) -> AttnDesc:
-    """qkv: [B, S, 3*H*D] fused projection output (q | k | v along the last dim)."""
+              dqkv: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
+              n_kv_heads: Optional[int] = None) -> AttnDesc:
+    """qkv: [B, S, (H + 2 H_kv) * D] fused projection output (q | k | v along the last dim);
+    ``n_kv_heads`` < H: grouped-query attention (H / n_kv_heads query heads per key / value head)."""
     require_cuda(qkv, o, lse, d_o, dqkv, delta)
-    B, S, three_hd = qkv.shape
-    HD = three_hd // 3
-    D = HD // H
+    B, S, width = qkv.shape
+    Hkv = H if n_kv_heads is None else n_kv_heads
+    assert 0 < Hkv <= H and H % Hkv == 0 and width % (H + 2 * Hkv) == 0
+    D = width // (H + 2 * Hkv)
+    HD, KD = H * D, Hkv * D
     assert qkv.stride(2) == 1 and o.is_contiguous() and o.shape == (B, S, HD)
     es = qkv.element_size()
     d = AttnDesc()
     base = qkv.data_ptr()
-    d.q, d.k, d.v = base, base + HD * es, base + 2 * HD * es
+    d.q, d.k, d.v = base, base + HD * es, base + (HD + KD) * es
+    d.kv_group = H // Hkv
     d.o, d.lse = o.data_ptr(), lse.data_ptr()
     d.B, d.S, d.H, d.D = B, S, H, D
     d.stride_b, d.stride_s = qkv.stride(0), qkv.stride(1)
@@ -582,18 +587,18 @@ def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, cau
         assert dqkv.shape == qkv.shape and dqkv.stride() == qkv.stride() and d_o.is_contiguous()
         gb = dqkv.data_ptr()
         d.d_o = d_o.data_ptr()
-        d.dq, d.dk, d.dv = gb, gb + HD * es, gb + 2 * HD * es
+        d.dq, d.dk, d.dv = gb, gb + HD * es, gb + (HD + KD) * es
         d.delta = delta.data_ptr()
     return d
 
 
-def attn_fwd(qkv, o, lse, H, causal, scale=None) -> None:
-    d = attn_desc(qkv, o, lse, H, causal, scale)
+def attn_fwd(qkv, o, lse, H, causal, scale=None, n_kv_heads=None) -> None:
+    d = attn_desc(qkv, o, lse, H, causal, scale, n_kv_heads=n_kv_heads)
     check(lib().pp_attn_fwd(C.byref(d), current_stream()), "pp_attn_fwd")
 
 
-def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None) -> None:
-    d = attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta)
+def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None, n_kv_heads=None) -> None:
+    d = attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads)
     check(lib().pp_attn_bwd(C.byref(d), current_stream()), "pp_attn_bwd")
 
 

@@ -439,8 +439,8 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
     return op
 
 
-def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None) -> N.Op:
-    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta)
+def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None) -> N.Op:
+    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads)
     op = N.Op()
     op.kind = kind
     for k, v in enumerate((d.q, d.k, d.v, d.o, d.lse, d.d_o, d.dq, d.dk, d.dv, d.delta)):
@@ -448,6 +448,7 @@ def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None) -> N.
     op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5] = d.B, d.S, d.H, d.D, d.stride_b, d.stride_s
     op.f[0] = d.scale
     op.j[0] = d.causal
+    op.j[1] = d.kv_group
     return op
 
 

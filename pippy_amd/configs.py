@@ -67,10 +67,11 @@ class LlamaStage(nn.Module):
     incoming activations ``[batch, seq, dim]`` (no embedding, no head)."""
 
     def __init__(self, n_layers=8, dim=4096, n_heads=32, ffn=11008, eps=1e-5, rope_theta=1e4,
-                 dtype=torch.bfloat16):
+                 dtype=torch.bfloat16, n_kv_heads=None):
         super().__init__()
         self.layers = nn.ModuleList([
-            LlamaLayer(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype) for _ in range(n_layers)])
+            LlamaLayer(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype, n_kv_heads=n_kv_heads)
+            for _ in range(n_layers)])
 
     def forward(self, x):
         for layer in self.layers:

@@ -36,6 +36,7 @@ struct AttnArgs {
     uint16_t* dq; uint16_t* dk; uint16_t* dv;
     float* delta;
     int64_t B, S, H, D, stride_b, stride_s;
+    int64_t G;  // query heads per key / value head (1: multi-head attention)
     float scale;
 };
 
@@ -76,13 +77,14 @@ struct AttnTileLoader {
             voff[i] = row * row_bytes + (((lane & 7) ^ swz_attn(row)) << 4);
         }
     }
-    __device__ __forceinline__ void load(uint16_t* lds, int64_t row0, int wave) const {
+    // `extra_bytes` shifts the columns (another head of the same rows)
+    __device__ __forceinline__ void load(uint16_t* lds, int64_t row0, int wave, int extra_bytes = 0) const {
 #pragma unroll
         for (int s = 0; s < DS; ++s)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
                 load_to_lds_b128(rsrc, lds + s * kTile + (i * 4 + wave) * 512, voff[i] + s * 128,
-                                 (int)row0 * row_bytes);
+                                 (int)row0 * row_bytes + extra_bytes);
     }
 };
 
@@ -207,8 +209,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
     // the 64-row tiles of a block are loaded by sets of four waves: waves 4 .. 7 take the second 64 keys
     const int lset = wave >> 2, lwave = wave & 3;
     AttnTileLoader<DS> lk, lv;
-    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, lwave, lane);
-    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, lwave, lane);
+    lk.init(a.k + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, lwave, lane);
+    lv.init(a.v + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, lwave, lane);
     const int64_t n_keys = CAUSAL ? q0 + 64 : a.S;
     const int64_t n_blocks = (n_keys + KB - 1) / KB;
     // LDS layout of an operand: [64-key tile of the block][64 columns of d] tiles of 64 x 64
@@ -381,14 +383,17 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     const int l32 = lane & 31, lh = lane >> 5;
     const uint32_t nx = (uint32_t)(a.S / 64);
     uint32_t bh, ord;
-    if (!attn_block_of(blockIdx.x, gridDim.x, nx, (uint32_t)(a.H * a.B), CAUSAL, &bh, &ord)) return;
-    const int64_t b = bh / a.H, h = bh % a.H;
+    // a work-group owns 64 keys of one key / value head and walks the query blocks of every query head
+    // of its group, one head after the other
+    const int64_t Hkv = a.H / a.G;
+    if (!attn_block_of(blockIdx.x, gridDim.x, nx, (uint32_t)(Hkv * a.B), CAUSAL, &bh, &ord)) return;
+    const int64_t b = bh / Hkv, hk = bh % Hkv, h = hk * a.G;  // h: first query head of the group
     const int64_t kv0 = (int64_t)ord * 64;  // early key blocks see the most queries
     const int64_t kvw0 = kv0 + 32 * grp;
     const int64_t kvi = kvw0 + l32;  // this lane's key row
 
-    const uint16_t* kp = a.k + b * a.stride_b + h * D;
-    const uint16_t* vp = a.v + b * a.stride_b + h * D;
+    const uint16_t* kp = a.k + b * a.stride_b + hk * D;
+    const uint16_t* vp = a.v + b * a.stride_b + hk * D;
     const int64_t ldo = a.H * D;
     AttnTileLoader<DS> lq, ldo_;
     lq.init(a.q + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
@@ -396,16 +401,23 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     // waves 0 and 2 fetch lse, waves 1 and 3 delta (the same values twice: every wave issues the
     // same number of loads, which keeps the vmcnt arithmetic uniform)
     const float* stat = ((wave & 1) ? a.delta : a.lse) + (b * a.H + h) * a.S;
-    const __amdgpu_buffer_rsrc_t rstat = make_rsrc(stat, (uint64_t)a.S * 4);
+    const __amdgpu_buffer_rsrc_t rstat = make_rsrc(stat, (uint64_t)a.G * (uint64_t)a.S * 4);
     const int stat_off = 2 * kOperand + ((wave & 1) ? 128 : 0);
 
-    const int64_t jq_begin = CAUSAL ? kv0 / 64 : 0;
-    const int64_t nb = a.S / 64 - jq_begin;
-    auto issue = [&](int stage, int64_t j) {
+    const int jq_begin = CAUSAL ? (int)(kv0 / 64) : 0;
+    const int nb_head = (int)(a.S / 64) - jq_begin;  // query blocks that see these keys, per query head
+    const int64_t nb = a.G * nb_head;                // steps: the blocks of head 0 of the group, of head 1, ...
+    int iss_g = 0, iss_b = 0;                        // head and block of the next step to be issued
+    auto issue = [&](int stage, int64_t) {           // steps are issued in order
         uint16_t* st = lds + stage * kStage;
-        lq.load(st, (jq_begin + j) * 64, wave);
-        ldo_.load(st + kOperand, (jq_begin + j) * 64, wave);
-        load_floats_to_lds(rstat, reinterpret_cast<float*>(st + stat_off), (jq_begin + j) * 64, lane);
+        const int row0 = (jq_begin + iss_b) * 64;
+        lq.load(st, row0, wave, iss_g * D * 2);
+        ldo_.load(st + kOperand, row0, wave, iss_g * D * 2);
+        load_floats_to_lds(rstat, reinterpret_cast<float*>(st + stat_off), iss_g * (int)a.S + row0, lane);
+        if (++iss_b == nb_head) {
+            iss_b = 0;
+            ++iss_g;
+        }
     };
 
     bf16x8_t kf[KS], vf[KS];
@@ -430,9 +442,10 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
 
     // (not unrolled by the number of stages as the other two kernels are: the per-lane offsets of its 24
     // fragment reads per block would not fit the register budget of three work-groups per CU)
-    int stage = 0;
+    int stage = 0, cur_b = 0;  // cur_b: block of the current step within its head
     for (int64_t j = 0; j < nb; ++j) {
-        const int64_t qc0 = (jq_begin + j) * 64;
+        const int64_t qc0 = (int64_t)(jq_begin + cur_b) * 64;
+        cur_b = cur_b + 1 == nb_head ? 0 : cur_b + 1;
         await_block<4 * DS + 1, NS>(j, nb);
         if (j + NS - 1 < nb) issue(stage == 0 ? NS - 1 : stage - 1, j + NS - 1);
         const uint16_t* Qs = lds + stage * kStage;
@@ -517,8 +530,8 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     }
     if (half != 0) return;
     // dvacc[dt][v]: d = 32 dt + 8 (v/4) + 4 lh + v%4, kv = kvi
-    uint16_t* dkp = a.dk + b * a.stride_b + h * D + kvi * a.stride_s;
-    uint16_t* dvp = a.dv + b * a.stride_b + h * D + kvi * a.stride_s;
+    uint16_t* dkp = a.dk + b * a.stride_b + hk * D + kvi * a.stride_s;
+    uint16_t* dvp = a.dv + b * a.stride_b + hk * D + kvi * a.stride_s;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -558,8 +571,8 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
     const int64_t ldo = a.H * D;
     const uint16_t* dop = a.d_o + b * a.S * ldo + h * D;
     AttnTileLoader<DS> lk, lv;
-    lk.init(a.k + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
-    lv.init(a.v + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
+    lk.init(a.k + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, wave, lane);
+    lv.init(a.v + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, wave, lane);
     const int64_t n_blocks = CAUSAL ? q0 / 64 + 1 : a.S / 64;
     auto issue = [&](int stage, int64_t j) {
         lk.load(lds + stage * kStage, j * 64, wave);
@@ -686,6 +699,8 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
     if (d->D != 64 && d->D != 128)
         return fail(PP_ERR_UNSUPPORTED, "%s: head_dim %lld (64 and 128 are built)", who, (long long)d->D);
     if (d->S % 64) return fail(PP_ERR_UNSUPPORTED, "%s: S %% 64 != 0 (S=%lld)", who, (long long)d->S);
+    if (d->kv_group < 0 || (d->kv_group > 1 && d->H % d->kv_group))
+        return fail(PP_ERR_INVALID, "%s: kv_group %d does not divide H = %lld", who, d->kv_group, (long long)d->H);
     if ((d->stride_s % 8) || (d->stride_b % 8)) return fail(PP_ERR_INVALID, "%s: strides must be multiples of 8", who);
     if (d->stride_s < d->H * d->D) return fail(PP_ERR_INVALID, "%s: stride_s < H*D", who);
     if (!d->q || !d->k || !d->v || !d->o || !d->lse) return fail(PP_ERR_INVALID, "%s: null pointer", who);
@@ -709,6 +724,7 @@ static AttnArgs to_args(const pp_attn_desc* d) {
     a.delta = d->delta;
     a.B = d->B; a.S = d->S; a.H = d->H; a.D = d->D;
     a.stride_b = d->stride_b; a.stride_s = d->stride_s;
+    a.G = d->kv_group > 1 ? d->kv_group : 1;
     a.scale = d->scale;
     return a;
 }
@@ -758,15 +774,17 @@ template <int D>
 static int attn_bwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
     // the dQ kernel goes first: it also computes delta = rowsum(dO * O), which the dK / dV kernel reads
     const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false);
+    // one work-group per 64 keys of a key / value head
+    const dim3 grid_kv((uint32_t)(((d->S / 64) * (d->H / a.G) * d->B + 7) / 8 * 8));
     int rc;
     if (d->causal) {
         rc = attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
         if (rc) return rc;
-        return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid, 256, lds_kv, st, a);
+        return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid_kv, 256, lds_kv, st, a);
     }
     rc = attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
     if (rc) return rc;
-    return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid, 256, lds_kv, st, a);
+    return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid_kv, 256, lds_kv, st, a);
 }
 
 }  // namespace pp

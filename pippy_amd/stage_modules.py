@@ -483,17 +483,23 @@ class LlamaLayer(NativeBlock):
     """One Llama-style decoder layer: RMSNorm, causal self-attention with rotary position embedding
     on a fused q|k|v projection, RMSNorm, SwiGLU feed-forward; no biases.  Parameter names follow the
     Hugging Face layer (``input_layernorm``, ``self_attn.o_proj``, ``post_attention_layernorm``,
-    ``mlp.gate_proj / up_proj / down_proj``) except for the fused ``self_attn.qkv_proj``."""
+    ``mlp.gate_proj / up_proj / down_proj``) except for the fused ``self_attn.qkv_proj``, whose rows are
+    the query heads, then the key heads, then the value heads.  ``n_kv_heads`` < ``n_heads`` makes it
+    grouped-query attention (``num_key_value_heads`` of the Hugging Face configuration): every
+    ``n_heads / n_kv_heads`` consecutive query heads share one key / value head."""
 
     def __init__(self, dim: int, n_heads: int, ffn: int, *, eps: float = 1e-5, rope_theta: float = 1e4,
-                 dtype=torch.bfloat16, init_std=0.02):
+                 dtype=torch.bfloat16, init_std=0.02, n_kv_heads: Optional[int] = None):
         super().__init__()
         assert dim % n_heads == 0 and (dim // n_heads) in (64, 128), "head dimension 64 or 128"
         self.dim, self.n_heads, self.ffn = dim, n_heads, ffn
+        self.n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
+        assert 0 < self.n_kv_heads <= n_heads and n_heads % self.n_kv_heads == 0, "n_kv_heads must divide n_heads"
         self.eps, self.rope_theta = eps, rope_theta
         self.input_layernorm = nn.RMSNorm(dim, eps=eps, dtype=dtype)
         self.self_attn = nn.Module()
-        self.self_attn.qkv_proj = nn.Linear(dim, 3 * dim, bias=False, dtype=dtype)
+        self.self_attn.qkv_proj = nn.Linear(dim, (n_heads + 2 * self.n_kv_heads) * (dim // n_heads), bias=False,
+                                            dtype=dtype)
         self.self_attn.o_proj = nn.Linear(dim, dim, bias=False, dtype=dtype)
         self.post_attention_layernorm = nn.RMSNorm(dim, eps=eps, dtype=dtype)
         self.mlp = nn.Module()
@@ -507,11 +513,15 @@ class LlamaLayer(NativeBlock):
     # torch statement of the layer
     def forward(self, x):
         Bn, S, Cc = x.shape
-        H, D = self.n_heads, Cc // self.n_heads
+        H, Hkv, D = self.n_heads, self.n_kv_heads, Cc // self.n_heads
         cos, sin = rope_tables(S, D, self.rope_theta, x.device)
         h = self.input_layernorm(x)
-        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self.self_attn.qkv_proj(h).split(Cc, dim=-1))
+        q, k, v = self.self_attn.qkv_proj(h).split([H * D, Hkv * D, Hkv * D], dim=-1)
+        q = q.reshape(Bn, S, H, D).transpose(1, 2)
+        k, v = (t.reshape(Bn, S, Hkv, D).transpose(1, 2) for t in (k, v))
         q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
+        if Hkv != H:  # query heads g * (H / Hkv) .. share key / value head g
+            k, v = (t.repeat_interleave(H // Hkv, dim=1) for t in (k, v))
         o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
         x = x + self.self_attn.o_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
         return x + self._feed_forward(self.post_attention_layernorm(x))
@@ -524,8 +534,9 @@ class LlamaLayer(NativeBlock):
             raise RuntimeError(f"{type(self).__name__} of width {self.dim} expects [batch, seq, dim], got "
                                f"{tuple(x.shape)}")
         Bn, S, Cc = x.shape
-        T, H = Bn * S, self.n_heads
+        T, H, Hkv = Bn * S, self.n_heads, self.n_kv_heads
         D = Cc // H
+        W = (H + 2 * Hkv) * D  # width of the fused projection
         x2d = x.view(T, Cc)
         cos = b.sp.shared(f"rope_cos:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
         sin = b.sp.shared(f"rope_sin:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
@@ -534,22 +545,22 @@ class LlamaLayer(NativeBlock):
         sin.copy_(s_)
         n1, rstd1 = lower_rmsnorm(b, "n1", self.input_layernorm, x2d)
         qkv, _ = lower_linear(b, "qkv", self.self_attn.qkv_proj, n1)
-        b.f(P.op_rope(qkv, cos, sin, S, 2 * H, D))
+        b.f(P.op_rope(qkv, cos, sin, S, H + Hkv, D))
         att = b.act("att", (T, Cc))
         lse = b.act("lse", (Bn, H, S), torch.float32)
-        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, True))
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, True, n_kv_heads=Hkv))
         x2, _ = lower_linear(b, "x2", self.self_attn.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         y, ffn_backward = self._lower_feed_forward(b, x2)
 
         def bwd(dy, need_dx, dx_out):
             d_x2 = ffn_backward(dy.view(T, Cc))
             d_att = linear_backward(b, "o", self.self_attn.o_proj, att, d_x2)
-            dqkv = b.grad("dqkv", (T, 3 * Cc))
+            dqkv = b.grad("dqkv", (T, W))
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
-            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, True,
-                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, True,
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv))
             # gradients w.r.t. the rotated q and k go back through the transposed rotation
-            b.i(P.op_rope(dqkv, cos, sin, S, 2 * H, D, inverse=True))
+            b.i(P.op_rope(dqkv, cos, sin, S, H + Hkv, D, inverse=True))
             d_n1 = linear_backward(b, "qkv", self.self_attn.qkv_proj, n1, dqkv)
             dx = rmsnorm_backward(b, "n1", self.input_layernorm, x2d, rstd1, d_n1, dres=d_x2,
                                   dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
@@ -641,8 +652,9 @@ class MoELayer(LlamaLayer):
     TOPK = 2
 
     def __init__(self, dim: int, n_heads: int, ffn: int, n_experts: int = 8, *, eps: float = 1e-5,
-                 rope_theta: float = 1e6, dtype=torch.bfloat16, init_std=0.02):
-        super().__init__(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype, init_std=init_std)
+                 rope_theta: float = 1e6, dtype=torch.bfloat16, init_std=0.02, n_kv_heads: Optional[int] = None):
+        super().__init__(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype, init_std=init_std,
+                         n_kv_heads=n_kv_heads)
         del self.mlp
         assert 2 <= n_experts <= 64
         self.n_experts = n_experts

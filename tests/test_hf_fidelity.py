@@ -116,11 +116,14 @@ def _llama_position_embeddings(cfg, x, S):
     return LlamaRotaryEmbedding(cfg)(x, torch.arange(S)[None])
 
 
-def test_llama_layer_is_a_llama_decoder_layer():
+@pytest.mark.parametrize("heads,kv_heads", [(2, 2), (4, 2), (4, 1)])
+def test_llama_layer_is_a_llama_decoder_layer(heads, kv_heads):
+    """Multi-head and grouped-query attention (``num_key_value_heads`` < ``num_attention_heads``: which
+    query heads share which key / value head is pinned here)."""
     from transformers import LlamaConfig
     from transformers.models.llama.modeling_llama import LlamaDecoderLayer
-    dim, heads, ffn, S, theta = 128, 2, 192, 24, 1e4
-    cfg = LlamaConfig(hidden_size=dim, num_attention_heads=heads, num_key_value_heads=heads,
+    dim, ffn, S, theta = 64 * heads, 192, 24, 1e4
+    cfg = LlamaConfig(hidden_size=dim, num_attention_heads=heads, num_key_value_heads=kv_heads,
                       intermediate_size=ffn, num_hidden_layers=1, rms_norm_eps=1e-5, rope_theta=theta,
                       max_position_embeddings=64, vocab_size=32, attention_dropout=0.0, hidden_act="silu")
     if getattr(cfg, "rope_parameters", None) is not None:
@@ -130,7 +133,7 @@ def test_llama_layer_is_a_llama_decoder_layer():
     torch.manual_seed(3)
     for p in hf.parameters():
         torch.nn.init.normal_(p, std=0.1)
-    mine = SM.LlamaLayer(dim, heads, ffn, eps=1e-5, rope_theta=theta, dtype=torch.float32)
+    mine = SM.LlamaLayer(dim, heads, ffn, eps=1e-5, rope_theta=theta, dtype=torch.float32, n_kv_heads=kv_heads)
     sd = hf.state_dict()
     with torch.no_grad():
         mine.self_attn.qkv_proj.weight.copy_(torch.cat([sd["self_attn.q_proj.weight"], sd["self_attn.k_proj.weight"],

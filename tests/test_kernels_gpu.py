@@ -563,6 +563,54 @@ def test_attention(causal, B, S, H, D):
         assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"attention {name}")
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,S,H,Hkv,D", [(2, 256, 4, 2, 64), (1, 192, 8, 2, 128), (1, 1024, 8, 1, 64),
+                                         (2, 128, 6, 3, 64), (1, 64, 16, 8, 64)])
+def test_grouped_query_attention(causal, B, S, H, Hkv, D):
+    """H query heads on Hkv key / value heads (q | k | v = H, Hkv, Hkv heads of the fused projection):
+    the gradients of a key / value head are the sums over its group of query heads."""
+    Nn = native()
+    torch.manual_seed(S + H + Hkv)
+    W = (H + 2 * Hkv) * D
+    qkv = torch.randn(B, S, W, device=DEV).to(torch.bfloat16)
+    o = torch.full((B, S, H * D), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    note(f"grouped-query attention B={B} S={S} H={H} Hkv={Hkv} D={D} causal={causal}")
+    Nn.attn_fwd(qkv, o, lse, H, causal, n_kv_heads=Hkv)
+    torch.cuda.synchronize()
+    qr = qkv.float().cpu().requires_grad_(True)
+    ref = O.attention_fused_qkv(qr, H, causal, n_kv_heads=Hkv)
+    assert_close_rel(o, ref, BF16_TOL, "attention fwd")
+    d_o = torch.randn(B, S, H * D, device=DEV).to(torch.bfloat16)
+    dqkv = torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, n_kv_heads=Hkv)
+    torch.cuda.synchronize()
+    ref.backward(d_o.float().cpu())
+    HD, KD = H * D, Hkv * D
+    for name, sl in (("dq", slice(0, HD)), ("dk", slice(HD, HD + KD)), ("dv", slice(HD + KD, HD + 2 * KD))):
+        assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"attention {name}")
+    # one key / value head per query head written out by hand gives the same bits as the grouping:
+    # the grouped form only shares the loads
+    if H <= 8:
+        G = H // Hkv
+        k_rep = qkv[..., HD:HD + KD].view(B, S, Hkv, D).repeat_interleave(G, dim=2).reshape(B, S, HD)
+        v_rep = qkv[..., HD + KD:].view(B, S, Hkv, D).repeat_interleave(G, dim=2).reshape(B, S, HD)
+        full = torch.cat([qkv[..., :HD], k_rep, v_rep], dim=-1).contiguous()
+        o2 = torch.empty_like(o)
+        lse2 = torch.empty_like(lse)
+        Nn.attn_fwd(full, o2, lse2, H, causal)
+        assert torch.equal(o2, o) and torch.equal(lse2, lse)
+
+
+def test_grouped_query_attention_rejects_a_group_that_does_not_divide_the_heads():
+    Nn = native()
+    qkv = torch.zeros(1, 64, (6 + 2 * 4) * 64, device=DEV, dtype=torch.bfloat16)
+    o = torch.zeros(1, 64, 6 * 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        Nn.attn_fwd(qkv, o, torch.zeros(1, 6, 64, device=DEV), 6, True, n_kv_heads=4)
+
+
 @pytest.mark.parametrize("B,S,H,D,causal", [(4, 1024, 12, 64, True), (8, 512, 12, 64, False),
                                            (1, 2048, 32, 128, True)])
 def test_attention_full_size_with_equal_keys_is_a_running_mean(B, S, H, D, causal):

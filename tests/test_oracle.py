@@ -54,6 +54,17 @@ def test_attention_matches_sdpa_and_brute_force(causal):
     # fused-qkv layout is the same function
     qkv = torch.cat([t.transpose(1, 2).reshape(2, 9, 12) for t in (q, k, v)], dim=-1)
     assert torch.allclose(O.attention_fused_qkv(qkv, 3, causal), ref.transpose(1, 2).reshape(2, 9, 12), atol=1e-12)
+    # grouped-query attention: 4 query heads on 2 key / value heads, against torch's own grouping and
+    # against the head-by-head statement (query head h uses key / value head h // 2)
+    q4 = torch.randn(2, 4, 9, 4, dtype=torch.float64)
+    k2, v2 = (torch.randn(2, 2, 9, 4, dtype=torch.float64) for _ in range(2))
+    ref_g = F.scaled_dot_product_attention(q4, k2, v2, is_causal=causal, enable_gqa=True)
+    by_head = torch.stack([O.attention(q4[:, h:h + 1], k2[:, h // 2:h // 2 + 1], v2[:, h // 2:h // 2 + 1], causal)[:, 0]
+                           for h in range(4)], dim=1)
+    assert torch.allclose(ref_g, by_head, atol=1e-12)
+    qkv_g = torch.cat([t.transpose(1, 2).reshape(2, 9, -1) for t in (q4, k2, v2)], dim=-1)
+    assert torch.allclose(O.attention_fused_qkv(qkv_g, 4, causal, n_kv_heads=2),
+                          ref_g.transpose(1, 2).reshape(2, 9, 16), atol=1e-12)
 
 
 def test_cross_entropy_matches_torch_with_ignore_index():

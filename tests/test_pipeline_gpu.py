@@ -578,6 +578,34 @@ def test_llama_fused_feed_forward_follows_parameter_updates_and_launches_fused_k
     _llama_grads_match(model, ref, losses, ref_losses, ref_out, upstream)
 
 
+@pytest.mark.parametrize("n_heads,n_kv_heads,dim", [(4, 2, 256), (4, 1, 256), (2, 1, 256)])
+def test_llama_grouped_query_attention_two_stages_matches_oracle(n_heads, n_kv_heads, dim):
+    """Llama-style layers whose query heads share key / value heads (head dimension 64 and 128), split
+    into two traced stages under 1F1B: the fused projection is narrower (q | k | v = H, Hkv, Hkv heads),
+    the rotary embedding covers H + Hkv heads, and a key / value head's gradient sums over its group."""
+    import pippy_amd as pp
+    import torch.nn as nn
+    from pippy_amd.configs import LlamaStage
+    torch.manual_seed(2)
+    M, S = 2, 128
+    model = LlamaStage(n_layers=2, dim=dim, n_heads=n_heads, ffn=256, n_kv_heads=n_kv_heads)
+    assert model.layers[0].self_attn.qkv_proj.weight.shape[0] == (n_heads + 2 * n_kv_heads) * (dim // n_heads)
+    ref = _fp32_cpu_copy(model)
+    x = torch.randn(2 * M, S, dim).to(torch.bfloat16)
+    upstream = torch.randn(2 * M, S, dim) * 1e-2
+    pipe = pp.pipeline(model, M, (x,), split_spec={"layers.1": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert all(st.is_native for st in stages)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=_upstream_loss)
+    losses = []
+    out = sched.step(x.to(DEV), target=upstream.to(DEV), losses=losses)
+    ref_stages = [nn.Sequential(ref.layers[0]), nn.Sequential(ref.layers[1])]
+    ref_out, ref_losses = OP.step(ref_stages, x.float(), upstream, M, _upstream_loss)
+    assert_close_rel(out, ref_out, BF16_TOL, "stage output")
+    worst = _llama_grads_match(model, ref, losses, ref_losses, ref_out, upstream)
+    note(f"Llama layers with {n_heads} query / {n_kv_heads} key-value heads: worst grad error {worst:.3e}")
+
+
 def test_llama_two_stages_1f1b_hand_off_matches_oracle():
     """The same layers split into two traced stages: the input gradient of the second stage (through
     RMSNorm, rotary embedding and attention backward) feeds the first."""
