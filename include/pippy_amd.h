@@ -268,6 +268,8 @@ int pp_gemm_bf16_dswiglu(const void* dy, const void* w_down_t, const void* gu, v
  *   pp_moe_permute: expert_of_slot [n_slots] -> seg_start [E + 1] (first row of every expert;
  *     seg_start[E] = rows placed), row_src [n_slots] (flat slot of every row), pos [n_slots] (row
  *     of every flat slot; -1 and dropped for an expert id outside [0, E)).  E <= 64.
+ *   (pp_moe_gate_bwd writes the columns [E, round_up(E, 8)) of dlogits as zeros: a router whose expert
+ *   count is not a multiple of 8 runs its GEMMs on logits padded to one.)
  *   pp_moe_gather: dst[r, :] = scale[f] * src[f / topk, :] with f = row_src[r] for r < *n_rows_dev
  *     (null: r < R); scale null = plain gather.  Tokens -> expert rows, and the weighted
  *     scatter of the output gradient in the backward pass.

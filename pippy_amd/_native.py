@@ -423,7 +423,7 @@ def moe_gate_bwd(dout, y, pos, topk_idx, gate, E: int, dlogits) -> None:
     require_cuda(dout, y, pos, topk_idx, gate, dlogits)
     T, Cc = dout.shape
     topk = pos.numel() // T
-    assert dlogits.shape == (T, E) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
+    assert dlogits.shape == (T, (E + 7) // 8 * 8) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
     check(lib().pp_moe_gate_bwd(dout.data_ptr(), dout.stride(0), y.data_ptr(), y.stride(0), pos.data_ptr(),
                                 topk_idx.data_ptr(), gate.data_ptr(), topk, E, dlogits.data_ptr(),
                                 dlogits.stride(0), T, Cc, current_stream()), "pp_moe_gate_bwd")

@@ -334,9 +334,11 @@ def op_gemm_seg(mode, A, ptr_list, seg_start, *, Cm=None, other=None, n_cols=Non
     return op
 
 
-def op_moe_router(logits, topk_idx, gate) -> N.Op:
-    T, E = logits.shape
-    assert logits.dtype == torch.bfloat16 and logits.stride(1) == 1
+def op_moe_router(logits, topk_idx, gate, E=None) -> N.Op:
+    """``E``: number of experts when ``logits`` carries padding columns after them."""
+    T = logits.shape[0]
+    E = logits.shape[1] if E is None else E
+    assert logits.dtype == torch.bfloat16 and logits.stride(1) == 1 and E <= logits.shape[1]
     assert topk_idx.dtype == torch.int32 and topk_idx.numel() == 2 * T and topk_idx.is_contiguous()
     assert gate.dtype == torch.float32 and gate.numel() == 2 * T and gate.is_contiguous()
     op = N.Op()
@@ -387,7 +389,7 @@ def op_moe_combine(y, pos, topk, out, gate=None, resid=None) -> N.Op:
 def op_moe_gate_bwd(dout, y, pos, topk_idx, gate, E, dlogits) -> N.Op:
     T, Cc = dout.shape
     topk = pos.numel() // T
-    assert dlogits.shape == (T, E) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
+    assert dlogits.shape == (T, (E + 7) // 8 * 8) and dlogits.dtype == torch.bfloat16 and dlogits.stride(1) == 1
     assert dout.stride(1) == 1 and y.stride(1) == 1 and y.shape[1] == Cc
     op = N.Op()
     op.kind = N.OP_MOE_GATE_BWD

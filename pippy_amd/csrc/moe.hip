@@ -208,7 +208,9 @@ __global__ __launch_bounds__(256) void moe_gate_bwd_kernel(const uint16_t* __res
             dg[k] = wave_sum(dg[k]);
             mean = fmaf(gate[t * topk + k], dg[k], mean);
         }
-        for (int e = lane; e < E; e += 64) {
+        // columns E .. round_up(E, 8) - 1 (the padding of a router with an expert count that is not a
+        // multiple of 8; ld_dl is a multiple of 8) are written as zeros
+        for (int e = lane; e < ((E + 7) & ~7); e += 64) {
             float v = 0.f;
 #pragma unroll
             for (int k = 0; k < kMoeMaxTopk; ++k) {
@@ -282,7 +284,7 @@ extern "C" int pp_moe_gate_bwd(const void* dout, int64_t ld_dout, const void* y,
                                const int32_t* pos, const int32_t* topk_idx, const float* gate, int topk, int E,
                                void* dlogits, int64_t ld_dl, int64_t T, int64_t C, pp_stream stream) {
     if (T < 0 || C < 0 || (C & 7) || topk < 1 || topk > kMoeMaxTopk || E < 1 || !pos || !topk_idx || !gate ||
-        !dlogits || ld_dl < E || !rows_ok(dout, ld_dout) || !rows_ok(y, ld_y) || ld_dout < C || ld_y < C)
+        !dlogits || ld_dl < ((E + 7) & ~7) || !rows_ok(dout, ld_dout) || !rows_ok(y, ld_y) || ld_dout < C || ld_y < C)
         return fail(PP_ERR_INVALID, "pp_moe_gate_bwd: bad arguments (T=%lld C=%lld topk=%d)", (long long)T,
                     (long long)C, topk);
     if (T == 0) return PP_OK;

@@ -642,7 +642,8 @@ class MoELayer(LlamaLayer):
     """A Mixtral-style decoder layer: the attention half of ``LlamaLayer`` and, in place of the dense
     feed-forward, a sparse mixture of ``n_experts`` SwiGLU experts of which a softmax router picks
     two per token (weights renormalised over the pair).  Parameters: ``block_sparse_moe.gate`` and
-    ``block_sparse_moe.experts.<e>.w1 / w2 / w3``.  The launch-list form takes 8, 16, .. 64 experts.
+    ``block_sparse_moe.experts.<e>.w1 / w2 / w3``.  The launch-list form takes 2 .. 64 experts (a count that is not a multiple of 8 runs with the router
+    weight and the logits padded to one).
 
     ``forced_routing`` (a list of int64 [tokens, 2] tensors, one per forward call, consumed in
     order) overrides the expert selection of the torch statement; a comparison against a lower
@@ -663,6 +664,12 @@ class MoELayer(LlamaLayer):
         nn.init.normal_(self.block_sparse_moe.gate.weight, std=init_std)
         self.block_sparse_moe.experts = nn.ModuleList([_Expert(dim, ffn, dtype, init_std) for _ in range(n_experts)])
         self.forced_routing = None
+
+    def _padded_experts(self) -> int:
+        return (self.n_experts + 7) // 8 * 8
+
+    def _pp_padded_rows(self):
+        return [(self.block_sparse_moe.gate.weight, self._padded_experts())] if self.n_experts % 8 else []
 
     def _feed_forward(self, h):
         shape = h.shape
@@ -690,18 +697,18 @@ class MoELayer(LlamaLayer):
     def _lower_feed_forward(self, b, x2):
         T, Cc = x2.shape
         E, K, ffn = self.n_experts, self.TOPK, self.ffn
-        if E % 8:
-            # the router GEMMs run with the expert count as a leading dimension and as a reduction length
-            raise RuntimeError(f"MoELayer lowers with a multiple of 8 experts, got {E}")
+        # the router GEMMs run with the expert count as a leading dimension and as a reduction length:
+        # the router weight is stored with zero rows up to a multiple of 8, and so are the logits
+        Ep = self._padded_experts()
         R = T * K
         moe = self.block_sparse_moe
         experts = list(moe.experts)
         n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
-        logits = b.act("router_logits", (T, E))
+        logits = b.act("router_logits", (T, Ep))
         lower_linear(b, "router", moe.gate, n2, out=logits)
         idx = b.act("topk_idx", (T, K), torch.int32)
         gate = b.act("gate", (T, K), torch.float32)
-        b.f(P.op_moe_router(logits, idx, gate))
+        b.f(P.op_moe_router(logits, idx, gate, E))
         seg = b.act("seg_start", (E + 1,), torch.int32)
         row_src = b.act("row_src", (R,), torch.int32)
         pos = b.act("pos", (R,), torch.int32)
@@ -726,7 +733,7 @@ class MoELayer(LlamaLayer):
             # expert rows receive the output gradient of their token times the routing weight
             d_yp = b.grad("d_yp", (R, Cc))
             b.i(P.op_moe_gather(dy2d, row_src, K, d_yp, scale=gate.view(-1)))
-            dlogits = b.grad("dlogits", (T, E))
+            dlogits = b.grad("dlogits", (T, Ep))
             b.i(P.op_moe_gate_bwd(dy2d, yp, pos, idx, gate, E, dlogits))
             w2t = self._pointer_list(b, "w2t", [b.weight_t(ex.w2.weight) for ex in experts])
             w1t = self._pointer_list(b, "w1t", [b.weight_t(ex.w1.weight) for ex in experts])

@@ -763,16 +763,17 @@ def _moe_reference_stages(ref, n_stages, per):
     return out
 
 
-@pytest.mark.parametrize("fused", [False, True, "staged"])
-def test_moe_interleaved_1f1b_matches_oracle(fused):
+@pytest.mark.parametrize("fused,E", [(False, 8), (True, 8), ("staged", 8), (False, 6), (False, 12), (True, 3)])
+def test_moe_interleaved_1f1b_matches_oracle(fused, E):
     """Config 5 at a reduced size: two virtual stages of MoE layers on one rank under interleaved
     1F1B.  The fp32 oracle is given the expert selection of the bf16 run (a token whose second and
     third router logits nearly tie may legitimately flip under rounding); that the selection itself
-    is the top-2 of the run's own logits is checked separately."""
+    is the top-2 of the run's own logits is checked separately.  Expert counts that are not a multiple
+    of 8 run with the router weight and the logits padded to one (zero rows / columns)."""
     import pippy_amd as pp
     from pippy_amd.configs import MoEDecoderLM, equal_split_spec
-    torch.manual_seed(0)
-    M, S, vocab, L, E = 4, 128, 512, 4, 8
+    torch.manual_seed(0 if E == 8 else E)
+    M, S, vocab, L = 4, 128, 512, 4
     model = MoEDecoderLM(vocab=vocab, dim=128, n_layers=L, n_heads=2, ffn=256, n_experts=E)
     with torch.no_grad():
         for layer in model.h:
@@ -797,7 +798,9 @@ def test_moe_interleaved_1f1b_matches_oracle(fused):
             seg = [v for k, v in acts.items() if k.endswith("seg_start")]
             assert len(idx) == L // 2
             for j in range(L // 2):
-                want, _ = OO.moe_route_top2(logits[j].float().cpu())
+                assert logits[j].shape[1] == (E + 7) // 8 * 8
+                assert float(logits[j][:, E:].float().abs().sum()) == 0.0      # the padding columns
+                want, _ = OO.moe_route_top2(logits[j][:, :E].float().cpu())
                 assert torch.equal(idx[j].cpu().long(), want)
                 assert int(seg[j][-1]) == 2 * 2 * S and int(seg[j][0]) == 0
                 routing[s * (L // 2) + j].append(idx[j].cpu().long())
