@@ -111,6 +111,136 @@ def _insert_markers(gm_graph: fx.Graph, split_spec: Dict[str, SplitPoint]):
             raise ValueError(f"Unknown split point type {point}")
 
 
+def _attr(root: nn.Module, target: str):
+    obj = root
+    for part in target.split("."):
+        obj = getattr(obj, part)
+    return obj
+
+
+def _fold_constants(gm: fx.GraphModule) -> None:
+    """Evaluates, once, every part of an exported graph that depends on no model input and no parameter
+    (position indices, attention masks built from the example's sequence length, ...), and replaces it by
+    non-persistent buffers of ``gm``.  Stages then receive only activations from their predecessor
+    instead of also such tensors computed by the first stage, and a stage's graph shows a constant mask
+    as what it is."""
+    graph = gm.graph
+    value: Dict[fx.Node, Any] = {}
+    for n in graph.nodes:
+        if n.op == "get_attr":
+            try:
+                obj = _attr(gm, n.target)
+            except AttributeError:
+                continue
+            written = any(u.op == "call_function" and getattr(getattr(u.target, "_schema", None), "is_mutable", False)
+                          for u in n.users)
+            if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) and not written:
+                value[n] = obj
+        elif n.op == "call_function" and isinstance(n.target, torch._ops.OpOverload):
+            if n.target.namespace != "aten" or torch.Tag.nondeterministic_seeded in n.target.tags \
+                    or n.target._schema.is_mutable or any(a not in value for a in n.all_input_nodes):
+                continue
+            try:
+                with torch.no_grad():
+                    value[n] = n.target(*fx.node.map_arg(n.args, lambda a: value[a]),
+                                        **fx.node.map_arg(n.kwargs, lambda a: value[a]))
+            except Exception:
+                continue
+    count = 0
+    for c in [n for n in value if n.op == "call_function" and torch.is_tensor(value[n])]:
+        outside = [u for u in c.users if u not in value]
+        if not outside:
+            continue
+        name = f"_folded_constant_{count}"
+        count += 1
+        gm.register_buffer(name, value[c].clone(), persistent=False)
+        for u in outside:
+            with graph.inserting_before(u):
+                const = graph.get_attr(name)
+            const.meta = {k: v for k, v in c.meta.items() if k == "val"}
+            u.replace_input_with(c, const)
+    for n in reversed(list(graph.nodes)):
+        if n in value and not n.users:
+            graph.erase_node(n)
+
+
+# Layers of torch.nn that take one tensor and whose exported nodes can be put back as one call of the layer
+_REROLLED_TYPES = (nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.Embedding, nn.Dropout, nn.GELU, nn.ReLU, nn.Identity)
+
+
+def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
+    """``torch.export`` dissolves every layer into ATen nodes.  This puts the standard leaf layers of
+    the model back: the nodes that the exporter recorded as coming from one call of such a layer, when
+    they read one tensor from outside and hand one tensor on, become a ``call_module`` node on the
+    model's own layer object (installed in ``gm`` under its qualified name).  A stage cut from the graph
+    then holds whole layers, which is what the stage runtime lowers to kernels; the result computed is
+    unchanged.  Besides the torch.nn types this covers layers of other libraries that are recognisably
+    an affine map with an [in, out] weight or an elementwise activation (checked on sample values, and
+    their exported nodes are checked against the layer itself)."""
+    from .stage_modules import activation_like, in_out_linear_like
+    graph = gm.graph
+    leaves = {}
+    for name, m in mod.named_modules():
+        if not name or next(m.children(), None) is not None:
+            continue
+        if isinstance(m, _REROLLED_TYPES):
+            leaves[name] = (m, False)
+        elif in_out_linear_like(m) or activation_like(m) is not None:
+            leaves[name] = (m, True)
+    calls: Dict[Tuple[str, str], List[fx.Node]] = {}
+    for n in graph.nodes:
+        stack = n.meta.get("nn_module_stack") if n.op == "call_function" else None
+        if not stack:
+            continue
+        key, entry = list(stack.items())[-1]
+        if entry[0] in leaves:
+            calls.setdefault((key, entry[0]), []).append(n)
+    for (_key, fqn), nodes in calls.items():
+        layer, verify = leaves[fqn]
+        inside = set(nodes)
+        external, own = [], []
+        for n in nodes:
+            for a in n.all_input_nodes:
+                if a in inside:
+                    continue
+                if a.op == "get_attr" and str(a.target).startswith(fqn + "."):
+                    own.append(a)
+                elif a not in external:
+                    external.append(a)
+        results = [n for n in nodes if any(u not in inside for u in n.users)]
+        if len(external) != 1 or len(results) != 1:
+            continue
+        src, res = external[0], results[0]
+        if verify:
+            fake = src.meta.get("val")
+            try:
+                x = torch.randn(tuple(int(d) for d in fake.shape), dtype=fake.dtype)
+                env = {src: x}
+                env.update({a: _attr(gm, a.target) for a in own})
+                with torch.no_grad():
+                    for n in nodes:
+                        env[n] = n.target(*fx.node.map_arg(n.args, lambda a: env[a]),
+                                          **fx.node.map_arg(n.kwargs, lambda a: env[a]))
+                    want, got = env[res], layer(x)
+                same = got.shape == want.shape and bool((got.float() - want.float()).abs().max()
+                                                        <= 1e-5 + 2e-2 * want.float().abs().max()
+                                                        * (want.dtype != torch.float32))
+            except Exception:
+                same = False
+            if not same:
+                continue
+        gm.add_submodule(fqn, layer)
+        with graph.inserting_after(nodes[-1]):
+            call = graph.call_module(fqn, (src,))
+        call.meta = dict(res.meta)
+        res.replace_all_uses_with(call)
+        for n in reversed(nodes):
+            graph.erase_node(n)
+    for n in reversed(list(graph.nodes)):
+        if n.op == "get_attr" and not n.users:
+            graph.erase_node(n)
+
+
 def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Optional[Dict[str, Any]],
                      split_spec: Optional[Dict[str, SplitPoint]]) -> Tuple[fx.GraphModule, fx.Graph]:
     """The route of the reference (``_IR.py:1141-1145``): ``torch.export`` on the inputs of one
@@ -123,9 +253,13 @@ def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Option
     gm = ep.module()
     graph = gm.graph
     for n in list(graph.nodes):
-        if n.op == "call_module" and str(n.target).startswith("_guards"):
-            graph.erase_node(n)   # shape guards of the example inputs: stages re-check nothing
-        elif n.op == "call_function" and n.target is torch.ops.pippy_amd._pipe_split.default:
+        if (n.op == "call_module" and str(n.target).startswith("_guards")) or \
+                (n.op == "call_function" and n.target is torch.ops.aten._assert_tensor_metadata.default):
+            graph.erase_node(n)   # guards of the example inputs' shapes and dtypes: stages re-check nothing
+    _fold_constants(gm)
+    _reroll_leaf_layers(mod, gm)
+    for n in list(graph.nodes):
+        if n.op == "call_function" and n.target is torch.ops.pippy_amd._pipe_split.default:
             n.target = pipe_split
     compute = [n for n in graph.nodes if n.op in ("call_function", "call_method", "call_module")]
     for name, point in (split_spec or {}).items():
@@ -258,7 +392,11 @@ class Pipe(nn.Module):
                     attr = sub.graph.create_node("get_attr", target)
                 ph.replace_all_uses_with(attr)
                 sub.graph.erase_node(ph)
-            setattr(split, name, fx.GraphModule(mod, sub.graph, class_name=name))
+            stage_mod = fx.GraphModule(mod, sub.graph, class_name=name)
+            # constants folded out of an exported graph are not part of the model's state
+            stage_mod._non_persistent_buffers_set.update(
+                b for b, _ in stage_mod.named_buffers(recurse=False) if b.startswith("_folded_constant_"))
+            setattr(split, name, stage_mod)
         split.recompile()
         found = [n for n, _ in split.named_children() if n.startswith("submod_")]
         if len(found) != num_stages:
@@ -297,8 +435,9 @@ class Pipe(nn.Module):
             # symbolic tracing cannot follow this model: export it on the first microbatch's inputs, as
             # the reference does (``_IR.py:1172-1185``); the stages are then ATen-level graphs
             logger.warning(f"torch.fx symbolic tracing failed ({type(fx_error).__name__}: {fx_error}); "
-                           "falling back to torch.export: the stages are ATen-level graphs and run through "
-                           "torch autograd, not as HIP launch lists")
+                           "falling back to torch.export on the inputs of one microbatch: the stages hold "
+                           "that microbatch's shapes; standard layers are put back into the ATen-level graph, "
+                           "and a stage whose structure is then recognised still runs as HIP launch lists")
             args_split, kwargs_split = split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks,
                                                                      args_chunk_spec, kwargs_chunk_spec)
             try:

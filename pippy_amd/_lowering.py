@@ -15,8 +15,9 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .stage_modules import (LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence,
-                            WrappedLMHead, WrappedTokenEmbedding, WrappedTransformerLayer)
+from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence,
+                            WrappedLMHead, WrappedTokenEmbedding, WrappedTransformerLayer, activation_like,
+                            in_out_linear_like)
 
 _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout,
                nn.Embedding)
@@ -24,7 +25,18 @@ _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GEL
 
 class _ChainTracer(fx.Tracer):
     def is_leaf_module(self, m, qualname):
-        return isinstance(m, _LEAF_TYPES) or super().is_leaf_module(m, qualname)
+        return isinstance(m, _LEAF_TYPES) or in_out_linear_like(m) or activation_like(m) is not None \
+            or super().is_leaf_module(m, qualname)
+
+
+def _as_linear(m: nn.Module) -> Optional[nn.Module]:
+    """``m`` itself when it is an ``nn.Linear``, an ``nn.Linear``-shaped view of it when it is an affine
+    layer with an [in, out] weight, else None."""
+    if isinstance(m, nn.Linear):
+        return m
+    if in_out_linear_like(m):
+        return InOutLinear(m)
+    return None
 
 
 def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
@@ -32,7 +44,9 @@ def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
     if node.op == "call_function":
         if node.target in (torch.relu, F.relu, torch.nn.functional.relu):
             return "relu"
-        if node.target is F.gelu:
+        if node.target is _ATEN.relu.default:
+            return "relu"
+        if node.target in (F.gelu, _ATEN.gelu.default):
             approx = node.kwargs.get("approximate", "none")
             return "gelu_tanh" if approx == "tanh" else "gelu_erf"
     if node.op == "call_method" and node.target == "relu":
@@ -47,7 +61,19 @@ def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
             return "identity"
         if isinstance(m, nn.Dropout) and (m.p == 0.0 or not m.training):
             return "identity"
+        return activation_like(m)
+    if node.op == "call_function" and node.target in _ATEN_DROPOUT:
+        p_drop, train = node.args[1], node.args[2] if len(node.args) > 2 else True
+        return "identity" if (p_drop == 0.0 or not train) else None
     return None
+
+
+_ATEN = torch.ops.aten
+_ATEN_DROPOUT = (_ATEN.dropout.default,)
+# ATen-level nodes of an exported stage that only change how a tensor is viewed; the walk over the
+# residual structure steps over them, and the numerical check of the recognised blocks covers them
+_ATEN_VIEWS = (_ATEN.view.default, _ATEN.reshape.default, _ATEN._unsafe_view.default, _ATEN.slice.Tensor,
+               _ATEN.contiguous.default, _ATEN.clone.default, _ATEN.alias.default, _ATEN.detach.default)
 
 
 class NotLowerable(Exception):
@@ -98,9 +124,10 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' is not a module call or a supported activation")
         m = root.get_submodule(n.target)
+        m = _as_linear(m) or m
         if isinstance(m, NativeBlock):
             blocks.append(m)
-        elif isinstance(m, nn.Linear):
+        elif isinstance(m, (nn.Linear, InOutLinear)):
             nxt = _activation_of(nodes[i + 1], root) if i + 1 < len(nodes) else None
             if nxt not in (None, "identity"):
                 blocks.append(LinearAct(m, nxt))
@@ -173,8 +200,9 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 # at which layers feed which residual add; how the model reshapes between them is not parsed but
 # checked: the torch statement of the recognised blocks must reproduce the stage's own forward on a
 # random input (fp32, on the host), otherwise the stage stays with torch autograd.
-_SDPA = F.scaled_dot_product_attention
-_ADD_FNS = (operator.add, operator.iadd, torch.add)
+_SDPA = (F.scaled_dot_product_attention, _ATEN.scaled_dot_product_attention.default)
+_ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor)
+_ACT_FNS = (F.gelu, F.relu, torch.relu, _ATEN.gelu.default, _ATEN.relu.default)
 
 
 def _is_add(n: fx.Node) -> bool:
@@ -191,40 +219,95 @@ def _branch_layers(y: fx.Node, stream: fx.Node, order: dict) -> List[fx.Node]:
         seen.add(n)
         if n.op == "placeholder":
             continue
-        if n.op == "call_module" or (n.op == "call_function" and n.target in (_SDPA, F.gelu, F.relu, torch.relu)) \
+        if n.op == "call_module" or (n.op == "call_function" and n.target in _SDPA + _ACT_FNS) \
                 or _is_add(n):
             found.append(n)
         stack.extend(a for a in n.all_input_nodes)
     return sorted(found, key=order.get)
 
 
+def _constant_of(root: nn.Module, node) -> Optional[torch.Tensor]:
+    """The tensor behind a ``get_attr`` node that reads a buffer or constant of ``root``, else None."""
+    if not isinstance(node, fx.Node) or node.op != "get_attr":
+        return None
+    obj = root
+    try:
+        for part in str(node.target).split("."):
+            obj = getattr(obj, part)
+    except AttributeError:
+        return None
+    return obj if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) else None
+
+
+def _is_causal_mask(mask: torch.Tensor) -> bool:
+    """A boolean (keep) or additive (0 / -inf or lowest) mask, broadcast over batch and heads, that lets
+    query i see exactly the keys 0..i."""
+    if mask.dim() < 2 or mask.shape[-1] != mask.shape[-2]:
+        return False
+    S = mask.shape[-1]
+    planes = mask.reshape(-1, S, S)
+    if not bool((planes == planes[0]).all()):
+        return False
+    m = planes[0]
+    keep = torch.ones(S, S, dtype=torch.bool, device=m.device).tril()
+    if m.dtype == torch.bool:
+        return bool((m == keep).all())
+    lowest = torch.finfo(m.dtype).min if m.dtype.is_floating_point else None
+    if lowest is None:
+        return False
+    masked = (m == float("-inf")) | (m <= lowest)
+    return bool((masked == ~keep).all()) and bool((m[keep] == 0).all())
+
+
+def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
+    """Reads the arguments of a scaled_dot_product_attention node; raises unless it is plain softmax
+    attention, causal or full, at the default scale."""
+    names = ("query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale", "enable_gqa")
+    given = dict(zip(names, sd.args))
+    given.update(sd.kwargs)
+    if given.get("dropout_p", 0.0) not in (0, 0.0) or given.get("enable_gqa"):
+        raise NotLowerable("scaled_dot_product_attention with dropout or grouped queries")
+    scale = given.get("scale")
+    if scale is not None and not any(abs(float(scale) - d ** -0.5) < 1e-6 for d in head_dims):
+        raise NotLowerable(f"scaled_dot_product_attention with the custom scale {scale}")
+    causal = bool(given.get("is_causal", False))
+    mask = given.get("attn_mask")
+    if mask is not None:
+        value = _constant_of(root, mask)
+        if value is None or causal or not _is_causal_mask(value):
+            raise NotLowerable("scaled_dot_product_attention with a mask tensor other than a constant causal mask")
+        causal = True
+    return causal
+
+
 def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     """("attn", ln, qkv, proj, causal) or ("mlp", ln, fc1, fc2, activation) for a residual branch."""
     mods = []
     for n in layers:
+        if _activation_of(n, root) == "identity":
+            continue
         if n.op == "call_module":
             m = root.get_submodule(n.target)
-            if _activation_of(n, root) == "identity":
-                continue
-            mods.append((n, m))
+            mods.append((n, _as_linear(m) or m))
         elif _is_add(n):
             raise NotLowerable(f"an addition inside a residual branch ('{n.format_node()}')")
         else:
             mods.append((n, None))
-    kinds = [type(m).__name__ if m is not None else ("sdpa" if n.target is _SDPA else "act") for n, m in mods]
+
+    def kind(n, m):
+        if m is None:
+            return "sdpa" if n.target in _SDPA else "act"
+        if isinstance(m, (nn.Linear, InOutLinear)):
+            return "Linear"
+        return "act" if _activation_of(n, root) is not None else type(m).__name__
+
+    kinds = [kind(n, m) for n, m in mods]
     if kinds == ["LayerNorm", "Linear", "sdpa", "Linear"]:
         (_, ln), (_, qkv), (sd, _), (_, proj) = mods
         if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
             raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection of width 3 d")
-        kw = dict(sd.kwargs)
-        extra = sd.args[3:]
-        if kw.get("attn_mask") is not None or kw.get("dropout_p", 0.0) not in (0, 0.0) or kw.get("scale") is not None \
-                or kw.get("enable_gqa") or any(a is not None and a != 0.0 and a is not False for a in extra[:2]):
-            raise NotLowerable("scaled_dot_product_attention with a mask tensor, dropout, a custom scale or grouped "
-                               "queries")
-        causal = bool(kw.get("is_causal", extra[2] if len(extra) > 2 else False))
-        return ("attn", ln, qkv, proj, causal)
-    if len(kinds) == 4 and kinds[0] == "LayerNorm" and kinds[1] == "Linear" and kinds[3] == "Linear":
+        return ("attn", ln, qkv, proj, _sdpa_is_causal(root, sd))
+    if kinds == ["LayerNorm", "Linear", "act", "Linear"]:
         (_, ln), (_, fc1), (an, am), (_, fc2) = mods
         act = _activation_of(an, root)
         if act not in ("gelu_tanh", "gelu_erf"):
@@ -252,7 +335,10 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
     # embedding front: the first addition of two embedding look-ups, or a lone token table
     emb = [n for n in nodes if n.op == "call_module" and isinstance(root.get_submodule(n.target), nn.Embedding)]
     if emb:
-        if len(emb) > 2 or emb[0].all_input_nodes != [stream]:
+        ids = emb[0].all_input_nodes[0] if len(emb[0].all_input_nodes) == 1 else None
+        while ids is not None and ids is not stream and ids.op == "call_function" and ids.target in _ATEN_VIEWS:
+            ids = ids.args[0]   # an exported model may re-view its indices first ([-1, seq])
+        if len(emb) > 2 or ids is not stream:
             raise NotLowerable("embedding tables other than one token table (and one position table)")
         wte = root.get_submodule(emb[0].target)
         if len(emb) == 2:
@@ -309,21 +395,22 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
         tail.append(cur)
     tail_mods = []
     for n in tail:
-        if _activation_of(n, root) == "identity":
+        if _activation_of(n, root) == "identity" or (n.op == "call_function" and n.target in _ATEN_VIEWS):
             continue
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
-        tail_mods.append(root.get_submodule(n.target))
-    kinds = [type(m).__name__ for m in tail_mods]
-    if kinds == ["LayerNorm", "Linear"] and tail_mods[1].bias is None:
+        m = root.get_submodule(n.target)
+        tail_mods.append(_as_linear(m) or m)
+    kinds = ["Linear" if isinstance(m, (nn.Linear, InOutLinear)) else type(m).__name__ for m in tail_mods]
+    if kinds == ["LayerNorm", "Linear"] and isinstance(tail_mods[1], nn.Linear) and tail_mods[1].bias is None:
         blocks.append(WrappedLMHead(tail_mods[0], tail_mods[1]))
-    elif kinds == ["Linear"] and tail_mods[0].bias is None and blocks:
+    elif kinds == ["Linear"] and isinstance(tail_mods[0], nn.Linear) and tail_mods[0].bias is None and blocks:
         blocks.append(WrappedLMHead(None, tail_mods[0]))
     else:
         for m in tail_mods:
             if isinstance(m, nn.LayerNorm):
                 blocks.append(LayerNormBlock(m))
-            elif isinstance(m, nn.Linear):
+            elif isinstance(m, (nn.Linear, InOutLinear)):
                 blocks.append(LinearAct(m, None))
             else:
                 raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
@@ -332,19 +419,26 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
     return blocks
 
 
-def _example_input(blocks: List[NativeBlock]) -> torch.Tensor:
+def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
+    """A random stage input; ``shape`` is given for exported stages, whose graphs hold the sizes of the
+    example microbatch."""
     g = torch.Generator().manual_seed(0)
     first = blocks[0]
     if isinstance(first, WrappedTokenEmbedding):
         seq = 16 if first.wpe is None else min(16, first.wpe.num_embeddings)
-        return torch.randint(0, first.wte.num_embeddings, (2, seq), generator=g)
+        return torch.randint(0, first.wte.num_embeddings, shape or (2, seq), generator=g)
     d = next(b for b in blocks if isinstance(b, WrappedTransformerLayer)).dim
-    return torch.randn(2, 16, d, generator=g)
+    return torch.randn(shape or (2, 16, d), generator=g)
 
 
 def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     """Blocks of a stage that is a stack of plain-torch transformer layers, verified numerically."""
     import copy
+    shape = None
+    if isinstance(submod, fx.GraphModule):
+        inputs = [n for n in submod.graph.nodes if n.op == "placeholder"]
+        if len(inputs) == 1 and hasattr(inputs[0].meta.get("val"), "shape"):
+            shape = tuple(int(s) for s in inputs[0].meta["val"].shape)
     try:
         graph = _ChainTracer().trace(submod)
     except Exception as e:
@@ -367,7 +461,7 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     reasons = []
     for n_heads in candidates:
         trial = _residual_blocks(probe, probe_graph, n_heads)
-        x = _example_input(trial)
+        x = _example_input(trial, shape)
         with torch.no_grad():
             want = probe(x)
             got = x

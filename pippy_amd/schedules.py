@@ -279,6 +279,9 @@ class PipelineSchedule(ABC):
         self._pipe_info = getattr(self._stages[0], "pipe_info", None)
         for stage in self._stages:
             stage.has_backward = self._has_backward
+            # a pipe built from the inputs of ONE microbatch (``pipeline(mod, mb_args=...)``) leaves the
+            # microbatch count to the schedule
+            stage.chunks = max(stage.chunks, self._n_microbatches)
 
 
 class PipelineScheduleSingle(PipelineSchedule):

@@ -126,6 +126,22 @@ class PipelineStageBase:
             logger.warning(f"{self.log_prefix} runs eagerly through torch autograd, not as HIP launch lists: "
                            f"{self.eager_reason}")
             self.submod.to(self.device)
+            self._move_ops_to_device()
+
+    def _move_ops_to_device(self):
+        """An exported graph holds the device of export time as a literal ``device=`` argument of the
+        ops that create tensors; an eager stage runs that graph, so the literals are pointed at the
+        stage's device (reference ``_PipelineStage.py:621-628``)."""
+        if not isinstance(self.submod, torch.fx.GraphModule):
+            return
+        changed = False
+        for node in self.submod.graph.nodes:
+            if node.op == "call_function" and isinstance(node.kwargs.get("device"), torch.device) \
+                    and node.kwargs["device"] != self.device:
+                node.kwargs = {**node.kwargs, "device": self.device}
+                changed = True
+        if changed:
+            self.submod.recompile()
 
     # -- reference properties -----------------------------------------------------------------
     @property
@@ -414,8 +430,11 @@ class PipelineStageBase:
                 entry = (lst, ws)
                 prog.loss_ops[key] = entry
             lst, _ = entry
-            if self._step_losses is None:
-                self._step_losses = torch.empty(self.chunks, dtype=torch.float32, device=self.device)
+            if self._step_losses is None or mb >= self._step_losses.numel():
+                # (a pipe built from one microbatch's inputs does not know the schedule's microbatch
+                # count; losses handed out earlier keep their old buffer)
+                self._step_losses = torch.empty(max(self.chunks, 2 * (mb + 1), 8), dtype=torch.float32,
+                                                device=self.device)
             if _CHECK_INPUTS:
                 bad = ((target < 0) | (target >= V)) & (target != native.ignore_index)
                 if bool(bad.any()):

@@ -43,7 +43,12 @@ def _as2d(t: torch.Tensor) -> torch.Tensor:
 def lower_linear(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, *, epilogue=N.EPI_BIAS,
                  aux_in=None, save_pre=False, out: Optional[torch.Tensor] = None):
     """y = epilogue(x W^T + bias).  Returns (y, pre_activation or None)."""
-    W = b.weight(lin.weight)
+    if getattr(lin, "weight_in_out", False):
+        if lin.weight.dtype != torch.bfloat16:
+            raise RuntimeError("a linear layer that stores its weight as [in, out] lowers in bf16 only")
+        W = b.weight_t(lin.weight)     # the [out, in] copy: both GEMM operands k-contiguous
+    else:
+        W = b.weight(lin.weight)
     bias = b.weight(lin.bias) if lin.bias is not None else None
     T = x2d.shape[0]
     y = out if out is not None else b.act(name, (T, W.shape[0]))
@@ -77,6 +82,20 @@ def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
 def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, dY2d: torch.Tensor, *,
                     need_dx=True, dx_out=None, dx_epilogue=N.EPI_NONE, dx_aux=None, padded=True):
     """I: dX = epilogue(dY W); W: dW = dY^T X, db = colsum(dY)."""
+    if getattr(lin, "weight_in_out", False):
+        # the stored [in, out] weight is what the input-gradient GEMM reads; its gradient is X^T dY
+        Wio = b.weight(lin.weight)
+        dx = None
+        if need_dx:
+            dx = dx_out if dx_out is not None else b.grad(name + ".dx", (dY2d.shape[0], Wio.shape[0]))
+            ws = None
+            copies = P.splitk_copies(dY2d.shape[0], Wio.shape[0], dY2d.shape[1])
+            if copies and dx_epilogue == N.EPI_NONE:
+                ws = b.workspace("splitk", (copies * dY2d.shape[0] * Wio.shape[0],), torch.float32)
+            b.i(P.op_gemm(dY2d, Wio, dx, epilogue=dx_epilogue, aux_in=dx_aux, splitk_workspace=ws))
+        b.w_weight_gemm(x2d, dY2d, lin.weight)
+        bias_grad(b, lin, dY2d)
+        return dx
     W = b.weight(lin.weight, padded)
     dx = None
     if need_dx:
@@ -840,6 +859,90 @@ class LMHead(NativeBlock):
 # A model written with plain torch layers (``nn.Embedding``, ``nn.LayerNorm``, ``nn.Linear``,
 # ``F.scaled_dot_product_attention``, residual adds) is lowered by recognising these groupings in its
 # graph and wrapping the user's own layer objects: no parameter is copied or renamed.
+class InOutLinear(nn.Module):
+    """A user's affine layer that stores its weight as [in, out] (``y = x W + b``; Hugging Face's
+    ``Conv1D`` is one), presented with the attributes of ``nn.Linear``.  The layer object, its
+    parameters and their names stay the user's; ``weight_in_out`` tells the lowering helpers which
+    GEMM operand the stored matrix is."""
+
+    weight_in_out = True
+
+    def __init__(self, layer: nn.Module):
+        super().__init__()
+        self.layer = layer
+        self.in_features, self.out_features = layer.weight.shape
+
+    @property
+    def weight(self):
+        return self.layer.weight
+
+    @property
+    def bias(self):
+        return self.layer.bias
+
+    def forward(self, x):
+        return self.layer(x)
+
+
+def in_out_linear_like(m: nn.Module) -> bool:
+    """Whether ``m`` is a leaf layer with a 2-d ``weight`` [in, out] and an optional 1-d ``bias`` whose
+    forward is ``x W + b`` over the last dimension — decided by running it on a few random rows."""
+    if isinstance(m, nn.Linear) or next(m.children(), None) is not None or next(m.buffers(), None) is not None:
+        return False
+    params = dict(m.named_parameters(recurse=False))
+    w = params.get("weight")
+    bias = params.get("bias", getattr(m, "bias", None))
+    if w is None or w.dim() != 2 or set(params) - {"weight", "bias"} or (bias is not None and bias.dim() != 1):
+        return False
+    cached = getattr(m, "_pp_in_out_linear", None)
+    if cached is not None:
+        return cached
+    try:
+        with torch.no_grad():
+            x = torch.randn(3, 2, w.shape[0], generator=torch.Generator().manual_seed(0)).to(w.device, w.dtype)
+            got = m(x).float()
+            want = x.float() @ w.float() + (bias.float() if bias is not None else 0.0)
+            ok = got.shape == want.shape and bool((got - want).abs().max() <= 2e-2 * want.abs().max() + 1e-6)
+    except Exception:
+        ok = False
+    try:
+        m._pp_in_out_linear = ok
+    except Exception:
+        pass
+    return ok
+
+
+def activation_like(m: nn.Module) -> Optional[str]:
+    """"relu", "gelu_tanh", "gelu_erf" or "identity" for a parameter-free leaf module that computes that
+    function elementwise (decided on sample values: activation classes of model libraries qualify),
+    else None."""
+    if next(m.children(), None) is not None or next(m.parameters(), None) is not None \
+            or next(m.buffers(), None) is not None:
+        return None
+    if isinstance(m, nn.Dropout):
+        return "identity" if (m.p == 0.0 or not m.training) else None
+    cached = getattr(m, "_pp_activation_like", 0)
+    if cached != 0:
+        return cached
+    found = None
+    try:
+        with torch.no_grad():
+            x = torch.linspace(-6.0, 6.0, 193).view(1, 1, -1)
+            y = m(x)
+            if torch.is_tensor(y) and y.shape == x.shape:
+                for name in ("relu", "gelu_tanh", "gelu_erf", "identity"):
+                    if (y - _torch_act(x, name if name != "identity" else None)).abs().max() <= 1e-5:
+                        found = name
+                        break
+    except Exception:
+        found = None
+    try:
+        m._pp_activation_like = found
+    except Exception:
+        pass
+    return found
+
+
 class WrappedTokenEmbedding(TokenEmbedding):
     def __init__(self, wte: nn.Embedding, wpe: Optional[nn.Embedding]):
         NativeBlock.__init__(self)

@@ -35,3 +35,64 @@ class GPT(nn.Module):
         for blk in self.h:
             x = blk(x)
         return self.lm_head(self.ln_f(x))
+
+
+# ---- the same model the way model libraries write it ---------------------------------------------------
+# Affine layers that keep their weight as [in, out], an activation class of their own, an explicit
+# boolean mask built from the sequence length, and Python control flow on shapes (torch.fx symbolic
+# tracing cannot follow it, so the front end goes through torch.export).
+class Affine(nn.Module):
+    def __init__(self, nx, nf):
+        super().__init__()
+        self.nf = nf
+        self.weight = nn.Parameter(torch.randn(nx, nf) * 0.02)
+        self.bias = nn.Parameter(torch.randn(nf) * 0.02)
+    def forward(self, x):
+        out_shape = x.size()[:-1] + (self.nf,)
+        return torch.addmm(self.bias, x.view(-1, x.size(-1)), self.weight).view(out_shape)
+class TanhGelu(nn.Module):
+    def forward(self, x):
+        return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * (x + 0.044715 * torch.pow(x, 3.0))))
+class LibAttention(nn.Module):
+    def __init__(self, d, h):
+        super().__init__()
+        self.c_attn = Affine(d, 3*d); self.c_proj = Affine(d, d); self.n_head = h
+        self.resid_dropout = nn.Dropout(0.0)
+    def forward(self, x, mask):
+        B, T, C = x.size()
+        q, k, v = self.c_attn(x).split(C, dim=2)
+        shape = (B, T, -1, C // self.n_head)
+        q, k, v = (t.view(shape).transpose(1, 2) for t in (q, k, v))
+        y = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, scale=(C // self.n_head) ** -0.5)
+        return self.resid_dropout(self.c_proj(y.transpose(1, 2).reshape(B, T, C)))
+class LibMLP(nn.Module):
+    def __init__(self, d):
+        super().__init__()
+        self.c_fc = Affine(d, 4*d); self.act = TanhGelu(); self.c_proj = Affine(4*d, d)
+    def forward(self, x):
+        return self.c_proj(self.act(self.c_fc(x)))
+class LibBlock(nn.Module):
+    def __init__(self, d, h):
+        super().__init__()
+        self.ln_1 = nn.LayerNorm(d); self.attn = LibAttention(d, h)
+        self.ln_2 = nn.LayerNorm(d); self.mlp = LibMLP(d)
+    def forward(self, x, mask):
+        x = self.attn(self.ln_1(x), mask) + x
+        return x + self.mlp(self.ln_2(x))
+class LibGPT(nn.Module):
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4):
+        super().__init__()
+        self.wte = nn.Embedding(vocab, d); self.wpe = nn.Embedding(seq, d)
+        self.h = nn.ModuleList([LibBlock(d, h) for _ in range(L)])
+        self.ln_f = nn.LayerNorm(d); self.lm_head = nn.Linear(d, vocab, bias=False)
+    def forward(self, idx):
+        idx = idx.view(-1, idx.shape[-1])
+        t = idx.shape[-1]
+        if t > self.wpe.num_embeddings:          # control flow on a shape
+            raise ValueError("sequence too long")
+        pos = torch.arange(t, device=idx.device).unsqueeze(0)
+        mask = (pos.unsqueeze(-1) >= pos.unsqueeze(-2))[:, None].expand(idx.shape[0], 1, t, t)
+        x = self.wte(idx) + self.wpe(pos)
+        for blk in self.h:
+            x = blk(x, mask)
+        return self.lm_head(self.ln_f(x))

@@ -112,3 +112,77 @@ def test_export_fallback_pipeline_trains_like_the_unsplit_model():
 def test_split_point_that_is_not_in_the_model_raises_on_the_export_route_too():
     with pytest.raises(ValueError, match="not a module called by the model"):
         pp.pipeline(_Model(), 2, (torch.randn(4, 8),), split_spec={"nowhere": pp.SplitPoint.BEGINNING})
+
+
+# ---- exported stages keep whole layers and lower to launch lists when their structure is recognised ----
+def _lib_gpt():
+    import os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import LibGPT
+    torch.manual_seed(0)
+    return LibGPT(vocab=500, seq=64, d=128, h=2, L=4)
+
+
+def test_exported_stages_hold_the_models_own_layers_and_no_constant_computation():
+    model = _lib_gpt()
+    with pytest.raises(Exception):
+        fx.symbolic_trace(model)
+    ids = torch.randint(0, 500, (2, 32))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    assert pipe.num_stages == 2
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    for i in range(2):
+        sm = pipe.get_stage_module(i)
+        layers = {n.target for n in sm.graph.nodes if n.op == "call_module"}
+        for name, layer in model.named_modules():
+            if name and next(layer.children(), None) is None and name.startswith(("h.0.", "h.1.") if i == 0 else ("h.2.", "h.3.")):
+                assert name in layers, f"{name} was not put back as a layer call"
+                assert sm.get_submodule(name) is layer
+        # one activation in, one activation out: the mask and the position indices are constants of the stage
+        assert len([n for n in sm.graph.nodes if n.op == "placeholder"]) == 1
+        assert not [n for n in sm.graph.nodes if n.op == "call_function" and "arange" in str(n.target)]
+        assert not [k for k in sm.state_dict() if "_folded_constant" in k]
+
+
+def test_exported_library_style_transformer_is_recognised_and_verified():
+    from pippy_amd._lowering import lower_stage_module
+    from pippy_amd.stage_modules import InOutLinear
+    model = _lib_gpt()
+    ids = torch.randint(0, 500, (2, 32))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    why = []
+    kinds = [[type(b).__name__ for b in lower_stage_module(pipe.get_stage_module(i), why)] for i in range(2)]
+    assert not why
+    assert kinds == [["WrappedTokenEmbedding"] + ["WrappedTransformerLayer"] * 2,
+                     ["WrappedTransformerLayer"] * 2 + ["WrappedLMHead"]]
+    layer = lower_stage_module(pipe.get_stage_module(1))[0]
+    # [in, out] affine layers are wrapped, not copied; the constant mask was read as causal
+    assert isinstance(layer.attn.c_attn, InOutLinear) and layer.attn.c_attn.layer is model.h[2].attn.c_attn
+    assert layer.causal and layer.n_heads == 2 and layer.activation == "gelu_tanh"
+    x = torch.randn(2, 32, 128)
+    torch.testing.assert_close(layer(x), model.h[2](x, torch.ones(32, 32, dtype=torch.bool).tril()))
+
+
+def test_a_mask_that_is_not_causal_keeps_the_stage_with_torch():
+    from pippy_amd._lowering import lower_stage_module
+    model = _lib_gpt()
+    orig = model.forward
+
+    def windowed(idx):
+        t = idx.shape[-1]
+        pos = torch.arange(t).unsqueeze(0)
+        mask = ((pos.unsqueeze(-1) >= pos.unsqueeze(-2)) & (pos.unsqueeze(-1) - pos.unsqueeze(-2) < 8))[:, None]
+        mask = mask.expand(idx.shape[0], 1, t, t)
+        x = model.wte(idx) + model.wpe(pos)
+        if t > 1:
+            for blk in model.h:
+                x = blk(x, mask)
+        return model.lm_head(model.ln_f(x))
+
+    model.forward = windowed
+    ids = torch.randint(0, 500, (2, 32))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None
+    assert "mask" in why[0]

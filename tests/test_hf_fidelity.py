@@ -184,3 +184,36 @@ def test_moe_feed_forward_is_a_mixtral_sparse_moe_block():
     w3 = torch.stack([ex.w3.weight for ex in mine.block_sparse_moe.experts]).detach()
     y = OO.moe_top2(h[0], sd["gate.weight"], w1, w2, w3)
     _close(y, out_hf.reshape(T, dim), "oracle moe_top2")
+
+
+def test_hugging_face_gpt2_stages_are_recognised_on_the_models_own_layers():
+    """The model of the reference's example (examples/huggingface/pippy_gpt2.py:50-65, embeddings untied)
+    goes through the torch.export route of the front end; its stages must come out as the blocks the
+    launch lists are built from, wrapped around the model's own Conv1D / LayerNorm / Embedding objects,
+    and those blocks must reproduce the model."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    from pippy_amd.stage_modules import InOutLinear
+    cfg = transformers.GPT2Config(n_layer=4, n_embd=128, n_head=2, vocab_size=500, n_positions=64,
+                                  attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False,
+                                  tie_word_embeddings=False, bos_token_id=0, eos_token_id=0)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.GPT2LMHeadModel(cfg)
+    ids = torch.randint(0, 500, (2, 48))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"transformer.h.2": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding"] + ["WrappedTransformerLayer"] * 2, ["WrappedTransformerLayer"] * 2 + ["WrappedLMHead"]]
+    first = blocks[0][1]
+    assert isinstance(first.attn.c_attn, InOutLinear) and first.attn.c_attn.layer is model.transformer.h[0].attn.c_attn
+    assert first.ln_1 is model.transformer.h[0].ln_1 and blocks[0][0].wte is model.transformer.wte
+    assert first.causal and first.n_heads == 2 and first.activation == "gelu_tanh"
+    assert blocks[1][-1].lm_head is model.lm_head
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against GPT2LMHeadModel")
