@@ -132,6 +132,34 @@ def build_other(args):
                          f"({args.accumulate_text})")
         args.batch, args.seq = 16, 1024
         return model, sched, stages, ids.cuda(), target.cuda()
+    if args.workload == "hf_gpt2":
+        # the headline configuration on the model class of the reference's example itself:
+        # transformers.GPT2LMHeadModel (GPT-2 small, random weights, embeddings untied), cut by the front
+        # end's torch.export route and run as launch lists on the model's own Conv1D parameters
+        import transformers
+        cfg = transformers.GPT2Config(attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False,
+                                      tie_word_embeddings=False)
+        cfg._attn_implementation = "sdpa"
+        model = transformers.GPT2LMHeadModel(cfg).to(torch.bfloat16)
+        M, B, S = 8, 32, 1024
+        ids = torch.randint(0, cfg.vocab_size, (B, S))
+        target = torch.randint(0, cfg.vocab_size, (B, S))
+        pipe = pp.pipeline(model, mb_args=(ids[:B // M],),
+                           split_spec={f"transformer.h.{i}": pp.SplitPoint.BEGINNING for i in (3, 6, 9)})
+        stages = [pp.PipelineStage(pipe, i, "cuda", fused_accumulate=args.fused_accumulate) for i in range(4)]
+        eager = [st.eager_reason for st in stages if not st.is_native]
+        if eager:
+            raise RuntimeError(f"a stage of the Hugging Face model did not lower: {eager}")
+        sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+        args.tokens, args.training = B * S, True
+        args.batch, args.seq = B, S
+        args.vocab, args.dim, args.layers, args.heads, args.ffn = cfg.vocab_size, 768, 12, 12, 3072
+        args.flops = flops_per_step(args)
+        args.describe = ("transformers.GPT2LMHeadModel (GPT-2 small: 12 layers, d_model 768, 12 heads, FFN 3072, "
+                         "vocab 50257, seq 1024; random weights, embeddings untied), exported and cut by "
+                         "pipeline(), 4 virtual stages on one GPU, schedule 1f1b, batch 32 in 8 microbatches, "
+                         f"bf16 with fp32 gradient accumulation ({args.accumulate_text})")
+        return model, sched, stages, ids.cuda(), target.cuda()
     raise ValueError(args.workload)
 
 
@@ -295,10 +323,11 @@ def main():
                     help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
                          "events, cold operands), torch.matmul (the vendor library) on the same operands beside "
                          "it, and sample the shader clock during each; one JSON line per shape")
-    ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe"],
+    ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe", "hf_gpt2"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
                          "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
-                         "configurations at full size")
+                         "configurations at full size; hf_gpt2: the headline configuration on "
+                         "transformers.GPT2LMHeadModel itself")
     # workload shape (defaults: GPT-2 small, configs[2])
     ap.add_argument("--vocab", type=int, default=50257)
     ap.add_argument("--seq", type=int, default=1024)
