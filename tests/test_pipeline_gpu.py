@@ -1089,3 +1089,50 @@ def test_hugging_face_gpt2_runs_natively_and_matches_the_oracle():
             return self.g(idx).logits
 
     _exported_model_against_the_oracle(model, Logits, 1000, 128, "transformer.h.2")
+
+
+def test_exported_stages_that_do_not_lower_run_through_autograd_on_the_gpu():
+    """An exported model whose attention mask is not the causal one (a sliding window) keeps its stages
+    with torch autograd.  Their graphs were exported on the host: the folded constants (mask, position
+    indices) must move to the GPU with the stage, and results must equal the unsplit model's."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import LibGPT
+    import pippy_amd as pp
+    torch.manual_seed(0)
+    model = LibGPT(vocab=300, seq=64, d=128, h=2, L=4)
+
+    def windowed(idx):
+        t = idx.shape[-1]
+        if t > model.wpe.num_embeddings:
+            raise ValueError("sequence too long")
+        pos = torch.arange(t, device=idx.device).unsqueeze(0)
+        mask = ((pos.unsqueeze(-1) >= pos.unsqueeze(-2)) & (pos.unsqueeze(-1) - pos.unsqueeze(-2) < 8))[:, None]
+        mask = mask.expand(idx.shape[0], 1, t, t)
+        x = model.wte(idx) + model.wpe(pos)
+        for blk in model.h:
+            x = blk(x, mask)
+        return model.lm_head(model.ln_f(x))
+
+    model.forward = windowed
+    M, mb, seq = 4, 2, 48
+    ids = torch.randint(0, 300, (mb * M, seq))
+    target = torch.randint(0, 300, (mb * M, seq))
+    pipe = pp.pipeline(model, mb_args=(ids[:mb],), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert not any(st.is_native for st in stages) and "mask" in stages[1].eager_reason
+    sched = pp.Schedule1F1B(stages, M, loss_fn=_ce)
+    losses = []
+    out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    for p in model.parameters():          # the stages moved the model's parameters to the GPU
+        assert p.is_cuda
+    grads = {n: p.grad.clone() for n, p in model.named_parameters()}
+    for p in model.parameters():
+        p.grad = None
+    ref_out = model(ids.to(DEV))
+    ref_losses = [_ce(o, t) for o, t in zip(ref_out.chunk(M), target.to(DEV).chunk(M))]
+    sum(ref_losses).backward()
+    torch.testing.assert_close(out, ref_out, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(torch.stack(losses), torch.stack(ref_losses), rtol=1e-4, atol=1e-5)
+    for name, p in model.named_parameters():
+        torch.testing.assert_close(grads[name], p.grad, rtol=1e-3, atol=1e-5, msg=lambda m: f"{name}: {m}")
