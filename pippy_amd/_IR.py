@@ -13,6 +13,7 @@ stage ``i`` is ``pipe.split_gm.submod_i`` and its parameters keep their original
 from __future__ import annotations
 
 import logging
+import operator
 from dataclasses import dataclass
 from enum import Enum
 from typing import Any, Callable, Dict, List, Optional, Tuple
@@ -118,6 +119,24 @@ def _attr(root: nn.Module, target: str):
     return obj
 
 
+# regions the model ran under torch.no_grad() / torch.autocast(...): exported as one higher-order node
+# around a sub-graph each
+_WRAPPED_REGIONS = tuple(op for op in (getattr(torch.ops.higher_order, name, None) for name in
+                                       ("wrap_with_set_grad_enabled", "wrap_with_autocast")) if op is not None)
+
+
+def _drop_noop_casts(gm: fx.GraphModule) -> None:
+    """``x.to(dtype)`` of a tensor that already has that dtype returns ``x``; the exporter still records a
+    node, which hides that the layers around it read the same tensor."""
+    for n in list(gm.graph.nodes):
+        if n.op == "call_function" and n.target is torch.ops.aten.to.dtype and len(n.args) == 2 and not n.kwargs:
+            src = n.args[0]
+            have = getattr(src.meta.get("val"), "dtype", None) if isinstance(src, fx.Node) else None
+            if have is not None and have == n.args[1]:
+                n.replace_all_uses_with(src)
+                gm.graph.erase_node(n)
+
+
 def _fold_constants(gm: fx.GraphModule) -> None:
     """Evaluates, once, every part of an exported graph that depends on no model input and no parameter
     (position indices, attention masks built from the example's sequence length, ...), and replaces it by
@@ -136,6 +155,18 @@ def _fold_constants(gm: fx.GraphModule) -> None:
                           for u in n.users)
             if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) and not written:
                 value[n] = obj
+            elif isinstance(obj, fx.GraphModule):
+                value[n] = obj     # the body of a higher-order operator (below)
+        elif n.op == "call_function" and (n.target is operator.getitem or n.target in _WRAPPED_REGIONS):
+            # with constant inputs such a region is a constant like any other
+            if any(a not in value for a in n.all_input_nodes):
+                continue
+            try:
+                with torch.no_grad():
+                    value[n] = n.target(*fx.node.map_arg(n.args, lambda a: value[a]),
+                                        **fx.node.map_arg(n.kwargs, lambda a: value[a]))
+            except Exception:
+                continue
         elif n.op == "call_function" and isinstance(n.target, torch._ops.OpOverload):
             if n.target.namespace != "aten" or torch.Tag.nondeterministic_seeded in n.target.tags \
                     or n.target._schema.is_mutable or any(a not in value for a in n.all_input_nodes):
@@ -151,7 +182,7 @@ def _fold_constants(gm: fx.GraphModule) -> None:
         outside = [u for u in c.users if u not in value]
         if not outside:
             continue
-        name = f"_folded_constant_{count}"
+        name = f"_folded_constant_{count}_tensor"   # (a name that fx's _1, _2 suffixes of node names cannot collide with)
         count += 1
         gm.register_buffer(name, value[c].clone(), persistent=False)
         for u in outside:
@@ -165,7 +196,8 @@ def _fold_constants(gm: fx.GraphModule) -> None:
 
 
 # Layers of torch.nn that take one tensor and whose exported nodes can be put back as one call of the layer
-_REROLLED_TYPES = (nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.Embedding, nn.Dropout, nn.GELU, nn.ReLU, nn.Identity)
+_REROLLED_TYPES = (nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.Embedding, nn.Dropout, nn.GELU, nn.ReLU, nn.SiLU,
+                   nn.Identity)
 
 
 def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
@@ -177,7 +209,7 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
     unchanged.  Besides the torch.nn types this covers layers of other libraries that are recognisably
     an affine map with an [in, out] weight or an elementwise activation (checked on sample values, and
     their exported nodes are checked against the layer itself)."""
-    from .stage_modules import activation_like, in_out_linear_like
+    from .stage_modules import activation_like, in_out_linear_like, rms_norm_like
     graph = gm.graph
     leaves = {}
     for name, m in mod.named_modules():
@@ -185,7 +217,7 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
             continue
         if isinstance(m, _REROLLED_TYPES):
             leaves[name] = (m, False)
-        elif in_out_linear_like(m) or activation_like(m) is not None:
+        elif in_out_linear_like(m) or activation_like(m) is not None or rms_norm_like(m) is not None:
             leaves[name] = (m, True)
     calls: Dict[Tuple[str, str], List[fx.Node]] = {}
     for n in graph.nodes:
@@ -256,6 +288,7 @@ def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Option
         if (n.op == "call_module" and str(n.target).startswith("_guards")) or \
                 (n.op == "call_function" and n.target is torch.ops.aten._assert_tensor_metadata.default):
             graph.erase_node(n)   # guards of the example inputs' shapes and dtypes: stages re-check nothing
+    _drop_noop_casts(gm)
     _fold_constants(gm)
     _reroll_leaf_layers(mod, gm)
     for n in list(graph.nodes):

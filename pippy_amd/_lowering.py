@@ -15,9 +15,9 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, StageSequence,
-                            WrappedLMHead, WrappedTokenEmbedding, WrappedTransformerLayer, activation_like,
-                            in_out_linear_like)
+from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, RMSNormLike,
+                            StageSequence, WrappedLlamaLayer, WrappedLMHead, WrappedTokenEmbedding,
+                            WrappedTransformerLayer, activation_like, in_out_linear_like, rms_norm_like)
 
 _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout,
                nn.Embedding)
@@ -26,7 +26,7 @@ _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GEL
 class _ChainTracer(fx.Tracer):
     def is_leaf_module(self, m, qualname):
         return isinstance(m, _LEAF_TYPES) or in_out_linear_like(m) or activation_like(m) is not None \
-            or super().is_leaf_module(m, qualname)
+            or rms_norm_like(m) is not None or super().is_leaf_module(m, qualname)
 
 
 def _as_linear(m: nn.Module) -> Optional[nn.Module]:
@@ -39,6 +39,15 @@ def _as_linear(m: nn.Module) -> Optional[nn.Module]:
     return None
 
 
+def _as_rms_norm(m: nn.Module) -> Optional[nn.Module]:
+    """``m`` itself when it is a usable ``nn.RMSNorm``, an ``nn.RMSNorm``-shaped view of it when it is a
+    root-mean-square norm layer of another library, else None."""
+    if isinstance(m, nn.RMSNorm):
+        return m if (len(m.normalized_shape) == 1 and m.weight is not None and m.eps is not None) else None
+    eps = rms_norm_like(m)
+    return RMSNormLike(m, eps) if eps is not None else None
+
+
 def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
     """Name of the activation a node applies, "identity" for a no-op, or None if it is neither."""
     if node.op == "call_function":
@@ -46,6 +55,8 @@ def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
             return "relu"
         if node.target is _ATEN.relu.default:
             return "relu"
+        if node.target in (F.silu, _ATEN.silu.default):
+            return "silu"
         if node.target in (F.gelu, _ATEN.gelu.default):
             approx = node.kwargs.get("approximate", "none")
             return "gelu_tanh" if approx == "tanh" else "gelu_erf"
@@ -55,6 +66,8 @@ def _activation_of(node: fx.Node, root: nn.Module) -> Optional[str]:
         m = root.get_submodule(node.target)
         if isinstance(m, nn.ReLU):
             return "relu"
+        if isinstance(m, nn.SiLU):
+            return "silu"
         if isinstance(m, nn.GELU):
             return "gelu_tanh" if m.approximate == "tanh" else "gelu_erf"
         if isinstance(m, nn.Identity):
@@ -129,6 +142,8 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
             blocks.append(m)
         elif isinstance(m, (nn.Linear, InOutLinear)):
             nxt = _activation_of(nodes[i + 1], root) if i + 1 < len(nodes) else None
+            if nxt == "silu":
+                raise NotLowerable("a linear layer followed by SiLU outside a gated feed-forward")
             if nxt not in (None, "identity"):
                 blocks.append(LinearAct(m, nxt))
                 i += 1
@@ -202,7 +217,7 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 # random input (fp32, on the host), otherwise the stage stays with torch autograd.
 _SDPA = (F.scaled_dot_product_attention, _ATEN.scaled_dot_product_attention.default)
 _ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor)
-_ACT_FNS = (F.gelu, F.relu, torch.relu, _ATEN.gelu.default, _ATEN.relu.default)
+_ACT_FNS = (F.gelu, F.relu, torch.relu, F.silu, _ATEN.gelu.default, _ATEN.relu.default, _ATEN.silu.default)
 
 
 def _is_add(n: fx.Node) -> bool:
@@ -281,16 +296,18 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
 
 
 def _classify_branch(root: nn.Module, layers: List[fx.Node]):
-    """("attn", ln, qkv, proj, causal) or ("mlp", ln, fc1, fc2, activation) for a residual branch."""
-    mods = []
+    """What a residual branch is, from the layers between the stream and the addition:
+    ("attn", ln, qkv, proj, causal) / ("mlp", ln, fc1, fc2, activation) for the GPT-2 family,
+    ("attn_rope", norm, q, k, v, o) / ("mlp_gated", norm, gate, up, down) for the Llama family."""
+    mods, inner_adds = [], []
     for n in layers:
         if _activation_of(n, root) == "identity":
             continue
         if n.op == "call_module":
             m = root.get_submodule(n.target)
-            mods.append((n, _as_linear(m) or m))
+            mods.append((n, _as_linear(m) or _as_rms_norm(m) or m))
         elif _is_add(n):
-            raise NotLowerable(f"an addition inside a residual branch ('{n.format_node()}')")
+            inner_adds.append(n)     # rotary embeddings add two products; nothing else may
         else:
             mods.append((n, None))
 
@@ -299,9 +316,38 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             return "sdpa" if n.target in _SDPA else "act"
         if isinstance(m, (nn.Linear, InOutLinear)):
             return "Linear"
+        if isinstance(m, (nn.RMSNorm, RMSNormLike)):
+            return "RMSNorm"
         return "act" if _activation_of(n, root) is not None else type(m).__name__
 
     kinds = [kind(n, m) for n, m in mods]
+    if kinds == ["RMSNorm", "Linear", "Linear", "Linear", "sdpa", "Linear"]:
+        (_, norm), (_, q), (_, k), (_, v), (sd, _), (_, o) = mods
+        if any(lin.bias is not None for lin in (q, k, v, o)) or not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
+            raise NotLowerable("rotary attention whose projections have biases or [in, out] weights")
+        if k.out_features != v.out_features or q.out_features != o.in_features or q.out_features != q.in_features \
+                or q.out_features % k.out_features:
+            raise NotLowerable("query / key / value projections of unexpected widths")
+        if not _sdpa_is_causal(root, sd):
+            raise NotLowerable("rotary attention that is not causal")
+        return ("attn_rope", norm, q, k, v, o)
+    if kinds == ["RMSNorm", "Linear", "act", "Linear", "Linear"] or kinds == ["RMSNorm", "Linear", "Linear", "act", "Linear"]:
+        norm, down = mods[0][1], mods[-1][1]
+        an = next(n for n, m in mods if kind(n, m) == "act")
+        if _activation_of(an, root) != "silu":
+            raise NotLowerable(f"gated feed-forward with the activation '{an.format_node()}' (SiLU is built)")
+        lins = {n: m for n, m in mods[1:-1] if kind(n, m) == "Linear"}
+        gate_node = an.all_input_nodes[0] if an.all_input_nodes else None
+        if gate_node not in lins or inner_adds:
+            raise NotLowerable("a feed-forward that is not down(silu(gate(x)) * up(x))")
+        gate = lins.pop(gate_node)
+        up = next(iter(lins.values()))
+        if any(lin.bias is not None or not isinstance(lin, nn.Linear) for lin in (gate, up, down)) or \
+                gate.out_features != up.out_features or down.in_features != gate.out_features:
+            raise NotLowerable("gated feed-forward projections with biases, [in, out] weights or unexpected widths")
+        return ("mlp_gated", norm, gate, up, down)
+    if inner_adds:
+        raise NotLowerable(f"an addition inside a residual branch ('{inner_adds[0].format_node()}')")
     if kinds == ["LayerNorm", "Linear", "sdpa", "Linear"]:
         (_, ln), (_, qkv), (sd, _), (_, proj) = mods
         if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
@@ -318,7 +364,7 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     raise NotLowerable(f"a residual branch made of {kinds}")
 
 
-def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[NativeBlock]:
+def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) -> List[NativeBlock]:
     nodes = list(graph.nodes)
     order = {n: i for i, n in enumerate(nodes)}
     placeholders = [n for n in nodes if n.op == "placeholder"]
@@ -363,19 +409,31 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
         if len(other) != 1:
             break
         kind = _classify_branch(root, [n for n in _branch_layers(other[0], stream, order)])
-        if kind[0] == "attn":
+        if kind[0] in ("attn", "attn_rope"):
             if pending is not None:
                 raise NotLowerable("two attention branches in a row")
             pending = kind
         else:
             if pending is None:
                 raise NotLowerable("a feed-forward branch without an attention branch before it")
-            _, ln1, qkv, proj, causal = pending
-            _, ln2, fc1, fc2, act = kind
-            d = qkv.in_features
+            if (pending[0], kind[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
+                raise NotLowerable(f"a '{pending[0]}' branch followed by a '{kind[0]}' branch")
+            d = pending[2].in_features
             if d % n_heads or d // n_heads not in (64, 128):
                 raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
-            blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
+            if kind[0] == "mlp":
+                _, ln1, qkv, proj, causal = pending
+                _, ln2, fc1, fc2, act = kind
+                blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
+            else:
+                _, norm1, q, k, v, o = pending
+                _, norm2, gate, up, down = kind
+                if k.out_features % (d // n_heads):
+                    raise NotLowerable("key / value projections that are not whole heads")
+                if rope is None:
+                    raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the "
+                                       "positions (exported models do)")
+                blocks.append(WrappedLlamaLayer(norm1, q, k, v, o, norm2, gate, up, down, n_heads, *rope))
             pending = None
         stream = add
         while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
@@ -400,8 +458,9 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
         m = root.get_submodule(n.target)
-        tail_mods.append(_as_linear(m) or m)
-    kinds = ["Linear" if isinstance(m, (nn.Linear, InOutLinear)) else type(m).__name__ for m in tail_mods]
+        tail_mods.append(_as_linear(m) or _as_rms_norm(m) or m)
+    kinds = ["Linear" if isinstance(m, (nn.Linear, InOutLinear)) else
+             "LayerNorm" if isinstance(m, (nn.RMSNorm, RMSNormLike)) else type(m).__name__ for m in tail_mods]
     if kinds == ["LayerNorm", "Linear"] and isinstance(tail_mods[1], nn.Linear) and tail_mods[1].bias is None:
         blocks.append(WrappedLMHead(tail_mods[0], tail_mods[1]))
     elif kinds == ["Linear"] and isinstance(tail_mods[0], nn.Linear) and tail_mods[0].bias is None and blocks:
@@ -410,11 +469,13 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int) -> List[Nat
         for m in tail_mods:
             if isinstance(m, nn.LayerNorm):
                 blocks.append(LayerNormBlock(m))
+            elif isinstance(m, (nn.RMSNorm, RMSNormLike)):
+                blocks.append(RMSNormBlock(m))
             elif isinstance(m, (nn.Linear, InOutLinear)):
                 blocks.append(LinearAct(m, None))
             else:
                 raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
-    if not any(isinstance(b, WrappedTransformerLayer) for b in blocks):
+    if not any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer)) for b in blocks):
         raise NotLowerable("no attention / feed-forward residual pair found")
     return blocks
 
@@ -427,8 +488,28 @@ def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
     if isinstance(first, WrappedTokenEmbedding):
         seq = 16 if first.wpe is None else min(16, first.wpe.num_embeddings)
         return torch.randint(0, first.wte.num_embeddings, shape or (2, seq), generator=g)
-    d = next(b for b in blocks if isinstance(b, WrappedTransformerLayer)).dim
+    d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer))).dim
     return torch.randn(shape or (2, 16, d), generator=g)
+
+
+def _rotary_tables(submod: nn.Module, d: int):
+    """(heads, (cos, sin)) read off the constants of an exported stage: two [.., positions, head_dim]
+    tensors whose halves repeat, whose squares add up to one and which are 1 and 0 at position 0.  The
+    tables are taken as the model made them (its base, scaling and rounding).  None when there are none."""
+    tables = []
+    for _, t in submod.named_buffers():
+        if not t.is_floating_point() or t.dim() < 2 or t.shape[-1] not in (64, 128) or d % t.shape[-1]:
+            continue
+        D, S = t.shape[-1], t.shape[-2]
+        planes = t.detach().float().cpu().reshape(-1, S, D)
+        if bool((planes == planes[0]).all()) and bool((planes[0][:, :D // 2] == planes[0][:, D // 2:]).all()):
+            tables.append(planes[0][:, :D // 2])
+    for c in tables:
+        for s_ in tables:
+            if c.shape == s_.shape and bool((c[0] == 1).all()) and bool((s_[0] == 0).all()) \
+                    and bool(((c * c + s_ * s_) - 1).abs().max() <= 2e-2):
+                return d // (2 * c.shape[1]), (c, s_)
+    return None
 
 
 def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
@@ -444,23 +525,29 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     except Exception as e:
         raise NotLowerable(f"torch.fx cannot trace {type(submod).__name__}: {type(e).__name__}: {e}") from e
     widths = {m.normalized_shape[0] for m in submod.modules()
-              if isinstance(m, nn.LayerNorm) and len(m.normalized_shape) == 1}
+              if isinstance(m, (nn.LayerNorm, nn.RMSNorm)) and len(m.normalized_shape) == 1}
+    widths |= {m.weight.shape[0] for m in submod.modules() if rms_norm_like(m) is not None}
     if len(widths) != 1:
-        raise NotLowerable("no single model width (the LayerNorms of the stage disagree)")
+        raise NotLowerable("no single model width (the normalisation layers of the stage disagree)")
     d = widths.pop()
     candidates = [h for h in (d // 64, d // 128) if h >= 1 and d % h == 0]
     if not candidates:
         raise NotLowerable(f"model width {d} allows no head dimension of 64 or 128")
-    _residual_blocks(submod, graph, candidates[0])   # raises unless the structure is recognised
+    rotary = _rotary_tables(submod, d)
+    if rotary is not None:
+        candidates = [rotary[0]]      # the table's width is the head size
+    rope = rotary[1] if rotary is not None else None
+    _residual_blocks(submod, graph, candidates[0], rope)   # raises unless the structure is recognised
     # the structure fits; which head count (if any) reproduces the stage is decided on an fp32 copy
     try:
         probe = copy.deepcopy(submod).float().cpu().eval()
     except Exception as e:
         raise NotLowerable(f"the stage module cannot be copied for verification: {e}") from e
     probe_graph = _ChainTracer().trace(probe)
+    tolerance = 1e-4
     reasons = []
     for n_heads in candidates:
-        trial = _residual_blocks(probe, probe_graph, n_heads)
+        trial = _residual_blocks(probe, probe_graph, n_heads, rope)
         x = _example_input(trial, shape)
         with torch.no_grad():
             want = probe(x)
@@ -470,8 +557,8 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
         if isinstance(want, (tuple, list)):
             want = want[0]
         err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30) if got.shape == want.shape else 1.0
-        if err <= 1e-4:
-            return _residual_blocks(submod, graph, n_heads)
+        if err <= tolerance:
+            return _residual_blocks(submod, graph, n_heads, rope)
         reasons.append(f"with {n_heads} heads the recognised blocks differ from the stage's own forward "
                        f"(relative error {err:.2e})")
     raise NotLowerable("; ".join(reasons))

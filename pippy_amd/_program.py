@@ -113,19 +113,21 @@ class ParamArena:
             self._transposed[id(p)] = ent
         return ent[1]
 
-    def weight_t_cat(self, p1: nn.Parameter, p2: nn.Parameter) -> torch.Tensor:
-        """[in, out1 + out2]: the transposed copies of two weights with the same input width side by
-        side, so that dY1 W1 + dY2 W2 is ONE product of [dY1 | dY2] with this matrix.  Kept in step
-        with both parameters by ``refresh_transposed``."""
-        key = ("cat", id(p1), id(p2))
+    def weight_t_cat(self, *ps: nn.Parameter) -> torch.Tensor:
+        """[in, out1 + out2 + ...]: the transposed copies of weights with the same input width side by
+        side, so that dY1 W1 + dY2 W2 + ... is ONE product of [dY1 | dY2 | ...] with this matrix.  Kept in
+        step with the parameters by ``refresh_transposed``."""
+        key = ("cat",) + tuple(id(p) for p in ps)
         ent = self._transposed.get(key)
         if ent is None:
-            w1, w2 = self.weight(p1, padded=True), self.weight(p2, padded=True)
-            assert w1.shape[1] == w2.shape[1]
-            t = torch.empty((w1.shape[1], w1.shape[0] + w2.shape[0]), dtype=w1.dtype, device=self.device)
-            for k, (p, lo, hi) in enumerate(((p1, 0, w1.shape[0]), (p2, w1.shape[0], t.shape[1]))):
-                view = t[:, lo:hi]
-                N.transpose_bf16(self.weight(p, padded=True), view)
+            ws = [self.weight(p, padded=True) for p in ps]
+            assert all(w.shape[1] == ws[0].shape[1] for w in ws)
+            t = torch.empty((ws[0].shape[1], sum(w.shape[0] for w in ws)), dtype=ws[0].dtype, device=self.device)
+            lo = 0
+            for k, (p, w) in enumerate(zip(ps, ws)):
+                view = t[:, lo:lo + w.shape[0]]
+                lo += w.shape[0]
+                N.transpose_bf16(w, view)
                 self._transposed[key + (k,)] = (p, view)
             ent = (None, t)
             self._transposed[key] = ent
@@ -646,8 +648,8 @@ class Builder:
     def weight_t(self, p):
         return self.sp.arena.weight_t(p)
 
-    def weight_t_cat(self, p1, p2):
-        return self.sp.arena.weight_t_cat(p1, p2)
+    def weight_t_cat(self, *ps):
+        return self.sp.arena.weight_t_cat(*ps)
 
     def grad_target(self, p, padded=True):
         """Where the W pass writes a microbatch gradient that no GEMM epilogue accumulates: the

@@ -146,6 +146,8 @@ _ACT_KIND = {"relu": N.ACT_RELU, "gelu_erf": N.ACT_GELU_ERF, "gelu_tanh": N.ACT_
 
 
 def _torch_act(y, activation):
+    if activation == "silu":
+        return F.silu(y)
     if activation == "relu":
         return torch.relu(y)
     if activation == "gelu_erf":
@@ -533,9 +535,9 @@ class LlamaLayer(NativeBlock):
     def forward(self, x):
         Bn, S, Cc = x.shape
         H, Hkv, D = self.n_heads, self.n_kv_heads, Cc // self.n_heads
-        cos, sin = rope_tables(S, D, self.rope_theta, x.device)
+        cos, sin = self._rope(S, D, x.device)
         h = self.input_layernorm(x)
-        q, k, v = self.self_attn.qkv_proj(h).split([H * D, Hkv * D, Hkv * D], dim=-1)
+        q, k, v = self._project_qkv(h).split([H * D, Hkv * D, Hkv * D], dim=-1)
         q = q.reshape(Bn, S, H, D).transpose(1, 2)
         k, v = (t.reshape(Bn, S, Hkv, D).transpose(1, 2) for t in (k, v))
         q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
@@ -548,6 +550,24 @@ class LlamaLayer(NativeBlock):
     def _feed_forward(self, h):
         return self.mlp.down_proj(F.silu(self.mlp.gate_proj(h)) * self.mlp.up_proj(h))
 
+    def _project_qkv(self, h):
+        return self.self_attn.qkv_proj(h)
+
+    def _rope(self, seq, head_dim, device):
+        """(cos, sin) [seq, head_dim / 2] in fp32 and a key that names their content."""
+        return rope_tables(seq, head_dim, self.rope_theta, device)
+
+    def _rope_key(self):
+        return str(self.rope_theta)
+
+    def _lower_qkv(self, b, n1):
+        """Emits the q|k|v projection of the normalised input; returns the [tokens, (H + 2 Hkv) D] buffer."""
+        return lower_linear(b, "qkv", self.self_attn.qkv_proj, n1)[0]
+
+    def _qkv_backward(self, b, n1, dqkv):
+        """Emits input and weight gradients of the q|k|v projection; returns the gradient of ``n1``."""
+        return linear_backward(b, "qkv", self.self_attn.qkv_proj, n1, dqkv)
+
     def lower(self, b, x):
         if x.dim() != 3 or x.shape[-1] != self.dim:
             raise RuntimeError(f"{type(self).__name__} of width {self.dim} expects [batch, seq, dim], got "
@@ -557,13 +577,13 @@ class LlamaLayer(NativeBlock):
         D = Cc // H
         W = (H + 2 * Hkv) * D  # width of the fused projection
         x2d = x.view(T, Cc)
-        cos = b.sp.shared(f"rope_cos:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
-        sin = b.sp.shared(f"rope_sin:{S}:{D}:{self.rope_theta}", (S, D // 2), torch.float32)
-        c, s_ = rope_tables(S, D, self.rope_theta, x.device)
+        cos = b.sp.shared(f"rope_cos:{S}:{D}:{self._rope_key()}", (S, D // 2), torch.float32)
+        sin = b.sp.shared(f"rope_sin:{S}:{D}:{self._rope_key()}", (S, D // 2), torch.float32)
+        c, s_ = self._rope(S, D, x.device)
         cos.copy_(c)
         sin.copy_(s_)
         n1, rstd1 = lower_rmsnorm(b, "n1", self.input_layernorm, x2d)
-        qkv, _ = lower_linear(b, "qkv", self.self_attn.qkv_proj, n1)
+        qkv = self._lower_qkv(b, n1)
         b.f(P.op_rope(qkv, cos, sin, S, H + Hkv, D))
         att = b.act("att", (T, Cc))
         lse = b.act("lse", (Bn, H, S), torch.float32)
@@ -580,7 +600,7 @@ class LlamaLayer(NativeBlock):
                           d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv))
             # gradients w.r.t. the rotated q and k go back through the transposed rotation
             b.i(P.op_rope(dqkv, cos, sin, S, H + Hkv, D, inverse=True))
-            d_n1 = linear_backward(b, "qkv", self.self_attn.qkv_proj, n1, dqkv)
+            d_n1 = self._qkv_backward(b, n1, dqkv)
             dx = rmsnorm_backward(b, "n1", self.input_layernorm, x2d, rstd1, d_n1, dres=d_x2,
                                   dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
             return dx.view(Bn, S, Cc)
@@ -823,7 +843,7 @@ class LMHead(NativeBlock):
         Bn, S, Cc = x.shape
         T, V, Vp = Bn * S, self.vocab, self.padded_vocab
         x2d = x.view(T, Cc)
-        rms = isinstance(self.ln_f, nn.RMSNorm)
+        rms = _is_rms(self.ln_f)
         if rms:
             h, rstd = lower_rmsnorm(b, "ln_f", self.ln_f, x2d)
         elif self.ln_f is not None:
@@ -912,8 +932,66 @@ def in_out_linear_like(m: nn.Module) -> bool:
     return ok
 
 
+class RMSNormLike(nn.Module):
+    """A user's root-mean-square norm layer of another library (one 1-d ``weight``, an epsilon attribute;
+    Hugging Face's ``LlamaRMSNorm`` is one), presented with the attributes of ``nn.RMSNorm``."""
+
+    def __init__(self, layer: nn.Module, eps: float):
+        super().__init__()
+        self.layer = layer
+        self.eps = eps
+        self.normalized_shape = tuple(layer.weight.shape)
+
+    @property
+    def weight(self):
+        return self.layer.weight
+
+    def forward(self, x):
+        return self.layer(x)
+
+
+def rms_norm_like(m: nn.Module) -> Optional[float]:
+    """The epsilon of a leaf layer that computes ``weight * x / sqrt(mean(x^2) + eps)`` over the last
+    dimension with its single 1-d parameter ``weight`` (decided by running it on a few random rows), else
+    None.  ``nn.RMSNorm`` itself is not meant."""
+    if isinstance(m, nn.RMSNorm) or next(m.children(), None) is not None or next(m.buffers(), None) is not None:
+        return None
+    params = dict(m.named_parameters(recurse=False))
+    w = params.get("weight")
+    if w is None or set(params) != {"weight"} or w.dim() != 1:
+        return None
+    cached = getattr(m, "_pp_rms_norm_like", 0)
+    if cached != 0:
+        return cached
+    found = None
+    for attr in ("eps", "variance_epsilon", "epsilon"):
+        eps = getattr(m, attr, None)
+        if not isinstance(eps, float):
+            continue
+        try:
+            with torch.no_grad():
+                x = torch.randn(3, 2, w.shape[0], generator=torch.Generator().manual_seed(0)).to(w.device, w.dtype)
+                got = m(x).float()
+                xf = x.float()
+                want = w.float() * xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+                if got.shape == want.shape and bool((got - want).abs().max() <= 2e-2 * want.abs().max() + 1e-6):
+                    found = eps
+        except Exception:
+            found = None
+        break
+    try:
+        m._pp_rms_norm_like = found
+    except Exception:
+        pass
+    return found
+
+
+def _is_rms(norm) -> bool:
+    return isinstance(norm, (nn.RMSNorm, RMSNormLike))
+
+
 def activation_like(m: nn.Module) -> Optional[str]:
-    """"relu", "gelu_tanh", "gelu_erf" or "identity" for a parameter-free leaf module that computes that
+    """"relu", "gelu_tanh", "gelu_erf", "silu" or "identity" for a parameter-free leaf module that computes that
     function elementwise (decided on sample values: activation classes of model libraries qualify),
     else None."""
     if next(m.children(), None) is not None or next(m.parameters(), None) is not None \
@@ -930,7 +1008,7 @@ def activation_like(m: nn.Module) -> Optional[str]:
             x = torch.linspace(-6.0, 6.0, 193).view(1, 1, -1)
             y = m(x)
             if torch.is_tensor(y) and y.shape == x.shape:
-                for name in ("relu", "gelu_tanh", "gelu_erf", "identity"):
+                for name in ("relu", "gelu_tanh", "gelu_erf", "silu", "identity"):
                     if (y - _torch_act(x, name if name != "identity" else None)).abs().max() <= 1e-5:
                         found = name
                         break
@@ -961,6 +1039,68 @@ class WrappedTransformerLayer(TransformerLayer):
         self.attn.c_attn, self.attn.c_proj = c_attn, c_proj
         self.mlp = nn.Module()
         self.mlp.c_fc, self.mlp.c_proj = c_fc, mlp_proj
+
+
+class WrappedLlamaLayer(LlamaLayer):
+    """``LlamaLayer`` around the layers of a user's model, which keeps separate query, key and value
+    projections (the Hugging Face layout).  The three forward GEMMs write their column ranges of the
+    one q|k|v buffer the attention kernels read; the gradient of the normalised input is one product of
+    the q|k|v gradient with the three transposed weights side by side; each weight gradient reads its
+    column range of that gradient."""
+
+    def __init__(self, input_layernorm, q_proj, k_proj, v_proj, o_proj, post_attention_layernorm,
+                 gate_proj, up_proj, down_proj, n_heads: int, cos: torch.Tensor, sin: torch.Tensor):
+        """``cos`` / ``sin``: the model's own rotary tables, [positions, head_dim / 2] (whatever base,
+        scaling or rounding the model applies is in them)."""
+        NativeBlock.__init__(self)
+        self.dim, self.n_heads, self.ffn = o_proj.out_features, n_heads, gate_proj.out_features
+        D = self.dim // n_heads
+        assert cos.shape == sin.shape and cos.shape[1] == D // 2
+        self.n_kv_heads = k_proj.out_features // D
+        self.eps, self.rope_theta = input_layernorm.eps, None
+        self._cos, self._sin = cos.detach().float().cpu().contiguous(), sin.detach().float().cpu().contiguous()
+        import hashlib
+        self._table_key = hashlib.sha1(self._cos.numpy().tobytes() + self._sin.numpy().tobytes()).hexdigest()[:16]
+        self.input_layernorm, self.post_attention_layernorm = input_layernorm, post_attention_layernorm
+        self.self_attn = nn.Module()
+        self.self_attn.q_proj, self.self_attn.k_proj, self.self_attn.v_proj = q_proj, k_proj, v_proj
+        self.self_attn.o_proj = o_proj
+        self.mlp = nn.Module()
+        self.mlp.gate_proj, self.mlp.up_proj, self.mlp.down_proj = gate_proj, up_proj, down_proj
+
+    def _rope(self, seq, head_dim, device):
+        if seq > self._cos.shape[0] or head_dim != 2 * self._cos.shape[1]:
+            raise RuntimeError(f"the model's rotary table covers {self._cos.shape[0]} positions of head size "
+                               f"{2 * self._cos.shape[1]}, asked for {seq} of {head_dim}")
+        return self._cos[:seq].to(device), self._sin[:seq].to(device)
+
+    def _rope_key(self):
+        return self._table_key
+
+    def _projections(self):
+        a = self.self_attn
+        return (a.q_proj, a.k_proj, a.v_proj)
+
+    def _project_qkv(self, h):
+        return torch.cat([lin(h) for lin in self._projections()], dim=-1)
+
+    def _lower_qkv(self, b, n1):
+        W = sum(lin.out_features for lin in self._projections())
+        qkv = b.act("qkv", (n1.shape[0], W))
+        lo = 0
+        for name, lin in zip("qkv", self._projections()):
+            lower_linear(b, name, lin, n1, out=qkv[:, lo:lo + lin.out_features])
+            lo += lin.out_features
+        return qkv
+
+    def _qkv_backward(self, b, n1, dqkv):
+        d_n1 = b.grad("qkv.dx", (n1.shape[0], n1.shape[1]))
+        b.i(P.op_gemm(dqkv, b.weight_t_cat(*(lin.weight for lin in self._projections())), d_n1))
+        lo = 0
+        for name, lin in zip("qkv", self._projections()):
+            linear_backward(b, name, lin, n1, dqkv[:, lo:lo + lin.out_features], need_dx=False)
+            lo += lin.out_features
+        return d_n1
 
 
 class WrappedLMHead(LMHead):

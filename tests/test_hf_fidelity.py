@@ -217,3 +217,43 @@ def test_hugging_face_gpt2_stages_are_recognised_on_the_models_own_layers():
         for b in blocks[0] + blocks[1]:
             x = b(x)
         _close(x, model(ids).logits, "blocks against GPT2LMHeadModel")
+
+
+def test_hugging_face_llama_stages_are_recognised_on_the_models_own_layers():
+    """The model class of the reference's Llama example (examples/llama/pippy_llama.py:18-39): the rotary
+    table (computed by the model under no_grad from a buffer) and the causal mask fold into constants, the
+    head size is read off that table and the table itself is kept, and the stages come out as Llama blocks around the
+    model's own q / k / v / o / gate / up / down projections and LlamaRMSNorm layers."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    from pippy_amd.stage_modules import RMSNormLike
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=4,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=500,
+                                   max_position_embeddings=64, use_cache=False, tie_word_embeddings=False,
+                                   attention_dropout=0.0, rope_theta=5e5)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.LlamaForCausalLM(cfg)
+    ids = torch.randint(0, 500, (2, 48))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"model.layers.2": pp.SplitPoint.BEGINNING})
+    _close(pipe(ids)[0] if isinstance(pipe(ids), (tuple, list)) else pipe(ids), model(ids).logits, "Pipe against the model")
+    for i in range(2):
+        assert len([n for n in pipe.get_stage_module(i).graph.nodes if n.op == "placeholder"]) == 1
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding"] + ["WrappedLlamaLayer"] * 2, ["WrappedLlamaLayer"] * 2 + ["WrappedLMHead"]]
+    layer = blocks[1][0]
+    hf = model.model.layers[2]
+    assert layer.self_attn.k_proj is hf.self_attn.k_proj and layer.mlp.gate_proj is hf.mlp.gate_proj
+    assert isinstance(layer.input_layernorm, RMSNormLike) and layer.input_layernorm.layer is hf.input_layernorm
+    assert (layer.n_heads, layer.n_kv_heads) == (4, 2)
+    cos, sin = SM.rope_tables(48, 64, 5e5, "cpu")
+    _close(layer._cos, cos, "the model's cosine table")
+    _close(layer._sin, sin, "the model's sine table")
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against LlamaForCausalLM")

@@ -1136,3 +1136,29 @@ def test_exported_stages_that_do_not_lower_run_through_autograd_on_the_gpu():
     torch.testing.assert_close(torch.stack(losses), torch.stack(ref_losses), rtol=1e-4, atol=1e-5)
     for name, p in model.named_parameters():
         torch.testing.assert_close(grads[name], p.grad, rtol=1e-3, atol=1e-5, msg=lambda m: f"{name}: {m}")
+
+
+@pytest.mark.parametrize("heads,kv_heads", [(4, 4), (4, 2)])
+def test_hugging_face_llama_runs_natively_and_matches_the_oracle(heads, kv_heads):
+    """The model class of the reference's Llama example (examples/llama/pippy_llama.py:18-39) with random
+    weights: separate q / k / v projections, rotary embedding from a table the model computes under
+    no_grad, LlamaRMSNorm, SwiGLU, grouped-query attention when kv_heads < heads."""
+    transformers = pytest.importorskip("transformers")
+    import torch.nn as nn
+    cfg = transformers.LlamaConfig(hidden_size=64 * heads, intermediate_size=512, num_hidden_layers=4,
+                                   num_attention_heads=heads, num_key_value_heads=kv_heads, vocab_size=1000,
+                                   max_position_embeddings=128, use_cache=False, tie_word_embeddings=False,
+                                   attention_dropout=0.0)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.LlamaForCausalLM(cfg)
+
+    class Logits(nn.Module):
+        def __init__(self, g):
+            super().__init__()
+            self.g = g
+
+        def forward(self, idx):
+            return self.g(idx).logits
+
+    _exported_model_against_the_oracle(model, Logits, 1000, 128, "model.layers.2")
