@@ -16,7 +16,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, RMSNormLike,
-                            StageSequence, WrappedLlamaLayer, WrappedLMHead, WrappedTokenEmbedding,
+                            StageSequence, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead,
+                            WrappedTokenEmbedding,
                             WrappedTransformerLayer, activation_like, in_out_linear_like, rms_norm_like)
 
 _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout,
@@ -274,6 +275,11 @@ def _is_causal_mask(mask: torch.Tensor) -> bool:
     return bool((masked == ~keep).all()) and bool((m[keep] == 0).all())
 
 
+def _is_full_mask(mask: torch.Tensor) -> bool:
+    """A boolean mask that keeps everything or an additive one that is zero everywhere."""
+    return bool(mask.all()) if mask.dtype == torch.bool else bool((mask == 0).all())
+
+
 def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
     """Reads the arguments of a scaled_dot_product_attention node; raises unless it is plain softmax
     attention, causal or full, at the default scale."""
@@ -289,6 +295,8 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
     mask = given.get("attn_mask")
     if mask is not None:
         value = _constant_of(root, mask)
+        if value is not None and _is_full_mask(value):
+            return causal     # a mask that masks nothing (an encoder without padding)
         if value is None or causal or not _is_causal_mask(value):
             raise NotLowerable("scaled_dot_product_attention with a mask tensor other than a constant causal mask")
         causal = True
@@ -297,7 +305,8 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
 
 def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     """What a residual branch is, from the layers between the stream and the addition:
-    ("attn", ln, qkv, proj, causal) / ("mlp", ln, fc1, fc2, activation) for the GPT-2 family,
+    ("attn", ln, qkv, proj, causal) / ("mlp", ln, fc1, fc2, activation) for the GPT-2 and BERT families
+    (ln is None when the branch does not start with a LayerNorm; qkv is one fused layer or three),
     ("attn_rope", norm, q, k, v, o) / ("mlp_gated", norm, gate, up, down) for the Llama family."""
     mods, inner_adds = [], []
     for n in layers:
@@ -348,13 +357,22 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         return ("mlp_gated", norm, gate, up, down)
     if inner_adds:
         raise NotLowerable(f"an addition inside a residual branch ('{inner_adds[0].format_node()}')")
-    if kinds == ["LayerNorm", "Linear", "sdpa", "Linear"]:
-        (_, ln), (_, qkv), (sd, _), (_, proj) = mods
+    ln = None
+    if kinds and kinds[0] == "LayerNorm":      # pre-LayerNorm; without it the norm follows the addition
+        ln, mods, kinds = mods[0][1], mods[1:], kinds[1:]
+    if kinds == ["Linear", "sdpa", "Linear"]:
+        (_, qkv), (sd, _), (_, proj) = mods
         if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
             raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection of width 3 d")
         return ("attn", ln, qkv, proj, _sdpa_is_causal(root, sd))
-    if kinds == ["LayerNorm", "Linear", "act", "Linear"]:
-        (_, ln), (_, fc1), (an, am), (_, fc2) = mods
+    if kinds == ["Linear", "Linear", "Linear", "sdpa", "Linear"]:
+        (_, q), (_, k), (_, v), (sd, _), (_, proj) = mods
+        if not all(isinstance(lin, nn.Linear) and lin.in_features == lin.out_features == proj.in_features
+                   for lin in (q, k, v)):
+            raise NotLowerable("separate query / key / value projections that are not d -> d nn.Linear layers")
+        return ("attn", ln, (q, k, v), proj, _sdpa_is_causal(root, sd))
+    if kinds == ["Linear", "act", "Linear"]:
+        (_, fc1), (an, am), (_, fc2) = mods
         act = _activation_of(an, root)
         if act not in ("gelu_tanh", "gelu_erf"):
             raise NotLowerable(f"feed-forward activation '{an.format_node()}' (tanh- and erf-GELU are built)")
@@ -384,10 +402,31 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         ids = emb[0].all_input_nodes[0] if len(emb[0].all_input_nodes) == 1 else None
         while ids is not None and ids is not stream and ids.op == "call_function" and ids.target in _ATEN_VIEWS:
             ids = ids.args[0]   # an exported model may re-view its indices first ([-1, seq])
-        if len(emb) > 2 or ids is not stream:
-            raise NotLowerable("embedding tables other than one token table (and one position table)")
+        if len(emb) > 3 or ids is not stream:
+            raise NotLowerable("embedding tables other than a token table, a position table and a token-type table")
         wte = root.get_submodule(emb[0].target)
-        if len(emb) == 2:
+        if len(emb) == 3:
+            # the encoder front: word + token type (all zero) + position (0 .. S-1), then a LayerNorm
+            joins = [n for n in nodes if _is_add(n) and
+                     set(_branch_layers(n, stream, order)) - {n} >= set(emb) and
+                     all(_is_add(x) or x in emb for x in _branch_layers(n, stream, order))]
+            roles = {}
+            for e in emb[1:]:
+                index = _constant_of(root, e.all_input_nodes[0]) if len(e.all_input_nodes) == 1 else None
+                if index is not None and index.dtype == torch.int64:
+                    if bool((index == 0).all()):
+                        roles["type"] = e
+                    elif bool((index.reshape(-1, index.shape[-1]) == torch.arange(index.shape[-1])).all()):
+                        roles["position"] = e
+            norm_users = [u for u in joins[0].users] if joins else []
+            norm = root.get_submodule(norm_users[0].target) if len(norm_users) == 1 and \
+                norm_users[0].op == "call_module" else None
+            if len(roles) != 2 or not isinstance(norm, nn.LayerNorm):
+                raise NotLowerable("three embedding tables that are not word + position + token type 0 under a LayerNorm")
+            stream = norm_users[0]
+            blocks.append(WrappedEncoderEmbedding(wte, root.get_submodule(roles["position"].target),
+                                                  root.get_submodule(roles["type"].target), norm))
+        elif len(emb) == 2:
             joins = [n for n in nodes if _is_add(n) and set(_branch_layers(n, stream, order)) == {emb[0], emb[1], n}]
             if not joins:
                 raise NotLowerable("token and position embeddings are not simply added")
@@ -399,7 +438,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
             stream = next(iter(stream.users))   # dropout that does nothing
     # residual pairs
-    pending = None
+    pending = pending_norm = None
     while True:
         adds = [u for u in stream.users if _is_add(u)]
         if len(adds) != 1:
@@ -409,22 +448,37 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         if len(other) != 1:
             break
         kind = _classify_branch(root, [n for n in _branch_layers(other[0], stream, order)])
+        # post-LayerNorm layers: the sum goes through a LayerNorm before anything else reads it
+        post_norm, after = None, add
+        if kind[0] in ("attn", "mlp") and kind[1] is None:
+            users = list(add.users)
+            m = root.get_submodule(users[0].target) if len(users) == 1 and users[0].op == "call_module" else None
+            if not isinstance(m, nn.LayerNorm):
+                raise NotLowerable("a residual branch without a LayerNorm before it or after its addition")
+            post_norm, after = m, users[0]
         if kind[0] in ("attn", "attn_rope"):
             if pending is not None:
                 raise NotLowerable("two attention branches in a row")
-            pending = kind
+            pending, pending_norm = kind, post_norm
         else:
             if pending is None:
                 raise NotLowerable("a feed-forward branch without an attention branch before it")
             if (pending[0], kind[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
                 raise NotLowerable(f"a '{pending[0]}' branch followed by a '{kind[0]}' branch")
-            d = pending[2].in_features
+            d = pending[3].in_features if pending[0] == "attn" else pending[2].in_features
             if d % n_heads or d // n_heads not in (64, 128):
                 raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
             if kind[0] == "mlp":
                 _, ln1, qkv, proj, causal = pending
                 _, ln2, fc1, fc2, act = kind
-                blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
+                if (ln1 is None) != (ln2 is None) or (ln1 is None) != (pending_norm is not None) \
+                        or (ln2 is None) != (post_norm is not None):
+                    raise NotLowerable("a layer that is neither pre-LayerNorm nor post-LayerNorm throughout")
+                if ln1 is None:
+                    blocks.append(WrappedTransformerLayer(pending_norm, qkv, proj, post_norm, fc1, fc2, n_heads,
+                                                          causal, act, pre_ln=False))
+                else:
+                    blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
             else:
                 _, norm1, q, k, v, o = pending
                 _, norm2, gate, up, down = kind
@@ -435,7 +489,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
                                        "positions (exported models do)")
                 blocks.append(WrappedLlamaLayer(norm1, q, k, v, o, norm2, gate, up, down, n_heads, *rope))
             pending = None
-        stream = add
+        stream = after
         while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
             stream = next(iter(stream.users))
     if pending is not None:
@@ -453,15 +507,23 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         tail.append(cur)
     tail_mods = []
     for n in tail:
-        if _activation_of(n, root) == "identity" or (n.op == "call_function" and n.target in _ATEN_VIEWS):
+        act = _activation_of(n, root)
+        if act == "identity" or (n.op == "call_function" and n.target in _ATEN_VIEWS):
+            continue
+        if act in ("relu", "gelu_tanh", "gelu_erf") and tail_mods and isinstance(tail_mods[-1], (nn.Linear, InOutLinear)):
+            tail_mods[-1] = LinearAct(tail_mods[-1], act)     # a projection with its activation
             continue
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
         m = root.get_submodule(n.target)
         tail_mods.append(_as_linear(m) or _as_rms_norm(m) or m)
+    lead = []
+    while tail_mods and isinstance(tail_mods[0], LinearAct):
+        lead.append(tail_mods.pop(0))       # e.g. the transform in front of a masked-language-model head
+    blocks.extend(lead)
     kinds = ["Linear" if isinstance(m, (nn.Linear, InOutLinear)) else
              "LayerNorm" if isinstance(m, (nn.RMSNorm, RMSNormLike)) else type(m).__name__ for m in tail_mods]
-    if kinds == ["LayerNorm", "Linear"] and isinstance(tail_mods[1], nn.Linear) and tail_mods[1].bias is None:
+    if kinds == ["LayerNorm", "Linear"] and isinstance(tail_mods[1], nn.Linear):
         blocks.append(WrappedLMHead(tail_mods[0], tail_mods[1]))
     elif kinds == ["Linear"] and isinstance(tail_mods[0], nn.Linear) and tail_mods[0].bias is None and blocks:
         blocks.append(WrappedLMHead(None, tail_mods[0]))
@@ -473,6 +535,8 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
                 blocks.append(RMSNormBlock(m))
             elif isinstance(m, (nn.Linear, InOutLinear)):
                 blocks.append(LinearAct(m, None))
+            elif isinstance(m, LinearAct):
+                blocks.append(m)
             else:
                 raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
     if not any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer)) for b in blocks):
@@ -488,6 +552,9 @@ def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
     if isinstance(first, WrappedTokenEmbedding):
         seq = 16 if first.wpe is None else min(16, first.wpe.num_embeddings)
         return torch.randint(0, first.wte.num_embeddings, shape or (2, seq), generator=g)
+    if isinstance(first, WrappedEncoderEmbedding):
+        seq = min(16, first.position_embeddings.num_embeddings)
+        return torch.randint(0, first.word_embeddings.num_embeddings, shape or (2, seq), generator=g)
     d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer))).dim
     return torch.randn(shape or (2, 16, d), generator=g)
 
@@ -549,11 +616,15 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     for n_heads in candidates:
         trial = _residual_blocks(probe, probe_graph, n_heads, rope)
         x = _example_input(trial, shape)
-        with torch.no_grad():
-            want = probe(x)
-            got = x
-            for blk in trial:
-                got = blk(got)
+        try:
+            with torch.no_grad():
+                want = probe(x)
+                got = x
+                for blk in trial:
+                    got = blk(got)
+        except Exception as e:
+            raise NotLowerable(f"the recognised blocks could not be compared with the stage's own forward "
+                               f"({type(e).__name__}: {e})") from e
         if isinstance(want, (tuple, list)):
             want = want[0]
         err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30) if got.shape == want.shape else 1.0

@@ -217,6 +217,14 @@ class LayerNormBlock(NativeBlock):
         return y.view(x.shape)
 
 
+def _zero_padding_row(b: "P.Builder", table: nn.Embedding, acc: torch.Tensor):
+    """``nn.Embedding(padding_idx=i)`` gives row i no gradient: the row of the accumulator that the
+    embedding backward has just added to is cleared again."""
+    pad = getattr(table, "padding_idx", None)
+    if pad is not None:
+        b.w(P.op_fill(acc[pad % acc.shape[0]]))
+
+
 class TokenEmbedding(NativeBlock):
     """Token + learned position embedding: ``wte[ids] + wpe[:S]`` (GPT-2 style);
     ``positions=False`` leaves the position table out (models with rotary embeddings)."""
@@ -264,6 +272,7 @@ class TokenEmbedding(NativeBlock):
             if acc_wpe is not None:
                 b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+            _zero_padding_row(b, self.wte, acc_wte)
             return None
 
         b.on_backward(bwd)
@@ -317,6 +326,7 @@ class EncoderEmbedding(NativeBlock):
             b.w(P.op_fill(acc_wte), tag="fill")
             b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+            _zero_padding_row(b, self.word_embeddings, acc_wte)
             # the type-0 row receives the gradient of every token; the other rows none
             g_tt = b.grad_target(self.token_type_embeddings.weight)
             ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)
@@ -354,7 +364,7 @@ class TransformerLayer(NativeBlock):
     def _attention(self, h):
         Bn, S, Cc = h.shape
         H, D = self.n_heads, Cc // self.n_heads
-        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self.attn.c_attn(h).split(Cc, dim=-1))
+        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self._project_qkv(h).split(Cc, dim=-1))
         o = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal)
         return self.attn.c_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
 
@@ -364,6 +374,41 @@ class TransformerLayer(NativeBlock):
             return x + self.mlp.c_proj(_torch_act(self.mlp.c_fc(self.ln_2(x)), self.activation))
         x = self.ln_1(x + self._attention(x))
         return self.ln_2(x + self.mlp.c_proj(_torch_act(self.mlp.c_fc(x), self.activation)))
+
+    # the q|k|v projection: one fused layer here; subclasses around a user's model may hold three
+    def _qkv_layers(self):
+        return (self.attn.c_attn,)
+
+    def _project_qkv(self, h):
+        return torch.cat([lin(h) for lin in self._qkv_layers()], dim=-1)
+
+    def _lower_qkv(self, b, h2d):
+        """Emits the projection; returns the [tokens, 3 d] buffer the attention kernels read."""
+        layers = self._qkv_layers()
+        if len(layers) == 1:
+            return lower_linear(b, "qkv", layers[0], h2d)[0]
+        qkv = b.act("qkv", (h2d.shape[0], sum(lin.out_features for lin in layers)))
+        lo = 0
+        for name, lin in zip("qkv", layers):      # each GEMM writes its column range
+            lower_linear(b, name, lin, h2d, out=qkv[:, lo:lo + lin.out_features])
+            lo += lin.out_features
+        return qkv
+
+    def _qkv_backward(self, b, h2d, dqkv, *, dx_epilogue=N.EPI_NONE, dx_aux=None, dx_out=None):
+        """Emits input and weight gradients of the projection; returns the gradient of its input."""
+        layers = self._qkv_layers()
+        if len(layers) == 1:
+            return linear_backward(b, "c_attn", layers[0], h2d, dqkv, dx_epilogue=dx_epilogue, dx_aux=dx_aux,
+                                   dx_out=dx_out)
+        # one product of the whole gradient with the transposed weights side by side
+        dx = dx_out if dx_out is not None else b.grad("c_attn.dx", tuple(h2d.shape))
+        b.i(P.op_gemm(dqkv, b.weight_t_cat(*(lin.weight for lin in layers)), dx, epilogue=dx_epilogue,
+                      aux_in=dx_aux))
+        lo = 0
+        for name, lin in zip("qkv", layers):
+            linear_backward(b, name, lin, h2d, dqkv[:, lo:lo + lin.out_features], need_dx=False)
+            lo += lin.out_features
+        return dx
 
     def lower(self, b, x):
         if x.dim() != 3:
@@ -379,7 +424,7 @@ class TransformerLayer(NativeBlock):
         x2d = x.view(T, Cc)
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         ln1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, x2d)
-        qkv, _ = lower_linear(b, "qkv", self.attn.c_attn, ln1)
+        qkv = self._lower_qkv(b, ln1)
         att = b.act("att", (T, Cc))
         lse = b.act("lse", (Bn, H, S), torch.float32)
         b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
@@ -400,7 +445,7 @@ class TransformerLayer(NativeBlock):
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
             b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
                           d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
-            d_ln1 = linear_backward(b, "c_attn", self.attn.c_attn, ln1, dqkv)
+            d_ln1 = self._qkv_backward(b, ln1, dqkv)
             dx = layernorm_backward(b, "ln1", self.ln_1, x2d, mean1, rstd1, d_ln1, dres=d_x2,
                                     dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
             return dx.view(Bn, S, Cc)
@@ -413,7 +458,7 @@ class TransformerLayer(NativeBlock):
         T, H = Bn * S, self.n_heads
         x2d = x.view(T, Cc)
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
-        qkv, _ = lower_linear(b, "qkv", self.attn.c_attn, x2d)
+        qkv = self._lower_qkv(b, x2d)
         att = b.act("att", (T, Cc))
         lse = b.act("lse", (Bn, H, S), torch.float32)
         b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
@@ -436,8 +481,8 @@ class TransformerLayer(NativeBlock):
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
             b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
                           d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
-            dx = linear_backward(b, "c_attn", self.attn.c_attn, x2d, dqkv, dx_epilogue=N.EPI_BIAS_RESIDUAL,
-                                 dx_aux=d_a, dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
+            dx = self._qkv_backward(b, x2d, dqkv, dx_epilogue=N.EPI_BIAS_RESIDUAL, dx_aux=d_a,
+                                    dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
             return dx.view(Bn, S, Cc)
 
         b.on_backward(bwd)
@@ -832,7 +877,10 @@ class LMHead(NativeBlock):
         return (self.vocab + self.VOCAB_ALIGN - 1) // self.VOCAB_ALIGN * self.VOCAB_ALIGN
 
     def _pp_padded_rows(self):
-        return [(self.lm_head.weight, self.padded_vocab)]
+        rows = [(self.lm_head.weight, self.padded_vocab)]
+        if self.lm_head.bias is not None:
+            rows.append((self.lm_head.bias, self.padded_vocab))   # zeros beyond the vocabulary, like the weight
+        return rows
 
     def forward(self, x):
         if self.ln_f is not None:
@@ -1028,17 +1076,38 @@ class WrappedTokenEmbedding(TokenEmbedding):
         self.wpe = wpe
 
 
+class WrappedEncoderEmbedding(EncoderEmbedding):
+    def __init__(self, word: nn.Embedding, position: nn.Embedding, token_type: nn.Embedding, norm: nn.LayerNorm):
+        NativeBlock.__init__(self)
+        self.word_embeddings, self.position_embeddings, self.token_type_embeddings = word, position, token_type
+        self.LayerNorm = norm
+
+
 class WrappedTransformerLayer(TransformerLayer):
-    def __init__(self, ln_1: nn.LayerNorm, c_attn: nn.Linear, c_proj: nn.Linear, ln_2: nn.LayerNorm,
-                 c_fc: nn.Linear, mlp_proj: nn.Linear, n_heads: int, causal: bool, activation: str):
+    """``TransformerLayer`` around a user's layers.  ``c_attn`` is the fused q|k|v projection or the
+    three separate ones; ``pre_ln=False`` is the encoder form, where ``ln_1`` / ``ln_2`` follow the two
+    residual additions."""
+
+    def __init__(self, ln_1: nn.LayerNorm, c_attn, c_proj: nn.Linear, ln_2: nn.LayerNorm,
+                 c_fc: nn.Linear, mlp_proj: nn.Linear, n_heads: int, causal: bool, activation: str,
+                 pre_ln: bool = True):
         NativeBlock.__init__(self)
         self.dim, self.n_heads, self.ffn = c_proj.out_features, n_heads, c_fc.out_features
-        self.causal, self.pre_ln, self.activation = causal, True, activation
+        self.causal, self.pre_ln, self.activation = causal, pre_ln, activation
         self.ln_1, self.ln_2 = ln_1, ln_2
         self.attn = nn.Module()
-        self.attn.c_attn, self.attn.c_proj = c_attn, c_proj
+        self.attn.c_proj = c_proj
+        if isinstance(c_attn, (tuple, list)):
+            self.attn.q, self.attn.k, self.attn.v = c_attn
+            self._qkv = tuple(c_attn)
+        else:
+            self.attn.c_attn = c_attn
+            self._qkv = (c_attn,)
         self.mlp = nn.Module()
         self.mlp.c_fc, self.mlp.c_proj = c_fc, mlp_proj
+
+    def _qkv_layers(self):
+        return self._qkv
 
 
 class WrappedLlamaLayer(LlamaLayer):

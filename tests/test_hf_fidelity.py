@@ -257,3 +257,36 @@ def test_hugging_face_llama_stages_are_recognised_on_the_models_own_layers():
         for b in blocks[0] + blocks[1]:
             x = b(x)
         _close(x, model(ids).logits, "blocks against LlamaForCausalLM")
+
+
+def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
+    """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
+    and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true
+    mask read as "no mask", and the masked-language-model head."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.BertConfig(hidden_size=128, intermediate_size=512, num_hidden_layers=4, num_attention_heads=2,
+                                  vocab_size=500, max_position_embeddings=64, hidden_dropout_prob=0.0,
+                                  attention_probs_dropout_prob=0.0, tie_word_embeddings=False)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.BertForMaskedLM(cfg)
+    ids = torch.randint(0, 500, (2, 48))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"bert.encoder.layer.2": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedEncoderEmbedding"] + ["WrappedTransformerLayer"] * 2,
+         ["WrappedTransformerLayer"] * 2 + ["LinearAct", "WrappedLMHead"]]
+    layer, hf = blocks[1][0], model.bert.encoder.layer[2]
+    assert not layer.pre_ln and not layer.causal and layer.activation == "gelu_erf" and layer.n_heads == 2
+    assert layer._qkv_layers() == (hf.attention.self.query, hf.attention.self.key, hf.attention.self.value)
+    assert layer.ln_1 is hf.attention.output.LayerNorm and layer.ln_2 is hf.output.LayerNorm
+    assert blocks[0][0].token_type_embeddings is model.bert.embeddings.token_type_embeddings
+    assert blocks[1][-1].lm_head is model.cls.predictions.decoder and blocks[1][-1].lm_head.bias is not None
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against BertForMaskedLM")
