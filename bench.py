@@ -160,6 +160,28 @@ def build_other(args):
                          "pipeline(), 4 virtual stages on one GPU, schedule 1f1b, batch 32 in 8 microbatches, "
                          f"bf16 with fp32 gradient accumulation ({args.accumulate_text})")
         return model, sched, stages, ids.cuda(), target.cuda()
+    if args.workload == "hf_bert":
+        # the BERT-base inference configuration on transformers.BertModel itself
+        import transformers
+        cfg = transformers.BertConfig(hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+        cfg._attn_implementation = "sdpa"
+        model = transformers.BertModel(cfg, add_pooling_layer=False).to(torch.bfloat16).eval()
+        ids = torch.randint(0, cfg.vocab_size, (64, 512))
+        pipe = pp.pipeline(model, mb_args=(ids[:8],),
+                           split_spec={f"encoder.layer.{i}": pp.SplitPoint.BEGINNING for i in (3, 6, 9)})
+        stages = [pp.PipelineStage(pipe, i, "cuda") for i in range(4)]
+        eager = [st.eager_reason for st in stages if not st.is_native]
+        if eager:
+            raise RuntimeError(f"a stage of the Hugging Face model did not lower: {eager}")
+        sched = pp.ScheduleGPipe(stages, 8)
+        args.tokens, args.training = ids.numel(), False
+        per_token = 12 * (2 * 768 * 3 * 768 + 2 * 768 * 768 + 4 * 768 * 3072 + 4 * 512 * 768)
+        args.flops = float(per_token) * ids.numel()
+        args.describe = ("transformers.BertModel (BERT-base: 12 post-LayerNorm layers, hidden 768, 12 heads, FFN "
+                         "3072, vocab 30522, seq 512; random weights), exported and cut by pipeline(), inference, "
+                         "4 virtual stages on one GPU, schedule gpipe, batch 64 in 8 microbatches, bf16")
+        args.batch, args.seq = 64, 512
+        return model, sched, stages, ids.cuda(), None
     raise ValueError(args.workload)
 
 
@@ -323,11 +345,11 @@ def main():
                     help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
                          "events, cold operands), torch.matmul (the vendor library) on the same operands beside "
                          "it, and sample the shader clock during each; one JSON line per shape")
-    ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe", "hf_gpt2"],
+    ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe", "hf_gpt2", "hf_bert"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
                          "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
-                         "configurations at full size; hf_gpt2: the headline configuration on "
-                         "transformers.GPT2LMHeadModel itself")
+                         "configurations at full size; hf_gpt2 / hf_bert: the headline and the BERT-base configurations on "
+                         "transformers.GPT2LMHeadModel / transformers.BertModel themselves")
     # workload shape (defaults: GPT-2 small, configs[2])
     ap.add_argument("--vocab", type=int, default=50257)
     ap.add_argument("--seq", type=int, default=1024)

@@ -2,8 +2,11 @@
 
 A stage lowers when it is a chain: its forward applies one lowerable piece after another to a
 single tensor.  Lowerable pieces are the blocks of ``stage_modules`` and the standard torch layers
-``nn.Linear`` (optionally followed by ReLU / GELU), ``nn.LayerNorm`` and ``nn.RMSNorm``.  Anything else returns
-None and the stage runs through torch autograd like the reference does.
+``nn.Linear`` (optionally followed by ReLU / GELU), ``nn.LayerNorm`` and ``nn.RMSNorm``.  A stage that is
+not such a chain still lowers when its graph is a stack of transformer layers written with plain
+layers (second half of this file): the GPT-2, BERT and Llama families, traced with ``torch.fx`` or
+exported with ``torch.export``.  Anything else returns None and the stage runs through torch autograd
+like the reference does.
 """
 from __future__ import annotations
 
@@ -209,13 +212,22 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 
 
 # ---- transformers written with plain torch layers ---------------------------------------------------
-# Recognised, in this order along the stage: an optional embedding front (token table, optionally plus
-# a position table indexed by arange), any number of pre-LayerNorm residual pairs
-#     x = x + proj(scaled_dot_product_attention(split(qkv(ln(x)))))      x = x + fc2(gelu(fc1(ln(x))))
-# and an optional tail of a final LayerNorm and a bias-free vocabulary projection.  The walk only looks
-# at which layers feed which residual add; how the model reshapes between them is not parsed but
-# checked: the torch statement of the recognised blocks must reproduce the stage's own forward on a
-# random input (fp32, on the host), otherwise the stage stays with torch autograd.
+# Recognised, in this order along the stage:
+#  * an optional embedding front: a token table, optionally plus a position table indexed by 0 .. S-1
+#    (GPT-2), or word + position + token-type-0 tables under a LayerNorm (BERT);
+#  * any number of residual pairs, attention then feed-forward, of one of three forms
+#      pre-LayerNorm    x = x + proj(sdpa(qkv(ln(x))))                 x = x + fc2(gelu(fc1(ln(x))))
+#      post-LayerNorm   x = ln(x + proj(sdpa(qkv(x))))                 x = ln(x + fc2(gelu(fc1(x))))
+#      rotary, gated    x = x + o(sdpa(rope(q(n(x)), k(n(x))), v(n(x)))) x = x + down(silu(gate(n(x))) * up(n(x)))
+#    where qkv is one fused projection or three separate ones, the affine layers are ``nn.Linear`` or
+#    layers with an [in, out] weight, the activations are functions, torch.nn modules or a library's own
+#    activation classes, n is an RMS norm, attention is ``scaled_dot_product_attention`` with
+#    ``is_causal``, no mask, or a constant mask that is causal or masks nothing, and the rotary tables
+#    are constants of the (exported) stage;
+#  * an optional tail: projections with activations, a final norm, the vocabulary projection.
+# The walk only looks at which layers feed which residual add; how the model reshapes between them is
+# not parsed but checked: the torch statement of the recognised blocks must reproduce the stage's own
+# forward on a random input (fp32, on the host), otherwise the stage stays with torch autograd.
 _SDPA = (F.scaled_dot_product_attention, _ATEN.scaled_dot_product_attention.default)
 _ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor)
 _ACT_FNS = (F.gelu, F.relu, torch.relu, F.silu, _ATEN.gelu.default, _ATEN.relu.default, _ATEN.silu.default)

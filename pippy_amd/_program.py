@@ -98,6 +98,7 @@ class ParamArena:
         self.named = params
         # transposed copies of linear weights ([in, out]) for the input-gradient GEMMs
         self._transposed: Dict[int, Tuple[nn.Parameter, torch.Tensor]] = {}
+        self._stacked: Dict[Tuple[int, ...], Tuple[torch.Tensor, List[Tuple[nn.Parameter, torch.Tensor]]]] = {}
         self._versions = None
         self._epoch = 0  # bumped by updates that write the arena directly (fused optimizers)
 
@@ -133,18 +134,38 @@ class ParamArena:
             self._transposed[key] = ent
         return ent[1]
 
+    def rows_cat(self, *ps: nn.Parameter) -> torch.Tensor:
+        """[out1 + out2 + ..., in] (or the 1-d analogue for biases): copies of parameters with the same
+        trailing shape stacked along dimension 0, so that projections which read the same input run as
+        ONE GEMM.  Kept in step with the parameters by ``refresh_transposed``."""
+        key = tuple(id(p) for p in ps)
+        ent = self._stacked.get(key)
+        if ent is None:
+            ws = [self.weight(p, padded=True) for p in ps]
+            t = torch.cat(ws, dim=0)
+            parts, lo = [], 0
+            for p, w in zip(ps, ws):
+                parts.append((p, t[lo:lo + w.shape[0]]))
+                lo += w.shape[0]
+            ent = (t, parts)
+            self._stacked[key] = ent
+        return ent[0]
+
     def refresh_transposed(self) -> None:
-        """Re-transposes the weights whose parameter changed since the last call (an optimizer
-        step bumps the parameter's version counter)."""
-        if not self._transposed:
+        """Re-transposes (re-copies) the weights whose parameter changed since the last call (an
+        optimizer step bumps the parameter's version counter)."""
+        if not self._transposed and not self._stacked:
             return
         live = [(p, t) for p, t in self._transposed.values() if p is not None]
-        versions = (self._epoch,) + tuple(p._version for p, _ in live)
+        stacked = [(p, view) for _, parts in self._stacked.values() for p, view in parts]
+        versions = (self._epoch,) + tuple(p._version for p, _ in live + stacked)
         if versions == self._versions:
             return
         self._versions = versions
         for p, t in live:
             N.transpose_bf16(self.weight(p, padded=True), t)
+        for p, view in stacked:
+            view.copy_(self.weight(p, padded=True))
 
     def mark_updated(self) -> None:
         """The parameter arena was written behind the parameters' version counters."""
@@ -650,6 +671,9 @@ class Builder:
 
     def weight_t_cat(self, *ps):
         return self.sp.arena.weight_t_cat(*ps)
+
+    def rows_cat(self, *ps):
+        return self.sp.arena.rows_cat(*ps)
 
     def grad_target(self, p, padded=True):
         """Where the W pass writes a microbatch gradient that no GEMM epilogue accumulates: the

@@ -59,6 +59,25 @@ def lower_linear(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor, *
     return y, pre
 
 
+def lower_stacked_linears(b: "P.Builder", name: str, layers, x2d: torch.Tensor) -> torch.Tensor:
+    """[y1 | y2 | ...] for ``nn.Linear`` layers that read the same input, as one GEMM with the arena's
+    stacked copy of their weights (and biases); three GEMMs into column ranges of the buffer when only
+    some of them have a bias."""
+    T = x2d.shape[0]
+    y = b.act(name, (T, sum(lin.out_features for lin in layers)))
+    biases = [lin.bias for lin in layers]
+    if all(bias is None for bias in biases) or all(bias is not None for bias in biases):
+        bias = b.rows_cat(*biases) if biases[0] is not None else None
+        b.f(P.op_gemm(x2d, b.rows_cat(*(lin.weight for lin in layers)), y,
+                      epilogue=N.EPI_BIAS if bias is not None else N.EPI_NONE, bias=bias))
+        return y
+    lo = 0
+    for k, lin in enumerate(layers):
+        lower_linear(b, f"{name}{k}", lin, x2d, out=y[:, lo:lo + lin.out_features])
+        lo += lin.out_features
+    return y
+
+
 def bias_grad(b: "P.Builder", lin: nn.Linear, dY2d: torch.Tensor):
     """db = column sum of dY (W pass)."""
     if lin.bias is None:
@@ -387,12 +406,7 @@ class TransformerLayer(NativeBlock):
         layers = self._qkv_layers()
         if len(layers) == 1:
             return lower_linear(b, "qkv", layers[0], h2d)[0]
-        qkv = b.act("qkv", (h2d.shape[0], sum(lin.out_features for lin in layers)))
-        lo = 0
-        for name, lin in zip("qkv", layers):      # each GEMM writes its column range
-            lower_linear(b, name, lin, h2d, out=qkv[:, lo:lo + lin.out_features])
-            lo += lin.out_features
-        return qkv
+        return lower_stacked_linears(b, "qkv", layers, h2d)
 
     def _qkv_backward(self, b, h2d, dqkv, *, dx_epilogue=N.EPI_NONE, dx_aux=None, dx_out=None):
         """Emits input and weight gradients of the projection; returns the gradient of its input."""
@@ -1154,13 +1168,7 @@ class WrappedLlamaLayer(LlamaLayer):
         return torch.cat([lin(h) for lin in self._projections()], dim=-1)
 
     def _lower_qkv(self, b, n1):
-        W = sum(lin.out_features for lin in self._projections())
-        qkv = b.act("qkv", (n1.shape[0], W))
-        lo = 0
-        for name, lin in zip("qkv", self._projections()):
-            lower_linear(b, name, lin, n1, out=qkv[:, lo:lo + lin.out_features])
-            lo += lin.out_features
-        return qkv
+        return lower_stacked_linears(b, "qkv", self._projections(), n1)
 
     def _qkv_backward(self, b, n1, dqkv):
         d_n1 = b.grad("qkv.dx", (n1.shape[0], n1.shape[1]))
