@@ -186,3 +186,37 @@ def test_a_mask_that_is_not_causal_keeps_the_stage_with_torch():
     why = []
     assert lower_stage_module(pipe.get_stage_module(1), why) is None
     assert "mask" in why[0]
+
+
+def test_shared_layers_mutated_buffers_and_keyword_inputs_survive_the_graph_passes():
+    """A layer called twice is put back twice; buffers that the forward writes (batch-norm statistics, a
+    step counter) are not mistaken for constants; keyword inputs reach the stage that reads them."""
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.shared, self.b = nn.Linear(8, 8), nn.Linear(8, 8), nn.Linear(8, 4)
+            self.bn = nn.BatchNorm1d(8)
+            self.register_buffer("steps", torch.zeros(()))
+
+        def forward(self, x, scale=None):
+            if x.shape[0] > 1:
+                x = self.a(x)
+            x = self.bn(self.shared(torch.relu(self.shared(x))))
+            self.steps += 1
+            pp.pipe_split()
+            if scale is not None:
+                x = x * scale
+            return self.b(x)
+
+    torch.manual_seed(0)
+    model, ref = Net(), Net()
+    ref.load_state_dict(model.state_dict())
+    x, scale = torch.randn(4, 8), torch.rand(4, 1)
+    pipe = pp.pipeline(model, mb_args=(x,), mb_kwargs={"scale": scale})
+    assert pipe.num_stages == 2
+    calls = [n.target for n in pipe.get_stage_module(0).graph.nodes if n.op == "call_module"]
+    assert calls == ["a", "shared", "shared"]
+    for _ in range(2):
+        torch.testing.assert_close(pipe(x, scale=scale), ref(x, scale=scale), rtol=0, atol=0)
+    assert model.steps.item() == ref.steps.item() == 2      # (exporting runs the forward on fake tensors only)
+    torch.testing.assert_close(model.bn.running_var, ref.bn.running_var)
