@@ -344,8 +344,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     kinds = [kind(n, m) for n, m in mods]
     if kinds == ["RMSNorm", "Linear", "Linear", "Linear", "sdpa", "Linear"]:
         (_, norm), (_, q), (_, k), (_, v), (sd, _), (_, o) = mods
-        if any(lin.bias is not None for lin in (q, k, v, o)) or not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
-            raise NotLowerable("rotary attention whose projections have biases or [in, out] weights")
+        if not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
+            raise NotLowerable("rotary attention whose projections keep [in, out] weights")
         if k.out_features != v.out_features or q.out_features != o.in_features or q.out_features != q.in_features \
                 or q.out_features % k.out_features:
             raise NotLowerable("query / key / value projections of unexpected widths")
@@ -443,7 +443,13 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
             if not joins:
                 raise NotLowerable("token and position embeddings are not simply added")
             stream = joins[0]
-            blocks.append(WrappedTokenEmbedding(wte, root.get_submodule(emb[1].target)))
+            after = list(stream.users)
+            norm = root.get_submodule(after[0].target) if len(after) == 1 and after[0].op == "call_module" else None
+            if isinstance(norm, nn.LayerNorm):      # an encoder front without token types
+                stream = after[0]
+                blocks.append(WrappedEncoderEmbedding(wte, root.get_submodule(emb[1].target), None, norm))
+            else:
+                blocks.append(WrappedTokenEmbedding(wte, root.get_submodule(emb[1].target)))
         else:
             stream = emb[0]
             blocks.append(WrappedTokenEmbedding(wte, None))

@@ -300,7 +300,8 @@ class TokenEmbedding(NativeBlock):
 
 class EncoderEmbedding(NativeBlock):
     """BERT-style embedding: ``LayerNorm(word[ids] + position[:S] + token_type[0])``.  All tokens
-    are of type 0, which is what the encoder computes when no ``token_type_ids`` are passed."""
+    are of type 0, which is what the encoder computes when no ``token_type_ids`` are passed.  A
+    wrapper around a user's layers may have no token-type table (``token_type_embeddings = None``)."""
 
     def __init__(self, vocab: int, max_seq: int, dim: int, n_types: int = 2, eps: float = 1e-12,
                  dtype=torch.bfloat16, init_std=0.02):
@@ -316,9 +317,10 @@ class EncoderEmbedding(NativeBlock):
         S = ids.shape[-1]
         pos = torch.arange(S, device=ids.device)
         # one rounding of the three-term sum, as the lowered kernel does
-        e = (self.word_embeddings(ids).float() + self.position_embeddings(pos).float()
-             + self.token_type_embeddings.weight[0].float()).to(self.word_embeddings.weight.dtype)
-        return self.LayerNorm(e)
+        e = self.word_embeddings(ids).float() + self.position_embeddings(pos).float()
+        if self.token_type_embeddings is not None:
+            e = e + self.token_type_embeddings.weight[0].float()
+        return self.LayerNorm(e.to(self.word_embeddings.weight.dtype))
 
     def _pp_direct_acc_params(self):
         return [self.word_embeddings.weight, self.position_embeddings.weight]
@@ -329,13 +331,13 @@ class EncoderEmbedding(NativeBlock):
                                f"{ids.dtype} {tuple(ids.shape)}")
         Bn, S = ids.shape
         wte, wpe = b.weight(self.word_embeddings.weight), b.weight(self.position_embeddings.weight)
-        wtt = b.weight(self.token_type_embeddings.weight)
+        wtt = b.weight(self.token_type_embeddings.weight) if self.token_type_embeddings is not None else None
         if S > wpe.shape[0]:
             raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
         Cc = wte.shape[1]
         T = Bn * S
         e = b.act("e", (T, Cc))
-        b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0]))
+        b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0] if wtt is not None else None))
         y, mean, rstd = lower_layernorm(b, "ln", self.LayerNorm, e)
 
         def bwd(dy, need_dx, dx_out):
@@ -346,10 +348,11 @@ class EncoderEmbedding(NativeBlock):
             b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
             _zero_padding_row(b, self.word_embeddings, acc_wte)
-            # the type-0 row receives the gradient of every token; the other rows none
-            g_tt = b.grad_target(self.token_type_embeddings.weight)
-            ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)
-            b.w_reduce(P.op_colsum(de, g_tt[0], ws))
+            if wtt is not None:
+                # the type-0 row receives the gradient of every token; the other rows none
+                g_tt = b.grad_target(self.token_type_embeddings.weight)
+                ws = b.workspace("colsum:tt", (2 * ((T + 127) // 128) * Cc,), torch.float32)
+                b.w_reduce(P.op_colsum(de, g_tt[0], ws))
             return None
 
         b.on_backward(bwd)

@@ -1212,3 +1212,56 @@ def test_hugging_face_bert_runs_natively_and_matches_the_oracle():
         return None
 
     _exported_model_against_the_oracle(model, Logits, 1003, 128, "bert.encoder.layer.2", scale_like=projection_group)
+
+
+def _qkv_group(name):
+    """The sibling query / key / value parameters of ``name`` (None if it is none of them)."""
+    for names in (("query", "key", "value"), ("q_lin", "k_lin", "v_lin"), ("q_proj", "k_proj", "v_proj")):
+        for part in names:
+            if f".{part}." in name:
+                return [name.replace(f".{part}.", f".{p}.") for p in names if p != part]
+    return None
+
+
+@pytest.mark.parametrize("family", ["qwen2", "mistral", "distilbert", "electra"])
+def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
+    """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
+    value projections), Mistral (Llama layout), DistilBERT (encoder without token types, its own layer
+    names), ELECTRA (BERT layout with a generator head)."""
+    T = pytest.importorskip("transformers")
+    import torch.nn as nn
+    common = dict(vocab_size=1000, tie_word_embeddings=False)
+    llama_like = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=4, num_attention_heads=4,
+                      num_key_value_heads=2, max_position_embeddings=128, attention_dropout=0.0, use_cache=False)
+    cls, cfg, split = {
+        "qwen2": lambda: (T.Qwen2ForCausalLM, T.Qwen2Config(**llama_like, **common), "model.layers.2"),
+        "mistral": lambda: (T.MistralForCausalLM, T.MistralConfig(sliding_window=None, **llama_like, **common),
+                            "model.layers.2"),
+        "distilbert": lambda: (T.DistilBertForMaskedLM,
+                               T.DistilBertConfig(dim=128, hidden_dim=512, n_layers=4, n_heads=2,
+                                                  max_position_embeddings=128, dropout=0.0, attention_dropout=0.0,
+                                                  **common), "distilbert.transformer.layer.2"),
+        "electra": lambda: (T.ElectraForMaskedLM,
+                            T.ElectraConfig(hidden_size=128, embedding_size=128, intermediate_size=512,
+                                            num_hidden_layers=4, num_attention_heads=2, max_position_embeddings=128,
+                                            hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, **common),
+                            "electra.encoder.layer.2"),
+    }[family]()
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = cls(cfg)
+    if family == "qwen2":
+        with torch.no_grad():      # the library initialises biases to zero: give them values
+            for name, p in model.named_parameters():
+                if name.endswith("_proj.bias"):
+                    p.normal_(std=0.05)
+
+    class Logits(nn.Module):
+        def __init__(self, g):
+            super().__init__()
+            self.g = g
+
+        def forward(self, idx):
+            return self.g(idx).logits
+
+    _exported_model_against_the_oracle(model, Logits, 1000, 128, split, scale_like=_qkv_group)
