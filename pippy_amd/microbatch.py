@@ -347,26 +347,44 @@ def cat_chunks(values: Sequence[torch.Tensor], dim: int) -> torch.Tensor:
     for v in values:
         d = v.size(dim)
         if v.numel():
-            rv = _row_view(v, dim)
-            if rv is None:  # arbitrary strides: gather into a contiguous staging tensor first
-                tmp = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-                _native.strided_copy_nd(tmp, v)
-                keep_alive.append(tmp)
-                v = tmp
-                rv = (outer, d * inner, d * inner, 1)
-            n_rows, row_bytes, src_stride, rows_per_outer = rv
-            if rows_per_outer == 1:
-                assert row_bytes == d * inner and n_rows == outer
-                dst_stride = total * inner
-            else:
-                assert outer == 1 and n_rows * row_bytes == d * inner
-                dst_stride = row_bytes
-            segs.append((v.data_ptr(), out.data_ptr() + lo * inner, n_rows, row_bytes, src_stride,
-                         dst_stride))
+            segs.append(_segment(v, out.data_ptr() + lo * inner, dim, total, outer, inner, keep_alive))
         lo += d
     _native.copy_rows(segs)
     del keep_alive
     return out
+
+
+def _segment(v: torch.Tensor, dst_ptr: int, dim: int, total: int, outer: int, inner: int, keep_alive: list):
+    """The row-copy segment that writes ``v`` into its place along ``dim`` of a contiguous tensor whose
+    size along ``dim`` is ``total`` (``outer`` / ``inner`` as ``_rows`` gives them for that tensor)."""
+    d = v.size(dim)
+    rv = _row_view(v, dim)
+    if rv is None:  # arbitrary strides: gather into a contiguous staging tensor first
+        tmp = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+        _native.strided_copy_nd(tmp, v)
+        keep_alive.append(tmp)
+        v = tmp
+        rv = (outer, d * inner, d * inner, 1)
+    n_rows, row_bytes, src_stride, rows_per_outer = rv
+    if rows_per_outer == 1:
+        assert row_bytes == d * inner and n_rows == outer
+        dst_stride = total * inner
+    else:
+        assert outer == 1 and n_rows * row_bytes == d * inner
+        dst_stride = row_bytes
+    return (v.data_ptr(), dst_ptr, n_rows, row_bytes, src_stride, dst_stride)
+
+
+def copy_into_rows(out: torch.Tensor, lo: int, v: torch.Tensor) -> None:
+    """``out[lo : lo + v.size(0)] = v`` for a contiguous device tensor ``out`` and a chunk ``v`` of any
+    strides, on the current stream: one microbatch's share of ``cat_chunks(values, 0)``."""
+    assert out.is_contiguous() and out.is_cuda and v.shape[1:] == out.shape[1:] and v.dtype == out.dtype
+    if not v.numel():
+        return
+    outer, inner = _rows(list(out.shape), 0, out.element_size())
+    keep_alive = []
+    _native.copy_rows([_segment(v, out.data_ptr() + lo * inner, 0, out.size(0), outer, inner, keep_alive)])
+    del keep_alive
 
 
 def _own_slices(values: Sequence[torch.Tensor], dim: int) -> List[torch.Tensor]:

@@ -24,10 +24,61 @@ from torch.profiler import record_function
 from contextlib import nullcontext
 
 from . import _schedule_order as order
-from .microbatch import merge_chunks, split_args_kwargs_into_chunks
+from . import microbatch as _microbatch
+from .microbatch import TensorChunkSpec, copy_into_rows, merge_chunks, split_args_kwargs_into_chunks
 from .stage import PipelineStageBase, link_stages
 
 logger = logging.getLogger(__name__)
+
+
+class _RunningMerge:
+    """Builds the merged output of a step while the step is still running: every microbatch output of
+    the last stage is copied into its rows of the result as soon as its forward pass has been issued,
+    on a stream of its own (an HBM-bound copy next to the MFMA-bound kernels of the other passes),
+    instead of all of them after the last backward pass.  The result is the same freshly allocated
+    contiguous tensor that ``merge_chunks`` returns.  Used when the output is one tensor merged along
+    dimension 0 and all microbatches have the same size; anything else is merged at the end as before."""
+
+    def __init__(self, n_microbatches: int, device):
+        self.n = n_microbatches
+        self.stream = torch.cuda.Stream(device=device)
+        self.out: Optional[torch.Tensor] = None
+        self.rows = 0
+        self.done = 0
+        self.ok = True
+
+    def reset(self):
+        self.out, self.rows, self.done, self.ok = None, 0, 0, True
+
+    def add(self, m: int, chunk, produced_on: "torch.cuda.Stream", main: "torch.cuda.Stream"):
+        if not self.ok:
+            return
+        if not isinstance(chunk, torch.Tensor) or not chunk.is_cuda or chunk.dim() == 0 or m != self.done:
+            self.ok = False
+            return
+        if self.out is None:
+            self.rows = chunk.shape[0]
+            with torch.cuda.stream(main):      # allocated (and later freed) under the caller's stream
+                self.out = torch.empty((self.n * self.rows,) + tuple(chunk.shape[1:]), dtype=chunk.dtype,
+                                       device=chunk.device)
+            self.out.record_stream(self.stream)
+        elif chunk.shape != (self.rows,) + tuple(self.out.shape[1:]) or chunk.dtype != self.out.dtype:
+            self.ok = False
+            return
+        ready = torch.cuda.Event()
+        ready.record(produced_on)
+        self.stream.wait_event(ready)
+        with torch.cuda.stream(self.stream):
+            copy_into_rows(self.out, m * self.rows, chunk)
+        self.done += 1
+
+    def result(self, main: "torch.cuda.Stream") -> Optional[torch.Tensor]:
+        """The merged tensor once every microbatch has been added (the caller's stream then waits for
+        the copies), else None."""
+        if not self.ok or self.out is None or self.done != self.n:
+            return None
+        main.wait_stream(self.stream)
+        return self.out
 
 
 class PipelineSchedule(ABC):
@@ -46,6 +97,10 @@ class PipelineSchedule(ABC):
         self._streams = None
         self._w_streams = None
         self._events: Dict[Any, Any] = {}
+        #: copy microbatch outputs into the merged result while the step runs (see ``_RunningMerge``)
+        self.merge_while_running = True
+        self._running_merge: Optional[_RunningMerge] = None
+        self._merge_active: Optional[_RunningMerge] = None
         logger.info(f"Using {self.__class__.__name__}")
 
     # -- losses (reference ``PipelineSchedule.py:39-80``) -------------------------------------------
@@ -164,6 +219,7 @@ class PipelineSchedule(ABC):
         main = torch.cuda.current_stream()
         start = self._event("start")
         start.record(main)
+        merger = self._merger(main)
         w_streams = self._w_streams
         for st in list(streams.values()) + list(w_streams.values()):
             st.wait_event(start)
@@ -191,6 +247,8 @@ class PipelineSchedule(ABC):
                 self._run_action(kind, s, m, arg_mbs, kwarg_mbs, target_mbs)
                 if kind == "F":
                     self._event(("F", s, m)).record(st)
+                    if merger is not None and s == last:
+                        merger.add(m, self._by_index[s].output_chunks[m], st, main)
                 elif kind in ("B", "I"):
                     self._event(("B", s, m)).record(st)
         for s, st in streams.items():
@@ -201,6 +259,21 @@ class PipelineSchedule(ABC):
             done = self._event(("done_w", s))
             done.record(w_streams[s])
             main.wait_event(done)
+
+    def _merger(self, main) -> Optional[_RunningMerge]:
+        """The running merge of this step, or None when outputs are merged at the end."""
+        default_spec = self._output_merge_spec is None or (
+            isinstance(self._output_merge_spec, TensorChunkSpec) and self._output_merge_spec.split_dim == 0)
+        self._merge_active = None
+        if not self.merge_while_running or os.environ.get("PIPPY_AMD_MERGE_AT_END") == "1" or not default_spec \
+                or _microbatch._debug_mask_minibatches:
+            return None
+        if self._running_merge is None or self._running_merge.n != self._n_microbatches:
+            self._running_merge = _RunningMerge(self._n_microbatches, main.device)
+        self._running_merge.stream.wait_stream(main)
+        self._running_merge.reset()
+        self._merge_active = self._running_merge
+        return self._running_merge
 
     @staticmethod
     def _range(name: str):
@@ -261,9 +334,15 @@ class PipelineSchedule(ABC):
             targets_split = list(torch.tensor_split(target, self._n_microbatches))
         else:
             targets_split = None
+        self._merge_active = None
         self._step_microbatches(args_split, kwargs_split, targets_split, losses)
         for stage in self._stages:
             if stage.is_last:
+                if self._merge_active is not None:
+                    merged = self._merge_active.result(torch.cuda.current_stream())
+                    self._merge_active.out = None
+                    if merged is not None:
+                        return merged
                 return self._merge_outputs(stage.output_chunks)
         return None
 

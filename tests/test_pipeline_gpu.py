@@ -1265,3 +1265,35 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
             return self.g(idx).logits
 
     _exported_model_against_the_oracle(model, Logits, 1000, 128, split, scale_like=_qkv_group)
+
+
+def test_outputs_merged_while_the_step_runs_are_the_merge_at_the_end(monkeypatch):
+    """The schedule copies each microbatch output of the last stage into the merged result as soon as
+    its forward pass is issued (a side stream).  The result must be bit for bit what merging after the
+    step gives, a tensor of its own (a later step must not change it), contiguous like torch.cat's, and
+    uneven microbatches must fall back to the merge at the end."""
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    target = torch.randint(0, 1000, ids.shape)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    ids2 = torch.randint(0, 1000, ids.shape)
+    out1 = sched.step(ids.to(DEV), target=target.to(DEV))
+    assert sched._merge_active is not None and out1.is_contiguous()
+    kept = out1.clone()
+    at_end1 = torch.cat([c.clone() for c in stages[-1].output_chunks])
+    assert torch.equal(out1, at_end1)
+    out2 = sched.step(ids2.to(DEV), target=target.to(DEV))
+    assert torch.equal(out1, kept) and not torch.equal(out2, out1)
+    monkeypatch.setenv("PIPPY_AMD_MERGE_AT_END", "1")
+    out2_at_end = sched.step(ids2.to(DEV), target=target.to(DEV))
+    assert sched._merge_active is None and torch.equal(out2, out2_at_end)
+    monkeypatch.delenv("PIPPY_AMD_MERGE_AT_END")
+    # 10 sequences in 4 microbatches: sizes 3, 3, 2, 2
+    uneven = torch.randint(0, 1000, (10, ids.shape[1]))
+    infer = pp.ScheduleGPipe(stages, M)
+    out = infer.step(uneven.to(DEV))
+    assert out.shape[0] == 10
+    assert torch.equal(out, torch.cat([c.clone() for c in stages[-1].output_chunks]))
+    ref_out, _ = OP.step(ref_stages, uneven, None, M, None)
+    assert_close_rel(out, ref_out, BF16_TOL, "uneven microbatches")
