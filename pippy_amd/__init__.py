@@ -7,6 +7,7 @@ virtual stages on one GPU; see ``schedules.py``.
 from . import _debug  # noqa: F401  (sets the logging level from PIPPY_VERBOSITY)
 from ._IR import (ArgsChunkSpec, KwargsChunkSpec, Pipe, PipeSplitWrapper, SplitPoint,
                   annotate_split_points, pipe_split, pipeline)
+from ._split_policies import split_by_graph, split_into_equal_size, split_on_size_threshold
 from .losses import CrossEntropyLoss
 from .optim import FusedAdamW, FusedSGD
 from .microbatch import TensorChunkSpec, merge_chunks, split_args_kwargs_into_chunks, sum_reducer
@@ -21,5 +22,6 @@ __all__ = [
     "KwargsChunkSpec", "TensorChunkSpec", "PipelineStage", "ManualPipelineStage", "Schedule1F1B",
     "ScheduleGPipe", "ScheduleInterleaved1F1B", "ScheduleLoopedBFS", "ScheduleZeroBubble",
     "split_args_kwargs_into_chunks", "merge_chunks", "sum_reducer", "CrossEntropyLoss",
-    "VirtualGroup", "PipeSplitWrapper", "FusedSGD", "FusedAdamW",
+    "VirtualGroup", "PipeSplitWrapper", "FusedSGD", "FusedAdamW", "split_into_equal_size",
+    "split_on_size_threshold", "split_by_graph",
 ]

@@ -46,13 +46,16 @@ class _RunningMerge:
         self.rows = 0
         self.done = 0
         self.ok = True
+        self.wrap = None
 
     def reset(self):
-        self.out, self.rows, self.done, self.ok = None, 0, 0, True
+        self.out, self.rows, self.done, self.ok, self.wrap = None, 0, 0, True, None
 
     def add(self, m: int, chunk, produced_on: "torch.cuda.Stream", main: "torch.cuda.Stream"):
         if not self.ok:
             return
+        if type(chunk) in (tuple, list) and len(chunk) == 1:     # exported models return 1-tuples
+            self.wrap, chunk = type(chunk), chunk[0]
         if not isinstance(chunk, torch.Tensor) or not chunk.is_cuda or chunk.dim() == 0 or m != self.done:
             self.ok = False
             return
@@ -78,7 +81,7 @@ class _RunningMerge:
         if not self.ok or self.out is None or self.done != self.n:
             return None
         main.wait_stream(self.stream)
-        return self.out
+        return self.out if self.wrap is None else self.wrap([self.out])
 
 
 class PipelineSchedule(ABC):

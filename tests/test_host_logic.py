@@ -538,3 +538,28 @@ def test_plain_torch_transformer_is_recognised_and_verified():
     why = []
     assert lower_stage_module(odd, why) is None
     assert "residual" in why[0]
+
+
+# ---- size-based split policies (reference pippy/ModelSplit.py:158-206) ---------------------------------
+def test_split_policies_cut_by_parameter_count():
+    from pippy_amd.configs import DecoderLM
+    torch.manual_seed(0)
+    model = DecoderLM(vocab=1000, max_seq=64, dim=128, n_layers=8, n_heads=2, ffn=512).float()
+    ids = torch.randint(0, 1000, (4, 64))
+    per_layer = sum(p.numel() for p in model.h[0].parameters())
+    pipe = pp.pipeline(model, 2, (ids,), split_policy=pp.split_into_equal_size(4))
+    assert pipe.num_stages == 4
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    sizes = [sum(p.numel() for p in pipe.get_stage_module(i).parameters()) for i in range(4)]
+    assert sum(sizes) == sum(p.numel() for p in model.parameters())
+    assert all(s <= sum(sizes) // 4 for s in sizes[:-1])          # only the last stage may run over
+    # a threshold of three layers: the embedding and two layers, then stages of three layers
+    pipe = pp.pipeline(model, 2, (ids,), split_policy=pp.split_on_size_threshold(3 * per_layer))
+    sizes = [sum(p.numel() for p in pipe.get_stage_module(i).parameters()) for i in range(pipe.num_stages)]
+    assert all(s <= 3 * per_layer for s in sizes) and sizes[1] == 3 * per_layer
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    with pytest.raises(ValueError):
+        pp.pipeline(model, 2, (ids,), split_spec={"h.4": pp.SplitPoint.BEGINNING},
+                    split_policy=pp.split_into_equal_size(2))
+    with pytest.raises(NotImplementedError):
+        pp.split_by_graph(2)
