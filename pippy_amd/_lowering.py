@@ -653,11 +653,34 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     raise NotLowerable("; ".join(reasons))
 
 
-def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None) -> Optional[List[NativeBlock]]:
+def _check_dtypes(submod: nn.Module, blocks: List[NativeBlock]) -> None:
+    """Launch lists compute in the parameter dtype.  The MFMA kernels (GEMM epilogues beyond bias / ReLU,
+    attention, norms, embeddings) are bf16; float32 stages can only be chains of ``nn.Linear`` with no
+    activation or ReLU."""
+    dtypes = {p.dtype for p in submod.parameters()}
+    if len(dtypes) > 1:
+        raise NotLowerable(f"parameters of several dtypes ({sorted(str(d) for d in dtypes)}); a launch-list stage "
+                           "keeps one")
+    if not dtypes or dtypes == {torch.bfloat16}:
+        return
+    if dtypes != {torch.float32}:
+        raise NotLowerable(f"parameters of dtype {dtypes.pop()} (bfloat16 and float32 are built)")
+    for blk in blocks:
+        plain = isinstance(blk, LinearAct) and isinstance(blk.lin, nn.Linear) and blk.activation in (None, "relu")
+        if not plain:
+            raise NotLowerable(f"float32 parameters: {type(blk).__name__} runs as bfloat16 kernels only (convert the "
+                               "model with .to(torch.bfloat16) to run it as launch lists)")
+
+
+def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None, check_dtypes: bool = False) -> Optional[List[NativeBlock]]:
     """Blocks of a lowerable stage module, or None when it has to run eagerly; the reason is then
-    appended to ``why``."""
+    appended to ``why``.  ``check_dtypes`` also requires parameter dtypes that the kernels compute in (the
+    stage runtime asks for it; recognising the structure of a model does not depend on its dtype)."""
     try:
-        return _lower(submod)
+        blocks = _lower(submod)
+        if check_dtypes:
+            _check_dtypes(submod, blocks)
+        return blocks
     except NotLowerable as e:
         if why is not None:
             why.append(str(e))

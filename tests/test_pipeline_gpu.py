@@ -1297,3 +1297,30 @@ def test_outputs_merged_while_the_step_runs_are_the_merge_at_the_end(monkeypatch
     assert torch.equal(out, torch.cat([c.clone() for c in stages[-1].output_chunks]))
     ref_out, _ = OP.step(ref_stages, uneven, None, M, None)
     assert_close_rel(out, ref_out, BF16_TOL, "uneven microbatches")
+
+
+def test_float32_transformer_stages_fall_back_to_autograd_and_say_so():
+    """The attention, norm and embedding kernels are bf16: a float32 model whose structure is recognised
+    still runs, through torch autograd on the GPU, and the stage says why."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import GPT
+    import pippy_amd as pp
+    torch.manual_seed(0)
+    M, vocab, seq = 2, 300, 32
+    model = GPT(vocab=vocab, seq=seq, d=128, h=2, L=2)
+    ref = copy.deepcopy(model)
+    ids = torch.randint(0, vocab, (2 * M, seq))
+    target = torch.randint(0, vocab, (2 * M, seq))
+    pipe = pp.pipeline(model, M, (ids,), split_spec={"h.1": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert not any(st.is_native for st in stages)
+    assert all("float32" in st.eager_reason and "bfloat16" in st.eager_reason for st in stages)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=_ce)
+    losses = []
+    out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    ref_out = ref(ids)
+    torch.testing.assert_close(out.cpu(), ref_out, rtol=1e-4, atol=1e-4)
+    sum(_ce(o, t) for o, t in zip(ref_out.chunk(M), target.chunk(M))).backward()
+    for (name, p), rp in zip(model.named_parameters(), ref.parameters()):
+        torch.testing.assert_close(p.grad.cpu(), rp.grad, rtol=1e-3, atol=1e-5, msg=lambda m: f"{name}: {m}")
