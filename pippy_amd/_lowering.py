@@ -189,7 +189,8 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
             try:
                 return blocks_from_residual_graph(submod)
             except NotLowerable as residual_reason:
-                raise NotLowerable(f"{chain_reason}; as a residual transformer stack: {residual_reason}") from None
+                raise NotLowerable(f"as a stack of transformer layers: {residual_reason}; as a plain chain of layers: "
+                                   f"{chain_reason}") from None
     if isinstance(submod, (nn.Linear, nn.LayerNorm, nn.RMSNorm)):
         # a stage that is one standard layer: the same rules as for that layer inside a chain
         holder = nn.Module()
@@ -208,7 +209,8 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
         try:
             return blocks_from_residual_graph(submod)
         except NotLowerable as residual_reason:
-            raise NotLowerable(f"{chain_reason}; as a residual transformer stack: {residual_reason}") from None
+            raise NotLowerable(f"as a stack of transformer layers: {residual_reason}; as a plain chain of layers: "
+                                   f"{chain_reason}") from None
 
 
 # ---- transformers written with plain torch layers ---------------------------------------------------
@@ -653,33 +655,39 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     raise NotLowerable("; ".join(reasons))
 
 
-def _check_dtypes(submod: nn.Module, blocks: List[NativeBlock]) -> None:
-    """Launch lists compute in the parameter dtype.  The MFMA kernels (GEMM epilogues beyond bias / ReLU,
-    attention, norms, embeddings) are bf16; float32 stages can only be chains of ``nn.Linear`` with no
-    activation or ReLU."""
+def _check_kernel_requirements(submod: nn.Module, blocks: List[NativeBlock]) -> None:
+    """What the kernels need beyond a recognised structure.  Launch lists compute in the parameter
+    dtype: the MFMA kernels (GEMM epilogues beyond bias / ReLU, attention, norms, embeddings) are bf16,
+    float32 stages can only be chains of ``nn.Linear`` with no activation or ReLU.  The attention
+    kernels take sequence lengths that are multiples of 64."""
     dtypes = {p.dtype for p in submod.parameters()}
     if len(dtypes) > 1:
         raise NotLowerable(f"parameters of several dtypes ({sorted(str(d) for d in dtypes)}); a launch-list stage "
                            "keeps one")
-    if not dtypes or dtypes == {torch.bfloat16}:
-        return
-    if dtypes != {torch.float32}:
+    if dtypes and dtypes != {torch.bfloat16} and dtypes != {torch.float32}:
         raise NotLowerable(f"parameters of dtype {dtypes.pop()} (bfloat16 and float32 are built)")
-    for blk in blocks:
+    # an exported stage runs at the shapes of its example microbatch: what the kernels cannot take is known now
+    if isinstance(submod, fx.GraphModule) and any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer))
+                                                   for b in blocks):
+        inputs = [n for n in submod.graph.nodes if n.op == "placeholder"]
+        shape = getattr(inputs[0].meta.get("val"), "shape", None) if len(inputs) == 1 else None
+        if shape is not None and len(shape) >= 2 and int(shape[1]) % 64:
+            raise NotLowerable(f"sequence length {int(shape[1])} (the attention kernels take multiples of 64)")
+    for blk in blocks if dtypes == {torch.float32} else ():
         plain = isinstance(blk, LinearAct) and isinstance(blk.lin, nn.Linear) and blk.activation in (None, "relu")
         if not plain:
             raise NotLowerable(f"float32 parameters: {type(blk).__name__} runs as bfloat16 kernels only (convert the "
                                "model with .to(torch.bfloat16) to run it as launch lists)")
 
 
-def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None, check_dtypes: bool = False) -> Optional[List[NativeBlock]]:
+def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None, for_kernels: bool = False) -> Optional[List[NativeBlock]]:
     """Blocks of a lowerable stage module, or None when it has to run eagerly; the reason is then
-    appended to ``why``.  ``check_dtypes`` also requires parameter dtypes that the kernels compute in (the
-    stage runtime asks for it; recognising the structure of a model does not depend on its dtype)."""
+    appended to ``why``.  ``for_kernels`` also requires what the kernels need of dtypes and (known) shapes;
+    the stage runtime asks for it, recognising the structure of a model does not depend on it."""
     try:
         blocks = _lower(submod)
-        if check_dtypes:
-            _check_dtypes(submod, blocks)
+        if for_kernels:
+            _check_kernel_requirements(submod, blocks)
         return blocks
     except NotLowerable as e:
         if why is not None:

@@ -115,7 +115,7 @@ class PipelineStageBase:
         if not force_eager and self.device.type != "cuda":
             force_eager = True
             why.append(f"its device is '{self.device}' and launch lists run on the GPU only")
-        self._blocks = None if force_eager else lower_stage_module(submodule, why, check_dtypes=True)
+        self._blocks = None if force_eager else lower_stage_module(submodule, why, for_kernels=True)
         self._program: Optional[P.StageProgram] = None
         #: why this stage runs through torch autograd instead of HIP launch lists (None: it is native)
         self.eager_reason: Optional[str] = None

@@ -220,3 +220,21 @@ def test_shared_layers_mutated_buffers_and_keyword_inputs_survive_the_graph_pass
         torch.testing.assert_close(pipe(x, scale=scale), ref(x, scale=scale), rtol=0, atol=0)
     assert model.steps.item() == ref.steps.item() == 2      # (exporting runs the forward on fake tensors only)
     torch.testing.assert_close(model.bn.running_var, ref.bn.running_var)
+
+
+def test_what_the_kernels_cannot_take_keeps_a_recognised_stage_with_torch():
+    """The structure of an exported stage may be recognised and still not run as launch lists: float32
+    parameters (the transformer kernels are bf16) and, known from the exported shapes, a sequence length
+    that is not a multiple of 64."""
+    from pippy_amd._lowering import lower_stage_module
+    model = _lib_gpt()
+    ids = torch.randint(0, 500, (2, 64))
+    stage = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING}).get_stage_module(1)
+    why = []
+    assert lower_stage_module(stage, why) is not None
+    assert lower_stage_module(stage, why, for_kernels=True) is None and "float32" in why[-1]
+    model = _lib_gpt().to(torch.bfloat16)
+    stage = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING}).get_stage_module(1)
+    assert lower_stage_module(stage, why, for_kernels=True) is not None
+    stage = pp.pipeline(model, 1, (ids[:, :48],), split_spec={"h.2": pp.SplitPoint.BEGINNING}).get_stage_module(1)
+    assert lower_stage_module(stage, why, for_kernels=True) is None and "sequence length 48" in why[-1]
