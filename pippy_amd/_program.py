@@ -465,6 +465,9 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
 
 
 def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None) -> N.Op:
+    if qkv.shape[1] % 64:
+        raise RuntimeError(f"the attention kernels take sequence lengths that are multiples of 64, got "
+                           f"{qkv.shape[1]} (pad the sequences, or build the stage with force_eager=True)")
     d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads)
     op = N.Op()
     op.kind = kind

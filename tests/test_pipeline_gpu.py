@@ -1324,3 +1324,20 @@ def test_float32_transformer_stages_fall_back_to_autograd_and_say_so():
     sum(_ce(o, t) for o, t in zip(ref_out.chunk(M), target.chunk(M))).backward()
     for (name, p), rp in zip(model.named_parameters(), ref.parameters()):
         torch.testing.assert_close(p.grad.cpu(), rp.grad, rtol=1e-3, atol=1e-5, msg=lambda m: f"{name}: {m}")
+
+
+def test_a_sequence_length_the_attention_kernels_do_not_take_is_refused_before_any_launch():
+    """A traced stage is shape-generic, so an unsupported sequence length shows when the launch lists are
+    built: the error names the limit and the way out, and ``force_eager=True`` runs the same pipe."""
+    import pippy_amd as pp
+    from pippy_amd.configs import DecoderLM, equal_split_spec
+    torch.manual_seed(0)
+    model = DecoderLM(vocab=300, max_seq=96, dim=128, n_layers=2, n_heads=2, ffn=256)
+    ids = torch.randint(0, 300, (4, 96))
+    pipe = pp.pipeline(model, 2, (ids,), split_spec=equal_split_spec(2, 2))
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    with pytest.raises(RuntimeError, match="multiples of 64"):
+        pp.ScheduleGPipe(stages, 2).step(ids.to(DEV))
+    eager = [pp.PipelineStage(pipe, i, DEV, force_eager=True) for i in range(2)]
+    out = pp.ScheduleGPipe(eager, 2).step(ids.to(DEV))
+    assert_close_rel(out, copy.deepcopy(model).float()(ids.to(DEV)), BF16_TOL, "eager logits")
