@@ -467,7 +467,8 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
 def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None) -> N.Op:
     if qkv.shape[1] % 64:
         raise RuntimeError(f"the attention kernels take sequence lengths that are multiples of 64, got "
-                           f"{qkv.shape[1]} (pad the sequences, or build the stage with force_eager=True)")
+                           f"{qkv.shape[1]} (causal layers pad by themselves; for attention without a mask pad "
+                           "the sequences, or build the stage with force_eager=True)")
     d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads)
     op = N.Op()
     op.kind = kind
@@ -526,6 +527,18 @@ def op_accum(acc, g, init=False) -> N.Op:
     op.p[0], op.p[1] = acc.data_ptr(), g.data_ptr()
     op.i[0] = acc.numel()
     op.j[0] = int(init)
+    return op
+
+
+def op_copy_rows(src, dst, n_rows, row_bytes, src_stride, dst_stride) -> N.Op:
+    """``n_rows`` runs of ``row_bytes`` bytes from ``src`` to ``dst`` with byte strides between runs."""
+    assert src_stride >= row_bytes and dst_stride >= row_bytes
+    assert (n_rows - 1) * src_stride + row_bytes <= src.numel() * src.element_size()
+    assert (n_rows - 1) * dst_stride + row_bytes <= dst.numel() * dst.element_size()
+    op = N.Op()
+    op.kind = N.OP_COPY_ROWS
+    op.p[0], op.p[1] = src.data_ptr(), dst.data_ptr()
+    op.i[0], op.i[1], op.i[2], op.i[3] = n_rows, row_bytes, src_stride, dst_stride
     return op
 
 
@@ -764,6 +777,7 @@ class StageProgram:
         self.arena = ParamArena(module, device, self.blocks)
         self.act_dtype = self.arena.dtype
         self._shared: Dict[str, torch.Tensor] = {}
+        self.zeroed_once = set()   # addresses of shared buffers whose padding a block cleared when it was built
         self.mbs: Dict[int, MicrobatchProgram] = {}
         self.acc_initialized = False  # False: the next W pass overwrites the accumulators
         # True once ``materialize_grads`` has set ``param.grad`` from the accumulators: a ``.grad`` that

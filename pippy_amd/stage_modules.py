@@ -135,6 +135,59 @@ def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor
     return dx
 
 
+def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, causal: bool,
+                    n_kv_heads: Optional[int] = None):
+    """Emits attention over the q|k|v rows ``qkv`` [Bn * S, W].  Returns the output [Bn * S, H * D] and the
+    emitter of the backward, ``d_att -> dqkv`` ([Bn * S, W]).
+
+    The kernels take sequence lengths that are multiples of 64.  Causal attention over any other length
+    runs on copies padded to the next multiple: a key past the end is never seen by a real query, a
+    query past the end receives no output gradient, so with zero rows in the padding (the value rows
+    must be finite) the real rows come out exactly as without padding, forward and backward."""
+    T, W = qkv.shape
+    Hkv = H if n_kv_heads is None else n_kv_heads
+    D = W // (H + 2 * Hkv)
+    Cc = H * D
+    att = b.act("att", (T, Cc))
+    if S % 64 == 0 or not causal:
+        lse = b.act("lse", (Bn, H, S), torch.float32)
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal, n_kv_heads=Hkv))
+
+        def backward(d_att):
+            dqkv = b.grad("dqkv", (T, W))
+            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
+            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal,
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv))
+            return dqkv
+
+        return att, backward
+    Sp = (S + 63) // 64 * 64
+    es = qkv.element_size()
+    qkv_p = b.act("qkv_padded", (Bn, Sp, W))
+    att_p = b.act("att_padded", (Bn, Sp, Cc))
+    lse = b.act("lse", (Bn, H, Sp), torch.float32)
+    qkv_p.zero_()       # once: the launch lists only ever write the real rows
+    b.f(P.op_copy_rows(qkv, qkv_p, Bn, S * W * es, S * W * es, Sp * W * es))
+    b.f(P.op_attn(N.OP_ATTN_FWD, qkv_p, att_p, lse, H, True, n_kv_heads=Hkv))
+    b.f(P.op_copy_rows(att_p, att, Bn, S * Cc * es, Sp * Cc * es, S * Cc * es))
+
+    def backward(d_att):
+        d_att_p = b.grad("d_att_padded", (Bn, Sp, Cc))
+        dqkv_p = b.grad("dqkv_padded", (Bn, Sp, W))
+        dqkv = b.grad("dqkv", (T, W))
+        delta = b.scratch("attn_delta", (Bn, H, Sp), torch.float32)
+        if d_att_p.data_ptr() not in b.sp.zeroed_once:      # (shared by the microbatches of a stage)
+            d_att_p.zero_()
+            b.sp.zeroed_once.add(d_att_p.data_ptr())
+        b.i(P.op_copy_rows(d_att, d_att_p, Bn, S * Cc * es, S * Cc * es, Sp * Cc * es))
+        b.i(P.op_attn(N.OP_ATTN_BWD, qkv_p, att_p, lse, H, True, d_o=d_att_p, dqkv=dqkv_p, delta=delta,
+                      n_kv_heads=Hkv))
+        b.i(P.op_copy_rows(dqkv_p, dqkv, Bn, S * W * es, Sp * W * es, S * W * es))
+        return dqkv
+
+    return att, backward
+
+
 def lower_layernorm(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d: torch.Tensor):
     T, Cc = x2d.shape
     y = b.act(name, (T, Cc))
@@ -442,9 +495,7 @@ class TransformerLayer(NativeBlock):
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         ln1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, x2d)
         qkv = self._lower_qkv(b, ln1)
-        att = b.act("att", (T, Cc))
-        lse = b.act("lse", (Bn, H, S), torch.float32)
-        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
         x2, _ = lower_linear(b, "x2", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         ln2, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, x2)
         h, h_pre = lower_linear(b, "h", self.mlp.c_fc, ln2, epilogue=act, save_pre=b.training)
@@ -458,10 +509,7 @@ class TransformerLayer(NativeBlock):
             d_x2 = layernorm_backward(b, "ln2", self.ln_2, x2, mean2, rstd2, d_ln2, dres=dy2d)
             # attention
             d_att = linear_backward(b, "attn_proj", self.attn.c_proj, att, d_x2)
-            dqkv = b.grad("dqkv", (T, 3 * Cc))
-            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
-            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
-                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            dqkv = attention_backward(d_att)
             d_ln1 = self._qkv_backward(b, ln1, dqkv)
             dx = layernorm_backward(b, "ln1", self.ln_1, x2d, mean1, rstd1, d_ln1, dres=d_x2,
                                     dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
@@ -476,9 +524,7 @@ class TransformerLayer(NativeBlock):
         x2d = x.view(T, Cc)
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         qkv = self._lower_qkv(b, x2d)
-        att = b.act("att", (T, Cc))
-        lse = b.act("lse", (Bn, H, S), torch.float32)
-        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal))
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
         a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         x1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, a)
         h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act, save_pre=b.training)
@@ -494,10 +540,7 @@ class TransformerLayer(NativeBlock):
                                    dx_aux=d_f)
             d_a = layernorm_backward(b, "ln1", self.ln_1, a, mean1, rstd1, d_x1)
             d_att = linear_backward(b, "attn_proj", self.attn.c_proj, att, d_a)
-            dqkv = b.grad("dqkv", (T, 3 * Cc))
-            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
-            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, 3 * Cc), att.view(Bn, S, Cc), lse, H, self.causal,
-                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, 3 * Cc), delta=delta))
+            dqkv = attention_backward(d_att)
             dx = self._qkv_backward(b, x2d, dqkv, dx_epilogue=N.EPI_BIAS_RESIDUAL, dx_aux=d_a,
                                     dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
             return dx.view(Bn, S, Cc)
@@ -647,19 +690,14 @@ class LlamaLayer(NativeBlock):
         n1, rstd1 = lower_rmsnorm(b, "n1", self.input_layernorm, x2d)
         qkv = self._lower_qkv(b, n1)
         b.f(P.op_rope(qkv, cos, sin, S, H + Hkv, D))
-        att = b.act("att", (T, Cc))
-        lse = b.act("lse", (Bn, H, S), torch.float32)
-        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, True, n_kv_heads=Hkv))
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, True, n_kv_heads=Hkv)
         x2, _ = lower_linear(b, "x2", self.self_attn.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         y, ffn_backward = self._lower_feed_forward(b, x2)
 
         def bwd(dy, need_dx, dx_out):
             d_x2 = ffn_backward(dy.view(T, Cc))
             d_att = linear_backward(b, "o", self.self_attn.o_proj, att, d_x2)
-            dqkv = b.grad("dqkv", (T, W))
-            delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
-            b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, True,
-                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv))
+            dqkv = attention_backward(d_att)
             # gradients w.r.t. the rotated q and k go back through the transposed rotation
             b.i(P.op_rope(dqkv, cos, sin, S, H + Hkv, D, inverse=True))
             d_n1 = self._qkv_backward(b, n1, dqkv)

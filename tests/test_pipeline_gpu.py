@@ -1326,13 +1326,46 @@ def test_float32_transformer_stages_fall_back_to_autograd_and_say_so():
         torch.testing.assert_close(p.grad.cpu(), rp.grad, rtol=1e-3, atol=1e-5, msg=lambda m: f"{name}: {m}")
 
 
-def test_a_sequence_length_the_attention_kernels_do_not_take_is_refused_before_any_launch():
-    """A traced stage is shape-generic, so an unsupported sequence length shows when the launch lists are
-    built: the error names the limit and the way out, and ``force_eager=True`` runs the same pipe."""
+@pytest.mark.parametrize("seq", [96, 100, 40])
+def test_causal_layers_pad_any_sequence_length_and_match_the_oracle(seq):
+    """The attention kernels take sequence lengths that are multiples of 64; causal layers run any other
+    length on zero-padded copies (a key past the end is never seen, a query past the end has no output
+    gradient), which must leave logits, losses and gradients those of the oracle."""
     import pippy_amd as pp
-    from pippy_amd.configs import DecoderLM, equal_split_spec
+    M = 2
+    model, ref, stages, ref_stages, ids = _build_decoder(2, n_layers=2, M=M, seq=seq)
+    _check_against_oracle(model, ref, stages, ref_stages, ids, pp.Schedule1F1B, M)
+
+
+def test_llama_layers_pad_any_sequence_length_and_match_the_oracle():
+    import pippy_amd as pp
+    from pippy_amd.configs import LlamaStage
     torch.manual_seed(0)
-    model = DecoderLM(vocab=300, max_seq=96, dim=128, n_layers=2, n_heads=2, ffn=256)
+    M, seq, dim = 2, 72, 256
+    model = LlamaStage(n_layers=2, dim=dim, n_heads=4, ffn=512, n_kv_heads=2)
+    ref = _fp32_cpu_copy(model)
+    x = (torch.randn(2 * M, seq, dim) * 0.5).to(torch.bfloat16)
+    upstream = torch.randn(2 * M, seq, dim) * 1e-2
+    stage = pp.ManualPipelineStage(model, 0, 1, DEV, M, input_args=(x[:2],))
+    loss_fn = lambda out, up: (out.float() * up).sum()
+    sched = pp.ScheduleZeroBubble([stage], M, loss_fn=loss_fn)
+    losses = []
+    out = sched.step(x.to(DEV), target=upstream.to(DEV), losses=losses)
+    ref_out, ref_losses = OP.step([ref], x.float(), upstream, M, loss_fn)
+    assert_close_rel(out, ref_out, BF16_TOL, "output")
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        err = max_rel(named[name].main_grad, rp.grad)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+
+
+def test_unmasked_attention_over_an_odd_sequence_length_is_refused_before_any_launch():
+    """Without a causal mask padding would be attended to: the limit shows when the launch lists of a
+    (shape-generic) traced stage are built; the error names it and the way out."""
+    import pippy_amd as pp
+    from pippy_amd.configs import EncoderModel, equal_split_spec
+    torch.manual_seed(0)
+    model = EncoderModel(vocab=300, max_seq=96, dim=128, n_layers=2, n_heads=2, ffn=256)
     ids = torch.randint(0, 300, (4, 96))
     pipe = pp.pipeline(model, 2, (ids,), split_spec=equal_split_spec(2, 2))
     stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
@@ -1340,4 +1373,4 @@ def test_a_sequence_length_the_attention_kernels_do_not_take_is_refused_before_a
         pp.ScheduleGPipe(stages, 2).step(ids.to(DEV))
     eager = [pp.PipelineStage(pipe, i, DEV, force_eager=True) for i in range(2)]
     out = pp.ScheduleGPipe(eager, 2).step(ids.to(DEV))
-    assert_close_rel(out, copy.deepcopy(model).float()(ids.to(DEV)), BF16_TOL, "eager logits")
+    assert_close_rel(out, copy.deepcopy(model).float()(ids.to(DEV)), BF16_TOL, "eager output")
