@@ -337,7 +337,10 @@ int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean, co
  * q, k, v: bf16, element (b, s, h, d) at base + b*stride_b + s*stride_s + h*head_dim + d, so the
  * three can alias one fused [B, S, 3*H*D] projection output.  o: bf16 [B, S, H*D] contiguous.
  * lse: fp32 [B, H, S] (log-sum-exp of the scaled scores; saved for backward).
- * head_dim in {64, 128}; S % 64 == 0.
+ * head_dim in {64, 128}; S % 64 == 0.  A shorter sequence is handed over padded to such an S with zero
+ * rows: kv_len = L makes the forward leave keys L .. S-1 out of the softmax (a causal mask does that
+ * for the real queries by itself).  The backward needs no mask: with zero key and value rows in the
+ * padding and zero d_o rows for the padded queries, the real rows of dq, dk, dv are exact.
  * Grouped-query attention: kv_group = G > 1 query heads share one key / value head, k and v (and dk,
  * dv) then hold H / G heads, query head h reads key / value head h / G, and dk, dv are sums over the
  * group (formed inside one work-group, in ascending query-head order); 0 or 1: one per query head.
@@ -353,7 +356,7 @@ typedef struct pp_attn_desc {
     float scale;           /* usually 1/sqrt(D) */
     int32_t causal;
     int32_t kv_group;      /* query heads per key / value head; 0 or 1: multi-head attention */
-    int32_t reserved;
+    int32_t kv_len;        /* 0: every key exists; L in 1..S: keys L..S-1 of each sequence are padding */
 } pp_attn_desc;
 int pp_attn_fwd(const pp_attn_desc* desc, pp_stream stream);
 int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
@@ -412,7 +415,7 @@ enum pp_op_kind {
  *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
- *                 | j: causal kv_group
+ *                 | j: causal kv_group kv_len
  *   EMBED_FWD     p: ids wte wpe y extra_row | i: n_tok seq C vocab
  *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab | j: round_bf16
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype

@@ -658,22 +658,13 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
 def _check_kernel_requirements(submod: nn.Module, blocks: List[NativeBlock]) -> None:
     """What the kernels need beyond a recognised structure.  Launch lists compute in the parameter
     dtype: the MFMA kernels (GEMM epilogues beyond bias / ReLU, attention, norms, embeddings) are bf16,
-    float32 stages can only be chains of ``nn.Linear`` with no activation or ReLU.  The attention
-    kernels take sequence lengths that are multiples of 64 (causal layers pad to one by themselves)."""
+    float32 stages can only be chains of ``nn.Linear`` with no activation or ReLU."""
     dtypes = {p.dtype for p in submod.parameters()}
     if len(dtypes) > 1:
         raise NotLowerable(f"parameters of several dtypes ({sorted(str(d) for d in dtypes)}); a launch-list stage "
                            "keeps one")
     if dtypes and dtypes != {torch.bfloat16} and dtypes != {torch.float32}:
         raise NotLowerable(f"parameters of dtype {dtypes.pop()} (bfloat16 and float32 are built)")
-    # an exported stage runs at the shapes of its example microbatch: what the kernels cannot take is known now
-    if isinstance(submod, fx.GraphModule) and any(isinstance(b, WrappedTransformerLayer) and not b.causal
-                                                   for b in blocks):
-        inputs = [n for n in submod.graph.nodes if n.op == "placeholder"]
-        shape = getattr(inputs[0].meta.get("val"), "shape", None) if len(inputs) == 1 else None
-        if shape is not None and len(shape) >= 2 and int(shape[1]) % 64:
-            raise NotLowerable(f"sequence length {int(shape[1])} without a causal mask (the attention kernels take "
-                               "multiples of 64; causal layers pad by themselves)")
     for blk in blocks if dtypes == {torch.float32} else ():
         plain = isinstance(blk, LinearAct) and isinstance(blk.lin, nn.Linear) and blk.activation in (None, "relu")
         if not plain:

@@ -464,12 +464,12 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
     return op
 
 
-def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None) -> N.Op:
+def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None, kv_len=None) -> N.Op:
     if qkv.shape[1] % 64:
         raise RuntimeError(f"the attention kernels take sequence lengths that are multiples of 64, got "
-                           f"{qkv.shape[1]} (causal layers pad by themselves; for attention without a mask pad "
-                           "the sequences, or build the stage with force_eager=True)")
-    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads)
+                           f"{qkv.shape[1]} (stage_modules.lower_attention pads)")
+    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
+                    kv_len=kv_len)
     op = N.Op()
     op.kind = kind
     for k, v in enumerate((d.q, d.k, d.v, d.o, d.lse, d.d_o, d.dq, d.dk, d.dv, d.delta)):
@@ -478,6 +478,7 @@ def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_
     op.f[0] = d.scale
     op.j[0] = d.causal
     op.j[1] = d.kv_group
+    op.j[2] = d.kv_len
     return op
 
 

@@ -37,6 +37,7 @@ struct AttnArgs {
     float* delta;
     int64_t B, S, H, D, stride_b, stride_s;
     int64_t G;  // query heads per key / value head (1: multi-head attention)
+    int64_t L;  // keys 0 .. L-1 of a sequence exist (L <= S); the forward masks the rest
     float scale;
 };
 
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
     AttnTileLoader<DS> lk, lv;
     lk.init(a.k + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, lwave, lane);
     lv.init(a.v + b * a.stride_b + (h / a.G) * D, a.stride_s, a.S, lwave, lane);
-    const int64_t n_keys = CAUSAL ? q0 + 64 : a.S;
+    const int64_t n_keys = CAUSAL ? q0 + 64 : a.L;
     const int64_t n_blocks = (n_keys + KB - 1) / KB;
     // LDS layout of an operand: [64-key tile of the block][64 columns of d] tiles of 64 x 64
     auto issue = [&](int stage, int64_t j) {
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
         const uint16_t* Ks = lds + stage * kStage + ktile * DS * kTile;
         const uint16_t* Vs = Ks + kOperand;
         // keys past the sequence (a last block of 128 that is half full) or past every query of the wave
-        const bool active = kt0 < a.S && (!CAUSAL || (kt0 <= qw0 + 31));
+        const bool active = kt0 < a.L && (!CAUSAL || (kt0 <= qw0 + 31));
         if (active) {
             bf16x8_t kf[KS];
 #pragma unroll
@@ -266,6 +267,12 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
             // sacc[v]: kv = kt0 + 8 (v/4) + 4 lh + v%4, q = qi
             if (CAUSAL && (kt0 + 31 > qw0)) {  // wave-uniform: only blocks on the diagonal pay for the mask
                 const int lim = (int)(qi - kt0) - 4 * lh;  // keys 8 (v/4) + v%4 up to lim are visible
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (8 * (v >> 2) + (v & 3) > lim) sacc[v] = -INFINITY;
+            }
+            if (kt0 + 31 >= a.L) {  // wave-uniform: the block that holds the end of a padded sequence
+                const int lim = (int)(a.L - 1 - kt0) - 4 * lh;
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
                     if (8 * (v >> 2) + (v & 3) > lim) sacc[v] = -INFINITY;
@@ -699,6 +706,8 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
     if (d->D != 64 && d->D != 128)
         return fail(PP_ERR_UNSUPPORTED, "%s: head_dim %lld (64 and 128 are built)", who, (long long)d->D);
     if (d->S % 64) return fail(PP_ERR_UNSUPPORTED, "%s: S %% 64 != 0 (S=%lld)", who, (long long)d->S);
+    if (d->kv_len < 0 || d->kv_len > d->S)
+        return fail(PP_ERR_INVALID, "%s: kv_len %d outside [0, S = %lld]", who, d->kv_len, (long long)d->S);
     if (d->kv_group < 0 || (d->kv_group > 1 && d->H % d->kv_group))
         return fail(PP_ERR_INVALID, "%s: kv_group %d does not divide H = %lld", who, d->kv_group, (long long)d->H);
     if ((d->stride_s % 8) || (d->stride_b % 8)) return fail(PP_ERR_INVALID, "%s: strides must be multiples of 8", who);
@@ -725,6 +734,7 @@ static AttnArgs to_args(const pp_attn_desc* d) {
     a.B = d->B; a.S = d->S; a.H = d->H; a.D = d->D;
     a.stride_b = d->stride_b; a.stride_s = d->stride_s;
     a.G = d->kv_group > 1 ? d->kv_group : 1;
+    a.L = d->kv_len > 0 ? d->kv_len : d->S;
     a.scale = d->scale;
     return a;
 }

@@ -140,16 +140,17 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
     """Emits attention over the q|k|v rows ``qkv`` [Bn * S, W].  Returns the output [Bn * S, H * D] and the
     emitter of the backward, ``d_att -> dqkv`` ([Bn * S, W]).
 
-    The kernels take sequence lengths that are multiples of 64.  Causal attention over any other length
-    runs on copies padded to the next multiple: a key past the end is never seen by a real query, a
-    query past the end receives no output gradient, so with zero rows in the padding (the value rows
-    must be finite) the real rows come out exactly as without padding, forward and backward."""
+    The kernels take sequence lengths that are multiples of 64.  Any other length runs on copies padded
+    to the next multiple with zero rows: the forward leaves the keys past the end out of the softmax
+    (``kv_len``; under a causal mask no real query sees them anyway), and in the backward a query past
+    the end has no output gradient while a key past the end has zero key and value rows, so the real
+    rows come out exactly as without padding, forward and backward."""
     T, W = qkv.shape
     Hkv = H if n_kv_heads is None else n_kv_heads
     D = W // (H + 2 * Hkv)
     Cc = H * D
     att = b.act("att", (T, Cc))
-    if S % 64 == 0 or not causal:
+    if S % 64 == 0:
         lse = b.act("lse", (Bn, H, S), torch.float32)
         b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal, n_kv_heads=Hkv))
 
@@ -168,7 +169,7 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
     lse = b.act("lse", (Bn, H, Sp), torch.float32)
     qkv_p.zero_()       # once: the launch lists only ever write the real rows
     b.f(P.op_copy_rows(qkv, qkv_p, Bn, S * W * es, S * W * es, Sp * W * es))
-    b.f(P.op_attn(N.OP_ATTN_FWD, qkv_p, att_p, lse, H, True, n_kv_heads=Hkv))
+    b.f(P.op_attn(N.OP_ATTN_FWD, qkv_p, att_p, lse, H, causal, n_kv_heads=Hkv, kv_len=S))
     b.f(P.op_copy_rows(att_p, att, Bn, S * Cc * es, Sp * Cc * es, S * Cc * es))
 
     def backward(d_att):
@@ -180,8 +181,8 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
             d_att_p.zero_()
             b.sp.zeroed_once.add(d_att_p.data_ptr())
         b.i(P.op_copy_rows(d_att, d_att_p, Bn, S * Cc * es, S * Cc * es, Sp * Cc * es))
-        b.i(P.op_attn(N.OP_ATTN_BWD, qkv_p, att_p, lse, H, True, d_o=d_att_p, dqkv=dqkv_p, delta=delta,
-                      n_kv_heads=Hkv))
+        b.i(P.op_attn(N.OP_ATTN_BWD, qkv_p, att_p, lse, H, causal, d_o=d_att_p, dqkv=dqkv_p, delta=delta,
+                      n_kv_heads=Hkv, kv_len=S))
         b.i(P.op_copy_rows(dqkv_p, dqkv, Bn, S * W * es, Sp * W * es, S * W * es))
         return dqkv
 

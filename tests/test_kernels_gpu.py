@@ -564,6 +564,46 @@ def test_attention(causal, B, S, H, D):
 
 
 @pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,L,H,Hkv,D", [(2, 100, 2, 2, 64), (1, 40, 3, 3, 64), (2, 193, 2, 1, 128), (1, 330, 4, 2, 64),
+                                         (3, 1, 1, 1, 64), (1, 449, 3, 3, 64), (1, 64, 2, 2, 64)])
+def test_attention_over_a_padded_sequence_is_attention_over_the_sequence(causal, B, L, H, Hkv, D):
+    """A sequence of L tokens handed over in S = the next multiple of 64 rows, the padding rows zero and
+    kv_len = L: the first L rows of the output, of the log-sum-exp and (with zero d_o rows in the padding)
+    of dq, dk, dv are those of attention over the L tokens."""
+    Nn = native()
+    torch.manual_seed(7 * L + H)
+    S = (L + 63) // 64 * 64
+    W = (H + 2 * Hkv) * D
+    real = torch.randn(B, L, W).to(torch.bfloat16)
+    qkv = torch.zeros(B, S, W, dtype=torch.bfloat16)
+    qkv[:, :L] = real
+    qkv = qkv.to(DEV)
+    o = torch.full((B, S, H * D), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    note(f"padded attention B={B} L={L} S={S} H={H} Hkv={Hkv} D={D} causal={causal}")
+    Nn.attn_fwd(qkv, o, lse, H, causal, n_kv_heads=Hkv, kv_len=L)
+    torch.cuda.synchronize()
+    qr = real.float().requires_grad_(True)
+    ref = O.attention_fused_qkv(qr, H, causal, n_kv_heads=Hkv)
+    assert_close_rel(o[:, :L], ref, BF16_TOL, "padded attention fwd")
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    d_real = torch.randn(B, L, H * D).to(torch.bfloat16)
+    d_o = torch.zeros(B, S, H * D, dtype=torch.bfloat16)
+    d_o[:, :L] = d_real
+    d_o = d_o.to(DEV)
+    dqkv = torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, n_kv_heads=Hkv, kv_len=L)
+    torch.cuda.synchronize()
+    ref.backward(d_real.float())
+    HD, KD = H * D, Hkv * D
+    for name, sl in (("dq", slice(0, HD)), ("dk", slice(HD, HD + KD)), ("dv", slice(HD + KD, HD + 2 * KD))):
+        assert_close_rel(dqkv[:, :L, sl], qr.grad[..., sl], BF16_TOL, f"padded attention {name}")
+    # the padded queries receive no gradient (their d_o rows are zero)
+    assert float(dqkv[:, L:, :HD].float().abs().max()) == 0.0 if L < S else True
+
+
+@pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,S,H,Hkv,D", [(2, 256, 4, 2, 64), (1, 192, 8, 2, 128), (1, 1024, 8, 1, 64),
                                          (2, 128, 6, 3, 64), (1, 64, 16, 8, 64)])
 def test_grouped_query_attention(causal, B, S, H, Hkv, D):
