@@ -143,7 +143,8 @@ typedef struct pp_gemm_desc {
     int32_t reserved;
 } pp_gemm_desc;
 
-/* Requirements: A, B 16-byte aligned; K % 8 == 0; lda, ldb % 8 == 0; a transposed operand needs
+/* Requirements: A, B 16-byte aligned; K % 8 == 0 unless both operands are transposed (then any K: the
+ * weight gradient over any number of tokens); lda, ldb % 8 == 0; a transposed operand needs
  * its contiguous extent (M resp. N) % 8 == 0; ldc, ld_aux % 4 == 0 (bf16) . */
 int pp_gemm_bf16(const pp_gemm_desc* desc, pp_stream stream);
 

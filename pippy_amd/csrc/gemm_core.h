@@ -519,9 +519,11 @@ static inline int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
     if (!d->A || !d->B || !d->C) return fail(PP_ERR_INVALID, "pp_gemm_bf16: null operand");
     if (!aligned(d->A, 16) || !aligned(d->B, 16))
         return fail(PP_ERR_INVALID, "pp_gemm_bf16: A and B must be 16-byte aligned");
-    if ((d->K & 7) || (d->lda & 7) || (d->ldb & 7))
-        return fail(PP_ERR_INVALID, "pp_gemm_bf16: K, lda, ldb must be multiples of 8 (K=%lld lda=%lld ldb=%lld)",
-                    (long long)d->K, (long long)d->lda, (long long)d->ldb);
+    // a k-contiguous operand is read in 16-byte chunks along k; a transposed one row of k by row, any K
+    // (rows past K fail the range check of the buffer loads and read as zero)
+    if ((d->lda & 7) || (d->ldb & 7) || ((d->K & 7) && !(d->a_trans && d->b_trans)))
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: lda, ldb (and K, unless both operands are transposed) must be "
+                    "multiples of 8 (K=%lld lda=%lld ldb=%lld)", (long long)d->K, (long long)d->lda, (long long)d->ldb);
     if (d->a_trans && (d->M & 7)) return fail(PP_ERR_INVALID, "pp_gemm_bf16: transposed A needs M %% 8 == 0");
     if (d->b_trans && (d->N & 7)) return fail(PP_ERR_INVALID, "pp_gemm_bf16: transposed B needs N %% 8 == 0");
     if (d->lda < (d->a_trans ? d->M : d->K) || d->ldb < (d->b_trans ? d->N : d->K) || d->ldc < d->N)

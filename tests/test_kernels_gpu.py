@@ -259,6 +259,30 @@ def test_gemm_bf16_rounded_accumulate_is_bit_exact(M, N, K, at, bt):
         Nn.gemm_bf16(A, B, bad, a_trans=at, b_trans=bt, epilogue=Nn.EPI_ACCUM_ROUNDED)
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 256, 100), (72, 136, 36), (768, 3072, 1001), (64, 64, 7), (256, 128, 65)])
+def test_gemm_bf16_transposed_operands_take_any_reduction_length(M, N, K):
+    """dW = dY^T X over a number of tokens that is not a multiple of 8 (both operands transposed: k is
+    the row index of both, rows past K read as zero), alone, into an accumulator, and in a grouped launch."""
+    Nn = native()
+    torch.manual_seed(K)
+    A = torch.randn(K, M, device=DEV).to(torch.bfloat16)
+    B = torch.randn(K, N, device=DEV).to(torch.bfloat16)
+    C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    note(f"gemm TT {M}x{N}x{K}")
+    Nn.gemm_bf16(A, B, C, a_trans=True, b_trans=True)
+    torch.cuda.synchronize()
+    ref = A.float().cpu().t() @ B.float().cpu()
+    assert_close_rel(C, ref, BF16_TOL, "TT gemm, odd K")
+    acc, acc2 = torch.ones(M, N, device=DEV), torch.zeros(M, N, device=DEV)
+    kw = dict(a_trans=True, b_trans=True, epilogue=Nn.EPI_ACCUM_F32, beta=1)
+    Nn.gemm_bf16_grouped([(A, B, acc, kw), (A, B, acc2, kw)])
+    torch.cuda.synchronize()
+    assert torch.equal(acc2.to(torch.bfloat16), C)
+    assert_close_rel(acc - 1.0, ref, BF16_TOL, "TT gemm into an accumulator, odd K")
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        Nn.gemm_bf16(A.t().contiguous(), B, torch.empty(M, N, device=DEV, dtype=torch.bfloat16), b_trans=True)
+
+
 def test_gemm_bf16_rejects_bad_arguments():
     Nn = native()
     A = torch.zeros(16, 12, device=DEV, dtype=torch.bfloat16)
