@@ -321,7 +321,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     """What a residual branch is, from the layers between the stream and the addition:
     ("attn", ln, qkv, proj, causal) / ("mlp", ln, fc1, fc2, activation) for the GPT-2 and BERT families
     (ln is None when the branch does not start with a LayerNorm; qkv is one fused layer or three),
-    ("attn_rope", norm, q, k, v, o) / ("mlp_gated", norm, gate, up, down) for the Llama family."""
+    ("attn_rope", norm, qkv, o) / ("mlp_gated", norm, gate_up, down) for the Llama family (qkv: the
+    fused projection or the three separate ones; gate_up: the fused projection or the two separate ones)."""
     mods, inner_adds = [], []
     for n in layers:
         if _activation_of(n, root) == "identity":
@@ -353,7 +354,15 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             raise NotLowerable("query / key / value projections of unexpected widths")
         if not _sdpa_is_causal(root, sd):
             raise NotLowerable("rotary attention that is not causal")
-        return ("attn_rope", norm, q, k, v, o)
+        return ("attn_rope", norm, (q, k, v), o)
+    if kinds == ["RMSNorm", "Linear", "sdpa", "Linear"] and inner_adds:
+        (_, norm), (_, qkv), (sd, _), (_, o) = mods       # one fused q|k|v projection under a rotary embedding
+        if not all(isinstance(lin, nn.Linear) for lin in (qkv, o)) or o.in_features != o.out_features \
+                or qkv.out_features <= o.in_features or (qkv.out_features - o.in_features) % 2:
+            raise NotLowerable("a fused projection in front of rotary attention that is not q|k|v")
+        if not _sdpa_is_causal(root, sd):
+            raise NotLowerable("rotary attention that is not causal")
+        return ("attn_rope", norm, qkv, o)
     if kinds == ["RMSNorm", "Linear", "act", "Linear", "Linear"] or kinds == ["RMSNorm", "Linear", "Linear", "act", "Linear"]:
         norm, down = mods[0][1], mods[-1][1]
         an = next(n for n, m in mods if kind(n, m) == "act")
@@ -368,7 +377,14 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         if any(lin.bias is not None or not isinstance(lin, nn.Linear) for lin in (gate, up, down)) or \
                 gate.out_features != up.out_features or down.in_features != gate.out_features:
             raise NotLowerable("gated feed-forward projections with biases, [in, out] weights or unexpected widths")
-        return ("mlp_gated", norm, gate, up, down)
+        return ("mlp_gated", norm, (gate, up), down)
+    if kinds == ["RMSNorm", "Linear", "act", "Linear"] and not inner_adds and \
+            _activation_of(mods[2][0], root) == "silu":
+        (_, norm), (_, packed), _, (_, down) = mods         # gate | up in one projection
+        if not all(isinstance(lin, nn.Linear) and lin.bias is None for lin in (packed, down)) or \
+                packed.out_features != 2 * down.in_features:
+            raise NotLowerable("a SiLU feed-forward that is not down(silu(gate) * up) over a fused gate|up projection")
+        return ("mlp_gated", norm, packed, down)
     if inner_adds:
         raise NotLowerable(f"an addition inside a residual branch ('{inner_adds[0].format_node()}')")
     ln = None
@@ -485,7 +501,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
                 raise NotLowerable("a feed-forward branch without an attention branch before it")
             if (pending[0], kind[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
                 raise NotLowerable(f"a '{pending[0]}' branch followed by a '{kind[0]}' branch")
-            d = pending[3].in_features if pending[0] == "attn" else pending[2].in_features
+            d = pending[3].in_features
             if d % n_heads or d // n_heads not in (64, 128):
                 raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
             if kind[0] == "mlp":
@@ -500,14 +516,16 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
                 else:
                     blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
             else:
-                _, norm1, q, k, v, o = pending
-                _, norm2, gate, up, down = kind
-                if k.out_features % (d // n_heads):
-                    raise NotLowerable("key / value projections that are not whole heads")
+                _, norm1, qkv, o = pending
+                _, norm2, gate_up, down = kind
+                width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
+                D = d // n_heads
+                if width % D or (width // D - n_heads) % 2 or width // D <= n_heads:
+                    raise NotLowerable("query / key / value projections that are not whole heads")
                 if rope is None:
                     raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the "
                                        "positions (exported models do)")
-                blocks.append(WrappedLlamaLayer(norm1, q, k, v, o, norm2, gate, up, down, n_heads, *rope))
+                blocks.append(WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope))
             pending = None
         stream = after
         while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":

@@ -1167,31 +1167,44 @@ class WrappedTransformerLayer(TransformerLayer):
 
 
 class WrappedLlamaLayer(LlamaLayer):
-    """``LlamaLayer`` around the layers of a user's model, which keeps separate query, key and value
-    projections (the Hugging Face layout).  The three forward GEMMs write their column ranges of the
-    one q|k|v buffer the attention kernels read; the gradient of the normalised input is one product of
-    the q|k|v gradient with the three transposed weights side by side; each weight gradient reads its
-    column range of that gradient."""
+    """``LlamaLayer`` around the layers of a user's model.  ``qkv`` is the fused q|k|v projection or the
+    three separate ones (the Hugging Face Llama layout), ``gate_up`` the fused gate|up projection or
+    the two separate ones.  Separate projections run as one forward GEMM over the arena's row-stacked
+    copy of their weights; the gradient of their common input is one product with the transposed
+    weights side by side; each weight gradient reads its column range of the output gradient."""
 
-    def __init__(self, input_layernorm, q_proj, k_proj, v_proj, o_proj, post_attention_layernorm,
-                 gate_proj, up_proj, down_proj, n_heads: int, cos: torch.Tensor, sin: torch.Tensor):
+    def __init__(self, input_layernorm, qkv, o_proj, post_attention_layernorm, gate_up, down_proj,
+                 n_heads: int, cos: torch.Tensor, sin: torch.Tensor):
         """``cos`` / ``sin``: the model's own rotary tables, [positions, head_dim / 2] (whatever base,
         scaling or rounding the model applies is in them)."""
         NativeBlock.__init__(self)
-        self.dim, self.n_heads, self.ffn = o_proj.out_features, n_heads, gate_proj.out_features
+        self._qkv = tuple(qkv) if isinstance(qkv, (tuple, list)) else (qkv,)
+        self._gate_up = tuple(gate_up) if isinstance(gate_up, (tuple, list)) else (gate_up,)
+        self.dim, self.n_heads = o_proj.out_features, n_heads
+        self.ffn = down_proj.in_features
         D = self.dim // n_heads
         assert cos.shape == sin.shape and cos.shape[1] == D // 2
-        self.n_kv_heads = k_proj.out_features // D
+        width = sum(lin.out_features for lin in self._qkv)
+        self.n_kv_heads = (width // D - n_heads) // 2
+        assert self.n_kv_heads > 0 and (n_heads + 2 * self.n_kv_heads) * D == width
+        assert sum(lin.out_features for lin in self._gate_up) == 2 * self.ffn
         self.eps, self.rope_theta = input_layernorm.eps, None
         self._cos, self._sin = cos.detach().float().cpu().contiguous(), sin.detach().float().cpu().contiguous()
         import hashlib
         self._table_key = hashlib.sha1(self._cos.numpy().tobytes() + self._sin.numpy().tobytes()).hexdigest()[:16]
         self.input_layernorm, self.post_attention_layernorm = input_layernorm, post_attention_layernorm
         self.self_attn = nn.Module()
-        self.self_attn.q_proj, self.self_attn.k_proj, self.self_attn.v_proj = q_proj, k_proj, v_proj
+        if len(self._qkv) == 3:
+            self.self_attn.q_proj, self.self_attn.k_proj, self.self_attn.v_proj = self._qkv
+        else:
+            self.self_attn.qkv_proj = self._qkv[0]
         self.self_attn.o_proj = o_proj
         self.mlp = nn.Module()
-        self.mlp.gate_proj, self.mlp.up_proj, self.mlp.down_proj = gate_proj, up_proj, down_proj
+        if len(self._gate_up) == 2:
+            self.mlp.gate_proj, self.mlp.up_proj = self._gate_up
+        else:
+            self.mlp.gate_up_proj = self._gate_up[0]
+        self.mlp.down_proj = down_proj
 
     def _rope(self, seq, head_dim, device):
         if seq > self._cos.shape[0] or head_dim != 2 * self._cos.shape[1]:
@@ -1202,24 +1215,55 @@ class WrappedLlamaLayer(LlamaLayer):
     def _rope_key(self):
         return self._table_key
 
-    def _projections(self):
-        a = self.self_attn
-        return (a.q_proj, a.k_proj, a.v_proj)
-
     def _project_qkv(self, h):
-        return torch.cat([lin(h) for lin in self._projections()], dim=-1)
+        return torch.cat([lin(h) for lin in self._qkv], dim=-1)
 
     def _lower_qkv(self, b, n1):
-        return lower_stacked_linears(b, "qkv", self._projections(), n1)
+        if len(self._qkv) == 1:
+            return lower_linear(b, "qkv", self._qkv[0], n1)[0]
+        return lower_stacked_linears(b, "qkv", self._qkv, n1)
 
     def _qkv_backward(self, b, n1, dqkv):
+        if len(self._qkv) == 1:
+            return linear_backward(b, "qkv", self._qkv[0], n1, dqkv)
         d_n1 = b.grad("qkv.dx", (n1.shape[0], n1.shape[1]))
-        b.i(P.op_gemm(dqkv, b.weight_t_cat(*(lin.weight for lin in self._projections())), d_n1))
+        b.i(P.op_gemm(dqkv, b.weight_t_cat(*(lin.weight for lin in self._qkv)), d_n1))
         lo = 0
-        for name, lin in zip("qkv", self._projections()):
+        for name, lin in zip("qkv", self._qkv):
             linear_backward(b, name, lin, n1, dqkv[:, lo:lo + lin.out_features], need_dx=False)
             lo += lin.out_features
         return d_n1
+
+    def _feed_forward(self, h):
+        if len(self._gate_up) == 2:
+            return super()._feed_forward(h)
+        gate, up = self._gate_up[0](h).chunk(2, dim=-1)
+        return self.mlp.down_proj(F.silu(gate) * up)
+
+    def _lower_feed_forward(self, b, x2):
+        if len(self._gate_up) == 2:
+            return super()._lower_feed_forward(b, x2)
+        # one [2 f, d] weight whose first f rows are the gate: both halves of the product come out of the
+        # SwiGLU GEMM as they do for two weights, and the backward treats the pair as the one layer it is
+        T, ffn, packed, down = x2.shape[0], self.ffn, self._gate_up[0], self.mlp.down_proj
+        if x2.dtype != torch.bfloat16 or ffn % 8 or packed.bias is not None:
+            raise RuntimeError("a fused gate|up projection lowers in bf16, without a bias, with a width that is a "
+                               "multiple of 8")
+        n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
+        w = b.weight(packed.weight)
+        gu = b.act("gu", (T, 2 * ffn))
+        h = b.act("h", (T, ffn))
+        b.f(P.op_gemm_swiglu(n2, w[:ffn], w[ffn:], gu, h))
+        y, _ = lower_linear(b, "y", down, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
+
+        def backward(dy2d):
+            dgu = b.grad("dgu", (T, 2 * ffn))
+            b.i(P.op_gemm_dswiglu(dy2d, b.weight_t(down.weight), gu, dgu))
+            d_n2 = linear_backward(b, "gate_up", packed, n2, dgu)
+            linear_backward(b, "down", down, h, dy2d, need_dx=False)
+            return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
+
+        return y, backward
 
 
 class WrappedLMHead(LMHead):

@@ -1223,11 +1223,12 @@ def _qkv_group(name):
     return None
 
 
-@pytest.mark.parametrize("family", ["qwen2", "mistral", "distilbert", "electra"])
+@pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra"])
 def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
-    value projections), Mistral (Llama layout), DistilBERT (encoder without token types, its own layer
-    names), ELECTRA (BERT layout with a generator head)."""
+    value projections), Mistral (Llama layout), Phi-3 (one fused q|k|v and one fused gate|up projection),
+    DistilBERT (encoder without token types, its own layer names), ELECTRA (BERT layout with a generator
+    head)."""
     T = pytest.importorskip("transformers")
     import torch.nn as nn
     common = dict(vocab_size=1000, tie_word_embeddings=False)
@@ -1237,6 +1238,9 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
         "qwen2": lambda: (T.Qwen2ForCausalLM, T.Qwen2Config(**llama_like, **common), "model.layers.2"),
         "mistral": lambda: (T.MistralForCausalLM, T.MistralConfig(sliding_window=None, **llama_like, **common),
                             "model.layers.2"),
+        "phi3": lambda: (T.Phi3ForCausalLM,
+                         T.Phi3Config(**{**llama_like, "num_key_value_heads": 4}, resid_pdrop=0.0, embd_pdrop=0.0,
+                                      pad_token_id=0, **common), "model.layers.2"),
         "distilbert": lambda: (T.DistilBertForMaskedLM,
                                T.DistilBertConfig(dim=128, hidden_dim=512, n_layers=4, n_heads=2,
                                                   max_position_embeddings=128, dropout=0.0, attention_dropout=0.0,
