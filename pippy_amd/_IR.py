@@ -478,9 +478,13 @@ class Pipe(nn.Module):
             except ValueError:
                 raise
             except Exception as export_error:
+                hint = ""
+                if "Cache" in str(export_error) and getattr(getattr(mod, "config", None), "use_cache", False):
+                    hint = ("; the model returns a key / value cache object, which torch.export cannot flatten: "
+                            "build it with config.use_cache = False")
                 raise RuntimeError(
                     f"pipeline(): neither torch.fx symbolic tracing ({type(fx_error).__name__}: {fx_error}) "
-                    f"nor torch.export ({type(export_error).__name__}: {export_error}) can trace this model"
+                    f"nor torch.export ({type(export_error).__name__}: {export_error}) can trace this model{hint}"
                 ) from export_error
         if split_policy is not None:
             gm = split_policy(fx.GraphModule(root, graph))

@@ -259,12 +259,14 @@ class PipelineStageBase:
     def _input_for(self, mb: int, args, kwargs):
         """(x, dx_target, patch_input) of microbatch ``mb`` for a native stage."""
         if self.is_first:
-            if kwargs:
-                raise RuntimeError(f"{self.log_prefix} native stages take positional tensor inputs only")
-            tensors = [a for a in args if isinstance(a, torch.Tensor)]
-            if len(tensors) != 1 or len(args) != 1:
+            # the stage's graph has one input: it may arrive by position or by keyword
+            # (``schedule.step(input_ids=ids)``, reference ``examples/huggingface/pippy_gpt2.py:73-77``)
+            values = [a for a in list(args) + list(kwargs.values()) if a is not None]
+            tensors = [a for a in values if isinstance(a, torch.Tensor)]
+            if len(tensors) != 1 or len(values) != 1:
                 raise RuntimeError(
-                    f"{self.log_prefix} a native stage takes exactly one tensor input, got {len(args)} args")
+                    f"{self.log_prefix} a native stage takes exactly one tensor input, got {len(args)} positional "
+                    f"and {len(kwargs)} keyword values")
             x = tensors[0]
             if not x.is_cuda:
                 raise RuntimeError(f"{self.log_prefix} input is on {x.device}; move it to {self.device}")

@@ -1392,3 +1392,32 @@ def test_encoder_layers_pad_any_sequence_length_and_match_the_oracle(seq):
             continue
         err = max_rel(named[name].main_grad, rp.grad)
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+
+
+def test_the_flow_of_the_reference_gpt2_example():
+    """examples/huggingface/pippy_gpt2.py:20-77 with the package's names: GPT2ForSequenceClassification in
+    eval mode, the microbatch given by keyword (``mb_kwargs``), ``pipe.build_stage``, ``ScheduleGPipe`` and
+    ``schedule.step(**inputs)``.  The decoder stage runs as launch lists; the last stage, which picks the
+    last token's scores out of the sequence, runs through torch; the result is the model's."""
+    transformers = pytest.importorskip("transformers")
+    from pippy_amd import ScheduleGPipe, SplitPoint, pipeline
+    config = transformers.GPT2Config(n_embd=128, n_layer=4, n_head=2, n_positions=256, vocab_size=1000,
+                                     attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False)
+    torch.manual_seed(0)
+    gpt2 = transformers.GPT2ForSequenceClassification(config).to(torch.bfloat16)
+    gpt2.eval()
+    chunks, batch, seq, world = 4, 4, 256, 2
+    mb_inputs = {"input_ids": torch.randint(0, 1000, (batch // chunks, seq))}
+    split_spec = {f"transformer.h.{i * 2}": SplitPoint.BEGINNING for i in range(1, world)}
+    pipe = pipeline(gpt2, mb_args=(), mb_kwargs=mb_inputs, split_spec=split_spec)
+    assert pipe.num_stages == world
+    stages = [pipe.build_stage(r, device=DEV) for r in range(world)]
+    assert stages[0].is_native and not stages[1].is_native
+    schedule = ScheduleGPipe(stages, chunks)
+    inputs = {"input_ids": torch.randint(0, 1000, (batch, seq), device=DEV)}
+    with torch.no_grad():
+        out = schedule.step(**inputs)
+        ref = torch.cat([copy.deepcopy(gpt2).float()(input_ids=inputs["input_ids"][i:i + 1]).logits
+                         for i in range(batch)])
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    assert_close_rel(out, ref, BF16_TOL, "classification scores")
