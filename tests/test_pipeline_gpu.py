@@ -1421,3 +1421,54 @@ def test_the_flow_of_the_reference_gpt2_example():
                          for i in range(batch)])
     out = out[0] if isinstance(out, (tuple, list)) else out
     assert_close_rel(out, ref, BF16_TOL, "classification scores")
+
+
+def test_hugging_face_vit_runs_its_encoder_stage_natively_between_two_torch_stages():
+    """transformers.ViTForImageClassification in three stages: the patch embedding (a convolution, the class
+    token) and the classifier head (the class token's row) run through torch autograd, the stage of plain
+    encoder layers between them as launch lists over 65 tokens (attention without a mask, padded to 128
+    keys inside the layer).  Activations and gradients cross both kinds of boundary."""
+    transformers = pytest.importorskip("transformers")
+    import pippy_amd as pp
+    cfg = transformers.ViTConfig(hidden_size=128, num_hidden_layers=6, num_attention_heads=2, intermediate_size=512,
+                                 image_size=64, patch_size=8, hidden_dropout_prob=0.0,
+                                 attention_probs_dropout_prob=0.0, num_labels=10)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.ViTForImageClassification(cfg).to(torch.bfloat16)
+    ref = copy.deepcopy(model).float()
+    M, mb = 4, 2
+    images = torch.randn(mb * M, 3, 64, 64)
+    labels = torch.randint(0, 10, (mb * M,))
+    pipe = pp.pipeline(model, mb_args=(images[:mb].to(torch.bfloat16),),
+                       split_spec={"vit.layers.2": pp.SplitPoint.BEGINNING, "vit.layers.4": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(3)]
+    assert [st.is_native for st in stages] == [False, True, False], [st.eager_reason for st in stages]
+    loss_fn = lambda out, tgt: torch.nn.functional.cross_entropy((out[0] if isinstance(out, tuple) else out).float(), tgt)
+    sched = pp.Schedule1F1B(stages, M, loss_fn=loss_fn)
+    losses = []
+    out = sched.step(images.to(DEV, torch.bfloat16), target=labels.to(DEV), losses=losses)
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    ref_losses = []
+    for x, t in zip(images.chunk(M), labels.chunk(M)):
+        logits = ref(x).logits
+        ref_losses.append(torch.nn.functional.cross_entropy(logits, t))
+        ref_losses[-1].backward()
+    assert_close_rel(out, ref(images).logits.detach(), BF16_TOL, "class scores")
+    for m in range(M):
+        assert_close_rel(losses[m].reshape(1), ref_losses[m].detach().reshape(1), BF16_TOL, f"loss {m}")
+    stages[1].materialize_grads()
+    named = dict(model.named_parameters())
+    for name, rp in ref.named_parameters():
+        got = named[name].grad
+        assert got is not None, name
+        group = _qkv_group(name)
+        err = max_rel(got, rp.grad)
+        if group:
+            ref_named = dict(ref.named_parameters())
+            scale = max(ref_named[n].grad.abs().max().item() for n in group + [name])
+            assert (got.float().cpu() - rp.grad).abs().max().item() / scale <= BF16_TOL, name
+            if rp.grad.abs().max().item() > 1e-3 * scale:
+                assert err <= 3 * BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+        else:
+            assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
