@@ -11,7 +11,7 @@ like the reference does.
 from __future__ import annotations
 
 import operator
-from typing import List, Optional
+from typing import List, Optional, Tuple
 
 import torch
 import torch.fx as fx
@@ -412,69 +412,155 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     raise NotLowerable(f"a residual branch made of {kinds}")
 
 
+def _skip_identities(root: nn.Module, stream: fx.Node) -> fx.Node:
+    """Steps over layers that do nothing (a dropout with p = 0 or in eval mode) behind ``stream``."""
+    while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
+        stream = next(iter(stream.users))
+    return stream
+
+
+def _only_layer_user(root: nn.Module, node: fx.Node) -> Tuple[Optional[fx.Node], Optional[nn.Module]]:
+    """(user, its module) when ``node`` feeds exactly one layer call, else (None, None)."""
+    users = list(node.users)
+    if len(users) == 1 and users[0].op == "call_module":
+        return users[0], root.get_submodule(users[0].target)
+    return None, None
+
+
+def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream: fx.Node):
+    """The embedding block at the head of a stage, if it has one: a lone token table, token + position
+    tables (GPT-2), or word + position (+ token type 0) tables under a LayerNorm (the BERT family).
+    Returns (blocks, the node that carries the residual stream from there on)."""
+    emb = [n for n in nodes if n.op == "call_module" and isinstance(root.get_submodule(n.target), nn.Embedding)]
+    if not emb:
+        return [], stream
+    ids = emb[0].all_input_nodes[0] if len(emb[0].all_input_nodes) == 1 else None
+    while ids is not None and ids is not stream and ids.op == "call_function" and ids.target in _ATEN_VIEWS:
+        ids = ids.args[0]   # an exported model may re-view its indices first ([-1, seq])
+    if len(emb) > 3 or ids is not stream:
+        raise NotLowerable("embedding tables other than a token table, a position table and a token-type table")
+    wte = root.get_submodule(emb[0].target)
+    if len(emb) == 1:
+        return [WrappedTokenEmbedding(wte, None)], _skip_identities(root, emb[0])
+    # the sum of all the look-ups: an addition fed by exactly these tables (and additions of them)
+    joins = [n for n in nodes if _is_add(n) and set(_branch_layers(n, stream, order)) - {n} >= set(emb) and
+             all(_is_add(x) or x in emb for x in _branch_layers(n, stream, order))]
+    if not joins:
+        raise NotLowerable("the embedding look-ups are not simply added")
+    norm_node, norm = _only_layer_user(root, joins[0])
+    if len(emb) == 2:
+        position = root.get_submodule(emb[1].target)
+        if isinstance(norm, nn.LayerNorm):      # an encoder front without token types
+            return [WrappedEncoderEmbedding(wte, position, None, norm)], _skip_identities(root, norm_node)
+        return [WrappedTokenEmbedding(wte, position)], _skip_identities(root, joins[0])
+    # three tables: which is which shows in their constant index tensors (all zero: token type 0; 0 .. S-1: positions)
+    roles = {}
+    for e in emb[1:]:
+        index = _constant_of(root, e.all_input_nodes[0]) if len(e.all_input_nodes) == 1 else None
+        if index is not None and index.dtype == torch.int64:
+            if bool((index == 0).all()):
+                roles["type"] = e
+            elif bool((index.reshape(-1, index.shape[-1]) == torch.arange(index.shape[-1])).all()):
+                roles["position"] = e
+    if len(roles) != 2 or not isinstance(norm, nn.LayerNorm):
+        raise NotLowerable("three embedding tables that are not word + position + token type 0 under a LayerNorm")
+    block = WrappedEncoderEmbedding(wte, root.get_submodule(roles["position"].target),
+                                    root.get_submodule(roles["type"].target), norm)
+    return [block], _skip_identities(root, norm_node)
+
+
+def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_heads: int, rope) -> NativeBlock:
+    """One transformer layer from its two classified branches (and, for post-LayerNorm layers, the
+    LayerNorms that follow their additions)."""
+    if (attention[0], feed_forward[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
+        raise NotLowerable(f"a '{attention[0]}' branch followed by a '{feed_forward[0]}' branch")
+    d = attention[3].in_features
+    if d % n_heads or d // n_heads not in (64, 128):
+        raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
+    if feed_forward[0] == "mlp":
+        _, ln1, qkv, proj, causal = attention
+        _, ln2, fc1, fc2, act = feed_forward
+        if (ln1 is None) != (ln2 is None) or (ln1 is None) != (attention_norm is not None) \
+                or (ln2 is None) != (feed_forward_norm is not None):
+            raise NotLowerable("a layer that is neither pre-LayerNorm nor post-LayerNorm throughout")
+        if ln1 is None:
+            return WrappedTransformerLayer(attention_norm, qkv, proj, feed_forward_norm, fc1, fc2, n_heads, causal,
+                                           act, pre_ln=False)
+        return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act)
+    _, norm1, qkv, o = attention
+    _, norm2, gate_up, down = feed_forward
+    width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
+    D = d // n_heads
+    if width % D or (width // D - n_heads) % 2 or width // D <= n_heads:
+        raise NotLowerable("query / key / value projections that are not whole heads")
+    if rope is None:
+        raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the positions "
+                           "(exported models do)")
+    return WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope)
+
+
+def _tail_blocks(root: nn.Module, stream: fx.Node, result: fx.Node, after_layers: bool) -> List[NativeBlock]:
+    """What follows the last residual addition must be a chain: projections with activations, a final
+    norm, the vocabulary projection."""
+    tail, cur = [], stream
+    while cur is not result:
+        users = list(cur.users)
+        if len(users) != 1:
+            raise NotLowerable(f"'{cur.format_node()}' feeds {len(users)} nodes after the last residual addition")
+        cur = users[0]
+        if cur.op == "output":
+            break
+        tail.append(cur)
+    mods = []
+    for n in tail:
+        act = _activation_of(n, root)
+        if act == "identity" or (n.op == "call_function" and n.target in _ATEN_VIEWS):
+            continue
+        if act in ("relu", "gelu_tanh", "gelu_erf") and mods and isinstance(mods[-1], (nn.Linear, InOutLinear)):
+            mods[-1] = LinearAct(mods[-1], act)     # a projection with its activation
+            continue
+        if n.op != "call_module":
+            raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
+        m = root.get_submodule(n.target)
+        mods.append(_as_linear(m) or _as_rms_norm(m) or m)
+    blocks: List[NativeBlock] = []
+    while mods and isinstance(mods[0], LinearAct):
+        blocks.append(mods.pop(0))       # e.g. the transform in front of a masked-language-model head
+    norm_types, linear_types = (nn.LayerNorm, nn.RMSNorm, RMSNormLike), (nn.Linear, InOutLinear)
+    if len(mods) == 2 and isinstance(mods[0], norm_types) and isinstance(mods[1], nn.Linear):
+        return blocks + [WrappedLMHead(mods[0], mods[1])]
+    if len(mods) == 1 and isinstance(mods[0], nn.Linear) and mods[0].bias is None and (after_layers or blocks):
+        return blocks + [WrappedLMHead(None, mods[0])]
+    for m in mods:
+        if isinstance(m, nn.LayerNorm):
+            blocks.append(LayerNormBlock(m))
+        elif isinstance(m, (nn.RMSNorm, RMSNormLike)):
+            blocks.append(RMSNormBlock(m))
+        elif isinstance(m, linear_types):
+            blocks.append(LinearAct(m, None))
+        elif isinstance(m, LinearAct):
+            blocks.append(m)
+        else:
+            raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
+    return blocks
+
+
 def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) -> List[NativeBlock]:
+    """The blocks of a stage that is an embedding front, residual layers and a tail (each optional except
+    that there must be a layer).  ``rope``: the (cos, sin) tables of rotary layers."""
     nodes = list(graph.nodes)
     order = {n: i for i, n in enumerate(nodes)}
     placeholders = [n for n in nodes if n.op == "placeholder"]
     if len(placeholders) != 1:
         raise NotLowerable(f"the stage takes {len(placeholders)} inputs; a launch-list stage takes one tensor")
-    out_node = next(n for n in nodes if n.op == "output")
-    result = out_node.args[0]
+    result = next(n for n in nodes if n.op == "output").args[0]
     if isinstance(result, (tuple, list)):
         if len(result) != 1:
             raise NotLowerable("the stage returns several values")
         result = result[0]
-    stream = placeholders[0]
-    blocks: List[NativeBlock] = []
-    # embedding front: the first addition of two embedding look-ups, or a lone token table
-    emb = [n for n in nodes if n.op == "call_module" and isinstance(root.get_submodule(n.target), nn.Embedding)]
-    if emb:
-        ids = emb[0].all_input_nodes[0] if len(emb[0].all_input_nodes) == 1 else None
-        while ids is not None and ids is not stream and ids.op == "call_function" and ids.target in _ATEN_VIEWS:
-            ids = ids.args[0]   # an exported model may re-view its indices first ([-1, seq])
-        if len(emb) > 3 or ids is not stream:
-            raise NotLowerable("embedding tables other than a token table, a position table and a token-type table")
-        wte = root.get_submodule(emb[0].target)
-        if len(emb) == 3:
-            # the encoder front: word + token type (all zero) + position (0 .. S-1), then a LayerNorm
-            joins = [n for n in nodes if _is_add(n) and
-                     set(_branch_layers(n, stream, order)) - {n} >= set(emb) and
-                     all(_is_add(x) or x in emb for x in _branch_layers(n, stream, order))]
-            roles = {}
-            for e in emb[1:]:
-                index = _constant_of(root, e.all_input_nodes[0]) if len(e.all_input_nodes) == 1 else None
-                if index is not None and index.dtype == torch.int64:
-                    if bool((index == 0).all()):
-                        roles["type"] = e
-                    elif bool((index.reshape(-1, index.shape[-1]) == torch.arange(index.shape[-1])).all()):
-                        roles["position"] = e
-            norm_users = [u for u in joins[0].users] if joins else []
-            norm = root.get_submodule(norm_users[0].target) if len(norm_users) == 1 and \
-                norm_users[0].op == "call_module" else None
-            if len(roles) != 2 or not isinstance(norm, nn.LayerNorm):
-                raise NotLowerable("three embedding tables that are not word + position + token type 0 under a LayerNorm")
-            stream = norm_users[0]
-            blocks.append(WrappedEncoderEmbedding(wte, root.get_submodule(roles["position"].target),
-                                                  root.get_submodule(roles["type"].target), norm))
-        elif len(emb) == 2:
-            joins = [n for n in nodes if _is_add(n) and set(_branch_layers(n, stream, order)) == {emb[0], emb[1], n}]
-            if not joins:
-                raise NotLowerable("token and position embeddings are not simply added")
-            stream = joins[0]
-            after = list(stream.users)
-            norm = root.get_submodule(after[0].target) if len(after) == 1 and after[0].op == "call_module" else None
-            if isinstance(norm, nn.LayerNorm):      # an encoder front without token types
-                stream = after[0]
-                blocks.append(WrappedEncoderEmbedding(wte, root.get_submodule(emb[1].target), None, norm))
-            else:
-                blocks.append(WrappedTokenEmbedding(wte, root.get_submodule(emb[1].target)))
-        else:
-            stream = emb[0]
-            blocks.append(WrappedTokenEmbedding(wte, None))
-        while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
-            stream = next(iter(stream.users))   # dropout that does nothing
-    # residual pairs
-    pending = pending_norm = None
+    blocks, stream = _embedding_front(root, nodes, order, placeholders[0])
+    # residual pairs: the stream feeds one addition whose other operand is a branch computed from the stream
+    attention = attention_norm = None
     while True:
         adds = [u for u in stream.users if _is_add(u)]
         if len(adds) != 1:
@@ -483,103 +569,28 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         other = [a for a in add.all_input_nodes if a is not stream]
         if len(other) != 1:
             break
-        kind = _classify_branch(root, [n for n in _branch_layers(other[0], stream, order)])
+        kind = _classify_branch(root, _branch_layers(other[0], stream, order))
         # post-LayerNorm layers: the sum goes through a LayerNorm before anything else reads it
         post_norm, after = None, add
         if kind[0] in ("attn", "mlp") and kind[1] is None:
-            users = list(add.users)
-            m = root.get_submodule(users[0].target) if len(users) == 1 and users[0].op == "call_module" else None
-            if not isinstance(m, nn.LayerNorm):
+            after, post_norm = _only_layer_user(root, add)
+            if not isinstance(post_norm, nn.LayerNorm):
                 raise NotLowerable("a residual branch without a LayerNorm before it or after its addition")
-            post_norm, after = m, users[0]
         if kind[0] in ("attn", "attn_rope"):
-            if pending is not None:
+            if attention is not None:
                 raise NotLowerable("two attention branches in a row")
-            pending, pending_norm = kind, post_norm
+            attention, attention_norm = kind, post_norm
         else:
-            if pending is None:
+            if attention is None:
                 raise NotLowerable("a feed-forward branch without an attention branch before it")
-            if (pending[0], kind[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
-                raise NotLowerable(f"a '{pending[0]}' branch followed by a '{kind[0]}' branch")
-            d = pending[3].in_features
-            if d % n_heads or d // n_heads not in (64, 128):
-                raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
-            if kind[0] == "mlp":
-                _, ln1, qkv, proj, causal = pending
-                _, ln2, fc1, fc2, act = kind
-                if (ln1 is None) != (ln2 is None) or (ln1 is None) != (pending_norm is not None) \
-                        or (ln2 is None) != (post_norm is not None):
-                    raise NotLowerable("a layer that is neither pre-LayerNorm nor post-LayerNorm throughout")
-                if ln1 is None:
-                    blocks.append(WrappedTransformerLayer(pending_norm, qkv, proj, post_norm, fc1, fc2, n_heads,
-                                                          causal, act, pre_ln=False))
-                else:
-                    blocks.append(WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act))
-            else:
-                _, norm1, qkv, o = pending
-                _, norm2, gate_up, down = kind
-                width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
-                D = d // n_heads
-                if width % D or (width // D - n_heads) % 2 or width // D <= n_heads:
-                    raise NotLowerable("query / key / value projections that are not whole heads")
-                if rope is None:
-                    raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the "
-                                       "positions (exported models do)")
-                blocks.append(WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope))
-            pending = None
-        stream = after
-        while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
-            stream = next(iter(stream.users))
-    if pending is not None:
+            blocks.append(_layer_block(attention, attention_norm, kind, post_norm, n_heads, rope))
+            attention = None
+        stream = _skip_identities(root, after)
+    if attention is not None:
         raise NotLowerable("an attention branch without its feed-forward branch in the same stage")
-    # tail: what is left must be a chain of layers
-    tail = []
-    cur = stream
-    while cur is not result:
-        users = [u for u in cur.users]
-        if len(users) != 1:
-            raise NotLowerable(f"'{cur.format_node()}' feeds {len(users)} nodes after the last residual addition")
-        cur = users[0]
-        if cur.op == "output":
-            break
-        tail.append(cur)
-    tail_mods = []
-    for n in tail:
-        act = _activation_of(n, root)
-        if act == "identity" or (n.op == "call_function" and n.target in _ATEN_VIEWS):
-            continue
-        if act in ("relu", "gelu_tanh", "gelu_erf") and tail_mods and isinstance(tail_mods[-1], (nn.Linear, InOutLinear)):
-            tail_mods[-1] = LinearAct(tail_mods[-1], act)     # a projection with its activation
-            continue
-        if n.op != "call_module":
-            raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
-        m = root.get_submodule(n.target)
-        tail_mods.append(_as_linear(m) or _as_rms_norm(m) or m)
-    lead = []
-    while tail_mods and isinstance(tail_mods[0], LinearAct):
-        lead.append(tail_mods.pop(0))       # e.g. the transform in front of a masked-language-model head
-    blocks.extend(lead)
-    kinds = ["Linear" if isinstance(m, (nn.Linear, InOutLinear)) else
-             "LayerNorm" if isinstance(m, (nn.RMSNorm, RMSNormLike)) else type(m).__name__ for m in tail_mods]
-    if kinds == ["LayerNorm", "Linear"] and isinstance(tail_mods[1], nn.Linear):
-        blocks.append(WrappedLMHead(tail_mods[0], tail_mods[1]))
-    elif kinds == ["Linear"] and isinstance(tail_mods[0], nn.Linear) and tail_mods[0].bias is None and blocks:
-        blocks.append(WrappedLMHead(None, tail_mods[0]))
-    else:
-        for m in tail_mods:
-            if isinstance(m, nn.LayerNorm):
-                blocks.append(LayerNormBlock(m))
-            elif isinstance(m, (nn.RMSNorm, RMSNormLike)):
-                blocks.append(RMSNormBlock(m))
-            elif isinstance(m, (nn.Linear, InOutLinear)):
-                blocks.append(LinearAct(m, None))
-            elif isinstance(m, LinearAct):
-                blocks.append(m)
-            else:
-                raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
     if not any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer)) for b in blocks):
         raise NotLowerable("no attention / feed-forward residual pair found")
-    return blocks
+    return blocks + _tail_blocks(root, stream, result, after_layers=True)
 
 
 def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
