@@ -255,6 +255,64 @@ GEMM_SHAPES = (
 )
 
 
+ATTENTION_SHAPES = (
+    # (batch, heads, seq, head_dim, causal, what)
+    (4, 12, 1024, 64, True, "gpt2 layer, one microbatch"),
+    (8, 12, 512, 64, False, "bert layer, one microbatch"),
+    (1, 32, 2048, 128, True, "llama layer, one sequence"),
+    (2, 16, 1024, 64, True, "mixtral-style layer, one microbatch"),
+)
+
+
+def attention_shapes():
+    """One JSON line per shape: the library's attention forward / backward and torch's
+    scaled_dot_product_attention (each of its fused backends that runs) on the same operands, timed with
+    events over back-to-back launches."""
+    import torch.nn.functional as F
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+    from pippy_amd import _native as N
+    N.lib()
+    torch.manual_seed(0)
+
+    def timed(fn, n=50):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+
+    for B, H, S, D, causal, what in ATTENTION_SHAPES:
+        qkv = torch.randn(B, S, 3 * H * D, device="cuda").to(torch.bfloat16)
+        o = torch.empty(B, S, H * D, device="cuda", dtype=torch.bfloat16)
+        lse, delta = torch.empty(B, H, S, device="cuda"), torch.empty(B, H, S, device="cuda")
+        d_o, dqkv = torch.randn_like(o), torch.empty_like(qkv)
+        fwd = timed(lambda: N.attn_fwd(qkv, o, lse, H, causal))
+        bwd = timed(lambda: N.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal))
+        q, k, v = (t.reshape(B, S, H, D).transpose(1, 2).contiguous().requires_grad_(True)
+                   for t in qkv.split(H * D, -1))
+        flops = 4.0 * B * H * S * S * D
+        row = {"shape": [B, H, S, D], "causal": causal, "what": what, "fwd_us": round(fwd, 1),
+               "bwd_us": round(bwd, 1), "fwd_tflops_dense_count": round(flops / fwd / 1e6, 1),
+               "bwd_tflops_dense_count": round(2.5 * flops / bwd / 1e6, 1)}
+        for name, backend in (("flash", SDPBackend.FLASH_ATTENTION), ("efficient", SDPBackend.EFFICIENT_ATTENTION)):
+            try:
+                with sdpa_kernel(backend):
+                    call = lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal)
+                    g = torch.randn_like(call())
+                    f_us = timed(call)
+                    fb_us = timed(lambda: torch.autograd.grad(call(), (q, k, v), g))
+                row[f"torch_sdpa_{name}_fwd_us"] = round(f_us, 1)
+                row[f"torch_sdpa_{name}_bwd_us"] = round(fb_us - f_us, 1)
+            except Exception as e:   # a backend that does not take the shape
+                row[f"torch_sdpa_{name}"] = f"{type(e).__name__}: {str(e)[:80]}"
+        print(json.dumps(row), flush=True)
+
+
 def gemm_shapes():
     """One JSON line per shape: the library's GEMM and torch.matmul on the same operands, each timed over
     rotating operand sets (so that operands are not L2-resident from the previous launch) with the shader
@@ -345,6 +403,10 @@ def main():
                     help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
                          "events, cold operands), torch.matmul (the vendor library) on the same operands beside "
                          "it, and sample the shader clock during each; one JSON line per shape")
+    ap.add_argument("--attention-shapes", action="store_true",
+                    help="instead of a step: time the attention kernels alone on the shapes of the workloads, "
+                         "torch's scaled_dot_product_attention backends on the same operands beside them; one "
+                         "JSON line per shape")
     ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe", "hf_gpt2", "hf_bert"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
                          "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
@@ -376,9 +438,12 @@ def main():
         sys.exit(2)
     # the CPU baseline runs first, in child processes started while this process holds no GPU state
     cpu_result = None
-    if not args.no_cpu_baseline and args.workload == "gpt2":
+    if not args.no_cpu_baseline and args.workload == "gpt2" and not (args.gemm_shapes or args.attention_shapes):
         cpu_result = cpu_baseline(args)
 
+    if args.attention_shapes:
+        attention_shapes()
+        return
     if args.gemm_shapes:
         gemm_shapes()
         return
