@@ -313,6 +313,61 @@ def attention_shapes():
         print(json.dumps(row), flush=True)
 
 
+def rowwise_shapes():
+    """One JSON line per kernel: the library's LayerNorm forward / input gradient and cross entropy
+    (loss + gradient) at the headline shapes, and torch's own operators on the same values."""
+    import torch.nn.functional as F
+    from pippy_amd import _native as N
+    N.lib()
+    torch.manual_seed(0)
+
+    def timed(fn, n=50):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+
+    T, Cc, V = 4096, 768, 50257
+    bf = dict(device="cuda", dtype=torch.bfloat16)
+    x, dy = torch.randn(T, Cc, **bf), torch.randn(T, Cc, **bf)
+    gamma, beta = torch.randn(Cc, **bf), torch.randn(Cc, **bf)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    mean, rstd = torch.empty(T, device="cuda"), torch.empty(T, device="cuda")
+    ours = timed(lambda: N.layernorm_fwd(x, gamma, beta, y, mean, rstd, 1e-5))
+    theirs = timed(lambda: F.layer_norm(x, (Cc,), gamma, beta, 1e-5))
+    print(json.dumps({"kernel": "layernorm forward", "shape": [T, Cc], "us": round(ours, 1),
+                      "GB/s": round(4.0 * T * Cc / ours / 1e3, 1), "torch_us": round(theirs, 1)}), flush=True)
+    ours = timed(lambda: N.layernorm_bwd_input(dy, x, gamma, mean, rstd, None, dx))
+    xr = x.clone().requires_grad_(True)
+    out = F.layer_norm(xr, (Cc,), gamma, beta, 1e-5)
+    theirs = timed(lambda: torch.autograd.grad(out, xr, dy, retain_graph=True))
+    print(json.dumps({"kernel": "layernorm input gradient", "shape": [T, Cc], "us": round(ours, 1),
+                      "GB/s": round(6.0 * T * Cc / ours / 1e3, 1), "torch_us": round(theirs, 1),
+                      "note": "torch's backward also forms the weight and bias gradients here"}), flush=True)
+    Vp = (V + 127) // 128 * 128
+    logits = torch.randn(T, Vp, **bf)
+    dlogits = torch.empty_like(logits)
+    target = torch.randint(0, V, (T,), device="cuda")
+    loss, ws = torch.empty(1, device="cuda"), torch.empty(T + 2, device="cuda")
+    ours = timed(lambda: N.ce_loss(logits, target, loss, dlogits, ws, V), n=20)
+    lr = logits[:, :V].clone().requires_grad_(True)
+
+    def torch_ce():
+        torch.autograd.grad(F.cross_entropy(lr.float(), target), lr)
+
+    theirs = timed(torch_ce, n=20)
+    print(json.dumps({"kernel": "cross entropy, loss and gradient", "shape": [T, V], "us": round(ours, 1),
+                      "GB/s": round(4.0 * T * V / ours / 1e3, 1), "torch_us": round(theirs, 1),
+                      "note": "torch: F.cross_entropy on the fp32 cast of the bf16 logits, and its backward"}),
+          flush=True)
+
+
 def gemm_shapes():
     """One JSON line per shape: the library's GEMM and torch.matmul on the same operands, each timed over
     rotating operand sets (so that operands are not L2-resident from the previous launch) with the shader
@@ -405,8 +460,9 @@ def main():
                          "it, and sample the shader clock during each; one JSON line per shape")
     ap.add_argument("--attention-shapes", action="store_true",
                     help="instead of a step: time the attention kernels alone on the shapes of the workloads, "
-                         "torch's scaled_dot_product_attention backends on the same operands beside them; one "
-                         "JSON line per shape")
+                         "torch's scaled_dot_product_attention backends on the same operands beside them, then "
+                         "LayerNorm and cross entropy at the headline shapes beside torch's operators; one JSON "
+                         "line per shape")
     ap.add_argument("--workload", default="gpt2", choices=["gpt2", "bert", "llama", "moe", "hf_gpt2", "hf_bert"],
                     help="gpt2: the headline configuration (default); bert / llama / moe: the BERT-base "
                          "inference, Llama-2-7B stage (zero-bubble) and Mixtral-style (interleaved 1F1B) "
@@ -443,6 +499,7 @@ def main():
 
     if args.attention_shapes:
         attention_shapes()
+        rowwise_shapes()
         return
     if args.gemm_shapes:
         gemm_shapes()
