@@ -1277,6 +1277,8 @@ def test_outputs_merged_while_the_step_runs_are_the_merge_at_the_end(monkeypatch
     step gives, a tensor of its own (a later step must not change it), contiguous like torch.cat's, and
     uneven microbatches must fall back to the merge at the end."""
     import pippy_amd as pp
+    monkeypatch.delenv("PIPPY_AMD_SERIAL_STAGES", raising=False)   # (the running merge needs the stage streams)
+    monkeypatch.delenv("PIPPY_AMD_MERGE_AT_END", raising=False)
     M = 4
     model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
     target = torch.randint(0, 1000, ids.shape)
