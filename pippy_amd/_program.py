@@ -134,6 +134,21 @@ class ParamArena:
             self._transposed[key] = ent
         return ent[1]
 
+    def weight_t_stack(self, p: nn.Parameter) -> torch.Tensor:
+        """[E, in, out]: the transposed copy of every [out, in] matrix of a stacked 3-d weight, kept in
+        step with the parameter by ``refresh_transposed``."""
+        key = ("stack", id(p))
+        ent = self._transposed.get(key)
+        if ent is None:
+            w = self.weight(p, padded=True)
+            t = torch.empty((w.shape[0], w.shape[2], w.shape[1]), dtype=w.dtype, device=self.device)
+            for e in range(w.shape[0]):
+                N.transpose_bf16(w[e], t[e])
+                self._transposed[key + (e,)] = (p, t[e], e)
+            ent = (None, t)
+            self._transposed[key] = ent
+        return ent[1]
+
     def rows_cat(self, *ps: nn.Parameter) -> torch.Tensor:
         """[out1 + out2 + ..., in] (or the 1-d analogue for biases): copies of parameters with the same
         trailing shape stacked along dimension 0, so that projections which read the same input run as
@@ -156,14 +171,15 @@ class ParamArena:
         optimizer step bumps the parameter's version counter)."""
         if not self._transposed and not self._stacked:
             return
-        live = [(p, t) for p, t in self._transposed.values() if p is not None]
+        live = [ent for ent in self._transposed.values() if ent[0] is not None]
         stacked = [(p, view) for _, parts in self._stacked.values() for p, view in parts]
-        versions = (self._epoch,) + tuple(p._version for p, _ in live + stacked)
+        versions = (self._epoch,) + tuple(ent[0]._version for ent in live) + tuple(p._version for p, _ in stacked)
         if versions == self._versions:
             return
         self._versions = versions
-        for p, t in live:
-            N.transpose_bf16(self.weight(p, padded=True), t)
+        for ent in live:      # (parameter, copy[, index of the matrix inside a stacked parameter])
+            src = self.weight(ent[0], padded=True)
+            N.transpose_bf16(src if len(ent) == 2 else src[ent[2]], ent[1])
         for p, view in stacked:
             view.copy_(self.weight(p, padded=True))
 

@@ -778,44 +778,110 @@ class _Expert(nn.Module):
         return self.w2(F.silu(self.w1(x)) * self.w3(x))
 
 
-class MoELayer(LlamaLayer):
-    """A Mixtral-style decoder layer: the attention half of ``LlamaLayer`` and, in place of the dense
-    feed-forward, a sparse mixture of ``n_experts`` SwiGLU experts of which a softmax router picks
-    two per token (weights renormalised over the pair).  Parameters: ``block_sparse_moe.gate`` and
-    ``block_sparse_moe.experts.<e>.w1 / w2 / w3``.  The launch-list form takes 2 .. 64 experts (a count that is not a multiple of 8 runs with the router
-    weight and the logits padded to one).
+class _ExpertModules:
+    """The expert weights of a layer that keeps one module per expert (``w1`` gate, ``w3`` up, ``w2``
+    down, each an ``nn.Linear``): per projection, the [out, in] weights, their transposed copies and the
+    places their gradients go, one tensor per expert."""
 
-    ``forced_routing`` (a list of int64 [tokens, 2] tensors, one per forward call, consumed in
-    order) overrides the expert selection of the torch statement; a comparison against a lower
-    precision run uses it so that tokens whose second and third logits nearly tie do not count as
-    errors of the arithmetic."""
+    _ATTR = {"gate": "w1", "up": "w3", "down": "w2"}
+
+    def __init__(self, experts):
+        self.experts = list(experts)
+
+    def __len__(self):
+        return len(self.experts)
+
+    def _params(self, which):
+        return [getattr(ex, self._ATTR[which]).weight for ex in self.experts]
+
+    def weights(self, b, which):
+        return [b.weight(p) for p in self._params(which)], None
+
+    def transposed(self, b, which):
+        return [b.weight_t(p) for p in self._params(which)], None
+
+    def grad_epilogue(self, b, which):
+        epis = {b.weight_grad_epilogue(p) for p in self._params(which)}
+        assert len(epis) == 1
+        return epis.pop()
+
+    def grad_accumulators(self, b, which):
+        return [b.grad_acc(p) for p in self._params(which)], None
+
+    def grad_targets(self, b, which):
+        return [b.grad_target(p) for p in self._params(which)], None
+
+    def apply(self, e, x):
+        """Torch statement of expert ``e``."""
+        return self.experts[e](x)
+
+
+class _ExpertTensors:
+    """The expert weights of a layer that keeps them stacked: ``gate_up`` [E, 2 f, d] (gate rows first)
+    and ``down`` [E, d, f] (the Hugging Face Mixtral layout).  Same interface as ``_ExpertModules``; the
+    second value of a pair is the leading dimension where a tensor is a column range of a wider one."""
+
+    def __init__(self, gate_up: nn.Parameter, down: nn.Parameter):
+        assert gate_up.dim() == 3 and down.dim() == 3 and gate_up.shape[0] == down.shape[0]
+        assert gate_up.shape[1] == 2 * down.shape[2] and gate_up.shape[2] == down.shape[1]
+        self.gate_up, self.down = gate_up, down
+        self.ffn = down.shape[2]
+
+    def __len__(self):
+        return self.gate_up.shape[0]
+
+    def _slices(self, stacked, which):
+        f = self.ffn
+        if which == "down":
+            return [stacked[e] for e in range(len(self))]
+        return [stacked[e, :f] if which == "gate" else stacked[e, f:] for e in range(len(self))]
+
+    def _param(self, which):
+        return self.down if which == "down" else self.gate_up
+
+    def weights(self, b, which):
+        return self._slices(b.weight(self._param(which)), which), None
+
+    def transposed(self, b, which):
+        t = b.sp.arena.weight_t_stack(self._param(which))      # [E, in, out]
+        if which == "down":
+            return [t[e] for e in range(len(self))], None
+        f = self.ffn
+        return [t[e][:, :f] if which == "gate" else t[e][:, f:] for e in range(len(self))], 2 * f
+
+    def grad_epilogue(self, b, which):
+        return b.weight_grad_epilogue(self._param(which))
+
+    def grad_accumulators(self, b, which):
+        return self._slices(b.grad_acc(self._param(which)), which), None
+
+    def grad_targets(self, b, which):
+        return self._slices(b.grad_target(self._param(which)), which), None
+
+    def apply(self, e, x):
+        f = self.ffn
+        gu = F.linear(x, self.gate_up[e])
+        return F.linear(F.silu(gu[..., :f]) * gu[..., f:], self.down[e])
+
+
+class _MoEFeedForward:
+    """The sparse feed-forward half of a Mixtral-style layer (mixed into a Llama-style layer class):
+    a softmax router picks two of ``n_experts`` SwiGLU experts per token, weights renormalised over the
+    pair.  Needs ``self.n_experts``, ``self.ffn``, ``self._experts`` (an expert-weight bank),
+    ``self._router`` (an ``nn.Linear``-shaped layer) and ``self.forced_routing``."""
 
     TOPK = 2
-
-    def __init__(self, dim: int, n_heads: int, ffn: int, n_experts: int = 8, *, eps: float = 1e-5,
-                 rope_theta: float = 1e6, dtype=torch.bfloat16, init_std=0.02, n_kv_heads: Optional[int] = None):
-        super().__init__(dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype, init_std=init_std,
-                         n_kv_heads=n_kv_heads)
-        del self.mlp
-        assert 2 <= n_experts <= 64
-        self.n_experts = n_experts
-        self.block_sparse_moe = nn.Module()
-        self.block_sparse_moe.gate = nn.Linear(dim, n_experts, bias=False, dtype=dtype)
-        nn.init.normal_(self.block_sparse_moe.gate.weight, std=init_std)
-        self.block_sparse_moe.experts = nn.ModuleList([_Expert(dim, ffn, dtype, init_std) for _ in range(n_experts)])
-        self.forced_routing = None
 
     def _padded_experts(self) -> int:
         return (self.n_experts + 7) // 8 * 8
 
     def _pp_padded_rows(self):
-        return [(self.block_sparse_moe.gate.weight, self._padded_experts())] if self.n_experts % 8 else []
+        return [(self._router.weight, self._padded_experts())] if self.n_experts % 8 else []
 
     def _feed_forward(self, h):
         shape = h.shape
         h = h.reshape(-1, shape[-1])
-        moe = self.block_sparse_moe
-        probs = torch.softmax(moe.gate(h).float(), dim=-1)
+        probs = torch.softmax(self._router(h).float(), dim=-1)
         if self.forced_routing:
             idx = self.forced_routing.pop(0).to(h.device)
         else:
@@ -823,10 +889,10 @@ class MoELayer(LlamaLayer):
         top = probs.gather(-1, idx)
         gate = top / top.sum(-1, keepdim=True)
         y = torch.zeros(h.shape, dtype=torch.float32, device=h.device)
-        for e, expert in enumerate(moe.experts):
+        for e in range(self.n_experts):
             tok, slot = torch.where(idx == e)
             if tok.numel():
-                y = y.index_add(0, tok, gate[tok, slot, None] * expert(h[tok]).float())
+                y = y.index_add(0, tok, gate[tok, slot, None] * self._experts.apply(e, h[tok]).float())
         return y.to(h.dtype).reshape(shape)
 
     def _pointer_list(self, b, name, tensors):
@@ -841,11 +907,10 @@ class MoELayer(LlamaLayer):
         # the router weight is stored with zero rows up to a multiple of 8, and so are the logits
         Ep = self._padded_experts()
         R = T * K
-        moe = self.block_sparse_moe
-        experts = list(moe.experts)
+        bank, router = self._experts, self._router
         n2, rstd2 = lower_rmsnorm(b, "n2", self.post_attention_layernorm, x2)
         logits = b.act("router_logits", (T, Ep))
-        lower_linear(b, "router", moe.gate, n2, out=logits)
+        lower_linear(b, "router", router, n2, out=logits)
         idx = b.act("topk_idx", (T, K), torch.int32)
         gate = b.act("gate", (T, K), torch.float32)
         b.f(P.op_moe_router(logits, idx, gate, E))
@@ -855,17 +920,22 @@ class MoELayer(LlamaLayer):
         b.f(P.op_moe_permute(idx.view(-1), E, seg, row_src, pos))
         xp = b.act("xp", (R, Cc))
         b.f(P.op_moe_gather(n2, row_src, K, xp))
-        w1 = self._pointer_list(b, "w1", [b.weight(ex.w1.weight) for ex in experts])
-        w2 = self._pointer_list(b, "w2", [b.weight(ex.w2.weight) for ex in experts])
-        w3 = self._pointer_list(b, "w3", [b.weight(ex.w3.weight) for ex in experts])
+
+        def pointers(name, pair):
+            tensors, ld = pair
+            return self._pointer_list(b, name, tensors), ld
+
+        w1, ld1 = pointers("w1", bank.weights(b, "gate"))
+        w3, ld3 = pointers("w3", bank.weights(b, "up"))
+        w2, ld2 = pointers("w2", bank.weights(b, "down"))
         g = b.act("g", (R, ffn))
         u = b.act("u", (R, ffn))
         h = b.act("h", (R, ffn))
         yp = b.act("yp", (R, Cc))
-        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w1, seg, Cm=g))
-        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w3, seg, Cm=u))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w1, seg, Cm=g, ld=ld1))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w3, seg, Cm=u, ld=ld3))
         b.f(P.op_swiglu_fwd(g, u, h))
-        b.f(P.op_gemm_seg(N.SEG_ROWS, h, w2, seg, Cm=yp))
+        b.f(P.op_gemm_seg(N.SEG_ROWS, h, w2, seg, Cm=yp, ld=ld2))
         y = b.act("y", (T, Cc))
         b.f(P.op_moe_combine(yp, pos, K, y, gate=gate.view(-1), resid=x2))
 
@@ -875,38 +945,70 @@ class MoELayer(LlamaLayer):
             b.i(P.op_moe_gather(dy2d, row_src, K, d_yp, scale=gate.view(-1)))
             dlogits = b.grad("dlogits", (T, Ep))
             b.i(P.op_moe_gate_bwd(dy2d, yp, pos, idx, gate, E, dlogits))
-            w2t = self._pointer_list(b, "w2t", [b.weight_t(ex.w2.weight) for ex in experts])
-            w1t = self._pointer_list(b, "w1t", [b.weight_t(ex.w1.weight) for ex in experts])
-            w3t = self._pointer_list(b, "w3t", [b.weight_t(ex.w3.weight) for ex in experts])
+            w2t, ld2t = pointers("w2t", bank.transposed(b, "down"))
+            w1t, ld1t = pointers("w1t", bank.transposed(b, "gate"))
+            w3t, ld3t = pointers("w3t", bank.transposed(b, "up"))
             d_h = b.grad("d_h", (R, ffn))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, d_yp, w2t, seg, Cm=d_h))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, d_yp, w2t, seg, Cm=d_h, ld=ld2t))
             dg = b.grad("dg", (R, ffn))
             du = b.grad("du", (R, ffn))
             b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
             d_xp = b.grad("d_xp", (R, Cc))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=d_xp))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp, ld=ld1t))
+            b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, ld=ld3t, epilogue=N.EPI_BIAS_RESIDUAL,
+                              aux_in=d_xp))
             # token gradient: its two expert rows, plus the router branch in the GEMM epilogue
             d_n2a = b.grad("d_n2a", (T, Cc))
             b.i(P.op_moe_combine(d_xp, pos, K, d_n2a))
-            d_n2 = linear_backward(b, "router", moe.gate, n2, dlogits, dx_epilogue=N.EPI_BIAS_RESIDUAL,
+            d_n2 = linear_backward(b, "router", router, n2, dlogits, dx_epilogue=N.EPI_BIAS_RESIDUAL,
                                    dx_aux=d_n2a)
             # expert weight gradients: one segmented GEMM per projection, reduced over each expert's rows
-            for name, dy_rows, x_rows in (("w1", dg, xp), ("w3", du, xp), ("w2", d_yp, h)):
-                params = [getattr(ex, name).weight for ex in experts]
-                epis = {b.weight_grad_epilogue(p) for p in params}
-                assert len(epis) == 1
-                epi = epis.pop()
+            for which, name, dy_rows, x_rows in (("gate", "w1", dg, xp), ("up", "w3", du, xp), ("down", "w2", d_yp, h)):
+                epi = bank.grad_epilogue(b, which)
                 if epi is not None:
-                    ptrs = self._pointer_list(b, "acc_" + name, [b.grad_acc(p) for p in params])
-                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, epilogue=epi,
+                    ptrs, ld = pointers("acc_" + name, bank.grad_accumulators(b, which))
+                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, ld=ld, epilogue=epi,
                                       beta=1, c_f32=True), tag="beta")
                 else:
-                    ptrs = self._pointer_list(b, "stage_" + name, [b.grad_target(p) for p in params])
-                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows))
+                    ptrs, ld = pointers("stage_" + name, bank.grad_targets(b, which))
+                    b.w(P.op_gemm_seg(N.SEG_K, dy_rows, ptrs, seg, other=x_rows, ld=ld))
             return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
 
         return y, backward
+
+
+class MoELayer(_MoEFeedForward, LlamaLayer):
+    """A Mixtral-style decoder layer: the attention half of ``LlamaLayer`` and, in place of the dense
+    feed-forward, a sparse mixture of ``n_experts`` SwiGLU experts of which a softmax router picks
+    two per token (weights renormalised over the pair).  Parameters: ``block_sparse_moe.gate`` and
+    ``block_sparse_moe.experts.<e>.w1 / w2 / w3``.  The launch-list form takes 2 .. 64 experts (a count
+    that is not a multiple of 8 runs with the router weight and the logits padded to one).
+
+    ``forced_routing`` (a list of int64 [tokens, 2] tensors, one per forward call, consumed in
+    order) overrides the expert selection of the torch statement; a comparison against a lower
+    precision run uses it so that tokens whose second and third logits nearly tie do not count as
+    errors of the arithmetic."""
+
+    def __init__(self, dim: int, n_heads: int, ffn: int, n_experts: int = 8, *, eps: float = 1e-5,
+                 rope_theta: float = 1e6, dtype=torch.bfloat16, init_std=0.02, n_kv_heads: Optional[int] = None):
+        LlamaLayer.__init__(self, dim, n_heads, ffn, eps=eps, rope_theta=rope_theta, dtype=dtype,
+                            init_std=init_std, n_kv_heads=n_kv_heads)
+        del self.mlp
+        assert 2 <= n_experts <= 64
+        self.n_experts = n_experts
+        self.block_sparse_moe = nn.Module()
+        self.block_sparse_moe.gate = nn.Linear(dim, n_experts, bias=False, dtype=dtype)
+        nn.init.normal_(self.block_sparse_moe.gate.weight, std=init_std)
+        self.block_sparse_moe.experts = nn.ModuleList([_Expert(dim, ffn, dtype, init_std) for _ in range(n_experts)])
+        self.forced_routing = None
+
+    @property
+    def _router(self):
+        return self.block_sparse_moe.gate
+
+    @property
+    def _experts(self):
+        return _ExpertModules(self.block_sparse_moe.experts)
 
 
 class LMHead(NativeBlock):
