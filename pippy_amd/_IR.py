@@ -482,6 +482,9 @@ class Pipe(nn.Module):
                 if "Cache" in str(export_error) and getattr(getattr(mod, "config", None), "use_cache", False):
                     hint = ("; the model returns a key / value cache object, which torch.export cannot flatten: "
                             "build it with config.use_cache = False")
+                if "data pointer" in str(export_error) and hasattr(getattr(mod, "config", None), "_experts_implementation"):
+                    hint = ("; the model's grouped expert product inspects tensor addresses, which torch.export "
+                            "cannot trace: build it with config._experts_implementation = 'batched_mm'")
                 raise RuntimeError(
                     f"pipeline(): neither torch.fx symbolic tracing ({type(fx_error).__name__}: {fx_error}) "
                     f"nor torch.export ({type(export_error).__name__}: {export_error}) can trace this model{hint}"

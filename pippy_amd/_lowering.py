@@ -19,7 +19,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, RMSNormLike,
-                            StageSequence, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead,
+                            StageSequence, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer,
                             WrappedTokenEmbedding,
                             WrappedTransformerLayer, activation_like, in_out_linear_like, rms_norm_like)
 
@@ -239,8 +239,9 @@ def _is_add(n: fx.Node) -> bool:
     return (n.op == "call_function" and n.target in _ADD_FNS) or (n.op == "call_method" and n.target in ("add", "add_"))
 
 
-def _branch_layers(y: fx.Node, stream: fx.Node, order: dict) -> List[fx.Node]:
-    """The layer and function nodes that ``y`` is computed from, back to ``stream`` (in graph order)."""
+def _branch_layers(y: fx.Node, stream: fx.Node, order: dict, state: bool = False) -> List[fx.Node]:
+    """The layer and function nodes that ``y`` is computed from, back to ``stream`` (in graph order);
+    with ``state`` also the ``get_attr`` nodes (parameters the model's own forward reads) and top-k nodes."""
     seen, stack, found = set(), [y], []
     while stack:
         n = stack.pop()
@@ -251,6 +252,8 @@ def _branch_layers(y: fx.Node, stream: fx.Node, order: dict) -> List[fx.Node]:
             continue
         if n.op == "call_module" or (n.op == "call_function" and n.target in _SDPA + _ACT_FNS) \
                 or _is_add(n):
+            found.append(n)
+        elif state and (n.op == "get_attr" or (n.op == "call_function" and n.target is _ATEN.topk.default)):
             found.append(n)
         stack.extend(a for a in n.all_input_nodes)
     return sorted(found, key=order.get)
@@ -304,7 +307,8 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
         raise NotLowerable("scaled_dot_product_attention with dropout or grouped queries")
     scale = given.get("scale")
     if scale is not None and not any(abs(float(scale) - d ** -0.5) < 1e-6 for d in head_dims):
-        raise NotLowerable(f"scaled_dot_product_attention with the custom scale {scale}")
+        raise NotLowerable(f"scaled_dot_product_attention with the scale {scale}, which is not the default for "
+                           f"a head size of {' or '.join(map(str, head_dims))}")
     causal = bool(given.get("is_causal", False))
     mask = given.get("attn_mask")
     if mask is not None:
@@ -317,14 +321,52 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
     return causal
 
 
+def _classify_expert_branch(root: nn.Module, norm, state: List[fx.Node]):
+    """("mlp_moe", norm, router module, experts module, gate_up, down) for a feed-forward branch that reads
+    a router weight [E, d] and two stacked expert parameters, gate|up [E, 2 f, d] and down [E, d, f], and
+    picks two experts per token.  How the model routes and combines is not parsed: the block's own
+    statement (softmax over all experts, top-2, renormalised) is compared with the stage numerically."""
+    params, owners = [], {}
+    for n in state:
+        if n.op != "get_attr":
+            continue
+        path = str(n.target).split(".")
+        try:
+            owner = root.get_submodule(".".join(path[:-1]))
+            value = getattr(owner, path[-1])
+        except AttributeError:
+            continue
+        if isinstance(value, nn.Parameter) and id(value) not in owners:
+            owners[id(value)] = owner
+            params.append(value)
+    top = [n for n in state if n.op == "call_function"]
+    if len(top) != 1 or top[0].args[1] != 2:
+        raise NotLowerable("a mixture-of-experts feed-forward that does not pick two experts per token")
+    routers = [p for p in params if p.dim() == 2]
+    stacked = [p for p in params if p.dim() == 3]
+    if len(params) != 3 or len(routers) != 1 or len(stacked) != 2:
+        raise NotLowerable("a mixture-of-experts feed-forward whose parameters are not a router weight and two "
+                           "stacked expert tensors")
+    router = routers[0]
+    E, d = router.shape
+    gate_up = next((p for p in stacked if p.shape[0] == E and p.shape[2] == d and p.shape[1] % 2 == 0), None)
+    down = next((p for p in stacked if p is not gate_up), None)
+    if gate_up is None or down is None or tuple(down.shape) != (E, d, gate_up.shape[1] // 2) or not 2 <= E <= 64:
+        raise NotLowerable("stacked expert tensors that are not gate|up [E, 2 f, d] and down [E, d, f]")
+    return ("mlp_moe", norm, owners[id(router)], owners[id(gate_up)], gate_up, down)
+
+
 def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     """What a residual branch is, from the layers between the stream and the addition:
     ("attn", ln, qkv, proj, causal) / ("mlp", ln, fc1, fc2, activation) for the GPT-2 and BERT families
     (ln is None when the branch does not start with a LayerNorm; qkv is one fused layer or three),
     ("attn_rope", norm, qkv, o) / ("mlp_gated", norm, gate_up, down) for the Llama family (qkv: the
     fused projection or the three separate ones; gate_up: the fused projection or the two separate ones)."""
-    mods, inner_adds = [], []
+    mods, inner_adds, state = [], [], []
     for n in layers:
+        if n.op == "get_attr" or (n.op == "call_function" and n.target is _ATEN.topk.default):
+            state.append(n)
+            continue
         if _activation_of(n, root) == "identity":
             continue
         if n.op == "call_module":
@@ -345,6 +387,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         return "act" if _activation_of(n, root) is not None else type(m).__name__
 
     kinds = [kind(n, m) for n, m in mods]
+    if kinds == ["RMSNorm", "act"] and _activation_of(mods[1][0], root) == "silu":
+        return _classify_expert_branch(root, mods[0][1], state)
     if kinds == ["RMSNorm", "Linear", "Linear", "Linear", "sdpa", "Linear"]:
         (_, norm), (_, q), (_, k), (_, v), (sd, _), (_, o) = mods
         if not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
@@ -472,7 +516,7 @@ def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream:
 def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_heads: int, rope) -> NativeBlock:
     """One transformer layer from its two classified branches (and, for post-LayerNorm layers, the
     LayerNorms that follow their additions)."""
-    if (attention[0], feed_forward[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated")):
+    if (attention[0], feed_forward[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated"), ("attn_rope", "mlp_moe")):
         raise NotLowerable(f"a '{attention[0]}' branch followed by a '{feed_forward[0]}' branch")
     d = attention[3].in_features
     if d % n_heads or d // n_heads not in (64, 128):
@@ -488,7 +532,6 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
                                            act, pre_ln=False)
         return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act)
     _, norm1, qkv, o = attention
-    _, norm2, gate_up, down = feed_forward
     width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
     D = d // n_heads
     if width % D or (width // D - n_heads) % 2 or width // D <= n_heads:
@@ -496,6 +539,10 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
     if rope is None:
         raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the positions "
                            "(exported models do)")
+    if feed_forward[0] == "mlp_moe":
+        _, norm2, router, experts, gate_up, down = feed_forward
+        return WrappedMoELayer(norm1, qkv, o, norm2, router, experts, gate_up, down, n_heads, *rope)
+    _, norm2, gate_up, down = feed_forward
     return WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope)
 
 
@@ -569,7 +616,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         other = [a for a in add.all_input_nodes if a is not stream]
         if len(other) != 1:
             break
-        kind = _classify_branch(root, _branch_layers(other[0], stream, order))
+        kind = _classify_branch(root, _branch_layers(other[0], stream, order, state=True))
         # post-LayerNorm layers: the sum goes through a LayerNorm before anything else reads it
         post_norm, after = None, add
         if kind[0] in ("attn", "mlp") and kind[1] is None:
@@ -659,6 +706,7 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
         probe = copy.deepcopy(submod).float().cpu().eval()
     except Exception as e:
         raise NotLowerable(f"the stage module cannot be copied for verification: {e}") from e
+    _widen_baked_casts(probe)
     probe_graph = _ChainTracer().trace(probe)
     tolerance = 1e-4
     reasons = []
@@ -682,6 +730,27 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
         reasons.append(f"with {n_heads} heads the recognised blocks differ from the stage's own forward "
                        f"(relative error {err:.2e})")
     raise NotLowerable("; ".join(reasons))
+
+
+def _widen_baked_casts(probe: nn.Module) -> None:
+    """A model exported in bf16 / fp16 holds the casts its forward made to "the input's dtype" as casts to
+    that dtype.  On the fp32 copy that the recognised blocks are compared with they would round where
+    nothing else does: they become casts to fp32."""
+    if not isinstance(probe, fx.GraphModule):
+        return
+    low = (torch.bfloat16, torch.float16)
+    changed = False
+    for n in probe.graph.nodes:
+        if n.op != "call_function":
+            continue
+        if n.target is _ATEN.to.dtype and len(n.args) > 1 and n.args[1] in low:
+            n.args = (n.args[0], torch.float32) + tuple(n.args[2:])
+            changed = True
+        elif n.target in (_ATEN._to_copy.default, _ATEN.to.dtype_layout) and n.kwargs.get("dtype") in low:
+            n.kwargs = {**n.kwargs, "dtype": torch.float32}
+            changed = True
+    if changed:
+        probe.recompile()
 
 
 def _check_kernel_requirements(submod: nn.Module, blocks: List[NativeBlock]) -> None:

@@ -1280,33 +1280,37 @@ class WrappedLlamaLayer(LlamaLayer):
         """``cos`` / ``sin``: the model's own rotary tables, [positions, head_dim / 2] (whatever base,
         scaling or rounding the model applies is in them)."""
         NativeBlock.__init__(self)
-        self._qkv = tuple(qkv) if isinstance(qkv, (tuple, list)) else (qkv,)
+        self._init_attention(input_layernorm, qkv, o_proj, n_heads, cos, sin)
+        self.post_attention_layernorm = post_attention_layernorm
         self._gate_up = tuple(gate_up) if isinstance(gate_up, (tuple, list)) else (gate_up,)
-        self.dim, self.n_heads = o_proj.out_features, n_heads
         self.ffn = down_proj.in_features
-        D = self.dim // n_heads
-        assert cos.shape == sin.shape and cos.shape[1] == D // 2
-        width = sum(lin.out_features for lin in self._qkv)
-        self.n_kv_heads = (width // D - n_heads) // 2
-        assert self.n_kv_heads > 0 and (n_heads + 2 * self.n_kv_heads) * D == width
         assert sum(lin.out_features for lin in self._gate_up) == 2 * self.ffn
-        self.eps, self.rope_theta = input_layernorm.eps, None
-        self._cos, self._sin = cos.detach().float().cpu().contiguous(), sin.detach().float().cpu().contiguous()
-        import hashlib
-        self._table_key = hashlib.sha1(self._cos.numpy().tobytes() + self._sin.numpy().tobytes()).hexdigest()[:16]
-        self.input_layernorm, self.post_attention_layernorm = input_layernorm, post_attention_layernorm
-        self.self_attn = nn.Module()
-        if len(self._qkv) == 3:
-            self.self_attn.q_proj, self.self_attn.k_proj, self.self_attn.v_proj = self._qkv
-        else:
-            self.self_attn.qkv_proj = self._qkv[0]
-        self.self_attn.o_proj = o_proj
         self.mlp = nn.Module()
         if len(self._gate_up) == 2:
             self.mlp.gate_proj, self.mlp.up_proj = self._gate_up
         else:
             self.mlp.gate_up_proj = self._gate_up[0]
         self.mlp.down_proj = down_proj
+
+    def _init_attention(self, input_layernorm, qkv, o_proj, n_heads, cos, sin):
+        self._qkv = tuple(qkv) if isinstance(qkv, (tuple, list)) else (qkv,)
+        self.dim, self.n_heads = o_proj.out_features, n_heads
+        D = self.dim // n_heads
+        assert cos.shape == sin.shape and cos.shape[1] == D // 2
+        width = sum(lin.out_features for lin in self._qkv)
+        self.n_kv_heads = (width // D - n_heads) // 2
+        assert self.n_kv_heads > 0 and (n_heads + 2 * self.n_kv_heads) * D == width
+        self.eps, self.rope_theta = input_layernorm.eps, None
+        self._cos, self._sin = cos.detach().float().cpu().contiguous(), sin.detach().float().cpu().contiguous()
+        import hashlib
+        self._table_key = hashlib.sha1(self._cos.numpy().tobytes() + self._sin.numpy().tobytes()).hexdigest()[:16]
+        self.input_layernorm = input_layernorm
+        self.self_attn = nn.Module()
+        if len(self._qkv) == 3:
+            self.self_attn.q_proj, self.self_attn.k_proj, self.self_attn.v_proj = self._qkv
+        else:
+            self.self_attn.qkv_proj = self._qkv[0]
+        self.self_attn.o_proj = o_proj
 
     def _rope(self, seq, head_dim, device):
         if seq > self._cos.shape[0] or head_dim != 2 * self._cos.shape[1]:
@@ -1366,6 +1370,54 @@ class WrappedLlamaLayer(LlamaLayer):
             return rmsnorm_backward(b, "n2", self.post_attention_layernorm, x2, rstd2, d_n2, dres=dy2d)
 
         return y, backward
+
+
+class RouterLayer(nn.Module):
+    """An ``nn.Linear``-shaped view of a router module that holds its [experts, d] weight itself and
+    does more than the projection in its forward (Hugging Face's ``MixtralTopKRouter``)."""
+
+    bias = None
+
+    def __init__(self, layer: nn.Module):
+        super().__init__()
+        self.layer = layer
+        self.out_features, self.in_features = layer.weight.shape
+
+    @property
+    def weight(self):
+        return self.layer.weight
+
+    def forward(self, x):
+        return F.linear(x, self.layer.weight)
+
+
+class WrappedMoELayer(_MoEFeedForward, WrappedLlamaLayer):
+    """A Mixtral-style layer around a user's model that keeps its experts stacked in two 3-d parameters
+    (``gate_up`` [E, 2 f, d], ``down`` [E, d, f]) and its router weight in a module of its own: the
+    attention half of ``WrappedLlamaLayer`` and the sparse feed-forward of ``MoELayer``, reading the
+    expert matrices in place."""
+
+    def __init__(self, input_layernorm, qkv, o_proj, post_attention_layernorm, router: nn.Module,
+                 experts: nn.Module, gate_up: nn.Parameter, down: nn.Parameter, n_heads: int,
+                 cos: torch.Tensor, sin: torch.Tensor):
+        NativeBlock.__init__(self)
+        self._init_attention(input_layernorm, qkv, o_proj, n_heads, cos, sin)
+        self.post_attention_layernorm = post_attention_layernorm
+        self.n_experts, self.ffn = gate_up.shape[0], down.shape[2]
+        assert 2 <= self.n_experts <= 64
+        self.mlp = nn.Module()
+        self.mlp.router = RouterLayer(router)
+        self.mlp.experts = experts      # the module that owns the two stacked parameters
+        self._bank = _ExpertTensors(gate_up, down)
+        self.forced_routing = None
+
+    @property
+    def _router(self):
+        return self.mlp.router
+
+    @property
+    def _experts(self):
+        return self._bank
 
 
 class WrappedLMHead(LMHead):

@@ -259,6 +259,49 @@ def test_hugging_face_llama_stages_are_recognised_on_the_models_own_layers():
         _close(x, model(ids).logits, "blocks against LlamaForCausalLM")
 
 
+def test_hugging_face_mixtral_stages_are_recognised_on_the_models_own_parameters():
+    """Mixtral keeps its experts as two stacked parameters (gate|up [E, 2 f, d] and down [E, d, f]) and
+    exports its sparse block as a soup of index arithmetic; the stage is recognised by what the branch
+    reads (an RMSNorm, a router weight, the two stacked parameters, a top-2, a SiLU) and checked
+    numerically against the stage itself, with the attention half handled as Llama's."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.MixtralConfig(hidden_size=256, intermediate_size=256, num_hidden_layers=2,
+                                     num_attention_heads=4, num_key_value_heads=2, vocab_size=500,
+                                     max_position_embeddings=64, use_cache=False, tie_word_embeddings=False,
+                                     num_local_experts=8, num_experts_per_tok=2, attention_dropout=0.0,
+                                     sliding_window=None, router_jitter_noise=0.0)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.MixtralForCausalLM(cfg)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() == 3:
+                p.normal_(std=0.05)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"model.layers.1": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding", "WrappedMoELayer"], ["WrappedMoELayer", "WrappedLMHead"]]
+    layer, hf = blocks[1][0], model.model.layers[1]
+    assert layer._experts.gate_up is hf.mlp.experts.gate_up_proj and layer._experts.down is hf.mlp.experts.down_proj
+    assert layer._router.weight is hf.mlp.gate.weight and layer.self_attn.q_proj is hf.self_attn.q_proj
+    assert (layer.n_experts, layer.ffn, layer.n_heads, layer.n_kv_heads) == (8, 256, 4, 2)
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against MixtralForCausalLM")
+    # a block that picks another number of experts per token is left to autograd, with the reason
+    cfg.num_experts_per_tok = 3
+    other = transformers.MixtralForCausalLM(cfg)
+    pipe = pp.pipeline(other, mb_args=(ids,), split_spec={"model.layers.1": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None and "two experts" in why[0]
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true

@@ -1271,6 +1271,77 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     _exported_model_against_the_oracle(model, Logits, 1000, 128, split, scale_like=_qkv_group)
 
 
+def test_hugging_face_mixtral_runs_natively_and_matches_the_oracle():
+    """Mixtral from the ``transformers`` package: experts stacked in two parameters per layer, the
+    sparse block recognised from what it reads.  The oracle is the fp32 copy of the model, pipelined and
+    recognised the same way on the host (those blocks equal the library's forward: a host test), so that
+    it can be given the expert selection of the bf16 run; that the selection is the top-2 of the run's own
+    router logits is checked here."""
+    T = pytest.importorskip("transformers")
+    import torch.nn as nn
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    M, mb, S, vocab, L, E = 4, 2, 128, 1000, 4, 8
+    cfg = T.MixtralConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=L, num_attention_heads=4,
+                          num_key_value_heads=2, vocab_size=vocab, max_position_embeddings=S, use_cache=False,
+                          tie_word_embeddings=False, num_local_experts=E, num_experts_per_tok=2,
+                          attention_dropout=0.0, sliding_window=None, router_jitter_noise=0.0)
+    cfg._attn_implementation = "sdpa"
+    cfg._experts_implementation = "batched_mm"    # (the grouped product looks at tensor addresses in bf16)
+    torch.manual_seed(0)
+    model = T.MixtralForCausalLM(cfg)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("mlp.gate.weight"):
+                p.mul_(10)                           # decisive routing: few near-ties
+    model = model.to(torch.bfloat16)
+    ref = copy.deepcopy(model).float()
+    ids = torch.randint(0, vocab, (mb * M, S))
+    target = torch.randint(0, vocab, (mb * M, S))
+    split = {f"model.layers.{L // 2}": pp.SplitPoint.BEGINNING}
+    pipe = pp.pipeline(model, mb_args=(ids[:mb],), split_spec=split)
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert all(st.is_native for st in stages), [st.eager_reason for st in stages]
+    sched = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    losses = []
+    out = sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    torch.cuda.synchronize()
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    ref_pipe = pp.pipeline(ref, mb_args=(ids[:mb],), split_spec=split)
+    ref_blocks = [lower_stage_module(ref_pipe.get_stage_module(i)) for i in range(2)]
+    for s, st in enumerate(stages):
+        layers = [b for b in ref_blocks[s] if type(b).__name__ == "WrappedMoELayer"]
+        assert len(layers) == L // 2
+        for layer in layers:
+            layer.forced_routing = []
+        for m in range(M):
+            acts = st.saved_activations(m)
+            idx = [v for k, v in acts.items() if k.endswith("topk_idx")]
+            logits = [v for k, v in acts.items() if k.endswith("router_logits")]
+            assert len(idx) == len(layers)
+            for j, layer in enumerate(layers):
+                want, _ = OO.moe_route_top2(logits[j][:, :E].float().cpu())
+                assert torch.equal(idx[j].cpu().long(), want)
+                layer.forced_routing.append(idx[j].cpu().long())
+    ref_out, ref_losses = OP.step([nn.Sequential(*bl) for bl in ref_blocks], ids, target, M, _ce)
+    assert_close_rel(out, ref_out, BF16_TOL, "merged logits")
+    for a, b in zip(losses, ref_losses):
+        assert_close_rel(a.reshape(1), b.reshape(1), BF16_TOL, "loss")
+    named = dict(model.named_parameters())
+    ref_named = dict(ref.named_parameters())
+    worst = 0.0
+    for name, rp in ref_named.items():
+        assert rp.grad is not None, name
+        group = _qkv_group(name)
+        err = max_rel(named[name].main_grad, rp.grad)
+        if group:
+            scale = max(ref_named[n].grad.abs().max().item() for n in list(group) + [name])
+            err = (named[name].main_grad.cpu() - rp.grad).abs().max().item() / scale
+        worst = max(worst, err)
+        assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+    note(f"Hugging Face Mixtral, 1F1B: worst grad error {worst:.3e}")
+
+
 def test_outputs_merged_while_the_step_runs_are_the_merge_at_the_end(monkeypatch):
     """The schedule copies each microbatch output of the last stage into the merged result as soon as
     its forward pass is issued (a side stream).  The result must be bit for bit what merging after the
