@@ -12,6 +12,7 @@ stage ``i`` is ``pipe.split_gm.submod_i`` and its parameters keep their original
 """
 from __future__ import annotations
 
+import copy
 import logging
 import operator
 from dataclasses import dataclass
@@ -215,10 +216,13 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
     for name, m in mod.named_modules():
         if not name or next(m.children(), None) is not None:
             continue
-        if isinstance(m, _REROLLED_TYPES):
-            leaves[name] = (m, False)
+        base = next((t for t in _REROLLED_TYPES if isinstance(m, t)), None)
+        if base is not None:
+            # a subclass with a forward of its own (a position table that shifts its indices, say) is
+            # put back only if that forward is what the exported nodes compute
+            leaves[name] = (m, type(m).forward is not base.forward, base)
         elif in_out_linear_like(m) or activation_like(m) is not None or rms_norm_like(m) is not None:
-            leaves[name] = (m, True)
+            leaves[name] = (m, True, None)
     calls: Dict[Tuple[str, str], List[fx.Node]] = {}
     for n in graph.nodes:
         stack = n.meta.get("nn_module_stack") if n.op == "call_function" else None
@@ -228,7 +232,7 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
         if entry[0] in leaves:
             calls.setdefault((key, entry[0]), []).append(n)
     for (_key, fqn), nodes in calls.items():
-        layer, verify = leaves[fqn]
+        layer, verify, base = leaves[fqn]
         inside = set(nodes)
         external, own = [], []
         for n in nodes:
@@ -245,22 +249,35 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
         src, res = external[0], results[0]
         if verify:
             fake = src.meta.get("val")
-            try:
-                x = torch.randn(tuple(int(d) for d in fake.shape), dtype=fake.dtype)
-                env = {src: x}
-                env.update({a: _attr(gm, a.target) for a in own})
-                with torch.no_grad():
-                    for n in nodes:
-                        env[n] = n.target(*fx.node.map_arg(n.args, lambda a: env[a]),
-                                          **fx.node.map_arg(n.kwargs, lambda a: env[a]))
-                    want, got = env[res], layer(x)
-                same = got.shape == want.shape and bool((got.float() - want.float()).abs().max()
-                                                        <= 1e-5 + 2e-2 * want.float().abs().max()
-                                                        * (want.dtype != torch.float32))
-            except Exception:
-                same = False
-            if not same:
-                continue
+
+            def same_as(forward) -> bool:
+                try:
+                    shape = tuple(int(d) for d in fake.shape)
+                    if fake.dtype.is_floating_point:
+                        x = torch.randn(shape, dtype=fake.dtype)
+                    else:       # indices into a table: the lower half of its rows
+                        x = torch.randint(0, max(1, getattr(layer, "num_embeddings", 2) // 2), shape, dtype=fake.dtype)
+                    env = {src: x}
+                    env.update({a: _attr(gm, a.target) for a in own})
+                    with torch.no_grad():
+                        for n in nodes:
+                            env[n] = n.target(*fx.node.map_arg(n.args, lambda a: env[a]),
+                                              **fx.node.map_arg(n.kwargs, lambda a: env[a]))
+                        want, got = env[res], forward(x)
+                    return got.shape == want.shape and bool((got.float() - want.float()).abs().max()
+                                                            <= 1e-5 + 2e-2 * want.float().abs().max()
+                                                            * (want.dtype != torch.float32))
+                except Exception:
+                    return False
+
+            if not same_as(layer):
+                # the nodes may still be the base layer's arithmetic on these parameters (the rest of the
+                # subclass's forward was folded into a constant or lies outside): then the base layer's
+                # view of the same parameter objects goes into the graph
+                if base is None or not same_as(lambda x: base.forward(layer, x)):
+                    continue
+                layer = copy.copy(layer)
+                layer.__class__ = base
         gm.add_submodule(fqn, layer)
         with graph.inserting_after(nodes[-1]):
             call = graph.call_module(fqn, (src,))

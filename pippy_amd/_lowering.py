@@ -306,7 +306,9 @@ def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
     if given.get("dropout_p", 0.0) not in (0, 0.0) or given.get("enable_gqa"):
         raise NotLowerable("scaled_dot_product_attention with dropout or grouped queries")
     scale = given.get("scale")
-    if scale is not None and not any(abs(float(scale) - d ** -0.5) < 1e-6 for d in head_dims):
+    # (a scale of 1 is what a model passes that has scaled its queries itself: whether it scaled them by
+    # the default factor shows when the recognised blocks are compared with the stage)
+    if scale is not None and float(scale) != 1.0 and not any(abs(float(scale) - d ** -0.5) < 1e-6 for d in head_dims):
         raise NotLowerable(f"scaled_dot_product_attention with the scale {scale}, which is not the default for "
                            f"a head size of {' or '.join(map(str, head_dims))}")
     causal = bool(given.get("is_causal", False))
@@ -448,8 +450,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     if kinds == ["Linear", "act", "Linear"]:
         (_, fc1), (an, am), (_, fc2) = mods
         act = _activation_of(an, root)
-        if act not in ("gelu_tanh", "gelu_erf"):
-            raise NotLowerable(f"feed-forward activation '{an.format_node()}' (tanh- and erf-GELU are built)")
+        if act not in ("gelu_tanh", "gelu_erf", "relu"):
+            raise NotLowerable(f"feed-forward activation '{an.format_node()}' (tanh-GELU, erf-GELU and ReLU are built)")
         if fc2.in_features != fc1.out_features or fc2.out_features != fc1.in_features:
             raise NotLowerable("feed-forward projections do not map d -> f -> d")
         return ("mlp", ln, fc1, fc2, act)
@@ -457,8 +459,15 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
 
 
 def _skip_identities(root: nn.Module, stream: fx.Node) -> fx.Node:
-    """Steps over layers that do nothing (a dropout with p = 0 or in eval mode) behind ``stream``."""
-    while len(stream.users) == 1 and _activation_of(next(iter(stream.users)), root) == "identity":
+    """Steps over what does nothing behind ``stream``: a dropout with p = 0 or in eval mode, a re-view of
+    the rows ([batch, seq, d] as [batch * seq, d] and back; the blocks work on rows either way, and the
+    comparison with the stage checks the final shape)."""
+    def passes(user: fx.Node) -> bool:
+        if _activation_of(user, root) == "identity":
+            return True
+        return user.op == "call_function" and user.target in (_ATEN.view.default, _ATEN.reshape.default,
+                                                              _ATEN._unsafe_view.default, _ATEN.alias.default)
+    while len(stream.users) == 1 and passes(next(iter(stream.users))):
         stream = next(iter(stream.users))
     return stream
 
@@ -496,7 +505,15 @@ def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream:
         position = root.get_submodule(emb[1].target)
         if isinstance(norm, nn.LayerNorm):      # an encoder front without token types
             return [WrappedEncoderEmbedding(wte, position, None, norm)], _skip_identities(root, norm_node)
-        return [WrappedTokenEmbedding(wte, position)], _skip_identities(root, joins[0])
+        # positions 0 .. S-1 may read the table from a later row on (a constant index of k .. k+S-1)
+        index = _constant_of(root, emb[1].all_input_nodes[0]) if len(emb[1].all_input_nodes) == 1 else None
+        offset = 0
+        if index is not None and index.dtype == torch.int64 and index.numel():
+            rows = index.reshape(-1, index.shape[-1])
+            offset = int(rows[0, 0])
+            if offset < 0 or not bool((rows == torch.arange(rows.shape[1]) + offset).all()):
+                raise NotLowerable("a position table that is not read at consecutive positions")
+        return [WrappedTokenEmbedding(wte, position, offset)], _skip_identities(root, joins[0])
     # three tables: which is which shows in their constant index tensors (all zero: token type 0; 0 .. S-1: positions)
     roles = {}
     for e in emb[1:]:

@@ -214,7 +214,7 @@ def layernorm_backward(b: "P.Builder", name: str, ln: nn.LayerNorm, x2d, mean, r
 
 _ACT_EPI = {None: N.EPI_BIAS, "relu": N.EPI_BIAS_RELU, "gelu_erf": N.EPI_BIAS_GELU_ERF,
             "gelu_tanh": N.EPI_BIAS_GELU_TANH}
-_ACT_DEPI = {"gelu_erf": N.EPI_DGELU_ERF, "gelu_tanh": N.EPI_DGELU_TANH}
+_ACT_DEPI = {"gelu_erf": N.EPI_DGELU_ERF, "gelu_tanh": N.EPI_DGELU_TANH, "relu": N.EPI_DRELU}
 _ACT_KIND = {"relu": N.ACT_RELU, "gelu_erf": N.ACT_GELU_ERF, "gelu_tanh": N.ACT_GELU_TANH}
 
 
@@ -312,11 +312,13 @@ class TokenEmbedding(NativeBlock):
             self.wpe = nn.Embedding(max_seq, dim, dtype=dtype)
             nn.init.normal_(self.wpe.weight, std=init_std)
 
+    position_offset = 0      # position p reads row p + position_offset of the table (OPT keeps two spare rows)
+
     def forward(self, ids):
         if self.wpe is None:
             return self.wte(ids)
         S = ids.shape[-1]
-        pos = torch.arange(S, device=ids.device)
+        pos = torch.arange(S, device=ids.device) + self.position_offset
         return self.wte(ids) + self.wpe(pos)
 
     def _pp_direct_acc_params(self):
@@ -328,9 +330,10 @@ class TokenEmbedding(NativeBlock):
                                f"{ids.dtype} {tuple(ids.shape)}")
         Bn, S = ids.shape
         wte = b.weight(self.wte.weight)
-        wpe = b.weight(self.wpe.weight) if self.wpe is not None else None
+        first = self.position_offset
+        wpe = b.weight(self.wpe.weight)[first:] if self.wpe is not None else None
         if wpe is not None and S > wpe.shape[0]:
-            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
+            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]} rows from row {first})")
         Cc = wte.shape[1]
         y = b.act("y", (Bn, S, Cc))
         b.f(P.op_embed_fwd(ids, wte, wpe, y.view(Bn * S, Cc), S))
@@ -344,7 +347,8 @@ class TokenEmbedding(NativeBlock):
             b.w(P.op_fill(acc_wte), tag="fill")
             if acc_wpe is not None:
                 b.w(P.op_fill(acc_wpe), tag="fill")
-            b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+            b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe[first:] if acc_wpe is not None else None,
+                               S, round_bf16=not b.fused_accumulate))
             _zero_padding_row(b, self.wte, acc_wte)
             return None
 
@@ -421,7 +425,7 @@ class TransformerLayer(NativeBlock):
     def __init__(self, dim: int, n_heads: int, ffn: int, *, causal: bool = True, pre_ln: bool = True,
                  activation: str = "gelu_tanh", eps: float = 1e-5, dtype=torch.bfloat16, init_std=0.02):
         super().__init__()
-        assert dim % n_heads == 0 and activation in ("gelu_tanh", "gelu_erf")
+        assert dim % n_heads == 0 and activation in ("gelu_tanh", "gelu_erf", "relu")
         self.dim, self.n_heads, self.ffn = dim, n_heads, ffn
         self.causal, self.pre_ln, self.activation = causal, pre_ln, activation
         self.ln_1 = nn.LayerNorm(dim, eps=eps, dtype=dtype)
@@ -499,7 +503,11 @@ class TransformerLayer(NativeBlock):
         att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
         x2, _ = lower_linear(b, "x2", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         ln2, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, x2)
-        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, ln2, epilogue=act, save_pre=b.training)
+        # (the derivative of a ReLU is read off its output; a GELU's needs the value before it)
+        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, ln2, epilogue=act,
+                                save_pre=b.training and self.activation != "relu")
+        if self.activation == "relu":
+            h_pre = h
         y, _ = lower_linear(b, "y", self.mlp.c_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2)
 
         def bwd(dy, need_dx, dx_out):
@@ -528,7 +536,10 @@ class TransformerLayer(NativeBlock):
         att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
         a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         x1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, a)
-        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act, save_pre=b.training)
+        h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act,
+                                save_pre=b.training and self.activation != "relu")
+        if self.activation == "relu":
+            h_pre = h
         f, _ = lower_linear(b, "f", self.mlp.c_proj, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x1)
         y, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, f)
 
@@ -1228,10 +1239,11 @@ def activation_like(m: nn.Module) -> Optional[str]:
 
 
 class WrappedTokenEmbedding(TokenEmbedding):
-    def __init__(self, wte: nn.Embedding, wpe: Optional[nn.Embedding]):
+    def __init__(self, wte: nn.Embedding, wpe: Optional[nn.Embedding], position_offset: int = 0):
         NativeBlock.__init__(self)
         self.wte = wte
         self.wpe = wpe
+        self.position_offset = position_offset
 
 
 class WrappedEncoderEmbedding(EncoderEmbedding):

@@ -238,3 +238,41 @@ def test_what_the_kernels_cannot_take_keeps_a_recognised_stage_with_torch():
     # any sequence length: the layers pad to a multiple of 64 by themselves
     stage = pp.pipeline(model, 1, (ids[:, :48],), split_spec={"h.2": pp.SplitPoint.BEGINNING}).get_stage_module(1)
     assert lower_stage_module(stage, why, for_kernels=True) is not None
+
+
+def test_a_layer_subclass_with_a_forward_of_its_own_is_not_put_back_blindly():
+    """OPT's position table is an ``nn.Embedding`` subclass whose forward shifts its indices by two.
+    After constant folding, the exported nodes of that call are a plain look-up at the shifted constant:
+    calling the subclass there would shift twice.  The look-up goes back as the base layer's view of the
+    same parameter, the stage lowers with the table read from row 2 on, and a ReLU feed-forward lowers."""
+    from pippy_amd._lowering import lower_stage_module
+    model = _lib_gpt()
+
+    class Shifted(nn.Embedding):
+        def forward(self, pos):
+            return super().forward(pos + 2)
+
+    class Relu(nn.Module):
+        def forward(self, x):
+            return torch.relu(x)
+
+    table = Shifted(66, 128)
+    model.wpe = table
+    for blk in model.h:
+        blk.mlp.act = Relu()
+    ids = torch.randint(0, 500, (2, 32))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    sm = pipe.get_stage_module(0)
+    assert type(sm.get_submodule("wpe")) is nn.Embedding and sm.get_submodule("wpe").weight is table.weight
+    why = []
+    blocks = lower_stage_module(sm, why)
+    assert blocks is not None, why
+    assert blocks[0].position_offset == 2 and blocks[0].wpe.weight is table.weight
+    assert blocks[1].activation == "relu"
+    x = ids
+    with torch.no_grad():
+        for b in blocks:
+            x = b(x)
+        torch.testing.assert_close(x, sm(ids), rtol=1e-4, atol=1e-4)

@@ -302,6 +302,38 @@ def test_hugging_face_mixtral_stages_are_recognised_on_the_models_own_parameters
     assert lower_stage_module(pipe.get_stage_module(1), why) is None and "two experts" in why[0]
 
 
+def test_hugging_face_opt_stages_are_recognised_on_the_models_own_layers():
+    """The model of the reference's examples/huggingface/pippy_opt.py, in eval mode as there: queries
+    scaled by the model before an attention call with scale 1, a position table that is a subclass of
+    nn.Embedding reading from row 2 on, ReLU feed-forward, the residual stream re-viewed as rows inside
+    each layer."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.OPTConfig(hidden_size=128, ffn_dim=256, num_hidden_layers=2, num_attention_heads=2,
+                                 max_position_embeddings=64, dropout=0.0, layerdrop=0.0, use_cache=False,
+                                 vocab_size=500, tie_word_embeddings=False)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.OPTForCausalLM(cfg).eval()
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"model.decoder.layers.1": pp.SplitPoint.BEGINNING})
+    got = pipe(ids)
+    _close(got[0] if isinstance(got, (tuple, list)) else got, model(ids).logits, "Pipe against the model")
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding", "WrappedTransformerLayer"], ["WrappedTransformerLayer", "WrappedLMHead"]]
+    front, layer, hf = blocks[0][0], blocks[1][0], model.model.decoder.layers[1]
+    assert front.position_offset == 2 and front.wpe.weight is model.model.decoder.embed_positions.weight
+    assert layer.activation == "relu" and layer.causal and layer.pre_ln and layer.mlp.c_fc is hf.fc1
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against OPTForCausalLM")
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true
