@@ -153,7 +153,7 @@ def _fold_constants(gm: fx.GraphModule) -> None:
             except AttributeError:
                 continue
             written = any(u.op == "call_function" and getattr(getattr(u.target, "_schema", None), "is_mutable", False)
-                          for u in n.users)
+                          and u.target is not torch.ops.aten.detach_.default for u in n.users)
             if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) and not written:
                 value[n] = obj
             elif isinstance(obj, fx.GraphModule):
@@ -168,6 +168,9 @@ def _fold_constants(gm: fx.GraphModule) -> None:
                                         **fx.node.map_arg(n.kwargs, lambda a: value[a]))
             except Exception:
                 continue
+        elif n.op == "call_function" and n.target is torch.ops.aten.detach_.default:
+            if n.args[0] in value:      # (in place, but it changes nothing about a constant)
+                value[n] = value[n.args[0]]
         elif n.op == "call_function" and isinstance(n.target, torch._ops.OpOverload):
             if n.target.namespace != "aten" or torch.Tag.nondeterministic_seeded in n.target.tags \
                     or n.target._schema.is_mutable or any(a not in value for a in n.all_input_nodes):
@@ -308,6 +311,15 @@ def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Option
     _drop_noop_casts(gm)
     _fold_constants(gm)
     _reroll_leaf_layers(mod, gm)
+    # what nothing reads (a pooling head whose result the model drops, say) would otherwise give the last
+    # layer a second reader; split markers and in-place operators stay
+    for n in reversed(list(graph.nodes)):
+        if n.users or n.op not in ("call_function", "call_module", "get_attr"):
+            continue
+        if n.op == "call_function" and (n.target is torch.ops.pippy_amd._pipe_split.default or
+                                        getattr(getattr(n.target, "_schema", None), "is_mutable", False)):
+            continue
+        graph.erase_node(n)
     for n in list(graph.nodes):
         if n.op == "call_function" and n.target is torch.ops.pippy_amd._pipe_split.default:
             n.target = pipe_split

@@ -231,7 +231,7 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 # not parsed but checked: the torch statement of the recognised blocks must reproduce the stage's own
 # forward on a random input (fp32, on the host), otherwise the stage stays with torch autograd.
 _SDPA = (F.scaled_dot_product_attention, _ATEN.scaled_dot_product_attention.default)
-_ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor)
+_ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor, _ATEN.add_.Tensor)
 _ACT_FNS = (F.gelu, F.relu, torch.relu, F.silu, _ATEN.gelu.default, _ATEN.relu.default, _ATEN.silu.default)
 
 
@@ -241,7 +241,8 @@ def _is_add(n: fx.Node) -> bool:
 
 def _branch_layers(y: fx.Node, stream: fx.Node, order: dict, state: bool = False) -> List[fx.Node]:
     """The layer and function nodes that ``y`` is computed from, back to ``stream`` (in graph order);
-    with ``state`` also the ``get_attr`` nodes (parameters the model's own forward reads) and top-k nodes."""
+    with ``state`` also the ``get_attr`` nodes (parameters the model's own forward reads), top-k and
+    softmax nodes."""
     seen, stack, found = set(), [y], []
     while stack:
         n = stack.pop()
@@ -253,7 +254,8 @@ def _branch_layers(y: fx.Node, stream: fx.Node, order: dict, state: bool = False
         if n.op == "call_module" or (n.op == "call_function" and n.target in _SDPA + _ACT_FNS) \
                 or _is_add(n):
             found.append(n)
-        elif state and (n.op == "get_attr" or (n.op == "call_function" and n.target is _ATEN.topk.default)):
+        elif state and (n.op == "get_attr" or (n.op == "call_function" and
+                                               n.target in (_ATEN.topk.default,) + _SOFTMAX)):
             found.append(n)
         stack.extend(a for a in n.all_input_nodes)
     return sorted(found, key=order.get)
@@ -273,8 +275,8 @@ def _constant_of(root: nn.Module, node) -> Optional[torch.Tensor]:
 
 
 def _is_causal_mask(mask: torch.Tensor) -> bool:
-    """A boolean (keep) or additive (0 / -inf or lowest) mask, broadcast over batch and heads, that lets
-    query i see exactly the keys 0..i."""
+    """A boolean (keep) or additive (0 / a huge negative number) mask, broadcast over batch and heads, that
+    lets query i see exactly the keys 0..i."""
     if mask.dim() < 2 or mask.shape[-1] != mask.shape[-2]:
         return False
     S = mask.shape[-1]
@@ -285,10 +287,11 @@ def _is_causal_mask(mask: torch.Tensor) -> bool:
     keep = torch.ones(S, S, dtype=torch.bool, device=m.device).tril()
     if m.dtype == torch.bool:
         return bool((m == keep).all())
-    lowest = torch.finfo(m.dtype).min if m.dtype.is_floating_point else None
-    if lowest is None:
+    if not m.dtype.is_floating_point:
         return False
-    masked = (m == float("-inf")) | (m <= lowest)
+    # -inf, the lowest value of some dtype (possibly of a narrower one than the tensor has now), -1e9,
+    # -10000: addends under which exp() is zero in any precision
+    masked = m <= -1e4
     return bool((masked == ~keep).all()) and bool((m[keep] == 0).all())
 
 
@@ -297,30 +300,101 @@ def _is_full_mask(mask: torch.Tensor) -> bool:
     return bool(mask.all()) if mask.dtype == torch.bool else bool((mask == 0).all())
 
 
-def _sdpa_is_causal(root: nn.Module, sd: fx.Node, head_dims=(64, 128)) -> bool:
-    """Reads the arguments of a scaled_dot_product_attention node; raises unless it is plain softmax
-    attention, causal or full, at the default scale."""
+_SOFTMAX = (_ATEN._softmax.default, _ATEN.softmax.int)
+_MATMULS = (_ATEN.matmul.default, _ATEN.bmm.default)
+_PASS_THROUGH = _ATEN_VIEWS + (_ATEN.transpose.int, _ATEN.permute.default, _ATEN.expand.default,
+                               _ATEN._to_copy.default, _ATEN.to.dtype, _ATEN.to.dtype_layout,
+                               _ATEN.unsqueeze.default, _ATEN.squeeze.dim, _ATEN.dropout.default)
+
+
+def _scalar_of(root: nn.Module, arg) -> Optional[float]:
+    """A Python number, or the value of a one-element constant tensor of the stage."""
+    if isinstance(arg, (int, float)) and not isinstance(arg, bool):
+        return float(arg)
+    value = _constant_of(root, arg)
+    if value is not None and value.numel() == 1 and (value.is_floating_point() or not value.dtype == torch.bool):
+        return float(value)
+    return None
+
+
+def _constant_factors_back(root: nn.Module, node):
+    """Walks from ``node`` towards its producer over views, casts and products / quotients with constants.
+    Returns (the first node that is none of those, the accumulated factor)."""
+    factor = 1.0
+    while isinstance(node, fx.Node) and node.op == "call_function":
+        if node.target in _PASS_THROUGH:
+            node = node.args[0]
+        elif node.target in (_ATEN.mul.Tensor, _ATEN.mul.Scalar, _ATEN.div.Tensor, _ATEN.div.Scalar) \
+                and _scalar_of(root, node.args[1]) is not None:
+            c = _scalar_of(root, node.args[1])
+            factor = factor * c if "mul" in str(node.target) else factor / c
+            node = node.args[0]
+        else:
+            break
+    return node, factor
+
+
+def _mask_is_causal(root: nn.Module, mask, causal: bool, inverted: bool = False) -> bool:
+    """Folds a constant mask into ``causal``; raises for a mask that is neither causal nor empty."""
+    value = _constant_of(root, mask)
+    if value is not None and inverted and value.dtype == torch.bool:
+        value = ~value
+    if value is not None and _is_full_mask(value):
+        return causal         # a mask that masks nothing (an encoder without padding)
+    if value is None or not _is_causal_mask(value):
+        raise NotLowerable("attention with a mask tensor other than a constant causal mask")
+    return True               # (a model may apply its causal mask twice, as a selection and as an addend)
+
+
+def _attention_form(root: nn.Module, node: fx.Node):
+    """(causal, (scale, factor)) of an attention, read off its scaled_dot_product_attention node or — for
+    a model that spells attention out as softmax(q k^T * c + mask) v — off its softmax node.  ``scale`` is
+    the explicit factor on the scores (None: the default 1 / sqrt(head size)), ``factor`` what the model
+    multiplied queries and keys with beforehand.  Raises unless it is plain softmax attention, causal or
+    full; whatever this reading misses shows when the recognised blocks are compared with the stage."""
+    if node.target in _SOFTMAX:
+        causal, factor = False, 1.0
+        x = node.args[0]
+        while isinstance(x, fx.Node) and x.op == "call_function" and x.target not in _MATMULS:
+            before, c = _constant_factors_back(root, x)
+            if before is not x:
+                x, factor = before, factor * c
+            elif x.target is _ATEN.add.Tensor:
+                causal = _mask_is_causal(root, x.args[1], causal)
+                x = x.args[0]
+            elif x.target is _ATEN.where.self:            # where(keep, scores, fill)
+                causal = _mask_is_causal(root, x.args[0], causal)
+                x = x.args[1]
+            elif x.target in (_ATEN.masked_fill.Scalar, _ATEN.masked_fill.Tensor):   # fill where the mask is set
+                causal = _mask_is_causal(root, x.args[1], causal, inverted=True)
+                x = x.args[0]
+            else:
+                raise NotLowerable(f"'{x.format_node()}' between the score product and the softmax")
+        if not (isinstance(x, fx.Node) and x.op == "call_function" and x.target in _MATMULS):
+            raise NotLowerable("a softmax that does not follow a product of queries and keys")
+        for operand in x.args[:2]:
+            factor *= _constant_factors_back(root, operand)[1]
+        return causal, (1.0, factor)
     names = ("query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale", "enable_gqa")
-    given = dict(zip(names, sd.args))
-    given.update(sd.kwargs)
+    given = dict(zip(names, node.args))
+    given.update(node.kwargs)
     if given.get("dropout_p", 0.0) not in (0, 0.0) or given.get("enable_gqa"):
         raise NotLowerable("scaled_dot_product_attention with dropout or grouped queries")
     scale = given.get("scale")
-    # (a scale of 1 is what a model passes that has scaled its queries itself: whether it scaled them by
-    # the default factor shows when the recognised blocks are compared with the stage)
-    if scale is not None and float(scale) != 1.0 and not any(abs(float(scale) - d ** -0.5) < 1e-6 for d in head_dims):
-        raise NotLowerable(f"scaled_dot_product_attention with the scale {scale}, which is not the default for "
-                           f"a head size of {' or '.join(map(str, head_dims))}")
+    factor = 1.0
+    if node.target in (_ATEN.scaled_dot_product_attention.default,):
+        factor = _constant_factors_back(root, given["query"])[1] * _constant_factors_back(root, given["key"])[1]
     causal = bool(given.get("is_causal", False))
-    mask = given.get("attn_mask")
-    if mask is not None:
-        value = _constant_of(root, mask)
-        if value is not None and _is_full_mask(value):
-            return causal     # a mask that masks nothing (an encoder without padding)
-        if value is None or causal or not _is_causal_mask(value):
-            raise NotLowerable("scaled_dot_product_attention with a mask tensor other than a constant causal mask")
-        causal = True
-    return causal
+    if given.get("attn_mask") is not None:
+        causal = _mask_is_causal(root, given["attn_mask"], causal)
+    return causal, (None if scale is None else float(scale), factor)
+
+
+def _score_factor(form, D: int) -> Optional[float]:
+    """The factor on the scores for head size ``D``; None when it is the default 1 / sqrt(D)."""
+    scale, factor = form
+    total = (D ** -0.5 if scale is None else scale) * factor
+    return None if abs(total - D ** -0.5) <= 1e-6 * D ** -0.5 else total
 
 
 def _classify_expert_branch(root: nn.Module, norm, state: List[fx.Node]):
@@ -364,10 +438,13 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     (ln is None when the branch does not start with a LayerNorm; qkv is one fused layer or three),
     ("attn_rope", norm, qkv, o) / ("mlp_gated", norm, gate_up, down) for the Llama family (qkv: the
     fused projection or the three separate ones; gate_up: the fused projection or the two separate ones)."""
-    mods, inner_adds, state = [], [], []
+    mods, inner_adds, state, soft = [], [], [], []
     for n in layers:
         if n.op == "get_attr" or (n.op == "call_function" and n.target is _ATEN.topk.default):
             state.append(n)
+            continue
+        if n.op == "call_function" and n.target in _SOFTMAX:
+            soft.append(n)
             continue
         if _activation_of(n, root) == "identity":
             continue
@@ -375,13 +452,15 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             m = root.get_submodule(n.target)
             mods.append((n, _as_linear(m) or _as_rms_norm(m) or m))
         elif _is_add(n):
+            if any(_constant_of(root, a) is not None for a in n.args[:2]):
+                continue             # a constant added on (the mask of an attention that is spelled out)
             inner_adds.append(n)     # rotary embeddings add two products; nothing else may
         else:
             mods.append((n, None))
 
     def kind(n, m):
         if m is None:
-            return "sdpa" if n.target in _SDPA else "act"
+            return "sdpa" if n.target in _SDPA + _SOFTMAX else "act"
         if isinstance(m, (nn.Linear, InOutLinear)):
             return "Linear"
         if isinstance(m, (nn.RMSNorm, RMSNormLike)):
@@ -391,6 +470,10 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
     kinds = [kind(n, m) for n, m in mods]
     if kinds == ["RMSNorm", "act"] and _activation_of(mods[1][0], root) == "silu":
         return _classify_expert_branch(root, mods[0][1], state)
+    if len(soft) == 1 and kinds and set(kinds[1:]) == {"Linear"} and kinds[-1] == "Linear":
+        # attention spelled out (softmax(q k^T) v between the projections): the softmax stands for the call
+        mods.insert(len(mods) - 1, (soft[0], None))
+        kinds.insert(len(kinds) - 1, "sdpa")
     if kinds == ["RMSNorm", "Linear", "Linear", "Linear", "sdpa", "Linear"]:
         (_, norm), (_, q), (_, k), (_, v), (sd, _), (_, o) = mods
         if not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
@@ -398,17 +481,19 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         if k.out_features != v.out_features or q.out_features != o.in_features or q.out_features != q.in_features \
                 or q.out_features % k.out_features:
             raise NotLowerable("query / key / value projections of unexpected widths")
-        if not _sdpa_is_causal(root, sd):
+        causal, form = _attention_form(root, sd)
+        if not causal:
             raise NotLowerable("rotary attention that is not causal")
-        return ("attn_rope", norm, (q, k, v), o)
+        return ("attn_rope", norm, (q, k, v), o, form)
     if kinds == ["RMSNorm", "Linear", "sdpa", "Linear"] and inner_adds:
         (_, norm), (_, qkv), (sd, _), (_, o) = mods       # one fused q|k|v projection under a rotary embedding
         if not all(isinstance(lin, nn.Linear) for lin in (qkv, o)) or o.in_features != o.out_features \
                 or qkv.out_features <= o.in_features or (qkv.out_features - o.in_features) % 2:
             raise NotLowerable("a fused projection in front of rotary attention that is not q|k|v")
-        if not _sdpa_is_causal(root, sd):
+        causal, form = _attention_form(root, sd)
+        if not causal:
             raise NotLowerable("rotary attention that is not causal")
-        return ("attn_rope", norm, qkv, o)
+        return ("attn_rope", norm, qkv, o, form)
     if kinds == ["RMSNorm", "Linear", "act", "Linear", "Linear"] or kinds == ["RMSNorm", "Linear", "Linear", "act", "Linear"]:
         norm, down = mods[0][1], mods[-1][1]
         an = next(n for n, m in mods if kind(n, m) == "act")
@@ -440,13 +525,13 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         (_, qkv), (sd, _), (_, proj) = mods
         if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
             raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection of width 3 d")
-        return ("attn", ln, qkv, proj, _sdpa_is_causal(root, sd))
+        return ("attn", ln, qkv, proj) + _attention_form(root, sd)
     if kinds == ["Linear", "Linear", "Linear", "sdpa", "Linear"]:
         (_, q), (_, k), (_, v), (sd, _), (_, proj) = mods
         if not all(isinstance(lin, nn.Linear) and lin.in_features == lin.out_features == proj.in_features
                    for lin in (q, k, v)):
             raise NotLowerable("separate query / key / value projections that are not d -> d nn.Linear layers")
-        return ("attn", ln, (q, k, v), proj, _sdpa_is_causal(root, sd))
+        return ("attn", ln, (q, k, v), proj) + _attention_form(root, sd)
     if kinds == ["Linear", "act", "Linear"]:
         (_, fc1), (an, am), (_, fc2) = mods
         act = _activation_of(an, root)
@@ -523,8 +608,10 @@ def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream:
                 roles["type"] = e
             elif bool((index.reshape(-1, index.shape[-1]) == torch.arange(index.shape[-1])).all()):
                 roles["position"] = e
-    if len(roles) != 2 or not isinstance(norm, nn.LayerNorm):
-        raise NotLowerable("three embedding tables that are not word + position + token type 0 under a LayerNorm")
+    if len(roles) != 2:
+        raise NotLowerable("three embedding tables that are not word + position + token type 0")
+    if not isinstance(norm, nn.LayerNorm):      # (a pre-LayerNorm encoder normalises inside its layers)
+        norm, norm_node = None, joins[0]
     block = WrappedEncoderEmbedding(wte, root.get_submodule(roles["position"].target),
                                     root.get_submodule(roles["type"].target), norm)
     return [block], _skip_identities(root, norm_node)
@@ -539,18 +626,22 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
     if d % n_heads or d // n_heads not in (64, 128):
         raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
     if feed_forward[0] == "mlp":
-        _, ln1, qkv, proj, causal = attention
+        _, ln1, qkv, proj, causal, form = attention
         _, ln2, fc1, fc2, act = feed_forward
+        scale = _score_factor(form, d // n_heads)
         if (ln1 is None) != (ln2 is None) or (ln1 is None) != (attention_norm is not None) \
                 or (ln2 is None) != (feed_forward_norm is not None):
             raise NotLowerable("a layer that is neither pre-LayerNorm nor post-LayerNorm throughout")
         if ln1 is None:
             return WrappedTransformerLayer(attention_norm, qkv, proj, feed_forward_norm, fc1, fc2, n_heads, causal,
-                                           act, pre_ln=False)
-        return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act)
-    _, norm1, qkv, o = attention
+                                           act, pre_ln=False, attn_scale=scale)
+        return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act, attn_scale=scale)
+    _, norm1, qkv, o, form = attention
     width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
     D = d // n_heads
+    if _score_factor(form, D) is not None:
+        raise NotLowerable(f"rotary attention with the score factor {_score_factor(form, D):.6g} (1 / sqrt(head "
+                           f"size) is built)")
     if width % D or (width // D - n_heads) % 2 or width // D <= n_heads:
         raise NotLowerable("query / key / value projections that are not whole heads")
     if rope is None:
@@ -588,13 +679,16 @@ def _tail_blocks(root: nn.Module, stream: fx.Node, result: fx.Node, after_layers
         m = root.get_submodule(n.target)
         mods.append(_as_linear(m) or _as_rms_norm(m) or m)
     blocks: List[NativeBlock] = []
-    while mods and isinstance(mods[0], LinearAct):
-        blocks.append(mods.pop(0))       # e.g. the transform in front of a masked-language-model head
+    head: List[NativeBlock] = []
     norm_types, linear_types = (nn.LayerNorm, nn.RMSNorm, RMSNormLike), (nn.Linear, InOutLinear)
-    if len(mods) == 2 and isinstance(mods[0], norm_types) and isinstance(mods[1], nn.Linear):
-        return blocks + [WrappedLMHead(mods[0], mods[1])]
-    if len(mods) == 1 and isinstance(mods[0], nn.Linear) and mods[0].bias is None and (after_layers or blocks):
-        return blocks + [WrappedLMHead(None, mods[0])]
+    # the chain ends in a norm and a projection (a language-model head; in front of it there may be the
+    # last norm of a pre-LayerNorm encoder and the transform of a masked-language-model head), or in a
+    # projection without a bias behind nothing but projections with activations
+    if len(mods) >= 2 and isinstance(mods[-2], norm_types) and isinstance(mods[-1], nn.Linear):
+        head, mods = [WrappedLMHead(mods[-2], mods[-1])], mods[:-2]
+    elif mods and isinstance(mods[-1], nn.Linear) and mods[-1].bias is None and (after_layers or len(mods) > 1) \
+            and all(isinstance(m, LinearAct) for m in mods[:-1]):
+        head, mods = [WrappedLMHead(None, mods[-1])], mods[:-1]
     for m in mods:
         if isinstance(m, nn.LayerNorm):
             blocks.append(LayerNormBlock(m))
@@ -606,7 +700,7 @@ def _tail_blocks(root: nn.Module, stream: fx.Node, result: fx.Node, after_layers
             blocks.append(m)
         else:
             raise NotLowerable(f"a {type(m).__name__} after the last residual addition")
-    return blocks
+    return blocks + head
 
 
 def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) -> List[NativeBlock]:

@@ -480,11 +480,13 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
     return op
 
 
-def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None, kv_len=None) -> N.Op:
+def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None, kv_len=None,
+            scale=None) -> N.Op:
+    """``scale``: the factor on the scores (None: 1 / sqrt(head size))."""
     if qkv.shape[1] % 64:
         raise RuntimeError(f"the attention kernels take sequence lengths that are multiples of 64, got "
                            f"{qkv.shape[1]} (stage_modules.lower_attention pads)")
-    d = N.attn_desc(qkv, o, lse, H, causal, None, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
+    d = N.attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
                     kv_len=kv_len)
     op = N.Op()
     op.kind = kind

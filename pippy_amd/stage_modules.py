@@ -136,7 +136,7 @@ def linear_backward(b: "P.Builder", name: str, lin: nn.Linear, x2d: torch.Tensor
 
 
 def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, causal: bool,
-                    n_kv_heads: Optional[int] = None):
+                    n_kv_heads: Optional[int] = None, scale: Optional[float] = None):
     """Emits attention over the q|k|v rows ``qkv`` [Bn * S, W].  Returns the output [Bn * S, H * D] and the
     emitter of the backward, ``d_att -> dqkv`` ([Bn * S, W]).
 
@@ -152,13 +152,15 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
     att = b.act("att", (T, Cc))
     if S % 64 == 0:
         lse = b.act("lse", (Bn, H, S), torch.float32)
-        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal, n_kv_heads=Hkv))
+        b.f(P.op_attn(N.OP_ATTN_FWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal, n_kv_heads=Hkv,
+                      scale=scale))
 
         def backward(d_att):
             dqkv = b.grad("dqkv", (T, W))
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
             b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal,
-                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv))
+                          d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv,
+                          scale=scale))
             return dqkv
 
         return att, backward
@@ -169,7 +171,7 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
     lse = b.act("lse", (Bn, H, Sp), torch.float32)
     qkv_p.zero_()       # once: the launch lists only ever write the real rows
     b.f(P.op_copy_rows(qkv, qkv_p, Bn, S * W * es, S * W * es, Sp * W * es))
-    b.f(P.op_attn(N.OP_ATTN_FWD, qkv_p, att_p, lse, H, causal, n_kv_heads=Hkv, kv_len=S))
+    b.f(P.op_attn(N.OP_ATTN_FWD, qkv_p, att_p, lse, H, causal, n_kv_heads=Hkv, kv_len=S, scale=scale))
     b.f(P.op_copy_rows(att_p, att, Bn, S * Cc * es, Sp * Cc * es, S * Cc * es))
 
     def backward(d_att):
@@ -182,7 +184,7 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
             b.sp.zeroed_once.add(d_att_p.data_ptr())
         b.i(P.op_copy_rows(d_att, d_att_p, Bn, S * Cc * es, S * Cc * es, Sp * Cc * es))
         b.i(P.op_attn(N.OP_ATTN_BWD, qkv_p, att_p, lse, H, causal, d_o=d_att_p, dqkv=dqkv_p, delta=delta,
-                      n_kv_heads=Hkv, kv_len=S))
+                      n_kv_heads=Hkv, kv_len=S, scale=scale))
         b.i(P.op_copy_rows(dqkv_p, dqkv, Bn, S * W * es, Sp * W * es, S * W * es))
         return dqkv
 
@@ -359,7 +361,8 @@ class TokenEmbedding(NativeBlock):
 class EncoderEmbedding(NativeBlock):
     """BERT-style embedding: ``LayerNorm(word[ids] + position[:S] + token_type[0])``.  All tokens
     are of type 0, which is what the encoder computes when no ``token_type_ids`` are passed.  A
-    wrapper around a user's layers may have no token-type table (``token_type_embeddings = None``)."""
+    wrapper around a user's layers may have no token-type table (``token_type_embeddings = None``) or no
+    LayerNorm (``LayerNorm = None``: an encoder that normalises inside its layers)."""
 
     def __init__(self, vocab: int, max_seq: int, dim: int, n_types: int = 2, eps: float = 1e-12,
                  dtype=torch.bfloat16, init_std=0.02):
@@ -378,7 +381,8 @@ class EncoderEmbedding(NativeBlock):
         e = self.word_embeddings(ids).float() + self.position_embeddings(pos).float()
         if self.token_type_embeddings is not None:
             e = e + self.token_type_embeddings.weight[0].float()
-        return self.LayerNorm(e.to(self.word_embeddings.weight.dtype))
+        e = e.to(self.word_embeddings.weight.dtype)
+        return self.LayerNorm(e) if self.LayerNorm is not None else e
 
     def _pp_direct_acc_params(self):
         return [self.word_embeddings.weight, self.position_embeddings.weight]
@@ -396,10 +400,15 @@ class EncoderEmbedding(NativeBlock):
         T = Bn * S
         e = b.act("e", (T, Cc))
         b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0] if wtt is not None else None))
-        y, mean, rstd = lower_layernorm(b, "ln", self.LayerNorm, e)
+        if self.LayerNorm is not None:
+            y, mean, rstd = lower_layernorm(b, "ln", self.LayerNorm, e)
+        else:
+            y = e
 
         def bwd(dy, need_dx, dx_out):
-            de = layernorm_backward(b, "ln", self.LayerNorm, e, mean, rstd, dy.view(T, Cc))
+            de = dy.view(T, Cc)
+            if self.LayerNorm is not None:
+                de = layernorm_backward(b, "ln", self.LayerNorm, e, mean, rstd, de)
             acc_wte = b.grad_acc(self.word_embeddings.weight)
             acc_wpe = b.grad_acc(self.position_embeddings.weight)
             b.w(P.op_fill(acc_wte), tag="fill")
@@ -440,12 +449,14 @@ class TransformerLayer(NativeBlock):
             nn.init.normal_(lin.weight, std=init_std)
             nn.init.zeros_(lin.bias)
 
+    attn_scale = None      # the factor on the attention scores; None: 1 / sqrt(head size)
+
     # torch statement of the layer
     def _attention(self, h):
         Bn, S, Cc = h.shape
         H, D = self.n_heads, Cc // self.n_heads
         q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self._project_qkv(h).split(Cc, dim=-1))
-        o = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal)
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal, scale=self.attn_scale)
         return self.attn.c_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
 
     def forward(self, x):
@@ -500,7 +511,7 @@ class TransformerLayer(NativeBlock):
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         ln1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, x2d)
         qkv = self._lower_qkv(b, ln1)
-        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, scale=self.attn_scale)
         x2, _ = lower_linear(b, "x2", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         ln2, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, x2)
         # (the derivative of a ReLU is read off its output; a GELU's needs the value before it)
@@ -533,7 +544,7 @@ class TransformerLayer(NativeBlock):
         x2d = x.view(T, Cc)
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         qkv = self._lower_qkv(b, x2d)
-        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal)
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, scale=self.attn_scale)
         a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         x1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, a)
         h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act,
@@ -1260,8 +1271,9 @@ class WrappedTransformerLayer(TransformerLayer):
 
     def __init__(self, ln_1: nn.LayerNorm, c_attn, c_proj: nn.Linear, ln_2: nn.LayerNorm,
                  c_fc: nn.Linear, mlp_proj: nn.Linear, n_heads: int, causal: bool, activation: str,
-                 pre_ln: bool = True):
+                 pre_ln: bool = True, attn_scale: Optional[float] = None):
         NativeBlock.__init__(self)
+        self.attn_scale = attn_scale
         self.dim, self.n_heads, self.ffn = c_proj.out_features, n_heads, c_fc.out_features
         self.causal, self.pre_ln, self.activation = causal, pre_ln, activation
         self.ln_1, self.ln_2 = ln_1, ln_2

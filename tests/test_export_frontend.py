@@ -276,3 +276,43 @@ def test_a_layer_subclass_with_a_forward_of_its_own_is_not_put_back_blindly():
         for b in blocks:
             x = b(x)
         torch.testing.assert_close(x, sm(ids), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("factor", ["default", "none", "queries"])
+def test_attention_spelled_out_is_recognised_with_its_mask_and_factor(factor):
+    """A model that writes attention as softmax(q k^T c, masked) v (the non-fused path of many code bases):
+    the softmax stands for the attention call, the constant mask filled in where it is *set* is read as
+    causal, and the factor on the scores — the default, none at all, or one applied to the queries
+    beforehand — becomes the block's ``attn_scale``."""
+    import math
+    import torch.nn.functional as F
+    from pippy_amd._lowering import lower_stage_module
+    model = _lib_gpt()
+
+    def spelled_out(self, x, mask):
+        B, T, C = x.size()
+        D = C // self.n_head
+        q, k, v = (t.view(B, T, self.n_head, D).transpose(1, 2) for t in self.c_attn(x).split(C, dim=2))
+        if factor == "queries":
+            q = q * 0.2
+        att = q @ k.transpose(-2, -1)
+        if factor == "default":
+            att = att / math.sqrt(D)
+        att = att.masked_fill(~mask, float("-inf"))
+        y = F.softmax(att, dim=-1) @ v
+        return self.resid_dropout(self.c_proj(y.transpose(1, 2).reshape(B, T, C)))
+
+    for blk in model.h:
+        blk.attn.forward = spelled_out.__get__(blk.attn)
+    ids = torch.randint(0, 500, (2, 32))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    for i in range(2):
+        sm = pipe.get_stage_module(i)
+        why = []
+        blocks = lower_stage_module(sm, why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2 and all(b.causal for b in layers)
+        want = {"default": None, "none": 1.0, "queries": 0.2}[factor]
+        assert all(b.attn_scale == want if want is None else abs(b.attn_scale - want) < 1e-9 for b in layers)

@@ -588,6 +588,34 @@ def test_attention(causal, B, S, H, D):
 
 
 @pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("scale,D", [(1.0, 64), (0.05, 128), (0.3, 64)])
+def test_attention_with_a_score_factor_of_the_callers(causal, scale, D):
+    """The factor on the scores is an argument (models that scale their queries themselves pass 1, some
+    pass a constant of their own): forward, log-sum-exp and the three gradients against attention with
+    the queries multiplied by scale * sqrt(D) beforehand, which is the same function."""
+    Nn = native()
+    B, S, H = 2, 192, 3
+    torch.manual_seed(int(scale * 100) + D)
+    HD = H * D
+    qkv = (torch.randn(B, S, 3 * HD, device=DEV) * 0.7).to(torch.bfloat16)
+    o = torch.full((B, S, HD), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    Nn.attn_fwd(qkv, o, lse, H, causal, scale=scale)
+    d_o = torch.randn(B, S, HD, device=DEV).to(torch.bfloat16)
+    dqkv = torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    Nn.attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=scale)
+    torch.cuda.synchronize()
+    qr = qkv.float().cpu().requires_grad_(True)
+    factor = torch.cat([torch.full((HD,), scale * math.sqrt(D)), torch.ones(2 * HD)])
+    ref = O.attention_fused_qkv(qr * factor, H, causal)
+    assert_close_rel(o, ref, BF16_TOL, "scaled attention fwd")
+    ref.backward(d_o.float().cpu())
+    for name, sl in (("dq", slice(0, HD)), ("dk", slice(HD, 2 * HD)), ("dv", slice(2 * HD, 3 * HD))):
+        assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"scaled attention {name}")
+
+
+@pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,L,H,Hkv,D", [(2, 100, 2, 2, 64), (1, 40, 3, 3, 64), (2, 193, 2, 1, 128), (1, 330, 4, 2, 64),
                                          (3, 1, 1, 1, 64), (1, 449, 3, 3, 64), (1, 64, 2, 2, 64)])
 def test_attention_over_a_padded_sequence_is_attention_over_the_sequence(causal, B, L, H, Hkv, D):

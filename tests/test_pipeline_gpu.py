@@ -1226,14 +1226,20 @@ def _qkv_group(name):
     return None
 
 
-@pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra", "opt"])
+@pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra", "opt", "gpt2_spelled_out",
+                                    "megatron_bert", "gpt_neo"])
 def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
     value projections), Mistral (Llama layout), Phi-3 (one fused q|k|v and one fused gate|up projection),
     DistilBERT (encoder without token types, its own layer names), ELECTRA (BERT layout with a generator
     head), OPT (the reference's examples/huggingface/pippy_opt.py: queries scaled before an attention
     call with scale 1, a position table read from row 2 on, ReLU feed-forward; exported in eval mode, as
-    the example runs it, since its training-mode layer drop branches on a random number)."""
+    the example runs it, since its training-mode layer drop branches on a random number); and models whose
+    attention is spelled out as softmax(q k^T c + mask) v instead of one call: GPT-2 with the library's
+    "eager" attention, Megatron-BERT (pre-LayerNorm encoder, embeddings without a LayerNorm, a final
+    LayerNorm in front of the head's transform; examples/huggingface/pippy_megatronBert.py) and GPT-Neo
+    (scores without the 1 / sqrt(head size) factor, the causal mask applied twice, projections without
+    biases, "local" layers whose window covers the sequence; examples/huggingface/pippy_gptNeo.py)."""
     T = pytest.importorskip("transformers")
     import torch.nn as nn
     common = dict(vocab_size=1000, tie_word_embeddings=False)
@@ -1259,8 +1265,23 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
                         T.OPTConfig(hidden_size=128, ffn_dim=512, num_hidden_layers=4, num_attention_heads=2,
                                     max_position_embeddings=128, dropout=0.0, layerdrop=0.0, use_cache=False,
                                     **common), "model.decoder.layers.2"),
+        "gpt2_spelled_out": lambda: (T.GPT2LMHeadModel,
+                                     T.GPT2Config(n_layer=4, n_embd=128, n_head=2, n_positions=128, attn_pdrop=0.0,
+                                                  embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False, bos_token_id=0,
+                                                  eos_token_id=0, **common), "transformer.h.2"),
+        "megatron_bert": lambda: (T.MegatronBertForMaskedLM,
+                                  T.MegatronBertConfig(hidden_size=128, intermediate_size=512, num_hidden_layers=4,
+                                                       num_attention_heads=2, max_position_embeddings=128,
+                                                       hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                                                       **common), "bert.encoder.layer.2"),
+        "gpt_neo": lambda: (T.GPTNeoForCausalLM,
+                            T.GPTNeoConfig(hidden_size=128, num_layers=4, num_heads=2, window_size=256,
+                                           attention_types=[[["global", "local"], 2]], max_position_embeddings=128,
+                                           embed_dropout=0.0, attention_dropout=0.0, resid_dropout=0.0,
+                                           use_cache=False, bos_token_id=0, eos_token_id=0, **common),
+                            "transformer.h.2"),
     }[family]()
-    cfg._attn_implementation = "sdpa"
+    cfg._attn_implementation = "eager" if family in ("gpt2_spelled_out", "megatron_bert", "gpt_neo") else "sdpa"
     torch.manual_seed(0)
     model = cls(cfg)
     if family == "opt":
