@@ -370,6 +370,17 @@ int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
  * ---------------------------------------------------------------------------------------- */
 int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe, const void* extra_row, void* y,
                  int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, pp_stream stream);
+/* The same sum with the position row given per token: wpe[pos_ids[t], :] (pos_ids int64 [n_tok], rows of
+ * an [n_pos, C] table; an index out of range reads row 0).  For encoders that count positions over the
+ * tokens that are not padding (the embeddings of the model in examples/huggingface/pippy_camemBert.py). */
+int pp_embed_fwd_at(const int64_t* ids, const int64_t* pos_ids, const void* wte, const void* wpe,
+                    const void* extra_row, void* y, int64_t n_tok, int64_t n_pos, int64_t C, int64_t vocab,
+                    pp_stream stream);
+/* Those positions: out[b, s] = pad where ids[b, s] == pad, else pad + the number of tokens != pad among
+ * ids[b, 0..s]  (ids, out int64 [n_seq, seq]; the position indices that the embeddings of the model in
+ * examples/huggingface/pippy_camemBert.py compute with ne / cumsum / mul / add). */
+int pp_position_ids_from_padding(const int64_t* ids, int64_t* out, int64_t n_seq, int64_t seq, int64_t pad,
+                                 pp_stream stream);
 /* Gradient of the lookup, added to fp32 accumulators (F.embedding's backward reached through
  * pippy/_backward.py:67-69, followed by the accumulation into the parameter's gradient):
  *   d_wte[v, :] += g[v, :],  g[v, :] = sum of dy[t, :] over the tokens t with ids[t] == v, formed in
@@ -404,7 +415,7 @@ enum pp_op_kind {
     PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16,
     PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
     PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
-    PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27
+    PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27, PP_OP_POSITION_IDS = 28
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -417,7 +428,9 @@ enum pp_op_kind {
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
  *                 | j: causal kv_group kv_len
- *   EMBED_FWD     p: ids wte wpe y extra_row | i: n_tok seq C vocab
+ *   EMBED_FWD     p: ids wte wpe y extra_row pos_ids | i: n_tok seq C vocab n_pos  (pos_ids non-null:
+ *                 pp_embed_fwd_at)
+ *   POSITION_IDS  p: ids out | i: n_seq seq pad
  *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab | j: round_bf16
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype
  *   ACCUM_*       p: acc g | i: n | j: init

@@ -104,6 +104,27 @@ def embedding(ids, wte, wpe=None):
     return y
 
 
+def position_ids_from_padding(ids, pad):
+    """Positions counted over the tokens that are not padding, as the embeddings of the encoder in the
+    reference's examples/huggingface/pippy_camemBert.py compute them (``transformers``' RoBERTa family;
+    pinned against that library's own routine in tests/test_hf_fidelity.py): a padding token gets
+    ``pad``, the k-th other token of its sequence (k = 1, 2, ...) gets ``pad + k``."""
+    out = torch.full_like(ids, pad)
+    for b in range(ids.shape[0]):
+        k = 0
+        for s in range(ids.shape[1]):
+            if int(ids[b, s]) != pad:
+                k += 1
+                out[b, s] = pad + k
+    return out
+
+
+def embedding_at(ids, pos_ids, wte, wpe, extra_row=None):
+    """wte[ids] + wpe[pos_ids] (+ one row added to every token)."""
+    y = wte[ids] + wpe[pos_ids]
+    return y if extra_row is None else y + extra_row
+
+
 # ---- top-2 mixture of experts (Mixtral-style block) -------------------------------------------
 def moe_route_top2(logits):
     """Softmax over all experts, the two largest probabilities (the lower expert index wins a tie),

@@ -600,7 +600,10 @@ def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream:
                 raise NotLowerable("a position table that is not read at consecutive positions")
         return [WrappedTokenEmbedding(wte, position, offset)], _skip_identities(root, joins[0])
     # three tables: which is which shows in their constant index tensors (all zero: token type 0; 0 .. S-1: positions)
-    roles = {}
+    # an index computed from the ids: positions counted over the tokens that are not padding, for a table
+    # with a padding row; else taken for token type 0 (RoBERTa gathers it from a buffer of zeros at those
+    # positions) — the comparison with the stage decides whether that reading holds
+    roles, pad = {}, None
     for e in emb[1:]:
         index = _constant_of(root, e.all_input_nodes[0]) if len(e.all_input_nodes) == 1 else None
         if index is not None and index.dtype == torch.int64:
@@ -608,12 +611,18 @@ def _embedding_front(root: nn.Module, nodes: List[fx.Node], order: dict, stream:
                 roles["type"] = e
             elif bool((index.reshape(-1, index.shape[-1]) == torch.arange(index.shape[-1])).all()):
                 roles["position"] = e
+        elif index is None and len(e.all_input_nodes) == 1:
+            table = root.get_submodule(e.target)
+            if table.padding_idx is not None and "position" not in roles:
+                roles["position"], pad = e, int(table.padding_idx)
+            elif table.padding_idx is None and "type" not in roles:
+                roles["type"] = e
     if len(roles) != 2:
         raise NotLowerable("three embedding tables that are not word + position + token type 0")
     if not isinstance(norm, nn.LayerNorm):      # (a pre-LayerNorm encoder normalises inside its layers)
         norm, norm_node = None, joins[0]
     block = WrappedEncoderEmbedding(wte, root.get_submodule(roles["position"].target),
-                                    root.get_submodule(roles["type"].target), norm)
+                                    root.get_submodule(roles["type"].target), norm, padding_positions=pad)
     return [block], _skip_identities(root, norm_node)
 
 
@@ -761,7 +770,11 @@ def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
         return torch.randint(0, first.wte.num_embeddings, shape or (2, seq), generator=g)
     if isinstance(first, WrappedEncoderEmbedding):
         seq = min(16, first.position_embeddings.num_embeddings)
-        return torch.randint(0, first.word_embeddings.num_embeddings, shape or (2, seq), generator=g)
+        x = torch.randint(0, first.word_embeddings.num_embeddings, shape or (2, seq), generator=g)
+        if first.padding_positions is not None:      # some padding, so that its handling is compared too
+            x[0, :1] = first.padding_positions
+            x[-1, x.shape[1] // 2:] = first.padding_positions
+        return x
     d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer))).dim
     return torch.randn(shape or (2, 16, d), generator=g)
 

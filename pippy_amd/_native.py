@@ -26,7 +26,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
- OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU) = range(1, 28)
+ OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU, OP_POSITION_IDS) = range(1, 29)
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
@@ -44,7 +44,7 @@ EXPORTED_SYMBOLS = (
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
     "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc", "pp_gemm_bf16_swiglu", "pp_gemm_bf16_dswiglu",
-    "pp_clock_probe",
+    "pp_clock_probe", "pp_embed_fwd_at", "pp_position_ids_from_padding",
 )
 
 
@@ -127,6 +127,8 @@ def lib() -> C.CDLL:
         "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
         "pp_embed_fwd": [vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
+        "pp_embed_fwd_at": [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
+        "pp_position_ids_from_padding": [vp, vp, i64, i64, i64, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
         "pp_run_ops": [C.POINTER(Op), i32, vp],
         "pp_activation_bwd": [vp, vp, vp, i64, i32, i32, vp],
@@ -614,6 +616,27 @@ def embed_fwd(ids, wte, wpe, y, seq: int, extra_row=None) -> None:
     assert extra_row is None or (extra_row.numel() == Cc and extra_row.is_contiguous())
     check(lib().pp_embed_fwd(ids.data_ptr(), wte.data_ptr(), ptr(wpe), ptr(extra_row), y.data_ptr(),
                              ids.numel(), seq, Cc, vocab, current_stream()), "pp_embed_fwd")
+
+
+def embed_fwd_at(ids, pos_ids, wte, wpe, y, extra_row=None) -> None:
+    """As ``embed_fwd`` with the row of the position table given per token (``pos_ids`` int64, like ``ids``)."""
+    require_cuda(ids, pos_ids, wte, wpe, y)
+    assert ids.dtype == pos_ids.dtype == torch.int64 and ids.is_contiguous() and pos_ids.is_contiguous()
+    assert pos_ids.numel() == ids.numel() and y.is_contiguous() and wpe.shape[1] == wte.shape[1]
+    vocab, Cc = wte.shape
+    assert extra_row is None or (extra_row.numel() == Cc and extra_row.is_contiguous())
+    check(lib().pp_embed_fwd_at(ids.data_ptr(), pos_ids.data_ptr(), wte.data_ptr(), wpe.data_ptr(), ptr(extra_row),
+                                y.data_ptr(), ids.numel(), wpe.shape[0], Cc, vocab, current_stream()),
+          "pp_embed_fwd_at")
+
+
+def position_ids_from_padding(ids, out, pad: int) -> None:
+    """out[b, s] = pad where ids[b, s] == pad, else pad + the count of tokens != pad among ids[b, :s + 1]."""
+    require_cuda(ids, out)
+    assert ids.dtype == out.dtype == torch.int64 and ids.dim() == 2 and out.shape == ids.shape
+    assert ids.is_contiguous() and out.is_contiguous()
+    check(lib().pp_position_ids_from_padding(ids.data_ptr(), out.data_ptr(), ids.shape[0], ids.shape[1], pad,
+                                             current_stream()), "pp_position_ids_from_padding")
 
 
 def embed_bwd(ids, dy, d_wte, d_wpe, seq: int, round_bf16: bool = False) -> None:

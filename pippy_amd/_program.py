@@ -500,7 +500,9 @@ def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_
     return op
 
 
-def op_embed_fwd(ids, wte, wpe, y, seq, extra_row=None) -> N.Op:
+def op_embed_fwd(ids, wte, wpe, y, seq, extra_row=None, pos_ids=None) -> N.Op:
+    """``pos_ids`` (int64, one per token): the row of ``wpe`` each token reads, instead of its index in
+    the sequence."""
     vocab, Cc = wte.shape
     assert ids.dtype == torch.int64 and y.shape == (ids.numel(), Cc) and y.is_contiguous()
     assert extra_row is None or (extra_row.numel() == Cc and extra_row.is_contiguous())
@@ -509,6 +511,21 @@ def op_embed_fwd(ids, wte, wpe, y, seq, extra_row=None) -> N.Op:
     op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), wte.data_ptr(), _p(wpe), y.data_ptr()
     op.p[4] = _p(extra_row)
     op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
+    if pos_ids is not None:
+        assert wpe is not None and pos_ids.dtype == torch.int64 and pos_ids.numel() == ids.numel() \
+            and pos_ids.is_contiguous()
+        op.p[5] = pos_ids.data_ptr()
+        op.i[4] = wpe.shape[0]
+    return op
+
+
+def op_position_ids(ids, out, pad: int) -> N.Op:
+    assert ids.dtype == out.dtype == torch.int64 and ids.dim() == 2 and out.shape == ids.shape
+    assert ids.is_contiguous() and out.is_contiguous()
+    op = N.Op()
+    op.kind = N.OP_POSITION_IDS
+    op.p[0], op.p[1] = ids.data_ptr(), out.data_ptr()
+    op.i[0], op.i[1], op.i[2] = ids.shape[0], ids.shape[1], pad
     return op
 
 

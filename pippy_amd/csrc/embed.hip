@@ -9,7 +9,8 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restric
                                                         const uint16_t* __restrict__ wpe,
                                                         const uint16_t* __restrict__ extra_row,
                                                         uint16_t* __restrict__ y, int64_t n_tok,
-                                                        int64_t seq, int C, int64_t vocab) {
+                                                        int64_t seq, int C, int64_t vocab,
+                                                        const int64_t* __restrict__ pos_ids, int64_t n_pos) {
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tok) return;
@@ -17,7 +18,13 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const int64_t* __restric
     // out-of-range ids read row 0 rather than faulting; callers validate ids on the host side
     if (id < 0 || id >= vocab) id = 0;
     const uint4* src = reinterpret_cast<const uint4*>(wte + id * C);
-    const uint4* pos = wpe ? reinterpret_cast<const uint4*>(wpe + (t % seq) * C) : nullptr;
+    // the row of the position table: t % seq, or the caller's own index (out of range reads row 0)
+    int64_t p = t % seq;
+    if (pos_ids) {
+        p = pos_ids[t];
+        if (p < 0 || p >= n_pos) p = 0;
+    }
+    const uint4* pos = wpe ? reinterpret_cast<const uint4*>(wpe + p * C) : nullptr;
     const uint4* ext = reinterpret_cast<const uint4*>(extra_row);
     uint4* dst = reinterpret_cast<uint4*>(y + t * C);
     for (int c = lane; c < (C >> 3); c += 64) {
@@ -128,6 +135,23 @@ __global__ __launch_bounds__(256) void embed_bwd_wpe_kernel(const uint16_t* __re
     dst[1] += s1;
 }
 
+// Positions counted over the tokens that are not padding: out[b, s] = pad for a padding token, else
+// pad + the number of non-padding tokens among ids[b, 0..s].  One wave per sequence.
+__global__ __launch_bounds__(64) void position_ids_kernel(const int64_t* __restrict__ ids,
+                                                          int64_t* __restrict__ out, int64_t seq, int64_t pad) {
+    const int lane = threadIdx.x;
+    const int64_t row = (int64_t)blockIdx.x * seq;
+    int64_t running = 0;
+    for (int64_t base = 0; base < seq; base += 64) {
+        const int64_t s = base + lane;
+        const bool real = s < seq && ids[row + s] != pad;
+        const uint64_t mask = __ballot(real);
+        const int upto = __builtin_popcountll(mask & ((lane == 63 ? ~0ull : ((1ull << (lane + 1)) - 1ull))));
+        if (s < seq) out[row + s] = real ? pad + running + upto : pad;
+        running += __builtin_popcountll(mask);
+    }
+}
+
 template <int NW>
 static void launch_embed_bwd_wte(const int64_t* ids, const void* dy, float* d_wte, int64_t n_tok, int C,
                                  int64_t vocab, int round_bf16, hipStream_t st) {
@@ -149,8 +173,35 @@ extern "C" int pp_embed_fwd(const int64_t* ids, const void* wte, const void* wpe
         return fail(PP_ERR_INVALID, "pp_embed_fwd: pointers must be 16-byte aligned");
     hipLaunchKernelGGL(embed_fwd_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), ids, (const uint16_t*)wte, (const uint16_t*)wpe,
-                       (const uint16_t*)extra_row, (uint16_t*)y, n_tok, seq, (int)C, vocab);
+                       (const uint16_t*)extra_row, (uint16_t*)y, n_tok, seq, (int)C, vocab,
+                       (const int64_t*)nullptr, (int64_t)0);
     return check_launch("embed_fwd_kernel");
+}
+
+extern "C" int pp_embed_fwd_at(const int64_t* ids, const int64_t* pos_ids, const void* wte, const void* wpe,
+                               const void* extra_row, void* y, int64_t n_tok, int64_t n_pos, int64_t C,
+                               int64_t vocab, pp_stream stream) {
+    if (n_tok < 0 || n_pos <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_fwd_at: bad shape");
+    if (C % 8) return fail(PP_ERR_UNSUPPORTED, "pp_embed_fwd_at: C %% 8 != 0");
+    if (n_tok == 0) return PP_OK;
+    if (!ids || !pos_ids || !wte || !wpe || !y) return fail(PP_ERR_INVALID, "pp_embed_fwd_at: null pointer");
+    if (!aligned(wte, 16) || !aligned(wpe, 16) || !aligned(extra_row, 16) || !aligned(y, 16))
+        return fail(PP_ERR_INVALID, "pp_embed_fwd_at: pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(embed_fwd_kernel, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), ids, (const uint16_t*)wte, (const uint16_t*)wpe,
+                       (const uint16_t*)extra_row, (uint16_t*)y, n_tok, (int64_t)1, (int)C, vocab, pos_ids, n_pos);
+    return check_launch("embed_fwd_kernel");
+}
+
+extern "C" int pp_position_ids_from_padding(const int64_t* ids, int64_t* out, int64_t n_seq, int64_t seq,
+                                            int64_t pad, pp_stream stream) {
+    if (n_seq < 0 || seq < 0) return fail(PP_ERR_INVALID, "pp_position_ids_from_padding: bad shape");
+    if (n_seq == 0 || seq == 0) return PP_OK;
+    if (!ids || !out) return fail(PP_ERR_INVALID, "pp_position_ids_from_padding: null pointer");
+    if (n_seq > 0x7fffffff) return fail(PP_ERR_UNSUPPORTED, "pp_position_ids_from_padding: more than 2^31 - 1 sequences");
+    hipLaunchKernelGGL(position_ids_kernel, dim3((uint32_t)n_seq), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       ids, out, seq, pad);
+    return check_launch("position_ids_kernel");
 }
 
 extern "C" int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe,

@@ -96,7 +96,13 @@ static int run_one(const pp_op& op, pp_stream st) {
             d.scale = op.f[0]; d.causal = op.j[0]; d.kv_group = op.j[1]; d.kv_len = op.j[2];
             return op.kind == PP_OP_ATTN_FWD ? pp_attn_fwd(&d, st) : pp_attn_bwd(&d, st);
         }
+        case PP_OP_POSITION_IDS:
+            return pp_position_ids_from_padding(static_cast<const int64_t*>(op.p[0]), static_cast<int64_t*>(op.p[1]),
+                                                op.i[0], op.i[1], op.i[2], st);
         case PP_OP_EMBED_FWD:
+            if (op.p[5])
+                return pp_embed_fwd_at(static_cast<const int64_t*>(op.p[0]), static_cast<const int64_t*>(op.p[5]),
+                                       op.p[1], op.p[2], op.p[4], op.p[3], op.i[0], op.i[4], op.i[2], op.i[3], st);
             return pp_embed_fwd(static_cast<const int64_t*>(op.p[0]), op.p[1], op.p[2], op.p[4], op.p[3], op.i[0],
                                 op.i[1], op.i[2], op.i[3], st);
         case PP_OP_EMBED_BWD:

@@ -374,9 +374,18 @@ class EncoderEmbedding(NativeBlock):
         for emb in (self.word_embeddings, self.position_embeddings, self.token_type_embeddings):
             nn.init.normal_(emb.weight, std=init_std)
 
+    # None: position s reads row s.  A token id: the positions are counted over the tokens that are not
+    # that (padding) id, starting one past it, and padding tokens read row ``padding_positions`` (RoBERTa)
+    padding_positions = None
+
+    def _positions(self, ids):
+        if self.padding_positions is None:
+            return torch.arange(ids.shape[-1], device=ids.device)
+        real = (ids != self.padding_positions).long()
+        return torch.cumsum(real, dim=-1) * real + self.padding_positions
+
     def forward(self, ids):
-        S = ids.shape[-1]
-        pos = torch.arange(S, device=ids.device)
+        pos = self._positions(ids)
         # one rounding of the three-term sum, as the lowered kernel does
         e = self.word_embeddings(ids).float() + self.position_embeddings(pos).float()
         if self.token_type_embeddings is not None:
@@ -394,12 +403,19 @@ class EncoderEmbedding(NativeBlock):
         Bn, S = ids.shape
         wte, wpe = b.weight(self.word_embeddings.weight), b.weight(self.position_embeddings.weight)
         wtt = b.weight(self.token_type_embeddings.weight) if self.token_type_embeddings is not None else None
-        if S > wpe.shape[0]:
-            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]})")
+        pad = self.padding_positions
+        if S + (0 if pad is None else pad + 1) > wpe.shape[0]:
+            raise RuntimeError(f"sequence length {S} exceeds the position table ({wpe.shape[0]} rows"
+                               f"{'' if pad is None else f', the first {pad + 1} not for positions'})")
         Cc = wte.shape[1]
         T = Bn * S
         e = b.act("e", (T, Cc))
-        b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0] if wtt is not None else None))
+        pos_ids = None
+        if pad is not None:
+            pos_ids = b.act("pos_ids", (Bn, S), torch.int64)
+            b.f(P.op_position_ids(ids, pos_ids, pad))
+        b.f(P.op_embed_fwd(ids, wte, wpe, e, S, extra_row=wtt[0] if wtt is not None else None,
+                           pos_ids=pos_ids.view(-1) if pos_ids is not None else None))
         if self.LayerNorm is not None:
             y, mean, rstd = lower_layernorm(b, "ln", self.LayerNorm, e)
         else:
@@ -413,7 +429,12 @@ class EncoderEmbedding(NativeBlock):
             acc_wpe = b.grad_acc(self.position_embeddings.weight)
             b.w(P.op_fill(acc_wte), tag="fill")
             b.w(P.op_fill(acc_wpe), tag="fill")
-            b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+            if pos_ids is None:
+                b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+            else:   # the position table is one more table read at computed indices
+                b.w(P.op_embed_bwd(ids, de, acc_wte, None, S, round_bf16=not b.fused_accumulate))
+                b.w(P.op_embed_bwd(pos_ids.view(-1), de, acc_wpe, None, S, round_bf16=not b.fused_accumulate))
+                _zero_padding_row(b, self.position_embeddings, acc_wpe)
             _zero_padding_row(b, self.word_embeddings, acc_wte)
             if wtt is not None:
                 # the type-0 row receives the gradient of every token; the other rows none
@@ -1258,10 +1279,12 @@ class WrappedTokenEmbedding(TokenEmbedding):
 
 
 class WrappedEncoderEmbedding(EncoderEmbedding):
-    def __init__(self, word: nn.Embedding, position: nn.Embedding, token_type: nn.Embedding, norm: nn.LayerNorm):
+    def __init__(self, word: nn.Embedding, position: nn.Embedding, token_type: nn.Embedding, norm: nn.LayerNorm,
+                 padding_positions: Optional[int] = None):
         NativeBlock.__init__(self)
         self.word_embeddings, self.position_embeddings, self.token_type_embeddings = word, position, token_type
         self.LayerNorm = norm
+        self.padding_positions = padding_positions
 
 
 class WrappedTransformerLayer(TransformerLayer):

@@ -334,6 +334,59 @@ def test_hugging_face_opt_stages_are_recognised_on_the_models_own_layers():
         _close(x, model(ids).logits, "blocks against OPTForCausalLM")
 
 
+def test_positions_counted_over_real_tokens_are_robertas():
+    """The oracle's loop against the library routine the RoBERTa family calls, on rows with padding at the
+    front, inside, at the end, everywhere and nowhere; and the block's own torch statement of it."""
+    from transformers.models.roberta.modeling_roberta import RobertaEmbeddings
+    from oracle import ops as OO2
+    g = torch.Generator().manual_seed(3)
+    for pad in (1, 0, 5):
+        ids = torch.randint(0, 9, (7, 37), generator=g)
+        ids[0, :4] = pad
+        ids[1, 30:] = pad
+        ids[2] = pad
+        ids[3][ids[3] == pad] = pad + 1
+        want = RobertaEmbeddings.create_position_ids_from_input_ids(ids, pad)
+        assert torch.equal(OO2.position_ids_from_padding(ids, pad), want)
+        blk = SM.EncoderEmbedding(16, 64, 8)
+        blk.padding_positions = pad
+        assert torch.equal(blk._positions(ids), want)
+
+
+def test_hugging_face_roberta_stages_are_recognised_on_the_models_own_layers():
+    """RoBERTa (the family of the reference's examples/huggingface/pippy_camemBert.py): position indices
+    computed from the input ids (a count over the tokens that are not padding), token types gathered from
+    a buffer of zeros at those positions."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.RobertaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                     num_attention_heads=2, max_position_embeddings=66, vocab_size=500,
+                                     hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                                     tie_word_embeddings=False)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.RobertaForMaskedLM(cfg)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"roberta.encoder.layer.1": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedEncoderEmbedding", "WrappedTransformerLayer"], ["WrappedTransformerLayer", "LinearAct", "WrappedLMHead"]]
+    front = blocks[0][0]
+    assert front.padding_positions == 1
+    assert front.position_embeddings is model.roberta.embeddings.position_embeddings
+    assert front.token_type_embeddings is model.roberta.embeddings.token_type_embeddings
+    other = torch.randint(0, 500, (2, 40))
+    other[0, :3] = 1
+    other[1, 20:] = 1
+    x = other
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(other).logits, "blocks against RobertaForMaskedLM on ids with padding")
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true

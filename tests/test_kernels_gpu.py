@@ -404,6 +404,37 @@ def test_embedding():
     assert_close_rel(d_wpe, pr.grad, 1e-5, "d_wpe")
 
 
+@pytest.mark.parametrize("B,S,pad", [(3, 128, 1), (2, 37, 0), (5, 200, 7), (1, 1, 1), (4, 64, 3)])
+def test_positions_counted_over_real_tokens_and_the_lookup_at_them(B, S, pad):
+    """Position indices of an encoder that skips padding tokens (bit-exact against the oracle's loop: rows
+    with padding at the front, inside, at the end, everywhere, nowhere) and the embedding sum read at
+    those indices (one rounding of the fp32 sum, like the positional form)."""
+    Nn = native()
+    g = torch.Generator().manual_seed(B * S + pad)
+    ids = torch.randint(0, 12, (B, S), generator=g)
+    ids[0, : S // 3] = pad
+    if B > 1:
+        ids[1, S // 2:] = pad
+    if B > 2:
+        ids[2] = pad
+    if B > 3:
+        ids[3][ids[3] == pad] = pad + 1
+    out = torch.full((B, S), -1, dtype=torch.int64, device=DEV)
+    Nn.position_ids_from_padding(ids.to(DEV), out, pad)
+    want = O.position_ids_from_padding(ids, pad)
+    assert torch.equal(out.cpu(), want)
+    C, vocab, n_pos = 256, 12, S + pad + 1
+    wte = torch.randn(vocab, C, generator=g).to(torch.bfloat16)
+    wpe = torch.randn(n_pos, C, generator=g).to(torch.bfloat16)
+    row = torch.randn(C, generator=g).to(torch.bfloat16)
+    for extra in (None, row):
+        y = torch.full((B * S, C), float("nan"), dtype=torch.bfloat16, device=DEV)
+        Nn.embed_fwd_at(ids.to(DEV), out, wte.to(DEV), wpe.to(DEV), y,
+                        extra_row=extra.to(DEV) if extra is not None else None)
+        ref = O.embedding_at(ids, want, wte.float(), wpe.float(), extra.float() if extra is not None else None)
+        assert torch.equal(y.cpu(), ref.reshape(B * S, C).to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("C,vocab,n_tok,seq", [(768, 50, 1024, 128), (64, 3, 333, 111), (4096, 17, 130, 65),
                                                (1024, 32000, 2048, 1024)])
 @pytest.mark.parametrize("rounded", [False, True])

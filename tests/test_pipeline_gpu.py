@@ -1026,7 +1026,8 @@ def test_plain_torch_gpt_runs_natively_and_matches_the_oracle():
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
 
 
-def _exported_model_against_the_oracle(model, whole, vocab, seq, split, scale_like=None, before_oracle=None):
+def _exported_model_against_the_oracle(model, whole, vocab, seq, split, scale_like=None, before_oracle=None,
+                                       padding=None):
     """Pipelines ``model`` (which torch.fx cannot trace: the front end exports it on one microbatch) in
     two stages, checks that both run as launch lists, and compares logits, losses and every parameter
     gradient with the fp32 oracle run of ``whole(copy of the model)``.  ``scale_like(name)`` may name
@@ -1036,12 +1037,18 @@ def _exported_model_against_the_oracle(model, whole, vocab, seq, split, scale_li
     initialisation the query and key parts are two orders smaller and carry the same absolute rounding
     noise), and, so that a wrong query or key gradient cannot hide behind that scale, at three times
     the tolerance on their own.  ``before_oracle(ref, stages, M)`` may prepare the fp32 copy from what
-    the run saved (a ReLU model is given the run's own active sets)."""
+    the run saved (a ReLU model is given the run's own active sets).  ``padding``: a token id written over
+    the end of some sequences, the start of one and a few places inside."""
     import pippy_amd as pp
     M, mb = 4, 2
     model = model.to(torch.bfloat16)
     ref = copy.deepcopy(model).float()
     ids = torch.randint(0, vocab, (mb * M, seq))
+    if padding is not None:
+        ids[0, seq - 9:] = padding
+        ids[3, seq // 2:] = padding
+        ids[5, :4] = padding
+        ids[6, 10:13] = padding
     target = torch.randint(0, vocab, (mb * M, seq))
     pipe = pp.pipeline(model, mb_args=(ids[:mb],), split_spec={split: pp.SplitPoint.BEGINNING})
     stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
@@ -1227,7 +1234,7 @@ def _qkv_group(name):
 
 
 @pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra", "opt", "gpt2_spelled_out",
-                                    "megatron_bert", "gpt_neo"])
+                                    "megatron_bert", "gpt_neo", "roberta"])
 def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
     value projections), Mistral (Llama layout), Phi-3 (one fused q|k|v and one fused gate|up projection),
@@ -1239,7 +1246,9 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     "eager" attention, Megatron-BERT (pre-LayerNorm encoder, embeddings without a LayerNorm, a final
     LayerNorm in front of the head's transform; examples/huggingface/pippy_megatronBert.py) and GPT-Neo
     (scores without the 1 / sqrt(head size) factor, the causal mask applied twice, projections without
-    biases, "local" layers whose window covers the sequence; examples/huggingface/pippy_gptNeo.py)."""
+    biases, "local" layers whose window covers the sequence; examples/huggingface/pippy_gptNeo.py); and
+    RoBERTa (the family of examples/huggingface/pippy_camemBert.py), whose position indices count the
+    tokens that are not padding: the input holds padding at the end, the start and inside of sequences."""
     T = pytest.importorskip("transformers")
     import torch.nn as nn
     common = dict(vocab_size=1000, tie_word_embeddings=False)
@@ -1280,6 +1289,11 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
                                            embed_dropout=0.0, attention_dropout=0.0, resid_dropout=0.0,
                                            use_cache=False, bos_token_id=0, eos_token_id=0, **common),
                             "transformer.h.2"),
+        "roberta": lambda: (T.RobertaForMaskedLM,
+                            T.RobertaConfig(hidden_size=128, intermediate_size=512, num_hidden_layers=4,
+                                            num_attention_heads=2, max_position_embeddings=132,
+                                            hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, **common),
+                            "roberta.encoder.layer.2"),
     }[family]()
     cfg._attn_implementation = "eager" if family in ("gpt2_spelled_out", "megatron_bert", "gpt_neo") else "sdpa"
     torch.manual_seed(0)
@@ -1301,7 +1315,8 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
             return self.g(idx).logits
 
     _exported_model_against_the_oracle(model, Logits, 1000, 128, split, scale_like=_qkv_group,
-                                       before_oracle=_relu_sets_of_the_run if family == "opt" else None)
+                                       before_oracle=_relu_sets_of_the_run if family == "opt" else None,
+                                       padding=cfg.pad_token_id if family == "roberta" else None)
 
 
 def _relu_sets_of_the_run(ref, stages, M):
