@@ -474,17 +474,32 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         # attention spelled out (softmax(q k^T) v between the projections): the softmax stands for the call
         mods.insert(len(mods) - 1, (soft[0], None))
         kinds.insert(len(kinds) - 1, "sdpa")
+    head_norms = {}
+    if kinds[:1] == ["RMSNorm"] and "sdpa" in kinds and kinds.count("RMSNorm") > 1:
+        # RMS norms inside the branch: over the values of each head of the queries / keys, each fed (through
+        # views) by the projection it belongs to
+        for n, m in [x for x in mods[1:] if kind(*x) == "RMSNorm"]:
+            src = _constant_factors_back(root, n.all_input_nodes[0])[0] if n.all_input_nodes else None
+            if not (isinstance(src, fx.Node) and src.op == "call_module" and m.weight.shape[0] in (64, 128)):
+                raise NotLowerable(f"a norm inside an attention branch that does not follow a projection "
+                                   f"('{n.format_node()}')")
+            head_norms[src] = m
+            mods.remove((n, m))
+        kinds = [kind(n, m) for n, m in mods]
     if kinds == ["RMSNorm", "Linear", "Linear", "Linear", "sdpa", "Linear"]:
-        (_, norm), (_, q), (_, k), (_, v), (sd, _), (_, o) = mods
+        (_, norm), (qn, q), (kn, k), (vn, v), (sd, _), (_, o) = mods
         if not all(isinstance(lin, nn.Linear) for lin in (q, k, v, o)):
             raise NotLowerable("rotary attention whose projections keep [in, out] weights")
-        if k.out_features != v.out_features or q.out_features != o.in_features or q.out_features != q.in_features \
-                or q.out_features % k.out_features:
+        if k.out_features != v.out_features or q.out_features != o.in_features or q.out_features % k.out_features:
             raise NotLowerable("query / key / value projections of unexpected widths")
+        if set(head_norms) - {qn, kn}:
+            raise NotLowerable("a per-head norm on something other than queries and keys")
         causal, form = _attention_form(root, sd)
         if not causal:
             raise NotLowerable("rotary attention that is not causal")
-        return ("attn_rope", norm, (q, k, v), o, form)
+        return ("attn_rope", norm, (q, k, v), o, form, (head_norms.get(qn), head_norms.get(kn)))
+    if head_norms:
+        raise NotLowerable("per-head norms in an attention branch without separate query / key / value projections")
     if kinds == ["RMSNorm", "Linear", "sdpa", "Linear"] and inner_adds:
         (_, norm), (_, qkv), (sd, _), (_, o) = mods       # one fused q|k|v projection under a rotary embedding
         if not all(isinstance(lin, nn.Linear) for lin in (qkv, o)) or o.in_features != o.out_features \
@@ -493,7 +508,7 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         causal, form = _attention_form(root, sd)
         if not causal:
             raise NotLowerable("rotary attention that is not causal")
-        return ("attn_rope", norm, qkv, o, form)
+        return ("attn_rope", norm, qkv, o, form, (None, None))
     if kinds == ["RMSNorm", "Linear", "act", "Linear", "Linear"] or kinds == ["RMSNorm", "Linear", "Linear", "act", "Linear"]:
         norm, down = mods[0][1], mods[-1][1]
         an = next(n for n, m in mods if kind(n, m) == "act")
@@ -632,6 +647,8 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
     if (attention[0], feed_forward[0]) not in (("attn", "mlp"), ("attn_rope", "mlp_gated"), ("attn_rope", "mlp_moe")):
         raise NotLowerable(f"a '{attention[0]}' branch followed by a '{feed_forward[0]}' branch")
     d = attention[3].in_features
+    if attention[0] == "attn_rope" and rope is not None:
+        n_heads = max(1, d // (2 * rope[0].shape[1]))     # the table's width is the head size
     if d % n_heads or d // n_heads not in (64, 128):
         raise NotLowerable(f"head dimension {d}/{n_heads} (64 and 128 are built)")
     if feed_forward[0] == "mlp":
@@ -645,7 +662,7 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
             return WrappedTransformerLayer(attention_norm, qkv, proj, feed_forward_norm, fc1, fc2, n_heads, causal,
                                            act, pre_ln=False, attn_scale=scale)
         return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act, attn_scale=scale)
-    _, norm1, qkv, o, form = attention
+    _, norm1, qkv, o, form, (q_norm, k_norm) = attention
     width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
     D = d // n_heads
     if _score_factor(form, D) is not None:
@@ -658,9 +675,11 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
                            "(exported models do)")
     if feed_forward[0] == "mlp_moe":
         _, norm2, router, experts, gate_up, down = feed_forward
+        if q_norm is not None or k_norm is not None:
+            raise NotLowerable("per-head norms in a mixture-of-experts layer")
         return WrappedMoELayer(norm1, qkv, o, norm2, router, experts, gate_up, down, n_heads, *rope)
     _, norm2, gate_up, down = feed_forward
-    return WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope)
+    return WrappedLlamaLayer(norm1, qkv, o, norm2, gate_up, down, n_heads, *rope, q_norm=q_norm, k_norm=k_norm)
 
 
 def _tail_blocks(root: nn.Module, stream: fx.Node, result: fx.Node, after_layers: bool) -> List[NativeBlock]:
@@ -814,6 +833,8 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     widths = {m.normalized_shape[0] for m in submod.modules()
               if isinstance(m, (nn.LayerNorm, nn.RMSNorm)) and len(m.normalized_shape) == 1}
     widths |= {m.weight.shape[0] for m in submod.modules() if rms_norm_like(m) is not None}
+    if len(widths) > 1 and all(w in (64, 128) for w in widths - {max(widths)}):
+        widths = {max(widths)}       # (norms over the values of one head, on queries and keys)
     if len(widths) != 1:
         raise NotLowerable("no single model width (the normalisation layers of the stage disagree)")
     d = widths.pop()

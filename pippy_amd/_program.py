@@ -568,9 +568,11 @@ def op_accum(acc, g, init=False) -> N.Op:
 
 def op_copy_rows(src, dst, n_rows, row_bytes, src_stride, dst_stride) -> N.Op:
     """``n_rows`` runs of ``row_bytes`` bytes from ``src`` to ``dst`` with byte strides between runs."""
+    def room(t):    # bytes from the tensor's first element to the end of its storage (t may be a strided view)
+        return t.untyped_storage().nbytes() - t.storage_offset() * t.element_size()
     assert src_stride >= row_bytes and dst_stride >= row_bytes
-    assert (n_rows - 1) * src_stride + row_bytes <= src.numel() * src.element_size()
-    assert (n_rows - 1) * dst_stride + row_bytes <= dst.numel() * dst.element_size()
+    assert (n_rows - 1) * src_stride + row_bytes <= room(src), "op_copy_rows: reads past the source"
+    assert (n_rows - 1) * dst_stride + row_bytes <= room(dst), "op_copy_rows: writes past the destination"
     op = N.Op()
     op.kind = N.OP_COPY_ROWS
     op.p[0], op.p[1] = src.data_ptr(), dst.data_ptr()

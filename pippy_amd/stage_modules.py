@@ -681,19 +681,37 @@ class LlamaLayer(NativeBlock):
             nn.init.normal_(lin.weight, std=init_std)
 
     # torch statement of the layer
+    # the size of a head when it is not dim / n_heads (the output projection then maps n_heads * head_dim
+    # back to dim), and RMS norms over each head's values of the queries / keys in front of the rotary
+    # embedding (Qwen3): attributes a wrapper around a user's layers may set
+    head_dim = None
+
+    def _head_dim(self) -> int:
+        return self.head_dim or self.dim // self.n_heads
+
+    def _head_norms(self):
+        """(q_norm, k_norm): submodules when set (a class attribute would hide a registered submodule)."""
+        return getattr(self, "q_norm", None), getattr(self, "k_norm", None)
+
     def forward(self, x):
         Bn, S, Cc = x.shape
-        H, Hkv, D = self.n_heads, self.n_kv_heads, Cc // self.n_heads
+        H, Hkv, D = self.n_heads, self.n_kv_heads, self._head_dim()
         cos, sin = self._rope(S, D, x.device)
         h = self.input_layernorm(x)
         q, k, v = self._project_qkv(h).split([H * D, Hkv * D, Hkv * D], dim=-1)
-        q = q.reshape(Bn, S, H, D).transpose(1, 2)
-        k, v = (t.reshape(Bn, S, Hkv, D).transpose(1, 2) for t in (k, v))
+        q = q.reshape(Bn, S, H, D)
+        k, v = (t.reshape(Bn, S, Hkv, D) for t in (k, v))
+        q_norm, k_norm = self._head_norms()
+        if q_norm is not None:
+            q = q_norm(q)
+        if k_norm is not None:
+            k = k_norm(k)
+        q, k, v = (t.transpose(1, 2) for t in (q, k, v))
         q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
         if Hkv != H:  # query heads g * (H / Hkv) .. share key / value head g
             k, v = (t.repeat_interleave(H // Hkv, dim=1) for t in (k, v))
         o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
-        x = x + self.self_attn.o_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
+        x = x + self.self_attn.o_proj(o.transpose(1, 2).reshape(Bn, S, H * D))
         return x + self._feed_forward(self.post_attention_layernorm(x))
 
     def _feed_forward(self, h):
@@ -723,7 +741,7 @@ class LlamaLayer(NativeBlock):
                                f"{tuple(x.shape)}")
         Bn, S, Cc = x.shape
         T, H, Hkv = Bn * S, self.n_heads, self.n_kv_heads
-        D = Cc // H
+        D = self._head_dim()
         W = (H + 2 * Hkv) * D  # width of the fused projection
         x2d = x.view(T, Cc)
         cos = b.sp.shared(f"rope_cos:{S}:{D}:{self._rope_key()}", (S, D // 2), torch.float32)
@@ -733,6 +751,20 @@ class LlamaLayer(NativeBlock):
         sin.copy_(s_)
         n1, rstd1 = lower_rmsnorm(b, "n1", self.input_layernorm, x2d)
         qkv = self._lower_qkv(b, n1)
+        # per-head norms: the heads of the queries (keys) leave the fused buffer as rows of their own, are
+        # normalised, and go back to where the rotary embedding and the attention read them
+        es = qkv.element_size()
+        head_norms = []
+        q_norm, k_norm = self._head_norms()
+        for name, norm, first, count in (("q", q_norm, 0, H), ("k", k_norm, H, Hkv)):
+            if norm is None:
+                continue
+            part = qkv[:, first * D:(first + count) * D]
+            pre = b.act(name + "_heads", (T * count, D))
+            b.f(P.op_copy_rows(part, pre, T, count * D * es, W * es, count * D * es))
+            normed, rstd = lower_rmsnorm(b, name + "_normed", norm, pre)
+            b.f(P.op_copy_rows(normed, part, T, count * D * es, count * D * es, W * es))
+            head_norms.append((name, norm, first, count, pre, rstd))
         b.f(P.op_rope(qkv, cos, sin, S, H + Hkv, D))
         att, attention_backward = lower_attention(b, qkv, Bn, S, H, True, n_kv_heads=Hkv)
         x2, _ = lower_linear(b, "x2", self.self_attn.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
@@ -744,6 +776,12 @@ class LlamaLayer(NativeBlock):
             dqkv = attention_backward(d_att)
             # gradients w.r.t. the rotated q and k go back through the transposed rotation
             b.i(P.op_rope(dqkv, cos, sin, S, H + Hkv, D, inverse=True))
+            for name, norm, first, count, pre, rstd in head_norms:
+                part = dqkv[:, first * D:(first + count) * D]
+                d_normed = b.grad(name + "_heads.dy", (T * count, D))
+                b.i(P.op_copy_rows(part, d_normed, T, count * D * es, W * es, count * D * es))
+                d_pre = rmsnorm_backward(b, name + "_heads", norm, pre, rstd, d_normed)
+                b.i(P.op_copy_rows(d_pre, part, T, count * D * es, count * D * es, W * es))
             d_n1 = self._qkv_backward(b, n1, dqkv)
             dx = rmsnorm_backward(b, "n1", self.input_layernorm, x2d, rstd1, d_n1, dres=d_x2,
                                   dx_out=dx_out.view(T, Cc) if dx_out is not None else None)
@@ -1323,11 +1361,12 @@ class WrappedLlamaLayer(LlamaLayer):
     weights side by side; each weight gradient reads its column range of the output gradient."""
 
     def __init__(self, input_layernorm, qkv, o_proj, post_attention_layernorm, gate_up, down_proj,
-                 n_heads: int, cos: torch.Tensor, sin: torch.Tensor):
+                 n_heads: int, cos: torch.Tensor, sin: torch.Tensor, q_norm=None, k_norm=None):
         """``cos`` / ``sin``: the model's own rotary tables, [positions, head_dim / 2] (whatever base,
-        scaling or rounding the model applies is in them)."""
+        scaling or rounding the model applies is in them); ``q_norm`` / ``k_norm``: RMS norms over each
+        head's values of the queries / keys."""
         NativeBlock.__init__(self)
-        self._init_attention(input_layernorm, qkv, o_proj, n_heads, cos, sin)
+        self._init_attention(input_layernorm, qkv, o_proj, n_heads, cos, sin, q_norm, k_norm)
         self.post_attention_layernorm = post_attention_layernorm
         self._gate_up = tuple(gate_up) if isinstance(gate_up, (tuple, list)) else (gate_up,)
         self.ffn = down_proj.in_features
@@ -1339,10 +1378,16 @@ class WrappedLlamaLayer(LlamaLayer):
             self.mlp.gate_up_proj = self._gate_up[0]
         self.mlp.down_proj = down_proj
 
-    def _init_attention(self, input_layernorm, qkv, o_proj, n_heads, cos, sin):
+    def _init_attention(self, input_layernorm, qkv, o_proj, n_heads, cos, sin, q_norm=None, k_norm=None):
         self._qkv = tuple(qkv) if isinstance(qkv, (tuple, list)) else (qkv,)
         self.dim, self.n_heads = o_proj.out_features, n_heads
-        D = self.dim // n_heads
+        assert o_proj.in_features % n_heads == 0
+        D = o_proj.in_features // n_heads
+        self.head_dim = D if D * n_heads != self.dim else None
+        if q_norm is not None:
+            self.q_norm = q_norm
+        if k_norm is not None:
+            self.k_norm = k_norm
         assert cos.shape == sin.shape and cos.shape[1] == D // 2
         width = sum(lin.out_features for lin in self._qkv)
         self.n_kv_heads = (width // D - n_heads) // 2

@@ -387,6 +387,41 @@ def test_hugging_face_roberta_stages_are_recognised_on_the_models_own_layers():
         _close(x, model(other).logits, "blocks against RobertaForMaskedLM on ids with padding")
 
 
+@pytest.mark.parametrize("head_dim", [64, 128])
+def test_hugging_face_qwen3_stages_are_recognised_with_their_per_head_norms(head_dim):
+    """Qwen3: RMS norms over the values of each head, on queries and keys, in front of the rotary
+    embedding; and a head size that need not be width / heads (128 with four heads on a width of 256: the
+    query projection maps 256 -> 512 and the output projection 512 -> 256)."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.Qwen3Config(hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, head_dim=head_dim, vocab_size=500,
+                                   max_position_embeddings=64, use_cache=False, tie_word_embeddings=False,
+                                   attention_dropout=0.0)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.Qwen3ForCausalLM(cfg)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith(("q_norm.weight", "k_norm.weight")):
+                p.add_(torch.randn_like(p) * 0.3)
+    ids = torch.randint(0, 500, (2, 48))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"model.layers.1": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding", "WrappedLlamaLayer"], ["WrappedLlamaLayer", "WrappedLMHead"]]
+    layer, hf = blocks[1][0], model.model.layers[1]
+    assert layer.q_norm.layer is hf.self_attn.q_norm and layer.k_norm.layer is hf.self_attn.k_norm
+    assert (layer.n_heads, layer.n_kv_heads, layer._head_dim()) == (4, 2, head_dim)
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against Qwen3ForCausalLM")
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true

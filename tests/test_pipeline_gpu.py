@@ -1083,7 +1083,11 @@ def _exported_model_against_the_oracle(model, whole, vocab, seq, split, scale_li
             if rp.grad.abs().max().item() > 5e-3 * scale:
                 assert err <= 3 * BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
         else:
-            assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
+            # (the weight of a per-head norm on queries / keys: D values, each a sum over all tokens and
+            # heads of terms that largely cancel; torch's own bf16 autograd through the same model is
+            # 0.9e-2 ... 2.6e-2 off the fp32 result there, this path 0.8e-2 ... 2.4e-2)
+            tol = 3 * BF16_TOL if name.endswith(("q_norm.weight", "k_norm.weight")) else BF16_TOL
+            assert err <= tol, f"grad of {name}: max relative error {err:.3e}"
 
 
 def test_exported_library_style_gpt_runs_natively_and_matches_the_oracle():
@@ -1237,7 +1241,7 @@ def _qkv_group(name):
 
 
 @pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra", "opt", "gpt2_spelled_out",
-                                    "megatron_bert", "gpt_neo", "roberta"])
+                                    "megatron_bert", "gpt_neo", "roberta", "qwen3", "qwen3_wide_heads"])
 def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
     value projections), Mistral (Llama layout), Phi-3 (one fused q|k|v and one fused gate|up projection),
@@ -1251,7 +1255,10 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     (scores without the 1 / sqrt(head size) factor, the causal mask applied twice, projections without
     biases, "local" layers whose window covers the sequence; examples/huggingface/pippy_gptNeo.py); and
     RoBERTa (the family of examples/huggingface/pippy_camemBert.py), whose position indices count the
-    tokens that are not padding: the input holds padding at the end, the start and inside of sequences."""
+    tokens that are not padding: the input holds padding at the end, the start and inside of sequences;
+    Qwen3 (RMS norms over each head's values of queries and keys in front of the rotary embedding; in
+    the second variant a head size of 128 that is not width / heads, so that the query projection widens
+    the stream and the output projection narrows it again)."""
     T = pytest.importorskip("transformers")
     import torch.nn as nn
     common = dict(vocab_size=1000, tie_word_embeddings=False)
@@ -1292,6 +1299,9 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
                                            embed_dropout=0.0, attention_dropout=0.0, resid_dropout=0.0,
                                            use_cache=False, bos_token_id=0, eos_token_id=0, **common),
                             "transformer.h.2"),
+        "qwen3": lambda: (T.Qwen3ForCausalLM, T.Qwen3Config(head_dim=64, **llama_like, **common), "model.layers.2"),
+        "qwen3_wide_heads": lambda: (T.Qwen3ForCausalLM, T.Qwen3Config(head_dim=128, **llama_like, **common),
+                                     "model.layers.2"),
         "roberta": lambda: (T.RobertaForMaskedLM,
                             T.RobertaConfig(hidden_size=128, intermediate_size=512, num_hidden_layers=4,
                                             num_attention_heads=2, max_position_embeddings=132,
@@ -1308,6 +1318,11 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
             for name, p in model.named_parameters():
                 if name.endswith("_proj.bias"):
                     p.normal_(std=0.05)
+    if family.startswith("qwen3"):
+        with torch.no_grad():      # (and per-head norm weights to one)
+            for name, p in model.named_parameters():
+                if name.endswith(("q_norm.weight", "k_norm.weight")):
+                    p.add_(torch.randn_like(p) * 0.3)
 
     class Logits(nn.Module):
         def __init__(self, g):
