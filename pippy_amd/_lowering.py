@@ -18,8 +18,8 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, NativeBlock, RMSNormBlock, RMSNormLike,
-                            StageSequence, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer,
+from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, LinearView, NativeBlock, RMSNormBlock, RMSNormLike,
+                            StageSequence, torch_encoder_layer_block, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer,
                             WrappedTokenEmbedding,
                             WrappedTransformerLayer, activation_like, in_out_linear_like, rms_norm_like)
 
@@ -29,7 +29,8 @@ _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GEL
 
 class _ChainTracer(fx.Tracer):
     def is_leaf_module(self, m, qualname):
-        return isinstance(m, _LEAF_TYPES) or in_out_linear_like(m) or activation_like(m) is not None \
+        return isinstance(m, _LEAF_TYPES + (nn.TransformerEncoderLayer,)) or in_out_linear_like(m) \
+            or activation_like(m) is not None \
             or rms_norm_like(m) is not None or super().is_leaf_module(m, qualname)
 
 
@@ -144,6 +145,8 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
         m = _as_linear(m) or m
         if isinstance(m, NativeBlock):
             blocks.append(m)
+        elif isinstance(m, nn.TransformerEncoderLayer):
+            blocks.append(_torch_layer(m, n))
         elif isinstance(m, (nn.Linear, InOutLinear)):
             nxt = _activation_of(nodes[i + 1], root) if i + 1 < len(nodes) else None
             if nxt == "silu":
@@ -170,6 +173,19 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
     if not blocks:
         raise NotLowerable("the stage holds no layer")
     return blocks
+
+
+def _torch_layer(m: nn.TransformerEncoderLayer, n: fx.Node) -> NativeBlock:
+    """torch's own encoder layer, called with its input alone (no mask, no padding mask)."""
+    if len(n.args) != 1 or any(v is not None for v in n.kwargs.values()):
+        raise NotLowerable(f"'{n.format_node()}': an nn.TransformerEncoderLayer called with a mask")
+    head = m.self_attn.embed_dim // m.self_attn.num_heads
+    if head not in (64, 128):
+        raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}' with head size {head} (64 and 128 are built)")
+    try:
+        return torch_encoder_layer_block(m)
+    except ValueError as e:
+        raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}': {e}") from None
 
 
 def _lower(submod: nn.Module) -> List[NativeBlock]:
@@ -232,6 +248,7 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 # forward on a random input (fp32, on the host), otherwise the stage stays with torch autograd.
 _SDPA = (F.scaled_dot_product_attention, _ATEN.scaled_dot_product_attention.default)
 _ADD_FNS = (operator.add, operator.iadd, torch.add, _ATEN.add.Tensor, _ATEN.add_.Tensor)
+_LINEAR_FNS = (_ATEN.linear.default,)      # an affine map written as a function of parameters
 _ACT_FNS = (F.gelu, F.relu, torch.relu, F.silu, _ATEN.gelu.default, _ATEN.relu.default, _ATEN.silu.default)
 
 
@@ -251,7 +268,7 @@ def _branch_layers(y: fx.Node, stream: fx.Node, order: dict, state: bool = False
         seen.add(n)
         if n.op == "placeholder":
             continue
-        if n.op == "call_module" or (n.op == "call_function" and n.target in _SDPA + _ACT_FNS) \
+        if n.op == "call_module" or (n.op == "call_function" and n.target in _SDPA + _ACT_FNS + _LINEAR_FNS) \
                 or _is_add(n):
             found.append(n)
         elif state and (n.op == "get_attr" or (n.op == "call_function" and
@@ -272,6 +289,19 @@ def _constant_of(root: nn.Module, node) -> Optional[torch.Tensor]:
     except AttributeError:
         return None
     return obj if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) else None
+
+
+def _parameter_of(root: nn.Module, node) -> Optional[nn.Parameter]:
+    """The parameter behind a ``get_attr`` node of ``root``, else None."""
+    if not isinstance(node, fx.Node) or node.op != "get_attr":
+        return None
+    obj = root
+    try:
+        for part in str(node.target).split("."):
+            obj = getattr(obj, part)
+    except AttributeError:
+        return None
+    return obj if isinstance(obj, nn.Parameter) else None
 
 
 def _is_causal_mask(mask: torch.Tensor) -> bool:
@@ -451,6 +481,13 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         if n.op == "call_module":
             m = root.get_submodule(n.target)
             mods.append((n, _as_linear(m) or _as_rms_norm(m) or m))
+        elif n.op == "call_function" and n.target in _LINEAR_FNS:
+            # (nn.MultiheadAttention applies its packed q|k|v parameters and its output projection this way)
+            weight = _parameter_of(root, n.args[1])
+            bias = _parameter_of(root, n.args[2]) if len(n.args) > 2 and n.args[2] is not None else None
+            if weight is None or weight.dim() != 2 or (len(n.args) > 2 and n.args[2] is not None and bias is None):
+                raise NotLowerable(f"'{n.format_node()}': a linear function of something other than parameters")
+            mods.append((n, LinearView(weight, bias)))
         elif _is_add(n):
             if any(_constant_of(root, a) is not None for a in n.args[:2]):
                 continue             # a constant added on (the mask of an attention that is spelled out)
@@ -748,6 +785,12 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
     # residual pairs: the stream feeds one addition whose other operand is a branch computed from the stream
     attention = attention_norm = None
     while True:
+        whole = next(iter(stream.users)) if len(stream.users) == 1 else None
+        if whole is not None and whole.op == "call_module" and attention is None and \
+                isinstance(root.get_submodule(whole.target), nn.TransformerEncoderLayer):
+            blocks.append(_torch_layer(root.get_submodule(whole.target), whole))    # a layer of torch's own
+            stream = _skip_identities(root, whole)
+            continue
         adds = [u for u in stream.users if _is_add(u)]
         if len(adds) != 1:
             break

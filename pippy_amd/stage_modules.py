@@ -1325,6 +1325,47 @@ class WrappedEncoderEmbedding(EncoderEmbedding):
         self.padding_positions = padding_positions
 
 
+class LinearView(nn.Linear):
+    """An ``nn.Linear`` around parameters that a module keeps without a layer of their own (the packed
+    q|k|v projection of ``nn.MultiheadAttention``): the same parameter objects, so names, gradients and
+    optimizer state stay with the owner."""
+
+    def __init__(self, weight: nn.Parameter, bias: Optional[nn.Parameter]):
+        nn.Module.__init__(self)
+        self.out_features, self.in_features = weight.shape
+        self.weight = weight
+        if bias is None:
+            self.register_parameter("bias", None)
+        else:
+            self.bias = bias
+
+
+def torch_encoder_layer_block(layer: nn.TransformerEncoderLayer, causal: bool = False) -> "WrappedTransformerLayer":
+    """``nn.TransformerEncoderLayer`` (called with its input alone: no mask) as a transformer block around
+    the layer's own parameters.  Raises ValueError with what keeps it from that."""
+    att = layer.self_attn
+    if not getattr(att, "batch_first", False):
+        raise ValueError("nn.TransformerEncoderLayer with batch_first=False (sequence-major activations)")
+    if not att._qkv_same_embed_dim or att.in_proj_weight is None or att.bias_k is not None or att.add_zero_attn:
+        raise ValueError("nn.MultiheadAttention with separate key / value widths, bias_k / bias_v or add_zero_attn")
+    drops = [layer.dropout, layer.dropout1, layer.dropout2]
+    if (layer.training and any(d.p > 0 for d in drops)) or (att.dropout > 0 and layer.training):
+        raise ValueError("dropout with p > 0 in training mode")
+    act = layer.activation
+    name = {F.relu: "relu", torch.relu: "relu"}.get(act)
+    if name is None and act is F.gelu:
+        name = "gelu_erf"
+    if name is None and isinstance(act, nn.Module):
+        name = activation_like(act)
+    if name not in ("relu", "gelu_erf", "gelu_tanh"):
+        raise ValueError(f"feed-forward activation {act!r} (ReLU, erf-GELU and tanh-GELU are built)")
+    if any(not isinstance(n, nn.LayerNorm) or not n.elementwise_affine or n.bias is None for n in (layer.norm1, layer.norm2)):
+        raise ValueError("norm layers other than affine LayerNorms with a bias")
+    qkv = LinearView(att.in_proj_weight, att.in_proj_bias)
+    return WrappedTransformerLayer(layer.norm1, qkv, att.out_proj, layer.norm2, layer.linear1, layer.linear2,
+                                   att.num_heads, causal, name, pre_ln=bool(layer.norm_first))
+
+
 class WrappedTransformerLayer(TransformerLayer):
     """``TransformerLayer`` around a user's layers.  ``c_attn`` is the fused q|k|v projection or the
     three separate ones; ``pre_ln=False`` is the encoder form, where ``ln_1`` / ``ln_2`` follow the two

@@ -96,3 +96,35 @@ class LibGPT(nn.Module):
         for blk in self.h:
             x = blk(x, mask)
         return self.lm_head(self.ln_f(x))
+
+
+# ---- an encoder built from torch's own layer class ------------------------------------------------------
+class TorchEncoderLM(nn.Module):
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4, norm_first=True, activation="gelu"):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, d); self.pos = nn.Embedding(seq, d)
+        self.layers = nn.ModuleList([nn.TransformerEncoderLayer(d, h, 4 * d, dropout=0.0, activation=activation,
+                                                                batch_first=True, norm_first=norm_first)
+                                     for _ in range(L)])
+        self.norm = nn.LayerNorm(d); self.head = nn.Linear(d, vocab, bias=False)
+    def forward(self, ids):
+        x = self.emb(ids) + self.pos(torch.arange(ids.shape[1], device=ids.device))
+        for layer in self.layers:
+            x = layer(x)
+        return self.head(self.norm(x))
+
+
+class TorchEncoderStackLM(nn.Module):
+    """The same with the layers inside ``nn.TransformerEncoder`` (whose forward torch.fx cannot follow: the
+    front end exports it, and the layers dissolve into ATen nodes on their parameters)."""
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4, norm_first=True, activation="gelu"):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, d); self.pos = nn.Embedding(seq, d)
+        layer = nn.TransformerEncoderLayer(d, h, 4 * d, dropout=0.0, activation=activation, batch_first=True,
+                                           norm_first=norm_first)
+        self.encoder = nn.TransformerEncoder(layer, L, norm=nn.LayerNorm(d) if norm_first else None,
+                                             enable_nested_tensor=False)
+        self.head = nn.Linear(d, vocab, bias=False)
+    def forward(self, ids):
+        x = self.emb(ids) + self.pos(torch.arange(ids.shape[1], device=ids.device))
+        return self.head(self.encoder(x))

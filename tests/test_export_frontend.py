@@ -316,3 +316,78 @@ def test_attention_spelled_out_is_recognised_with_its_mask_and_factor(factor):
         assert len(layers) == 2 and all(b.causal for b in layers)
         want = {"default": None, "none": 1.0, "queries": 0.2}[factor]
         assert all(b.attn_scale == want if want is None else abs(b.attn_scale - want) < 1e-9 for b in layers)
+
+
+@pytest.mark.parametrize("norm_first,activation", [(True, "gelu"), (False, "relu")])
+def test_torchs_own_encoder_layers_become_transformer_blocks(norm_first, activation):
+    """``nn.TransformerEncoderLayer`` (batch first, called without a mask) is taken as a whole: a transformer
+    block around its own parameters, the packed q|k|v projection of ``nn.MultiheadAttention`` seen through
+    an ``nn.Linear`` view of the same parameter objects.  What it cannot take is said."""
+    import os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchEncoderLM
+    from pippy_amd._lowering import lower_stage_module
+    torch.manual_seed(0)
+    model = TorchEncoderLM(vocab=500, seq=64, norm_first=norm_first, activation=activation)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    x = ids
+    for i in range(2):
+        why = []
+        blocks = lower_stage_module(pipe.get_stage_module(i), why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2
+        for b, own in zip(layers, model.layers[2 * i:2 * i + 2]):
+            assert b.attn.c_attn.weight is own.self_attn.in_proj_weight and b.attn.c_attn.bias is own.self_attn.in_proj_bias
+            assert b.attn.c_proj is own.self_attn.out_proj and b.mlp.c_fc is own.linear1 and b.ln_2 is own.norm2
+            assert (b.pre_ln, b.causal, b.n_heads) == (norm_first, False, 2)
+            assert b.activation == {"gelu": "gelu_erf", "relu": "relu"}[activation]
+        with torch.no_grad():
+            for b in blocks:
+                x = b(x)
+    torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+    # sequence-major layers and head sizes the kernels do not have stay with torch, with the reason
+    other = TorchEncoderLM(vocab=500, seq=64, d=96, h=2)
+    pipe = pp.pipeline(other, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None and "head size 48" in why[0]
+    other = TorchEncoderLM(vocab=500, seq=64)
+    for layer in other.layers:
+        layer.self_attn.batch_first = False
+    pipe = pp.pipeline(other, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None and "batch_first" in why[0]
+
+
+@pytest.mark.parametrize("norm_first", [True, False])
+def test_torchs_encoder_stack_is_recognised_through_its_exported_graph(norm_first):
+    """``nn.TransformerEncoder`` goes through torch.export; ``nn.MultiheadAttention`` applies its packed
+    q|k|v parameters and its output projection as functions of parameters, which are taken as linear layers
+    (views of the same parameter objects); the sequence-major reshaping inside is not parsed but checked."""
+    import os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchEncoderStackLM
+    from pippy_amd._lowering import lower_stage_module
+    torch.manual_seed(0)
+    model = TorchEncoderStackLM(vocab=500, seq=64, norm_first=norm_first)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"encoder.layers.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    x = ids
+    for i in range(2):
+        why = []
+        blocks = lower_stage_module(pipe.get_stage_module(i), why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2
+        for b, own in zip(layers, model.encoder.layers[2 * i:2 * i + 2]):
+            assert b.attn.c_attn.weight is own.self_attn.in_proj_weight
+            assert b.attn.c_proj.weight is own.self_attn.out_proj.weight and b.mlp.c_fc is own.linear1
+            assert (b.pre_ln, b.causal, b.n_heads, b.activation) == (norm_first, False, 2, "gelu_erf")
+        with torch.no_grad():
+            for b in blocks:
+                x = b(x)
+    torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)

@@ -1126,6 +1126,58 @@ def test_hugging_face_gpt2_runs_natively_and_matches_the_oracle():
     _exported_model_against_the_oracle(model, Logits, 1000, 128, "transformer.h.2")
 
 
+@pytest.mark.parametrize("norm_first,activation", [(True, "gelu"), (False, "relu")])
+def test_torchs_own_encoder_layers_run_natively_and_match_the_oracle(norm_first, activation):
+    """A model built from ``nn.TransformerEncoderLayer`` (torch.fx keeps each layer whole): both stages
+    run as launch lists on the layers' own parameters, the packed q|k|v weight of ``nn.MultiheadAttention``
+    included, and match the fp32 oracle run of the same model."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchEncoderLM
+    torch.manual_seed(0)
+    model = TorchEncoderLM(vocab=1000, seq=128, d=128, h=2, L=4, norm_first=norm_first, activation=activation)
+    _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "layers.2",
+                                       before_oracle=_relu_sets_of_torch_layers if activation == "relu" else None)
+
+
+def test_torchs_encoder_stack_runs_natively_and_matches_the_oracle():
+    """The layers inside ``nn.TransformerEncoder``: exported, recognised on the parameters that
+    ``nn.MultiheadAttention`` applies as functions, run as launch lists."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchEncoderStackLM
+    torch.manual_seed(0)
+    model = TorchEncoderStackLM(vocab=1000, seq=128, d=128, h=2, L=4)
+    _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "encoder.layers.2")
+
+
+def _relu_sets_of_torch_layers(ref, stages, M):
+    """The run's ReLU active sets for a model of ``nn.TransformerEncoderLayer``s (see _relu_sets_of_the_run)."""
+    import torch.nn as nn
+    layers = [m for m in ref.modules() if isinstance(m, nn.TransformerEncoderLayer)]
+    at = 0
+    for st in stages:
+        count = 0
+        for m in range(M):
+            hs = [v for k, v in st.saved_activations(m).items() if k.split(".")[-1] == "h"]
+            count = len(hs)
+            for j, h in enumerate(hs):
+                layers[at + j].__dict__.setdefault("_sets", []).append((h > 0).cpu())
+        at += count
+    assert at == len(layers)
+    for layer in layers:
+        sets = layer.__dict__["_sets"]
+
+        def forced(x, sets=sets):
+            active = sets.pop(0).reshape(x.shape)
+            flipped = active != (x > 0)
+            assert flipped.float().mean() < 0.02 and (not flipped.any() or x[flipped].abs().max() < 2e-2 * x.abs().max())
+            return x * active
+
+        layer.activation = forced
+        layer.activation_relu_or_gelu = 0
+
+
 def test_exported_stages_that_do_not_lower_run_through_autograd_on_the_gpu():
     """An exported model whose attention mask is not the causal one (a sliding window) keeps its stages
     with torch autograd.  Their graphs were exported on the host: the folded constants (mask, position
