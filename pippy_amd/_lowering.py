@@ -505,8 +505,10 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         return "act" if _activation_of(n, root) is not None else type(m).__name__
 
     kinds = [kind(n, m) for n, m in mods]
-    if kinds == ["RMSNorm", "act"] and _activation_of(mods[1][0], root) == "silu":
-        return _classify_expert_branch(root, mods[0][1], state)
+    # (a router applied as a function of its weight is among the parameters the expert branch reads)
+    modules = [(n, m) for n, m in mods if not isinstance(m, LinearView)]
+    if [kind(n, m) for n, m in modules] == ["RMSNorm", "act"] and _activation_of(modules[1][0], root) == "silu":
+        return _classify_expert_branch(root, modules[0][1], state)
     if len(soft) == 1 and kinds and set(kinds[1:]) == {"Linear"} and kinds[-1] == "Linear":
         # attention spelled out (softmax(q k^T) v between the projections): the softmax stands for the call
         mods.insert(len(mods) - 1, (soft[0], None))
