@@ -231,18 +231,27 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 
 # ---- transformers written with plain torch layers ---------------------------------------------------
 # Recognised, in this order along the stage:
-#  * an optional embedding front: a token table, optionally plus a position table indexed by 0 .. S-1
-#    (GPT-2), or word + position + token-type-0 tables under a LayerNorm (BERT);
-#  * any number of residual pairs, attention then feed-forward, of one of three forms
-#      pre-LayerNorm    x = x + proj(sdpa(qkv(ln(x))))                 x = x + fc2(gelu(fc1(ln(x))))
-#      post-LayerNorm   x = ln(x + proj(sdpa(qkv(x))))                 x = ln(x + fc2(gelu(fc1(x))))
-#      rotary, gated    x = x + o(sdpa(rope(q(n(x)), k(n(x))), v(n(x)))) x = x + down(silu(gate(n(x))) * up(n(x)))
-#    where qkv is one fused projection or three separate ones, the affine layers are ``nn.Linear`` or
-#    layers with an [in, out] weight, the activations are functions, torch.nn modules or a library's own
-#    activation classes, n is an RMS norm, attention is ``scaled_dot_product_attention`` with
-#    ``is_causal``, no mask, or a constant mask that is causal or masks nothing, and the rotary tables
-#    are constants of the (exported) stage;
-#  * an optional tail: projections with activations, a final norm, the vocabulary projection.
+#  * an optional embedding front: a token table, optionally plus a position table read at k .. k+S-1
+#    (GPT-2; OPT reads from row 2 on), or word + position + token-type-0 tables, under a LayerNorm (BERT) or
+#    not (a pre-LayerNorm encoder), the positions 0 .. S-1 or counted over the tokens that are not padding
+#    (RoBERTa);
+#  * any number of layers: a whole ``nn.TransformerEncoderLayer`` (batch first, no mask), or a residual
+#    pair, attention then feed-forward, of one of these forms
+#      pre-LayerNorm    x = x + proj(attn(qkv(ln(x))))                 x = x + fc2(act(fc1(ln(x))))
+#      post-LayerNorm   x = ln(x + proj(attn(qkv(x))))                 x = ln(x + fc2(act(fc1(x))))
+#      rotary, gated    x = x + o(attn(rope(q(n(x)), k(n(x))), v(n(x)))) x = x + down(silu(gate(n(x))) * up(n(x)))
+#      rotary, experts  the same attention; x = x + (two of E gated experts per token, weights in stacked
+#                       tensors, chosen by a softmax router)
+#    where qkv is one fused projection or three separate ones; the affine layers are ``nn.Linear``, layers
+#    with an [in, out] weight, or ``linear`` applied as a function to parameters; act is tanh-GELU,
+#    erf-GELU or ReLU, as a function, a torch.nn module or a library's own activation class; n is an RMS
+#    norm, and queries and keys may have an RMS norm over each head's values in front of the rotary
+#    embedding; attn is ``scaled_dot_product_attention`` or softmax(q k^T c + mask) v spelled out, with
+#    ``is_causal``, no mask, or a constant mask that is causal or masks nothing, and any constant factor
+#    c on the scores (also applied to queries or keys beforehand); the rotary tables are constants of the
+#    (exported) stage, and their width is the head size;
+#  * an optional tail: norms and projections with activations, then a final norm and / or the vocabulary
+#    projection.
 # The walk only looks at which layers feed which residual add; how the model reshapes between them is
 # not parsed but checked: the torch statement of the recognised blocks must reproduce the stage's own
 # forward on a random input (fp32, on the host), otherwise the stage stays with torch autograd.
