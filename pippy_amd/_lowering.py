@@ -172,6 +172,15 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
         i += 1
     if not blocks:
         raise NotLowerable("the stage holds no layer")
+    # a last projection onto a width that is no multiple of 8 (a vocabulary of 50257): the head block keeps
+    # its weight rows and its output padded to one, which the GEMM and the loss kernel need
+    last = blocks[-1]
+    if type(last) is LinearAct and last.activation is None and isinstance(last.lin, nn.Linear) \
+            and last.lin.weight.dtype == torch.bfloat16 and last.lin.out_features % 8:
+        norm = None
+        if len(blocks) > 1 and type(blocks[-2]) in (LayerNormBlock, RMSNormBlock):
+            norm = blocks[-2].ln if type(blocks[-2]) is LayerNormBlock else blocks[-2].norm
+        blocks = blocks[:-2 if norm is not None else -1] + [WrappedLMHead(norm, last.lin)]
     return blocks
 
 

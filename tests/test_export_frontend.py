@@ -348,6 +348,11 @@ def test_torchs_own_encoder_layers_become_transformer_blocks(norm_first, activat
             for b in blocks:
                 x = b(x)
     torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+    # a last projection onto a width that is no multiple of 8 becomes the head block (padded rows) in bf16
+    odd = TorchEncoderLM(vocab=501, seq=64, norm_first=norm_first, activation=activation).to(torch.bfloat16)
+    pipe = pp.pipeline(odd, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    tail = lower_stage_module(pipe.get_stage_module(1), [])[-1]
+    assert type(tail).__name__ == "WrappedLMHead" and tail.lm_head is odd.head and tail.ln_f is odd.norm
     # sequence-major layers and head sizes the kernels do not have stay with torch, with the reason
     other = TorchEncoderLM(vocab=500, seq=64, d=96, h=2)
     pipe = pp.pipeline(other, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
