@@ -976,6 +976,25 @@ def _check_kernel_requirements(submod: nn.Module, blocks: List[NativeBlock]) -> 
         if not plain:
             raise NotLowerable(f"float32 parameters: {type(blk).__name__} runs as bfloat16 kernels only (convert the "
                                "model with .to(torch.bfloat16) to run it as launch lists)")
+    if dtypes == {torch.bfloat16}:
+        # the bf16 kernels move 16-byte groups: widths are multiples of 8, except where a block keeps a
+        # weight's rows padded (a vocabulary projection, a router)
+        padded = set()
+        for blk in blocks:
+            for m in blk.modules():
+                padded |= {id(p) for p, _ in getattr(m, "_pp_padded_rows", lambda: [])()}
+        for blk in blocks:
+            for name, m in blk.named_modules():
+                if isinstance(m, (nn.Linear, InOutLinear)):
+                    widths = [("in", m.in_features)] + ([] if id(m.weight) in padded else [("out", m.out_features)])
+                elif isinstance(m, (nn.LayerNorm, nn.Embedding)):
+                    widths = [("", m.weight.shape[-1])] if getattr(m, "weight", None) is not None else []
+                else:
+                    continue
+                for which, w in widths:
+                    if w % 8:
+                        raise NotLowerable(f"{type(m).__name__} '{name}' of {type(blk).__name__} has {which + ' ' if which else ''}"
+                                           f"width {w}; the bfloat16 kernels take multiples of 8")
 
 
 def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None, for_kernels: bool = False) -> Optional[List[NativeBlock]]:

@@ -238,6 +238,16 @@ def test_what_the_kernels_cannot_take_keeps_a_recognised_stage_with_torch():
     # any sequence length: the layers pad to a multiple of 64 by themselves
     stage = pp.pipeline(model, 1, (ids[:, :48],), split_spec={"h.2": pp.SplitPoint.BEGINNING}).get_stage_module(1)
     assert lower_stage_module(stage, why, for_kernels=True) is not None
+    # widths: the bf16 kernels move groups of 8 values; fp32 chains of linear layers take any width; a
+    # vocabulary projection keeps its rows padded and may have any number of them
+    chain = nn.Sequential(nn.Linear(64, 100), nn.ReLU(), nn.Linear(100, 8))
+    assert lower_stage_module(chain, why, for_kernels=True) is not None
+    del why[:]
+    assert lower_stage_module(chain.to(torch.bfloat16), why, for_kernels=True) is None
+    assert "out width 100" in why[0] and "multiples of 8" in why[0]
+    head = nn.Sequential(nn.Linear(64, 64), nn.LayerNorm(64), nn.Linear(64, 1001, bias=False)).to(torch.bfloat16)
+    blocks = lower_stage_module(head, why, for_kernels=True)
+    assert blocks is not None and type(blocks[-1]).__name__ == "WrappedLMHead"
 
 
 def test_a_layer_subclass_with_a_forward_of_its_own_is_not_put_back_blindly():
