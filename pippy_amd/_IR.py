@@ -488,22 +488,14 @@ class Pipe(nn.Module):
         split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks, args_chunk_spec,
                                       kwargs_chunk_spec)
         names = list(split_spec.keys()) if split_spec else None
-        root = mod
-        try:
-            graph = _ModuleGranularityTracer(names).trace(mod)
-            if split_spec:
-                _insert_markers(graph, split_spec)
-        except Exception as fx_error:
-            # symbolic tracing cannot follow this model: export it on the first microbatch's inputs, as
-            # the reference does (``_IR.py:1172-1185``); the stages are then ATen-level graphs
-            logger.warning(f"torch.fx symbolic tracing failed ({type(fx_error).__name__}: {fx_error}); "
-                           "falling back to torch.export on the inputs of one microbatch: the stages hold "
-                           "that microbatch's shapes; standard layers are put back into the ATen-level graph, "
-                           "and a stage whose structure is then recognised still runs as HIP launch lists")
+
+        def exported(fx_error):
+            """(root, graph) over torch.export on the first microbatch's inputs, as the reference traces
+            (``_IR.py:1172-1185``); the stages are then ATen-level graphs."""
             args_split, kwargs_split = split_args_kwargs_into_chunks(example_args, example_kwargs, num_chunks,
                                                                      args_chunk_spec, kwargs_chunk_spec)
             try:
-                root, graph = _export_and_mark(mod, args_split[0], kwargs_split[0], split_spec)
+                return _export_and_mark(mod, args_split[0], kwargs_split[0], split_spec)
             except ValueError:
                 raise
             except Exception as export_error:
@@ -518,10 +510,44 @@ class Pipe(nn.Module):
                     f"pipeline(): neither torch.fx symbolic tracing ({type(fx_error).__name__}: {fx_error}) "
                     f"nor torch.export ({type(export_error).__name__}: {export_error}) can trace this model{hint}"
                 ) from export_error
-        if split_policy is not None:
-            gm = split_policy(fx.GraphModule(root, graph))
-            graph = gm.graph
-        pipe = Pipe._from_traced(root, graph)
+
+        def build(root, graph):
+            if split_policy is not None:
+                graph = split_policy(fx.GraphModule(root, graph)).graph
+            return Pipe._from_traced(root, graph)
+
+        def widest_boundary(pipe):
+            return max([len([n for n in pipe.get_stage_module(i).graph.nodes if n.op == "placeholder"])
+                        for i in range(1, pipe.num_stages)] or [0])
+
+        try:
+            graph = _ModuleGranularityTracer(names).trace(mod)
+            if split_spec:
+                _insert_markers(graph, split_spec)
+        except Exception as fx_error:
+            # symbolic tracing cannot follow this model
+            logger.warning(f"torch.fx symbolic tracing failed ({type(fx_error).__name__}: {fx_error}); "
+                           "falling back to torch.export on the inputs of one microbatch: the stages hold "
+                           "that microbatch's shapes; standard layers are put back into the ATen-level graph, "
+                           "and a stage whose structure is then recognised still runs as HIP launch lists")
+            pipe = build(*exported(fx_error))
+        else:
+            pipe = build(mod, graph)
+            if widest_boundary(pipe) > 1:
+                # a symbolically traced forward keeps what it computes from shapes (a mask built from the
+                # sequence length, say) as values that travel from stage to stage; exported on an example
+                # they are constants of each stage.  The exported pipeline is taken when that leaves fewer
+                # values on the boundaries; otherwise (real skip connections) the traced one stays.
+                try:
+                    other = build(*exported(None))
+                except Exception:
+                    other = None
+                if other is not None and other.num_stages == pipe.num_stages and \
+                        widest_boundary(other) < widest_boundary(pipe):
+                    logger.warning("the symbolically traced stages would hand more than one tensor on (values "
+                                   "computed from shapes); using torch.export on the inputs of one microbatch "
+                                   "instead, where they are constants: the stages hold that microbatch's shapes")
+                    pipe = other
         pipe.pipe_info = PipeInfo(graph=pipe.split_gm.graph, num_stages=pipe.num_stages,
                                   num_chunks=num_chunks, has_loss_and_backward=False,
                                   args_chunk_spec=args_chunk_spec, kwargs_chunk_spec=kwargs_chunk_spec)

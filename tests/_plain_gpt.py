@@ -128,3 +128,23 @@ class TorchEncoderStackLM(nn.Module):
     def forward(self, ids):
         x = self.emb(ids) + self.pos(torch.arange(ids.shape[1], device=ids.device))
         return self.head(self.encoder(x))
+
+
+class TorchCausalLM(nn.Module):
+    """A decoder-only language model the way tutorials build it from torch's encoder layers: a causal
+    mask made in forward from the sequence length, handed to every layer."""
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4, flag=True):
+        super().__init__()
+        self.flag = flag
+        self.emb = nn.Embedding(vocab, d); self.pos = nn.Embedding(seq, d)
+        self.layers = nn.ModuleList([nn.TransformerEncoderLayer(d, h, 4 * d, dropout=0.0, activation="gelu",
+                                                                batch_first=True, norm_first=True)
+                                     for _ in range(L)])
+        self.norm = nn.LayerNorm(d); self.head = nn.Linear(d, vocab, bias=False)
+    def forward(self, ids):
+        S = ids.shape[1]
+        x = self.emb(ids) + self.pos(torch.arange(S, device=ids.device))
+        mask = nn.Transformer.generate_square_subsequent_mask(S, device=ids.device)
+        for layer in self.layers:
+            x = layer(x, src_mask=mask, is_causal=True) if self.flag else layer(x, src_mask=mask)
+        return self.head(self.norm(x))

@@ -406,3 +406,50 @@ def test_torchs_encoder_stack_is_recognised_through_its_exported_graph(norm_firs
             for b in blocks:
                 x = b(x)
     torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("flag", [True, False])
+def test_values_computed_from_shapes_do_not_travel_between_stages(flag, caplog):
+    """torch.fx can trace this model (each encoder layer is one call), but the causal mask that forward
+    builds from the sequence length would then be a second tensor on every stage boundary.  The front end
+    notices, exports the model instead, where the mask is a constant of each stage, and says so; the
+    stages are then recognised as causal transformer layers.  A real skip connection keeps the traced
+    pipeline (its exported form has the same boundary)."""
+    import logging, os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchCausalLM
+    from pippy_amd._lowering import lower_stage_module
+    torch.manual_seed(0)
+    model = TorchCausalLM(vocab=500, seq=64, flag=flag)
+    ids = torch.randint(0, 500, (2, 40))
+    with caplog.at_level(logging.WARNING, logger="pippy_amd._IR"):
+        pipe = pp.pipeline(model, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    assert "more than one tensor" in caplog.text
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    for i in range(2):
+        sm = pipe.get_stage_module(i)
+        assert len([n for n in sm.graph.nodes if n.op == "placeholder"]) == 1
+        why = []
+        blocks = lower_stage_module(sm, why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2 and all(b.causal and b.pre_ln for b in layers)
+
+    class Skip(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b, self.c = nn.Linear(16, 16), nn.Linear(16, 16), nn.Linear(16, 16)
+
+        def forward(self, x):
+            first = torch.relu(self.a(x))
+            pp.pipe_split()
+            y = torch.relu(self.b(first))
+            pp.pipe_split()
+            return self.c(y + first)
+
+    caplog.clear()
+    with caplog.at_level(logging.WARNING, logger="pippy_amd._IR"):
+        skip = pp.pipeline(Skip(), 1, (torch.randn(4, 16),))
+    assert "more than one tensor" not in caplog.text and skip.num_stages == 3
+    assert any(n.op == "call_module" and n.target == "b" for n in skip.get_stage_module(1).graph.nodes)

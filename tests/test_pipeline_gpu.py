@@ -1141,6 +1141,18 @@ def test_torchs_own_encoder_layers_run_natively_and_match_the_oracle(norm_first,
                                        before_oracle=_relu_sets_of_torch_layers if activation == "relu" else None)
 
 
+def test_a_causal_model_of_torchs_encoder_layers_runs_natively_and_matches_the_oracle():
+    """A decoder-only model made of ``nn.TransformerEncoderLayer`` with a causal mask built in forward
+    from the sequence length: exported (so that the mask is a constant of each stage), recognised as
+    causal layers, run as launch lists."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TorchCausalLM
+    torch.manual_seed(0)
+    model = TorchCausalLM(vocab=1000, seq=128, d=128, h=2, L=4)
+    _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "layers.2")
+
+
 def test_torchs_encoder_stack_runs_natively_and_matches_the_oracle():
     """The layers inside ``nn.TransformerEncoder``: exported, recognised on the parameters that
     ``nn.MultiheadAttention`` applies as functions, run as launch lists."""
