@@ -86,6 +86,12 @@ class _ModuleGranularityTracer(fx.Tracer):
     def is_leaf_module(self, m: nn.Module, qualname: str) -> bool:
         if isinstance(m, NativeBlock):
             return True
+        if next(m.children(), None) is None and not type(m).__module__.startswith("torch.nn"):
+            # a library's or a user's own affine layer, norm or activation stays one call, as torch.nn's do
+            from .stage_modules import activation_like, in_out_linear_like, layer_norm_like, rms_norm_like
+            if in_out_linear_like(m) or activation_like(m) is not None or rms_norm_like(m) is not None \
+                    or layer_norm_like(m) is not None:
+                return True
         if self._split_names is None:
             return super().is_leaf_module(m, qualname)
         # descend only into modules that contain a split point
@@ -138,12 +144,14 @@ def _drop_noop_casts(gm: fx.GraphModule) -> None:
                 gm.graph.erase_node(n)
 
 
-def _fold_constants(gm: fx.GraphModule) -> None:
-    """Evaluates, once, every part of an exported graph that depends on no model input and no parameter
-    (position indices, attention masks built from the example's sequence length, ...), and replaces it by
-    non-persistent buffers of ``gm``.  Stages then receive only activations from their predecessor
-    instead of also such tensors computed by the first stage, and a stage's graph shows a constant mask
-    as what it is."""
+def _fold_constants(gm: fx.GraphModule, state: frozenset = frozenset()) -> None:
+    """Evaluates, once, every part of an exported graph that depends on no model input and no part of the
+    model's state (position indices, attention masks built from the example's sequence length, ...), and
+    replaces it by non-persistent buffers of ``gm``.  Stages then receive only activations from their
+    predecessor instead of also such tensors computed by the first stage, and a stage's graph shows a
+    constant mask as what it is.  ``state``: the names of the model's persistent buffers; like parameters
+    they may be loaded from a checkpoint after the pipeline is built, so what is computed from them stays
+    in the graph (and they stay in their stage's state_dict)."""
     graph = gm.graph
     value: Dict[fx.Node, Any] = {}
     for n in graph.nodes:
@@ -154,7 +162,7 @@ def _fold_constants(gm: fx.GraphModule) -> None:
                 continue
             written = any(u.op == "call_function" and getattr(getattr(u.target, "_schema", None), "is_mutable", False)
                           and u.target is not torch.ops.aten.detach_.default for u in n.users)
-            if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) and not written:
+            if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) and not written and n.target not in state:
                 value[n] = obj
             elif isinstance(obj, fx.GraphModule):
                 value[n] = obj     # the body of a higher-order operator (below)
@@ -213,7 +221,7 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
     unchanged.  Besides the torch.nn types this covers layers of other libraries that are recognisably
     an affine map with an [in, out] weight or an elementwise activation (checked on sample values, and
     their exported nodes are checked against the layer itself)."""
-    from .stage_modules import activation_like, in_out_linear_like, rms_norm_like
+    from .stage_modules import activation_like, in_out_linear_like, layer_norm_like, rms_norm_like
     graph = gm.graph
     leaves = {}
     for name, m in mod.named_modules():
@@ -224,7 +232,8 @@ def _reroll_leaf_layers(mod: nn.Module, gm: fx.GraphModule) -> None:
             # a subclass with a forward of its own (a position table that shifts its indices, say) is
             # put back only if that forward is what the exported nodes compute
             leaves[name] = (m, type(m).forward is not base.forward, base)
-        elif in_out_linear_like(m) or activation_like(m) is not None or rms_norm_like(m) is not None:
+        elif in_out_linear_like(m) or activation_like(m) is not None or rms_norm_like(m) is not None \
+                or layer_norm_like(m) is not None:
             leaves[name] = (m, True, None)
     calls: Dict[Tuple[str, str], List[fx.Node]] = {}
     for n in graph.nodes:
@@ -309,7 +318,7 @@ def _export_and_mark(mod: nn.Module, mb_args: Tuple[Any, ...], mb_kwargs: Option
                 (n.op == "call_function" and n.target is torch.ops.aten._assert_tensor_metadata.default):
             graph.erase_node(n)   # guards of the example inputs' shapes and dtypes: stages re-check nothing
     _drop_noop_casts(gm)
-    _fold_constants(gm)
+    _fold_constants(gm, frozenset(k for k, _ in mod.named_buffers()) & frozenset(mod.state_dict().keys()))
     _reroll_leaf_layers(mod, gm)
     # what nothing reads (a pooling head whose result the model drops, say) would otherwise give the last
     # layer a second reader; split markers and in-place operators stay

@@ -21,7 +21,7 @@ import torch.nn.functional as F
 from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, LinearView, NativeBlock, RMSNormBlock, RMSNormLike,
                             StageSequence, torch_encoder_layer_block, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer,
                             WrappedTokenEmbedding,
-                            WrappedTransformerLayer, activation_like, in_out_linear_like, rms_norm_like)
+                            WrappedTransformerLayer, activation_like, in_out_linear_like, layer_norm_like, rms_norm_like)
 
 _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GELU, nn.Identity, nn.Dropout,
                nn.Embedding)
@@ -30,7 +30,7 @@ _LEAF_TYPES = (NativeBlock, nn.Linear, nn.LayerNorm, nn.RMSNorm, nn.ReLU, nn.GEL
 class _ChainTracer(fx.Tracer):
     def is_leaf_module(self, m, qualname):
         return isinstance(m, _LEAF_TYPES + (nn.TransformerEncoderLayer,)) or in_out_linear_like(m) \
-            or activation_like(m) is not None \
+            or activation_like(m) is not None or layer_norm_like(m) is not None \
             or rms_norm_like(m) is not None or super().is_leaf_module(m, qualname)
 
 
@@ -42,6 +42,13 @@ def _as_linear(m: nn.Module) -> Optional[nn.Module]:
     if in_out_linear_like(m):
         return InOutLinear(m)
     return None
+
+
+def _layer_of(root: nn.Module, target: str) -> nn.Module:
+    """The submodule ``target`` of ``root``, seen as the torch.nn layer it amounts to where it is a layer of
+    another library (an affine layer with an [in, out] weight, an RMS norm, a layer norm)."""
+    m = root.get_submodule(target)
+    return _as_linear(m) or _as_rms_norm(m) or layer_norm_like(m) or m
 
 
 def _as_rms_norm(m: nn.Module) -> Optional[nn.Module]:
@@ -141,8 +148,7 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
             continue
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' is not a module call or a supported activation")
-        m = root.get_submodule(n.target)
-        m = _as_linear(m) or m
+        m = _layer_of(root, n.target)
         if isinstance(m, NativeBlock):
             blocks.append(m)
         elif isinstance(m, nn.TransformerEncoderLayer):
@@ -164,6 +170,8 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
         elif isinstance(m, nn.RMSNorm):
             if len(m.normalized_shape) != 1 or m.weight is None or m.eps is None:
                 raise NotLowerable(f"RMSNorm '{n.target}' needs one normalised dimension, a weight and an eps")
+            blocks.append(RMSNormBlock(m))
+        elif isinstance(m, RMSNormLike):
             blocks.append(RMSNormBlock(m))
         else:
             # a user container (e.g. a block that wraps a linear and an activation): lower it as
@@ -296,17 +304,39 @@ def _branch_layers(y: fx.Node, stream: fx.Node, order: dict, state: bool = False
     return sorted(found, key=order.get)
 
 
-def _constant_of(root: nn.Module, node) -> Optional[torch.Tensor]:
-    """The tensor behind a ``get_attr`` node that reads a buffer or constant of ``root``, else None."""
-    if not isinstance(node, fx.Node) or node.op != "get_attr":
+def _constant_of(root: nn.Module, node, depth: int = 0) -> Optional[torch.Tensor]:
+    """The tensor behind a ``get_attr`` node that reads a buffer or constant of ``root``, or what a few
+    ATen operators make of such tensors (a mask cut out of a registered lower-triangular buffer and
+    compared with zero: persistent buffers are not folded when a model is exported), else None."""
+    if not isinstance(node, fx.Node):
         return None
-    obj = root
+    if node.op == "get_attr":
+        obj = root
+        try:
+            for part in str(node.target).split("."):
+                obj = getattr(obj, part)
+        except AttributeError:
+            return None
+        return obj if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) else None
+    if node.op != "call_function" or not isinstance(node.target, torch._ops.OpOverload) or depth > 16:
+        return None
+    op = node.target
+    if op.namespace != "aten" or op._schema.is_mutable or torch.Tag.nondeterministic_seeded in op.tags:
+        return None
+    inputs = {}
+    for a in node.all_input_nodes:
+        value = _constant_of(root, a, depth + 1)
+        if value is None or value.numel() > (1 << 26):
+            return None
+        inputs[a] = value
+    if not inputs:
+        return None
     try:
-        for part in str(node.target).split("."):
-            obj = getattr(obj, part)
-    except AttributeError:
+        with torch.no_grad():
+            out = op(*fx.node.map_arg(node.args, lambda a: inputs[a]), **fx.node.map_arg(node.kwargs, lambda a: inputs[a]))
+    except Exception:
         return None
-    return obj if torch.is_tensor(obj) and not isinstance(obj, nn.Parameter) else None
+    return out if torch.is_tensor(out) else None
 
 
 def _parameter_of(root: nn.Module, node) -> Optional[nn.Parameter]:
@@ -497,8 +527,7 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         if _activation_of(n, root) == "identity":
             continue
         if n.op == "call_module":
-            m = root.get_submodule(n.target)
-            mods.append((n, _as_linear(m) or _as_rms_norm(m) or m))
+            mods.append((n, _layer_of(root, n.target)))
         elif n.op == "call_function" and n.target in _LINEAR_FNS:
             # (nn.MultiheadAttention applies its packed q|k|v parameters and its output projection this way)
             weight = _parameter_of(root, n.args[1])
@@ -520,6 +549,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             return "Linear"
         if isinstance(m, (nn.RMSNorm, RMSNormLike)):
             return "RMSNorm"
+        if isinstance(m, nn.LayerNorm):
+            return "LayerNorm"
         return "act" if _activation_of(n, root) is not None else type(m).__name__
 
     kinds = [kind(n, m) for n, m in mods]
@@ -633,7 +664,7 @@ def _only_layer_user(root: nn.Module, node: fx.Node) -> Tuple[Optional[fx.Node],
     """(user, its module) when ``node`` feeds exactly one layer call, else (None, None)."""
     users = list(node.users)
     if len(users) == 1 and users[0].op == "call_module":
-        return users[0], root.get_submodule(users[0].target)
+        return users[0], _layer_of(root, users[0].target)
     return None, None
 
 
@@ -761,8 +792,7 @@ def _tail_blocks(root: nn.Module, stream: fx.Node, result: fx.Node, after_layers
             continue
         if n.op != "call_module":
             raise NotLowerable(f"'{n.format_node()}' after the last residual addition")
-        m = root.get_submodule(n.target)
-        mods.append(_as_linear(m) or _as_rms_norm(m) or m)
+        mods.append(_layer_of(root, n.target))
     blocks: List[NativeBlock] = []
     head: List[NativeBlock] = []
     norm_types, linear_types = (nn.LayerNorm, nn.RMSNorm, RMSNormLike), (nn.Linear, InOutLinear)
@@ -895,7 +925,7 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
         raise NotLowerable(f"torch.fx cannot trace {type(submod).__name__}: {type(e).__name__}: {e}") from e
     widths = {m.normalized_shape[0] for m in submod.modules()
               if isinstance(m, (nn.LayerNorm, nn.RMSNorm)) and len(m.normalized_shape) == 1}
-    widths |= {m.weight.shape[0] for m in submod.modules() if rms_norm_like(m) is not None}
+    widths |= {m.weight.shape[0] for m in submod.modules() if rms_norm_like(m) is not None or layer_norm_like(m) is not None}
     if len(widths) > 1 and all(w in (64, 128) for w in widths - {max(widths)}):
         widths = {max(widths)}       # (norms over the values of one head, on queries and keys)
     if len(widths) != 1:

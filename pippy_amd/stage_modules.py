@@ -1273,6 +1273,56 @@ def rms_norm_like(m: nn.Module) -> Optional[float]:
     return found
 
 
+class LayerNormView(nn.LayerNorm):
+    """An ``nn.LayerNorm`` around the parameters of a user's own layer-norm layer (the same parameter
+    objects; a layer without a bias gives ``bias = None``)."""
+
+    def __init__(self, weight: nn.Parameter, bias: Optional[nn.Parameter], eps: float):
+        nn.Module.__init__(self)
+        self.normalized_shape, self.eps, self.elementwise_affine = (weight.shape[0],), eps, True
+        self.weight = weight
+        if bias is None:
+            self.register_parameter("bias", None)
+        else:
+            self.bias = bias
+
+
+def layer_norm_like(m: nn.Module) -> Optional[LayerNormView]:
+    """An ``nn.LayerNorm`` view of a leaf layer that is not one but computes one over the last dimension
+    with its 1-d ``weight`` and optional 1-d ``bias`` (decided by running a float32 copy on rows of small
+    variance, which also tells its epsilon: the attribute ``eps`` / ``variance_epsilon`` / ``epsilon`` if
+    there is one, else 1e-5, 1e-6 or 1e-12), else None."""
+    import copy
+    if isinstance(m, (nn.LayerNorm, nn.RMSNorm)) or next(m.children(), None) is not None \
+            or next(m.buffers(), None) is not None:
+        return None
+    params = dict(m.named_parameters(recurse=False))
+    w, bias = params.get("weight"), params.get("bias")
+    if w is None or not set(params) <= {"weight", "bias"} or w.dim() != 1 or (bias is not None and bias.shape != w.shape):
+        return None
+    cached = m.__dict__.get("_pp_layer_norm_like", 0)      # (kept out of the layer's registered submodules)
+    if cached != 0:
+        return cached
+    found = None
+    named = [getattr(m, a) for a in ("eps", "variance_epsilon", "epsilon") if isinstance(getattr(m, a, None), float)]
+    try:
+        probe = copy.deepcopy(m).float().cpu()
+        pw, pb = probe.weight, getattr(probe, "bias", None)
+        with torch.no_grad():
+            g = torch.Generator().manual_seed(0)
+            x = torch.randn(3, 2, w.shape[0], generator=g) * 1e-3 + torch.randn(3, 2, 1, generator=g)
+            got = probe(x)
+            for eps in named or (1e-5, 1e-6, 1e-12):
+                want = F.layer_norm(x, (w.shape[0],), pw, pb, eps)
+                if got.shape == want.shape and bool((got - want).abs().max() <= 1e-4 * want.abs().max() + 1e-7):
+                    found = LayerNormView(w, bias, eps)
+                    break
+    except Exception:
+        found = None
+    m.__dict__["_pp_layer_norm_like"] = found
+    return found
+
+
 def _is_rms(norm) -> bool:
     return isinstance(norm, (nn.RMSNorm, RMSNormLike))
 

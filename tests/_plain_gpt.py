@@ -148,3 +148,72 @@ class TorchCausalLM(nn.Module):
         for layer in self.layers:
             x = layer(x, src_mask=mask, is_causal=True) if self.flag else layer(x, src_mask=mask)
         return self.head(self.norm(x))
+
+
+# ---- a GPT in the style of small teaching code bases ------------------------------------------------------
+# (a layer norm class of its own with an optional bias, a ModuleDict of parts, attention through the fused
+# call or spelled out against a registered lower-triangular buffer, linear layers with or without biases)
+import math
+
+
+class OwnLayerNorm(nn.Module):
+    def __init__(self, d, bias):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(d) + 0.1 * torch.randn(d))
+        self.bias = nn.Parameter(0.1 * torch.randn(d)) if bias else None
+    def forward(self, x):
+        return F.layer_norm(x, self.weight.shape, self.weight, self.bias, 1e-5)
+class TeachingAttention(nn.Module):
+    def __init__(self, d, h, seq, bias, flash):
+        super().__init__()
+        self.c_attn = nn.Linear(d, 3 * d, bias=bias); self.c_proj = nn.Linear(d, d, bias=bias)
+        self.attn_dropout = nn.Dropout(0.0); self.resid_dropout = nn.Dropout(0.0)
+        self.n_head, self.n_embd, self.flash = h, d, flash
+        if not flash:
+            self.register_buffer("bias", torch.tril(torch.ones(seq, seq)).view(1, 1, seq, seq))
+    def forward(self, x):
+        B, T, C = x.size()
+        q, k, v = self.c_attn(x).split(self.n_embd, dim=2)
+        k = k.view(B, T, self.n_head, C // self.n_head).transpose(1, 2)
+        q = q.view(B, T, self.n_head, C // self.n_head).transpose(1, 2)
+        v = v.view(B, T, self.n_head, C // self.n_head).transpose(1, 2)
+        if self.flash:
+            y = F.scaled_dot_product_attention(q, k, v, attn_mask=None, dropout_p=0.0, is_causal=True)
+        else:
+            att = (q @ k.transpose(-2, -1)) * (1.0 / math.sqrt(k.size(-1)))
+            att = att.masked_fill(self.bias[:, :, :T, :T] == 0, float("-inf"))
+            att = self.attn_dropout(F.softmax(att, dim=-1))
+            y = att @ v
+        y = y.transpose(1, 2).contiguous().view(B, T, C)
+        return self.resid_dropout(self.c_proj(y))
+class TeachingMLP(nn.Module):
+    def __init__(self, d, bias):
+        super().__init__()
+        self.c_fc = nn.Linear(d, 4 * d, bias=bias); self.gelu = nn.GELU()
+        self.c_proj = nn.Linear(4 * d, d, bias=bias); self.dropout = nn.Dropout(0.0)
+    def forward(self, x):
+        return self.dropout(self.c_proj(self.gelu(self.c_fc(x))))
+class TeachingBlock(nn.Module):
+    def __init__(self, d, h, seq, bias, flash):
+        super().__init__()
+        self.ln_1 = OwnLayerNorm(d, bias); self.attn = TeachingAttention(d, h, seq, bias, flash)
+        self.ln_2 = OwnLayerNorm(d, bias); self.mlp = TeachingMLP(d, bias)
+    def forward(self, x):
+        x = x + self.attn(self.ln_1(x))
+        return x + self.mlp(self.ln_2(x))
+class TeachingGPT(nn.Module):
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4, bias=True, flash=True):
+        super().__init__()
+        self.block_size = seq
+        self.transformer = nn.ModuleDict(dict(
+            wte=nn.Embedding(vocab, d), wpe=nn.Embedding(seq, d), drop=nn.Dropout(0.0),
+            h=nn.ModuleList([TeachingBlock(d, h, seq, bias, flash) for _ in range(L)]), ln_f=OwnLayerNorm(d, bias)))
+        self.lm_head = nn.Linear(d, vocab, bias=False)
+    def forward(self, idx):
+        b, t = idx.size()
+        assert t <= self.block_size, "sequence longer than the block size"
+        pos = torch.arange(0, t, dtype=torch.long, device=idx.device)
+        x = self.transformer.drop(self.transformer.wte(idx) + self.transformer.wpe(pos))
+        for block in self.transformer.h:
+            x = block(x)
+        return self.lm_head(self.transformer.ln_f(x))

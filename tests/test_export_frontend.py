@@ -453,3 +453,41 @@ def test_values_computed_from_shapes_do_not_travel_between_stages(flag, caplog):
         skip = pp.pipeline(Skip(), 1, (torch.randn(4, 16),))
     assert "more than one tensor" not in caplog.text and skip.num_stages == 3
     assert any(n.op == "call_module" and n.target == "b" for n in skip.get_stage_module(1).graph.nodes)
+
+
+@pytest.mark.parametrize("bias,flash", [(True, True), (True, False), (False, True), (False, False)])
+def test_a_teaching_style_gpt_with_its_own_layer_norm_is_recognised(bias, flash):
+    """The GPT of small teaching code bases: a layer-norm class of its own (``F.layer_norm`` on its
+    parameters, the bias optional) is taken as the ``nn.LayerNorm`` it amounts to (a view of the same
+    parameter objects, the epsilon found by comparison), attention through the fused call or spelled out
+    against a registered lower-triangular buffer, layers with or without biases."""
+    import os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TeachingGPT
+    from pippy_amd._lowering import lower_stage_module
+    from pippy_amd.stage_modules import layer_norm_like
+    torch.manual_seed(0)
+    model = TeachingGPT(vocab=500, seq=64, bias=bias, flash=flash)
+    keys = set(model.state_dict())
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"transformer.h.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    x = ids
+    for i in range(2):
+        why = []
+        blocks = lower_stage_module(pipe.get_stage_module(i), why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2 and all(b.causal and b.pre_ln and b.activation == "gelu_erf" for b in layers)
+        own = model.transformer.h[2 * i]
+        assert layers[0].ln_1.weight is own.ln_1.weight and layers[0].ln_1.eps == 1e-5
+        assert (layers[0].ln_1.bias is own.ln_1.bias) if bias else layers[0].ln_1.bias is None
+        with torch.no_grad():
+            for b in blocks:
+                x = b(x)
+    torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+    assert set(model.state_dict()) == keys          # recognising the layers left the model as it was
+    view = layer_norm_like(model.transformer.ln_f)
+    assert view is layer_norm_like(model.transformer.ln_f) and isinstance(view, nn.LayerNorm)
+    assert layer_norm_like(nn.LayerNorm(8)) is None and layer_norm_like(nn.Linear(8, 8)) is None

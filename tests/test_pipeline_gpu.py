@@ -1153,6 +1153,18 @@ def test_a_causal_model_of_torchs_encoder_layers_runs_natively_and_matches_the_o
     _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "layers.2")
 
 
+@pytest.mark.parametrize("bias,flash", [(True, False), (False, True)])
+def test_a_teaching_style_gpt_runs_natively_and_matches_the_oracle(bias, flash):
+    """A GPT with a layer-norm class of its own (optionally without biases anywhere) and attention through
+    the fused call or spelled out against a lower-triangular buffer."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import TeachingGPT
+    torch.manual_seed(0)
+    model = TeachingGPT(vocab=1000, seq=128, d=128, h=2, L=4, bias=bias, flash=flash)
+    _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "transformer.h.2")
+
+
 def test_torchs_encoder_stack_runs_natively_and_matches_the_oracle():
     """The layers inside ``nn.TransformerEncoder``: exported, recognised on the parameters that
     ``nn.MultiheadAttention`` applies as functions, run as launch lists."""
