@@ -379,7 +379,7 @@ def _is_full_mask(mask: torch.Tensor) -> bool:
 
 
 _SOFTMAX = (_ATEN._softmax.default, _ATEN.softmax.int)
-_MATMULS = (_ATEN.matmul.default, _ATEN.bmm.default)
+_MATMULS = (_ATEN.matmul.default, _ATEN.bmm.default, _ATEN.baddbmm.default)
 _PASS_THROUGH = _ATEN_VIEWS + (_ATEN.transpose.int, _ATEN.permute.default, _ATEN.expand.default,
                                _ATEN._to_copy.default, _ATEN.to.dtype, _ATEN.to.dtype_layout,
                                _ATEN.unsqueeze.default, _ATEN.squeeze.dim, _ATEN.dropout.default)
@@ -424,12 +424,37 @@ def _mask_is_causal(root: nn.Module, mask, causal: bool, inverted: bool = False)
     return True               # (a model may apply its causal mask twice, as a selection and as an addend)
 
 
+_WHOLE_ATTENTION = object()      # stands for the attention inside a call of nn.MultiheadAttention
+
+
+def _check_whole_attention(att: nn.MultiheadAttention, n: fx.Node) -> None:
+    """Raises unless the call ``n`` of ``att`` is plain self-attention over batch-first activations whose
+    averaged weights nobody reads."""
+    given = dict(zip(("query", "key", "value", "key_padding_mask", "need_weights", "attn_mask",
+                      "average_attn_weights", "is_causal"), n.args))
+    given.update(n.kwargs)
+    if not (given.get("query") is given.get("key") is given.get("value")):
+        raise NotLowerable(f"'{n.format_node()}': nn.MultiheadAttention on different query / key / value tensors")
+    if given.get("key_padding_mask") is not None or given.get("attn_mask") is not None or given.get("is_causal"):
+        raise NotLowerable(f"'{n.format_node()}': nn.MultiheadAttention with a mask that is not a constant of the stage")
+    if not att.batch_first or not att._qkv_same_embed_dim or att.in_proj_weight is None or att.bias_k is not None \
+            or att.add_zero_attn or (att.dropout > 0 and att.training):
+        raise NotLowerable(f"nn.MultiheadAttention '{n.target}': sequence-major, separate key / value widths, "
+                           "bias_k / bias_v, add_zero_attn or dropout")
+    for user in n.users:
+        first = user.op == "call_function" and user.target is operator.getitem and user.args[1] == 0
+        if not first and user.users:
+            raise NotLowerable(f"'{n.format_node()}': the attention weights of nn.MultiheadAttention are read")
+
+
 def _attention_form(root: nn.Module, node: fx.Node):
     """(causal, (scale, factor)) of an attention, read off its scaled_dot_product_attention node or — for
     a model that spells attention out as softmax(q k^T * c + mask) v — off its softmax node.  ``scale`` is
     the explicit factor on the scores (None: the default 1 / sqrt(head size)), ``factor`` what the model
     multiplied queries and keys with beforehand.  Raises unless it is plain softmax attention, causal or
     full; whatever this reading misses shows when the recognised blocks are compared with the stage."""
+    if node.op == "call_module":          # a whole nn.MultiheadAttention, checked by _check_whole_attention
+        return False, (None, 1.0)
     if node.target in _SOFTMAX:
         causal, factor = False, 1.0
         x = node.args[0]
@@ -450,7 +475,13 @@ def _attention_form(root: nn.Module, node: fx.Node):
                 raise NotLowerable(f"'{x.format_node()}' between the score product and the softmax")
         if not (isinstance(x, fx.Node) and x.op == "call_function" and x.target in _MATMULS):
             raise NotLowerable("a softmax that does not follow a product of queries and keys")
-        for operand in x.args[:2]:
+        operands = x.args[:2]
+        if x.target is _ATEN.baddbmm.default:      # mask + q k^T in one operator
+            if x.kwargs.get("beta", 1) != 1 or x.kwargs.get("alpha", 1) != 1:
+                raise NotLowerable(f"'{x.format_node()}' with factors of its own")
+            causal = _mask_is_causal(root, x.args[0], causal)
+            operands = x.args[1:3]
+        for operand in operands:
             factor *= _constant_factors_back(root, operand)[1]
         return causal, (1.0, factor)
     names = ("query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale", "enable_gqa")
@@ -526,7 +557,12 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             continue
         if _activation_of(n, root) == "identity":
             continue
-        if n.op == "call_module":
+        if n.op == "call_module" and isinstance(root.get_submodule(n.target), nn.MultiheadAttention):
+            # torch's attention layer as one call: its packed projection, the attention, its output projection
+            att = root.get_submodule(n.target)
+            _check_whole_attention(att, n)
+            mods += [(n, LinearView(att.in_proj_weight, att.in_proj_bias)), (n, _WHOLE_ATTENTION), (n, att.out_proj)]
+        elif n.op == "call_module":
             mods.append((n, _layer_of(root, n.target)))
         elif n.op == "call_function" and n.target in _LINEAR_FNS:
             # (nn.MultiheadAttention applies its packed q|k|v parameters and its output projection this way)
@@ -543,6 +579,8 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
             mods.append((n, None))
 
     def kind(n, m):
+        if m is _WHOLE_ATTENTION:
+            return "sdpa"
         if m is None:
             return "sdpa" if n.target in _SDPA + _SOFTMAX else "act"
         if isinstance(m, (nn.Linear, InOutLinear)):

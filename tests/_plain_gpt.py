@@ -217,3 +217,30 @@ class TeachingGPT(nn.Module):
         for block in self.transformer.h:
             x = block(x)
         return self.lm_head(self.transformer.ln_f(x))
+
+
+# ---- blocks of one's own around torch's attention layer ----------------------------------------------------
+class MHABlock(nn.Module):
+    def __init__(self, d, h, need_weights, causal):
+        super().__init__()
+        self.ln1 = nn.LayerNorm(d); self.attn = nn.MultiheadAttention(d, h, batch_first=True)
+        self.ln2 = nn.LayerNorm(d); self.ff = nn.Sequential(nn.Linear(d, 4 * d), nn.GELU(), nn.Linear(4 * d, d))
+        self.need_weights, self.causal = need_weights, causal
+    def forward(self, x):
+        h = self.ln1(x)
+        mask = None
+        if self.causal:
+            mask = torch.triu(torch.ones(x.shape[1], x.shape[1], dtype=torch.bool, device=x.device), 1)
+        x = x + self.attn(h, h, h, need_weights=self.need_weights, attn_mask=mask)[0]
+        return x + self.ff(self.ln2(x))
+class MHAModel(nn.Module):
+    def __init__(self, vocab=1000, seq=128, d=128, h=2, L=4, need_weights=True, causal=False):
+        super().__init__()
+        self.emb = nn.Embedding(vocab, d); self.pos = nn.Embedding(seq, d)
+        self.blocks = nn.ModuleList([MHABlock(d, h, need_weights, causal) for _ in range(L)])
+        self.norm = nn.LayerNorm(d); self.head = nn.Linear(d, vocab, bias=False)
+    def forward(self, ids):
+        x = self.emb(ids) + self.pos(torch.arange(ids.shape[1], device=ids.device))
+        for b in self.blocks:
+            x = b(x)
+        return self.head(self.norm(x))

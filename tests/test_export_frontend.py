@@ -491,3 +491,35 @@ def test_a_teaching_style_gpt_with_its_own_layer_norm_is_recognised(bias, flash)
     view = layer_norm_like(model.transformer.ln_f)
     assert view is layer_norm_like(model.transformer.ln_f) and isinstance(view, nn.LayerNorm)
     assert layer_norm_like(nn.LayerNorm(8)) is None and layer_norm_like(nn.Linear(8, 8)) is None
+
+
+@pytest.mark.parametrize("need_weights,causal", [(True, False), (True, True), (False, False), (False, True)])
+def test_blocks_around_torchs_attention_layer_are_recognised(need_weights, causal):
+    """``nn.MultiheadAttention`` inside a block of one's own.  Without a mask torch.fx keeps the layer as one
+    call, which is taken as its packed projection, the attention and its output projection; with a mask
+    built from the sequence length the model is exported, and with ``need_weights`` (the layer's default)
+    the layer spells its attention out (the mask added by ``baddbmm``); the averaged weights, which nobody
+    reads, are dropped."""
+    import os, sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import MHAModel
+    from pippy_amd._lowering import lower_stage_module
+    torch.manual_seed(0)
+    model = MHAModel(vocab=500, seq=64, need_weights=need_weights, causal=causal)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"blocks.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    _check_partition(pipe, model)
+    x = ids
+    for i in range(2):
+        why = []
+        blocks = lower_stage_module(pipe.get_stage_module(i), why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2 and all(b.causal == causal and b.pre_ln and b.attn_scale is None for b in layers)
+        own = model.blocks[2 * i].attn
+        assert layers[0].attn.c_attn.weight is own.in_proj_weight and layers[0].attn.c_proj.weight is own.out_proj.weight
+        with torch.no_grad():
+            for b in blocks:
+                x = b(x)
+    torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)

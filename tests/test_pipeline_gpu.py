@@ -1165,6 +1165,19 @@ def test_a_teaching_style_gpt_runs_natively_and_matches_the_oracle(bias, flash):
     _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "transformer.h.2")
 
 
+@pytest.mark.parametrize("need_weights,causal", [(True, False), (True, True)])
+def test_blocks_around_torchs_attention_layer_run_natively_and_match_the_oracle(need_weights, causal):
+    """Blocks of one's own around ``nn.MultiheadAttention`` called the default way (averaged weights
+    computed and dropped), without a mask (traced: the layer is one call) and with a causal mask built
+    from the sequence length (exported: the layer spells its attention out)."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import MHAModel
+    torch.manual_seed(0)
+    model = MHAModel(vocab=1000, seq=128, d=128, h=2, L=4, need_weights=need_weights, causal=causal)
+    _exported_model_against_the_oracle(model, lambda g: g, 1000, 128, "blocks.2")
+
+
 def test_torchs_encoder_stack_runs_natively_and_matches_the_oracle():
     """The layers inside ``nn.TransformerEncoder``: exported, recognised on the parameters that
     ``nn.MultiheadAttention`` applies as functions, run as launch lists."""
