@@ -200,9 +200,23 @@ def _torch_layer(m: nn.TransformerEncoderLayer, n: fx.Node) -> NativeBlock:
     if head not in (64, 128):
         raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}' with head size {head} (64 and 128 are built)")
     try:
-        return torch_encoder_layer_block(m)
+        block = torch_encoder_layer_block(m)
+        # like every recognised stage, the block is compared with what it stands for (fp32, on the host)
+        import copy
+        probe = copy.deepcopy(m).float().cpu().eval()
+        x = torch.randn(2, 16, m.self_attn.embed_dim, generator=torch.Generator().manual_seed(0))
+        with torch.no_grad():
+            want, got = probe(x), torch_encoder_layer_block(probe)(x)
+        err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30)
     except ValueError as e:
         raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}': {e}") from None
+    except Exception as e:
+        raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}' could not be compared with its block "
+                           f"({type(e).__name__}: {e})") from None
+    if err > 1e-4:
+        raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}': the block differs from the layer's own "
+                           f"forward (relative error {err:.2e})")
+    return block
 
 
 def _lower(submod: nn.Module) -> List[NativeBlock]:
