@@ -678,8 +678,10 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         ln, mods, kinds = mods[0][1], mods[1:], kinds[1:]
     if kinds == ["Linear", "sdpa", "Linear"]:
         (_, qkv), (sd, _), (_, proj) = mods
-        if qkv.out_features != 3 * qkv.in_features or proj.in_features != qkv.in_features:
-            raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection of width 3 d")
+        d = qkv.in_features
+        if proj.in_features != d or not d < qkv.out_features <= 3 * d or (qkv.out_features - d) % 2:
+            raise NotLowerable("the projection in front of the attention is not a fused q|k|v projection (width 3 d, "
+                               "or d + 2 k for fewer key / value heads)")
         return ("attn", ln, qkv, proj) + _attention_form(root, sd)
     if kinds == ["Linear", "Linear", "Linear", "sdpa", "Linear"]:
         (_, q), (_, k), (_, v), (sd, _), (_, proj) = mods
@@ -795,13 +797,21 @@ def _layer_block(attention, attention_norm, feed_forward, feed_forward_norm, n_h
         _, ln1, qkv, proj, causal, form = attention
         _, ln2, fc1, fc2, act = feed_forward
         scale = _score_factor(form, d // n_heads)
+        kv_heads = None
+        if not isinstance(qkv, tuple) and qkv.out_features != 3 * d:      # multi-query / grouped-query q|k|v
+            D = d // n_heads
+            kv_heads = (qkv.out_features - d) // (2 * D)
+            if kv_heads < 1 or kv_heads * 2 * D != qkv.out_features - d or n_heads % kv_heads:
+                raise NotLowerable(f"a fused projection of width {qkv.out_features} that is not {n_heads} query heads "
+                                   f"plus whole key / value heads of size {D}")
         if (ln1 is None) != (ln2 is None) or (ln1 is None) != (attention_norm is not None) \
                 or (ln2 is None) != (feed_forward_norm is not None):
             raise NotLowerable("a layer that is neither pre-LayerNorm nor post-LayerNorm throughout")
         if ln1 is None:
             return WrappedTransformerLayer(attention_norm, qkv, proj, feed_forward_norm, fc1, fc2, n_heads, causal,
-                                           act, pre_ln=False, attn_scale=scale)
-        return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act, attn_scale=scale)
+                                           act, pre_ln=False, attn_scale=scale, n_kv_heads=kv_heads)
+        return WrappedTransformerLayer(ln1, qkv, proj, ln2, fc1, fc2, n_heads, causal, act, attn_scale=scale,
+                                       n_kv_heads=kv_heads)
     _, norm1, qkv, o, form, (q_norm, k_norm) = attention
     width = sum(lin.out_features for lin in qkv) if isinstance(qkv, tuple) else qkv.out_features
     D = d // n_heads

@@ -471,12 +471,16 @@ class TransformerLayer(NativeBlock):
             nn.init.zeros_(lin.bias)
 
     attn_scale = None      # the factor on the attention scores; None: 1 / sqrt(head size)
+    n_kv_heads = None      # fewer key / value heads than query heads (multi-query: 1); None: as many
 
     # torch statement of the layer
     def _attention(self, h):
         Bn, S, Cc = h.shape
         H, D = self.n_heads, Cc // self.n_heads
-        q, k, v = (t.reshape(Bn, S, H, D).transpose(1, 2) for t in self._project_qkv(h).split(Cc, dim=-1))
+        Hkv = self.n_kv_heads or H
+        q, k, v = self._project_qkv(h).split([H * D, Hkv * D, Hkv * D], dim=-1)
+        q = q.reshape(Bn, S, H, D).transpose(1, 2)
+        k, v = (t.reshape(Bn, S, Hkv, D).transpose(1, 2).repeat_interleave(H // Hkv, dim=1) for t in (k, v))
         o = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal, scale=self.attn_scale)
         return self.attn.c_proj(o.transpose(1, 2).reshape(Bn, S, Cc))
 
@@ -532,7 +536,7 @@ class TransformerLayer(NativeBlock):
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         ln1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, x2d)
         qkv = self._lower_qkv(b, ln1)
-        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, scale=self.attn_scale)
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, n_kv_heads=self.n_kv_heads, scale=self.attn_scale)
         x2, _ = lower_linear(b, "x2", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         ln2, mean2, rstd2 = lower_layernorm(b, "ln2", self.ln_2, x2)
         # (the derivative of a ReLU is read off its output; a GELU's needs the value before it)
@@ -565,7 +569,7 @@ class TransformerLayer(NativeBlock):
         x2d = x.view(T, Cc)
         act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
         qkv = self._lower_qkv(b, x2d)
-        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, scale=self.attn_scale)
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, self.causal, n_kv_heads=self.n_kv_heads, scale=self.attn_scale)
         a, _ = lower_linear(b, "a", self.attn.c_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)
         x1, mean1, rstd1 = lower_layernorm(b, "ln1", self.ln_1, a)
         h, h_pre = lower_linear(b, "h", self.mlp.c_fc, x1, epilogue=act,
@@ -1423,9 +1427,10 @@ class WrappedTransformerLayer(TransformerLayer):
 
     def __init__(self, ln_1: nn.LayerNorm, c_attn, c_proj: nn.Linear, ln_2: nn.LayerNorm,
                  c_fc: nn.Linear, mlp_proj: nn.Linear, n_heads: int, causal: bool, activation: str,
-                 pre_ln: bool = True, attn_scale: Optional[float] = None):
+                 pre_ln: bool = True, attn_scale: Optional[float] = None, n_kv_heads: Optional[int] = None):
         NativeBlock.__init__(self)
         self.attn_scale = attn_scale
+        self.n_kv_heads = n_kv_heads
         self.dim, self.n_heads, self.ffn = c_proj.out_features, n_heads, c_fc.out_features
         self.causal, self.pre_ln, self.activation = causal, pre_ln, activation
         self.ln_1, self.ln_2 = ln_1, ln_2

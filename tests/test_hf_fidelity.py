@@ -422,6 +422,33 @@ def test_hugging_face_qwen3_stages_are_recognised_with_their_per_head_norms(head
         _close(x, model(ids).logits, "blocks against Qwen3ForCausalLM")
 
 
+@pytest.mark.parametrize("attention", ["sdpa", "eager"])
+def test_hugging_face_gpt_bigcode_stages_are_recognised_with_multi_query_attention(attention):
+    """GPT-BigCode: a GPT-2-style layer whose fused projection is q (d) | k (D) | v (D): every query head
+    attends to the one key / value head."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    cfg = transformers.GPTBigCodeConfig(n_embd=256, n_layer=2, n_head=4, n_positions=64, attn_pdrop=0.0,
+                                        embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False, multi_query=True,
+                                        vocab_size=500, tie_word_embeddings=False)
+    cfg._attn_implementation = attention
+    torch.manual_seed(0)
+    model = transformers.GPTBigCodeForCausalLM(cfg)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"transformer.h.1": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    layer, hf = blocks[1][0], model.transformer.h[1]
+    assert type(layer).__name__ == "WrappedTransformerLayer" and layer.attn.c_attn is hf.attn.c_attn
+    assert (layer.n_heads, layer.n_kv_heads, layer.causal, layer.attn.c_attn.out_features) == (4, 1, True, 256 + 128)
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against GPTBigCodeForCausalLM")
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true
