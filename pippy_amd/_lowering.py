@@ -19,7 +19,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .stage_modules import (InOutLinear, LayerNormBlock, LinearAct, LinearView, NativeBlock, RMSNormBlock, RMSNormLike,
-                            StageSequence, torch_encoder_layer_block, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer,
+                            StageSequence, torch_encoder_layer_block, WrappedEncoderEmbedding, WrappedLlamaLayer, WrappedLMHead, WrappedMoELayer, WrappedParallelLayer,
                             WrappedTokenEmbedding,
                             WrappedTransformerLayer, activation_like, in_out_linear_like, layer_norm_like, rms_norm_like)
 
@@ -271,6 +271,7 @@ def _lower(submod: nn.Module) -> List[NativeBlock]:
 #      pre-LayerNorm    x = x + proj(attn(qkv(ln(x))))                 x = x + fc2(act(fc1(ln(x))))
 #      post-LayerNorm   x = ln(x + proj(attn(qkv(x))))                 x = ln(x + fc2(act(fc1(x))))
 #      rotary, gated    x = x + o(attn(rope(q(n(x)), k(n(x))), v(n(x)))) x = x + down(silu(gate(n(x))) * up(n(x)))
+#      side by side     x = x + o(attn(rope(qkv(ln(x))))) + fc2(act(fc1(ln'(x))))   (ln' = ln or a second LayerNorm)
 #      rotary, experts  the same attention; x = x + (two of E gated experts per token, weights in stacked
 #                       tensors, chosen by a softmax router)
 #    where qkv is one fused projection or three separate ones; the affine layers are ``nn.Linear``, layers
@@ -640,6 +641,24 @@ def _classify_branch(root: nn.Module, layers: List[fx.Node]):
         return ("attn_rope", norm, (q, k, v), o, form, (head_norms.get(qn), head_norms.get(kn)))
     if head_norms:
         raise NotLowerable("per-head norms in an attention branch without separate query / key / value projections")
+    norms = 2 if kinds[:2] == ["LayerNorm", "LayerNorm"] else 1
+    if kinds[:norms] == ["LayerNorm"] * norms and kinds[norms:] == ["Linear", "sdpa", "Linear", "Linear", "act", "Linear"] \
+            and inner_adds:
+        # attention and feed-forward side by side on one stream (their sum is one of the inner additions,
+        # the rotary embedding makes the others), behind one LayerNorm or one each
+        (qn, qkv), (sd, _), (_, o), (fn, fc1), (an, _), (_, fc2) = mods[norms:]
+        feeds = {node: m for node, m in mods[:norms]}
+        ln_a = feeds.get(_constant_factors_back(root, qn.all_input_nodes[0])[0])
+        ln_m = feeds.get(_constant_factors_back(root, fn.all_input_nodes[0])[0])
+        act = _activation_of(an, root)
+        if ln_a is None or ln_m is None or not all(isinstance(lin, nn.Linear) for lin in (qkv, o, fc1, fc2)) \
+                or act not in ("gelu_tanh", "gelu_erf", "relu") or fc2.in_features != fc1.out_features:
+            raise NotLowerable("attention and feed-forward side by side, but not as ln -> q|k|v -> attention -> o "
+                               "next to ln -> fc1 -> GELU / ReLU -> fc2")
+        causal, form = _attention_form(root, sd)
+        if not causal:
+            raise NotLowerable("rotary attention that is not causal")
+        return ("parallel", ln_a, ln_m, qkv, o, fc1, fc2, act, form)
     if kinds == ["RMSNorm", "Linear", "sdpa", "Linear"] and inner_adds:
         (_, norm), (_, qkv), (sd, _), (_, o) = mods       # one fused q|k|v projection under a rotary embedding
         if not all(isinstance(lin, nn.Linear) for lin in (qkv, o)) or o.in_features != o.out_features \
@@ -917,6 +936,23 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
             after, post_norm = _only_layer_user(root, add)
             if not isinstance(post_norm, nn.LayerNorm):
                 raise NotLowerable("a residual branch without a LayerNorm before it or after its addition")
+        if kind[0] == "parallel":
+            if attention is not None:
+                raise NotLowerable("an attention branch without its feed-forward branch before a side-by-side layer")
+            _, ln_a, ln_m, qkv, o, fc1, fc2, act, form = kind
+            if rope is None:
+                raise NotLowerable("rotary attention, but the stage holds no constant cos / sin table of the positions")
+            D = 2 * rope[0].shape[1]
+            if o.in_features % D or _score_factor(form, D) is not None:
+                raise NotLowerable("a side-by-side layer whose heads do not match the rotary table, or with a score "
+                                   "factor other than 1 / sqrt(head size)")
+            heads = o.in_features // D
+            if qkv.out_features % D or (qkv.out_features // D - heads) % 2 or qkv.out_features // D <= heads \
+                    or heads % ((qkv.out_features // D - heads) // 2):
+                raise NotLowerable("a fused projection that is not whole query, key and value heads")
+            blocks.append(WrappedParallelLayer(ln_a, ln_m, qkv, o, fc1, fc2, heads, act, *rope))
+            stream = _skip_identities(root, add)
+            continue
         if kind[0] in ("attn", "attn_rope"):
             if attention is not None:
                 raise NotLowerable("two attention branches in a row")
@@ -929,7 +965,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         stream = _skip_identities(root, after)
     if attention is not None:
         raise NotLowerable("an attention branch without its feed-forward branch in the same stage")
-    if not any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer)) for b in blocks):
+    if not any(isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer, WrappedParallelLayer)) for b in blocks):
         raise NotLowerable("no attention / feed-forward residual pair found")
     return blocks + _tail_blocks(root, stream, result, after_layers=True)
 
@@ -949,7 +985,7 @@ def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
             x[0, :1] = first.padding_positions
             x[-1, x.shape[1] // 2:] = first.padding_positions
         return x
-    d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer))).dim
+    d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer, WrappedParallelLayer))).dim
     return torch.randn(shape or (2, 16, d), generator=g)
 
 

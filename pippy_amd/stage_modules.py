@@ -1379,6 +1379,104 @@ class WrappedEncoderEmbedding(EncoderEmbedding):
         self.padding_positions = padding_positions
 
 
+class WrappedParallelLayer(NativeBlock):
+    """A decoder layer whose attention and feed-forward read the same residual stream side by side
+    (Falcon): ``x + o(attn(rope(qkv(ln_a(x))))) + fc2(act(fc1(ln_m(x))))`` around a user's layers.  ``qkv``
+    is one fused projection, query heads first, then the key heads, then the value heads (fewer of them
+    than query heads for multi-query / grouped-query attention); ``ln_m`` may be ``ln_a`` itself;
+    ``cos`` / ``sin`` are the model's own rotary tables [positions, head_dim / 2]."""
+
+    def __init__(self, ln_a: nn.LayerNorm, ln_m: nn.LayerNorm, qkv: nn.Linear, o_proj: nn.Linear, fc1: nn.Linear,
+                 fc2: nn.Linear, n_heads: int, activation: str, cos: torch.Tensor, sin: torch.Tensor):
+        super().__init__()
+        assert activation in _ACT_DEPI and cos.shape == sin.shape
+        self.dim, self.n_heads, self.activation = o_proj.out_features, n_heads, activation
+        D = 2 * cos.shape[1]
+        assert o_proj.in_features == n_heads * D
+        self.head_dim = D
+        self.n_kv_heads = (qkv.out_features // D - n_heads) // 2
+        assert self.n_kv_heads > 0 and (n_heads + 2 * self.n_kv_heads) * D == qkv.out_features \
+            and n_heads % self.n_kv_heads == 0
+        self.ln_a, self.qkv, self.o_proj, self.fc1, self.fc2 = ln_a, qkv, o_proj, fc1, fc2
+        if ln_m is not ln_a:
+            self.ln_m = ln_m
+        self._cos, self._sin = cos.detach().float().cpu().contiguous(), sin.detach().float().cpu().contiguous()
+        import hashlib
+        self._table_key = hashlib.sha1(self._cos.numpy().tobytes() + self._sin.numpy().tobytes()).hexdigest()[:16]
+
+    def _ln_m(self):
+        return getattr(self, "ln_m", None) or self.ln_a
+
+    def _tables(self, seq, device):
+        if seq > self._cos.shape[0]:
+            raise RuntimeError(f"the model's rotary table covers {self._cos.shape[0]} positions, asked for {seq}")
+        return self._cos[:seq].to(device), self._sin[:seq].to(device)
+
+    # torch statement of the layer
+    def forward(self, x):
+        Bn, S, Cc = x.shape
+        H, Hkv, D = self.n_heads, self.n_kv_heads, self.head_dim
+        cos, sin = self._tables(S, x.device)
+        q, k, v = self.qkv(self.ln_a(x)).split([H * D, Hkv * D, Hkv * D], dim=-1)
+        q = q.reshape(Bn, S, H, D).transpose(1, 2)
+        k, v = (t.reshape(Bn, S, Hkv, D).transpose(1, 2) for t in (k, v))
+        q, k = _apply_rope(q, cos, sin), _apply_rope(k, cos, sin)
+        if Hkv != H:
+            k, v = (t.repeat_interleave(H // Hkv, dim=1) for t in (k, v))
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        a = self.o_proj(o.transpose(1, 2).reshape(Bn, S, H * D))
+        return x + a + self.fc2(_torch_act(self.fc1(self._ln_m()(x)), self.activation))
+
+    def lower(self, b, x):
+        if x.dim() != 3 or x.shape[-1] != self.dim:
+            raise RuntimeError(f"{type(self).__name__} of width {self.dim} expects [batch, seq, dim], got "
+                               f"{tuple(x.shape)}")
+        Bn, S, Cc = x.shape
+        T, H, Hkv, D = Bn * S, self.n_heads, self.n_kv_heads, self.head_dim
+        x2d = x.view(T, Cc)
+        ln_a, ln_m = self.ln_a, self._ln_m()
+        shared = ln_m is ln_a
+        act, dact = _ACT_EPI[self.activation], _ACT_DEPI[self.activation]
+        cos = b.sp.shared(f"rope_cos:{S}:{D}:{self._table_key}", (S, D // 2), torch.float32)
+        sin = b.sp.shared(f"rope_sin:{S}:{D}:{self._table_key}", (S, D // 2), torch.float32)
+        c, s_ = self._tables(S, x.device)
+        cos.copy_(c)
+        sin.copy_(s_)
+        na, mean_a, rstd_a = lower_layernorm(b, "na", ln_a, x2d)
+        nm, mean_m, rstd_m = (na, mean_a, rstd_a) if shared else lower_layernorm(b, "nm", ln_m, x2d)
+        qkv, _ = lower_linear(b, "qkv", self.qkv, na)
+        b.f(P.op_rope(qkv, cos, sin, S, H + Hkv, D))
+        att, attention_backward = lower_attention(b, qkv, Bn, S, H, True, n_kv_heads=Hkv)
+        a, _ = lower_linear(b, "a", self.o_proj, att, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=x2d)      # x + attention
+        relu = self.activation == "relu"
+        h, h_pre = lower_linear(b, "h", self.fc1, nm, epilogue=act, save_pre=b.training and not relu)
+        if relu:
+            h_pre = h
+        y, _ = lower_linear(b, "y", self.fc2, h, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=a)
+
+        def bwd(dy, need_dx, dx_out):
+            dy2d = dy.view(T, Cc)
+            d_hpre = linear_backward(b, "fc2", self.fc2, h, dy2d, dx_epilogue=dact, dx_aux=h_pre)
+            d_nm = linear_backward(b, "fc1", self.fc1, nm, d_hpre)
+            d_att = linear_backward(b, "o", self.o_proj, att, dy2d)
+            dqkv = attention_backward(d_att)
+            b.i(P.op_rope(dqkv, cos, sin, S, H + Hkv, D, inverse=True))
+            out = dx_out.view(T, Cc) if dx_out is not None else None
+            if shared:
+                # the two gradients of the one norm's output are added by the residual epilogue of the
+                # second input-gradient GEMM
+                d_n = linear_backward(b, "qkv", self.qkv, na, dqkv, dx_epilogue=N.EPI_BIAS_RESIDUAL, dx_aux=d_nm)
+                dx = layernorm_backward(b, "na", ln_a, x2d, mean_a, rstd_a, d_n, dres=dy2d, dx_out=out)
+            else:
+                d_na = linear_backward(b, "qkv", self.qkv, na, dqkv)
+                dx1 = layernorm_backward(b, "nm", ln_m, x2d, mean_m, rstd_m, d_nm, dres=dy2d)
+                dx = layernorm_backward(b, "na", ln_a, x2d, mean_a, rstd_a, d_na, dres=dx1, dx_out=out)
+            return dx.view(Bn, S, Cc)
+
+        b.on_backward(bwd)
+        return y.view(Bn, S, Cc)
+
+
 class LinearView(nn.Linear):
     """An ``nn.Linear`` around parameters that a module keeps without a layer of their own (the packed
     q|k|v projection of ``nn.MultiheadAttention``): the same parameter objects, so names, gradients and

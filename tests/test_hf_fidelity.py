@@ -449,6 +449,43 @@ def test_hugging_face_gpt_bigcode_stages_are_recognised_with_multi_query_attenti
         _close(x, model(ids).logits, "blocks against GPTBigCodeForCausalLM")
 
 
+def test_hugging_face_falcon_stages_are_recognised_as_side_by_side_layers():
+    """Falcon: attention and feed-forward read the same LayerNorm output and are added to the residual
+    stream together; rotary embedding; multi-query attention through one fused projection; no biases.
+    The newer decoder layout of the family interleaves q, k and v per key / value group in that projection:
+    the numerical comparison notices, and such stages stay with torch."""
+    import pippy_amd as pp
+    from pippy_amd._lowering import lower_stage_module
+    kw = dict(hidden_size=256, num_hidden_layers=2, num_attention_heads=4, hidden_dropout=0.0, attention_dropout=0.0,
+              use_cache=False, tie_word_embeddings=False, vocab_size=500, max_position_embeddings=64)
+    cfg = transformers.FalconConfig(**kw)
+    cfg._attn_implementation = "sdpa"
+    torch.manual_seed(0)
+    model = transformers.FalconForCausalLM(cfg)
+    ids = torch.randint(0, 500, (2, 40))
+    pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"transformer.h.1": pp.SplitPoint.BEGINNING})
+    why = []
+    blocks = [lower_stage_module(pipe.get_stage_module(i), why) for i in range(2)]
+    assert not why, why
+    assert [[type(b).__name__ for b in bl] for bl in blocks] == \
+        [["WrappedTokenEmbedding", "WrappedParallelLayer"], ["WrappedParallelLayer", "WrappedLMHead"]]
+    layer, hf = blocks[1][0], model.transformer.h[1]
+    assert layer.qkv is hf.self_attention.query_key_value and layer.ln_a is hf.input_layernorm
+    assert layer._ln_m() is layer.ln_a and layer.fc1 is hf.mlp.dense_h_to_4h
+    assert (layer.n_heads, layer.n_kv_heads, layer.head_dim, layer.activation) == (4, 1, 64, "gelu_erf")
+    x = ids
+    with torch.no_grad():
+        for b in blocks[0] + blocks[1]:
+            x = b(x)
+        _close(x, model(ids).logits, "blocks against FalconForCausalLM")
+    cfg = transformers.FalconConfig(new_decoder_architecture=True, num_kv_heads=2, **kw)
+    cfg._attn_implementation = "sdpa"
+    other = transformers.FalconForCausalLM(cfg)
+    pipe = pp.pipeline(other, mb_args=(ids,), split_spec={"transformer.h.1": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None and "differ from the stage's own forward" in why[0]
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true

@@ -1331,7 +1331,7 @@ def _qkv_group(name):
 
 
 @pytest.mark.parametrize("family", ["qwen2", "mistral", "phi3", "distilbert", "electra", "opt", "gpt2_spelled_out",
-                                    "megatron_bert", "gpt_neo", "roberta", "qwen3", "qwen3_wide_heads", "gpt_bigcode"])
+                                    "megatron_bert", "gpt_neo", "roberta", "qwen3", "qwen3_wide_heads", "gpt_bigcode", "falcon"])
 def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     """Families that the same recognisers cover: Qwen2 (Llama layout with biases on the query / key /
     value projections), Mistral (Llama layout), Phi-3 (one fused q|k|v and one fused gate|up projection),
@@ -1349,7 +1349,9 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
     Qwen3 (RMS norms over each head's values of queries and keys in front of the rotary embedding; in
     the second variant a head size of 128 that is not width / heads, so that the query projection widens
     the stream and the output projection narrows it again); GPT-BigCode (multi-query attention in a
-    GPT-2-style layer: one fused projection of width d + 2 D, all query heads on one key / value head)."""
+    GPT-2-style layer: one fused projection of width d + 2 D, all query heads on one key / value head);
+    Falcon (attention and feed-forward side by side on the residual stream behind one LayerNorm, rotary
+    embedding, multi-query attention, no biases)."""
     T = pytest.importorskip("transformers")
     import torch.nn as nn
     common = dict(vocab_size=1000, tie_word_embeddings=False)
@@ -1397,6 +1399,10 @@ def test_more_hugging_face_families_run_natively_and_match_the_oracle(family):
                                 T.GPTBigCodeConfig(n_embd=256, n_layer=4, n_head=4, n_positions=128, attn_pdrop=0.0,
                                                    embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False, multi_query=True,
                                                    bos_token_id=0, eos_token_id=0, **common), "transformer.h.2"),
+        "falcon": lambda: (T.FalconForCausalLM,
+                           T.FalconConfig(hidden_size=256, num_hidden_layers=4, num_attention_heads=4,
+                                          hidden_dropout=0.0, attention_dropout=0.0, use_cache=False,
+                                          max_position_embeddings=128, **common), "transformer.h.2"),
         "roberta": lambda: (T.RobertaForMaskedLM,
                             T.RobertaConfig(hidden_size=128, intermediate_size=512, num_hidden_layers=4,
                                             num_attention_heads=2, max_position_embeddings=132,
