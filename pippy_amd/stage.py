@@ -317,9 +317,29 @@ class PipelineStageBase:
     def _check_live_shapes(self, flat_inputs, output_tuple) -> None:
         """Hook for stages that were given example values (``ManualPipelineStage``)."""
 
+    def _exported_input_shape(self):
+        """The per-sample input shape a stage was exported on (None for a stage traced symbolically, which
+        holds no shapes).  What an exported stage computes was fixed for that shape (a mask cut for that
+        sequence length, a sliding window known to cover it, position indices): the launch lists run any
+        batch size, samples being independent, but no other sequence length."""
+        if "_exported_shape" not in self.__dict__:
+            shape = None
+            graph = getattr(self.submod, "graph", None)
+            inputs = [n for n in graph.nodes if n.op == "placeholder"] if graph is not None else []
+            if len(inputs) == 1 and hasattr(inputs[0].meta.get("val"), "shape") and \
+                    any(b.startswith("_folded_constant_") for b, _ in self.submod.named_buffers(recurse=False)):
+                shape = tuple(int(d) for d in inputs[0].meta["val"].shape[1:])
+            self._exported_shape = shape
+        return self._exported_shape
+
     def _forward_native(self, mb, args, kwargs):
         sp = self._stage_program()
         x, dx_target, patch = self._input_for(mb, args, kwargs)
+        expected = self._exported_input_shape()
+        if expected is not None and tuple(x.shape[1:]) != expected:
+            raise RuntimeError(f"{self.log_prefix} was exported on inputs of shape [batch, {', '.join(map(str, expected))}] "
+                               f"and holds constants made for it; got {tuple(x.shape)} (build the pipeline on an "
+                               "example of the shape it will run on)")
         prog = sp.mbs.get(mb)
         if patch:
             xc = None

@@ -1216,6 +1216,36 @@ def _relu_sets_of_torch_layers(ref, stages, M):
         layer.activation_relu_or_gelu = 0
 
 
+def test_an_exported_stage_runs_any_batch_size_but_only_its_sequence_length():
+    """An exported stage holds constants made for the example's shape (here a causal mask cut for 64
+    positions).  Its launch lists take other batch sizes, samples being independent; another sequence
+    length is refused with the reason instead of being computed with whatever the blocks would assume.  A
+    symbolically traced model holds no shapes and runs both."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import GPT, LibGPT
+    import pippy_amd as pp
+    for cls, exported in ((LibGPT, True), (GPT, False)):
+        torch.manual_seed(0)
+        model = cls(vocab=300, seq=128, d=128, h=2, L=4).to(torch.bfloat16)
+        ids = torch.randint(0, 300, (2, 64))
+        pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"h.2": pp.SplitPoint.BEGINNING})
+        stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+        assert all(st.is_native for st in stages)
+        sched = pp.ScheduleGPipe(stages, 2)
+        big = torch.randint(0, 300, (6, 64))
+        out = sched.step(big.to(DEV))
+        assert_close_rel(out, model.to(DEV)(big.to(DEV)), BF16_TOL, "another batch size")
+        model.cpu()
+        longer = torch.randint(0, 300, (4, 96))
+        if exported:
+            with pytest.raises(RuntimeError, match="exported on inputs of shape"):
+                sched.step(longer.to(DEV))
+        else:
+            out = sched.step(longer.to(DEV))
+            assert_close_rel(out, model.to(DEV)(longer.to(DEV)), BF16_TOL, "another sequence length")
+
+
 def test_exported_stages_that_do_not_lower_run_through_autograd_on_the_gpu():
     """An exported model whose attention mask is not the causal one (a sliding window) keeps its stages
     with torch autograd.  Their graphs were exported on the host: the folded constants (mask, position
