@@ -508,6 +508,22 @@ class Pipe(nn.Module):
             except ValueError:
                 raise
             except Exception as export_error:
+                config = getattr(mod, "config", None)
+                if "data pointer" in str(export_error) and getattr(config, "_experts_implementation", None) not in \
+                        (None, "batched_mm"):
+                    # a library's grouped expert product inspects tensor addresses, which torch.export cannot
+                    # trace; its batched form computes the same and traces: export with that one selected
+                    chosen = config._experts_implementation
+                    config._experts_implementation = "batched_mm"
+                    try:
+                        traced = _export_and_mark(mod, args_split[0], kwargs_split[0], split_spec)
+                        logger.warning("exported with config._experts_implementation = 'batched_mm' (the "
+                                       f"'{chosen}' form inspects tensor addresses, which torch.export cannot trace)")
+                        return traced
+                    except Exception:
+                        pass
+                    finally:
+                        config._experts_implementation = chosen
                 hint = ""
                 if "Cache" in str(export_error) and getattr(getattr(mod, "config", None), "use_cache", False):
                     hint = ("; the model returns a key / value cache object, which torch.export cannot flatten: "
