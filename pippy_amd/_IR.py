@@ -524,6 +524,19 @@ class Pipe(nn.Module):
                         pass
                     finally:
                         config._experts_implementation = chosen
+                if "Cache" in str(export_error) and getattr(config, "use_cache", False):
+                    # the model returns a key / value cache object, which torch.export cannot flatten and a
+                    # training or scoring pipeline has no use for: export without it
+                    config.use_cache = False
+                    try:
+                        traced = _export_and_mark(mod, args_split[0], kwargs_split[0], split_spec)
+                        logger.warning("exported with config.use_cache = False: the model's key / value cache object "
+                                       "cannot be exported, and the pipeline's stages do not return one")
+                        return traced
+                    except Exception:
+                        pass
+                    finally:
+                        config.use_cache = True
                 hint = ""
                 if "Cache" in str(export_error) and getattr(getattr(mod, "config", None), "use_cache", False):
                     hint = ("; the model returns a key / value cache object, which torch.export cannot flatten: "

@@ -486,6 +486,40 @@ def test_hugging_face_falcon_stages_are_recognised_as_side_by_side_layers():
     assert lower_stage_module(pipe.get_stage_module(1), why) is None and "differ from the stage's own forward" in why[0]
 
 
+def test_library_defaults_that_cannot_be_exported_are_set_aside_for_the_export(caplog):
+    """The reference's example builds ``GPT2LMHeadModel(config)`` as the library configures it, which today
+    returns a key / value cache object that torch.export cannot flatten; Mixtral's default expert product
+    inspects tensor addresses in bf16.  The front end exports with the cache off (a pipeline's stages do not
+    return one) and with the library's batched expert form, says so, and leaves the configuration as it was."""
+    import logging
+    import pippy_amd as pp
+    cfg = transformers.GPT2Config(n_layer=2, n_embd=128, n_head=2, n_positions=64, attn_pdrop=0.0, embd_pdrop=0.0,
+                                  resid_pdrop=0.0, tie_word_embeddings=False, vocab_size=500)
+    torch.manual_seed(0)
+    model = transformers.GPT2LMHeadModel(cfg)
+    assert model.config.use_cache
+    ids = torch.randint(0, 500, (2, 32))
+    with caplog.at_level(logging.WARNING, logger="pippy_amd._IR"):
+        pipe = pp.pipeline(model, mb_args=(ids,), split_spec={"transformer.h.1": pp.SplitPoint.BEGINNING})
+    assert "use_cache = False" in caplog.text and model.config.use_cache
+    out = pipe(ids)
+    _close(out[0] if isinstance(out, (tuple, list)) else out, model(ids).logits, "Pipe against the model")
+    cfg = transformers.MixtralConfig(hidden_size=128, intermediate_size=128, num_hidden_layers=2,
+                                     num_attention_heads=2, num_key_value_heads=1, vocab_size=300,
+                                     max_position_embeddings=32, use_cache=False, tie_word_embeddings=False,
+                                     num_local_experts=4, num_experts_per_tok=2, attention_dropout=0.0,
+                                     sliding_window=None)
+    moe = transformers.MixtralForCausalLM(cfg).to(torch.bfloat16)
+    chosen = moe.config._experts_implementation
+    ids = torch.randint(0, 300, (2, 16))
+    caplog.clear()
+    with caplog.at_level(logging.WARNING, logger="pippy_amd._IR"):
+        pipe = pp.pipeline(moe, mb_args=(ids,), split_spec={"model.layers.1": pp.SplitPoint.BEGINNING})
+    assert pipe.num_stages == 2 and moe.config._experts_implementation == chosen
+    if chosen != "batched_mm":
+        assert "batched_mm" in caplog.text
+
+
 def test_hugging_face_bert_stages_are_recognised_on_the_models_own_layers():
     """transformers.BertForMaskedLM (examples/huggingface/pippy_bert.py): the encoder front (three tables
     and a LayerNorm), post-LayerNorm layers with separate query / key / value projections, the all-true
