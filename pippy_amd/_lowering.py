@@ -152,7 +152,7 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
         if isinstance(m, NativeBlock):
             blocks.append(m)
         elif isinstance(m, nn.TransformerEncoderLayer):
-            blocks.append(_torch_layer(m, n))
+            blocks.append(_torch_layer(m, n, root))
         elif isinstance(m, (nn.Linear, InOutLinear)):
             nxt = _activation_of(nodes[i + 1], root) if i + 1 < len(nodes) else None
             if nxt == "silu":
@@ -192,21 +192,36 @@ def blocks_from_graph(root: nn.Module, graph: fx.Graph) -> Optional[List[NativeB
     return blocks
 
 
-def _torch_layer(m: nn.TransformerEncoderLayer, n: fx.Node) -> NativeBlock:
-    """torch's own encoder layer, called with its input alone (no mask, no padding mask)."""
-    if len(n.args) != 1 or any(v is not None for v in n.kwargs.values()):
-        raise NotLowerable(f"'{n.format_node()}': an nn.TransformerEncoderLayer called with a mask")
+def _torch_layer(m: nn.TransformerEncoderLayer, n: fx.Node, root: Optional[nn.Module] = None) -> NativeBlock:
+    """torch's own encoder layer, called with its input alone or with a constant causal mask (a registered
+    buffer: additive, or boolean with True for what is masked) and / or ``is_causal=True``."""
+    given = dict(zip(("src", "src_mask", "src_key_padding_mask", "is_causal"), n.args))
+    given.update(n.kwargs)
+    causal = False
+    if given.get("src_key_padding_mask") is not None:
+        raise NotLowerable(f"'{n.format_node()}': an nn.TransformerEncoderLayer called with a padding mask")
+    if given.get("src_mask") is not None:
+        value = _constant_of(root, given["src_mask"]) if root is not None else None
+        if value is not None and value.dtype == torch.bool:
+            value = ~value
+        if value is None or not _is_causal_mask(value):
+            raise NotLowerable(f"'{n.format_node()}': an nn.TransformerEncoderLayer called with a mask that is not a "
+                               "constant causal mask")
+        causal = True
+    elif given.get("is_causal"):
+        raise NotLowerable(f"'{n.format_node()}': is_causal without the mask it describes")
     head = m.self_attn.embed_dim // m.self_attn.num_heads
     if head not in (64, 128):
         raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}' with head size {head} (64 and 128 are built)")
     try:
-        block = torch_encoder_layer_block(m)
+        block = torch_encoder_layer_block(m, causal)
         # like every recognised stage, the block is compared with what it stands for (fp32, on the host)
         import copy
         probe = copy.deepcopy(m).float().cpu().eval()
         x = torch.randn(2, 16, m.self_attn.embed_dim, generator=torch.Generator().manual_seed(0))
+        mask = nn.Transformer.generate_square_subsequent_mask(16) if causal else None
         with torch.no_grad():
-            want, got = probe(x), torch_encoder_layer_block(probe)(x)
+            want, got = probe(x, src_mask=mask), torch_encoder_layer_block(probe, causal)(x)
         err = (got - want).abs().max().item() / max(want.abs().max().item(), 1e-30)
     except ValueError as e:
         raise NotLowerable(f"nn.TransformerEncoderLayer '{n.target}': {e}") from None
@@ -919,7 +934,7 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
         whole = next(iter(stream.users)) if len(stream.users) == 1 else None
         if whole is not None and whole.op == "call_module" and attention is None and \
                 isinstance(root.get_submodule(whole.target), nn.TransformerEncoderLayer):
-            blocks.append(_torch_layer(root.get_submodule(whole.target), whole))    # a layer of torch's own
+            blocks.append(_torch_layer(root.get_submodule(whole.target), whole, root))    # a layer of torch's own
             stream = _skip_identities(root, whole)
             continue
         adds = [u for u in stream.users if _is_add(u)]
@@ -970,23 +985,24 @@ def _residual_blocks(root: nn.Module, graph: fx.Graph, n_heads: int, rope=None) 
     return blocks + _tail_blocks(root, stream, result, after_layers=True)
 
 
-def _example_input(blocks: List[NativeBlock], shape=None) -> torch.Tensor:
+def _example_input(blocks: List[NativeBlock], shape=None, seq: int = 16) -> torch.Tensor:
     """A random stage input; ``shape`` is given for exported stages, whose graphs hold the sizes of the
-    example microbatch."""
+    example microbatch; ``seq``: the sequence length otherwise (a stage that holds a square mask runs at
+    that mask's size only)."""
     g = torch.Generator().manual_seed(0)
     first = blocks[0]
     if isinstance(first, WrappedTokenEmbedding):
-        seq = 16 if first.wpe is None else min(16, first.wpe.num_embeddings)
+        seq = seq if first.wpe is None else min(seq, first.wpe.num_embeddings)
         return torch.randint(0, first.wte.num_embeddings, shape or (2, seq), generator=g)
     if isinstance(first, WrappedEncoderEmbedding):
-        seq = min(16, first.position_embeddings.num_embeddings)
+        seq = min(seq, first.position_embeddings.num_embeddings)
         x = torch.randint(0, first.word_embeddings.num_embeddings, shape or (2, seq), generator=g)
         if first.padding_positions is not None:      # some padding, so that its handling is compared too
             x[0, :1] = first.padding_positions
             x[-1, x.shape[1] // 2:] = first.padding_positions
         return x
     d = next(b for b in blocks if isinstance(b, (WrappedTransformerLayer, WrappedLlamaLayer, WrappedParallelLayer))).dim
-    return torch.randn(shape or (2, 16, d), generator=g)
+    return torch.randn(shape or (2, seq, d), generator=g)
 
 
 def _rotary_tables(submod: nn.Module, d: int):
@@ -1043,12 +1059,16 @@ def blocks_from_residual_graph(submod: nn.Module) -> List[NativeBlock]:
     except Exception as e:
         raise NotLowerable(f"the stage module cannot be copied for verification: {e}") from e
     _widen_baked_casts(probe)
+    # a mask kept as a buffer of fixed size (a traced model that hands it to its layers) fixes the length
+    square = [t.shape[-1] for _, t in submod.named_buffers() if t.dim() >= 2 and t.shape[-1] == t.shape[-2] > 1
+              and (t.dtype == torch.bool or t.is_floating_point())]
+    seq = min(square) if square and shape is None else 16
     probe_graph = _ChainTracer().trace(probe)
     tolerance = 1e-4
     reasons = []
     for n_heads in candidates:
         trial = _residual_blocks(probe, probe_graph, n_heads, rope)
-        x = _example_input(trial, shape)
+        x = _example_input(trial, shape, seq)
         try:
             with torch.no_grad():
                 want = probe(x)

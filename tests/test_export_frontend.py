@@ -523,3 +523,50 @@ def test_blocks_around_torchs_attention_layer_are_recognised(need_weights, causa
             for b in blocks:
                 x = b(x)
     torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("boolean,flag", [(False, True), (True, False)])
+def test_torchs_encoder_layers_called_with_a_registered_causal_mask(boolean, flag):
+    """``layer(x, src_mask=self.mask)`` with the mask a registered buffer (additive, or boolean with True for
+    what is masked), with or without ``is_causal=True``: torch.fx keeps the calls whole, the mask is read
+    from the buffer, and the comparison with the stage runs at the mask's size."""
+    from pippy_amd._lowering import lower_stage_module
+
+    class Model(nn.Module):
+        def __init__(self, vocab=300, d=128, h=2, L=4, seq=48):
+            super().__init__()
+            self.emb = nn.Embedding(vocab, d)
+            self.layers = nn.ModuleList([nn.TransformerEncoderLayer(d, h, 2 * d, dropout=0.0, batch_first=True,
+                                                                    norm_first=True) for _ in range(L)])
+            self.head = nn.Linear(d, vocab, bias=False)
+            mask = torch.triu(torch.ones(seq, seq, dtype=torch.bool), 1) if boolean else \
+                nn.Transformer.generate_square_subsequent_mask(seq)
+            self.register_buffer("mask", mask, persistent=False)
+
+        def forward(self, ids):
+            x = self.emb(ids)
+            for layer in self.layers:
+                x = layer(x, src_mask=self.mask, is_causal=True) if flag else layer(x, src_mask=self.mask)
+            return self.head(x)
+
+    torch.manual_seed(0)
+    model = Model()
+    ids = torch.randint(0, 300, (2, 48))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    torch.testing.assert_close(pipe(ids), model(ids), rtol=0, atol=0)
+    x = ids
+    for i in range(2):
+        why = []
+        blocks = lower_stage_module(pipe.get_stage_module(i), why)
+        assert blocks is not None, why
+        layers = [b for b in blocks if type(b).__name__ == "WrappedTransformerLayer"]
+        assert len(layers) == 2 and all(b.causal for b in layers)
+        with torch.no_grad():
+            for b in blocks:
+                x = b(x)
+    torch.testing.assert_close(x, model(ids), rtol=1e-4, atol=1e-4)
+    # a mask that is not causal keeps the stage with torch
+    model.mask = torch.zeros(48, 48).fill_diagonal_(float("-inf"))
+    pipe = pp.pipeline(model, 1, (ids,), split_spec={"layers.2": pp.SplitPoint.BEGINNING})
+    why = []
+    assert lower_stage_module(pipe.get_stage_module(1), why) is None and "not a constant causal mask" in why[0]
