@@ -193,14 +193,15 @@ def flops_per_step(args):
     return 3.0 * per_token_fwd * T
 
 
-def cpu_baseline(args, budget_seconds=45.0):
+def cpu_baseline(args, budget_seconds=120.0):
     """The reference's own way of running this workload on host cores (its tests: backend gloo, one
     process per stage, ``test/test_fwd.py:117-129``), restated in ``oracle/gloo_pipeline.py``: S fresh
     CPU-only child processes over gloo on 127.0.0.1, each running its rank's program of the same 1F1B
     schedule on its stage of the same model, ``cores // S`` threads each, in the arithmetic of the
     configuration (bf16 parameters, activations and gradients).  One warm-up microbatch through the
-    whole pipeline, then one timed step; if the warm-up says a full step would overrun the budget the
-    first half (quarter ...) of the step's microbatches is timed instead, and ``sample`` says so.
+    whole pipeline, one untimed warm-up step, then three timed steps whose median is reported; if the
+    warm-up microbatch says that this would overrun the budget, one timed step (or the first half,
+    quarter ... of its microbatches) without the warm-up step, and ``sample`` says so.
     Must be called before this process touches the GPU: the children are started from a parent that
     holds no GPU state."""
     import socket
@@ -234,12 +235,15 @@ def cpu_baseline(args, budget_seconds=45.0):
                 "sample": f"a CPU pipeline process failed (exit codes {[p.returncode for p in procs]})"}
     rep = json.loads([ln for ln in out0.splitlines() if ln.startswith("{")][-1])
     n, M = rep["microbatches_timed"], rep["microbatches"]
-    what = "one full step" if n == M else f"the first {n} of {M} microbatches of one step"
+    k = len(rep["step_times_s"])
+    what = (f"median of {k} full steps after {rep['warmup_steps']} warm-up step" if n == M and k > 1 else
+            "one full step" if n == M else f"the first {n} of {M} microbatches of one step")
     return {"value": round(rep["tokens"] / rep["step_s"], 1), "unit": "tokens/s", "cores": S * threads,
             "kind": "port", "dtype": "bf16", "processes": S, "threads_per_process": threads,
             "sample": f"{what} ({rep['tokens']} tokens) of the same workload: {S} CPU processes over gloo, one "
                       f"per stage, 1F1B, bf16, after a warm-up of {rep['warmup_microbatches']} microbatch "
-                      f"({rep['warmup_s']:.1f} s); timed {rep['step_s']:.1f} s"}
+                      f"({rep['warmup_s']:.1f} s); timed steps "
+                      f"{', '.join(f'{t:.1f}' for t in rep['step_times_s'])} s"}
 
 
 GEMM_SHAPES = (
@@ -370,15 +374,12 @@ def rowwise_shapes():
 
 def gemm_shapes():
     """One JSON line per shape: the library's GEMM and torch.matmul on the same operands, each timed over
-    rotating operand sets (so that operands are not L2-resident from the previous launch) with the shader
-    clock sampled by a one-wave probe on a second stream while the launches run."""
+    rotating operand sets (so that operands are not L2-resident from the previous launch)."""
     from pippy_amd import _native as N
     from pippy_amd._program import splitk_copies
     N.lib()
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    side = torch.cuda.Stream()
-    clk = torch.zeros(2, dtype=torch.int64, device=dev)
 
     def timed(fns, flops):
         for f in fns:
@@ -392,15 +393,7 @@ def gemm_shapes():
                 f()
         ev1.record()
         torch.cuda.synchronize()
-        us = ev0.elapsed_time(ev1) * 1e3 / (reps * len(fns))
-        # the same launches again, enough of them to outlast the 2 ms probe
-        for _ in range(max(reps, int(4e3 / (us * len(fns))) + 1)):
-            for f in fns:
-                f()
-        N.clock_probe(clk, 2e-3, side.cuda_stream)
-        torch.cuda.synchronize()
-        c, w = clk.tolist()
-        return us, c / max(w, 1) * 100.0   # MHz
+        return ev0.elapsed_time(ev1) * 1e3 / (reps * len(fns))
 
     for (M, Nn, K, at, bt, what) in GEMM_SHAPES:
         sets = []
@@ -416,8 +409,8 @@ def gemm_shapes():
             ours = [(lambda s=s: N.gemm_bf16_splitk(s[0], s[1], s[2], ws)) for s in sets]
         else:
             ours = [(lambda s=s: N.gemm_bf16(s[0], s[1], s[2], a_trans=bool(at), b_trans=bool(bt))) for s in sets]
-        ours_us, ours_mhz = timed(ours, flops)
-        lib_us, lib_mhz = timed([(lambda s=s: torch.matmul(s[0].t() if at else s[0], s[1] if bt else s[1].t(),
+        ours_us = timed(ours, flops)
+        lib_us = timed([(lambda s=s: torch.matmul(s[0].t() if at else s[0], s[1] if bt else s[1].t(),
                                                            out=s[2])) for s in sets], flops)
         # the per-layer shapes once more as 2 and 4 independent problems in one grouped launch: what the
         # same-shaped GEMMs of several pipeline stages would cost each if the stages ran in lock step
@@ -426,13 +419,12 @@ def gemm_shapes():
             for k in (2, 4):
                 more = [[(torch.randn_like(s[0]), torch.randn_like(s[1]) * 0.05, torch.empty_like(s[2]),
                           dict(a_trans=bool(at), b_trans=bool(bt))) for _ in range(k)] for s in sets]
-                us_k, _ = timed([(lambda ps=ps: N.gemm_bf16_grouped(ps)) for ps in more], k * flops)
+                us_k = timed([(lambda ps=ps: N.gemm_bf16_grouped(ps)) for ps in more], k * flops)
                 grouped[f"grouped{k}_us_each"] = round(us_k / k, 1)
                 del more
         print(json.dumps({"shape": [M, Nn, K], "a_trans": at, "b_trans": bt, "what": what, "k_splits": copies,
                           "us": round(ours_us, 1), "tflops": round(flops / ours_us / 1e6, 1),
-                          "shader_mhz": round(ours_mhz), "vendor_us": round(lib_us, 1),
-                          "vendor_tflops": round(flops / lib_us / 1e6, 1), "vendor_shader_mhz": round(lib_mhz),
+                          "vendor_us": round(lib_us, 1), "vendor_tflops": round(flops / lib_us / 1e6, 1),
                           **grouped}),
               flush=True)
         del sets
@@ -456,8 +448,8 @@ def main():
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--gemm-shapes", action="store_true",
                     help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
-                         "events, cold operands), torch.matmul (the vendor library) on the same operands beside "
-                         "it, and sample the shader clock during each; one JSON line per shape")
+                         "events, cold operands) and torch.matmul (the vendor library) on the same operands beside "
+                         "it; one JSON line per shape")
     ap.add_argument("--attention-shapes", action="store_true",
                     help="instead of a step: time the attention kernels alone on the shapes of the workloads, "
                          "torch's scaled_dot_product_attention backends on the same operands beside them, then "

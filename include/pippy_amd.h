@@ -169,6 +169,19 @@ int pp_gemm_bf16_splitk(const pp_gemm_desc* desc, float* workspace, int64_t work
 #define PP_GEMM_MAX_GROUP 28
 int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream);
 
+/* The weight gradients of several microbatches in one launch.  Problem i is
+ *   C_i = (beta ? C_i : 0) + g_0 + g_1 + ... + g_{n_seg-1},   g_s = A_{i,s}^T B_{i,s}
+ * with the terms added one at a time in ascending s in fp32 (g_s rounded to bf16 first under
+ * PP_EPI_ACCUM_ROUNDED): bit for bit what n_seg accumulating pp_gemm_bf16_grouped launches, one per
+ * microbatch in ascending order, leave in C (the reference reaches them through one autograd pass per
+ * microbatch, pippy/_backward.py:67-69, accumulating in backward-microbatch order,
+ * pippy/PipelineSchedule.py:327,401-438).  A tile keeps its running sum in registers, so C moves once
+ * instead of n_seg times.  Every descriptor: a_trans = b_trans = 1, fp32 C, PP_EPI_ACCUM_F32 or _ROUNDED;
+ * desc->A and desc->B are DEVICE arrays of n_seg device pointers to the [K, M] and [K, N] operands of the
+ * segments (each 16-byte aligned, which the caller vouches for; K, lda, ldb are shared by the segments). */
+#define PP_GEMM_MAX_KSEG 1024
+int pp_gemm_bf16_grouped_kseg(const pp_gemm_desc* descs, int n, int n_seg, pp_stream stream);
+
 /* One GEMM per segment of a row-partitioned operand, with the segment bounds in DEVICE memory:
  * seg_start[0 .. n_seg] ascending row indices (int32), read by the kernel, so that sizes produced on
  * the device (the token counts of the experts of a mixture-of-experts layer, which the reference
@@ -415,7 +428,8 @@ enum pp_op_kind {
     PP_OP_ACCUM_F32 = 13, PP_OP_COPY_ROWS = 14, PP_OP_FILL = 15, PP_OP_ACT_BWD = 16,
     PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
     PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
-    PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27, PP_OP_POSITION_IDS = 28
+    PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27, PP_OP_POSITION_IDS = 28,
+    PP_OP_GEMM_KSEG = 29
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -448,6 +462,9 @@ enum pp_op_kind {
  *   MOE_GATE_BWD  p: dout y pos topk_idx gate dlogits | i: ld_dout ld_y topk E ld_dl T C
  *   GEMM_SWIGLU   p: x w_gate w_up gu h | i: M N K ldx ldw ld_gu ldh
  *   GEMM_DSWIGLU  p: dy w_down_t gu dgu | i: M N K ldy ldw ld_gu ld_dgu
+ *   GEMM_KSEG     as GEMM_BF16 with p[0], p[1]: device arrays of the segments' A and B pointers
+ *                 | i[7]: n_seg; consecutive GEMM_KSEG ops with the same n_seg go out as ONE
+ *                 pp_gemm_bf16_grouped_kseg call (they must not depend on each other)
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped
@@ -479,12 +496,6 @@ int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream);
 int pp_profile_start(int max_records);
 int pp_profile_stop(void);
 int pp_profile_read(int kind, double* total_ms, double* total_work, int64_t* count);
-
-/* Samples the shader clock (measurement aid; no reference counterpart): one wave idles for
- * `wall_ticks` ticks of the constant 100 MHz counter (at most 1e8 = one second) and writes
- * out[0] = shader clocks elapsed, out[1] = ticks elapsed (device memory, two int64).  Launched on a
- * stream of its own beside other work, out[0] / out[1] * 100 MHz is the clock that work runs at. */
-int pp_clock_probe(int64_t* out, int64_t wall_ticks, pp_stream stream);
 
 #ifdef __cplusplus
 }

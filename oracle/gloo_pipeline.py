@@ -12,7 +12,7 @@ gradients accumulate in ``param.grad`` in the parameter dtype as they do in the 
 process group is started as in the reference's tests (test/test_fwd.py:117-129: backend gloo on CPU).
 
 Run as ``python -m oracle.gloo_pipeline --rank R --world S ...`` with MASTER_ADDR / MASTER_PORT set;
-rank 0 prints one JSON line with the wall time of the timed step.
+rank 0 prints one JSON line with the wall times of the timed steps (their median is the figure).
 """
 import argparse
 import json
@@ -92,9 +92,12 @@ def main():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--microbatches", type=int, default=8)
     ap.add_argument("--warmup-microbatches", type=int, default=1)
+    ap.add_argument("--warmup-steps", type=int, default=1, help="untimed full steps before the timed ones")
+    ap.add_argument("--timed-steps", type=int, default=3, help="timed full steps; the median is reported")
     ap.add_argument("--budget-seconds", type=float, default=0.0,
-                    help="if > 0, time the first M' = M, M/2, M/4 ... microbatches of the step, the largest "
-                         "count whose time, estimated from the warm-up, stays within the budget")
+                    help="if > 0 and the warm-up microbatch says that the warm-up and timed steps would "
+                         "overrun it: one timed step without a warm-up step, over the first M' = M, M/2, "
+                         "M/4 ... microbatches, the largest count that stays within the budget")
     args = ap.parse_args()
 
     torch.set_num_threads(max(1, args.threads))
@@ -119,24 +122,39 @@ def main():
     for p in stage.parameters():
         p.grad = None
 
-    # how much of the step is timed: all of it unless the warm-up says that would overrun the budget
-    # (a pipelined step of M microbatches over S stages lasts about (M + S - 1) / S single-microbatch
-    # passes through the whole pipeline, which is what the warm-up timed)
-    n_timed = args.microbatches
+    # how much is timed: by default whole steps (warm-up steps, then timed steps); when the warm-up
+    # microbatch says that this would overrun the budget, one step, or the first half (quarter ...) of
+    # its microbatches (a pipelined step of M microbatches over S stages lasts about (M + S - 1) / S
+    # single-microbatch passes through the whole pipeline, which is what the warm-up timed)
+    n_timed, warm_steps, timed_steps = args.microbatches, max(0, args.warmup_steps), max(1, args.timed_steps)
     if args.budget_seconds > 0:
         per_pass = warm_s / w
-        while n_timed > 1 and per_pass * (n_timed + args.world - 1) / args.world > args.budget_seconds:
-            n_timed //= 2
-    decided = torch.tensor([n_timed])
+        est = lambda n: per_pass * (n + args.world - 1) / args.world  # noqa: E731
+        if est(n_timed) * (warm_steps + timed_steps) > args.budget_seconds:
+            warm_steps, timed_steps = 0, 1
+            while n_timed > 1 and est(n_timed) > args.budget_seconds:
+                n_timed //= 2
+    decided = torch.tensor([n_timed, warm_steps, timed_steps])
     dist.broadcast(decided, src=0)
-    n_timed = int(decided[0])
+    n_timed, warm_steps, timed_steps = (int(v) for v in decided)
 
-    dist.barrier()
-    t0 = time.perf_counter()
-    losses = run_step(stage, args.rank, args.world, n_timed, ids_mbs[:n_timed], target_mbs[:n_timed], act_shape,
-                      dtype)
-    dist.barrier()
-    step_s = time.perf_counter() - t0
+    def zero_grads():
+        for p in stage.parameters():
+            p.grad = None
+
+    step_times, losses = [], None
+    for it in range(warm_steps + timed_steps):
+        zero_grads()
+        dist.barrier()
+        t0 = time.perf_counter()
+        got = run_step(stage, args.rank, args.world, n_timed, ids_mbs[:n_timed], target_mbs[:n_timed], act_shape,
+                       dtype)
+        dist.barrier()
+        if it >= warm_steps:
+            step_times.append(time.perf_counter() - t0)
+        if losses is None:
+            losses = got  # of the first step run after the gradients were cleared: what a test compares
+    step_s = sorted(step_times)[len(step_times) // 2]
     if args.rank == args.world - 1 and args.world > 1:
         # the last rank holds the losses; rank 0 reports, so send them over
         dist.send(torch.stack(losses).float(), dst=0)
@@ -146,7 +164,9 @@ def main():
             dist.recv(got, src=args.world - 1)
         else:
             got = torch.stack(losses).float()
-        print(json.dumps({"step_s": step_s, "warmup_s": warm_s, "warmup_microbatches": w,
+        print(json.dumps({"step_s": step_s, "step_times_s": step_times, "warmup_steps": warm_steps,
+                          "warmup_s": warm_s, "warmup_microbatches": w,
+                          "losses": [float(v) for v in got],
                           "tokens": n_timed * mb * args.seq, "microbatches_timed": n_timed,
                           "microbatches": args.microbatches, "threads_per_rank": torch.get_num_threads(),
                           "world": args.world, "dtype": args.dtype,

@@ -26,7 +26,8 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
 (OP_GEMM_BF16, OP_GEMM_F32, OP_COLSUM, OP_LN_FWD, OP_LN_BWD_INPUT, OP_LN_BWD_WEIGHT, OP_ATTN_FWD,
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
- OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU, OP_POSITION_IDS) = range(1, 29)
+ OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU, OP_POSITION_IDS,
+ OP_GEMM_KSEG) = range(1, 30)
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
@@ -38,13 +39,13 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_bf16_grouped_kseg", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
     "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc", "pp_gemm_bf16_swiglu", "pp_gemm_bf16_dswiglu",
-    "pp_clock_probe", "pp_embed_fwd_at", "pp_position_ids_from_padding",
+    "pp_embed_fwd_at", "pp_position_ids_from_padding",
 )
 
 
@@ -117,6 +118,7 @@ def lib() -> C.CDLL:
         "pp_gemm_f32": [C.POINTER(GemmDesc), vp],
         "pp_gemm_bf16_splitk": [C.POINTER(GemmDesc), vp, i64, vp],
         "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
+        "pp_gemm_bf16_grouped_kseg": [C.POINTER(GemmDesc), i32, i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
         "pp_colsum_bf16_noalloc": [vp, i64, i64, i64, vp, i32, vp],
         "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],
@@ -135,7 +137,6 @@ def lib() -> C.CDLL:
         "pp_transpose_bf16": [vp, i64, i64, i64, vp, i64, vp],
         "pp_profile_start": [i32],
         "pp_profile_stop": [],
-        "pp_clock_probe": [vp, i64, vp],
         "pp_profile_read": [i32, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i64)],
         "pp_swiglu_fwd": [vp, vp, vp, i64, vp],
         "pp_swiglu_bwd": [vp, vp, vp, vp, vp, i64, vp],
@@ -500,6 +501,49 @@ def gemm_bf16_grouped(problems) -> None:
     check(lib().pp_gemm_bf16_grouped(arr, len(problems), current_stream()), "pp_gemm_bf16_grouped")
 
 
+class KsegLaunch:
+    """Descriptors and device pointer tables of one ``pp_gemm_bf16_grouped_kseg`` launch, built once.
+
+    problems: list of (As, Bs, C, kwargs): the weight gradient C (fp32) over the segments (microbatches)
+    s of As[s]^T Bs[s], added in ascending s, all problems in one launch."""
+
+    def __init__(self, problems):
+        self.n_seg = len(problems[0][0])
+        self.n = len(problems)
+        self.arr = (GemmDesc * self.n)()
+        ptrs = []
+        for As, Bs, Cm, kw in problems:
+            assert len(As) == len(Bs) == self.n_seg
+            for t in list(As) + list(Bs):
+                assert t.data_ptr() % 16 == 0 and t.dtype == torch.bfloat16
+            assert all(a.shape == As[0].shape and a.stride() == As[0].stride() for a in As)
+            assert all(b.shape == Bs[0].shape and b.stride() == Bs[0].stride() for b in Bs)
+            ptrs += [a.data_ptr() for a in As] + [b.data_ptr() for b in Bs]
+        # one table for the whole launch: problem k's A pointers at [2 k n_seg, ...), its B pointers after them
+        self.table = torch.tensor(ptrs, dtype=torch.int64, device=problems[0][2].device)
+        for k, (As, Bs, Cm, kw) in enumerate(problems):
+            d = gemm_desc(As[0], Bs[0], Cm, a_trans=True, b_trans=True, **kw)
+            d.A = self.table.data_ptr() + 8 * (2 * k * self.n_seg)
+            d.B = self.table.data_ptr() + 8 * ((2 * k + 1) * self.n_seg)
+            C.memmove(C.byref(self.arr, k * C.sizeof(GemmDesc)), C.byref(d), C.sizeof(GemmDesc))
+        self.keep = problems
+
+    def run(self) -> None:
+        check(lib().pp_gemm_bf16_grouped_kseg(self.arr, self.n, self.n_seg, current_stream()),
+              "pp_gemm_bf16_grouped_kseg")
+
+
+def gemm_bf16_grouped_kseg(problems, keep=None) -> None:
+    """One launch of ``KsegLaunch(problems)``; ``keep`` (a list) receives the launch object, whose pointer
+    table must outlive the kernel (without it the call waits for the stream)."""
+    launch = KsegLaunch(problems)
+    launch.run()
+    if keep is not None:
+        keep.append(launch)
+    else:
+        torch.cuda.current_stream().synchronize()
+
+
 def gemm_f32(A, B, Cm, **kw) -> None:
     assert A.dtype == torch.float32 and B.dtype == torch.float32 and Cm.dtype == torch.float32
     d = gemm_desc(A, B, Cm, **kw)
@@ -688,14 +732,6 @@ def profile_start(max_records: int = 1 << 16) -> None:
 
 def profile_stop() -> None:
     check(lib().pp_profile_stop(), "pp_profile_stop")
-
-
-def clock_probe(out: torch.Tensor, seconds: float, stream: int) -> None:
-    """Launches the clock sampler on ``stream`` for ``seconds``; afterwards out[0] / out[1] * 1e8 is the
-    shader clock in Hz (``out``: two int64 on the device)."""
-    require_cuda(out)
-    assert out.dtype == torch.int64 and out.numel() >= 2 and out.is_contiguous()
-    check(lib().pp_clock_probe(out.data_ptr(), int(seconds * 1e8), stream), "pp_clock_probe")
 
 
 def profile_read(kind: int):

@@ -13,14 +13,16 @@ from ._IR import _attr, pipe_split
 
 def _state_of_nodes(gm: fx.GraphModule) -> List[Tuple[fx.Node, Dict[int, int], bool]]:
     """(node, {id(tensor): elements}, whole) for every node that reads parameters or buffers, in graph
-    order: a layer call reads the state of its module (``whole``: always counted in full, reference
+    order: a layer call reads the parameters of its module (``whole``: always counted in full, reference
     ``ModelSplit.py:107-110``), any other node the tensors that ``get_attr`` nodes hand it."""
     found = []
     for node in gm.graph.nodes:
         state: Dict[int, int] = {}
         if node.op == "call_module":
             sub = gm.get_submodule(node.target)
-            for t in list(sub.parameters()) + list(sub.buffers()):
+            # parameters only, and in full on every call of the module, as the reference counts a layer
+            # (``ModelSplit.py:45-52``: ``named_parameters``; buffers of a layer are not counted)
+            for t in sub.parameters():
                 state[id(t)] = t.numel()
             whole = True
         else:

@@ -213,14 +213,6 @@ struct WaveTile {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "a wave's part of the tile is made of 32 x 32 MFMA tiles");
 };
 
-// Measurement builds only: PP_GEMM_KNOCKOUT removes one ingredient of the k-loop, so that timing the
-// kernels with and without it shows what each costs (1: no loads inside the loop, 2: no LDS fragment
-// reads after a tile's first two, 3: no MFMAs).  Results are wrong by construction; an ordinary build
-// does not define it.
-#ifndef PP_GEMM_KNOCKOUT
-#define PP_GEMM_KNOCKOUT 0
-#endif
-
 // Main loop of one BM x BN output tile over the k-tiles [kt_begin, kt_end) of KT values each, through
 // NS LDS stages filled by direct-to-LDS loads; the products are added to acc.  Starts with a barrier,
 // so that it may follow an epilogue (or another main loop) that used the same LDS.
@@ -267,14 +259,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
 #pragma unroll
     for (int t = 0; t < TN; ++t) rb[t].init(wn0 + t * 32, lane);
     bf16x8_t fa[2][TM], fb[2][TN];
-#if PP_GEMM_KNOCKOUT == 2
-    bool first_reads = true;
-#endif
     auto read_frags = [&](int sel, const uint16_t* st, int ks) {
-#if PP_GEMM_KNOCKOUT == 2
-        if (!first_reads && ks >= 2) return;
-        if (ks == 1) first_reads = false;
-#endif
 #pragma unroll
         for (int t = 0; t < TM; ++t) fa[sel][t] = ra[t].read(st, ks);
 #pragma unroll
@@ -285,11 +270,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
         for (int a = a_lo; a < a_hi; ++a)
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
-#if PP_GEMM_KNOCKOUT == 3
-                asm volatile("" ::"v"(fb[sel][a]), "v"(fa[sel][b]));  // the fragments stay live
-#else
                 acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[sel][a], fa[sel][b], acc[a][b], 0, 0, 0);
-#endif
             }
     };
     auto interleave = [&]() { interleave_reads<kReadsPerStep, TM * TN, 0>(); };
@@ -322,9 +303,7 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
         else wait_vmcnt<0>();
         wait_lds();  // this wave's reads of the current stage are done: the stage may be refilled
         __builtin_amdgcn_s_barrier();
-#if PP_GEMM_KNOCKOUT != 1
         if (kt + NS < nk) issue(stage, kt + NS);
-#endif
         stage = stage + 1 == NS ? 0 : stage + 1;
         if (kt + 1 < nk) read_frags(0, smem + stage * kStageElems, 0);
         mma(kLast, TN / 2, TN);

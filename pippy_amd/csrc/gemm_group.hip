@@ -7,6 +7,14 @@
 #include "gemm_core.h"
 #include <vector>
 
+#ifndef PP_KSEG_BM
+#define PP_KSEG_BM 128
+#define PP_KSEG_BN 128
+#define PP_KSEG_W 4
+#define PP_KSEG_NS 2
+#define PP_KSEG_KT 64
+#endif
+
 namespace pp {
 
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT>
@@ -56,9 +64,164 @@ static int launch_layout(GemmGroupArgs& ga, int at, int bt, hipStream_t st) {
     return launch_auto<true, true, EPI, CF32>(ga, st);
 }
 
+// ---- weight gradients of several microbatches in one launch --------------------------------------
+// Problem i is  C_i = (beta ? C_i : 0) + g_0 + g_1 + ... + g_{S-1}  with  g_s = A_{i,s}^T B_{i,s}  (rounded to
+// bf16 first when the problem says so), the terms added one by one in ascending s in fp32: bit for bit
+// what S accumulating launches, one per microbatch, leave in C.  A tile keeps the running sum in
+// registers over all S reductions, so C is read (at most) once and written once instead of S times, and
+// the k-loop of a tile is S times as long.  GemmArgs::A and ::B of a problem point to DEVICE arrays of
+// its S operand pointers.
+template <int BM, int BN, int W>
+__device__ __forceinline__ void load_c_as_accumulators(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
+                                                       f32x16_t (&t)[WaveTile<BM, BN, W>::TN][WaveTile<BM, BN, W>::TM]) {
+    typedef WaveTile<BM, BN, W> WT;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int64_t m_base = (int64_t)tile_m * BM + (wave % WT::WGM) * WT::WTM + l32;
+    const int64_t n_base = (int64_t)tile_n * BN + (wave / WT::WGM) * WT::WTN + 4 * lh;
+    const float* C = static_cast<const float*>(g.C);
+    const bool vec_ok = (g.ldc & 3) == 0 && aligned(g.C, 16);
+#pragma unroll
+    for (int a = 0; a < WT::TN; ++a)
+#pragma unroll
+        for (int b = 0; b < WT::TM; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                // the accumulator layout of v_mfma_f32_32x32x16 with B as the first operand: a lane holds,
+                // for one row, four groups of four consecutive columns
+                const int64_t m = m_base + b * 32, n = n_base + a * 32 + 8 * q;
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                if (m < g.M) {
+                    if (vec_ok && n + 3 < g.N) {
+                        const float4 w = *reinterpret_cast<const float4*>(C + m * g.ldc + n);
+                        v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (n + e < g.N) v[e] = C[m * g.ldc + n + e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[a][b][4 * q + e] = v[e];
+            }
+}
+
+template <int BM, int BN, int NS, int KT, int W>
+__global__ __launch_bounds__(W * 64) void gemm_bf16_group_kseg_kernel(const GemmGroupArgs ga, const int n_seg) {
+    uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= ga.tile_start[ga.n]) return;
+    int i = 0;
+    while (i + 1 < ga.n && bid >= ga.tile_start[i + 1]) ++i;
+    bid -= ga.tile_start[i];
+    GemmArgs g = ga.p[i];
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    typedef WaveTile<BM, BN, W> WT;
+    const uint16_t* const* seg_a = reinterpret_cast<const uint16_t* const*>(g.A);
+    const uint16_t* const* seg_b = reinterpret_cast<const uint16_t* const*>(g.B);
+    f32x16_t total[WT::TN][WT::TM], acc[WT::TN][WT::TM];
+    if (g.beta) load_c_as_accumulators<BM, BN, W>(g, tile_m, tile_n, total);
+    const int nk = (int)((g.K + KT - 1) / KT);
+    for (int s = 0; s < n_seg; ++s) {
+        g.A = seg_a[s];
+        g.B = seg_b[s];
+#pragma unroll
+        for (int a = 0; a < WT::TN; ++a)
+#pragma unroll
+            for (int b = 0; b < WT::TM; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+        gemm_mainloop<BM, BN, true, true, NS, KT, false, W>(g, tile_m, tile_n, 0, nk, acc);
+        const bool first = s == 0 && !g.beta;  // the first term of a fresh sum is stored, not added to zero
+#pragma unroll
+        for (int a = 0; a < WT::TN; ++a)
+#pragma unroll
+            for (int b = 0; b < WT::TM; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; e += 2) {
+                    float lo = acc[a][b][e], hi = acc[a][b][e + 1];
+                    if (g.round_bf16) {
+                        const uint32_t w = pack_bf16(lo, hi);
+                        lo = bf16lo(w);
+                        hi = bf16hi(w);
+                    }
+                    total[a][b][e] = first ? lo : total[a][b][e] + lo;
+                    total[a][b][e + 1] = first ? hi : total[a][b][e + 1] + hi;
+                }
+    }
+    g.beta = 0;
+    g.round_bf16 = 0;
+    gemm_epilogue<BM, BN, PP_EPI_NONE, true, 0, W>(g, tile_m, tile_n, total);
+}
+
+template <int BM, int BN, int NS, int KT, int W>
+static int launch_group_kseg(GemmGroupArgs& ga, int n_seg, hipStream_t st) {
+    constexpr size_t lds = (size_t)NS * (BM + BN) * KT * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_group_kseg_kernel<BM, BN, NS, KT, W>, lds);
+    if (attr_rc) return attr_rc;
+    uint64_t total = 0;
+    for (int i = 0; i < ga.n; ++i) {
+        int rc = count_tiles<BM, BN>(ga.p[i]);
+        if (rc) return rc;
+        ga.tile_start[i] = (uint32_t)total;
+        total += ga.p[i].n_blocks;
+    }
+    if (total > 0x7fffff00ull) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_grouped_kseg: too many tiles");
+    ga.tile_start[ga.n] = (uint32_t)total;
+    if (total == 0) return PP_OK;
+    const uint32_t grid = ((uint32_t)total + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_group_kseg_kernel<BM, BN, NS, KT, W>), dim3(grid), dim3(W * 64), lds, st, ga,
+                       n_seg);
+    return check_launch("gemm_bf16_group_kseg_kernel");
+}
+
 }  // namespace pp
 
 using namespace pp;
+
+extern "C" int pp_gemm_bf16_grouped_kseg(const pp_gemm_desc* descs, int n, int n_seg, pp_stream stream) {
+    if (n < 0 || (n > 0 && !descs)) return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped_kseg: bad list");
+    if (n_seg < 1 || n_seg > PP_GEMM_MAX_KSEG)
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped_kseg: n_seg %d out of [1, %d]", n_seg, PP_GEMM_MAX_KSEG);
+    std::vector<GemmArgs> probs;
+    probs.reserve(n);
+    for (int i = 0; i < n; ++i) {
+        const pp_gemm_desc& d = descs[i];
+        if (!d.a_trans || !d.b_trans || d.c_dtype != PP_F32 ||
+            (d.epilogue != PP_EPI_ACCUM_F32 && d.epilogue != PP_EPI_ACCUM_ROUNDED))
+            return fail(PP_ERR_UNSUPPORTED, "pp_gemm_bf16_grouped_kseg: problem %d is not a transposed-operand "
+                        "product accumulated into an fp32 C", i);
+        if (!aligned(d.A, 8) || !aligned(d.B, 8))
+            return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped_kseg: problem %d: A and B are device arrays of "
+                        "pointers", i);
+        // the operand checks of a single product, on a copy whose operands pass the alignment test (the
+        // real operand pointers live in device memory; the caller vouches for their 16-byte alignment)
+        pp_gemm_desc probe = d;
+        probe.A = probe.B = reinterpret_cast<const void*>(uintptr_t(16));
+        GemmArgs g;
+        bool empty;
+        int rc = convert(&probe, &g, &empty);
+        if (rc) return rc;
+        if (empty) continue;
+        g.A = static_cast<const uint16_t*>(d.A);
+        g.B = static_cast<const uint16_t*>(d.B);
+        probs.push_back(g);
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int total = (int)probs.size();
+    const int launches = (total + PP_GEMM_MAX_GROUP - 1) / PP_GEMM_MAX_GROUP;
+    int done = 0;
+    for (int l = 0; l < launches; ++l) {
+        const int cnt = (total - done + (launches - l) - 1) / (launches - l);
+        GemmGroupArgs ga;
+        ga.n = cnt;
+        for (int i = 0; i < cnt; ++i) ga.p[i] = probs[done + i];
+        done += cnt;
+        int rc = launch_group_kseg<PP_KSEG_BM, PP_KSEG_BN, PP_KSEG_NS, PP_KSEG_KT, PP_KSEG_W>(ga, n_seg, st);
+        if (rc) return rc;
+    }
+    return PP_OK;
+}
 
 extern "C" int pp_gemm_bf16_grouped(const pp_gemm_desc* descs, int n, pp_stream stream) {
     if (n < 0 || (n > 0 && !descs)) return fail(PP_ERR_INVALID, "pp_gemm_bf16_grouped: bad list");

@@ -31,6 +31,16 @@ static int group_length(const pp_op* ops, int i, int n_ops) {
     return len;
 }
 
+// Number of consecutive weight-gradient ops over several microbatches (same segment count) from ops[i].
+static int kseg_group_length(const pp_op* ops, int i, int n_ops) {
+    if (ops[i].kind != PP_OP_GEMM_KSEG || (ops[i].flags & PP_OP_SKIP)) return 0;
+    int len = 1;
+    while (i + len < n_ops && ops[i + len].kind == PP_OP_GEMM_KSEG && !(ops[i + len].flags & PP_OP_SKIP) &&
+           ops[i + len].i[7] == ops[i].i[7])
+        ++len;
+    return len;
+}
+
 static bool is_colreduce(const pp_op& o) {
     return (o.kind == PP_OP_COLSUM || o.kind == PP_OP_LN_BWD_WEIGHT) && (o.flags & PP_OP_GROUPED) &&
            !(o.flags & PP_OP_SKIP);
@@ -192,6 +202,8 @@ double op_work(const pp_op& op) {
         case PP_OP_GEMM_DSWIGLU:
         case PP_OP_GEMM_SEG:  // the segments partition the rows (rows mode: M, k mode: K)
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
+        case PP_OP_GEMM_KSEG:  // one product per segment
+            return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2] * (double)op.i[7];
         case PP_OP_GEMM_SWIGLU:  // two products of N columns each
             return 4.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_ATTN_FWD:  // dense count: QK^T and PV
@@ -237,31 +249,6 @@ double op_work(const pp_op& op) {
     }
 }
 }  // namespace
-
-// One wave that idles for `wall_ticks` ticks of the constant 100 MHz counter and reports how many
-// shader clocks passed meanwhile: launched on a stream of its own beside other work, it samples the
-// clock that the work runs at.
-__global__ void clock_probe_kernel(long long* out, long long wall_ticks) {
-    const long long c0 = clock64(), w0 = wall_clock64();
-    long long w1 = w0;
-    while (w1 - w0 < wall_ticks) {
-        __builtin_amdgcn_s_sleep(8);
-        w1 = wall_clock64();
-    }
-    const long long c1 = clock64();
-    if (threadIdx.x == 0) {
-        out[0] = c1 - c0;
-        out[1] = w1 - w0;
-    }
-}
-
-extern "C" int pp_clock_probe(int64_t* out, int64_t wall_ticks, pp_stream stream) {
-    if (!out) return fail(PP_ERR_INVALID, "pp_clock_probe: null pointer");
-    if (wall_ticks < 0 || wall_ticks > 100000000) return fail(PP_ERR_INVALID, "pp_clock_probe: 0 <= wall_ticks <= 1e8 (one second)");
-    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
-                       reinterpret_cast<long long*>(out), (long long)wall_ticks);
-    return check_launch("clock_probe_kernel");
-}
 
 extern "C" int pp_profile_start(int max_records) {
     if (max_records <= 0) return fail(PP_ERR_INVALID, "pp_profile_start: max_records <= 0");
@@ -312,6 +299,8 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
         int glen = group_length(ops, i, n_ops);
         const int clen = glen ? 0 : colreduce_group_length(ops, i, n_ops);
         if (clen > 1) glen = clen;
+        const int klen = kseg_group_length(ops, i, n_ops);
+        if (klen) glen = klen;
         ProfRecord* rec = nullptr;
         if (g_prof_on) {
             if (g_prof_used < g_prof.size()) {
@@ -325,7 +314,12 @@ extern "C" int pp_run_ops(const pp_op* ops, int n_ops, pp_stream stream) {
             }
         }
         int rc;
-        if (clen > 1) {
+        if (klen) {
+            std::vector<pp_gemm_desc> descs;
+            descs.reserve(klen);
+            for (int q = 0; q < klen; ++q) descs.push_back(gemm_desc_of(ops[i + q]));
+            rc = pp_gemm_bf16_grouped_kseg(descs.data(), klen, (int)ops[i].i[7], stream);
+        } else if (clen > 1) {
             std::vector<pp_colreduce_desc> descs;
             descs.reserve(clen);
             for (int q = 0; q < clen; ++q) descs.push_back(colreduce_desc_of(ops[i + q]));

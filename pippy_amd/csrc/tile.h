@@ -68,6 +68,41 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 // flight.
 typedef __attribute__((address_space(3))) void* lds_void_ptr_t;
 
+// The loads are written as inline assembly on purpose.  Issued through the compiler's builtin, the
+// compiler knows that they write LDS, cannot tell which part, and therefore makes every later LDS read
+// wait for ALL outstanding loads (s_waitcnt vmcnt(0) in front of the first fragment read of the next
+// tile): the loads of tile t + 2 would then finish before tile t + 1 is touched, and nothing would
+// overlap.  The kernels order loads and reads themselves, with explicit vmcnt waits and barriers.
+struct LdsDmaRsrc {
+    u32x4_t w;  // buffer resource words, wave-uniform (SGPRs)
+};
+
+__device__ __forceinline__ LdsDmaRsrc make_lds_dma_rsrc(const void* base, uint64_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+    LdsDmaRsrc r;
+    r.w.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    r.w.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);  // stride 0: raw buffer
+    r.w.z = __builtin_amdgcn_readfirstlane(n);
+    r.w.w = 0x00020000u;
+    return r;
+}
+
+// One wave load of 64 x 16 bytes to `lds_wave_base` + 16 * lane; `soffset` must be wave-uniform.
+__device__ __forceinline__ void load_to_lds_b128(const LdsDmaRsrc& rsrc, uint16_t* lds_wave_base, int voffset,
+                                                 int soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_void_ptr_t)lds_wave_base;
+    asm volatile("s_mov_b32 m0, %0\n\t"
+                 "s_nop 0\n\t"
+                 "buffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc.w),
+                   "s"(__builtin_amdgcn_readfirstlane(soffset))
+                 : "memory", "m0");
+#endif
+}
+
 __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint16_t* lds_wave_base,
                                                  int voffset, int soffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -96,14 +131,14 @@ struct DmaStage<ROWS, false, KT, W> {
     static constexpr int kRowsPerLoad = 64 / kChunks;   // rows covered by one wave load
     static constexpr int kLoads = ROWS / kRowsPerLoad / W;
     static_assert(ROWS % (kRowsPerLoad * W) == 0, "tile rows must divide over the waves' loads");
-    __amdgpu_buffer_rsrc_t rsrc;
+    LdsDmaRsrc rsrc;
     int voff[kLoads];
     int kcol[kLoads];  // first k of this lane's chunk within a tile
     int K;
     __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
                                          int64_t rows_total, int64_t K_, int wave, int lane) {
         const uint64_t bytes = (uint64_t)(rows_total - row0) * (uint64_t)ld * 2;
-        rsrc = make_rsrc(base + row0 * ld, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
+        rsrc = make_lds_dma_rsrc(base + row0 * ld, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
         K = (int)K_;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
@@ -139,13 +174,13 @@ struct DmaStage<ROWS, true, KT, W> {
     static constexpr int kLoads = KT / kRowsPerLoad / W;
     static_assert(ROWS % 128 == 0 && ROWS <= 512, "transposed tiles are staged 128 rows at a time");
     static_assert(kLoads >= 1, "a wave load must not span more k-rows than a quarter of the tile");
-    __amdgpu_buffer_rsrc_t rsrc;
+    LdsDmaRsrc rsrc;
     int voff[kLoads];
     int ld2;  // bytes per k-row of the operand
     __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int64_t row0,
                                          int64_t rows_total, int64_t K_, int wave, int lane) {
         const uint64_t bytes = ((uint64_t)K_ * (uint64_t)ld - (uint64_t)row0) * 2;
-        rsrc = make_rsrc(base + row0, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
+        rsrc = make_lds_dma_rsrc(base + row0, bytes < 0x7ffffff0ull ? bytes : 0x7ffffff0ull);
         ld2 = (int)(ld * 2);
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {

@@ -262,6 +262,10 @@ class PipelineSchedule(ABC):
             done = self._event(("done_w", s))
             done.record(w_streams[s])
             main.wait_event(done)
+        if merger is not None:
+            # also for a caller that drives _step_microbatches itself and never asks for the merged result:
+            # the copies read the per-microbatch output buffers that the next step overwrites
+            main.wait_stream(merger.stream)
 
     def _merger(self, main) -> Optional[_RunningMerge]:
         """The running merge of this step, or None when outputs are merged at the end."""

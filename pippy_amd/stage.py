@@ -116,6 +116,13 @@ class PipelineStageBase:
             force_eager = True
             why.append(f"its device is '{self.device}' and launch lists run on the GPU only")
         self._blocks = None if force_eager else lower_stage_module(submodule, why, for_kernels=True)
+        # Whether a dropout does nothing is decided when the stage is lowered (p == 0, or eval mode).  The
+        # layers that were taken as identity only because of the mode are remembered: a launch-list stage
+        # whose module is switched to training mode afterwards would otherwise train without dropout.
+        self._mode_bound_dropouts: List[nn.Module] = [] if self._blocks is None else [
+            m for m in submodule.modules()
+            if (isinstance(m, nn.modules.dropout._DropoutNd) and m.p > 0)
+            or (isinstance(m, nn.MultiheadAttention) and m.dropout > 0)]
         self._program: Optional[P.StageProgram] = None
         #: why this stage runs through torch autograd instead of HIP launch lists (None: it is native)
         self.eager_reason: Optional[str] = None
@@ -333,6 +340,12 @@ class PipelineStageBase:
         return self._exported_shape
 
     def _forward_native(self, mb, args, kwargs):
+        if self._mode_bound_dropouts and any(m.training for m in self._mode_bound_dropouts):
+            raise RuntimeError(
+                f"{self.log_prefix} was lowered to launch lists in eval mode, where its dropout layers (p > 0) do "
+                "nothing, and its module is in training mode now: the launch lists hold no dropout.  Set the mode "
+                "before the stage is built (a stage built in training mode with p > 0 runs through torch "
+                "autograd), or set the dropout probabilities to 0")
         sp = self._stage_program()
         x, dx_target, patch = self._input_for(mb, args, kwargs)
         expected = self._exported_input_shape()

@@ -179,3 +179,52 @@ def test_copy_rows_with_unaligned_rows_is_bit_exact(dtype, V, ld, rows):
         got = dst[shift:shift + rows * V].view(rows, V)
         assert torch.equal(got, src[:, :V])
         assert float(dst[:shift].float().abs().sum()) == 0 and float(dst[shift + rows * V:].float().abs().sum()) == 0
+
+
+@pytest.mark.parametrize("epi_name", ["rounded", "f32"])
+@pytest.mark.parametrize("beta", [0, 1])
+def test_weight_gradients_of_several_microbatches_in_one_launch_equal_one_launch_each(epi_name, beta):
+    """``pp_gemm_bf16_grouped_kseg``: C = (beta ? C : 0) + g_0 + g_1 + ... added in microbatch order must
+    leave the bits that one accumulating launch per microbatch leaves (fp32 addition is not associative,
+    so the order and the per-microbatch rounding both show), for ragged shapes too."""
+    from pippy_amd import _native as N
+    N.lib()
+    torch.manual_seed(5)
+    epi = N.EPI_ACCUM_ROUNDED if epi_name == "rounded" else N.EPI_ACCUM_F32
+    n_seg, T = 5, 392                      # a token count that is no multiple of the k-tile
+    shapes = [(2304, 768), (768, 768), (136, 200), (8, 8), (3072, 256)]
+    problems, want = [], []
+    for out_f, in_f in shapes:
+        dYs = [torch.randn(T, out_f, device=DEV).to(torch.bfloat16) for _ in range(n_seg)]
+        Xs = [torch.randn(T, in_f, device=DEV).to(torch.bfloat16) for _ in range(n_seg)]
+        C0 = torch.randn(out_f, in_f, device=DEV) * 30
+        ref = C0.clone()
+        for s in range(n_seg):
+            N.gemm_bf16(dYs[s], Xs[s], ref, a_trans=True, b_trans=True, epilogue=epi, beta=1 if (s or beta) else 0)
+        got = C0.clone()
+        problems.append((dYs, Xs, got, dict(epilogue=epi, beta=beta)))
+        want.append(ref)
+    keep = []
+    N.gemm_bf16_grouped_kseg(problems, keep)
+    torch.cuda.synchronize()
+    for (_, _, got, _), ref in zip(problems, want):
+        assert torch.equal(got, ref)
+    # the sum is not the sum of a different order: adding the microbatches backwards differs somewhere
+    dYs, Xs, _, kw = problems[0]
+    back = (torch.zeros_like(want[0]) if not beta else None)
+    if back is not None:
+        N.gemm_bf16_grouped_kseg([(dYs[::-1], Xs[::-1], back, kw)], keep)
+        torch.cuda.synchronize()
+        assert not torch.equal(back, want[0])
+        assert torch.allclose(back, want[0], rtol=1e-3, atol=1e-2)
+
+
+def test_kseg_rejects_what_it_does_not_compute():
+    from pippy_amd import _native as N
+    A = torch.zeros(16, 16, device=DEV, dtype=torch.bfloat16)
+    Cb = torch.zeros(16, 16, device=DEV, dtype=torch.bfloat16)
+    Cf = torch.zeros(16, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="accumulated into an fp32 C"):
+        N.gemm_bf16_grouped_kseg([([A], [A], Cb, {})], [])
+    with pytest.raises(RuntimeError, match="accumulated into an fp32 C"):
+        N.gemm_bf16_grouped_kseg([([A], [A], Cf, {})], [])      # epilogue NONE does not accumulate

@@ -563,3 +563,50 @@ def test_split_policies_cut_by_parameter_count():
                     split_policy=pp.split_into_equal_size(2))
     with pytest.raises(NotImplementedError):
         pp.split_by_graph(2)
+
+
+def test_whether_a_dropout_is_a_no_op_is_decided_when_the_stage_is_lowered():
+    """A dropout with p > 0 is identity in eval mode only.  Lowering takes the decision once: in eval
+    mode the stage becomes launch lists, in training mode it stays with torch autograd (and says why)."""
+    from pippy_amd._lowering import lower_stage_module
+    m = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Dropout(0.1), nn.Linear(32, 16)).to(torch.bfloat16)
+    m.eval()
+    why = []
+    assert lower_stage_module(m, why, for_kernels=True) is not None
+    m.train()
+    why = []
+    assert lower_stage_module(m, why, for_kernels=True) is None
+    assert "dropout" in why[0]
+    # p == 0 is a no-op in either mode
+    m[2].p = 0.0
+    assert lower_stage_module(m, [], for_kernels=True) is not None
+
+
+def test_a_launch_list_stage_refuses_to_run_after_its_dropout_was_switched_on():
+    """The launch lists hold no dropout: a stage lowered in eval mode whose module is then put into
+    training mode (p > 0) raises instead of training without dropout; back in eval mode it runs."""
+    import pippy_amd as pp
+    from pippy_amd import stage as stage_mod
+    m = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Dropout(0.1), nn.Linear(32, 16)).to(torch.bfloat16).eval()
+    st = pp.ManualPipelineStage(m, 0, 1, "cpu", 1, input_args=(torch.zeros(2, 16, dtype=torch.bfloat16),))
+    assert st._mode_bound_dropouts == []          # eager on the CPU: torch's own dropout applies, nothing to guard
+    # the guard itself, on a stage object made to look lowered (launch lists need the GPU)
+    st._mode_bound_dropouts = [m[2]]
+    m.train()
+    with pytest.raises(RuntimeError, match="dropout"):
+        stage_mod.PipelineStageBase._forward_native(st, 0, (), {})
+
+
+def test_size_policy_counts_a_layers_parameters_not_its_buffers():
+    """Reference ``ModelSplit.py:45-52``: a layer call weighs what ``named_parameters`` holds.  The running
+    statistics of a normalisation layer (buffers) must not move the cut."""
+    import pippy_amd as pp
+    model = nn.Sequential(nn.Linear(8, 8), nn.BatchNorm1d(8), nn.Linear(8, 8), nn.BatchNorm1d(8),
+                          nn.Linear(8, 8), nn.BatchNorm1d(8), nn.Linear(8, 8), nn.BatchNorm1d(8)).eval()
+    pair = (8 * 8 + 8) + 2 * 8           # a linear layer and the weight and bias of its normalisation
+    # two pairs per stage by their parameters; with the 17 buffer elements of each BatchNorm counted too the
+    # second pair would not fit
+    pipe = pp.pipeline(model, 1, (torch.zeros(2, 8),), split_policy=pp.split_on_size_threshold(2 * pair))
+    assert pipe.num_stages == 2
+    keys0 = set(pipe.get_stage_module(0).state_dict())
+    assert {k.split(".")[0] for k in keys0} == {"0", "1", "2", "3"}

@@ -388,3 +388,63 @@ def test_moe_layer_equals_dense_sum_with_zero_weights_and_module_statement():
         assert layer.forced_routing == []
         assert torch.allclose(y_forced, O.moe_top2(x, moe.gate.weight, w1, w2, w3, idx=forced), rtol=1e-5, atol=1e-6)
         assert not torch.allclose(y_forced, y, atol=1e-3)
+
+
+def test_embedding_at_matches_torch_embedding():
+    torch.manual_seed(11)
+    wte, wpe = torch.randn(13, 6, dtype=torch.float64), torch.randn(9, 6, dtype=torch.float64)
+    ids, pos = torch.randint(0, 13, (3, 5)), torch.randint(0, 9, (3, 5))
+    extra = torch.randn(6, dtype=torch.float64)
+    want = F.embedding(ids, wte) + F.embedding(pos, wpe)
+    assert torch.equal(O.embedding_at(ids, pos, wte, wpe), want)
+    assert torch.equal(O.embedding_at(ids, pos, wte, wpe, extra), want + extra)
+    # a position index is not the token's place in its sequence: swapping two positions moves the rows
+    pos2 = pos.clone()
+    pos2[0, 0], pos2[0, 1] = pos[0, 1], pos[0, 0]
+    if pos[0, 0] != pos[0, 1]:
+        assert not torch.equal(O.embedding_at(ids, pos2, wte, wpe), want)
+
+
+def test_gloo_pipeline_processes_compute_the_losses_of_the_step_oracle():
+    """The CPU baseline of the bench (one process per stage over gloo, each running its rank's 1F1B
+    program) against ``oracle.pipeline.step`` on the same model, ids and targets: same per-microbatch
+    losses (fp32; the hand-offs move values, they do not change them)."""
+    import json
+    import os
+    import socket
+    import subprocess
+    import sys
+
+    from pippy_amd.configs import DecoderLM
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = dict(vocab=97, seq=16, dim=32, layers=2, heads=2, ffn=64, batch=8, microbatches=4)
+    with socket.socket() as sock:
+        sock.bind(("127.0.0.1", 0))
+        port = sock.getsockname()[1]
+    env = dict(os.environ, MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port), OMP_NUM_THREADS="1",
+               HIP_VISIBLE_DEVICES="", CUDA_VISIBLE_DEVICES="")
+    common = ["--world", "2", "--threads", "1", "--dtype", "fp32", "--warmup-steps", "0", "--timed-steps", "1"]
+    for k, v in cfg.items():
+        common += ["--" + k, str(v)]
+    procs = [subprocess.Popen([sys.executable, "-m", "oracle.gloo_pipeline", "--rank", str(r)] + common, cwd=root,
+                              env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True) for r in range(2)]
+    outs = [p.communicate(timeout=240) for p in procs]
+    assert all(p.returncode == 0 for p in procs), [o[1][-2000:] for o in outs]
+    rep = json.loads([ln for ln in outs[0][0].splitlines() if ln.startswith("{")][-1])
+    assert rep["microbatches_timed"] == 4 and rep["tokens"] == 8 * 16
+
+    # the same model (seed 0), ids and targets (generator seed 1) as the processes build them
+    torch.manual_seed(0)
+    model = DecoderLM(vocab=97, max_seq=16, dim=32, n_layers=2, n_heads=2, ffn=64, dtype=torch.float32)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, 97, (8, 16), generator=g)
+    target = torch.randint(0, 97, (8, 16), generator=g)
+    stages = [nn.Sequential(model.embed, model.h[0]), nn.Sequential(model.h[1], model.head)]
+    ce = lambda o, t: F.cross_entropy(o.reshape(-1, o.shape[-1]).float(), t.reshape(-1))  # noqa: E731
+    _, losses = OP.step(stages, ids, target, 4, ce)
+    want = torch.stack(losses)
+    got = torch.tensor(rep["losses"])
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-6), (got, want)
+    # each microbatch has its own loss: an index mix-up would show
+    assert len(set(round(float(v), 4) for v in want)) == 4

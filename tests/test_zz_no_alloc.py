@@ -65,3 +65,25 @@ def test_noalloc_colsum_rejects_what_does_not_fit():
     M_ok = (limit // Nn) * 128
     ok = dY[:M_ok]
     assert torch.equal(_colsum_noalloc(ok, torch.bfloat16), _colsum_ws(ok, torch.bfloat16))
+
+
+def test_noalloc_colsum_allocates_nothing_on_a_warm_call():
+    """What the entry point is for: after the first call on a device (which looks up the address of the
+    library's array), a call leaves the device's free memory and torch's allocator untouched."""
+    dY = torch.randn(2048, 1024, device="cuda").to(torch.bfloat16)
+    out = torch.empty(1024, dtype=torch.bfloat16, device="cuda")
+
+    def call():
+        N.check(N.lib().pp_colsum_bf16_noalloc(dY.data_ptr(), 2048, 1024, 1024, out.data_ptr(), N.PP_BF16,
+                                               N.current_stream()), "pp_colsum_bf16_noalloc")
+
+    call()                                   # warm: the per-device set-up happens here
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    held0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_allocated() == held0 and torch.cuda.memory_reserved() == reserved0
+    assert free1 == free0
