@@ -72,7 +72,10 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr_t;
 // compiler knows that they write LDS, cannot tell which part, and therefore makes every later LDS read
 // wait for ALL outstanding loads (s_waitcnt vmcnt(0) in front of the first fragment read of the next
 // tile): the loads of tile t + 2 would then finish before tile t + 1 is touched, and nothing would
-// overlap.  The kernels order loads and reads themselves, with explicit vmcnt waits and barriers.
+// overlap.  The kernels order loads and reads themselves, with explicit vmcnt waits and barriers: the
+// statements carry no "memory" clobber (it would pin every LDS read of a loop body to its side of them);
+// a stage is only ever refilled behind the barrier that follows its last read, and the compiler moves no
+// memory access across a barrier.
 struct LdsDmaRsrc {
     u32x4_t w;  // buffer resource words, wave-uniform (SGPRs)
 };
@@ -99,10 +102,11 @@ __device__ __forceinline__ void load_to_lds_b128(const LdsDmaRsrc& rsrc, uint16_
                  :
                  : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc.w),
                    "s"(__builtin_amdgcn_readfirstlane(soffset))
-                 : "memory", "m0");
+                 : "m0");
 #endif
 }
 
+// The builtin form, for kernels that were tuned around the compiler's own waits (attention).
 __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint16_t* lds_wave_base,
                                                  int voffset, int soffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
