@@ -371,7 +371,16 @@ typedef struct pp_attn_desc {
     int32_t causal;
     int32_t kv_group;      /* query heads per key / value head; 0 or 1: multi-head attention */
     int32_t kv_len;        /* 0: every key exists; L in 1..S: keys L..S-1 of each sequence are padding */
+    int32_t flags;         /* PP_ATTN_* bits */
 } pp_attn_desc;
+/* Backward: correct dq for the rounding of the forward's output.  The backward starts from
+ * delta = rowsum(dO * O) of the bf16 output; the sum of P * dP over the keys is the same number in exact
+ * arithmetic and the one under which the rows of dS sum to zero.  The dQ kernel always forms it (it is
+ * what `delta` holds afterwards and what the dK / dV kernel uses); with this bit it also corrects its own
+ * result, dQ -= (that sum - delta) * (P K), for one more MFMA per key block and tile.  For models whose
+ * attention is nearly uniform while their keys share a large common part (an encoder at initialisation),
+ * where the query gradients are small differences of large terms. */
+#define PP_ATTN_EXACT_DQ 1
 int pp_attn_fwd(const pp_attn_desc* desc, pp_stream stream);
 int pp_attn_bwd(const pp_attn_desc* desc, pp_stream stream);
 
@@ -441,7 +450,7 @@ enum pp_op_kind {
  *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
- *                 | j: causal kv_group kv_len
+ *                 | j: causal kv_group kv_len flags
  *   EMBED_FWD     p: ids wte wpe y extra_row pos_ids | i: n_tok seq C vocab n_pos  (pos_ids non-null:
  *                 pp_embed_fwd_at)
  *   POSITION_IDS  p: ids out | i: n_seq seq pad

@@ -31,6 +31,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
+ATTN_EXACT_DQ = 1
 ACT_RELU, ACT_GELU_ERF, ACT_GELU_TANH = 0, 1, 2
 
 PP_COPY_MAX_SEGS = 64
@@ -78,7 +79,8 @@ class AttnDesc(C.Structure):
                 ("delta", C.c_void_p),
                 ("B", C.c_int64), ("S", C.c_int64), ("H", C.c_int64), ("D", C.c_int64),
                 ("stride_b", C.c_int64), ("stride_s", C.c_int64),
-                ("scale", C.c_float), ("causal", C.c_int32), ("kv_group", C.c_int32), ("kv_len", C.c_int32)]
+                ("scale", C.c_float), ("causal", C.c_int32), ("kv_group", C.c_int32), ("kv_len", C.c_int32),
+                ("flags", C.c_int32)]
 
 
 class Op(C.Structure):
@@ -608,10 +610,11 @@ def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:
 def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, causal: bool,
               scale: Optional[float] = None, d_o: Optional[torch.Tensor] = None,
               dqkv: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
-              n_kv_heads: Optional[int] = None, kv_len: Optional[int] = None) -> AttnDesc:
+              n_kv_heads: Optional[int] = None, kv_len: Optional[int] = None, exact_dq: bool = False) -> AttnDesc:
     """qkv: [B, S, (H + 2 H_kv) * D] fused projection output (q | k | v along the last dim);
     ``n_kv_heads`` < H: grouped-query attention (H / n_kv_heads query heads per key / value head);
-    ``kv_len`` < S: rows kv_len .. S-1 of every sequence are (zero) padding that the forward masks."""
+    ``kv_len`` < S: rows kv_len .. S-1 of every sequence are (zero) padding that the forward masks;
+    ``exact_dq``: the backward corrects dq for the rounding of the forward's output (PP_ATTN_EXACT_DQ)."""
     require_cuda(qkv, o, lse, d_o, dqkv, delta)
     B, S, width = qkv.shape
     Hkv = H if n_kv_heads is None else n_kv_heads
@@ -631,6 +634,7 @@ def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, cau
     d.causal = int(causal)
     assert kv_len is None or 0 < kv_len <= S
     d.kv_len = 0 if kv_len is None else kv_len
+    d.flags = ATTN_EXACT_DQ if exact_dq else 0
     if d_o is not None:
         assert dqkv is not None and delta is not None
         assert dqkv.shape == qkv.shape and dqkv.stride() == qkv.stride() and d_o.is_contiguous()
@@ -646,9 +650,10 @@ def attn_fwd(qkv, o, lse, H, causal, scale=None, n_kv_heads=None, kv_len=None) -
     check(lib().pp_attn_fwd(C.byref(d), current_stream()), "pp_attn_fwd")
 
 
-def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None, n_kv_heads=None, kv_len=None) -> None:
+def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None, n_kv_heads=None, kv_len=None,
+             exact_dq=False) -> None:
     d = attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
-                  kv_len=kv_len)
+                  kv_len=kv_len, exact_dq=exact_dq)
     check(lib().pp_attn_bwd(C.byref(d), current_stream()), "pp_attn_bwd")
 
 

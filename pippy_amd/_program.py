@@ -481,13 +481,13 @@ def op_ln_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, ws) -> N.Op:
 
 
 def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_heads=None, kv_len=None,
-            scale=None) -> N.Op:
-    """``scale``: the factor on the scores (None: 1 / sqrt(head size))."""
+            scale=None, exact_dq=False) -> N.Op:
+    """``scale``: the factor on the scores (None: 1 / sqrt(head size)); ``exact_dq``: see ``N.attn_desc``."""
     if qkv.shape[1] % 64:
         raise RuntimeError(f"the attention kernels take sequence lengths that are multiples of 64, got "
                            f"{qkv.shape[1]} (stage_modules.lower_attention pads)")
     d = N.attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
-                    kv_len=kv_len)
+                    kv_len=kv_len, exact_dq=exact_dq)
     op = N.Op()
     op.kind = kind
     for k, v in enumerate((d.q, d.k, d.v, d.o, d.lse, d.d_o, d.dq, d.dk, d.dv, d.delta)):
@@ -497,6 +497,7 @@ def op_attn(kind, qkv, o, lse, H, causal, d_o=None, dqkv=None, delta=None, n_kv_
     op.j[0] = d.causal
     op.j[1] = d.kv_group
     op.j[2] = d.kv_len
+    op.j[3] = d.flags
     return op
 
 

@@ -64,13 +64,17 @@ __device__ __forceinline__ int swz_attn(int r) { return ((r ^ (r >> 3)) & 7) ^ (
 
 // Direct-to-LDS loader of 64-row blocks out of a [rows][stride] operand: DS tiles of 64 columns
 // (128 B per row and tile), tile s at lds + s * kTile.
-template <int DS>
+// ASM: the loads go out as inline assembly, which lets tiles stay in flight across LDS reads (the forward
+// and the dQ kernel); the dK / dV kernel keeps the builtin form: it spills a few registers, and the waits
+// of its scratch loads would cover the assembly loads anyway.
+template <int DS, bool ASM = true>
 struct AttnTileLoader {
-    __amdgpu_buffer_rsrc_t rsrc;
+    typename std::conditional<ASM, LdsDmaRsrc, __amdgpu_buffer_rsrc_t>::type rsrc;
     int voff[2];
     int row_bytes;
     __device__ __forceinline__ void init(const uint16_t* base, int64_t stride, int64_t rows, int wave, int lane) {
-        rsrc = make_rsrc(base, (uint64_t)rows * (uint64_t)stride * 2);
+        if constexpr (ASM) rsrc = make_lds_dma_rsrc(base, (uint64_t)rows * (uint64_t)stride * 2);
+        else rsrc = make_rsrc(base, (uint64_t)rows * (uint64_t)stride * 2);
         row_bytes = (int)(stride * 2);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -227,6 +231,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t)
         if (t < n_blocks) issue(t, t);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) settle(qf[ks]);
 
     f32x16_t oacc[DT];
 #pragma unroll
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     const uint16_t* kp = a.k + b * a.stride_b + hk * D;
     const uint16_t* vp = a.v + b * a.stride_b + hk * D;
     const int64_t ldo = a.H * D;
-    AttnTileLoader<DS> lq, ldo_;
+    AttnTileLoader<DS, false> lq, ldo_;
     lq.init(a.q + b * a.stride_b + h * D, a.stride_s, a.S, wave, lane);
     ldo_.init(a.d_o + b * a.S * ldo + h * D, ldo, a.S, wave, lane);
     // waves 0 and 2 fetch lse, waves 1 and 3 delta (the same values twice: every wave issues the
@@ -554,8 +560,8 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
 }
 
 // ---- backward: dQ (parallel over query blocks) ---------------------------------------------------
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+template <int D, bool CAUSAL, bool EXACT>
+__global__ __launch_bounds__(256, D == 64 ? 3 : (EXACT ? 1 : 2)) void attn_bwd_dq_kernel(const AttnArgs a) {
     static_assert(D == 64 || D == 128, "head dimension 64 or 128");
     constexpr int KS = D / 16, DT = D / 32, DS = D / 64, NS = attn_stages(D);
     constexpr int kOperand = DS * kTile;   // one staged 64-row block of K or V
@@ -592,7 +598,7 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
         qf[ks] = *reinterpret_cast<const bf16x8_t*>(qp + qi * a.stride_s + 16 * ks + 8 * lh);
         dof[ks] = *reinterpret_cast<const bf16x8_t*>(dop + qi * ldo + 16 * ks + 8 * lh);
     }
-    const float lse_q = a.lse[(b * a.H + h) * a.S + qi] * kLog2e;
+    float lse_q = a.lse[(b * a.H + h) * a.S + qi] * kLog2e;
     // delta = rowsum(dO * O) of this lane's query row: the lane pair (lh = 0, 1) holds the row of dO, so
     // the same pieces of O make the dot product; it is stored for the dK / dV kernel, which runs next
     float delta_q = 0.f;
@@ -609,11 +615,31 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
                        bf16lo(x.u.w) * bf16lo(y.u.w) + bf16hi(x.u.w) * bf16hi(y.u.w);
         }
         delta_q += __shfl_xor(delta_q, 32, 64);
-        if (half == 0 && lh == 0) a.delta[(b * a.H + h) * a.S + qi] = delta_q;
+    }
+    // The row sum above comes from the rounded output of the forward; the sum of P * dP over the keys, which
+    // this kernel forms anyway, is the same number in exact arithmetic and the one that is consistent with
+    // the dS = P (dP - delta) of both backward kernels (their rows then sum to zero).  It is only complete
+    // after the loop: it is what the dK / dV kernel gets, and with EXACT this kernel corrects its own
+    // result by the difference, dQ -= (D - delta) * (P K), at the cost of one more MFMA per block and tile
+    // (the error term is a multiple of the attention-weighted mean key, which dwarfs the true gradient of
+    // the queries where attention is nearly uniform and the keys share a large common part).
+    float d_consistent = 0.f;
+    f32x16_t pkacc[EXACT ? DT : 1];
+    if constexpr (EXACT) {
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) pkacc[t][e] = 0.f;
     }
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t)
         if (t < n_blocks) issue(t, t);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        settle(qf[ks]);
+        settle(dof[ks]);
+    }
+    settle(lse_q);
     const float c = a.scale * kLog2e;
 
     f32x16_t dqacc[DT];
@@ -660,6 +686,13 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
                     if (kt0 + 8 * (v >> 2) + 4 * lh + (v & 3) > qi) dsv[v] = 0.f;
             }
 #pragma unroll
+            for (int v = 0; v < 16; ++v) d_consistent = fmaf(dsv[v], dpacc[v], d_consistent);
+            bf16x8_t pb[EXACT ? 2 : 1];
+            if constexpr (EXACT) {
+                pb[0] = pack8(dsv);
+                pb[1] = pack8(dsv + 8);
+            }
+#pragma unroll
             for (int v = 0; v < 16; ++v) dsv[v] *= dpacc[v] - delta_q;
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
@@ -668,26 +701,41 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void attn_bwd_dq_kernel(const
                 for (int dt = 0; dt < DT; ++dt) {
                     const bf16x8_t ktf = read_col_frag(Ks + (dt / 2) * kTile, 32 * t + 16 * gp, 32 * (dt % 2), lane);
                     dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf, dsb, dqacc[dt], 0, 0, 0);
+                    if constexpr (EXACT)
+                        pkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf, pb[gp], pkacc[dt], 0, 0, 0);
                 }
             }
         }
       });
-    // add the partial sums of the two key halves: [grp][16 DT values][64 lanes] floats
+    // this lane's keys and its partner's (lane ^ 32) make the row's share of this wave
+    d_consistent += __shfl_xor(d_consistent, 32, 64);
+    // add the partial sums of the two key halves: [grp][(EXACT ? 32 : 16) DT + 1 values][64 lanes] floats
     wait_lds();
     __builtin_amdgcn_s_barrier();
-    float* xs = reinterpret_cast<float*>(lds) + grp * (16 * DT * 64) + lane;
+    constexpr int kMergeVals = (EXACT ? 32 : 16) * DT + 1;
+    float* xs = reinterpret_cast<float*>(lds) + grp * (kMergeVals * 64) + lane;
     if (half == 1) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) xs[(16 * dt + e) * 64] = dqacc[dt][e];
+            for (int e = 0; e < 16; ++e) {
+                xs[(16 * dt + e) * 64] = dqacc[dt][e];
+                if constexpr (EXACT) xs[(16 * DT + 16 * dt + e) * 64] = pkacc[dt][e];
+            }
+        xs[(kMergeVals - 1) * 64] = d_consistent;
     }
     __syncthreads();
     if (half != 0) return;
+    d_consistent += xs[(kMergeVals - 1) * 64];
+    if (lh == 0) a.delta[(b * a.H + h) * a.S + qi] = d_consistent;
+    const float r = d_consistent - delta_q;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) dqacc[dt][e] += xs[(16 * dt + e) * 64];
+        for (int e = 0; e < 16; ++e) {
+            dqacc[dt][e] += xs[(16 * dt + e) * 64];
+            if constexpr (EXACT) dqacc[dt][e] -= r * (pkacc[dt][e] + xs[(16 * DT + 16 * dt + e) * 64]);
+        }
     uint16_t* dqp = a.dq + b * a.stride_b + h * D + qi * a.stride_s;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -740,9 +788,9 @@ static AttnArgs to_args(const pp_attn_desc* d) {
 }
 
 // Dynamic LDS of the three kernels: stages, or the merge buffers of the epilogue if those are larger.
-static size_t attn_lds_bytes(int D, bool dkv) {
+static size_t attn_lds_bytes(int D, bool dkv, bool exact_dq = false) {
     const size_t stage = (size_t)2 * (D / 64) * kTile * 2 + (dkv ? 512 : 0);
-    const size_t merge = (size_t)2 * (16 * (D / 32) + 2) * 64 * 4;
+    const size_t merge = (size_t)2 * ((exact_dq ? 32 : 16) * (D / 32) + 2) * 64 * 4;
     const size_t stages = (size_t)attn_stages(D) * stage;
     return stages > merge ? stages : merge;
 }
@@ -783,16 +831,19 @@ static int attn_fwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipSt
 template <int D>
 static int attn_bwd_d(const pp_attn_desc* d, const AttnArgs& a, dim3 grid, hipStream_t st) {
     // the dQ kernel goes first: it also computes delta = rowsum(dO * O), which the dK / dV kernel reads
-    const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false);
+    const bool exact = (d->flags & PP_ATTN_EXACT_DQ) != 0;
+    const size_t lds_kv = attn_lds_bytes(D, true), lds_q = attn_lds_bytes(D, false, exact);
     // one work-group per 64 keys of a key / value head
     const dim3 grid_kv((uint32_t)(((d->S / 64) * (d->H / a.G) * d->B + 7) / 8 * 8));
     int rc;
     if (d->causal) {
-        rc = attn_launch<attn_bwd_dq_kernel<D, true>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
+        rc = exact ? attn_launch<attn_bwd_dq_kernel<D, true, true>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a)
+                   : attn_launch<attn_bwd_dq_kernel<D, true, false>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
         if (rc) return rc;
         return attn_launch<attn_bwd_dkv_kernel<D, true>>("attn_bwd_dkv_kernel", grid_kv, 256, lds_kv, st, a);
     }
-    rc = attn_launch<attn_bwd_dq_kernel<D, false>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
+    rc = exact ? attn_launch<attn_bwd_dq_kernel<D, false, true>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a)
+               : attn_launch<attn_bwd_dq_kernel<D, false, false>>("attn_bwd_dq_kernel", grid, 256, lds_q, st, a);
     if (rc) return rc;
     return attn_launch<attn_bwd_dkv_kernel<D, false>>("attn_bwd_dkv_kernel", grid_kv, 256, lds_kv, st, a);
 }

@@ -449,8 +449,8 @@ struct GemmGroupArgs {
     int n;
 };
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK>
-__global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const GemmGroupArgs ga) {
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT = BK, int W = 4>
+__global__ __launch_bounds__(W * 64) void gemm_bf16_group_kernel(const GemmGroupArgs ga) {
     uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
     if (bid >= ga.tile_start[ga.n]) return;
     int i = 0;
@@ -459,7 +459,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_group_kernel(const Gem
     const GemmArgs& g = ga.p[i];
     uint32_t tile_m, tile_n;
     grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT>(g, tile_m, tile_n);
+    gemm_tile_dma<BM, BN, AT, BT, NS, EPI, CF32, KT, 0, W>(g, tile_m, tile_n);
 }
 
 

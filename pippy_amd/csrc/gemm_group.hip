@@ -17,10 +17,10 @@
 
 namespace pp {
 
-template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT>
+template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT, int W = 4>
 static int launch_group(GemmGroupArgs& ga, hipStream_t st) {
     constexpr size_t lds = (size_t)NS * (BM + BN) * KT * sizeof(uint16_t);
-    static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>, lds);
+    static const int attr_rc = reserve_lds(&gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT, W>, lds);
     if (attr_rc) return attr_rc;
     uint64_t total = 0;
     for (int i = 0; i < ga.n; ++i) {
@@ -33,7 +33,7 @@ static int launch_group(GemmGroupArgs& ga, hipStream_t st) {
     ga.tile_start[ga.n] = (uint32_t)total;
     if (total == 0) return PP_OK;
     const uint32_t grid = ((uint32_t)total + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT>), dim3(grid), dim3(kGemmThreads),
+    hipLaunchKernelGGL((gemm_bf16_group_kernel<BM, BN, AT, BT, NS, EPI, CF32, KT, W>), dim3(grid), dim3(W * 64),
                        lds, st, ga);
     return check_launch("gemm_bf16_group_kernel");
 }
@@ -48,10 +48,15 @@ static uint64_t tiles_128(const GemmGroupArgs& ga) {
 // 128 x 128 tiles: with at most one tile per CU a work-group has the CU to itself and takes 3 LDS
 // stages; with more tiles 2 stages leave room for two resident work-groups.  (Wider tiles were
 // measured on groups of 2 to 4 transformer-sized problems per launch, 256 x 128, 128 x 256 and
-// 256 x 256 with 2 to 4 stages of 32 or 64 k: none ran a forward-shaped group faster than 128 x 128,
-// and the weight-gradient groups gained 2 % at best.)
+// 256 x 256 with 2 to 4 stages of 32 or 64 k: none ran a forward-shaped group faster than 128 x 128.)
 template <bool AT, bool BT, int EPI, bool CF32>
 static int launch_auto(GemmGroupArgs& ga, hipStream_t st) {
+    if constexpr (AT && BT && CF32) {
+        // the weight gradients of a stage pass: more 128 x 128 tiles than two per CU.  256 x 128 tiles on
+        // 8 waves load a quarter less per flop and, with the CU to themselves, keep 3 stages (two tiles
+        // in flight): 880 against 800 TFLOP/s on the 12 problems of three GPT-2-small layers
+        if (tiles_128(ga) > 2 * kComputeUnits) return launch_group<256, 128, AT, BT, 3, EPI, CF32, 64, 8>(ga, st);
+    }
     return tiles_128(ga) <= kComputeUnits ? launch_group<128, 128, AT, BT, 3, EPI, CF32, 64>(ga, st)
                                           : launch_group<128, 128, AT, BT, 2, EPI, CF32, 64>(ga, st);
 }

@@ -103,7 +103,7 @@ static int run_one(const pp_op& op, pp_stream st) {
             d.dq = op.p[6]; d.dk = op.p[7]; d.dv = op.p[8]; d.delta = static_cast<float*>(op.p[9]);
             d.B = op.i[0]; d.S = op.i[1]; d.H = op.i[2]; d.D = op.i[3];
             d.stride_b = op.i[4]; d.stride_s = op.i[5];
-            d.scale = op.f[0]; d.causal = op.j[0]; d.kv_group = op.j[1]; d.kv_len = op.j[2];
+            d.scale = op.f[0]; d.causal = op.j[0]; d.kv_group = op.j[1]; d.kv_len = op.j[2]; d.flags = op.j[3];
             return op.kind == PP_OP_ATTN_FWD ? pp_attn_fwd(&d, st) : pp_attn_bwd(&d, st);
         }
         case PP_OP_POSITION_IDS:

@@ -149,6 +149,12 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
     Hkv = H if n_kv_heads is None else n_kv_heads
     D = W // (H + 2 * Hkv)
     Cc = H * D
+    # Without a causal mask every query sees every key: at initialisation attention is then nearly uniform
+    # over the whole sequence and the query gradients are small differences of large terms, which the
+    # rounding of the forward's output would swamp (the dQ kernel corrects for it at one more MFMA per
+    # block).  Under a causal mask the early queries see few keys and the effect stays below the rounding
+    # of the operands themselves.
+    exact_dq = not causal
     att = b.act("att", (T, Cc))
     if S % 64 == 0:
         lse = b.act("lse", (Bn, H, S), torch.float32)
@@ -160,7 +166,7 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
             delta = b.scratch("attn_delta", (Bn, H, S), torch.float32)
             b.i(P.op_attn(N.OP_ATTN_BWD, qkv.view(Bn, S, W), att.view(Bn, S, Cc), lse, H, causal,
                           d_o=d_att.view(Bn, S, Cc), dqkv=dqkv.view(Bn, S, W), delta=delta, n_kv_heads=Hkv,
-                          scale=scale))
+                          scale=scale, exact_dq=exact_dq))
             return dqkv
 
         return att, backward
@@ -184,7 +190,7 @@ def lower_attention(b: "P.Builder", qkv: torch.Tensor, Bn: int, S: int, H: int, 
             b.sp.zeroed_once.add(d_att_p.data_ptr())
         b.i(P.op_copy_rows(d_att, d_att_p, Bn, S * Cc * es, S * Cc * es, Sp * Cc * es))
         b.i(P.op_attn(N.OP_ATTN_BWD, qkv_p, att_p, lse, H, causal, d_o=d_att_p, dqkv=dqkv_p, delta=delta,
-                      n_kv_heads=Hkv, kv_len=S, scale=scale))
+                      n_kv_heads=Hkv, kv_len=S, scale=scale, exact_dq=exact_dq))
         b.i(P.op_copy_rows(dqkv_p, dqkv, Bn, S * W * es, Sp * W * es, S * W * es))
         return dqkv
 
