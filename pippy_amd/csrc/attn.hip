@@ -64,10 +64,11 @@ __device__ __forceinline__ int swz_attn(int r) { return ((r ^ (r >> 3)) & 7) ^ (
 
 // Direct-to-LDS loader of 64-row blocks out of a [rows][stride] operand: DS tiles of 64 columns
 // (128 B per row and tile), tile s at lds + s * kTile.
-// ASM: the loads go out as inline assembly, which lets tiles stay in flight across LDS reads (the forward
-// and the dQ kernel); the dK / dV kernel keeps the builtin form: it spills a few registers, and the waits
-// of its scratch loads would cover the assembly loads anyway.
-template <int DS, bool ASM = true>
+// ASM: the loads go out as inline assembly (see tile.h), which lets tiles stay in flight across LDS reads.
+// Measured on the three kernels it changed nothing (forward 1.92 against 1.95 ms, backward 5.12 against
+// 5.29 ms per GPT-2-small step, within the scatter between machines): a work-group's chain of dependent
+// block steps, not its loads, sets the pace.  The kernels stay on the builtin form.
+template <int DS, bool ASM = false>
 struct AttnTileLoader {
     typename std::conditional<ASM, LdsDmaRsrc, __amdgpu_buffer_rsrc_t>::type rsrc;
     int voff[2];
@@ -231,8 +232,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 2 : (D == 64 ? 3 : 2)) voi
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t)
         if (t < n_blocks) issue(t, t);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) settle(qf[ks]);
 
     f32x16_t oacc[DT];
 #pragma unroll
@@ -634,12 +633,6 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : (EXACT ? 1 : 2)) void attn_bwd_d
 #pragma unroll
     for (int t = 0; t < NS - 1; ++t)
         if (t < n_blocks) issue(t, t);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        settle(qf[ks]);
-        settle(dof[ks]);
-    }
-    settle(lse_q);
     const float c = a.scale * kLog2e;
 
     f32x16_t dqacc[DT];

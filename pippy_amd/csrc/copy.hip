@@ -155,77 +155,7 @@ __global__ __launch_bounds__(kThreads) void copy_rows_unaligned_kernel(const Cop
     }
 }
 
-// The same rows when every source row starts on a 16-byte boundary (the padded logits of a stage: rows of
-// 100 608 bytes merged into rows of 100 514): both sides move as aligned 16-byte vectors.  Destination
-// vector i of a row holds source bytes [head + 16 i, head + 16 i + 16), which straddle the aligned source
-// vectors i and i + 1; a lane loads both (the second is its neighbour's first: the same lines) and shifts
-// the pair by `head` bytes in registers.  The vector that holds a row's last bytes may be read past the
-// row's end, never past the end of its 16-byte unit, so never into another page.
-template <int Q>
-__device__ __forceinline__ copy_u32x4_t shift_pair(const copy_u32x4_t lo, const copy_u32x4_t hi, const int b) {
-    const uint32_t d[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    copy_u32x4_t r;
-    // alignbyte(h, l, b) = low 32 bits of ((h:l) >> 8 b); b < 4
-    r.x = __builtin_amdgcn_alignbyte(d[Q + 1], d[Q], b);
-    r.y = __builtin_amdgcn_alignbyte(d[Q + 2], d[Q + 1], b);
-    r.z = __builtin_amdgcn_alignbyte(d[Q + 3], d[Q + 2], b);
-    r.w = __builtin_amdgcn_alignbyte(d[Q + 4], d[Q + 3], b);
-    return r;
-}
-
 template <int A>
-__global__ __launch_bounds__(kThreads) void copy_rows_realign_kernel(const CopyTable t) {
-    typedef typename VecT<A>::type elem;
-    uint32_t b = blockIdx.x;
-    int s = 0;
-    while (s + 1 < t.n && b >= t.block_start[s + 1]) ++s;
-    b -= t.block_start[s];
-    const DevSeg& g = t.seg[s];
-    const int tid = threadIdx.x;
-    const int64_t row = b / g.col_blocks;
-    const uint32_t cblk = b % g.col_blocks;
-    const char* sp = g.src + row * g.src_stride;  // 16-byte aligned
-    char* dp = g.dst + row * g.dst_stride;
-    int64_t head = (16 - (reinterpret_cast<uintptr_t>(dp) & 15)) & 15;  // wave-uniform: one row per block
-    if (head > g.row_bytes) head = g.row_bytes;
-    const int64_t nv = (g.row_bytes - head) >> 4;
-    const int64_t v0 = (int64_t)cblk * (kThreads * kUnroll);
-    const int q = (int)(head >> 2), bsh = (int)(head & 3);
-    copy_u32x4_t lo[kUnroll], hi[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const int64_t vi = v0 + u * kThreads + tid;
-        if (vi < nv) {
-            lo[u] = __builtin_nontemporal_load(reinterpret_cast<const copy_u32x4_t*>(sp + vi * 16));
-            // (head == 0: the second vector is not needed and may lie past the row)
-            hi[u] = head ? *reinterpret_cast<const copy_u32x4_t*>(sp + vi * 16 + 16) : lo[u];
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const int64_t vi = v0 + u * kThreads + tid;
-        if (vi < nv) {
-            copy_u32x4_t w;
-            switch (q) {
-                case 0: w = shift_pair<0>(lo[u], hi[u], bsh); break;
-                case 1: w = shift_pair<1>(lo[u], hi[u], bsh); break;
-                case 2: w = shift_pair<2>(lo[u], hi[u], bsh); break;
-                default: w = shift_pair<3>(lo[u], hi[u], bsh); break;
-            }
-            __builtin_nontemporal_store(w, reinterpret_cast<copy_u32x4_t*>(dp + head + vi * 16));
-        }
-    }
-    if (cblk == 0) {
-        for (int64_t i = (int64_t)tid * A; i < head; i += kThreads * A)
-            *reinterpret_cast<elem*>(dp + i) = *reinterpret_cast<const elem*>(sp + i);
-    }
-    if (cblk == g.col_blocks - 1) {
-        for (int64_t i = head + nv * 16 + (int64_t)tid * A; i < g.row_bytes; i += kThreads * A)
-            *reinterpret_cast<elem*>(dp + i) = *reinterpret_cast<const elem*>(sp + i);
-    }
-}
-
-template <int A, bool REALIGN>
 static int launch_unaligned(const pp_copy_seg* segs, int n, hipStream_t stream) {
     CopyTable t;
     uint64_t blocks = 0;
@@ -253,10 +183,7 @@ static int launch_unaligned(const pp_copy_seg* segs, int n, hipStream_t stream) 
     if (m == 0) return PP_OK;
     t.block_start[m] = (uint32_t)blocks;
     t.n = m;
-    if (REALIGN)
-        hipLaunchKernelGGL(copy_rows_realign_kernel<A>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, t);
-    else
-        hipLaunchKernelGGL(copy_rows_unaligned_kernel<A>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, t);
+    hipLaunchKernelGGL(copy_rows_unaligned_kernel<A>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, t);
     return check_launch("copy_rows_unaligned_kernel");
 }
 
@@ -334,22 +261,11 @@ static int copy_rows_impl(const pp_copy_seg* segs, int n_segs, hipStream_t strea
         for (int i = 0; i < n; ++i)
             if (segs[i0 + i].n_rows > 0 && segs[i0 + i].row_bytes < 2048) long_rows = false;
         if (vec < 16 && long_rows) {
-            // every source row on a 16-byte boundary: aligned loads, realigned in registers
-            bool src16 = true;
-            for (int i = 0; i < n; ++i) {
-                const pp_copy_seg& sg = segs[i0 + i];
-                if (sg.n_rows == 0 || sg.row_bytes == 0) continue;
-                if ((reinterpret_cast<uintptr_t>(sg.src) & 15) || (sg.n_rows > 1 && (sg.src_stride & 15))) src16 = false;
-            }
             switch (vec) {
-                case 8: rc = src16 ? launch_unaligned<8, true>(segs + i0, n, stream)
-                                   : launch_unaligned<8, false>(segs + i0, n, stream); break;
-                case 4: rc = src16 ? launch_unaligned<4, true>(segs + i0, n, stream)
-                                   : launch_unaligned<4, false>(segs + i0, n, stream); break;
-                case 2: rc = src16 ? launch_unaligned<2, true>(segs + i0, n, stream)
-                                   : launch_unaligned<2, false>(segs + i0, n, stream); break;
-                default: rc = src16 ? launch_unaligned<1, true>(segs + i0, n, stream)
-                                    : launch_unaligned<1, false>(segs + i0, n, stream); break;
+                case 8: rc = launch_unaligned<8>(segs + i0, n, stream); break;
+                case 4: rc = launch_unaligned<4>(segs + i0, n, stream); break;
+                case 2: rc = launch_unaligned<2>(segs + i0, n, stream); break;
+                default: rc = launch_unaligned<1>(segs + i0, n, stream); break;
             }
             if (rc != PP_OK) return rc;
             continue;

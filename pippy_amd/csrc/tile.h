@@ -109,34 +109,7 @@ __device__ __forceinline__ void load_to_lds_b128(const LdsDmaRsrc& rsrc, uint16_
 #endif
 }
 
-// The same with 4 bytes per lane: 64 consecutive dwords to `lds_wave_base` + 4 * lane.
-__device__ __forceinline__ void load_to_lds_b32(const LdsDmaRsrc& rsrc, void* lds_wave_base, int voffset,
-                                                int soffset) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_void_ptr_t)lds_wave_base;
-    asm volatile("s_mov_b32 m0, %0\n\t"
-                 "s_nop 3\n\t"
-                 "buffer_load_dword %1, %2, %3 offen lds"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voffset), "s"(rsrc.w),
-                   "s"(__builtin_amdgcn_readfirstlane(soffset))
-                 : "m0");
-#endif
-}
-
-// A value that an ordinary global load fetched into registers before the first of these loads was
-// issued: passing it through here makes the compiler place its wait for that load at this point (once,
-// in the prologue).  Left to itself it puts the wait at the value's first use, inside the main loop, as
-// "vmcnt(0)" - computed without the loads above, which it does not see, but executed with them: every
-// iteration would wait for every tile in flight.
-__device__ __forceinline__ void settle(bf16x8_t& f) {
-    u32x4_t t = __builtin_bit_cast(u32x4_t, f);
-    asm volatile("" : "+v"(t));
-    f = __builtin_bit_cast(bf16x8_t, t);
-}
-__device__ __forceinline__ void settle(float& f) { asm volatile("" : "+v"(f)); }
-
-// The builtin form.
+// The builtin form, for kernels that were tuned around the compiler's own waits (attention).
 __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint16_t* lds_wave_base,
                                                  int voffset, int soffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
