@@ -446,6 +446,9 @@ def main():
     ap.add_argument("--serial-stages", action="store_true",
                     help="run all virtual stages on one stream instead of two")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--batch-weight-grads", default="auto", choices=["auto", "on", "off"],
+                    help="one batched weight-gradient pass per stage and step (auto: the schedule's own choice: "
+                         "zero-bubble schedules and stages with expert weights)")
     ap.add_argument("--gemm-shapes", action="store_true",
                     help="instead of a step: time the stage GEMM alone on the shapes of the workloads (HIP "
                          "events, cold operands) and torch.matmul (the vendor library) on the same operands beside "
@@ -504,6 +507,8 @@ def main():
     tokens = ids.numel() if default_workload else args.tokens
     training = True if default_workload else args.training
     sched.concurrent_stages = not args.serial_stages
+    if args.batch_weight_grads != "auto":
+        sched.batch_weight_grads = args.batch_weight_grads == "on"
 
     def step():
         losses = []
@@ -559,6 +564,11 @@ def main():
         ms, work, cnt = N.profile_read(N.OP_GEMM_BF16)
         sms_, swork, scnt = N.profile_read(N.OP_GEMM_SEG)   # expert GEMMs of a mixture-of-experts layer
         ms, work, cnt = ms + sms_, work + swork, cnt + scnt
+        bcnt = 0
+        for kind in (N.OP_GEMM_KSEG, N.OP_GEMM_SEG_KSEG):   # weight gradients of all microbatches in one launch
+            kms, kwork, kcnt = N.profile_read(kind)
+            ms, work, cnt, bcnt = ms + kms, work + kwork, cnt + kcnt, bcnt + kcnt
+            scnt += kcnt if kind == N.OP_GEMM_SEG_KSEG else 0
         gcnt = 0
         for kind in (N.OP_GEMM_SWIGLU, N.OP_GEMM_DSWIGLU):   # feed-forward GEMMs with SwiGLU in the epilogue
             kms, kwork, kcnt = N.profile_read(kind)
@@ -570,7 +580,8 @@ def main():
                               "traffic_source": gemm_traffic()[1] if default_workload else None,
                               "kernel": "gemm_bf16_dma_kernel + gemm_bf16_dma8_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
                                         + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else "")
-                                        + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else ""),
+                                        + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else "")
+                                        + (" + gemm_bf16_group_kseg_kernel / gemm_bf16_seg_k_multi_kernel" if bcnt else ""),
                               "launches_per_step": cnt // n_prof,
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),
                               "gemm_ms_per_step": round(ms / n_prof, 3)}

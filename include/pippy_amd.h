@@ -200,6 +200,19 @@ enum pp_gemm_seg_mode { PP_SEG_ROWS = 0, PP_SEG_K = 1 };
 int pp_gemm_bf16_segmented(const pp_gemm_desc* desc, const int32_t* seg_start, const void* const* seg_ptr,
                            int n_seg, int mode, pp_stream stream);
 
+/* PP_SEG_K over several microbatches in one launch (the expert weight gradients of a mixture-of-experts
+ * layer for all microbatches of a step):  for every segment e,
+ *   C_e = (beta ? C_e : 0) + g_{e,0} + ... + g_{e,n_mb-1},   g_{e,m} = A_m[r0:r1, :]^T * B_m[r0:r1, :],
+ *   r0 = seg_start_of[m][e], r1 = seg_start_of[m][e + 1]
+ * added one term at a time in ascending m in fp32 (g rounded to bf16 first under PP_EPI_ACCUM_ROUNDED): bit
+ * for bit what one accumulating PP_SEG_K launch per microbatch, in ascending order, leaves in C_e.  a_of,
+ * b_of, seg_start_of ([n_mb]) and seg_ptr ([n_seg]) are DEVICE arrays of device pointers; desc gives M, N,
+ * lda, ldb, ldc, epilogue (ACCUM_F32 / ACCUM_ROUNDED) and beta, its A, B, C and K are ignored.  The
+ * accumulators C_e, which outweigh a microbatch's operands, move once instead of n_mb times. */
+int pp_gemm_bf16_segmented_kseg(const pp_gemm_desc* desc, const void* const* a_of, const void* const* b_of,
+                                const int32_t* const* seg_start_of, const void* const* seg_ptr, int n_seg,
+                                int n_mb, pp_stream stream);
+
 /* fp32 GEMM with the same descriptor (A, B, C, bias, aux fp32; config 1 of the baseline, the
  * README MLP).  Only a_trans / b_trans, NONE, BIAS, BIAS_RELU, DRELU and ACCUM_F32 epilogues. */
 int pp_gemm_f32(const pp_gemm_desc* desc, pp_stream stream);
@@ -438,7 +451,7 @@ enum pp_op_kind {
     PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
     PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
     PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27, PP_OP_POSITION_IDS = 28,
-    PP_OP_GEMM_KSEG = 29
+    PP_OP_GEMM_KSEG = 29, PP_OP_GEMM_SEG_KSEG = 30
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -474,6 +487,8 @@ enum pp_op_kind {
  *   GEMM_KSEG     as GEMM_BF16 with p[0], p[1]: device arrays of the segments' A and B pointers
  *                 | i[7]: n_seg; consecutive GEMM_KSEG ops with the same n_seg go out as ONE
  *                 pp_gemm_bf16_grouped_kseg call (they must not depend on each other)
+ *   GEMM_SEG_KSEG as GEMM_SEG in k mode with p[0], p[1]: device arrays of the microbatches' A and B, p[6]:
+ *                 device array of their seg_start arrays | i[7]: n_seg, i[8]: n_mb
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped

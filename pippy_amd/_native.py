@@ -27,7 +27,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
  OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU, OP_POSITION_IDS,
- OP_GEMM_KSEG) = range(1, 30)
+ OP_GEMM_KSEG, OP_GEMM_SEG_KSEG) = range(1, 31)
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
@@ -40,7 +40,7 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_bf16_grouped_kseg", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_bf16_grouped_kseg", "pp_gemm_bf16_segmented_kseg", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
@@ -121,6 +121,7 @@ def lib() -> C.CDLL:
         "pp_gemm_bf16_splitk": [C.POINTER(GemmDesc), vp, i64, vp],
         "pp_gemm_bf16_grouped": [C.POINTER(GemmDesc), i32, vp],
         "pp_gemm_bf16_grouped_kseg": [C.POINTER(GemmDesc), i32, i32, vp],
+        "pp_gemm_bf16_segmented_kseg": [C.POINTER(GemmDesc), vp, vp, vp, vp, i32, i32, vp],
         "pp_colsum_bf16": [vp, i64, i64, i64, vp, i32, vp, vp],
         "pp_colsum_bf16_noalloc": [vp, i64, i64, i64, vp, i32, vp],
         "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],

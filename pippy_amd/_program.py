@@ -654,6 +654,7 @@ class MicrobatchProgram:
         self.init_toggle_accum: List[int] = []  # W ops whose init flag follows the stage state
         self.init_toggle_beta: List[int] = []   # W GEMMs that accumulate in their epilogue
         self.loss_ops: Dict[int, Tuple[OpList, torch.Tensor, torch.Tensor]] = {}
+        self.w_tags: List[Optional[str]] = []   # per W op: how it follows the accumulation state
 
 
 class Builder:
@@ -818,6 +819,7 @@ class StageProgram:
         self._shared: Dict[str, torch.Tensor] = {}
         self.zeroed_once = set()   # addresses of shared buffers whose padding a block cleared when it was built
         self.mbs: Dict[int, MicrobatchProgram] = {}
+        self._batched_w: Dict[Tuple[int, ...], "BatchedW"] = {}
         self.acc_initialized = False  # False: the next W pass overwrites the accumulators
         # True once ``materialize_grads`` has set ``param.grad`` from the accumulators: a ``.grad`` that
         # is None afterwards was cleared by the user's optimizer
@@ -884,18 +886,29 @@ class StageProgram:
                        "fill": prog.init_toggle_fill}
             for op, tag in b._w_gemm + b._w_reduce + b._w_other:
                 k = prog.W.append(op)
+                prog.w_tags.append(tag)
                 if tag is not None:
                     toggles[tag].append(k)
             # fold this microbatch's staged parameter gradients into the fp32 accumulators
             # (those that no GEMM epilogue has added already)
             for lo, hi in self.arena.staged_ranges(self.epilogue_accumulated):
                 k = prog.W.append(op_accum(self.arena.acc[lo:hi], self.arena.staging[lo:hi], init=False))
+                prog.w_tags.append("accum")
                 prog.init_toggle_accum.append(k)
         prog.F.freeze()
         prog.I.freeze()
         prog.W.freeze()
         self.mbs[mb] = prog
         return prog
+
+    def batched_w(self, mbs: Tuple[int, ...]) -> "BatchedW":
+        """The weight-gradient passes of the microbatches ``mbs`` (ascending) as ONE launch list in which
+        every weight-gradient GEMM runs once over all of them (see ``BatchedW``)."""
+        key = tuple(mbs)
+        got = self._batched_w.get(key)
+        if got is None or any(self.mbs[m] is not p for m, p in zip(key, got.progs)):
+            got = self._batched_w[key] = BatchedW(self, key)
+        return got
 
     def set_accumulate_mode(self, prog: MicrobatchProgram, init: bool) -> None:
         """Patches the W list for the first (init) or a later microbatch of an accumulation."""
@@ -908,6 +921,125 @@ class StageProgram:
                 prog.W[k].flags &= ~OP_SKIP
             else:
                 prog.W[k].flags |= OP_SKIP
+
+
+class BatchedW:
+    """The weight-gradient passes of several microbatches of a stage as one launch list.
+
+    The reference accumulates parameter gradients microbatch by microbatch (one autograd pass each,
+    ``pippy/_backward.py:67-69``, in backward-microbatch order, ``pippy/PipelineSchedule.py:327,401-438``).
+    With every microbatch's operands still resident, a weight-gradient GEMM can instead run ONCE over all of
+    them: a tile walks the microbatches in ascending order, rounds each microbatch's product as the
+    single-microbatch kernel would, and adds it to a running fp32 sum in registers - the same additions in
+    the same order, so the accumulators end up bit-identical, but they are read and written once instead of
+    once per microbatch (``pp_gemm_bf16_grouped_kseg``; ``pp_gemm_bf16_segmented_kseg`` for the expert
+    weights of a mixture-of-experts layer, whose accumulators outweigh a microbatch's operands by far).
+    Everything else of the passes (column reductions, embedding gradients, the accumulate op over the small
+    tensors) follows per microbatch, in order."""
+
+    def __init__(self, sp: "StageProgram", mbs: Tuple[int, ...]):
+        self.progs = [sp.mbs[m] for m in mbs]
+        first = self.progs[0]
+        n_ops = first.W.n if first.W._arr is not None else len(first.W.ops)
+        for p in self.progs:
+            assert (p.W.n if p.W._arr is not None else len(p.W.ops)) == n_ops and p.w_tags == first.w_tags
+        dev = sp.device
+        self.list = OpList()
+        self.beta_ops: List[int] = []                     # batched GEMMs: beta follows the accumulation state
+        self.rest: List[Tuple[int, int, str]] = []        # (index, position of its microbatch, tag) of the others
+        batched = set()
+        dense, seg = [], []
+        for k in range(n_ops):
+            op = first.W[k]
+            accumulating = op.j[2] in (N.EPI_ACCUM_F32, N.EPI_ACCUM_ROUNDED) and op.j[3] == N.PP_F32
+            if op.kind == N.OP_GEMM_BF16 and op.j[0] and op.j[1] and accumulating and first.w_tags[k] == "beta" \
+                    and not op.p[8]:
+                dense.append(k)
+            elif op.kind == N.OP_GEMM_SEG and op.j[5] == N.SEG_K and accumulating and first.w_tags[k] == "beta":
+                seg.append(k)
+        n_mb = len(self.progs)
+        # where the copies of this list hold a pointer that a forward pass re-points at the stage's current
+        # input (a first stage reads the caller's tensors): (position of the microbatch, op, pointer slot)
+        patched = [(pos, k, q) for pos, p in enumerate(self.progs) for (lst, k, q) in p.input_patches if lst is p.W]
+        self._tables: Dict[int, Tuple[torch.Tensor, List[int]]] = {}   # op -> (device table, its host copy)
+        self._copy_of: Dict[Tuple[int, int], int] = {}                 # (position, op) -> index in this list
+        for k in dense:
+            ops = [p.W[k] for p in self.progs]
+            assert all(o.p[2] == ops[0].p[2] and tuple(o.i[:6]) == tuple(ops[0].i[:6]) for o in ops)
+            host = [o.p[0] for o in ops] + [o.p[1] for o in ops]
+            table = torch.tensor(host, dtype=torch.int64, device=dev)
+            self._tables[k] = (table, host)
+            op = N.Op()
+            C.memmove(C.byref(op), C.byref(ops[0]), C.sizeof(N.Op))
+            op.kind = N.OP_GEMM_KSEG
+            op.flags = 0
+            op.p[0], op.p[1] = table.data_ptr(), table.data_ptr() + 8 * n_mb
+            op.i[7] = n_mb
+            self.beta_ops.append(self.list.append(op))
+            batched.add(k)
+        for k in seg:
+            ops = [p.W[k] for p in self.progs]
+            assert all(o.p[7] == ops[0].p[7] and tuple(o.i[:2]) == tuple(ops[0].i[:2]) and
+                       tuple(o.i[3:6]) == tuple(ops[0].i[3:6]) and o.i[7] == ops[0].i[7] for o in ops)
+            host = [o.p[0] for o in ops] + [o.p[1] for o in ops] + [o.p[6] for o in ops]
+            table = torch.tensor(host, dtype=torch.int64, device=dev)
+            self._tables[k] = (table, host)
+            op = N.Op()
+            C.memmove(C.byref(op), C.byref(ops[0]), C.sizeof(N.Op))
+            op.kind = N.OP_GEMM_SEG_KSEG
+            op.flags = 0
+            op.p[0], op.p[1] = table.data_ptr(), table.data_ptr() + 8 * n_mb
+            op.p[6] = table.data_ptr() + 16 * n_mb
+            op.i[8] = n_mb
+            self.beta_ops.append(self.list.append(op))
+            batched.add(k)
+        for pos, p in enumerate(self.progs):
+            for k in range(n_ops):
+                if k in batched:
+                    continue
+                op = N.Op()
+                C.memmove(C.byref(op), C.byref(p.W[k]), C.sizeof(N.Op))
+                idx = self.list.append(op)
+                self._copy_of[(pos, k)] = idx
+                if p.w_tags[k] is not None:
+                    self.rest.append((idx, pos, p.w_tags[k]))
+        self.list.freeze()
+        self.n_batched = len(batched)
+        self._patched = patched
+        self._table_slot = {0: 0, 1: 1, 6: 2}     # pointer slot of an op -> which third of its table
+
+    def _follow_input_patches(self) -> None:
+        """Re-points the copies at what the per-microbatch lists point at now."""
+        n_mb = len(self.progs)
+        for pos, k, q in self._patched:
+            ptr = self.progs[pos].W[k].p[q]
+            if k in self._tables:
+                table, host = self._tables[k]
+                at = self._table_slot[q] * n_mb + pos
+                if host[at] != ptr:
+                    host[at] = ptr
+                    table[at] = ptr
+            else:
+                self.list[self._copy_of[(pos, k)]].p[q] = ptr
+
+    def run(self, init: bool) -> None:
+        """``init``: the accumulation starts with this batch (the accumulators are overwritten)."""
+        lst = self.list
+        self._follow_input_patches()
+        for k in self.beta_ops:
+            lst[k].j[4] = 0 if init else 1
+        for k, pos, tag in self.rest:
+            first = init and pos == 0
+            if tag == "accum":
+                lst[k].j[0] = int(first)
+            elif tag == "beta":
+                lst[k].j[4] = 0 if first else 1
+            elif tag == "fill":
+                if first:
+                    lst[k].flags &= ~OP_SKIP
+                else:
+                    lst[k].flags |= OP_SKIP
+        lst.run()
 
 
 def _like_view(padded_grad: torch.Tensor, out_view: torch.Tensor, padded_out: torch.Tensor) -> torch.Tensor:

@@ -76,41 +76,6 @@ static int launch_layout(GemmGroupArgs& ga, int at, int bt, hipStream_t st) {
 // registers over all S reductions, so C is read (at most) once and written once instead of S times, and
 // the k-loop of a tile is S times as long.  GemmArgs::A and ::B of a problem point to DEVICE arrays of
 // its S operand pointers.
-template <int BM, int BN, int W>
-__device__ __forceinline__ void load_c_as_accumulators(const GemmArgs& g, uint32_t tile_m, uint32_t tile_n,
-                                                       f32x16_t (&t)[WaveTile<BM, BN, W>::TN][WaveTile<BM, BN, W>::TM]) {
-    typedef WaveTile<BM, BN, W> WT;
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int l32 = lane & 31, lh = lane >> 5;
-    const int64_t m_base = (int64_t)tile_m * BM + (wave % WT::WGM) * WT::WTM + l32;
-    const int64_t n_base = (int64_t)tile_n * BN + (wave / WT::WGM) * WT::WTN + 4 * lh;
-    const float* C = static_cast<const float*>(g.C);
-    const bool vec_ok = (g.ldc & 3) == 0 && aligned(g.C, 16);
-#pragma unroll
-    for (int a = 0; a < WT::TN; ++a)
-#pragma unroll
-        for (int b = 0; b < WT::TM; ++b)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                // the accumulator layout of v_mfma_f32_32x32x16 with B as the first operand: a lane holds,
-                // for one row, four groups of four consecutive columns
-                const int64_t m = m_base + b * 32, n = n_base + a * 32 + 8 * q;
-                float v[4] = {0.f, 0.f, 0.f, 0.f};
-                if (m < g.M) {
-                    if (vec_ok && n + 3 < g.N) {
-                        const float4 w = *reinterpret_cast<const float4*>(C + m * g.ldc + n);
-                        v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (n + e < g.N) v[e] = C[m * g.ldc + n + e];
-                    }
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) t[a][b][4 * q + e] = v[e];
-            }
-}
-
 template <int BM, int BN, int NS, int KT, int W>
 __global__ __launch_bounds__(W * 64) void gemm_bf16_group_kseg_kernel(const GemmGroupArgs ga, const int n_seg) {
     uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);

@@ -156,6 +156,13 @@ static int run_one(const pp_op& op, pp_stream st) {
             return pp_gemm_bf16_segmented(&d, static_cast<const int32_t*>(op.p[6]),
                                           static_cast<const void* const*>(op.p[7]), (int)op.i[7], op.j[5], st);
         }
+        case PP_OP_GEMM_SEG_KSEG: {
+            const pp_gemm_desc d = gemm_desc_of(op);
+            return pp_gemm_bf16_segmented_kseg(&d, static_cast<const void* const*>(op.p[0]),
+                                               static_cast<const void* const*>(op.p[1]),
+                                               static_cast<const int32_t* const*>(op.p[6]),
+                                               static_cast<const void* const*>(op.p[7]), (int)op.i[7], (int)op.i[8], st);
+        }
         case PP_OP_MOE_ROUTER:
             return pp_moe_router_top2(op.p[0], op.i[0], op.i[1], (int)op.i[2], static_cast<int32_t*>(op.p[1]),
                                       static_cast<float*>(op.p[2]), st);
@@ -202,6 +209,8 @@ double op_work(const pp_op& op) {
         case PP_OP_GEMM_DSWIGLU:
         case PP_OP_GEMM_SEG:  // the segments partition the rows (rows mode: M, k mode: K)
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
+        case PP_OP_GEMM_SEG_KSEG:  // per microbatch the segments partition K (the upper bound given in i[2])
+            return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2] * (double)op.i[8];
         case PP_OP_GEMM_KSEG:  // one product per segment
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2] * (double)op.i[7];
         case PP_OP_GEMM_SWIGLU:  // two products of N columns each

@@ -111,6 +111,9 @@ class PipelineStageBase:
 
         self.fused_accumulate = fused_accumulate
         self.split_backward = False
+        #: run the weight-gradient passes of a step as one batched pass (``flush_weight_grads``) instead of
+        #: one per microbatch; set by the schedule, needs ``split_backward``
+        self.batch_weight_grads = False
         why: List[str] = []
         if not force_eager and self.device.type != "cuda":
             force_eager = True
@@ -495,6 +498,8 @@ class PipelineStageBase:
         if self.is_native:
             self._backward_input_native(mb, loss)
             self.bwd_chunk_id += 1
+            if self.batch_weight_grads and self.split_backward:
+                return                      # the weight gradients of the step follow in one batched pass
             self._backward_weight_native(mb)
             self.bwd_weight_chunk_id += 1
         else:
@@ -517,11 +522,42 @@ class PipelineStageBase:
         """Weight-gradient pass (dW) of the oldest microbatch whose input-gradient pass has run."""
         if not self.is_native:
             raise RuntimeError("split backward needs a native stage")
+        if self.batch_weight_grads:
+            return                          # deferred to ``flush_weight_grads``
         mb = self.bwd_weight_chunk_id
         if mb >= self.bwd_chunk_id:
             raise RuntimeError(f"{self.log_prefix} weight-gradient pass of microbatch {mb} before its input-gradient pass")
         self._backward_weight_native(mb)
         self.bwd_weight_chunk_id += 1
+
+    @property
+    def prefers_batched_weight_grads(self) -> bool:
+        """Whether one batched weight-gradient pass per step pays for this stage whatever the schedule:
+        stages whose blocks say so (expert weights: their fp32 accumulators outweigh a microbatch's
+        operands, so moving them once per step instead of once per microbatch is the larger part of the
+        pass)."""
+        return bool(self._blocks) and any(getattr(b, "_pp_batch_weight_grads", False) for b in self._blocks)
+
+    def flush_weight_grads(self) -> int:
+        """Runs the weight-gradient passes of all microbatches whose input-gradient pass has run and whose
+        weight-gradient pass has not, as one batched pass (``_program.BatchedW``: every weight-gradient GEMM
+        once over all of them, accumulation order and bits as microbatch by microbatch).  Returns how many
+        microbatches it covered."""
+        if not self.is_native:
+            return 0
+        lo, hi = self.bwd_weight_chunk_id, self.bwd_chunk_id
+        if hi <= lo:
+            return 0
+        if hi - lo == 1:
+            self._backward_weight_native(lo)
+            self.bwd_weight_chunk_id = hi
+            return 1
+        sp = self._program
+        self._start_accumulation_if_cleared(sp)
+        sp.batched_w(tuple(range(lo, hi))).run(init=not sp.acc_initialized)
+        self._after_weight_pass(sp)
+        self.bwd_weight_chunk_id = hi
+        return hi - lo
 
     def _backward_input_native(self, mb, loss):
         if mb not in self.fwd_cache:
@@ -546,22 +582,30 @@ class PipelineStageBase:
         self._bwd_done[mb] = True
         self.grads_input = [prog.input_grad]
 
-    def _backward_weight_native(self, mb):
-        sp = self._program
-        prog = sp.mbs[mb]
+    @staticmethod
+    def _start_accumulation_if_cleared(sp):
         fp32_params = sp.arena.dtype == torch.float32
         if (fp32_params or sp.grads_handed_over) and sp.acc_initialized and \
                 any(p.grad is None for _, p in sp.arena.named):
             # the user cleared the gradients (optimizer.zero_grad()): start a new accumulation
             sp.acc_initialized = False
             sp.grads_handed_over = False
-        sp.set_accumulate_mode(prog, init=not sp.acc_initialized)
-        prog.W.run()
+
+    @staticmethod
+    def _after_weight_pass(sp):
         sp.acc_initialized = True
-        if fp32_params:
+        if sp.arena.dtype == torch.float32:
             for _, p in sp.arena.named:
                 if p.grad is None:
                     p.grad = p.main_grad
+
+    def _backward_weight_native(self, mb):
+        sp = self._program
+        prog = sp.mbs[mb]
+        self._start_accumulation_if_cleared(sp)
+        sp.set_accumulate_mode(prog, init=not sp.acc_initialized)
+        prog.W.run()
+        self._after_weight_pass(sp)
 
     def _grad_from(self, consumer: "PipelineStageBase", pos: int, mb: int):
         if not consumer._bwd_done.get(mb):

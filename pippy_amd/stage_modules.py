@@ -962,6 +962,7 @@ class _MoEFeedForward:
     ``self._router`` (an ``nn.Linear``-shaped layer) and ``self.forced_routing``."""
 
     TOPK = 2
+    _pp_batch_weight_grads = True      # see PipelineStageBase.prefers_batched_weight_grads
 
     def _padded_experts(self) -> int:
         return (self.n_experts + 7) // 8 * 8

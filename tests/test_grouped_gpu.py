@@ -228,3 +228,47 @@ def test_kseg_rejects_what_it_does_not_compute():
         N.gemm_bf16_grouped_kseg([([A], [A], Cb, {})], [])
     with pytest.raises(RuntimeError, match="accumulated into an fp32 C"):
         N.gemm_bf16_grouped_kseg([([A], [A], Cf, {})], [])      # epilogue NONE does not accumulate
+
+
+@pytest.mark.parametrize("epi_name,beta", [("rounded", 0), ("rounded", 1), ("f32", 1)])
+def test_expert_weight_gradients_of_several_microbatches_in_one_launch(epi_name, beta):
+    """``pp_gemm_bf16_segmented_kseg``: every expert's C_e = (beta ? C_e : 0) + its product over each
+    microbatch's rows of that expert, added in microbatch order, against one accumulating k-mode launch per
+    microbatch (bit for bit); every microbatch has its own row partition, with empty and ragged segments."""
+    import ctypes as C
+    from pippy_amd import _native as N
+    N.lib()
+    torch.manual_seed(9)
+    epi = N.EPI_ACCUM_ROUNDED if epi_name == "rounded" else N.EPI_ACCUM_F32
+    E, n_mb, Mo, Ni = 5, 3, 256, 136
+    rows = [[70, 0, 131, 8, 47], [0, 0, 256, 0, 0], [33, 64, 1, 100, 58]]
+    As, Bs, segs = [], [], []
+    for m in range(n_mb):
+        R = sum(rows[m])
+        As.append(torch.randn(R, Mo, device=DEV).to(torch.bfloat16))
+        Bs.append(torch.randn(R, Ni, device=DEV).to(torch.bfloat16))
+        segs.append(torch.tensor([0] + list(torch.tensor(rows[m]).cumsum(0)), dtype=torch.int32, device=DEV))
+    C0 = [torch.randn(Mo, Ni, device=DEV) * 20 for _ in range(E)]
+    want = [c.clone() for c in C0]
+    want_ptrs = torch.tensor([c.data_ptr() for c in want], dtype=torch.int64, device=DEV)
+    for m in range(n_mb):
+        N.gemm_bf16_segmented(As[m], want_ptrs, None, segs[m], N.SEG_K, other=Bs[m], ld=Ni, epilogue=epi,
+                              beta=1 if (m or beta) else 0, c_dtype=torch.float32)
+    got = [c.clone() for c in C0]
+    got_ptrs = torch.tensor([c.data_ptr() for c in got], dtype=torch.int64, device=DEV)
+    a_of = torch.tensor([a.data_ptr() for a in As], dtype=torch.int64, device=DEV)
+    b_of = torch.tensor([b.data_ptr() for b in Bs], dtype=torch.int64, device=DEV)
+    s_of = torch.tensor([s.data_ptr() for s in segs], dtype=torch.int64, device=DEV)
+    d = N.GemmDesc()
+    d.M, d.N, d.K = Mo, Ni, max(sum(r) for r in rows)
+    d.lda, d.ldb, d.ldc = Mo, Ni, Ni
+    d.a_trans = d.b_trans = 1
+    d.c_dtype, d.epilogue, d.beta = N.PP_F32, epi, beta
+    N.check(N.lib().pp_gemm_bf16_segmented_kseg(C.byref(d), a_of.data_ptr(), b_of.data_ptr(), s_of.data_ptr(),
+                                                got_ptrs.data_ptr(), E, n_mb, N.current_stream()),
+            "pp_gemm_bf16_segmented_kseg")
+    torch.cuda.synchronize()
+    for e in range(E):
+        assert torch.equal(got[e], want[e]), f"expert {e}"
+    if not beta:
+        assert float(got[1].abs().max()) > 0          # expert 1 has rows in the last microbatch only

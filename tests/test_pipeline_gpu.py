@@ -1742,3 +1742,77 @@ def test_hugging_face_vit_runs_its_encoder_stage_natively_between_two_torch_stag
         assert named[name].grad is not None, name
     check_gradients({n: _Grad(p) for n, p in named.items()}, dict(ref.named_parameters()), run_in_bf16,
                     "ViT between two torch stages", note)
+
+
+# ---- the weight-gradient passes of a step as one batched pass ----------------------------------------
+def _grads_after_steps(sched_cls, batch, steps, n_stages=2, fused=False, zero_between=True):
+    import pippy_amd as pp
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(n_stages, M=M, fused=fused)
+    torch.manual_seed(123)
+    target = torch.randint(0, 1000, ids.shape)
+    sched = sched_cls(stages, M, loss_fn=pp.CrossEntropyLoss())
+    sched.batch_weight_grads = batch
+    for step in range(steps):
+        if zero_between or step == 0:
+            sched.zero_grad()
+        losses = []
+        sched.step(ids.to(DEV), target=target.to(DEV), losses=losses)
+    torch.cuda.synchronize()
+    n_batched = [st._program.batched_w(tuple(range(M))).n_batched if st.batch_weight_grads else 0 for st in stages]
+    return {n: p.main_grad.clone() for n, p in model.named_parameters()}, [l.clone() for l in losses], n_batched
+
+
+@pytest.mark.parametrize("schedule", ["1f1b", "gpipe", "zero_bubble", "interleaved"])
+@pytest.mark.parametrize("fused", [False, True])
+def test_weight_gradients_in_one_batched_pass_leave_the_bits_of_one_pass_per_microbatch(schedule, fused):
+    """With ``schedule.batch_weight_grads`` every weight-gradient GEMM of a stage runs once per step over all
+    microbatches, a tile adding the microbatches' (rounded) products to its running sum in ascending order:
+    the fp32 accumulators must hold the bits that one accumulating pass per microbatch leaves, after one
+    step from cleared gradients and after a second step that keeps accumulating (the sums then start from
+    what the accumulators hold)."""
+    import pippy_amd as pp
+    cls = {"1f1b": pp.Schedule1F1B, "gpipe": pp.ScheduleGPipe, "zero_bubble": pp.ScheduleZeroBubble,
+           "interleaved": pp.ScheduleInterleaved1F1B}[schedule]
+    for steps, zero_between in ((1, True), (2, False)):
+        got, losses_b, n_batched = _grads_after_steps(cls, True, steps, fused=fused, zero_between=zero_between)
+        want, losses_p, none = _grads_after_steps(cls, False, steps, fused=fused, zero_between=zero_between)
+        assert all(n >= 4 for n in n_batched) and not any(none), (n_batched, none)   # the GEMMs of a layer, at least
+        for a, b in zip(losses_b, losses_p):
+            assert torch.equal(a, b)
+        for name in want:
+            assert torch.equal(got[name], want[name]), f"{schedule}, {steps} step(s): grad of {name}"
+
+
+def test_expert_stages_batch_their_weight_gradients_by_default():
+    """Left to itself (``batch_weight_grads = None``) a schedule batches where it pays: stages with expert
+    weights, under any schedule; dense stages keep one weight-gradient pass per microbatch."""
+    import pippy_amd as pp
+    from pippy_amd.configs import MoEDecoderLM, equal_split_spec
+    M = 4
+    model, ref, stages, ref_stages, ids = _build_decoder(2, M=M)
+    target = torch.randint(0, 1000, ids.shape)
+    plain = pp.Schedule1F1B(stages, M, loss_fn=pp.CrossEntropyLoss())
+    plain.step(ids.to(DEV), target=target.to(DEV))
+    assert not any(st.batch_weight_grads for st in stages)
+
+    def moe_grads(batch):
+        torch.manual_seed(0)
+        S, vocab, L = 128, 512, 4
+        moe = MoEDecoderLM(vocab=vocab, dim=128, n_layers=L, n_heads=2, ffn=256, n_experts=8)
+        mids = torch.randint(0, vocab, (2 * M, S))
+        mtarget = torch.randint(0, vocab, (2 * M, S))
+        pipe = pp.pipeline(moe, M, (mids,), split_spec=equal_split_spec(L, 2))
+        mstages = [pp.PipelineStage(pipe, i, DEV, group=1) for i in range(2)]
+        sched = pp.ScheduleInterleaved1F1B(mstages, M, loss_fn=pp.CrossEntropyLoss())
+        sched.batch_weight_grads = batch
+        sched.step(mids.to(DEV), target=mtarget.to(DEV))
+        torch.cuda.synchronize()
+        return {n: p.main_grad.clone() for n, p in moe.named_parameters()}, [st.batch_weight_grads for st in mstages]
+
+    auto, flags = moe_grads(None)
+    assert all(flags)
+    per_microbatch, flags = moe_grads(False)
+    assert not any(flags)
+    for name in auto:
+        assert torch.equal(auto[name], per_microbatch[name]), f"grad of {name}"
