@@ -141,7 +141,13 @@ typedef struct pp_gemm_desc {
     int64_t ld_aux;
     int32_t beta;          /* PP_EPI_ACCUM_F32 / _ROUNDED: 0 overwrite, 1 accumulate */
     int32_t reserved;
+    float* colsum;         /* PP_EPI_DGELU_* / PP_EPI_DRELU with a bf16 C, or null: fp32
+                              [ceil(M / PP_GEMM_COLSUM_ROWS), N], row r receives the column sums of rows
+                              32 r .. 32 r + 31 of C as stored: partial sums of the bias gradient of the
+                              layer in front of the activation, for pp_colreduce_grouped with
+                              n_part_ready = ceil(M / 32) (pp_gemm_bf16 and pp_gemm_bf16_grouped only) */
 } pp_gemm_desc;
+#define PP_GEMM_COLSUM_ROWS 32
 
 /* Requirements: A, B 16-byte aligned; K % 8 == 0 unless both operands are transposed (then any K: the
  * weight gradient over any number of tokens); lda, ldb % 8 == 0; a transposed operand needs
@@ -325,7 +331,10 @@ int pp_moe_gate_bwd(const void* dout, int64_t ld_dout, const void* y, int64_t ld
  *   out_sum[c] = sum_r dy[r, c]                                   (bias gradient / dbeta), and, if
  *   out_dot is non-null, out_dot[c] = sum_r dy[r, c] * (x[r, c] - mean[r]) * rstd[r]   (dgamma).
  * workspace: fp32 [2, ceil(rows / 128), C] per descriptor, distinct between descriptors.  Sums are
- * formed in a fixed order, so results do not depend on scheduling. */
+ * formed in a fixed order, so results do not depend on scheduling.
+ * n_part_ready = P > 0: the kernel that produced dy has already left P rows of partial sums in the
+ * workspace (fp32 [2, P, C]: sums, then dots; pp_layernorm_bwd_input_sums writes that form), so dy
+ * and x are not read again (they may be null) and only the final sums are formed. */
 typedef struct pp_colreduce_desc {
     const void* dy;      /* bf16 [rows, C] with row stride ld_dy */
     const void* x;       /* bf16 [rows, C] contiguous, or null */
@@ -336,7 +345,7 @@ typedef struct pp_colreduce_desc {
     float* workspace;
     int64_t ld_dy, rows, C;
     int32_t out_dtype;   /* PP_BF16 or PP_F32 */
-    int32_t reserved;
+    int32_t n_part_ready; /* 0: reduce dy; P > 0: the workspace holds P rows of partial sums */
 } pp_colreduce_desc;
 #define PP_COLREDUCE_MAX_GROUP 24
 int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_stream stream);
@@ -353,6 +362,19 @@ int pp_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y
 int pp_layernorm_bwd_input(const void* dy, const void* x, const void* gamma, const float* mean,
                            const float* rstd, const void* dres, void* dx, int64_t rows, int64_t C,
                            pp_stream stream);
+/* pp_layernorm_bwd_input that also leaves column sums for the weight-gradient pass, so that dy, x and
+ * dx are not read a second time: per block of PP_LN_SUM_ROWS rows one row of partial sums,
+ *   ws_weight fp32 [2, P, C]: sum of dy (dbeta), then sum of dy * xhat (dgamma),
+ *   ws_dx     fp32 [P, C]:    sum of dx as written (rounded to bf16): the bias gradient of the linear
+ *                             layer whose output gradient dx is,
+ * with P = ceil(rows / PP_LN_SUM_ROWS); either may be null.  pp_colreduce_grouped with n_part_ready = P
+ * forms the final sums.  C <= PP_LN_SUM_MAX_C.  Same reference arithmetic as the two separate passes
+ * (F.layer_norm's backward reached from pippy/_backward.py:67-69), in a fixed summation order. */
+#define PP_LN_SUM_ROWS 16
+#define PP_LN_SUM_MAX_C 1024
+int pp_layernorm_bwd_input_sums(const void* dy, const void* x, const void* gamma, const float* mean,
+                                const float* rstd, const void* dres, void* dx, int64_t rows, int64_t C,
+                                float* ws_weight, float* ws_dx, pp_stream stream);
 /* dgamma, dbeta (bf16 [C] or fp32 by out_dtype): the weight-gradient pass.
  * workspace: fp32 [2, ceil(rows/128), C]. */
 int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean, const float* rstd,
@@ -457,11 +479,13 @@ enum pp_op_kind {
 /* Field use per kind (unused fields are ignored):
  *   GEMM_*        p: A B C bias aux_in aux_out | i: M N K lda ldb ldc ld_aux | j: a_trans b_trans
  *                 epilogue c_dtype beta; GEMM_BF16 also p[8]: split-K workspace or null, i[10]: its
- *                 size in floats (then the op is pp_gemm_bf16_splitk)
- *   COLSUM        p: dY out workspace | i: M N ld | j: out_dtype
+ *                 size in floats (then the op is pp_gemm_bf16_splitk), p[9]: colsum or null
+ *   COLSUM        p: dY out workspace | i: M N ld | j: out_dtype n_part_ready
  *   LN_FWD        p: x gamma beta y mean rstd | i: rows C | f: eps
- *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx | i: rows C
- *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype
+ *   LN_BWD_INPUT  p: dy x gamma mean rstd dres dx ws_weight ws_dx | i: rows C  (a non-null ws_weight or
+ *                 ws_dx: pp_layernorm_bwd_input_sums)
+ *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype n_part_ready
+ *                 (n_part_ready > 0, here and for COLSUM: the op runs through pp_colreduce_grouped)
  *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
  *                 | j: causal kv_group kv_len flags
  *   EMBED_FWD     p: ids wte wpe y extra_row pos_ids | i: n_tok seq C vocab n_pos  (pos_ids non-null:

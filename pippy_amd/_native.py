@@ -40,7 +40,7 @@ PP_COPY_MAX_SEGS = 64
 EXPORTED_SYMBOLS = (
     "pp_abi_version", "pp_last_error", "pp_copy_rows", "pp_split_copy", "pp_merge_copy",
     "pp_strided_copy_nd", "pp_grad_accum_f32_bf16", "pp_grad_accum_f32_f32", "pp_fill_bytes",
-    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_bf16_grouped_kseg", "pp_gemm_bf16_segmented_kseg", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input",
+    "pp_gemm_bf16", "pp_gemm_bf16_splitk", "pp_gemm_bf16_grouped", "pp_gemm_bf16_grouped_kseg", "pp_gemm_bf16_segmented_kseg", "pp_gemm_f32", "pp_colsum_bf16", "pp_colreduce_grouped", "pp_layernorm_fwd", "pp_layernorm_bwd_input", "pp_layernorm_bwd_input_sums",
     "pp_layernorm_bwd_weight", "pp_attn_fwd", "pp_attn_bwd", "pp_embed_fwd", "pp_embed_bwd",
     "pp_ce_loss", "pp_run_ops", "pp_activation_bwd", "pp_transpose_bf16", "pp_profile_start", "pp_profile_stop",
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
@@ -62,14 +62,14 @@ class GemmDesc(C.Structure):
                 ("a_trans", C.c_int32), ("b_trans", C.c_int32),
                 ("epilogue", C.c_int32), ("c_dtype", C.c_int32),
                 ("bias", C.c_void_p), ("aux_in", C.c_void_p), ("aux_out", C.c_void_p),
-                ("ld_aux", C.c_int64), ("beta", C.c_int32), ("reserved", C.c_int32)]
+                ("ld_aux", C.c_int64), ("beta", C.c_int32), ("reserved", C.c_int32), ("colsum", C.c_void_p)]
 
 
 class ColReduceDesc(C.Structure):
     _fields_ = [("dy", C.c_void_p), ("x", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p),
                 ("out_sum", C.c_void_p), ("out_dot", C.c_void_p), ("workspace", C.c_void_p),
                 ("ld_dy", C.c_int64), ("rows", C.c_int64), ("C", C.c_int64),
-                ("out_dtype", C.c_int32), ("reserved", C.c_int32)]
+                ("out_dtype", C.c_int32), ("n_part_ready", C.c_int32)]
 
 
 class AttnDesc(C.Structure):
@@ -127,6 +127,7 @@ def lib() -> C.CDLL:
         "pp_colreduce_grouped": [C.POINTER(ColReduceDesc), i32, vp],
         "pp_layernorm_fwd": [vp, vp, vp, vp, vp, vp, i64, i64, f32, vp],
         "pp_layernorm_bwd_input": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp],
+        "pp_layernorm_bwd_input_sums": [vp, vp, vp, vp, vp, vp, vp, i64, i64, vp, vp, vp],
         "pp_layernorm_bwd_weight": [vp, vp, vp, vp, vp, vp, i32, vp, i64, i64, vp],
         "pp_attn_fwd": [C.POINTER(AttnDesc), vp],
         "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
@@ -446,7 +447,7 @@ def fill_bytes(t: torch.Tensor, value: int = 0) -> None:
 def gemm_desc(A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, *, a_trans: bool = False,
               b_trans: bool = False, epilogue: int = EPI_NONE, bias: Optional[torch.Tensor] = None,
               aux_in: Optional[torch.Tensor] = None, aux_out: Optional[torch.Tensor] = None,
-              beta: int = 0) -> GemmDesc:
+              beta: int = 0, colsum: Optional[torch.Tensor] = None) -> GemmDesc:
     """A: [M,K] (or [K,M] if a_trans); B: [N,K] (or [K,N] if b_trans); Cm: [M,N].
     Row-major 2-d tensors whose last stride is 1 (a row stride larger than the row is fine)."""
     require_cuda(A, B, Cm, bias, aux_in, aux_out)
@@ -476,6 +477,10 @@ def gemm_desc(A: torch.Tensor, B: torch.Tensor, Cm: torch.Tensor, *, a_trans: bo
             ld_aux = t.stride(0)
     d.ld_aux = ld_aux
     d.beta = beta
+    if colsum is not None:
+        require_cuda(colsum)
+        assert colsum.dtype == torch.float32 and colsum.numel() >= ((M + GEMM_COLSUM_ROWS - 1) // GEMM_COLSUM_ROWS) * N
+    d.colsum = ptr(colsum)
     return d
 
 
@@ -564,7 +569,8 @@ def colsum(dY: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor) -> None
 
 
 def colreduce_grouped(items) -> None:
-    """items: dicts with dy, out_sum and/or out_dot, workspace and, for out_dot, x, mean, rstd."""
+    """items: dicts with dy, out_sum and/or out_dot, workspace and, for out_dot, x, mean, rstd; with
+    ``n_part_ready`` = P the workspace already holds P rows of partial sums and dy only gives the shape."""
     arr = (ColReduceDesc * len(items))()
     for d, it in zip(arr, items):
         dy = it["dy"]
@@ -573,7 +579,8 @@ def colreduce_grouped(items) -> None:
         d.x, d.mean, d.rstd = ptr(it.get("x")), ptr(it.get("mean")), ptr(it.get("rstd"))
         d.out_sum, d.out_dot = ptr(it.get("out_sum")), ptr(it.get("out_dot"))
         d.workspace = it["workspace"].data_ptr()
-        assert it["workspace"].numel() >= 2 * ((dy.shape[0] + 127) // 128) * dy.shape[1]
+        d.n_part_ready = int(it.get("n_part_ready", 0))
+        assert it["workspace"].numel() >= (d.n_part_ready or 2 * ((dy.shape[0] + 127) // 128)) * dy.shape[1]
         out = it.get("out_sum") if it.get("out_sum") is not None else it.get("out_dot")
         d.out_dtype = PP_F32 if out.dtype == torch.float32 else PP_BF16
     check(lib().pp_colreduce_grouped(arr, len(items), current_stream()), "pp_colreduce_grouped")
@@ -594,6 +601,25 @@ def layernorm_bwd_input(dy, x, gamma, mean, rstd, dres, dx) -> None:
     check(lib().pp_layernorm_bwd_input(dy.data_ptr(), x.data_ptr(), gamma.data_ptr(),
                                        ptr(mean), rstd.data_ptr(), ptr(dres), dx.data_ptr(),
                                        rows, Cc, current_stream()), "pp_layernorm_bwd_input")
+
+
+GEMM_COLSUM_ROWS = 32  # PP_GEMM_COLSUM_ROWS: rows of C per row of column sums that a GEMM epilogue leaves
+LN_SUM_ROWS = 16     # PP_LN_SUM_ROWS: rows per partial-sum row of pp_layernorm_bwd_input_sums
+LN_SUM_MAX_C = 1024  # PP_LN_SUM_MAX_C
+
+
+def layernorm_bwd_input_sums(dy, x, gamma, mean, rstd, dres, dx, ws_weight=None, ws_dx=None) -> int:
+    """The input gradient plus rows of partial column sums (one per ``LN_SUM_ROWS`` rows): ``ws_weight``
+    fp32 [2, P, C] (sum of dy, sum of dy * xhat), ``ws_dx`` fp32 [P, C] (sum of dx).  Returns P."""
+    require_cuda(dy, x, gamma, mean, rstd, dres, dx, ws_weight, ws_dx)
+    rows, Cc = x.shape
+    n_part = (rows + LN_SUM_ROWS - 1) // LN_SUM_ROWS
+    assert ws_weight is None or (ws_weight.dtype == torch.float32 and ws_weight.numel() >= 2 * n_part * Cc)
+    assert ws_dx is None or (ws_dx.dtype == torch.float32 and ws_dx.numel() >= n_part * Cc)
+    check(lib().pp_layernorm_bwd_input_sums(dy.data_ptr(), x.data_ptr(), gamma.data_ptr(), ptr(mean),
+                                            rstd.data_ptr(), ptr(dres), dx.data_ptr(), rows, Cc, ptr(ws_weight),
+                                            ptr(ws_dx), current_stream()), "pp_layernorm_bwd_input_sums")
+    return n_part
 
 
 def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:

@@ -21,6 +21,7 @@ input gradient straight into it: the hand-off is a pointer, not a copy).
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -794,6 +795,77 @@ class Builder:
         self._backward.append(scoped)
 
 
+# Pointer fields that an op of the input-gradient pass writes, by kind (kinds that are absent write through
+# fields that never hold a gradient tensor which a column reduction reads).
+_WRITTEN_FIELDS = {
+    N.OP_GEMM_BF16: (2, 5), N.OP_GEMM_F32: (2, 5), N.OP_GEMM_SEG: (2, 5), N.OP_LN_BWD_INPUT: (6,),
+    N.OP_ATTN_BWD: (6, 7, 8, 9), N.OP_ACT_BWD: (2,), N.OP_SWIGLU_BWD: (3, 4), N.OP_ROPE: (0,),
+    N.OP_COPY_ROWS: (1,), N.OP_FILL: (0,), N.OP_ACCUM_BF16: (0,), N.OP_ACCUM_F32: (0,),
+    N.OP_MOE_GATHER: (4,), N.OP_MOE_COMBINE: (4,), N.OP_MOE_GATE_BWD: (5,), N.OP_GEMM_DSWIGLU: (3,),
+    N.OP_EMBED_BWD: (2, 3), N.OP_CE_LOSS: (2, 3),
+}
+
+
+def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
+    """Lets the kernels of the I pass that produce a gradient tensor leave the partial column sums that the W
+    pass needs of it, so that its column reductions do not read the tensor from memory a second time:
+
+    * the dgamma / dbeta reduction of a LayerNorm takes them from that LayerNorm's own input-gradient op;
+    * a bias-gradient column sum over a tensor that a LayerNorm input-gradient op wrote as its ``dx`` (the
+      gradient of the residual stream, which is the output gradient of the linear layer in front of the
+      norm) takes the sums of ``dx`` from that op;
+    * a bias-gradient column sum over the output of a GEMM with an activation-derivative epilogue (the
+      gradient in front of a GELU or ReLU) takes them from that GEMM's epilogue.
+
+    Only exact matches are rewired: same pointers, same shape, a contiguous tensor, and no other op of the I
+    pass writing to the same address."""
+    if os.environ.get("PIPPY_AMD_TWO_PASS_COLUMN_SUMS") == "1":  # for A / B measurements of this rewiring
+        return
+    I = prog.I.ops
+    ln_ops = [op for op in I if op.kind == N.OP_LN_BWD_INPUT and 0 < op.i[1] <= N.LN_SUM_MAX_C]
+    act_ops = [op for op in I if op.kind == N.OP_GEMM_BF16 and op.j[3] == N.PP_BF16 and not op.p[8]
+               and op.j[2] in (N.EPI_DGELU_ERF, N.EPI_DGELU_TANH, N.EPI_DRELU)]
+    if not ln_ops and not act_ops:
+        return
+    written: Dict[int, int] = {}
+    for op in I:
+        for q in _WRITTEN_FIELDS.get(op.kind, range(10)):
+            if op.p[q]:
+                written[op.p[q]] = written.get(op.p[q], 0) + 1
+    for k, (op, _tag) in enumerate(b._w_reduce):
+        if op.j[1]:
+            continue
+        if op.kind == N.OP_LN_BWD_WEIGHT:
+            src = [l for l in ln_ops if l.p[0] == op.p[0] and l.p[1] == op.p[1] and l.i[0] == op.i[0]
+                   and l.i[1] == op.i[1] and not l.p[7]]
+            if len(src) != 1:
+                continue
+            rows, Cc = op.i[0], op.i[1]
+            n_part = (rows + N.LN_SUM_ROWS - 1) // N.LN_SUM_ROWS
+            ws = b.grad(f"colsums.{k}", (2 * n_part * Cc,), torch.float32)
+            src[0].p[7] = ws.data_ptr()
+            op.p[6], op.j[1] = ws.data_ptr(), n_part
+        elif op.kind == N.OP_COLSUM:
+            rows, Cc, ld = op.i[0], op.i[1], op.i[2]
+            if written.get(op.p[0], 0) != 1:
+                continue
+            src = [l for l in ln_ops if l.p[6] == op.p[0] and l.i[0] == rows and l.i[1] == Cc and not l.p[8]]
+            if len(src) == 1 and ld == Cc:
+                n_part = (rows + N.LN_SUM_ROWS - 1) // N.LN_SUM_ROWS
+                ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
+                src[0].p[8] = ws.data_ptr()
+                op.p[2], op.j[1] = ws.data_ptr(), n_part
+                continue
+            # the input gradient of an activation, written by the epilogue of the GEMM in front of it
+            src = [g for g in act_ops if g.p[2] == op.p[0] and g.i[0] == rows and g.i[1] == Cc and g.i[5] == ld
+                   and not g.p[9]]
+            if len(src) == 1:
+                n_part = (rows + N.GEMM_COLSUM_ROWS - 1) // N.GEMM_COLSUM_ROWS
+                ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
+                src[0].p[9] = ws.data_ptr()
+                op.p[2], op.j[1] = ws.data_ptr(), n_part
+
+
 class StageProgram:
     """All microbatch programs of one stage plus its arenas and shared buffers."""
 
@@ -882,6 +954,7 @@ class StageProgram:
             if dx_target is not None:
                 assert dy is not None and dy.data_ptr() == dx_target.data_ptr()
             prog.input_grad = dy
+            _fuse_column_sums(b, prog)
             toggles = {"accum": prog.init_toggle_accum, "beta": prog.init_toggle_beta,
                        "fill": prog.init_toggle_fill}
             for op, tag in b._w_gemm + b._w_reduce + b._w_other:

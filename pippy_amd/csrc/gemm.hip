@@ -522,7 +522,8 @@ extern "C" int pp_gemm_bf16_splitk(const pp_gemm_desc* d, float* workspace, int6
     int rc = convert(d, &g, &empty);
     if (rc || empty) return rc;
     int kt_per_split = 0;
-    const int splits = (workspace && aligned(workspace, 16)) ? splitk_plan(d, workspace_elems, &kt_per_split) : 0;
+    // the column sums of an activation-derivative epilogue are formed by the single-launch epilogue only
+    const int splits = (workspace && aligned(workspace, 16) && !g.colsum) ? splitk_plan(d, workspace_elems, &kt_per_split) : 0;
     if (!splits) return pp_gemm_bf16(d, stream);
     rc = count_tiles<256, 256>(g);
     if (rc) return rc;

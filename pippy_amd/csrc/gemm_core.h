@@ -22,7 +22,13 @@ struct GemmArgs {
     int round_bf16;  // fp32 C: round the sums to bf16 before they are stored or added
     int epi;         // the problem's epilogue, for kernels that take it at run time (kEpiRuntime)
     uint32_t tiles_m, tiles_n, n_blocks;
+    // activation-derivative epilogues: fp32 [ceil(M / 32)][N], the column sums of every band of 32 rows of C
+    // as stored (what the bias gradient of the layer in front of the activation is the sum of), or null
+    float* colsum = nullptr;
 };
+__host__ __device__ constexpr bool epi_may_sum_columns(int epi) {
+    return epi == PP_EPI_DGELU_ERF || epi == PP_EPI_DGELU_TANH || epi == PP_EPI_DRELU;
+}
 
 // Template value of EPI for kernels whose problems bring their own epilogue (GemmArgs::epi): the
 // grouped launches of problems that differ in it.  Only for a bf16 C.
@@ -107,7 +113,8 @@ __device__ __forceinline__ void epilogue_math4(float (&v)[4], float (&pre)[4], c
 // and columns past the edge of C and unaligned operands.
 template <int EPI, bool CF32>
 __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t n0, float v0, float v1,
-                                          float v2, float v3, const float (&bias)[4], bool vec_ok) {
+                                          float v2, float v3, const float (&bias)[4], bool vec_ok,
+                                          float* colsum4 = nullptr) {
     if (m >= g.M || n0 >= g.N) return;
     float v[4] = {v0, v1, v2, v3}, pre[4];
     const int nv = (g.N - n0 >= 4) ? 4 : (int)(g.N - n0);
@@ -165,6 +172,11 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int64_t m, int64_t 
         }
     } else {
         uint16_t* cp = static_cast<uint16_t*>(g.C) + m * g.ldc + n0;
+        if (colsum4) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nv) colsum4[e] += bf16_to_f32(f32_to_bf16(v[e]));
+        }
         if (full) {
             *reinterpret_cast<uint2*>(cp) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
         } else {
@@ -365,6 +377,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
                     make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
             }
         const int64_t gm = m0 + wm0 + b * 32 + rr;  // row of pass 0; pass i adds i * RPP
+        constexpr bool kMaySum = !CF32 && (EPI == kEpiRuntime || epi_may_sum_columns(EPI));
+        const bool sums = kMaySum && g.colsum && epi_may_sum_columns(epi);
+        float cs[4] = {0.f, 0.f, 0.f, 0.f};  // this lane's rows of the band, its 4 columns
         if (interior && lane_on) {
 #pragma unroll EpiUnroll<EPI>::value
           for (int i0 = 0; i0 < kPasses; i0 += kBatch) {
@@ -410,8 +425,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
                     else
                         *reinterpret_cast<float4*>(cp) = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
-                    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(g.C) + row * g.ldc + gn) =
-                        make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+                    const uint32_t w0 = pack_bf16(v[0], v[1]), w1 = pack_bf16(v[2], v[3]);
+                    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(g.C) + row * g.ldc + gn) = make_uint2(w0, w1);
+                    if (kMaySum && sums) {
+                        cs[0] += bf16lo(w0); cs[1] += bf16hi(w0); cs[2] += bf16lo(w1); cs[3] += bf16hi(w1);
+                    }
                 }
             }
           }
@@ -420,7 +438,23 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
             for (int i = 0; i < kPasses; ++i) {
                 const int m = i * RPP + rr;
                 const float4 v = *reinterpret_cast<const float4*>(cw + m * WTN + (unit_at(ru, m) << 2));
-                epilogue4<EPI, CF32>(g, gm + i * RPP, gn, v.x, v.y, v.z, v.w, bias, vec_ok);
+                epilogue4<EPI, CF32>(g, gm + i * RPP, gn, v.x, v.y, v.z, v.w, bias, vec_ok,
+                                     kMaySum && sums ? cs : nullptr);
+            }
+        }
+        if (kMaySum && sums) {
+            // the RPP lanes that share these 4 columns, added in row order; the first of them writes
+            float t[4] = {cs[0], cs[1], cs[2], cs[3]};
+#pragma unroll
+            for (int r = 1; r < RPP; ++r)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[e] += __shfl(cs[e], ru + r * UPR, 64);
+            const int64_t band_row = m0 + wm0 + b * 32;
+            if (lane < UPR && band_row < g.M) {
+                float* out = g.colsum + (band_row >> 5) * g.N + gn;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (gn + e < g.N) out[e] = t[e];
             }
         }
     });
@@ -573,6 +607,10 @@ static inline int convert(const pp_gemm_desc* d, GemmArgs* g, bool* empty) {
     g->round_bf16 = d->epilogue == PP_EPI_ACCUM_ROUNDED;
     g->epi = epi;
     g->tiles_m = g->tiles_n = g->n_blocks = 0;
+    if (d->colsum && (!epi_may_sum_columns(epi) || d->c_dtype != PP_BF16))
+        return fail(PP_ERR_INVALID, "pp_gemm_bf16: column sums come with the activation-derivative epilogues "
+                    "and a bf16 C (epilogue %d)", epi);
+    g->colsum = d->colsum;
     return PP_OK;
 }
 

@@ -125,6 +125,7 @@ extern "C" int pp_gemm_f32(const pp_gemm_desc* d, pp_stream stream) {
     if (d->M == 0 || d->N == 0) return PP_OK;
     if (!d->A || !d->B || !d->C) return fail(PP_ERR_INVALID, "pp_gemm_f32: null operand");
     if (d->c_dtype != PP_F32) return fail(PP_ERR_INVALID, "pp_gemm_f32: C must be fp32");
+    if (d->colsum) return fail(PP_ERR_UNSUPPORTED, "pp_gemm_f32: no column sums (pp_gemm_bf16 forms them)");
     if (d->lda < (d->a_trans ? d->M : d->K) || d->ldb < (d->b_trans ? d->N : d->K) || d->ldc < d->N)
         return fail(PP_ERR_INVALID, "pp_gemm_f32: leading dimension too small");
     if (d->epilogue == PP_EPI_DRELU && (!d->aux_in || d->ld_aux < d->N))

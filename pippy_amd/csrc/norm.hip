@@ -78,6 +78,14 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const uint16_t* __re
     }
 }
 
+// a * b + c with the product rounded before the sum, whatever contraction the compiler is allowed elsewhere:
+// the two input-gradient kernels below must write the same bits
+__device__ __forceinline__ float mul_then_add(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float p = a * b;
+    return p + c;
+}
+
 // ---- input gradient ---------------------------------------------------------------------------
 template <int NV>
 __global__ __launch_bounds__(256) void layernorm_bwd_input_kernel(
@@ -121,16 +129,151 @@ __global__ __launch_bounds__(256) void layernorm_bwd_input_kernel(
         const int c = lane + 64 * i;
         if (c < nchunk) {
             float o[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (wd[i][e] - c1 * xh[i][e] - c2) * rstd;
+            float rf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if (dres) {
                 const uint4 rw = reinterpret_cast<const uint4*>(dres + row * C)[c];
-                o[0] += bf16lo(rw.x); o[1] += bf16hi(rw.x); o[2] += bf16lo(rw.y); o[3] += bf16hi(rw.y);
-                o[4] += bf16lo(rw.z); o[5] += bf16hi(rw.z); o[6] += bf16lo(rw.w); o[7] += bf16hi(rw.w);
+                rf[0] = bf16lo(rw.x); rf[1] = bf16hi(rw.x); rf[2] = bf16lo(rw.y); rf[3] = bf16hi(rw.y);
+                rf[4] = bf16lo(rw.z); rf[5] = bf16hi(rw.z); rf[6] = bf16lo(rw.w); rf[7] = bf16hi(rw.w);
             }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = mul_then_add(wd[i][e] - c1 * xh[i][e] - c2, rstd, rf[e]);
             outr[c] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]),
                                  pack_bf16(o[6], o[7]));
         }
+    }
+}
+
+// ---- input gradient that also leaves column sums --------------------------------------------
+// The same arithmetic per row; a block owns kSumRows consecutive rows (WAVES waves of RW rows each) and
+// writes one row of partial column sums per requested quantity: sum of dy (dbeta) and of dy * xhat
+// (dgamma) into ws_w [2][n_part][C], sum of the rounded dx (the bias gradient of the linear layer that
+// produced the normalised tensor's input) into ws_dx [n_part][C].  Rows are added in ascending order
+// within a wave and the waves in wave order, so the sums do not depend on scheduling.
+constexpr int kSumRows = PP_LN_SUM_ROWS;
+
+template <int NV, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void layernorm_bwd_input_sums_kernel(
+    const uint16_t* __restrict__ dy, const uint16_t* __restrict__ x, const uint16_t* __restrict__ gamma,
+    const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+    const uint16_t* __restrict__ dres, uint16_t* __restrict__ dx, int64_t rows, int C,
+    float* __restrict__ ws_w, float* __restrict__ ws_dx, int64_t n_part) {
+    constexpr int RW = kSumRows / WAVES;  // rows per wave, their loads in flight together
+    static_assert(RW * WAVES == kSumRows, "the waves share the block's rows evenly");
+    extern __shared__ __attribute__((aligned(16))) float red[];  // [quantities][WAVES][C]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nchunk = C >> 3;
+    float gf[NV][8];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = lane + 64 * i;
+        const uint4 gw = c < nchunk ? reinterpret_cast<const uint4*>(gamma)[c] : make_uint4(0, 0, 0, 0);
+        gf[i][0] = bf16lo(gw.x); gf[i][1] = bf16hi(gw.x); gf[i][2] = bf16lo(gw.y); gf[i][3] = bf16hi(gw.y);
+        gf[i][4] = bf16lo(gw.z); gf[i][5] = bf16hi(gw.z); gf[i][6] = bf16lo(gw.w); gf[i][7] = bf16hi(gw.w);
+    }
+    float sb[NV][8], sg[NV][8], sx[NV][8];
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sb[i][e] = sg[i][e] = sx[i][e] = 0.f;
+    const int64_t row0 = (int64_t)blockIdx.x * kSumRows + wave * RW;
+    uint4 xw[RW][NV], dw[RW][NV], rw[RW][NV];
+    float mean[RW], rstd[RW];
+#pragma unroll
+    for (int j = 0; j < RW; ++j) {
+        const int64_t row = row0 + j;
+        const bool live = row < rows;
+        mean[j] = live && mean_in ? mean_in[row] : 0.f;
+        rstd[j] = live ? rstd_in[row] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane + 64 * i;
+            const bool on = live && c < nchunk;
+            xw[j][i] = on ? reinterpret_cast<const uint4*>(x + row * C)[c] : make_uint4(0, 0, 0, 0);
+            dw[j][i] = on ? reinterpret_cast<const uint4*>(dy + row * C)[c] : make_uint4(0, 0, 0, 0);
+            rw[j][i] = on && dres ? reinterpret_cast<const uint4*>(dres + row * C)[c] : make_uint4(0, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < RW; ++j) {
+        const int64_t row = row0 + j;
+        if (row >= rows) continue;  // wave-uniform
+        float xh[NV][8], wd[NV][8];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint4 a = xw[j][i], d = dw[j][i];
+            const float xf[8] = {bf16lo(a.x), bf16hi(a.x), bf16lo(a.y), bf16hi(a.y),
+                                 bf16lo(a.z), bf16hi(a.z), bf16lo(a.w), bf16hi(a.w)};
+            const float df[8] = {bf16lo(d.x), bf16hi(d.x), bf16lo(d.y), bf16hi(d.y),
+                                 bf16lo(d.z), bf16hi(d.z), bf16lo(d.w), bf16hi(d.w)};
+            const bool on = lane + 64 * i < nchunk;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                xh[i][e] = on ? (xf[e] - mean[j]) * rstd[j] : 0.f;
+                wd[i][e] = df[e] * gf[i][e];
+                s1 += wd[i][e] * xh[i][e];
+                s2 += wd[i][e];
+                sb[i][e] += df[e];
+                sg[i][e] += df[e] * xh[i][e];
+            }
+        }
+        const float c1 = wave_sum(s1) / (float)C;
+        const float c2 = mean_in ? wave_sum(s2) / (float)C : 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane + 64 * i;
+            if (c < nchunk) {
+                const uint4 r = rw[j][i];
+                const float rf[8] = {bf16lo(r.x), bf16hi(r.x), bf16lo(r.y), bf16hi(r.y),
+                                     bf16lo(r.z), bf16hi(r.z), bf16lo(r.w), bf16hi(r.w)};
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float o0 = mul_then_add(wd[i][e] - c1 * xh[i][e] - c2, rstd[j], rf[e]);
+                    const float o1 = mul_then_add(wd[i][e + 1] - c1 * xh[i][e + 1] - c2, rstd[j], rf[e + 1]);
+                    w[e >> 1] = pack_bf16(o0, o1);
+                    sx[i][e] += bf16lo(w[e >> 1]);
+                    sx[i][e + 1] += bf16hi(w[e >> 1]);
+                }
+                reinterpret_cast<uint4*>(dx + row * C)[c] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
+    // the waves' sums, in wave order; the requested quantities side by side in LDS, one barrier for all
+    const int kRowFloats = C, kSetFloats = WAVES * C;
+    float* const outs[3] = {ws_w, ws_w ? ws_w + n_part * C : nullptr, ws_dx};
+    int set = 0;
+#pragma unroll
+    for (int pass = 0; pass < 3; ++pass) {
+        if (!outs[pass]) continue;  // uniform over the grid
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            if (lane + 64 * i >= nchunk) continue;
+            const float* s = pass == 0 ? sb[i] : pass == 1 ? sg[i] : sx[i];
+            float4* r = reinterpret_cast<float4*>(&red[set * kSetFloats + wave * kRowFloats + (lane + 64 * i) * 8]);
+            r[0] = make_float4(s[0], s[1], s[2], s[3]);
+            r[1] = make_float4(s[4], s[5], s[6], s[7]);
+        }
+        ++set;
+    }
+    __syncthreads();
+    // four columns per lane and step, over the requested quantities laid end to end
+    const int n_sets = set, quads = C >> 2;
+    for (int q = threadIdx.x; q < n_sets * quads; q += WAVES * 64) {
+        const int which = q / quads, c4 = q - which * quads;
+        const float4* r = reinterpret_cast<const float4*>(red + which * kSetFloats) + c4;
+        float4 v[WAVES];
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) v[w] = r[w * (kRowFloats >> 2)];
+        float4 t = v[0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) { t.x += v[w].x; t.y += v[w].y; t.z += v[w].z; t.w += v[w].w; }
+        // set number `which` is the which-th requested quantity
+        int pass = 0, seen = 0;
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+            if (outs[p]) { if (seen == which) pass = p; ++seen; }
+        reinterpret_cast<float4*>(outs[pass] + (int64_t)blockIdx.x * C)[c4] = t;
     }
 }
 
@@ -230,6 +373,7 @@ struct ColDesc {
     float* ws;       // [2][n_part][C]: sums, then dots
     int64_t ld_dy;
     int rows, C, n_part, n_cb, out_f32;
+    int ready;  // the workspace already holds n_part rows of partial sums (a producer kernel wrote them)
 };
 
 struct ColGroupArgs {
@@ -297,6 +441,39 @@ __global__ __launch_bounds__(256) void colgroup_final_kernel(const ColGroupArgs 
     while (i + 1 < ga.n && b >= ga.final_start[i + 1]) ++i;
     b -= ga.final_start[i];
     const ColDesc& d = ga.d[i];
+    if (d.ready) {
+        // partial sums left by a producer, many rows of them: 32 columns per block, the rows dealt out to 8
+        // phases (phase p adds rows p, p + 8, ... in ascending order), the phases added in phase order
+        __shared__ float red[8][32 + 1];
+        const int cc = threadIdx.x & 31, rp = threadIdx.x >> 5;
+        const int c = b * 32 + cc;
+        for (int pass = 0; pass < 2; ++pass) {
+            void* out = pass == 0 ? d.out_sum : d.out_dot;
+            if (!out) continue;  // uniform over the block
+            const float* part = d.ws + (int64_t)pass * d.n_part * d.C + c;
+            float t = 0.f;
+            if (c < d.C) {
+                int p = rp;
+                for (; p + 24 < d.n_part; p += 32) {
+                    const float v0 = part[(int64_t)p * d.C], v1 = part[(int64_t)(p + 8) * d.C],
+                                v2 = part[(int64_t)(p + 16) * d.C], v3 = part[(int64_t)(p + 24) * d.C];
+                    t += v0; t += v1; t += v2; t += v3;
+                }
+                for (; p < d.n_part; p += 8) t += part[(int64_t)p * d.C];
+            }
+            __syncthreads();
+            red[rp][cc] = t;
+            __syncthreads();
+            if (rp == 0 && c < d.C) {
+                float sum = 0.f;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) sum += red[q][cc];
+                if (d.out_f32) static_cast<float*>(out)[c] = sum;
+                else static_cast<uint16_t*>(out)[c] = f32_to_bf16(sum);
+            }
+        }
+        return;
+    }
     const int c = b * 256 + threadIdx.x;
     if (c >= d.C) return;
     for (int pass = 0; pass < 2; ++pass) {
@@ -324,6 +501,30 @@ static void launch_ln_bwd_in(const void* dy, const void* x, const void* gamma, c
     hipLaunchKernelGGL(layernorm_bwd_input_kernel<NV>, dim3(nb), dim3(256), 0, st, (const uint16_t*)dy,
                        (const uint16_t*)x, (const uint16_t*)gamma, mean, rstd, (const uint16_t*)dres,
                        (uint16_t*)dx, rows, C);
+}
+
+#ifndef PP_LN_SUM_WAVES
+#define PP_LN_SUM_WAVES 8
+#endif
+template <int NV>
+static int launch_ln_bwd_in_sums(const void* dy, const void* x, const void* gamma, const float* mean,
+                                 const float* rstd, const void* dres, void* dx, int64_t rows, int C,
+                                 float* ws_w, float* ws_dx, hipStream_t st) {
+    constexpr int WAVES = PP_LN_SUM_WAVES;
+    // one set of WAVES rows per requested quantity
+    const size_t lds = (size_t)((ws_w ? 2 : 0) + (ws_dx ? 1 : 0)) * WAVES * C * sizeof(float);
+    static_assert((size_t)3 * WAVES * PP_LN_SUM_MAX_C * sizeof(float) <= 160 * 1024, "LDS of one CU");
+    static const hipError_t attr_rc = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&layernorm_bwd_input_sums_kernel<NV, WAVES>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)3 * WAVES * PP_LN_SUM_MAX_C * sizeof(float)));
+    if (attr_rc != hipSuccess)
+        return fail(PP_ERR_LAUNCH, "pp_layernorm_bwd_input_sums: cannot reserve %zu bytes of LDS: %s", lds,
+                    hipGetErrorString(attr_rc));
+    const int64_t n_part = (rows + kSumRows - 1) / kSumRows;
+    hipLaunchKernelGGL((layernorm_bwd_input_sums_kernel<NV, WAVES>), dim3((uint32_t)n_part), dim3(WAVES * 64), lds, st,
+                       (const uint16_t*)dy, (const uint16_t*)x, (const uint16_t*)gamma, mean, rstd,
+                       (const uint16_t*)dres, (uint16_t*)dx, rows, C, ws_w, ws_dx, n_part);
+    return PP_OK;
 }
 
 static int ln_check(const char* who, int64_t rows, int64_t C) {
@@ -375,6 +576,28 @@ extern "C" int pp_layernorm_bwd_input(const void* dy, const void* x, const void*
     else if (nv <= 8) launch_ln_bwd_in<8>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
     else launch_ln_bwd_in<16>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, st);
     return check_launch("layernorm_bwd_input_kernel");
+}
+
+extern "C" int pp_layernorm_bwd_input_sums(const void* dy, const void* x, const void* gamma, const float* mean,
+                                           const float* rstd, const void* dres, void* dx, int64_t rows,
+                                           int64_t C, float* ws_weight, float* ws_dx, pp_stream stream) {
+    if (!ws_weight && !ws_dx) return pp_layernorm_bwd_input(dy, x, gamma, mean, rstd, dres, dx, rows, C, stream);
+    int rc = ln_check("pp_layernorm_bwd_input_sums", rows, C);
+    if (rc) return rc;
+    if (C > PP_LN_SUM_MAX_C)
+        return fail(PP_ERR_UNSUPPORTED, "pp_layernorm_bwd_input_sums: C = %lld exceeds %d (the waves' sums of a block meet in "
+                    "LDS); use pp_layernorm_bwd_input and the column reductions", (long long)C, PP_LN_SUM_MAX_C);
+    if (rows == 0) return PP_OK;
+    if (!dy || !x || !gamma || !rstd || !dx)
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input_sums: null pointer");
+    if (!aligned(x, 16) || !aligned(dy, 16) || !aligned(gamma, 16) || !aligned(dres, 16) || !aligned(dx, 16))
+        return fail(PP_ERR_INVALID, "pp_layernorm_bwd_input_sums: pointers must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int nv = (int)((C / 8 + 63) / 64);
+    if (nv <= 1) rc = launch_ln_bwd_in_sums<1>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, ws_weight, ws_dx, st);
+    else rc = launch_ln_bwd_in_sums<2>(dy, x, gamma, mean, rstd, dres, dx, rows, (int)C, ws_weight, ws_dx, st);
+    if (rc) return rc;
+    return check_launch("layernorm_bwd_input_sums_kernel");
 }
 
 extern "C" int pp_layernorm_bwd_weight(const void* dy, const void* x, const float* mean,
@@ -487,9 +710,11 @@ extern "C" int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_st
         for (int i = 0; i < cnt; ++i) {
             const pp_colreduce_desc& s = descs[i0 + i];
             if (s.rows < 0 || s.C <= 0 || s.ld_dy < s.C) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: bad shape in %d", i0 + i);
-            if ((s.C % 8) || (s.ld_dy % 8)) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: C and ld must be multiples of 8");
-            if (!s.dy || !s.workspace || (!s.out_sum && !s.out_dot)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: null pointer in %d", i0 + i);
-            if (s.out_dot && (!s.x || !s.rstd)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: out_dot needs x and rstd");
+            if (!(s.n_part_ready > 0) && ((s.C % 8) || (s.ld_dy % 8))) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: C and ld must be multiples of 8");
+            const bool ready = s.n_part_ready > 0;
+            if ((!ready && !s.dy) || !s.workspace || (!s.out_sum && !s.out_dot)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: null pointer in %d", i0 + i);
+            if (!ready && s.out_dot && (!s.x || !s.rstd)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: out_dot needs x and rstd");
+            if (s.n_part_ready < 0) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: negative n_part_ready in %d", i0 + i);
             if (!aligned(s.dy, 16) || !aligned(s.x, 16)) return fail(PP_ERR_INVALID, "pp_colreduce_grouped: dy and x must be 16-byte aligned");
             if (s.rows > 0x7fffffff || s.C > 0x7fffffff) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: shape too large");
             ColDesc& d = ga.d[ga.n];
@@ -500,13 +725,14 @@ extern "C" int pp_colreduce_grouped(const pp_colreduce_desc* descs, int n, pp_st
             d.ws = s.workspace;
             d.ld_dy = s.ld_dy;
             d.rows = (int)s.rows; d.C = (int)s.C;
-            d.n_part = (int)((s.rows + 127) / 128);
+            d.ready = ready;
+            d.n_part = ready ? s.n_part_ready : (int)((s.rows + 127) / 128);
             d.n_cb = (int)((s.C + 255) / 256);
             d.out_f32 = s.out_dtype == PP_F32;
             ga.part_start[ga.n] = (uint32_t)pb;
             ga.final_start[ga.n] = (uint32_t)fb;
-            pb += (uint64_t)d.n_part * d.n_cb;
-            fb += (uint64_t)d.n_cb;
+            if (!ready) pb += (uint64_t)d.n_part * d.n_cb;
+            fb += ready ? (uint64_t)((s.C + 31) / 32) : (uint64_t)d.n_cb;
             ++ga.n;
         }
         if (pb > 0x7fffffffull) return fail(PP_ERR_UNSUPPORTED, "pp_colreduce_grouped: too many blocks");

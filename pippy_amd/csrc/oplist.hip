@@ -14,6 +14,7 @@ static pp_gemm_desc gemm_desc_of(const pp_op& op) {
     d.lda = op.i[3]; d.ldb = op.i[4]; d.ldc = op.i[5]; d.ld_aux = op.i[6];
     d.a_trans = op.j[0]; d.b_trans = op.j[1]; d.epilogue = op.j[2]; d.c_dtype = op.j[3];
     d.beta = op.j[4]; d.reserved = 0;
+    d.colsum = op.kind == PP_OP_GEMM_BF16 ? static_cast<float*>(op.p[9]) : nullptr;
     return d;
 }
 
@@ -68,7 +69,7 @@ static pp_colreduce_desc colreduce_desc_of(const pp_op& op) {
         d.rows = op.i[0]; d.C = op.i[1]; d.ld_dy = op.i[1];
     }
     d.out_dtype = op.j[0];
-    d.reserved = 0;
+    d.n_part_ready = op.j[1];
     return d;
 }
 
@@ -82,16 +83,25 @@ static int run_one(const pp_op& op, pp_stream st) {
             return op.kind == PP_OP_GEMM_BF16 ? pp_gemm_bf16(&d, st) : pp_gemm_f32(&d, st);
         }
         case PP_OP_COLSUM:
+            if (op.j[1] > 0) {  // partial sums are there already: only the grouped call takes them
+                const pp_colreduce_desc d = colreduce_desc_of(op);
+                return pp_colreduce_grouped(&d, 1, st);
+            }
             return pp_colsum_bf16(op.p[0], op.i[0], op.i[1], op.i[2], op.p[1], op.j[0],
                                   static_cast<float*>(op.p[2]), st);
         case PP_OP_LN_FWD:
             return pp_layernorm_fwd(op.p[0], op.p[1], op.p[2], op.p[3], static_cast<float*>(op.p[4]),
                                     static_cast<float*>(op.p[5]), op.i[0], op.i[1], op.f[0], st);
         case PP_OP_LN_BWD_INPUT:
-            return pp_layernorm_bwd_input(op.p[0], op.p[1], op.p[2], static_cast<const float*>(op.p[3]),
-                                          static_cast<const float*>(op.p[4]), op.p[5], op.p[6], op.i[0],
-                                          op.i[1], st);
+            return pp_layernorm_bwd_input_sums(op.p[0], op.p[1], op.p[2], static_cast<const float*>(op.p[3]),
+                                               static_cast<const float*>(op.p[4]), op.p[5], op.p[6], op.i[0],
+                                               op.i[1], static_cast<float*>(op.p[7]), static_cast<float*>(op.p[8]),
+                                               st);
         case PP_OP_LN_BWD_WEIGHT:
+            if (op.j[1] > 0) {
+                const pp_colreduce_desc d = colreduce_desc_of(op);
+                return pp_colreduce_grouped(&d, 1, st);
+            }
             return pp_layernorm_bwd_weight(op.p[0], op.p[1], static_cast<const float*>(op.p[2]),
                                            static_cast<const float*>(op.p[3]), op.p[4], op.p[5], op.j[0],
                                            static_cast<float*>(op.p[6]), op.i[0], op.i[1], st);
@@ -229,10 +239,10 @@ double op_work(const pp_op& op) {
             return 4.0 * (double)op.i[0] * (double)op.i[1];  // read x, write y (bf16)
         case PP_OP_LN_BWD_INPUT:
             return (op.p[5] ? 8.0 : 6.0) * (double)op.i[0] * (double)op.i[1];
-        case PP_OP_LN_BWD_WEIGHT:
-            return 4.0 * (double)op.i[0] * (double)op.i[1];
+        case PP_OP_LN_BWD_WEIGHT:  // dy and x, or the partial sums that their producer left
+            return op.j[1] > 0 ? 8.0 * (double)op.j[1] * (double)op.i[1] : 4.0 * (double)op.i[0] * (double)op.i[1];
         case PP_OP_COLSUM:
-            return 2.0 * (double)op.i[0] * (double)op.i[1];
+            return op.j[1] > 0 ? 4.0 * (double)op.j[1] * (double)op.i[1] : 2.0 * (double)op.i[0] * (double)op.i[1];
         case PP_OP_CE_LOSS:  // read logits, write their gradient
             return (op.p[3] ? 2.0 : 1.0) * (double)op.i[0] * (double)op.i[2] * (op.j[0] == PP_F32 ? 4.0 : 2.0);
         case PP_OP_EMBED_FWD:

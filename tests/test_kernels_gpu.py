@@ -227,6 +227,43 @@ def test_gemm_bf16_epilogues(M, N, K):
     assert_close_rel(acc, lin, 1e-5, "accumulate init")
 
 
+@pytest.mark.parametrize("M,N,K,bt", [(4096, 3072, 264, False), (4096, 768, 136, False), (1000, 376, 136, False),
+                                       (384, 264, 136, True), (300, 3072, 72, False)])
+def test_gemm_activation_derivative_epilogue_leaves_the_column_sums(M, N, K, bt):
+    """With ``colsum`` the epilogue also writes, per band of 32 rows, the column sums of C as stored: C itself
+    is unchanged bit for bit, every band's sums are the fp32 sums of the stored bf16 values (at most one
+    rounding per addition apart from the ascending-order sum), and pp_colreduce_grouped forms from them the
+    bias gradient that the two-pass reduction of C gives.  Shapes cover 192-, 96- and 128-column tiles, ragged
+    edges in both directions and a transposed weight."""
+    Nn = native()
+    torch.manual_seed(51)
+    A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    W = (torch.randn(K, N, device=DEV) * 0.1).to(torch.bfloat16) if bt else \
+        (torch.randn(N, K, device=DEV) * 0.1).to(torch.bfloat16)
+    R = torch.randn(M, N, device=DEV).to(torch.bfloat16)
+    n_part = (M + Nn.GEMM_COLSUM_ROWS - 1) // Nn.GEMM_COLSUM_ROWS
+    for epi in (Nn.EPI_DGELU_TANH, Nn.EPI_DGELU_ERF, Nn.EPI_DRELU):
+        C0 = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+        C1 = torch.empty_like(C0)
+        part = torch.full((n_part, N), float("nan"), device=DEV)
+        Nn.gemm_bf16(A, W, C0, b_trans=bt, epilogue=epi, aux_in=R)
+        Nn.gemm_bf16(A, W, C1, b_trans=bt, epilogue=epi, aux_in=R, colsum=part)
+        assert torch.equal(C0, C1)
+        pad = torch.zeros(n_part * 32, N, device=DEV, dtype=torch.float64)
+        pad[:M] = C1.double()
+        bands = pad.view(n_part, 32, N)
+        exact = bands.sum(1)
+        assert not bool(torch.isnan(part).any())
+        assert (part.double() - exact).abs().max() <= 32 * 2.0 ** -24 * bands.abs().sum(1).max()
+        out, ref = torch.empty(N, device=DEV), torch.empty(N, device=DEV)
+        Nn.colreduce_grouped([dict(dy=C1, out_sum=out, workspace=part, n_part_ready=n_part)])
+        ws = torch.empty(2 * ((M + 127) // 128) * N, device=DEV)
+        Nn.colreduce_grouped([dict(dy=C1, out_sum=ref, workspace=ws)])
+        assert (out - ref).abs().max() <= 1e-6 * float(C1.float().abs().sum(0).max())
+    with pytest.raises(RuntimeError, match="column sums"):
+        Nn.gemm_bf16(A, W, C0, b_trans=bt, epilogue=Nn.EPI_NONE, colsum=part)
+
+
 @pytest.mark.parametrize("M,N,K,at,bt", [(768, 2304, 4096, True, True), (200, 136, 264, True, True),
                                           (50304, 768, 4096, True, True), (11008, 4096, 2048, True, True),
                                           (256, 96, 512, False, False), (4096, 768, 64, False, True)])
@@ -372,6 +409,65 @@ def test_layernorm(rows, C):
     Nn.layernorm_bwd_weight(dy, x, mean, rstd, dg16, db16, ws)
     assert_close_rel(dg16, gr.grad, BF16_TOL, "ln dgamma bf16")
     assert_close_rel(db16, br.grad, BF16_TOL, "ln dbeta bf16")
+
+
+@pytest.mark.parametrize("rows,C,rms", [(4096, 768, False), (1000, 768, False), (37, 64, False), (512, 1024, True),
+                                        (130, 1024, False)])
+def test_layernorm_input_gradient_that_leaves_the_column_sums(rows, C, rms):
+    """pp_layernorm_bwd_input_sums: the input gradient bit for bit as pp_layernorm_bwd_input writes it, and
+    the final sums that pp_colreduce_grouped forms from its partial sums against the definition (fp64) and
+    against the two-pass reductions, for LayerNorm and RMSNorm, with ragged last blocks of rows."""
+    Nn = native()
+    torch.manual_seed(81)
+    x = (torch.randn(rows, C, device=DEV) * 2 + 0.5).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(C, device=DEV)).to(torch.bfloat16)
+    dy = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+    dres = torch.randn(rows, C, device=DEV).to(torch.bfloat16)
+    y, rstd = torch.empty_like(x), torch.empty(rows, device=DEV)
+    mean = None if rms else torch.empty(rows, device=DEV)
+    Nn.layernorm_fwd(x, gamma, None, y, mean, rstd, 1e-5)
+    for res in (None, dres):
+        dx_ref, dx = torch.empty_like(x), torch.full_like(x, 7.0)
+        Nn.layernorm_bwd_input(dy, x, gamma, mean, rstd, res, dx_ref)
+        n_part = (rows + Nn.LN_SUM_ROWS - 1) // Nn.LN_SUM_ROWS
+        ws_w = torch.full((2 * n_part * C,), float("nan"), device=DEV)
+        ws_dx = torch.full((n_part * C,), float("nan"), device=DEV)
+        assert Nn.layernorm_bwd_input_sums(dy, x, gamma, mean, rstd, res, dx, ws_w, ws_dx) == n_part
+        assert torch.equal(dx, dx_ref)
+        # the final sums from the partial sums
+        dg, db, dbias = (torch.empty(C, device=DEV) for _ in range(3))
+        Nn.colreduce_grouped([
+            dict(dy=dy, out_sum=db, out_dot=dg, workspace=ws_w, n_part_ready=n_part),
+            dict(dy=dx, out_sum=dbias, workspace=ws_dx, n_part_ready=n_part)])
+        xh = (x.double() - (0 if rms else mean.double()[:, None])) * rstd.double()[:, None]
+        scale = float(rows) ** 0.5
+        assert (dg.double() - (dy.double() * xh).sum(0)).abs().max() <= 1e-5 * scale * 8
+        assert (db.double() - dy.double().sum(0)).abs().max() <= 1e-5 * scale * 8
+        assert (dbias.double() - dx.double().sum(0)).abs().max() <= 1e-5 * scale * 8
+        # and the two-pass reductions over the same tensors: the same sums up to fp32 summation order
+        ws2 = torch.empty(2 * ((rows + 127) // 128) * C, device=DEV)
+        dg2, db2, dbias2 = (torch.empty(C, device=DEV) for _ in range(3))
+        Nn.colreduce_grouped([dict(dy=dy, x=x, mean=mean, rstd=rstd, out_sum=db2, out_dot=dg2, workspace=ws2)])
+        Nn.colreduce_grouped([dict(dy=dx, out_sum=dbias2, workspace=ws2)])
+        for a, b_ in ((dg, dg2), (db, db2), (dbias, dbias2)):
+            assert (a - b_).abs().max() <= 1e-5 * scale * 8
+    # only one of the two kinds of sums asked for; bf16 results
+    ws_dx = torch.empty(n_part * C, device=DEV)
+    dx2 = torch.empty_like(x)
+    Nn.layernorm_bwd_input_sums(dy, x, gamma, mean, rstd, dres, dx2, None, ws_dx)
+    assert torch.equal(dx2, dx_ref)
+    b16 = torch.empty(C, device=DEV, dtype=torch.bfloat16)
+    Nn.colreduce_grouped([dict(dy=dx2, out_sum=b16, workspace=ws_dx, n_part_ready=n_part)])
+    assert torch.equal(b16, dbias.to(torch.bfloat16))
+
+
+def test_layernorm_input_gradient_sums_reject_a_wide_row():
+    Nn = native()
+    C = Nn.LN_SUM_MAX_C + 8
+    x = torch.zeros(16, C, device=DEV, dtype=torch.bfloat16)
+    ws = torch.empty(2 * C, device=DEV)
+    with pytest.raises(RuntimeError, match="exceeds"):
+        Nn.layernorm_bwd_input_sums(x, x, x[0], None, torch.ones(16, device=DEV), None, torch.empty_like(x), ws, None)
 
 
 # ---- embedding / loss ----------------------------------------------------------------------------
