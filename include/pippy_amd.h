@@ -443,9 +443,11 @@ int pp_position_ids_from_padding(const int64_t* ids, int64_t* out, int64_t n_seq
  *   d_wte[v, :] += g[v, :],  g[v, :] = sum of dy[t, :] over the tokens t with ids[t] == v, formed in
  *   fp32 in ascending t;  d_wpe[p, :] += sum over the batch of dy[b * seq + p, :] in ascending b.
  * round_bf16 != 0 rounds g to bf16 before it is added: bit for bit what a bf16 gradient tensor folded
- * in by pp_grad_accum_f32_bf16 leaves.  No atomics: results do not depend on scheduling.  C <= 8192. */
+ * in by pp_grad_accum_f32_bf16 leaves.  No atomics: results do not depend on scheduling.  C <= 8192.
+ * padding_idx >= 0: row padding_idx of d_wte is left untouched (nn.Embedding(padding_idx=...) gives that row
+ * no gradient) and its tokens are not summed; negative: no such row. */
 int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe, int64_t n_tok,
-                 int64_t seq, int64_t C, int64_t vocab, int round_bf16, pp_stream stream);
+                 int64_t seq, int64_t C, int64_t vocab, int round_bf16, int64_t padding_idx, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
  * Cross-entropy loss of one microbatch (loss_fn at pippy/PipelineSchedule.py:154-155 when it is
@@ -491,7 +493,7 @@ enum pp_op_kind {
  *   EMBED_FWD     p: ids wte wpe y extra_row pos_ids | i: n_tok seq C vocab n_pos  (pos_ids non-null:
  *                 pp_embed_fwd_at)
  *   POSITION_IDS  p: ids out | i: n_seq seq pad
- *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab | j: round_bf16
+ *   EMBED_BWD     p: ids dy d_wte d_wpe | i: n_tok seq C vocab padding_idx+1 (0: none) | j: round_bf16
  *   CE_LOSS       p: logits target loss dlogits workspace | i: rows V ld ignore_index | j: dtype
  *   ACCUM_*       p: acc g | i: n | j: init
  *   COPY_ROWS     p: src dst | i: n_rows row_bytes src_stride dst_stride

@@ -132,7 +132,7 @@ def lib() -> C.CDLL:
         "pp_attn_fwd": [C.POINTER(AttnDesc), vp],
         "pp_attn_bwd": [C.POINTER(AttnDesc), vp],
         "pp_embed_fwd": [vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
-        "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
+        "pp_embed_bwd": [vp, vp, vp, vp, i64, i64, i64, i64, i32, i64, vp],
         "pp_embed_fwd_at": [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp],
         "pp_position_ids_from_padding": [vp, vp, i64, i64, i64, vp],
         "pp_ce_loss": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp],
@@ -715,11 +715,13 @@ def position_ids_from_padding(ids, out, pad: int) -> None:
                                              current_stream()), "pp_position_ids_from_padding")
 
 
-def embed_bwd(ids, dy, d_wte, d_wpe, seq: int, round_bf16: bool = False) -> None:
+def embed_bwd(ids, dy, d_wte, d_wpe, seq: int, round_bf16: bool = False, padding_idx: Optional[int] = None) -> None:
+    """``padding_idx``: the row of ``d_wte`` that receives no gradient (its tokens are skipped)."""
     require_cuda(ids, dy, d_wte, d_wpe)
     vocab, Cc = d_wte.shape
+    pad = -1 if padding_idx is None else padding_idx % vocab
     check(lib().pp_embed_bwd(ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), ptr(d_wpe),
-                             ids.numel(), seq, Cc, vocab, int(round_bf16), current_stream()), "pp_embed_bwd")
+                             ids.numel(), seq, Cc, vocab, int(round_bf16), pad, current_stream()), "pp_embed_bwd")
 
 
 def ce_loss(logits, target, loss, dlogits, workspace, V: int, ignore_index: int = -100) -> None:

@@ -531,15 +531,17 @@ def op_position_ids(ids, out, pad: int) -> N.Op:
     return op
 
 
-def op_embed_bwd(ids, dy, d_wte, d_wpe, seq, round_bf16=False) -> N.Op:
+def op_embed_bwd(ids, dy, d_wte, d_wpe, seq, round_bf16=False, padding_idx=None) -> N.Op:
     """``round_bf16``: the per-microbatch row sums are rounded to bf16 before they are added (the bits
-    of a bf16 gradient tensor folded into the fp32 accumulator)."""
+    of a bf16 gradient tensor folded into the fp32 accumulator).  ``padding_idx``: the row of ``d_wte``
+    that gets no gradient, as ``nn.Embedding(padding_idx=...)`` has it."""
     vocab, Cc = d_wte.shape
     assert d_wte.dtype == torch.float32 and dy.shape == (ids.numel(), Cc) and dy.is_contiguous()
     op = N.Op()
     op.kind = N.OP_EMBED_BWD
     op.p[0], op.p[1], op.p[2], op.p[3] = ids.data_ptr(), dy.data_ptr(), d_wte.data_ptr(), _p(d_wpe)
     op.i[0], op.i[1], op.i[2], op.i[3] = ids.numel(), seq, Cc, vocab
+    op.i[4] = 0 if padding_idx is None else padding_idx % vocab + 1
     op.j[0] = int(round_bf16)
     return op
 

@@ -58,12 +58,15 @@ template <int NW>
 __global__ __launch_bounds__(256) void embed_bwd_wte_kernel(const int64_t* __restrict__ ids,
                                                             const uint16_t* __restrict__ dy,
                                                             float* __restrict__ d_wte, int64_t n_tok,
-                                                            int C, int64_t vocab, int round_bf16) {
+                                                            int C, int64_t vocab, int round_bf16,
+                                                            int64_t skip_id) {
     const int lane = threadIdx.x & 63;
     const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tok) return;
     const int64_t id = ids[t];
-    if (id < 0 || id >= vocab) return;
+    // the padding row gets no gradient: its occurrences (often most of a padded batch, all owned by one
+    // wave) are not summed at all
+    if (id < 0 || id >= vocab || id == skip_id) return;
     const int half_c = C >> 1;
     float lo[NW], hi[NW];
 #pragma unroll
@@ -154,9 +157,9 @@ __global__ __launch_bounds__(64) void position_ids_kernel(const int64_t* __restr
 
 template <int NW>
 static void launch_embed_bwd_wte(const int64_t* ids, const void* dy, float* d_wte, int64_t n_tok, int C,
-                                 int64_t vocab, int round_bf16, hipStream_t st) {
+                                 int64_t vocab, int round_bf16, int64_t skip_id, hipStream_t st) {
     hipLaunchKernelGGL(embed_bwd_wte_kernel<NW>, dim3((uint32_t)((n_tok + 3) / 4)), dim3(256), 0, st, ids,
-                       (const uint16_t*)dy, d_wte, n_tok, C, vocab, round_bf16);
+                       (const uint16_t*)dy, d_wte, n_tok, C, vocab, round_bf16, skip_id);
 }
 
 }  // namespace pp
@@ -206,7 +209,7 @@ extern "C" int pp_position_ids_from_padding(const int64_t* ids, int64_t* out, in
 
 extern "C" int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, float* d_wpe,
                             int64_t n_tok, int64_t seq, int64_t C, int64_t vocab, int round_bf16,
-                            pp_stream stream) {
+                            int64_t padding_idx, pp_stream stream) {
     if (n_tok < 0 || seq <= 0 || C <= 0 || vocab <= 0) return fail(PP_ERR_INVALID, "pp_embed_bwd: bad shape");
     if (C % 2) return fail(PP_ERR_UNSUPPORTED, "pp_embed_bwd: C %% 2 != 0");
     if (C > 8192) return fail(PP_ERR_UNSUPPORTED, "pp_embed_bwd: C > 8192");
@@ -215,11 +218,11 @@ extern "C" int pp_embed_bwd(const int64_t* ids, const void* dy, float* d_wte, fl
     if (!aligned(dy, 4) || !aligned(d_wte, 8)) return fail(PP_ERR_INVALID, "pp_embed_bwd: misaligned pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int words = (int)((C / 2 + 63) / 64);
-    if (words <= 2) launch_embed_bwd_wte<2>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
-    else if (words <= 8) launch_embed_bwd_wte<8>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
-    else if (words <= 16) launch_embed_bwd_wte<16>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
-    else if (words <= 32) launch_embed_bwd_wte<32>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
-    else launch_embed_bwd_wte<64>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, st);
+    if (words <= 2) launch_embed_bwd_wte<2>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, padding_idx, st);
+    else if (words <= 8) launch_embed_bwd_wte<8>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, padding_idx, st);
+    else if (words <= 16) launch_embed_bwd_wte<16>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, padding_idx, st);
+    else if (words <= 32) launch_embed_bwd_wte<32>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, padding_idx, st);
+    else launch_embed_bwd_wte<64>(ids, dy, d_wte, n_tok, (int)C, vocab, round_bf16, padding_idx, st);
     if (d_wpe) {
         const int64_t work = seq * (C / 2);
         hipLaunchKernelGGL(embed_bwd_wpe_kernel, dim3((uint32_t)((work + 255) / 256)), dim3(256), 0, st,

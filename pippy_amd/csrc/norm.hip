@@ -453,11 +453,15 @@ __global__ __launch_bounds__(256) void colgroup_final_kernel(const ColGroupArgs 
             const float* part = d.ws + (int64_t)pass * d.n_part * d.C + c;
             float t = 0.f;
             if (c < d.C) {
+                // 16 loads in flight per lane (a loop of load-then-add pays one memory latency per term); the
+                // additions stay a chain in ascending row order
                 int p = rp;
-                for (; p + 24 < d.n_part; p += 32) {
-                    const float v0 = part[(int64_t)p * d.C], v1 = part[(int64_t)(p + 8) * d.C],
-                                v2 = part[(int64_t)(p + 16) * d.C], v3 = part[(int64_t)(p + 24) * d.C];
-                    t += v0; t += v1; t += v2; t += v3;
+                for (; p + 8 * 15 < d.n_part; p += 8 * 16) {
+                    float v[16];
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) v[k] = part[(int64_t)(p + 8 * k) * d.C];
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) t += v[k];
                 }
                 for (; p < d.n_part; p += 8) t += part[(int64_t)p * d.C];
             }

@@ -127,7 +127,8 @@ static int run_one(const pp_op& op, pp_stream st) {
                                 op.i[1], op.i[2], op.i[3], st);
         case PP_OP_EMBED_BWD:
             return pp_embed_bwd(static_cast<const int64_t*>(op.p[0]), op.p[1], static_cast<float*>(op.p[2]),
-                                static_cast<float*>(op.p[3]), op.i[0], op.i[1], op.i[2], op.i[3], op.j[0], st);
+                                static_cast<float*>(op.p[3]), op.i[0], op.i[1], op.i[2], op.i[3], op.j[0],
+                                op.i[4] - 1, st);
         case PP_OP_CE_LOSS:
             return pp_ce_loss(op.p[0], static_cast<const int64_t*>(op.p[1]), static_cast<float*>(op.p[2]),
                               op.p[3], static_cast<float*>(op.p[4]), op.i[0], op.i[1], op.i[2], op.i[3],

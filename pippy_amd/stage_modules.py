@@ -298,12 +298,10 @@ class LayerNormBlock(NativeBlock):
         return y.view(x.shape)
 
 
-def _zero_padding_row(b: "P.Builder", table: nn.Embedding, acc: torch.Tensor):
-    """``nn.Embedding(padding_idx=i)`` gives row i no gradient: the row of the accumulator that the
-    embedding backward has just added to is cleared again."""
-    pad = getattr(table, "padding_idx", None)
-    if pad is not None:
-        b.w(P.op_fill(acc[pad % acc.shape[0]]))
+def _padding_idx(table: nn.Embedding) -> Optional[int]:
+    """``nn.Embedding(padding_idx=i)`` gives row i no gradient: the embedding backward leaves that row of the
+    accumulator (zero since the accumulation started) alone."""
+    return getattr(table, "padding_idx", None)
 
 
 class TokenEmbedding(NativeBlock):
@@ -356,8 +354,7 @@ class TokenEmbedding(NativeBlock):
             if acc_wpe is not None:
                 b.w(P.op_fill(acc_wpe), tag="fill")
             b.w(P.op_embed_bwd(ids, dy.view(Bn * S, Cc), acc_wte, acc_wpe[first:] if acc_wpe is not None else None,
-                               S, round_bf16=not b.fused_accumulate))
-            _zero_padding_row(b, self.wte, acc_wte)
+                               S, round_bf16=not b.fused_accumulate, padding_idx=_padding_idx(self.wte)))
             return None
 
         b.on_backward(bwd)
@@ -435,13 +432,13 @@ class EncoderEmbedding(NativeBlock):
             acc_wpe = b.grad_acc(self.position_embeddings.weight)
             b.w(P.op_fill(acc_wte), tag="fill")
             b.w(P.op_fill(acc_wpe), tag="fill")
+            pad_w = _padding_idx(self.word_embeddings)
             if pos_ids is None:
-                b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate))
+                b.w(P.op_embed_bwd(ids, de, acc_wte, acc_wpe, S, round_bf16=not b.fused_accumulate, padding_idx=pad_w))
             else:   # the position table is one more table read at computed indices
-                b.w(P.op_embed_bwd(ids, de, acc_wte, None, S, round_bf16=not b.fused_accumulate))
-                b.w(P.op_embed_bwd(pos_ids.view(-1), de, acc_wpe, None, S, round_bf16=not b.fused_accumulate))
-                _zero_padding_row(b, self.position_embeddings, acc_wpe)
-            _zero_padding_row(b, self.word_embeddings, acc_wte)
+                b.w(P.op_embed_bwd(ids, de, acc_wte, None, S, round_bf16=not b.fused_accumulate, padding_idx=pad_w))
+                b.w(P.op_embed_bwd(pos_ids.view(-1), de, acc_wpe, None, S, round_bf16=not b.fused_accumulate,
+                                   padding_idx=_padding_idx(self.position_embeddings)))
             if wtt is not None:
                 # the type-0 row receives the gradient of every token; the other rows none
                 g_tt = b.grad_target(self.token_type_embeddings.weight)

@@ -560,6 +560,28 @@ def test_embedding_backward_is_ordered_and_bit_exact(C, vocab, n_tok, seq, round
         assert torch.equal(d_wpe.cpu(), start_p), f"d_wpe, call {call}"
 
 
+def test_embedding_backward_leaves_the_padding_row_alone():
+    """``padding_idx``: that row of the table's gradient keeps what it held (here a marker value), however
+    many padding tokens the batch has (most of it here), negative indices count from the end of the table
+    as in ``nn.Embedding``, and every other row is what the call without a padding row leaves."""
+    Nn = native()
+    g = torch.Generator().manual_seed(12)
+    vocab, C, seq, n_tok = 50, 64, 32, 512
+    ids = torch.randint(0, vocab, (n_tok,), generator=g)
+    pad = 1
+    ids[torch.rand(n_tok, generator=g) < 0.7] = pad
+    dy = torch.randn(n_tok, C, generator=g).to(torch.bfloat16)
+    for given in (pad, pad - vocab):
+        ref = torch.zeros(vocab, C, device=DEV)
+        got = torch.zeros(vocab, C, device=DEV)
+        got[pad] = 5.0
+        Nn.embed_bwd(ids.to(DEV), dy.to(DEV), ref, None, seq)
+        Nn.embed_bwd(ids.to(DEV), dy.to(DEV), got, None, seq, padding_idx=given)
+        assert bool((got[pad] == 5.0).all())
+        keep = torch.arange(vocab) != pad
+        assert torch.equal(got[keep], ref[keep])
+
+
 def test_embedding_and_layernorm_full_size_closed_forms():
     """The embedding and LayerNorm shapes of the GPT-2-small stage (4096 tokens, width 768, 50257
     tokens in the table).  A zero position table makes the embedding an exact gather; rows of the
