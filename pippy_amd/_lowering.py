@@ -1156,5 +1156,15 @@ def lower_stage_module(submod: nn.Module, why: Optional[List[str]] = None, for_k
         return blocks
     except NotLowerable as e:
         if why is not None:
-            why.append(str(e))
+            reason = str(e)
+            # the most common cause, and one that the structural messages do not name: a dropout that does
+            # something keeps its residual branch from being recognised
+            live = [n for n, m in submod.named_modules()
+                    if (isinstance(m, nn.modules.dropout._DropoutNd) and m.p > 0 and m.training)
+                    or (isinstance(m, nn.MultiheadAttention) and m.dropout > 0 and m.training)]
+            if live and "dropout" not in reason:
+                shown = ", ".join(live[:3]) + (", ..." if len(live) > 3 else "")
+                reason = (f"dropout with p > 0 in training mode ({shown}): the launch lists hold no dropout; "
+                          f"set p = 0 or build the stage in eval mode.  The recogniser says: {reason}")
+            why.append(reason)
         return None

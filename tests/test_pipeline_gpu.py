@@ -1026,6 +1026,46 @@ def test_plain_torch_gpt_runs_natively_and_matches_the_oracle():
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
 
 
+def test_a_stage_lowered_in_eval_mode_refuses_to_train_with_its_dropout_switched_on():
+    """Dropout with p > 0 is identity in eval mode, so a model built that way lowers to launch lists — which
+    hold no dropout.  Put into training mode afterwards the stage must raise rather than train without
+    dropout; back in eval mode it runs again, with the same result as before."""
+    import sys, os
+    import torch.nn as nn
+    sys.path.insert(0, os.path.dirname(__file__))
+    from _plain_gpt import GPT
+    import pippy_amd as pp
+    torch.manual_seed(0)
+    M, vocab, seq = 2, 1000, 64
+    model = GPT(vocab=vocab, seq=seq, d=128, h=2, L=2).to(torch.bfloat16)
+    for m in model.modules():
+        if isinstance(m, nn.Dropout):
+            m.p = 0.1
+    model.eval()
+    ids = torch.randint(0, vocab, (2 * M, seq))
+    pipe = pp.pipeline(model, M, (ids,), split_spec={"h.1": pp.SplitPoint.BEGINNING})
+    stages = [pp.PipelineStage(pipe, i, DEV) for i in range(2)]
+    assert all(st.is_native for st in stages), [st.eager_reason for st in stages]
+    sched = pp.ScheduleGPipe(stages, M)
+    first = sched.step(ids.to(DEV)).clone()
+    for st in stages:
+        st.submod.train()
+    with pytest.raises(RuntimeError, match="dropout"):
+        sched.step(ids.to(DEV))
+    for st in stages:
+        st.submod.eval()
+    assert torch.equal(sched.step(ids.to(DEV)), first)
+    # the other direction: built in training mode with p > 0, the stages stay with torch autograd and say why
+    model2 = GPT(vocab=vocab, seq=seq, d=128, h=2, L=2).to(torch.bfloat16)
+    for m in model2.modules():
+        if isinstance(m, nn.Dropout):
+            m.p = 0.1
+    model2.train()
+    pipe2 = pp.pipeline(model2, M, (ids,), split_spec={"h.1": pp.SplitPoint.BEGINNING})
+    st2 = pp.PipelineStage(pipe2, 0, DEV)
+    assert not st2.is_native and "dropout" in st2.eager_reason
+
+
 def _exported_model_against_the_oracle(model, whole, vocab, seq, split, before_oracle=None, padding=None):
     """Pipelines ``model`` (which torch.fx cannot trace: the front end exports it on one microbatch) in
     two stages, checks that both run as launch lists, and compares logits, losses and every parameter
