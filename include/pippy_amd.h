@@ -407,6 +407,13 @@ typedef struct pp_attn_desc {
     int32_t kv_group;      /* query heads per key / value head; 0 or 1: multi-head attention */
     int32_t kv_len;        /* 0: every key exists; L in 1..S: keys L..S-1 of each sequence are padding */
     int32_t flags;         /* PP_ATTN_* bits */
+    float* colsum;         /* backward, head_dim 64, or null: fp32 [B * S / 64, ld_colsum]; row b * (S / 64) + j
+                              receives the sums over the 64 tokens of block j of every column of dq, dk and dv
+                              as stored, at the column that the element has relative to dq (dq, dk, dv are then
+                              sections of one row of a fused projection's gradient, dq first): the partial sums
+                              of that projection's bias gradient, for pp_colreduce_grouped with
+                              n_part_ready = B * S / 64 */
+    int64_t ld_colsum;     /* row length of colsum, in floats */
 } pp_attn_desc;
 /* Backward: correct dq for the rounding of the forward's output.  The backward starts from
  * delta = rowsum(dO * O) of the bf16 output; the sum of P * dP over the keys is the same number in exact
@@ -488,7 +495,7 @@ enum pp_op_kind {
  *                 ws_dx: pp_layernorm_bwd_input_sums)
  *   LN_BWD_WEIGHT p: dy x mean rstd dgamma dbeta workspace | i: rows C | j: out_dtype n_part_ready
  *                 (n_part_ready > 0, here and for COLSUM: the op runs through pp_colreduce_grouped)
- *   ATTN_*        p: q k v o lse d_o dq dk dv delta | i: B S H D stride_b stride_s | f: scale
+ *   ATTN_*        p: q k v o lse d_o dq dk dv delta colsum | i: B S H D stride_b stride_s ld_colsum | f: scale
  *                 | j: causal kv_group kv_len flags
  *   EMBED_FWD     p: ids wte wpe y extra_row pos_ids | i: n_tok seq C vocab n_pos  (pos_ids non-null:
  *                 pp_embed_fwd_at)
@@ -525,7 +532,7 @@ enum pp_op_kind {
 typedef struct pp_op {
     int32_t kind;   /* enum pp_op_kind */
     int32_t flags;
-    void* p[10];
+    void* p[12];
     int64_t i[12];
     float f[2];
     int32_t j[6];

@@ -80,11 +80,11 @@ class AttnDesc(C.Structure):
                 ("B", C.c_int64), ("S", C.c_int64), ("H", C.c_int64), ("D", C.c_int64),
                 ("stride_b", C.c_int64), ("stride_s", C.c_int64),
                 ("scale", C.c_float), ("causal", C.c_int32), ("kv_group", C.c_int32), ("kv_len", C.c_int32),
-                ("flags", C.c_int32)]
+                ("flags", C.c_int32), ("colsum", C.c_void_p), ("ld_colsum", C.c_int64)]
 
 
 class Op(C.Structure):
-    _fields_ = [("kind", C.c_int32), ("flags", C.c_int32), ("p", C.c_void_p * 10),
+    _fields_ = [("kind", C.c_int32), ("flags", C.c_int32), ("p", C.c_void_p * 12),
                 ("i", C.c_int64 * 12), ("f", C.c_float * 2), ("j", C.c_int32 * 6)]
 
 
@@ -637,11 +637,14 @@ def layernorm_bwd_weight(dy, x, mean, rstd, dgamma, dbeta, workspace) -> None:
 def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, causal: bool,
               scale: Optional[float] = None, d_o: Optional[torch.Tensor] = None,
               dqkv: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
-              n_kv_heads: Optional[int] = None, kv_len: Optional[int] = None, exact_dq: bool = False) -> AttnDesc:
+              n_kv_heads: Optional[int] = None, kv_len: Optional[int] = None, exact_dq: bool = False,
+              colsum: Optional[torch.Tensor] = None) -> AttnDesc:
     """qkv: [B, S, (H + 2 H_kv) * D] fused projection output (q | k | v along the last dim);
     ``n_kv_heads`` < H: grouped-query attention (H / n_kv_heads query heads per key / value head);
     ``kv_len`` < S: rows kv_len .. S-1 of every sequence are (zero) padding that the forward masks;
-    ``exact_dq``: the backward corrects dq for the rounding of the forward's output (PP_ATTN_EXACT_DQ)."""
+    ``exact_dq``: the backward corrects dq for the rounding of the forward's output (PP_ATTN_EXACT_DQ);
+    ``colsum`` (backward, head size 64): fp32 [B * S / 64, width], receives the column sums of every block of
+    64 tokens of dqkv as stored."""
     require_cuda(qkv, o, lse, d_o, dqkv, delta)
     B, S, width = qkv.shape
     Hkv = H if n_kv_heads is None else n_kv_heads
@@ -669,6 +672,10 @@ def attn_desc(qkv: torch.Tensor, o: torch.Tensor, lse: torch.Tensor, H: int, cau
         d.d_o = d_o.data_ptr()
         d.dq, d.dk, d.dv = gb, gb + HD * es, gb + (HD + KD) * es
         d.delta = delta.data_ptr()
+        if colsum is not None:
+            require_cuda(colsum)
+            assert colsum.dtype == torch.float32 and colsum.is_contiguous() and colsum.shape == (B * S // 64, width)
+            d.colsum, d.ld_colsum = colsum.data_ptr(), width
     return d
 
 
@@ -678,9 +685,9 @@ def attn_fwd(qkv, o, lse, H, causal, scale=None, n_kv_heads=None, kv_len=None) -
 
 
 def attn_bwd(qkv, o, lse, d_o, dqkv, delta, H, causal, scale=None, n_kv_heads=None, kv_len=None,
-             exact_dq=False) -> None:
+             exact_dq=False, colsum=None) -> None:
     d = attn_desc(qkv, o, lse, H, causal, scale, d_o=d_o, dqkv=dqkv, delta=delta, n_kv_heads=n_kv_heads,
-                  kv_len=kv_len, exact_dq=exact_dq)
+                  kv_len=kv_len, exact_dq=exact_dq, colsum=colsum)
     check(lib().pp_attn_bwd(C.byref(d), current_stream()), "pp_attn_bwd")
 
 

@@ -633,7 +633,7 @@ class OpList:
             self.freeze()
         hits = []
         for k in range(self.n):
-            for q in range(10):
+            for q in range(12):
                 if self._arr[k].p[q] == ptr:
                     hits.append((k, q))
         return hits
@@ -817,7 +817,9 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
       gradient of the residual stream, which is the output gradient of the linear layer in front of the
       norm) takes the sums of ``dx`` from that op;
     * a bias-gradient column sum over the output of a GEMM with an activation-derivative epilogue (the
-      gradient in front of a GELU or ReLU) takes them from that GEMM's epilogue.
+      gradient in front of a GELU or ReLU) takes them from that GEMM's epilogue;
+    * the bias gradient of a fused q | k | v projection takes them from the attention backward kernels (head
+      size 64), which write that projection's output gradient.
 
     Only exact matches are rewired: same pointers, same shape, a contiguous tensor, and no other op of the I
     pass writing to the same address."""
@@ -827,11 +829,12 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
     ln_ops = [op for op in I if op.kind == N.OP_LN_BWD_INPUT and 0 < op.i[1] <= N.LN_SUM_MAX_C]
     act_ops = [op for op in I if op.kind == N.OP_GEMM_BF16 and op.j[3] == N.PP_BF16 and not op.p[8]
                and op.j[2] in (N.EPI_DGELU_ERF, N.EPI_DGELU_TANH, N.EPI_DRELU)]
-    if not ln_ops and not act_ops:
+    attn_ops = [op for op in I if op.kind == N.OP_ATTN_BWD and op.i[3] == 64 and not op.p[10]]
+    if not ln_ops and not act_ops and not attn_ops:
         return
     written: Dict[int, int] = {}
     for op in I:
-        for q in _WRITTEN_FIELDS.get(op.kind, range(10)):
+        for q in _WRITTEN_FIELDS.get(op.kind, range(12)):
             if op.p[q]:
                 written[op.p[q]] = written.get(op.p[q], 0) + 1
     for k, (op, _tag) in enumerate(b._w_reduce):
@@ -865,6 +868,20 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
                 n_part = (rows + N.GEMM_COLSUM_ROWS - 1) // N.GEMM_COLSUM_ROWS
                 ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
                 src[0].p[9] = ws.data_ptr()
+                op.p[2], op.j[1] = ws.data_ptr(), n_part
+                continue
+            # the gradient of a fused q | k | v projection, written by the attention backward: dq at the head
+            # of every row, dk and dv behind it, the rows of all sequences back to back
+            def fused(a):
+                Bn, S, H, D, sb, ss = (a.i[q] for q in range(6))
+                Hkv = H // max(a.j[1], 1)
+                return (a.p[6] == op.p[0] and a.p[7] == a.p[6] + 2 * H * D and a.p[8] == a.p[7] + 2 * Hkv * D
+                        and Cc == (H + 2 * Hkv) * D and ss == ld and sb == S * ss and rows == Bn * S)
+            src = [a for a in attn_ops if fused(a)]
+            if len(src) == 1 and written.get(src[0].p[7], 0) == 1 and written.get(src[0].p[8], 0) == 1:
+                n_part = rows // 64
+                ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
+                src[0].p[10], src[0].i[6] = ws.data_ptr(), Cc
                 op.p[2], op.j[1] = ws.data_ptr(), n_part
 
 

@@ -39,7 +39,27 @@ struct AttnArgs {
     int64_t G;  // query heads per key / value head (1: multi-head attention)
     int64_t L;  // keys 0 .. L-1 of a sequence exist (L <= S); the forward masks the rest
     float scale;
+    // backward, head dimension 64: fp32 [B * S / 64][ld_cs], row b * (S / 64) + j receives the column sums
+    // over block j (64 tokens) of dq, dk and dv as stored, at the columns that the elements have relative
+    // to dq (cs_k, cs_v: where the dk and dv sections start); null: no sums
+    float* colsum;
+    int64_t ld_cs, cs_k, cs_v;
 };
+
+// Column sums of a 64 x 64 block that its owners have written to `cs` as [column][65] floats (row = token
+// within the block): every wave adds 16 rows of each column in ascending order, wave 0 then adds the four
+// partial sums in wave order and writes the 64 sums.  Called by all 256 threads of the work-group.
+constexpr int kColsumScratchFloats = 64 * 65 + 4 * 64;
+__device__ __forceinline__ void attn_block_column_sums(float* cs, int tid, float* out) {
+    const int c = tid & 63, rq = tid >> 6;
+    float t = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t += cs[c * 65 + rq * 16 + r];
+    float* part = cs + 64 * 65;
+    part[rq * 64 + c] = t;
+    __syncthreads();
+    if (rq == 0) out[c] = ((part[c] + part[64 + c]) + part[128 + c]) + part[192 + c];
+}
 
 union Frag {
     uint4 u;
@@ -540,22 +560,46 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
         }
         __syncthreads();
     }
-    if (half != 0) return;
     // dvacc[dt][v]: d = 32 dt + 8 (v/4) + 4 lh + v%4, kv = kvi
-    uint16_t* dkp = a.dk + b * a.stride_b + hk * D + kvi * a.stride_s;
-    uint16_t* dvp = a.dv + b * a.stride_b + hk * D + kvi * a.stride_s;
+    bool sums = false;
+    if constexpr (D == 64) sums = a.colsum != nullptr;  // uniform over the grid
+    if (half != 0 && !sums) return;
+    float* cs = reinterpret_cast<float*>(lds) + 2 * (16 * DT * 64);  // behind the exchange buffers above
+    const int row = 32 * grp + l32;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int pass = 0; pass < 2; ++pass) {
+        if (half == 0) {
+            f32x16_t(&acc)[DT] = pass == 0 ? dvacc : dkacc;
+            uint16_t* outp = (pass == 0 ? a.dv : a.dk) + b * a.stride_b + hk * D + kvi * a.stride_s;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int d = 32 * dt + 8 * g + 4 * lh;
-            *reinterpret_cast<uint2*>(dvp + d) =
-                make_uint2(pack_bf16(dvacc[dt][4 * g + 0], dvacc[dt][4 * g + 1]),
-                           pack_bf16(dvacc[dt][4 * g + 2], dvacc[dt][4 * g + 3]));
-            *reinterpret_cast<uint2*>(dkp + d) =
-                make_uint2(pack_bf16(dkacc[dt][4 * g + 0] * a.scale, dkacc[dt][4 * g + 1] * a.scale),
-                           pack_bf16(dkacc[dt][4 * g + 2] * a.scale, dkacc[dt][4 * g + 3] * a.scale));
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = 32 * dt + 8 * g + 4 * lh;
+                    float v[4] = {acc[dt][4 * g + 0], acc[dt][4 * g + 1], acc[dt][4 * g + 2], acc[dt][4 * g + 3]};
+                    if (pass == 1) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] *= a.scale;
+                    }
+                    const uint32_t w0 = pack_bf16(v[0], v[1]), w1 = pack_bf16(v[2], v[3]);
+                    *reinterpret_cast<uint2*>(outp + d) = make_uint2(w0, w1);
+                    if constexpr (D == 64) {
+                        if (sums) {
+                            cs[(d + 0) * 65 + row] = bf16lo(w0); cs[(d + 1) * 65 + row] = bf16hi(w0);
+                            cs[(d + 2) * 65 + row] = bf16lo(w1); cs[(d + 3) * 65 + row] = bf16hi(w1);
+                        }
+                    }
+                }
         }
+        if constexpr (D == 64) {
+            if (sums) {
+                __syncthreads();
+                attn_block_column_sums(cs, tid, a.colsum + (b * (a.S / 64) + kv0 / 64) * a.ld_cs +
+                                                    (pass == 0 ? a.cs_v : a.cs_k) + hk * D);
+                __syncthreads();
+            }
+        }
+    }
 }
 
 // ---- backward: dQ (parallel over query blocks) ---------------------------------------------------
@@ -718,27 +762,45 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : (EXACT ? 1 : 2)) void attn_bwd_d
         xs[(kMergeVals - 1) * 64] = d_consistent;
     }
     __syncthreads();
-    if (half != 0) return;
-    d_consistent += xs[(kMergeVals - 1) * 64];
-    if (lh == 0) a.delta[(b * a.H + h) * a.S + qi] = d_consistent;
-    const float r = d_consistent - delta_q;
+    bool sums = false;
+    if constexpr (D == 64) sums = a.colsum != nullptr;  // uniform over the grid
+    if (half != 0 && !sums) return;
+    float* cs = reinterpret_cast<float*>(lds) + 2 * (kMergeVals * 64);  // behind the exchange buffers
+    if (half == 0) {
+        d_consistent += xs[(kMergeVals - 1) * 64];
+        if (lh == 0) a.delta[(b * a.H + h) * a.S + qi] = d_consistent;
+        const float r = d_consistent - delta_q;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            dqacc[dt][e] += xs[(16 * dt + e) * 64];
-            if constexpr (EXACT) dqacc[dt][e] -= r * (pkacc[dt][e] + xs[(16 * DT + 16 * dt + e) * 64]);
+            for (int e = 0; e < 16; ++e) {
+                dqacc[dt][e] += xs[(16 * dt + e) * 64];
+                if constexpr (EXACT) dqacc[dt][e] -= r * (pkacc[dt][e] + xs[(16 * DT + 16 * dt + e) * 64]);
+            }
+        uint16_t* dqp = a.dq + b * a.stride_b + h * D + qi * a.stride_s;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * dt + 8 * g + 4 * lh;
+                const uint32_t w0 = pack_bf16(dqacc[dt][4 * g + 0] * a.scale, dqacc[dt][4 * g + 1] * a.scale);
+                const uint32_t w1 = pack_bf16(dqacc[dt][4 * g + 2] * a.scale, dqacc[dt][4 * g + 3] * a.scale);
+                *reinterpret_cast<uint2*>(dqp + d) = make_uint2(w0, w1);
+                if constexpr (D == 64) {
+                    if (sums) {
+                        const int row = 32 * grp + l32;
+                        cs[(d + 0) * 65 + row] = bf16lo(w0); cs[(d + 1) * 65 + row] = bf16hi(w0);
+                        cs[(d + 2) * 65 + row] = bf16lo(w1); cs[(d + 3) * 65 + row] = bf16hi(w1);
+                    }
+                }
+            }
+    }
+    if constexpr (D == 64) {
+        if (sums) {
+            __syncthreads();
+            attn_block_column_sums(cs, tid, a.colsum + (b * (a.S / 64) + q0 / 64) * a.ld_cs + h * D);
         }
-    uint16_t* dqp = a.dq + b * a.stride_b + h * D + qi * a.stride_s;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int d = 32 * dt + 8 * g + 4 * lh;
-            *reinterpret_cast<uint2*>(dqp + d) =
-                make_uint2(pack_bf16(dqacc[dt][4 * g + 0] * a.scale, dqacc[dt][4 * g + 1] * a.scale),
-                           pack_bf16(dqacc[dt][4 * g + 2] * a.scale, dqacc[dt][4 * g + 3] * a.scale));
-        }
+    }
 }
 
 static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
@@ -760,6 +822,16 @@ static int attn_check(const char* who, const pp_attn_desc* d, bool bwd) {
         if (!d->d_o || !d->dq || !d->dk || !d->dv || !d->delta) return fail(PP_ERR_INVALID, "%s: null pointer", who);
         if (!aligned(d->d_o, 16) || !aligned(d->dq, 16) || !aligned(d->dk, 16) || !aligned(d->dv, 16))
             return fail(PP_ERR_INVALID, "%s: gradients must be 16-byte aligned", who);
+        if (d->colsum) {
+            if (d->D != 64) return fail(PP_ERR_UNSUPPORTED, "%s: column sums are built for head_dim 64", who);
+            const int64_t g = d->kv_group > 1 ? d->kv_group : 1;
+            const int64_t off_k = static_cast<const uint16_t*>(d->dk) - static_cast<const uint16_t*>(d->dq);
+            const int64_t off_v = static_cast<const uint16_t*>(d->dv) - static_cast<const uint16_t*>(d->dq);
+            if (off_k < d->H * d->D || off_v < d->H * d->D || off_k + d->H / g * d->D > d->ld_colsum ||
+                off_v + d->H / g * d->D > d->ld_colsum || d->H * d->D > d->ld_colsum)
+                return fail(PP_ERR_INVALID, "%s: column sums need dq, dk, dv as sections of one row of at most "
+                            "ld_colsum = %lld elements, dq first", who, (long long)d->ld_colsum);
+        }
     }
     if ((d->S / 64) * d->H * d->B > 0x7fffff00ll) return fail(PP_ERR_UNSUPPORTED, "%s: grid too large", who);
     return PP_OK;
@@ -777,13 +849,19 @@ static AttnArgs to_args(const pp_attn_desc* d) {
     a.G = d->kv_group > 1 ? d->kv_group : 1;
     a.L = d->kv_len > 0 ? d->kv_len : d->S;
     a.scale = d->scale;
+    a.colsum = d->dq ? d->colsum : nullptr;
+    a.ld_cs = d->ld_colsum;
+    a.cs_k = d->dq ? static_cast<const uint16_t*>(d->dk) - static_cast<const uint16_t*>(d->dq) : 0;
+    a.cs_v = d->dq ? static_cast<const uint16_t*>(d->dv) - static_cast<const uint16_t*>(d->dq) : 0;
     return a;
 }
 
 // Dynamic LDS of the three kernels: stages, or the merge buffers of the epilogue if those are larger.
 static size_t attn_lds_bytes(int D, bool dkv, bool exact_dq = false) {
     const size_t stage = (size_t)2 * (D / 64) * kTile * 2 + (dkv ? 512 : 0);
-    const size_t merge = (size_t)2 * ((exact_dq ? 32 : 16) * (D / 32) + 2) * 64 * 4;
+    // the exchange buffers of the epilogue and, behind them, the scratch of the column sums (head size 64)
+    const size_t merge = (size_t)2 * ((exact_dq ? 32 : 16) * (D / 32) + 2) * 64 * 4 +
+                         (D == 64 ? (size_t)kColsumScratchFloats * 4 : 0);
     const size_t stages = (size_t)attn_stages(D) * stage;
     return stages > merge ? stages : merge;
 }

@@ -452,9 +452,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, uint32_t tile_m
             const int64_t band_row = m0 + wm0 + b * 32;
             if (lane < UPR && band_row < g.M) {
                 float* out = g.colsum + (band_row >> 5) * g.N + gn;
+                if (gn + 3 < g.N && aligned(out, 16)) {
+                    *reinterpret_cast<float4*>(out) = make_float4(t[0], t[1], t[2], t[3]);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (gn + e < g.N) out[e] = t[e];
+                    for (int e = 0; e < 4; ++e)
+                        if (gn + e < g.N) out[e] = t[e];
+                }
             }
         }
     });

@@ -114,6 +114,7 @@ static int run_one(const pp_op& op, pp_stream st) {
             d.B = op.i[0]; d.S = op.i[1]; d.H = op.i[2]; d.D = op.i[3];
             d.stride_b = op.i[4]; d.stride_s = op.i[5];
             d.scale = op.f[0]; d.causal = op.j[0]; d.kv_group = op.j[1]; d.kv_len = op.j[2]; d.flags = op.j[3];
+            d.colsum = static_cast<float*>(op.p[10]); d.ld_colsum = op.i[6];
             return op.kind == PP_OP_ATTN_FWD ? pp_attn_fwd(&d, st) : pp_attn_bwd(&d, st);
         }
         case PP_OP_POSITION_IDS:

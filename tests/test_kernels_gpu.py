@@ -736,6 +736,53 @@ def test_attention(causal, B, S, H, D):
         assert_close_rel(dqkv[..., sl], qr.grad[..., sl], BF16_TOL, f"attention {name}")
 
 
+@pytest.mark.parametrize("causal,exact", [(True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("B,S,H,Hkv", [(2, 256, 3, 3), (4, 1024, 12, 12), (1, 64, 2, 2), (2, 192, 4, 2), (1, 320, 6, 1)])
+def test_attention_backward_leaves_the_column_sums_of_its_gradients(causal, exact, B, S, H, Hkv):
+    """With ``colsum`` (head size 64) the two backward kernels also write, per block of 64 tokens, the column
+    sums of dq, dk and dv as stored: the gradients themselves are unchanged bit for bit, every row of sums is
+    the fp32 sum of the 64 stored bf16 rows (up to the rounding of the additions), and pp_colreduce_grouped
+    forms from them the bias gradient of the fused projection that the two-pass reduction gives.  Multi-head
+    and grouped-query layouts, with and without the query-gradient correction."""
+    Nn = native()
+    torch.manual_seed(3 + S + H)
+    D = 64
+    width = (H + 2 * Hkv) * D
+    qkv = torch.randn(B, S, width, device=DEV).to(torch.bfloat16)
+    o = torch.empty(B, S, H * D, device=DEV, dtype=torch.bfloat16)
+    lse = torch.empty(B, H, S, device=DEV)
+    Nn.attn_fwd(qkv, o, lse, H, causal, n_kv_heads=Hkv)
+    d_o = torch.randn(B, S, H * D, device=DEV).to(torch.bfloat16)
+    ref, got = torch.full_like(qkv, float("nan")), torch.full_like(qkv, float("nan"))
+    delta = torch.empty(B, H, S, device=DEV)
+    Nn.attn_bwd(qkv, o, lse, d_o, ref, delta, H, causal, n_kv_heads=Hkv, exact_dq=exact)
+    n_part = B * S // 64
+    part = torch.full((n_part, width), float("nan"), device=DEV)
+    note(f"attention bwd with column sums B={B} S={S} H={H} Hkv={Hkv} causal={causal} exact={exact}")
+    Nn.attn_bwd(qkv, o, lse, d_o, got, delta, H, causal, n_kv_heads=Hkv, exact_dq=exact, colsum=part)
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)
+    blocks = got.double().view(n_part, 64, width)
+    assert not bool(torch.isnan(part).any())
+    assert (part.double() - blocks.sum(1)).abs().max() <= 64 * 2.0 ** -24 * float(blocks.abs().sum(1).max())
+    flat = got.view(B * S, width)
+    bias, two_pass = torch.empty(width, device=DEV), torch.empty(width, device=DEV)
+    Nn.colreduce_grouped([dict(dy=flat, out_sum=bias, workspace=part, n_part_ready=n_part)])
+    ws = torch.empty(2 * ((B * S + 127) // 128) * width, device=DEV)
+    Nn.colreduce_grouped([dict(dy=flat, out_sum=two_pass, workspace=ws)])
+    assert (bias - two_pass).abs().max() <= 1e-6 * float(flat.float().abs().sum(0).max())
+
+
+def test_attention_column_sums_are_for_head_size_64():
+    Nn = native()
+    qkv = torch.zeros(1, 64, 3 * 128, device=DEV, dtype=torch.bfloat16)
+    o = torch.zeros(1, 64, 128, device=DEV, dtype=torch.bfloat16)
+    lse, delta = torch.zeros(1, 1, 64, device=DEV), torch.zeros(1, 1, 64, device=DEV)
+    part = torch.zeros(1, 3 * 128, device=DEV)
+    with pytest.raises(RuntimeError, match="head_dim 64"):
+        Nn.attn_bwd(qkv, o, lse, o, torch.empty_like(qkv), delta, 1, True, colsum=part)
+
+
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("D", [64, 128])
 def test_attention_backward_where_query_gradients_are_small_differences(causal, D):
