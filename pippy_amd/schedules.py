@@ -95,8 +95,10 @@ class PipelineSchedule(ABC):
         self._internal_losses: List[torch.Tensor] = []
         self._stages: List[PipelineStageBase] = []
         self._by_index: Dict[int, PipelineStageBase] = {}
-        #: spread the virtual stages over two HIP streams (natively lowered stages only)
-        self.concurrent_stages = True
+        #: spread the virtual stages over two HIP streams (natively lowered stages only): True, False, or
+        #: None = when a stage pass holds enough work for it (see ``_stage_streams``)
+        self.concurrent_stages: Optional[bool] = None
+        self._small_step: Dict[Any, bool] = {}
         self._streams = None
         self._w_streams = None
         self._events: Dict[Any, Any] = {}
@@ -182,7 +184,7 @@ class PipelineSchedule(ABC):
         return merge_chunks(output_chunks, self._output_merge_spec)
 
     # -- execution of a merged action order on the device -------------------------------------------
-    def _stage_streams(self):
+    def _stage_streams(self, arg_mbs=None):
         """The HIP stream of every virtual stage (two streams, half of the stages on each), or None
         when the actions run on the caller's stream.
 
@@ -191,9 +193,12 @@ class PipelineSchedule(ABC):
         tiles than CUs, the tail of any grid, the dependent chain of a causal attention block)
         shares the machine with a kernel of another stage.  Only natively lowered stages qualify:
         their buffers are allocated once, so no allocator block changes hands between streams."""
-        if not self.concurrent_stages or os.environ.get("PIPPY_AMD_SERIAL_STAGES") == "1":
+        if self.concurrent_stages is False or os.environ.get("PIPPY_AMD_SERIAL_STAGES") == "1":
             return None
         if len(self._stages) < 2 or not all(getattr(st, "is_native", False) for st in self._stages):
+            return None
+        if self.concurrent_stages is None and os.environ.get("PIPPY_AMD_CONCURRENT_STAGES") != "1" \
+                and self._is_small_step(arg_mbs):
             return None
         dev = self._stages[0].device
         if torch.device(dev).type != "cuda":
@@ -213,6 +218,24 @@ class PipelineSchedule(ABC):
             self._events = {}
         return self._streams
 
+    #: below this many floating-point operations per stage pass (2 x parameters x rows of a microbatch) the
+    #: kernels of a pass are shorter than what switching streams and recording events costs the host
+    #: (about 50 us per pass): the README-sized MLP runs 0.5 ms per step on one stream, 1.1 ms on two
+    _CONCURRENT_MIN_FLOP = 1.0e10
+
+    def _is_small_step(self, arg_mbs) -> bool:
+        first = None
+        if arg_mbs:
+            first = next((a for a in arg_mbs[0] if isinstance(a, torch.Tensor)), None)
+        if first is None:
+            return False
+        rows = first.numel() if not first.is_floating_point() or first.dim() < 2 else first.numel() // first.shape[-1]
+        got = self._small_step.get(rows)
+        if got is None:
+            params = max(sum(p.numel() for p in st.submod.parameters()) for st in self._stages)
+            got = self._small_step[rows] = 2.0 * params * rows < self._CONCURRENT_MIN_FLOP
+        return got
+
     def _event(self, key):
         ev = self._events.get(key)
         if ev is None:
@@ -220,7 +243,7 @@ class PipelineSchedule(ABC):
         return ev
 
     def _execute(self, actions: Sequence[order.Action], arg_mbs, kwarg_mbs, target_mbs):
-        streams = self._stage_streams()
+        streams = self._stage_streams(arg_mbs)
         self._choose_weight_grad_batching()
         if streams is None:
             for kind, s, m in actions:

@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # the test models are small: left to itself a schedule would run their stages on one stream (the host cost
+    # of two exceeds their kernels), and the two-stream path — events between stages, the running merge —
+    # would go untested.  A test of the automatic choice clears this.
+    os.environ.setdefault("PIPPY_AMD_CONCURRENT_STAGES", "1")
 
 
 def pytest_collection_modifyitems(config, items):

@@ -1026,6 +1026,30 @@ def test_plain_torch_gpt_runs_natively_and_matches_the_oracle():
         assert err <= BF16_TOL, f"grad of {name}: max relative error {err:.3e}"
 
 
+def test_small_steps_run_on_one_stream_and_give_the_same_bits(monkeypatch):
+    """A schedule left to itself (``concurrent_stages = None``) runs the stages of a small model on the caller's
+    stream — the host cost of two streams exceeds such kernels — and a large one on two; either way the
+    results are the same bits."""
+    import pippy_amd as pp
+    model, ref, stages, ref_stages, ids = _build_decoder(2, n_layers=2, M=4)
+    target = torch.randint(0, 1000, ids.shape)
+    sched = pp.Schedule1F1B(stages, 4, loss_fn=pp.CrossEntropyLoss())
+    assert sched.concurrent_stages is None
+    monkeypatch.setenv("PIPPY_AMD_CONCURRENT_STAGES", "1")
+    la = []
+    out_a = sched.step(ids.to(DEV), target=target.to(DEV), losses=la).clone()
+    assert sched._stage_streams([(ids,)]) is not None
+    grads_a = [p.main_grad.clone() for p in model.parameters()]
+    monkeypatch.delenv("PIPPY_AMD_CONCURRENT_STAGES")
+    sched.zero_grad()
+    lb = []
+    out_b = sched.step(ids.to(DEV), target=target.to(DEV), losses=lb)
+    assert sched._stage_streams([(ids[:2],)]) is None          # 256 rows x 1 M parameters: a small step
+    assert sched._stage_streams([(ids.repeat(64, 8)[:2048],)]) is not None   # 2 M rows: not small
+    assert torch.equal(out_a, out_b) and all(torch.equal(a, b) for a, b in zip(la, lb))
+    assert all(torch.equal(p.main_grad, g) for p, g in zip(model.parameters(), grads_a))
+
+
 def test_a_stage_lowered_in_eval_mode_refuses_to_train_with_its_dropout_switched_on():
     """Dropout with p > 0 is identity in eval mode, so a model built that way lowers to launch lists — which
     hold no dropout.  Put into training mode afterwards the stage must raise rather than train without
