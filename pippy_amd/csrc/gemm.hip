@@ -296,11 +296,12 @@ static int launch_gemm(const GemmArgs* probs, hipStream_t st) {
             // traffic per MFMA; on 8 waves, so that every SIMD has a second wave to run while the first
             // waits (vocabulary projection 4096 x 50304 x 768: 880 against 840 TFLOP/s on 4 waves and
             // 710 on 128 x 128 tiles; 4096 x 4096 x 1024: 970 against 860).  Taken when the tiles fill at
-            // least four fifths of the rounds of 256 work-groups they need.
+            // least seven tenths of the rounds of 256 work-groups they need (the Llama qkv projection,
+            // 2048 x 12288 x 4096 = 384 tiles: 903 against 833 TFLOP/s on 128 x 128).
             GemmArgs big = probs[0];
             const int64_t t256 = ((big.M + 255) / 256) * ((big.N + 255) / 256);
             const int64_t rounds = (t256 + kComputeUnits - 1) / kComputeUnits;
-            if (t256 >= kComputeUnits && 5 * t256 >= 4 * rounds * kComputeUnits) {
+            if (t256 >= kComputeUnits && 10 * t256 >= 7 * rounds * kComputeUnits) {
                 int rc = count_tiles<256, 256>(big);
                 if (rc) return rc;
                 return launch_single8<256, 256, AT, BT, 2, EPI, CF32>(big, st);
@@ -324,6 +325,18 @@ static int launch_gemm(const GemmArgs* probs, hipStream_t st) {
                 int rc = count_tiles<128, 192>(narrow);
                 if (rc) return rc;
                 return launch_single<128, 192, AT, BT, 2, EPI, CF32>(narrow, st);
+            }
+        }
+        if constexpr (!AT && !BT && !CF32 && (EPI == PP_EPI_NONE || EPI == PP_EPI_BIAS_RESIDUAL)) {
+            // a long reduction into an output with at least one 128 x 256 tile per CU (the Llama-sized
+            // down and input-gradient projections, 2048 x 4096 with K = 11008 ... 22016): tiles twice as wide
+            // on 8 waves load a quarter fewer operand bytes per flop (921 -> 983, 938 -> 1016 TFLOP/s); with
+            // K = 4096 the longer prologue and epilogue of the larger tile still outweigh that (1003 -> 930)
+            GemmArgs w = probs[0];
+            if (w.K >= 8192) {
+                int rc = count_tiles<128, 256>(w);
+                if (rc) return rc;
+                if (w.n_blocks >= kComputeUnits) return launch_single8<128, 256, AT, BT, 3, EPI, CF32>(w, st);
             }
         }
         GemmArgs g = probs[0];
