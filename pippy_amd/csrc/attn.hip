@@ -564,11 +564,14 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
     bool sums = false;
     if constexpr (D == 64) sums = a.colsum != nullptr;  // uniform over the grid
     if (half != 0 && !sums) return;
-    float* cs = reinterpret_cast<float*>(lds) + 2 * (16 * DT * 64);  // behind the exchange buffers above
+    // column sums of the two tiles: the exchange buffers above are done with, so the scratch starts at the
+    // head of LDS: [dv, dk][64 columns][65], then [dv, dk][4 waves][64]
+    float* cs = reinterpret_cast<float*>(lds);
+    constexpr int kTileScratch = 64 * 65;
     const int row = 32 * grp + l32;
+    if (half == 0) {
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        if (half == 0) {
+        for (int pass = 0; pass < 2; ++pass) {
             f32x16_t(&acc)[DT] = pass == 0 ? dvacc : dkacc;
             uint16_t* outp = (pass == 0 ? a.dv : a.dk) + b * a.stride_b + hk * D + kvi * a.stride_s;
 #pragma unroll
@@ -585,18 +588,33 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 1) void attn_bwd_dkv_kernel(cons
                     *reinterpret_cast<uint2*>(outp + d) = make_uint2(w0, w1);
                     if constexpr (D == 64) {
                         if (sums) {
-                            cs[(d + 0) * 65 + row] = bf16lo(w0); cs[(d + 1) * 65 + row] = bf16hi(w0);
-                            cs[(d + 2) * 65 + row] = bf16lo(w1); cs[(d + 3) * 65 + row] = bf16hi(w1);
+                            float* t = cs + pass * kTileScratch + row;
+                            t[(d + 0) * 65] = bf16lo(w0); t[(d + 1) * 65] = bf16hi(w0);
+                            t[(d + 2) * 65] = bf16lo(w1); t[(d + 3) * 65] = bf16hi(w1);
                         }
                     }
                 }
         }
-        if constexpr (D == 64) {
-            if (sums) {
-                __syncthreads();
-                attn_block_column_sums(cs, tid, a.colsum + (b * (a.S / 64) + kv0 / 64) * a.ld_cs +
-                                                    (pass == 0 ? a.cs_v : a.cs_k) + hk * D);
-                __syncthreads();
+    }
+    if constexpr (D == 64) {
+        if (sums) {
+            __syncthreads();
+            // every wave adds 16 rows of each column of both tiles in ascending order; waves 0 and 1 then
+            // add the four partial sums of dv and of dk in wave order
+            const int c = tid & 63, rq = tid >> 6;
+            float* part = cs + 2 * kTileScratch;
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                float t = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) t += cs[pass * kTileScratch + c * 65 + rq * 16 + r];
+                part[(pass * 4 + rq) * 64 + c] = t;
+            }
+            __syncthreads();
+            if (rq < 2) {
+                const float* pp_ = part + rq * 4 * 64 + c;
+                float* out = a.colsum + (b * (a.S / 64) + kv0 / 64) * a.ld_cs + (rq == 0 ? a.cs_v : a.cs_k) + hk * D;
+                out[c] = ((pp_[0] + pp_[64]) + pp_[128]) + pp_[192];
             }
         }
     }
