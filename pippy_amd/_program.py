@@ -821,8 +821,8 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
     * the bias gradient of a fused q | k | v projection takes them from the attention backward kernels (head
       size 64), which write that projection's output gradient.
 
-    Only exact matches are rewired: same pointers, same shape, a contiguous tensor, and no other op of the I
-    pass writing to the same address."""
+    Only exact matches are rewired: same pointers, same shape, and no other op of the I pass writing anywhere
+    into the tensor."""
     if os.environ.get("PIPPY_AMD_TWO_PASS_COLUMN_SUMS") == "1":  # for A / B measurements of this rewiring
         return
     I = prog.I.ops
@@ -832,11 +832,14 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
     attn_ops = [op for op in I if op.kind == N.OP_ATTN_BWD and op.i[3] == 64 and not op.p[10]]
     if not ln_ops and not act_ops and not attn_ops:
         return
-    written: Dict[int, int] = {}
-    for op in I:
-        for q in _WRITTEN_FIELDS.get(op.kind, range(12)):
-            if op.p[q]:
-                written[op.p[q]] = written.get(op.p[q], 0) + 1
+    writes = [(op.p[q], op) for op in I for q in _WRITTEN_FIELDS.get(op.kind, range(12)) if op.p[q]]
+
+    def only_writer(src, lo: int, n_bytes: int) -> bool:
+        """No op of the pass other than ``src`` writes through a pointer into [lo, lo + n_bytes): the tensor
+        that the reduction reads is what ``src`` left there (an in-place rotary embedding or a row copy into
+        a part of it, which start inside the range, rule the rewiring out)."""
+        return not any(lo <= ptr < lo + n_bytes and op is not src for ptr, op in writes)
+
     for k, (op, _tag) in enumerate(b._w_reduce):
         if op.j[1]:
             continue
@@ -852,10 +855,9 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
             op.p[6], op.j[1] = ws.data_ptr(), n_part
         elif op.kind == N.OP_COLSUM:
             rows, Cc, ld = op.i[0], op.i[1], op.i[2]
-            if written.get(op.p[0], 0) != 1:
-                continue
+            n_bytes = 2 * ((rows - 1) * ld + Cc) if rows else 0
             src = [l for l in ln_ops if l.p[6] == op.p[0] and l.i[0] == rows and l.i[1] == Cc and not l.p[8]]
-            if len(src) == 1 and ld == Cc:
+            if len(src) == 1 and ld == Cc and only_writer(src[0], op.p[0], n_bytes):
                 n_part = (rows + N.LN_SUM_ROWS - 1) // N.LN_SUM_ROWS
                 ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
                 src[0].p[8] = ws.data_ptr()
@@ -864,7 +866,7 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
             # the input gradient of an activation, written by the epilogue of the GEMM in front of it
             src = [g for g in act_ops if g.p[2] == op.p[0] and g.i[0] == rows and g.i[1] == Cc and g.i[5] == ld
                    and not g.p[9]]
-            if len(src) == 1:
+            if len(src) == 1 and only_writer(src[0], op.p[0], n_bytes):
                 n_part = (rows + N.GEMM_COLSUM_ROWS - 1) // N.GEMM_COLSUM_ROWS
                 ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
                 src[0].p[9] = ws.data_ptr()
@@ -878,7 +880,7 @@ def _fuse_column_sums(b: "Builder", prog: MicrobatchProgram) -> None:
                 return (a.p[6] == op.p[0] and a.p[7] == a.p[6] + 2 * H * D and a.p[8] == a.p[7] + 2 * Hkv * D
                         and Cc == (H + 2 * Hkv) * D and ss == ld and sb == S * ss and rows == Bn * S)
             src = [a for a in attn_ops if fused(a)]
-            if len(src) == 1 and written.get(src[0].p[7], 0) == 1 and written.get(src[0].p[8], 0) == 1:
+            if len(src) == 1 and only_writer(src[0], op.p[0], n_bytes):
                 n_part = rows // 64
                 ws = b.grad(f"colsums.{k}", (n_part * Cc,), torch.float32)
                 src[0].p[10], src[0].i[6] = ws.data_ptr(), Cc
