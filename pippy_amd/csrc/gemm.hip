@@ -292,19 +292,21 @@ template <int BM, int BN, bool AT, bool BT, int EPI, bool CF32>
 static int launch_gemm(const GemmArgs* probs, hipStream_t st) {
     {
         if constexpr (EPI == PP_EPI_NONE && !CF32 && BM == 128 && !AT && !BT) {
-            // a large output with both operands k-contiguous: 256 x 256 tiles halve the LDS and L2
-            // traffic per MFMA; on 8 waves, so that every SIMD has a second wave to run while the first
-            // waits (vocabulary projection 4096 x 50304 x 768: 880 against 840 TFLOP/s on 4 waves and
-            // 710 on 128 x 128 tiles; 4096 x 4096 x 1024: 970 against 860).  Taken when the tiles fill at
-            // least seven tenths of the rounds of 256 work-groups they need (the Llama qkv projection,
-            // 2048 x 12288 x 4096 = 384 tiles: 903 against 833 TFLOP/s on 128 x 128).
+            // a large output with both operands k-contiguous: 256-row tiles halve the LDS and L2 traffic
+            // per MFMA; on 8 waves, so that every SIMD has a second wave to run while the first waits
+            // (vocabulary projection 4096 x 50304 x 768: 880 against 840 TFLOP/s on 4 waves and 710 on
+            // 128 x 128 tiles; 4096 x 4096 x 1024: 970 against 860)
             GemmArgs big = probs[0];
-            const int64_t t256 = ((big.M + 255) / 256) * ((big.N + 255) / 256);
-            const int64_t rounds = (t256 + kComputeUnits - 1) / kComputeUnits;
-            if (t256 >= kComputeUnits && 10 * t256 >= 7 * rounds * kComputeUnits) {
+            const int wide = wide_tile_for(big.M, big.N, true);
+            if (wide == 256) {
                 int rc = count_tiles<256, 256>(big);
                 if (rc) return rc;
                 return launch_single8<256, 256, AT, BT, 2, EPI, CF32>(big, st);
+            }
+            if (wide == 192) {
+                int rc = count_tiles<256, 192>(big);
+                if (rc) return rc;
+                return launch_single8<256, 192, AT, BT, 2, EPI, CF32>(big, st);
             }
         }
         if constexpr (BM == 128 && BN == 128 && !AT && !BT) {

@@ -268,8 +268,12 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs& g, uint32_t tile_m
     FragReader<BN, BT, KT> rb[TN];
 #pragma unroll
     for (int t = 0; t < TM; ++t) ra[t].init(wm0 + t * 32, lane);
+    // DUAL: the first half of a wave's accumulator tiles is its columns of the first product, the second
+    // half the same columns of the second product (rows BN / 2 ... of the B tile)
+    static_assert(!DUAL || TN % 2 == 0, "two products per tile: an even number of accumulator tiles per wave");
 #pragma unroll
-    for (int t = 0; t < TN; ++t) rb[t].init(wn0 + t * 32, lane);
+    for (int t = 0; t < TN; ++t)
+        rb[t].init(DUAL ? (t < TN / 2 ? 0 : BN / 2) + wn0 / 2 + (t % (TN / 2 > 0 ? TN / 2 : 1)) * 32 : wn0 + t * 32, lane);
     bf16x8_t fa[2][TM], fb[2][TN];
     auto read_frags = [&](int sel, const uint16_t* st, int ks) {
 #pragma unroll
@@ -559,6 +563,24 @@ static inline int count_tiles(GemmArgs& g) {
 
 
 constexpr uint32_t kComputeUnits = 256;
+
+// Whether an M x N output with both operands k-contiguous takes 256-row tiles on 8 waves (one work-group
+// per CU), and how wide: 256 (half the LDS and L2 traffic per MFMA of a 128 x 128 tile) when the tiles fill at
+// least seven tenths of the rounds of 256 work-groups they need, 192 when those fill at least 85 %; with both
+// eligible, the one with fewer rounds x tile width, the narrower tile counted 6 % dearer per column (measured:
+// 2048 x 12288 x 4096, 384 tiles in 2 rounds against 512 in 2: 224 -> 203 us; 2048 x 11008 x 4096, 344 tiles
+// (too empty) against 464: 208 -> 184 us; 2048 x 22016 x 4096, 3 rounds against 4: 347 against 367 us;
+// 4096 x 50304 x 768, 13 rounds against 17: 364 against 397 us).  Returns 0, 192 or 256.
+static inline int wide_tile_for(int64_t M, int64_t N, bool allow_192) {
+    const int64_t cu = kComputeUnits, rows = (M + 255) / 256;
+    const int64_t t256 = rows * ((N + 255) / 256), t192 = rows * ((N + 191) / 192);
+    const int64_t r256 = (t256 + cu - 1) / cu, r192 = (t192 + cu - 1) / cu;
+    const bool ok256 = t256 >= cu && 10 * t256 >= 7 * r256 * cu;
+    const bool ok192 = allow_192 && t192 >= cu && 100 * t192 >= 85 * r192 * cu;
+    if (!ok256 && !ok192) return 0;
+    if (ok256 && ok192) return r192 * 192 * 106 < r256 * 256 * 100 ? 192 : 256;
+    return ok256 ? 256 : 192;
+}
 
 // Validates one descriptor and converts it to kernel arguments.  Returns PP_OK with *empty set
 // when the problem has no output (M or N zero).

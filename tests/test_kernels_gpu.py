@@ -1267,7 +1267,10 @@ def test_swiglu_matches_oracle(n):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,F", [(4096, 1024, 2816), (130, 72, 200), (1, 8, 8), (257, 4096, 344)])
+@pytest.mark.parametrize("M,K,F", [(4096, 1024, 2816), (130, 72, 200), (1, 8, 8), (257, 4096, 344),
+                                   # outputs that fill the CUs with 256-row tiles on 8 waves: forward 256 x 256,
+                                   # backward 256 x 192 (first) and 256 x 256 (the other two), the second with ragged edges
+                                   (2048, 264, 11008), (2050, 72, 11016), (2048, 136, 8192)])
 def test_gemm_fused_swiglu_equals_the_separate_kernels_and_the_oracle(M, K, F):
     """The gate / up GEMM that applies SwiGLU in its epilogue, and the down projection's input-gradient
     GEMM that applies its derivative, leave the bits of the GEMMs followed by the element-wise kernels
