@@ -126,49 +126,58 @@ __global__ __launch_bounds__(W * 64) void gemm_bf16_dswiglu_kernel(const GemmArg
     const int64_t col = (int64_t)tile_n * BN + wn * WTN + ru * 4;
     const int64_t row0 = (int64_t)tile_m * BM + wm * WTM;
     uint16_t* const out = static_cast<uint16_t*>(g.C);  // dgu [M, 2 N] with row stride ldc
-    static_for<TM>([&](auto band) {
-        constexpr int b = decltype(band)::value;
+    // The passes of the tile's bands run in batches of kBatch; the g and u values of a batch are fetched one
+    // batch ahead (two register sets), so that their way from memory overlaps the arithmetic and the stores
+    // of the batch before (with one work-group per CU nothing else would run meanwhile).
+    constexpr int kPerBand = kPasses / kBatch, kBatches = TM * kPerBand;
+    uint2 gw[2][kBatch], uw[2][kBatch];
+    auto fetch = [&](auto set_c, int k) {
+        constexpr int set = decltype(set_c)::value;
 #pragma unroll
-        for (int a = 0; a < TN; ++a)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int u = a * 8 + 2 * q + lh;
-                *reinterpret_cast<float4*>(cw + l32 * WTN + (unit_at(u, l32) << 2)) =
-                    make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
+        for (int j = 0; j < kBatch; ++j) {
+            const int64_t row = row0 + (k / kPerBand) * 32 + ((k % kPerBand) * kBatch + j) * RPP + rr;
+            if (lane_on && row < g.M && col < g.N) {
+                gw[set][j] = *reinterpret_cast<const uint2*>(gu + row * ld_gu + col);
+                uw[set][j] = *reinterpret_cast<const uint2*>(gu + row * ld_gu + g.N + col);
             }
-        // the region is private to the wave: its own LDS accesses complete in order
+        }
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    static_for<kBatches>([&](auto batch) {
+        constexpr int k = decltype(batch)::value, b = k / kPerBand, i0 = (k % kPerBand) * kBatch, set = k & 1;
+        if constexpr (k + 1 < kBatches) fetch(std::integral_constant<int, (k + 1) & 1>{}, k + 1);
+        if constexpr (i0 == 0) {
 #pragma unroll
-        for (int i0 = 0; i0 < kPasses; i0 += kBatch) {
-            float4 dh[kBatch];
-            uint2 gw[kBatch], uw[kBatch];
-            bool ok[kBatch];
+            for (int a = 0; a < TN; ++a)
 #pragma unroll
-            for (int j = 0; j < kBatch; ++j) {
-                const int m = (i0 + j) * RPP + rr;
-                const int64_t row = row0 + b * 32 + m;
-                dh[j] = *reinterpret_cast<const float4*>(cw + (lane_on ? m : 0) * WTN + (unit_at(lane_on ? ru : 0, m) << 2));
-                ok[j] = lane_on && row < g.M && col < g.N;
-                if (ok[j]) {
-                    gw[j] = *reinterpret_cast<const uint2*>(gu + row * ld_gu + col);
-                    uw[j] = *reinterpret_cast<const uint2*>(gu + row * ld_gu + g.N + col);
+                for (int q = 0; q < 4; ++q) {
+                    const int u = a * 8 + 2 * q + lh;
+                    *reinterpret_cast<float4*>(cw + l32 * WTN + (unit_at(u, l32) << 2)) =
+                        make_float4(acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2], acc[a][b][4 * q + 3]);
                 }
-            }
+        }
+        // the region is private to the wave: its own LDS accesses complete in order
+        float4 dh[kBatch];
 #pragma unroll
-            for (int j = 0; j < kBatch; ++j) {
-                if (!ok[j]) continue;
-                const int64_t row = row0 + b * 32 + (i0 + j) * RPP + rr;
-                // dh is rounded to bf16 first: what a separate GEMM would have stored
-                const uint32_t d0 = pack_bf16(dh[j].x, dh[j].y), d1 = pack_bf16(dh[j].z, dh[j].w);
-                const float d[4] = {bf16lo(d0), bf16hi(d0), bf16lo(d1), bf16hi(d1)};
-                const float gg[4] = {bf16lo(gw[j].x), bf16hi(gw[j].x), bf16lo(gw[j].y), bf16hi(gw[j].y)};
-                const float uu[4] = {bf16lo(uw[j].x), bf16hi(uw[j].x), bf16lo(uw[j].y), bf16hi(uw[j].y)};
-                float dg[4], du[4];
+        for (int j = 0; j < kBatch; ++j) {
+            const int m = (i0 + j) * RPP + rr;
+            dh[j] = *reinterpret_cast<const float4*>(cw + (lane_on ? m : 0) * WTN + (unit_at(lane_on ? ru : 0, m) << 2));
+        }
 #pragma unroll
-                for (int e = 0; e < 4; ++e) swiglu_grads(gg[e], uu[e], d[e], &dg[e], &du[e]);
-                *reinterpret_cast<uint2*>(out + row * g.ldc + col) = make_uint2(pack_bf16(dg[0], dg[1]), pack_bf16(dg[2], dg[3]));
-                *reinterpret_cast<uint2*>(out + row * g.ldc + g.N + col) =
-                    make_uint2(pack_bf16(du[0], du[1]), pack_bf16(du[2], du[3]));
-            }
+        for (int j = 0; j < kBatch; ++j) {
+            const int64_t row = row0 + b * 32 + (i0 + j) * RPP + rr;
+            if (!(lane_on && row < g.M && col < g.N)) continue;
+            // dh is rounded to bf16 first: what a separate GEMM would have stored
+            const uint32_t d0 = pack_bf16(dh[j].x, dh[j].y), d1 = pack_bf16(dh[j].z, dh[j].w);
+            const float d[4] = {bf16lo(d0), bf16hi(d0), bf16lo(d1), bf16hi(d1)};
+            const float gg[4] = {bf16lo(gw[set][j].x), bf16hi(gw[set][j].x), bf16lo(gw[set][j].y), bf16hi(gw[set][j].y)};
+            const float uu[4] = {bf16lo(uw[set][j].x), bf16hi(uw[set][j].x), bf16lo(uw[set][j].y), bf16hi(uw[set][j].y)};
+            float dg[4], du[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) swiglu_grads(gg[e], uu[e], d[e], &dg[e], &du[e]);
+            *reinterpret_cast<uint2*>(out + row * g.ldc + col) = make_uint2(pack_bf16(dg[0], dg[1]), pack_bf16(dg[2], dg[3]));
+            *reinterpret_cast<uint2*>(out + row * g.ldc + g.N + col) =
+                make_uint2(pack_bf16(du[0], du[1]), pack_bf16(du[2], du[3]));
         }
     });
 }
@@ -205,8 +214,9 @@ using namespace pp;
 // Tile choice.  Small problems keep 128 x 128 tiles on 4 waves (two work-groups per CU).  A problem whose
 // 256-row tiles on 8 waves fill the CUs takes those: the forward 256 x 256 (128 columns of h), the backward
 // 256 x 192 or 256 x 256, whichever needs less time by rounds of work-groups x tile area (Llama-2-7B feed-forward,
-// 2048 tokens: forward 466 -> 413 us, backward 247 -> 240 us; with one work-group per CU nothing runs beside
-// a tile's epilogue, which is why the gain is smaller than that of the plain GEMM on the same tiles).
+// 2048 tokens: forward 466 -> 403 us, backward 247 -> 226 us; with one work-group per CU nothing runs beside
+// a tile's epilogue and all CUs reach it together, which is why the gain is smaller than that of the plain
+// GEMM on the same tiles).
 template <int BM, int BN, int NS, int W>
 static int launch_swiglu(GemmArgs& g, uint16_t* gu, int64_t ld_gu, hipStream_t st) {
     g.tiles_m = (uint32_t)((g.M + BM - 1) / BM);
