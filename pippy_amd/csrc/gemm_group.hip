@@ -7,14 +7,6 @@
 #include "gemm_core.h"
 #include <vector>
 
-#ifndef PP_KSEG_BM
-#define PP_KSEG_BM 128
-#define PP_KSEG_BN 128
-#define PP_KSEG_W 4
-#define PP_KSEG_NS 2
-#define PP_KSEG_KT 64
-#endif
-
 namespace pp {
 
 template <int BM, int BN, bool AT, bool BT, int NS, int EPI, bool CF32, int KT, int W = 4>
@@ -187,7 +179,11 @@ extern "C" int pp_gemm_bf16_grouped_kseg(const pp_gemm_desc* descs, int n, int n
         ga.n = cnt;
         for (int i = 0; i < cnt; ++i) ga.p[i] = probs[done + i];
         done += cnt;
-        int rc = launch_group_kseg<PP_KSEG_BM, PP_KSEG_BN, PP_KSEG_NS, PP_KSEG_KT, PP_KSEG_W>(ga, n_seg, st);
+        // as for one pass: 256 x 128 tiles on 8 waves once there are more 128 x 128 tiles than two per CU (the
+        // running sum doubles the accumulator registers, which 8 waves per CU leave room for; Llama-2-7B
+        // stage step with one pass per step: 389 -> 375 ms)
+        int rc = tiles_128(ga) > 2 * kComputeUnits ? launch_group_kseg<256, 128, 3, 64, 8>(ga, n_seg, st)
+                                                   : launch_group_kseg<128, 128, 2, 64, 4>(ga, n_seg, st);
         if (rc) return rc;
     }
     return PP_OK;

@@ -105,9 +105,11 @@ class PipelineSchedule(ABC):
         #: run the weight-gradient passes of a stage as ONE batched pass after its last input-gradient pass
         #: (every weight-gradient GEMM once over all microbatches, bit-identical accumulators, see
         #: ``_program.BatchedW``).  None: where it pays - stages with expert weights, whose fp32 accumulators
-        #: outweigh a microbatch's operands (53.2 against 58.3 ms per Mixtral-style step; dense stages gain
-        #: nothing: 408 against 407 ms per Llama-stage step, 44.0 against 42.6 ms per GPT-2-small step, where
-        #: the batched pass at the end of the step no longer hides behind other stages' kernels);
+        #: outweigh a microbatch's operands (53.2 against 58.3 ms per Mixtral-style step), and a schedule's
+        #: only native stage, whose passes have no other stage's kernels to run beside (the accumulators then
+        #: move once per step instead of once per microbatch: 375 against 386 ms per Llama-stage step); with
+        #: several stages on this device the batched pass at the end of the step no longer hides behind other
+        #: stages' kernels (43.5 against 43.2 ms per GPT-2-small step);
         #: True / False: every native stage / none
         self.batch_weight_grads: Optional[bool] = None
         #: copy microbatch outputs into the merged result while the step runs (see ``_RunningMerge``)
@@ -316,12 +318,13 @@ class PipelineSchedule(ABC):
     def _choose_weight_grad_batching(self):
         """Sets ``batch_weight_grads`` (and with it ``split_backward``: per-microbatch gradient buffers) on
         the stages, before the step's first forward pass builds their launch lists."""
+        n_native = sum(1 for st in self._stages if getattr(st, "is_native", False))
         for st in self._stages:
             if not getattr(st, "is_native", False) or not self._has_backward:
                 continue
             want = self.batch_weight_grads
             if want is None:
-                want = st.prefers_batched_weight_grads
+                want = st.prefers_batched_weight_grads or n_native == 1
             if want and not st.split_backward:
                 st.split_backward = True
             st.batch_weight_grads = bool(want)
