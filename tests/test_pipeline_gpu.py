@@ -1892,9 +1892,26 @@ def test_weight_gradients_in_one_batched_pass_leave_the_bits_of_one_pass_per_mic
             assert torch.equal(got[name], want[name]), f"{schedule}, {steps} step(s): grad of {name}"
 
 
+@pytest.mark.parametrize("schedule", ["1f1b", "zero_bubble"])
+def test_a_schedules_only_stage_batches_its_weight_gradients_by_default(schedule):
+    """A schedule that drives one launch-list stage has no other stage's kernels to run beside that stage's
+    weight-gradient launches: left to itself it forms them in one pass per step, with the bits of one pass per
+    microbatch."""
+    import pippy_amd as pp
+    cls = {"1f1b": pp.Schedule1F1B, "zero_bubble": pp.ScheduleZeroBubble}[schedule]
+    got, losses_b, n_batched = _grads_after_steps(cls, None, 1, n_stages=1)
+    want, losses_p, none = _grads_after_steps(cls, False, 1, n_stages=1)
+    assert n_batched[0] >= 4 and not any(none), (n_batched, none)
+    for a, b in zip(losses_b, losses_p):
+        assert torch.equal(a, b)
+    for name in want:
+        assert torch.equal(got[name], want[name]), f"grad of {name}"
+
+
 def test_expert_stages_batch_their_weight_gradients_by_default():
     """Left to itself (``batch_weight_grads = None``) a schedule batches where it pays: stages with expert
-    weights, under any schedule; dense stages keep one weight-gradient pass per microbatch."""
+    weights, under any schedule; dense stages that share the device keep one weight-gradient pass per
+    microbatch."""
     import pippy_amd as pp
     from pippy_amd.configs import MoEDecoderLM, equal_split_spec
     M = 4
