@@ -569,10 +569,13 @@ def main():
             kms, kwork, kcnt = N.profile_read(kind)
             ms, work, cnt, bcnt = ms + kms, work + kwork, cnt + kcnt, bcnt + kcnt
             scnt += kcnt if kind == N.OP_GEMM_SEG_KSEG else 0
-        gcnt = 0
+        gcnt = sgcnt = 0
         for kind in (N.OP_GEMM_SWIGLU, N.OP_GEMM_DSWIGLU):   # feed-forward GEMMs with SwiGLU in the epilogue
             kms, kwork, kcnt = N.profile_read(kind)
             ms, work, cnt, gcnt = ms + kms, work + kwork, cnt + kcnt, gcnt + kcnt
+        for kind in (N.OP_GEMM_SEG_SWIGLU, N.OP_GEMM_SEG_DSWIGLU):   # the same over expert segments
+            kms, kwork, kcnt = N.profile_read(kind)
+            ms, work, cnt, sgcnt = ms + kms, work + kwork, cnt + kcnt, sgcnt + kcnt
         achieved = work / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
         result["roofline"] = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS, 4),
@@ -581,6 +584,7 @@ def main():
                               "kernel": "gemm_bf16_dma_kernel + gemm_bf16_dma8_kernel + gemm_bf16_group_kernel + gemm_bf16_splitk_kernel"
                                         + (" + gemm_bf16_seg_rows_kernel + gemm_bf16_seg_k_kernel" if scnt else "")
                                         + (" + gemm_bf16_swiglu_kernel + gemm_bf16_dswiglu_kernel" if gcnt else "")
+                                        + (" + gemm_bf16_seg_gated_kernel" if sgcnt else "")
                                         + (" + gemm_bf16_group_kseg_kernel / gemm_bf16_seg_k_multi_kernel" if bcnt else ""),
                               "launches_per_step": cnt // n_prof,
                               "avg_launch_us": round(ms / max(cnt, 1) * 1e3, 2),

@@ -288,6 +288,20 @@ int pp_gemm_bf16_swiglu(const void* x, const void* w_gate, const void* w_up, voi
 int pp_gemm_bf16_dswiglu(const void* dy, const void* w_down_t, const void* gu, void* dgu, int64_t M,
                          int64_t N, int64_t K, int64_t ldy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu,
                          pp_stream stream);
+/* The same two calls over rows that are partitioned into n_seg consecutive segments with weights of their
+ * own (the experts of a mixture-of-experts feed-forward over its permuted token rows, replacing the per-expert
+ * F.linear calls reached from pippy/_PipelineStage.py:420-428 and their backward, pippy/_backward.py:67-69):
+ * rows [seg_start[e], seg_start[e+1]) use w_gate_of[e] / w_up_of[e] (forward) or w_down_t_of[e] (backward).
+ * seg_start [n_seg + 1] (int32) and the pointer arrays live in DEVICE memory; M is the total number of
+ * rows (seg_start[n_seg] <= M), every weight [N, K] with the same ldw.  Rows outside every segment are not
+ * written.  Bits as pp_gemm_bf16_segmented (rows mode) followed by pp_swiglu_fwd / pp_swiglu_bwd. */
+int pp_gemm_bf16_segmented_swiglu(const void* x, const void* const* w_gate_of, const void* const* w_up_of,
+                                  const int32_t* seg_start, int n_seg, void* gu, void* h, int64_t M, int64_t N,
+                                  int64_t K, int64_t ldx, int64_t ldw, int64_t ld_gu, int64_t ldh,
+                                  pp_stream stream);
+int pp_gemm_bf16_segmented_dswiglu(const void* dy, const void* const* w_down_t_of, const int32_t* seg_start,
+                                   int n_seg, const void* gu, void* dgu, int64_t M, int64_t N, int64_t K,
+                                   int64_t ldy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu, pp_stream stream);
 
 /* ------------------------------------------------------------------------------------------
  * Routing of a top-2 mixture-of-experts layer (a Mixtral-style block inside the stage module;
@@ -482,7 +496,7 @@ enum pp_op_kind {
     PP_OP_SWIGLU_FWD = 17, PP_OP_SWIGLU_BWD = 18, PP_OP_ROPE = 19, PP_OP_GEMM_SEG = 20,
     PP_OP_MOE_ROUTER = 21, PP_OP_MOE_PERMUTE = 22, PP_OP_MOE_GATHER = 23, PP_OP_MOE_COMBINE = 24,
     PP_OP_MOE_GATE_BWD = 25, PP_OP_GEMM_SWIGLU = 26, PP_OP_GEMM_DSWIGLU = 27, PP_OP_POSITION_IDS = 28,
-    PP_OP_GEMM_KSEG = 29, PP_OP_GEMM_SEG_KSEG = 30
+    PP_OP_GEMM_KSEG = 29, PP_OP_GEMM_SEG_KSEG = 30, PP_OP_GEMM_SEG_SWIGLU = 31, PP_OP_GEMM_SEG_DSWIGLU = 32
 };
 
 /* Field use per kind (unused fields are ignored):
@@ -522,6 +536,8 @@ enum pp_op_kind {
  *                 pp_gemm_bf16_grouped_kseg call (they must not depend on each other)
  *   GEMM_SEG_KSEG as GEMM_SEG in k mode with p[0], p[1]: device arrays of the microbatches' A and B, p[6]:
  *                 device array of their seg_start arrays | i[7]: n_seg, i[8]: n_mb
+ *   GEMM_SEG_SWIGLU  p: x w_gate_of w_up_of gu h seg_start | i: M N K ldx ldw ld_gu ldh n_seg
+ *   GEMM_SEG_DSWIGLU p: dy w_down_t_of gu dgu seg_start | i: M N K ldy ldw ld_gu ld_dgu n_seg
  * flags bit 0 (PP_OP_SKIP): the op is stepped over.
  * flags bit 1 (PP_OP_GROUPED): a GEMM_BF16 op that may be launched together with the grouped
  * GEMM_BF16 ops next to it (they must not depend on each other); likewise consecutive grouped

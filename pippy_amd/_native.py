@@ -27,7 +27,7 @@ EPI_DGELU_ERF, EPI_DGELU_TANH, EPI_ACCUM_F32, EPI_BIAS_RELU, EPI_DRELU, EPI_ACCU
  OP_ATTN_BWD, OP_EMBED_FWD, OP_EMBED_BWD, OP_CE_LOSS, OP_ACCUM_BF16, OP_ACCUM_F32, OP_COPY_ROWS,
  OP_FILL, OP_ACT_BWD, OP_SWIGLU_FWD, OP_SWIGLU_BWD, OP_ROPE, OP_GEMM_SEG, OP_MOE_ROUTER, OP_MOE_PERMUTE,
  OP_MOE_GATHER, OP_MOE_COMBINE, OP_MOE_GATE_BWD, OP_GEMM_SWIGLU, OP_GEMM_DSWIGLU, OP_POSITION_IDS,
- OP_GEMM_KSEG, OP_GEMM_SEG_KSEG) = range(1, 31)
+ OP_GEMM_KSEG, OP_GEMM_SEG_KSEG, OP_GEMM_SEG_SWIGLU, OP_GEMM_SEG_DSWIGLU) = range(1, 33)
 SEG_ROWS, SEG_K = 0, 1
 OP_SKIP = 1
 OP_GROUPED = 2
@@ -46,7 +46,8 @@ EXPORTED_SYMBOLS = (
     "pp_profile_read", "pp_sgd_step", "pp_adamw_step", "pp_swiglu_fwd", "pp_swiglu_bwd", "pp_rope",
     "pp_gemm_bf16_segmented", "pp_moe_router_top2", "pp_moe_permute", "pp_moe_gather", "pp_moe_combine",
     "pp_moe_gate_bwd", "pp_colsum_bf16_noalloc", "pp_gemm_bf16_swiglu", "pp_gemm_bf16_dswiglu",
-    "pp_embed_fwd_at", "pp_position_ids_from_padding",
+    "pp_embed_fwd_at", "pp_position_ids_from_padding", "pp_gemm_bf16_segmented_swiglu",
+    "pp_gemm_bf16_segmented_dswiglu",
 )
 
 
@@ -147,6 +148,8 @@ def lib() -> C.CDLL:
         "pp_rope": [vp, vp, vp, i64, i64, i64, i64, i64, i32, vp],
         "pp_gemm_bf16_swiglu": [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
         "pp_gemm_bf16_dswiglu": [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
+        "pp_gemm_bf16_segmented_swiglu": [vp, vp, vp, vp, i32, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
+        "pp_gemm_bf16_segmented_dswiglu": [vp, vp, vp, i32, vp, vp, i64, i64, i64, i64, i64, i64, i64, vp],
         "pp_gemm_bf16_segmented": [C.POINTER(GemmDesc), vp, vp, i32, i32, vp],
         "pp_moe_router_top2": [vp, i64, i64, i32, vp, vp, vp],
         "pp_moe_permute": [vp, i64, i32, vp, vp, vp, vp],
@@ -346,6 +349,41 @@ def rope(x2d, cos, sin, seq: int, n_heads: int, D: int, inverse: bool = False) -
 
 
 # ---- mixture-of-experts routing and segmented GEMMs ---------------------------------------------
+def gemm_segmented_swiglu(x, w_gate_list: torch.Tensor, w_up_list: torch.Tensor, seg_start: torch.Tensor, gu, h, *,
+                          ld: Optional[int] = None) -> None:
+    """``gemm_swiglu`` over row segments with weights of their own: rows [seg_start[e], seg_start[e + 1]) of
+    ``x`` [R, K] use the [N, K] weights (leading dimension ``ld``) whose addresses are entry e of the int64
+    device tensors ``w_gate_list`` and ``w_up_list``; ``gu`` [R, 2 N], ``h`` [R, N]."""
+    require_cuda(x, w_gate_list, w_up_list, seg_start, gu, h)
+    assert seg_start.dtype == torch.int32 and w_gate_list.dtype == w_up_list.dtype == torch.int64
+    n_seg = seg_start.numel() - 1
+    assert w_gate_list.numel() == w_up_list.numel() == n_seg
+    R, K = x.shape
+    Nn = h.shape[1]
+    assert gu.shape == (R, 2 * Nn) and h.shape[0] == R and x.stride(1) == gu.stride(1) == h.stride(1) == 1
+    check(lib().pp_gemm_bf16_segmented_swiglu(x.data_ptr(), w_gate_list.data_ptr(), w_up_list.data_ptr(),
+                                              seg_start.data_ptr(), n_seg, gu.data_ptr(), h.data_ptr(), R, Nn, K,
+                                              x.stride(0), ld if ld is not None else K, gu.stride(0), h.stride(0),
+                                              current_stream()), "pp_gemm_bf16_segmented_swiglu")
+
+
+def gemm_segmented_dswiglu(dy, w_down_t_list: torch.Tensor, seg_start: torch.Tensor, gu, dgu, *,
+                           ld: Optional[int] = None) -> None:
+    """``gemm_dswiglu`` over row segments: rows [seg_start[e], seg_start[e + 1]) of ``dy`` [R, K] use the
+    transposed down projection [N, K] (leading dimension ``ld``) at entry e of ``w_down_t_list``."""
+    require_cuda(dy, w_down_t_list, seg_start, gu, dgu)
+    assert seg_start.dtype == torch.int32 and w_down_t_list.dtype == torch.int64
+    n_seg = seg_start.numel() - 1
+    assert w_down_t_list.numel() == n_seg
+    R, K = dy.shape
+    Nn = gu.shape[1] // 2
+    assert gu.shape == dgu.shape == (R, 2 * Nn) and dy.stride(1) == gu.stride(1) == dgu.stride(1) == 1
+    check(lib().pp_gemm_bf16_segmented_dswiglu(dy.data_ptr(), w_down_t_list.data_ptr(), seg_start.data_ptr(), n_seg,
+                                               gu.data_ptr(), dgu.data_ptr(), R, Nn, K, dy.stride(0),
+                                               ld if ld is not None else K, gu.stride(0), dgu.stride(0),
+                                               current_stream()), "pp_gemm_bf16_segmented_dswiglu")
+
+
 def gemm_bf16_segmented(A, B_or_C_list: torch.Tensor, Cm, seg_start: torch.Tensor, mode: int, *, other=None,
                         N: Optional[int] = None, ld: Optional[int] = None, epilogue: int = EPI_NONE,
                         aux_in=None, beta: int = 0, c_dtype=None) -> None:

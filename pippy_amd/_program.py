@@ -342,6 +342,46 @@ def op_rope(x2d, cos, sin, seq, n_heads, D, inverse=False) -> N.Op:
     return op
 
 
+def op_gemm_seg_swiglu(x, w_gate_list, w_up_list, seg_start, gu, h, *, ld=None) -> N.Op:
+    """``op_gemm_swiglu`` over the expert segments of permuted rows: the [F, K] weights of segment e (leading
+    dimension ``ld``) are entry e of the int64 device tensors ``w_gate_list`` / ``w_up_list``."""
+    T, K = x.shape
+    Fn = h.shape[1]
+    assert gu.shape == (T, 2 * Fn) and h.shape == (T, Fn) and Fn % 8 == 0 and K % 8 == 0
+    for t in (x, gu, h):
+        assert t.dtype == torch.bfloat16 and t.stride(1) == 1
+    assert seg_start.dtype == torch.int32 and w_gate_list.dtype == w_up_list.dtype == torch.int64
+    assert w_gate_list.numel() == w_up_list.numel() == seg_start.numel() - 1
+    op = N.Op()
+    op.kind = N.OP_GEMM_SEG_SWIGLU
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4], op.p[5] = (x.data_ptr(), w_gate_list.data_ptr(), w_up_list.data_ptr(),
+                                                            gu.data_ptr(), h.data_ptr(), seg_start.data_ptr())
+    op.i[0], op.i[1], op.i[2] = T, Fn, K
+    op.i[3], op.i[4], op.i[5], op.i[6] = x.stride(0), ld if ld is not None else K, gu.stride(0), h.stride(0)
+    op.i[7] = w_gate_list.numel()
+    return op
+
+
+def op_gemm_seg_dswiglu(dy, w_down_t_list, seg_start, gu, dgu, *, ld=None) -> N.Op:
+    """``op_gemm_dswiglu`` over the expert segments: the transposed down projection [F, K] of segment e is
+    entry e of ``w_down_t_list``."""
+    T, K = dy.shape
+    Fn = gu.shape[1] // 2
+    assert gu.shape == dgu.shape == (T, 2 * Fn) and Fn % 8 == 0 and K % 8 == 0
+    for t in (dy, gu, dgu):
+        assert t.dtype == torch.bfloat16 and t.stride(1) == 1
+    assert seg_start.dtype == torch.int32 and w_down_t_list.dtype == torch.int64
+    assert w_down_t_list.numel() == seg_start.numel() - 1
+    op = N.Op()
+    op.kind = N.OP_GEMM_SEG_DSWIGLU
+    op.p[0], op.p[1], op.p[2], op.p[3], op.p[4] = (dy.data_ptr(), w_down_t_list.data_ptr(), gu.data_ptr(),
+                                                   dgu.data_ptr(), seg_start.data_ptr())
+    op.i[0], op.i[1], op.i[2] = T, Fn, K
+    op.i[3], op.i[4], op.i[5], op.i[6] = dy.stride(0), ld if ld is not None else K, gu.stride(0), dgu.stride(0)
+    op.i[7] = w_down_t_list.numel()
+    return op
+
+
 def op_gemm_seg(mode, A, ptr_list, seg_start, *, Cm=None, other=None, n_cols=None, ld=None,
                 epilogue=N.EPI_NONE, aux_in=None, beta=0, c_f32=False) -> N.Op:
     """Segmented GEMM over the expert segments of permuted rows (sizes read on the device).
@@ -804,6 +844,7 @@ _WRITTEN_FIELDS = {
     N.OP_ATTN_BWD: (6, 7, 8, 9), N.OP_ACT_BWD: (2,), N.OP_SWIGLU_BWD: (3, 4), N.OP_ROPE: (0,),
     N.OP_COPY_ROWS: (1,), N.OP_FILL: (0,), N.OP_ACCUM_BF16: (0,), N.OP_ACCUM_F32: (0,),
     N.OP_MOE_GATHER: (4,), N.OP_MOE_COMBINE: (4,), N.OP_MOE_GATE_BWD: (5,), N.OP_GEMM_DSWIGLU: (3,),
+    N.OP_GEMM_SEG_DSWIGLU: (3,),
     N.OP_EMBED_BWD: (2, 3), N.OP_CE_LOSS: (2, 3),
 }
 

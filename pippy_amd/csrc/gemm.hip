@@ -112,53 +112,10 @@ struct GemmSegArgs {
 
 template <int BM, int BN, int NS, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gemm_bf16_seg_rows_kernel(const GemmSegArgs sa) {
-    // tiles of every segment, then an XCD-contiguous numbering of exactly that many ids
-    int e = 0;
+    int e;
     int32_t r0, r1;
     uint32_t tiles_m, bid;
-    if (sa.n_seg < 64) {
-        // one vector load of the bounds (lane l holds segment l) and a prefix sum over the lanes,
-        // instead of a chain of dependent scalar loads that would cost as much as a third of a tile
-        const int lane = threadIdx.x & 63;
-        const int32_t lo = sa.seg_start[min(lane, sa.n_seg)], hi = sa.seg_start[min(lane + 1, sa.n_seg)];
-        const uint32_t mine = (uint32_t)((hi - lo + BM - 1) / BM) * sa.g.tiles_n;  // 0 for lanes past n_seg
-        uint32_t incl = mine;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t up = __shfl_up(incl, o, 64);
-            if (lane >= o) incl += up;
-        }
-        const uint32_t total = __shfl(incl, 63, 64);
-        const uint32_t total8 = (total + 7) & ~7u;
-        if (blockIdx.x >= total8) return;
-        bid = xcd_remap(blockIdx.x, total8);
-        if (bid >= total) return;
-        const uint64_t past = __ballot(incl > bid);  // lanes whose segments end after this tile
-        e = __builtin_amdgcn_readfirstlane(__builtin_ctzll(past));
-        bid = __builtin_amdgcn_readfirstlane(bid - __shfl(incl - mine, e, 64));
-        r0 = __builtin_amdgcn_readfirstlane(__shfl(lo, e, 64));
-        r1 = __builtin_amdgcn_readfirstlane(__shfl(hi, e, 64));
-        tiles_m = (uint32_t)((r1 - r0 + BM - 1) / BM);
-    } else {
-        uint32_t total = 0;
-        for (int q = 0; q < sa.n_seg; ++q)
-            total += (uint32_t)((sa.seg_start[q + 1] - sa.seg_start[q] + BM - 1) / BM) * sa.g.tiles_n;
-        const uint32_t total8 = (total + 7) & ~7u;
-        if (blockIdx.x >= total8) return;
-        bid = xcd_remap(blockIdx.x, total8);
-        if (bid >= total) return;
-        r0 = sa.seg_start[0];
-        r1 = r0;
-        tiles_m = 0;
-        for (; e < sa.n_seg; ++e) {
-            r1 = sa.seg_start[e + 1];
-            tiles_m = (uint32_t)((r1 - r0 + BM - 1) / BM);
-            const uint32_t nt = tiles_m * sa.g.tiles_n;
-            if (bid < nt) break;
-            bid -= nt;
-            r0 = r1;
-        }
-    }
+    if (!seg_rows_locate<BM>(sa.seg_start, sa.n_seg, sa.g.tiles_n, &e, &r0, &r1, &tiles_m, &bid)) return;
     GemmArgs g = sa.g;
     g.M = r1 - r0;
     g.A += (int64_t)r0 * g.lda;

@@ -562,6 +562,68 @@ static inline int count_tiles(GemmArgs& g) {
 }
 
 
+// The tile of a rows-segmented launch: the rows of A are partitioned into n_seg consecutive segments whose
+// bounds seg_start[0 .. n_seg] live in device memory; every segment has its own ceil(rows / BM) x tiles_n
+// tiles, numbered segment after segment, and the grid is an upper bound.  Finds the segment e, its rows
+// [r0, r1), its tiles_m and the tile's number inside it for this work-group; false when the work-group has
+// no tile.  The ids that exist are renumbered XCD-contiguously.
+template <int BM>
+__device__ __forceinline__ bool seg_rows_locate(const int32_t* seg_start, int n_seg, uint32_t tiles_n, int* e_out,
+                                                int32_t* r0_out, int32_t* r1_out, uint32_t* tiles_m_out,
+                                                uint32_t* bid_out) {
+    int e = 0;
+    int32_t r0, r1;
+    uint32_t tiles_m, bid;
+    if (n_seg < 64) {
+        // one vector load of the bounds (lane l holds segment l) and a prefix sum over the lanes,
+        // instead of a chain of dependent scalar loads that would cost as much as a third of a tile
+        const int lane = threadIdx.x & 63;
+        const int32_t lo = seg_start[min(lane, n_seg)], hi = seg_start[min(lane + 1, n_seg)];
+        const uint32_t mine = (uint32_t)((hi - lo + BM - 1) / BM) * tiles_n;  // 0 for lanes past n_seg
+        uint32_t incl = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
+        }
+        const uint32_t total = __shfl(incl, 63, 64);
+        const uint32_t total8 = (total + 7) & ~7u;
+        if (blockIdx.x >= total8) return false;
+        bid = xcd_remap(blockIdx.x, total8);
+        if (bid >= total) return false;
+        const uint64_t past = __ballot(incl > bid);  // lanes whose segments end after this tile
+        e = __builtin_amdgcn_readfirstlane(__builtin_ctzll(past));
+        bid = __builtin_amdgcn_readfirstlane(bid - __shfl(incl - mine, e, 64));
+        r0 = __builtin_amdgcn_readfirstlane(__shfl(lo, e, 64));
+        r1 = __builtin_amdgcn_readfirstlane(__shfl(hi, e, 64));
+        tiles_m = (uint32_t)((r1 - r0 + BM - 1) / BM);
+    } else {
+        uint32_t total = 0;
+        for (int q = 0; q < n_seg; ++q) total += (uint32_t)((seg_start[q + 1] - seg_start[q] + BM - 1) / BM) * tiles_n;
+        const uint32_t total8 = (total + 7) & ~7u;
+        if (blockIdx.x >= total8) return false;
+        bid = xcd_remap(blockIdx.x, total8);
+        if (bid >= total) return false;
+        r0 = seg_start[0];
+        r1 = r0;
+        tiles_m = 0;
+        for (; e < n_seg; ++e) {
+            r1 = seg_start[e + 1];
+            tiles_m = (uint32_t)((r1 - r0 + BM - 1) / BM);
+            const uint32_t nt = tiles_m * tiles_n;
+            if (bid < nt) break;
+            bid -= nt;
+            r0 = r1;
+        }
+    }
+    *e_out = e;
+    *r0_out = r0;
+    *r1_out = r1;
+    *tiles_m_out = tiles_m;
+    *bid_out = bid;
+    return true;
+}
+
 constexpr uint32_t kComputeUnits = 256;
 
 // Whether an M x N output with both operands k-contiguous takes 256-row tiles on 8 waves (one work-group

@@ -21,7 +21,8 @@ namespace pp {
 // (the first half of its accumulator tiles is the gate, the second the up product), so that a band of 32
 // rows goes through the wave's own LDS region and comes back with both values of an element in one lane.
 template <int BM, int BN, int NS, int W>
-__global__ __launch_bounds__(W * 64) void gemm_bf16_swiglu_kernel(const GemmArgs g, uint16_t* gu, int64_t ld_gu) {
+__device__ __forceinline__ void swiglu_tile(const GemmArgs& g, uint16_t* gu, int64_t ld_gu, uint32_t tile_m,
+                                            uint32_t tile_n) {
     typedef WaveTile<BM, BN, W> WT;
     constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     constexpr int H = WTN / 2;      // columns of h per wave
@@ -30,10 +31,6 @@ __global__ __launch_bounds__(W * 64) void gemm_bf16_swiglu_kernel(const GemmArgs
     constexpr int RPP = 64 / UPH;   // rows per pass
     constexpr int kPasses = 32 / RPP;
     static_assert(TN % 2 == 0 && (UPR & (UPR - 1)) == 0 && 64 % UPH == 0 && 32 % RPP == 0, "wave tile of 64 or 128 columns");
-    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
-    if (bid >= g.n_blocks) return;
-    uint32_t tile_m, tile_n;
-    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
     f32x16_t acc[TN][TM];
 #pragma unroll
     for (int a = 0; a < TN; ++a)
@@ -90,7 +87,8 @@ __global__ __launch_bounds__(W * 64) void gemm_bf16_swiglu_kernel(const GemmArgs
 
 // Backward tile: an ordinary tile of dh = dy Wd whose epilogue turns it into dg and du.
 template <int BM, int BN, int NS, int W>
-__global__ __launch_bounds__(W * 64) void gemm_bf16_dswiglu_kernel(const GemmArgs g, const uint16_t* gu, int64_t ld_gu) {
+__device__ __forceinline__ void dswiglu_tile(const GemmArgs& g, const uint16_t* gu, int64_t ld_gu, uint32_t tile_m,
+                                             uint32_t tile_n) {
     typedef WaveTile<BM, BN, W> WT;
     constexpr int WTM = WT::WTM, WTN = WT::WTN, TM = WT::TM, TN = WT::TN;
     constexpr int UPR = WTN / 4;   // 16-byte units per row
@@ -98,10 +96,6 @@ __global__ __launch_bounds__(W * 64) void gemm_bf16_dswiglu_kernel(const GemmArg
     constexpr int kPasses = 32 / RPP;
     constexpr int kBatch = kPasses < 8 ? kPasses : 8;  // passes whose loads are in flight together
     static_assert(UPR % 8 == 0 && 32 % RPP == 0 && kPasses % kBatch == 0, "the unit swizzle works on groups of 8 units");
-    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
-    if (bid >= g.n_blocks) return;
-    uint32_t tile_m, tile_n;
-    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
     f32x16_t acc[TN][TM];
 #pragma unroll
     for (int a = 0; a < TN; ++a)
@@ -180,6 +174,54 @@ __global__ __launch_bounds__(W * 64) void gemm_bf16_dswiglu_kernel(const GemmArg
                 make_uint2(pack_bf16(du[0], du[1]), pack_bf16(du[2], du[3]));
         }
     });
+}
+
+template <int BM, int BN, int NS, int W>
+__global__ __launch_bounds__(W * 64) void gemm_bf16_swiglu_kernel(const GemmArgs g, uint16_t* gu, int64_t ld_gu) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks) return;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    swiglu_tile<BM, BN, NS, W>(g, gu, ld_gu, tile_m, tile_n);
+}
+
+template <int BM, int BN, int NS, int W>
+__global__ __launch_bounds__(W * 64) void gemm_bf16_dswiglu_kernel(const GemmArgs g, const uint16_t* gu, int64_t ld_gu) {
+    const uint32_t bid = xcd_remap(blockIdx.x, gridDim.x);
+    if (bid >= g.n_blocks) return;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+    dswiglu_tile<BM, BN, NS, W>(g, gu, ld_gu, tile_m, tile_n);
+}
+
+// The same two tiles over rows that are partitioned into segments with a weight of their own each (the
+// experts of a mixture-of-experts layer over its permuted token rows): segment e multiplies its rows by
+// w_a[e] (and w_b[e], forward).  The segment bounds live in device memory; see seg_rows_locate.
+struct GatedSegArgs {
+    GemmArgs g;  // M = total rows; B and B2 unused
+    const int32_t* seg_start;
+    const void* const* w_a;
+    const void* const* w_b;
+    int n_seg;
+};
+
+template <int BM, int BN, int NS, int W, bool FWD>
+__global__ __launch_bounds__(W * 64) void gemm_bf16_seg_gated_kernel(const GatedSegArgs sa, uint16_t* gu, int64_t ld_gu) {
+    int e;
+    int32_t r0, r1;
+    uint32_t tiles_m, bid;
+    if (!seg_rows_locate<BM>(sa.seg_start, sa.n_seg, sa.g.tiles_n, &e, &r0, &r1, &tiles_m, &bid)) return;
+    GemmArgs g = sa.g;
+    g.M = r1 - r0;
+    g.A += (int64_t)r0 * g.lda;
+    g.B = static_cast<const uint16_t*>(sa.w_a[e]);
+    if (FWD) g.B2 = static_cast<const uint16_t*>(sa.w_b[e]);
+    g.C = static_cast<uint16_t*>(g.C) + (int64_t)r0 * g.ldc;
+    gu += (int64_t)r0 * ld_gu;
+    uint32_t tile_m, tile_n;
+    grouped_tile(bid, tiles_m, g.tiles_n, &tile_m, &tile_n);
+    if constexpr (FWD) swiglu_tile<BM, BN, NS, W>(g, gu, ld_gu, tile_m, tile_n);
+    else dswiglu_tile<BM, BN, NS, W>(g, gu, ld_gu, tile_m, tile_n);
 }
 
 static int gated_check(const char* who, const void* a, const void* b, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -283,4 +325,71 @@ extern "C" int pp_gemm_bf16_dswiglu(const void* dy, const void* w_down_t, const 
         case 192: return launch_dswiglu<256, 192, 2, 8>(g, gup, ld_gu, st);
         default: return launch_dswiglu<128, 128, 2, 4>(g, gup, ld_gu, st);
     }
+}
+
+// Rows-segmented forms (the expert feed-forwards of a mixture-of-experts layer): 128 x 128 tiles on 4 waves,
+// two work-groups per CU, as the segmented GEMMs they replace; the grid is an upper bound on the tiles.
+template <bool FWD>
+static int launch_seg_gated(GatedSegArgs& sa, uint16_t* gu, int64_t ld_gu, hipStream_t st, const char* who) {
+    constexpr int BM = 128, BN = 128, NS = 2, W = 4;
+    constexpr size_t lds = (size_t)NS * (BM + BN) * BK * sizeof(uint16_t);
+    static const int attr_rc = reserve_lds(&gemm_bf16_seg_gated_kernel<BM, BN, NS, W, FWD>, lds);
+    if (attr_rc) return attr_rc;
+    const int64_t cols = FWD ? BN / 2 : BN;  // columns of N per tile
+    sa.g.tiles_n = (uint32_t)((sa.g.N + cols - 1) / cols);
+    // every segment may end in a partly filled tile row
+    const uint64_t bound = ((uint64_t)(sa.g.M + BM - 1) / BM + (uint64_t)sa.n_seg) * sa.g.tiles_n;
+    if (bound > 0x0fffff00ull) return fail(PP_ERR_UNSUPPORTED, "%s: too many tiles", who);
+    const uint32_t grid = ((uint32_t)bound + 7) / 8 * 8;
+    hipLaunchKernelGGL((gemm_bf16_seg_gated_kernel<BM, BN, NS, W, FWD>), dim3(grid), dim3(W * 64), lds, st, sa, gu, ld_gu);
+    return check_launch("gemm_bf16_seg_gated_kernel");
+}
+
+extern "C" int pp_gemm_bf16_segmented_swiglu(const void* x, const void* const* w_gate_of, const void* const* w_up_of,
+                                             const int32_t* seg_start, int n_seg, void* gu, void* h, int64_t M,
+                                             int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ld_gu,
+                                             int64_t ldh, pp_stream stream) {
+    const char* who = "pp_gemm_bf16_segmented_swiglu";
+    if (!w_gate_of || !w_up_of || !seg_start || n_seg < 1 || n_seg > PP_GEMM_MAX_SEGMENTS)
+        return fail(PP_ERR_INVALID, "%s: bad segment list (n_seg=%d)", who, n_seg);
+    // the weights are checked for null only: their pointers live in device memory
+    int rc = gated_check(who, x, x, M, N, K, ldx, ldw);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return PP_OK;
+    if (!gu || !h) return fail(PP_ERR_INVALID, "%s: null pointer", who);
+    if (!aligned(gu, 8) || !aligned(h, 8)) return fail(PP_ERR_INVALID, "%s: misaligned pointer", who);
+    if (ld_gu < 2 * N || (ld_gu & 3) || ldh < N || (ldh & 3))
+        return fail(PP_ERR_INVALID, "%s: ld_gu >= 2 N and ldh >= N, both multiples of 4", who);
+    GatedSegArgs sa;
+    fill_args(sa.g, x, nullptr, h, M, N, K, ldx, ldw, ldh);
+    sa.seg_start = seg_start;
+    sa.w_a = w_gate_of;
+    sa.w_b = w_up_of;
+    sa.n_seg = n_seg;
+    return launch_seg_gated<true>(sa, static_cast<uint16_t*>(gu), ld_gu, static_cast<hipStream_t>(stream), who);
+}
+
+extern "C" int pp_gemm_bf16_segmented_dswiglu(const void* dy, const void* const* w_down_t_of, const int32_t* seg_start,
+                                              int n_seg, const void* gu, void* dgu, int64_t M, int64_t N, int64_t K,
+                                              int64_t ldy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu,
+                                              pp_stream stream) {
+    const char* who = "pp_gemm_bf16_segmented_dswiglu";
+    if (!w_down_t_of || !seg_start || n_seg < 1 || n_seg > PP_GEMM_MAX_SEGMENTS)
+        return fail(PP_ERR_INVALID, "%s: bad segment list (n_seg=%d)", who, n_seg);
+    int rc = gated_check(who, dy, dy, M, N, K, ldy, ldw);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return PP_OK;
+    if (!gu || !dgu) return fail(PP_ERR_INVALID, "%s: null pointer", who);
+    if (!aligned(gu, 8) || !aligned(dgu, 8)) return fail(PP_ERR_INVALID, "%s: misaligned pointer", who);
+    if (ld_gu < 2 * N || (ld_gu & 3) || ld_dgu < 2 * N || (ld_dgu & 3))
+        return fail(PP_ERR_INVALID, "%s: ld_gu and ld_dgu >= 2 N, multiples of 4", who);
+    GatedSegArgs sa;
+    fill_args(sa.g, dy, nullptr, dgu, M, N, K, ldy, ldw, ld_dgu);
+    sa.seg_start = seg_start;
+    sa.w_a = w_down_t_of;
+    sa.w_b = nullptr;
+    sa.n_seg = n_seg;
+    // the kernel reads gu; it is passed through the same parameter as the forward's output
+    return launch_seg_gated<false>(sa, const_cast<uint16_t*>(static_cast<const uint16_t*>(gu)), ld_gu,
+                                   static_cast<hipStream_t>(stream), who);
 }

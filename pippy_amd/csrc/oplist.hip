@@ -160,6 +160,15 @@ static int run_one(const pp_op& op, pp_stream st) {
         case PP_OP_GEMM_DSWIGLU:
             return pp_gemm_bf16_dswiglu(op.p[0], op.p[1], op.p[2], op.p[3], op.i[0], op.i[1], op.i[2], op.i[3], op.i[4],
                                         op.i[5], op.i[6], st);
+        case PP_OP_GEMM_SEG_SWIGLU:
+            return pp_gemm_bf16_segmented_swiglu(op.p[0], static_cast<const void* const*>(op.p[1]),
+                                                 static_cast<const void* const*>(op.p[2]),
+                                                 static_cast<const int32_t*>(op.p[5]), (int)op.i[7], op.p[3], op.p[4],
+                                                 op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5], op.i[6], st);
+        case PP_OP_GEMM_SEG_DSWIGLU:
+            return pp_gemm_bf16_segmented_dswiglu(op.p[0], static_cast<const void* const*>(op.p[1]),
+                                                  static_cast<const int32_t*>(op.p[4]), (int)op.i[7], op.p[2], op.p[3],
+                                                  op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.i[5], op.i[6], st);
         case PP_OP_ROPE:
             return pp_rope(op.p[0], static_cast<const float*>(op.p[1]), static_cast<const float*>(op.p[2]),
                            op.i[0], op.i[1], op.i[2], op.i[3], op.i[4], op.j[0], st);
@@ -219,6 +228,7 @@ double op_work(const pp_op& op) {
         case PP_OP_GEMM_BF16:
         case PP_OP_GEMM_F32:
         case PP_OP_GEMM_DSWIGLU:
+        case PP_OP_GEMM_SEG_DSWIGLU:
         case PP_OP_GEMM_SEG:  // the segments partition the rows (rows mode: M, k mode: K)
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_GEMM_SEG_KSEG:  // per microbatch the segments partition K (the upper bound given in i[2])
@@ -226,6 +236,7 @@ double op_work(const pp_op& op) {
         case PP_OP_GEMM_KSEG:  // one product per segment
             return 2.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2] * (double)op.i[7];
         case PP_OP_GEMM_SWIGLU:  // two products of N columns each
+        case PP_OP_GEMM_SEG_SWIGLU:
             return 4.0 * (double)op.i[0] * (double)op.i[1] * (double)op.i[2];
         case PP_OP_ATTN_FWD:  // dense count: QK^T and PV
             return 4.0 * (double)op.i[0] * (double)op.i[2] * (double)op.i[1] * (double)op.i[1] * (double)op.i[3];

@@ -1017,13 +1017,21 @@ class _MoEFeedForward:
         w1, ld1 = pointers("w1", bank.weights(b, "gate"))
         w3, ld3 = pointers("w3", bank.weights(b, "up"))
         w2, ld2 = pointers("w2", bank.weights(b, "down"))
-        g = b.act("g", (R, ffn))
-        u = b.act("u", (R, ffn))
         h = b.act("h", (R, ffn))
         yp = b.act("yp", (R, Cc))
-        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w1, seg, Cm=g, ld=ld1))
-        b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w3, seg, Cm=u, ld=ld3))
-        b.f(P.op_swiglu_fwd(g, u, h))
+        # SwiGLU inside the expert GEMMs (gate and up products side by side, as those kernels write and read
+        # them) when both weights of a tile share a leading dimension; else GEMMs and element-wise kernels
+        fused = ld1 == ld3
+        if fused:
+            gu = b.act("gu", (R, 2 * ffn))
+            g, u = gu[:, :ffn], gu[:, ffn:]
+            b.f(P.op_gemm_seg_swiglu(xp, w1, w3, seg, gu, h, ld=ld1))
+        else:
+            g = b.act("g", (R, ffn))
+            u = b.act("u", (R, ffn))
+            b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w1, seg, Cm=g, ld=ld1))
+            b.f(P.op_gemm_seg(N.SEG_ROWS, xp, w3, seg, Cm=u, ld=ld3))
+            b.f(P.op_swiglu_fwd(g, u, h))
         b.f(P.op_gemm_seg(N.SEG_ROWS, h, w2, seg, Cm=yp, ld=ld2))
         y = b.act("y", (T, Cc))
         b.f(P.op_moe_combine(yp, pos, K, y, gate=gate.view(-1), resid=x2))
@@ -1037,11 +1045,16 @@ class _MoEFeedForward:
             w2t, ld2t = pointers("w2t", bank.transposed(b, "down"))
             w1t, ld1t = pointers("w1t", bank.transposed(b, "gate"))
             w3t, ld3t = pointers("w3t", bank.transposed(b, "up"))
-            d_h = b.grad("d_h", (R, ffn))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, d_yp, w2t, seg, Cm=d_h, ld=ld2t))
-            dg = b.grad("dg", (R, ffn))
-            du = b.grad("du", (R, ffn))
-            b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
+            if fused:
+                dgu = b.grad("dgu", (R, 2 * ffn))
+                dg, du = dgu[:, :ffn], dgu[:, ffn:]
+                b.i(P.op_gemm_seg_dswiglu(d_yp, w2t, seg, gu, dgu, ld=ld2t))
+            else:
+                d_h = b.grad("d_h", (R, ffn))
+                b.i(P.op_gemm_seg(N.SEG_ROWS, d_yp, w2t, seg, Cm=d_h, ld=ld2t))
+                dg = b.grad("dg", (R, ffn))
+                du = b.grad("du", (R, ffn))
+                b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
             d_xp = b.grad("d_xp", (R, Cc))
             b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp, ld=ld1t))
             b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, ld=ld3t, epilogue=N.EPI_BIAS_RESIDUAL,

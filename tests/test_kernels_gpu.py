@@ -1323,6 +1323,12 @@ def test_gemm_fused_swiglu_rejects_bad_arguments():
         N.gemm_swiglu(x, w, w, gu, h)
     with pytest.raises(RuntimeError, match="multiple of 8"):
         N.gemm_dswiglu(x, w, gu, gu.clone())
+    seg = torch.tensor([0, 16], dtype=torch.int32, device="cuda")
+    ptr = torch.tensor([w.data_ptr()], dtype=torch.int64, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        N.gemm_segmented_swiglu(x, ptr, ptr, seg, gu, h)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        N.gemm_segmented_dswiglu(x, ptr, seg, gu, gu.clone())
 
 
 @pytest.mark.gpu
@@ -1485,6 +1491,51 @@ def test_segmented_gemm_rows_mode(R, K, Nn, E):
     assert_close_rel(Cm, ref, BF16_TOL, "segmented rows")
     N.gemm_bf16_segmented(Ad, ptrs, Cm, segd, N.SEG_ROWS, epilogue=N.EPI_BIAS_RESIDUAL, aux_in=auxd)
     assert_close_rel(Cm, ref + aux.float(), BF16_TOL, "segmented rows + residual")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,K,F,E", [(4096, 1024, 512, 8), (1000, 256, 384, 5), (130, 64, 128, 3),
+                                     (3000, 64, 136, 63), (2000, 64, 128, 130)])
+def test_segmented_gemms_with_swiglu_inside_leave_the_bits_of_the_separate_kernels(R, K, F, E):
+    """The expert feed-forward's gate / up GEMM with SwiGLU in its epilogue, and the down projection's
+    input-gradient GEMM with its derivative, over ragged row segments with a weight each (one of them
+    empty): the bits of the segmented GEMMs followed by the element-wise kernels; rows and columns that
+    belong to no tile of a segment keep their fill."""
+    N = native()
+    torch.manual_seed(R + F)
+    seg = _segments(R, E, R + 1)
+    seg[2] = seg[1]
+    x = (torch.randn(R, K) * 0.5).to(torch.bfloat16).to(DEV)
+    dy = (torch.randn(R, K) * 0.5).to(torch.bfloat16).to(DEV)
+    wg = (torch.randn(E, F, K) * 0.1).to(torch.bfloat16).to(DEV)
+    wu = (torch.randn(E, F, K) * 0.05).to(torch.bfloat16).to(DEV)
+    wdt = (torch.randn(E, F, K) * 0.05).to(torch.bfloat16).to(DEV)
+    ptrs = lambda w: torch.tensor([w[e].data_ptr() for e in range(E)], dtype=torch.int64, device=DEV)
+    pg, pu, pd = ptrs(wg), ptrs(wu), ptrs(wdt)
+    segd = seg.int().to(DEV)
+    g = torch.empty(R, F, dtype=torch.bfloat16, device=DEV)
+    u, h, dh, dg, du = (torch.empty_like(g) for _ in range(5))
+    N.gemm_bf16_segmented(x, pg, g, segd, N.SEG_ROWS)
+    N.gemm_bf16_segmented(x, pu, u, segd, N.SEG_ROWS)
+    N.swiglu_fwd(g, u, h)
+    N.gemm_bf16_segmented(dy, pd, dh, segd, N.SEG_ROWS)
+    N.swiglu_bwd(g, u, dh, dg, du)
+    gu = torch.full((R, 2 * F + 8), 7.0, dtype=torch.bfloat16, device=DEV)      # a leading dimension beyond 2 F
+    hf = torch.full((R, F), 7.0, dtype=torch.bfloat16, device=DEV)
+    dgu = torch.full((R, 2 * F + 8), 7.0, dtype=torch.bfloat16, device=DEV)
+    N.gemm_segmented_swiglu(x, pg, pu, segd, gu[:, :2 * F], hf)
+    N.gemm_segmented_dswiglu(dy, pd, segd, gu[:, :2 * F], dgu[:, :2 * F])
+    torch.cuda.synchronize()
+    assert torch.equal(gu[:, :F], g) and torch.equal(gu[:, F:2 * F], u), "gate / up products"
+    assert torch.equal(hf, h), "activation"
+    assert torch.equal(dgu[:, :F], dg) and torch.equal(dgu[:, F:2 * F], du), "gate / up gradients"
+    assert bool((gu[:, 2 * F:] == 7.0).all()) and bool((dgu[:, 2 * F:] == 7.0).all()), "stray writes"
+    # fp32 statement of one non-empty segment
+    e = int(torch.argmax(seg[1:] - seg[:-1]))
+    r0, r1 = int(seg[e]), int(seg[e + 1])
+    gr = x[r0:r1].float() @ wg[e].float().T
+    ur = x[r0:r1].float() @ wu[e].float().T
+    assert_close_rel(hf[r0:r1], torch.nn.functional.silu(gr) * ur, BF16_TOL, "segment of h")
 
 
 @pytest.mark.gpu
