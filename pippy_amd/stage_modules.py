@@ -888,6 +888,11 @@ class _ExpertModules:
     def transposed(self, b, which):
         return [b.weight_t(p) for p in self._params(which)], None
 
+    def transposed_gate_up(self, b):
+        """Per expert [in, 2 f]: the transposed gate and up weights side by side, so that the input gradient
+        of both projections is one product with [dg | du]."""
+        return [b.weight_t_cat(g, u) for g, u in zip(self._params("gate"), self._params("up"))], None
+
     def grad_epilogue(self, b, which):
         epis = {b.weight_grad_epilogue(p) for p in self._params(which)}
         assert len(epis) == 1
@@ -936,6 +941,10 @@ class _ExpertTensors:
             return [t[e] for e in range(len(self))], None
         f = self.ffn
         return [t[e][:, :f] if which == "gate" else t[e][:, f:] for e in range(len(self))], 2 * f
+
+    def transposed_gate_up(self, b):
+        t = b.sp.arena.weight_t_stack(self.gate_up)             # [E, in, 2 f]: gate columns first
+        return [t[e] for e in range(len(self))], None
 
     def grad_epilogue(self, b, which):
         return b.weight_grad_epilogue(self._param(which))
@@ -1043,8 +1052,6 @@ class _MoEFeedForward:
             dlogits = b.grad("dlogits", (T, Ep))
             b.i(P.op_moe_gate_bwd(dy2d, yp, pos, idx, gate, E, dlogits))
             w2t, ld2t = pointers("w2t", bank.transposed(b, "down"))
-            w1t, ld1t = pointers("w1t", bank.transposed(b, "gate"))
-            w3t, ld3t = pointers("w3t", bank.transposed(b, "up"))
             if fused:
                 dgu = b.grad("dgu", (R, 2 * ffn))
                 dg, du = dgu[:, :ffn], dgu[:, ffn:]
@@ -1056,9 +1063,16 @@ class _MoEFeedForward:
                 du = b.grad("du", (R, ffn))
                 b.i(P.op_swiglu_bwd(g, u, d_h, dg, du))
             d_xp = b.grad("d_xp", (R, Cc))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp, ld=ld1t))
-            b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, ld=ld3t, epilogue=N.EPI_BIAS_RESIDUAL,
-                              aux_in=d_xp))
+            if fused:
+                # dg W1 + du W3 as one product of [dg | du] with the two transposed weights side by side
+                w13t, ld13t = pointers("w13t", bank.transposed_gate_up(b))
+                b.i(P.op_gemm_seg(N.SEG_ROWS, dgu, w13t, seg, Cm=d_xp, ld=ld13t))
+            else:
+                w1t, ld1t = pointers("w1t", bank.transposed(b, "gate"))
+                w3t, ld3t = pointers("w3t", bank.transposed(b, "up"))
+                b.i(P.op_gemm_seg(N.SEG_ROWS, dg, w1t, seg, Cm=d_xp, ld=ld1t))
+                b.i(P.op_gemm_seg(N.SEG_ROWS, du, w3t, seg, Cm=d_xp, ld=ld3t, epilogue=N.EPI_BIAS_RESIDUAL,
+                                  aux_in=d_xp))
             # token gradient: its two expert rows, plus the router branch in the GEMM epilogue
             d_n2a = b.grad("d_n2a", (T, Cc))
             b.i(P.op_moe_combine(d_xp, pos, K, d_n2a))
