@@ -176,6 +176,27 @@ def test_gemm_bf16_large_output_takes_256_wide_tiles():
     assert bool(torch.isnan(Cbuf[:, N:]).all())
 
 
+def test_gemm_bf16_output_that_fills_its_rounds_better_takes_256_x_192_tiles():
+    """An output whose 256 x 192 tiles fill two rounds of work-groups where 256 x 256 tiles leave the second
+    a quarter empty (the shape of a Llama-2-7B q | k | v projection over 2048 tokens) runs on the 192-wide
+    tile variant: edges in M and N, a k tail, a ragged leading dimension, and the same bits as the rows
+    computed alone on the small tiles (the reduction order does not depend on the tile)."""
+    Nn = native()
+    torch.manual_seed(12)
+    M, N, K = 2048 - 8, 12288 - 8, 200
+    A = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    B = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    Cbuf = torch.full((M, N + 4), float("nan"), device=DEV, dtype=torch.bfloat16)
+    C = Cbuf[:, :N]
+    Nn.gemm_bf16(A, B, C)
+    ref = A.float() @ B.float().t()
+    assert_close_rel(C, ref.cpu(), BF16_TOL, "gemm, 256 x 192 tiles")
+    assert bool(torch.isnan(Cbuf[:, N:]).all())
+    part = torch.empty(M, 768, device=DEV, dtype=torch.bfloat16)      # 16 x 8 tiles of 128 x 96: the small path
+    Nn.gemm_bf16(A, B[4096:4096 + 768], part)
+    assert torch.equal(part, C[:, 4096:4096 + 768])
+
+
 @pytest.mark.parametrize("M,N,K", [(384, 264, 136), (512, 380, 136), (4096, 768, 264), (4096, 2304, 136)])
 def test_gemm_bf16_epilogues(M, N, K):
     """The second and third shapes run on 96-column tiles (they fill more CUs than 128-column ones),
